@@ -1,0 +1,270 @@
+"""CPU oracle bindings -- TEST INFRASTRUCTURE ONLY.
+
+ctypes front-end of ``oracle/splatad_oracle.c`` (a plain-C restatement of the
+reference's rendering path).  Only ``tests/``, ``__graft_entry__.smoke()`` and
+the ``cpu_baseline`` leg of ``bench.py`` may import this package; the shipped
+``splatad_amd`` package never does.
+
+All functions take and return numpy arrays (float32 inputs; outputs are
+float32 for ``precision="f32"`` and float64 for ``"f64"``).  Integer outputs
+(tile intersections, sort order, offsets) exist only in single precision,
+because the reference computes the tile bounds in float32
+(``gsplat/cuda/csrc/rasterization.cu:46-56, 321-357``).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_DIR = os.path.dirname(os.path.abspath(__file__))
+_LIBS = {}
+
+
+def build(force: bool = False) -> None:
+    """Compile both oracle libraries with gcc (``make -C oracle``)."""
+    if force:
+        subprocess.check_call(["make", "-C", _DIR, "clean"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(["make", "-C", _DIR], stdout=subprocess.DEVNULL)
+
+
+def _lib(precision: str):
+    if precision not in ("f32", "f64"):
+        raise ValueError(precision)
+    if precision not in _LIBS:
+        path = os.path.join(_DIR, f"liboracle_{precision}.so")
+        if not os.path.exists(path):
+            build()
+        _LIBS[precision] = ctypes.CDLL(path)
+    return _LIBS[precision]
+
+
+def _real(precision):
+    return np.float32 if precision == "f32" else np.float64
+
+
+def _f32(a):
+    return None if a is None else np.ascontiguousarray(np.asarray(a, dtype=np.float32))
+
+
+def _p(a):
+    if a is None:
+        return ctypes.c_void_p(0)
+    assert a.flags["C_CONTIGUOUS"]
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def set_num_threads(n: int) -> None:
+    """OpenMP thread count used by the oracle loops (``OMP_NUM_THREADS``)."""
+    os.environ["OMP_NUM_THREADS"] = str(n)
+    try:
+        omp = ctypes.CDLL("libgomp.so.1")
+        omp.omp_set_num_threads(int(n))
+    except OSError:
+        pass
+
+
+# ---------------------------------------------------------------------------
+# projection
+# ---------------------------------------------------------------------------
+def projection_fwd(means, covars, quats, scales, velocities, viewmats, Ks, width, height,
+                   linear_velocity, angular_velocity, rolling_shutter_time, eps2d=0.3,
+                   near_plane=0.01, far_plane=1e10, radius_clip=0.0, calc_compensations=False,
+                   precision="f32"):
+    """Restates ``fully_fused_projection_fwd`` (projection.cu:605-751).
+
+    Returns (radii int32[C,N,2], means2d, depths, conics, compensations|None, pix_vels).
+    """
+    lib, rt = _lib(precision), _real(precision)
+    means = _f32(means); covars = _f32(covars); quats = _f32(quats); scales = _f32(scales)
+    velocities = _f32(velocities); viewmats = _f32(viewmats); Ks = _f32(Ks)
+    lv = _f32(linear_velocity); av = _f32(angular_velocity); rs = _f32(rolling_shutter_time)
+    C, N = viewmats.shape[0], means.shape[0]
+    radii = np.zeros((C, N, 2), np.int32)
+    means2d = np.zeros((C, N, 2), rt); depths = np.zeros((C, N), rt)
+    conics = np.zeros((C, N, 3), rt); pix_vels = np.zeros((C, N, 2), rt)
+    comps = np.zeros((C, N), rt) if calc_compensations else None
+    fn = getattr(lib, f"oracle_{precision}_projection_fwd")
+    fn.restype = None
+    fn(ctypes.c_int(C), ctypes.c_int(N), _p(means), _p(covars), _p(quats), _p(scales),
+       _p(velocities), _p(viewmats), _p(Ks), ctypes.c_int(width), ctypes.c_int(height), _p(lv),
+       _p(av), _p(rs), ctypes.c_float(eps2d), ctypes.c_float(near_plane),
+       ctypes.c_float(far_plane), ctypes.c_float(radius_clip), _p(radii), _p(means2d),
+       _p(depths), _p(conics), _p(comps), _p(pix_vels))
+    return radii, means2d, depths, conics, comps, pix_vels
+
+
+def lidar_projection_fwd(means, covars, quats, scales, velocities, viewmats, min_elevation,
+                         max_elevation, min_azimuth, max_azimuth, linear_velocity,
+                         angular_velocity, rolling_shutter_time, eps2d=0.01, near_plane=0.01,
+                         far_plane=1e10, radius_clip=0.0, calc_compensations=False,
+                         precision="f32"):
+    """Restates ``fully_fused_lidar_projection_fwd`` (projection.cu:2268-2417).
+
+    Returns (radii[C,N,2], means2d, depths, conics, compensations|None, pix_vels[C,N,3],
+    depth_compensations[C,N,2]).
+    """
+    lib, rt = _lib(precision), _real(precision)
+    means = _f32(means); covars = _f32(covars); quats = _f32(quats); scales = _f32(scales)
+    velocities = _f32(velocities); viewmats = _f32(viewmats)
+    lv = _f32(linear_velocity); av = _f32(angular_velocity); rs = _f32(rolling_shutter_time)
+    C, N = viewmats.shape[0], means.shape[0]
+    radii = np.zeros((C, N, 2), rt)
+    means2d = np.zeros((C, N, 2), rt); depths = np.zeros((C, N), rt)
+    conics = np.zeros((C, N, 3), rt); pix_vels = np.zeros((C, N, 3), rt)
+    dcomps = np.zeros((C, N, 2), rt)
+    comps = np.zeros((C, N), rt) if calc_compensations else None
+    fn = getattr(lib, f"oracle_{precision}_lidar_projection_fwd")
+    fn.restype = None
+    fn(ctypes.c_int(C), ctypes.c_int(N), _p(means), _p(covars), _p(quats), _p(scales),
+       _p(velocities), _p(viewmats), ctypes.c_float(min_elevation), ctypes.c_float(max_elevation),
+       ctypes.c_float(min_azimuth), ctypes.c_float(max_azimuth), _p(lv), _p(av), _p(rs),
+       ctypes.c_float(eps2d), ctypes.c_float(near_plane), ctypes.c_float(far_plane),
+       ctypes.c_float(radius_clip), _p(radii), _p(means2d), _p(depths), _p(conics), _p(comps),
+       _p(pix_vels), _p(dcomps))
+    return radii, means2d, depths, conics, comps, pix_vels, dcomps
+
+
+def spherical_harmonics(degree, dirs, coeffs, masks=None, precision="f32"):
+    """Restates ``compute_sh_fwd`` (sh.cu:13-93, 355-374); masked rows are zero."""
+    lib, rt = _lib(precision), _real(precision)
+    dirs = _f32(dirs); coeffs = _f32(coeffs)
+    K = coeffs.shape[-2]
+    n = dirs.size // 3
+    m = None if masks is None else np.ascontiguousarray(np.asarray(masks, dtype=np.uint8))
+    colors = np.zeros(dirs.shape, rt)
+    fn = getattr(lib, f"oracle_{precision}_sh_fwd")
+    fn.restype = None
+    fn(ctypes.c_long(n), ctypes.c_int(K), ctypes.c_int(degree), _p(dirs), _p(coeffs), _p(m),
+       _p(colors))
+    return colors
+
+
+# ---------------------------------------------------------------------------
+# intersection / sort / offsets (single precision only)
+# ---------------------------------------------------------------------------
+def bit_width(v: int) -> int:
+    return int(v).bit_length()
+
+
+def _isect(lidar, means2d, radii, depths, tile_size, tile_w, tile_h, elev_boundaries,
+           tile_azim_res, min_azim, sort, n_cameras, camera_ids):
+    lib = _lib("f32")
+    means2d = _f32(means2d); depths = _f32(depths)
+    radii = _f32(radii) if lidar else np.ascontiguousarray(np.asarray(radii, dtype=np.int32))
+    eb = _f32(elev_boundaries)
+    packed = means2d.ndim == 2
+    if packed:
+        total = means2d.shape[0]; N = 0; C = n_cameras
+        cam = np.ascontiguousarray(np.asarray(camera_ids, dtype=np.int64))
+    else:
+        C, N = means2d.shape[:2]; total = C * N; cam = None
+    tpg = np.zeros(depths.shape, np.int32)
+    lib.oracle_isect_count.restype = ctypes.c_long
+    n_isects = lib.oracle_isect_count(
+        ctypes.c_int(lidar), ctypes.c_long(total), _p(means2d), _p(radii),
+        ctypes.c_uint32(tile_size), ctypes.c_uint32(tile_w), ctypes.c_uint32(tile_h), _p(eb),
+        ctypes.c_float(tile_azim_res), ctypes.c_float(min_azim), _p(tpg))
+    ids = np.zeros((n_isects,), np.int64); flat = np.zeros((n_isects,), np.int32)
+    lib.oracle_isect_emit.restype = None
+    lib.oracle_isect_emit(
+        ctypes.c_int(lidar), ctypes.c_long(total), ctypes.c_long(N), _p(cam), _p(means2d),
+        _p(radii), _p(depths), ctypes.c_uint32(tile_size), ctypes.c_uint32(tile_w),
+        ctypes.c_uint32(tile_h), _p(eb), ctypes.c_float(tile_azim_res), ctypes.c_float(min_azim),
+        _p(ids), _p(flat))
+    if sort and n_isects:
+        end_bit = 32 + bit_width(tile_w * tile_h) + bit_width(C)
+        lib.oracle_sort_pairs.restype = None
+        lib.oracle_sort_pairs(ctypes.c_long(n_isects), ctypes.c_int(end_bit), _p(ids), _p(flat))
+    return tpg, ids, flat
+
+
+def isect_tiles(means2d, radii, depths, tile_size, tile_width, tile_height, sort=True,
+                n_cameras=None, camera_ids=None):
+    """Restates ``isect_tiles`` (rasterization.cu:15-216)."""
+    return _isect(0, means2d, radii, depths, tile_size, tile_width, tile_height, None, 0.0, 0.0,
+                  sort, n_cameras, camera_ids)
+
+
+def isect_lidar_tiles(means2d, radii, depths, elev_boundaries, tile_azim_resolution, min_azim,
+                      sort=True, n_cameras=None, camera_ids=None):
+    """Restates ``isect_lidar_tiles`` (rasterization.cu:287-529)."""
+    import math
+    # rasterization.cu:435-436: float32 division, ceil
+    n_tiles_azim = int(math.ceil(float(np.float32(360.0) / np.float32(tile_azim_resolution))))
+    n_tiles_elev = int(np.asarray(elev_boundaries).shape[0] - 1)
+    return _isect(1, means2d, radii, depths, 0, n_tiles_azim, n_tiles_elev, elev_boundaries,
+                  tile_azim_resolution, min_azim, sort, n_cameras, camera_ids)
+
+
+def isect_offset_encode(isect_ids, n_cameras, tile_width, tile_height):
+    """Restates ``isect_offset_encode`` (rasterization.cu:218-285)."""
+    lib = _lib("f32")
+    ids = np.ascontiguousarray(np.asarray(isect_ids, dtype=np.int64))
+    offsets = np.zeros((n_cameras, tile_height, tile_width), np.int32)
+    lib.oracle_isect_offset_encode.restype = None
+    lib.oracle_isect_offset_encode(ctypes.c_long(ids.shape[0]), _p(ids),
+                                   ctypes.c_uint32(n_cameras),
+                                   ctypes.c_uint32(tile_width * tile_height), _p(offsets))
+    return offsets
+
+
+# ---------------------------------------------------------------------------
+# rasterization
+# ---------------------------------------------------------------------------
+def rasterize_to_pixels_fwd(means2d, conics, colors, opacities, pix_vels, rolling_shutter_time,
+                            backgrounds, width, height, tile_size, isect_offsets, flatten_ids,
+                            precision="f32"):
+    """Restates ``rasterize_to_pixels_fwd`` (rasterization.cu:1360-1518).
+
+    Returns (render_colors[C,H,W,D], render_alphas[C,H,W,1], last_ids int32[C,H,W]).
+    """
+    lib, rt = _lib(precision), _real(precision)
+    means2d = _f32(means2d); conics = _f32(conics); colors = _f32(colors)
+    opacities = _f32(opacities); pix_vels = _f32(pix_vels); rs = _f32(rolling_shutter_time)
+    bg = _f32(backgrounds)
+    offs = np.ascontiguousarray(np.asarray(isect_offsets, dtype=np.int32))
+    flat = np.ascontiguousarray(np.asarray(flatten_ids, dtype=np.int32))
+    C, th, tw = offs.shape
+    D = colors.shape[-1]
+    rc = np.zeros((C, height, width, D), rt); ra = np.zeros((C, height, width, 1), rt)
+    last = np.zeros((C, height, width), np.int32)
+    fn = getattr(lib, f"oracle_{precision}_rasterize_to_pixels_fwd")
+    fn.restype = None
+    fn(ctypes.c_int(C), ctypes.c_long(flat.shape[0]), ctypes.c_int(D), _p(means2d), _p(conics),
+       _p(colors), _p(opacities), _p(pix_vels), _p(rs), _p(bg), ctypes.c_int(width),
+       ctypes.c_int(height), ctypes.c_int(tile_size), ctypes.c_int(tw), ctypes.c_int(th),
+       _p(offs), _p(flat), _p(rc), _p(ra), _p(last))
+    return rc, ra, last
+
+
+def rasterize_to_points_fwd(means2d, conics, colors, opacities, pix_vels, depth_compensations,
+                            backgrounds, raster_pts, width, height, tile_width, tile_height,
+                            compute_alpha_sum_until_points, threshold, isect_offsets, flatten_ids,
+                            depth_channel_idx, precision="f32"):
+    """Restates ``rasterize_to_points_fwd`` (rasterization.cu:2021-2219).
+
+    Returns (render_colors, render_alphas, last_ids, alpha_sum_until_points|None,
+    median_depths), the order of the reference's C++ op.
+    """
+    lib, rt = _lib(precision), _real(precision)
+    means2d = _f32(means2d); conics = _f32(conics); colors = _f32(colors)
+    opacities = _f32(opacities); pix_vels = _f32(pix_vels); dc = _f32(depth_compensations)
+    bg = _f32(backgrounds); rp = _f32(raster_pts)
+    offs = np.ascontiguousarray(np.asarray(isect_offsets, dtype=np.int32))
+    flat = np.ascontiguousarray(np.asarray(flatten_ids, dtype=np.int32))
+    C, gh, gw = offs.shape
+    D = colors.shape[-1]
+    rc = np.zeros((C, height, width, D), rt); ra = np.zeros((C, height, width, 1), rt)
+    asum = np.zeros((C, height, width, 1), rt) if compute_alpha_sum_until_points else None
+    med = np.zeros((C, height, width, 1), rt)
+    last = np.zeros((C, height, width), np.int32)
+    fn = getattr(lib, f"oracle_{precision}_rasterize_to_points_fwd")
+    fn.restype = None
+    fn(ctypes.c_int(C), ctypes.c_long(flat.shape[0]), ctypes.c_int(D), _p(means2d), _p(conics),
+       _p(colors), _p(opacities), _p(pix_vels), _p(dc), _p(bg), _p(rp), ctypes.c_int(width),
+       ctypes.c_int(height), ctypes.c_int(tile_width), ctypes.c_int(tile_height),
+       ctypes.c_int(gw), ctypes.c_int(gh), ctypes.c_int(bool(compute_alpha_sum_until_points)),
+       ctypes.c_float(threshold), _p(offs), _p(flat), ctypes.c_int(depth_channel_idx), _p(rc),
+       _p(ra), _p(asum), _p(last), _p(med))
+    return rc, ra, last, asum, med
