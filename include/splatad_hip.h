@@ -1,0 +1,241 @@
+/*
+ * C ABI of libsplatad_hip.so: the MI355X (gfx950) kernels behind the operator
+ * interface of carlinds/splatad's rendering path.
+ *
+ * Conventions (they replace the pybind11/torch::Tensor boundary of the
+ * reference, gsplat/cuda/csrc/ext.cpp:4-52 and bindings.h:123-468):
+ *   - every pointer is a DEVICE pointer to contiguous row-major memory unless
+ *     its name ends in _host; optional tensors are passed as NULL;
+ *   - the caller allocates every output and every workspace (sizes from the
+ *     *_workspace_bytes queries); the library never allocates or frees device
+ *     memory;
+ *   - all work is enqueued on `stream` (a hipStream_t); the only host
+ *     synchronisation is inside the *_count entry points, which copy one
+ *     integer back to the host (the reference does the same through
+ *     Tensor::item(): rasterization.cu:154,465, projection.cu:1421);
+ *   - return value 0 = success, negative = error; splatad_last_error() gives a
+ *     thread-local message (the reference raises through TORCH_CHECK,
+ *     bindings.h:9-13).
+ * dtypes: float = IEEE binary32; radii are int32 for cameras and float for
+ * lidars; isect ids int64; flatten ids / offsets / last ids int32; camera and
+ * gaussian ids int64; masks are one byte per element.
+ */
+#ifndef SPLATAD_HIP_H
+#define SPLATAD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *splatad_stream_t; /* hipStream_t */
+
+const char *splatad_last_error(void);
+int splatad_abi_version(void);
+
+/* ---- projection ------------------------------------------------------- */
+
+/* fully_fused_projection_fwd_tensor, projection.cu:966-1045 (kernel :605-751).
+ * Exactly one of covars or (quats, scales) is non-NULL.  compensations may be
+ * NULL.  Rows of culled Gaussians are written as zeros. */
+int splatad_projection_fwd(uint32_t C, uint32_t N, const float *means, const float *covars,
+                           const float *quats, const float *scales, const float *velocities,
+                           const float *viewmats, const float *Ks, uint32_t image_width,
+                           uint32_t image_height, const float *linear_velocity,
+                           const float *angular_velocity, const float *rolling_shutter_time,
+                           float eps2d, float near_plane, float far_plane, float radius_clip,
+                           int32_t *radii, float *means2d, float *depths, float *conics,
+                           float *compensations, float *pix_vels, splatad_stream_t stream);
+
+/* fully_fused_projection_packed_fwd_tensor, projection.cu:1355-1464, as a
+ * two-call protocol: _count projects into the workspace and returns nnz on the
+ * host, _fill compacts into [nnz,...] outputs ordered by (camera, gaussian). */
+size_t splatad_projection_packed_workspace_bytes(uint32_t C, uint32_t N);
+int splatad_projection_packed_count(uint32_t C, uint32_t N, const float *means,
+                                    const float *covars, const float *quats, const float *scales,
+                                    const float *velocities, const float *viewmats,
+                                    const float *Ks, uint32_t image_width, uint32_t image_height,
+                                    const float *linear_velocity, const float *angular_velocity,
+                                    const float *rolling_shutter_time, float eps2d,
+                                    float near_plane, float far_plane, float radius_clip,
+                                    int calc_compensations, void *workspace, int64_t *nnz_host,
+                                    splatad_stream_t stream);
+int splatad_projection_packed_fill(uint32_t C, uint32_t N, int64_t nnz, const void *workspace,
+                                   int32_t *indptr, int64_t *camera_ids, int64_t *gaussian_ids,
+                                   int32_t *radii, float *means2d, float *depths, float *conics,
+                                   float *compensations, float *pix_vels,
+                                   splatad_stream_t stream);
+
+/* fully_fused_lidar_projection_fwd_tensor, projection.cu:2631-2714 (kernel :2268-2417). */
+int splatad_lidar_projection_fwd(uint32_t C, uint32_t N, const float *means, const float *covars,
+                                 const float *quats, const float *scales, const float *velocities,
+                                 const float *viewmats, float min_elevation, float max_elevation,
+                                 float min_azimuth, float max_azimuth,
+                                 const float *linear_velocity, const float *angular_velocity,
+                                 const float *rolling_shutter_time, float eps2d, float near_plane,
+                                 float far_plane, float radius_clip, float *radii, float *means2d,
+                                 float *depths, float *conics, float *compensations,
+                                 float *pix_vels, float *depth_compensations,
+                                 splatad_stream_t stream);
+
+/* fully_fused_projection_bwd_tensor, projection.cu:1047-1155 (kernel :753-964).
+ * Gradient outputs must be zero-filled by the caller; v_covars xor (v_quats,
+ * v_scales); v_viewmats and v_velocities may be NULL.  v_velocities is an
+ * extension: the reference computes and drops it (projection.cu:874-877). */
+int splatad_projection_bwd(uint32_t C, uint32_t N, const float *means, const float *covars,
+                           const float *quats, const float *scales, const float *velocities,
+                           const float *viewmats, const float *Ks, uint32_t image_width,
+                           uint32_t image_height, const float *linear_velocity,
+                           const float *angular_velocity, const float *rolling_shutter_time,
+                           float eps2d, const int64_t *camera_ids, const int64_t *gaussian_ids,
+                           int64_t nnz, const int32_t *radii, const float *conics,
+                           const float *compensations, const float *v_means2d,
+                           const float *v_depths, const float *v_conics,
+                           const float *v_compensations, const float *v_pix_vels, int sparse_grad,
+                           float *v_means, float *v_covars, float *v_quats, float *v_scales,
+                           float *v_viewmats, float *v_velocities, splatad_stream_t stream);
+
+/* fully_fused_lidar_projection_bwd_tensor, projection.cu:2716-2826 (kernel :2419-2629). */
+int splatad_lidar_projection_bwd(uint32_t C, uint32_t N, const float *means, const float *covars,
+                                 const float *quats, const float *scales, const float *velocities,
+                                 const float *viewmats, const float *linear_velocity,
+                                 const float *angular_velocity, const float *rolling_shutter_time,
+                                 float eps2d, const float *radii, const float *conics,
+                                 const float *compensations, const float *v_means2d,
+                                 const float *v_depths, const float *v_conics,
+                                 const float *v_compensations, const float *v_pix_vels,
+                                 const float *v_depth_compensations, float *v_means,
+                                 float *v_covars, float *v_quats, float *v_scales,
+                                 float *v_viewmats, float *v_velocities, splatad_stream_t stream);
+
+/* ---- spherical harmonics ------------------------------------------------ */
+
+/* compute_sh_fwd_tensor / compute_sh_bwd_tensor, sh.cu:408-468.  n = number of
+ * directions, K = number of bases in coeffs.  Masked-out rows are zero.
+ * v_coeffs must be zero-filled; v_dirs may be NULL. */
+int splatad_sh_fwd(uint32_t n, uint32_t K, uint32_t degree, const float *dirs,
+                   const float *coeffs, const uint8_t *masks, float *colors,
+                   splatad_stream_t stream);
+int splatad_sh_bwd(uint32_t n, uint32_t K, uint32_t degree, const float *dirs,
+                   const float *coeffs, const uint8_t *masks, const float *v_colors,
+                   float *v_coeffs, float *v_dirs, splatad_stream_t stream);
+
+/* ---- tile intersection, sort, offsets ----------------------------------- */
+
+/* isect_tiles_tensor (rasterization.cu:92-216) and isect_lidar_tiles_tensor
+ * (:397-529) as a two-call protocol.  total = C*N (camera_ids NULL) or nnz
+ * (packed, camera_ids given).  _count writes tiles_per_gauss and returns
+ * n_isects on the host; _fill writes isect_ids/flatten_ids, sorted by
+ * (camera, tile, depth bits) with ties in emission order when sort != 0, in
+ * emission order otherwise.  Depths must be non-negative (sign bit clear).
+ * For lidars tile_width/tile_height are the azimuth/elevation tile counts and
+ * elev_boundaries has tile_height+1 entries.  The workspace of _count needs
+ * splatad_isect_workspace_bytes(total, C, n_tiles, 0) bytes, that of _fill
+ * splatad_isect_workspace_bytes(total, C, n_tiles, n_isects); nothing has to
+ * survive between the two calls except tiles_per_gauss. */
+size_t splatad_isect_workspace_bytes(uint64_t total, uint32_t C, uint32_t n_tiles,
+                                     int64_t n_isects);
+int splatad_isect_tiles_count(uint64_t total, const float *means2d, const int32_t *radii,
+                              uint32_t C, uint32_t tile_size, uint32_t tile_width,
+                              uint32_t tile_height, int32_t *tiles_per_gauss, void *workspace,
+                              int64_t *n_isects_host, splatad_stream_t stream);
+int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_ids,
+                             const float *means2d, const int32_t *radii, const float *depths,
+                             uint32_t C, uint32_t tile_size, uint32_t tile_width,
+                             uint32_t tile_height, int sort, int64_t n_isects,
+                             const int32_t *tiles_per_gauss, void *workspace, int64_t *isect_ids,
+                             int32_t *flatten_ids, splatad_stream_t stream);
+int splatad_isect_lidar_tiles_count(uint64_t total, const float *means2d, const float *radii,
+                                    uint32_t C, const float *elev_boundaries,
+                                    float tile_azim_resolution, float min_azim,
+                                    uint32_t tile_width, uint32_t tile_height,
+                                    int32_t *tiles_per_gauss, void *workspace,
+                                    int64_t *n_isects_host, splatad_stream_t stream);
+int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_ids,
+                                   const float *means2d, const float *radii, const float *depths,
+                                   uint32_t C, const float *elev_boundaries,
+                                   float tile_azim_resolution, float min_azim,
+                                   uint32_t tile_width, uint32_t tile_height, int sort,
+                                   int64_t n_isects, const int32_t *tiles_per_gauss,
+                                   void *workspace, int64_t *isect_ids, int32_t *flatten_ids,
+                                   splatad_stream_t stream);
+
+/* isect_offset_encode_tensor, rasterization.cu:264-285 (kernel :218-262). */
+int splatad_isect_offset_encode(int64_t n_isects, const int64_t *isect_ids, uint32_t C,
+                                uint32_t n_tiles, int32_t *offsets, splatad_stream_t stream);
+
+/* ---- rasterization ------------------------------------------------------ */
+
+/* rasterize_to_pixels_fwd_tensor, rasterization.cu:1520-2018 (kernel
+ * :1360-1518).  Any channel count >= 1 is accepted (wide inputs are rendered in
+ * passes).  backgrounds may be NULL. */
+int splatad_rasterize_to_pixels_fwd(uint32_t C, int64_t n_isects, uint32_t channels,
+                                    const float *means2d, const float *conics,
+                                    const float *colors, const float *opacities,
+                                    const float *pix_vels, const float *rolling_shutter_time,
+                                    const float *backgrounds, uint32_t image_width,
+                                    uint32_t image_height, uint32_t tile_size,
+                                    uint32_t tile_width, uint32_t tile_height,
+                                    const int32_t *tile_offsets, const int32_t *flatten_ids,
+                                    float *render_colors, float *render_alphas,
+                                    int32_t *last_ids, splatad_stream_t stream);
+
+/* rasterize_to_pixels_bwd_tensor, rasterization.cu:3091-3726 (kernel
+ * :2833-3089).  Gradient outputs must be zero-filled; v_means2d_abs may be NULL. */
+int splatad_rasterize_to_pixels_bwd(uint32_t C, int64_t n_isects, uint32_t channels,
+                                    const float *means2d, const float *conics,
+                                    const float *colors, const float *opacities,
+                                    const float *pix_vels, const float *rolling_shutter_time,
+                                    const float *backgrounds, uint32_t image_width,
+                                    uint32_t image_height, uint32_t tile_size,
+                                    uint32_t tile_width, uint32_t tile_height,
+                                    const int32_t *tile_offsets, const int32_t *flatten_ids,
+                                    const float *render_alphas, const int32_t *last_ids,
+                                    const float *v_render_colors, const float *v_render_alphas,
+                                    float *v_means2d_abs, float *v_means2d, float *v_conics,
+                                    float *v_colors, float *v_opacities, float *v_pix_vels,
+                                    splatad_stream_t stream);
+
+/* rasterize_to_points_fwd_tensor, rasterization.cu:2221-2831 (kernel
+ * :2021-2219).  Outputs of inactive points (range <= 0) are zero.
+ * alpha_sum_until_points may be NULL when compute_alpha_sum_until_points == 0. */
+int splatad_rasterize_to_points_fwd(uint32_t C, int64_t n_isects, uint32_t channels,
+                                    const float *means2d, const float *conics,
+                                    const float *colors, const float *opacities,
+                                    const float *pix_vels, const float *depth_compensations,
+                                    const float *backgrounds, const float *raster_pts,
+                                    uint32_t image_width, uint32_t image_height,
+                                    uint32_t tile_width, uint32_t tile_height,
+                                    uint32_t tile_grid_width, uint32_t tile_grid_height,
+                                    int compute_alpha_sum_until_points, float threshold,
+                                    const int32_t *tile_offsets, const int32_t *flatten_ids,
+                                    uint32_t depth_channel_idx, float *render_colors,
+                                    float *render_alphas, float *alpha_sum_until_points,
+                                    int32_t *last_ids, float *median_depths,
+                                    splatad_stream_t stream);
+
+/* rasterize_to_points_bwd_tensor, rasterization.cu:4056-4851 (kernel :3728-4054). */
+int splatad_rasterize_to_points_bwd(uint32_t C, int64_t n_isects, uint32_t channels,
+                                    const float *means2d, const float *conics,
+                                    const float *colors, const float *opacities,
+                                    const float *pix_vels, const float *depth_compensations,
+                                    const float *backgrounds, const float *raster_pts,
+                                    uint32_t image_width, uint32_t image_height,
+                                    uint32_t tile_width, uint32_t tile_height,
+                                    uint32_t tile_grid_width, uint32_t tile_grid_height,
+                                    int compute_alpha_sum_until_points, float threshold,
+                                    const int32_t *tile_offsets, const int32_t *flatten_ids,
+                                    uint32_t depth_channel_idx, const float *render_alphas,
+                                    const int32_t *last_ids, const float *v_render_colors,
+                                    const float *v_render_alphas,
+                                    const float *v_alpha_sum_until_points, float *v_means2d_abs,
+                                    float *v_means2d, float *v_conics, float *v_colors,
+                                    float *v_opacities, float *v_pix_vels,
+                                    float *v_depth_compensations, splatad_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPLATAD_HIP_H */

@@ -580,7 +580,10 @@ void oracle_isect_emit(int lidar, long total, long N, const int64_t *camera_ids,
                             tile_h, rect);
             for (int32_t i = rect[1]; i < rect[3]; ++i)
                 for (int32_t j = rect[0]; j < rect[2]; ++j) {
-                    int32_t wj = (j + (int32_t)tile_w) % (int32_t)tile_w;
+                    /* mathematical modulo: identical to (j + n) % n of the reference
+                     * (rasterization.cu:384) for j >= -n; azimuth extents below -360
+                     * degrees (j < -n) would make that expression negative */
+                    int32_t wj = ((j % (int32_t)tile_w) + (int32_t)tile_w) % (int32_t)tile_w;
                     int64_t tile_id = (int64_t)i * tile_w + wj;
                     isect_ids[cur] = cid_enc | (tile_id << 32) | depth_enc;
                     flatten_ids[cur] = (int32_t)idx;

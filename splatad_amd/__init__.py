@@ -1,1 +1,31 @@
-"""MI355X-native rendering hot path of SplatAD behind the gsplat operator API."""
+"""MI355X-native rendering hot path of SplatAD behind the gsplat operator API.
+
+Exports the operators and end-to-end functions of the reference's gsplat/__init__.py:3-24 that
+lie on the path projection -> tile intersection -> rasterization.
+"""
+from .hip._wrapper import (
+    fully_fused_lidar_projection,
+    fully_fused_projection,
+    isect_lidar_tiles,
+    isect_offset_encode,
+    isect_tiles,
+    rasterize_to_pixels,
+    rasterize_to_points,
+    spherical_harmonics,
+)
+from .rendering import lidar_rasterization, rasterization
+
+__version__ = "0.1.0"
+
+__all__ = [
+    "rasterization",
+    "lidar_rasterization",
+    "fully_fused_projection",
+    "fully_fused_lidar_projection",
+    "isect_tiles",
+    "isect_lidar_tiles",
+    "isect_offset_encode",
+    "rasterize_to_pixels",
+    "rasterize_to_points",
+    "spherical_harmonics",
+]

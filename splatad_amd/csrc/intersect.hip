@@ -1,0 +1,489 @@
+// Tile intersection, segmented sort and tile-offset encoding for gfx950.
+//
+// Results are bit-identical to gsplat/cuda/csrc/rasterization.cu:15-529 of the reference
+// (two-pass emit + cub::DeviceRadixSort on (camera | tile | depth) keys) but are produced
+// differently:
+//   1. a histogram pass counts intersections per (camera, tile);
+//   2. an exclusive scan of the histogram gives every tile's segment in the output;
+//   3. a scatter pass drops (depth bits, flatten id) pairs into their tile's segment;
+//   4. one workgroup per tile sorts its segment in LDS (bitonic network on the 64-bit
+//      composite depth<<32 | id) and writes the final 64-bit keys and the ids.
+// A stable sort by (camera, tile, depth) with ties kept in emission order equals a sort
+// by (camera, tile, depth, flatten id), because the emission loop visits flatten ids in
+// ascending order and emits each id at most once per tile; that is what makes the
+// unordered scatter of step 3 legal.  Depths must have a clear sign bit.
+//
+// Built with -ffp-contract=off: the tile bounds are float32 expressions whose rounding
+// decides which tiles a Gaussian touches.
+#include "common.h"
+#include "scan.h"
+
+namespace {
+
+struct TileGrid {
+    uint32_t tile_size;   // camera only
+    uint32_t tile_w, tile_h;
+    float azim_res, min_azim; // lidar only
+    const float *elev_boundaries;
+};
+
+__device__ __forceinline__ uint32_t f2u_sat(float v) {
+    if (!(v > 0.0f)) return 0u;
+    if (v >= 4294967296.0f) return 0xFFFFFFFFu;
+    return (uint32_t)v;
+}
+
+// Tile rectangle of one projected Gaussian: x in [x0, x1), y in [y0, y1).  For lidars x
+// may be negative or exceed tile_w (wrapped at emission).
+template <bool LIDAR>
+__device__ __forceinline__ bool tile_rect(const TileGrid &g, const float *__restrict__ means2d,
+                                          const void *__restrict__ radii_v, uint64_t idx,
+                                          int32_t &x0, int32_t &y0, int32_t &x1, int32_t &y1) {
+    const float2 mu = reinterpret_cast<const float2 *>(means2d)[idx];
+    if (!LIDAR) {
+        const int2 r = reinterpret_cast<const int2 *>(radii_v)[idx];
+        if (r.x <= 0) return false;
+        const float ts = (float)g.tile_size;
+        const float ex = (float)r.x / ts, ey = (float)r.y / ts;
+        const float tx = mu.x / ts, ty = mu.y / ts;
+        x0 = (int32_t)min(f2u_sat(floorf(tx - ex)), g.tile_w);
+        y0 = (int32_t)min(f2u_sat(floorf(ty - ey)), g.tile_h);
+        x1 = (int32_t)min(f2u_sat(ceilf(tx + ex)), g.tile_w);
+        y1 = (int32_t)min(f2u_sat(ceilf(ty + ey)), g.tile_h);
+    } else {
+        const float2 r = reinterpret_cast<const float2 *>(radii_v)[idx];
+        if (r.x <= 0.f) return false;
+        const float elev_low = mu.y - r.y, elev_high = mu.y + r.y;
+        const float azim = mu.x - g.min_azim;
+        const float azim_low = azim - r.x, azim_high = azim + r.x;
+        const float azim_max = (float)g.tile_w * g.azim_res;
+        float t_low, t_high;
+        if (azim_low >= 0.f)
+            t_low = azim_low / g.azim_res;
+        else
+            t_low = (fmodf(azim_low + 360.f, 360.f) - azim_max) / g.azim_res;
+        if (azim_high <= 360.f)
+            t_high = azim_high / g.azim_res;
+        else
+            t_high = (float)g.tile_w + fmodf(azim_high + 360.f, 360.f) / g.azim_res;
+        x0 = (int32_t)floorf(t_low);
+        x1 = (int32_t)ceilf(t_high);
+        const int32_t n = (int32_t)g.tile_h;
+        int32_t i = 0;
+        while (i <= n && g.elev_boundaries[i] < elev_low) ++i;
+        y0 = max(i - 1, 0);
+        while (i <= n && g.elev_boundaries[i] < elev_high) ++i;
+        y1 = min(i, n);
+    }
+    return true;
+}
+
+template <bool LIDAR>
+__device__ __forceinline__ uint32_t tile_index(const TileGrid &g, int32_t y, int32_t x) {
+    if (LIDAR) {
+        // Mathematical modulo.  For x >= -tile_w this equals (x + tile_w) % tile_w of the
+        // reference (rasterization.cu:384); an azimuth extent reaching below -360 degrees
+        // gives x < -tile_w, where that expression would go negative.
+        const int32_t n = (int32_t)g.tile_w;
+        x = ((x % n) + n) % n;
+    }
+    return (uint32_t)y * g.tile_w + (uint32_t)x;
+}
+
+template <bool LIDAR>
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d,
+                   const void *__restrict__ radii, int32_t *__restrict__ tiles_per_gauss,
+                   unsigned long long *__restrict__ n_isects) {
+    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int32_t cnt = 0;
+    if (idx < total) {
+        int32_t x0, y0, x1, y1;
+        if (tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) cnt = (y1 - y0) * (x1 - x0);
+        tiles_per_gauss[idx] = cnt;
+    }
+    // workgroup total -> one atomic per workgroup
+    long long s = cnt;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, SPLATAD_WAVE);
+    __shared__ long long wsum[SPLATAD_THREADS / SPLATAD_WAVE];
+    if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        long long t = 0;
+        for (int w = 0; w < SPLATAD_THREADS / SPLATAD_WAVE; ++w) t += wsum[w];
+        if (t != 0) atomicAdd(n_isects, (unsigned long long)t);
+    }
+}
+
+__device__ __forceinline__ uint32_t camera_of(uint64_t idx, uint32_t N,
+                                              const int64_t *__restrict__ camera_ids) {
+    return camera_ids ? (uint32_t)camera_ids[idx] : (uint32_t)(idx / N);
+}
+
+template <bool LIDAR>
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+isect_histogram_kernel(TileGrid g, uint64_t total, uint32_t N,
+                       const int64_t *__restrict__ camera_ids, const float *__restrict__ means2d,
+                       const void *__restrict__ radii, int32_t *__restrict__ tile_counts) {
+    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    int32_t x0, y0, x1, y1;
+    if (!tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) return;
+    const uint32_t base = camera_of(idx, N, camera_ids) * g.tile_w * g.tile_h;
+    for (int32_t y = y0; y < y1; ++y)
+        for (int32_t x = x0; x < x1; ++x) atomicAdd(&tile_counts[base + tile_index<LIDAR>(g, y, x)], 1);
+}
+
+template <bool LIDAR>
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+isect_scatter_kernel(TileGrid g, uint64_t total, uint32_t N,
+                     const int64_t *__restrict__ camera_ids, const float *__restrict__ means2d,
+                     const void *__restrict__ radii, const float *__restrict__ depths,
+                     const int32_t *__restrict__ tile_starts, int32_t *__restrict__ tile_fill,
+                     uint64_t *__restrict__ pairs) {
+    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    int32_t x0, y0, x1, y1;
+    if (!tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) return;
+    const uint32_t base = camera_of(idx, N, camera_ids) * g.tile_w * g.tile_h;
+    const uint64_t pair = ((uint64_t)__float_as_uint(depths[idx]) << 32) | (uint64_t)(uint32_t)idx;
+    for (int32_t y = y0; y < y1; ++y)
+        for (int32_t x = x0; x < x1; ++x) {
+            const uint32_t t = base + tile_index<LIDAR>(g, y, x);
+            const int32_t slot = atomicAdd(&tile_fill[t], 1);
+            pairs[(int64_t)tile_starts[t] + slot] = pair;
+        }
+}
+
+// Emission order without sorting (sort == false): rasterization.cu:65-89 / :366-394.
+template <bool LIDAR>
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+isect_emit_kernel(TileGrid g, uint64_t total, uint32_t N, const int64_t *__restrict__ camera_ids,
+                  const float *__restrict__ means2d, const void *__restrict__ radii,
+                  const float *__restrict__ depths, const int64_t *__restrict__ cum_before,
+                  uint32_t tile_n_bits, int64_t *__restrict__ isect_ids,
+                  int32_t *__restrict__ flatten_ids) {
+    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    int32_t x0, y0, x1, y1;
+    if (!tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) return;
+    const int64_t cid_enc = (int64_t)camera_of(idx, N, camera_ids) << (32 + tile_n_bits);
+    const int64_t depth_enc = (int64_t)(int32_t)__float_as_uint(depths[idx]);
+    int64_t cur = cum_before[idx];
+    for (int32_t y = y0; y < y1; ++y)
+        for (int32_t x = x0; x < x1; ++x) {
+            const int64_t tile_id = tile_index<LIDAR>(g, y, x);
+            isect_ids[cur] = cid_enc | (tile_id << 32) | depth_enc;
+            flatten_ids[cur] = (int32_t)idx;
+            ++cur;
+        }
+}
+
+// All comparators of this bitonic network point the same way (the first stage of every
+// merge is a "flip"), so a virtual +inf tail needs no storage: pairs whose upper index is
+// >= n are skipped.
+template <typename Ptr>
+__device__ __forceinline__ void bitonic_sort_ascending(Ptr a, uint32_t n, uint32_t tid,
+                                                       uint32_t nthreads) {
+    uint32_t m = 1;
+    while (m < n) m <<= 1;
+    for (uint32_t k = 2; k <= m; k <<= 1) {
+        for (uint32_t i = tid; i < m / 2; i += nthreads) {
+            const uint32_t lo = ((i / (k / 2)) * k) + (i % (k / 2));
+            const uint32_t hi = lo ^ (k - 1);
+            if (hi < n) {
+                const uint64_t x = a[lo], y = a[hi];
+                if (y < x) { a[lo] = y; a[hi] = x; }
+            }
+        }
+        __syncthreads();
+        for (uint32_t j = k / 4; j > 0; j >>= 1) {
+            for (uint32_t i = tid; i < m / 2; i += nthreads) {
+                const uint32_t lo = ((i / j) * (2 * j)) + (i % j);
+                const uint32_t hi = lo + j;
+                if (hi < n) {
+                    const uint64_t x = a[lo], y = a[hi];
+                    if (y < x) { a[lo] = y; a[hi] = x; }
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+// One workgroup per (camera, tile).  Segments with min_n < n <= max_n are handled here;
+// use_lds selects LDS staging (n <= lds capacity) or in-place sorting in global memory.
+__global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
+                                          uint32_t tile_n_bits, uint32_t min_n, uint32_t max_n,
+                                          int use_lds, const int32_t *__restrict__ tile_starts,
+                                          const int32_t *__restrict__ tile_counts,
+                                          uint64_t *__restrict__ pairs,
+                                          int64_t *__restrict__ isect_ids,
+                                          int32_t *__restrict__ flatten_ids) {
+    extern __shared__ uint64_t lds_pairs[];
+    const uint32_t seg = blockIdx.x;
+    if (seg >= n_segments) return;
+    const uint32_t n = (uint32_t)tile_counts[seg];
+    if (n <= min_n || n > max_n) return; // uniform across the workgroup
+    const int64_t start = tile_starts[seg];
+    uint64_t *g = pairs + start;
+    const uint32_t tid = threadIdx.x, nt = blockDim.x;
+    const uint64_t cam = seg / n_tiles, tile = seg % n_tiles;
+    const uint64_t hi = ((cam << tile_n_bits) | tile) << 32;
+    if (use_lds) {
+        for (uint32_t i = tid; i < n; i += nt) lds_pairs[i] = g[i];
+        __syncthreads();
+        bitonic_sort_ascending(lds_pairs, n, tid, nt);
+        for (uint32_t i = tid; i < n; i += nt) {
+            const uint64_t p = lds_pairs[i];
+            isect_ids[start + i] = (int64_t)(hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
+            flatten_ids[start + i] = (int32_t)(uint32_t)p;
+        }
+    } else {
+        __syncthreads();
+        bitonic_sort_ascending(g, n, tid, nt);
+        for (uint32_t i = tid; i < n; i += nt) {
+            const uint64_t p = g[i];
+            isect_ids[start + i] = (int64_t)(hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
+            flatten_ids[start + i] = (int32_t)(uint32_t)p;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+isect_offset_encode_kernel(int64_t n_isects, const int64_t *__restrict__ isect_ids,
+                           uint32_t n_tiles, uint32_t tile_n_bits, int64_t total_tiles,
+                           int32_t *__restrict__ offsets) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_isects) return;
+    const int64_t mask = ((int64_t)1 << tile_n_bits) - 1;
+    const int64_t hi = isect_ids[idx] >> 32;
+    const int64_t id_curr = (hi >> tile_n_bits) * n_tiles + (hi & mask);
+    int64_t first; // first table entry this intersection is responsible for
+    if (idx == 0) {
+        first = 0;
+    } else {
+        const int64_t hp = isect_ids[idx - 1] >> 32;
+        if (hp == hi) {
+            first = id_curr + 1; // nothing to write
+        } else {
+            first = (hp >> tile_n_bits) * n_tiles + (hp & mask) + 1;
+        }
+    }
+    for (int64_t i = first; i <= id_curr && i < total_tiles; ++i) offsets[i] = (int32_t)idx;
+    if (idx == n_isects - 1)
+        for (int64_t i = id_curr + 1; i < total_tiles; ++i) offsets[i] = (int32_t)n_isects;
+}
+
+__global__ void fill_zero_i32_kernel(int32_t *p, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+__global__ void fill_zero_u64_kernel(unsigned long long *p) { *p = 0ull; }
+
+struct IsectWorkspace {
+    unsigned long long *n_isects; // [1]
+    int64_t *scan_total;          // [1]
+    int32_t *tile_counts;         // [C * n_tiles]
+    int32_t *tile_starts;         // [C * n_tiles]
+    int32_t *tile_fill;           // [C * n_tiles]
+    int64_t *cum_before;          // [total] (sort == false only)
+    int64_t *block_sums;          // scan scratch
+    uint64_t *pairs;              // [n_isects]
+};
+
+static size_t isect_ws_bytes(uint64_t total, uint64_t segs, int64_t n_isects) {
+    uint64_t scan_n = total > segs ? total : segs;
+    return 512 + 3 * splatad_align256(segs * 4) + splatad_align256(total * 8) +
+           scan_workspace_bytes((int64_t)scan_n) + splatad_align256((uint64_t)n_isects * 8);
+}
+
+static IsectWorkspace carve_isect(void *ws, uint64_t total, uint64_t segs) {
+    char *p = (char *)ws;
+    IsectWorkspace w;
+    w.n_isects = (unsigned long long *)p;   p += 256;
+    w.scan_total = (int64_t *)p;            p += 256;
+    w.tile_counts = (int32_t *)p;           p += splatad_align256(segs * 4);
+    w.tile_starts = (int32_t *)p;           p += splatad_align256(segs * 4);
+    w.tile_fill = (int32_t *)p;             p += splatad_align256(segs * 4);
+    w.cum_before = (int64_t *)p;            p += splatad_align256(total * 8);
+    uint64_t scan_n = total > segs ? total : segs;
+    w.block_sums = (int64_t *)p;            p += scan_workspace_bytes((int64_t)scan_n);
+    w.pairs = (uint64_t *)p;
+    return w;
+}
+
+static inline dim3 grid_for(uint64_t n) {
+    return dim3((uint32_t)((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS));
+}
+
+template <bool LIDAR>
+static int isect_count(TileGrid g, uint64_t total, const float *means2d, const void *radii,
+                       uint32_t C, int32_t *tiles_per_gauss, void *workspace,
+                       int64_t *n_isects_host, hipStream_t stream) {
+    SPLATAD_REQUIRE(n_isects_host != nullptr, "isect: n_isects_host is null");
+    *n_isects_host = 0;
+    if (total == 0) return 0;
+    SPLATAD_REQUIRE(total < (1ull << 31), "isect: number of projected Gaussians must be below 2^31");
+    SPLATAD_REQUIRE(means2d && radii && tiles_per_gauss && workspace, "isect: null pointer argument");
+    const uint32_t n_tiles = g.tile_w * g.tile_h;
+    SPLATAD_REQUIRE(n_tiles > 0 && C > 0, "isect: empty tile grid");
+    SPLATAD_REQUIRE(splatad_bit_width(n_tiles) + splatad_bit_width(C) <= 32,
+                    "isect: camera and tile ids need more than 32 bits");
+    IsectWorkspace w = carve_isect(workspace, total, (uint64_t)C * n_tiles);
+    hipLaunchKernelGGL(fill_zero_u64_kernel, dim3(1), dim3(1), 0, stream, w.n_isects);
+    hipLaunchKernelGGL(isect_count_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
+                       stream, g, total, means2d, radii, tiles_per_gauss, w.n_isects);
+    SPLATAD_LAUNCH_CHECK();
+    unsigned long long n = 0;
+    SPLATAD_CHECK_HIP(hipMemcpyAsync(&n, w.n_isects, sizeof(n), hipMemcpyDeviceToHost, stream));
+    SPLATAD_CHECK_HIP(hipStreamSynchronize(stream));
+    SPLATAD_REQUIRE(n < (1ull << 31), "isect: %llu intersections exceed the int32 offset range", n);
+    *n_isects_host = (int64_t)n;
+    return 0;
+}
+
+template <bool LIDAR>
+static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *camera_ids,
+                      const float *means2d, const void *radii, const float *depths, uint32_t C,
+                      int sort, int64_t n_isects, const int32_t *tiles_per_gauss,
+                      void *workspace, int64_t *isect_ids, int32_t *flatten_ids,
+                      hipStream_t stream) {
+    if (total == 0 || n_isects == 0) return 0;
+    SPLATAD_REQUIRE(means2d && radii && depths && workspace && isect_ids && flatten_ids,
+                    "isect: null pointer argument");
+    SPLATAD_REQUIRE(camera_ids != nullptr || N > 0, "isect: N is zero for unpacked input");
+    const uint32_t n_tiles = g.tile_w * g.tile_h;
+    const uint32_t tile_n_bits = splatad_bit_width(n_tiles);
+    const uint64_t segs = (uint64_t)C * n_tiles;
+    IsectWorkspace w = carve_isect(workspace, total, segs);
+    if (!sort) {
+        SPLATAD_REQUIRE(tiles_per_gauss != nullptr, "isect: tiles_per_gauss is null");
+        int rc = launch_exclusive_scan<int64_t>(tiles_per_gauss, (int64_t)total, 1, 0,
+                                                w.cum_before, w.scan_total, w.block_sums, stream);
+        if (rc) return rc;
+        hipLaunchKernelGGL(isect_emit_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
+                           stream, g, total, N, camera_ids, means2d, radii, depths,
+                           (const int64_t *)w.cum_before, tile_n_bits, isect_ids, flatten_ids);
+        SPLATAD_LAUNCH_CHECK();
+        return 0;
+    }
+    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream,
+                       w.tile_counts, (int64_t)segs);
+    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream,
+                       w.tile_fill, (int64_t)segs);
+    hipLaunchKernelGGL(isect_histogram_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
+                       stream, g, total, N, camera_ids, means2d, radii, w.tile_counts);
+    SPLATAD_LAUNCH_CHECK();
+    int rc = launch_exclusive_scan<int32_t>(w.tile_counts, (int64_t)segs, 1, 0, w.tile_starts,
+                                            w.scan_total, w.block_sums, stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL(isect_scatter_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
+                       stream, g, total, N, camera_ids, means2d, radii, depths, w.tile_starts,
+                       w.tile_fill, w.pairs);
+    SPLATAD_LAUNCH_CHECK();
+    // three size classes: small and medium in LDS, the rest in place in global memory
+    const uint32_t small_cap = 2048, medium_cap = 16384;
+    static bool attr_set = false;
+    if (!attr_set) {
+        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)isect_segment_sort_kernel,
+                                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              medium_cap * 8));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(isect_segment_sort_kernel, dim3((uint32_t)segs), dim3(256), small_cap * 8,
+                       stream, (uint32_t)segs, n_tiles, tile_n_bits, 0u, small_cap, 1,
+                       w.tile_starts, w.tile_counts, w.pairs, isect_ids, flatten_ids);
+    hipLaunchKernelGGL(isect_segment_sort_kernel, dim3((uint32_t)segs), dim3(1024),
+                       medium_cap * 8, stream, (uint32_t)segs, n_tiles, tile_n_bits, small_cap,
+                       medium_cap, 1, w.tile_starts, w.tile_counts, w.pairs, isect_ids,
+                       flatten_ids);
+    hipLaunchKernelGGL(isect_segment_sort_kernel, dim3((uint32_t)segs), dim3(1024), 0, stream,
+                       (uint32_t)segs, n_tiles, tile_n_bits, medium_cap, 0x7FFFFFFFu, 0,
+                       w.tile_starts, w.tile_counts, w.pairs, isect_ids, flatten_ids);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
+}
+
+} // namespace
+
+extern "C" size_t splatad_isect_workspace_bytes(uint64_t total, uint32_t C, uint32_t n_tiles,
+                                                int64_t n_isects) {
+    return isect_ws_bytes(total, (uint64_t)C * n_tiles, n_isects < 0 ? 0 : n_isects);
+}
+
+extern "C" int splatad_isect_tiles_count(uint64_t total, const float *means2d,
+                                         const int32_t *radii, uint32_t C, uint32_t tile_size,
+                                         uint32_t tile_width, uint32_t tile_height,
+                                         int32_t *tiles_per_gauss, void *workspace,
+                                         int64_t *n_isects_host, splatad_stream_t stream) {
+    SPLATAD_REQUIRE(tile_size > 0, "isect_tiles: tile_size is zero");
+    TileGrid g{tile_size, tile_width, tile_height, 0.f, 0.f, nullptr};
+    return isect_count<false>(g, total, means2d, radii, C, tiles_per_gauss, workspace,
+                              n_isects_host, (hipStream_t)stream);
+}
+
+extern "C" int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_ids,
+                                        const float *means2d, const int32_t *radii,
+                                        const float *depths, uint32_t C, uint32_t tile_size,
+                                        uint32_t tile_width, uint32_t tile_height, int sort,
+                                        int64_t n_isects, const int32_t *tiles_per_gauss,
+                                        void *workspace, int64_t *isect_ids, int32_t *flatten_ids,
+                                        splatad_stream_t stream) {
+    SPLATAD_REQUIRE(tile_size > 0, "isect_tiles: tile_size is zero");
+    TileGrid g{tile_size, tile_width, tile_height, 0.f, 0.f, nullptr};
+    return isect_fill<false>(g, total, N, camera_ids, means2d, radii, depths, C, sort, n_isects,
+                             tiles_per_gauss, workspace, isect_ids, flatten_ids,
+                             (hipStream_t)stream);
+}
+
+extern "C" int splatad_isect_lidar_tiles_count(uint64_t total, const float *means2d,
+                                               const float *radii, uint32_t C,
+                                               const float *elev_boundaries,
+                                               float tile_azim_resolution, float min_azim,
+                                               uint32_t tile_width, uint32_t tile_height,
+                                               int32_t *tiles_per_gauss, void *workspace,
+                                               int64_t *n_isects_host, splatad_stream_t stream) {
+    SPLATAD_REQUIRE(elev_boundaries != nullptr, "isect_lidar_tiles: elev_boundaries is null");
+    TileGrid g{0u, tile_width, tile_height, tile_azim_resolution, min_azim, elev_boundaries};
+    return isect_count<true>(g, total, means2d, radii, C, tiles_per_gauss, workspace,
+                             n_isects_host, (hipStream_t)stream);
+}
+
+extern "C" int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N,
+                                              const int64_t *camera_ids, const float *means2d,
+                                              const float *radii, const float *depths, uint32_t C,
+                                              const float *elev_boundaries,
+                                              float tile_azim_resolution, float min_azim,
+                                              uint32_t tile_width, uint32_t tile_height, int sort,
+                                              int64_t n_isects, const int32_t *tiles_per_gauss,
+                                              void *workspace, int64_t *isect_ids,
+                                              int32_t *flatten_ids, splatad_stream_t stream) {
+    SPLATAD_REQUIRE(elev_boundaries != nullptr, "isect_lidar_tiles: elev_boundaries is null");
+    TileGrid g{0u, tile_width, tile_height, tile_azim_resolution, min_azim, elev_boundaries};
+    return isect_fill<true>(g, total, N, camera_ids, means2d, radii, depths, C, sort, n_isects,
+                            tiles_per_gauss, workspace, isect_ids, flatten_ids,
+                            (hipStream_t)stream);
+}
+
+extern "C" int splatad_isect_offset_encode(int64_t n_isects, const int64_t *isect_ids, uint32_t C,
+                                           uint32_t n_tiles, int32_t *offsets,
+                                           splatad_stream_t stream) {
+    const int64_t total_tiles = (int64_t)C * n_tiles;
+    if (total_tiles == 0) return 0;
+    SPLATAD_REQUIRE(offsets != nullptr, "isect_offset_encode: offsets is null");
+    if (n_isects == 0) {
+        hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for((uint64_t)total_tiles),
+                           dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, offsets, total_tiles);
+        SPLATAD_LAUNCH_CHECK();
+        return 0;
+    }
+    SPLATAD_REQUIRE(isect_ids != nullptr, "isect_offset_encode: isect_ids is null");
+    hipLaunchKernelGGL(isect_offset_encode_kernel, grid_for((uint64_t)n_isects),
+                       dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, n_isects, isect_ids, n_tiles,
+                       splatad_bit_width(n_tiles), total_tiles, offsets);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
+}

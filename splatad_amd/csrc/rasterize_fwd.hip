@@ -1,0 +1,404 @@
+// Front-to-back alpha compositing for camera pixels and lidar points on gfx950.
+//
+// One workgroup per (sensor, tile); one lane per pixel / point.  A tile's depth-sorted
+// Gaussian list is streamed through LDS in batches of one Gaussian per lane: the batch is
+// gathered once (coalesced over the id list, 16-byte records in LDS, colours included) and
+// then every lane walks the batch reading LDS at a wave-uniform address, which the LDS
+// serves as a broadcast without bank conflicts.  A 16x16 tile is four wavefronts of 16x4
+// pixels; a wavefront leaves the batch loop as soon as its 64 pixels are saturated and the
+// workgroup stops fetching batches once all of its pixels are.
+//
+// Compositing rules follow gsplat/cuda/csrc/rasterization.cu:1360-1518 (pixels) and
+// :2021-2219 (points) of the reference: alpha = min(0.999, o * exp(-sigma)); a Gaussian is
+// skipped when sigma < 0 or alpha < 1/255; a pixel stops, without taking the Gaussian,
+// when its transmittance would fall to 1e-4 or below.
+//
+// Channels: the kernels are compiled for CH accumulators per lane and take the real
+// channel count, stride and offset at run time, so any channel count is rendered without
+// host-side padding (wide inputs in passes of up to 32 channels).
+#include "common.h"
+
+namespace {
+
+struct PixelArgs {
+    uint32_t C;
+    int64_t n_isects;
+    uint32_t color_stride; // channels of the colour tensor
+    uint32_t ch_offset;    // first channel of this pass
+    uint32_t n_ch;         // channels of this pass (<= CH)
+    const float *means2d, *conics, *colors, *opacities, *pix_vels, *rs_time, *backgrounds;
+    uint32_t W, H, tile_size, tile_w, tile_h;
+    const int32_t *tile_offsets, *flatten_ids;
+    float *render_colors, *render_alphas;
+    int32_t *last_ids;
+    int write_aux; // first pass also writes alphas and last ids
+};
+
+template <int CH>
+__global__ void __launch_bounds__(1024)
+rasterize_to_pixels_fwd_kernel(PixelArgs a) {
+    extern __shared__ float4 lds4[];
+    const uint32_t block_size = blockDim.x * blockDim.y;
+    float4 *s_xyv = lds4;                           // {x, y, vx, vy}
+    float4 *s_con = lds4 + block_size;              // {conic a, b, c, opacity}
+    float *s_col = reinterpret_cast<float *>(lds4 + 2 * block_size); // [block_size][CH]
+
+    const uint32_t tiles_per_cam = a.tile_w * a.tile_h;
+    const uint32_t cam = blockIdx.x / tiles_per_cam;
+    const uint32_t tile_id = blockIdx.x % tiles_per_cam;
+    const uint32_t tile_y = tile_id / a.tile_w, tile_x = tile_id % a.tile_w;
+    const uint32_t i = tile_y * a.tile_size + threadIdx.y;
+    const uint32_t j = tile_x * a.tile_size + threadIdx.x;
+    const uint32_t tr = threadIdx.y * blockDim.x + threadIdx.x;
+
+    const float px = (float)j + 0.5f, py = (float)i + 0.5f;
+    const float roll = a.rs_time[cam] * ((py - 0.5f) / (float)(a.H - 1) - 0.5f);
+    const bool inside = (i < a.H && j < a.W);
+    bool done = !inside;
+
+    const int32_t *offs = a.tile_offsets + (size_t)cam * tiles_per_cam;
+    const int32_t range_start = offs[tile_id];
+    const int32_t range_end = (cam == a.C - 1 && tile_id == tiles_per_cam - 1)
+                                  ? (int32_t)a.n_isects
+                                  : offs[tile_id + 1];
+    const uint32_t num_batches = (uint32_t)(range_end - range_start + block_size - 1) / block_size;
+
+    float T = 1.0f;
+    uint32_t cur_idx = 0;
+    float out[CH];
+#pragma unroll
+    for (int k = 0; k < CH; ++k) out[k] = 0.f;
+
+    for (uint32_t b = 0; b < num_batches; ++b) {
+        // also orders the previous batch's LDS reads before this batch's writes
+        if (__syncthreads_count(done) >= (int)block_size) break;
+
+        const uint32_t batch_start = (uint32_t)range_start + block_size * b;
+        const uint32_t idx = batch_start + tr;
+        if (idx < (uint32_t)range_end) {
+            const int32_t g = a.flatten_ids[idx];
+            const float2 xy = reinterpret_cast<const float2 *>(a.means2d)[g];
+            const float2 v = reinterpret_cast<const float2 *>(a.pix_vels)[g];
+            const float *cn = a.conics + (size_t)g * 3;
+            s_xyv[tr] = make_float4(xy.x, xy.y, v.x, v.y);
+            s_con[tr] = make_float4(cn[0], cn[1], cn[2], a.opacities[g]);
+            const float *c = a.colors + (size_t)g * a.color_stride + a.ch_offset;
+#pragma unroll
+            for (int k = 0; k < CH; ++k) s_col[tr * CH + k] = (uint32_t)k < a.n_ch ? c[k] : 0.f;
+        }
+        __syncthreads();
+
+        const uint32_t batch_size = min(block_size, (uint32_t)range_end - batch_start);
+        for (uint32_t t = 0; t < batch_size && !done; ++t) {
+            const float4 xyv = s_xyv[t];
+            const float4 con = s_con[t];
+            const float dx = xyv.x + roll * xyv.z - px;
+            const float dy = xyv.y + roll * xyv.w - py;
+            const float sigma = 0.5f * (con.x * dx * dx + con.z * dy * dy) + con.y * dx * dy;
+            const float alpha = fminf(0.999f, con.w * __expf(-sigma));
+            if (sigma < 0.f || alpha < 1.f / 255.f) continue;
+            const float next_T = T * (1.0f - alpha);
+            if (next_T <= 1e-4f) {
+                done = true;
+                break;
+            }
+            const float vis = alpha * T;
+#pragma unroll
+            for (int k = 0; k < CH; ++k) out[k] += s_col[t * CH + k] * vis;
+            cur_idx = batch_start + t;
+            T = next_T;
+        }
+    }
+
+    if (inside) {
+        const size_t pix = ((size_t)cam * a.H + i) * a.W + j;
+        float *dst = a.render_colors + pix * a.color_stride + a.ch_offset;
+        const float *bg = a.backgrounds ? a.backgrounds + (size_t)cam * a.color_stride + a.ch_offset : nullptr;
+#pragma unroll
+        for (int k = 0; k < CH; ++k)
+            if ((uint32_t)k < a.n_ch) dst[k] = bg ? out[k] + T * bg[k] : out[k];
+        if (a.write_aux) {
+            a.render_alphas[pix] = 1.0f - T;
+            a.last_ids[pix] = (int32_t)cur_idx;
+        }
+    }
+}
+
+struct PointArgs {
+    uint32_t C;
+    int64_t n_isects;
+    uint32_t color_stride, ch_offset, n_ch;
+    const float *means2d, *conics, *colors, *opacities, *pix_vels, *depth_comps, *backgrounds,
+        *raster_pts;
+    uint32_t W, H, tile_width, tile_height, grid_w, grid_h;
+    int compute_alpha_sum;
+    float threshold;
+    const int32_t *tile_offsets, *flatten_ids;
+    uint32_t depth_idx;
+    float *render_colors, *render_alphas, *alpha_sum;
+    int32_t *last_ids;
+    float *median_depths;
+    int write_aux;
+};
+
+// fmodf(a - b + 180, 360) - 180, folded into (-180, 180]; the common case (argument of
+// fmodf already in [0, 360)) skips the library call, with the same result.
+__device__ __forceinline__ float angle_difference(float a, float b) {
+    const float d = a - b + 180.f;
+    const float m = (d >= 0.f && d < 360.f) ? d : fmodf(d, 360.f);
+    const float r = m - 180.f;
+    return r < -180.f ? r + 360.f : r;
+}
+
+template <int CH>
+__global__ void __launch_bounds__(256)
+rasterize_to_points_fwd_kernel(PointArgs a) {
+    extern __shared__ float4 lds4[];
+    const uint32_t block_size = blockDim.x * blockDim.y;
+    float4 *s_xyv = lds4;                  // {az, el, v_az, v_el}
+    float4 *s_con = lds4 + block_size;     // {conic a, b, c, opacity}
+    float4 *s_ext = lds4 + 2 * block_size; // {v_range, depth comp 0, depth comp 1, depth}
+    float *s_col = reinterpret_cast<float *>(lds4 + 3 * block_size);
+
+    const uint32_t tiles_per_cam = a.grid_w * a.grid_h;
+    const uint32_t cam = blockIdx.x / tiles_per_cam;
+    const uint32_t tile_id = blockIdx.x % tiles_per_cam;
+    const uint32_t i = (tile_id / a.grid_w) * a.tile_height + threadIdx.y;
+    const uint32_t j = (tile_id % a.grid_w) * a.tile_width + threadIdx.x;
+    const uint32_t tr = threadIdx.y * blockDim.x + threadIdx.x;
+
+    const bool in_image = (i < a.H && j < a.W);
+    const size_t pix = ((size_t)cam * a.H + i) * a.W + j;
+    float px = 0.f, py = 0.f, pz = 0.f, roll = 0.f;
+    if (in_image) {
+        const float4 p = reinterpret_cast<const float4 *>(a.raster_pts)[pix];
+        px = p.x; py = p.y; pz = p.z; roll = p.w;
+    }
+    const bool inside = in_image && pz > 0.f;
+    bool done = !inside;
+
+    const int32_t *offs = a.tile_offsets + (size_t)cam * tiles_per_cam;
+    const int32_t range_start = offs[tile_id];
+    const int32_t range_end = (cam == a.C - 1 && tile_id == tiles_per_cam - 1)
+                                  ? (int32_t)a.n_isects
+                                  : offs[tile_id + 1];
+    const uint32_t num_batches = (uint32_t)(range_end - range_start + block_size - 1) / block_size;
+    const bool has_depth = a.depth_idx >= a.ch_offset && a.depth_idx < a.ch_offset + a.n_ch;
+
+    float T = 1.0f, asum = 0.f, median = 0.f, depth_extra = 0.f;
+    uint32_t cur_idx = 0;
+    float out[CH];
+#pragma unroll
+    for (int k = 0; k < CH; ++k) out[k] = 0.f;
+
+    for (uint32_t b = 0; b < num_batches; ++b) {
+        if (__syncthreads_count(done) >= (int)block_size) break;
+        const uint32_t batch_start = (uint32_t)range_start + block_size * b;
+        const uint32_t idx = batch_start + tr;
+        if (idx < (uint32_t)range_end) {
+            const int32_t g = a.flatten_ids[idx];
+            const float2 xy = reinterpret_cast<const float2 *>(a.means2d)[g];
+            const float *v = a.pix_vels + (size_t)g * 3;
+            const float2 dc = reinterpret_cast<const float2 *>(a.depth_comps)[g];
+            const float *cn = a.conics + (size_t)g * 3;
+            const float *crow = a.colors + (size_t)g * a.color_stride;
+            s_xyv[tr] = make_float4(xy.x, xy.y, v[0], v[1]);
+            s_con[tr] = make_float4(cn[0], cn[1], cn[2], a.opacities[g]);
+            s_ext[tr] = make_float4(v[2], dc.x, dc.y, crow[a.depth_idx]);
+            const float *c = crow + a.ch_offset;
+#pragma unroll
+            for (int k = 0; k < CH; ++k) s_col[tr * CH + k] = (uint32_t)k < a.n_ch ? c[k] : 0.f;
+        }
+        __syncthreads();
+
+        const uint32_t batch_size = min(block_size, (uint32_t)range_end - batch_start);
+        for (uint32_t t = 0; t < batch_size && !done; ++t) {
+            const float4 xyv = s_xyv[t];
+            const float4 con = s_con[t];
+            const float dx = angle_difference(xyv.x + roll * xyv.z, px);
+            const float dy = angle_difference(xyv.y + roll * xyv.w, py);
+            const float sigma = 0.5f * (con.x * dx * dx + con.z * dy * dy) + con.y * dx * dy;
+            const float alpha = fminf(0.999f, con.w * __expf(-sigma));
+            if (sigma < 0.f || alpha < 1.f / 255.f) continue;
+            const float next_T = T * (1.0f - alpha);
+            if (next_T <= 1e-4f) {
+                done = true;
+                break;
+            }
+            const float vis = alpha * T;
+#pragma unroll
+            for (int k = 0; k < CH; ++k) out[k] += s_col[t * CH + k] * vis;
+            const float4 ext = s_ext[t];
+            const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
+            depth_extra += extra * vis;
+            if (T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
+            if (a.compute_alpha_sum && ext.w < pz - a.threshold) asum += alpha;
+            cur_idx = batch_start + t;
+            T = next_T;
+        }
+    }
+
+    if (in_image) {
+        float *dst = a.render_colors + pix * a.color_stride + a.ch_offset;
+        const float *bg = a.backgrounds ? a.backgrounds + (size_t)cam * a.color_stride + a.ch_offset : nullptr;
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+            if ((uint32_t)k < a.n_ch) {
+                float v = out[k];
+                if (has_depth && (uint32_t)k == a.depth_idx - a.ch_offset) v += depth_extra;
+                if (bg && inside) v += T * bg[k];
+                dst[k] = inside ? v : 0.f;
+            }
+        }
+        if (a.write_aux) {
+            a.render_alphas[pix] = inside ? 1.0f - T : 0.f;
+            a.last_ids[pix] = inside ? (int32_t)cur_idx : 0;
+            a.median_depths[pix] = median;
+            if (a.alpha_sum) a.alpha_sum[pix] = asum;
+        }
+    }
+}
+
+// Compiled accumulator widths; a pass of n channels uses the smallest width >= n.
+constexpr int kWidths[] = {1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33};
+constexpr int kMaxPass = 33;
+
+static inline int pick_width(uint32_t n) {
+    for (int w : kWidths)
+        if ((uint32_t)w >= n) return w;
+    return -1;
+}
+
+template <int CH>
+static int launch_pixels(const PixelArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
+    const size_t lds = (size_t)block.x * block.y * (32 + 4 * CH);
+    if (lds > 64 * 1024)
+        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_to_pixels_fwd_kernel<CH>,
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(rasterize_to_pixels_fwd_kernel<CH>, grid, block, lds, stream, a);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
+}
+
+template <int CH>
+static int launch_points(const PointArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
+    const size_t lds = (size_t)block.x * block.y * (48 + 4 * CH);
+    hipLaunchKernelGGL(rasterize_to_points_fwd_kernel<CH>, grid, block, lds, stream, a);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
+}
+
+#define DISPATCH_WIDTH(w, CALL)                                                              \
+    switch (w) {                                                                             \
+    case 1: return CALL(1);                                                                  \
+    case 2: return CALL(2);                                                                  \
+    case 3: return CALL(3);                                                                  \
+    case 4: return CALL(4);                                                                  \
+    case 5: return CALL(5);                                                                  \
+    case 8: return CALL(8);                                                                  \
+    case 9: return CALL(9);                                                                  \
+    case 16: return CALL(16);                                                                \
+    case 17: return CALL(17);                                                                \
+    case 32: return CALL(32);                                                                \
+    case 33: return CALL(33);                                                                \
+    default: break;                                                                          \
+    }
+
+static int dispatch_pixels(int w, const PixelArgs &a, dim3 grid, dim3 block, hipStream_t s) {
+#define CALL_PIX(W) launch_pixels<W>(a, grid, block, s)
+    DISPATCH_WIDTH(w, CALL_PIX)
+#undef CALL_PIX
+    splatad_set_error("rasterize_to_pixels: no kernel for %d channels per pass", w);
+    return -1;
+}
+
+static int dispatch_points(int w, const PointArgs &a, dim3 grid, dim3 block, hipStream_t s) {
+#define CALL_PTS(W) launch_points<W>(a, grid, block, s)
+    DISPATCH_WIDTH(w, CALL_PTS)
+#undef CALL_PTS
+    splatad_set_error("rasterize_to_points: no kernel for %d channels per pass", w);
+    return -1;
+}
+
+} // namespace
+
+extern "C" int splatad_rasterize_to_pixels_fwd(
+    uint32_t C, int64_t n_isects, uint32_t channels, const float *means2d, const float *conics,
+    const float *colors, const float *opacities, const float *pix_vels, const float *rs_time,
+    const float *backgrounds, uint32_t W, uint32_t H, uint32_t tile_size, uint32_t tile_w,
+    uint32_t tile_h, const int32_t *tile_offsets, const int32_t *flatten_ids,
+    float *render_colors, float *render_alphas, int32_t *last_ids, splatad_stream_t stream) {
+    SPLATAD_REQUIRE(channels >= 1, "rasterize_to_pixels: zero channels");
+    SPLATAD_REQUIRE(tile_size >= 1 && tile_size * tile_size <= 1024,
+                    "rasterize_to_pixels: tile_size %u is outside 1..32", tile_size);
+    if (C == 0 || W == 0 || H == 0) return 0;
+    SPLATAD_REQUIRE((uint64_t)tile_w * tile_size >= W && (uint64_t)tile_h * tile_size >= H,
+                    "rasterize_to_pixels: tile grid %ux%u of size %u does not cover %ux%u", tile_w,
+                    tile_h, tile_size, W, H);
+    SPLATAD_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31), "rasterize_to_pixels: bad n_isects");
+    SPLATAD_REQUIRE(rs_time && tile_offsets && render_colors && render_alphas && last_ids,
+                    "rasterize_to_pixels: null pointer argument");
+    SPLATAD_REQUIRE(n_isects == 0 || (means2d && conics && colors && opacities && pix_vels && flatten_ids),
+                    "rasterize_to_pixels: null pointer argument");
+    PixelArgs a;
+    a.C = C; a.n_isects = n_isects; a.color_stride = channels;
+    a.means2d = means2d; a.conics = conics; a.colors = colors; a.opacities = opacities;
+    a.pix_vels = pix_vels; a.rs_time = rs_time; a.backgrounds = backgrounds;
+    a.W = W; a.H = H; a.tile_size = tile_size; a.tile_w = tile_w; a.tile_h = tile_h;
+    a.tile_offsets = tile_offsets; a.flatten_ids = flatten_ids;
+    a.render_colors = render_colors; a.render_alphas = render_alphas; a.last_ids = last_ids;
+    const dim3 grid(C * tile_w * tile_h), block(tile_size, tile_size);
+    const uint32_t pass = channels <= (uint32_t)kMaxPass ? channels : 32u;
+    for (uint32_t off = 0; off < channels; off += pass) {
+        a.ch_offset = off;
+        a.n_ch = min(pass, channels - off);
+        a.write_aux = off == 0;
+        int rc = dispatch_pixels(pick_width(a.n_ch), a, grid, block, (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+extern "C" int splatad_rasterize_to_points_fwd(
+    uint32_t C, int64_t n_isects, uint32_t channels, const float *means2d, const float *conics,
+    const float *colors, const float *opacities, const float *pix_vels, const float *depth_comps,
+    const float *backgrounds, const float *raster_pts, uint32_t W, uint32_t H,
+    uint32_t tile_width, uint32_t tile_height, uint32_t grid_w, uint32_t grid_h,
+    int compute_alpha_sum, float threshold, const int32_t *tile_offsets,
+    const int32_t *flatten_ids, uint32_t depth_idx, float *render_colors, float *render_alphas,
+    float *alpha_sum, int32_t *last_ids, float *median_depths, splatad_stream_t stream) {
+    SPLATAD_REQUIRE(channels >= 1, "rasterize_to_points: zero channels");
+    SPLATAD_REQUIRE(depth_idx < channels, "rasterize_to_points: depth channel %u of %u", depth_idx, channels);
+    SPLATAD_REQUIRE(tile_width >= 1 && tile_height >= 1 && tile_width * tile_height <= 256,
+                    "rasterize_to_points: tile %ux%u exceeds 256 points", tile_width, tile_height);
+    if (C == 0 || W == 0 || H == 0) return 0;
+    SPLATAD_REQUIRE((uint64_t)grid_w * tile_width >= W && (uint64_t)grid_h * tile_height >= H,
+                    "rasterize_to_points: tile grid does not cover the point image");
+    SPLATAD_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31), "rasterize_to_points: bad n_isects");
+    SPLATAD_REQUIRE(raster_pts && tile_offsets && render_colors && render_alphas && last_ids && median_depths,
+                    "rasterize_to_points: null pointer argument");
+    SPLATAD_REQUIRE(!compute_alpha_sum || alpha_sum, "rasterize_to_points: alpha_sum output is null");
+    SPLATAD_REQUIRE(n_isects == 0 || (means2d && conics && colors && opacities && pix_vels && depth_comps && flatten_ids),
+                    "rasterize_to_points: null pointer argument");
+    PointArgs a;
+    a.C = C; a.n_isects = n_isects; a.color_stride = channels;
+    a.means2d = means2d; a.conics = conics; a.colors = colors; a.opacities = opacities;
+    a.pix_vels = pix_vels; a.depth_comps = depth_comps; a.backgrounds = backgrounds;
+    a.raster_pts = raster_pts; a.W = W; a.H = H; a.tile_width = tile_width;
+    a.tile_height = tile_height; a.grid_w = grid_w; a.grid_h = grid_h;
+    a.compute_alpha_sum = compute_alpha_sum; a.threshold = threshold;
+    a.tile_offsets = tile_offsets; a.flatten_ids = flatten_ids; a.depth_idx = depth_idx;
+    a.render_colors = render_colors; a.render_alphas = render_alphas;
+    a.alpha_sum = compute_alpha_sum ? alpha_sum : nullptr;
+    a.last_ids = last_ids; a.median_depths = median_depths;
+    const dim3 grid(C * grid_w * grid_h), block(tile_width, tile_height);
+    const uint32_t pass = channels <= (uint32_t)kMaxPass ? channels : 32u;
+    for (uint32_t off = 0; off < channels; off += pass) {
+        a.ch_offset = off;
+        a.n_ch = min(pass, channels - off);
+        a.write_aux = off == 0;
+        int rc = dispatch_points(pick_width(a.n_ch), a, grid, block, (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    return 0;
+}

@@ -1,0 +1,131 @@
+// Device-wide exclusive prefix sum used by the compaction and intersection code.
+//
+// Three launches: per-block totals, a single-workgroup scan of those totals, and a
+// per-block scan that adds the block's base.  2048 items per workgroup of 256 lanes;
+// wave64 shuffles inside a wavefront, LDS across the four wavefronts.
+#pragma once
+
+#include "common.h"
+
+#ifdef __HIPCC__
+
+#define SCAN_ITEMS 8
+#define SCAN_TILE (SPLATAD_THREADS * SCAN_ITEMS)
+
+namespace { // one private copy of the kernels per translation unit
+
+// Value of element i of a strided int32 input, optionally reduced to a 0/1 flag (v > 0).
+__device__ __forceinline__ int32_t scan_load(const int32_t *in, int64_t i, int64_t n, int stride,
+                                             int as_flag) {
+    if (i >= n) return 0;
+    int32_t v = in[i * stride];
+    return as_flag ? (v > 0 ? 1 : 0) : v;
+}
+
+// Exclusive scan of one int64 per lane across the workgroup; returns the lane's
+// exclusive prefix and the workgroup total.
+__device__ __forceinline__ int64_t block_exclusive_scan(int64_t v, int64_t *total) {
+    __shared__ int64_t wave_tot[SPLATAD_THREADS / SPLATAD_WAVE];
+    const int lane = threadIdx.x & (SPLATAD_WAVE - 1);
+    const int wave = threadIdx.x / SPLATAD_WAVE;
+    int64_t incl = v;
+#pragma unroll
+    for (int off = 1; off < SPLATAD_WAVE; off <<= 1) {
+        int64_t o = __shfl_up(incl, off, SPLATAD_WAVE);
+        if (lane >= off) incl += o;
+    }
+    if (lane == SPLATAD_WAVE - 1) wave_tot[wave] = incl;
+    __syncthreads();
+    int64_t base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < SPLATAD_THREADS / SPLATAD_WAVE; ++w) {
+        int64_t t = wave_tot[w];
+        if (w < wave) base += t;
+        tot += t;
+    }
+    __syncthreads();
+    *total = tot;
+    return base + incl - v;
+}
+
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+scan_block_totals_kernel(const int32_t *__restrict__ in, int64_t n, int stride, int as_flag,
+                         int64_t *__restrict__ block_sums) {
+    const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+    int64_t s = 0;
+#pragma unroll
+    for (int k = 0; k < SCAN_ITEMS; ++k) s += scan_load(in, base + k, n, stride, as_flag);
+    int64_t tot;
+    block_exclusive_scan(s, &tot);
+    if (threadIdx.x == 0) block_sums[blockIdx.x] = tot;
+}
+
+// One workgroup: in-place exclusive scan of block_sums, grand total to *total.
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+scan_block_sums_kernel(int64_t *__restrict__ block_sums, int64_t n_blocks,
+                       int64_t *__restrict__ total) {
+    int64_t carry = 0;
+    for (int64_t start = 0; start < n_blocks; start += SPLATAD_THREADS) {
+        int64_t i = start + threadIdx.x;
+        int64_t v = i < n_blocks ? block_sums[i] : 0;
+        int64_t tot;
+        int64_t ex = block_exclusive_scan(v, &tot);
+        if (i < n_blocks) block_sums[i] = carry + ex;
+        carry += tot;
+    }
+    if (threadIdx.x == 0) *total = carry;
+}
+
+template <typename OutT>
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+scan_apply_kernel(const int32_t *__restrict__ in, int64_t n, int stride, int as_flag,
+                  const int64_t *__restrict__ block_sums, OutT *__restrict__ out) {
+    const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+    int32_t v[SCAN_ITEMS];
+    int64_t s = 0;
+#pragma unroll
+    for (int k = 0; k < SCAN_ITEMS; ++k) {
+        v[k] = scan_load(in, base + k, n, stride, as_flag);
+        s += v[k];
+    }
+    int64_t tot;
+    int64_t run = block_exclusive_scan(s, &tot) + block_sums[blockIdx.x];
+#pragma unroll
+    for (int k = 0; k < SCAN_ITEMS; ++k) {
+        if (base + k < n) out[base + k] = (OutT)run;
+        run += v[k];
+    }
+}
+
+static inline size_t scan_workspace_bytes(int64_t n) {
+    int64_t n_blocks = (n + SCAN_TILE - 1) / SCAN_TILE;
+    return splatad_align256((size_t)(n_blocks > 0 ? n_blocks : 1) * sizeof(int64_t));
+}
+
+// out[i] = sum_{j<i} f(in[j*stride]); *total (device) = sum over all.  `block_sums` is
+// scan_workspace_bytes(n) of scratch.  n == 0 only writes *total = 0.
+template <typename OutT>
+static inline int launch_exclusive_scan(const int32_t *in, int64_t n, int stride, int as_flag,
+                                        OutT *out, int64_t *total, int64_t *block_sums,
+                                        hipStream_t stream) {
+    int64_t n_blocks = (n + SCAN_TILE - 1) / SCAN_TILE;
+    if (n_blocks > 0) {
+        hipLaunchKernelGGL(scan_block_totals_kernel, dim3((uint32_t)n_blocks), dim3(SPLATAD_THREADS),
+                           0, stream, in, n, stride, as_flag, block_sums);
+        SPLATAD_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL(scan_block_sums_kernel, dim3(1), dim3(SPLATAD_THREADS), 0, stream,
+                       block_sums, n_blocks, total);
+    SPLATAD_LAUNCH_CHECK();
+    if (n_blocks > 0 && out != nullptr) {
+        hipLaunchKernelGGL(scan_apply_kernel<OutT>, dim3((uint32_t)n_blocks),
+                           dim3(SPLATAD_THREADS), 0, stream, in, n, stride, as_flag,
+                           (const int64_t *)block_sums, out);
+        SPLATAD_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+} // namespace
+
+#endif // __HIPCC__

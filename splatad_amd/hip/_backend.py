@@ -1,0 +1,503 @@
+"""Loader of libsplatad_hip.so and the `_C`-shaped operator table built on it.
+
+Counterpart of the reference's extension loader and pybind11 module
+(gsplat/cuda/_backend.py:80-142, gsplat/cuda/csrc/ext.cpp:4-52): `_C.<name>(*args)` takes the
+same positional arguments and returns the same tuples of tensors as the reference's C++ ops
+(gsplat/cuda/csrc/bindings.h:123-468).  Behind it sits a plain C ABI (include/splatad_hip.h)
+called through ctypes with raw device pointers; outputs and workspaces are allocated here with
+torch so that they live in torch's caching allocator, on torch's current stream.
+
+There is no CPU path: without the built library, or with non-GPU tensors, the ops raise.
+"""
+import ctypes
+import math
+import os
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+_PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG_DIR, "libsplatad_hip.so")
+
+_lib = None
+
+
+def load_library():
+    """Returns the ctypes handle of libsplatad_hip.so; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build the HIP kernels first with "
+                "`python -m splatad_amd.build` (needs hipcc). There is no CPU fallback."
+            )
+        lib = ctypes.CDLL(LIB_PATH)
+        lib.splatad_last_error.restype = ctypes.c_char_p
+        lib.splatad_abi_version.restype = ctypes.c_int
+        for name in ("splatad_projection_packed_workspace_bytes", "splatad_isect_workspace_bytes"):
+            getattr(lib, name).restype = ctypes.c_size_t
+        _lib = lib
+    return _lib
+
+
+def _check(rc: int):
+    if rc != 0:
+        msg = load_library().splatad_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"splatad_hip error {rc}: {msg}")
+
+
+def _in(t: Optional[Tensor], name: str, dtype=torch.float32) -> Optional[Tensor]:
+    """Input check (bindings.h:9-13 of the reference): GPU, contiguous, expected dtype."""
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name} must have dtype {dtype}, got {t.dtype}")
+    if t.data_ptr() % 16 != 0 and t.numel() > 0:
+        t = t.clone()  # the kernels use 8/16-byte vector accesses
+    return t
+
+
+def _p(t: Optional[Tensor]):
+    return ctypes.c_void_p(0 if t is None or t.numel() == 0 else t.data_ptr())
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+_u32, _i32, _i64, _u64, _f32 = ctypes.c_uint32, ctypes.c_int, ctypes.c_int64, ctypes.c_uint64, ctypes.c_float
+
+
+def _workspace(nbytes: int, device) -> Tensor:
+    return torch.empty((max(int(nbytes), 256),), dtype=torch.uint8, device=device)
+
+
+class _Ops:
+    """Operator table with the names and calling conventions of the reference's `_C`."""
+
+    # ------------------------------------------------------------------ projection
+    def fully_fused_projection_fwd(self, means, covars, quats, scales, velocities, viewmats, Ks,
+                                   image_width, image_height, linear_velocity, angular_velocity,
+                                   rolling_shutter_time, eps2d, near_plane, far_plane, radius_clip,
+                                   calc_compensations):
+        lib = load_library()
+        means = _in(means, "means"); covars = _in(covars, "covars"); quats = _in(quats, "quats")
+        scales = _in(scales, "scales"); velocities = _in(velocities, "velocities")
+        viewmats = _in(viewmats, "viewmats"); Ks = _in(Ks, "Ks")
+        lv = _in(linear_velocity, "linear_velocity"); av = _in(angular_velocity, "angular_velocity")
+        rs = _in(rolling_shutter_time, "rolling_shutter_time")
+        N, C, dev = means.shape[0], viewmats.shape[0], means.device
+        f = dict(dtype=torch.float32, device=dev)
+        radii = torch.empty((C, N, 2), dtype=torch.int32, device=dev)
+        means2d = torch.empty((C, N, 2), **f); depths = torch.empty((C, N), **f)
+        conics = torch.empty((C, N, 3), **f); pix_vels = torch.empty((C, N, 2), **f)
+        comps = torch.empty((C, N), **f) if calc_compensations else None
+        with torch.cuda.device(dev):
+            _check(lib.splatad_projection_fwd(
+                _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
+                _p(viewmats), _p(Ks), _u32(image_width), _u32(image_height), _p(lv), _p(av), _p(rs),
+                _f32(eps2d), _f32(near_plane), _f32(far_plane), _f32(radius_clip), _p(radii),
+                _p(means2d), _p(depths), _p(conics), _p(comps), _p(pix_vels), _stream(dev)))
+        return radii, means2d, depths, conics, comps, pix_vels
+
+    def fully_fused_projection_packed_fwd(self, means, covars, quats, scales, velocities, viewmats,
+                                          Ks, image_width, image_height, linear_velocity,
+                                          angular_velocity, rolling_shutter_time, eps2d, near_plane,
+                                          far_plane, radius_clip, calc_compensations):
+        lib = load_library()
+        means = _in(means, "means"); covars = _in(covars, "covars"); quats = _in(quats, "quats")
+        scales = _in(scales, "scales"); velocities = _in(velocities, "velocities")
+        viewmats = _in(viewmats, "viewmats"); Ks = _in(Ks, "Ks")
+        lv = _in(linear_velocity, "linear_velocity"); av = _in(angular_velocity, "angular_velocity")
+        rs = _in(rolling_shutter_time, "rolling_shutter_time")
+        N, C, dev = means.shape[0], viewmats.shape[0], means.device
+        f = dict(dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            ws = _workspace(lib.splatad_projection_packed_workspace_bytes(_u32(C), _u32(N)), dev)
+            nnz_host = _i64(0)
+            _check(lib.splatad_projection_packed_count(
+                _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
+                _p(viewmats), _p(Ks), _u32(image_width), _u32(image_height), _p(lv), _p(av), _p(rs),
+                _f32(eps2d), _f32(near_plane), _f32(far_plane), _f32(radius_clip),
+                _i32(bool(calc_compensations)), _p(ws), ctypes.byref(nnz_host), _stream(dev)))
+            nnz = int(nnz_host.value)
+            indptr = torch.empty((C + 1,), dtype=torch.int32, device=dev)
+            camera_ids = torch.empty((nnz,), dtype=torch.int64, device=dev)
+            gaussian_ids = torch.empty((nnz,), dtype=torch.int64, device=dev)
+            radii = torch.empty((nnz, 2), dtype=torch.int32, device=dev)
+            means2d = torch.empty((nnz, 2), **f); depths = torch.empty((nnz,), **f)
+            conics = torch.empty((nnz, 3), **f); pix_vels = torch.empty((nnz, 2), **f)
+            comps = torch.empty((nnz,), **f) if calc_compensations else None
+            _check(lib.splatad_projection_packed_fill(
+                _u32(C), _u32(N), _i64(nnz), _p(ws), _p(indptr), _p(camera_ids), _p(gaussian_ids),
+                _p(radii), _p(means2d), _p(depths), _p(conics), _p(comps), _p(pix_vels),
+                _stream(dev)))
+        return indptr, camera_ids, gaussian_ids, radii, means2d, depths, conics, comps, pix_vels
+
+    def fully_fused_lidar_projection_fwd(self, means, covars, quats, scales, velocities, viewmats,
+                                         min_elevation, max_elevation, min_azimuth, max_azimuth,
+                                         linear_velocity, angular_velocity, rolling_shutter_time,
+                                         eps2d, near_plane, far_plane, radius_clip,
+                                         calc_compensations):
+        lib = load_library()
+        means = _in(means, "means"); covars = _in(covars, "covars"); quats = _in(quats, "quats")
+        scales = _in(scales, "scales"); velocities = _in(velocities, "velocities")
+        viewmats = _in(viewmats, "viewmats")
+        lv = _in(linear_velocity, "linear_velocity"); av = _in(angular_velocity, "angular_velocity")
+        rs = _in(rolling_shutter_time, "rolling_shutter_time")
+        N, C, dev = means.shape[0], viewmats.shape[0], means.device
+        f = dict(dtype=torch.float32, device=dev)
+        radii = torch.empty((C, N, 2), **f)
+        means2d = torch.empty((C, N, 2), **f); depths = torch.empty((C, N), **f)
+        conics = torch.empty((C, N, 3), **f); pix_vels = torch.empty((C, N, 3), **f)
+        dcomps = torch.empty((C, N, 2), **f)
+        comps = torch.empty((C, N), **f) if calc_compensations else None
+        with torch.cuda.device(dev):
+            _check(lib.splatad_lidar_projection_fwd(
+                _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
+                _p(viewmats), _f32(min_elevation), _f32(max_elevation), _f32(min_azimuth),
+                _f32(max_azimuth), _p(lv), _p(av), _p(rs), _f32(eps2d), _f32(near_plane),
+                _f32(far_plane), _f32(radius_clip), _p(radii), _p(means2d), _p(depths), _p(conics),
+                _p(comps), _p(pix_vels), _p(dcomps), _stream(dev)))
+        return radii, means2d, depths, conics, comps, pix_vels, dcomps
+
+    def fully_fused_projection_bwd(self, means, covars, quats, scales, velocities, viewmats, Ks,
+                                   image_width, image_height, linear_velocity, angular_velocity,
+                                   rolling_shutter_time, eps2d, radii, conics, compensations,
+                                   v_means2d, v_depths, v_conics, v_compensations, v_pix_vels,
+                                   viewmats_requires_grad, velocities_requires_grad=False):
+        return self._projection_bwd(means, covars, quats, scales, velocities, viewmats, Ks,
+                                    image_width, image_height, linear_velocity, angular_velocity,
+                                    rolling_shutter_time, eps2d, None, None, radii, conics,
+                                    compensations, v_means2d, v_depths, v_conics, v_compensations,
+                                    v_pix_vels, viewmats_requires_grad, False,
+                                    velocities_requires_grad)
+
+    def fully_fused_projection_packed_bwd(self, means, covars, quats, scales, velocities, viewmats,
+                                          Ks, image_width, image_height, linear_velocity,
+                                          angular_velocity, rolling_shutter_time, eps2d, camera_ids,
+                                          gaussian_ids, conics, compensations, pix_vels, v_means2d,
+                                          v_depths, v_conics, v_compensations, v_pix_vels,
+                                          viewmats_requires_grad, sparse_grad,
+                                          velocities_requires_grad=False):
+        return self._projection_bwd(means, covars, quats, scales, velocities, viewmats, Ks,
+                                    image_width, image_height, linear_velocity, angular_velocity,
+                                    rolling_shutter_time, eps2d, camera_ids, gaussian_ids, None,
+                                    conics, compensations, v_means2d, v_depths, v_conics,
+                                    v_compensations, v_pix_vels, viewmats_requires_grad, sparse_grad,
+                                    velocities_requires_grad)
+
+    def _projection_bwd(self, means, covars, quats, scales, velocities, viewmats, Ks, image_width,
+                        image_height, linear_velocity, angular_velocity, rolling_shutter_time, eps2d,
+                        camera_ids, gaussian_ids, radii, conics, compensations, v_means2d, v_depths,
+                        v_conics, v_compensations, v_pix_vels, viewmats_requires_grad, sparse_grad,
+                        velocities_requires_grad):
+        lib = load_library()
+        means = _in(means, "means"); covars = _in(covars, "covars"); quats = _in(quats, "quats")
+        scales = _in(scales, "scales"); velocities = _in(velocities, "velocities")
+        viewmats = _in(viewmats, "viewmats"); Ks = _in(Ks, "Ks")
+        lv = _in(linear_velocity, "linear_velocity"); av = _in(angular_velocity, "angular_velocity")
+        rs = _in(rolling_shutter_time, "rolling_shutter_time")
+        camera_ids = _in(camera_ids, "camera_ids", torch.int64)
+        gaussian_ids = _in(gaussian_ids, "gaussian_ids", torch.int64)
+        radii = _in(radii, "radii", torch.int32); conics = _in(conics, "conics")
+        compensations = _in(compensations, "compensations")
+        v_means2d = _in(v_means2d, "v_means2d"); v_depths = _in(v_depths, "v_depths")
+        v_conics = _in(v_conics, "v_conics"); v_compensations = _in(v_compensations, "v_compensations")
+        v_pix_vels = _in(v_pix_vels, "v_pix_vels")
+        N, C, dev = means.shape[0], viewmats.shape[0], means.device
+        packed = camera_ids is not None
+        nnz = camera_ids.shape[0] if packed else 0
+        rows = nnz if (packed and sparse_grad) else N
+        f = dict(dtype=torch.float32, device=dev)
+        v_means = torch.zeros((rows, 3), **f)
+        v_covars = torch.zeros((rows, 6), **f) if covars is not None else None
+        v_quats = torch.zeros((rows, 4), **f) if covars is None else None
+        v_scales = torch.zeros((rows, 3), **f) if covars is None else None
+        v_viewmats = torch.zeros_like(viewmats) if viewmats_requires_grad else None
+        v_velocities = (torch.zeros_like(velocities)
+                        if (velocities_requires_grad and velocities is not None) else None)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_projection_bwd(
+                _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
+                _p(viewmats), _p(Ks), _u32(image_width), _u32(image_height), _p(lv), _p(av), _p(rs),
+                _f32(eps2d), _p(camera_ids), _p(gaussian_ids), _i64(nnz), _p(radii), _p(conics),
+                _p(compensations), _p(v_means2d), _p(v_depths), _p(v_conics), _p(v_compensations),
+                _p(v_pix_vels), _i32(bool(sparse_grad)), _p(v_means), _p(v_covars), _p(v_quats),
+                _p(v_scales), _p(v_viewmats), _p(v_velocities), _stream(dev)))
+        if velocities_requires_grad:
+            return v_means, v_covars, v_quats, v_scales, v_viewmats, v_velocities
+        return v_means, v_covars, v_quats, v_scales, v_viewmats
+
+    def fully_fused_lidar_projection_bwd(self, means, covars, quats, scales, velocities, viewmats,
+                                         min_elevation, max_elevation, min_azimuth, max_azimuth,
+                                         linear_velocity, angular_velocity, rolling_shutter_time,
+                                         eps2d, radii, conics, compensations, v_means2d, v_depths,
+                                         v_conics, v_compensations, v_pix_vels,
+                                         v_depth_compensations, viewmats_requires_grad,
+                                         velocities_requires_grad=False):
+        lib = load_library()
+        means = _in(means, "means"); covars = _in(covars, "covars"); quats = _in(quats, "quats")
+        scales = _in(scales, "scales"); velocities = _in(velocities, "velocities")
+        viewmats = _in(viewmats, "viewmats")
+        lv = _in(linear_velocity, "linear_velocity"); av = _in(angular_velocity, "angular_velocity")
+        rs = _in(rolling_shutter_time, "rolling_shutter_time")
+        radii = _in(radii, "radii"); conics = _in(conics, "conics")
+        compensations = _in(compensations, "compensations")
+        v_means2d = _in(v_means2d, "v_means2d"); v_depths = _in(v_depths, "v_depths")
+        v_conics = _in(v_conics, "v_conics"); v_compensations = _in(v_compensations, "v_compensations")
+        v_pix_vels = _in(v_pix_vels, "v_pix_vels")
+        v_dc = _in(v_depth_compensations, "v_depth_compensations")
+        N, C, dev = means.shape[0], viewmats.shape[0], means.device
+        v_means = torch.zeros_like(means)
+        v_covars = torch.zeros_like(covars) if covars is not None else None
+        v_quats = torch.zeros_like(quats) if covars is None else None
+        v_scales = torch.zeros_like(scales) if covars is None else None
+        v_viewmats = torch.zeros_like(viewmats) if viewmats_requires_grad else None
+        v_velocities = (torch.zeros_like(velocities)
+                        if (velocities_requires_grad and velocities is not None) else None)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_lidar_projection_bwd(
+                _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
+                _p(viewmats), _p(lv), _p(av), _p(rs), _f32(eps2d), _p(radii), _p(conics),
+                _p(compensations), _p(v_means2d), _p(v_depths), _p(v_conics), _p(v_compensations),
+                _p(v_pix_vels), _p(v_dc), _p(v_means), _p(v_covars), _p(v_quats), _p(v_scales),
+                _p(v_viewmats), _p(v_velocities), _stream(dev)))
+        if velocities_requires_grad:
+            return v_means, v_covars, v_quats, v_scales, v_viewmats, v_velocities
+        return v_means, v_covars, v_quats, v_scales, v_viewmats
+
+    # ------------------------------------------------------------------ spherical harmonics
+    def compute_sh_fwd(self, degrees_to_use, dirs, coeffs, masks):
+        lib = load_library()
+        dirs = _in(dirs, "dirs"); coeffs = _in(coeffs, "coeffs")
+        masks = _in(masks, "masks", torch.bool)
+        if coeffs.shape[-1] != 3:
+            raise RuntimeError("coeffs must have last dimension 3")
+        if dirs.shape[-1] != 3:
+            raise RuntimeError("dirs must have last dimension 3")
+        K, n, dev = coeffs.shape[-2], dirs.numel() // 3, dirs.device
+        colors = torch.empty_like(dirs)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_sh_fwd(_u32(n), _u32(K), _u32(degrees_to_use), _p(dirs), _p(coeffs),
+                                      _p(masks), _p(colors), _stream(dev)))
+        return colors
+
+    def compute_sh_bwd(self, K, degrees_to_use, dirs, coeffs, masks, v_colors, compute_v_dirs):
+        lib = load_library()
+        dirs = _in(dirs, "dirs"); coeffs = _in(coeffs, "coeffs")
+        masks = _in(masks, "masks", torch.bool); v_colors = _in(v_colors, "v_colors")
+        n, dev = dirs.numel() // 3, dirs.device
+        v_coeffs = torch.zeros_like(coeffs)
+        v_dirs = torch.zeros_like(dirs) if compute_v_dirs else None
+        with torch.cuda.device(dev):
+            _check(lib.splatad_sh_bwd(_u32(n), _u32(K), _u32(degrees_to_use), _p(dirs), _p(coeffs),
+                                      _p(masks), _p(v_colors), _p(v_coeffs), _p(v_dirs),
+                                      _stream(dev)))
+        return v_coeffs, v_dirs
+
+    # ------------------------------------------------------------------ intersection
+    def _isect(self, lidar, means2d, radii, depths, camera_ids, gaussian_ids, C, grid_args,
+               tile_w, tile_h, sort):
+        lib = load_library()
+        means2d = _in(means2d, "means2d"); depths = _in(depths, "depths")
+        radii = _in(radii, "radii", torch.float32 if lidar else torch.int32)
+        camera_ids = _in(camera_ids, "camera_ids", torch.int64)
+        _in(gaussian_ids, "gaussian_ids", torch.int64)
+        packed = means2d.dim() == 2
+        dev = means2d.device
+        if packed:
+            assert camera_ids is not None and gaussian_ids is not None
+            total, N = means2d.shape[0], 0
+        else:
+            N = means2d.shape[1]
+            total = C * N
+            camera_ids = None
+        n_tiles = tile_w * tile_h
+        # reference: assert(tile_n_bits + cam_n_bits <= 32), rasterization.cu:138
+        assert n_tiles.bit_length() + int(C).bit_length() <= 32
+        tiles_per_gauss = torch.empty(depths.shape, dtype=torch.int32, device=dev)
+        count = lib.splatad_isect_lidar_tiles_count if lidar else lib.splatad_isect_tiles_count
+        fill = lib.splatad_isect_lidar_tiles_fill if lidar else lib.splatad_isect_tiles_fill
+        with torch.cuda.device(dev):
+            ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(total), _u32(C), _u32(n_tiles),
+                                                              _i64(0)), dev)
+            n_host = _i64(0)
+            _check(count(_u64(total), _p(means2d), _p(radii), _u32(C), *grid_args, _u32(tile_w),
+                         _u32(tile_h), _p(tiles_per_gauss), _p(ws), ctypes.byref(n_host),
+                         _stream(dev)))
+            n_isects = int(n_host.value)
+            isect_ids = torch.empty((n_isects,), dtype=torch.int64, device=dev)
+            flatten_ids = torch.empty((n_isects,), dtype=torch.int32, device=dev)
+            if n_isects:
+                ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(total), _u32(C),
+                                                                  _u32(n_tiles), _i64(n_isects)), dev)
+                _check(fill(_u64(total), _u32(N), _p(camera_ids), _p(means2d), _p(radii),
+                            _p(depths), _u32(C), *grid_args, _u32(tile_w), _u32(tile_h),
+                            _i32(bool(sort)), _i64(n_isects), _p(tiles_per_gauss), _p(ws),
+                            _p(isect_ids), _p(flatten_ids), _stream(dev)))
+        return tiles_per_gauss, isect_ids, flatten_ids
+
+    def isect_tiles(self, means2d, radii, depths, camera_ids, gaussian_ids, C, tile_size,
+                    tile_width, tile_height, sort, double_buffer):
+        return self._isect(False, means2d, radii, depths, camera_ids, gaussian_ids, C,
+                           (_u32(tile_size),), tile_width, tile_height, sort)
+
+    def isect_lidar_tiles(self, means2d, radii, depths, camera_ids, gaussian_ids, C,
+                          elev_boundaries, tile_azim_resolution, min_azim, sort, double_buffer):
+        eb = _in(elev_boundaries, "elev_boundaries")
+        # rasterization.cu:435-436: float32 division, then ceil
+        res32 = torch.tensor(tile_azim_resolution, dtype=torch.float32)
+        n_tiles_azim = int(math.ceil((torch.tensor(360.0, dtype=torch.float32) / res32).item()))
+        n_tiles_elev = eb.shape[0] - 1
+        return self._isect(True, means2d, radii, depths, camera_ids, gaussian_ids, C,
+                           (_p(eb), _f32(tile_azim_resolution), _f32(min_azim)), n_tiles_azim,
+                           n_tiles_elev, sort)
+
+    def isect_offset_encode(self, isect_ids, C, tile_width, tile_height):
+        lib = load_library()
+        isect_ids = _in(isect_ids, "isect_ids", torch.int64)
+        dev = isect_ids.device
+        offsets = torch.empty((C, tile_height, tile_width), dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_isect_offset_encode(_i64(isect_ids.shape[0]), _p(isect_ids), _u32(C),
+                                                   _u32(tile_width * tile_height), _p(offsets),
+                                                   _stream(dev)))
+        return offsets
+
+    # ------------------------------------------------------------------ rasterization
+    def rasterize_to_pixels_fwd(self, means2d, conics, colors, opacities, pix_vels,
+                                rolling_shutter_time, backgrounds, image_width, image_height,
+                                tile_size, tile_offsets, flatten_ids):
+        lib = load_library()
+        means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
+        colors = _in(colors, "colors"); opacities = _in(opacities, "opacities")
+        pix_vels = _in(pix_vels, "pix_vels"); rs = _in(rolling_shutter_time, "rolling_shutter_time")
+        backgrounds = _in(backgrounds, "backgrounds")
+        tile_offsets = _in(tile_offsets, "tile_offsets", torch.int32)
+        flatten_ids = _in(flatten_ids, "flatten_ids", torch.int32)
+        C, th, tw = tile_offsets.shape
+        D, dev = colors.shape[-1], means2d.device
+        f = dict(dtype=torch.float32, device=dev)
+        renders = torch.empty((C, image_height, image_width, D), **f)
+        alphas = torch.empty((C, image_height, image_width, 1), **f)
+        last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_rasterize_to_pixels_fwd(
+                _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics), _p(colors),
+                _p(opacities), _p(pix_vels), _p(rs), _p(backgrounds), _u32(image_width),
+                _u32(image_height), _u32(tile_size), _u32(tw), _u32(th), _p(tile_offsets),
+                _p(flatten_ids), _p(renders), _p(alphas), _p(last_ids), _stream(dev)))
+        return renders, alphas, last_ids
+
+    def rasterize_to_pixels_bwd(self, means2d, conics, colors, opacities, pix_vels,
+                                rolling_shutter_time, backgrounds, image_width, image_height,
+                                tile_size, tile_offsets, flatten_ids, render_alphas, last_ids,
+                                v_render_colors, v_render_alphas, absgrad):
+        lib = load_library()
+        means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
+        colors = _in(colors, "colors"); opacities = _in(opacities, "opacities")
+        pix_vels = _in(pix_vels, "pix_vels"); rs = _in(rolling_shutter_time, "rolling_shutter_time")
+        backgrounds = _in(backgrounds, "backgrounds")
+        tile_offsets = _in(tile_offsets, "tile_offsets", torch.int32)
+        flatten_ids = _in(flatten_ids, "flatten_ids", torch.int32)
+        render_alphas = _in(render_alphas, "render_alphas")
+        last_ids = _in(last_ids, "last_ids", torch.int32)
+        v_render_colors = _in(v_render_colors, "v_render_colors")
+        v_render_alphas = _in(v_render_alphas, "v_render_alphas")
+        C, th, tw = tile_offsets.shape
+        D, dev = colors.shape[-1], means2d.device
+        v_means2d = torch.zeros_like(means2d); v_conics = torch.zeros_like(conics)
+        v_colors = torch.zeros_like(colors); v_opacities = torch.zeros_like(opacities)
+        v_pix_vels = torch.zeros_like(pix_vels)
+        v_means2d_abs = torch.zeros_like(means2d) if absgrad else None
+        if flatten_ids.shape[0]:
+            with torch.cuda.device(dev):
+                _check(lib.splatad_rasterize_to_pixels_bwd(
+                    _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics),
+                    _p(colors), _p(opacities), _p(pix_vels), _p(rs), _p(backgrounds),
+                    _u32(image_width), _u32(image_height), _u32(tile_size), _u32(tw), _u32(th),
+                    _p(tile_offsets), _p(flatten_ids), _p(render_alphas), _p(last_ids),
+                    _p(v_render_colors), _p(v_render_alphas), _p(v_means2d_abs), _p(v_means2d),
+                    _p(v_conics), _p(v_colors), _p(v_opacities), _p(v_pix_vels), _stream(dev)))
+        return v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities, v_pix_vels
+
+    def rasterize_to_points_fwd(self, means2d, conics, colors, opacities, pix_vels,
+                                depth_compensations, backgrounds, raster_pts, image_width,
+                                image_height, tile_width, tile_height,
+                                compute_alpha_sum_until_points,
+                                compute_alpha_sum_until_points_threshold, tile_offsets, flatten_ids,
+                                depth_channel_idx):
+        lib = load_library()
+        means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
+        colors = _in(colors, "colors"); opacities = _in(opacities, "opacities")
+        pix_vels = _in(pix_vels, "pix_vels"); dc = _in(depth_compensations, "depth_compensations")
+        backgrounds = _in(backgrounds, "backgrounds"); raster_pts = _in(raster_pts, "raster_pts")
+        tile_offsets = _in(tile_offsets, "tile_offsets", torch.int32)
+        flatten_ids = _in(flatten_ids, "flatten_ids", torch.int32)
+        C, gh, gw = tile_offsets.shape
+        D, dev = colors.shape[-1], means2d.device
+        f = dict(dtype=torch.float32, device=dev)
+        renders = torch.empty((C, image_height, image_width, D), **f)
+        alphas = torch.empty((C, image_height, image_width, 1), **f)
+        medians = torch.empty((C, image_height, image_width, 1), **f)
+        asum = (torch.empty((C, image_height, image_width, 1), **f)
+                if compute_alpha_sum_until_points else None)
+        last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_rasterize_to_points_fwd(
+                _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics), _p(colors),
+                _p(opacities), _p(pix_vels), _p(dc), _p(backgrounds), _p(raster_pts),
+                _u32(image_width), _u32(image_height), _u32(tile_width), _u32(tile_height),
+                _u32(gw), _u32(gh), _i32(bool(compute_alpha_sum_until_points)),
+                _f32(compute_alpha_sum_until_points_threshold), _p(tile_offsets), _p(flatten_ids),
+                _u32(depth_channel_idx), _p(renders), _p(alphas), _p(asum), _p(last_ids),
+                _p(medians), _stream(dev)))
+        return renders, alphas, last_ids, asum, medians
+
+    def rasterize_to_points_bwd(self, means2d, conics, colors, opacities, pix_vels,
+                                depth_compensations, backgrounds, raster_pts, image_width,
+                                image_height, tile_width, tile_height, tile_offsets, flatten_ids,
+                                render_alphas, last_ids, v_render_colors, v_render_alphas,
+                                v_alpha_sum_until_points, absgrad, compute_alpha_sum_until_points,
+                                compute_alpha_sum_until_points_threshold, depth_channel_idx):
+        lib = load_library()
+        means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
+        colors = _in(colors, "colors"); opacities = _in(opacities, "opacities")
+        pix_vels = _in(pix_vels, "pix_vels"); dc = _in(depth_compensations, "depth_compensations")
+        backgrounds = _in(backgrounds, "backgrounds"); raster_pts = _in(raster_pts, "raster_pts")
+        tile_offsets = _in(tile_offsets, "tile_offsets", torch.int32)
+        flatten_ids = _in(flatten_ids, "flatten_ids", torch.int32)
+        render_alphas = _in(render_alphas, "render_alphas")
+        last_ids = _in(last_ids, "last_ids", torch.int32)
+        v_render_colors = _in(v_render_colors, "v_render_colors")
+        v_render_alphas = _in(v_render_alphas, "v_render_alphas")
+        v_asum = _in(v_alpha_sum_until_points, "v_alpha_sum_until_points")
+        C, gh, gw = tile_offsets.shape
+        D, dev = colors.shape[-1], means2d.device
+        v_means2d = torch.zeros_like(means2d); v_conics = torch.zeros_like(conics)
+        v_colors = torch.zeros_like(colors); v_opacities = torch.zeros_like(opacities)
+        v_pix_vels = torch.zeros_like(pix_vels); v_dc = torch.zeros_like(dc)
+        v_means2d_abs = torch.zeros_like(means2d) if absgrad else None
+        if flatten_ids.shape[0]:
+            with torch.cuda.device(dev):
+                _check(lib.splatad_rasterize_to_points_bwd(
+                    _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics),
+                    _p(colors), _p(opacities), _p(pix_vels), _p(dc), _p(backgrounds),
+                    _p(raster_pts), _u32(image_width), _u32(image_height), _u32(tile_width),
+                    _u32(tile_height), _u32(gw), _u32(gh),
+                    _i32(bool(compute_alpha_sum_until_points)),
+                    _f32(compute_alpha_sum_until_points_threshold), _p(tile_offsets),
+                    _p(flatten_ids), _u32(depth_channel_idx), _p(render_alphas), _p(last_ids),
+                    _p(v_render_colors), _p(v_render_alphas), _p(v_asum), _p(v_means2d_abs),
+                    _p(v_means2d), _p(v_conics), _p(v_colors), _p(v_opacities), _p(v_pix_vels),
+                    _p(v_dc), _stream(dev)))
+        return v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_dc
+
+
+_C = _Ops()

@@ -1,0 +1,600 @@
+"""Operator wrappers and autograd glue over the HIP kernels.
+
+Same public names, argument order, defaults and return values as the reference's
+gsplat/cuda/_wrapper.py (functions at :17, :230, :390, :533, :606, :680, :811, :951; autograd
+classes at :1495-2351), so code written against those operators runs unchanged.  Differences,
+all on the permissive side:
+  * channel counts are passed to the kernels as they are (no host-side zero padding);
+  * rows of culled Gaussians and masked SH rows are zeros instead of uninitialised memory;
+  * the fused projections return a gradient for per-Gaussian `velocities` (the reference
+    computes it and drops it, gsplat/cuda/csrc/projection.cu:874-877).
+"""
+from typing import Callable, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+MAX_CHANNELS = 513  # same ceiling as the reference (gsplat/cuda/_wrapper.py:878)
+
+
+def _make_lazy_hip_func(name: str) -> Callable:
+    """Late lookup in the op table, so importing this module needs no GPU and no library."""
+
+    def call_hip(*args, **kwargs):
+        from ._backend import _C
+
+        return getattr(_C, name)(*args, **kwargs)
+
+    return call_hip
+
+
+def _c(t: Optional[Tensor]) -> Optional[Tensor]:
+    return None if t is None else t.contiguous()
+
+
+def _check_gaussians(means, covars, quats, scales, velocities):
+    N = means.size(0)
+    assert means.size() == (N, 3), means.size()
+    if covars is not None:
+        assert covars.size() == (N, 6), covars.size()
+    else:
+        assert quats is not None, "covars or quats is required"
+        assert scales is not None, "covars or scales is required"
+        assert quats.size() == (N, 4), quats.size()
+        assert scales.size() == (N, 3), scales.size()
+    if velocities is not None:
+        assert velocities.size() == (N, 3), velocities.size()
+    return N
+
+
+def spherical_harmonics(
+    degrees_to_use: int,
+    dirs: Tensor,  # [..., 3]
+    coeffs: Tensor,  # [..., K, 3]
+    masks: Optional[Tensor] = None,  # [...]
+) -> Tensor:
+    """Evaluates real spherical harmonics of degree `degrees_to_use` (0..4) in the directions
+    `dirs` (need not be unit length) with coefficients `coeffs`; returns [..., 3].  Rows whose
+    mask is False are skipped (zeros)."""
+    assert (degrees_to_use + 1) ** 2 <= coeffs.shape[-2], coeffs.shape
+    assert dirs.shape[:-1] == coeffs.shape[:-2], (dirs.shape, coeffs.shape)
+    assert dirs.shape[-1] == 3, dirs.shape
+    assert coeffs.shape[-1] == 3, coeffs.shape
+    if masks is not None:
+        assert masks.shape == dirs.shape[:-1], masks.shape
+        masks = masks.contiguous()
+    return _SphericalHarmonics.apply(degrees_to_use, dirs.contiguous(), coeffs.contiguous(), masks)
+
+
+def fully_fused_projection(
+    means: Tensor,  # [N, 3]
+    covars: Optional[Tensor],  # [N, 6] or None
+    quats: Optional[Tensor],  # [N, 4] or None
+    scales: Optional[Tensor],  # [N, 3] or None
+    velocities: Optional[Tensor],  # [N, 3] or None
+    viewmats: Tensor,  # [C, 4, 4]
+    Ks: Tensor,  # [C, 3, 3]
+    width: int,
+    height: int,
+    linear_velocity: Tensor,  # [C, 3]
+    angular_velocity: Tensor,  # [C, 3]
+    rolling_shutter_time: Tensor,  # [C]
+    eps2d: float = 0.3,
+    near_plane: float = 0.01,
+    far_plane: float = 1e10,
+    radius_clip: float = 0.0,
+    packed: bool = False,
+    sparse_grad: bool = False,
+    calc_compensations: bool = False,
+):
+    """Projects Gaussians onto C pinhole image planes (EWA splatting) with rolling-shutter
+    pixel velocities.
+
+    Returns, unpacked: (radii int32[C,N,2], means2d[C,N,2], depths[C,N], conics[C,N,3],
+    compensations[C,N] | None, pix_vels[C,N,2]); a zero radius marks a culled Gaussian.
+    Packed: (camera_ids[nnz], gaussian_ids[nnz], radii[nnz,2], means2d[nnz,2], depths[nnz],
+    conics[nnz,3], compensations[nnz] | None, pix_vels[nnz,2]) in (camera, gaussian) order.
+    """
+    C = viewmats.size(0)
+    _check_gaussians(means, covars, quats, scales, velocities)
+    assert viewmats.size() == (C, 4, 4), viewmats.size()
+    assert Ks.size() == (C, 3, 3), Ks.size()
+    assert linear_velocity.size() == (C, 3), linear_velocity.size()
+    assert angular_velocity.size() == (C, 3), angular_velocity.size()
+    assert rolling_shutter_time.size() == (C,), rolling_shutter_time.size()
+    if sparse_grad:
+        assert packed, "sparse_grad is only supported when packed is True"
+    args = (
+        means.contiguous(), _c(covars), _c(quats), _c(scales), _c(velocities),
+        viewmats.contiguous(), Ks.contiguous(), width, height, linear_velocity.contiguous(),
+        angular_velocity.contiguous(), rolling_shutter_time.contiguous(), eps2d, near_plane,
+        far_plane, radius_clip,
+    )
+    if packed:
+        return _FullyFusedProjectionPacked.apply(*args, sparse_grad, calc_compensations)
+    return _FullyFusedProjection.apply(*args, calc_compensations)
+
+
+def fully_fused_lidar_projection(
+    means: Tensor,  # [N, 3]
+    covars: Optional[Tensor],  # [N, 6] or None
+    quats: Optional[Tensor],  # [N, 4] or None
+    scales: Optional[Tensor],  # [N, 3] or None
+    velocities: Optional[Tensor],  # [N, 3] or None
+    viewmats: Tensor,  # [C, 4, 4]
+    linear_velocity: Tensor,  # [C, 3]
+    angular_velocity: Tensor,  # [C, 3]
+    rolling_shutter_time: Tensor,  # [C]
+    min_elevation: float = -45,
+    max_elevation: float = 45,
+    min_azimuth: float = -180,
+    max_azimuth: float = 180,
+    eps2d: float = 0.01,
+    near_plane: float = 0.01,
+    far_plane: float = 1e10,
+    radius_clip: float = 0.0,
+    packed: bool = False,
+    sparse_grad: bool = False,
+    calc_compensations: bool = False,
+):
+    """Projects Gaussians into the spherical frame (azimuth deg, elevation deg, range) of C
+    lidars.
+
+    Returns (radii float[C,N,2] in degrees, means2d[C,N,2] in degrees, depths[C,N] = range,
+    conics[C,N,3], compensations[C,N] | None, pix_vels[C,N,3] = (deg/s, deg/s, m/s),
+    depth_compensations[C,N,2] = change of range per degree of angular offset).
+    Packed mode does not exist for lidars.
+    """
+    C = viewmats.size(0)
+    _check_gaussians(means, covars, quats, scales, velocities)
+    assert viewmats.size() == (C, 4, 4), viewmats.size()
+    if sparse_grad:
+        assert packed, "sparse_grad is only supported when packed is True"
+    if packed:
+        raise NotImplementedError("FullyFusedLidarProjectionPacked is not implemented yet")
+    return _FullyFusedLidarProjection.apply(
+        means.contiguous(), _c(covars), _c(quats), _c(scales), _c(velocities),
+        viewmats.contiguous(), min_elevation, max_elevation, min_azimuth, max_azimuth,
+        linear_velocity.contiguous(), angular_velocity.contiguous(),
+        rolling_shutter_time.contiguous(), eps2d, near_plane, far_plane, radius_clip,
+        calc_compensations,
+    )
+
+
+def _check_projected(means2d, radii, depths, packed, n_cameras, camera_ids, gaussian_ids):
+    if packed:
+        nnz = means2d.size(0)
+        assert means2d.shape == (nnz, 2), means2d.size()
+        assert radii.shape == (nnz, 2), radii.size()
+        assert depths.shape == (nnz,), depths.size()
+        assert camera_ids is not None, "camera_ids is required if packed is True"
+        assert gaussian_ids is not None, "gaussian_ids is required if packed is True"
+        assert n_cameras is not None, "n_cameras is required if packed is True"
+        return n_cameras, camera_ids.contiguous(), gaussian_ids.contiguous()
+    C, N, _ = means2d.shape
+    assert means2d.shape == (C, N, 2), means2d.size()
+    assert radii.shape == (C, N, 2), radii.size()
+    assert depths.shape == (C, N), depths.size()
+    return C, camera_ids, gaussian_ids
+
+
+@torch.no_grad()
+def isect_tiles(
+    means2d: Tensor,  # [C, N, 2] or [nnz, 2]
+    radii: Tensor,  # [C, N, 2] or [nnz, 2]
+    depths: Tensor,  # [C, N] or [nnz]
+    tile_size: int,
+    tile_width: int,
+    tile_height: int,
+    sort: bool = True,
+    packed: bool = False,
+    n_cameras: Optional[int] = None,
+    camera_ids: Optional[Tensor] = None,
+    gaussian_ids: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """Lists the image tiles every projected Gaussian touches.
+
+    Returns (tiles_per_gauss int32[C,N] | [nnz], isect_ids int64[n_isects] with layout
+    camera | tile | float bits of depth, flatten_ids int32[n_isects]); sorted by isect id
+    (ties in emission order) when `sort`.
+    """
+    C, camera_ids, gaussian_ids = _check_projected(
+        means2d, radii, depths, packed, n_cameras, camera_ids, gaussian_ids
+    )
+    return _make_lazy_hip_func("isect_tiles")(
+        means2d.contiguous(), radii.contiguous(), depths.contiguous(), camera_ids, gaussian_ids,
+        C, tile_size, tile_width, tile_height, sort, True,
+    )
+
+
+@torch.no_grad()
+def isect_lidar_tiles(
+    means2d: Tensor,  # [C, N, 2] or [nnz, 2]
+    radii: Tensor,  # [C, N, 2] or [nnz, 2]
+    depths: Tensor,  # [C, N] or [nnz]
+    elev_boundaries: Tensor,
+    tile_azim_resolution: float,
+    min_azim: float,
+    sort: bool = True,
+    packed: bool = False,
+    n_cameras: Optional[int] = None,
+    camera_ids: Optional[Tensor] = None,
+    gaussian_ids: Optional[Tensor] = None,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """Lists the lidar tiles (uniform in azimuth with wrap-around, `elev_boundaries` in
+    elevation) every projected Gaussian touches.  Same outputs as :func:`isect_tiles`."""
+    C, camera_ids, gaussian_ids = _check_projected(
+        means2d, radii, depths, packed, n_cameras, camera_ids, gaussian_ids
+    )
+    return _make_lazy_hip_func("isect_lidar_tiles")(
+        means2d.contiguous(), radii.contiguous(), depths.contiguous(), camera_ids, gaussian_ids,
+        C, elev_boundaries.contiguous(), tile_azim_resolution, min_azim, sort, True,
+    )
+
+
+@torch.no_grad()
+def isect_offset_encode(isect_ids: Tensor, n_cameras: int, tile_width: int, tile_height: int) -> Tensor:
+    """Start of every (camera, tile) segment in the sorted intersection list,
+    int32 [C, tile_height, tile_width]."""
+    return _make_lazy_hip_func("isect_offset_encode")(
+        isect_ids.contiguous(), n_cameras, tile_width, tile_height
+    )
+
+
+def rasterize_to_pixels(
+    means2d: Tensor,  # [C, N, 2] or [nnz, 2]
+    conics: Tensor,  # [C, N, 3] or [nnz, 3]
+    colors: Tensor,  # [C, N, channels] or [nnz, channels]
+    opacities: Tensor,  # [C, N] or [nnz]
+    pix_vels: Tensor,  # [C, N, 2] or [nnz, 2]
+    image_width: int,
+    image_height: int,
+    tile_size: int,
+    isect_offsets: Tensor,  # [C, tile_height, tile_width]
+    flatten_ids: Tensor,  # [n_isects]
+    rolling_shutter_time: Optional[Tensor] = None,  # [C]
+    backgrounds: Optional[Tensor] = None,  # [C, channels]
+    packed: bool = False,
+    absgrad: bool = False,
+) -> Tuple[Tensor, Tensor]:
+    """Front-to-back alpha compositing of the sorted per-tile Gaussian lists onto the pixel
+    grid, with a per-row rolling-shutter shift of the Gaussian centres.
+
+    Returns (render_colors[C,H,W,channels], render_alphas[C,H,W,1]).
+    """
+    C = isect_offsets.size(0)
+    device = means2d.device
+    if packed:
+        nnz = means2d.size(0)
+        assert means2d.shape == (nnz, 2), means2d.shape
+        assert conics.shape == (nnz, 3), conics.shape
+        assert colors.shape[0] == nnz, colors.shape
+        assert opacities.shape == (nnz,), opacities.shape
+        assert pix_vels.shape == (nnz, 2), pix_vels.shape
+    else:
+        N = means2d.size(1)
+        assert means2d.shape == (C, N, 2), means2d.shape
+        assert conics.shape == (C, N, 3), conics.shape
+        assert colors.shape[:2] == (C, N), colors.shape
+        assert opacities.shape == (C, N), opacities.shape
+        assert pix_vels.shape == (C, N, 2), pix_vels.shape
+    if rolling_shutter_time is not None:
+        assert rolling_shutter_time.shape == (C,), rolling_shutter_time.shape
+    else:
+        rolling_shutter_time = torch.zeros(C, device=device)
+    if backgrounds is not None:
+        assert backgrounds.shape == (C, colors.shape[-1]), backgrounds.shape
+        backgrounds = backgrounds.contiguous()
+    channels = colors.shape[-1]
+    if channels > MAX_CHANNELS or channels == 0:
+        raise ValueError(f"Unsupported number of color channels: {channels}")
+    tile_height, tile_width = isect_offsets.shape[1:3]
+    assert tile_height * tile_size >= image_height, f"Assert Failed: {tile_height} * {tile_size} >= {image_height}"
+    assert tile_width * tile_size >= image_width, f"Assert Failed: {tile_width} * {tile_size} >= {image_width}"
+
+    return _RasterizeToPixels.apply(
+        means2d.contiguous(), conics.contiguous(), colors.contiguous(), opacities.contiguous(),
+        pix_vels.contiguous(), rolling_shutter_time.contiguous(), backgrounds, image_width,
+        image_height, tile_size, isect_offsets.contiguous(), flatten_ids.contiguous(), absgrad,
+    )
+
+
+def rasterize_to_points(
+    means2d: Tensor,  # [C, N, 2] or [nnz, 2]
+    conics: Tensor,  # [C, N, 3] or [nnz, 3]
+    lidar_features: Tensor,  # [C, N, channels] or [nnz, channels]; last channel = range
+    opacities: Tensor,  # [C, N] or [nnz]
+    pix_vels: Tensor,  # [C, N, 3] or [nnz, 3]
+    depth_compensations: Tensor,  # [C, N, 2] or [nnz, 2]
+    raster_pts: Tensor,  # [C, H, W, 4] = (azimuth, elevation, range, time)
+    image_width: int,
+    image_height: int,
+    tile_width: int,
+    tile_height: int,
+    isect_offsets: Tensor,  # [C, tile_grid_height, tile_grid_width]
+    flatten_ids: Tensor,  # [n_isects]
+    compute_alpha_sum_until_points: bool,
+    compute_alpha_sum_until_points_threshold: float,
+    backgrounds: Optional[Tensor] = None,  # [C, channels]
+    packed: bool = False,
+    absgrad: bool = False,
+) -> Tuple[Tensor, Tensor, Optional[Tensor], Tensor]:
+    """Alpha compositing onto a grid of lidar points given in spherical coordinates; the last
+    feature channel is the Gaussian's range and receives the depth-compensation and range-rate
+    terms.  Points with range <= 0 are skipped (zeros).
+
+    Returns (render_features[C,H,W,channels], render_alphas[C,H,W,1],
+    alpha_sum_until_points[C,H,W,1] | None, median_depths[C,H,W,1]).
+    """
+    C = isect_offsets.size(0)
+    if packed:
+        nnz = means2d.size(0)
+        assert means2d.shape == (nnz, 2), means2d.shape
+        assert conics.shape == (nnz, 3), conics.shape
+        assert lidar_features.shape[0] == nnz, lidar_features.shape
+        assert opacities.shape == (nnz,), opacities.shape
+        assert pix_vels.shape == (nnz, 3), pix_vels.shape
+        assert depth_compensations.shape == (nnz, 2), depth_compensations.shape
+    else:
+        N = means2d.size(1)
+        assert means2d.shape == (C, N, 2), means2d.shape
+        assert conics.shape == (C, N, 3), conics.shape
+        assert lidar_features.shape[:2] == (C, N), lidar_features.shape
+        assert opacities.shape == (C, N), opacities.shape
+        assert pix_vels.shape == (C, N, 3), pix_vels.shape
+        assert depth_compensations.shape == (C, N, 2), depth_compensations.shape
+    if backgrounds is not None:
+        assert backgrounds.shape == (C, lidar_features.shape[-1]), backgrounds.shape
+        backgrounds = backgrounds.contiguous()
+    channels = lidar_features.shape[-1]
+    depth_channel_idx = channels - 1
+    if channels > MAX_CHANNELS or channels == 0:
+        raise ValueError(f"Unsupported number of lidar_features channels: {channels}")
+    tile_grid_height, tile_grid_width = isect_offsets.shape[1:3]
+    assert tile_grid_height * tile_height >= image_height, f"Assert Failed: {tile_grid_height} * {tile_height} >= {image_height}"
+    assert tile_grid_width * tile_width >= image_width, f"Assert Failed: {tile_grid_width} * {tile_width} >= {image_width}"
+    assert raster_pts.shape == (C, image_height, image_width, 4), "raster_pts does not have the correct shape"
+
+    return _RasterizeToPoints.apply(
+        means2d.contiguous(), conics.contiguous(), lidar_features.contiguous(),
+        opacities.contiguous(), pix_vels.contiguous(), depth_compensations.contiguous(),
+        backgrounds, raster_pts.contiguous(), image_width, image_height, tile_width, tile_height,
+        isect_offsets.contiguous(), flatten_ids.contiguous(), compute_alpha_sum_until_points,
+        compute_alpha_sum_until_points_threshold, absgrad, depth_channel_idx,
+    )
+
+
+# ---------------------------------------------------------------------------------------------
+# autograd pairing of the forward and backward kernels
+# ---------------------------------------------------------------------------------------------
+def _gate(grads, needs):
+    return tuple(g if n else None for g, n in zip(grads, needs))
+
+
+class _FullyFusedProjection(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, means, covars, quats, scales, velocities, viewmats, Ks, width, height,
+                linear_velocity, angular_velocity, rolling_shutter_time, eps2d, near_plane,
+                far_plane, radius_clip, calc_compensations):
+        radii, means2d, depths, conics, compensations, pix_vels = _make_lazy_hip_func(
+            "fully_fused_projection_fwd"
+        )(means, covars, quats, scales, velocities, viewmats, Ks, width, height, linear_velocity,
+          angular_velocity, rolling_shutter_time, eps2d, near_plane, far_plane, radius_clip,
+          calc_compensations)
+        if not calc_compensations:
+            compensations = None
+        ctx.save_for_backward(means, covars, quats, scales, velocities, viewmats, Ks,
+                              linear_velocity, angular_velocity, rolling_shutter_time, radii,
+                              conics, compensations)
+        ctx.width, ctx.height, ctx.eps2d = width, height, eps2d
+        ctx.mark_non_differentiable(radii)
+        return radii, means2d, depths, conics, compensations, pix_vels
+
+    @staticmethod
+    def backward(ctx, v_radii, v_means2d, v_depths, v_conics, v_compensations, v_pix_vels):
+        (means, covars, quats, scales, velocities, viewmats, Ks, linear_velocity,
+         angular_velocity, rolling_shutter_time, radii, conics, compensations) = ctx.saved_tensors
+        want_vel = velocities is not None and ctx.needs_input_grad[4]
+        out = _make_lazy_hip_func("fully_fused_projection_bwd")(
+            means, covars, quats, scales, velocities, viewmats, Ks, ctx.width, ctx.height,
+            linear_velocity, angular_velocity, rolling_shutter_time, ctx.eps2d, radii, conics,
+            compensations, v_means2d.contiguous(), v_depths.contiguous(), v_conics.contiguous(),
+            _c(v_compensations), v_pix_vels.contiguous(), ctx.needs_input_grad[5], want_vel)
+        v_means, v_covars, v_quats, v_scales, v_viewmats = out[:5]
+        v_velocities = out[5] if want_vel else None
+        grads = _gate((v_means, v_covars, v_quats, v_scales, v_velocities, v_viewmats),
+                      ctx.needs_input_grad[:6])
+        return grads + (None,) * 11
+
+
+class _FullyFusedLidarProjection(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, means, covars, quats, scales, velocities, viewmats, min_elevation,
+                max_elevation, min_azimuth, max_azimuth, linear_velocity, angular_velocity,
+                rolling_shutter_time, eps2d, near_plane, far_plane, radius_clip,
+                calc_compensations):
+        (radii, means2d, depths, conics, compensations, pix_vels,
+         depth_compensations) = _make_lazy_hip_func("fully_fused_lidar_projection_fwd")(
+            means, covars, quats, scales, velocities, viewmats, min_elevation, max_elevation,
+            min_azimuth, max_azimuth, linear_velocity, angular_velocity, rolling_shutter_time,
+            eps2d, near_plane, far_plane, radius_clip, calc_compensations)
+        if not calc_compensations:
+            compensations = None
+        ctx.save_for_backward(means, covars, quats, scales, velocities, viewmats,
+                              linear_velocity, angular_velocity, rolling_shutter_time, radii,
+                              conics, compensations)
+        ctx.bounds = (min_elevation, max_elevation, min_azimuth, max_azimuth)
+        ctx.eps2d = eps2d
+        ctx.mark_non_differentiable(radii)
+        return radii, means2d, depths, conics, compensations, pix_vels, depth_compensations
+
+    @staticmethod
+    def backward(ctx, v_radii, v_means2d, v_depths, v_conics, v_compensations, v_pix_vels,
+                 v_depth_compensations):
+        (means, covars, quats, scales, velocities, viewmats, linear_velocity, angular_velocity,
+         rolling_shutter_time, radii, conics, compensations) = ctx.saved_tensors
+        want_vel = velocities is not None and ctx.needs_input_grad[4]
+        out = _make_lazy_hip_func("fully_fused_lidar_projection_bwd")(
+            means, covars, quats, scales, velocities, viewmats, *ctx.bounds, linear_velocity,
+            angular_velocity, rolling_shutter_time, ctx.eps2d, radii, conics, compensations,
+            v_means2d.contiguous(), v_depths.contiguous(), v_conics.contiguous(),
+            _c(v_compensations), v_pix_vels.contiguous(), v_depth_compensations.contiguous(),
+            ctx.needs_input_grad[5], want_vel)
+        v_means, v_covars, v_quats, v_scales, v_viewmats = out[:5]
+        v_velocities = out[5] if want_vel else None
+        grads = _gate((v_means, v_covars, v_quats, v_scales, v_velocities, v_viewmats),
+                      ctx.needs_input_grad[:6])
+        return grads + (None,) * 12
+
+
+class _FullyFusedProjectionPacked(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, means, covars, quats, scales, velocities, viewmats, Ks, width, height,
+                linear_velocity, angular_velocity, rolling_shutter_time, eps2d, near_plane,
+                far_plane, radius_clip, sparse_grad, calc_compensations):
+        (indptr, camera_ids, gaussian_ids, radii, means2d, depths, conics, compensations,
+         pix_vels) = _make_lazy_hip_func("fully_fused_projection_packed_fwd")(
+            means, covars, quats, scales, velocities, viewmats, Ks, width, height,
+            linear_velocity, angular_velocity, rolling_shutter_time, eps2d, near_plane, far_plane,
+            radius_clip, calc_compensations)
+        if not calc_compensations:
+            compensations = None
+        ctx.save_for_backward(camera_ids, gaussian_ids, means, covars, quats, scales, velocities,
+                              viewmats, Ks, linear_velocity, angular_velocity,
+                              rolling_shutter_time, conics, compensations, pix_vels)
+        ctx.width, ctx.height, ctx.eps2d, ctx.sparse_grad = width, height, eps2d, sparse_grad
+        ctx.mark_non_differentiable(camera_ids, gaussian_ids, radii)
+        return camera_ids, gaussian_ids, radii, means2d, depths, conics, compensations, pix_vels
+
+    @staticmethod
+    def backward(ctx, v_camera_ids, v_gaussian_ids, v_radii, v_means2d, v_depths, v_conics,
+                 v_compensations, v_pix_vels):
+        (camera_ids, gaussian_ids, means, covars, quats, scales, velocities, viewmats, Ks,
+         linear_velocity, angular_velocity, rolling_shutter_time, conics, compensations,
+         pix_vels) = ctx.saved_tensors
+        sparse_grad = ctx.sparse_grad
+        want_vel = velocities is not None and ctx.needs_input_grad[4]
+        out = _make_lazy_hip_func("fully_fused_projection_packed_bwd")(
+            means, covars, quats, scales, velocities, viewmats, Ks, ctx.width, ctx.height,
+            linear_velocity, angular_velocity, rolling_shutter_time, ctx.eps2d, camera_ids,
+            gaussian_ids, conics, compensations, pix_vels, v_means2d.contiguous(),
+            v_depths.contiguous(), v_conics.contiguous(), _c(v_compensations),
+            v_pix_vels.contiguous(), ctx.needs_input_grad[5], sparse_grad, want_vel)
+        v_means, v_covars, v_quats, v_scales, v_viewmats = out[:5]
+        v_velocities = out[5] if want_vel else None
+
+        def coo(values, like):
+            # rows of `values` belong to gaussian_ids; duplicates (several cameras) are summed
+            # by the sparse tensor's consumer
+            return torch.sparse_coo_tensor(indices=gaussian_ids[None], values=values, size=like.size())
+
+        if sparse_grad:
+            if ctx.needs_input_grad[0]:
+                v_means = coo(v_means, means)
+            if covars is not None and ctx.needs_input_grad[1]:
+                v_covars = coo(v_covars, covars)
+            if quats is not None and ctx.needs_input_grad[2]:
+                v_quats = coo(v_quats, quats)
+            if scales is not None and ctx.needs_input_grad[3]:
+                v_scales = coo(v_scales, scales)
+        grads = _gate((v_means, v_covars, v_quats, v_scales, v_velocities, v_viewmats),
+                      ctx.needs_input_grad[:6])
+        return grads + (None,) * 12
+
+
+class _RasterizeToPixels(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, means2d, conics, colors, opacities, pix_vels, rolling_shutter_time,
+                backgrounds, width, height, tile_size, isect_offsets, flatten_ids, absgrad):
+        render_colors, render_alphas, last_ids = _make_lazy_hip_func("rasterize_to_pixels_fwd")(
+            means2d, conics, colors, opacities, pix_vels, rolling_shutter_time, backgrounds, width,
+            height, tile_size, isect_offsets, flatten_ids)
+        ctx.save_for_backward(means2d, conics, colors, opacities, pix_vels, rolling_shutter_time,
+                              backgrounds, isect_offsets, flatten_ids, render_alphas, last_ids)
+        ctx.width, ctx.height, ctx.tile_size, ctx.absgrad = width, height, tile_size, absgrad
+        return render_colors, render_alphas.float()
+
+    @staticmethod
+    def backward(ctx, v_render_colors, v_render_alphas):
+        (means2d, conics, colors, opacities, pix_vels, rolling_shutter_time, backgrounds,
+         isect_offsets, flatten_ids, render_alphas, last_ids) = ctx.saved_tensors
+        (v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities,
+         v_pix_vels) = _make_lazy_hip_func("rasterize_to_pixels_bwd")(
+            means2d, conics, colors, opacities, pix_vels, rolling_shutter_time, backgrounds,
+            ctx.width, ctx.height, ctx.tile_size, isect_offsets, flatten_ids, render_alphas,
+            last_ids, v_render_colors.contiguous(), v_render_alphas.contiguous(), ctx.absgrad)
+        if ctx.absgrad:
+            means2d.absgrad = v_means2d_abs
+        v_backgrounds = None
+        if ctx.needs_input_grad[6]:
+            v_backgrounds = (v_render_colors * (1.0 - render_alphas).float()).sum(dim=(1, 2))
+        return (v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, None, v_backgrounds,
+                None, None, None, None, None, None)
+
+
+class _RasterizeToPoints(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, means2d, conics, colors, opacities, pix_vels, depth_compensations,
+                backgrounds, raster_pts, width, height, tile_width, tile_height, isect_offsets,
+                flatten_ids, compute_alpha_sum_until_points,
+                compute_alpha_sum_until_points_threshold, absgrad, depth_channel_idx):
+        (render_colors, render_alphas, last_ids, alpha_sum_until_points,
+         median_depths) = _make_lazy_hip_func("rasterize_to_points_fwd")(
+            means2d, conics, colors, opacities, pix_vels, depth_compensations, backgrounds,
+            raster_pts, width, height, tile_width, tile_height, compute_alpha_sum_until_points,
+            compute_alpha_sum_until_points_threshold, isect_offsets, flatten_ids,
+            depth_channel_idx)
+        ctx.save_for_backward(means2d, conics, colors, opacities, pix_vels, depth_compensations,
+                              backgrounds, raster_pts, isect_offsets, flatten_ids, render_alphas,
+                              last_ids)
+        ctx.geom = (width, height, tile_width, tile_height)
+        ctx.absgrad = absgrad
+        ctx.alpha_sum = (compute_alpha_sum_until_points, compute_alpha_sum_until_points_threshold)
+        ctx.depth_channel_idx = depth_channel_idx
+        ctx.mark_non_differentiable(median_depths)
+        alpha_sum_until_points = (
+            alpha_sum_until_points.float() if compute_alpha_sum_until_points else None
+        )
+        return render_colors, render_alphas.float(), alpha_sum_until_points, median_depths
+
+    @staticmethod
+    def backward(ctx, v_render_colors, v_render_alphas, v_alpha_sum_until_points, v_median_depths):
+        (means2d, conics, colors, opacities, pix_vels, depth_compensations, backgrounds,
+         raster_pts, isect_offsets, flatten_ids, render_alphas, last_ids) = ctx.saved_tensors
+        compute_sum, threshold = ctx.alpha_sum
+        if compute_sum and v_alpha_sum_until_points is not None:
+            v_sum = v_alpha_sum_until_points.contiguous()
+        else:
+            v_sum = torch.zeros_like(v_render_alphas)
+        (v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities, v_pix_vels,
+         v_depth_compensations) = _make_lazy_hip_func("rasterize_to_points_bwd")(
+            means2d, conics, colors, opacities, pix_vels, depth_compensations, backgrounds,
+            raster_pts, *ctx.geom, isect_offsets, flatten_ids, render_alphas, last_ids,
+            v_render_colors.contiguous(), v_render_alphas.contiguous(), v_sum, ctx.absgrad,
+            compute_sum, threshold, ctx.depth_channel_idx)
+        if ctx.absgrad:
+            means2d.absgrad = v_means2d_abs
+        v_backgrounds = None
+        if ctx.needs_input_grad[6]:
+            v_backgrounds = (v_render_colors * (1.0 - render_alphas).float()).sum(dim=(1, 2))
+        return (v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_depth_compensations,
+                v_backgrounds) + (None,) * 11
+
+
+class _SphericalHarmonics(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, sh_degree, dirs, coeffs, masks):
+        colors = _make_lazy_hip_func("compute_sh_fwd")(sh_degree, dirs, coeffs, masks)
+        ctx.save_for_backward(dirs, coeffs, masks)
+        ctx.sh_degree = sh_degree
+        ctx.num_bases = coeffs.shape[-2]
+        return colors
+
+    @staticmethod
+    def backward(ctx, v_colors):
+        dirs, coeffs, masks = ctx.saved_tensors
+        compute_v_dirs = ctx.needs_input_grad[1]
+        v_coeffs, v_dirs = _make_lazy_hip_func("compute_sh_bwd")(
+            ctx.num_bases, ctx.sh_degree, dirs, coeffs, masks, v_colors.contiguous(),
+            compute_v_dirs)
+        return None, (v_dirs if compute_v_dirs else None), v_coeffs, None

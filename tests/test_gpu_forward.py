@@ -1,0 +1,379 @@
+"""GPU parity of the forward operators against the CPU oracle (same seeded inputs).
+
+Bars: tile intersection lists, sort order and offsets bit-exact; projected and rendered
+floats within 1e-4 (absolute, plus 1e-4 relative where values reach hundreds of pixels);
+radii exact up to the truncation of a float that differs in its last bits (|diff| <= 1 on
+<0.1% of rows).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from tests.gpu_util import DEV, assert_close, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _gaussians(n, seed, spread=2.0, log_scale=-3.0):
+    rng = np.random.default_rng(seed)
+    means = (rng.uniform(-1, 1, (n, 3)) * spread).astype(np.float32)
+    quats = rng.normal(size=(n, 4)).astype(np.float32)
+    scales = np.exp(rng.normal(size=(n, 3)) * 0.5 + log_scale).astype(np.float32)
+    vel = rng.normal(size=(n, 3)).astype(np.float32)
+    return rng, means, quats, scales, vel
+
+
+def _cameras(rng, C, W, H, f=300.0):
+    from scipy.spatial.transform import Rotation
+    vms, Ks = [], []
+    for _ in range(C):
+        vm = np.eye(4)
+        vm[:3, :3] = Rotation.from_rotvec(rng.normal(size=3) * 0.3).as_matrix()
+        vm[:3, 3] = [rng.normal() * 0.2, rng.normal() * 0.2, 3.0]
+        vms.append(vm)
+        Ks.append([[f, 0, W / 2 + 1.5], [0, f * 0.97, H / 2 - 2.0], [0, 0, 1]])
+    return np.array(vms, np.float32), np.array(Ks, np.float32)
+
+
+def _covars6(quats, scales):
+    from scipy.spatial.transform import Rotation
+    R = Rotation.from_quat(quats[:, [1, 2, 3, 0]].astype(np.float64)).as_matrix()
+    cov = np.einsum("nij,nj,nkj->nik", R, scales.astype(np.float64) ** 2, R)
+    return cov.reshape(-1, 9)[:, [0, 1, 2, 4, 5, 8]].astype(np.float32)
+
+
+def _check_projection(out, ref32, ref64, lidar=False):
+    radii = to_np(out[0])
+    valid = (radii[..., 0] > 0) & (ref32[0][..., 0] > 0) & (ref64[0][..., 0] > 0)
+    # the same Gaussians survive the culls (boundary cases may flip with the last float bit)
+    agree = ((radii[..., 0] > 0) == (ref32[0][..., 0] > 0)).mean()
+    assert agree > 0.999, agree
+    assert valid.sum() > 100
+    if lidar:
+        assert_close(radii[valid], ref64[0][valid], atol=1e-4, rtol=1e-4, name="radii")
+    else:
+        d = np.abs(radii[valid].astype(np.int64) - ref32[0][valid])
+        assert d.max() <= 1 and (d > 0).mean() < 1e-3, (d.max(), (d > 0).mean())
+    names = ["means2d", "depths", "conics", "compensations", "pix_vels", "depth_compensations"]
+    for k, name in enumerate(names[: len(out) - 1], start=1):
+        if out[k] is None:
+            assert ref64[k] is None
+            continue
+        got = to_np(out[k])
+        assert_close(got[valid], ref64[k][valid], atol=1e-4, rtol=1e-4, name=name)
+        assert (got[radii[..., 0] <= 0] == 0).all(), f"{name}: culled rows must be zero"
+
+
+@pytest.mark.parametrize("use_covars", [False, True])
+@pytest.mark.parametrize("use_vel", [False, True])
+@pytest.mark.parametrize("comp", [False, True])
+def test_projection_camera(use_covars, use_vel, comp):
+    from splatad_amd import fully_fused_projection
+    C, N, W, H = 3, 20000, 320, 240
+    rng, means, quats, scales, vel = _gaussians(N, 10)
+    viewmats, Ks = _cameras(rng, C, W, H)
+    lin = rng.normal(size=(C, 3)).astype(np.float32)
+    ang = (rng.normal(size=(C, 3)) * 0.3).astype(np.float32)
+    rs = np.array([0.03, 0.0, 0.01], np.float32)
+    covars = _covars6(quats, scales) if use_covars else None
+    kw = dict(eps2d=0.3, near_plane=0.5, far_plane=4.5, radius_clip=0.5, calc_compensations=comp)
+    args = (means, covars, None if use_covars else quats, None if use_covars else scales,
+            vel if use_vel else None, viewmats, Ks, W, H, lin, ang, rs)
+    ref32 = oracle.projection_fwd(*args, precision="f32", **kw)
+    ref64 = oracle.projection_fwd(*args, precision="f64", **kw)
+    t = [to_dev(a) if isinstance(a, np.ndarray) else a for a in args]
+    out = fully_fused_projection(*t, packed=False, **kw)
+    _check_projection(out, ref32, ref64)
+
+    # packed == compacted unpacked, in (camera, gaussian) order
+    pk = fully_fused_projection(*t, packed=True, **kw)
+    cam, gid = to_np(pk[0]), to_np(pk[1])
+    radii = to_np(out[0])
+    sel = np.argwhere(radii[..., 0] > 0)
+    np.testing.assert_array_equal(cam, sel[:, 0])
+    np.testing.assert_array_equal(gid, sel[:, 1])
+    assert pk[0].dtype == torch.int64 and pk[1].dtype == torch.int64
+    for a, b in zip(pk[2:], out):
+        if b is None:
+            assert a is None
+        else:
+            np.testing.assert_array_equal(to_np(a), to_np(b)[sel[:, 0], sel[:, 1]])
+
+
+@pytest.mark.parametrize("use_covars", [False, True])
+@pytest.mark.parametrize("use_vel", [False, True])
+def test_projection_lidar(use_covars, use_vel):
+    from splatad_amd import fully_fused_lidar_projection
+    from scipy.spatial.transform import Rotation
+    C, N = 2, 20000
+    rng, means, quats, scales, vel = _gaussians(N, 11, spread=30.0, log_scale=-1.5)
+    means[:, 2] *= 0.15
+    vms = []
+    for _ in range(C):
+        vm = np.eye(4)
+        vm[:3, :3] = Rotation.from_rotvec(rng.normal(size=3) * 0.1).as_matrix()
+        vm[:3, 3] = rng.normal(size=3)
+        vms.append(vm)
+    viewmats = np.array(vms, np.float32)
+    lin = (rng.normal(size=(C, 3)) * 5).astype(np.float32)
+    ang = (rng.normal(size=(C, 3)) * 0.2).astype(np.float32)
+    rs = np.array([0.1, 0.0], np.float32)
+    covars = _covars6(quats, scales) if use_covars else None
+    kw = dict(eps2d=0.017, near_plane=1.0, far_plane=40.0, radius_clip=0.05, calc_compensations=True)
+    args = (means, covars, None if use_covars else quats, None if use_covars else scales,
+            vel if use_vel else None, viewmats, -20.0, 15.0, -170.0, 175.0, lin, ang, rs)
+    ref32 = oracle.lidar_projection_fwd(*args, precision="f32", **kw)
+    ref64 = oracle.lidar_projection_fwd(*args, precision="f64", **kw)
+    t = [to_dev(a) if isinstance(a, np.ndarray) else a for a in args]
+    # API order: (..., viewmats, lin, ang, rs, min_el, max_el, min_az, max_az)
+    out = fully_fused_lidar_projection(t[0], t[1], t[2], t[3], t[4], t[5], t[10], t[11], t[12],
+                                       t[6], t[7], t[8], t[9], **kw)
+    _check_projection(out, ref32, ref64, lidar=True)
+
+
+def test_isect_camera_reference_recipe():
+    # input recipe of the reference's test_isect (tests/test_basic.py:704-712)
+    from splatad_amd import isect_offset_encode, isect_tiles
+    rng = np.random.default_rng(42)
+    C, N, W, H, ts = 3, 1000, 40, 60, 16
+    tw, th = math.ceil(W / ts), math.ceil(H / ts)
+    means2d = (rng.normal(size=(C, N, 2)) * W).astype(np.float32)
+    radii = rng.integers(0, W, (C, N, 2)).astype(np.int32)
+    depths = rng.random((C, N)).astype(np.float32)
+    for sort in (True, False):
+        tpg, ids, flat = isect_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), ts, tw, th, sort=sort)
+        o_tpg, o_ids, o_flat = oracle.isect_tiles(means2d, radii, depths, ts, tw, th, sort=sort)
+        np.testing.assert_array_equal(to_np(tpg), o_tpg)
+        np.testing.assert_array_equal(to_np(ids), o_ids)
+        np.testing.assert_array_equal(to_np(flat), o_flat)
+        assert ids.dtype == torch.int64 and flat.dtype == torch.int32 and tpg.dtype == torch.int32
+    offs = isect_offset_encode(ids if sort else to_dev(o_ids), C, tw, th)
+    tpg, ids, flat = isect_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), ts, tw, th)
+    offs = isect_offset_encode(ids, C, tw, th)
+    np.testing.assert_array_equal(to_np(offs), oracle.isect_offset_encode(to_np(ids), C, tw, th))
+
+
+@pytest.mark.parametrize("n,C,W,H,ts,rmax", [(200000, 2, 640, 480, 16, 40), (3000, 1, 64, 64, 16, 600),
+                                              (50000, 4, 200, 120, 8, 12), (0, 1, 64, 64, 16, 5)])
+def test_isect_camera_sizes_and_packed(n, C, W, H, ts, rmax):
+    from splatad_amd import isect_offset_encode, isect_tiles
+    rng = np.random.default_rng(n + C)
+    tw, th = math.ceil(W / ts), math.ceil(H / ts)
+    means2d = np.stack([rng.uniform(-20, W + 20, (C, n)), rng.uniform(-20, H + 20, (C, n))], -1).astype(np.float32)
+    radii = rng.integers(0, rmax, (C, n, 2)).astype(np.int32)
+    depths = rng.uniform(0.01, 100, (C, n)).astype(np.float32)
+    depths[:, : n // 10] = 7.5   # many exact depth ties: order must follow the flatten id
+    tpg, ids, flat = isect_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), ts, tw, th)
+    o_tpg, o_ids, o_flat = oracle.isect_tiles(means2d, radii, depths, ts, tw, th)
+    np.testing.assert_array_equal(to_np(tpg), o_tpg)
+    np.testing.assert_array_equal(to_np(ids), o_ids)
+    np.testing.assert_array_equal(to_np(flat), o_flat)
+    offs = isect_offset_encode(ids, C, tw, th)
+    np.testing.assert_array_equal(to_np(offs), oracle.isect_offset_encode(o_ids, C, tw, th))
+    if n == 0:
+        return
+    # packed input gives the same keys; ids index the packed rows
+    sel = np.nonzero(radii[..., 0].reshape(-1) > 0)[0]
+    cam_ids = (sel // n).astype(np.int64)
+    tpg_p, ids_p, flat_p = isect_tiles(
+        to_dev(means2d.reshape(-1, 2)[sel]), to_dev(radii.reshape(-1, 2)[sel]),
+        to_dev(depths.reshape(-1)[sel]), ts, tw, th, packed=True, n_cameras=C,
+        camera_ids=to_dev(cam_ids), gaussian_ids=to_dev((sel % n).astype(np.int64)))
+    np.testing.assert_array_equal(to_np(ids_p), o_ids)
+    np.testing.assert_array_equal(sel[to_np(flat_p)], o_flat)
+
+
+def test_isect_lidar_reference_recipe_and_wrap():
+    # input recipe of the reference's test_isect_lidar (tests/test_basic.py:733-751)
+    from splatad_amd import isect_lidar_tiles, isect_offset_encode
+    rng = np.random.default_rng(42)
+    C, N = 3, 100
+    res, min_az = 0.2 * 16, -180.0
+    n_az = math.ceil(360 / res)
+    eb = np.linspace(-45.0, 45.0, 17).astype(np.float32)
+    means2d = np.zeros((C, N, 2), np.float32)
+    means2d[..., 0] = rng.random((C, N)) * 360 - 180
+    means2d[..., 1] = rng.random((C, N)) * 90 - 45
+    radii = (rng.random((C, N, 2)) / 2).astype(np.float32)
+    depths = rng.random((C, N)).astype(np.float32)
+    means2d[0, 0] = [-179.9, 0.0]; radii[0, 0] = [0.4, 0.3]
+    means2d[0, 1] = [179.8, 10.0]; radii[0, 1] = [0.45, 0.2]
+    for sort in (True, False):
+        tpg, ids, flat = isect_lidar_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), to_dev(eb),
+                                           res, min_az, sort=sort)
+        o = oracle.isect_lidar_tiles(means2d, radii, depths, eb, res, min_az, sort=sort)
+        np.testing.assert_array_equal(to_np(tpg), o[0])
+        np.testing.assert_array_equal(to_np(ids), o[1])
+        np.testing.assert_array_equal(to_np(flat), o[2])
+    tpg, ids, flat = isect_lidar_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), to_dev(eb), res, min_az)
+    offs = isect_offset_encode(ids, C, n_az, 16)
+    np.testing.assert_array_equal(to_np(offs), oracle.isect_offset_encode(to_np(ids), C, n_az, 16))
+
+
+def test_isect_lidar_large_nonuniform():
+    from splatad_amd import isect_lidar_tiles
+    from splatad_amd import workloads
+    rng = np.random.default_rng(5)
+    C, N = 2, 100000
+    elev = workloads.lidar_beam_elevations(128)
+    eb = workloads.lidar_tile_elevation_boundaries(elev, 4).numpy()
+    res, min_az = 360.0 / 2048 * 64, -180.0
+    means2d = np.stack([rng.uniform(-180, 180, (C, N)), rng.uniform(-30, 20, (C, N))], -1).astype(np.float32)
+    radii = (rng.exponential(1.5, (C, N, 2))).astype(np.float32)
+    radii[rng.random((C, N)) < 0.2] = 0
+    depths = rng.uniform(0.5, 80, (C, N)).astype(np.float32)
+    tpg, ids, flat = isect_lidar_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), to_dev(eb), res, min_az)
+    o = oracle.isect_lidar_tiles(means2d, radii, depths, eb, res, min_az)
+    np.testing.assert_array_equal(to_np(tpg), o[0])
+    np.testing.assert_array_equal(to_np(ids), o[1])
+    np.testing.assert_array_equal(to_np(flat), o[2])
+
+
+def _projected_scene(C, N, W, H, D, seed, rs=(0.02, 0.0)):
+    from splatad_amd import fully_fused_projection
+    rng, means, quats, scales, vel = _gaussians(N, seed, log_scale=-2.6)
+    viewmats, Ks = _cameras(rng, C, W, H, f=0.9 * W)
+    lin = rng.normal(size=(C, 3)).astype(np.float32)
+    ang = (rng.normal(size=(C, 3)) * 0.3).astype(np.float32)
+    rs = np.array(rs[:C], np.float32)
+    radii, means2d, depths, conics, _, pix_vels = fully_fused_projection(
+        to_dev(means), None, to_dev(quats), to_dev(scales), to_dev(vel), to_dev(viewmats), to_dev(Ks),
+        W, H, to_dev(lin), to_dev(ang), to_dev(rs))
+    colors = rng.normal(size=(C, N, D)).astype(np.float32)
+    opac = rng.uniform(0.05, 1.0, (C, N)).astype(np.float32)
+    bg = rng.uniform(size=(C, D)).astype(np.float32)
+    return dict(radii=radii, means2d=means2d, depths=depths, conics=conics, pix_vels=pix_vels,
+                colors=to_dev(colors), opacities=to_dev(opac), backgrounds=to_dev(bg), rs=to_dev(rs))
+
+
+@pytest.mark.parametrize("D,ts", [(3, 16), (4, 16), (1, 16), (32, 16), (33, 16), (7, 8), (64, 4), (70, 16)])
+def test_rasterize_to_pixels(D, ts):
+    from splatad_amd import isect_offset_encode, isect_tiles, rasterize_to_pixels
+    C, N, W, H = 2, 2500, 200, 136
+    s = _projected_scene(C, N, W, H, D, seed=20 + D)
+    tw, th = math.ceil(W / ts), math.ceil(H / ts)
+    _, ids, flat = isect_tiles(s["means2d"], s["radii"], s["depths"], ts, tw, th)
+    offs = isect_offset_encode(ids, C, tw, th)
+    for bg in (s["backgrounds"], None):
+        rc, ra = rasterize_to_pixels(s["means2d"], s["conics"], s["colors"], s["opacities"],
+                                     s["pix_vels"], W, H, ts, offs, flat,
+                                     rolling_shutter_time=s["rs"], backgrounds=bg)
+        o_rc, o_ra, _ = oracle.rasterize_to_pixels_fwd(
+            to_np(s["means2d"]), to_np(s["conics"]), to_np(s["colors"]), to_np(s["opacities"]),
+            to_np(s["pix_vels"]), to_np(s["rs"]), to_np(bg), W, H, ts, to_np(offs), to_np(flat),
+            precision="f64")
+        assert rc.shape == (C, H, W, D) and ra.shape == (C, H, W, 1)
+        assert_close(to_np(rc), o_rc, atol=1e-4, name=f"colors D={D}")
+        assert_close(to_np(ra), o_ra, atol=1e-4, name="alphas")
+    lo, hi = float(ra.min()), float(ra.max())
+    assert hi > 0.9 and lo < 0.9, (lo, hi)
+
+
+def test_rasterize_to_pixels_last_ids_and_termination():
+    # dense, opaque scene so that most pixels terminate early
+    from splatad_amd.hip._backend import _C
+    from splatad_amd import isect_offset_encode, isect_tiles
+    C, N, W, H, D, ts = 1, 30000, 96, 64, 3, 16
+    s = _projected_scene(C, N, W, H, D, seed=3, rs=(0.0,))
+    s["opacities"] = torch.full_like(s["opacities"], 0.95)
+    tw, th = math.ceil(W / ts), math.ceil(H / ts)
+    _, ids, flat = isect_tiles(s["means2d"], s["radii"], s["depths"], ts, tw, th)
+    offs = isect_offset_encode(ids, C, tw, th)
+    rc, ra, last = _C.rasterize_to_pixels_fwd(s["means2d"], s["conics"], s["colors"], s["opacities"],
+                                             s["pix_vels"], s["rs"], None, W, H, ts, offs, flat)
+    o_rc, o_ra, o_last = oracle.rasterize_to_pixels_fwd(
+        to_np(s["means2d"]), to_np(s["conics"]), to_np(s["colors"]), to_np(s["opacities"]),
+        to_np(s["pix_vels"]), to_np(s["rs"]), None, W, H, ts, to_np(offs), to_np(flat), precision="f32")
+    assert_close(to_np(rc), o_rc, atol=1e-4, name="colors")
+    assert (to_np(last) == o_last).mean() > 0.999
+    assert (o_ra > 0.9998).mean() > 0.5   # the scene really saturates
+
+
+def _lidar_scene(N, seed, H=16, W=256, tw=32, th=4, D=5, C=1):
+    from splatad_amd import fully_fused_lidar_projection
+    from splatad_amd import workloads
+    l = workloads.lidar_sweep(n=N, seed=seed, n_beams=H, n_azimuth=W, feature_dim=D - 1,
+                              tile_width=tw, tile_height=th, with_velocities=True)
+    l["scales"] = l["scales"] * 3.0
+    rng = np.random.default_rng(seed)
+    rp = l["raster_pts"].numpy().copy()
+    rp[..., 2] = rng.uniform(2, 60, rp.shape[:-1])
+    rp[..., :2] += rng.normal(size=rp[..., :2].shape).astype(np.float32) * 0.01
+    rp[0, 0, :7, 2] = 0.0
+    rp[0, 3, 5, 2] = -1.0
+    l["raster_pts"] = torch.from_numpy(rp)
+    l["angular_velocity"] = torch.tensor([[0.0, 0.05, 0.3]])
+    d = workloads.to_device(l, DEV)
+    proj = fully_fused_lidar_projection(
+        d["means"], None, d["quats"], d["scales"], d["velocities"], d["viewmats"],
+        d["linear_velocity"], d["angular_velocity"], d["rolling_shutter_time"],
+        d["min_elevation"], d["max_elevation"], d["min_azimuth"], d["max_azimuth"], eps2d=0.017)
+    return d, proj
+
+
+@pytest.mark.parametrize("D,asum", [(5, True), (5, False), (33, True), (2, True), (40, True)])
+def test_rasterize_to_points(D, asum):
+    from splatad_amd import isect_lidar_tiles, isect_offset_encode, rasterize_to_points
+    H, W, tw, th = 16, 256, 32, 4
+    d, proj = _lidar_scene(8000, 30 + D, H, W, tw, th, D)
+    radii, means2d, depths, conics, _, pix_vels, dcomp = proj
+    res = d["azimuth_resolution"] * tw
+    _, ids, flat = isect_lidar_tiles(means2d, radii, depths, d["tile_elevation_boundaries"], res, -180.0)
+    offs = isect_offset_encode(ids, 1, W // tw, H // th)
+    feats = torch.cat([d["lidar_features"], depths[..., None]], -1)
+    opac = d["opacities"][None].contiguous()
+    rf, ra, rsum, med = rasterize_to_points(means2d, conics, feats, opac, pix_vels, dcomp,
+                                            d["raster_pts"], W, H, tw, th, offs, flat, asum, 0.3)
+    o = oracle.rasterize_to_points_fwd(
+        to_np(means2d), to_np(conics), to_np(feats), to_np(opac), to_np(pix_vels), to_np(dcomp),
+        None, to_np(d["raster_pts"]), W, H, tw, th, asum, 0.3, to_np(offs), to_np(flat), D - 1,
+        precision="f64")
+    assert_close(to_np(rf), o[0], atol=2e-4, rtol=1e-4, name="features")
+    assert_close(to_np(ra), o[1], atol=1e-4, name="alphas")
+    if asum:
+        assert_close(to_np(rsum), o[3], atol=1e-4, rtol=1e-4, name="alpha_sum")
+    else:
+        assert rsum is None
+    # the median switches Gaussians where T crosses 0.5 within float error: allow rare flips
+    assert_close(to_np(med), o[4], atol=1e-3, rtol=1e-4, frac=0.999, name="median")
+    assert float(ra.max()) > 0.5
+    assert (to_np(rf)[0, 0, :7] == 0).all() and (to_np(ra)[0, 3, 5] == 0).all()
+
+
+@pytest.mark.parametrize("deg", [0, 1, 2, 3, 4])
+def test_spherical_harmonics_forward(deg):
+    from splatad_amd import spherical_harmonics
+    rng = np.random.default_rng(deg)
+    n, K = 5000, 25
+    dirs = (rng.normal(size=(n, 3)) * 2).astype(np.float32)
+    coeffs = rng.normal(size=(n, K, 3)).astype(np.float32)
+    masks = rng.random(n) > 0.3
+    col = spherical_harmonics(deg, to_dev(dirs), to_dev(coeffs))
+    assert_close(to_np(col), oracle.spherical_harmonics(deg, dirs, coeffs, precision="f64"),
+                 atol=1e-4, name="sh")
+    colm = spherical_harmonics(deg, to_dev(dirs), to_dev(coeffs), masks=to_dev(masks))
+    assert_close(to_np(colm), oracle.spherical_harmonics(deg, dirs, coeffs, masks, precision="f64"),
+                 atol=1e-4, name="sh masked")
+    # batched shapes [C, N, ...]
+    col2 = spherical_harmonics(deg, to_dev(dirs.reshape(5, 1000, 3)), to_dev(coeffs.reshape(5, 1000, K, 3)))
+    np.testing.assert_array_equal(to_np(col2).reshape(n, 3), to_np(col))
+
+
+def test_isect_lidar_extent_beyond_a_full_turn():
+    # regression: azimuth extents below -360 degrees must wrap inside the tile grid
+    from splatad_amd import isect_lidar_tiles
+    rng = np.random.default_rng(9)
+    N = 2000
+    means2d = np.stack([rng.uniform(-180, 180, (1, N)), rng.uniform(-20, 20, (1, N))], -1).astype(np.float32)
+    radii = rng.uniform(0.0, 900.0, (1, N, 2)).astype(np.float32)
+    depths = rng.uniform(0.1, 50, (1, N)).astype(np.float32)
+    eb = np.linspace(-25, 25, 5).astype(np.float32)
+    res = 360.0 / 16
+    tpg, ids, flat = isect_lidar_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), to_dev(eb), res, -180.0)
+    o = oracle.isect_lidar_tiles(means2d, radii, depths, eb, res, -180.0)
+    np.testing.assert_array_equal(to_np(tpg), o[0])
+    np.testing.assert_array_equal(to_np(ids), o[1])
+    np.testing.assert_array_equal(to_np(flat), o[2])

@@ -205,3 +205,20 @@ def test_lidar_isect_full_circle_tiles():
     np.testing.assert_array_equal(tpg, tpg_b)
     np.testing.assert_array_equal(ids, ids_b)
     np.testing.assert_array_equal(flat, flat_b)
+
+
+def test_lidar_isect_extent_beyond_a_full_turn():
+    # A Gaussian next to the sensor can span more than 360 degrees: tile columns wrap with a
+    # true modulo, every tile index stays inside the grid and the counts match the bounds.
+    means2d = np.array([[[-100.0, 0.0], [120.0, 1.0]]], np.float32)
+    radii = np.array([[[700.0, 2.0], [800.0, 1.0]]], np.float32)
+    depths = np.array([[1.0, 2.0]], np.float32)
+    eb = np.array([-30.0, 0.0, 30.0], np.float32)
+    res = 360.0 / 8
+    tpg, ids, flat = oracle.isect_lidar_tiles(means2d, radii, depths, eb, res, -180.0, sort=False)
+    cam, tile, _ = _decode(ids, 8 * 2, 1)
+    assert (cam == 0).all() and (tile >= 0).all() and (tile < 16).all()
+    assert tpg.sum() == ids.shape[0] and (tpg > 16).all()
+    # consecutive emissions walk the columns cyclically
+    cols = tile[: tpg[0, 0] // 2] % 8
+    assert ((np.diff(cols) % 8) == 1).all()
