@@ -1,0 +1,318 @@
+"""Benchmark of the forward rendering path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--n N]
+
+A step is one complete forward call of `rasterization()` (projection + SH + tile intersection
++ sort + offsets + rasterize) on the driving-camera workload: 1M Gaussians, 1920x1080 pinhole,
+SH degree 3, rolling shutter, RGB+D.  All inputs are resident in HBM before the timed region.
+The same is done for `lidar_rasterization()` on the 128x2048 lidar sweep and reported in the
+"lidar" object of the same JSON line.  "roofline" describes the dominant kernel
+(rasterize_to_pixels forward), timed with events on the launch stream; "cpu_baseline" times the
+CPU oracle (a C restatement of the reference's algorithm, OpenMP) on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def _sync():
+    import torch
+
+    torch.cuda.synchronize()
+
+
+def time_steps(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    _sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    _sync()
+    return (time.perf_counter() - t0) / steps
+
+
+def time_kernel(fn, iters, warmup=2):
+    """Average duration in ms of the work fn() enqueues on torch's current stream."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    _sync()
+    start = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    stop = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    for i in range(iters):
+        start[i].record()
+        fn()
+        stop[i].record()
+    _sync()
+    return sum(s.elapsed_time(e) for s, e in zip(start, stop)) / iters
+
+
+def consumed_isects(last_ids, alphas, offsets, n_isects, tile_w, tile_h):
+    """Per-tile prefix of the sorted list that the tile's pixels/points really consume:
+    the whole list when some pixel never saturates, else up to the last contributing entry."""
+    import torch
+
+    C, H, W = last_ids.shape
+    gh, gw = offsets.shape[1:]
+    flat_off = offsets.reshape(-1).long()
+    ends = torch.cat([flat_off[1:], torch.tensor([n_isects], device=flat_off.device)])
+    Hp, Wp = gh * tile_h, gw * tile_w
+    li = torch.zeros((C, Hp, Wp), dtype=torch.long, device=last_ids.device)
+    li[:, :H, :W] = last_ids.long()
+    unsat = torch.zeros((C, Hp, Wp), dtype=torch.bool, device=last_ids.device)
+    unsat[:, :H, :W] = alphas.reshape(C, H, W) < 0.9998
+    li = li.reshape(C, gh, tile_h, gw, tile_w).permute(0, 1, 3, 2, 4).reshape(C * gh * gw, -1)
+    unsat = unsat.reshape(C, gh, tile_h, gw, tile_w).permute(0, 1, 3, 2, 4).reshape(C * gh * gw, -1)
+    full = ends - flat_off
+    need = (li.max(dim=1).values + 1 - flat_off).clamp(min=0)
+    need = torch.where(unsat.any(dim=1), full, torch.minimum(need, full))
+    need = torch.where(full > 0, need, torch.zeros_like(need))
+    return int(need.sum().item()), int(full.sum().item())
+
+
+def bench_camera(args):
+    import torch
+
+    from splatad_amd import rasterization, workloads
+    from splatad_amd.hip._backend import _C
+
+    dev = torch.device("cuda:0")
+    s = workloads.to_device(workloads.camera_driving(n=args.n), dev)
+
+    def run(packed=False):
+        return rasterization(
+            s["means"], s["quats"], s["scales"], s["opacities"], s["colors"], s["velocities"],
+            s["viewmats"], s["Ks"], s["width"], s["height"], s["linear_velocity"],
+            s["angular_velocity"], s["rolling_shutter_time"], sh_degree=s["sh_degree"],
+            packed=packed, render_mode="RGB+D", near_plane=s["near_plane"],
+            far_plane=s["far_plane"], eps2d=s["eps2d"], tile_size=s["tile_size"])
+
+    with torch.no_grad():
+        sec = time_steps(run, args.steps, args.warmup)
+        sec_packed = time_steps(lambda: run(True), max(2, args.steps // 2), 1)
+        rc, ra, meta = run()
+        C, H, W = 1, s["height"], s["width"]
+        # dominant kernel, isolated
+        colors = None
+
+        # rebuild the rasterizer's inputs exactly as rasterization() does
+        from splatad_amd import spherical_harmonics
+        camtoworlds = torch.inverse(s["viewmats"])
+        dirs = s["means"][None] - camtoworlds[:, None, :3, 3]
+        cols = spherical_harmonics(3, dirs, s["colors"].expand(C, -1, -1, -1), masks=meta["radii"][..., 0] > 0)
+        cols = torch.cat([torch.clamp_min(cols + 0.5, 0.0), meta["depths"][..., None]], -1).contiguous()
+        ts = s["tile_size"]
+
+        def raster():
+            return _C.rasterize_to_pixels_fwd(
+                meta["means2d"], meta["conics"], cols, meta["opacities"], meta["pix_vels"],
+                s["rolling_shutter_time"], None, W, H, ts, meta["isect_offsets"], meta["flatten_ids"])
+
+        k_ms = time_kernel(raster, iters=max(5, args.steps))
+        _, alphas, last_ids = raster()
+        n_isects = int(meta["flatten_ids"].shape[0])
+        i_need, i_full = consumed_isects(last_ids, alphas, meta["isect_offsets"], n_isects, ts, ts)
+        D = cols.shape[-1]
+        P, T = C * H * W, meta["isect_offsets"].numel()
+        alg_bytes = i_need * (36 + 4 * D) + P * (4 * D + 8) + T * 4
+        # per-stage times of the same call
+        stages = {}
+        proj = lambda: _C.fully_fused_projection_fwd(
+            s["means"], None, s["quats"], s["scales"], s["velocities"], s["viewmats"], s["Ks"], W, H,
+            s["linear_velocity"], s["angular_velocity"], s["rolling_shutter_time"], s["eps2d"],
+            s["near_plane"], s["far_plane"], 0.0, False)
+        stages["projection_ms"] = time_kernel(proj, 5)
+        isect = lambda: _C.isect_tiles(meta["means2d"], meta["radii"], meta["depths"], None, None, C,
+                                       ts, meta["tile_width"], meta["tile_height"], True, True)
+        stages["isect_sort_ms"] = time_kernel(isect, 5)
+        stages["offset_encode_ms"] = time_kernel(
+            lambda: _C.isect_offset_encode(meta["isect_ids"], C, meta["tile_width"], meta["tile_height"]), 5)
+        stages["sh_ms"] = time_kernel(
+            lambda: _C.compute_sh_fwd(3, dirs.contiguous(), s["colors"].expand(C, -1, -1, -1).contiguous(),
+                                      (meta["radii"][..., 0] > 0).contiguous()), 5)
+        stages["rasterize_ms"] = k_ms
+    return dict(sec=sec, sec_packed=sec_packed, pixels=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
+                n_isects=n_isects, i_need=i_need, nnz=int((meta["radii"][..., 0] > 0).sum().item()),
+                stages=stages, channels=D)
+
+
+def bench_lidar(args):
+    import torch
+
+    from splatad_amd import lidar_rasterization, workloads
+    from splatad_amd.hip._backend import _C
+
+    dev = torch.device("cuda:0")
+    s = workloads.to_device(workloads.lidar_sweep(n=args.n), dev)
+
+    def run(chunk=33):
+        return lidar_rasterization(
+            s["means"], s["quats"], s["scales"], s["opacities"], s["lidar_features"],
+            s["velocities"], s["viewmats"], s["raster_pts"], s["tile_elevation_boundaries"],
+            s["linear_velocity"], s["angular_velocity"], s["rolling_shutter_time"],
+            min_azimuth=s["min_azimuth"], max_azimuth=s["max_azimuth"],
+            min_elevation=s["min_elevation"], max_elevation=s["max_elevation"],
+            n_elevation_channels=s["n_elevation_channels"],
+            azimuth_resolution=s["azimuth_resolution"], tile_width=s["tile_width"],
+            tile_height=s["tile_height"], near_plane=s["near_plane"], far_plane=s["far_plane"],
+            eps2d=s["eps2d"], channel_chunk=chunk)
+
+    with torch.no_grad():
+        sec = time_steps(run, args.steps, args.warmup)
+        sec_chunk32 = time_steps(lambda: run(32), max(2, args.steps // 2), 1)
+        rf, ra, asum, meta = run()
+        C, H, W = ra.shape[:3]
+        proj = _C.fully_fused_lidar_projection_fwd(
+            s["means"], None, s["quats"], s["scales"], s["velocities"], s["viewmats"],
+            s["min_elevation"], s["max_elevation"], s["min_azimuth"], s["max_azimuth"],
+            s["linear_velocity"], s["angular_velocity"], s["rolling_shutter_time"], s["eps2d"],
+            s["near_plane"], s["far_plane"], 0.0, False)
+        feats = torch.cat([s["lidar_features"], meta["depths"][..., None]], -1).contiguous()
+        D = feats.shape[-1]
+
+        def raster():
+            return _C.rasterize_to_points_fwd(
+                meta["means2d"], meta["conics"], feats, meta["opacities"], meta["pix_vels"], proj[6],
+                None, s["raster_pts"], W, H, s["tile_width"], s["tile_height"], True, 0.2,
+                meta["isect_offsets"], meta["flatten_ids"], D - 1)
+
+        k_ms = time_kernel(raster, iters=max(5, args.steps))
+        _, alphas, last_ids, _, _ = raster()
+        n_isects = int(meta["flatten_ids"].shape[0])
+        i_need, _ = consumed_isects(last_ids, alphas, meta["isect_offsets"], n_isects,
+                                    s["tile_width"], s["tile_height"])
+        P, T = C * H * W, meta["isect_offsets"].numel()
+        alg_bytes = i_need * (48 + 4 * D) + P * (4 * D + 32) + T * 4
+    return dict(sec=sec, sec_chunk32=sec_chunk32, points=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
+                n_isects=n_isects, i_need=i_need, channels=D)
+
+
+def cpu_baseline_camera(args):
+    """The CPU oracle on the same camera workload (same seed and distributions), OpenMP over
+    all host cores given to the process; bounded by using fewer Gaussians when needed."""
+    import numpy as np
+
+    import oracle
+    from splatad_amd import workloads
+
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else os.cpu_count()
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    oracle.set_num_threads(cores)
+    n = args.cpu_n
+    s = workloads.camera_driving(n=n)
+    npy = lambda t: t.numpy()
+    W, H, ts = s["width"], s["height"], s["tile_size"]
+    tw, th = -(-W // ts), -(-H // ts)
+    t0 = time.perf_counter()
+    radii, m2, depths, conics, _, pv = oracle.projection_fwd(
+        npy(s["means"]), None, npy(s["quats"]), npy(s["scales"]), None, npy(s["viewmats"]),
+        npy(s["Ks"]), W, H, npy(s["linear_velocity"]), npy(s["angular_velocity"]),
+        npy(s["rolling_shutter_time"]), eps2d=s["eps2d"], near_plane=s["near_plane"],
+        far_plane=s["far_plane"], precision="f32")
+    c2w = np.linalg.inv(npy(s["viewmats"]))
+    dirs = npy(s["means"])[None] - c2w[:, None, :3, 3]
+    cols = oracle.spherical_harmonics(3, dirs, np.broadcast_to(npy(s["colors"])[None], (1, n, 16, 3)),
+                                      masks=radii[..., 0] > 0, precision="f32")
+    cols = np.concatenate([np.maximum(cols + 0.5, 0.0), depths[..., None]], -1)
+    _, ids, flat = oracle.isect_tiles(m2, radii, depths, ts, tw, th)
+    offs = oracle.isect_offset_encode(ids, 1, tw, th)
+    opac = npy(s["opacities"])[None]
+    oracle.rasterize_to_pixels_fwd(m2, conics, cols, opac, pv, npy(s["rolling_shutter_time"]), None,
+                                   W, H, ts, offs, flat, precision="f32")
+    dt = time.perf_counter() - t0
+    return dict(value=W * H / dt / 1e6, unit="Mpix/s", cores=cores, kind="port",
+                sample=f"one full 1920x1080 forward frame of the same workload with {n} Gaussians "
+                       f"({dt:.1f} s; C oracle, OpenMP in projection/SH/compositing, serial "
+                       "intersection and merge sort)")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--n", type=int, default=1_000_000, help="Gaussians (default: the benchmark's 1M)")
+    ap.add_argument("--cpu-n", type=int, default=1_000_000, help="Gaussians of the CPU baseline sample")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-lidar", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three 1 GiB device-to-device copies (known HBM traffic, used "
+                         "to scale FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build renders on one GPU; --gpus must be 1 "
+              "(sensors would shard across GPUs, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    cam = bench_camera(args)
+    lid = None if args.no_lidar else bench_lidar(args)
+    achieved = cam["alg_bytes"] / (cam["kernel_ms"] * 1e-3) / 1e9
+    out = {
+        "metric": "camera Mpix/s (fwd)",
+        "value": cam["pixels"] / cam["sec"] / 1e6,
+        "unit": "Mpix/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": cam["sec"] * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "driving camera, rolling shutter: %d Gaussians, 1920x1080, SH degree 3, "
+                        "RGB+D, packed=False (BASELINE configs[1])" % args.n,
+            "n_isects": cam["n_isects"], "n_isects_consumed": cam["i_need"],
+            "visible_gaussians": cam["nnz"], "ms_per_step_packed": cam["sec_packed"] * 1e3,
+            "stage_ms": {k: round(v, 4) for k, v in cam["stages"].items()},
+        },
+        "roofline": {
+            "kernel": "rasterize_to_pixels_fwd_kernel<%d>" % cam["channels"],
+            "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "algorithmic_bytes": cam["alg_bytes"], "kernel_ms": cam["kernel_ms"],
+        },
+    }
+    if lid is not None:
+        l_ach = lid["alg_bytes"] / (lid["kernel_ms"] * 1e-3) / 1e9
+        out["lidar"] = {
+            "metric": "lidar Mpts/s (fwd)", "value": lid["points"] / lid["sec"] / 1e6,
+            "unit": "Mpts/s", "ms_per_step": lid["sec"] * 1e3,
+            "ms_per_step_channel_chunk_32": lid["sec_chunk32"] * 1e3,
+            "workload": "128x2048 lidar sweep, %d Gaussians, 32 features + range, tile 64x4, "
+                        "channel_chunk=33 (BASELINE configs[2])" % args.n,
+            "n_isects": lid["n_isects"], "n_isects_consumed": lid["i_need"],
+            "roofline": {"kernel": "rasterize_to_points_fwd_kernel<%d>" % lid["channels"],
+                         "bound": "hbm", "achieved": l_ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": l_ach / HBM_PEAK_GBS, "traffic": None,
+                         "algorithmic_bytes": lid["alg_bytes"], "kernel_ms": lid["kernel_ms"]},
+        }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_camera(args)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

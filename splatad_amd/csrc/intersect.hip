@@ -121,18 +121,88 @@ __device__ __forceinline__ uint32_t camera_of(uint64_t idx, uint32_t N,
     return camera_ids ? (uint32_t)camera_ids[idx] : (uint32_t)(idx / N);
 }
 
+// Work item of one lane: the tile rectangle of its Gaussian plus what the emitters need.
+struct LaneWork {
+    int32_t x0, y0, w, cnt; // rectangle origin, width and number of tiles (0 = nothing)
+    uint32_t base;          // camera * tiles per camera
+    uint32_t idx;           // flatten id
+    uint32_t depth_bits;
+    int64_t cum;            // emission position of the first tile (unsorted output only)
+};
+
+__device__ __forceinline__ LaneWork broadcast_work(const LaneWork &w, int leader) {
+    LaneWork o;
+    o.x0 = __shfl(w.x0, leader, SPLATAD_WAVE);
+    o.y0 = __shfl(w.y0, leader, SPLATAD_WAVE);
+    o.w = __shfl(w.w, leader, SPLATAD_WAVE);
+    o.cnt = __shfl(w.cnt, leader, SPLATAD_WAVE);
+    o.base = __shfl(w.base, leader, SPLATAD_WAVE);
+    o.idx = __shfl(w.idx, leader, SPLATAD_WAVE);
+    o.depth_bits = __shfl(w.depth_bits, leader, SPLATAD_WAVE);
+    o.cum = __shfl(w.cum, leader, SPLATAD_WAVE);
+    return o;
+}
+
+// Tile counts per Gaussian span four orders of magnitude (a Gaussian next to the sensor
+// covers thousands of tiles, a distant one a single tile), so a lane-per-Gaussian loop
+// leaves 63 lanes idle behind one busy lane.  Rectangles above kCoopTiles are therefore
+// expanded by the whole wavefront, 64 tiles per step; the rest stay lane-private.
+constexpr int32_t kCoopTiles = 16;
+
+template <typename Emit>
+__device__ __forceinline__ void for_each_tile_balanced(const LaneWork &mine, Emit &&emit) {
+    const int lane = threadIdx.x & (SPLATAD_WAVE - 1);
+    uint64_t big = __ballot(mine.cnt > kCoopTiles);
+    while (big) {
+        const int leader = __ffsll((unsigned long long)big) - 1;
+        big &= big - 1;
+        const LaneWork w = broadcast_work(mine, leader);
+        for (int32_t t = lane; t < w.cnt; t += SPLATAD_WAVE) emit(w, w.y0 + t / w.w, w.x0 + t % w.w, t);
+    }
+    if (mine.cnt <= kCoopTiles)
+        for (int32_t t = 0; t < mine.cnt; ++t) emit(mine, mine.y0 + t / mine.w, mine.x0 + t % mine.w, t);
+}
+
+template <bool LIDAR>
+__device__ __forceinline__ LaneWork load_work(const TileGrid &g, uint64_t idx, uint64_t total,
+                                              uint32_t N, const int64_t *__restrict__ camera_ids,
+                                              const float *__restrict__ means2d,
+                                              const void *__restrict__ radii,
+                                              const float *__restrict__ depths,
+                                              const int64_t *__restrict__ cum_before) {
+    LaneWork w;
+    w.x0 = w.y0 = w.cnt = 0;
+    w.w = 1;
+    w.base = 0;
+    w.idx = (uint32_t)idx;
+    w.depth_bits = 0;
+    w.cum = 0;
+    if (idx < total) {
+        int32_t x0, y0, x1, y1;
+        if (tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) {
+            w.x0 = x0; w.y0 = y0;
+            w.w = max(x1 - x0, 1);
+            w.cnt = max(x1 - x0, 0) * max(y1 - y0, 0);
+            w.base = camera_of(idx, N, camera_ids) * g.tile_w * g.tile_h;
+            if (depths) w.depth_bits = __float_as_uint(depths[idx]);
+            if (cum_before) w.cum = cum_before[idx];
+        }
+    }
+    return w;
+}
+
 template <bool LIDAR>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 isect_histogram_kernel(TileGrid g, uint64_t total, uint32_t N,
                        const int64_t *__restrict__ camera_ids, const float *__restrict__ means2d,
-                       const void *__restrict__ radii, int32_t *__restrict__ tile_counts) {
+                       const void *__restrict__ radii, uint32_t copies,
+                       uint32_t n_segments, int32_t *__restrict__ tile_counts) {
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    int32_t x0, y0, x1, y1;
-    if (!tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) return;
-    const uint32_t base = camera_of(idx, N, camera_ids) * g.tile_w * g.tile_h;
-    for (int32_t y = y0; y < y1; ++y)
-        for (int32_t x = x0; x < x1; ++x) atomicAdd(&tile_counts[base + tile_index<LIDAR>(g, y, x)], 1);
+    const LaneWork mine = load_work<LIDAR>(g, idx, total, N, camera_ids, means2d, radii, nullptr, nullptr);
+    const size_t copy_base = (size_t)(blockIdx.x & (copies - 1)) * n_segments;
+    for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t) {
+        atomicAdd(&tile_counts[copy_base + w.base + tile_index<LIDAR>(g, y, x)], 1);
+    });
 }
 
 template <bool LIDAR>
@@ -140,20 +210,17 @@ __global__ void __launch_bounds__(SPLATAD_THREADS)
 isect_scatter_kernel(TileGrid g, uint64_t total, uint32_t N,
                      const int64_t *__restrict__ camera_ids, const float *__restrict__ means2d,
                      const void *__restrict__ radii, const float *__restrict__ depths,
+                     uint32_t copies, uint32_t n_segments,
                      const int32_t *__restrict__ tile_starts, int32_t *__restrict__ tile_fill,
                      uint64_t *__restrict__ pairs) {
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    int32_t x0, y0, x1, y1;
-    if (!tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) return;
-    const uint32_t base = camera_of(idx, N, camera_ids) * g.tile_w * g.tile_h;
-    const uint64_t pair = ((uint64_t)__float_as_uint(depths[idx]) << 32) | (uint64_t)(uint32_t)idx;
-    for (int32_t y = y0; y < y1; ++y)
-        for (int32_t x = x0; x < x1; ++x) {
-            const uint32_t t = base + tile_index<LIDAR>(g, y, x);
-            const int32_t slot = atomicAdd(&tile_fill[t], 1);
-            pairs[(int64_t)tile_starts[t] + slot] = pair;
-        }
+    const LaneWork mine = load_work<LIDAR>(g, idx, total, N, camera_ids, means2d, radii, depths, nullptr);
+    const size_t copy_base = (size_t)(blockIdx.x & (copies - 1)) * n_segments;
+    for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t) {
+        const size_t t = copy_base + w.base + tile_index<LIDAR>(g, y, x);
+        const int32_t slot = atomicAdd(&tile_fill[t], 1);
+        pairs[(int64_t)tile_starts[t] + slot] = ((uint64_t)w.depth_bits << 32) | (uint64_t)w.idx;
+    });
 }
 
 // Emission order without sorting (sort == false): rasterization.cu:65-89 / :366-394.
@@ -165,19 +232,15 @@ isect_emit_kernel(TileGrid g, uint64_t total, uint32_t N, const int64_t *__restr
                   uint32_t tile_n_bits, int64_t *__restrict__ isect_ids,
                   int32_t *__restrict__ flatten_ids) {
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    int32_t x0, y0, x1, y1;
-    if (!tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) return;
-    const int64_t cid_enc = (int64_t)camera_of(idx, N, camera_ids) << (32 + tile_n_bits);
-    const int64_t depth_enc = (int64_t)(int32_t)__float_as_uint(depths[idx]);
-    int64_t cur = cum_before[idx];
-    for (int32_t y = y0; y < y1; ++y)
-        for (int32_t x = x0; x < x1; ++x) {
-            const int64_t tile_id = tile_index<LIDAR>(g, y, x);
-            isect_ids[cur] = cid_enc | (tile_id << 32) | depth_enc;
-            flatten_ids[cur] = (int32_t)idx;
-            ++cur;
-        }
+    const LaneWork mine = load_work<LIDAR>(g, idx, total, N, camera_ids, means2d, radii, depths, cum_before);
+    const uint32_t tiles_per_cam = g.tile_w * g.tile_h;
+    for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t t) {
+        const int64_t cid_enc = (int64_t)(w.base / tiles_per_cam) << (32 + tile_n_bits);
+        const int64_t depth_enc = (int64_t)(int32_t)w.depth_bits;
+        const int64_t tile_id = tile_index<LIDAR>(g, y, x);
+        isect_ids[w.cum + t] = cid_enc | (tile_id << 32) | depth_enc;
+        flatten_ids[w.cum + t] = (int32_t)w.idx;
+    });
 }
 
 // All comparators of this bitonic network point the same way (the first stage of every
@@ -216,17 +279,19 @@ __device__ __forceinline__ void bitonic_sort_ascending(Ptr a, uint32_t n, uint32
 // use_lds selects LDS staging (n <= lds capacity) or in-place sorting in global memory.
 __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
                                           uint32_t tile_n_bits, uint32_t min_n, uint32_t max_n,
-                                          int use_lds, const int32_t *__restrict__ tile_starts,
-                                          const int32_t *__restrict__ tile_counts,
+                                          int use_lds, int64_t n_isects,
+                                          const int32_t *__restrict__ tile_starts,
                                           uint64_t *__restrict__ pairs,
                                           int64_t *__restrict__ isect_ids,
                                           int32_t *__restrict__ flatten_ids) {
     extern __shared__ uint64_t lds_pairs[];
     const uint32_t seg = blockIdx.x;
     if (seg >= n_segments) return;
-    const uint32_t n = (uint32_t)tile_counts[seg];
-    if (n <= min_n || n > max_n) return; // uniform across the workgroup
+    // a segment is the concatenation of the tile's sub-segments; copy 0 comes first
     const int64_t start = tile_starts[seg];
+    const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
+    const uint32_t n = (uint32_t)(stop - start);
+    if (n <= min_n || n > max_n) return; // uniform across the workgroup
     uint64_t *g = pairs + start;
     const uint32_t tid = threadIdx.x, nt = blockDim.x;
     const uint64_t cam = seg / n_tiles, tile = seg % n_tiles;
@@ -286,21 +351,35 @@ __global__ void fill_zero_u64_kernel(unsigned long long *p) { *p = 0ull; }
 struct IsectWorkspace {
     unsigned long long *n_isects; // [1]
     int64_t *scan_total;          // [1]
-    int32_t *tile_counts;         // [C * n_tiles]
-    int32_t *tile_starts;         // [C * n_tiles]
-    int32_t *tile_fill;           // [C * n_tiles]
+    int32_t *tile_counts;         // [C * n_tiles * copies]
+    int32_t *tile_starts;         // [C * n_tiles * copies]
+    int32_t *tile_fill;           // [C * n_tiles * copies]
     int64_t *cum_before;          // [total] (sort == false only)
     int64_t *block_sums;          // scan scratch
     uint64_t *pairs;              // [n_isects]
 };
 
-static size_t isect_ws_bytes(uint64_t total, uint64_t segs, int64_t n_isects) {
+// Atomics on one cache line are serialised by the L2, and a tile table of a few thousand
+// counters is only a few hundred lines.  Every counter is therefore replicated `copies`
+// times (a power of two, chosen so that the table has about half a million entries);
+// workgroup b updates copy b % copies.  A tile's output segment is the concatenation of its
+// sub-segments, so nothing downstream sees the replication.  The table is laid out
+// [copy][segment]: lanes expanding one rectangle update neighbouring words of one line.
+static uint32_t isect_copies(uint64_t segs) {
+    uint32_t k = 1;
+    while (k < 256 && (uint64_t)(2 * k) * segs <= (1ull << 19)) k *= 2;
+    return k;
+}
+
+static size_t isect_ws_bytes(uint64_t total, uint64_t segs_in, int64_t n_isects) {
+    const uint64_t segs = segs_in * isect_copies(segs_in);
     uint64_t scan_n = total > segs ? total : segs;
     return 512 + 3 * splatad_align256(segs * 4) + splatad_align256(total * 8) +
            scan_workspace_bytes((int64_t)scan_n) + splatad_align256((uint64_t)n_isects * 8);
 }
 
-static IsectWorkspace carve_isect(void *ws, uint64_t total, uint64_t segs) {
+static IsectWorkspace carve_isect(void *ws, uint64_t total, uint64_t segs_in) {
+    const uint64_t segs = segs_in * isect_copies(segs_in);
     char *p = (char *)ws;
     IsectWorkspace w;
     w.n_isects = (unsigned long long *)p;   p += 256;
@@ -370,39 +449,48 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         SPLATAD_LAUNCH_CHECK();
         return 0;
     }
-    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream,
-                       w.tile_counts, (int64_t)segs);
-    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream,
-                       w.tile_fill, (int64_t)segs);
+    const uint32_t copies = isect_copies(segs);
+    const uint64_t slots = segs * copies;
+    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(slots), dim3(SPLATAD_THREADS), 0, stream,
+                       w.tile_counts, (int64_t)slots);
+    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(slots), dim3(SPLATAD_THREADS), 0, stream,
+                       w.tile_fill, (int64_t)slots);
     hipLaunchKernelGGL(isect_histogram_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
-                       stream, g, total, N, camera_ids, means2d, radii, w.tile_counts);
+                       stream, g, total, N, camera_ids, means2d, radii, copies, (uint32_t)segs,
+                       w.tile_counts);
     SPLATAD_LAUNCH_CHECK();
-    int rc = launch_exclusive_scan<int32_t>(w.tile_counts, (int64_t)segs, 1, 0, w.tile_starts,
+    // counters are stored [copy][segment] (so that a wavefront's atomics on neighbouring
+    // tiles share cache lines) and scanned segment-major
+    int rc = launch_exclusive_scan<int32_t>(w.tile_counts, (int64_t)slots,
+                                            copies > 1 ? -(int)copies : 1, 0, w.tile_starts,
                                             w.scan_total, w.block_sums, stream);
     if (rc) return rc;
     hipLaunchKernelGGL(isect_scatter_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
-                       stream, g, total, N, camera_ids, means2d, radii, depths, w.tile_starts,
-                       w.tile_fill, w.pairs);
+                       stream, g, total, N, camera_ids, means2d, radii, depths, copies,
+                       (uint32_t)segs, w.tile_starts, w.tile_fill, w.pairs);
     SPLATAD_LAUNCH_CHECK();
-    // three size classes: small and medium in LDS, the rest in place in global memory
-    const uint32_t small_cap = 2048, medium_cap = 16384;
+    // Size classes: each launch visits every segment and only works on those of its class, so
+    // that LDS per workgroup (and with it the number of resident workgroups) fits the
+    // segment length.  Segments above the last LDS class are sorted in place in global memory.
+    struct SortClass { uint32_t cap, threads; };
+    static const SortClass classes[] = {{256, 64}, {1024, 256}, {4096, 1024}, {16384, 1024}};
     static bool attr_set = false;
     if (!attr_set) {
         SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)isect_segment_sort_kernel,
                                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                                              medium_cap * 8));
+                                              16384 * 8));
         attr_set = true;
     }
-    hipLaunchKernelGGL(isect_segment_sort_kernel, dim3((uint32_t)segs), dim3(256), small_cap * 8,
-                       stream, (uint32_t)segs, n_tiles, tile_n_bits, 0u, small_cap, 1,
-                       w.tile_starts, w.tile_counts, w.pairs, isect_ids, flatten_ids);
-    hipLaunchKernelGGL(isect_segment_sort_kernel, dim3((uint32_t)segs), dim3(1024),
-                       medium_cap * 8, stream, (uint32_t)segs, n_tiles, tile_n_bits, small_cap,
-                       medium_cap, 1, w.tile_starts, w.tile_counts, w.pairs, isect_ids,
-                       flatten_ids);
+    uint32_t lo = 0;
+    for (const SortClass &c : classes) {
+        hipLaunchKernelGGL(isect_segment_sort_kernel, dim3((uint32_t)segs), dim3(c.threads),
+                           c.cap * 8, stream, (uint32_t)segs, n_tiles, tile_n_bits, lo, c.cap, 1,
+                           n_isects, w.tile_starts, w.pairs, isect_ids, flatten_ids);
+        lo = c.cap;
+    }
     hipLaunchKernelGGL(isect_segment_sort_kernel, dim3((uint32_t)segs), dim3(1024), 0, stream,
-                       (uint32_t)segs, n_tiles, tile_n_bits, medium_cap, 0x7FFFFFFFu, 0,
-                       w.tile_starts, w.tile_counts, w.pairs, isect_ids, flatten_ids);
+                       (uint32_t)segs, n_tiles, tile_n_bits, lo, 0x7FFFFFFFu, 0, n_isects,
+                       w.tile_starts, w.pairs, isect_ids, flatten_ids);
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }

@@ -14,11 +14,20 @@
 
 namespace { // one private copy of the kernels per translation unit
 
-// Value of element i of a strided int32 input, optionally reduced to a 0/1 flag (v > 0).
+// How logical element i of a scan maps to memory.  stride > 0: element i sits at i * stride.
+// stride < 0: the data is a [-stride][n / -stride] matrix scanned column by column, i.e.
+// logical i = col * rows + row sits at row * cols + col.
+__device__ __forceinline__ int64_t scan_phys(int64_t i, int64_t n, int stride) {
+    if (stride > 0) return i * stride;
+    const int64_t rows = -stride, cols = n / rows;
+    return (i % rows) * cols + (i / rows);
+}
+
+// Value of logical element i of an int32 input, optionally reduced to a 0/1 flag (v > 0).
 __device__ __forceinline__ int32_t scan_load(const int32_t *in, int64_t i, int64_t n, int stride,
                                              int as_flag) {
     if (i >= n) return 0;
-    int32_t v = in[i * stride];
+    int32_t v = in[scan_phys(i, n, stride)];
     return as_flag ? (v > 0 ? 1 : 0) : v;
 }
 
@@ -92,7 +101,7 @@ scan_apply_kernel(const int32_t *__restrict__ in, int64_t n, int stride, int as_
     int64_t run = block_exclusive_scan(s, &tot) + block_sums[blockIdx.x];
 #pragma unroll
     for (int k = 0; k < SCAN_ITEMS; ++k) {
-        if (base + k < n) out[base + k] = (OutT)run;
+        if (base + k < n) out[stride > 0 ? base + k : scan_phys(base + k, n, stride)] = (OutT)run;
         run += v[k];
     }
 }
@@ -102,8 +111,9 @@ static inline size_t scan_workspace_bytes(int64_t n) {
     return splatad_align256((size_t)(n_blocks > 0 ? n_blocks : 1) * sizeof(int64_t));
 }
 
-// out[i] = sum_{j<i} f(in[j*stride]); *total (device) = sum over all.  `block_sums` is
-// scan_workspace_bytes(n) of scratch.  n == 0 only writes *total = 0.
+// out[i] = sum_{j<i} f(in[phys(j)]); *total (device) = sum over all.  The output is dense for
+// stride > 0 and uses the input's transposed layout for stride < 0 (see scan_phys).
+// `block_sums` is scan_workspace_bytes(n) of scratch.  n == 0 only writes *total = 0.
 template <typename OutT>
 static inline int launch_exclusive_scan(const int32_t *in, int64_t n, int stride, int as_flag,
                                         OutT *out, int64_t *total, int64_t *block_sums,
