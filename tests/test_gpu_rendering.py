@@ -1,0 +1,286 @@
+"""End-to-end GPU parity of rasterization() / lidar_rasterization() against the CPU oracle,
+plus size-independent properties at the full benchmark sizes."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import torch_ref
+from splatad_amd import workloads
+from tests.gpu_util import DEV, assert_close, to_dev, to_np
+from tests.oracle_backend import OracleOps
+
+pytestmark = pytest.mark.gpu
+
+T64 = lambda a: torch.from_numpy(np.ascontiguousarray(a)).double()
+
+
+def _cam_scene(n=10000, rolling=True):
+    s = workloads.camera_small(n=n)
+    if rolling:
+        s["linear_velocity"] = torch.tensor([[1.0, 0.5, 0.2]])
+        s["angular_velocity"] = torch.tensor([[0.0, 0.1, 0.05]])
+        s["rolling_shutter_time"] = torch.tensor([0.03])
+    return s
+
+
+def _render(s, dev_scene=None, **kw):
+    from splatad_amd import rasterization
+    d = dev_scene or workloads.to_device(s, DEV)
+    return rasterization(d["means"], d["quats"], d["scales"], d["opacities"], d["colors"], d["velocities"],
+                         d["viewmats"], d["Ks"], d["width"], d["height"], d["linear_velocity"],
+                         d["angular_velocity"], d["rolling_shutter_time"], near_plane=d["near_plane"],
+                         far_plane=d["far_plane"], eps2d=d["eps2d"], tile_size=d["tile_size"], **kw)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_camera_small_config_against_oracle_pipeline(packed, monkeypatch):
+    """10k Gaussians, 320x240 (the CPU-runnable benchmark configuration)."""
+    s = _cam_scene()
+    rc, ra, meta = _render(s, packed=packed, render_mode="RGB+D")
+    # (1) every stage against the oracle on the GPU's own inputs to that stage
+    m2, radii, depths = to_np(meta["means2d"]), to_np(meta["radii"]), to_np(meta["depths"])
+    cam_ids = to_np(meta["camera_ids"]) if packed else None
+    o_tpg, o_ids, o_flat = oracle.isect_tiles(m2, radii, depths, 16, meta["tile_width"], meta["tile_height"],
+                                              n_cameras=1, camera_ids=cam_ids)
+    np.testing.assert_array_equal(to_np(meta["tiles_per_gauss"]), o_tpg)
+    np.testing.assert_array_equal(to_np(meta["isect_ids"]), o_ids)
+    np.testing.assert_array_equal(to_np(meta["flatten_ids"]), o_flat)
+    np.testing.assert_array_equal(to_np(meta["isect_offsets"]),
+                                  oracle.isect_offset_encode(o_ids, 1, meta["tile_width"], meta["tile_height"]))
+    cols = s["colors"].numpy()
+    cols = cols[to_np(meta["gaussian_ids"])] if packed else cols[None]
+    cols = np.concatenate([cols, depths[..., None]], -1)
+    o_rc, o_ra, _ = oracle.rasterize_to_pixels_fwd(
+        m2, to_np(meta["conics"]), cols, to_np(meta["opacities"]), to_np(meta["pix_vels"]),
+        s["rolling_shutter_time"].numpy(), None, s["width"], s["height"], 16, to_np(meta["isect_offsets"]),
+        to_np(meta["flatten_ids"]), precision="f64")
+    assert_close(to_np(rc), o_rc, atol=1e-4, name="render")
+    assert_close(to_np(ra), o_ra, atol=1e-4, name="alpha")
+    # (2) the whole call against the whole oracle pipeline (float32 oracle projection may cull
+    # or truncate a boundary Gaussian differently: allow that on a sliver of the pixels)
+    from splatad_amd import rasterization
+    from splatad_amd.hip import _backend
+    monkeypatch.setattr(_backend, "_C", OracleOps())
+    e_rc, e_ra, e_meta = rasterization(s["means"], s["quats"], s["scales"], s["opacities"], s["colors"], None,
+                                       s["viewmats"], s["Ks"], s["width"], s["height"], s["linear_velocity"],
+                                       s["angular_velocity"], s["rolling_shutter_time"], packed=packed,
+                                       render_mode="RGB+D")
+    assert_close(to_np(rc), e_rc.numpy(), atol=1e-4, rtol=1e-4, frac=0.999, name="render vs full oracle")
+    assert_close(to_np(ra), e_ra.numpy(), atol=1e-4, frac=0.999, name="alpha vs full oracle")
+    assert abs(e_meta["flatten_ids"].shape[0] - meta["flatten_ids"].shape[0]) <= 20
+
+
+def test_camera_render_modes_backgrounds_sh_and_determinism():
+    s = workloads.camera_driving(n=20000, width=320, height=180, with_velocities=True)
+    d = workloads.to_device(s, DEV)
+    bg = torch.rand(1, 3, device=DEV)
+    outs = {}
+    for mode in ("RGB", "D", "ED", "RGB+D", "RGB+ED"):
+        rc, ra, meta = _render(s, d, sh_degree=3, packed=False, render_mode=mode, backgrounds=bg)
+        outs[mode] = (rc, ra)
+        X = {"RGB": 3, "RGB+D": 4, "RGB+ED": 4, "D": 1, "ED": 1}[mode]
+        assert rc.shape == (1, 180, 320, X)
+    torch.testing.assert_close(outs["RGB+D"][0][..., :3], outs["RGB"][0], rtol=0, atol=1e-6)
+    torch.testing.assert_close(outs["RGB+D"][0][..., 3:], outs["D"][0], rtol=0, atol=1e-5)
+    ed = outs["D"][0] / outs["D"][1].clamp(min=1e-10)
+    torch.testing.assert_close(outs["ED"][0], ed, rtol=1e-6, atol=1e-6)
+    # bitwise reproducible
+    again = _render(s, d, sh_degree=3, packed=False, render_mode="RGB+D", backgrounds=bg)
+    assert torch.equal(again[0], outs["RGB+D"][0]) and torch.equal(again[1], outs["RGB+D"][1])
+    # SH colours against the oracle
+    cam2world = np.linalg.inv(s["viewmats"].numpy())
+    dirs = s["means"].numpy()[None] - cam2world[:, None, :3, 3]
+    _, _, meta = _render(s, d, sh_degree=3, packed=False)
+    sh = oracle.spherical_harmonics(3, dirs, s["colors"].numpy()[None], to_np(meta["radii"])[..., 0] > 0, "f64")
+    # packed and unpacked agree
+    p = _render(s, d, sh_degree=3, packed=True, render_mode="RGB+D", backgrounds=bg)
+    torch.testing.assert_close(p[0], outs["RGB+D"][0], rtol=0, atol=1e-5)
+    # channel chunking agrees with one pass
+    feat = torch.rand(20000, 40, device=DEV)
+    from splatad_amd import rasterization
+    a = rasterization(d["means"], d["quats"], d["scales"], d["opacities"], feat, None, d["viewmats"], d["Ks"],
+                      320, 180, packed=False, channel_chunk=64)
+    b = rasterization(d["means"], d["quats"], d["scales"], d["opacities"], feat, None, d["viewmats"], d["Ks"],
+                      320, 180, packed=False, channel_chunk=16)
+    torch.testing.assert_close(a[0], b[0], rtol=0, atol=1e-5)
+    assert sh.shape == (1, 20000, 3)
+
+
+def _lidar(n=20000, D=8, **kw):
+    l = workloads.lidar_sweep(n=n, n_beams=32, n_azimuth=512, feature_dim=D, tile_width=64, tile_height=4,
+                              with_velocities=True, **kw)
+    l["scales"] = l["scales"] * 2.0
+    return l
+
+
+def _lidar_render(d, **kw):
+    from splatad_amd import lidar_rasterization
+    return lidar_rasterization(
+        d["means"], d["quats"], d["scales"], d["opacities"], d["lidar_features"], d["velocities"],
+        d["viewmats"], d["raster_pts"], d["tile_elevation_boundaries"], d["linear_velocity"],
+        d["angular_velocity"], d["rolling_shutter_time"], min_azimuth=d["min_azimuth"],
+        max_azimuth=d["max_azimuth"], min_elevation=d["min_elevation"], max_elevation=d["max_elevation"],
+        n_elevation_channels=d["n_elevation_channels"], azimuth_resolution=d["azimuth_resolution"],
+        tile_width=d["tile_width"], tile_height=d["tile_height"], eps2d=d["eps2d"], **kw)
+
+
+def test_lidar_end_to_end_against_oracle(monkeypatch):
+    l = _lidar()
+    d = workloads.to_device(l, DEV)
+    rf, ra, asum, meta = _lidar_render(d)
+    assert rf.shape == (1, 32, 512, 9)
+    o = oracle.isect_lidar_tiles(to_np(meta["means2d"]), to_np(meta["radii"]), to_np(meta["depths"]),
+                                 l["tile_elevation_boundaries"].numpy(), l["azimuth_resolution"] * 64, -180.0)
+    np.testing.assert_array_equal(to_np(meta["isect_ids"]), o[1])
+    np.testing.assert_array_equal(to_np(meta["flatten_ids"]), o[2])
+    from splatad_amd import lidar_rasterization
+    from splatad_amd.hip import _backend
+    monkeypatch.setattr(_backend, "_C", OracleOps())
+    e = lidar_rasterization(
+        l["means"], l["quats"], l["scales"], l["opacities"], l["lidar_features"], l["velocities"],
+        l["viewmats"], l["raster_pts"], l["tile_elevation_boundaries"], l["linear_velocity"],
+        l["angular_velocity"], l["rolling_shutter_time"], min_azimuth=-180.0, max_azimuth=180.0,
+        min_elevation=-26.0, max_elevation=16.0, n_elevation_channels=32,
+        azimuth_resolution=l["azimuth_resolution"], tile_width=64, tile_height=4, eps2d=0.017)
+    assert_close(to_np(rf), e[0].numpy(), atol=3e-4, rtol=1e-4, frac=0.999, name="features")
+    assert_close(to_np(ra), e[1].numpy(), atol=1e-4, frac=0.999, name="alphas")
+    assert_close(to_np(asum), e[2].numpy(), atol=1e-4, rtol=1e-4, frac=0.999, name="alpha sum")
+    assert_close(to_np(meta["median_depths"]), e[3]["median_depths"].numpy(), atol=1e-3, rtol=1e-4, frac=0.995,
+                 name="median")
+    assert float(ra.max()) > 0.5
+
+
+def test_camera_pipeline_gradients_end_to_end():
+    """loss -> rasterize -> SH -> projection, against float64 autograd on the same tile lists."""
+    s = workloads.camera_driving(n=3000, width=96, height=64, with_velocities=True, sh_degree=2)
+    s["colors"] = s["colors"][:, :9]
+    s["means"][:, 2] = s["means"][:, 2] * 0.2 + 3.0     # keep the scene close enough to cover pixels
+    s["means"][:, :2] *= 0.1
+    s["scales"] = s["scales"] * 0.5
+    d = workloads.to_device(s, DEV)
+    names = ("means", "quats", "scales", "opacities", "colors", "velocities")
+    for k in names:
+        d[k] = d[k].clone().requires_grad_()
+    rc, ra, meta = _render(s, d, sh_degree=2, packed=False, render_mode="RGB+D")
+    rng = np.random.default_rng(0)
+    wc = rng.normal(size=tuple(rc.shape)).astype(np.float32)
+    wa = rng.normal(size=tuple(ra.shape)).astype(np.float32)
+    grads = torch.autograd.grad((rc * to_dev(wc)).sum() + (ra * to_dev(wa)).sum(), [d[k] for k in names])
+    # float64 pipeline with the GPU's culling decisions and tile lists
+    r = {k: T64(s[k].numpy()).requires_grad_() for k in names}
+    m2, depths, conics, _, pv = torch_ref.projection_fwd(
+        r["means"], None, r["quats"], r["scales"], r["velocities"], T64(s["viewmats"].numpy()),
+        T64(s["Ks"].numpy()), 96, 64, T64(s["linear_velocity"].numpy()), T64(s["angular_velocity"].numpy()),
+        T64(s["rolling_shutter_time"].numpy()), eps2d=0.3)
+    c2w = torch.inverse(T64(s["viewmats"].numpy()))
+    dirs = r["means"][None] - c2w[:, None, :3, 3]
+    cols = torch.clamp_min(torch_ref.spherical_harmonics(2, dirs, r["colors"][None]) + 0.5, 0.0)
+    cols = torch.cat([cols, depths[..., None]], -1)
+    o_rc, o_ra = torch_ref.rasterize_to_pixels(m2, conics, cols, r["opacities"][None], pv,
+                                               T64(s["rolling_shutter_time"].numpy()), None, 96, 64, 16,
+                                               meta["isect_offsets"].cpu(), meta["flatten_ids"].cpu())
+    assert_close(to_np(rc), o_rc.detach().numpy(), atol=2e-4, rtol=1e-4, name="render")
+    ref = torch.autograd.grad((o_rc * T64(wc)).sum() + (o_ra * T64(wa)).sum(), [r[k] for k in names])
+    from tests.test_gpu_backward import assert_grad_close
+    for k, a, b in zip(names, grads, ref):
+        assert_grad_close(to_np(a), b.numpy(), k, frac=0.99, loose=5e-2)
+    # the densification hook: absgrad lands on meta["means2d"], which is a non-leaf of the graph
+    rc, ra, meta = _render(s, d, sh_degree=2, packed=True, absgrad=True)
+    meta["means2d"].retain_grad()
+    rc.sum().backward()
+    assert meta["means2d"].grad is not None and meta["means2d"].absgrad.shape == meta["means2d"].shape
+    assert (meta["means2d"].absgrad >= meta["means2d"].grad.abs() - 1e-6).all()
+
+
+def test_lidar_pipeline_gradients_end_to_end():
+    l = _lidar(n=3000, D=4)
+    d = workloads.to_device(l, DEV)
+    names = ("means", "quats", "scales", "opacities", "lidar_features", "velocities")
+    for k in names:
+        d[k] = d[k].clone().requires_grad_()
+    rf, ra, asum, meta = _lidar_render(d)
+    rng = np.random.default_rng(0)
+    wc = rng.normal(size=tuple(rf.shape)).astype(np.float32)
+    wa = rng.normal(size=tuple(ra.shape)).astype(np.float32)
+    ws = rng.normal(size=tuple(ra.shape)).astype(np.float32)
+    loss = (rf * to_dev(wc)).sum() + (ra * to_dev(wa)).sum() + (asum * to_dev(ws)).sum()
+    grads = torch.autograd.grad(loss, [d[k] for k in names])
+    r = {k: T64(l[k].numpy()).requires_grad_() for k in names}
+    m2, depths, conics, _, pv, dc = torch_ref.lidar_projection_fwd(
+        r["means"], None, r["quats"], r["scales"], r["velocities"], T64(l["viewmats"].numpy()),
+        T64(l["linear_velocity"].numpy()), T64(l["angular_velocity"].numpy()),
+        T64(l["rolling_shutter_time"].numpy()), eps2d=0.017)
+    feats = torch.cat([r["lidar_features"], depths[..., None]], -1)
+    o = torch_ref.rasterize_to_points(m2, conics, feats, r["opacities"][None], pv, dc, None,
+                                      T64(l["raster_pts"].numpy()), 64, 4, True, 0.2,
+                                      meta["isect_offsets"].cpu(), meta["flatten_ids"].cpu(), 4)
+    assert_close(to_np(rf), o[0].detach().numpy(), atol=3e-4, rtol=1e-4, name="features")
+    ref = torch.autograd.grad((o[0] * T64(wc)).sum() + (o[1] * T64(wa)).sum() + (o[2] * T64(ws)).sum(),
+                              [r[k] for k in names])
+    from tests.test_gpu_backward import assert_grad_close
+    for k, a, b in zip(names, grads, ref):
+        assert_grad_close(to_np(a), b.numpy(), k, frac=0.99, loose=5e-2)
+
+
+def _check_isect_invariants(meta, C, n_tiles):
+    ids = meta["isect_ids"]
+    assert int(meta["tiles_per_gauss"].sum()) == ids.shape[0] == meta["flatten_ids"].shape[0]
+    assert bool((ids[1:] >= ids[:-1]).all())
+    offs = meta["isect_offsets"].reshape(-1).long()
+    assert bool((offs[1:] >= offs[:-1]).all()) and int(offs[-1]) <= ids.shape[0]
+    tb = int(n_tiles).bit_length()
+    hi = ids >> 32
+    lin = (hi >> tb) * n_tiles + (hi & ((1 << tb) - 1))
+    counts = torch.bincount(lin, minlength=C * n_tiles)
+    ends = torch.cat([offs[1:], torch.tensor([ids.shape[0]], device=offs.device)])
+    assert torch.equal(ends - offs, counts)
+
+
+def test_full_size_driving_camera_properties():
+    """1M Gaussians, 1920x1080, SH degree 3, rolling shutter: properties that need no oracle."""
+    s = workloads.camera_driving()
+    d = workloads.to_device(s, DEV)
+    rc, ra, meta = _render(s, d, sh_degree=3, packed=False, render_mode="RGB+D")
+    assert rc.shape == (1, 1080, 1920, 4) and torch.isfinite(rc).all()
+    assert float(ra.min()) >= 0.0 and float(ra.max()) <= 1.0 - 1e-4 + 1e-6
+    _check_isect_invariants(meta, 1, meta["tile_width"] * meta["tile_height"])
+    # compositing is linear in the colours: render(a) + render(b) == render(a + b)
+    from splatad_amd import rasterize_to_pixels
+    N = s["means"].shape[0]
+    ca, cb = torch.rand(1, N, 3, device=DEV), torch.rand(1, N, 3, device=DEV)
+    args = (meta["opacities"], meta["pix_vels"], 1920, 1080, 16, meta["isect_offsets"], meta["flatten_ids"])
+    kw = dict(rolling_shutter_time=d["rolling_shutter_time"])
+    ra_, _ = rasterize_to_pixels(meta["means2d"], meta["conics"], ca, *args, **kw)
+    rb_, _ = rasterize_to_pixels(meta["means2d"], meta["conics"], cb, *args, **kw)
+    rab, alpha_ab = rasterize_to_pixels(meta["means2d"], meta["conics"], ca + cb, *args, **kw)
+    torch.testing.assert_close(ra_ + rb_, rab, rtol=1e-5, atol=2e-5)
+    # with all colours equal to one the image is the accumulated alpha
+    ones, a1 = rasterize_to_pixels(meta["means2d"], meta["conics"], torch.ones(1, N, 1, device=DEV), *args, **kw)
+    torch.testing.assert_close(ones, a1, rtol=1e-5, atol=1e-5)
+    # packed and unpacked agree
+    p = _render(s, d, sh_degree=3, packed=True, render_mode="RGB+D")
+    torch.testing.assert_close(p[0], rc, rtol=1e-5, atol=1e-4)
+    assert p[2]["camera_ids"].shape[0] == int((meta["radii"][..., 0] > 0).sum())
+
+
+def test_full_size_lidar_sweep_properties():
+    """1M Gaussians, 128 x 2048 lidar sweep with 32 features."""
+    l = workloads.lidar_sweep()
+    d = workloads.to_device(l, DEV)
+    rf, ra, asum, meta = _lidar_render(d, channel_chunk=33)
+    assert rf.shape == (1, 128, 2048, 33) and torch.isfinite(rf).all()
+    assert float(ra.min()) >= 0.0 and float(ra.max()) <= 1.0
+    assert float(asum.min()) >= 0.0
+    _check_isect_invariants(meta, 1, meta["tile_grid_width"] * meta["tile_grid_height"])
+    # two chunks (31 features + range, 1 feature + range) reproduce the single pass
+    rf2, ra2, asum2, meta2 = _lidar_render(d, channel_chunk=32)
+    torch.testing.assert_close(rf2, rf, rtol=1e-5, atol=1e-4)
+    torch.testing.assert_close(ra2, ra, rtol=0, atol=1e-6)
+    assert meta2["median_depths"].shape[-1] == 2
+    # expected range lies between the nearest and the farthest Gaussian range where opaque
+    opaque = ra[..., 0] > 0.99
+    rng_ch = rf[..., -1][opaque]
+    assert float(rng_ch.min()) > 0.0 and float(rng_ch.max()) < 60.0
