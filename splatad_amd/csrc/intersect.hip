@@ -18,6 +18,8 @@
 #include "common.h"
 #include "scan.h"
 
+#include <mutex>
+
 namespace {
 
 struct TileGrid {
@@ -275,45 +277,215 @@ __device__ __forceinline__ void bitonic_sort_ascending(Ptr a, uint32_t n, uint32
     }
 }
 
-// One workgroup per (camera, tile).  Segments with min_n < n <= max_n are handled here;
-// use_lds selects LDS staging (n <= lds capacity) or in-place sorting in global memory.
+constexpr uint32_t kSortMaxBuckets = 2048; // per segment
+constexpr uint32_t kSortBucketMean = 12;   // upper bound of the mean entries per bucket
+constexpr uint32_t kSortRankMax = 1024;    // largest bucket ordered by rank counting
+constexpr uint32_t kSortWindow = 12288;    // entries ranked per step when staging is global
+
+__host__ __device__ inline uint32_t sort_bucket_count(uint32_t n) {
+    uint32_t nb = 1;
+    while (nb < kSortMaxBuckets && nb * kSortBucketMean < n) nb <<= 1;
+    return nb;
+}
+
+// One workgroup per (camera, tile) segment: a bucket sort on the depth.  The segment's range
+// of depth bits (for positive floats a piecewise-linear logarithm of the depth) is cut into
+// up to 2048 equal buckets; the entries are counted per bucket (LDS atomics), scattered
+// bucket by bucket into a staging array, and every entry then finds its place inside its
+// bucket by counting the bucket's smaller (depth bits, flatten id) keys; equal keys (a lidar
+// Gaussian wider than a full turn meets a tile twice) are ordered by staging position.
+// Lanes of one bucket read the same staging words, so those reads are LDS broadcasts.
+//   ER     > 0: the segment (n <= ER * blockDim.x) is held in registers between the passes;
+//          = 0: it is read from global memory three times.
+//   IN_LDS: the staging array is LDS (lds_words entries), and the output is written
+//          directly.  Otherwise the isect_ids output is the staging array, LDS holds a
+//          window of kSortWindow entries (plus one maximal bucket on either side) of it at
+//          a time, the ranked entries go back to `pairs` and are converted at the end.
+// Buckets above 1024 entries (many equal depths) are ordered by a workgroup-wide bitonic
+// network instead.  Segments with min_n < n <= max_n are handled, the others skipped.
+// Dynamic LDS: lds_words * 8 bytes of staging, then 2 * sort_bucket_count(max_n) counters.
+template <int ER, bool IN_LDS>
 __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
                                           uint32_t tile_n_bits, uint32_t min_n, uint32_t max_n,
-                                          int use_lds, int64_t n_isects,
+                                          uint32_t lds_words, int64_t n_isects,
                                           const int32_t *__restrict__ tile_starts,
-                                          uint64_t *__restrict__ pairs,
-                                          int64_t *__restrict__ isect_ids,
+                                          uint64_t *pairs, int64_t *isect_ids,
                                           int32_t *__restrict__ flatten_ids) {
-    extern __shared__ uint64_t lds_pairs[];
+    extern __shared__ uint64_t lds_staged[];
+    __shared__ uint32_t s_wave[2 * (1024 / SPLATAD_WAVE)];
+    __shared__ uint32_t s_big;
     const uint32_t seg = blockIdx.x;
     if (seg >= n_segments) return;
-    // a segment is the concatenation of the tile's sub-segments; copy 0 comes first
     const int64_t start = tile_starts[seg];
     const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
     const uint32_t n = (uint32_t)(stop - start);
     if (n <= min_n || n > max_n) return; // uniform across the workgroup
+    const uint32_t nb = sort_bucket_count(n);
+    uint32_t *s_cursor = reinterpret_cast<uint32_t *>(lds_staged + lds_words);
+    uint32_t *s_first = s_cursor + sort_bucket_count(max_n);
     uint64_t *g = pairs + start;
+    int64_t *ids_out = isect_ids + start;
+    int32_t *flat_out = flatten_ids + start;
+    uint64_t *staged = IN_LDS ? lds_staged : reinterpret_cast<uint64_t *>(ids_out);
     const uint32_t tid = threadIdx.x, nt = blockDim.x;
+    const uint32_t lane = tid & (SPLATAD_WAVE - 1), wave = tid / SPLATAD_WAVE;
+    const uint32_t n_waves = nt / SPLATAD_WAVE;
     const uint64_t cam = seg / n_tiles, tile = seg % n_tiles;
-    const uint64_t hi = ((cam << tile_n_bits) | tile) << 32;
-    if (use_lds) {
-        for (uint32_t i = tid; i < n; i += nt) lds_pairs[i] = g[i];
-        __syncthreads();
-        bitonic_sort_ascending(lds_pairs, n, tid, nt);
-        for (uint32_t i = tid; i < n; i += nt) {
-            const uint64_t p = lds_pairs[i];
-            isect_ids[start + i] = (int64_t)(hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
-            flatten_ids[start + i] = (int32_t)(uint32_t)p;
-        }
-    } else {
-        __syncthreads();
-        bitonic_sort_ascending(g, n, tid, nt);
-        for (uint32_t i = tid; i < n; i += nt) {
-            const uint64_t p = g[i];
-            isect_ids[start + i] = (int64_t)(hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
-            flatten_ids[start + i] = (int32_t)(uint32_t)p;
+    const uint64_t key_hi = ((cam << tile_n_bits) | tile) << 32;
+
+    constexpr int NR = ER > 0 ? ER : 1;
+    uint64_t held[NR];
+    if (ER > 0) {
+#pragma unroll
+        for (int k = 0; k < NR; ++k) {
+            const uint32_t i = tid + k * nt;
+            held[k] = i < n ? g[i] : ~0ull;
         }
     }
+    // for_each_entry(f): f(entry) for the entries this thread owns
+    auto for_each_entry = [&](auto &&f) {
+        if (ER > 0) {
+#pragma unroll
+            for (int k = 0; k < NR; ++k)
+                if (tid + k * nt < n) f(held[k]);
+        } else {
+            for (uint32_t i = tid; i < n; i += nt) f(g[i]);
+        }
+    };
+
+    uint32_t lo = 0xFFFFFFFFu, hi = 0u;
+    for_each_entry([&](uint64_t p) {
+        const uint32_t d = (uint32_t)(p >> 32);
+        lo = min(lo, d);
+        hi = max(hi, d);
+    });
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        lo = min(lo, (uint32_t)__shfl_xor((int)lo, off, SPLATAD_WAVE));
+        hi = max(hi, (uint32_t)__shfl_xor((int)hi, off, SPLATAD_WAVE));
+    }
+    if (lane == 0) { s_wave[2 * wave] = lo; s_wave[2 * wave + 1] = hi; }
+    if (tid == 0) s_big = 0;
+    for (uint32_t b = tid; b < nb; b += nt) s_cursor[b] = 0;
+    __syncthreads();
+    for (uint32_t w = 0; w < n_waves; ++w) {
+        lo = min(lo, s_wave[2 * w]);
+        hi = max(hi, s_wave[2 * w + 1]);
+    }
+    const float scale = (float)nb / ((float)(hi - lo) + 1.f);
+    auto bucket_of = [&](uint64_t p) -> uint32_t {
+        return min(nb - 1, (uint32_t)((float)((uint32_t)(p >> 32) - lo) * scale));
+    };
+    __syncthreads(); // s_wave is reused by the scan
+
+    // entries per bucket
+    for_each_entry([&](uint64_t p) { atomicAdd(&s_cursor[bucket_of(p)], 1u); });
+    __syncthreads();
+
+    // exclusive scan over the buckets: thread t owns `per` consecutive buckets
+    {
+        const uint32_t per = nb > nt ? nb / nt : 1;
+        const uint32_t b0 = tid * per;
+        uint32_t sum = 0;
+        if (b0 < nb)
+            for (uint32_t k = 0; k < per; ++k) sum += s_cursor[b0 + k];
+        uint32_t incl = sum;
+#pragma unroll
+        for (int off = 1; off < SPLATAD_WAVE; off <<= 1) {
+            const uint32_t o = (uint32_t)__shfl_up((int)incl, off, SPLATAD_WAVE);
+            if ((int)lane >= off) incl += o;
+        }
+        if (lane == SPLATAD_WAVE - 1) s_wave[wave] = incl;
+        __syncthreads();
+        uint32_t run = incl - sum;
+        for (uint32_t w = 0; w < wave; ++w) run += s_wave[w];
+        if (b0 < nb)
+            for (uint32_t k = 0; k < per; ++k) {
+                const uint32_t c = s_cursor[b0 + k];
+                s_cursor[b0 + k] = run;
+                s_first[b0 + k] = run;
+                run += c;
+                if (c > kSortRankMax) s_big = 1;
+            }
+    }
+    __syncthreads();
+
+    // scatter into buckets
+    for_each_entry([&](uint64_t p) { staged[atomicAdd(&s_cursor[bucket_of(p)], 1u)] = p; });
+    __syncthreads(); // s_cursor[b] is now the end of bucket b
+
+    if (s_big) { // uniform
+        for (uint32_t b = 0; b < nb; ++b) {
+            const uint32_t s0 = s_first[b], s = s_cursor[b] - s0;
+            if (s > kSortRankMax) bitonic_sort_ascending(staged + s0, s, tid, nt); // uniform
+        }
+    }
+
+    // place = first of the bucket + number of smaller keys in the bucket; `view` is the
+    // staging array seen through LDS, view[j - view_lo] == staged[j]
+    auto place_of = [&](uint64_t p, uint32_t i, const uint64_t *view, uint32_t view_lo) -> uint32_t {
+        const uint32_t b = bucket_of(p);
+        const uint32_t s0 = s_first[b], s1 = s_cursor[b];
+        if (s1 - s0 > kSortRankMax) return i; // ordered by the network above
+        uint32_t place = s0;
+        for (uint32_t j = s0; j < s1; ++j) {
+            const uint64_t q = view[j - view_lo];
+            place += (q < p || (q == p && j < i)) ? 1u : 0u;
+        }
+        return place;
+    };
+    if (IN_LDS) {
+        for (uint32_t i = tid; i < n; i += nt) {
+            const uint64_t p = lds_staged[i];
+            const uint32_t place = place_of(p, i, lds_staged, 0);
+            ids_out[place] = (int64_t)(key_hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
+            flat_out[place] = (int32_t)(uint32_t)p;
+        }
+    } else {
+        for (uint32_t w0 = 0; w0 < n; w0 += kSortWindow) { // uniform
+            const uint32_t w1 = min(n, w0 + kSortWindow);
+            const uint32_t v0 = w0 > kSortRankMax ? w0 - kSortRankMax : 0;
+            const uint32_t v1 = min(n, w1 + kSortRankMax);
+            for (uint32_t j = v0 + tid; j < v1; j += nt) lds_staged[j - v0] = staged[j];
+            __syncthreads();
+            for (uint32_t i = w0 + tid; i < w1; i += nt) {
+                const uint64_t p = lds_staged[i - v0];
+                g[place_of(p, i, lds_staged, v0)] = p; // the input is free by now
+            }
+            __syncthreads();
+        }
+        for (uint32_t i = tid; i < n; i += nt) {
+            const uint64_t p = g[i];
+            ids_out[i] = (int64_t)(key_hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
+            flat_out[i] = (int32_t)(uint32_t)p;
+        }
+    }
+}
+
+template <int ER, bool IN_LDS>
+static int launch_segment_sort(uint32_t threads, uint32_t min_n, uint32_t max_n, uint32_t segs,
+                               uint32_t n_tiles, uint32_t tile_n_bits, int64_t n_isects,
+                               const int32_t *tile_starts, uint64_t *pairs, int64_t *isect_ids,
+                               int32_t *flatten_ids, hipStream_t stream) {
+    const uint32_t lds_words = IN_LDS ? max_n : kSortWindow + 2 * kSortRankMax;
+    const uint32_t cap = IN_LDS ? max_n : 0x7FFFFFFFu;
+    const size_t lds_bytes = (size_t)lds_words * 8 + 2 * sort_bucket_count(cap) * 4;
+    {   // raise the kernel's dynamic LDS limit once per instantiation and size
+        static std::mutex guard;
+        static size_t allowed = 0;
+        std::lock_guard<std::mutex> lock(guard);
+        if (lds_bytes > allowed) {
+            SPLATAD_CHECK_HIP(hipFuncSetAttribute(
+                (const void *)isect_segment_sort_kernel<ER, IN_LDS>,
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+            allowed = lds_bytes;
+        }
+    }
+    hipLaunchKernelGGL((isect_segment_sort_kernel<ER, IN_LDS>), dim3(segs), dim3(threads),
+                       lds_bytes, stream, segs, n_tiles, tile_n_bits, min_n, cap, lds_words,
+                       n_isects, tile_starts, pairs, isect_ids, flatten_ids);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
 }
 
 __global__ void __launch_bounds__(SPLATAD_THREADS)
@@ -470,27 +642,21 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                        (uint32_t)segs, w.tile_starts, w.tile_fill, w.pairs);
     SPLATAD_LAUNCH_CHECK();
     // Size classes: each launch visits every segment and only works on those of its class, so
-    // that LDS per workgroup (and with it the number of resident workgroups) fits the
-    // segment length.  Segments above the last LDS class are sorted in place in global memory.
-    struct SortClass { uint32_t cap, threads; };
-    static const SortClass classes[] = {{256, 64}, {1024, 256}, {4096, 1024}, {16384, 1024}};
-    static bool attr_set = false;
-    if (!attr_set) {
-        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)isect_segment_sort_kernel,
-                                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                                              16384 * 8));
-        attr_set = true;
-    }
-    uint32_t lo = 0;
-    for (const SortClass &c : classes) {
-        hipLaunchKernelGGL(isect_segment_sort_kernel, dim3((uint32_t)segs), dim3(c.threads),
-                           c.cap * 8, stream, (uint32_t)segs, n_tiles, tile_n_bits, lo, c.cap, 1,
-                           n_isects, w.tile_starts, w.pairs, isect_ids, flatten_ids);
-        lo = c.cap;
-    }
-    hipLaunchKernelGGL(isect_segment_sort_kernel, dim3((uint32_t)segs), dim3(1024), 0, stream,
-                       (uint32_t)segs, n_tiles, tile_n_bits, lo, 0x7FFFFFFFu, 0, n_isects,
-                       w.tile_starts, w.pairs, isect_ids, flatten_ids);
+    // that the LDS per workgroup (and with it the number of resident workgroups) fits the
+    // segment length.
+    const uint32_t nseg = (uint32_t)segs;
+#define SPLATAD_SORT_CLASS(ER, IN_LDS, threads, lo, hi)                                          \
+    if ((rc = launch_segment_sort<ER, IN_LDS>(threads, lo, hi, nseg, n_tiles, tile_n_bits,        \
+                                              n_isects, w.tile_starts, w.pairs, isect_ids,        \
+                                              flatten_ids, stream)) != 0)                         \
+        return rc;
+    SPLATAD_SORT_CLASS(4, true, 128, 0u, 512u)
+    SPLATAD_SORT_CLASS(8, true, 256, 512u, 2048u)
+    SPLATAD_SORT_CLASS(8, true, 512, 2048u, 4096u)
+    SPLATAD_SORT_CLASS(8, true, 1024, 4096u, 8192u)
+    SPLATAD_SORT_CLASS(16, true, 1024, 8192u, 16384u)
+    SPLATAD_SORT_CLASS(0, false, 1024, 16384u, 0x7FFFFFFFu)
+#undef SPLATAD_SORT_CLASS
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }

@@ -186,6 +186,25 @@ def test_isect_camera_sizes_and_packed(n, C, W, H, ts, rmax):
     np.testing.assert_array_equal(sel[to_np(flat_p)], o_flat)
 
 
+@pytest.mark.parametrize("n,tie_frac", [(1500, 0.8), (6000, 0.0), (6000, 0.5), (12000, 0.3),
+                                        (40000, 0.0), (40000, 0.4), (3000, 1.0)])
+def test_isect_sort_long_segments_and_depth_ties(n, tie_frac):
+    # every Gaussian covers all four tiles, so each tile's segment has n entries: exercises
+    # every segment-length class of the sort and, with many equal depths, oversized buckets
+    from splatad_amd import isect_tiles
+    rng = np.random.default_rng(n + int(10 * tie_frac))
+    means2d = rng.uniform(10, 22, (1, n, 2)).astype(np.float32)
+    radii = np.full((1, n, 2), 40, np.int32)
+    depths = np.exp(rng.uniform(-3, 5, (1, n))).astype(np.float32)
+    depths[0, rng.random(n) < tie_frac] = 3.25
+    tpg, ids, flat = isect_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), 16, 2, 2)
+    o_tpg, o_ids, o_flat = oracle.isect_tiles(means2d, radii, depths, 16, 2, 2)
+    assert o_ids.shape[0] == 4 * n
+    np.testing.assert_array_equal(to_np(tpg), o_tpg)
+    np.testing.assert_array_equal(to_np(ids), o_ids)
+    np.testing.assert_array_equal(to_np(flat), o_flat)
+
+
 def test_isect_lidar_reference_recipe_and_wrap():
     # input recipe of the reference's test_isect_lidar (tests/test_basic.py:733-751)
     from splatad_amd import isect_lidar_tiles, isect_offset_encode
