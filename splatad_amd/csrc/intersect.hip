@@ -2,16 +2,20 @@
 //
 // Results are bit-identical to gsplat/cuda/csrc/rasterization.cu:15-529 of the reference
 // (two-pass emit + cub::DeviceRadixSort on (camera | tile | depth) keys) but are produced
-// differently:
-//   1. a histogram pass counts intersections per (camera, tile);
-//   2. an exclusive scan of the histogram gives every tile's segment in the output;
-//   3. a scatter pass drops (depth bits, flatten id) pairs into their tile's segment;
-//   4. one workgroup per tile sorts its segment in LDS (bitonic network on the 64-bit
-//      composite depth<<32 | id) and writes the final 64-bit keys and the ids.
+// differently, by binning instead of a global sort:
+//   1. coarse binning: every Gaussian is entered, with one global atomic each in a counting
+//      and a filling pass, into the lists of the coarse blocks (4 x 4 tiles) it touches,
+//      together with the 16-bit mask of the block's tiles it covers;
+//   2. tile binning: wavefronts walk the coarse lists, 64 entries of one block at a time,
+//      and turn the masks into per-tile counts and ranks with ballots, so that a tile
+//      counter sees one atomic per wavefront instead of one per intersection; an exclusive
+//      scan of the tile counts in between gives every tile's segment in the output;
+//   3. one workgroup per tile sorts its segment of (depth bits, flatten id) pairs in LDS and
+//      writes the final 64-bit keys and the ids.
 // A stable sort by (camera, tile, depth) with ties kept in emission order equals a sort
 // by (camera, tile, depth, flatten id), because the emission loop visits flatten ids in
-// ascending order and emits each id at most once per tile; that is what makes the
-// unordered scatter of step 3 legal.  Depths must have a clear sign bit.
+// ascending order; that is what makes the unordered binning legal.  Depths must have a
+// clear sign bit.
 //
 // Built with -ffp-contract=off: the tile bounds are float32 expressions whose rounding
 // decides which tiles a Gaussian touches.
@@ -130,6 +134,7 @@ struct LaneWork {
     uint32_t idx;           // flatten id
     uint32_t depth_bits;
     int64_t cum;            // emission position of the first tile (unsorted output only)
+    int32_t tx0, ty0, tx1, ty1; // tile rectangle, when x0.. describe coarse blocks instead
 };
 
 __device__ __forceinline__ LaneWork broadcast_work(const LaneWork &w, int leader) {
@@ -142,6 +147,10 @@ __device__ __forceinline__ LaneWork broadcast_work(const LaneWork &w, int leader
     o.idx = __shfl(w.idx, leader, SPLATAD_WAVE);
     o.depth_bits = __shfl(w.depth_bits, leader, SPLATAD_WAVE);
     o.cum = __shfl(w.cum, leader, SPLATAD_WAVE);
+    o.tx0 = __shfl(w.tx0, leader, SPLATAD_WAVE);
+    o.ty0 = __shfl(w.ty0, leader, SPLATAD_WAVE);
+    o.tx1 = __shfl(w.tx1, leader, SPLATAD_WAVE);
+    o.ty1 = __shfl(w.ty1, leader, SPLATAD_WAVE);
     return o;
 }
 
@@ -179,9 +188,11 @@ __device__ __forceinline__ LaneWork load_work(const TileGrid &g, uint64_t idx, u
     w.idx = (uint32_t)idx;
     w.depth_bits = 0;
     w.cum = 0;
+    w.tx0 = w.ty0 = w.tx1 = w.ty1 = 0;
     if (idx < total) {
         int32_t x0, y0, x1, y1;
         if (tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) {
+            w.tx0 = x0; w.ty0 = y0; w.tx1 = x1; w.ty1 = y1;
             w.x0 = x0; w.y0 = y0;
             w.w = max(x1 - x0, 1);
             w.cnt = max(x1 - x0, 0) * max(y1 - y0, 0);
@@ -193,36 +204,147 @@ __device__ __forceinline__ LaneWork load_work(const TileGrid &g, uint64_t idx, u
     return w;
 }
 
-template <bool LIDAR>
-__global__ void __launch_bounds__(SPLATAD_THREADS)
-isect_histogram_kernel(TileGrid g, uint64_t total, uint32_t N,
-                       const int64_t *__restrict__ camera_ids, const float *__restrict__ means2d,
-                       const void *__restrict__ radii, uint32_t copies,
-                       uint32_t n_segments, int32_t *__restrict__ tile_counts) {
-    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const LaneWork mine = load_work<LIDAR>(g, idx, total, N, camera_ids, means2d, radii, nullptr, nullptr);
-    const size_t copy_base = (size_t)(blockIdx.x & (copies - 1)) * n_segments;
-    for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t) {
-        atomicAdd(&tile_counts[copy_base + w.base + tile_index<LIDAR>(g, y, x)], 1);
-    });
+// Coarse blocks of (1 << bshift) x 4 tiles.  The width is 4 tiles for cameras; for lidars,
+// whose tile columns wrap around, it is the largest of 4, 2, 1 that divides the number of
+// columns, so that an unwrapped block column maps onto one wrapped block column.
+struct CoarseGrid {
+    uint32_t bshift;
+    uint32_t cw, ch; // blocks per row and per column
+};
+constexpr uint32_t kCoarseRowShift = 2;
+
+// Turns the tile rectangle of a lane's work into the rectangle of coarse blocks to visit.
+__device__ __forceinline__ void to_coarse(LaneWork &w, const CoarseGrid &cg) {
+    if (w.cnt <= 0) return;
+    const int32_t cx0 = w.tx0 >> cg.bshift, cx1 = ((w.tx1 - 1) >> cg.bshift) + 1;
+    const int32_t cy0 = w.ty0 >> kCoarseRowShift, cy1 = ((w.ty1 - 1) >> kCoarseRowShift) + 1;
+    w.x0 = cx0; w.y0 = cy0;
+    w.w = cx1 - cx0;
+    w.cnt = (cx1 - cx0) * (cy1 - cy0);
 }
 
 template <bool LIDAR>
+__device__ __forceinline__ uint32_t coarse_index(const CoarseGrid &cg, int32_t cy, int32_t cx) {
+    if (LIDAR) {
+        const int32_t n = (int32_t)cg.cw;
+        cx = ((cx % n) + n) % n;
+    }
+    return (uint32_t)cy * cg.cw + (uint32_t)cx;
+}
+
+// Bit (ly << bshift | lx) is set when tile (lx, ly) of block (cx, cy) lies in the rectangle.
+__device__ __forceinline__ uint32_t coarse_mask(const LaneWork &w, const CoarseGrid &cg,
+                                                int32_t cy, int32_t cx) {
+    const int32_t bx = 1 << cg.bshift;
+    const int32_t by = 1 << kCoarseRowShift;
+    const int32_t xa = max(w.tx0 - cx * bx, 0), xb = min(w.tx1 - cx * bx, bx);
+    const int32_t ya = max(w.ty0 - cy * by, 0), yb = min(w.ty1 - cy * by, by);
+    const uint32_t row = ((1u << xb) - 1u) & ~((1u << xa) - 1u);
+    uint32_t m = 0;
+    for (int32_t ly = ya; ly < yb; ++ly) m |= row << (ly << cg.bshift);
+    return m;
+}
+
+// The coarse counters are replicated `copies` times (atomics on one cache line are
+// serialised; workgroup b updates copy b % copies) and stored [copy][block], so that a
+// wavefront expanding one large rectangle updates neighbouring words.
+template <bool LIDAR>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
-isect_scatter_kernel(TileGrid g, uint64_t total, uint32_t N,
-                     const int64_t *__restrict__ camera_ids, const float *__restrict__ means2d,
-                     const void *__restrict__ radii, const float *__restrict__ depths,
-                     uint32_t copies, uint32_t n_segments,
-                     const int32_t *__restrict__ tile_starts, int32_t *__restrict__ tile_fill,
-                     uint64_t *__restrict__ pairs) {
+isect_coarse_count_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
+                          const int64_t *__restrict__ camera_ids,
+                          const float *__restrict__ means2d, const void *__restrict__ radii,
+                          uint32_t copies, uint32_t n_blocks, int32_t *__restrict__ counts) {
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const LaneWork mine = load_work<LIDAR>(g, idx, total, N, camera_ids, means2d, radii, depths, nullptr);
-    const size_t copy_base = (size_t)(blockIdx.x & (copies - 1)) * n_segments;
+    LaneWork mine = load_work<LIDAR>(g, idx, total, N, camera_ids, means2d, radii, nullptr, nullptr);
+    mine.base = (mine.base / (g.tile_w * g.tile_h)) * cg.cw * cg.ch;
+    to_coarse(mine, cg);
+    const size_t copy_base = (size_t)(blockIdx.x & (copies - 1)) * n_blocks;
     for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t) {
-        const size_t t = copy_base + w.base + tile_index<LIDAR>(g, y, x);
-        const int32_t slot = atomicAdd(&tile_fill[t], 1);
-        pairs[(int64_t)tile_starts[t] + slot] = ((uint64_t)w.depth_bits << 32) | (uint64_t)w.idx;
+        atomicAdd(&counts[copy_base + w.base + coarse_index<LIDAR>(cg, y, x)], 1);
     });
+}
+
+// Coarse list entry: {flatten id, depth bits, block, tile mask}
+template <bool LIDAR>
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+isect_coarse_fill_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
+                         const int64_t *__restrict__ camera_ids,
+                         const float *__restrict__ means2d, const void *__restrict__ radii,
+                         const float *__restrict__ depths, uint32_t copies, uint32_t n_blocks,
+                         const int32_t *__restrict__ starts, int32_t *__restrict__ fill,
+                         uint4 *__restrict__ entries) {
+    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    LaneWork mine = load_work<LIDAR>(g, idx, total, N, camera_ids, means2d, radii, depths, nullptr);
+    mine.base = (mine.base / (g.tile_w * g.tile_h)) * cg.cw * cg.ch;
+    to_coarse(mine, cg);
+    const size_t copy_base = (size_t)(blockIdx.x & (copies - 1)) * n_blocks;
+    for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t) {
+        const uint32_t block = w.base + coarse_index<LIDAR>(cg, y, x);
+        const size_t t = copy_base + block;
+        const int32_t slot = atomicAdd(&fill[t], 1);
+        entries[(int64_t)starts[t] + slot] =
+            make_uint4(w.idx, w.depth_bits, block, coarse_mask(w, cg, y, x));
+    });
+}
+
+// Tile binning.  A wavefront takes 64 consecutive coarse entries; those of one block (nearly
+// always all 64, the lists being contiguous) are handled together: for each tile of the
+// block a ballot over the mask bit gives the number of entries and every entry's rank, and
+// the lane that owns the tile issues the one atomic.  FILL == false adds to the tile counts,
+// FILL == true reserves the run in the tile's segment and writes the pairs.
+template <bool FILL>
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t copies,
+                      uint32_t n_segments, const int64_t *__restrict__ n_entries_ptr,
+                      const uint4 *__restrict__ entries, int32_t *__restrict__ tile_counts,
+                      const int32_t *__restrict__ tile_starts, int32_t *__restrict__ tile_fill,
+                      uint64_t *__restrict__ pairs) {
+    const int64_t n_entries = *n_entries_ptr;
+    const uint32_t lane = threadIdx.x & (SPLATAD_WAVE - 1);
+    const int64_t wave_id = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / SPLATAD_WAVE;
+    const int64_t n_waves = (int64_t)gridDim.x * blockDim.x / SPLATAD_WAVE;
+    const uint32_t bits = 4u << cg.bshift, per_cam = cg.cw * cg.ch;
+    const uint64_t below = (1ull << lane) - 1ull;
+    // the tile counters are replicated like the coarse ones; both passes run on the same
+    // grid, so an entry meets the same copy in both
+    const int64_t copy_base = (int64_t)(wave_id & (copies - 1)) * n_segments;
+    for (int64_t e0 = wave_id * SPLATAD_WAVE; e0 < n_entries; e0 += n_waves * SPLATAD_WAVE) {
+        const bool has = e0 + lane < n_entries;
+        const uint4 rec = has ? entries[e0 + lane] : make_uint4(0, 0, 0xFFFFFFFFu, 0);
+        uint64_t todo = __ballot(has);
+        while (todo) {
+            const int leader = __ffsll((unsigned long long)todo) - 1;
+            const uint32_t block = (uint32_t)__shfl((int)rec.z, leader, SPLATAD_WAVE);
+            const bool in = has && rec.z == block;
+            todo &= ~__ballot(in);
+            uint32_t my_cnt = 0;
+            for (uint32_t t = 0; t < bits; ++t) {
+                const uint64_t b = __ballot(in && ((rec.w >> t) & 1u));
+                if (lane == t) my_cnt = (uint32_t)__popcll(b);
+            }
+            // lane t < bits owns tile t of the block
+            int64_t tile = copy_base;
+            if (lane < bits) {
+                const uint32_t cam = block / per_cam, r = block % per_cam;
+                const uint32_t x = ((r % cg.cw) << cg.bshift) + (lane & ((1u << cg.bshift) - 1u));
+                const uint32_t y = ((r / cg.cw) << kCoarseRowShift) + (lane >> cg.bshift);
+                tile += (int64_t)cam * tile_w * tile_h + (int64_t)y * tile_w + x;
+            }
+            if (!FILL) {
+                if (my_cnt) atomicAdd(&tile_counts[tile], (int32_t)my_cnt);
+            } else {
+                int32_t dst = 0;
+                if (my_cnt) dst = tile_starts[tile] + atomicAdd(&tile_fill[tile], (int32_t)my_cnt);
+                const uint64_t pair = ((uint64_t)rec.y << 32) | (uint64_t)rec.x;
+                for (uint32_t t = 0; t < bits; ++t) {
+                    const bool hit = in && ((rec.w >> t) & 1u);
+                    const uint64_t b = __ballot(hit);
+                    const int32_t first = __shfl(dst, (int)t, SPLATAD_WAVE);
+                    if (hit) pairs[(int64_t)first + __popcll(b & below)] = pair;
+                }
+            }
+        }
+    }
 }
 
 // Emission order without sorting (sort == false): rasterization.cu:65-89 / :366-394.
@@ -522,48 +644,74 @@ __global__ void fill_zero_u64_kernel(unsigned long long *p) { *p = 0ull; }
 
 struct IsectWorkspace {
     unsigned long long *n_isects; // [1]
+    int64_t *n_entries;           // [1] length of the coarse lists
     int64_t *scan_total;          // [1]
-    int32_t *tile_counts;         // [C * n_tiles * copies]
-    int32_t *tile_starts;         // [C * n_tiles * copies]
-    int32_t *tile_fill;           // [C * n_tiles * copies]
-    int64_t *cum_before;          // [total] (sort == false only)
+    int32_t *zeroed;              // coarse_counts .. tile_fill are contiguous, cleared together
+    uint64_t n_zeroed;
+    int32_t *coarse_counts;       // [copies * C * blocks]
+    int32_t *coarse_fill;         // same
+    int32_t *tile_counts;         // [tile copies * C * n_tiles]
+    int32_t *tile_fill;           // same
+    int32_t *coarse_starts;       // [copies * C * blocks]
+    int32_t *tile_starts;         // [tile copies * C * n_tiles]
     int64_t *block_sums;          // scan scratch
+    int64_t *cum_before;          // [total] (sort == false)
+    uint4 *entries;               // [n_isects] (sort == true), shares memory with cum_before
     uint64_t *pairs;              // [n_isects]
 };
 
-// Atomics on one cache line are serialised by the L2, and a tile table of a few thousand
-// counters is only a few hundred lines.  Every counter is therefore replicated `copies`
-// times (a power of two, chosen so that the table has about half a million entries);
-// workgroup b updates copy b % copies.  A tile's output segment is the concatenation of its
-// sub-segments, so nothing downstream sees the replication.  The table is laid out
-// [copy][segment]: lanes expanding one rectangle update neighbouring words of one line.
-static uint32_t isect_copies(uint64_t segs) {
+template <bool LIDAR>
+static CoarseGrid coarse_grid(const TileGrid &g) {
+    CoarseGrid cg;
+    cg.bshift = !LIDAR ? 2 : (g.tile_w % 4 == 0 ? 2 : (g.tile_w % 2 == 0 ? 1 : 0));
+    cg.cw = (g.tile_w + (1u << cg.bshift) - 1) >> cg.bshift;
+    cg.ch = (g.tile_h + (1u << kCoarseRowShift) - 1) >> kCoarseRowShift;
+    return cg;
+}
+
+// Copies of a counter table: a power of two chosen so that the table has about half a
+// million entries, i.e. thousands of cache lines for the atomics to spread over.
+static uint32_t isect_copies(uint64_t blocks) {
     uint32_t k = 1;
-    while (k < 256 && (uint64_t)(2 * k) * segs <= (1ull << 19)) k *= 2;
+    while (k < 256 && (uint64_t)(2 * k) * blocks <= (1ull << 19)) k *= 2;
     return k;
 }
 
-static size_t isect_ws_bytes(uint64_t total, uint64_t segs_in, int64_t n_isects) {
-    const uint64_t segs = segs_in * isect_copies(segs_in);
-    uint64_t scan_n = total > segs ? total : segs;
-    return 512 + 3 * splatad_align256(segs * 4) + splatad_align256(total * 8) +
-           scan_workspace_bytes((int64_t)scan_n) + splatad_align256((uint64_t)n_isects * 8);
-}
-
-static IsectWorkspace carve_isect(void *ws, uint64_t total, uint64_t segs_in) {
-    const uint64_t segs = segs_in * isect_copies(segs_in);
+// Layout from sizes only; cslots is the length of the replicated coarse counter table, or
+// an upper bound of it when only the number of tiles is known (workspace sizing).
+static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslots,
+                          int64_t n_isects, IsectWorkspace *out) {
+    const uint64_t tslots = segs * isect_copies(segs);
+    uint64_t scan_n = total > cslots ? total : cslots;
+    if (tslots > scan_n) scan_n = tslots;
     char *p = (char *)ws;
     IsectWorkspace w;
     w.n_isects = (unsigned long long *)p;   p += 256;
+    w.n_entries = (int64_t *)p;             p += 256;
     w.scan_total = (int64_t *)p;            p += 256;
-    w.tile_counts = (int32_t *)p;           p += splatad_align256(segs * 4);
-    w.tile_starts = (int32_t *)p;           p += splatad_align256(segs * 4);
-    w.tile_fill = (int32_t *)p;             p += splatad_align256(segs * 4);
-    w.cum_before = (int64_t *)p;            p += splatad_align256(total * 8);
-    uint64_t scan_n = total > segs ? total : segs;
+    w.zeroed = (int32_t *)p;
+    w.coarse_counts = (int32_t *)p;         p += splatad_align256(cslots * 4);
+    w.coarse_fill = (int32_t *)p;           p += splatad_align256(cslots * 4);
+    w.tile_counts = (int32_t *)p;           p += splatad_align256(tslots * 4);
+    w.tile_fill = (int32_t *)p;             p += splatad_align256(tslots * 4);
+    w.n_zeroed = (uint64_t)(p - (char *)w.zeroed) / 4;
+    w.coarse_starts = (int32_t *)p;         p += splatad_align256(cslots * 4);
+    w.tile_starts = (int32_t *)p;           p += splatad_align256(tslots * 4);
     w.block_sums = (int64_t *)p;            p += scan_workspace_bytes((int64_t)scan_n);
-    w.pairs = (uint64_t *)p;
-    return w;
+    const uint64_t list_bytes = splatad_align256((uint64_t)n_isects * 16);
+    const uint64_t cum_bytes = splatad_align256(total * 8);
+    w.cum_before = (int64_t *)p;
+    w.entries = (uint4 *)p;                 p += list_bytes > cum_bytes ? list_bytes : cum_bytes;
+    w.pairs = (uint64_t *)p;                p += splatad_align256((uint64_t)n_isects * 8);
+    if (out) *out = w;
+    return (size_t)(p - (char *)ws);
+}
+
+static size_t isect_ws_bytes(uint64_t total, uint64_t segs, int64_t n_isects) {
+    // there are at most as many coarse blocks as tiles, and isect_copies() keeps the table
+    // below 2^19 entries unless the blocks alone exceed that
+    const uint64_t cslots_bound = segs > (1ull << 19) ? segs : (1ull << 19);
+    return carve_isect(nullptr, total, segs, cslots_bound, n_isects, nullptr);
 }
 
 static inline dim3 grid_for(uint64_t n) {
@@ -583,7 +731,8 @@ static int isect_count(TileGrid g, uint64_t total, const float *means2d, const v
     SPLATAD_REQUIRE(n_tiles > 0 && C > 0, "isect: empty tile grid");
     SPLATAD_REQUIRE(splatad_bit_width(n_tiles) + splatad_bit_width(C) <= 32,
                     "isect: camera and tile ids need more than 32 bits");
-    IsectWorkspace w = carve_isect(workspace, total, (uint64_t)C * n_tiles);
+    IsectWorkspace w;
+    carve_isect(workspace, total, (uint64_t)C * n_tiles, 0, 0, &w);
     hipLaunchKernelGGL(fill_zero_u64_kernel, dim3(1), dim3(1), 0, stream, w.n_isects);
     hipLaunchKernelGGL(isect_count_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
                        stream, g, total, means2d, radii, tiles_per_gauss, w.n_isects);
@@ -609,11 +758,17 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     const uint32_t n_tiles = g.tile_w * g.tile_h;
     const uint32_t tile_n_bits = splatad_bit_width(n_tiles);
     const uint64_t segs = (uint64_t)C * n_tiles;
-    IsectWorkspace w = carve_isect(workspace, total, segs);
+    const CoarseGrid cg = coarse_grid<LIDAR>(g);
+    const uint64_t blocks = (uint64_t)C * cg.cw * cg.ch;
+    const uint32_t copies = isect_copies(blocks);
+    const uint64_t cslots = blocks * copies;
+    IsectWorkspace w;
+    carve_isect(workspace, total, segs, sort ? cslots : 0, n_isects, &w);
+    int rc;
     if (!sort) {
         SPLATAD_REQUIRE(tiles_per_gauss != nullptr, "isect: tiles_per_gauss is null");
-        int rc = launch_exclusive_scan<int64_t>(tiles_per_gauss, (int64_t)total, 1, 0,
-                                                w.cum_before, w.scan_total, w.block_sums, stream);
+        rc = launch_exclusive_scan<int64_t>(tiles_per_gauss, (int64_t)total, 1, 0, w.cum_before,
+                                            w.scan_total, w.block_sums, stream);
         if (rc) return rc;
         hipLaunchKernelGGL(isect_emit_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
                            stream, g, total, N, camera_ids, means2d, radii, depths,
@@ -621,25 +776,42 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         SPLATAD_LAUNCH_CHECK();
         return 0;
     }
-    const uint32_t copies = isect_copies(segs);
-    const uint64_t slots = segs * copies;
-    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(slots), dim3(SPLATAD_THREADS), 0, stream,
-                       w.tile_counts, (int64_t)slots);
-    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(slots), dim3(SPLATAD_THREADS), 0, stream,
-                       w.tile_fill, (int64_t)slots);
-    hipLaunchKernelGGL(isect_histogram_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
-                       stream, g, total, N, camera_ids, means2d, radii, copies, (uint32_t)segs,
-                       w.tile_counts);
+    SPLATAD_REQUIRE(blocks < (1ull << 32) && cslots < (1ull << 31), "isect: tile grid too large");
+    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(w.n_zeroed), dim3(SPLATAD_THREADS), 0, stream,
+                       w.zeroed, (int64_t)w.n_zeroed);
+    // coarse lists: count, scan (the table is stored [copy][block] and scanned block-major,
+    // which makes a block's list contiguous), fill
+    hipLaunchKernelGGL(isect_coarse_count_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
+                       stream, g, cg, total, N, camera_ids, means2d, radii, copies,
+                       (uint32_t)blocks, w.coarse_counts);
     SPLATAD_LAUNCH_CHECK();
-    // counters are stored [copy][segment] (so that a wavefront's atomics on neighbouring
-    // tiles share cache lines) and scanned segment-major
-    int rc = launch_exclusive_scan<int32_t>(w.tile_counts, (int64_t)slots,
-                                            copies > 1 ? -(int)copies : 1, 0, w.tile_starts,
-                                            w.scan_total, w.block_sums, stream);
+    rc = launch_exclusive_scan<int32_t>(w.coarse_counts, (int64_t)cslots,
+                                        copies > 1 ? -(int)copies : 1, 0, w.coarse_starts,
+                                        w.n_entries, w.block_sums, stream);
     if (rc) return rc;
-    hipLaunchKernelGGL(isect_scatter_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
-                       stream, g, total, N, camera_ids, means2d, radii, depths, copies,
-                       (uint32_t)segs, w.tile_starts, w.tile_fill, w.pairs);
+    hipLaunchKernelGGL(isect_coarse_fill_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
+                       stream, g, cg, total, N, camera_ids, means2d, radii, depths, copies,
+                       (uint32_t)blocks, w.coarse_starts, w.coarse_fill, w.entries);
+    SPLATAD_LAUNCH_CHECK();
+    // tile segments: count, scan, fill.  The number of coarse entries stays on the device;
+    // the grid is sized for the bound n_isects and strides.
+    const uint32_t tcopies = isect_copies(segs);
+    uint64_t bin_wgs = ((uint64_t)n_isects + SPLATAD_THREADS - 1) / SPLATAD_THREADS;
+    if (bin_wgs > 8192) bin_wgs = 8192;
+    hipLaunchKernelGGL(isect_tile_bin_kernel<false>, dim3((uint32_t)bin_wgs),
+                       dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, tcopies,
+                       (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
+                       w.tile_counts, (const int32_t *)nullptr, (int32_t *)nullptr,
+                       (uint64_t *)nullptr);
+    SPLATAD_LAUNCH_CHECK();
+    rc = launch_exclusive_scan<int32_t>(w.tile_counts, (int64_t)(segs * tcopies),
+                                        tcopies > 1 ? -(int)tcopies : 1, 0, w.tile_starts,
+                                        w.scan_total, w.block_sums, stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL(isect_tile_bin_kernel<true>, dim3((uint32_t)bin_wgs),
+                       dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, tcopies,
+                       (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
+                       w.tile_counts, (const int32_t *)w.tile_starts, w.tile_fill, w.pairs);
     SPLATAD_LAUNCH_CHECK();
     // Size classes: each launch visits every segment and only works on those of its class, so
     // that the LDS per workgroup (and with it the number of resident workgroups) fits the
