@@ -112,6 +112,12 @@ __device__ __forceinline__ Mat3 quat_to_rotmat(float w, float x, float y, float 
 }
 
 // Sum over the 64 lanes of a wavefront; every lane gets the total.
+// Lane mask of a predicate.  Unlike __ballot(int) this takes the condition as it is held
+// (one bit per lane in a scalar register pair), without a round trip through a vector register.
+__device__ __forceinline__ uint64_t wave_ballot(bool pred) {
+    return __builtin_amdgcn_ballot_w64(pred);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, SPLATAD_WAVE);

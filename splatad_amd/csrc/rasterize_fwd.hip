@@ -34,27 +34,74 @@ struct PixelArgs {
     int write_aux; // first pass also writes alphas and last ids
 };
 
+// Conservative test of one Gaussian against the footprint of a wavefront.  With the staged
+// record {A, B, C, L} (see the kernel), alpha = exp2(L - p(d)), p(d) = A dx^2 + B dx dy +
+// C dy^2.  The smallest value of p over the box of offsets d = mean - pixel that the
+// wavefront's pixels can see (widened by the rolling-shutter shift of the mean across the
+// wavefront's rows) is compared with the largest p that still passes the alpha >= 1/255
+// test, L + log2(255).  p is convex for a positive definite conic, so off the centre its
+// minimum over the box lies on one of the four edges.  A margin covers the rounding of this
+// test; Gaussians with a degenerate conic are never culled.
+struct WaveCull {
+    bool enabled;
+    float cx, cy;     // centre of the footprint
+    float hx, hy;     // half extents
+    float roll_mid, roll_half;
+
+    __device__ __forceinline__ static float edge_min(float a2, float c2, float b, float fixed,
+                                                     float lo, float hi) {
+        // fixed coordinate uses a2 (= a / 2), free coordinate uses c2 (= c / 2)
+        const float free_c = fminf(fmaxf(-b * fixed / (2.f * c2), lo), hi);
+        return a2 * fixed * fixed + c2 * free_c * free_c + b * fixed * free_c;
+    }
+
+    __device__ __forceinline__ bool may_touch(const float4 xyv, const float4 con) const {
+        const float mx = xyv.x + roll_mid * xyv.z - cx, my = xyv.y + roll_mid * xyv.w - cy;
+        const float ex = hx + fabsf(xyv.z) * roll_half, ey = hy + fabsf(xyv.w) * roll_half;
+        const float x0 = mx - ex, x1 = mx + ex, y0 = my - ey, y1 = my + ey;
+        const float a2 = con.x, c2 = con.z, b = con.y;
+        const bool definite = a2 > 0.f && c2 > 0.f && 4.f * a2 * c2 - b * b > 0.f;
+        const bool centre_in = x0 <= 0.f && x1 >= 0.f && y0 <= 0.f && y1 >= 0.f;
+        const float q = fminf(fminf(edge_min(a2, c2, b, x0, y0, y1), edge_min(a2, c2, b, x1, y0, y1)),
+                              fminf(edge_min(c2, a2, b, y0, x0, x1), edge_min(c2, a2, b, y1, x0, x1)));
+        const float limit = con.w + 7.99435343685886f; // log2(255)
+        const bool cull = definite && !centre_in && q > limit + 1e-3f * fabsf(limit) + 0.02f;
+        return !cull;
+    }
+};
+
 template <int CH>
 __global__ void __launch_bounds__(1024)
 rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     extern __shared__ float4 lds4[];
     const uint32_t block_size = blockDim.x * blockDim.y;
-    float4 *s_xyv = lds4;                           // {x, y, vx, vy}
-    float4 *s_con = lds4 + block_size;              // {conic a, b, c, opacity}
-    float *s_col = reinterpret_cast<float *>(lds4 + 2 * block_size); // [block_size][CH]
+    // per Gaussian: {x, y, vx, vy} and {A, B, C, L}, where sigma * log2(e) = A dx^2 + B dx dy +
+    // C dy^2 and L = log2(opacity), so that alpha = exp2(L - (A dx^2 + B dx dy + C dy^2))
+    // followed by the CH colours, padded to a multiple of four floats
+    constexpr int RECORD = 2 + (CH + 3) / 4; // float4 per Gaussian
+    float4 *s_rec = lds4;
 
     const uint32_t tiles_per_cam = a.tile_w * a.tile_h;
     const uint32_t cam = blockIdx.x / tiles_per_cam;
     const uint32_t tile_id = blockIdx.x % tiles_per_cam;
     const uint32_t tile_y = tile_id / a.tile_w, tile_x = tile_id % a.tile_w;
-    const uint32_t i = tile_y * a.tile_size + threadIdx.y;
-    const uint32_t j = tile_x * a.tile_size + threadIdx.x;
     const uint32_t tr = threadIdx.y * blockDim.x + threadIdx.x;
+    const uint32_t lane = tr & (SPLATAD_WAVE - 1);
+    // pixel of this lane: wavefronts cover 8x8 squares when the tile allows it (a compact
+    // footprint is what makes the per-wavefront culling below effective), rows otherwise
+    uint32_t lx = threadIdx.x, ly = threadIdx.y;
+    if (a.tile_size % 8 == 0) {
+        const uint32_t squares_per_row = a.tile_size / 8, square = tr / SPLATAD_WAVE;
+        lx = (square % squares_per_row) * 8 + (lane & 7);
+        ly = (square / squares_per_row) * 8 + (lane >> 3);
+    }
+    const uint32_t i = tile_y * a.tile_size + ly;
+    const uint32_t j = tile_x * a.tile_size + lx;
 
     const float px = (float)j + 0.5f, py = (float)i + 0.5f;
     const float roll = a.rs_time[cam] * ((py - 0.5f) / (float)(a.H - 1) - 0.5f);
     const bool inside = (i < a.H && j < a.W);
-    bool done = !inside;
+    bool alive = inside; // still compositing
 
     const int32_t *offs = a.tile_offsets + (size_t)cam * tiles_per_cam;
     const int32_t range_start = offs[tile_id];
@@ -62,6 +109,28 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
                                   ? (int32_t)a.n_isects
                                   : offs[tile_id + 1];
     const uint32_t num_batches = (uint32_t)(range_end - range_start + block_size - 1) / block_size;
+
+    // footprint of this wavefront (all 64 lanes exist when the workgroup is a multiple of 64)
+    WaveCull cull;
+    cull.enabled = block_size % SPLATAD_WAVE == 0;
+    {
+        float x_lo = px, x_hi = px, y_lo = py, y_hi = py, r_lo = roll, r_hi = roll;
+        if (cull.enabled) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                x_lo = fminf(x_lo, __shfl_xor(x_lo, off, SPLATAD_WAVE));
+                x_hi = fmaxf(x_hi, __shfl_xor(x_hi, off, SPLATAD_WAVE));
+                y_lo = fminf(y_lo, __shfl_xor(y_lo, off, SPLATAD_WAVE));
+                y_hi = fmaxf(y_hi, __shfl_xor(y_hi, off, SPLATAD_WAVE));
+                r_lo = fminf(r_lo, __shfl_xor(r_lo, off, SPLATAD_WAVE));
+                r_hi = fmaxf(r_hi, __shfl_xor(r_hi, off, SPLATAD_WAVE));
+            }
+        }
+        cull.cx = 0.5f * (x_lo + x_hi); cull.hx = 0.5f * (x_hi - x_lo);
+        cull.cy = 0.5f * (y_lo + y_hi); cull.hy = 0.5f * (y_hi - y_lo);
+        cull.roll_mid = 0.5f * (r_lo + r_hi);
+        cull.roll_half = 0.5f * (r_hi - r_lo) * 1.0001f + 1e-12f;
+    }
 
     float T = 1.0f;
     uint32_t cur_idx = 0;
@@ -71,7 +140,7 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
 
     for (uint32_t b = 0; b < num_batches; ++b) {
         // also orders the previous batch's LDS reads before this batch's writes
-        if (__syncthreads_count(done) >= (int)block_size) break;
+        if (__syncthreads_count(!alive) >= (int)block_size) break;
 
         const uint32_t batch_start = (uint32_t)range_start + block_size * b;
         const uint32_t idx = batch_start + tr;
@@ -80,33 +149,50 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
             const float2 xy = reinterpret_cast<const float2 *>(a.means2d)[g];
             const float2 v = reinterpret_cast<const float2 *>(a.pix_vels)[g];
             const float *cn = a.conics + (size_t)g * 3;
-            s_xyv[tr] = make_float4(xy.x, xy.y, v.x, v.y);
-            s_con[tr] = make_float4(cn[0], cn[1], cn[2], a.opacities[g]);
+            constexpr float kLog2e = 1.44269504088896341f;
+            const float opac = a.opacities[g];
+            s_rec[RECORD * tr] = make_float4(xy.x, xy.y, v.x, v.y);
+            s_rec[RECORD * tr + 1] = make_float4(0.5f * kLog2e * cn[0], kLog2e * cn[1],
+                                            0.5f * kLog2e * cn[2], opac > 0.f ? __log2f(opac) : -INFINITY);
             const float *c = a.colors + (size_t)g * a.color_stride + a.ch_offset;
 #pragma unroll
-            for (int k = 0; k < CH; ++k) s_col[tr * CH + k] = (uint32_t)k < a.n_ch ? c[k] : 0.f;
+            for (int k = 0; k < CH; ++k)
+                reinterpret_cast<float *>(s_rec + RECORD * tr + 2)[k] = (uint32_t)k < a.n_ch ? c[k] : 0.f;
         }
         __syncthreads();
 
         const uint32_t batch_size = min(block_size, (uint32_t)range_end - batch_start);
-        for (uint32_t t = 0; t < batch_size && !done; ++t) {
-            const float4 xyv = s_xyv[t];
-            const float4 con = s_con[t];
-            const float dx = xyv.x + roll * xyv.z - px;
-            const float dy = xyv.y + roll * xyv.w - py;
-            const float sigma = 0.5f * (con.x * dx * dx + con.z * dy * dy) + con.y * dx * dy;
-            const float alpha = fminf(0.999f, con.w * __expf(-sigma));
-            if (sigma < 0.f || alpha < 1.f / 255.f) continue;
-            const float next_T = T * (1.0f - alpha);
-            if (next_T <= 1e-4f) {
-                done = true;
-                break;
-            }
-            const float vis = alpha * T;
+        for (uint32_t base = 0; base < batch_size && wave_ballot(alive); base += SPLATAD_WAVE) {
+            // lanes test 64 Gaussians against the wavefront's footprint, then all lanes walk
+            // the survivors (a wave-uniform loop over the set bits)
+            bool keep = base + lane < batch_size;
+            if (keep && cull.enabled) keep = cull.may_touch(s_rec[RECORD * (base + lane)], s_rec[RECORD * (base + lane) + 1]);
+            uint64_t todo = wave_ballot(keep);
+            while (todo) {
+                const uint32_t t = base + (uint32_t)__ffsll((unsigned long long)todo) - 1u;
+                todo &= todo - 1;
+                const float4 *rec = s_rec + RECORD * t;
+                const float4 xyv = rec[0];
+                const float4 con = rec[1];
+                const float dx = (xyv.x + roll * xyv.z) - px;
+                const float dy = (xyv.y + roll * xyv.w) - py;
+                const float power = dx * (con.x * dx + con.y * dy) + con.z * dy * dy;
+                const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
+                const float next_T = T * (1.0f - alpha);
+                // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
+                const bool valid = alive && !(power < 0.f) && !(alpha < 1.f / 255.f);
+                const bool stop = valid && next_T <= 1e-4f;
+                const bool take = valid && !stop;
+                alive = alive && !stop;
+                if (CH > 8 ? wave_ballot(take) != 0 : true) {
+                    const float vis = take ? alpha * T : 0.f;
 #pragma unroll
-            for (int k = 0; k < CH; ++k) out[k] += s_col[t * CH + k] * vis;
-            cur_idx = batch_start + t;
-            T = next_T;
+                    for (int k = 0; k < CH; ++k) out[k] += reinterpret_cast<const float *>(rec + 2)[k] * vis;
+                }
+                cur_idx = take ? batch_start + t : cur_idx;
+                T = take ? next_T : T;
+                if (wave_ballot(alive) == 0) break;
+            }
         }
     }
 
@@ -271,7 +357,7 @@ static inline int pick_width(uint32_t n) {
 
 template <int CH>
 static int launch_pixels(const PixelArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
-    const size_t lds = (size_t)block.x * block.y * (32 + 4 * CH);
+    const size_t lds = (size_t)block.x * block.y * 16 * (2 + (CH + 3) / 4);
     if (lds > 64 * 1024)
         SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_to_pixels_fwd_kernel<CH>,
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
