@@ -227,31 +227,74 @@ struct PointArgs {
     int write_aux;
 };
 
-// fmodf(a - b + 180, 360) - 180, folded into (-180, 180]; the common case (argument of
-// fmodf already in [0, 360)) skips the library call, with the same result.
+// Difference of two angles in degrees folded into [-180, 180), as the reference's
+// fmodf(a - b + 180, 360) - 180 with negative results raised by 360.  Without the detour
+// through +180 / -180 the difference of two nearby angles is exact in float32.
 __device__ __forceinline__ float angle_difference(float a, float b) {
-    const float d = a - b + 180.f;
-    const float m = (d >= 0.f && d < 360.f) ? d : fmodf(d, 360.f);
-    const float r = m - 180.f;
-    return r < -180.f ? r + 360.f : r;
+    const float d = a - b;
+    if (d >= -180.f && d < 180.f) return d;
+    float m = fmodf(d + 180.f, 360.f);
+    if (m < 0.f) m += 360.f;
+    return m - 180.f;
 }
+
+// Footprint test for a wavefront of lidar points, the counterpart of WaveCull.  All angles
+// are taken relative to a reference point of the tile, so that neither the +-180 degree
+// seam nor the size of the absolute angles matters: the staged record holds u = (mean -
+// reference) and the lane r = (point - reference), both folded, and the offset of a pair is
+// u + roll * velocity - r as long as that cannot leave (-180, 180).  The test decides for
+// every Gaussian whether any lane can reach alpha >= 1/255 and whether the unfolded
+// difference is safe (it is unless the Gaussian sits half a turn away from the tile).
+struct WavePointCull {
+    bool enabled;
+    float x_lo, x_hi, y_lo, y_hi; // box of the lanes' r
+    float roll_mid, roll_half;
+
+    __device__ __forceinline__ bool may_touch(const float4 uv, const float4 con, bool &unfolded_ok) const {
+        const float cx = uv.x + roll_mid * uv.z, cy = uv.y + roll_mid * uv.w;
+        const float ex = fabsf(uv.z) * roll_half, ey = fabsf(uv.w) * roll_half;
+        const float x0 = cx - x_hi - ex, x1 = cx - x_lo + ex;
+        const float y0 = cy - y_hi - ey, y1 = cy - y_lo + ey;
+        unfolded_ok = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(y0), fabsf(y1))) < 179.f;
+        if (!unfolded_ok || !enabled) return true;
+        const float a2 = con.x, c2 = con.z, b = con.y;
+        const bool definite = a2 > 0.f && c2 > 0.f && 4.f * a2 * c2 - b * b > 0.f;
+        const bool centre_in = x0 <= 0.f && x1 >= 0.f && y0 <= 0.f && y1 >= 0.f;
+        const float q = fminf(fminf(WaveCull::edge_min(a2, c2, b, x0, y0, y1), WaveCull::edge_min(a2, c2, b, x1, y0, y1)),
+                              fminf(WaveCull::edge_min(c2, a2, b, y0, x0, x1), WaveCull::edge_min(c2, a2, b, y1, x0, x1)));
+        const float limit = con.w + 7.99435343685886f; // log2(255)
+        const bool cull = definite && !centre_in && q > limit + 1e-3f * fabsf(limit) + 0.02f;
+        return !cull;
+    }
+};
 
 template <int CH>
 __global__ void __launch_bounds__(256)
 rasterize_to_points_fwd_kernel(PointArgs a) {
     extern __shared__ float4 lds4[];
+    __shared__ uint32_t s_ref_thread;
+    __shared__ float s_ref[2];
     const uint32_t block_size = blockDim.x * blockDim.y;
-    float4 *s_xyv = lds4;                  // {az, el, v_az, v_el}
-    float4 *s_con = lds4 + block_size;     // {conic a, b, c, opacity}
-    float4 *s_ext = lds4 + 2 * block_size; // {v_range, depth comp 0, depth comp 1, depth}
-    float *s_col = reinterpret_cast<float *>(lds4 + 3 * block_size);
+    // per Gaussian: {u_az, u_el, v_az, v_el} (u relative to the tile's reference point),
+    // {A, B, C, L} as in the pixel kernel, {v_range, depth comp 0, depth comp 1, depth} and
+    // the CH colours padded to a multiple of four floats
+    constexpr int RECORD = 3 + (CH + 3) / 4; // float4 per Gaussian
+    float4 *s_rec = lds4;
 
     const uint32_t tiles_per_cam = a.grid_w * a.grid_h;
     const uint32_t cam = blockIdx.x / tiles_per_cam;
     const uint32_t tile_id = blockIdx.x % tiles_per_cam;
-    const uint32_t i = (tile_id / a.grid_w) * a.tile_height + threadIdx.y;
-    const uint32_t j = (tile_id % a.grid_w) * a.tile_width + threadIdx.x;
     const uint32_t tr = threadIdx.y * blockDim.x + threadIdx.x;
+    const uint32_t lane = tr & (SPLATAD_WAVE - 1);
+    // point of this lane: a wavefront covers 16 columns of all four rows when the tile
+    // allows it (the compact footprint culls better than one row of 64 columns)
+    uint32_t lx = threadIdx.x, ly = threadIdx.y;
+    if (a.tile_height == 4 && a.tile_width % 16 == 0) {
+        lx = (tr / SPLATAD_WAVE) * 16 + (lane & 15);
+        ly = lane >> 4;
+    }
+    const uint32_t i = (tile_id / a.grid_w) * a.tile_height + ly;
+    const uint32_t j = (tile_id % a.grid_w) * a.tile_width + lx;
 
     const bool in_image = (i < a.H && j < a.W);
     const size_t pix = ((size_t)cam * a.H + i) * a.W + j;
@@ -261,15 +304,56 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
         px = p.x; py = p.y; pz = p.z; roll = p.w;
     }
     const bool inside = in_image && pz > 0.f;
-    bool done = !inside;
+    bool alive = inside;
+
+    // reference point of the tile: its first valid point
+    if (tr == 0) s_ref_thread = 0xFFFFFFFFu;
+    __syncthreads();
+    if (inside) atomicMin(&s_ref_thread, tr);
+    __syncthreads();
+    if (tr == s_ref_thread) { s_ref[0] = px; s_ref[1] = py; }
+    __syncthreads();
+    const bool any_point = s_ref_thread != 0xFFFFFFFFu; // uniform
+    const float ref_x = any_point ? s_ref[0] : 0.f, ref_y = any_point ? s_ref[1] : 0.f;
+    const float rx = angle_difference(px, ref_x), ry = angle_difference(py, ref_y);
 
     const int32_t *offs = a.tile_offsets + (size_t)cam * tiles_per_cam;
     const int32_t range_start = offs[tile_id];
     const int32_t range_end = (cam == a.C - 1 && tile_id == tiles_per_cam - 1)
                                   ? (int32_t)a.n_isects
                                   : offs[tile_id + 1];
-    const uint32_t num_batches = (uint32_t)(range_end - range_start + block_size - 1) / block_size;
+    const uint32_t num_batches =
+        any_point ? (uint32_t)(range_end - range_start + block_size - 1) / block_size : 0u;
     const bool has_depth = a.depth_idx >= a.ch_offset && a.depth_idx < a.ch_offset + a.n_ch;
+
+    // footprint of this wavefront over its valid lanes
+    WavePointCull cull;
+    cull.enabled = block_size % SPLATAD_WAVE == 0;
+    {
+        const float inf = INFINITY;
+        float x_lo = alive ? rx : inf, x_hi = alive ? rx : -inf;
+        float y_lo = alive ? ry : inf, y_hi = alive ? ry : -inf;
+        float r_lo = alive ? roll : inf, r_hi = alive ? roll : -inf;
+        if (cull.enabled) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                x_lo = fminf(x_lo, __shfl_xor(x_lo, off, SPLATAD_WAVE));
+                x_hi = fmaxf(x_hi, __shfl_xor(x_hi, off, SPLATAD_WAVE));
+                y_lo = fminf(y_lo, __shfl_xor(y_lo, off, SPLATAD_WAVE));
+                y_hi = fmaxf(y_hi, __shfl_xor(y_hi, off, SPLATAD_WAVE));
+                r_lo = fminf(r_lo, __shfl_xor(r_lo, off, SPLATAD_WAVE));
+                r_hi = fmaxf(r_hi, __shfl_xor(r_hi, off, SPLATAD_WAVE));
+            }
+        } else { // partial wavefront: no culling, bounds of the whole (-180, 180] range
+            x_lo = y_lo = -180.f; x_hi = y_hi = 180.f;
+            r_lo = r_hi = roll;
+        }
+        // slightly widened against the rounding of the test itself
+        cull.x_lo = x_lo - 1e-4f; cull.x_hi = x_hi + 1e-4f;
+        cull.y_lo = y_lo - 1e-4f; cull.y_hi = y_hi + 1e-4f;
+        cull.roll_mid = 0.5f * (r_lo + r_hi);
+        cull.roll_half = 0.5f * (r_hi - r_lo) * 1.0001f + 1e-12f;
+    }
 
     float T = 1.0f, asum = 0.f, median = 0.f, depth_extra = 0.f;
     uint32_t cur_idx = 0;
@@ -278,7 +362,8 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
     for (int k = 0; k < CH; ++k) out[k] = 0.f;
 
     for (uint32_t b = 0; b < num_batches; ++b) {
-        if (__syncthreads_count(done) >= (int)block_size) break;
+        // also orders the previous batch's LDS reads before this batch's writes
+        if (__syncthreads_count(!alive) >= (int)block_size) break;
         const uint32_t batch_start = (uint32_t)range_start + block_size * b;
         const uint32_t idx = batch_start + tr;
         if (idx < (uint32_t)range_end) {
@@ -288,39 +373,61 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
             const float2 dc = reinterpret_cast<const float2 *>(a.depth_comps)[g];
             const float *cn = a.conics + (size_t)g * 3;
             const float *crow = a.colors + (size_t)g * a.color_stride;
-            s_xyv[tr] = make_float4(xy.x, xy.y, v[0], v[1]);
-            s_con[tr] = make_float4(cn[0], cn[1], cn[2], a.opacities[g]);
-            s_ext[tr] = make_float4(v[2], dc.x, dc.y, crow[a.depth_idx]);
+            constexpr float kLog2e = 1.44269504088896341f;
+            const float opac = a.opacities[g];
+            float4 *rec = s_rec + RECORD * tr;
+            rec[0] = make_float4(angle_difference(xy.x, ref_x), angle_difference(xy.y, ref_y), v[0], v[1]);
+            rec[1] = make_float4(0.5f * kLog2e * cn[0], kLog2e * cn[1], 0.5f * kLog2e * cn[2],
+                                 opac > 0.f ? __log2f(opac) : -INFINITY);
+            rec[2] = make_float4(v[2], dc.x, dc.y, crow[a.depth_idx]);
             const float *c = crow + a.ch_offset;
 #pragma unroll
-            for (int k = 0; k < CH; ++k) s_col[tr * CH + k] = (uint32_t)k < a.n_ch ? c[k] : 0.f;
+            for (int k = 0; k < CH; ++k)
+                reinterpret_cast<float *>(rec + 3)[k] = (uint32_t)k < a.n_ch ? c[k] : 0.f;
         }
         __syncthreads();
 
         const uint32_t batch_size = min(block_size, (uint32_t)range_end - batch_start);
-        for (uint32_t t = 0; t < batch_size && !done; ++t) {
-            const float4 xyv = s_xyv[t];
-            const float4 con = s_con[t];
-            const float dx = angle_difference(xyv.x + roll * xyv.z, px);
-            const float dy = angle_difference(xyv.y + roll * xyv.w, py);
-            const float sigma = 0.5f * (con.x * dx * dx + con.z * dy * dy) + con.y * dx * dy;
-            const float alpha = fminf(0.999f, con.w * __expf(-sigma));
-            if (sigma < 0.f || alpha < 1.f / 255.f) continue;
-            const float next_T = T * (1.0f - alpha);
-            if (next_T <= 1e-4f) {
-                done = true;
-                break;
-            }
-            const float vis = alpha * T;
+        for (uint32_t base = 0; base < batch_size && wave_ballot(alive); base += SPLATAD_WAVE) {
+            bool keep = base + lane < batch_size, unfolded_ok = true;
+            if (keep) keep = cull.may_touch(s_rec[RECORD * (base + lane)], s_rec[RECORD * (base + lane) + 1], unfolded_ok);
+            uint64_t todo = wave_ballot(keep);
+            const uint64_t folded = wave_ballot(keep && !unfolded_ok);
+            while (todo) {
+                const uint32_t bit = (uint32_t)__ffsll((unsigned long long)todo) - 1u;
+                const uint32_t t = base + bit;
+                todo &= todo - 1;
+                const float4 *rec = s_rec + RECORD * t;
+                const float4 uv = rec[0];
+                const float4 con = rec[1];
+                float dx = (uv.x + roll * uv.z) - rx;
+                float dy = (uv.y + roll * uv.w) - ry;
+                if ((folded >> bit) & 1ull) { // uniform, rare: half a turn away from the tile
+                    dx = angle_difference(uv.x + roll * uv.z, rx);
+                    dy = angle_difference(uv.y + roll * uv.w, ry);
+                }
+                const float power = dx * (con.x * dx + con.y * dy) + con.z * dy * dy;
+                const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
+                const float next_T = T * (1.0f - alpha);
+                // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
+                const bool valid = alive && !(power < 0.f) && !(alpha < 1.f / 255.f);
+                const bool stop = valid && next_T <= 1e-4f;
+                const bool take = valid && !stop;
+                alive = alive && !stop;
+                if (wave_ballot(take) != 0) {
+                    const float vis = take ? alpha * T : 0.f;
 #pragma unroll
-            for (int k = 0; k < CH; ++k) out[k] += s_col[t * CH + k] * vis;
-            const float4 ext = s_ext[t];
-            const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
-            depth_extra += extra * vis;
-            if (T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
-            if (a.compute_alpha_sum && ext.w < pz - a.threshold) asum += alpha;
-            cur_idx = batch_start + t;
-            T = next_T;
+                    for (int k = 0; k < CH; ++k) out[k] += reinterpret_cast<const float *>(rec + 3)[k] * vis;
+                    const float4 ext = rec[2];
+                    const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
+                    depth_extra += extra * vis;
+                    if (take && T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
+                    if (take && a.compute_alpha_sum && ext.w < pz - a.threshold) asum += alpha;
+                    cur_idx = take ? batch_start + t : cur_idx;
+                    T = take ? next_T : T;
+                }
+                if (wave_ballot(alive) == 0) break;
+            }
         }
     }
 
@@ -368,7 +475,7 @@ static int launch_pixels(const PixelArgs &a, dim3 grid, dim3 block, hipStream_t 
 
 template <int CH>
 static int launch_points(const PointArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
-    const size_t lds = (size_t)block.x * block.y * (48 + 4 * CH);
+    const size_t lds = (size_t)block.x * block.y * 16 * (3 + (CH + 3) / 4);
     hipLaunchKernelGGL(rasterize_to_points_fwd_kernel<CH>, grid, block, lds, stream, a);
     SPLATAD_LAUNCH_CHECK();
     return 0;
