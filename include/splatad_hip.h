@@ -134,7 +134,10 @@ int splatad_sh_bwd(uint32_t n, uint32_t K, uint32_t degree, const float *dirs,
  * elev_boundaries has tile_height+1 entries.  The workspace of _count needs
  * splatad_isect_workspace_bytes(total, C, n_tiles, 0) bytes, that of _fill
  * splatad_isect_workspace_bytes(total, C, n_tiles, n_isects); nothing has to
- * survive between the two calls except tiles_per_gauss. */
+ * survive between the two calls except tiles_per_gauss.  tile_offsets may be
+ * NULL; with sort != 0 it receives the [C, tile_height, tile_width] table that
+ * splatad_isect_offset_encode would derive from isect_ids (the binning knows
+ * every tile's first intersection before the sort runs). */
 size_t splatad_isect_workspace_bytes(uint64_t total, uint32_t C, uint32_t n_tiles,
                                      int64_t n_isects);
 int splatad_isect_tiles_count(uint64_t total, const float *means2d, const int32_t *radii,
@@ -146,7 +149,8 @@ int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_i
                              uint32_t C, uint32_t tile_size, uint32_t tile_width,
                              uint32_t tile_height, int sort, int64_t n_isects,
                              const int32_t *tiles_per_gauss, void *workspace, int64_t *isect_ids,
-                             int32_t *flatten_ids, splatad_stream_t stream);
+                             int32_t *flatten_ids, int32_t *tile_offsets,
+                             splatad_stream_t stream);
 int splatad_isect_lidar_tiles_count(uint64_t total, const float *means2d, const float *radii,
                                     uint32_t C, const float *elev_boundaries,
                                     float tile_azim_resolution, float min_azim,
@@ -160,7 +164,7 @@ int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N, const int64_t *ca
                                    uint32_t tile_width, uint32_t tile_height, int sort,
                                    int64_t n_isects, const int32_t *tiles_per_gauss,
                                    void *workspace, int64_t *isect_ids, int32_t *flatten_ids,
-                                   splatad_stream_t stream);
+                                   int32_t *tile_offsets, splatad_stream_t stream);
 
 /* isect_offset_encode_tensor, rasterization.cu:264-285 (kernel :218-262). */
 int splatad_isect_offset_encode(int64_t n_isects, const int64_t *isect_ids, uint32_t C,

@@ -39,6 +39,27 @@ __device__ __forceinline__ uint32_t f2u_sat(float v) {
     return (uint32_t)v;
 }
 
+// Number of leading boundaries below v (boundaries ascending).
+__device__ __forceinline__ int32_t elev_lower_bound(const float *b, int32_t count, float v) {
+    int32_t lo = 0, hi = count;
+    while (lo < hi) {
+        const int32_t mid = (lo + hi) >> 1;
+        if (b[mid] < v) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
+// Lidar kernels read the elevation boundaries from LDS when they fit.
+constexpr uint32_t kElevLds = 1025;
+#define SPLATAD_STAGE_ELEVATIONS(g)                                                          \
+    __shared__ float s_elev[kElevLds];                                                       \
+    if (LIDAR && (g).tile_h + 1 <= kElevLds) {                                               \
+        for (uint32_t e = threadIdx.x; e <= (g).tile_h; e += blockDim.x)                     \
+            s_elev[e] = (g).elev_boundaries[e];                                              \
+        __syncthreads();                                                                     \
+        (g).elev_boundaries = s_elev;                                                        \
+    }
+
 // Tile rectangle of one projected Gaussian: x in [x0, x1), y in [y0, y1).  For lidars x
 // may be negative or exceed tile_w (wrapped at emission).
 template <bool LIDAR>
@@ -74,12 +95,14 @@ __device__ __forceinline__ bool tile_rect(const TileGrid &g, const float *__rest
             t_high = (float)g.tile_w + fmodf(azim_high + 360.f, 360.f) / g.azim_res;
         x0 = (int32_t)floorf(t_low);
         x1 = (int32_t)ceilf(t_high);
+        // The reference walks the boundaries upwards (rasterization.cu:346-356): i = first
+        // boundary >= elev_low, then on to the first >= elev_high.  For ascending boundaries
+        // these are two lower bounds, found here by bisection.
         const int32_t n = (int32_t)g.tile_h;
-        int32_t i = 0;
-        while (i <= n && g.elev_boundaries[i] < elev_low) ++i;
-        y0 = max(i - 1, 0);
-        while (i <= n && g.elev_boundaries[i] < elev_high) ++i;
-        y1 = min(i, n);
+        const int32_t i_low = elev_lower_bound(g.elev_boundaries, n + 1, elev_low);
+        const int32_t i_high = max(i_low, elev_lower_bound(g.elev_boundaries, n + 1, elev_high));
+        y0 = max(i_low - 1, 0);
+        y1 = min(i_high, n);
     }
     return true;
 }
@@ -96,20 +119,22 @@ __device__ __forceinline__ uint32_t tile_index(const TileGrid &g, int32_t y, int
     return (uint32_t)y * g.tile_w + (uint32_t)x;
 }
 
+// Grid-stride: a few hundred workgroups, each ending in one atomic on the total (thousands
+// of atomics on one address would take longer than the rest of the kernel).
 template <bool LIDAR>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d,
                    const void *__restrict__ radii, int32_t *__restrict__ tiles_per_gauss,
                    unsigned long long *__restrict__ n_isects) {
-    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    int32_t cnt = 0;
-    if (idx < total) {
-        int32_t x0, y0, x1, y1;
+    SPLATAD_STAGE_ELEVATIONS(g)
+    long long s = 0;
+    for (uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (uint64_t)gridDim.x * blockDim.x) {
+        int32_t cnt = 0, x0, y0, x1, y1;
         if (tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) cnt = (y1 - y0) * (x1 - x0);
         tiles_per_gauss[idx] = cnt;
+        s += cnt;
     }
-    // workgroup total -> one atomic per workgroup
-    long long s = cnt;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, SPLATAD_WAVE);
     __shared__ long long wsum[SPLATAD_THREADS / SPLATAD_WAVE];
@@ -245,46 +270,48 @@ __device__ __forceinline__ uint32_t coarse_mask(const LaneWork &w, const CoarseG
     return m;
 }
 
-// The coarse counters are replicated `copies` times (atomics on one cache line are
-// serialised; workgroup b updates copy b % copies) and stored [copy][block], so that a
-// wavefront expanding one large rectangle updates neighbouring words.
-template <bool LIDAR>
-__global__ void __launch_bounds__(SPLATAD_THREADS)
-isect_coarse_count_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
-                          const int64_t *__restrict__ camera_ids,
-                          const float *__restrict__ means2d, const void *__restrict__ radii,
-                          uint32_t copies, uint32_t n_blocks, int32_t *__restrict__ counts) {
-    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    LaneWork mine = load_work<LIDAR>(g, idx, total, N, camera_ids, means2d, radii, nullptr, nullptr);
-    mine.base = (mine.base / (g.tile_w * g.tile_h)) * cg.cw * cg.ch;
-    to_coarse(mine, cg);
-    const size_t copy_base = (size_t)(blockIdx.x & (copies - 1)) * n_blocks;
-    for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t) {
-        atomicAdd(&counts[copy_base + w.base + coarse_index<LIDAR>(cg, y, x)], 1);
-    });
-}
+// Coarse binning without global atomics.  A fixed grid of workgroups strides over the
+// Gaussians; each keeps the counters of all coarse blocks in LDS.  COUNT pass: the
+// workgroup's counts go to its own row of a [workgroup][block] table.  The table is then
+// scanned block-major, which gives every (block, workgroup) its own run in the block's
+// list.  FILL pass: the same workgroup meets the same Gaussians, starts its LDS cursors at
+// those runs and writes the entries {flatten id, depth bits, block, tile mask}.
+// One launch covers the cameras [cam_lo, cam_hi) (as many as the LDS holds counters for).
+constexpr uint32_t kCoarseThreads = 1024;
+constexpr uint32_t kCoarseLdsBlocks = 36864; // counters per workgroup, 144 KB
 
-// Coarse list entry: {flatten id, depth bits, block, tile mask}
-template <bool LIDAR>
-__global__ void __launch_bounds__(SPLATAD_THREADS)
-isect_coarse_fill_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
-                         const int64_t *__restrict__ camera_ids,
-                         const float *__restrict__ means2d, const void *__restrict__ radii,
-                         const float *__restrict__ depths, uint32_t copies, uint32_t n_blocks,
-                         const int32_t *__restrict__ starts, int32_t *__restrict__ fill,
-                         uint4 *__restrict__ entries) {
-    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    LaneWork mine = load_work<LIDAR>(g, idx, total, N, camera_ids, means2d, radii, depths, nullptr);
-    mine.base = (mine.base / (g.tile_w * g.tile_h)) * cg.cw * cg.ch;
-    to_coarse(mine, cg);
-    const size_t copy_base = (size_t)(blockIdx.x & (copies - 1)) * n_blocks;
-    for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t) {
-        const uint32_t block = w.base + coarse_index<LIDAR>(cg, y, x);
-        const size_t t = copy_base + block;
-        const int32_t slot = atomicAdd(&fill[t], 1);
-        entries[(int64_t)starts[t] + slot] =
-            make_uint4(w.idx, w.depth_bits, block, coarse_mask(w, cg, y, x));
-    });
+template <bool LIDAR, bool FILL>
+__global__ void __launch_bounds__(kCoarseThreads)
+isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
+                    const int64_t *__restrict__ camera_ids, const float *__restrict__ means2d,
+                    const void *__restrict__ radii, const float *__restrict__ depths,
+                    uint32_t cam_lo, uint32_t cam_hi, uint32_t n_blocks, int32_t *table,
+                    uint4 *__restrict__ entries) {
+    extern __shared__ int32_t s_blocks[];
+    SPLATAD_STAGE_ELEVATIONS(g)
+    const uint32_t per_cam = cg.cw * cg.ch, tiles_per_cam = g.tile_w * g.tile_h;
+    const uint32_t first = cam_lo * per_cam, count = (cam_hi - cam_lo) * per_cam;
+    int32_t *row = table + (size_t)blockIdx.x * n_blocks + first;
+    for (uint32_t b = threadIdx.x; b < count; b += blockDim.x) s_blocks[b] = FILL ? row[b] : 0;
+    __syncthreads();
+    for (uint64_t base = (uint64_t)blockIdx.x * blockDim.x; base < total;
+         base += (uint64_t)gridDim.x * blockDim.x) { // uniform across the workgroup
+        LaneWork mine = load_work<LIDAR>(g, base + threadIdx.x, total, N, camera_ids, means2d,
+                                         radii, FILL ? depths : nullptr, nullptr);
+        const uint32_t cam = mine.base / tiles_per_cam;
+        if (cam < cam_lo || cam >= cam_hi) mine.cnt = 0;
+        mine.base = (cam - cam_lo) * per_cam;
+        to_coarse(mine, cg);
+        for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t) {
+            const uint32_t local = w.base + coarse_index<LIDAR>(cg, y, x);
+            const int32_t slot = atomicAdd(&s_blocks[local], 1);
+            if (FILL) entries[slot] = make_uint4(w.idx, w.depth_bits, first + local, coarse_mask(w, cg, y, x));
+        });
+    }
+    if (!FILL) {
+        __syncthreads();
+        for (uint32_t b = threadIdx.x; b < count; b += blockDim.x) row[b] = s_blocks[b];
+    }
 }
 
 // Tile binning.  A wavefront takes 64 consecutive coarse entries; those of one block (nearly
@@ -355,6 +382,7 @@ isect_emit_kernel(TileGrid g, uint64_t total, uint32_t N, const int64_t *__restr
                   const float *__restrict__ depths, const int64_t *__restrict__ cum_before,
                   uint32_t tile_n_bits, int64_t *__restrict__ isect_ids,
                   int32_t *__restrict__ flatten_ids) {
+    SPLATAD_STAGE_ELEVATIONS(g)
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const LaneWork mine = load_work<LIDAR>(g, idx, total, N, camera_ids, means2d, radii, depths, cum_before);
     const uint32_t tiles_per_cam = g.tile_w * g.tile_h;
@@ -399,39 +427,78 @@ __device__ __forceinline__ void bitonic_sort_ascending(Ptr a, uint32_t n, uint32
     }
 }
 
-constexpr uint32_t kSortMaxBuckets = 2048; // per segment
-constexpr uint32_t kSortBucketMean = 12;   // upper bound of the mean entries per bucket
-constexpr uint32_t kSortRankMax = 1024;    // largest bucket ordered by rank counting
-constexpr uint32_t kSortWindow = 12288;    // entries ranked per step when staging is global
+constexpr uint32_t kSortFineBins = 512;     // first-level depth bins per segment
+constexpr uint32_t kSortBucketMean = 8;     // aimed-at entries per bucket
+constexpr uint32_t kSortSplit = 4096;       // buckets at most, beyond the fine bins
+constexpr uint32_t kSortRankMax = 1024;     // largest bucket ordered by rank counting
+constexpr uint32_t kSortWindow = 15360;     // LDS window (entries) when staging is global
 
-__host__ __device__ inline uint32_t sort_bucket_count(uint32_t n) {
-    uint32_t nb = 1;
-    while (nb < kSortMaxBuckets && nb * kSortBucketMean < n) nb <<= 1;
-    return nb;
+// Bucket counters a segment of up to max_n entries can need.
+__host__ __device__ inline uint32_t sort_bucket_capacity(uint32_t max_n) {
+    const uint32_t split = max_n / kSortBucketMean < kSortSplit ? max_n / kSortBucketMean : kSortSplit;
+    return split + kSortFineBins + 1;
 }
 
-// One workgroup per (camera, tile) segment: a bucket sort on the depth.  The segment's range
-// of depth bits (for positive floats a piecewise-linear logarithm of the depth) is cut into
-// up to 2048 equal buckets; the entries are counted per bucket (LDS atomics), scattered
-// bucket by bucket into a staging array, and every entry then finds its place inside its
-// bucket by counting the bucket's smaller (depth bits, flatten id) keys; equal keys (a lidar
-// Gaussian wider than a full turn meets a tile twice) are ordered by staging position.
-// Lanes of one bucket read the same staging words, so those reads are LDS broadcasts.
+// Exclusive scan over L values held in LDS by a workgroup of nt threads (a multiple of 64):
+// thread t owns ceil(L / nt) consecutive values; load(i) gives value i, store(i, before, v)
+// receives the sum of the values before i.  Returns the total.  Ends with a barrier.
+template <typename Load, typename Store>
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t L, uint32_t tid, uint32_t nt,
+                                                         uint32_t *s_wave, Load &&load, Store &&store) {
+    const uint32_t lane = tid & (SPLATAD_WAVE - 1), wave = tid / SPLATAD_WAVE;
+    const uint32_t per = (L + nt - 1) / nt;
+    const uint32_t b0 = min(L, tid * per), b1 = min(L, b0 + per);
+    uint32_t sum = 0;
+    for (uint32_t b = b0; b < b1; ++b) sum += load(b);
+    uint32_t incl = sum;
+#pragma unroll
+    for (int off = 1; off < SPLATAD_WAVE; off <<= 1) {
+        const uint32_t o = (uint32_t)__shfl_up((int)incl, off, SPLATAD_WAVE);
+        if ((int)lane >= off) incl += o;
+    }
+    if (lane == SPLATAD_WAVE - 1) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - sum, total = 0;
+    for (uint32_t w = 0; w < nt / SPLATAD_WAVE; ++w) {
+        const uint32_t v = s_wave[w];
+        if (w < wave) run += v;
+        total += v;
+    }
+    for (uint32_t b = b0; b < b1; ++b) {
+        const uint32_t v = load(b);
+        store(b, run, v);
+        run += v;
+    }
+    __syncthreads();
+    return total;
+}
+
+// One workgroup per (camera, tile) segment: a bucket sort on the depth in three steps.
+//  1. The segment's range of depth bits (for positive floats a piecewise-linear logarithm
+//     of the depth) is cut into up to 512 equal fine bins and the entries are counted per
+//     bin (LDS atomics).
+//  2. Every fine bin is given ceil(count / 8) buckets that divide it evenly, so that the
+//     buckets hold about eight entries whatever the distribution of the depths is; the
+//     entries are counted per bucket, the counts scanned, and the entries scattered bucket
+//     by bucket into a staging array.
+//  3. Every entry finds its place inside its bucket by counting the bucket's smaller
+//     (depth bits, flatten id) keys; equal keys (a lidar Gaussian wider than a full turn
+//     meets a tile twice) are ordered by staging position.  Lanes of one bucket read the
+//     same staging words, so those reads are LDS broadcasts.
 //   ER     > 0: the segment (n <= ER * blockDim.x) is held in registers between the passes;
-//          = 0: it is read from global memory three times.
-//   IN_LDS: the staging array is LDS (lds_words entries), and the output is written
-//          directly.  Otherwise the isect_ids output is the staging array, LDS holds a
-//          window of kSortWindow entries (plus one maximal bucket on either side) of it at
-//          a time, the ranked entries go back to `pairs` and are converted at the end.
+//          = 0: it is read from global memory once per pass.
+//   IN_LDS: the staging array is LDS (lds_words entries).  Otherwise the isect_ids output
+//          is the staging array and passes through LDS in windows of whole buckets.
 // Buckets above 1024 entries (many equal depths) are ordered by a workgroup-wide bitonic
 // network instead.  Segments with min_n < n <= max_n are handled, the others skipped.
-// Dynamic LDS: lds_words * 8 bytes of staging, then 2 * sort_bucket_count(max_n) counters.
+// Dynamic LDS: lds_words * 8 bytes of staging, the fine bins, 2 * bucket_cap counters.
 template <int ER, bool IN_LDS>
 __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
                                           uint32_t tile_n_bits, uint32_t min_n, uint32_t max_n,
-                                          uint32_t lds_words, int64_t n_isects,
+                                          uint32_t lds_words, uint32_t bucket_cap,
+                                          int64_t n_isects,
                                           const int32_t *__restrict__ tile_starts,
-                                          uint64_t *pairs, int64_t *isect_ids,
+                                          const uint64_t *__restrict__ pairs, int64_t *isect_ids,
                                           int32_t *__restrict__ flatten_ids) {
     extern __shared__ uint64_t lds_staged[];
     __shared__ uint32_t s_wave[2 * (1024 / SPLATAD_WAVE)];
@@ -442,10 +509,10 @@ __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
     const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
     const uint32_t n = (uint32_t)(stop - start);
     if (n <= min_n || n > max_n) return; // uniform across the workgroup
-    const uint32_t nb = sort_bucket_count(n);
-    uint32_t *s_cursor = reinterpret_cast<uint32_t *>(lds_staged + lds_words);
-    uint32_t *s_first = s_cursor + sort_bucket_count(max_n);
-    uint64_t *g = pairs + start;
+    uint32_t *s_fine = reinterpret_cast<uint32_t *>(lds_staged + lds_words);
+    uint32_t *s_cursor = s_fine + kSortFineBins;
+    uint32_t *s_first = s_cursor + bucket_cap;
+    const uint64_t *g = pairs + start;
     int64_t *ids_out = isect_ids + start;
     int32_t *flat_out = flatten_ids + start;
     uint64_t *staged = IN_LDS ? lds_staged : reinterpret_cast<uint64_t *>(ids_out);
@@ -471,10 +538,16 @@ __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
             for (int k = 0; k < NR; ++k)
                 if (tid + k * nt < n) f(held[k]);
         } else {
-            for (uint32_t i = tid; i < n; i += nt) f(g[i]);
+            uint32_t i = tid;
+            for (; i + 3 * nt < n; i += 4 * nt) { // independent loads in flight together
+                const uint64_t p0 = g[i], p1 = g[i + nt], p2 = g[i + 2 * nt], p3 = g[i + 3 * nt];
+                f(p0); f(p1); f(p2); f(p3);
+            }
+            for (; i < n; i += nt) f(g[i]);
         }
     };
 
+    // range of the depth bits
     uint32_t lo = 0xFFFFFFFFu, hi = 0u;
     for_each_entry([&](uint64_t p) {
         const uint32_t d = (uint32_t)(p >> 32);
@@ -488,49 +561,56 @@ __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
     }
     if (lane == 0) { s_wave[2 * wave] = lo; s_wave[2 * wave + 1] = hi; }
     if (tid == 0) s_big = 0;
-    for (uint32_t b = tid; b < nb; b += nt) s_cursor[b] = 0;
+    uint32_t n_fine = 1;
+    while (n_fine < kSortFineBins && n_fine * 16 < n) n_fine <<= 1;
+    for (uint32_t f = tid; f < n_fine; f += nt) s_fine[f] = 0;
     __syncthreads();
     for (uint32_t w = 0; w < n_waves; ++w) {
         lo = min(lo, s_wave[2 * w]);
         hi = max(hi, s_wave[2 * w + 1]);
     }
-    const float scale = (float)nb / ((float)(hi - lo) + 1.f);
-    auto bucket_of = [&](uint64_t p) -> uint32_t {
-        return min(nb - 1, (uint32_t)((float)((uint32_t)(p >> 32) - lo) * scale));
+    const float scale = (float)n_fine / ((float)(hi - lo) + 1.f);
+    // position on the fine-bin axis, non-decreasing in the depth bits
+    auto fine_pos = [&](uint64_t p, uint32_t &f) -> float {
+        const float x = (float)((uint32_t)(p >> 32) - lo) * scale;
+        f = min(n_fine - 1, (uint32_t)x);
+        return x;
     };
-    __syncthreads(); // s_wave is reused by the scan
+    __syncthreads(); // s_wave is reused by the scans
 
-    // entries per bucket
+    // 1. entries per fine bin
+    for_each_entry([&](uint64_t p) {
+        uint32_t f;
+        fine_pos(p, f);
+        atomicAdd(&s_fine[f], 1u);
+    });
+    __syncthreads();
+
+    // 2. buckets per fine bin; s_fine[f] becomes (first bucket | buckets << 16)
+    const uint32_t mean = max(kSortBucketMean, (n + kSortSplit - 1) / kSortSplit);
+    const uint32_t nb = block_exclusive_scan(
+        n_fine, tid, nt, s_wave,
+        [&](uint32_t f) { return (s_fine[f] + mean - 1) / mean; },
+        [&](uint32_t f, uint32_t before, uint32_t v) { s_fine[f] = before | (v << 16); });
+    auto bucket_of = [&](uint64_t p) -> uint32_t {
+        uint32_t f;
+        const float x = fine_pos(p, f);
+        const uint32_t packed = s_fine[f];
+        const uint32_t k = packed >> 16;
+        const uint32_t sub = min(k - 1, (uint32_t)((x - (float)f) * (float)k));
+        return (packed & 0xFFFFu) + sub;
+    };
+    for (uint32_t b = tid; b < nb; b += nt) s_cursor[b] = 0;
+    __syncthreads();
     for_each_entry([&](uint64_t p) { atomicAdd(&s_cursor[bucket_of(p)], 1u); });
     __syncthreads();
-
-    // exclusive scan over the buckets: thread t owns `per` consecutive buckets
-    {
-        const uint32_t per = nb > nt ? nb / nt : 1;
-        const uint32_t b0 = tid * per;
-        uint32_t sum = 0;
-        if (b0 < nb)
-            for (uint32_t k = 0; k < per; ++k) sum += s_cursor[b0 + k];
-        uint32_t incl = sum;
-#pragma unroll
-        for (int off = 1; off < SPLATAD_WAVE; off <<= 1) {
-            const uint32_t o = (uint32_t)__shfl_up((int)incl, off, SPLATAD_WAVE);
-            if ((int)lane >= off) incl += o;
-        }
-        if (lane == SPLATAD_WAVE - 1) s_wave[wave] = incl;
-        __syncthreads();
-        uint32_t run = incl - sum;
-        for (uint32_t w = 0; w < wave; ++w) run += s_wave[w];
-        if (b0 < nb)
-            for (uint32_t k = 0; k < per; ++k) {
-                const uint32_t c = s_cursor[b0 + k];
-                s_cursor[b0 + k] = run;
-                s_first[b0 + k] = run;
-                run += c;
-                if (c > kSortRankMax) s_big = 1;
-            }
-    }
-    __syncthreads();
+    block_exclusive_scan(
+        nb, tid, nt, s_wave, [&](uint32_t b) { return s_cursor[b]; },
+        [&](uint32_t b, uint32_t before, uint32_t v) {
+            s_cursor[b] = before;
+            s_first[b] = before;
+            if (v > kSortRankMax) s_big = 1;
+        });
 
     // scatter into buckets
     for_each_entry([&](uint64_t p) { staged[atomicAdd(&s_cursor[bucket_of(p)], 1u)] = p; });
@@ -543,7 +623,7 @@ __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
         }
     }
 
-    // place = first of the bucket + number of smaller keys in the bucket; `view` is the
+    // 3. place = first of the bucket + number of smaller keys in the bucket; `view` is the
     // staging array seen through LDS, view[j - view_lo] == staged[j]
     auto place_of = [&](uint64_t p, uint32_t i, const uint64_t *view, uint32_t view_lo) -> uint32_t {
         const uint32_t b = bucket_of(p);
@@ -556,30 +636,49 @@ __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
         }
         return place;
     };
+    auto emit = [&](uint32_t place, uint64_t p) {
+        ids_out[place] = (int64_t)(key_hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
+        flat_out[place] = (int32_t)(uint32_t)p;
+    };
     if (IN_LDS) {
         for (uint32_t i = tid; i < n; i += nt) {
             const uint64_t p = lds_staged[i];
-            const uint32_t place = place_of(p, i, lds_staged, 0);
-            ids_out[place] = (int64_t)(key_hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
-            flat_out[place] = (int32_t)(uint32_t)p;
+            emit(place_of(p, i, lds_staged, 0), p);
         }
     } else {
-        for (uint32_t w0 = 0; w0 < n; w0 += kSortWindow) { // uniform
-            const uint32_t w1 = min(n, w0 + kSortWindow);
-            const uint32_t v0 = w0 > kSortRankMax ? w0 - kSortRankMax : 0;
-            const uint32_t v1 = min(n, w1 + kSortRankMax);
-            for (uint32_t j = v0 + tid; j < v1; j += nt) lds_staged[j - v0] = staged[j];
+        // windows of whole buckets, as many as fit the LDS: a window is loaded, then its
+        // entries are ranked and written over the staging array they came from
+        uint32_t b0 = 0;
+        while (b0 < nb) { // uniform
+            const uint32_t v0 = s_first[b0];
+            uint32_t lo_b = b0, hi_b = nb; // largest b1 with end(b1 - 1) - v0 <= lds_words
+            while (lo_b < hi_b) {
+                const uint32_t mid = (lo_b + hi_b + 1) / 2;
+                if (s_cursor[mid - 1] - v0 <= lds_words) lo_b = mid; else hi_b = mid - 1;
+            }
+            if (lo_b == b0) {
+                // a single bucket beyond the window: ordered by the network already
+                const uint32_t v1 = s_cursor[b0];
+                for (uint32_t i = v0 + tid; i < v1; i += nt) emit(i, staged[i]);
+                b0 = b0 + 1;
+                continue;
+            }
+            const uint32_t count = s_cursor[lo_b - 1] - v0;
+            uint32_t j = tid;
+            for (; j + 3 * nt < count; j += 4 * nt) { // independent loads in flight together
+                const uint64_t q0 = staged[v0 + j], q1 = staged[v0 + j + nt];
+                const uint64_t q2 = staged[v0 + j + 2 * nt], q3 = staged[v0 + j + 3 * nt];
+                lds_staged[j] = q0; lds_staged[j + nt] = q1;
+                lds_staged[j + 2 * nt] = q2; lds_staged[j + 3 * nt] = q3;
+            }
+            for (; j < count; j += nt) lds_staged[j] = staged[v0 + j];
             __syncthreads();
-            for (uint32_t i = w0 + tid; i < w1; i += nt) {
+            for (uint32_t i = v0 + tid; i < v0 + count; i += nt) {
                 const uint64_t p = lds_staged[i - v0];
-                g[place_of(p, i, lds_staged, v0)] = p; // the input is free by now
+                emit(place_of(p, i, lds_staged, v0), p);
             }
             __syncthreads();
-        }
-        for (uint32_t i = tid; i < n; i += nt) {
-            const uint64_t p = g[i];
-            ids_out[i] = (int64_t)(key_hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
-            flat_out[i] = (int32_t)(uint32_t)p;
+            b0 = lo_b;
         }
     }
 }
@@ -587,11 +686,11 @@ __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
 template <int ER, bool IN_LDS>
 static int launch_segment_sort(uint32_t threads, uint32_t min_n, uint32_t max_n, uint32_t segs,
                                uint32_t n_tiles, uint32_t tile_n_bits, int64_t n_isects,
-                               const int32_t *tile_starts, uint64_t *pairs, int64_t *isect_ids,
-                               int32_t *flatten_ids, hipStream_t stream) {
-    const uint32_t lds_words = IN_LDS ? max_n : kSortWindow + 2 * kSortRankMax;
-    const uint32_t cap = IN_LDS ? max_n : 0x7FFFFFFFu;
-    const size_t lds_bytes = (size_t)lds_words * 8 + 2 * sort_bucket_count(cap) * 4;
+                               const int32_t *tile_starts, const uint64_t *pairs,
+                               int64_t *isect_ids, int32_t *flatten_ids, hipStream_t stream) {
+    const uint32_t lds_words = IN_LDS ? max_n : kSortWindow;
+    const uint32_t bucket_cap = sort_bucket_capacity(max_n);
+    const size_t lds_bytes = (size_t)lds_words * 8 + (kSortFineBins + 2 * (size_t)bucket_cap) * 4;
     {   // raise the kernel's dynamic LDS limit once per instantiation and size
         static std::mutex guard;
         static size_t allowed = 0;
@@ -604,8 +703,8 @@ static int launch_segment_sort(uint32_t threads, uint32_t min_n, uint32_t max_n,
         }
     }
     hipLaunchKernelGGL((isect_segment_sort_kernel<ER, IN_LDS>), dim3(segs), dim3(threads),
-                       lds_bytes, stream, segs, n_tiles, tile_n_bits, min_n, cap, lds_words,
-                       n_isects, tile_starts, pairs, isect_ids, flatten_ids);
+                       lds_bytes, stream, segs, n_tiles, tile_n_bits, min_n, max_n, lds_words,
+                       bucket_cap, n_isects, tile_starts, pairs, isect_ids, flatten_ids);
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }
@@ -642,17 +741,22 @@ __global__ void fill_zero_i32_kernel(int32_t *p, int64_t n) {
 
 __global__ void fill_zero_u64_kernel(unsigned long long *p) { *p = 0ull; }
 
+__global__ void copy_i32_kernel(const int32_t *__restrict__ src, int32_t *__restrict__ dst,
+                                int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
 struct IsectWorkspace {
     unsigned long long *n_isects; // [1]
     int64_t *n_entries;           // [1] length of the coarse lists
     int64_t *scan_total;          // [1]
-    int32_t *zeroed;              // coarse_counts .. tile_fill are contiguous, cleared together
+    int32_t *zeroed;              // tile_counts, tile_fill are contiguous, cleared together
     uint64_t n_zeroed;
-    int32_t *coarse_counts;       // [copies * C * blocks]
-    int32_t *coarse_fill;         // same
     int32_t *tile_counts;         // [tile copies * C * n_tiles]
     int32_t *tile_fill;           // same
-    int32_t *coarse_starts;       // [copies * C * blocks]
+    int32_t *coarse_counts;       // [coarse workgroups * C * blocks]
+    int32_t *coarse_starts;       // same
     int32_t *tile_starts;         // [tile copies * C * n_tiles]
     int64_t *block_sums;          // scan scratch
     int64_t *cum_before;          // [total] (sort == false)
@@ -677,8 +781,19 @@ static uint32_t isect_copies(uint64_t blocks) {
     return k;
 }
 
-// Layout from sizes only; cslots is the length of the replicated coarse counter table, or
-// an upper bound of it when only the number of tiles is known (workspace sizing).
+// Workgroups of the coarse binning (= rows of its counter table): enough to fill the GPU,
+// fewer when many blocks would make the table long.
+static uint32_t coarse_workgroups(uint64_t total, uint64_t blocks) {
+    uint64_t wgs = (1ull << 19) / (blocks ? blocks : 1);
+    if (wgs > 512) wgs = 512;
+    if (wgs < 64) wgs = 64;
+    const uint64_t needed = (total + kCoarseThreads - 1) / kCoarseThreads;
+    if (wgs > needed) wgs = needed ? needed : 1;
+    return (uint32_t)wgs;
+}
+
+// Layout from sizes only; cslots is the length of the coarse counter table, or an upper
+// bound of it when only the number of tiles is known (workspace sizing).
 static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslots,
                           int64_t n_isects, IsectWorkspace *out) {
     const uint64_t tslots = segs * isect_copies(segs);
@@ -690,11 +805,10 @@ static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslo
     w.n_entries = (int64_t *)p;             p += 256;
     w.scan_total = (int64_t *)p;            p += 256;
     w.zeroed = (int32_t *)p;
-    w.coarse_counts = (int32_t *)p;         p += splatad_align256(cslots * 4);
-    w.coarse_fill = (int32_t *)p;           p += splatad_align256(cslots * 4);
     w.tile_counts = (int32_t *)p;           p += splatad_align256(tslots * 4);
     w.tile_fill = (int32_t *)p;             p += splatad_align256(tslots * 4);
     w.n_zeroed = (uint64_t)(p - (char *)w.zeroed) / 4;
+    w.coarse_counts = (int32_t *)p;         p += splatad_align256(cslots * 4);
     w.coarse_starts = (int32_t *)p;         p += splatad_align256(cslots * 4);
     w.tile_starts = (int32_t *)p;           p += splatad_align256(tslots * 4);
     w.block_sums = (int64_t *)p;            p += scan_workspace_bytes((int64_t)scan_n);
@@ -708,9 +822,9 @@ static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslo
 }
 
 static size_t isect_ws_bytes(uint64_t total, uint64_t segs, int64_t n_isects) {
-    // there are at most as many coarse blocks as tiles, and isect_copies() keeps the table
-    // below 2^19 entries unless the blocks alone exceed that
-    const uint64_t cslots_bound = segs > (1ull << 19) ? segs : (1ull << 19);
+    // there are at most as many coarse blocks as tiles, and coarse_workgroups() keeps the
+    // table at 2^19 entries unless 64 rows exceed that
+    const uint64_t cslots_bound = segs * 64 > (1ull << 19) ? segs * 64 : (1ull << 19);
     return carve_isect(nullptr, total, segs, cslots_bound, n_isects, nullptr);
 }
 
@@ -734,8 +848,10 @@ static int isect_count(TileGrid g, uint64_t total, const float *means2d, const v
     IsectWorkspace w;
     carve_isect(workspace, total, (uint64_t)C * n_tiles, 0, 0, &w);
     hipLaunchKernelGGL(fill_zero_u64_kernel, dim3(1), dim3(1), 0, stream, w.n_isects);
-    hipLaunchKernelGGL(isect_count_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
-                       stream, g, total, means2d, radii, tiles_per_gauss, w.n_isects);
+    dim3 count_grid = grid_for(total);
+    if (count_grid.x > 512) count_grid.x = 512;
+    hipLaunchKernelGGL(isect_count_kernel<LIDAR>, count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
+                       total, means2d, radii, tiles_per_gauss, w.n_isects);
     SPLATAD_LAUNCH_CHECK();
     unsigned long long n = 0;
     SPLATAD_CHECK_HIP(hipMemcpyAsync(&n, w.n_isects, sizeof(n), hipMemcpyDeviceToHost, stream));
@@ -745,13 +861,48 @@ static int isect_count(TileGrid g, uint64_t total, const float *means2d, const v
     return 0;
 }
 
+// Helper streams (default priority) and events of the segment sort, one set per device,
+// created at first use and kept for the life of the process.  `guard` serialises the
+// enqueueing of a fork .. join sequence, which shares the events.
+struct SortStreams {
+    hipStream_t aux[2];
+    hipEvent_t fork, join[2];
+    std::mutex guard;
+};
+
+static int sort_streams(SortStreams **out) {
+    static std::mutex table_guard;
+    static SortStreams *table[64] = {};
+    int dev = 0;
+    SPLATAD_CHECK_HIP(hipGetDevice(&dev));
+    SPLATAD_REQUIRE(dev >= 0 && dev < 64, "isect: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(table_guard);
+    if (!table[dev]) {
+        SortStreams *s = new SortStreams();
+        for (hipStream_t &a : s->aux) SPLATAD_CHECK_HIP(hipStreamCreateWithFlags(&a, hipStreamNonBlocking));
+        SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->fork, hipEventDisableTiming));
+        for (hipEvent_t &e : s->join) SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        table[dev] = s;
+    }
+    *out = table[dev];
+    return 0;
+}
+
 template <bool LIDAR>
 static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *camera_ids,
                       const float *means2d, const void *radii, const float *depths, uint32_t C,
                       int sort, int64_t n_isects, const int32_t *tiles_per_gauss,
                       void *workspace, int64_t *isect_ids, int32_t *flatten_ids,
-                      hipStream_t stream) {
-    if (total == 0 || n_isects == 0) return 0;
+                      int32_t *tile_offsets, hipStream_t stream) {
+    if (total == 0 || n_isects == 0) {
+        if (tile_offsets && sort && (uint64_t)C * g.tile_w * g.tile_h > 0) {
+            const uint64_t tiles = (uint64_t)C * g.tile_w * g.tile_h;
+            hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(tiles), dim3(SPLATAD_THREADS), 0,
+                               stream, tile_offsets, (int64_t)tiles);
+            SPLATAD_LAUNCH_CHECK();
+        }
+        return 0;
+    }
     SPLATAD_REQUIRE(means2d && radii && depths && workspace && isect_ids && flatten_ids,
                     "isect: null pointer argument");
     SPLATAD_REQUIRE(camera_ids != nullptr || N > 0, "isect: N is zero for unpacked input");
@@ -760,8 +911,8 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     const uint64_t segs = (uint64_t)C * n_tiles;
     const CoarseGrid cg = coarse_grid<LIDAR>(g);
     const uint64_t blocks = (uint64_t)C * cg.cw * cg.ch;
-    const uint32_t copies = isect_copies(blocks);
-    const uint64_t cslots = blocks * copies;
+    const uint32_t coarse_wgs = coarse_workgroups(total, blocks);
+    const uint64_t cslots = blocks * coarse_wgs;
     IsectWorkspace w;
     carve_isect(workspace, total, segs, sort ? cslots : 0, n_isects, &w);
     int rc;
@@ -776,22 +927,48 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         SPLATAD_LAUNCH_CHECK();
         return 0;
     }
-    SPLATAD_REQUIRE(blocks < (1ull << 32) && cslots < (1ull << 31), "isect: tile grid too large");
+    const uint32_t per_cam = cg.cw * cg.ch;
+    SPLATAD_REQUIRE(per_cam <= kCoarseLdsBlocks, "isect: %u x %u tiles per sensor exceed the "
+                    "binning capacity", g.tile_w, g.tile_h);
+    SPLATAD_REQUIRE(blocks < (1ull << 31) && cslots < (1ull << 31), "isect: tile grid too large");
+    const uint32_t cams_per_launch = kCoarseLdsBlocks / per_cam;
+    {
+        static std::mutex guard;
+        static bool raised = false;
+        std::lock_guard<std::mutex> lock(guard);
+        if (!raised) {
+            SPLATAD_CHECK_HIP(hipFuncSetAttribute(
+                (const void *)isect_coarse_kernel<LIDAR, false>,
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kCoarseLdsBlocks * 4)));
+            SPLATAD_CHECK_HIP(hipFuncSetAttribute(
+                (const void *)isect_coarse_kernel<LIDAR, true>,
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kCoarseLdsBlocks * 4)));
+            raised = true;
+        }
+    }
     hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(w.n_zeroed), dim3(SPLATAD_THREADS), 0, stream,
                        w.zeroed, (int64_t)w.n_zeroed);
-    // coarse lists: count, scan (the table is stored [copy][block] and scanned block-major,
-    // which makes a block's list contiguous), fill
-    hipLaunchKernelGGL(isect_coarse_count_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
-                       stream, g, cg, total, N, camera_ids, means2d, radii, copies,
-                       (uint32_t)blocks, w.coarse_counts);
+    // coarse lists: count, scan (the table is stored [workgroup][block] and scanned
+    // block-major, which makes a block's list contiguous), fill
+    for (uint32_t c0 = 0; c0 < C; c0 += cams_per_launch) {
+        const uint32_t c1 = C - c0 < cams_per_launch ? C : c0 + cams_per_launch;
+        hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, false>), dim3(coarse_wgs),
+                           dim3(kCoarseThreads), (size_t)(c1 - c0) * per_cam * 4, stream, g, cg,
+                           total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)blocks,
+                           w.coarse_counts, (uint4 *)nullptr);
+    }
     SPLATAD_LAUNCH_CHECK();
     rc = launch_exclusive_scan<int32_t>(w.coarse_counts, (int64_t)cslots,
-                                        copies > 1 ? -(int)copies : 1, 0, w.coarse_starts,
+                                        coarse_wgs > 1 ? -(int)coarse_wgs : 1, 0, w.coarse_starts,
                                         w.n_entries, w.block_sums, stream);
     if (rc) return rc;
-    hipLaunchKernelGGL(isect_coarse_fill_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
-                       stream, g, cg, total, N, camera_ids, means2d, radii, depths, copies,
-                       (uint32_t)blocks, w.coarse_starts, w.coarse_fill, w.entries);
+    for (uint32_t c0 = 0; c0 < C; c0 += cams_per_launch) {
+        const uint32_t c1 = C - c0 < cams_per_launch ? C : c0 + cams_per_launch;
+        hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, true>), dim3(coarse_wgs),
+                           dim3(kCoarseThreads), (size_t)(c1 - c0) * per_cam * 4, stream, g, cg,
+                           total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)blocks,
+                           w.coarse_starts, w.entries);
+    }
     SPLATAD_LAUNCH_CHECK();
     // tile segments: count, scan, fill.  The number of coarse entries stays on the device;
     // the grid is sized for the bound n_isects and strides.
@@ -808,6 +985,11 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                                         tcopies > 1 ? -(int)tcopies : 1, 0, w.tile_starts,
                                         w.scan_total, w.block_sums, stream);
     if (rc) return rc;
+    if (tile_offsets) {
+        // a tile's offset is the start of its segment: the first row of the scanned table
+        hipLaunchKernelGGL(copy_i32_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream,
+                           (const int32_t *)w.tile_starts, tile_offsets, (int64_t)segs);
+    }
     hipLaunchKernelGGL(isect_tile_bin_kernel<true>, dim3((uint32_t)bin_wgs),
                        dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, tcopies,
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
@@ -815,20 +997,32 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     SPLATAD_LAUNCH_CHECK();
     // Size classes: each launch visits every segment and only works on those of its class, so
     // that the LDS per workgroup (and with it the number of resident workgroups) fits the
-    // segment length.
+    // segment length.  The classes touch disjoint segments; they run on two helper streams
+    // beside the caller's, forked and joined with events, so that the few long workgroups
+    // of the upper classes overlap the many short ones of the lower classes.
     const uint32_t nseg = (uint32_t)segs;
-#define SPLATAD_SORT_CLASS(ER, IN_LDS, threads, lo, hi)                                          \
+    SortStreams *ss = nullptr;
+    if ((rc = sort_streams(&ss)) != 0) return rc;
+    std::lock_guard<std::mutex> fork_lock(ss->guard);
+    SPLATAD_CHECK_HIP(hipEventRecord(ss->fork, stream));
+    for (hipStream_t aux : ss->aux) SPLATAD_CHECK_HIP(hipStreamWaitEvent(aux, ss->fork, 0));
+#define SPLATAD_SORT_CLASS(ER, IN_LDS, threads, lo, hi, on)                                      \
     if ((rc = launch_segment_sort<ER, IN_LDS>(threads, lo, hi, nseg, n_tiles, tile_n_bits,        \
                                               n_isects, w.tile_starts, w.pairs, isect_ids,        \
-                                              flatten_ids, stream)) != 0)                         \
+                                              flatten_ids, on)) != 0)                             \
         return rc;
-    SPLATAD_SORT_CLASS(4, true, 128, 0u, 512u)
-    SPLATAD_SORT_CLASS(8, true, 256, 512u, 2048u)
-    SPLATAD_SORT_CLASS(8, true, 512, 2048u, 4096u)
-    SPLATAD_SORT_CLASS(8, true, 1024, 4096u, 8192u)
-    SPLATAD_SORT_CLASS(16, true, 1024, 8192u, 16384u)
-    SPLATAD_SORT_CLASS(0, false, 1024, 16384u, 0x7FFFFFFFu)
+    SPLATAD_SORT_CLASS(32, false, 1024, 16384u, 32768u, ss->aux[0])
+    SPLATAD_SORT_CLASS(0, false, 1024, 32768u, 0x7FFFFFFFu, ss->aux[0])
+    SPLATAD_SORT_CLASS(16, true, 1024, 8192u, 16384u, ss->aux[1])
+    SPLATAD_SORT_CLASS(8, true, 1024, 4096u, 8192u, ss->aux[1])
+    SPLATAD_SORT_CLASS(8, true, 512, 2048u, 4096u, stream)
+    SPLATAD_SORT_CLASS(8, true, 256, 512u, 2048u, stream)
+    SPLATAD_SORT_CLASS(4, true, 128, 0u, 512u, stream)
 #undef SPLATAD_SORT_CLASS
+    for (int k = 0; k < 2; ++k) {
+        SPLATAD_CHECK_HIP(hipEventRecord(ss->join[k], ss->aux[k]));
+        SPLATAD_CHECK_HIP(hipStreamWaitEvent(stream, ss->join[k], 0));
+    }
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }
@@ -857,11 +1051,11 @@ extern "C" int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_
                                         uint32_t tile_width, uint32_t tile_height, int sort,
                                         int64_t n_isects, const int32_t *tiles_per_gauss,
                                         void *workspace, int64_t *isect_ids, int32_t *flatten_ids,
-                                        splatad_stream_t stream) {
+                                        int32_t *tile_offsets, splatad_stream_t stream) {
     SPLATAD_REQUIRE(tile_size > 0, "isect_tiles: tile_size is zero");
     TileGrid g{tile_size, tile_width, tile_height, 0.f, 0.f, nullptr};
     return isect_fill<false>(g, total, N, camera_ids, means2d, radii, depths, C, sort, n_isects,
-                             tiles_per_gauss, workspace, isect_ids, flatten_ids,
+                             tiles_per_gauss, workspace, isect_ids, flatten_ids, tile_offsets,
                              (hipStream_t)stream);
 }
 
@@ -886,11 +1080,12 @@ extern "C" int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N,
                                               uint32_t tile_width, uint32_t tile_height, int sort,
                                               int64_t n_isects, const int32_t *tiles_per_gauss,
                                               void *workspace, int64_t *isect_ids,
-                                              int32_t *flatten_ids, splatad_stream_t stream) {
+                                              int32_t *flatten_ids, int32_t *tile_offsets,
+                                              splatad_stream_t stream) {
     SPLATAD_REQUIRE(elev_boundaries != nullptr, "isect_lidar_tiles: elev_boundaries is null");
     TileGrid g{0u, tile_width, tile_height, tile_azim_resolution, min_azim, elev_boundaries};
     return isect_fill<true>(g, total, N, camera_ids, means2d, radii, depths, C, sort, n_isects,
-                            tiles_per_gauss, workspace, isect_ids, flatten_ids,
+                            tiles_per_gauss, workspace, isect_ids, flatten_ids, tile_offsets,
                             (hipStream_t)stream);
 }
 

@@ -334,13 +334,19 @@ class _Ops:
             n_isects = int(n_host.value)
             isect_ids = torch.empty((n_isects,), dtype=torch.int64, device=dev)
             flatten_ids = torch.empty((n_isects,), dtype=torch.int32, device=dev)
+            # the binning knows every tile's first intersection: keep that table with the
+            # ids so that isect_offset_encode() on the same, unmodified tensor is free
+            offsets = (torch.empty((C, tile_h, tile_w), dtype=torch.int32, device=dev)
+                       if sort and n_isects else None)
             if n_isects:
                 ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(total), _u32(C),
                                                                   _u32(n_tiles), _i64(n_isects)), dev)
                 _check(fill(_u64(total), _u32(N), _p(camera_ids), _p(means2d), _p(radii),
                             _p(depths), _u32(C), *grid_args, _u32(tile_w), _u32(tile_h),
                             _i32(bool(sort)), _i64(n_isects), _p(tiles_per_gauss), _p(ws),
-                            _p(isect_ids), _p(flatten_ids), _stream(dev)))
+                            _p(isect_ids), _p(flatten_ids), _p(offsets), _stream(dev)))
+            if offsets is not None:
+                isect_ids._splatad_tile_offsets = (offsets, isect_ids._version)
         return tiles_per_gauss, isect_ids, flatten_ids
 
     def isect_tiles(self, means2d, radii, depths, camera_ids, gaussian_ids, C, tile_size,
@@ -361,6 +367,10 @@ class _Ops:
 
     def isect_offset_encode(self, isect_ids, C, tile_width, tile_height):
         lib = load_library()
+        cached = getattr(isect_ids, "_splatad_tile_offsets", None)
+        if (cached is not None and cached[1] == isect_ids._version
+                and tuple(cached[0].shape) == (C, tile_height, tile_width)):
+            return cached[0]
         isect_ids = _in(isect_ids, "isect_ids", torch.int64)
         dev = isect_ids.device
         offsets = torch.empty((C, tile_height, tile_width), dtype=torch.int32, device=dev)

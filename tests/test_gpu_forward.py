@@ -164,7 +164,9 @@ def test_isect_camera_reference_recipe():
 
 
 @pytest.mark.parametrize("n,C,W,H,ts,rmax", [(200000, 2, 640, 480, 16, 40), (3000, 1, 64, 64, 16, 600),
-                                              (50000, 4, 200, 120, 8, 12), (0, 1, 64, 64, 16, 5)])
+                                              (50000, 4, 200, 120, 8, 12), (0, 1, 64, 64, 16, 5),
+                                              # 150 sensors x 256 coarse blocks: two binning launches
+                                              (300, 150, 1024, 1024, 16, 30)])
 def test_isect_camera_sizes_and_packed(n, C, W, H, ts, rmax):
     from splatad_amd import isect_offset_encode, isect_tiles
     rng = np.random.default_rng(n + C)
@@ -178,8 +180,10 @@ def test_isect_camera_sizes_and_packed(n, C, W, H, ts, rmax):
     np.testing.assert_array_equal(to_np(tpg), o_tpg)
     np.testing.assert_array_equal(to_np(ids), o_ids)
     np.testing.assert_array_equal(to_np(flat), o_flat)
-    offs = isect_offset_encode(ids, C, tw, th)
+    offs = isect_offset_encode(ids, C, tw, th)               # table kept by isect_tiles
+    offs_k = isect_offset_encode(ids.clone(), C, tw, th)     # derived from the keys
     np.testing.assert_array_equal(to_np(offs), oracle.isect_offset_encode(o_ids, C, tw, th))
+    np.testing.assert_array_equal(to_np(offs_k), to_np(offs))
     if n == 0:
         return
     # packed input gives the same keys; ids index the packed rows
@@ -194,7 +198,7 @@ def test_isect_camera_sizes_and_packed(n, C, W, H, ts, rmax):
 
 
 @pytest.mark.parametrize("n,tie_frac", [(1500, 0.8), (6000, 0.0), (6000, 0.5), (12000, 0.3),
-                                        (40000, 0.0), (40000, 0.4), (3000, 1.0)])
+                                        (20000, 0.1), (40000, 0.0), (40000, 0.4), (3000, 1.0)])
 def test_isect_sort_long_segments_and_depth_ties(n, tie_frac):
     # every Gaussian covers all four tiles, so each tile's segment has n entries: exercises
     # every segment-length class of the sort and, with many equal depths, oversized buckets
@@ -237,6 +241,9 @@ def test_isect_lidar_reference_recipe_and_wrap():
     tpg, ids, flat = isect_lidar_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), to_dev(eb), res, min_az)
     offs = isect_offset_encode(ids, C, n_az, 16)
     np.testing.assert_array_equal(to_np(offs), oracle.isect_offset_encode(to_np(ids), C, n_az, 16))
+    np.testing.assert_array_equal(to_np(isect_offset_encode(ids.clone(), C, n_az, 16)), to_np(offs))
+    ids.add_(0)  # an in-place change invalidates the kept table
+    assert not (isect_offset_encode(ids, C, n_az, 16) is offs)
 
 
 def test_isect_lidar_large_nonuniform():
