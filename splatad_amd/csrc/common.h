@@ -124,6 +124,36 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// Sums NV (a power of two, 2..64) per-lane values over the 64 lanes of a wavefront with
+// NV - 1 + log2(64 / NV) shuffles instead of 6 NV: at every step a lane hands half of its
+// values to the partner that keeps accumulating them.  Afterwards every lane holds, in
+// v[0], the wavefront total of value `wave_reduce_slot<NV>(lane)`; 64 / NV lanes hold each.
+template <int NV>
+__device__ __forceinline__ void wave_reduce_scatter(float (&v)[NV], int lane) {
+    int off = 32;
+#pragma unroll
+    for (int half = NV / 2; half >= 1; half /= 2) {
+        // bit masks instead of selects: a select between two array elements would be turned
+        // into a dynamically indexed access, i.e. a compare-and-select chain over the array
+        const uint32_t m = (lane & off) != 0 ? 0xFFFFFFFFu : 0u; // upper half of the pair
+#pragma unroll
+        for (int k = 0; k < half; ++k) {
+            const uint32_t lo = __float_as_uint(v[k]), hi = __float_as_uint(v[k + half]);
+            const float send = __uint_as_float((lo & m) | (hi & ~m));
+            const float keep = __uint_as_float((hi & m) | (lo & ~m));
+            v[k] = keep + __shfl_xor(send, off, SPLATAD_WAVE);
+        }
+        off >>= 1;
+    }
+#pragma unroll
+    for (int rest = 32 / NV; rest >= 1; rest /= 2) v[0] += __shfl_xor(v[0], rest, SPLATAD_WAVE);
+}
+
+template <int NV>
+__device__ __forceinline__ int wave_reduce_slot(int lane) {
+    return NV == 64 ? lane : lane / (64 / NV);
+}
+
 __device__ __forceinline__ int wave_max_i32(int v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {

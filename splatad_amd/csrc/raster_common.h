@@ -1,0 +1,171 @@
+// Pieces shared by the forward and backward compositing kernels: the staged form of a
+// Gaussian's exponent, the folded angle difference of the lidar path and the per-wavefront
+// footprint tests that let a wavefront skip Gaussians none of its 64 lanes can see.
+#pragma once
+
+#include "common.h"
+
+#ifdef __HIPCC__
+namespace {
+
+constexpr float kLog2e = 1.44269504088896341f;
+constexpr float kLn2 = 0.693147180559945309f;
+constexpr float kLog2Of255 = 7.99435343685886f;
+
+// Staged exponent of a Gaussian: alpha = exp2(L - (A dx^2 + B dx dy + C dy^2)), i.e.
+// A = a log2(e) / 2, B = b log2(e), C = c log2(e) / 2 for the conic (a, b, c) and
+// L = log2(opacity) (-inf for opacity <= 0, which can then never reach alpha >= 1/255).
+__device__ __forceinline__ float4 staged_exponent(float a, float b, float c, float opacity) {
+    return make_float4(0.5f * kLog2e * a, kLog2e * b, 0.5f * kLog2e * c,
+                       opacity > 0.f ? __log2f(opacity) : -INFINITY);
+}
+
+// Difference of two angles in degrees folded into [-180, 180), as the reference's
+// fmodf(a - b + 180, 360) - 180 with negative results raised by 360
+// (gsplat/cuda/csrc/utils.cuh:552-555).  Without the detour through +180 / -180 the difference of two
+// nearby angles is exact in float32.
+__device__ __forceinline__ float angle_difference(float a, float b) {
+    const float d = a - b;
+    if (d >= -180.f && d < 180.f) return d;
+    float m = fmodf(d + 180.f, 360.f);
+    if (m < 0.f) m += 360.f;
+    return m - 180.f;
+}
+
+// Smallest value of p(d) = A dx^2 + B dx dy + C dy^2 over the box [x0, x1] x [y0, y1] of
+// offsets, compared with the largest p that still passes alpha >= 1/255, L + log2(255).
+// p is convex for a positive definite conic, so off the centre its minimum over the box lies
+// on one of the four edges.  A margin covers the rounding of the test itself; Gaussians with
+// a degenerate conic are never rejected.  Returns false when no offset in the box can pass.
+__device__ __forceinline__ float edge_min(float fixed_coef, float free_coef, float cross,
+                                          float fixed, float lo, float hi) {
+    const float free_c = fminf(fmaxf(-cross * fixed / (2.f * free_coef), lo), hi);
+    return fixed_coef * fixed * fixed + free_coef * free_c * free_c + cross * fixed * free_c;
+}
+
+__device__ __forceinline__ bool box_may_pass(const float4 e, float x0, float x1, float y0, float y1) {
+    const float A = e.x, B = e.y, C = e.z;
+    const bool definite = A > 0.f && C > 0.f && 4.f * A * C - B * B > 0.f;
+    const bool centre_in = x0 <= 0.f && x1 >= 0.f && y0 <= 0.f && y1 >= 0.f;
+    const float q = fminf(fminf(edge_min(A, C, B, x0, y0, y1), edge_min(A, C, B, x1, y0, y1)),
+                          fminf(edge_min(C, A, B, y0, x0, x1), edge_min(C, A, B, y1, x0, x1)));
+    const float limit = e.w + kLog2Of255;
+    return !(definite && !centre_in && q > limit + 1e-3f * fabsf(limit) + 0.02f);
+}
+
+// Footprint of a wavefront of camera pixels: bounding box of the pixel centres and range of
+// the rolling-shutter factor over its lanes (all 64 lanes must exist).
+struct WaveCull {
+    bool enabled;
+    float cx, cy, hx, hy;
+    float roll_mid, roll_half;
+
+    __device__ __forceinline__ void init(float px, float py, float roll, bool full_wavefront) {
+        enabled = full_wavefront;
+        float x_lo = px, x_hi = px, y_lo = py, y_hi = py, r_lo = roll, r_hi = roll;
+        if (enabled) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                x_lo = fminf(x_lo, __shfl_xor(x_lo, off, SPLATAD_WAVE));
+                x_hi = fmaxf(x_hi, __shfl_xor(x_hi, off, SPLATAD_WAVE));
+                y_lo = fminf(y_lo, __shfl_xor(y_lo, off, SPLATAD_WAVE));
+                y_hi = fmaxf(y_hi, __shfl_xor(y_hi, off, SPLATAD_WAVE));
+                r_lo = fminf(r_lo, __shfl_xor(r_lo, off, SPLATAD_WAVE));
+                r_hi = fmaxf(r_hi, __shfl_xor(r_hi, off, SPLATAD_WAVE));
+            }
+        }
+        cx = 0.5f * (x_lo + x_hi); hx = 0.5f * (x_hi - x_lo);
+        cy = 0.5f * (y_lo + y_hi); hy = 0.5f * (y_hi - y_lo);
+        roll_mid = 0.5f * (r_lo + r_hi);
+        roll_half = 0.5f * (r_hi - r_lo) * 1.0001f + 1e-12f;
+    }
+
+    // xyv = {mean x, mean y, pixel velocity x, y}: the offsets mean + roll * velocity -
+    // pixel of the wavefront lie in a box around (mean + roll_mid * velocity - centre)
+    __device__ __forceinline__ bool may_touch(const float4 xyv, const float4 e) const {
+        if (!enabled) return true;
+        const float mx = xyv.x + roll_mid * xyv.z - cx, my = xyv.y + roll_mid * xyv.w - cy;
+        const float ex = hx + fabsf(xyv.z) * roll_half, ey = hy + fabsf(xyv.w) * roll_half;
+        return box_may_pass(e, mx - ex, mx + ex, my - ey, my + ey);
+    }
+};
+
+// Footprint of a wavefront of lidar points.  All angles are taken relative to a reference
+// point of the tile, so that neither the +-180 degree seam nor the size of the absolute
+// angles matters: the staged record holds u = (mean - reference) and the lane r = (point -
+// reference), both folded, and the offset of a pair is u + roll * velocity - r as long as
+// that cannot leave (-180, 180).  The test decides for every Gaussian whether any lane can
+// reach alpha >= 1/255 and whether the unfolded difference is safe (it is unless the
+// Gaussian sits half a turn away from the tile).
+struct WavePointCull {
+    bool enabled;
+    float x_lo, x_hi, y_lo, y_hi; // box of the lanes' r
+    float roll_mid, roll_half;
+
+    __device__ __forceinline__ void init(bool alive, float rx, float ry, float roll,
+                                         bool full_wavefront) {
+        enabled = full_wavefront;
+        const float inf = INFINITY;
+        float xl = alive ? rx : inf, xh = alive ? rx : -inf;
+        float yl = alive ? ry : inf, yh = alive ? ry : -inf;
+        float rl = alive ? roll : inf, rh = alive ? roll : -inf;
+        if (enabled) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                xl = fminf(xl, __shfl_xor(xl, off, SPLATAD_WAVE));
+                xh = fmaxf(xh, __shfl_xor(xh, off, SPLATAD_WAVE));
+                yl = fminf(yl, __shfl_xor(yl, off, SPLATAD_WAVE));
+                yh = fmaxf(yh, __shfl_xor(yh, off, SPLATAD_WAVE));
+                rl = fminf(rl, __shfl_xor(rl, off, SPLATAD_WAVE));
+                rh = fmaxf(rh, __shfl_xor(rh, off, SPLATAD_WAVE));
+            }
+        } else { // partial wavefront: no culling, bounds of the whole folded range
+            xl = yl = -180.f; xh = yh = 180.f;
+            rl = rh = roll;
+        }
+        // slightly widened against the rounding of the test itself
+        x_lo = xl - 1e-4f; x_hi = xh + 1e-4f;
+        y_lo = yl - 1e-4f; y_hi = yh + 1e-4f;
+        roll_mid = 0.5f * (rl + rh);
+        roll_half = 0.5f * (rh - rl) * 1.0001f + 1e-12f;
+    }
+
+    __device__ __forceinline__ bool may_touch(const float4 uv, const float4 e, bool &unfolded_ok) const {
+        const float cx = uv.x + roll_mid * uv.z, cy = uv.y + roll_mid * uv.w;
+        const float ex = fabsf(uv.z) * roll_half, ey = fabsf(uv.w) * roll_half;
+        const float x0 = cx - x_hi - ex, x1 = cx - x_lo + ex;
+        const float y0 = cy - y_hi - ey, y1 = cy - y_lo + ey;
+        unfolded_ok = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(y0), fabsf(y1))) < 179.f;
+        if (!unfolded_ok || !enabled) return true;
+        return box_may_pass(e, x0, x1, y0, y1);
+    }
+};
+
+// Lane -> pixel inside a camera tile: wavefronts cover 8x8 squares when the tile allows it
+// (a compact footprint is what makes the per-wavefront test effective), rows otherwise.
+__device__ __forceinline__ void pixel_of_lane(uint32_t tile_size, uint32_t tr, uint32_t &lx, uint32_t &ly) {
+    lx = tr % tile_size;
+    ly = tr / tile_size;
+    if (tile_size % 8 == 0) {
+        const uint32_t squares_per_row = tile_size / 8, square = tr / SPLATAD_WAVE;
+        const uint32_t lane = tr & (SPLATAD_WAVE - 1);
+        lx = (square % squares_per_row) * 8 + (lane & 7);
+        ly = (square / squares_per_row) * 8 + (lane >> 3);
+    }
+}
+
+// Lane -> point inside a lidar tile: a wavefront covers 16 columns of all four rows when the
+// tile allows it (more compact than one row of 64 columns).
+__device__ __forceinline__ void point_of_lane(uint32_t tile_width, uint32_t tile_height, uint32_t tr,
+                                              uint32_t &lx, uint32_t &ly) {
+    lx = tr % tile_width;
+    ly = tr / tile_width;
+    if (tile_height == 4 && tile_width % 16 == 0) {
+        const uint32_t lane = tr & (SPLATAD_WAVE - 1);
+        lx = (tr / SPLATAD_WAVE) * 16 + (lane & 15);
+        ly = lane >> 4;
+    }
+}
+
+} // namespace
+#endif // __HIPCC__

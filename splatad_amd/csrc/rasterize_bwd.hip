@@ -1,29 +1,24 @@
 // Backward of the alpha compositing for camera pixels and lidar points on gfx950.
 //
-// One workgroup per (sensor, tile), one lane per pixel / point.  Each pixel replays its
-// tile's list back to front, starting at the last Gaussian it took in the forward pass,
-// and recovers the transmittance by dividing (T_before = T_after / (1 - alpha)).  Batches of
-// the list are staged in LDS together with the colours.  Per Gaussian, the pixel gradients
-// are summed over the 64 lanes of each wavefront, accumulated across the wavefronts of the
-// workgroup in LDS, and flushed with one global atomic per value and (tile, Gaussian) when
-// the batch is finished.  Batches behind the deepest entry any pixel of the tile consumed
-// are never loaded.
+// One workgroup per (sensor, tile), one lane per pixel / point, lanes laid out as in the
+// forward kernels.  Each pixel replays its tile's list back to front, starting at the last
+// Gaussian it took in the forward pass, and recovers the transmittance by dividing
+// (T_before = T_after / (1 - alpha)).  Batches of the list are staged in LDS in the same form
+// as in the forward pass, so that both passes take the same alpha >= 1/255 decisions.  Every
+// wavefront first tests the batch against its footprint, 64 Gaussians at a time, and then
+// walks only those Gaussians some lane of it can see.  Per Gaussian, the pixel gradients
+// (colours and geometry, up to 46 values) are summed over the wavefront with one
+// reduce-scatter, accumulated across the wavefronts of the workgroup in LDS, and flushed
+// with one global atomic per value and (tile, Gaussian) when the batch is finished.  Batches
+// behind the deepest entry any pixel of the tile consumed are never loaded.
 //
 // Gradient rules follow gsplat/cuda/csrc/rasterization.cu:2833-3089 (pixels) and :3728-4054
 // (points) of the reference.  Channels beyond 33 are handled in passes; the geometry
 // gradients are linear in the per-channel terms, so the passes add up exactly (the absolute
 // gradient v_means2d_abs then adds the per-pass magnitudes).
-#include "common.h"
+#include "raster_common.h"
 
 namespace {
-
-// fmodf(a - b + 180, 360) - 180 folded into (-180, 180], see the forward kernel
-__device__ __forceinline__ float angle_difference(float a, float b) {
-    const float d = a - b + 180.f;
-    const float m = (d >= 0.f && d < 360.f) ? d : fmodf(d, 360.f);
-    const float r = m - 180.f;
-    return r < -180.f ? r + 360.f : r;
-}
 
 struct BwdArgs {
     uint32_t C;
@@ -43,32 +38,43 @@ struct BwdArgs {
     int first_pass; // adds the alpha / alpha-sum terms exactly once over the channel passes
 };
 
-// Geometry gradient slots per Gaussian in the LDS accumulator, after the CH colour slots.
-enum { G_CONIC = 0, G_XY = 3, G_ABS = 5, G_VEL = 7, G_OPAC = 10, G_DC = 11, G_COUNT = 13 };
+// Geometry gradient slots per Gaussian in the LDS accumulator, after the CH colour slots;
+// the last three exist for lidars only.
+enum { G_CONIC = 0, G_XY = 3, G_ABS = 5, G_VEL = 7, G_OPAC = 9, G_VELZ = 10, G_DC = 11, G_COUNT = 13 };
+
+constexpr int pow2_at_least(int n) { return n <= 16 ? 16 : (n <= 32 ? 32 : 64); }
 
 template <int CH, bool LIDAR>
 __global__ void __launch_bounds__(256)
 rasterize_bwd_kernel(BwdArgs a) {
     extern __shared__ float4 lds4[];
-    const uint32_t block_size = blockDim.x * blockDim.y;
-    float4 *s_xyv = lds4;                  // {x, y, vx, vy}
-    float4 *s_con = lds4 + block_size;     // {conic a, b, c, opacity}
-    float4 *s_ext = lds4 + 2 * block_size; // lidar: {v_range, depth comp 0, depth comp 1, depth}
-    int32_t *s_id = reinterpret_cast<int32_t *>(lds4 + 3 * block_size);
-    float *s_col = reinterpret_cast<float *>(s_id + block_size);        // [block_size][CH]
-    float *s_acc = s_col + (size_t)block_size * CH;                     // [block_size][CH + G_COUNT]
     __shared__ int32_t s_block_final;
-    constexpr int ACC = CH + G_COUNT;
+    __shared__ uint32_t s_ref_thread;
+    __shared__ float s_ref[2];
+    // the workgroup is one-dimensional and padded to whole wavefronts: the wavefront
+    // reductions below need all 64 lanes; lanes beyond the tile own no pixel
+    const uint32_t block_size = blockDim.x;
+    constexpr int RECORD = LIDAR ? 3 : 2; // {x, y, vx, vy}, staged exponent, lidar extras
+    constexpr int GEO = LIDAR ? G_COUNT : G_VELZ;
+    constexpr int ACC = CH + GEO;
+    constexpr int NV = pow2_at_least(ACC);
+    float4 *s_rec = lds4;
+    float2 *s_aux = reinterpret_cast<float2 *>(lds4 + (size_t)RECORD * block_size); // {id, 1/opacity}
+    float *s_col = reinterpret_cast<float *>(s_aux + block_size);                   // [block_size][CH]
+    float *s_acc = s_col + (size_t)block_size * CH;                                 // [block_size][ACC]
 
     const uint32_t tiles_per_cam = a.grid_w * a.grid_h;
     const uint32_t cam = blockIdx.x / tiles_per_cam;
     const uint32_t tile_id = blockIdx.x % tiles_per_cam;
-    const uint32_t i = (tile_id / a.grid_w) * a.tile_h_px + threadIdx.y;
-    const uint32_t j = (tile_id % a.grid_w) * a.tile_w_px + threadIdx.x;
-    const uint32_t tr = threadIdx.y * blockDim.x + threadIdx.x;
+    const uint32_t tr = threadIdx.x;
     const int lane = tr & (SPLATAD_WAVE - 1);
+    uint32_t lx, ly;
+    if (LIDAR) point_of_lane(a.tile_w_px, a.tile_h_px, tr, lx, ly);
+    else pixel_of_lane(a.tile_w_px, tr, lx, ly);
+    const uint32_t i = (tile_id / a.grid_w) * a.tile_h_px + ly;
+    const uint32_t j = (tile_id % a.grid_w) * a.tile_w_px + lx;
 
-    const bool in_image = (i < a.H && j < a.W);
+    const bool in_image = (tr < a.tile_w_px * a.tile_h_px && i < a.H && j < a.W);
     const size_t pix = in_image ? ((size_t)cam * a.H + i) * a.W + j : 0;
     float px, py, pz = 1.f, roll;
     if (LIDAR) {
@@ -84,6 +90,20 @@ rasterize_bwd_kernel(BwdArgs a) {
         roll = a.rs_time[cam] * ((py - 0.5f) / (float)(a.H - 1) - 0.5f);
     }
     const bool inside = in_image && pz > 0.f;
+
+    // lidar: angles relative to the tile's first valid point, as in the forward kernel
+    float ref_x = 0.f, ref_y = 0.f;
+    if (tr == 0) { s_block_final = -1; s_ref_thread = 0xFFFFFFFFu; }
+    __syncthreads();
+    if (LIDAR) {
+        if (inside) atomicMin(&s_ref_thread, tr);
+        __syncthreads();
+        if (tr == s_ref_thread) { s_ref[0] = px; s_ref[1] = py; }
+        __syncthreads();
+        if (s_ref_thread != 0xFFFFFFFFu) { ref_x = s_ref[0]; ref_y = s_ref[1]; }
+        px = angle_difference(px, ref_x); // from here on px, py are relative
+        py = angle_difference(py, ref_y);
+    }
 
     const int32_t *offs = a.tile_offsets + (size_t)cam * tiles_per_cam;
     const int32_t range_start = offs[tile_id];
@@ -118,14 +138,18 @@ rasterize_bwd_kernel(BwdArgs a) {
         if (k == depth_local) v_out_depth = v_out[k];
 
     // deepest entry any pixel of the tile consumed
-    if (tr == 0) s_block_final = -1;
-    __syncthreads();
     const int32_t wave_final = wave_max_i32(bin_final);
     if (lane == 0 && wave_final >= 0) atomicMax(&s_block_final, wave_final);
     __syncthreads();
     const int32_t list_end = min(range_end, s_block_final + 1); // exclusive
     if (list_end <= range_start) return;
     const uint32_t num_batches = (uint32_t)(list_end - range_start + block_size - 1) / block_size;
+
+    // footprint of this wavefront over the lanes that consumed anything
+    WaveCull cull;
+    WavePointCull pcull;
+    if (LIDAR) pcull.init(inside && bin_final >= range_start, px, py, roll, true);
+    else cull.init(px, py, roll, true);
 
     for (uint32_t b = 0; b < num_batches; ++b) {
         __syncthreads(); // previous batch fully flushed
@@ -134,134 +158,141 @@ rasterize_bwd_kernel(BwdArgs a) {
         const int32_t idx = batch_end - (int32_t)tr;
         if (idx >= range_start) {
             const int32_t g = a.flatten_ids[idx];
-            s_id[tr] = g;
             const float2 xy = reinterpret_cast<const float2 *>(a.means2d)[g];
             const float *cn = a.conics + (size_t)g * 3;
-            s_con[tr] = make_float4(cn[0], cn[1], cn[2], a.opacities[g]);
+            const float opac = a.opacities[g];
             const float *crow = a.colors + (size_t)g * a.color_stride;
+            float4 *rec = s_rec + (size_t)RECORD * tr;
             if (LIDAR) {
                 const float *v = a.pix_vels + (size_t)g * 3;
                 const float2 dc = reinterpret_cast<const float2 *>(a.depth_comps)[g];
-                s_xyv[tr] = make_float4(xy.x, xy.y, v[0], v[1]);
-                s_ext[tr] = make_float4(v[2], dc.x, dc.y, crow[a.depth_idx]);
+                rec[0] = make_float4(angle_difference(xy.x, ref_x), angle_difference(xy.y, ref_y), v[0], v[1]);
+                rec[RECORD - 1] = make_float4(v[2], dc.x, dc.y, crow[a.depth_idx]);
             } else {
                 const float2 v = reinterpret_cast<const float2 *>(a.pix_vels)[g];
-                s_xyv[tr] = make_float4(xy.x, xy.y, v.x, v.y);
+                rec[0] = make_float4(xy.x, xy.y, v.x, v.y);
             }
+            rec[1] = staged_exponent(cn[0], cn[1], cn[2], opac);
+            s_aux[tr] = make_float2(__int_as_float(g), 1.0f / opac);
 #pragma unroll
             for (int k = 0; k < CH; ++k) s_col[tr * CH + k] = (uint32_t)k < a.n_ch ? crow[a.ch_offset + k] : 0.f;
         }
         for (uint32_t k = tr; k < (uint32_t)batch_size * ACC; k += block_size) s_acc[k] = 0.f;
         __syncthreads();
 
-        // entry t of the batch sits at list position batch_end - t
+        // entry t of the batch sits at list position batch_end - t; this wavefront starts at
+        // the deepest entry any of its lanes consumed
         const int32_t t0 = max(0, batch_end - wave_final);
-        for (int32_t t = t0; t < batch_size; ++t) {
-            bool valid = inside && (batch_end - t <= bin_final);
-            float alpha = 0.f, opac = 0.f, vis = 0.f, dx = 0.f, dy = 0.f;
-            float4 con = make_float4(0.f, 0.f, 0.f, 0.f), ext = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (valid) {
-                con = s_con[t];
-                const float4 xyv = s_xyv[t];
-                opac = con.w;
-                if (LIDAR) {
-                    ext = s_ext[t];
+        for (int32_t base = t0 & ~(SPLATAD_WAVE - 1); base < batch_size; base += SPLATAD_WAVE) {
+            const int32_t tt = base + lane;
+            bool keep = tt >= t0 && tt < batch_size, unfolded_ok = true;
+            if (keep) {
+                const float4 *rec = s_rec + (size_t)RECORD * tt;
+                keep = LIDAR ? pcull.may_touch(rec[0], rec[1], unfolded_ok) : cull.may_touch(rec[0], rec[1]);
+            }
+            uint64_t todo = wave_ballot(keep);
+            const uint64_t folded = wave_ballot(keep && !unfolded_ok);
+            while (todo) {
+                const int32_t bit = __ffsll((unsigned long long)todo) - 1;
+                const int32_t t = base + bit;
+                todo &= todo - 1;
+                const float4 *rec = s_rec + (size_t)RECORD * t;
+                const float4 xyv = rec[0];
+                const float4 e = rec[1];
+                float dx = (xyv.x + roll * xyv.z) - px;
+                float dy = (xyv.y + roll * xyv.w) - py;
+                if (LIDAR && ((folded >> bit) & 1ull)) { // uniform, rare
                     dx = angle_difference(xyv.x + roll * xyv.z, px);
                     dy = angle_difference(xyv.y + roll * xyv.w, py);
-                } else {
-                    dx = xyv.x + roll * xyv.z - px;
-                    dy = xyv.y + roll * xyv.w - py;
                 }
-                const float sigma = 0.5f * (con.x * dx * dx + con.z * dy * dy) + con.y * dx * dy;
-                vis = __expf(-sigma);
-                alpha = fminf(0.999f, opac * vis);
-                if (sigma < 0.f || alpha < 1.f / 255.f) valid = false;
-            }
-            if (__ballot(valid) == 0) continue;
+                const float power = dx * (e.x * dx + e.y * dy) + e.z * dy * dy;
+                const float au = __builtin_amdgcn_exp2f(e.w - power); // opacity * exp(-sigma)
+                const float alpha = fminf(0.999f, au);
+                const bool valid = inside && (batch_end - t <= bin_final) && !(power < 0.f) &&
+                                   !(alpha < 1.f / 255.f);
+                if (wave_ballot(valid) == 0) continue;
 
-            float g_col[CH];
-            float g_conic0 = 0.f, g_conic1 = 0.f, g_conic2 = 0.f, g_x = 0.f, g_y = 0.f, g_ax = 0.f,
-                  g_ay = 0.f, g_vx = 0.f, g_vy = 0.f, g_vz = 0.f, g_op = 0.f, g_dc0 = 0.f, g_dc1 = 0.f;
+                float v[NV];
 #pragma unroll
-            for (int k = 0; k < CH; ++k) g_col[k] = 0.f;
-            if (valid) {
-                const float ra = 1.0f / (1.0f - alpha);
-                T *= ra; // transmittance in front of this Gaussian
-                const float fac = alpha * T;
-                float v_alpha = 0.f;
+                for (int k = 0; k < NV; ++k) v[k] = 0.f;
+                if (valid) {
+                    const float ra = 1.0f / (1.0f - alpha);
+                    T *= ra; // transmittance in front of this Gaussian
+                    const float fac = alpha * T;
+                    float v_alpha = 0.f;
 #pragma unroll
-                for (int k = 0; k < CH; ++k) {
-                    g_col[k] = fac * v_out[k];
-                    v_alpha += (s_col[t * CH + k] * T - buffer[k] * ra) * v_out[k];
-                }
-                float extra = 0.f;
-                if (LIDAR) {
-                    extra = ext.y * dx + ext.z * dy + ext.x * roll;
-                    // depth channel = colour + extra: both enter c*T and the buffer
-                    v_alpha += (extra * T - buffer_extra * ra) * v_out_depth;
-                }
-                v_alpha += T_final * ra * v_render_a;
-                v_alpha += -T_final * ra * bg_dot;
-                const float g_depth = fac * v_out_depth; // gradient of the depth channel value
-                if (opac * vis <= 0.999f) {
-                    const float v_sigma = -opac * vis * v_alpha;
-                    g_conic0 = 0.5f * v_sigma * dx * dx;
-                    g_conic1 = v_sigma * dx * dy;
-                    g_conic2 = 0.5f * v_sigma * dy * dy;
-                    g_x = v_sigma * (con.x * dx + con.y * dy);
-                    g_y = v_sigma * (con.y * dx + con.z * dy);
-                    if (LIDAR) {
-                        g_dc0 = g_depth * dx;
-                        g_dc1 = g_depth * dy;
-                        g_vz = g_depth * roll;
-                        g_x += g_depth * ext.y;
-                        g_y += g_depth * ext.z;
+                    for (int k = 0; k < CH; ++k) {
+                        v[k] = fac * v_out[k];
+                        v_alpha += (s_col[t * CH + k] * T - buffer[k] * ra) * v_out[k];
                     }
-                    g_vx = g_x * roll;
-                    g_vy = g_y * roll;
-                    g_ax = fabsf(g_x);
-                    g_ay = fabsf(g_y);
-                    g_op = vis * v_alpha;
-                }
-#pragma unroll
-                for (int k = 0; k < CH; ++k) buffer[k] += s_col[t * CH + k] * fac;
-                if (LIDAR) {
-                    buffer_extra += extra * fac;
-                    if (a.compute_alpha_sum && ext.w < pz - a.threshold) {
-                        const float v_sig2 = v_asum * -opac * vis;
-                        const float ex = v_sig2 * (con.x * dx + con.y * dy);
-                        const float ey = v_sig2 * (con.y * dx + con.z * dy);
-                        g_x += ex; g_y += ey;
-                        g_vx += ex * roll; g_vy += ey * roll;
-                        g_ax += fabsf(ex); g_ay += fabsf(ey);
-                        g_conic0 += v_sig2 * 0.5f * dx * dx;
-                        g_conic1 += v_sig2 * dx * dy;
-                        g_conic2 += v_sig2 * 0.5f * dy * dy;
-                        g_op += v_asum * vis;
+                    float4 ext = make_float4(0.f, 0.f, 0.f, 0.f);
+                    float extra = 0.f;
+                    if constexpr (LIDAR) {
+                        ext = rec[RECORD - 1];
+                        extra = ext.y * dx + ext.z * dy + ext.x * roll;
+                        // depth channel = colour + extra: both enter c*T and the buffer
+                        v_alpha += (extra * T - buffer_extra * ra) * v_out_depth;
                     }
+                    v_alpha += T_final * ra * v_render_a;
+                    v_alpha += -T_final * ra * bg_dot;
+                    const float g_depth = fac * v_out_depth; // gradient of the depth channel value
+                    const float rop = s_aux[t].y;
+                    // conic row products a dx + b dy and b dx + c dy from the staged form
+                    const float row_x = kLn2 * (2.f * e.x * dx + e.y * dy);
+                    const float row_y = kLn2 * (e.y * dx + 2.f * e.z * dy);
+                    float g_x = 0.f, g_y = 0.f, g_ax = 0.f, g_ay = 0.f;
+                    if (au <= 0.999f) {
+                        const float v_sigma = -au * v_alpha;
+                        v[CH + G_CONIC] = 0.5f * v_sigma * dx * dx;
+                        v[CH + G_CONIC + 1] = v_sigma * dx * dy;
+                        v[CH + G_CONIC + 2] = 0.5f * v_sigma * dy * dy;
+                        g_x = v_sigma * row_x;
+                        g_y = v_sigma * row_y;
+                        if constexpr (LIDAR) {
+                            v[CH + G_DC] = g_depth * dx;
+                            v[CH + G_DC + 1] = g_depth * dy;
+                            v[CH + G_VELZ] = g_depth * roll;
+                            g_x += g_depth * ext.y;
+                            g_y += g_depth * ext.z;
+                        }
+                        g_ax = fabsf(g_x);
+                        g_ay = fabsf(g_y);
+                        v[CH + G_OPAC] = au * rop * v_alpha;
+                    }
+#pragma unroll
+                    for (int k = 0; k < CH; ++k) buffer[k] += s_col[t * CH + k] * fac;
+                    if constexpr (LIDAR) {
+                        buffer_extra += extra * fac;
+                        if (a.compute_alpha_sum && ext.w < pz - a.threshold) {
+                            const float v_sig2 = -v_asum * au;
+                            const float ex = v_sig2 * row_x, ey = v_sig2 * row_y;
+                            g_x += ex; g_y += ey;
+                            g_ax += fabsf(ex); g_ay += fabsf(ey);
+                            v[CH + G_CONIC] += v_sig2 * 0.5f * dx * dx;
+                            v[CH + G_CONIC + 1] += v_sig2 * dx * dy;
+                            v[CH + G_CONIC + 2] += v_sig2 * 0.5f * dy * dy;
+                            v[CH + G_OPAC] += v_asum * au * rop;
+                        }
+                    }
+                    v[CH + G_XY] = g_x;
+                    v[CH + G_XY + 1] = g_y;
+                    v[CH + G_ABS] = g_ax;
+                    v[CH + G_ABS + 1] = g_ay;
+                    v[CH + G_VEL] = g_x * roll;
+                    v[CH + G_VEL + 1] = g_y * roll;
                 }
-            }
-            // sum over the wavefront, then one LDS atomic per value and wavefront
-            float *acc = s_acc + (size_t)t * ACC;
-#pragma unroll
-            for (int k = 0; k < CH; ++k) {
-                const float s = wave_sum(g_col[k]);
-                if (lane == 0 && (uint32_t)k < a.n_ch) atomicAdd(acc + k, s);
-            }
-            float geo[G_COUNT] = {g_conic0, g_conic1, g_conic2, g_x, g_y, g_ax, g_ay,
-                                  g_vx, g_vy, g_vz, g_op, g_dc0, g_dc1};
-#pragma unroll
-            for (int q = 0; q < G_COUNT; ++q) {
-                if (!LIDAR && (q == G_VEL + 2 || q >= G_DC)) continue;
-                const float s = wave_sum(geo[q]);
-                if (lane == 0) atomicAdd(acc + CH + q, s);
+                // sum over the wavefront; the lane that ends up with slot s adds it in LDS
+                wave_reduce_scatter<NV>(v, lane);
+                const int slot = wave_reduce_slot<NV>(lane);
+                if (slot < ACC && (lane & (64 / NV - 1)) == 0 && v[0] != 0.f)
+                    atomicAdd(s_acc + (size_t)t * ACC + slot, v[0]);
             }
         }
         __syncthreads();
 
         // flush the batch: lane tr owns Gaussian tr of the batch
         if ((int32_t)tr < batch_size) {
-            const int32_t g = s_id[tr];
+            const int32_t g = __float_as_int(s_aux[tr].x);
             const float *acc = s_acc + (size_t)tr * ACC;
             float *vc = a.v_colors + (size_t)g * a.color_stride + a.ch_offset;
 #pragma unroll
@@ -284,10 +315,13 @@ rasterize_bwd_kernel(BwdArgs a) {
                 atomicAdd(a.v_pix_vels + (size_t)g * nv + 1, geo[G_VEL + 1]);
                 atomicAdd(a.v_opacities + g, geo[G_OPAC]);
             }
-            if (LIDAR && (geo[G_VEL + 2] != 0.f || geo[G_DC] != 0.f || geo[G_DC + 1] != 0.f)) {
-                atomicAdd(a.v_pix_vels + (size_t)g * 3 + 2, geo[G_VEL + 2]);
-                atomicAdd(a.v_depth_comps + (size_t)g * 2, geo[G_DC]);
-                atomicAdd(a.v_depth_comps + (size_t)g * 2 + 1, geo[G_DC + 1]);
+            if constexpr (LIDAR) {
+                const float gz = acc[CH + G_VELZ], d0 = acc[CH + G_DC], d1 = acc[CH + G_DC + 1];
+                if (gz != 0.f || d0 != 0.f || d1 != 0.f) {
+                    atomicAdd(a.v_pix_vels + (size_t)g * 3 + 2, gz);
+                    atomicAdd(a.v_depth_comps + (size_t)g * 2, d0);
+                    atomicAdd(a.v_depth_comps + (size_t)g * 2 + 1, d1);
+                }
             }
         }
     }
@@ -305,7 +339,7 @@ static inline int pick_width(uint32_t n) {
 template <int CH, bool LIDAR>
 static int launch_bwd(const BwdArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
     const size_t bs = (size_t)block.x * block.y;
-    const size_t lds = bs * (48 + 4) + bs * 4 * CH + bs * 4 * (CH + G_COUNT);
+    const size_t lds = bs * ((LIDAR ? 48 : 32) + 8) + bs * 4 * CH + bs * 4 * (CH + (LIDAR ? G_COUNT : G_VELZ));
     if (lds > 64 * 1024)
         SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_bwd_kernel<CH, LIDAR>,
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -378,8 +412,8 @@ extern "C" int splatad_rasterize_to_pixels_bwd(
     a.v_render_colors = v_render_colors; a.v_render_alphas = v_render_alphas;
     a.v_means2d_abs = v_means2d_abs; a.v_means2d = v_means2d; a.v_conics = v_conics;
     a.v_colors = v_colors; a.v_opacities = v_opacities; a.v_pix_vels = v_pix_vels;
-    return run_passes<false>(a, channels, dim3(C * tile_w * tile_h), dim3(tile_size, tile_size),
-                             (hipStream_t)stream);
+    return run_passes<false>(a, channels, dim3(C * tile_w * tile_h),
+                             dim3((tile_size * tile_size + 63) / 64 * 64), (hipStream_t)stream);
 }
 
 extern "C" int splatad_rasterize_to_points_bwd(
@@ -418,6 +452,6 @@ extern "C" int splatad_rasterize_to_points_bwd(
     a.v_means2d_abs = v_means2d_abs; a.v_means2d = v_means2d; a.v_conics = v_conics;
     a.v_colors = v_colors; a.v_opacities = v_opacities; a.v_pix_vels = v_pix_vels;
     a.v_depth_comps = v_depth_comps;
-    return run_passes<true>(a, channels, dim3(C * grid_w * grid_h), dim3(tile_width, tile_height),
-                            (hipStream_t)stream);
+    return run_passes<true>(a, channels, dim3(C * grid_w * grid_h),
+                            dim3((tile_width * tile_height + 63) / 64 * 64), (hipStream_t)stream);
 }

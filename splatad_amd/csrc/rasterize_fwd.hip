@@ -16,7 +16,7 @@
 // Channels: the kernels are compiled for CH accumulators per lane and take the real
 // channel count, stride and offset at run time, so any channel count is rendered without
 // host-side padding (wide inputs in passes of up to 32 channels).
-#include "common.h"
+#include "raster_common.h"
 
 namespace {
 
@@ -32,42 +32,6 @@ struct PixelArgs {
     float *render_colors, *render_alphas;
     int32_t *last_ids;
     int write_aux; // first pass also writes alphas and last ids
-};
-
-// Conservative test of one Gaussian against the footprint of a wavefront.  With the staged
-// record {A, B, C, L} (see the kernel), alpha = exp2(L - p(d)), p(d) = A dx^2 + B dx dy +
-// C dy^2.  The smallest value of p over the box of offsets d = mean - pixel that the
-// wavefront's pixels can see (widened by the rolling-shutter shift of the mean across the
-// wavefront's rows) is compared with the largest p that still passes the alpha >= 1/255
-// test, L + log2(255).  p is convex for a positive definite conic, so off the centre its
-// minimum over the box lies on one of the four edges.  A margin covers the rounding of this
-// test; Gaussians with a degenerate conic are never culled.
-struct WaveCull {
-    bool enabled;
-    float cx, cy;     // centre of the footprint
-    float hx, hy;     // half extents
-    float roll_mid, roll_half;
-
-    __device__ __forceinline__ static float edge_min(float a2, float c2, float b, float fixed,
-                                                     float lo, float hi) {
-        // fixed coordinate uses a2 (= a / 2), free coordinate uses c2 (= c / 2)
-        const float free_c = fminf(fmaxf(-b * fixed / (2.f * c2), lo), hi);
-        return a2 * fixed * fixed + c2 * free_c * free_c + b * fixed * free_c;
-    }
-
-    __device__ __forceinline__ bool may_touch(const float4 xyv, const float4 con) const {
-        const float mx = xyv.x + roll_mid * xyv.z - cx, my = xyv.y + roll_mid * xyv.w - cy;
-        const float ex = hx + fabsf(xyv.z) * roll_half, ey = hy + fabsf(xyv.w) * roll_half;
-        const float x0 = mx - ex, x1 = mx + ex, y0 = my - ey, y1 = my + ey;
-        const float a2 = con.x, c2 = con.z, b = con.y;
-        const bool definite = a2 > 0.f && c2 > 0.f && 4.f * a2 * c2 - b * b > 0.f;
-        const bool centre_in = x0 <= 0.f && x1 >= 0.f && y0 <= 0.f && y1 >= 0.f;
-        const float q = fminf(fminf(edge_min(a2, c2, b, x0, y0, y1), edge_min(a2, c2, b, x1, y0, y1)),
-                              fminf(edge_min(c2, a2, b, y0, x0, x1), edge_min(c2, a2, b, y1, x0, x1)));
-        const float limit = con.w + 7.99435343685886f; // log2(255)
-        const bool cull = definite && !centre_in && q > limit + 1e-3f * fabsf(limit) + 0.02f;
-        return !cull;
-    }
 };
 
 template <int CH>
@@ -87,14 +51,8 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     const uint32_t tile_y = tile_id / a.tile_w, tile_x = tile_id % a.tile_w;
     const uint32_t tr = threadIdx.y * blockDim.x + threadIdx.x;
     const uint32_t lane = tr & (SPLATAD_WAVE - 1);
-    // pixel of this lane: wavefronts cover 8x8 squares when the tile allows it (a compact
-    // footprint is what makes the per-wavefront culling below effective), rows otherwise
-    uint32_t lx = threadIdx.x, ly = threadIdx.y;
-    if (a.tile_size % 8 == 0) {
-        const uint32_t squares_per_row = a.tile_size / 8, square = tr / SPLATAD_WAVE;
-        lx = (square % squares_per_row) * 8 + (lane & 7);
-        ly = (square / squares_per_row) * 8 + (lane >> 3);
-    }
+    uint32_t lx, ly;
+    pixel_of_lane(a.tile_size, tr, lx, ly);
     const uint32_t i = tile_y * a.tile_size + ly;
     const uint32_t j = tile_x * a.tile_size + lx;
 
@@ -112,25 +70,7 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
 
     // footprint of this wavefront (all 64 lanes exist when the workgroup is a multiple of 64)
     WaveCull cull;
-    cull.enabled = block_size % SPLATAD_WAVE == 0;
-    {
-        float x_lo = px, x_hi = px, y_lo = py, y_hi = py, r_lo = roll, r_hi = roll;
-        if (cull.enabled) {
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) {
-                x_lo = fminf(x_lo, __shfl_xor(x_lo, off, SPLATAD_WAVE));
-                x_hi = fmaxf(x_hi, __shfl_xor(x_hi, off, SPLATAD_WAVE));
-                y_lo = fminf(y_lo, __shfl_xor(y_lo, off, SPLATAD_WAVE));
-                y_hi = fmaxf(y_hi, __shfl_xor(y_hi, off, SPLATAD_WAVE));
-                r_lo = fminf(r_lo, __shfl_xor(r_lo, off, SPLATAD_WAVE));
-                r_hi = fmaxf(r_hi, __shfl_xor(r_hi, off, SPLATAD_WAVE));
-            }
-        }
-        cull.cx = 0.5f * (x_lo + x_hi); cull.hx = 0.5f * (x_hi - x_lo);
-        cull.cy = 0.5f * (y_lo + y_hi); cull.hy = 0.5f * (y_hi - y_lo);
-        cull.roll_mid = 0.5f * (r_lo + r_hi);
-        cull.roll_half = 0.5f * (r_hi - r_lo) * 1.0001f + 1e-12f;
-    }
+    cull.init(px, py, roll, block_size % SPLATAD_WAVE == 0);
 
     float T = 1.0f;
     uint32_t cur_idx = 0;
@@ -149,11 +89,8 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
             const float2 xy = reinterpret_cast<const float2 *>(a.means2d)[g];
             const float2 v = reinterpret_cast<const float2 *>(a.pix_vels)[g];
             const float *cn = a.conics + (size_t)g * 3;
-            constexpr float kLog2e = 1.44269504088896341f;
-            const float opac = a.opacities[g];
             s_rec[RECORD * tr] = make_float4(xy.x, xy.y, v.x, v.y);
-            s_rec[RECORD * tr + 1] = make_float4(0.5f * kLog2e * cn[0], kLog2e * cn[1],
-                                            0.5f * kLog2e * cn[2], opac > 0.f ? __log2f(opac) : -INFINITY);
+            s_rec[RECORD * tr + 1] = staged_exponent(cn[0], cn[1], cn[2], a.opacities[g]);
             const float *c = a.colors + (size_t)g * a.color_stride + a.ch_offset;
 #pragma unroll
             for (int k = 0; k < CH; ++k)
@@ -166,7 +103,7 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
             // lanes test 64 Gaussians against the wavefront's footprint, then all lanes walk
             // the survivors (a wave-uniform loop over the set bits)
             bool keep = base + lane < batch_size;
-            if (keep && cull.enabled) keep = cull.may_touch(s_rec[RECORD * (base + lane)], s_rec[RECORD * (base + lane) + 1]);
+            if (keep) keep = cull.may_touch(s_rec[RECORD * (base + lane)], s_rec[RECORD * (base + lane) + 1]);
             uint64_t todo = wave_ballot(keep);
             while (todo) {
                 const uint32_t t = base + (uint32_t)__ffsll((unsigned long long)todo) - 1u;
@@ -227,47 +164,6 @@ struct PointArgs {
     int write_aux;
 };
 
-// Difference of two angles in degrees folded into [-180, 180), as the reference's
-// fmodf(a - b + 180, 360) - 180 with negative results raised by 360.  Without the detour
-// through +180 / -180 the difference of two nearby angles is exact in float32.
-__device__ __forceinline__ float angle_difference(float a, float b) {
-    const float d = a - b;
-    if (d >= -180.f && d < 180.f) return d;
-    float m = fmodf(d + 180.f, 360.f);
-    if (m < 0.f) m += 360.f;
-    return m - 180.f;
-}
-
-// Footprint test for a wavefront of lidar points, the counterpart of WaveCull.  All angles
-// are taken relative to a reference point of the tile, so that neither the +-180 degree
-// seam nor the size of the absolute angles matters: the staged record holds u = (mean -
-// reference) and the lane r = (point - reference), both folded, and the offset of a pair is
-// u + roll * velocity - r as long as that cannot leave (-180, 180).  The test decides for
-// every Gaussian whether any lane can reach alpha >= 1/255 and whether the unfolded
-// difference is safe (it is unless the Gaussian sits half a turn away from the tile).
-struct WavePointCull {
-    bool enabled;
-    float x_lo, x_hi, y_lo, y_hi; // box of the lanes' r
-    float roll_mid, roll_half;
-
-    __device__ __forceinline__ bool may_touch(const float4 uv, const float4 con, bool &unfolded_ok) const {
-        const float cx = uv.x + roll_mid * uv.z, cy = uv.y + roll_mid * uv.w;
-        const float ex = fabsf(uv.z) * roll_half, ey = fabsf(uv.w) * roll_half;
-        const float x0 = cx - x_hi - ex, x1 = cx - x_lo + ex;
-        const float y0 = cy - y_hi - ey, y1 = cy - y_lo + ey;
-        unfolded_ok = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(y0), fabsf(y1))) < 179.f;
-        if (!unfolded_ok || !enabled) return true;
-        const float a2 = con.x, c2 = con.z, b = con.y;
-        const bool definite = a2 > 0.f && c2 > 0.f && 4.f * a2 * c2 - b * b > 0.f;
-        const bool centre_in = x0 <= 0.f && x1 >= 0.f && y0 <= 0.f && y1 >= 0.f;
-        const float q = fminf(fminf(WaveCull::edge_min(a2, c2, b, x0, y0, y1), WaveCull::edge_min(a2, c2, b, x1, y0, y1)),
-                              fminf(WaveCull::edge_min(c2, a2, b, y0, x0, x1), WaveCull::edge_min(c2, a2, b, y1, x0, x1)));
-        const float limit = con.w + 7.99435343685886f; // log2(255)
-        const bool cull = definite && !centre_in && q > limit + 1e-3f * fabsf(limit) + 0.02f;
-        return !cull;
-    }
-};
-
 template <int CH>
 __global__ void __launch_bounds__(256)
 rasterize_to_points_fwd_kernel(PointArgs a) {
@@ -286,13 +182,8 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
     const uint32_t tile_id = blockIdx.x % tiles_per_cam;
     const uint32_t tr = threadIdx.y * blockDim.x + threadIdx.x;
     const uint32_t lane = tr & (SPLATAD_WAVE - 1);
-    // point of this lane: a wavefront covers 16 columns of all four rows when the tile
-    // allows it (the compact footprint culls better than one row of 64 columns)
-    uint32_t lx = threadIdx.x, ly = threadIdx.y;
-    if (a.tile_height == 4 && a.tile_width % 16 == 0) {
-        lx = (tr / SPLATAD_WAVE) * 16 + (lane & 15);
-        ly = lane >> 4;
-    }
+    uint32_t lx, ly;
+    point_of_lane(a.tile_width, a.tile_height, tr, lx, ly);
     const uint32_t i = (tile_id / a.grid_w) * a.tile_height + ly;
     const uint32_t j = (tile_id % a.grid_w) * a.tile_width + lx;
 
@@ -328,32 +219,7 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
 
     // footprint of this wavefront over its valid lanes
     WavePointCull cull;
-    cull.enabled = block_size % SPLATAD_WAVE == 0;
-    {
-        const float inf = INFINITY;
-        float x_lo = alive ? rx : inf, x_hi = alive ? rx : -inf;
-        float y_lo = alive ? ry : inf, y_hi = alive ? ry : -inf;
-        float r_lo = alive ? roll : inf, r_hi = alive ? roll : -inf;
-        if (cull.enabled) {
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) {
-                x_lo = fminf(x_lo, __shfl_xor(x_lo, off, SPLATAD_WAVE));
-                x_hi = fmaxf(x_hi, __shfl_xor(x_hi, off, SPLATAD_WAVE));
-                y_lo = fminf(y_lo, __shfl_xor(y_lo, off, SPLATAD_WAVE));
-                y_hi = fmaxf(y_hi, __shfl_xor(y_hi, off, SPLATAD_WAVE));
-                r_lo = fminf(r_lo, __shfl_xor(r_lo, off, SPLATAD_WAVE));
-                r_hi = fmaxf(r_hi, __shfl_xor(r_hi, off, SPLATAD_WAVE));
-            }
-        } else { // partial wavefront: no culling, bounds of the whole (-180, 180] range
-            x_lo = y_lo = -180.f; x_hi = y_hi = 180.f;
-            r_lo = r_hi = roll;
-        }
-        // slightly widened against the rounding of the test itself
-        cull.x_lo = x_lo - 1e-4f; cull.x_hi = x_hi + 1e-4f;
-        cull.y_lo = y_lo - 1e-4f; cull.y_hi = y_hi + 1e-4f;
-        cull.roll_mid = 0.5f * (r_lo + r_hi);
-        cull.roll_half = 0.5f * (r_hi - r_lo) * 1.0001f + 1e-12f;
-    }
+    cull.init(alive, rx, ry, roll, block_size % SPLATAD_WAVE == 0);
 
     float T = 1.0f, asum = 0.f, median = 0.f, depth_extra = 0.f;
     uint32_t cur_idx = 0;
@@ -373,12 +239,9 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
             const float2 dc = reinterpret_cast<const float2 *>(a.depth_comps)[g];
             const float *cn = a.conics + (size_t)g * 3;
             const float *crow = a.colors + (size_t)g * a.color_stride;
-            constexpr float kLog2e = 1.44269504088896341f;
-            const float opac = a.opacities[g];
             float4 *rec = s_rec + RECORD * tr;
             rec[0] = make_float4(angle_difference(xy.x, ref_x), angle_difference(xy.y, ref_y), v[0], v[1]);
-            rec[1] = make_float4(0.5f * kLog2e * cn[0], kLog2e * cn[1], 0.5f * kLog2e * cn[2],
-                                 opac > 0.f ? __log2f(opac) : -INFINITY);
+            rec[1] = staged_exponent(cn[0], cn[1], cn[2], a.opacities[g]);
             rec[2] = make_float4(v[2], dc.x, dc.y, crow[a.depth_idx]);
             const float *c = crow + a.ch_offset;
 #pragma unroll
