@@ -65,6 +65,33 @@ __device__ __forceinline__ void sh_for_each_basis(uint32_t degree, float x, floa
     f(24, k4 * c3, k4 * 4.f * c2, -k4 * 4.f * s2, 0.f);
 }
 
+// Coefficient rows ([K][3] floats per direction) are 12 K bytes apart, so a lane-per-row
+// store writes 4 bytes into each of 64 cache lines per instruction.  The backward kernel
+// therefore collects a workgroup's gradient rows in LDS (rows padded by one float so that
+// the lanes of a wavefront hit different banks) and stores them with coalesced accesses
+// (consecutive lanes, consecutive floats).  Only the first `used` floats of a row
+// (3 (degree + 1)^2) are moved.
+struct ShRows {
+    uint32_t K3;     // floats per row in global memory
+    uint32_t used;   // floats per row that the degree needs
+    uint32_t dq, dr; // blockDim.x / K3 and blockDim.x % K3
+};
+
+// f(lds_index, global_index) for every used float of the workgroup's `rows` rows
+template <typename F>
+__device__ __forceinline__ void sh_for_each_float(const ShRows &r, uint32_t rows, F &&f) {
+    uint32_t row = threadIdx.x / r.K3, col = threadIdx.x % r.K3;
+    const uint32_t total = rows * r.K3;
+    for (uint32_t e = threadIdx.x; e < total; e += blockDim.x) {
+        if (col < r.used) f(row * (r.used + 1) + col, e);
+        row += r.dq;
+        col += r.dr;
+        if (col >= r.K3) { col -= r.K3; ++row; }
+    }
+}
+
+// Forward: every lane reads its own row; the rows are read completely, so the cache lines a
+// wavefront touches are all used (measured faster than staging through LDS).
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, const float *__restrict__ dirs,
               const float *__restrict__ coeffs, const uint8_t *__restrict__ masks,
@@ -89,37 +116,67 @@ sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, const float *__restrict__
 }
 
 __global__ void __launch_bounds__(SPLATAD_THREADS)
-sh_bwd_kernel(uint32_t n, uint32_t K, uint32_t degree, const float *__restrict__ dirs,
+sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, const float *__restrict__ dirs,
               const float *__restrict__ coeffs, const uint8_t *__restrict__ masks,
               const float *__restrict__ v_colors, float *__restrict__ v_coeffs,
               float *__restrict__ v_dirs) {
-    const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n) return;
-    if (masks != nullptr && !masks[e]) return; // gradients stay zero
-    const float dx = dirs[(size_t)e * 3], dy = dirs[(size_t)e * 3 + 1], dz = dirs[(size_t)e * 3 + 2];
-    const float inorm = rsqrtf(dx * dx + dy * dy + dz * dz);
-    const float x = dx * inorm, y = dy * inorm, z = dz * inorm;
-    const float vr = v_colors[(size_t)e * 3], vg = v_colors[(size_t)e * 3 + 1], vb = v_colors[(size_t)e * 3 + 2];
-    const float *cf = coeffs + (size_t)e * K * 3;
-    float *vcf = v_coeffs + (size_t)e * K * 3;
-    float gx = 0.f, gy = 0.f, gz = 0.f;
+    extern __shared__ float s_rows[];
+    const uint32_t first = blockIdx.x * blockDim.x;
+    const uint32_t here = min(blockDim.x, n - first);
     const bool want_dirs = v_dirs != nullptr;
-    sh_for_each_basis(degree, x, y, z, [&](int k, float v, float bx, float by, float bz) {
-        vcf[k * 3] = v * vr;
-        vcf[k * 3 + 1] = v * vg;
-        vcf[k * 3 + 2] = v * vb;
-        if (want_dirs) {
-            const float w = cf[k * 3] * vr + cf[k * 3 + 1] * vg + cf[k * 3 + 2] * vb;
-            gx += w * bx; gy += w * by; gz += w * bz;
+    const uint32_t e = first + threadIdx.x;
+    // every lane writes its row of coefficient gradients to LDS, from where the workgroup
+    // stores them coalesced; rows of masked directions are zeros (their gradients are zero)
+    float *row = s_rows + (size_t)threadIdx.x * (rows.used + 1);
+    const float *cf = coeffs + (size_t)min(e, n - 1) * rows.K3;
+    if (e < n) {
+        const bool active = masks == nullptr || masks[e];
+        const float dx = active ? dirs[(size_t)e * 3] : 0.f, dy = active ? dirs[(size_t)e * 3 + 1] : 0.f;
+        const float dz = active ? dirs[(size_t)e * 3 + 2] : 0.f;
+        const float inorm = active ? rsqrtf(dx * dx + dy * dy + dz * dz) : 0.f;
+        const float x = dx * inorm, y = dy * inorm, z = active ? dz * inorm : 1.f;
+        const float vr = active ? v_colors[(size_t)e * 3] : 0.f;
+        const float vg = active ? v_colors[(size_t)e * 3 + 1] : 0.f;
+        const float vb = active ? v_colors[(size_t)e * 3 + 2] : 0.f;
+        float gx = 0.f, gy = 0.f, gz = 0.f;
+        sh_for_each_basis(degree, x, y, z, [&](int k, float v, float bx, float by, float bz) {
+            if (want_dirs) {
+                const float w = cf[k * 3] * vr + cf[k * 3 + 1] * vg + cf[k * 3 + 2] * vb;
+                gx += w * bx; gy += w * by; gz += w * bz;
+            }
+            row[k * 3] = v * vr;
+            row[k * 3 + 1] = v * vg;
+            row[k * 3 + 2] = v * vb;
+        });
+        if (want_dirs && active) {
+            // through the normalisation: (I - n n^T) g / |d|
+            const float dot = gx * x + gy * y + gz * z;
+            v_dirs[(size_t)e * 3] = (gx - dot * x) * inorm;
+            v_dirs[(size_t)e * 3 + 1] = (gy - dot * y) * inorm;
+            v_dirs[(size_t)e * 3 + 2] = (gz - dot * z) * inorm;
         }
-    });
-    if (want_dirs) {
-        // through the normalisation: (I - n n^T) g / |d|
-        const float dot = gx * x + gy * y + gz * z;
-        v_dirs[(size_t)e * 3] = (gx - dot * x) * inorm;
-        v_dirs[(size_t)e * 3 + 1] = (gy - dot * y) * inorm;
-        v_dirs[(size_t)e * 3 + 2] = (gz - dot * z) * inorm;
     }
+    __syncthreads();
+    float *gout = v_coeffs + (size_t)first * rows.K3;
+    sh_for_each_float(rows, here, [&](uint32_t l, uint32_t f) { gout[f] = s_rows[l]; });
+}
+
+static ShRows sh_rows(uint32_t K, uint32_t degree) {
+    ShRows r;
+    r.K3 = K * 3;
+    r.used = (degree + 1) * (degree + 1) * 3;
+    r.dq = SPLATAD_THREADS / r.K3;
+    r.dr = SPLATAD_THREADS % r.K3;
+    return r;
+}
+
+template <typename Kernel>
+static int sh_lds(Kernel kernel, const ShRows &r, size_t *bytes) {
+    *bytes = (size_t)SPLATAD_THREADS * (r.used + 1) * sizeof(float);
+    if (*bytes > 64 * 1024)
+        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)kernel,
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)*bytes));
+    return 0;
 }
 
 } // namespace
@@ -145,8 +202,11 @@ extern "C" int splatad_sh_bwd(uint32_t n, uint32_t K, uint32_t degree, const flo
     SPLATAD_REQUIRE((degree + 1) * (degree + 1) <= K, "spherical harmonics: %u bases for degree %u", K, degree);
     if (n == 0) return 0;
     SPLATAD_REQUIRE(dirs && coeffs && v_colors && v_coeffs, "spherical harmonics: null pointer argument");
+    const ShRows r = sh_rows(K, degree);
+    size_t lds = 0;
+    if (int rc = sh_lds(sh_bwd_kernel, r, &lds)) return rc;
     hipLaunchKernelGGL(sh_bwd_kernel, dim3((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS),
-                       dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, n, K, degree, dirs, coeffs,
+                       dim3(SPLATAD_THREADS), lds, (hipStream_t)stream, n, r, degree, dirs, coeffs,
                        masks, v_colors, v_coeffs, v_dirs);
     SPLATAD_LAUNCH_CHECK();
     return 0;
