@@ -22,6 +22,16 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
+# HBM bytes per launch of the two compositing kernels on the default workloads, from
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this file (KiB per dispatch,
+# scaled by what the same counters read for a 1 GiB device-to-device copy: FETCH_SIZE reads
+# 0.5 KiB per KiB, WRITE_SIZE 1.0).  Summaries: profiles/rasterize_kernels_counters_1M.txt.
+# They describe the 1M-Gaussian default only; other sizes report null.
+MEASURED_TRAFFIC_BYTES = {
+    "camera": int((12972.2 * 2.0 + 48600.0) * 1024),
+    "lidar": int((36864.9 * 2.0 + 40193.0) * 1024),
+}
+
 
 def _sync():
     import torch
@@ -197,6 +207,57 @@ def bench_lidar(args):
                 n_isects=n_isects, i_need=i_need, channels=D)
 
 
+def bench_backward(args):
+    """Forward + backward (L1 losses on colour, depth and alpha against random targets, the
+    shape of BASELINE configs[4]) of the camera and the lidar call, ms per step."""
+    import torch
+
+    from splatad_amd import lidar_rasterization, rasterization, workloads
+
+    dev = torch.device("cuda:0")
+    out = {}
+    s = workloads.to_device(workloads.camera_driving(n=args.n), dev)
+    names = ("means", "quats", "scales", "opacities", "colors")
+    p = {k: s[k].clone().requires_grad_(True) for k in names}
+    g = torch.Generator(device=dev).manual_seed(7)
+    target = torch.rand((1, s["height"], s["width"], 4), device=dev, generator=g)
+
+    def cam_step():
+        rc, ra, _ = rasterization(
+            p["means"], p["quats"], p["scales"], p["opacities"], p["colors"], s["velocities"],
+            s["viewmats"], s["Ks"], s["width"], s["height"], s["linear_velocity"],
+            s["angular_velocity"], s["rolling_shutter_time"], sh_degree=s["sh_degree"],
+            packed=False, render_mode="RGB+D", near_plane=s["near_plane"],
+            far_plane=s["far_plane"], eps2d=s["eps2d"], tile_size=s["tile_size"])
+        ((rc - target).abs().mean() + ra.mean()).backward()
+        for t in p.values():
+            t.grad = None
+
+    out["camera_fwd_bwd_ms"] = time_steps(cam_step, max(3, args.steps // 2), 2) * 1e3
+    del s, p, target
+    l = workloads.to_device(workloads.lidar_sweep(n=args.n), dev)
+    lnames = ("means", "quats", "scales", "opacities", "lidar_features")
+    q = {k: l[k].clone().requires_grad_(True) for k in lnames}
+
+    def lidar_step():
+        rf, ra, _, _ = lidar_rasterization(
+            q["means"], q["quats"], q["scales"], q["opacities"], q["lidar_features"],
+            l["velocities"], l["viewmats"], l["raster_pts"], l["tile_elevation_boundaries"],
+            l["linear_velocity"], l["angular_velocity"], l["rolling_shutter_time"],
+            min_azimuth=l["min_azimuth"], max_azimuth=l["max_azimuth"],
+            min_elevation=l["min_elevation"], max_elevation=l["max_elevation"],
+            n_elevation_channels=l["n_elevation_channels"],
+            azimuth_resolution=l["azimuth_resolution"], tile_width=l["tile_width"],
+            tile_height=l["tile_height"], near_plane=l["near_plane"], far_plane=l["far_plane"],
+            eps2d=l["eps2d"], channel_chunk=33)
+        (rf.abs().mean() + ra.mean()).backward()
+        for t in q.values():
+            t.grad = None
+
+    out["lidar_fwd_bwd_ms"] = time_steps(lidar_step, max(3, args.steps // 2), 2) * 1e3
+    return out
+
+
 def cpu_baseline_camera(args):
     """The CPU oracle on the same camera workload (same seed and distributions), OpenMP over
     all host cores given to the process; bounded by using fewer Gaussians when needed."""
@@ -245,6 +306,7 @@ def main():
     ap.add_argument("--cpu-n", type=int, default=1_000_000, help="Gaussians of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-lidar", action="store_true")
+    ap.add_argument("--no-bwd", action="store_true", help="skip the forward + backward timing")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (known HBM traffic, used "
                          "to scale FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -291,7 +353,8 @@ def main():
         "roofline": {
             "kernel": "rasterize_to_pixels_fwd_kernel<%d>" % cam["channels"],
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": MEASURED_TRAFFIC_BYTES["camera"] if args.n == 1_000_000 else None,
             "algorithmic_bytes": cam["alg_bytes"], "kernel_ms": cam["kernel_ms"],
         },
     }
@@ -306,9 +369,12 @@ def main():
             "n_isects": lid["n_isects"], "n_isects_consumed": lid["i_need"],
             "roofline": {"kernel": "rasterize_to_points_fwd_kernel<%d>" % lid["channels"],
                          "bound": "hbm", "achieved": l_ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": l_ach / HBM_PEAK_GBS, "traffic": None,
+                         "frac": l_ach / HBM_PEAK_GBS,
+                         "traffic": MEASURED_TRAFFIC_BYTES["lidar"] if args.n == 1_000_000 else None,
                          "algorithmic_bytes": lid["alg_bytes"], "kernel_ms": lid["kernel_ms"]},
         }
+    if not args.no_bwd:
+        out["config"].update({k: round(v, 4) for k, v in bench_backward(args).items()})
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_camera(args)
     print(json.dumps(out))
