@@ -170,6 +170,39 @@ int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N, const int64_t *ca
 int splatad_isect_offset_encode(int64_t n_isects, const int64_t *isect_ids, uint32_t C,
                                 uint32_t n_tiles, int32_t *offsets, splatad_stream_t stream);
 
+/* ---- lidar point binning -------------------------------------------- */
+
+/* map_points_to_lidar_tiles_tensor, rasterization.cu:658-770 (kernel :596-656; op declared
+ * in bindings.h next to isect_lidar_tiles).  One key (camera << 32 | tile) and one id per
+ * point; points2d is [C, N, 2] (camera_ids NULL, N given) or packed [total, 2] with
+ * camera_ids [total].  With sort != 0 the keys ascend and equal keys keep the point order;
+ * that mode needs a workspace of splatad_map_points_to_lidar_tiles_workspace_bytes(total,
+ * C, n_tiles_azim * n_tiles_elev) bytes and at most 36864 (sensor, tile) pairs. */
+size_t splatad_map_points_to_lidar_tiles_workspace_bytes(uint64_t total, uint32_t C,
+                                                         uint32_t n_tiles);
+int splatad_map_points_to_lidar_tiles(uint64_t total, uint32_t N, const int64_t *camera_ids,
+                                      const float *points2d, uint32_t C,
+                                      const float *elev_boundaries, float tile_azim_resolution,
+                                      float min_azim, uint32_t n_tiles_azim,
+                                      uint32_t n_tiles_elev, int sort, void *workspace,
+                                      int64_t *tile_ids, int32_t *flatten_ids,
+                                      splatad_stream_t stream);
+
+/* points_mapping_offset_encode_tensor, rasterization.cu:576-594 (kernel :531-574). */
+int splatad_points_mapping_offset_encode(int64_t n_points, const int64_t *point_ids, uint32_t C,
+                                         uint32_t n_tiles, int32_t *offsets,
+                                         splatad_stream_t stream);
+
+/* populate_image_from_points_tensor, rasterization.cu:807-833 (kernel :772-805).  points is
+ * [.., 5]; image [C, image_height, image_width, 5] is written completely (zeros where no
+ * point lands). */
+int splatad_populate_image_from_points(uint32_t C, int64_t n_points, const float *points,
+                                       uint32_t image_width, uint32_t image_height,
+                                       uint32_t tile_width, uint32_t tile_height,
+                                       uint32_t grid_w, uint32_t grid_h,
+                                       const int32_t *tile_offsets, const int32_t *flatten_ids,
+                                       float *image, splatad_stream_t stream);
+
 /* ---- rasterization ------------------------------------------------------ */
 
 /* rasterize_to_pixels_fwd_tensor, rasterization.cu:1520-2018 (kernel

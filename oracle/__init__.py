@@ -210,6 +210,65 @@ def isect_offset_encode(isect_ids, n_cameras, tile_width, tile_height):
 
 
 # ---------------------------------------------------------------------------
+# lidar point binning
+# ---------------------------------------------------------------------------
+def map_points_to_lidar_tiles(points2d, elev_boundaries, tile_azim_resolution, min_azim,
+                              n_cameras=None, camera_ids=None, sort=True):
+    """Restates ``map_points_to_lidar_tiles`` (rasterization.cu:596-770).
+
+    Returns (tile_ids int64[total], flatten_ids int32[total])."""
+    import math
+    lib = _lib("f32")
+    pts = _f32(points2d); eb = _f32(elev_boundaries)
+    if pts.ndim == 2:
+        total, N = pts.shape[0], 0
+        cam = np.ascontiguousarray(np.asarray(camera_ids, dtype=np.int64))
+    else:
+        C, N = pts.shape[:2]; total = C * N; cam = None
+    n_az = int(math.ceil(float(np.float32(360.0) / np.float32(tile_azim_resolution))))
+    n_el = int(eb.shape[0] - 1)
+    ids = np.zeros((total,), np.int64); flat = np.zeros((total,), np.int32)
+    lib.oracle_map_points_to_lidar_tiles.restype = None
+    lib.oracle_map_points_to_lidar_tiles(
+        ctypes.c_long(total), ctypes.c_long(N), _p(cam), _p(pts), _p(eb),
+        ctypes.c_float(tile_azim_resolution), ctypes.c_float(min_azim), ctypes.c_uint32(n_az),
+        ctypes.c_uint32(n_el), _p(ids), _p(flat))
+    if sort and total:
+        lib.oracle_sort_pairs.restype = None
+        lib.oracle_sort_pairs(ctypes.c_long(total), ctypes.c_int(64), _p(ids), _p(flat))
+    return ids, flat
+
+
+def points_mapping_offset_encode(point_ids, n_lidars, tile_width, tile_height):
+    """Restates ``points_mapping_offset_encode`` (rasterization.cu:531-594)."""
+    lib = _lib("f32")
+    ids = np.ascontiguousarray(np.asarray(point_ids, dtype=np.int64))
+    offsets = np.zeros((n_lidars, tile_height, tile_width), np.int32)
+    lib.oracle_points_mapping_offset_encode.restype = None
+    lib.oracle_points_mapping_offset_encode(
+        ctypes.c_long(ids.shape[0]), _p(ids), ctypes.c_uint32(n_lidars),
+        ctypes.c_uint32(tile_width * tile_height), _p(offsets))
+    return offsets
+
+
+def populate_image_from_points(points, image_width, image_height, tile_width, tile_height,
+                               tile_offsets, flatten_ids):
+    """Restates ``populate_image_from_points`` (rasterization.cu:772-833)."""
+    lib = _lib("f32")
+    pts = _f32(points)
+    offs = np.ascontiguousarray(np.asarray(tile_offsets, dtype=np.int32))
+    flat = np.ascontiguousarray(np.asarray(flatten_ids, dtype=np.int32))
+    C, gh, gw = offs.shape
+    image = np.zeros((C, image_height, image_width, 5), np.float32)
+    lib.oracle_populate_image_from_points.restype = None
+    lib.oracle_populate_image_from_points(
+        ctypes.c_uint32(C), ctypes.c_long(flat.shape[0]), _p(pts), ctypes.c_uint32(image_width),
+        ctypes.c_uint32(image_height), ctypes.c_uint32(tile_width), ctypes.c_uint32(tile_height),
+        ctypes.c_uint32(gw), ctypes.c_uint32(gh), _p(offs), _p(flat), _p(image))
+    return image
+
+
+# ---------------------------------------------------------------------------
 # rasterization
 # ---------------------------------------------------------------------------
 def rasterize_to_pixels_fwd(means2d, conics, colors, opacities, pix_vels, rolling_shutter_time,

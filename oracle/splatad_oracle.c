@@ -650,6 +650,85 @@ void oracle_isect_offset_encode(long n_isects, const int64_t *isect_ids, uint32_
     while (next < total) offsets[next++] = (int32_t)n_isects;
 }
 
+/* ------------------------------------------------------------------ */
+/* Lidar point binning (rasterization.cu:531-833)                       */
+/* ------------------------------------------------------------------ */
+
+/* map_points_to_lidar_tiles, rasterization.cu:596-656: one key (camera << 32 | tile) per
+ * point, no radius.  The azimuth column is the truncated quotient (wrapped with fmodf only
+ * outside [0, 360)), the elevation row the last boundary below the point, found by a linear
+ * scan over the first n_tiles_elev boundaries with strict <. */
+void oracle_map_points_to_lidar_tiles(long total, long N, const int64_t *camera_ids,
+                                      const float *points2d, const float *elev_boundaries,
+                                      float tile_azim_res, float min_azim, uint32_t n_tiles_azim,
+                                      uint32_t n_tiles_elev, int64_t *tile_ids,
+                                      int32_t *flatten_ids) {
+    for (long idx = 0; idx < total; ++idx) {
+        float tile_elev = points2d[idx * 2 + 1];
+        float azim = points2d[idx * 2] - min_azim;
+        float tile_azim;
+        if (azim >= 0.f && azim < 360.f)
+            tile_azim = azim / tile_azim_res;
+        else
+            tile_azim = fmodf(azim + 360.f, 360.f) / tile_azim_res;
+        int32_t x = (int32_t)tile_azim;
+        int32_t i = 0;
+        while (i < (int32_t)n_tiles_elev && elev_boundaries[i] < tile_elev) ++i;
+        int32_t y = i - 1 > 0 ? i - 1 : 0;
+        int64_t cid = camera_ids ? camera_ids[idx] : idx / N;
+        int64_t tile_id = (int64_t)y * n_tiles_azim + x;
+        tile_ids[idx] = (cid << 32) | tile_id;
+        flatten_ids[idx] = (int32_t)idx;
+    }
+}
+
+/* points_mapping_offset_encode, rasterization.cu:531-574: offsets[camera * n_tiles + tile] =
+ * index of the first sorted point whose (camera, tile) >= that entry; all zero when empty. */
+void oracle_points_mapping_offset_encode(long n_points, const int64_t *point_ids, uint32_t C,
+                                         uint32_t n_tiles, int32_t *offsets) {
+    long total = (long)C * n_tiles;
+    if (n_points == 0) {
+        for (long i = 0; i < total; ++i) offsets[i] = 0;
+        return;
+    }
+    long next = 0;
+    for (long idx = 0; idx < n_points; ++idx) {
+        int64_t cid = point_ids[idx] >> 32;
+        int64_t tid = point_ids[idx] & 0xFFFFFFFFll;
+        long id = (long)(cid * n_tiles + tid);
+        while (next <= id && next < total) offsets[next++] = (int32_t)idx;
+    }
+    while (next < total) offsets[next++] = (int32_t)n_points;
+}
+
+/* populate_image_from_points, rasterization.cu:772-833: the k-th point of a tile's list
+ * (k < tile_width * tile_height) lands on the tile's k-th pixel in row-major order, if that
+ * pixel is inside the image; everything else stays zero. */
+void oracle_populate_image_from_points(uint32_t C, long n_points, const float *points,
+                                       uint32_t image_width, uint32_t image_height,
+                                       uint32_t tile_width, uint32_t tile_height,
+                                       uint32_t grid_w, uint32_t grid_h,
+                                       const int32_t *tile_offsets, const int32_t *flatten_ids,
+                                       float *image) {
+    long n_tiles = (long)grid_w * grid_h;
+    for (uint32_t c = 0; c < C; ++c)
+        for (long t = 0; t < n_tiles; ++t) {
+            long start = tile_offsets[c * n_tiles + t];
+            long end = (c == C - 1 && t == n_tiles - 1) ? n_points : tile_offsets[c * n_tiles + t + 1];
+            long cap = start + (long)tile_width * tile_height;
+            if (end > cap) end = cap;
+            for (long k = start; k < end; ++k) {
+                long tr = k - start;
+                uint32_t i = (uint32_t)(t / grid_w) * tile_height + (uint32_t)(tr / tile_width);
+                uint32_t j = (uint32_t)(t % grid_w) * tile_width + (uint32_t)(tr % tile_width);
+                if (i >= image_height || j >= image_width) continue;
+                const float *src = points + (long)flatten_ids[k] * 5;
+                float *dst = image + (((long)c * image_height + i) * image_width + j) * 5;
+                for (int q = 0; q < 5; ++q) dst[q] = src[q];
+            }
+        }
+}
+
 #endif /* !ORACLE_F64 */
 
 /* ------------------------------------------------------------------ */

@@ -1,7 +1,8 @@
 """MI355X-native rendering hot path of SplatAD behind the gsplat operator API.
 
 Exports the operators and end-to-end functions of the reference's gsplat/__init__.py:3-24 that
-lie on the path projection -> tile intersection -> rasterization.
+lie on the path projection -> tile intersection -> rasterization, and the lidar point binning
+that prepares the points to render.
 """
 from .hip._wrapper import (
     fully_fused_lidar_projection,
@@ -9,6 +10,9 @@ from .hip._wrapper import (
     isect_lidar_tiles,
     isect_offset_encode,
     isect_tiles,
+    map_points_to_lidar_tiles,
+    points_mapping_offset_encode,
+    populate_image_from_points,
     rasterize_to_pixels,
     rasterize_to_points,
     spherical_harmonics,
@@ -28,4 +32,7 @@ __all__ = [
     "rasterize_to_pixels",
     "rasterize_to_points",
     "spherical_harmonics",
+    "map_points_to_lidar_tiles",
+    "points_mapping_offset_encode",
+    "populate_image_from_points",
 ]

@@ -35,7 +35,8 @@ def load_library():
         lib = ctypes.CDLL(LIB_PATH)
         lib.splatad_last_error.restype = ctypes.c_char_p
         lib.splatad_abi_version.restype = ctypes.c_int
-        for name in ("splatad_projection_packed_workspace_bytes", "splatad_isect_workspace_bytes"):
+        for name in ("splatad_projection_packed_workspace_bytes", "splatad_isect_workspace_bytes",
+                     "splatad_map_points_to_lidar_tiles_workspace_bytes"):
             getattr(lib, name).restype = ctypes.c_size_t
         _lib = lib
     return _lib
@@ -379,6 +380,66 @@ class _Ops:
                                                    _u32(tile_width * tile_height), _p(offsets),
                                                    _stream(dev)))
         return offsets
+
+    # ------------------------------------------------------------------ lidar point binning
+    def map_points_to_lidar_tiles(self, points2d, camera_ids, C, elev_boundaries,
+                                  tile_azim_resolution, min_azim, sort, double_buffer):
+        lib = load_library()
+        points2d = _in(points2d, "points2d"); eb = _in(elev_boundaries, "elev_boundaries")
+        camera_ids = _in(camera_ids, "camera_ids", torch.int64)
+        dev = points2d.device
+        packed = points2d.dim() == 2
+        if packed:
+            assert camera_ids is not None
+            total, N = points2d.shape[0], 0
+        else:
+            N = points2d.shape[1]
+            total = C * N
+            camera_ids = None
+        # rasterization.cu:689-690: float32 division, then ceil
+        res32 = torch.tensor(tile_azim_resolution, dtype=torch.float32)
+        n_az = int(math.ceil((torch.tensor(360.0, dtype=torch.float32) / res32).item()))
+        n_el = eb.shape[0] - 1
+        tile_ids = torch.empty((total,), dtype=torch.int64, device=dev)
+        flatten_ids = torch.empty((total,), dtype=torch.int32, device=dev)
+        if total:
+            with torch.cuda.device(dev):
+                ws = _workspace(lib.splatad_map_points_to_lidar_tiles_workspace_bytes(
+                    _u64(total), _u32(C), _u32(n_az * n_el)), dev) if sort else None
+                _check(lib.splatad_map_points_to_lidar_tiles(
+                    _u64(total), _u32(N), _p(camera_ids), _p(points2d), _u32(C), _p(eb),
+                    _f32(tile_azim_resolution), _f32(min_azim), _u32(n_az), _u32(n_el),
+                    _i32(bool(sort)), _p(ws), _p(tile_ids), _p(flatten_ids), _stream(dev)))
+        return tile_ids, flatten_ids
+
+    def points_mapping_offset_encode(self, point_ids, C, tile_width, tile_height):
+        lib = load_library()
+        point_ids = _in(point_ids, "point_ids", torch.int64)
+        dev = point_ids.device
+        offsets = torch.empty((C, tile_height, tile_width), dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_points_mapping_offset_encode(
+                _i64(point_ids.shape[0]), _p(point_ids), _u32(C), _u32(tile_width * tile_height),
+                _p(offsets), _stream(dev)))
+        return offsets
+
+    def populate_image_from_points(self, points, image_width, image_height, tile_width,
+                                   tile_height, tile_offsets, flatten_ids):
+        lib = load_library()
+        points = _in(points, "points")
+        tile_offsets = _in(tile_offsets, "tile_offsets", torch.int32)
+        flatten_ids = _in(flatten_ids, "flatten_ids", torch.int32)
+        if points.shape[-1] != 5:
+            raise ValueError("populate_image_from_points: points must have 5 values each")
+        dev = points.device
+        C, gh, gw = tile_offsets.shape
+        image = torch.empty((C, image_height, image_width, 5), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_populate_image_from_points(
+                _u32(C), _i64(flatten_ids.shape[0]), _p(points), _u32(image_width),
+                _u32(image_height), _u32(tile_width), _u32(tile_height), _u32(gw), _u32(gh),
+                _p(tile_offsets), _p(flatten_ids), _p(image), _stream(dev)))
+        return image
 
     # ------------------------------------------------------------------ rasterization
     def rasterize_to_pixels_fwd(self, means2d, conics, colors, opacities, pix_vels,

@@ -241,6 +241,56 @@ def isect_offset_encode(isect_ids: Tensor, n_cameras: int, tile_width: int, tile
     )
 
 
+@torch.no_grad()
+def map_points_to_lidar_tiles(
+    points2d: Tensor,  # [C, N, 2] or [nnz, 2]
+    elev_boundaries: Tensor,
+    tile_azim_resolution: float,
+    min_azim: float,
+    packed: bool = False,
+    n_cameras: Optional[int] = None,
+    camera_ids: Optional[Tensor] = None,
+    sort: bool = True,
+) -> Tuple[Tensor, Tensor]:
+    """Tile of every lidar point (no extent), `gsplat/cuda/_wrapper.py:698-757`.
+
+    Returns (tile ids int64 [total]: camera << 32 | tile, flatten ids int32 [total]); with
+    `sort` the ids ascend and the points of one tile keep their order."""
+    if packed:
+        nnz = points2d.size(0)
+        assert points2d.shape == (nnz, 2), points2d.size()
+        assert camera_ids is not None, "camera_ids is required if packed is True"
+        assert n_cameras is not None, "n_cameras is required if packed is True"
+        camera_ids = camera_ids.contiguous()
+        C = n_cameras
+    else:
+        C, N, _ = points2d.shape
+        assert points2d.shape == (C, N, 2), points2d.size()
+    return _make_lazy_hip_func("map_points_to_lidar_tiles")(
+        points2d.contiguous(), camera_ids, C, elev_boundaries.contiguous(), tile_azim_resolution,
+        min_azim, sort, True)
+
+
+@torch.no_grad()
+def points_mapping_offset_encode(point_ids: Tensor, n_lidars: int, tile_width: int,
+                                 tile_height: int) -> Tensor:
+    """Offsets [n_lidars, tile_height, tile_width] of sorted point tile ids,
+    `gsplat/cuda/_wrapper.py:759-776`."""
+    return _make_lazy_hip_func("points_mapping_offset_encode")(
+        point_ids.contiguous(), n_lidars, tile_width, tile_height)
+
+
+@torch.no_grad()
+def populate_image_from_points(points: Tensor, image_width: int, image_height: int,
+                               tile_width: int, tile_height: int, tile_offsets: Tensor,
+                               flatten_id: Tensor) -> Tensor:
+    """Image [C, image_height, image_width, 5] whose tiles are filled, in order, with the
+    points binned into them (`gsplat/cuda/_wrapper.py:778-809`)."""
+    return _make_lazy_hip_func("populate_image_from_points")(
+        points.contiguous(), image_width, image_height, tile_width, tile_height,
+        tile_offsets.contiguous(), flatten_id.contiguous())
+
+
 def rasterize_to_pixels(
     means2d: Tensor,  # [C, N, 2] or [nnz, 2]
     conics: Tensor,  # [C, N, 3] or [nnz, 3]
