@@ -272,6 +272,83 @@ int splatad_rasterize_to_points_bwd(uint32_t C, int64_t n_isects, uint32_t chann
                                     float *v_opacities, float *v_pix_vels,
                                     float *v_depth_compensations, splatad_stream_t stream);
 
+/* ---- unfused projection operators ------------------------------------ */
+/* Every operator streams [C, N, ...] (or [N, ...]) rows; gradients of a forward input are
+ * written completely unless stated otherwise. */
+
+/* quat_scale_to_covar_preci_{fwd,bwd}_tensor, projection.cu:161-228 (kernels :18-159).
+ * covars / precis are [N, 3, 3], or [N, 6] upper triangles with triu != 0; either may be
+ * NULL (not computed / no gradient given). */
+int splatad_quat_scale_to_covar_preci_fwd(uint32_t N, const float *quats, const float *scales,
+                                          int triu, float *covars, float *precis,
+                                          splatad_stream_t stream);
+int splatad_quat_scale_to_covar_preci_bwd(uint32_t N, const float *quats, const float *scales,
+                                          const float *v_covars, const float *v_precis, int triu,
+                                          float *v_quats, float *v_scales, splatad_stream_t stream);
+
+/* world_to_cam_{fwd,bwd}_tensor, projection.cu:386-599.  The backward outputs v_means [N, 3],
+ * v_covars [N, 3, 3], v_viewmats [C, 4, 4] are accumulated into (zero-fill them) and may each
+ * be NULL. */
+int splatad_world_to_cam_fwd(uint32_t C, uint32_t N, const float *means, const float *covars,
+                             const float *viewmats, float *means_c, float *covars_c,
+                             splatad_stream_t stream);
+int splatad_world_to_cam_bwd(uint32_t C, uint32_t N, const float *means, const float *covars,
+                             const float *viewmats, const float *v_means_c,
+                             const float *v_covars_c, float *v_means, float *v_covars,
+                             float *v_viewmats, splatad_stream_t stream);
+
+/* persp_proj_{fwd,bwd}_tensor, projection.cu:230-384: means [C, N, 3], covars [C, N, 3, 3] ->
+ * means2d [C, N, 2], covars2d [C, N, 2, 2]. */
+int splatad_persp_proj_fwd(uint32_t C, uint32_t N, const float *means, const float *covars,
+                           const float *Ks, uint32_t width, uint32_t height, float *means2d,
+                           float *covars2d, splatad_stream_t stream);
+int splatad_persp_proj_bwd(uint32_t C, uint32_t N, const float *means, const float *covars,
+                           const float *Ks, uint32_t width, uint32_t height,
+                           const float *v_means2d, const float *v_covars2d, float *v_means,
+                           float *v_covars, splatad_stream_t stream);
+
+/* compute_pix_velocity_{fwd,bwd}_tensor, projection.cu:2118-2266: p_view and velocities are
+ * [C, N, 3] in the sensor frame; vel is [C, N, 2]. */
+int splatad_compute_pix_velocity_fwd(uint32_t C, uint32_t N, const float *p_view,
+                                     const float *lin_vel, const float *ang_vel,
+                                     const float *velocities, const float *Ks, uint32_t width,
+                                     uint32_t height, float *vel, splatad_stream_t stream);
+int splatad_compute_pix_velocity_bwd(uint32_t C, uint32_t N, const float *p_view,
+                                     const float *lin_vel, const float *ang_vel,
+                                     const float *velocities, const float *Ks, uint32_t width,
+                                     uint32_t height, const float *v_vel, float *v_p_view,
+                                     float *v_velocities, splatad_stream_t stream);
+
+/* lidar_proj_{fwd,bwd}_tensor, projection.cu:1841-1988: means2d (azimuth, elevation in degrees)
+ * [C, N, 2], covars2d [C, N, 2, 2], depth_compensations [C, N, 2]. */
+int splatad_lidar_proj_fwd(uint32_t C, uint32_t N, const float *means, const float *covars,
+                           float eps2d, float *means2d, float *covars2d,
+                           float *depth_compensations, splatad_stream_t stream);
+int splatad_lidar_proj_bwd(uint32_t C, uint32_t N, const float *means, const float *covars,
+                           float eps2d, const float *v_means2d, const float *v_covars2d,
+                           const float *v_depth_compensations, float *v_means, float *v_covars,
+                           splatad_stream_t stream);
+
+/* compute_lidar_velocity_{fwd,bwd}_tensor, projection.cu:1990-2116: vel is [C, N, 3]
+ * (azimuth rate, elevation rate in degrees, range rate). */
+int splatad_compute_lidar_velocity_fwd(uint32_t C, uint32_t N, const float *p_view,
+                                       const float *lin_vel, const float *ang_vel,
+                                       const float *velocities, float *vel,
+                                       splatad_stream_t stream);
+int splatad_compute_lidar_velocity_bwd(uint32_t C, uint32_t N, const float *p_view,
+                                       const float *lin_vel, const float *ang_vel,
+                                       const float *velocities, const float *v_vel,
+                                       float *v_p_view, float *v_velocities,
+                                       splatad_stream_t stream);
+
+/* ---- densification helper --------------------------------------------- */
+
+/* compute_relocation_tensor, gsplat/cuda/csrc/relocation.cu:32-56 (kernel :4-30; op
+ * declared in bindings.h).  ratios are int32 in [1, n_max]; binoms is [n_max, n_max]. */
+int splatad_compute_relocation(uint32_t N, const float *opacities, const float *scales,
+                               const int32_t *ratios, const float *binoms, int32_t n_max,
+                               float *new_opacities, float *new_scales, splatad_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

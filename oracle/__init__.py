@@ -268,6 +268,19 @@ def populate_image_from_points(points, image_width, image_height, tile_width, ti
     return image
 
 
+def compute_relocation(opacities, scales, ratios, binoms):
+    """Restates ``compute_relocation`` (gsplat/relocation.py:10-49, relocation.cu:4-30)."""
+    lib = _lib("f32")
+    o = _f32(opacities); sc = _f32(scales); b = _f32(binoms)
+    n_max = b.shape[0]
+    r = np.ascontiguousarray(np.clip(np.asarray(ratios), 1, n_max).astype(np.int32))
+    new_o = np.zeros_like(o); new_s = np.zeros_like(sc)
+    lib.oracle_compute_relocation.restype = None
+    lib.oracle_compute_relocation(ctypes.c_long(o.shape[0]), _p(o), _p(sc), _p(r), _p(b),
+                                  ctypes.c_int(n_max), _p(new_o), _p(new_s))
+    return new_o, new_s
+
+
 # ---------------------------------------------------------------------------
 # rasterization
 # ---------------------------------------------------------------------------

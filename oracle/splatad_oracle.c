@@ -729,6 +729,27 @@ void oracle_populate_image_from_points(uint32_t C, long n_points, const float *p
         }
 }
 
+/* compute_relocation, gsplat/cuda/csrc/relocation.cu:4-30: powers and square root in double
+ * (pow / sqrt on mixed arguments promote), sum in float. */
+void oracle_compute_relocation(long N, const float *opacities, const float *scales,
+                               const int32_t *ratios, const float *binoms, int n_max,
+                               float *new_opacities, float *new_scales) {
+    for (long idx = 0; idx < N; ++idx) {
+        int n_idx = ratios[idx];
+        float denom_sum = 0.0f;
+        new_opacities[idx] = 1.0f - powf(1.0f - opacities[idx], 1.0f / n_idx);
+        for (int i = 1; i <= n_idx; ++i)
+            for (int k = 0; k <= i - 1; ++k) {
+                float bin_coeff = binoms[(long)(i - 1) * n_max + k];
+                float term = (float)((pow(-1.0, k) / sqrt((double)(float)(k + 1))) *
+                                     pow((double)new_opacities[idx], k + 1));
+                denom_sum += bin_coeff * term;
+            }
+        float coeff = opacities[idx] / denom_sum;
+        for (int q = 0; q < 3; ++q) new_scales[idx * 3 + q] = coeff * scales[idx * 3 + q];
+    }
+}
+
 #endif /* !ORACLE_F64 */
 
 /* ------------------------------------------------------------------ */

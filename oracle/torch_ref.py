@@ -263,3 +263,100 @@ def rasterize_to_points(means2d, conics, colors, opacities, pix_vels, depth_comp
         asum[c, i0:i1, j0:j1, 0] = s.reshape(i1 - i0, j1 - j0)
         med[c, i0:i1, j0:j1, 0] = m.detach().reshape(i1 - i0, j1 - j0)
     return out, alph, (asum if compute_alpha_sum else None), med
+
+
+# ---------------------------------------------------------------------------
+# the unfused projection operators (gsplat/cuda/_torch_impl.py:10-200 of the reference
+# holds the torch restatement its own tests compare against)
+# ---------------------------------------------------------------------------
+def _quat_to_rotmat(quats):
+    q = quats / quats.norm(dim=-1, keepdim=True)
+    w, x, y, z = q.unbind(-1)
+    return torch.stack([
+        1 - 2 * (y * y + z * z), 2 * (x * y - w * z), 2 * (x * z + w * y),
+        2 * (x * y + w * z), 1 - 2 * (x * x + z * z), 2 * (y * z - w * x),
+        2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)], dim=-1).reshape(-1, 3, 3)
+
+
+def quat_scale_to_covar_preci(quats, scales, compute_covar=True, compute_preci=True, triu=False):
+    """covar = R S S R^T, preci = R S^-1 S^-1 R^T; `triu` returns (xx, xy, xz, yy, yz, zz)."""
+    R = _quat_to_rotmat(quats)
+    covars = precis = None
+    if compute_covar:
+        M = R * scales[:, None, :]
+        covars = M @ M.transpose(-1, -2)
+    if compute_preci:
+        P = R * (1.0 / scales[:, None, :])
+        precis = P @ P.transpose(-1, -2)
+    if triu:
+        pick = lambda m: None if m is None else torch.stack(
+            [m[:, 0, 0], m[:, 0, 1], m[:, 0, 2], m[:, 1, 1], m[:, 1, 2], m[:, 2, 2]], dim=-1)
+        covars, precis = pick(covars), pick(precis)
+    return covars, precis
+
+
+def world_to_cam(means, covars, viewmats):
+    R = viewmats[:, :3, :3]
+    t = viewmats[:, :3, 3]
+    means_c = torch.einsum("cij,nj->cni", R, means) + t[:, None, :]
+    covars_c = torch.einsum("cij,njk,clk->cnil", R, covars, R)
+    return means_c, covars_c
+
+
+def _persp_jacobian(means, Ks, width, height):
+    x, y, z = means.unbind(-1)
+    fx, fy = Ks[:, 0, 0, None], Ks[:, 1, 1, None]
+    cx, cy = Ks[:, 0, 2, None], Ks[:, 1, 2, None]
+    tan_fovx, tan_fovy = 0.5 * width / fx, 0.5 * height / fy
+    lim_x_pos = (width - cx) / fx + 0.3 * tan_fovx
+    lim_x_neg = cx / fx + 0.3 * tan_fovx
+    lim_y_pos = (height - cy) / fy + 0.3 * tan_fovy
+    lim_y_neg = cy / fy + 0.3 * tan_fovy
+    tx = z * torch.minimum(lim_x_pos, torch.maximum(-lim_x_neg, x / z))
+    ty = z * torch.minimum(lim_y_pos, torch.maximum(-lim_y_neg, y / z))
+    O = torch.zeros_like(z)
+    J = torch.stack([fx / z, O, -fx * tx / z ** 2, O, fy / z, -fy * ty / z ** 2], dim=-1).reshape(*z.shape, 2, 3)
+    means2d = torch.stack([fx * x / z + cx, fy * y / z + cy], dim=-1)
+    return J, means2d
+
+
+def persp_proj(means, covars, Ks, width, height):
+    J, means2d = _persp_jacobian(means, Ks, width, height)
+    return means2d, J @ covars @ J.transpose(-1, -2)
+
+
+def compute_pix_velocity(p_view, lin_vel, ang_vel, velocities, Ks, width, height):
+    J, _ = _persp_jacobian(p_view, Ks, width, height)
+    tv = lin_vel[:, None, :] + torch.cross(ang_vel[:, None, :].expand_as(p_view), p_view, dim=-1) - velocities
+    return -(J @ tv[..., None])[..., 0]
+
+
+def _lidar_jacobian(means):
+    x, y, z = means.unbind(-1)
+    rho2 = x * x + y * y
+    r2 = rho2 + z * z
+    r, rho = torch.sqrt(r2), torch.sqrt(rho2)
+    O = torch.zeros_like(z)
+    J = torch.stack([
+        -y / rho2 * RAD2DEG, x / rho2 * RAD2DEG, O,
+        -x * z / (r2 * rho) * RAD2DEG, -y * z / (r2 * rho) * RAD2DEG, rho / r2 * RAD2DEG,
+        x / r, y / r, z / r], dim=-1).reshape(*z.shape, 3, 3)
+    means2d = torch.stack([torch.atan2(y, x) * RAD2DEG, torch.asin(z / r) * RAD2DEG], dim=-1)
+    return J, means2d
+
+
+def lidar_proj(means, covars, eps2d):
+    J, means2d = _lidar_jacobian(means)
+    cs = J @ covars @ J.transpose(-1, -2)
+    a1, a2 = cs[..., 0, 0] + eps2d, cs[..., 0, 1]
+    b1, b2 = cs[..., 1, 0], cs[..., 1, 1] + eps2d
+    c1, c2 = cs[..., 2, 0], cs[..., 2, 1]
+    D = a1 * b2 - a2 * b1
+    dcomp = torch.stack([(b1 * c2 - b2 * c1) / D, (a2 * c1 - a1 * c2) / D], dim=-1)
+    return means2d, cs[..., :2, :2], dcomp
+
+
+def compute_lidar_velocity(p_view, lin_vel, ang_vel, velocities):
+    J, _ = _lidar_jacobian(p_view)
+    tv = lin_vel[:, None, :] + torch.cross(ang_vel[:, None, :].expand_as(p_view), p_view, dim=-1) - velocities
+    return -(J @ tv[..., None])[..., 0]

@@ -5,6 +5,12 @@ lie on the path projection -> tile intersection -> rasterization, and the lidar 
 that prepares the points to render.
 """
 from .hip._wrapper import (
+    compute_lidar_velocity,
+    compute_pix_velocity,
+    lidar_proj,
+    persp_proj,
+    quat_scale_to_covar_preci,
+    world_to_cam,
     fully_fused_lidar_projection,
     fully_fused_projection,
     isect_lidar_tiles,
@@ -32,6 +38,12 @@ __all__ = [
     "rasterize_to_pixels",
     "rasterize_to_points",
     "spherical_harmonics",
+    "quat_scale_to_covar_preci",
+    "world_to_cam",
+    "persp_proj",
+    "lidar_proj",
+    "compute_pix_velocity",
+    "compute_lidar_velocity",
     "map_points_to_lidar_tiles",
     "points_mapping_offset_encode",
     "populate_image_from_points",

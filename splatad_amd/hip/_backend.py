@@ -441,6 +441,167 @@ class _Ops:
                 _p(tile_offsets), _p(flatten_ids), _p(image), _stream(dev)))
         return image
 
+    # ------------------------------------------------------------------ unfused projection ops
+    def quat_scale_to_covar_preci_fwd(self, quats, scales, compute_covar, compute_preci, triu):
+        lib = load_library()
+        quats = _in(quats, "quats"); scales = _in(scales, "scales")
+        N, dev = quats.shape[0], quats.device
+        shape = (N, 6) if triu else (N, 3, 3)
+        covars = torch.empty(shape, dtype=torch.float32, device=dev) if compute_covar else None
+        precis = torch.empty(shape, dtype=torch.float32, device=dev) if compute_preci else None
+        with torch.cuda.device(dev):
+            _check(lib.splatad_quat_scale_to_covar_preci_fwd(
+                _u32(N), _p(quats), _p(scales), _i32(bool(triu)), _p(covars), _p(precis), _stream(dev)))
+        return covars, precis
+
+    def quat_scale_to_covar_preci_bwd(self, quats, scales, v_covars, v_precis, triu):
+        lib = load_library()
+        quats = _in(quats, "quats"); scales = _in(scales, "scales")
+        v_covars = _in(v_covars, "v_covars"); v_precis = _in(v_precis, "v_precis")
+        dev = quats.device
+        v_quats = torch.empty_like(quats); v_scales = torch.empty_like(scales)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_quat_scale_to_covar_preci_bwd(
+                _u32(quats.shape[0]), _p(quats), _p(scales), _p(v_covars), _p(v_precis),
+                _i32(bool(triu)), _p(v_quats), _p(v_scales), _stream(dev)))
+        return v_quats, v_scales
+
+    def world_to_cam_fwd(self, means, covars, viewmats):
+        lib = load_library()
+        means = _in(means, "means"); covars = _in(covars, "covars"); viewmats = _in(viewmats, "viewmats")
+        C, N, dev = viewmats.shape[0], means.shape[0], means.device
+        means_c = torch.empty((C, N, 3), dtype=torch.float32, device=dev)
+        covars_c = torch.empty((C, N, 3, 3), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_world_to_cam_fwd(_u32(C), _u32(N), _p(means), _p(covars), _p(viewmats),
+                                                _p(means_c), _p(covars_c), _stream(dev)))
+        return means_c, covars_c
+
+    def world_to_cam_bwd(self, means, covars, viewmats, v_means_c, v_covars_c, means_grad,
+                         covars_grad, viewmats_grad):
+        lib = load_library()
+        means = _in(means, "means"); covars = _in(covars, "covars"); viewmats = _in(viewmats, "viewmats")
+        v_means_c = _in(v_means_c, "v_means_c"); v_covars_c = _in(v_covars_c, "v_covars_c")
+        C, N, dev = viewmats.shape[0], means.shape[0], means.device
+        v_means = torch.zeros_like(means) if means_grad else None
+        v_covars = torch.zeros_like(covars) if covars_grad else None
+        v_viewmats = torch.zeros_like(viewmats) if viewmats_grad else None
+        with torch.cuda.device(dev):
+            _check(lib.splatad_world_to_cam_bwd(
+                _u32(C), _u32(N), _p(means), _p(covars), _p(viewmats), _p(v_means_c), _p(v_covars_c),
+                _p(v_means), _p(v_covars), _p(v_viewmats), _stream(dev)))
+        return v_means, v_covars, v_viewmats
+
+    def persp_proj_fwd(self, means, covars, Ks, width, height):
+        lib = load_library()
+        means = _in(means, "means"); covars = _in(covars, "covars"); Ks = _in(Ks, "Ks")
+        C, N, dev = means.shape[0], means.shape[1], means.device
+        means2d = torch.empty((C, N, 2), dtype=torch.float32, device=dev)
+        covars2d = torch.empty((C, N, 2, 2), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_persp_proj_fwd(_u32(C), _u32(N), _p(means), _p(covars), _p(Ks), _u32(width),
+                                              _u32(height), _p(means2d), _p(covars2d), _stream(dev)))
+        return means2d, covars2d
+
+    def persp_proj_bwd(self, means, covars, Ks, width, height, v_means2d, v_covars2d):
+        lib = load_library()
+        means = _in(means, "means"); covars = _in(covars, "covars"); Ks = _in(Ks, "Ks")
+        v_means2d = _in(v_means2d, "v_means2d"); v_covars2d = _in(v_covars2d, "v_covars2d")
+        C, N, dev = means.shape[0], means.shape[1], means.device
+        v_means = torch.empty_like(means); v_covars = torch.empty_like(covars)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_persp_proj_bwd(
+                _u32(C), _u32(N), _p(means), _p(covars), _p(Ks), _u32(width), _u32(height),
+                _p(v_means2d), _p(v_covars2d), _p(v_means), _p(v_covars), _stream(dev)))
+        return v_means, v_covars
+
+    def compute_pix_velocity_fwd(self, p_view, lin_vel, ang_vel, velocities, Ks, width, height):
+        lib = load_library()
+        p_view = _in(p_view, "p_view"); lin_vel = _in(lin_vel, "lin_vel"); ang_vel = _in(ang_vel, "ang_vel")
+        velocities = _in(velocities, "velocities"); Ks = _in(Ks, "Ks")
+        C, N, dev = p_view.shape[0], p_view.shape[1], p_view.device
+        vel = torch.empty((C, N, 2), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_compute_pix_velocity_fwd(
+                _u32(C), _u32(N), _p(p_view), _p(lin_vel), _p(ang_vel), _p(velocities), _p(Ks),
+                _u32(width), _u32(height), _p(vel), _stream(dev)))
+        return vel
+
+    def compute_pix_velocity_bwd(self, p_view, lin_vel, ang_vel, velocities, Ks, width, height, v_vel):
+        lib = load_library()
+        p_view = _in(p_view, "p_view"); lin_vel = _in(lin_vel, "lin_vel"); ang_vel = _in(ang_vel, "ang_vel")
+        velocities = _in(velocities, "velocities"); Ks = _in(Ks, "Ks"); v_vel = _in(v_vel, "v_vel")
+        C, N, dev = p_view.shape[0], p_view.shape[1], p_view.device
+        v_p_view = torch.empty_like(p_view); v_velocities = torch.empty_like(velocities)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_compute_pix_velocity_bwd(
+                _u32(C), _u32(N), _p(p_view), _p(lin_vel), _p(ang_vel), _p(velocities), _p(Ks),
+                _u32(width), _u32(height), _p(v_vel), _p(v_p_view), _p(v_velocities), _stream(dev)))
+        return v_p_view, v_velocities
+
+    def lidar_proj_fwd(self, means, covars, eps2d):
+        lib = load_library()
+        means = _in(means, "means"); covars = _in(covars, "covars")
+        C, N, dev = means.shape[0], means.shape[1], means.device
+        means2d = torch.empty((C, N, 2), dtype=torch.float32, device=dev)
+        covars2d = torch.empty((C, N, 2, 2), dtype=torch.float32, device=dev)
+        depth_comps = torch.empty((C, N, 2), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_lidar_proj_fwd(_u32(C), _u32(N), _p(means), _p(covars), _f32(eps2d),
+                                              _p(means2d), _p(covars2d), _p(depth_comps), _stream(dev)))
+        return means2d, covars2d, depth_comps
+
+    def lidar_proj_bwd(self, means, covars, eps2d, v_means2d, v_covars2d, v_depth_compensations):
+        lib = load_library()
+        means = _in(means, "means"); covars = _in(covars, "covars")
+        v_means2d = _in(v_means2d, "v_means2d"); v_covars2d = _in(v_covars2d, "v_covars2d")
+        v_dc = _in(v_depth_compensations, "v_depth_compensations")
+        C, N, dev = means.shape[0], means.shape[1], means.device
+        v_means = torch.empty_like(means); v_covars = torch.empty_like(covars)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_lidar_proj_bwd(
+                _u32(C), _u32(N), _p(means), _p(covars), _f32(eps2d), _p(v_means2d), _p(v_covars2d),
+                _p(v_dc), _p(v_means), _p(v_covars), _stream(dev)))
+        return v_means, v_covars
+
+    def compute_lidar_velocity_fwd(self, p_view, lin_vel, ang_vel, velocities):
+        lib = load_library()
+        p_view = _in(p_view, "p_view"); lin_vel = _in(lin_vel, "lin_vel"); ang_vel = _in(ang_vel, "ang_vel")
+        velocities = _in(velocities, "velocities")
+        C, N, dev = p_view.shape[0], p_view.shape[1], p_view.device
+        vel = torch.empty((C, N, 3), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_compute_lidar_velocity_fwd(
+                _u32(C), _u32(N), _p(p_view), _p(lin_vel), _p(ang_vel), _p(velocities), _p(vel),
+                _stream(dev)))
+        return vel
+
+    def compute_lidar_velocity_bwd(self, p_view, lin_vel, ang_vel, velocities, v_vel):
+        lib = load_library()
+        p_view = _in(p_view, "p_view"); lin_vel = _in(lin_vel, "lin_vel"); ang_vel = _in(ang_vel, "ang_vel")
+        velocities = _in(velocities, "velocities"); v_vel = _in(v_vel, "v_vel")
+        C, N, dev = p_view.shape[0], p_view.shape[1], p_view.device
+        v_p_view = torch.empty_like(p_view); v_velocities = torch.empty_like(velocities)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_compute_lidar_velocity_bwd(
+                _u32(C), _u32(N), _p(p_view), _p(lin_vel), _p(ang_vel), _p(velocities), _p(v_vel),
+                _p(v_p_view), _p(v_velocities), _stream(dev)))
+        return v_p_view, v_velocities
+
+    # ------------------------------------------------------------------ densification helper
+    def compute_relocation(self, opacities, scales, ratios, binoms, n_max):
+        lib = load_library()
+        opacities = _in(opacities, "opacities"); scales = _in(scales, "scales")
+        ratios = _in(ratios, "ratios", torch.int32); binoms = _in(binoms, "binoms")
+        dev = opacities.device
+        new_opacities = torch.empty_like(opacities)
+        new_scales = torch.empty_like(scales)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_compute_relocation(
+                _u32(opacities.shape[0]), _p(opacities), _p(scales), _p(ratios), _p(binoms),
+                _i32(n_max), _p(new_opacities), _p(new_scales), _stream(dev)))
+        return new_opacities, new_scales
+
     # ------------------------------------------------------------------ rasterization
     def rasterize_to_pixels_fwd(self, means2d, conics, colors, opacities, pix_vels,
                                 rolling_shutter_time, backgrounds, image_width, image_height,

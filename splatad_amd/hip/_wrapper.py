@@ -631,6 +631,185 @@ class _RasterizeToPoints(torch.autograd.Function):
                 v_backgrounds) + (None,) * 11
 
 
+# ---------------------------------------------------------------------------
+# the unfused projection operators (gsplat/cuda/_wrapper.py:46-228, 1283-1493)
+# ---------------------------------------------------------------------------
+def quat_scale_to_covar_preci(
+    quats: Tensor,  # [N, 4]
+    scales: Tensor,  # [N, 3]
+    compute_covar: bool = True,
+    compute_preci: bool = True,
+    triu: bool = False,
+) -> Tuple[Optional[Tensor], Optional[Tensor]]:
+    """Covariances R S S R^T and precisions R S^-1 S^-1 R^T of (unnormalised) quaternions and
+    scales, [N, 3, 3] each or upper triangles [N, 6] with `triu`; a matrix that is not asked
+    for is None."""
+    assert quats.dim() == 2 and quats.size(1) == 4, quats.size()
+    assert scales.dim() == 2 and scales.size(1) == 3, scales.size()
+    covars, precis = _QuatScaleToCovarPreci.apply(
+        quats.contiguous(), scales.contiguous(), compute_covar, compute_preci, triu)
+    return covars if compute_covar else None, precis if compute_preci else None
+
+
+def persp_proj(means: Tensor, covars: Tensor, Ks: Tensor, width: int, height: int) -> Tuple[Tensor, Tensor]:
+    """Pinhole projection of sensor-frame means [C, N, 3] and covariances [C, N, 3, 3]:
+    means2d [C, N, 2] and covars2d [C, N, 2, 2]."""
+    C, N, _ = means.shape
+    assert means.shape == (C, N, 3), means.size()
+    assert covars.shape == (C, N, 3, 3), covars.size()
+    assert Ks.shape == (C, 3, 3), Ks.size()
+    return _PerspProj.apply(means.contiguous(), covars.contiguous(), Ks.contiguous(), width, height)
+
+
+def compute_pix_velocity(p_view: Tensor, lin_vel: Tensor, ang_vel: Tensor, velocities: Tensor,
+                         Ks: Tensor, width: int, height: int) -> Tensor:
+    """Image-space velocity [C, N, 2] of sensor-frame points [C, N, 3] moving with
+    `velocities` [C, N, 3] while the camera moves with `lin_vel`, `ang_vel` [C, 3]."""
+    C, N, _ = p_view.shape
+    assert p_view.shape == (C, N, 3), p_view.size()
+    assert lin_vel.shape == (C, 3), lin_vel.size()
+    assert ang_vel.shape == (C, 3), ang_vel.size()
+    assert velocities.shape == (C, N, 3), velocities.size()
+    assert Ks.shape == (C, 3, 3), Ks.size()
+    return _ComputePixVelocity.apply(p_view.contiguous(), lin_vel.contiguous(), ang_vel.contiguous(),
+                                     velocities.contiguous(), Ks.contiguous(), width, height)
+
+
+def world_to_cam(means: Tensor, covars: Tensor, viewmats: Tensor) -> Tuple[Tensor, Tensor]:
+    """World-frame means [N, 3] and covariances [N, 3, 3] in the frames of C sensors:
+    [C, N, 3] and [C, N, 3, 3]."""
+    C = viewmats.size(0)
+    N = means.size(0)
+    assert means.size() == (N, 3), means.size()
+    assert covars.size() == (N, 3, 3), covars.size()
+    assert viewmats.size() == (C, 4, 4), viewmats.size()
+    return _WorldToCam.apply(means.contiguous(), covars.contiguous(), viewmats.contiguous())
+
+
+def lidar_proj(means: Tensor, covars: Tensor, eps2d: float) -> Tuple[Tensor, Tensor, Tensor]:
+    """Spherical projection of sensor-frame Gaussians: means2d (azimuth, elevation above the
+    xy-plane, degrees) [C, N, 2], covars2d [C, N, 2, 2], depth compensations [C, N, 2]."""
+    C, N, _ = means.shape
+    assert means.shape == (C, N, 3), means.size()
+    assert covars.shape == (C, N, 3, 3), covars.size()
+    return _LidarProj.apply(means.contiguous(), covars.contiguous(), eps2d)
+
+
+def compute_lidar_velocity(p_view: Tensor, lin_vel: Tensor, ang_vel: Tensor, velocities: Tensor) -> Tensor:
+    """Spherical velocity (azimuth rate, elevation rate, range rate) [C, N, 3] of sensor-frame
+    points under sensor motion."""
+    C, N, _ = p_view.shape
+    assert p_view.shape == (C, N, 3), p_view.size()
+    assert lin_vel.shape == (C, 3), lin_vel.size()
+    assert ang_vel.shape == (C, 3), ang_vel.size()
+    assert velocities.shape == (C, N, 3), velocities.size()
+    return _ComputeLidarVelocity.apply(p_view.contiguous(), lin_vel.contiguous(), ang_vel.contiguous(),
+                                       velocities.contiguous())
+
+
+class _QuatScaleToCovarPreci(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, quats, scales, compute_covar=True, compute_preci=True, triu=False):
+        covars, precis = _make_lazy_hip_func("quat_scale_to_covar_preci_fwd")(
+            quats, scales, compute_covar, compute_preci, triu)
+        ctx.save_for_backward(quats, scales)
+        ctx.compute_covar, ctx.compute_preci, ctx.triu = compute_covar, compute_preci, triu
+        return covars, precis
+
+    @staticmethod
+    def backward(ctx, v_covars, v_precis):
+        quats, scales = ctx.saved_tensors
+        if ctx.compute_covar and v_covars is not None and v_covars.is_sparse:
+            v_covars = v_covars.to_dense()
+        if ctx.compute_preci and v_precis is not None and v_precis.is_sparse:
+            v_precis = v_precis.to_dense()
+        v_quats, v_scales = _make_lazy_hip_func("quat_scale_to_covar_preci_bwd")(
+            quats, scales,
+            v_covars.contiguous() if ctx.compute_covar and v_covars is not None else None,
+            v_precis.contiguous() if ctx.compute_preci and v_precis is not None else None, ctx.triu)
+        return v_quats, v_scales, None, None, None
+
+
+class _PerspProj(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, means, covars, Ks, width, height):
+        means2d, covars2d = _make_lazy_hip_func("persp_proj_fwd")(means, covars, Ks, width, height)
+        ctx.save_for_backward(means, covars, Ks)
+        ctx.width, ctx.height = width, height
+        return means2d, covars2d
+
+    @staticmethod
+    def backward(ctx, v_means2d, v_covars2d):
+        means, covars, Ks = ctx.saved_tensors
+        v_means, v_covars = _make_lazy_hip_func("persp_proj_bwd")(
+            means, covars, Ks, ctx.width, ctx.height, v_means2d.contiguous(), v_covars2d.contiguous())
+        return v_means, v_covars, None, None, None
+
+
+class _ComputePixVelocity(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, p_view, lin_vel, ang_vel, velocities, Ks, width, height):
+        vel = _make_lazy_hip_func("compute_pix_velocity_fwd")(p_view, lin_vel, ang_vel, velocities, Ks,
+                                                              width, height)
+        ctx.save_for_backward(p_view, lin_vel, ang_vel, velocities, Ks)
+        ctx.width, ctx.height = width, height
+        return vel
+
+    @staticmethod
+    def backward(ctx, v_vel):
+        p_view, lin_vel, ang_vel, velocities, Ks = ctx.saved_tensors
+        v_p_view, v_velocities = _make_lazy_hip_func("compute_pix_velocity_bwd")(
+            p_view, lin_vel, ang_vel, velocities, Ks, ctx.width, ctx.height, v_vel.contiguous())
+        return v_p_view, None, None, v_velocities, None, None, None
+
+
+class _WorldToCam(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, means, covars, viewmats):
+        means_c, covars_c = _make_lazy_hip_func("world_to_cam_fwd")(means, covars, viewmats)
+        ctx.save_for_backward(means, covars, viewmats)
+        return means_c, covars_c
+
+    @staticmethod
+    def backward(ctx, v_means_c, v_covars_c):
+        means, covars, viewmats = ctx.saved_tensors
+        return _make_lazy_hip_func("world_to_cam_bwd")(
+            means, covars, viewmats, v_means_c.contiguous(), v_covars_c.contiguous(),
+            ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2])
+
+
+class _LidarProj(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, means, covars, eps2d):
+        means2d, covars2d, depth_compensations = _make_lazy_hip_func("lidar_proj_fwd")(means, covars, eps2d)
+        ctx.save_for_backward(means, covars)
+        ctx.eps2d = eps2d
+        return means2d, covars2d, depth_compensations
+
+    @staticmethod
+    def backward(ctx, v_means2d, v_covars2d, v_depth_compensations):
+        means, covars = ctx.saved_tensors
+        v_means, v_covars = _make_lazy_hip_func("lidar_proj_bwd")(
+            means, covars, ctx.eps2d, v_means2d.contiguous(), v_covars2d.contiguous(),
+            v_depth_compensations.contiguous())
+        return v_means, v_covars, None
+
+
+class _ComputeLidarVelocity(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, p_view, lin_vel, ang_vel, velocities):
+        vel = _make_lazy_hip_func("compute_lidar_velocity_fwd")(p_view, lin_vel, ang_vel, velocities)
+        ctx.save_for_backward(p_view, lin_vel, ang_vel, velocities)
+        return vel
+
+    @staticmethod
+    def backward(ctx, v_vel):
+        p_view, lin_vel, ang_vel, velocities = ctx.saved_tensors
+        v_p_view, v_velocities = _make_lazy_hip_func("compute_lidar_velocity_bwd")(
+            p_view, lin_vel, ang_vel, velocities, v_vel.contiguous())
+        return v_p_view, None, None, v_velocities
+
+
 class _SphericalHarmonics(torch.autograd.Function):
     @staticmethod
     def forward(ctx, sh_degree, dirs, coeffs, masks):
