@@ -341,6 +341,62 @@ int splatad_compute_lidar_velocity_bwd(uint32_t C, uint32_t N, const float *p_vi
                                        float *v_p_view, float *v_velocities,
                                        splatad_stream_t stream);
 
+/* ---- (Gaussian, pixel) index lists -------------------------------------- */
+
+/* rasterize_to_indices_in_range_tensor, rasterization.cu:1003-1092 (kernel :839-1001)
+ * and rasterize_to_indices_in_range_lidar_tensor, :1270-1358 (kernel :1100-1268).
+ *
+ * The reference runs its kernel twice inside one op, with a host read of the number of
+ * pairs in between to size the outputs.  Here the two passes are two entry points so that
+ * the caller owns every allocation:
+ *   *_count  counts the pairs of every pixel for batches [range_start, range_end) of each
+ *            tile's list (a batch is as many Gaussians as a tile has pixels), writes the
+ *            exclusive prefix sums to chunk_starts [C * H * W] (int64, row-major pixels,
+ *            sensor by sensor) and the number of pairs to *n_elems (device memory);
+ *   *_fill   writes gaussian_ids [n_elems] (index in [0, N)) and indices [n_elems]
+ *            (pixel + sensor * H * W), front to back within a pixel, with the same arguments
+ *            and the chunk_starts of the counting call.
+ * transmittances [C, H, W] is the transmittance reached before range_start.  range_end
+ * beyond the longest list is allowed (values above 2^32 - 1 are clamped).  workspace is
+ * splatad_rasterize_to_indices_workspace_bytes(C, W, H) of scratch. */
+size_t splatad_rasterize_to_indices_workspace_bytes(uint32_t C, uint32_t image_width,
+                                                    uint32_t image_height);
+int splatad_rasterize_to_indices_in_range_count(
+    int64_t range_start, int64_t range_end, uint32_t C, uint32_t N, int64_t n_isects,
+    const float *transmittances, const float *means2d, const float *conics,
+    const float *opacities, const float *pix_vels, const float *rolling_shutter_time,
+    uint32_t image_width, uint32_t image_height, uint32_t tile_size, uint32_t tile_width,
+    uint32_t tile_height, const int32_t *tile_offsets, const int32_t *flatten_ids,
+    void *workspace, size_t workspace_bytes, int64_t *chunk_starts, int64_t *n_elems,
+    splatad_stream_t stream);
+int splatad_rasterize_to_indices_in_range_fill(
+    int64_t range_start, int64_t range_end, uint32_t C, uint32_t N, int64_t n_isects,
+    const float *transmittances, const float *means2d, const float *conics,
+    const float *opacities, const float *pix_vels, const float *rolling_shutter_time,
+    uint32_t image_width, uint32_t image_height, uint32_t tile_size, uint32_t tile_width,
+    uint32_t tile_height, const int32_t *tile_offsets, const int32_t *flatten_ids,
+    const int64_t *chunk_starts, int64_t *gaussian_ids, int64_t *indices,
+    splatad_stream_t stream);
+/* Lidar: pix_vels is [C, N, 3], raster_pts [C, H, W, 4] = azimuth, elevation (degrees),
+ * range, time; tile_width x tile_height points per tile (at most 256), grid of
+ * tile_grid_width x tile_grid_height tiles. */
+int splatad_rasterize_to_indices_in_range_lidar_count(
+    int64_t range_start, int64_t range_end, uint32_t C, uint32_t N, int64_t n_isects,
+    const float *transmittances, const float *means2d, const float *conics,
+    const float *opacities, const float *pix_vels, const float *raster_pts,
+    uint32_t image_width, uint32_t image_height, uint32_t tile_width, uint32_t tile_height,
+    uint32_t tile_grid_width, uint32_t tile_grid_height, const int32_t *tile_offsets,
+    const int32_t *flatten_ids, void *workspace, size_t workspace_bytes,
+    int64_t *chunk_starts, int64_t *n_elems, splatad_stream_t stream);
+int splatad_rasterize_to_indices_in_range_lidar_fill(
+    int64_t range_start, int64_t range_end, uint32_t C, uint32_t N, int64_t n_isects,
+    const float *transmittances, const float *means2d, const float *conics,
+    const float *opacities, const float *pix_vels, const float *raster_pts,
+    uint32_t image_width, uint32_t image_height, uint32_t tile_width, uint32_t tile_height,
+    uint32_t tile_grid_width, uint32_t tile_grid_height, const int32_t *tile_offsets,
+    const int32_t *flatten_ids, const int64_t *chunk_starts, int64_t *gaussian_ids,
+    int64_t *indices, splatad_stream_t stream);
+
 /* ---- densification helper --------------------------------------------- */
 
 /* compute_relocation_tensor, gsplat/cuda/csrc/relocation.cu:32-56 (kernel :4-30; op

@@ -340,3 +340,130 @@ def rasterize_to_points_fwd(means2d, conics, colors, opacities, pix_vels, depth_
        ctypes.c_float(threshold), _p(offs), _p(flat), ctypes.c_int(depth_channel_idx), _p(rc),
        _p(ra), _p(asum), _p(last), _p(med))
     return rc, ra, last, asum, med
+
+
+# ---------------------------------------------------------------------------
+# (Gaussian, pixel) index lists and compositing over them
+# ---------------------------------------------------------------------------
+def _indices_in_range(lidar, range_start, range_end, transmittances, means2d, conics, opacities,
+                      pix_vels, sensor, width, height, tile_width, tile_height, isect_offsets,
+                      flatten_ids, precision):
+    lib = _lib(precision)
+    trans = _f32(transmittances); means2d = _f32(means2d); conics = _f32(conics)
+    opacities = _f32(opacities); pix_vels = _f32(pix_vels); sensor = _f32(sensor)
+    offs = np.ascontiguousarray(np.asarray(isect_offsets, dtype=np.int32))
+    flat = np.ascontiguousarray(np.asarray(flatten_ids, dtype=np.int32))
+    C, gh, gw = offs.shape
+    N = means2d.shape[1]
+    fn = getattr(lib, f"oracle_{precision}_rasterize_to_indices_in_range")
+    fn.restype = None
+    cap = 2 ** 40
+
+    def run(counts, starts, gids, idx):
+        fn(ctypes.c_int(bool(lidar)), ctypes.c_long(min(int(range_start), cap)),
+           ctypes.c_long(min(int(range_end), cap)), ctypes.c_int(C), ctypes.c_long(N),
+           ctypes.c_long(flat.shape[0]), _p(trans), _p(means2d), _p(conics), _p(opacities),
+           _p(pix_vels), _p(sensor), ctypes.c_int(width), ctypes.c_int(height),
+           ctypes.c_int(tile_width), ctypes.c_int(tile_height), ctypes.c_int(gw), ctypes.c_int(gh),
+           _p(offs), _p(flat), _p(counts), _p(starts), _p(gids), _p(idx))
+
+    counts = np.zeros(C * height * width, np.int32)
+    run(counts, None, None, None)
+    starts = np.ascontiguousarray(np.cumsum(counts, dtype=np.int64) - counts)
+    total = int(counts.sum(dtype=np.int64))
+    gids = np.zeros(total, np.int64); idx = np.zeros(total, np.int64)
+    if total:
+        run(None, starts, gids, idx)
+    return gids, idx % (width * height), idx // (width * height)
+
+
+def rasterize_to_indices_in_range(range_start, range_end, transmittances, means2d, conics,
+                                  opacities, pix_vels, width, height, tile_size, isect_offsets,
+                                  flatten_ids, rolling_shutter_time=None, precision="f32"):
+    """Restates ``rasterize_to_indices_in_range`` (_wrapper.py:1115-1198; kernel and its two
+    passes rasterization.cu:839-1092).  Returns (gaussian_ids, pixel_ids, camera_ids), int64."""
+    C = np.asarray(means2d).shape[0]
+    rs = np.zeros(C, np.float32) if rolling_shutter_time is None else rolling_shutter_time
+    return _indices_in_range(False, range_start, range_end, transmittances, means2d, conics,
+                             opacities, pix_vels, rs, width, height, tile_size, tile_size,
+                             isect_offsets, flatten_ids, precision)
+
+
+def rasterize_to_indices_in_range_lidar(range_start, range_end, transmittances, means2d, conics,
+                                        opacities, pix_vels, raster_pts, width, height,
+                                        tile_width, tile_height, isect_offsets, flatten_ids,
+                                        precision="f32"):
+    """Restates ``rasterize_to_indices_in_range_lidar`` (_wrapper.py:1200-1281; kernel
+    rasterization.cu:1100-1358)."""
+    return _indices_in_range(True, range_start, range_end, transmittances, means2d, conics,
+                             opacities, pix_vels, raster_pts, width, height, tile_width,
+                             tile_height, isect_offsets, flatten_ids, precision)
+
+
+def _composite_rays(alphas, values, rays, n_rays):
+    """Per ray, in list order: T_k = prod_{j<k} (1 - alpha_j), weight_k = T_k alpha_k; returns
+    (sum_k weight_k values_k [n_rays, D], sum_k weight_k [n_rays, 1]).  This is what the
+    reference obtains from nerfacc's render_weight_from_alpha and accumulate_along_rays
+    (_torch_impl.py:694-704); nerfacc is not vendored by the reference and no version is
+    pinned, so the published definition is restated as a scalar loop."""
+    out = np.zeros((n_rays, values.shape[-1]), np.float64)
+    acc = np.zeros((n_rays, 1), np.float64)
+    T, prev = 1.0, -1
+    for k in range(alphas.shape[0]):
+        r = int(rays[k])
+        if r != prev:
+            T, prev = 1.0, r
+        w = T * float(alphas[k])
+        out[r] += w * values[k]
+        acc[r, 0] += w
+        T *= 1.0 - float(alphas[k])
+    return out, acc
+
+
+def accumulate(means2d, conics, opacities, colors, pix_vels, rolling_shutter_time, gaussian_ids,
+               pixel_ids, camera_ids, width, height):
+    """Restates ``accumulate`` (_torch_impl.py:610-706) in float64.  Returns
+    (renders[C,H,W,D], alphas[C,H,W,1])."""
+    f = lambda a: np.asarray(a, np.float64)
+    means2d, conics, opacities, colors, pix_vels = map(f, (means2d, conics, opacities, colors, pix_vels))
+    rs = f(rolling_shutter_time)
+    g, p, c = (np.asarray(a, np.int64) for a in (gaussian_ids, pixel_ids, camera_ids))
+    C, D = means2d.shape[0], colors.shape[-1]
+    col, row = p % width, p // width
+    roll = rs[c] * (row / (height - 1) - 0.5)
+    d = means2d[c, g] + roll[:, None] * pix_vels[c, g] - (np.stack([col, row], -1) + 0.5)
+    cn = conics[c, g]
+    sigma = 0.5 * (cn[:, 0] * d[:, 0] ** 2 + cn[:, 2] * d[:, 1] ** 2) + cn[:, 1] * d[:, 0] * d[:, 1]
+    alpha = np.minimum(opacities[c, g] * np.exp(-sigma), 0.999)
+    out, acc = _composite_rays(alpha, colors[c, g], c * height * width + p, C * height * width)
+    return out.reshape(C, height, width, D), acc.reshape(C, height, width, 1)
+
+
+def accumulate_lidar(means2d, conics, opacities, lidar_features, pix_vels, depth_compensations,
+                     raster_pts, gaussian_ids, pixel_ids, camera_ids, width, height,
+                     compute_alpha_sum_until_pts, compute_alpha_sum_until_pts_threshold):
+    """Restates ``accumulate_lidar`` (_torch_impl.py:709-830) in float64.  Returns
+    (renders, alphas, alpha_sum_until_points | None)."""
+    f = lambda a: np.asarray(a, np.float64)
+    means2d, conics, opacities, feats, pix_vels, dc, pts = map(
+        f, (means2d, conics, opacities, lidar_features, pix_vels, depth_compensations, raster_pts))
+    g, p, c = (np.asarray(a, np.int64) for a in (gaussian_ids, pixel_ids, camera_ids))
+    C, D = means2d.shape[0], feats.shape[-1]
+    col, row = p % width, p // width
+    pt = pts[c, row, col]
+    roll = pt[:, 3]
+    d = np.mod(means2d[c, g] + roll[:, None] * pix_vels[c, g][:, :2] - pt[:, :2] + 180, 360) - 180
+    cn = conics[c, g]
+    sigma = 0.5 * (cn[:, 0] * d[:, 0] ** 2 + cn[:, 2] * d[:, 1] ** 2) + cn[:, 1] * d[:, 0] * d[:, 1]
+    alpha = np.minimum(opacities[c, g] * np.exp(-sigma), 0.999)
+    vals = feats[c, g].copy()
+    vals[:, -1] += (d * dc[c, g]).sum(-1) + pix_vels[c, g][:, 2] * roll
+    rays, n_rays = c * height * width + p, C * height * width
+    out, acc = _composite_rays(alpha, vals, rays, n_rays)
+    asum = None
+    if compute_alpha_sum_until_pts:
+        before = feats[c, g][:, -1] < pt[:, 2] - compute_alpha_sum_until_pts_threshold
+        asum = np.zeros(n_rays, np.float64)
+        np.add.at(asum, rays, np.where(before, alpha, 0.0))
+        asum = asum.reshape(C, height, width, 1)
+    return out.reshape(C, height, width, D), acc.reshape(C, height, width, 1), asum

@@ -872,4 +872,77 @@ void NAME(rasterize_to_points_fwd)(int C, long n_isects, int D, const float *mea
     }
 }
 
+/* ------------------------------------------------------------------ */
+/* (Gaussian, pixel) index lists: rasterize_to_indices_in_range_kernel   */
+/* (rasterization.cu:839-1001) and its lidar twin (:1100-1268).          */
+/* One scalar loop per pixel over batches [range_start, range_end) of    */
+/* its tile's list, a batch being tile_width * tile_height entries; the  */
+/* pixel starts from transmittances[pix].  With chunk_starts == NULL the */
+/* pairs of every pixel are counted into counts[pix]; otherwise they are */
+/* written from chunk_starts[pix] on (the reference's two passes,        */
+/* :1054-1090).  lidar: sensor = raster_pts [C,H,W,4], points with       */
+/* range <= 0 take nothing (:1218-1222); camera: sensor = rolling        */
+/* shutter time [C].                                                     */
+/* ------------------------------------------------------------------ */
+void NAME(rasterize_to_indices_in_range)(int lidar, long range_start, long range_end, int C,
+                                         long N, long n_isects, const float *transmittances,
+                                         const float *means2d, const float *conics,
+                                         const float *opacities, const float *pix_vels,
+                                         const float *sensor, int W, int H, int tile_width,
+                                         int tile_height, int grid_w, int grid_h,
+                                         const int32_t *tile_offsets, const int32_t *flatten_ids,
+                                         int32_t *counts, const int64_t *chunk_starts,
+                                         int64_t *gaussian_ids, int64_t *indices) {
+    long n_tiles = (long)grid_w * grid_h;
+    long block = (long)tile_width * tile_height;
+    int vs = lidar ? 3 : 2;
+#pragma omp parallel for schedule(dynamic, 64)
+    for (long pix = 0; pix < (long)C * H * W; ++pix) {
+        int cid = (int)(pix / ((long)H * W));
+        long rem = pix % ((long)H * W);
+        int i = (int)(rem / W), j = (int)(rem % W);
+        long tile_id = (long)(i / tile_height) * grid_w + (j / tile_width);
+        long t_glob = cid * n_tiles + tile_id;
+        long start = tile_offsets[t_glob];
+        long end = (cid == C - 1 && tile_id == n_tiles - 1) ? n_isects : tile_offsets[t_glob + 1];
+        long num_batches = (end - start + block - 1) / block;
+        long b_end = range_end < num_batches ? range_end : num_batches;
+        long cnt = 0;
+        real px, py, roll;
+        int active = 1;
+        if (lidar) {
+            const float *rp = sensor + pix * 4;
+            px = rp[0]; py = rp[1]; roll = rp[3];
+            active = rp[2] > 0;
+        } else {
+            px = (real)j + RC(0.5); py = (real)i + RC(0.5);
+            roll = RC(sensor[cid]) * ((py - RC(0.5)) / (real)(H - 1) - RC(0.5)); /* :876 */
+        }
+        real T = transmittances[pix];
+        if (active && range_start < num_batches) {
+            long s_end = start + b_end * block < end ? start + b_end * block : end;
+            for (long s = start + range_start * block; s < s_end; ++s) {
+                long g = flatten_ids[s];
+                real dx = RC(means2d[g * 2]) + roll * RC(pix_vels[g * vs]);
+                real dy = RC(means2d[g * 2 + 1]) + roll * RC(pix_vels[g * vs + 1]);
+                if (lidar) { dx = angle_difference(dx, px); dy = angle_difference(dy, py); }
+                else { dx -= px; dy -= py; }
+                real ca = conics[g * 3], cb = conics[g * 3 + 1], cc = conics[g * 3 + 2];
+                real sigma = RC(0.5) * (ca * dx * dx + cc * dy * dy) + cb * dx * dy;
+                real alpha = R_FMIN(RC(0.999), RC(opacities[g]) * R_EXP(-sigma));
+                if (sigma < 0 || alpha < RC(1) / RC(255)) continue;
+                real next_T = T * (RC(1) - alpha);
+                if (next_T <= RC(1e-4)) break;
+                if (chunk_starts) {
+                    gaussian_ids[chunk_starts[pix] + cnt] = g % N;
+                    indices[chunk_starts[pix] + cnt] = pix;
+                }
+                ++cnt;
+                T = next_T;
+            }
+        }
+        if (!chunk_starts) counts[pix] = (int32_t)cnt;
+    }
+}
+
 int NAME(sizeof_real)(void) { return (int)sizeof(real); }

@@ -4,6 +4,7 @@ Exports the operators and end-to-end functions of the reference's gsplat/__init_
 lie on the path projection -> tile intersection -> rasterization, and the lidar point binning
 that prepares the points to render.
 """
+from .hip._torch_impl import accumulate, accumulate_lidar
 from .hip._wrapper import (
     compute_lidar_velocity,
     compute_pix_velocity,
@@ -19,6 +20,8 @@ from .hip._wrapper import (
     map_points_to_lidar_tiles,
     points_mapping_offset_encode,
     populate_image_from_points,
+    rasterize_to_indices_in_range,
+    rasterize_to_indices_in_range_lidar,
     rasterize_to_pixels,
     rasterize_to_points,
     spherical_harmonics,
@@ -47,4 +50,8 @@ __all__ = [
     "map_points_to_lidar_tiles",
     "points_mapping_offset_encode",
     "populate_image_from_points",
+    "rasterize_to_indices_in_range",
+    "rasterize_to_indices_in_range_lidar",
+    "accumulate",
+    "accumulate_lidar",
 ]

@@ -36,7 +36,8 @@ def load_library():
         lib.splatad_last_error.restype = ctypes.c_char_p
         lib.splatad_abi_version.restype = ctypes.c_int
         for name in ("splatad_projection_packed_workspace_bytes", "splatad_isect_workspace_bytes",
-                     "splatad_map_points_to_lidar_tiles_workspace_bytes"):
+                     "splatad_map_points_to_lidar_tiles_workspace_bytes",
+                     "splatad_rasterize_to_indices_workspace_bytes"):
             getattr(lib, name).restype = ctypes.c_size_t
         _lib = lib
     return _lib
@@ -730,6 +731,67 @@ class _Ops:
                     _p(v_means2d), _p(v_conics), _p(v_colors), _p(v_opacities), _p(v_pix_vels),
                     _p(v_dc), _stream(dev)))
         return v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_dc
+
+    # ------------------------------------------------------------------ index lists
+    def _indices_in_range(self, lidar, range_start, range_end, transmittances, means2d, conics,
+                          opacities, pix_vels, sensor, image_width, image_height, tile_width,
+                          tile_height, tile_offsets, flatten_ids):
+        lib = load_library()
+        transmittances = _in(transmittances, "transmittances")
+        means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
+        opacities = _in(opacities, "opacities"); pix_vels = _in(pix_vels, "pix_vels")
+        sensor = _in(sensor, "raster_pts" if lidar else "rolling_shutter_time")
+        tile_offsets = _in(tile_offsets, "tile_offsets", torch.int32)
+        flatten_ids = _in(flatten_ids, "flatten_ids", torch.int32)
+        C, N = means2d.shape[0], means2d.shape[1]
+        gh, gw = tile_offsets.shape[1], tile_offsets.shape[2]
+        dev = means2d.device
+        i64 = dict(dtype=torch.int64, device=dev)
+        n_pixels, n_isects = C * image_height * image_width, flatten_ids.shape[0]
+        if n_pixels == 0 or n_isects == 0:
+            return torch.empty((0,), **i64), torch.empty((0,), **i64)
+        count = (lib.splatad_rasterize_to_indices_in_range_lidar_count if lidar
+                 else lib.splatad_rasterize_to_indices_in_range_count)
+        fill = (lib.splatad_rasterize_to_indices_in_range_lidar_fill if lidar
+                else lib.splatad_rasterize_to_indices_in_range_fill)
+        tiles = ((_u32(tile_width), _u32(tile_height), _u32(gw), _u32(gh)) if lidar
+                 else (_u32(tile_width), _u32(gw), _u32(gh)))
+        head = (_i64(int(min(range_start, 2 ** 62))), _i64(int(min(range_end, 2 ** 62))), _u32(C),
+                _u32(N), _i64(n_isects), _p(transmittances), _p(means2d), _p(conics), _p(opacities),
+                _p(pix_vels), _p(sensor), _u32(image_width), _u32(image_height), *tiles,
+                _p(tile_offsets), _p(flatten_ids))
+        with torch.cuda.device(dev):
+            nbytes = lib.splatad_rasterize_to_indices_workspace_bytes(
+                _u32(C), _u32(image_width), _u32(image_height))
+            ws = _workspace(nbytes, dev)
+            chunk_starts = torch.empty((n_pixels,), **i64)
+            n_elems = torch.empty((1,), **i64)
+            _check(count(*head, _p(ws), ctypes.c_size_t(ws.numel()), _p(chunk_starts), _p(n_elems),
+                         _stream(dev)))
+            total = int(n_elems.item())  # the one host read: sizes the outputs
+            gaussian_ids = torch.empty((total,), **i64)
+            indices = torch.empty((total,), **i64)
+            if total:
+                _check(fill(*head, _p(chunk_starts), _p(gaussian_ids), _p(indices), _stream(dev)))
+        return gaussian_ids, indices
+
+    def rasterize_to_indices_in_range(self, range_start, range_end, transmittances, means2d,
+                                      conics, opacities, pix_vels, rolling_shutter_time,
+                                      image_width, image_height, tile_size, tile_offsets,
+                                      flatten_ids):
+        return self._indices_in_range(False, range_start, range_end, transmittances, means2d,
+                                      conics, opacities, pix_vels, rolling_shutter_time,
+                                      image_width, image_height, tile_size, tile_size,
+                                      tile_offsets, flatten_ids)
+
+    def rasterize_to_indices_in_range_lidar(self, range_start, range_end, transmittances, means2d,
+                                            conics, opacities, pix_vels, raster_pts, image_width,
+                                            image_height, tile_width, tile_height, tile_offsets,
+                                            flatten_ids):
+        return self._indices_in_range(True, range_start, range_end, transmittances, means2d,
+                                      conics, opacities, pix_vels, raster_pts, image_width,
+                                      image_height, tile_width, tile_height, tile_offsets,
+                                      flatten_ids)
 
 
 _C = _Ops()

@@ -414,6 +414,98 @@ def rasterize_to_points(
     )
 
 
+@torch.no_grad()
+def rasterize_to_indices_in_range(
+    range_start: int,
+    range_end: int,
+    transmittances: Tensor,  # [C, image_height, image_width]
+    means2d: Tensor,  # [C, N, 2]
+    conics: Tensor,  # [C, N, 3]
+    opacities: Tensor,  # [C, N]
+    pix_vels: Tensor,  # [C, N, 2]
+    image_width: int,
+    image_height: int,
+    tile_size: int,
+    isect_offsets: Tensor,  # [C, tile_height, tile_width]
+    flatten_ids: Tensor,  # [n_isects]
+    rolling_shutter_time: Optional[Tensor] = None,  # [C]
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """Lists the (Gaussian, pixel, camera) triples that take part in compositing, for batches
+    `[range_start, range_end)` of every tile's depth-sorted list (a batch is tile_size**2
+    Gaussians), starting from the transmittance reached so far.  A very large `range_end`
+    walks every list to its end in one call.  (Reference: gsplat/cuda/_wrapper.py:1115-1198.)
+
+    Returns (gaussian_ids[M], pixel_ids[M] (row-major), camera_ids[M]), int64; within a pixel
+    front to back, pixels in row-major order, camera by camera.
+    """
+    C, N, _ = means2d.shape
+    assert conics.shape == (C, N, 3), conics.shape
+    assert opacities.shape == (C, N), opacities.shape
+    assert isect_offsets.shape[0] == C, isect_offsets.shape
+    assert pix_vels.shape == (C, N, 2), pix_vels.shape
+    assert transmittances.shape == (C, image_height, image_width), transmittances.shape
+    if rolling_shutter_time is not None:
+        assert rolling_shutter_time.shape == (C,), rolling_shutter_time.shape
+    else:
+        rolling_shutter_time = torch.zeros(C, device=means2d.device)
+    tile_height, tile_width = isect_offsets.shape[1:3]
+    assert tile_height * tile_size >= image_height, f"Assert Failed: {tile_height} * {tile_size} >= {image_height}"
+    assert tile_width * tile_size >= image_width, f"Assert Failed: {tile_width} * {tile_size} >= {image_width}"
+
+    out_gauss_ids, out_indices = _make_lazy_hip_func("rasterize_to_indices_in_range")(
+        range_start, range_end, transmittances.contiguous(), means2d.contiguous(),
+        conics.contiguous(), opacities.contiguous(), pix_vels.contiguous(),
+        rolling_shutter_time.contiguous(), image_width, image_height, tile_size,
+        isect_offsets.contiguous(), flatten_ids.contiguous(),
+    )
+    out_pixel_ids = out_indices % (image_width * image_height)
+    out_camera_ids = out_indices // (image_width * image_height)
+    return out_gauss_ids, out_pixel_ids, out_camera_ids
+
+
+@torch.no_grad()
+def rasterize_to_indices_in_range_lidar(
+    range_start: int,
+    range_end: int,
+    transmittances: Tensor,  # [C, image_height, image_width]
+    means2d: Tensor,  # [C, N, 2]
+    conics: Tensor,  # [C, N, 3]
+    opacities: Tensor,  # [C, N]
+    pix_vels: Tensor,  # [C, N, 3]
+    raster_pts: Tensor,  # [C, image_height, image_width, 4]
+    image_width: int,
+    image_height: int,
+    tile_width: int,
+    tile_height: int,
+    isect_offsets: Tensor,  # [C, tile_grid_height, tile_grid_width]
+    flatten_ids: Tensor,  # [n_isects]
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """`rasterize_to_indices_in_range` for lidar points given as (azimuth, elevation, range,
+    time); a batch is tile_width * tile_height Gaussians and points with range <= 0 take
+    nothing.  (Reference: gsplat/cuda/_wrapper.py:1200-1281.)
+    """
+    C, N, _ = means2d.shape
+    assert conics.shape == (C, N, 3), conics.shape
+    assert opacities.shape == (C, N), opacities.shape
+    assert isect_offsets.shape[0] == C, isect_offsets.shape
+    assert pix_vels.shape == (C, N, 3), pix_vels.shape
+    assert transmittances.shape == (C, image_height, image_width), transmittances.shape
+    assert raster_pts.shape == (C, image_height, image_width, 4), raster_pts.shape
+    tile_grid_height, tile_grid_width = isect_offsets.shape[1:3]
+    assert tile_grid_height * tile_height >= image_height, f"Assert Failed: {tile_grid_height} * {tile_height} >= {image_height}"
+    assert tile_grid_width * tile_width >= image_width, f"Assert Failed: {tile_grid_width} * {tile_width} >= {image_width}"
+
+    out_gauss_ids, out_indices = _make_lazy_hip_func("rasterize_to_indices_in_range_lidar")(
+        range_start, range_end, transmittances.contiguous(), means2d.contiguous(),
+        conics.contiguous(), opacities.contiguous(), pix_vels.contiguous(),
+        raster_pts.contiguous(), image_width, image_height, tile_width, tile_height,
+        isect_offsets.contiguous(), flatten_ids.contiguous(),
+    )
+    out_pixel_ids = out_indices % (image_width * image_height)
+    out_camera_ids = out_indices // (image_width * image_height)
+    return out_gauss_ids, out_pixel_ids, out_camera_ids
+
+
 # ---------------------------------------------------------------------------------------------
 # autograd pairing of the forward and backward kernels
 # ---------------------------------------------------------------------------------------------
