@@ -10,9 +10,9 @@
  *     *_workspace_bytes queries); the library never allocates or frees device
  *     memory;
  *   - all work is enqueued on `stream` (a hipStream_t); the only host
- *     synchronisation is inside the *_count entry points, which copy one
- *     integer back to the host (the reference does the same through
- *     Tensor::item(): rasterization.cu:154,465, projection.cu:1421);
+ *     waits are inside the *_count entry points, which copy one integer back
+ *     to the host (the reference does the same through Tensor::item():
+ *     rasterization.cu:154,465, projection.cu:1421);
  *   - return value 0 = success, negative = error; splatad_last_error() gives a
  *     thread-local message (the reference raises through TORCH_CHECK,
  *     bindings.h:9-13).
@@ -122,6 +122,29 @@ int splatad_sh_bwd(uint32_t n, uint32_t K, uint32_t degree, const float *dirs,
                    const float *coeffs, const uint8_t *masks, const float *v_colors,
                    float *v_coeffs, float *v_dirs, splatad_stream_t stream);
 
+/* View-dependent colours of the rendering pipeline in one launch: the block of
+ * gsplat/rendering.py:325-351 (inverse of the view matrices, viewing directions, visibility
+ * masks, spherical_harmonics(), max(c + 1/2, 0) and, optionally, the depth as fourth channel).
+ * Row e is (sensor e / N, Gaussian e % N) for n == C * N, or (camera_ids[e], gaussian_ids[e])
+ * for packed input; its direction is means[g] minus the sensor position -A^-1 t of
+ * viewmats[c] = [A | t] (last row (0, 0, 0, 1), as the projection kernels assume); it is
+ * active when radii[e][0] > 0 and inactive rows evaluate to max(1/2, 0).  coeffs is [N, K, 3]
+ * (coeffs_per_sensor == 0) or [C, N, K, 3] (== 1).  colors has 3 channels, or 4 with depths.
+ * _bwd takes the forward's colors (a channel passes its gradient only where it is positive)
+ * and writes one row per e: v_coeffs [n, K, 3] (zero-filled by the caller) and, unless NULL,
+ * v_dirs [n, 3]; the caller sums rows that share a Gaussian. */
+int splatad_view_colors_fwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
+                            const float *means, const float *viewmats, const int64_t *camera_ids,
+                            const int64_t *gaussian_ids, const int32_t *radii, const float *coeffs,
+                            int coeffs_per_sensor, const float *depths, float *colors,
+                            splatad_stream_t stream);
+int splatad_view_colors_bwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
+                            const float *means, const float *viewmats, const int64_t *camera_ids,
+                            const int64_t *gaussian_ids, const int32_t *radii, const float *coeffs,
+                            int coeffs_per_sensor, uint32_t channels, const float *colors,
+                            const float *v_colors, float *v_coeffs, float *v_dirs,
+                            splatad_stream_t stream);
+
 /* ---- tile intersection, sort, offsets ----------------------------------- */
 
 /* isect_tiles_tensor (rasterization.cu:92-216) and isect_lidar_tiles_tensor
@@ -131,31 +154,41 @@ int splatad_sh_bwd(uint32_t n, uint32_t K, uint32_t degree, const float *dirs,
  * (camera, tile, depth bits) with ties in emission order when sort != 0, in
  * emission order otherwise.  Depths must be non-negative (sign bit clear).
  * For lidars tile_width/tile_height are the azimuth/elevation tile counts and
- * elev_boundaries has tile_height+1 entries.  The workspace of _count needs
- * splatad_isect_workspace_bytes(total, C, n_tiles, 0) bytes, that of _fill
- * splatad_isect_workspace_bytes(total, C, n_tiles, n_isects); nothing has to
- * survive between the two calls except tiles_per_gauss.  tile_offsets may be
- * NULL; with sort != 0 it receives the [C, tile_height, tile_width] table that
- * splatad_isect_offset_encode would derive from isect_ids (the binning knows
- * every tile's first intersection before the sort runs). */
-size_t splatad_isect_workspace_bytes(uint64_t total, uint32_t C, uint32_t n_tiles,
-                                     int64_t n_isects);
-int splatad_isect_tiles_count(uint64_t total, const float *means2d, const int32_t *radii,
-                              uint32_t C, uint32_t tile_size, uint32_t tile_width,
-                              uint32_t tile_height, int32_t *tiles_per_gauss, void *workspace,
+ * elev_boundaries has tile_height+1 entries.
+ *
+ * Memory: `workspace` is splatad_isect_workspace_bytes(total, C, n_tiles) bytes
+ * and is shared by the two calls: with sort != 0, _count also enqueues the first
+ * stages of the binning (they do not depend on n_isects) behind the counting
+ * kernel, so that the GPU has work while the host sizes the outputs, and _fill
+ * continues from what they left there.  Pass both calls the same sort flag, inputs
+ * and stream, and leave the workspace untouched in between.  `lists` is
+ * splatad_isect_lists_bytes(total, n_isects) bytes of scratch for _fill alone.
+ * _count waits for the counting kernel only (the kernel writes n_isects into a
+ * pinned host slot, one per device, kept for the life of the process, and the
+ * host spins on it), not for the work enqueued behind it.
+ *
+ * tile_offsets may be NULL; with sort != 0 it receives the [C, tile_height,
+ * tile_width] table that splatad_isect_offset_encode would derive from isect_ids
+ * (the binning knows every tile's first intersection before the sort runs). */
+size_t splatad_isect_workspace_bytes(uint64_t total, uint32_t C, uint32_t n_tiles);
+size_t splatad_isect_lists_bytes(uint64_t total, int64_t n_isects);
+int splatad_isect_tiles_count(uint64_t total, uint32_t N, const int64_t *camera_ids,
+                              const float *means2d, const int32_t *radii, uint32_t C,
+                              uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
+                              int sort, int32_t *tiles_per_gauss, void *workspace,
                               int64_t *n_isects_host, splatad_stream_t stream);
 int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_ids,
                              const float *means2d, const int32_t *radii, const float *depths,
                              uint32_t C, uint32_t tile_size, uint32_t tile_width,
                              uint32_t tile_height, int sort, int64_t n_isects,
-                             const int32_t *tiles_per_gauss, void *workspace, int64_t *isect_ids,
-                             int32_t *flatten_ids, int32_t *tile_offsets,
+                             const int32_t *tiles_per_gauss, void *workspace, void *lists,
+                             int64_t *isect_ids, int32_t *flatten_ids, int32_t *tile_offsets,
                              splatad_stream_t stream);
-int splatad_isect_lidar_tiles_count(uint64_t total, const float *means2d, const float *radii,
-                                    uint32_t C, const float *elev_boundaries,
-                                    float tile_azim_resolution, float min_azim,
-                                    uint32_t tile_width, uint32_t tile_height,
-                                    int32_t *tiles_per_gauss, void *workspace,
+int splatad_isect_lidar_tiles_count(uint64_t total, uint32_t N, const int64_t *camera_ids,
+                                    const float *means2d, const float *radii, uint32_t C,
+                                    const float *elev_boundaries, float tile_azim_resolution,
+                                    float min_azim, uint32_t tile_width, uint32_t tile_height,
+                                    int sort, int32_t *tiles_per_gauss, void *workspace,
                                     int64_t *n_isects_host, splatad_stream_t stream);
 int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_ids,
                                    const float *means2d, const float *radii, const float *depths,
@@ -163,8 +196,9 @@ int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N, const int64_t *ca
                                    float tile_azim_resolution, float min_azim,
                                    uint32_t tile_width, uint32_t tile_height, int sort,
                                    int64_t n_isects, const int32_t *tiles_per_gauss,
-                                   void *workspace, int64_t *isect_ids, int32_t *flatten_ids,
-                                   int32_t *tile_offsets, splatad_stream_t stream);
+                                   void *workspace, void *lists, int64_t *isect_ids,
+                                   int32_t *flatten_ids, int32_t *tile_offsets,
+                                   splatad_stream_t stream);
 
 /* isect_offset_encode_tensor, rasterization.cu:264-285 (kernel :218-262). */
 int splatad_isect_offset_encode(int64_t n_isects, const int64_t *isect_ids, uint32_t C,

@@ -125,7 +125,8 @@ template <bool LIDAR>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d,
                    const void *__restrict__ radii, int32_t *__restrict__ tiles_per_gauss,
-                   unsigned long long *__restrict__ n_isects) {
+                   unsigned long long *__restrict__ n_isects,
+                   unsigned long long *__restrict__ n_isects_host) {
     SPLATAD_STAGE_ELEVATIONS(g)
     long long s = 0;
     for (uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
@@ -144,6 +145,14 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
         long long t = 0;
         for (int w = 0; w < SPLATAD_THREADS / SPLATAD_WAVE; ++w) t += wsum[w];
         if (t != 0) atomicAdd(n_isects, (unsigned long long)t);
+        // The workgroup that finishes last hands the total to the host, which spins on the
+        // pinned slot: no copy command, no event and no system-scope fence (which would write
+        // back whatever other kernels have dirtied in L2) stand between this kernel and the
+        // host or the work enqueued behind it.  n_isects[1] counts the finished workgroups.
+        __threadfence();
+        if (atomicAdd(n_isects + 1, 1ull) == gridDim.x - 1)
+            __hip_atomic_store(n_isects_host, atomicAdd(n_isects, 0ull), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_SYSTEM);
     }
 }
 
@@ -493,22 +502,16 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t L, uint32_t ti
 // network instead.  Segments with min_n < n <= max_n are handled, the others skipped.
 // Dynamic LDS: lds_words * 8 bytes of staging, the fine bins, 2 * bucket_cap counters.
 template <int ER, bool IN_LDS>
-__global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
-                                          uint32_t tile_n_bits, uint32_t min_n, uint32_t max_n,
-                                          uint32_t lds_words, uint32_t bucket_cap,
-                                          int64_t n_isects,
-                                          const int32_t *__restrict__ tile_starts,
-                                          const uint64_t *__restrict__ pairs, int64_t *isect_ids,
-                                          int32_t *__restrict__ flatten_ids) {
-    extern __shared__ uint64_t lds_staged[];
-    __shared__ uint32_t s_wave[2 * (1024 / SPLATAD_WAVE)];
-    __shared__ uint32_t s_big;
-    const uint32_t seg = blockIdx.x;
-    if (seg >= n_segments) return;
+__device__ __forceinline__ void sort_segment(uint32_t seg, uint32_t n_segments, uint32_t n_tiles,
+                                             uint32_t tile_n_bits, uint32_t lds_words,
+                                             uint32_t bucket_cap, int64_t n_isects,
+                                             const int32_t *__restrict__ tile_starts,
+                                             const uint64_t *__restrict__ pairs, int64_t *isect_ids,
+                                             int32_t *__restrict__ flatten_ids,
+                                             uint64_t *lds_staged, uint32_t *s_wave, uint32_t &s_big) {
     const int64_t start = tile_starts[seg];
     const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
     const uint32_t n = (uint32_t)(stop - start);
-    if (n <= min_n || n > max_n) return; // uniform across the workgroup
     uint32_t *s_fine = reinterpret_cast<uint32_t *>(lds_staged + lds_words);
     uint32_t *s_cursor = s_fine + kSortFineBins;
     uint32_t *s_first = s_cursor + bucket_cap;
@@ -683,11 +686,73 @@ __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
     }
 }
 
+// Size classes of the segment sort: class c holds the segments with kSortClassMin[c] < n <=
+// kSortClassMin[c + 1]; the host launches one kernel configuration per class.
+constexpr int kSortClasses = 7;
+__constant__ const uint32_t kSortClassMin[kSortClasses + 1] = {0u,    512u,   2048u,  4096u,
+                                                               8192u, 16384u, 32768u, 0x7FFFFFFFu};
+
+// Lists the segments of every class: seg_lists[c * n_segments + k], k < seg_counts[c] (zeroed
+// beforehand).  The order inside a class is whatever the atomics give; every segment is sorted
+// on its own, so the result does not depend on it.
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+isect_classify_segments_kernel(uint32_t n_segments, int64_t n_isects,
+                               const int32_t *__restrict__ tile_starts,
+                               uint32_t *__restrict__ seg_counts, uint32_t *__restrict__ seg_lists) {
+    const uint32_t seg = blockIdx.x * blockDim.x + threadIdx.x;
+    uint32_t n = 0;
+    if (seg < n_segments) {
+        const int64_t start = tile_starts[seg];
+        const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
+        n = (uint32_t)(stop - start);
+    }
+    int c = n == 0 ? -1 : 0;
+    while (c >= 0 && c + 1 < kSortClasses && n > kSortClassMin[c + 1]) ++c;
+    // one atomic per wavefront and class: thousands of segments share a class, and atomics on
+    // one address are served one after the other
+    const uint32_t lane = threadIdx.x & (SPLATAD_WAVE - 1);
+    for (int k = 0; k < kSortClasses; ++k) {
+        const uint64_t members = wave_ballot(c == k);
+        if (members == 0) continue; // uniform
+        const int leader = __ffsll((unsigned long long)members) - 1;
+        uint32_t base = 0;
+        if ((int)lane == leader) base = atomicAdd(&seg_counts[k], (uint32_t)__popcll(members));
+        base = (uint32_t)__shfl((int)base, leader, SPLATAD_WAVE);
+        if (c == k)
+            seg_lists[(size_t)k * n_segments + base + (uint32_t)__popcll(members & ((1ull << lane) - 1ull))] = seg;
+    }
+}
+
+// The workgroups of a launch share out the segments of one class; a launch has no more
+// workgroups than can be resident, so a class without segments costs next to nothing.
 template <int ER, bool IN_LDS>
-static int launch_segment_sort(uint32_t threads, uint32_t min_n, uint32_t max_n, uint32_t segs,
-                               uint32_t n_tiles, uint32_t tile_n_bits, int64_t n_isects,
-                               const int32_t *tile_starts, const uint64_t *pairs,
-                               int64_t *isect_ids, int32_t *flatten_ids, hipStream_t stream) {
+__global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
+                                          uint32_t tile_n_bits, uint32_t lds_words,
+                                          uint32_t bucket_cap, int64_t n_isects,
+                                          const uint32_t *__restrict__ seg_count,
+                                          const uint32_t *__restrict__ seg_list,
+                                          const int32_t *__restrict__ tile_starts,
+                                          const uint64_t *__restrict__ pairs, int64_t *isect_ids,
+                                          int32_t *__restrict__ flatten_ids) {
+    extern __shared__ uint64_t lds_staged[];
+    __shared__ uint32_t s_wave[2 * (1024 / SPLATAD_WAVE)];
+    __shared__ uint32_t s_big;
+    const uint32_t count = *seg_count;
+    for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) { // uniform across the workgroup
+        sort_segment<ER, IN_LDS>(seg_list[k], n_segments, n_tiles, tile_n_bits, lds_words, bucket_cap,
+                                 n_isects, tile_starts, pairs, isect_ids, flatten_ids, lds_staged,
+                                 s_wave, s_big);
+        __syncthreads(); // the next segment reuses the LDS
+    }
+}
+
+template <int ER, bool IN_LDS>
+static int launch_segment_sort(int cls, uint32_t threads, uint32_t max_n, uint32_t workgroups,
+                               uint32_t segs, uint32_t n_tiles, uint32_t tile_n_bits,
+                               int64_t n_isects, const uint32_t *seg_counts,
+                               const uint32_t *seg_lists, const int32_t *tile_starts,
+                               const uint64_t *pairs, int64_t *isect_ids, int32_t *flatten_ids,
+                               hipStream_t stream) {
     const uint32_t lds_words = IN_LDS ? max_n : kSortWindow;
     const uint32_t bucket_cap = sort_bucket_capacity(max_n);
     const size_t lds_bytes = (size_t)lds_words * 8 + (kSortFineBins + 2 * (size_t)bucket_cap) * 4;
@@ -702,9 +767,10 @@ static int launch_segment_sort(uint32_t threads, uint32_t min_n, uint32_t max_n,
             allowed = lds_bytes;
         }
     }
-    hipLaunchKernelGGL((isect_segment_sort_kernel<ER, IN_LDS>), dim3(segs), dim3(threads),
-                       lds_bytes, stream, segs, n_tiles, tile_n_bits, min_n, max_n, lds_words,
-                       bucket_cap, n_isects, tile_starts, pairs, isect_ids, flatten_ids);
+    hipLaunchKernelGGL((isect_segment_sort_kernel<ER, IN_LDS>), dim3(workgroups < segs ? workgroups : segs),
+                       dim3(threads), lds_bytes, stream, segs, n_tiles, tile_n_bits, lds_words,
+                       bucket_cap, n_isects, seg_counts + cls, seg_lists + (size_t)cls * segs,
+                       tile_starts, pairs, isect_ids, flatten_ids);
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }
@@ -739,7 +805,7 @@ __global__ void fill_zero_i32_kernel(int32_t *p, int64_t n) {
     if (i < n) p[i] = 0;
 }
 
-__global__ void fill_zero_u64_kernel(unsigned long long *p) { *p = 0ull; }
+__global__ void fill_zero_u64_kernel(unsigned long long *p) { p[threadIdx.x] = 0ull; }
 
 __global__ void copy_i32_kernel(const int32_t *__restrict__ src, int32_t *__restrict__ dst,
                                 int64_t n) {
@@ -758,7 +824,10 @@ struct IsectWorkspace {
     int32_t *coarse_counts;       // [coarse workgroups * C * blocks]
     int32_t *coarse_starts;       // same
     int32_t *tile_starts;         // [tile copies * C * n_tiles]
+    uint32_t *seg_counts;         // [kSortClasses] segments per size class (in the cleared part)
+    uint32_t *seg_lists;          // [kSortClasses * C * n_tiles]
     int64_t *block_sums;          // scan scratch
+    // the lists, whose size depends on the number of intersections
     int64_t *cum_before;          // [total] (sort == false)
     uint4 *entries;               // [n_isects] (sort == true), shares memory with cum_before
     uint64_t *pairs;              // [n_isects]
@@ -792,146 +861,118 @@ static uint32_t coarse_workgroups(uint64_t total, uint64_t blocks) {
     return (uint32_t)wgs;
 }
 
-// Layout from sizes only; cslots is the length of the coarse counter table, or an upper
-// bound of it when only the number of tiles is known (workspace sizing).
+// Everything the two calls derive from the sizes alone, the same way in both.
+struct IsectPlan {
+    uint32_t n_tiles, tile_n_bits, per_cam, coarse_wgs, cams_per_launch;
+    uint64_t segs, blocks, cslots;
+    CoarseGrid cg;
+};
+
+template <bool LIDAR>
+static IsectPlan isect_plan(const TileGrid &g, uint64_t total, uint32_t C) {
+    IsectPlan pl;
+    pl.n_tiles = g.tile_w * g.tile_h;
+    pl.tile_n_bits = splatad_bit_width(pl.n_tiles);
+    pl.segs = (uint64_t)C * pl.n_tiles;
+    pl.cg = coarse_grid<LIDAR>(g);
+    pl.per_cam = pl.cg.cw * pl.cg.ch;
+    pl.blocks = (uint64_t)C * pl.per_cam;
+    pl.coarse_wgs = coarse_workgroups(total, pl.blocks);
+    pl.cslots = pl.blocks * pl.coarse_wgs;
+    pl.cams_per_launch = pl.per_cam ? kCoarseLdsBlocks / pl.per_cam : 0;
+    return pl;
+}
+
+// Layout of the workspace from sizes only; cslots is the length of the coarse counter table,
+// or an upper bound of it when only the number of tiles is known (workspace sizing).
 static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslots,
-                          int64_t n_isects, IsectWorkspace *out) {
+                          IsectWorkspace *out) {
     const uint64_t tslots = segs * isect_copies(segs);
     uint64_t scan_n = total > cslots ? total : cslots;
     if (tslots > scan_n) scan_n = tslots;
     char *p = (char *)ws;
-    IsectWorkspace w;
+    IsectWorkspace w = {};
     w.n_isects = (unsigned long long *)p;   p += 256;
     w.n_entries = (int64_t *)p;             p += 256;
     w.scan_total = (int64_t *)p;            p += 256;
     w.zeroed = (int32_t *)p;
     w.tile_counts = (int32_t *)p;           p += splatad_align256(tslots * 4);
     w.tile_fill = (int32_t *)p;             p += splatad_align256(tslots * 4);
+    w.seg_counts = (uint32_t *)p;           p += 256;
     w.n_zeroed = (uint64_t)(p - (char *)w.zeroed) / 4;
     w.coarse_counts = (int32_t *)p;         p += splatad_align256(cslots * 4);
     w.coarse_starts = (int32_t *)p;         p += splatad_align256(cslots * 4);
     w.tile_starts = (int32_t *)p;           p += splatad_align256(tslots * 4);
+    w.seg_lists = (uint32_t *)p;            p += splatad_align256(segs * kSortClasses * 4);
     w.block_sums = (int64_t *)p;            p += scan_workspace_bytes((int64_t)scan_n);
-    const uint64_t list_bytes = splatad_align256((uint64_t)n_isects * 16);
-    const uint64_t cum_bytes = splatad_align256(total * 8);
-    w.cum_before = (int64_t *)p;
-    w.entries = (uint4 *)p;                 p += list_bytes > cum_bytes ? list_bytes : cum_bytes;
-    w.pairs = (uint64_t *)p;                p += splatad_align256((uint64_t)n_isects * 8);
     if (out) *out = w;
     return (size_t)(p - (char *)ws);
 }
 
-static size_t isect_ws_bytes(uint64_t total, uint64_t segs, int64_t n_isects) {
+static size_t carve_lists(void *lists, uint64_t total, int64_t n_isects, IsectWorkspace *w) {
+    char *p = (char *)lists;
+    const uint64_t list_bytes = splatad_align256((uint64_t)n_isects * 16);
+    const uint64_t cum_bytes = splatad_align256(total * 8);
+    if (w) { w->cum_before = (int64_t *)p; w->entries = (uint4 *)p; }
+    p += list_bytes > cum_bytes ? list_bytes : cum_bytes;
+    if (w) w->pairs = (uint64_t *)p;
+    p += splatad_align256((uint64_t)n_isects * 8);
+    return (size_t)(p - (char *)lists);
+}
+
+static size_t isect_ws_bytes(uint64_t total, uint64_t segs) {
     // there are at most as many coarse blocks as tiles, and coarse_workgroups() keeps the
     // table at 2^19 entries unless 64 rows exceed that
     const uint64_t cslots_bound = segs * 64 > (1ull << 19) ? segs * 64 : (1ull << 19);
-    return carve_isect(nullptr, total, segs, cslots_bound, n_isects, nullptr);
+    return carve_isect(nullptr, total, segs, cslots_bound, nullptr);
 }
 
 static inline dim3 grid_for(uint64_t n) {
     return dim3((uint32_t)((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS));
 }
 
-template <bool LIDAR>
-static int isect_count(TileGrid g, uint64_t total, const float *means2d, const void *radii,
-                       uint32_t C, int32_t *tiles_per_gauss, void *workspace,
-                       int64_t *n_isects_host, hipStream_t stream) {
-    SPLATAD_REQUIRE(n_isects_host != nullptr, "isect: n_isects_host is null");
-    *n_isects_host = 0;
-    if (total == 0) return 0;
-    SPLATAD_REQUIRE(total < (1ull << 31), "isect: number of projected Gaussians must be below 2^31");
-    SPLATAD_REQUIRE(means2d && radii && tiles_per_gauss && workspace, "isect: null pointer argument");
-    const uint32_t n_tiles = g.tile_w * g.tile_h;
-    SPLATAD_REQUIRE(n_tiles > 0 && C > 0, "isect: empty tile grid");
-    SPLATAD_REQUIRE(splatad_bit_width(n_tiles) + splatad_bit_width(C) <= 32,
-                    "isect: camera and tile ids need more than 32 bits");
-    IsectWorkspace w;
-    carve_isect(workspace, total, (uint64_t)C * n_tiles, 0, 0, &w);
-    hipLaunchKernelGGL(fill_zero_u64_kernel, dim3(1), dim3(1), 0, stream, w.n_isects);
-    dim3 count_grid = grid_for(total);
-    if (count_grid.x > 512) count_grid.x = 512;
-    hipLaunchKernelGGL(isect_count_kernel<LIDAR>, count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
-                       total, means2d, radii, tiles_per_gauss, w.n_isects);
-    SPLATAD_LAUNCH_CHECK();
-    unsigned long long n = 0;
-    SPLATAD_CHECK_HIP(hipMemcpyAsync(&n, w.n_isects, sizeof(n), hipMemcpyDeviceToHost, stream));
-    SPLATAD_CHECK_HIP(hipStreamSynchronize(stream));
-    SPLATAD_REQUIRE(n < (1ull << 31), "isect: %llu intersections exceed the int32 offset range", n);
-    *n_isects_host = (int64_t)n;
-    return 0;
-}
-
-// Helper streams (default priority) and events of the segment sort, one set per device,
-// created at first use and kept for the life of the process.  `guard` serialises the
-// enqueueing of a fork .. join sequence, which shares the events.
-struct SortStreams {
+// Per device, created at first use and kept for the life of the process: the helper streams
+// (default priority) and events of the segment sort, and the pinned host slot through which
+// the number of intersections reaches the host.  `guard` serialises the
+// enqueueing of sequences that share them.
+struct IsectDevice {
     hipStream_t aux[2];
     hipEvent_t fork, join[2];
+    unsigned long long *n_host, *n_device; // pinned slot: host address, address for kernels
     std::mutex guard;
 };
 
-static int sort_streams(SortStreams **out) {
+static int isect_device(IsectDevice **out) {
     static std::mutex table_guard;
-    static SortStreams *table[64] = {};
+    static IsectDevice *table[64] = {};
     int dev = 0;
     SPLATAD_CHECK_HIP(hipGetDevice(&dev));
     SPLATAD_REQUIRE(dev >= 0 && dev < 64, "isect: device index %d out of range", dev);
     std::lock_guard<std::mutex> lock(table_guard);
     if (!table[dev]) {
-        SortStreams *s = new SortStreams();
+        IsectDevice *s = new IsectDevice();
         for (hipStream_t &a : s->aux) SPLATAD_CHECK_HIP(hipStreamCreateWithFlags(&a, hipStreamNonBlocking));
         SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->fork, hipEventDisableTiming));
         for (hipEvent_t &e : s->join) SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        SPLATAD_CHECK_HIP(hipHostMalloc((void **)&s->n_host, 64, hipHostMallocDefault));
+        SPLATAD_CHECK_HIP(hipHostGetDevicePointer((void **)&s->n_device, s->n_host, 0));
         table[dev] = s;
     }
     *out = table[dev];
     return 0;
 }
 
+// First stages of the binning, which need no list memory: clear the tile counters, count the
+// coarse lists and scan the counts (the table is stored [workgroup][block] and scanned
+// block-major, which makes a block's list contiguous).
 template <bool LIDAR>
-static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *camera_ids,
-                      const float *means2d, const void *radii, const float *depths, uint32_t C,
-                      int sort, int64_t n_isects, const int32_t *tiles_per_gauss,
-                      void *workspace, int64_t *isect_ids, int32_t *flatten_ids,
-                      int32_t *tile_offsets, hipStream_t stream) {
-    if (total == 0 || n_isects == 0) {
-        if (tile_offsets && sort && (uint64_t)C * g.tile_w * g.tile_h > 0) {
-            const uint64_t tiles = (uint64_t)C * g.tile_w * g.tile_h;
-            hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(tiles), dim3(SPLATAD_THREADS), 0,
-                               stream, tile_offsets, (int64_t)tiles);
-            SPLATAD_LAUNCH_CHECK();
-        }
-        return 0;
-    }
-    SPLATAD_REQUIRE(means2d && radii && depths && workspace && isect_ids && flatten_ids,
-                    "isect: null pointer argument");
-    SPLATAD_REQUIRE(camera_ids != nullptr || N > 0, "isect: N is zero for unpacked input");
-    const uint32_t n_tiles = g.tile_w * g.tile_h;
-    const uint32_t tile_n_bits = splatad_bit_width(n_tiles);
-    const uint64_t segs = (uint64_t)C * n_tiles;
-    const CoarseGrid cg = coarse_grid<LIDAR>(g);
-    const uint64_t blocks = (uint64_t)C * cg.cw * cg.ch;
-    const uint32_t coarse_wgs = coarse_workgroups(total, blocks);
-    const uint64_t cslots = blocks * coarse_wgs;
-    IsectWorkspace w;
-    carve_isect(workspace, total, segs, sort ? cslots : 0, n_isects, &w);
-    int rc;
-    if (!sort) {
-        SPLATAD_REQUIRE(tiles_per_gauss != nullptr, "isect: tiles_per_gauss is null");
-        rc = launch_exclusive_scan<int64_t>(tiles_per_gauss, (int64_t)total, 1, 0, w.cum_before,
-                                            w.scan_total, w.block_sums, stream);
-        if (rc) return rc;
-        hipLaunchKernelGGL(isect_emit_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
-                           stream, g, total, N, camera_ids, means2d, radii, depths,
-                           (const int64_t *)w.cum_before, tile_n_bits, isect_ids, flatten_ids);
-        SPLATAD_LAUNCH_CHECK();
-        return 0;
-    }
-    const uint32_t per_cam = cg.cw * cg.ch;
-    SPLATAD_REQUIRE(per_cam <= kCoarseLdsBlocks, "isect: %u x %u tiles per sensor exceed the "
+static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const IsectWorkspace &w,
+                                uint64_t total, uint32_t N, const int64_t *camera_ids,
+                                const float *means2d, const void *radii, uint32_t C,
+                                hipStream_t stream) {
+    SPLATAD_REQUIRE(pl.per_cam <= kCoarseLdsBlocks, "isect: %u x %u tiles per sensor exceed the "
                     "binning capacity", g.tile_w, g.tile_h);
-    SPLATAD_REQUIRE(blocks < (1ull << 31) && cslots < (1ull << 31), "isect: tile grid too large");
-    const uint32_t cams_per_launch = kCoarseLdsBlocks / per_cam;
+    SPLATAD_REQUIRE(pl.blocks < (1ull << 31) && pl.cslots < (1ull << 31), "isect: tile grid too large");
     {
         static std::mutex guard;
         static bool raised = false;
@@ -948,25 +989,114 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     }
     hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(w.n_zeroed), dim3(SPLATAD_THREADS), 0, stream,
                        w.zeroed, (int64_t)w.n_zeroed);
-    // coarse lists: count, scan (the table is stored [workgroup][block] and scanned
-    // block-major, which makes a block's list contiguous), fill
-    for (uint32_t c0 = 0; c0 < C; c0 += cams_per_launch) {
-        const uint32_t c1 = C - c0 < cams_per_launch ? C : c0 + cams_per_launch;
-        hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, false>), dim3(coarse_wgs),
-                           dim3(kCoarseThreads), (size_t)(c1 - c0) * per_cam * 4, stream, g, cg,
-                           total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)blocks,
-                           w.coarse_counts, (uint4 *)nullptr);
+    for (uint32_t c0 = 0; c0 < C; c0 += pl.cams_per_launch) {
+        const uint32_t c1 = C - c0 < pl.cams_per_launch ? C : c0 + pl.cams_per_launch;
+        hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, false>), dim3(pl.coarse_wgs),
+                           dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, pl.cg,
+                           total, N, camera_ids, means2d, radii, (const float *)nullptr, c0, c1,
+                           (uint32_t)pl.blocks, w.coarse_counts, (uint4 *)nullptr);
     }
     SPLATAD_LAUNCH_CHECK();
-    rc = launch_exclusive_scan<int32_t>(w.coarse_counts, (int64_t)cslots,
-                                        coarse_wgs > 1 ? -(int)coarse_wgs : 1, 0, w.coarse_starts,
-                                        w.n_entries, w.block_sums, stream);
-    if (rc) return rc;
-    for (uint32_t c0 = 0; c0 < C; c0 += cams_per_launch) {
-        const uint32_t c1 = C - c0 < cams_per_launch ? C : c0 + cams_per_launch;
-        hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, true>), dim3(coarse_wgs),
-                           dim3(kCoarseThreads), (size_t)(c1 - c0) * per_cam * 4, stream, g, cg,
-                           total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)blocks,
+    return launch_exclusive_scan<int32_t>(w.coarse_counts, (int64_t)pl.cslots,
+                                          pl.coarse_wgs > 1 ? -(int)pl.coarse_wgs : 1, 0,
+                                          w.coarse_starts, w.n_entries, w.block_sums, stream);
+}
+
+template <bool LIDAR>
+static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *camera_ids,
+                       const float *means2d, const void *radii, uint32_t C, int sort,
+                       int32_t *tiles_per_gauss, void *workspace, int64_t *n_isects_host,
+                       hipStream_t stream) {
+    SPLATAD_REQUIRE(n_isects_host != nullptr, "isect: n_isects_host is null");
+    *n_isects_host = 0;
+    if (total == 0) return 0;
+    SPLATAD_REQUIRE(total < (1ull << 31), "isect: number of projected Gaussians must be below 2^31");
+    SPLATAD_REQUIRE(means2d && radii && tiles_per_gauss && workspace, "isect: null pointer argument");
+    SPLATAD_REQUIRE(camera_ids != nullptr || N > 0, "isect: N is zero for unpacked input");
+    const IsectPlan pl = isect_plan<LIDAR>(g, total, C);
+    SPLATAD_REQUIRE(pl.n_tiles > 0 && C > 0, "isect: empty tile grid");
+    SPLATAD_REQUIRE(pl.tile_n_bits + splatad_bit_width(C) <= 32,
+                    "isect: camera and tile ids need more than 32 bits");
+    IsectWorkspace w;
+    carve_isect(workspace, total, pl.segs, sort ? pl.cslots : 0, &w);
+    IsectDevice *dv = nullptr;
+    if (int rc = isect_device(&dv)) return rc;
+    std::lock_guard<std::mutex> lock(dv->guard);
+    volatile unsigned long long *slot = dv->n_host;
+    const unsigned long long pending = ~0ull;
+    *slot = pending;
+    hipLaunchKernelGGL(fill_zero_u64_kernel, dim3(1), dim3(2), 0, stream, w.n_isects);
+    dim3 count_grid = grid_for(total);
+    if (count_grid.x > 512) count_grid.x = 512;
+    hipLaunchKernelGGL(isect_count_kernel<LIDAR>, count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
+                       total, means2d, radii, tiles_per_gauss, w.n_isects, dv->n_device);
+    SPLATAD_LAUNCH_CHECK();
+    // work for the GPU while the host learns the count and sizes the lists
+    if (sort)
+        if (int rc = enqueue_coarse_count<LIDAR>(g, pl, w, total, N, camera_ids, means2d, radii, C, stream))
+            return rc;
+    // wait for the counting kernel's word only, not for the work behind it; now and then ask
+    // the stream, so that a failed launch or a fault ends the wait with its error
+    unsigned long long n = pending;
+    for (uint32_t spin = 1; (n = *slot) == pending; ++spin) {
+        __builtin_ia32_pause();
+        if ((spin & 0xFFFFu) == 0) {
+            const hipError_t q = hipStreamQuery(stream);
+            if (q == hipErrorNotReady) { (void)hipGetLastError(); continue; }
+            SPLATAD_CHECK_HIP(q);
+            n = *slot; // the stream has drained: the word is there, or never will be
+            SPLATAD_REQUIRE(n != pending, "isect: the counting kernel left no result");
+            break;
+        }
+    }
+    SPLATAD_REQUIRE(n < (1ull << 31), "isect: %llu intersections exceed the int32 offset range", n);
+    *n_isects_host = (int64_t)n;
+    return 0;
+}
+
+template <bool LIDAR>
+static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *camera_ids,
+                      const float *means2d, const void *radii, const float *depths, uint32_t C,
+                      int sort, int64_t n_isects, const int32_t *tiles_per_gauss,
+                      void *workspace, void *lists, int64_t *isect_ids, int32_t *flatten_ids,
+                      int32_t *tile_offsets, hipStream_t stream) {
+    if (total == 0 || n_isects == 0) {
+        if (tile_offsets && sort && (uint64_t)C * g.tile_w * g.tile_h > 0) {
+            const uint64_t tiles = (uint64_t)C * g.tile_w * g.tile_h;
+            hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(tiles), dim3(SPLATAD_THREADS), 0,
+                               stream, tile_offsets, (int64_t)tiles);
+            SPLATAD_LAUNCH_CHECK();
+        }
+        return 0;
+    }
+    SPLATAD_REQUIRE(means2d && radii && depths && workspace && lists && isect_ids && flatten_ids,
+                    "isect: null pointer argument");
+    SPLATAD_REQUIRE(camera_ids != nullptr || N > 0, "isect: N is zero for unpacked input");
+    const IsectPlan pl = isect_plan<LIDAR>(g, total, C);
+    const uint32_t n_tiles = pl.n_tiles, tile_n_bits = pl.tile_n_bits;
+    const uint64_t segs = pl.segs;
+    const CoarseGrid cg = pl.cg;
+    IsectWorkspace w;
+    carve_isect(workspace, total, segs, sort ? pl.cslots : 0, &w);
+    carve_lists(lists, total, n_isects, &w);
+    int rc;
+    if (!sort) {
+        SPLATAD_REQUIRE(tiles_per_gauss != nullptr, "isect: tiles_per_gauss is null");
+        rc = launch_exclusive_scan<int64_t>(tiles_per_gauss, (int64_t)total, 1, 0, w.cum_before,
+                                            w.scan_total, w.block_sums, stream);
+        if (rc) return rc;
+        hipLaunchKernelGGL(isect_emit_kernel<LIDAR>, grid_for(total), dim3(SPLATAD_THREADS), 0,
+                           stream, g, total, N, camera_ids, means2d, radii, depths,
+                           (const int64_t *)w.cum_before, tile_n_bits, isect_ids, flatten_ids);
+        SPLATAD_LAUNCH_CHECK();
+        return 0;
+    }
+    // the coarse lists were counted and scanned by the counting call; fill them
+    for (uint32_t c0 = 0; c0 < C; c0 += pl.cams_per_launch) {
+        const uint32_t c1 = C - c0 < pl.cams_per_launch ? C : c0 + pl.cams_per_launch;
+        hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, true>), dim3(pl.coarse_wgs),
+                           dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, cg,
+                           total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)pl.blocks,
                            w.coarse_starts, w.entries);
     }
     SPLATAD_LAUNCH_CHECK();
@@ -995,29 +1125,32 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
                        w.tile_counts, (const int32_t *)w.tile_starts, w.tile_fill, w.pairs);
     SPLATAD_LAUNCH_CHECK();
-    // Size classes: each launch visits every segment and only works on those of its class, so
-    // that the LDS per workgroup (and with it the number of resident workgroups) fits the
-    // segment length.  The classes touch disjoint segments; they run on two helper streams
-    // beside the caller's, forked and joined with events, so that the few long workgroups
-    // of the upper classes overlap the many short ones of the lower classes.
+    // Size classes: one launch per class, so that the LDS per workgroup (and with it the number
+    // of resident workgroups) fits the segment length; the segments of a class come from a list
+    // made on the device.  The classes touch disjoint segments; they run on two helper streams
+    // beside the caller's, forked and joined with events, so that the few long workgroups of the
+    // upper classes overlap the many short ones of the lower classes.
     const uint32_t nseg = (uint32_t)segs;
-    SortStreams *ss = nullptr;
-    if ((rc = sort_streams(&ss)) != 0) return rc;
+    hipLaunchKernelGGL(isect_classify_segments_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream,
+                       nseg, n_isects, (const int32_t *)w.tile_starts, w.seg_counts, w.seg_lists);
+    SPLATAD_LAUNCH_CHECK();
+    IsectDevice *ss = nullptr;
+    if ((rc = isect_device(&ss)) != 0) return rc;
     std::lock_guard<std::mutex> fork_lock(ss->guard);
     SPLATAD_CHECK_HIP(hipEventRecord(ss->fork, stream));
     for (hipStream_t aux : ss->aux) SPLATAD_CHECK_HIP(hipStreamWaitEvent(aux, ss->fork, 0));
-#define SPLATAD_SORT_CLASS(ER, IN_LDS, threads, lo, hi, on)                                      \
-    if ((rc = launch_segment_sort<ER, IN_LDS>(threads, lo, hi, nseg, n_tiles, tile_n_bits,        \
-                                              n_isects, w.tile_starts, w.pairs, isect_ids,        \
-                                              flatten_ids, on)) != 0)                             \
+#define SPLATAD_SORT_CLASS(cls, ER, IN_LDS, threads, hi, wgs, on)                                \
+    if ((rc = launch_segment_sort<ER, IN_LDS>(cls, threads, hi, wgs, nseg, n_tiles, tile_n_bits,  \
+                                              n_isects, w.seg_counts, w.seg_lists, w.tile_starts, \
+                                              w.pairs, isect_ids, flatten_ids, on)) != 0)         \
         return rc;
-    SPLATAD_SORT_CLASS(32, false, 1024, 16384u, 32768u, ss->aux[0])
-    SPLATAD_SORT_CLASS(0, false, 1024, 32768u, 0x7FFFFFFFu, ss->aux[0])
-    SPLATAD_SORT_CLASS(16, true, 1024, 8192u, 16384u, ss->aux[1])
-    SPLATAD_SORT_CLASS(8, true, 1024, 4096u, 8192u, ss->aux[1])
-    SPLATAD_SORT_CLASS(8, true, 512, 2048u, 4096u, stream)
-    SPLATAD_SORT_CLASS(8, true, 256, 512u, 2048u, stream)
-    SPLATAD_SORT_CLASS(4, true, 128, 0u, 512u, stream)
+    SPLATAD_SORT_CLASS(5, 32, false, 1024, 32768u, 256u, ss->aux[0])
+    SPLATAD_SORT_CLASS(6, 0, false, 1024, 0x7FFFFFFFu, 256u, ss->aux[0])
+    SPLATAD_SORT_CLASS(4, 16, true, 1024, 16384u, 256u, ss->aux[1])
+    SPLATAD_SORT_CLASS(3, 8, true, 1024, 8192u, 512u, ss->aux[1])
+    SPLATAD_SORT_CLASS(2, 8, true, 512, 4096u, 1024u, stream)
+    SPLATAD_SORT_CLASS(1, 8, true, 256, 2048u, 2048u, stream)
+    SPLATAD_SORT_CLASS(0, 4, true, 128, 512u, 4096u, stream)
 #undef SPLATAD_SORT_CLASS
     for (int k = 0; k < 2; ++k) {
         SPLATAD_CHECK_HIP(hipEventRecord(ss->join[k], ss->aux[k]));
@@ -1029,20 +1162,24 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
 
 } // namespace
 
-extern "C" size_t splatad_isect_workspace_bytes(uint64_t total, uint32_t C, uint32_t n_tiles,
-                                                int64_t n_isects) {
-    return isect_ws_bytes(total, (uint64_t)C * n_tiles, n_isects < 0 ? 0 : n_isects);
+extern "C" size_t splatad_isect_workspace_bytes(uint64_t total, uint32_t C, uint32_t n_tiles) {
+    return isect_ws_bytes(total, (uint64_t)C * n_tiles);
 }
 
-extern "C" int splatad_isect_tiles_count(uint64_t total, const float *means2d,
-                                         const int32_t *radii, uint32_t C, uint32_t tile_size,
-                                         uint32_t tile_width, uint32_t tile_height,
-                                         int32_t *tiles_per_gauss, void *workspace,
-                                         int64_t *n_isects_host, splatad_stream_t stream) {
+extern "C" size_t splatad_isect_lists_bytes(uint64_t total, int64_t n_isects) {
+    return carve_lists(nullptr, total, n_isects < 0 ? 0 : n_isects, nullptr);
+}
+
+extern "C" int splatad_isect_tiles_count(uint64_t total, uint32_t N, const int64_t *camera_ids,
+                                         const float *means2d, const int32_t *radii, uint32_t C,
+                                         uint32_t tile_size, uint32_t tile_width,
+                                         uint32_t tile_height, int sort, int32_t *tiles_per_gauss,
+                                         void *workspace, int64_t *n_isects_host,
+                                         splatad_stream_t stream) {
     SPLATAD_REQUIRE(tile_size > 0, "isect_tiles: tile_size is zero");
     TileGrid g{tile_size, tile_width, tile_height, 0.f, 0.f, nullptr};
-    return isect_count<false>(g, total, means2d, radii, C, tiles_per_gauss, workspace,
-                              n_isects_host, (hipStream_t)stream);
+    return isect_count<false>(g, total, N, camera_ids, means2d, radii, C, sort, tiles_per_gauss,
+                              workspace, n_isects_host, (hipStream_t)stream);
 }
 
 extern "C" int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_ids,
@@ -1050,26 +1187,28 @@ extern "C" int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_
                                         const float *depths, uint32_t C, uint32_t tile_size,
                                         uint32_t tile_width, uint32_t tile_height, int sort,
                                         int64_t n_isects, const int32_t *tiles_per_gauss,
-                                        void *workspace, int64_t *isect_ids, int32_t *flatten_ids,
-                                        int32_t *tile_offsets, splatad_stream_t stream) {
+                                        void *workspace, void *lists, int64_t *isect_ids,
+                                        int32_t *flatten_ids, int32_t *tile_offsets,
+                                        splatad_stream_t stream) {
     SPLATAD_REQUIRE(tile_size > 0, "isect_tiles: tile_size is zero");
     TileGrid g{tile_size, tile_width, tile_height, 0.f, 0.f, nullptr};
     return isect_fill<false>(g, total, N, camera_ids, means2d, radii, depths, C, sort, n_isects,
-                             tiles_per_gauss, workspace, isect_ids, flatten_ids, tile_offsets,
-                             (hipStream_t)stream);
+                             tiles_per_gauss, workspace, lists, isect_ids, flatten_ids,
+                             tile_offsets, (hipStream_t)stream);
 }
 
-extern "C" int splatad_isect_lidar_tiles_count(uint64_t total, const float *means2d,
+extern "C" int splatad_isect_lidar_tiles_count(uint64_t total, uint32_t N,
+                                               const int64_t *camera_ids, const float *means2d,
                                                const float *radii, uint32_t C,
                                                const float *elev_boundaries,
                                                float tile_azim_resolution, float min_azim,
-                                               uint32_t tile_width, uint32_t tile_height,
+                                               uint32_t tile_width, uint32_t tile_height, int sort,
                                                int32_t *tiles_per_gauss, void *workspace,
                                                int64_t *n_isects_host, splatad_stream_t stream) {
     SPLATAD_REQUIRE(elev_boundaries != nullptr, "isect_lidar_tiles: elev_boundaries is null");
     TileGrid g{0u, tile_width, tile_height, tile_azim_resolution, min_azim, elev_boundaries};
-    return isect_count<true>(g, total, means2d, radii, C, tiles_per_gauss, workspace,
-                             n_isects_host, (hipStream_t)stream);
+    return isect_count<true>(g, total, N, camera_ids, means2d, radii, C, sort, tiles_per_gauss,
+                             workspace, n_isects_host, (hipStream_t)stream);
 }
 
 extern "C" int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N,
@@ -1079,13 +1218,13 @@ extern "C" int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N,
                                               float tile_azim_resolution, float min_azim,
                                               uint32_t tile_width, uint32_t tile_height, int sort,
                                               int64_t n_isects, const int32_t *tiles_per_gauss,
-                                              void *workspace, int64_t *isect_ids,
+                                              void *workspace, void *lists, int64_t *isect_ids,
                                               int32_t *flatten_ids, int32_t *tile_offsets,
                                               splatad_stream_t stream) {
     SPLATAD_REQUIRE(elev_boundaries != nullptr, "isect_lidar_tiles: elev_boundaries is null");
     TileGrid g{0u, tile_width, tile_height, tile_azim_resolution, min_azim, elev_boundaries};
     return isect_fill<true>(g, total, N, camera_ids, means2d, radii, depths, C, sort, n_isects,
-                            tiles_per_gauss, workspace, isect_ids, flatten_ids, tile_offsets,
+                            tiles_per_gauss, workspace, lists, isect_ids, flatten_ids, tile_offsets,
                             (hipStream_t)stream);
 }
 

@@ -90,19 +90,72 @@ __device__ __forceinline__ void sh_for_each_float(const ShRows &r, uint32_t rows
     }
 }
 
+// Where a kernel takes its directions, masks and coefficient rows from.  The plain operator
+// reads them from tensors; the rendering pipeline (VIEW) derives them from the scene: the
+// direction of row e is the Gaussian's mean minus the position of its sensor, the row is
+// active when the Gaussian's projected radius is positive, and the coefficient row is the
+// Gaussian's own unless every sensor has its own coefficients.  This replaces the inverse of
+// the view matrices, the gathers and the mask tensor of gsplat/rendering.py:325-345.
+struct ShView {
+    const float *means;                       // [N, 3]
+    const float *viewmats;                    // [C, 4, 4], rows [A | t], last row (0, 0, 0, 1)
+    const int64_t *camera_ids, *gaussian_ids; // per row for packed input, else null
+    const int32_t *radii;                     // [n, 2]
+    uint32_t N;
+    int coeffs_per_sensor; // coefficient rows: 1 = one per row e, 0 = one per Gaussian
+};
+
+// Position of the sensor in the world: the translation column of the inverse of [A | t], -A^-1 t.
+__device__ __forceinline__ void sensor_position(const float *vm, float &px, float &py, float &pz) {
+    const float a = vm[0], b = vm[1], c = vm[2], d = vm[4], e = vm[5], f = vm[6], g = vm[8], h = vm[9], i = vm[10];
+    const float tx = vm[3], ty = vm[7], tz = vm[11];
+    const float c00 = e * i - f * h, c01 = c * h - b * i, c02 = b * f - c * e;
+    const float c10 = f * g - d * i, c11 = a * i - c * g, c12 = c * d - a * f;
+    const float c20 = d * h - e * g, c21 = b * g - a * h, c22 = a * e - b * d;
+    const float inv_det = 1.f / (a * c00 + b * c10 + c * c20);
+    px = -(c00 * tx + c01 * ty + c02 * tz) * inv_det;
+    py = -(c10 * tx + c11 * ty + c12 * tz) * inv_det;
+    pz = -(c20 * tx + c21 * ty + c22 * tz) * inv_det;
+}
+
+// Direction, activity and coefficient row of row e
+template <bool VIEW>
+__device__ __forceinline__ bool sh_row(uint32_t e, const ShView &v, const float *dirs,
+                                       const uint8_t *masks, float &dx, float &dy, float &dz,
+                                       size_t &coeff_row) {
+    if (!VIEW) {
+        coeff_row = e;
+        if (masks != nullptr && !masks[e]) return false;
+        dx = dirs[(size_t)e * 3]; dy = dirs[(size_t)e * 3 + 1]; dz = dirs[(size_t)e * 3 + 2];
+        return true;
+    }
+    const uint32_t g = v.gaussian_ids ? (uint32_t)v.gaussian_ids[e] : e % v.N;
+    const uint32_t cam = v.camera_ids ? (uint32_t)v.camera_ids[e] : e / v.N;
+    coeff_row = v.coeffs_per_sensor ? (v.camera_ids ? (size_t)cam * v.N + g : (size_t)e) : (size_t)g;
+    if (v.radii[(size_t)e * 2] <= 0) return false;
+    float px, py, pz;
+    sensor_position(v.viewmats + (size_t)cam * 16, px, py, pz);
+    dx = v.means[(size_t)g * 3] - px; dy = v.means[(size_t)g * 3 + 1] - py; dz = v.means[(size_t)g * 3 + 2] - pz;
+    return true;
+}
+
 // Forward: every lane reads its own row; the rows are read completely, so the cache lines a
-// wavefront touches are all used (measured faster than staging through LDS).
+// wavefront touches are all used (measured faster than staging through LDS).  VIEW also
+// applies the colour activation of the pipeline, max(c + 1/2, 0) (gsplat/rendering.py:347),
+// and writes rows of `stride` floats, with the depth as fourth channel when given (:351).
+template <bool VIEW>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
-sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, const float *__restrict__ dirs,
+sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, ShView view, const float *__restrict__ dirs,
               const float *__restrict__ coeffs, const uint8_t *__restrict__ masks,
-              float *__restrict__ colors) {
+              const float *__restrict__ depths, uint32_t stride, float *__restrict__ colors) {
     const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= n) return;
     float r = 0.f, g = 0.f, b = 0.f;
-    if (masks == nullptr || masks[e]) {
-        const float dx = dirs[(size_t)e * 3], dy = dirs[(size_t)e * 3 + 1], dz = dirs[(size_t)e * 3 + 2];
+    float dx = 0.f, dy = 0.f, dz = 0.f;
+    size_t coeff_row;
+    if (sh_row<VIEW>(e, view, dirs, masks, dx, dy, dz, coeff_row)) {
         const float inorm = rsqrtf(dx * dx + dy * dy + dz * dz);
-        const float *cf = coeffs + (size_t)e * K * 3;
+        const float *cf = coeffs + coeff_row * K * 3;
         sh_for_each_basis(degree, dx * inorm, dy * inorm, dz * inorm,
                           [&](int k, float v, float, float, float) {
                               r += v * cf[k * 3];
@@ -110,14 +163,24 @@ sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, const float *__restrict__
                               b += v * cf[k * 3 + 2];
                           });
     }
-    colors[(size_t)e * 3] = r;
-    colors[(size_t)e * 3 + 1] = g;
-    colors[(size_t)e * 3 + 2] = b;
+    float *out = colors + (size_t)e * stride;
+    if (VIEW) {
+        out[0] = fmaxf(r + 0.5f, 0.f);
+        out[1] = fmaxf(g + 0.5f, 0.f);
+        out[2] = fmaxf(b + 0.5f, 0.f);
+        if (depths != nullptr) out[3] = depths[e];
+    } else {
+        out[0] = r; out[1] = g; out[2] = b;
+    }
 }
 
+// VIEW: v_colors are rows of `stride` floats, the gradients of the activated colours
+// `colors` (same layout), so a channel passes its gradient on only where it is positive.
+template <bool VIEW>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
-sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, const float *__restrict__ dirs,
+sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, ShView view, const float *__restrict__ dirs,
               const float *__restrict__ coeffs, const uint8_t *__restrict__ masks,
+              const float *__restrict__ colors, uint32_t stride,
               const float *__restrict__ v_colors, float *__restrict__ v_coeffs,
               float *__restrict__ v_dirs) {
     extern __shared__ float s_rows[];
@@ -128,16 +191,21 @@ sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, const float *__restrict_
     // every lane writes its row of coefficient gradients to LDS, from where the workgroup
     // stores them coalesced; rows of masked directions are zeros (their gradients are zero)
     float *row = s_rows + (size_t)threadIdx.x * (rows.used + 1);
-    const float *cf = coeffs + (size_t)min(e, n - 1) * rows.K3;
     if (e < n) {
-        const bool active = masks == nullptr || masks[e];
-        const float dx = active ? dirs[(size_t)e * 3] : 0.f, dy = active ? dirs[(size_t)e * 3 + 1] : 0.f;
-        const float dz = active ? dirs[(size_t)e * 3 + 2] : 0.f;
+        float dx = 0.f, dy = 0.f, dz = 0.f;
+        size_t coeff_row;
+        const bool active = sh_row<VIEW>(e, view, dirs, masks, dx, dy, dz, coeff_row);
+        const float *cf = coeffs + coeff_row * rows.K3;
         const float inorm = active ? rsqrtf(dx * dx + dy * dy + dz * dz) : 0.f;
         const float x = dx * inorm, y = dy * inorm, z = active ? dz * inorm : 1.f;
-        const float vr = active ? v_colors[(size_t)e * 3] : 0.f;
-        const float vg = active ? v_colors[(size_t)e * 3 + 1] : 0.f;
-        const float vb = active ? v_colors[(size_t)e * 3 + 2] : 0.f;
+        const float *vc = v_colors + (size_t)e * stride;
+        float vr = active ? vc[0] : 0.f, vg = active ? vc[1] : 0.f, vb = active ? vc[2] : 0.f;
+        if (VIEW) {
+            const float *c = colors + (size_t)e * stride;
+            vr = c[0] > 0.f ? vr : 0.f;
+            vg = c[1] > 0.f ? vg : 0.f;
+            vb = c[2] > 0.f ? vb : 0.f;
+        }
         float gx = 0.f, gy = 0.f, gz = 0.f;
         sh_for_each_basis(degree, x, y, z, [&](int k, float v, float bx, float by, float bz) {
             if (want_dirs) {
@@ -148,8 +216,8 @@ sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, const float *__restrict_
             row[k * 3 + 1] = v * vg;
             row[k * 3 + 2] = v * vb;
         });
-        if (want_dirs && active) {
-            // through the normalisation: (I - n n^T) g / |d|
+        if (want_dirs && (active || VIEW)) {
+            // through the normalisation: (I - n n^T) g / |d|; zero for inactive rows
             const float dot = gx * x + gy * y + gz * z;
             v_dirs[(size_t)e * 3] = (gx - dot * x) * inorm;
             v_dirs[(size_t)e * 3 + 1] = (gy - dot * y) * inorm;
@@ -179,35 +247,103 @@ static int sh_lds(Kernel kernel, const ShRows &r, size_t *bytes) {
     return 0;
 }
 
+static int sh_check(uint32_t K, uint32_t degree) {
+    SPLATAD_REQUIRE(degree <= 4, "spherical harmonics: degree %u is above 4", degree);
+    SPLATAD_REQUIRE((degree + 1) * (degree + 1) <= K, "spherical harmonics: %u bases for degree %u", K, degree);
+    return 0;
+}
+
+template <bool VIEW>
+static int sh_forward(uint32_t n, uint32_t K, uint32_t degree, const ShView &view, const float *dirs,
+                      const float *coeffs, const uint8_t *masks, const float *depths,
+                      uint32_t stride, float *colors, hipStream_t stream) {
+    hipLaunchKernelGGL(sh_fwd_kernel<VIEW>, dim3((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS),
+                       dim3(SPLATAD_THREADS), 0, stream, n, K, degree, view, dirs, coeffs, masks,
+                       depths, stride, colors);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
+}
+
+template <bool VIEW>
+static int sh_backward(uint32_t n, uint32_t K, uint32_t degree, const ShView &view, const float *dirs,
+                       const float *coeffs, const uint8_t *masks, const float *colors,
+                       uint32_t stride, const float *v_colors, float *v_coeffs, float *v_dirs,
+                       hipStream_t stream) {
+    const ShRows r = sh_rows(K, degree);
+    size_t lds = 0;
+    if (int rc = sh_lds(sh_bwd_kernel<VIEW>, r, &lds)) return rc;
+    hipLaunchKernelGGL(sh_bwd_kernel<VIEW>, dim3((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS),
+                       dim3(SPLATAD_THREADS), lds, stream, n, r, degree, view, dirs, coeffs, masks,
+                       colors, stride, v_colors, v_coeffs, v_dirs);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
+}
+
+static int sh_view_args(uint32_t n, uint32_t C, uint32_t N, const float *means, const float *viewmats,
+                        const int64_t *camera_ids, const int64_t *gaussian_ids, const int32_t *radii,
+                        int coeffs_per_sensor, ShView *view) {
+    SPLATAD_REQUIRE(means && viewmats && radii, "view colours: null pointer argument");
+    SPLATAD_REQUIRE((camera_ids == nullptr) == (gaussian_ids == nullptr),
+                    "view colours: camera_ids and gaussian_ids go together");
+    SPLATAD_REQUIRE(N > 0 && C > 0, "view colours: no Gaussians or no sensors");
+    SPLATAD_REQUIRE(camera_ids != nullptr || (uint64_t)n == (uint64_t)C * N,
+                    "view colours: %u rows for %u sensors x %u Gaussians", n, C, N);
+    *view = ShView{means, viewmats, camera_ids, gaussian_ids, radii, N, coeffs_per_sensor};
+    return 0;
+}
+
 } // namespace
 
 extern "C" int splatad_sh_fwd(uint32_t n, uint32_t K, uint32_t degree, const float *dirs,
                               const float *coeffs, const uint8_t *masks, float *colors,
                               splatad_stream_t stream) {
-    SPLATAD_REQUIRE(degree <= 4, "spherical harmonics: degree %u is above 4", degree);
-    SPLATAD_REQUIRE((degree + 1) * (degree + 1) <= K, "spherical harmonics: %u bases for degree %u", K, degree);
+    if (int rc = sh_check(K, degree)) return rc;
     if (n == 0) return 0;
     SPLATAD_REQUIRE(dirs && coeffs && colors, "spherical harmonics: null pointer argument");
-    hipLaunchKernelGGL(sh_fwd_kernel, dim3((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS),
-                       dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, n, K, degree, dirs, coeffs,
-                       masks, colors);
-    SPLATAD_LAUNCH_CHECK();
-    return 0;
+    return sh_forward<false>(n, K, degree, ShView{}, dirs, coeffs, masks, nullptr, 3, colors,
+                             (hipStream_t)stream);
 }
 
 extern "C" int splatad_sh_bwd(uint32_t n, uint32_t K, uint32_t degree, const float *dirs,
                               const float *coeffs, const uint8_t *masks, const float *v_colors,
                               float *v_coeffs, float *v_dirs, splatad_stream_t stream) {
-    SPLATAD_REQUIRE(degree <= 4, "spherical harmonics: degree %u is above 4", degree);
-    SPLATAD_REQUIRE((degree + 1) * (degree + 1) <= K, "spherical harmonics: %u bases for degree %u", K, degree);
+    if (int rc = sh_check(K, degree)) return rc;
     if (n == 0) return 0;
     SPLATAD_REQUIRE(dirs && coeffs && v_colors && v_coeffs, "spherical harmonics: null pointer argument");
-    const ShRows r = sh_rows(K, degree);
-    size_t lds = 0;
-    if (int rc = sh_lds(sh_bwd_kernel, r, &lds)) return rc;
-    hipLaunchKernelGGL(sh_bwd_kernel, dim3((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS),
-                       dim3(SPLATAD_THREADS), lds, (hipStream_t)stream, n, r, degree, dirs, coeffs,
-                       masks, v_colors, v_coeffs, v_dirs);
-    SPLATAD_LAUNCH_CHECK();
-    return 0;
+    return sh_backward<false>(n, K, degree, ShView{}, dirs, coeffs, masks, nullptr, 3, v_colors,
+                              v_coeffs, v_dirs, (hipStream_t)stream);
+}
+
+extern "C" int splatad_view_colors_fwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K,
+                                       uint32_t degree, const float *means, const float *viewmats,
+                                       const int64_t *camera_ids, const int64_t *gaussian_ids,
+                                       const int32_t *radii, const float *coeffs,
+                                       int coeffs_per_sensor, const float *depths, float *colors,
+                                       splatad_stream_t stream) {
+    if (int rc = sh_check(K, degree)) return rc;
+    if (n == 0) return 0;
+    ShView view;
+    if (int rc = sh_view_args(n, C, N, means, viewmats, camera_ids, gaussian_ids, radii,
+                              coeffs_per_sensor, &view)) return rc;
+    SPLATAD_REQUIRE(coeffs && colors, "view colours: null pointer argument");
+    return sh_forward<true>(n, K, degree, view, nullptr, coeffs, nullptr, depths, depths ? 4u : 3u,
+                            colors, (hipStream_t)stream);
+}
+
+extern "C" int splatad_view_colors_bwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K,
+                                       uint32_t degree, const float *means, const float *viewmats,
+                                       const int64_t *camera_ids, const int64_t *gaussian_ids,
+                                       const int32_t *radii, const float *coeffs,
+                                       int coeffs_per_sensor, uint32_t channels, const float *colors,
+                                       const float *v_colors, float *v_coeffs, float *v_dirs,
+                                       splatad_stream_t stream) {
+    if (int rc = sh_check(K, degree)) return rc;
+    if (n == 0) return 0;
+    ShView view;
+    if (int rc = sh_view_args(n, C, N, means, viewmats, camera_ids, gaussian_ids, radii,
+                              coeffs_per_sensor, &view)) return rc;
+    SPLATAD_REQUIRE(channels == 3 || channels == 4, "view colours: %u channels per row", channels);
+    SPLATAD_REQUIRE(coeffs && colors && v_colors && v_coeffs, "view colours: null pointer argument");
+    return sh_backward<true>(n, K, degree, view, nullptr, coeffs, nullptr, colors, channels, v_colors,
+                             v_coeffs, v_dirs, (hipStream_t)stream);
 }

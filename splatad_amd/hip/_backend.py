@@ -36,6 +36,7 @@ def load_library():
         lib.splatad_last_error.restype = ctypes.c_char_p
         lib.splatad_abi_version.restype = ctypes.c_int
         for name in ("splatad_projection_packed_workspace_bytes", "splatad_isect_workspace_bytes",
+                     "splatad_isect_lists_bytes",
                      "splatad_map_points_to_lidar_tiles_workspace_bytes",
                      "splatad_rasterize_to_indices_workspace_bytes"):
             getattr(lib, name).restype = ctypes.c_size_t
@@ -303,6 +304,51 @@ class _Ops:
                                       _stream(dev)))
         return v_coeffs, v_dirs
 
+    def view_colors_fwd(self, degrees_to_use, means, viewmats, camera_ids, gaussian_ids, radii,
+                        coeffs, depths):
+        """Colours max(SH(mean - sensor position) + 1/2, 0) per (sensor, Gaussian), with the
+        depth as fourth channel when given.  No counterpart among the reference's C++ ops: it
+        replaces the tensor operations of gsplat/rendering.py:325-351."""
+        lib = load_library()
+        means = _in(means, "means"); viewmats = _in(viewmats, "viewmats")
+        camera_ids = _in(camera_ids, "camera_ids", torch.int64)
+        gaussian_ids = _in(gaussian_ids, "gaussian_ids", torch.int64)
+        radii = _in(radii, "radii", torch.int32); coeffs = _in(coeffs, "coeffs")
+        depths = _in(depths, "depths")
+        C, N, dev = viewmats.shape[0], means.shape[0], means.device
+        lead = tuple(radii.shape[:-1])
+        n = int(math.prod(lead))
+        colors = torch.empty(lead + (4 if depths is not None else 3,), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_view_colors_fwd(
+                _u32(n), _u32(C), _u32(N), _u32(coeffs.shape[-2]), _u32(degrees_to_use), _p(means),
+                _p(viewmats), _p(camera_ids), _p(gaussian_ids), _p(radii), _p(coeffs),
+                _i32(coeffs.dim() == 4), _p(depths), _p(colors), _stream(dev)))
+        return colors
+
+    def view_colors_bwd(self, degrees_to_use, means, viewmats, camera_ids, gaussian_ids, radii,
+                        coeffs, colors, v_colors, compute_v_dirs):
+        """Per-row gradients (v_coeffs [..., K, 3], v_dirs [..., 3] | None) of view_colors_fwd."""
+        lib = load_library()
+        means = _in(means, "means"); viewmats = _in(viewmats, "viewmats")
+        camera_ids = _in(camera_ids, "camera_ids", torch.int64)
+        gaussian_ids = _in(gaussian_ids, "gaussian_ids", torch.int64)
+        radii = _in(radii, "radii", torch.int32); coeffs = _in(coeffs, "coeffs")
+        colors = _in(colors, "colors"); v_colors = _in(v_colors, "v_colors")
+        C, N, dev = viewmats.shape[0], means.shape[0], means.device
+        lead = tuple(radii.shape[:-1])
+        n, K = int(math.prod(lead)), coeffs.shape[-2]
+        f = dict(dtype=torch.float32, device=dev)
+        v_coeffs = torch.zeros(lead + (K, 3), **f)
+        v_dirs = torch.empty(lead + (3,), **f) if compute_v_dirs else None
+        with torch.cuda.device(dev):
+            _check(lib.splatad_view_colors_bwd(
+                _u32(n), _u32(C), _u32(N), _u32(K), _u32(degrees_to_use), _p(means), _p(viewmats),
+                _p(camera_ids), _p(gaussian_ids), _p(radii), _p(coeffs), _i32(coeffs.dim() == 4),
+                _u32(colors.shape[-1]), _p(colors), _p(v_colors), _p(v_coeffs), _p(v_dirs),
+                _stream(dev)))
+        return v_coeffs, v_dirs
+
     # ------------------------------------------------------------------ intersection
     def _isect(self, lidar, means2d, radii, depths, camera_ids, gaussian_ids, C, grid_args,
                tile_w, tile_h, sort):
@@ -327,26 +373,26 @@ class _Ops:
         count = lib.splatad_isect_lidar_tiles_count if lidar else lib.splatad_isect_tiles_count
         fill = lib.splatad_isect_lidar_tiles_fill if lidar else lib.splatad_isect_tiles_fill
         with torch.cuda.device(dev):
-            ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(total), _u32(C), _u32(n_tiles),
-                                                              _i64(0)), dev)
+            # one workspace for both calls: the counting call leaves the start of the binning in it
+            ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(total), _u32(C), _u32(n_tiles)), dev)
+            # the binning knows every tile's first intersection: keep that table with the
+            # ids so that isect_offset_encode() on the same, unmodified tensor is free
+            offsets = (torch.empty((C, tile_h, tile_w), dtype=torch.int32, device=dev)
+                       if sort else None)
+            head = (_u64(total), _u32(N), _p(camera_ids), _p(means2d), _p(radii))
+            tail = (_u32(C), *grid_args, _u32(tile_w), _u32(tile_h), _i32(bool(sort)))
             n_host = _i64(0)
-            _check(count(_u64(total), _p(means2d), _p(radii), _u32(C), *grid_args, _u32(tile_w),
-                         _u32(tile_h), _p(tiles_per_gauss), _p(ws), ctypes.byref(n_host),
+            _check(count(*head, *tail, _p(tiles_per_gauss), _p(ws), ctypes.byref(n_host),
                          _stream(dev)))
             n_isects = int(n_host.value)
             isect_ids = torch.empty((n_isects,), dtype=torch.int64, device=dev)
             flatten_ids = torch.empty((n_isects,), dtype=torch.int32, device=dev)
-            # the binning knows every tile's first intersection: keep that table with the
-            # ids so that isect_offset_encode() on the same, unmodified tensor is free
-            offsets = (torch.empty((C, tile_h, tile_w), dtype=torch.int32, device=dev)
-                       if sort and n_isects else None)
             if n_isects:
-                ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(total), _u32(C),
-                                                                  _u32(n_tiles), _i64(n_isects)), dev)
-                _check(fill(_u64(total), _u32(N), _p(camera_ids), _p(means2d), _p(radii),
-                            _p(depths), _u32(C), *grid_args, _u32(tile_w), _u32(tile_h),
-                            _i32(bool(sort)), _i64(n_isects), _p(tiles_per_gauss), _p(ws),
-                            _p(isect_ids), _p(flatten_ids), _p(offsets), _stream(dev)))
+                lists = _workspace(lib.splatad_isect_lists_bytes(_u64(total), _i64(n_isects)), dev)
+                _check(fill(*head, _p(depths), *tail, _i64(n_isects), _p(tiles_per_gauss), _p(ws),
+                            _p(lists), _p(isect_ids), _p(flatten_ids), _p(offsets), _stream(dev)))
+            else:
+                offsets = None
             if offsets is not None:
                 isect_ids._splatad_tile_offsets = (offsets, isect_ids._version)
         return tiles_per_gauss, isect_ids, flatten_ids

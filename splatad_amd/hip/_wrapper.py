@@ -9,6 +9,7 @@ all on the permissive side:
   * the fused projections return a gradient for per-Gaussian `velocities` (the reference
     computes it and drops it, gsplat/cuda/csrc/projection.cu:874-877).
 """
+import contextlib
 from typing import Callable, Optional, Tuple
 
 import torch
@@ -64,6 +65,51 @@ def spherical_harmonics(
         assert masks.shape == dirs.shape[:-1], masks.shape
         masks = masks.contiguous()
     return _SphericalHarmonics.apply(degrees_to_use, dirs.contiguous(), coeffs.contiguous(), masks)
+
+
+def view_dependent_colors(
+    degrees_to_use: int,
+    means: Tensor,  # [N, 3]
+    viewmats: Tensor,  # [C, 4, 4]
+    coeffs: Tensor,  # [N, K, 3] or [C, N, K, 3]
+    radii: Tensor,  # [C, N, 2] or [nnz, 2], int32
+    depths: Optional[Tensor] = None,  # [C, N] or [nnz]
+    camera_ids: Optional[Tensor] = None,  # [nnz]
+    gaussian_ids: Optional[Tensor] = None,  # [nnz]
+    launch_context=None,
+) -> Tensor:
+    """Activated view-dependent colours of every (sensor, Gaussian) pair in one kernel:
+    max(SH(mean - sensor position) + 1/2, 0) for pairs with a positive projected radius
+    (1/2 for the others), with `depths` appended as fourth channel when given.  Same values as
+    inverting the view matrices, forming the directions and masks, `spherical_harmonics`,
+    the activation and the concatenation (gsplat/rendering.py:325-351 of the reference),
+    without materialising any of them.  Differentiable in `means`, `coeffs` and `depths`;
+    `viewmats` are treated as constants (rows [A | t], last row (0, 0, 0, 1)).
+    `launch_context`, if given, is a context manager entered around the forward kernel launch
+    only (e.g. a helper stream); the autograd node, and with it the backward pass, stays on the
+    caller's stream.
+
+    Returns [C, N, 3 or 4], or [nnz, 3 or 4] for packed input.
+    """
+    N, C = means.shape[0], viewmats.shape[0]
+    packed = radii.dim() == 2
+    assert means.shape == (N, 3), means.shape
+    assert viewmats.shape == (C, 4, 4), viewmats.shape
+    assert coeffs.shape[-1] == 3 and (degrees_to_use + 1) ** 2 <= coeffs.shape[-2], coeffs.shape
+    assert coeffs.shape[:-2] in ((N,), (C, N)), coeffs.shape
+    if packed:
+        assert camera_ids is not None and gaussian_ids is not None
+        assert camera_ids.shape == gaussian_ids.shape == radii.shape[:1], radii.shape
+        camera_ids, gaussian_ids = camera_ids.contiguous(), gaussian_ids.contiguous()
+    else:
+        assert radii.shape == (C, N, 2), radii.shape
+        camera_ids, gaussian_ids = None, None
+    if depths is not None:
+        assert depths.shape == radii.shape[:-1], depths.shape
+        depths = depths.contiguous()
+    return _ViewColors.apply(degrees_to_use, means.contiguous(), viewmats.contiguous(),
+                             coeffs.contiguous(), radii.contiguous(), depths, camera_ids, gaussian_ids,
+                             launch_context)
 
 
 def fully_fused_projection(
@@ -900,6 +946,47 @@ class _ComputeLidarVelocity(torch.autograd.Function):
         v_p_view, v_velocities = _make_lazy_hip_func("compute_lidar_velocity_bwd")(
             p_view, lin_vel, ang_vel, velocities, v_vel.contiguous())
         return v_p_view, None, None, v_velocities
+
+
+class _ViewColors(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, sh_degree, means, viewmats, coeffs, radii, depths, camera_ids, gaussian_ids,
+                launch_context):
+        with (launch_context if launch_context is not None else contextlib.nullcontext()):
+            colors = _make_lazy_hip_func("view_colors_fwd")(
+                sh_degree, means, viewmats, camera_ids, gaussian_ids, radii, coeffs, depths)
+        ctx.save_for_backward(means, viewmats, coeffs, radii, camera_ids, gaussian_ids, colors)
+        ctx.sh_degree = sh_degree
+        ctx.has_depths = depths is not None
+        return colors
+
+    @staticmethod
+    def backward(ctx, v_colors):
+        means, viewmats, coeffs, radii, camera_ids, gaussian_ids, colors = ctx.saved_tensors
+        need_means, need_coeffs = ctx.needs_input_grad[1], ctx.needs_input_grad[3]
+        v_means = v_coeffs = v_depths = None
+        if need_means or need_coeffs:
+            v_rows, v_dirs = _make_lazy_hip_func("view_colors_bwd")(
+                ctx.sh_degree, means, viewmats, camera_ids, gaussian_ids, radii, coeffs, colors,
+                v_colors.contiguous(), need_means)
+            # rows of one Gaussian seen by several sensors add up
+            packed = camera_ids is not None
+            if need_coeffs:
+                if coeffs.dim() == 4:
+                    v_coeffs = (torch.zeros_like(coeffs).index_put_((camera_ids, gaussian_ids), v_rows, accumulate=True)
+                                if packed else v_rows)
+                elif packed:
+                    v_coeffs = torch.zeros_like(coeffs).index_add_(0, gaussian_ids, v_rows)
+                else:
+                    v_coeffs = v_rows[0] if v_rows.shape[0] == 1 else v_rows.sum(0)
+            if need_means:
+                if packed:
+                    v_means = torch.zeros_like(means).index_add_(0, gaussian_ids, v_dirs)
+                else:
+                    v_means = v_dirs[0] if v_dirs.shape[0] == 1 else v_dirs.sum(0)
+        if ctx.has_depths and ctx.needs_input_grad[5]:
+            v_depths = v_colors[..., 3]
+        return None, v_means, None, v_coeffs, None, v_depths, None, None, None
 
 
 class _SphericalHarmonics(torch.autograd.Function):

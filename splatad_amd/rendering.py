@@ -20,6 +20,7 @@ from .hip._wrapper import (
     rasterize_to_pixels,
     rasterize_to_points,
     spherical_harmonics,
+    view_dependent_colors,
 )
 
 
@@ -38,6 +39,68 @@ def _sensor_motion(C, device, linear_velocity, angular_velocity, rolling_shutter
     else:
         rolling_shutter_time = torch.zeros(C, device=device)
     return linear_velocity, angular_velocity, rolling_shutter_time
+
+
+_HELPER_STREAMS: Dict[int, "torch.cuda.Stream"] = {}
+
+
+class _Beside:
+    """Runs the work of `with` blocks on a helper stream, beside what the caller's stream does
+    between the creation of the object (the fork) and `join()`.
+
+    The tile intersection ends with a segment sort whose few long workgroups leave most of the
+    GPU idle; work that only depends on the projection -- the colours of the Gaussians -- is
+    enqueued on a helper stream (default priority) to run meanwhile.  Create the object when
+    the inputs of that work are enqueued on the caller's stream: the helper stream waits for
+    that point only, not for what the caller's stream is given afterwards.  `join()` makes the
+    caller's stream wait for the helper and tells the allocator that the tensors made there
+    are used on the caller's stream from now on.  On a CPU device, or while a graph is being
+    captured, the blocks simply run in place.
+    """
+
+    def __init__(self, device):
+        self.main = self.side = self.fork = self._ctx = None
+        if device.type == "cuda" and not torch.cuda.is_current_stream_capturing():
+            idx = device.index if device.index is not None else torch.cuda.current_device()
+            if idx not in _HELPER_STREAMS:
+                _HELPER_STREAMS[idx] = torch.cuda.Stream(device=idx)
+            self.main = torch.cuda.current_stream(idx)
+            self.side = _HELPER_STREAMS[idx]
+            self.fork = self.main.record_event()
+
+    def __enter__(self):
+        if self.side is not None:
+            self.side.wait_event(self.fork)
+            self._ctx = torch.cuda.stream(self.side)
+            self._ctx.__enter__()
+        return self
+
+    def __exit__(self, *exc):
+        if self._ctx is not None:
+            self._ctx.__exit__(*exc)
+            self._ctx = None
+        return False
+
+    def join(self, *tensors):
+        if self.side is not None:
+            self.main.wait_stream(self.side)
+            for t in tensors:
+                if t is not None:
+                    t.record_stream(self.main)
+
+
+class _AppendChannel(torch.autograd.Function):
+    """torch.cat([features, extra[..., None]], -1) with the copy enqueued inside `beside`;
+    the autograd node, and with it the backward pass, stays on the caller's stream."""
+
+    @staticmethod
+    def forward(ctx, beside, features, extra):
+        with beside:
+            return torch.cat([features, extra[..., None]], dim=-1)
+
+    @staticmethod
+    def backward(ctx, v_out):
+        return None, v_out[..., :-1], v_out[..., -1]
 
 
 def rasterization(
@@ -125,6 +188,7 @@ def rasterization(
         opacities = opacities * compensations
 
     # 2. tile intersection, sort, offsets
+    beside = _Beside(means.device)  # fork: everything the colours need is enqueued
     tile_width = math.ceil(width / float(tile_size))
     tile_height = math.ceil(height / float(tile_size))
     tiles_per_gauss, isect_ids, flatten_ids = isect_tiles(
@@ -133,8 +197,19 @@ def rasterization(
     )
     isect_offsets = isect_offset_encode(isect_ids, C, tile_width, tile_height)
 
-    # 3. per-(camera, Gaussian) colours
-    if sh_degree is None:
+    # 3. per-(camera, Gaussian) colours.  The intersection has just enqueued its segment sort,
+    # whose long workgroups leave most of the GPU idle: the colours are computed beside it, on
+    # a helper stream.
+    depth_appended = False
+    fused_colors = sh_degree is not None and not viewmats.requires_grad
+    if fused_colors:
+        # one kernel for directions, masks, SH, activation and the depth channel
+        depth_appended = render_mode in ["RGB+D", "RGB+ED"]
+        colors = view_dependent_colors(sh_degree, means, viewmats, colors, radii,
+                                       depths if depth_appended else None, camera_ids,
+                                       gaussian_ids, launch_context=beside)
+        beside.join(colors)
+    elif sh_degree is None:
         if packed:
             colors = colors[gaussian_ids] if colors.dim() == 2 else colors[camera_ids, gaussian_ids]
         elif colors.dim() == 2:
@@ -154,7 +229,8 @@ def rasterization(
 
     # 4. channels to composite
     if render_mode in ["RGB+D", "RGB+ED"]:
-        colors = torch.cat((colors, depths[..., None]), dim=-1)
+        if not depth_appended:
+            colors = torch.cat((colors, depths[..., None]), dim=-1)
         if backgrounds is not None:
             backgrounds = torch.cat(
                 [backgrounds, torch.zeros(C, 1, device=backgrounds.device)], dim=-1
@@ -309,19 +385,32 @@ def lidar_rasterization(
     n_elevation_tiles = math.ceil(n_elevation_channels / tile_height)
     tile_azimuth_resolution = azimuth_resolution * tile_width
     n_azimuth_tiles = math.ceil((max_azimuth - min_azimuth) / tile_azimuth_resolution)
+    # features to composite (the range is appended as last channel further down, on a helper
+    # stream beside the segment sort of the tile intersection).  Chunks carry channel_chunk-1 features plus the range; the
+    # chunk count is the reference's (rendering.py:735): features beyond
+    # n_chunks*(channel_chunk-1) are not rendered, e.g. D=63 with channel_chunk=32.
+    if (D + 1) > channel_chunk:
+        n_chunks = (D + channel_chunk) // channel_chunk
+        chunks = [lidar_features[..., i * (channel_chunk - 1) : (i + 1) * (channel_chunk - 1)]
+                  for i in range(n_chunks)]
+    else:
+        chunks = [lidar_features]
+    beside = _Beside(means.device)  # fork: features and ranges are enqueued
     tiles_per_gauss, isect_ids, flatten_ids = isect_lidar_tiles(
         means2d, radii, depths, elev_boundaries=tile_elevation_boundaries,
         tile_azim_resolution=tile_azimuth_resolution, min_azim=min_azimuth, packed=packed,
         n_cameras=C, camera_ids=camera_ids, gaussian_ids=gaussian_ids,
     )
     isect_offsets = isect_offset_encode(isect_ids, C, n_azimuth_tiles, n_elevation_tiles)
+    chunks = [_AppendChannel.apply(beside, f, depths) for f in chunks]
+    beside.join(*chunks)
 
     image_width = raster_pts.shape[-2]
     image_height = raster_pts.shape[-3]
 
     def composite(feats):
         return rasterize_to_points(
-            means2d, conics, torch.cat([feats, depths[..., None]], dim=-1), opacities, pix_vels,
+            means2d, conics, feats, opacities, pix_vels,
             depth_compensations, raster_pts, image_width, image_height, tile_width, tile_height,
             isect_offsets, flatten_ids,
             compute_alpha_sum_until_points=compute_alpha_sum_until_points,
@@ -329,16 +418,11 @@ def lidar_rasterization(
             packed=packed, absgrad=absgrad,
         )
 
-    if (D + 1) > channel_chunk:
-        # Chunks carry channel_chunk-1 features plus the range channel.  The chunk count is
-        # the reference's (rendering.py:735): features beyond n_chunks*(channel_chunk-1) are
-        # not rendered, e.g. D=63 with channel_chunk=32.
-        n_chunks = (D + channel_chunk) // channel_chunk
+    if len(chunks) > 1:
         feats_out, alphas_out, sums_out, medians_out = [], [], [], []
-        for i in range(n_chunks):
-            chunk = lidar_features[..., i * (channel_chunk - 1) : (i + 1) * (channel_chunk - 1)]
+        for i, chunk in enumerate(chunks):
             rf, ra, rs_, md = composite(chunk)
-            feats_out.append(rf if i == n_chunks - 1 else rf[..., :-1])
+            feats_out.append(rf if i == len(chunks) - 1 else rf[..., :-1])
             alphas_out.append(ra)
             sums_out.append(rs_)
             medians_out.append(md)
@@ -348,7 +432,7 @@ def lidar_rasterization(
         alpha_sum_until_points = sums_out[0]
     else:
         render_lidar_features, render_alphas, alpha_sum_until_points, median_depths = composite(
-            lidar_features
+            chunks[0]
         )
 
     meta = {

@@ -54,6 +54,24 @@ class OracleOps:
     def compute_sh_fwd(self, degree, dirs, coeffs, masks):
         return _t(oracle.spherical_harmonics(degree, _n(dirs), _n(coeffs), _n(masks), precision="f32"))
 
+    def view_colors_fwd(self, degree, means, viewmats, camera_ids, gaussian_ids, radii, coeffs, depths):
+        # the chain of gsplat/rendering.py:325-351 on the oracle's spherical harmonics
+        means, viewmats, radii, coeffs = _n(means), _n(viewmats), _n(radii), _n(coeffs)
+        pos = np.linalg.inv(viewmats.astype(np.float64))[:, :3, 3]
+        if camera_ids is not None:
+            cam, gid = _n(camera_ids), _n(gaussian_ids)
+            dirs = means[gid] - pos[cam]
+            shs = coeffs[gid] if coeffs.ndim == 3 else coeffs[cam, gid]
+        else:
+            dirs = means[None] - pos[:, None]
+            shs = np.broadcast_to(coeffs, (viewmats.shape[0],) + coeffs.shape[-3:]) if coeffs.ndim == 3 else coeffs
+        cols = oracle.spherical_harmonics(degree, dirs.astype(np.float32), np.ascontiguousarray(shs),
+                                          radii[..., 0] > 0, precision="f32")
+        cols = np.maximum(cols + 0.5, 0.0).astype(np.float32)
+        if depths is not None:
+            cols = np.concatenate([cols, _n(depths)[..., None]], -1)
+        return _t(cols)
+
     def isect_tiles(self, means2d, radii, depths, camera_ids, gaussian_ids, C, tile_size, tw, th, sort,
                     double_buffer):
         out = oracle.isect_tiles(_n(means2d), _n(radii), _n(depths), tile_size, tw, th, sort, C,

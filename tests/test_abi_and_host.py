@@ -28,14 +28,16 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in include/splatad_hip.h but not exported"
     lib.splatad_abi_version.restype = ctypes.c_int
-    assert lib.splatad_abi_version() == 2
+    assert lib.splatad_abi_version() == 3
     lib.splatad_last_error.restype = ctypes.c_char_p
     assert isinstance(lib.splatad_last_error(), bytes)
     # size queries are pure host code
     lib.splatad_isect_workspace_bytes.restype = ctypes.c_size_t
-    a = lib.splatad_isect_workspace_bytes(ctypes.c_uint64(1000), ctypes.c_uint32(2), ctypes.c_uint32(100), ctypes.c_int64(0))
-    b = lib.splatad_isect_workspace_bytes(ctypes.c_uint64(1000), ctypes.c_uint32(2), ctypes.c_uint32(100), ctypes.c_int64(5000))
-    assert b >= a + 5000 * 8
+    lib.splatad_isect_lists_bytes.restype = ctypes.c_size_t
+    assert lib.splatad_isect_workspace_bytes(ctypes.c_uint64(1000), ctypes.c_uint32(2), ctypes.c_uint32(100)) >= 3 * 256
+    a = lib.splatad_isect_lists_bytes(ctypes.c_uint64(1000), ctypes.c_int64(0))
+    b = lib.splatad_isect_lists_bytes(ctypes.c_uint64(1000), ctypes.c_int64(5000))
+    assert a >= 1000 * 8 and b >= 5000 * 24
     lib.splatad_projection_packed_workspace_bytes.restype = ctypes.c_size_t
     assert lib.splatad_projection_packed_workspace_bytes(ctypes.c_uint32(2), ctypes.c_uint32(1000)) >= 2000 * 48
 
