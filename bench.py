@@ -147,9 +147,9 @@ def bench_camera(args):
         stages["isect_sort_ms"] = time_kernel(isect, 5)
         stages["offset_encode_ms"] = time_kernel(
             lambda: _C.isect_offset_encode(meta["isect_ids"], C, meta["tile_width"], meta["tile_height"]), 5)
-        stages["sh_ms"] = time_kernel(
-            lambda: _C.compute_sh_fwd(3, dirs.contiguous(), s["colors"].expand(C, -1, -1, -1).contiguous(),
-                                      (meta["radii"][..., 0] > 0).contiguous()), 5)
+        stages["view_colors_ms"] = time_kernel(
+            lambda: _C.view_colors_fwd(3, s["means"], s["viewmats"], None, None, meta["radii"],
+                                       s["colors"], meta["depths"]), 5)
         stages["rasterize_ms"] = k_ms
     return dict(sec=sec, sec_packed=sec_packed, pixels=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
                 n_isects=n_isects, i_need=i_need, nnz=int((meta["radii"][..., 0] > 0).sum().item()),

@@ -124,29 +124,60 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// Sums NV (a power of two, 2..64) per-lane values over the 64 lanes of a wavefront with
-// NV - 1 + log2(64 / NV) shuffles instead of 6 NV: at every step a lane hands half of its
-// values to the partner that keeps accumulating them.  Afterwards every lane holds, in
-// v[0], the wavefront total of value `wave_reduce_slot<NV>(lane)`; 64 / NV lanes hold each.
+// Lane permutations inside the vector ALU (no LDS round trip): `pattern` is a DPP control --
+// 0x140 mirrors each row of 16 lanes, 0x141 each half row of 8, 0x4E swaps the pairs of a quad
+// (lane ^ 2), 0xB1 the neighbours (lane ^ 1).  All lanes of the wavefront must be active.
+template <int pattern>
+__device__ __forceinline__ float wave_dpp(float v) {
+    return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), pattern, 0xF, 0xF, false));
+}
+
+// One step of a reduce-scatter between lanes that differ in bit `BIT` (5..0) of the lane
+// index: afterwards the lanes whose bit is clear hold, in `a`, the pair's sum of `a`, the
+// others the pair's sum of `b`.  Bits 5 and 4 use the gfx950 half-swaps (the upper 32 or the
+// odd 16 lanes of one register change places with the lower 32 or even 16 of the other, so a
+// single add finishes the step); bits 3 and 2 pair lanes by mirroring a row or a half row,
+// which also flips lower bits -- harmless, those have not been used yet.
+template <int BIT>
+__device__ __forceinline__ float wave_pair_step(float a, float b, int lane) {
+    if constexpr (BIT == 5) {
+        const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+        return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    } else if constexpr (BIT == 4) {
+        const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+        return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    } else {
+        constexpr int pattern = BIT == 3 ? 0x140 : (BIT == 2 ? 0x141 : (BIT == 1 ? 0x4E : 0xB1));
+        const float sa = a + wave_dpp<pattern>(a), sb = b + wave_dpp<pattern>(b);
+        return (lane & (1 << BIT)) == 0 ? sa : sb;
+    }
+}
+
+template <int NV, int BIT>
+__device__ __forceinline__ void wave_reduce_scatter_from(float (&v)[NV], int lane) {
+    constexpr int half = NV >> (6 - BIT); // values still held per lane, halved by this step
+    if constexpr (half >= 1) {
+#pragma unroll
+        for (int k = 0; k < half; ++k) v[k] = wave_pair_step<BIT>(v[k], v[k + half], lane);
+        if constexpr (BIT > 0) wave_reduce_scatter_from<NV, BIT - 1>(v, lane);
+    } else {
+        // one value left per lane: the lanes that share it add up their parts
+        constexpr int pattern = BIT == 3 ? 0x140 : (BIT == 2 ? 0x141 : (BIT == 1 ? 0x4E : 0xB1));
+        static_assert(BIT <= 3, "at least four values per lane");
+        v[0] += wave_dpp<pattern>(v[0]);
+        if constexpr (BIT > 0) wave_reduce_scatter_from<NV, BIT - 1>(v, lane);
+    }
+}
+
+// Sums NV (a power of two, 4..64) per-lane values over the 64 lanes of a wavefront: at every
+// step a lane hands half of its values to a partner that keeps accumulating them, so the
+// work halves from step to step (NV - 1 exchanges instead of 6 NV).  Afterwards every lane
+// holds, in v[0], the wavefront total of value `wave_reduce_slot<NV>(lane)`; 64 / NV lanes
+// hold each.  All 64 lanes must be active.
 template <int NV>
 __device__ __forceinline__ void wave_reduce_scatter(float (&v)[NV], int lane) {
-    int off = 32;
-#pragma unroll
-    for (int half = NV / 2; half >= 1; half /= 2) {
-        // bit masks instead of selects: a select between two array elements would be turned
-        // into a dynamically indexed access, i.e. a compare-and-select chain over the array
-        const uint32_t m = (lane & off) != 0 ? 0xFFFFFFFFu : 0u; // upper half of the pair
-#pragma unroll
-        for (int k = 0; k < half; ++k) {
-            const uint32_t lo = __float_as_uint(v[k]), hi = __float_as_uint(v[k + half]);
-            const float send = __uint_as_float((lo & m) | (hi & ~m));
-            const float keep = __uint_as_float((hi & m) | (lo & ~m));
-            v[k] = keep + __shfl_xor(send, off, SPLATAD_WAVE);
-        }
-        off >>= 1;
-    }
-#pragma unroll
-    for (int rest = 32 / NV; rest >= 1; rest /= 2) v[0] += __shfl_xor(v[0], rest, SPLATAD_WAVE);
+    static_assert(NV >= 4 && NV <= 64 && (NV & (NV - 1)) == 0, "NV must be a power of two in 4..64");
+    wave_reduce_scatter_from<NV, 5>(v, lane);
 }
 
 template <int NV>

@@ -216,7 +216,7 @@ rasterize_bwd_kernel(BwdArgs a) {
 #pragma unroll
                 for (int k = 0; k < NV; ++k) v[k] = 0.f;
                 if (valid) {
-                    const float ra = 1.0f / (1.0f - alpha);
+                    const float ra = __builtin_amdgcn_rcpf(1.0f - alpha); // 1 ulp, no division sequence
                     T *= ra; // transmittance in front of this Gaussian
                     const float fac = alpha * T;
                     float v_alpha = 0.f;

@@ -76,6 +76,25 @@ def _stream(device):
 _u32, _i32, _i64, _u64, _f32 = ctypes.c_uint32, ctypes.c_int, ctypes.c_int64, ctypes.c_uint64, ctypes.c_float
 
 
+def _zeros_many(device, *shapes):
+    """Zero-filled float32 tensors of the given shapes (None stays None), carved out of one
+    buffer that a single fill clears: gradient outputs come in groups of four to seven, and a
+    fill per tensor costs more in launches than in bandwidth."""
+    counts = [0 if sh is None else int(math.prod(sh)) for sh in shapes]
+    sizes = [(n + 63) // 64 * 64 for n in counts]  # pieces of whole 256 bytes
+    pool = torch.zeros((sum(sizes),), dtype=torch.float32, device=device)
+    out, at = [], 0
+    for sh, n, size in zip(shapes, counts, sizes):
+        out.append(None if sh is None else pool[at:at + n].view(tuple(sh)))
+        at += size
+    return out
+
+
+def _zeros_like_many(*tensors):
+    ref = next(t for t in tensors if t is not None)
+    return _zeros_many(ref.device, *(None if t is None else t.shape for t in tensors))
+
+
 def _workspace(nbytes: int, device) -> Tensor:
     return torch.empty((max(int(nbytes), 256),), dtype=torch.uint8, device=device)
 
@@ -218,13 +237,11 @@ class _Ops:
         nnz = camera_ids.shape[0] if packed else 0
         rows = nnz if (packed and sparse_grad) else N
         f = dict(dtype=torch.float32, device=dev)
-        v_means = torch.zeros((rows, 3), **f)
-        v_covars = torch.zeros((rows, 6), **f) if covars is not None else None
-        v_quats = torch.zeros((rows, 4), **f) if covars is None else None
-        v_scales = torch.zeros((rows, 3), **f) if covars is None else None
-        v_viewmats = torch.zeros_like(viewmats) if viewmats_requires_grad else None
-        v_velocities = (torch.zeros_like(velocities)
-                        if (velocities_requires_grad and velocities is not None) else None)
+        v_means, v_covars, v_quats, v_scales, v_viewmats, v_velocities = _zeros_many(
+            dev, (rows, 3), (rows, 6) if covars is not None else None,
+            (rows, 4) if covars is None else None, (rows, 3) if covars is None else None,
+            viewmats.shape if viewmats_requires_grad else None,
+            velocities.shape if (velocities_requires_grad and velocities is not None) else None)
         with torch.cuda.device(dev):
             _check(lib.splatad_projection_bwd(
                 _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
@@ -257,13 +274,10 @@ class _Ops:
         v_pix_vels = _in(v_pix_vels, "v_pix_vels")
         v_dc = _in(v_depth_compensations, "v_depth_compensations")
         N, C, dev = means.shape[0], viewmats.shape[0], means.device
-        v_means = torch.zeros_like(means)
-        v_covars = torch.zeros_like(covars) if covars is not None else None
-        v_quats = torch.zeros_like(quats) if covars is None else None
-        v_scales = torch.zeros_like(scales) if covars is None else None
-        v_viewmats = torch.zeros_like(viewmats) if viewmats_requires_grad else None
-        v_velocities = (torch.zeros_like(velocities)
-                        if (velocities_requires_grad and velocities is not None) else None)
+        v_means, v_covars, v_quats, v_scales, v_viewmats, v_velocities = _zeros_like_many(
+            means, covars, quats if covars is None else None, scales if covars is None else None,
+            viewmats if viewmats_requires_grad else None,
+            velocities if (velocities_requires_grad and velocities is not None) else None)
         with torch.cuda.device(dev):
             _check(lib.splatad_lidar_projection_bwd(
                 _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
@@ -296,7 +310,9 @@ class _Ops:
         dirs = _in(dirs, "dirs"); coeffs = _in(coeffs, "coeffs")
         masks = _in(masks, "masks", torch.bool); v_colors = _in(v_colors, "v_colors")
         n, dev = dirs.numel() // 3, dirs.device
-        v_coeffs = torch.zeros_like(coeffs)
+        # the kernel writes the floats of the bases in use; the others must read zero
+        full = (degrees_to_use + 1) ** 2 == K
+        v_coeffs = torch.empty_like(coeffs) if full else torch.zeros_like(coeffs)
         v_dirs = torch.zeros_like(dirs) if compute_v_dirs else None
         with torch.cuda.device(dev):
             _check(lib.splatad_sh_bwd(_u32(n), _u32(K), _u32(degrees_to_use), _p(dirs), _p(coeffs),
@@ -339,7 +355,9 @@ class _Ops:
         lead = tuple(radii.shape[:-1])
         n, K = int(math.prod(lead)), coeffs.shape[-2]
         f = dict(dtype=torch.float32, device=dev)
-        v_coeffs = torch.zeros(lead + (K, 3), **f)
+        # the kernel writes the floats of the bases in use; the others must read zero
+        full = (degrees_to_use + 1) ** 2 == K
+        v_coeffs = (torch.empty if full else torch.zeros)(lead + (K, 3), **f)
         v_dirs = torch.empty(lead + (3,), **f) if compute_v_dirs else None
         with torch.cuda.device(dev):
             _check(lib.splatad_view_colors_bwd(
@@ -691,10 +709,8 @@ class _Ops:
         v_render_alphas = _in(v_render_alphas, "v_render_alphas")
         C, th, tw = tile_offsets.shape
         D, dev = colors.shape[-1], means2d.device
-        v_means2d = torch.zeros_like(means2d); v_conics = torch.zeros_like(conics)
-        v_colors = torch.zeros_like(colors); v_opacities = torch.zeros_like(opacities)
-        v_pix_vels = torch.zeros_like(pix_vels)
-        v_means2d_abs = torch.zeros_like(means2d) if absgrad else None
+        v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_means2d_abs = _zeros_like_many(
+            means2d, conics, colors, opacities, pix_vels, means2d if absgrad else None)
         if flatten_ids.shape[0]:
             with torch.cuda.device(dev):
                 _check(lib.splatad_rasterize_to_pixels_bwd(
@@ -759,10 +775,8 @@ class _Ops:
         v_asum = _in(v_alpha_sum_until_points, "v_alpha_sum_until_points")
         C, gh, gw = tile_offsets.shape
         D, dev = colors.shape[-1], means2d.device
-        v_means2d = torch.zeros_like(means2d); v_conics = torch.zeros_like(conics)
-        v_colors = torch.zeros_like(colors); v_opacities = torch.zeros_like(opacities)
-        v_pix_vels = torch.zeros_like(pix_vels); v_dc = torch.zeros_like(dc)
-        v_means2d_abs = torch.zeros_like(means2d) if absgrad else None
+        v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_dc, v_means2d_abs = _zeros_like_many(
+            means2d, conics, colors, opacities, pix_vels, dc, means2d if absgrad else None)
         if flatten_ids.shape[0]:
             with torch.cuda.device(dev):
                 _check(lib.splatad_rasterize_to_points_bwd(
