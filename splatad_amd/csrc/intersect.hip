@@ -1144,11 +1144,12 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                                               n_isects, w.seg_counts, w.seg_lists, w.tile_starts, \
                                               w.pairs, isect_ids, flatten_ids, on)) != 0)         \
         return rc;
+    // the longest workgroups first on every stream
     SPLATAD_SORT_CLASS(5, 32, false, 1024, 32768u, 256u, ss->aux[0])
-    SPLATAD_SORT_CLASS(6, 0, false, 1024, 0x7FFFFFFFu, 256u, ss->aux[0])
     SPLATAD_SORT_CLASS(4, 16, true, 1024, 16384u, 256u, ss->aux[1])
+    SPLATAD_SORT_CLASS(6, 0, false, 1024, 0x7FFFFFFFu, 256u, stream)
+    SPLATAD_SORT_CLASS(2, 8, true, 512, 4096u, 1024u, ss->aux[0])
     SPLATAD_SORT_CLASS(3, 8, true, 1024, 8192u, 512u, ss->aux[1])
-    SPLATAD_SORT_CLASS(2, 8, true, 512, 4096u, 1024u, stream)
     SPLATAD_SORT_CLASS(1, 8, true, 256, 2048u, 2048u, stream)
     SPLATAD_SORT_CLASS(0, 4, true, 128, 512u, 4096u, stream)
 #undef SPLATAD_SORT_CLASS
