@@ -698,13 +698,16 @@ __constant__ const uint32_t kSortClassMin[kSortClasses + 1] = {0u,    512u,   20
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 isect_classify_segments_kernel(uint32_t n_segments, int64_t n_isects,
                                const int32_t *__restrict__ tile_starts,
-                               uint32_t *__restrict__ seg_counts, uint32_t *__restrict__ seg_lists) {
+                               uint32_t *__restrict__ seg_counts, uint32_t *__restrict__ seg_lists,
+                               int32_t *__restrict__ tile_offsets) {
     const uint32_t seg = blockIdx.x * blockDim.x + threadIdx.x;
     uint32_t n = 0;
     if (seg < n_segments) {
         const int64_t start = tile_starts[seg];
         const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
         n = (uint32_t)(stop - start);
+        // a tile's offset is the start of its segment: the first row of the scanned table
+        if (tile_offsets != nullptr) tile_offsets[seg] = (int32_t)start;
     }
     int c = n == 0 ? -1 : 0;
     while (c >= 0 && c + 1 < kSortClasses && n > kSortClassMin[c + 1]) ++c;
@@ -806,12 +809,6 @@ __global__ void fill_zero_i32_kernel(int32_t *p, int64_t n) {
 }
 
 __global__ void fill_zero_u64_kernel(unsigned long long *p) { p[threadIdx.x] = 0ull; }
-
-__global__ void copy_i32_kernel(const int32_t *__restrict__ src, int32_t *__restrict__ dst,
-                                int64_t n) {
-    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) dst[i] = src[i];
-}
 
 struct IsectWorkspace {
     unsigned long long *n_isects; // [1]
@@ -1115,11 +1112,6 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                                         tcopies > 1 ? -(int)tcopies : 1, 0, w.tile_starts,
                                         w.scan_total, w.block_sums, stream);
     if (rc) return rc;
-    if (tile_offsets) {
-        // a tile's offset is the start of its segment: the first row of the scanned table
-        hipLaunchKernelGGL(copy_i32_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream,
-                           (const int32_t *)w.tile_starts, tile_offsets, (int64_t)segs);
-    }
     hipLaunchKernelGGL(isect_tile_bin_kernel<true>, dim3((uint32_t)bin_wgs),
                        dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, tcopies,
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
@@ -1132,7 +1124,8 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     // upper classes overlap the many short ones of the lower classes.
     const uint32_t nseg = (uint32_t)segs;
     hipLaunchKernelGGL(isect_classify_segments_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream,
-                       nseg, n_isects, (const int32_t *)w.tile_starts, w.seg_counts, w.seg_lists);
+                       nseg, n_isects, (const int32_t *)w.tile_starts, w.seg_counts, w.seg_lists,
+                       tile_offsets);
     SPLATAD_LAUNCH_CHECK();
     IsectDevice *ss = nullptr;
     if ((rc = isect_device(&ss)) != 0) return rc;

@@ -1,7 +1,8 @@
 // Device-wide exclusive prefix sum used by the compaction and intersection code.
 //
-// Three launches: per-block totals, a single-workgroup scan of those totals, and a
-// per-block scan that adds the block's base.  2048 items per workgroup of 256 lanes;
+// Per-block totals, then a per-block scan that adds the block's base; the base comes from a
+// single-workgroup scan of the totals in between or, for up to two million elements, is added
+// up by every block itself (two launches instead of three).  2048 items per workgroup of 256 lanes;
 // wave64 shuffles inside a wavefront, LDS across the four wavefronts.
 #pragma once
 
@@ -85,10 +86,22 @@ scan_block_sums_kernel(int64_t *__restrict__ block_sums, int64_t n_blocks,
     if (threadIdx.x == 0) *total = carry;
 }
 
-template <typename OutT>
+// FOLD: block_sums holds the blocks' totals, not yet scanned; every workgroup adds up the
+// totals before its own (a few hundred at most, see kScanFoldBlocks) and the last one writes
+// the grand total, which saves the launch of scan_block_sums_kernel.
+template <typename OutT, bool FOLD>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 scan_apply_kernel(const int32_t *__restrict__ in, int64_t n, int stride, int as_flag,
-                  const int64_t *__restrict__ block_sums, OutT *__restrict__ out) {
+                  const int64_t *__restrict__ block_sums, OutT *__restrict__ out,
+                  int64_t *__restrict__ total) {
+    int64_t before = 0;
+    if (FOLD) {
+        int64_t part = 0;
+        for (uint32_t j = threadIdx.x; j < blockIdx.x; j += SPLATAD_THREADS) part += block_sums[j];
+        block_exclusive_scan(part, &before);
+    } else {
+        before = block_sums[blockIdx.x];
+    }
     const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
     int32_t v[SCAN_ITEMS];
     int64_t s = 0;
@@ -98,13 +111,16 @@ scan_apply_kernel(const int32_t *__restrict__ in, int64_t n, int stride, int as_
         s += v[k];
     }
     int64_t tot;
-    int64_t run = block_exclusive_scan(s, &tot) + block_sums[blockIdx.x];
+    int64_t run = block_exclusive_scan(s, &tot) + before;
+    if (FOLD && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) *total = before + tot;
 #pragma unroll
     for (int k = 0; k < SCAN_ITEMS; ++k) {
         if (base + k < n) out[stride > 0 ? base + k : scan_phys(base + k, n, stride)] = (OutT)run;
         run += v[k];
     }
 }
+
+constexpr int64_t kScanFoldBlocks = 1024; // up to 2M elements: two launches instead of three
 
 static inline size_t scan_workspace_bytes(int64_t n) {
     int64_t n_blocks = (n + SCAN_TILE - 1) / SCAN_TILE;
@@ -124,13 +140,20 @@ static inline int launch_exclusive_scan(const int32_t *in, int64_t n, int stride
                            0, stream, in, n, stride, as_flag, block_sums);
         SPLATAD_LAUNCH_CHECK();
     }
+    if (n_blocks > 0 && n_blocks <= kScanFoldBlocks && out != nullptr) {
+        hipLaunchKernelGGL((scan_apply_kernel<OutT, true>), dim3((uint32_t)n_blocks),
+                           dim3(SPLATAD_THREADS), 0, stream, in, n, stride, as_flag,
+                           (const int64_t *)block_sums, out, total);
+        SPLATAD_LAUNCH_CHECK();
+        return 0;
+    }
     hipLaunchKernelGGL(scan_block_sums_kernel, dim3(1), dim3(SPLATAD_THREADS), 0, stream,
                        block_sums, n_blocks, total);
     SPLATAD_LAUNCH_CHECK();
     if (n_blocks > 0 && out != nullptr) {
-        hipLaunchKernelGGL(scan_apply_kernel<OutT>, dim3((uint32_t)n_blocks),
+        hipLaunchKernelGGL((scan_apply_kernel<OutT, false>), dim3((uint32_t)n_blocks),
                            dim3(SPLATAD_THREADS), 0, stream, in, n, stride, as_flag,
-                           (const int64_t *)block_sums, out);
+                           (const int64_t *)block_sums, out, total);
         SPLATAD_LAUNCH_CHECK();
     }
     return 0;
