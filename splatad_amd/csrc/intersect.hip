@@ -1016,6 +1016,11 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
                     "isect: camera and tile ids need more than 32 bits");
     IsectWorkspace w;
     carve_isect(workspace, total, pl.segs, sort ? pl.cslots : 0, &w);
+    // the host waits for the count below, which a stream under graph capture would never deliver
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    SPLATAD_CHECK_HIP(hipStreamIsCapturing(stream, &capturing));
+    SPLATAD_REQUIRE(capturing == hipStreamCaptureStatusNone,
+                    "isect: the counting call returns a number to the host and cannot be captured in a graph");
     IsectDevice *dv = nullptr;
     if (int rc = isect_device(&dv)) return rc;
     std::lock_guard<std::mutex> lock(dv->guard);
