@@ -115,20 +115,21 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
                 const float dy = (xyv.y + roll * xyv.w) - py;
                 const float power = dx * (con.x * dx + con.y * dy) + con.z * dy * dy;
                 const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
-                const float next_T = T * (1.0f - alpha);
+                const float weight = alpha * T;
+                const float next_T = T - weight; // T (1 - alpha)
                 // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
                 const bool valid = alive && !(power < 0.f) && !(alpha < 1.f / 255.f);
                 const bool stop = valid && next_T <= 1e-4f;
                 const bool take = valid && !stop;
                 alive = alive && !stop;
+                const float vis = take ? weight : 0.f;
                 if (CH > 8 ? wave_ballot(take) != 0 : true) {
-                    const float vis = take ? alpha * T : 0.f;
 #pragma unroll
                     for (int k = 0; k < CH; ++k) out[k] += reinterpret_cast<const float *>(rec + 2)[k] * vis;
                 }
                 cur_idx = take ? batch_start + t : cur_idx;
-                T = take ? next_T : T;
-                if (wave_ballot(alive) == 0) break;
+                T -= vis;
+                // whether the whole wavefront is done is looked at once per 64 candidates, above
             }
         }
     }
@@ -271,14 +272,15 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
                 }
                 const float power = dx * (con.x * dx + con.y * dy) + con.z * dy * dy;
                 const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
-                const float next_T = T * (1.0f - alpha);
+                const float weight = alpha * T;
+                const float next_T = T - weight; // T (1 - alpha)
                 // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
                 const bool valid = alive && !(power < 0.f) && !(alpha < 1.f / 255.f);
                 const bool stop = valid && next_T <= 1e-4f;
                 const bool take = valid && !stop;
                 alive = alive && !stop;
                 if (wave_ballot(take) != 0) {
-                    const float vis = take ? alpha * T : 0.f;
+                    const float vis = take ? weight : 0.f;
 #pragma unroll
                     for (int k = 0; k < CH; ++k) out[k] += reinterpret_cast<const float *>(rec + 3)[k] * vis;
                     const float4 ext = rec[2];
@@ -287,9 +289,9 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
                     if (take && T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
                     if (take && a.compute_alpha_sum && ext.w < pz - a.threshold) asum += alpha;
                     cur_idx = take ? batch_start + t : cur_idx;
-                    T = take ? next_T : T;
+                    T -= vis;
                 }
-                if (wave_ballot(alive) == 0) break;
+                // whether the whole wavefront is done is looked at once per 64 candidates, above
             }
         }
     }

@@ -157,7 +157,7 @@ rasterize_to_indices_kernel(IndexArgs a) {
                 }
                 const float power = dx * (con.x * dx + con.y * dy) + con.z * dy * dy;
                 const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
-                const float next_T = T * (1.0f - alpha);
+                const float next_T = T - alpha * T; // as in the compositing kernels
                 const bool valid = alive && !(power < 0.f) && !(alpha < 1.f / 255.f);
                 const bool stop = valid && next_T <= 1e-4f;
                 const bool take = valid && !stop;
