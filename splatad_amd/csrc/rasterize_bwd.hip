@@ -36,6 +36,11 @@ struct BwdArgs {
     const float *v_render_colors, *v_render_alphas, *v_alpha_sum;
     float *v_means2d_abs, *v_means2d, *v_conics, *v_colors, *v_opacities, *v_pix_vels, *v_depth_comps;
     int first_pass; // adds the alpha / alpha-sum terms exactly once over the channel passes
+    // Packed accumulation: when given, the gradients of Gaussian g go to packed[g * packed_stride
+    // + slot] (slot = channel of the pass, then the geometry slots below) instead of the v_*
+    // arrays; unpack_gradients_kernel distributes them afterwards.
+    float *packed;
+    uint32_t packed_stride;
 };
 
 // Geometry gradient slots per Gaussian in the LDS accumulator, after the CH colour slots;
@@ -173,7 +178,7 @@ rasterize_bwd_kernel(BwdArgs a) {
                 rec[0] = make_float4(xy.x, xy.y, v.x, v.y);
             }
             rec[1] = staged_exponent(cn[0], cn[1], cn[2], opac);
-            s_aux[tr] = make_float2(__int_as_float(g), 1.0f / opac);
+            s_aux[tr] = make_float2(__int_as_float(g), opac > 0.f ? 1.0f / opac : 0.f); // finite
 #pragma unroll
             for (int k = 0; k < CH; ++k) s_col[tr * CH + k] = (uint32_t)k < a.n_ch ? crow[a.ch_offset + k] : 0.f;
         }
@@ -212,75 +217,77 @@ rasterize_bwd_kernel(BwdArgs a) {
                                    !(alpha < 1.f / 255.f);
                 if (wave_ballot(valid) == 0) continue;
 
+                // Branch-free from here on: a lane that does not take this Gaussian runs the same
+                // arithmetic with alpha = 0 and alpha-before-clamping = 0, which makes every
+                // gradient term an exact zero (all other factors are finite) and leaves its
+                // transmittance and colour buffer as they are.
+                const float alpha_s = valid ? alpha : 0.f;
+                const float ra = __builtin_amdgcn_rcpf(1.0f - alpha_s); // 1 ulp; exactly 1 for alpha = 0
+                T *= ra; // transmittance in front of this Gaussian
+                const float fac = alpha_s * T;
+                // a clamped alpha passes no gradient on to the exponent or the opacity
+                const float au_g = (valid && au <= 0.999f) ? au : 0.f;
                 float v[NV];
 #pragma unroll
-                for (int k = 0; k < NV; ++k) v[k] = 0.f;
-                if (valid) {
-                    const float ra = __builtin_amdgcn_rcpf(1.0f - alpha); // 1 ulp, no division sequence
-                    T *= ra; // transmittance in front of this Gaussian
-                    const float fac = alpha * T;
-                    float v_alpha = 0.f;
+                for (int k = ACC; k < NV; ++k) v[k] = 0.f;
+                float v_alpha = 0.f;
 #pragma unroll
-                    for (int k = 0; k < CH; ++k) {
-                        v[k] = fac * v_out[k];
-                        v_alpha += (s_col[t * CH + k] * T - buffer[k] * ra) * v_out[k];
-                    }
-                    float4 ext = make_float4(0.f, 0.f, 0.f, 0.f);
-                    float extra = 0.f;
-                    if constexpr (LIDAR) {
-                        ext = rec[RECORD - 1];
-                        extra = ext.y * dx + ext.z * dy + ext.x * roll;
-                        // depth channel = colour + extra: both enter c*T and the buffer
-                        v_alpha += (extra * T - buffer_extra * ra) * v_out_depth;
-                    }
-                    v_alpha += T_final * ra * v_render_a;
-                    v_alpha += -T_final * ra * bg_dot;
-                    const float g_depth = fac * v_out_depth; // gradient of the depth channel value
-                    const float rop = s_aux[t].y;
-                    // conic row products a dx + b dy and b dx + c dy from the staged form
-                    const float row_x = kLn2 * (2.f * e.x * dx + e.y * dy);
-                    const float row_y = kLn2 * (e.y * dx + 2.f * e.z * dy);
-                    float g_x = 0.f, g_y = 0.f, g_ax = 0.f, g_ay = 0.f;
-                    if (au <= 0.999f) {
-                        const float v_sigma = -au * v_alpha;
-                        v[CH + G_CONIC] = 0.5f * v_sigma * dx * dx;
-                        v[CH + G_CONIC + 1] = v_sigma * dx * dy;
-                        v[CH + G_CONIC + 2] = 0.5f * v_sigma * dy * dy;
-                        g_x = v_sigma * row_x;
-                        g_y = v_sigma * row_y;
-                        if constexpr (LIDAR) {
-                            v[CH + G_DC] = g_depth * dx;
-                            v[CH + G_DC + 1] = g_depth * dy;
-                            v[CH + G_VELZ] = g_depth * roll;
-                            g_x += g_depth * ext.y;
-                            g_y += g_depth * ext.z;
-                        }
-                        g_ax = fabsf(g_x);
-                        g_ay = fabsf(g_y);
-                        v[CH + G_OPAC] = au * rop * v_alpha;
-                    }
-#pragma unroll
-                    for (int k = 0; k < CH; ++k) buffer[k] += s_col[t * CH + k] * fac;
-                    if constexpr (LIDAR) {
-                        buffer_extra += extra * fac;
-                        if (a.compute_alpha_sum && ext.w < pz - a.threshold) {
-                            const float v_sig2 = -v_asum * au;
-                            const float ex = v_sig2 * row_x, ey = v_sig2 * row_y;
-                            g_x += ex; g_y += ey;
-                            g_ax += fabsf(ex); g_ay += fabsf(ey);
-                            v[CH + G_CONIC] += v_sig2 * 0.5f * dx * dx;
-                            v[CH + G_CONIC + 1] += v_sig2 * dx * dy;
-                            v[CH + G_CONIC + 2] += v_sig2 * 0.5f * dy * dy;
-                            v[CH + G_OPAC] += v_asum * au * rop;
-                        }
-                    }
-                    v[CH + G_XY] = g_x;
-                    v[CH + G_XY + 1] = g_y;
-                    v[CH + G_ABS] = g_ax;
-                    v[CH + G_ABS + 1] = g_ay;
-                    v[CH + G_VEL] = g_x * roll;
-                    v[CH + G_VEL + 1] = g_y * roll;
+                for (int k = 0; k < CH; ++k) {
+                    v[k] = fac * v_out[k];
+                    v_alpha += (s_col[t * CH + k] * T - buffer[k] * ra) * v_out[k];
                 }
+                float4 ext = make_float4(0.f, 0.f, 0.f, 0.f);
+                float extra = 0.f;
+                if constexpr (LIDAR) {
+                    ext = rec[RECORD - 1];
+                    extra = ext.y * dx + ext.z * dy + ext.x * roll;
+                    // depth channel = colour + extra: both enter c*T and the buffer
+                    v_alpha += (extra * T - buffer_extra * ra) * v_out_depth;
+                }
+                v_alpha += T_final * ra * v_render_a;
+                v_alpha += -T_final * ra * bg_dot;
+                const float rop = s_aux[t].y;
+                // conic row products a dx + b dy and b dx + c dy from the staged form
+                const float row_x = kLn2 * (2.f * e.x * dx + e.y * dy);
+                const float row_y = kLn2 * (e.y * dx + 2.f * e.z * dy);
+                const float v_sigma = -au_g * v_alpha;
+                v[CH + G_CONIC] = 0.5f * v_sigma * dx * dx;
+                v[CH + G_CONIC + 1] = v_sigma * dx * dy;
+                v[CH + G_CONIC + 2] = 0.5f * v_sigma * dy * dy;
+                float g_x = v_sigma * row_x, g_y = v_sigma * row_y;
+                if constexpr (LIDAR) {
+                    // gradient of the depth channel value, under the same clamp rule
+                    const float g_depth = au_g != 0.f ? fac * v_out_depth : 0.f;
+                    v[CH + G_DC] = g_depth * dx;
+                    v[CH + G_DC + 1] = g_depth * dy;
+                    v[CH + G_VELZ] = g_depth * roll;
+                    g_x += g_depth * ext.y;
+                    g_y += g_depth * ext.z;
+                }
+                float g_ax = fabsf(g_x), g_ay = fabsf(g_y);
+                v[CH + G_OPAC] = au_g * rop * v_alpha;
+#pragma unroll
+                for (int k = 0; k < CH; ++k) buffer[k] += s_col[t * CH + k] * fac;
+                if constexpr (LIDAR) {
+                    buffer_extra += extra * fac;
+                    if (a.compute_alpha_sum) { // uniform
+                        const float au_s = (valid && ext.w < pz - a.threshold) ? au : 0.f;
+                        const float v_sig2 = -v_asum * au_s;
+                        const float ex = v_sig2 * row_x, ey = v_sig2 * row_y;
+                        g_x += ex; g_y += ey;
+                        g_ax += fabsf(ex); g_ay += fabsf(ey);
+                        v[CH + G_CONIC] += v_sig2 * 0.5f * dx * dx;
+                        v[CH + G_CONIC + 1] += v_sig2 * dx * dy;
+                        v[CH + G_CONIC + 2] += v_sig2 * 0.5f * dy * dy;
+                        v[CH + G_OPAC] += v_asum * au_s * rop;
+                    }
+                }
+                v[CH + G_XY] = g_x;
+                v[CH + G_XY + 1] = g_y;
+                v[CH + G_ABS] = g_ax;
+                v[CH + G_ABS + 1] = g_ay;
+                v[CH + G_VEL] = g_x * roll;
+                v[CH + G_VEL + 1] = g_y * roll;
                 // sum over the wavefront; the lane that ends up with slot s adds it in LDS
                 wave_reduce_scatter<NV>(v, lane);
                 const int slot = wave_reduce_slot<NV>(lane);
@@ -290,8 +297,19 @@ rasterize_bwd_kernel(BwdArgs a) {
         }
         __syncthreads();
 
-        // flush the batch: lane tr owns Gaussian tr of the batch
-        if ((int32_t)tr < batch_size) {
+        // Flush the batch.  Global atomics are served per memory request, about one per clock and
+        // L2 channel, so what counts is how many requests an instruction spreads over: with the
+        // packed layout the slots of one Gaussian are neighbours in memory and in the wavefront
+        // (lane = (Gaussian, slot)), and a Gaussian costs one or two requests instead of one per
+        // value.
+        if (a.packed != nullptr) {
+            for (uint32_t idx = tr; idx < (uint32_t)batch_size * ACC; idx += block_size) {
+                const uint32_t t = idx / ACC, slot = idx - t * ACC;
+                const float val = s_acc[idx];
+                if (val != 0.f)
+                    atomicAdd(a.packed + (size_t)__float_as_int(s_aux[t].x) * a.packed_stride + slot, val);
+            }
+        } else if ((int32_t)tr < batch_size) { // lane tr owns Gaussian tr of the batch
             const int32_t g = __float_as_int(s_aux[tr].x);
             const float *acc = s_acc + (size_t)tr * ACC;
             float *vc = a.v_colors + (size_t)g * a.color_stride + a.ch_offset;
@@ -325,6 +343,40 @@ rasterize_bwd_kernel(BwdArgs a) {
             }
         }
     }
+}
+
+// Adds the packed gradients of one channel pass into the arrays of the interface: one thread
+// per (Gaussian, slot), `width` colour slots (the first n_ch of them in use) followed by the
+// geometry slots.  Every output element has exactly one writer.
+template <bool LIDAR>
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+unpack_gradients_kernel(uint64_t total, uint32_t stride, uint32_t width, BwdArgs a) {
+    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total * stride) return;
+    const uint64_t g = idx / stride;
+    const uint32_t slot = (uint32_t)(idx - g * stride);
+    constexpr uint32_t GEO = LIDAR ? G_COUNT : G_VELZ;
+    if (slot >= width + GEO) return;
+    const float val = a.packed[idx];
+    if (val == 0.f) return;
+    if (slot < width) {
+        if (slot < a.n_ch) a.v_colors[g * a.color_stride + a.ch_offset + slot] += val;
+        return;
+    }
+    const uint32_t geo = slot - width;
+    constexpr uint32_t nv = LIDAR ? 3 : 2;
+    if (geo < G_XY) a.v_conics[g * 3 + geo] += val;
+    else if (geo < G_ABS) a.v_means2d[g * 2 + (geo - G_XY)] += val;
+    else if (geo < G_VEL) { if (a.v_means2d_abs != nullptr) a.v_means2d_abs[g * 2 + (geo - G_ABS)] += val; }
+    else if (geo < G_OPAC) a.v_pix_vels[g * nv + (geo - G_VEL)] += val;
+    else if (geo == G_OPAC) a.v_opacities[g] += val;
+    else if (geo == G_VELZ) a.v_pix_vels[g * 3 + 2] += val;
+    else a.v_depth_comps[g * 2 + (geo - G_DC)] += val;
+}
+
+__global__ void __launch_bounds__(SPLATAD_THREADS) fill_zero_f32x4_kernel(float4 *p, uint64_t n4) {
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n4) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
 constexpr int kWidths[] = {1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33};
@@ -368,20 +420,57 @@ static int dispatch_bwd(int w, const BwdArgs &a, dim3 grid, dim3 block, hipStrea
     return -1;
 }
 
-template <bool LIDAR>
-static int run_passes(BwdArgs &a, uint32_t channels, dim3 grid, dim3 block, hipStream_t stream) {
+// Floats per Gaussian of the packed accumulation buffer: the widest pass plus the geometry
+// slots, in whole 64-byte lines.
+static uint32_t packed_stride(uint32_t channels, bool lidar) {
     const uint32_t pass = channels <= (uint32_t)kMaxPass ? channels : 32u;
+    const uint32_t acc = (uint32_t)pick_width(pass) + (lidar ? G_COUNT : G_VELZ);
+    return (acc + 15u) / 16u * 16u;
+}
+
+template <bool LIDAR>
+static int run_passes(BwdArgs &a, uint32_t channels, dim3 grid, dim3 block, uint64_t total,
+                      void *workspace, size_t workspace_bytes, hipStream_t stream) {
+    const uint32_t pass = channels <= (uint32_t)kMaxPass ? channels : 32u;
+    const uint32_t stride = packed_stride(channels, LIDAR);
+    a.packed = nullptr;
+    if (workspace != nullptr) {
+        SPLATAD_REQUIRE(total > 0 && total < (1ull << 31), "rasterize backward: bad number of Gaussians");
+        SPLATAD_REQUIRE(workspace_bytes >= total * stride * sizeof(float),
+                        "rasterize backward: workspace of %zu bytes, %zu needed", workspace_bytes,
+                        (size_t)(total * stride * sizeof(float)));
+        SPLATAD_REQUIRE(((uintptr_t)workspace & 15) == 0, "rasterize backward: workspace is not 16-byte aligned");
+        a.packed = reinterpret_cast<float *>(workspace);
+        a.packed_stride = stride;
+    }
     for (uint32_t off = 0; off < channels; off += pass) {
         a.ch_offset = off;
         a.n_ch = min(pass, channels - off);
         a.first_pass = off == 0;
-        int rc = dispatch_bwd<LIDAR>(pick_width(a.n_ch), a, grid, block, stream);
+        const int width = pick_width(a.n_ch);
+        if (a.packed != nullptr) {
+            const uint64_t n4 = total * stride / 4;
+            hipLaunchKernelGGL(fill_zero_f32x4_kernel, dim3((uint32_t)((n4 + SPLATAD_THREADS - 1) / SPLATAD_THREADS)),
+                               dim3(SPLATAD_THREADS), 0, stream, reinterpret_cast<float4 *>(a.packed), n4);
+            SPLATAD_LAUNCH_CHECK();
+        }
+        int rc = dispatch_bwd<LIDAR>(width, a, grid, block, stream);
         if (rc) return rc;
+        if (a.packed != nullptr) {
+            const uint64_t n = total * stride;
+            hipLaunchKernelGGL(unpack_gradients_kernel<LIDAR>, dim3((uint32_t)((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS)),
+                               dim3(SPLATAD_THREADS), 0, stream, total, stride, (uint32_t)width, a);
+            SPLATAD_LAUNCH_CHECK();
+        }
     }
     return 0;
 }
 
 } // namespace
+
+extern "C" size_t splatad_rasterize_bwd_workspace_bytes(uint64_t total, uint32_t channels, int lidar) {
+    return (size_t)(total * packed_stride(channels ? channels : 1, lidar != 0) * sizeof(float));
+}
 
 extern "C" int splatad_rasterize_to_pixels_bwd(
     uint32_t C, int64_t n_isects, uint32_t channels, const float *means2d, const float *conics,
@@ -390,7 +479,8 @@ extern "C" int splatad_rasterize_to_pixels_bwd(
     uint32_t tile_h, const int32_t *tile_offsets, const int32_t *flatten_ids,
     const float *render_alphas, const int32_t *last_ids, const float *v_render_colors,
     const float *v_render_alphas, float *v_means2d_abs, float *v_means2d, float *v_conics,
-    float *v_colors, float *v_opacities, float *v_pix_vels, splatad_stream_t stream) {
+    float *v_colors, float *v_opacities, float *v_pix_vels, uint64_t total, void *workspace,
+    size_t workspace_bytes, splatad_stream_t stream) {
     SPLATAD_REQUIRE(channels >= 1, "rasterize_to_pixels bwd: zero channels");
     SPLATAD_REQUIRE(tile_size >= 1 && tile_size * tile_size <= 256,
                     "rasterize_to_pixels bwd: tile_size %u is outside 1..16", tile_size);
@@ -413,7 +503,8 @@ extern "C" int splatad_rasterize_to_pixels_bwd(
     a.v_means2d_abs = v_means2d_abs; a.v_means2d = v_means2d; a.v_conics = v_conics;
     a.v_colors = v_colors; a.v_opacities = v_opacities; a.v_pix_vels = v_pix_vels;
     return run_passes<false>(a, channels, dim3(C * tile_w * tile_h),
-                             dim3((tile_size * tile_size + 63) / 64 * 64), (hipStream_t)stream);
+                             dim3((tile_size * tile_size + 63) / 64 * 64), total, workspace,
+                             workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int splatad_rasterize_to_points_bwd(
@@ -425,8 +516,8 @@ extern "C" int splatad_rasterize_to_points_bwd(
     const int32_t *flatten_ids, uint32_t depth_idx, const float *render_alphas,
     const int32_t *last_ids, const float *v_render_colors, const float *v_render_alphas,
     const float *v_alpha_sum, float *v_means2d_abs, float *v_means2d, float *v_conics,
-    float *v_colors, float *v_opacities, float *v_pix_vels, float *v_depth_comps,
-    splatad_stream_t stream) {
+    float *v_colors, float *v_opacities, float *v_pix_vels, float *v_depth_comps, uint64_t total,
+    void *workspace, size_t workspace_bytes, splatad_stream_t stream) {
     SPLATAD_REQUIRE(channels >= 1, "rasterize_to_points bwd: zero channels");
     SPLATAD_REQUIRE(depth_idx < channels, "rasterize_to_points bwd: depth channel %u of %u", depth_idx, channels);
     SPLATAD_REQUIRE(tile_width >= 1 && tile_height >= 1 && tile_width * tile_height <= 256,
@@ -453,5 +544,6 @@ extern "C" int splatad_rasterize_to_points_bwd(
     a.v_colors = v_colors; a.v_opacities = v_opacities; a.v_pix_vels = v_pix_vels;
     a.v_depth_comps = v_depth_comps;
     return run_passes<true>(a, channels, dim3(C * grid_w * grid_h),
-                            dim3((tile_width * tile_height + 63) / 64 * 64), (hipStream_t)stream);
+                            dim3((tile_width * tile_height + 63) / 64 * 64), total, workspace,
+                            workspace_bytes, (hipStream_t)stream);
 }

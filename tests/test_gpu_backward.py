@@ -239,7 +239,7 @@ def test_rasterize_to_pixels_absgrad():
     assert_grad_close(to_np(m.grad), torch.autograd.grad(per_pixel.sum(), rm)[0].numpy(), "means2d")
 
 
-@pytest.mark.parametrize("D,asum", [(5, True), (5, False), (33, True), (36, True)])
+@pytest.mark.parametrize("D,asum", [(5, True), (5, False), (33, True), (36, True), (2, True), (3, False)])
 def test_rasterize_to_points_backward(D, asum):
     from splatad_amd import isect_lidar_tiles, isect_offset_encode, rasterize_to_points
     H, W, tw, th = 8, 128, 32, 4
