@@ -118,6 +118,13 @@ __device__ __forceinline__ uint64_t wave_ballot(bool pred) {
     return __builtin_amdgcn_ballot_w64(pred);
 }
 
+// The reverse: a per-lane predicate from a lane mask held in scalar registers (free: the
+// hardware keeps predicates as such masks).  Predicates that are combined with scalar logic on
+// their masks cost no vector instructions, and "no lane left" is a scalar compare.
+__device__ __forceinline__ bool wave_lanes(uint64_t mask) {
+    return __builtin_amdgcn_inverse_ballot_w64(mask);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, SPLATAD_WAVE);

@@ -95,6 +95,7 @@ rasterize_bwd_kernel(BwdArgs a) {
         roll = a.rs_time[cam] * ((py - 0.5f) / (float)(a.H - 1) - 0.5f);
     }
     const bool inside = in_image && pz > 0.f;
+    const uint64_t inside_bits = wave_ballot(inside);
 
     // lidar: angles relative to the tile's first valid point, as in the forward kernel
     float ref_x = 0.f, ref_y = 0.f;
@@ -213,9 +214,11 @@ rasterize_bwd_kernel(BwdArgs a) {
                 const float power = dx * (e.x * dx + e.y * dy) + e.z * dy * dy;
                 const float au = __builtin_amdgcn_exp2f(e.w - power); // opacity * exp(-sigma)
                 const float alpha = fminf(0.999f, au);
-                const bool valid = inside && (batch_end - t <= bin_final) && !(power < 0.f) &&
-                                   !(alpha < 1.f / 255.f);
-                if (wave_ballot(valid) == 0) continue;
+                // the lanes that took this Gaussian in the forward pass, by scalar logic on lane masks
+                const uint64_t valid_bits = inside_bits & wave_ballot(batch_end - t <= bin_final) &
+                                            wave_ballot(!(power < 0.f)) & wave_ballot(!(alpha < 1.f / 255.f));
+                if (valid_bits == 0) continue;
+                const bool valid = wave_lanes(valid_bits);
 
                 // Branch-free from here on: a lane that does not take this Gaussian runs the same
                 // arithmetic with alpha = 0 and alpha-before-clamping = 0, which makes every

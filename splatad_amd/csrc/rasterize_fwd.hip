@@ -59,7 +59,9 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     const float px = (float)j + 0.5f, py = (float)i + 0.5f;
     const float roll = a.rs_time[cam] * ((py - 0.5f) / (float)(a.H - 1) - 0.5f);
     const bool inside = (i < a.H && j < a.W);
-    bool alive = inside; // still compositing
+    // lanes still compositing, as a lane mask: the decisions of the inner loop are taken with
+    // scalar logic on such masks
+    uint64_t alive_bits = wave_ballot(inside);
 
     const int32_t *offs = a.tile_offsets + (size_t)cam * tiles_per_cam;
     const int32_t range_start = offs[tile_id];
@@ -80,7 +82,7 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
 
     for (uint32_t b = 0; b < num_batches; ++b) {
         // also orders the previous batch's LDS reads before this batch's writes
-        if (__syncthreads_count(!alive) >= (int)block_size) break;
+        if (__syncthreads_count(!wave_lanes(alive_bits)) >= (int)block_size) break;
 
         const uint32_t batch_start = (uint32_t)range_start + block_size * b;
         const uint32_t idx = batch_start + tr;
@@ -99,7 +101,7 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
         __syncthreads();
 
         const uint32_t batch_size = min(block_size, (uint32_t)range_end - batch_start);
-        for (uint32_t base = 0; base < batch_size && wave_ballot(alive); base += SPLATAD_WAVE) {
+        for (uint32_t base = 0; base < batch_size && alive_bits != 0; base += SPLATAD_WAVE) {
             // lanes test 64 Gaussians against the wavefront's footprint, then all lanes walk
             // the survivors (a wave-uniform loop over the set bits)
             bool keep = base + lane < batch_size;
@@ -118,18 +120,20 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
                 const float weight = alpha * T;
                 const float next_T = T - weight; // T (1 - alpha)
                 // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
-                const bool valid = alive && !(power < 0.f) && !(alpha < 1.f / 255.f);
-                const bool stop = valid && next_T <= 1e-4f;
-                const bool take = valid && !stop;
-                alive = alive && !stop;
+                const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
+                                            wave_ballot(!(alpha < 1.f / 255.f));
+                const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
+                const uint64_t take_bits = valid_bits & ~stop_bits;
+                alive_bits &= ~stop_bits;
+                const bool take = wave_lanes(take_bits);
                 const float vis = take ? weight : 0.f;
-                if (CH > 8 ? wave_ballot(take) != 0 : true) {
+                if (CH > 8 ? take_bits != 0 : true) {
 #pragma unroll
                     for (int k = 0; k < CH; ++k) out[k] += reinterpret_cast<const float *>(rec + 2)[k] * vis;
                 }
                 cur_idx = take ? batch_start + t : cur_idx;
                 T -= vis;
-                // whether the whole wavefront is done is looked at once per 64 candidates, above
+                if (alive_bits == 0) break;
             }
         }
     }
@@ -196,7 +200,7 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
         px = p.x; py = p.y; pz = p.z; roll = p.w;
     }
     const bool inside = in_image && pz > 0.f;
-    bool alive = inside;
+    uint64_t alive_bits = wave_ballot(inside); // lanes still compositing, as in the pixel kernel
 
     // reference point of the tile: its first valid point
     if (tr == 0) s_ref_thread = 0xFFFFFFFFu;
@@ -220,7 +224,7 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
 
     // footprint of this wavefront over its valid lanes
     WavePointCull cull;
-    cull.init(alive, rx, ry, roll, block_size % SPLATAD_WAVE == 0);
+    cull.init(inside, rx, ry, roll, block_size % SPLATAD_WAVE == 0);
 
     float T = 1.0f, asum = 0.f, median = 0.f, depth_extra = 0.f;
     uint32_t cur_idx = 0;
@@ -230,7 +234,7 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
 
     for (uint32_t b = 0; b < num_batches; ++b) {
         // also orders the previous batch's LDS reads before this batch's writes
-        if (__syncthreads_count(!alive) >= (int)block_size) break;
+        if (__syncthreads_count(!wave_lanes(alive_bits)) >= (int)block_size) break;
         const uint32_t batch_start = (uint32_t)range_start + block_size * b;
         const uint32_t idx = batch_start + tr;
         if (idx < (uint32_t)range_end) {
@@ -252,7 +256,7 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
         __syncthreads();
 
         const uint32_t batch_size = min(block_size, (uint32_t)range_end - batch_start);
-        for (uint32_t base = 0; base < batch_size && wave_ballot(alive); base += SPLATAD_WAVE) {
+        for (uint32_t base = 0; base < batch_size && alive_bits != 0; base += SPLATAD_WAVE) {
             bool keep = base + lane < batch_size, unfolded_ok = true;
             if (keep) keep = cull.may_touch(s_rec[RECORD * (base + lane)], s_rec[RECORD * (base + lane) + 1], unfolded_ok);
             uint64_t todo = wave_ballot(keep);
@@ -275,11 +279,13 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
                 const float weight = alpha * T;
                 const float next_T = T - weight; // T (1 - alpha)
                 // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
-                const bool valid = alive && !(power < 0.f) && !(alpha < 1.f / 255.f);
-                const bool stop = valid && next_T <= 1e-4f;
-                const bool take = valid && !stop;
-                alive = alive && !stop;
-                if (wave_ballot(take) != 0) {
+                const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
+                                            wave_ballot(!(alpha < 1.f / 255.f));
+                const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
+                const uint64_t take_bits = valid_bits & ~stop_bits;
+                alive_bits &= ~stop_bits;
+                if (take_bits != 0) {
+                    const bool take = wave_lanes(take_bits);
                     const float vis = take ? weight : 0.f;
 #pragma unroll
                     for (int k = 0; k < CH; ++k) out[k] += reinterpret_cast<const float *>(rec + 3)[k] * vis;
@@ -291,7 +297,7 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
                     cur_idx = take ? batch_start + t : cur_idx;
                     T -= vis;
                 }
-                // whether the whole wavefront is done is looked at once per 64 candidates, above
+                if (alive_bits == 0) break;
             }
         }
     }

@@ -90,7 +90,7 @@ rasterize_to_indices_kernel(IndexArgs a) {
     } else {
         roll = a.rs_time[cam] * ((py - 0.5f) / (float)(a.H - 1) - 0.5f);
     }
-    bool alive = inside;
+    uint64_t alive_bits = wave_ballot(inside); // lanes still compositing, as in the compositing kernels
 
     const int32_t *offs = a.tile_offsets + (size_t)cam * tiles_per_cam;
     const int32_t list_start = offs[tile_id];
@@ -104,7 +104,7 @@ rasterize_to_indices_kernel(IndexArgs a) {
     WaveCull cull;
     WavePointCull pcull;
     const bool full = block_size % SPLATAD_WAVE == 0;
-    if (LIDAR) pcull.init(alive, px, py, roll, full);
+    if (LIDAR) pcull.init(inside, px, py, roll, full);
     else cull.init(px, py, roll, full);
 
     float T = inside ? a.transmittances[pix] : 0.f;
@@ -118,7 +118,7 @@ rasterize_to_indices_kernel(IndexArgs a) {
 
     for (uint32_t b = a.range_start; b < batch_end; ++b) {
         // also orders the previous batch's LDS reads before this batch's writes
-        if (__syncthreads_count(!alive) >= (int)block_size) break;
+        if (__syncthreads_count(!wave_lanes(alive_bits)) >= (int)block_size) break;
         const uint32_t batch_start = (uint32_t)list_start + block_size * b;
         const uint32_t idx = batch_start + tr;
         if (idx < (uint32_t)list_end) {
@@ -135,7 +135,7 @@ rasterize_to_indices_kernel(IndexArgs a) {
         __syncthreads();
 
         const uint32_t batch_size = min(block_size, (uint32_t)list_end - batch_start);
-        for (uint32_t base = 0; base < batch_size && wave_ballot(alive); base += SPLATAD_WAVE) {
+        for (uint32_t base = 0; base < batch_size && alive_bits != 0; base += SPLATAD_WAVE) {
             bool keep = base + lane < batch_size, unfolded_ok = true;
             if (keep) {
                 const float4 r0 = s_rec[2 * (base + lane)], r1 = s_rec[2 * (base + lane) + 1];
@@ -158,11 +158,11 @@ rasterize_to_indices_kernel(IndexArgs a) {
                 const float power = dx * (con.x * dx + con.y * dy) + con.z * dy * dy;
                 const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
                 const float next_T = T - alpha * T; // as in the compositing kernels
-                const bool valid = alive && !(power < 0.f) && !(alpha < 1.f / 255.f);
-                const bool stop = valid && next_T <= 1e-4f;
-                const bool take = valid && !stop;
-                alive = alive && !stop;
-                if (take) {
+                const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
+                                            wave_ballot(!(alpha < 1.f / 255.f));
+                const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
+                alive_bits &= ~stop_bits;
+                if (wave_lanes(valid_bits & ~stop_bits)) {
                     if (WRITE) {
                         out_g[cnt] = (int64_t)s_id[t];
                         out_i[cnt] = (int64_t)pix;
@@ -170,7 +170,7 @@ rasterize_to_indices_kernel(IndexArgs a) {
                     ++cnt;
                     T = next_T;
                 }
-                if (wave_ballot(alive) == 0) break;
+                if (alive_bits == 0) break;
             }
         }
     }
