@@ -81,9 +81,14 @@ int splatad_lidar_projection_fwd(uint32_t C, uint32_t N, const float *means, con
                                  splatad_stream_t stream);
 
 /* fully_fused_projection_bwd_tensor, projection.cu:1047-1155 (kernel :753-964).
- * Gradient outputs must be zero-filled by the caller; v_covars xor (v_quats,
- * v_scales); v_viewmats and v_velocities may be NULL.  v_velocities is an
- * extension: the reference computes and drops it (projection.cu:874-877). */
+ * v_covars xor (v_quats, v_scales); v_viewmats and v_velocities may be NULL.
+ * Unpacked input (camera_ids == NULL): every row of v_means, v_covars, v_quats,
+ * v_scales and v_velocities is stored, summed over the sensors in a fixed order
+ * (no atomics: the same bits on every run); only v_viewmats is accumulated into and
+ * must be zero-filled by the caller.  Packed input: all gradient outputs must be
+ * zero-filled by the caller.  The same holds for splatad_lidar_projection_bwd, whose
+ * input is always unpacked.  v_velocities is an extension: the reference computes and
+ * drops it (projection.cu:874-877). */
 int splatad_projection_bwd(uint32_t C, uint32_t N, const float *means, const float *covars,
                            const float *quats, const float *scales, const float *velocities,
                            const float *viewmats, const float *Ks, uint32_t image_width,

@@ -20,6 +20,7 @@
 // Built with -ffp-contract=off: the tile bounds are float32 expressions whose rounding
 // decides which tiles a Gaussian touches.
 #include "common.h"
+#include "host_word.h"
 #include "scan.h"
 
 #include <mutex>
@@ -935,7 +936,7 @@ static inline dim3 grid_for(uint64_t n) {
 struct IsectDevice {
     hipStream_t aux[2];
     hipEvent_t fork, join[2];
-    unsigned long long *n_host, *n_device; // pinned slot: host address, address for kernels
+    HostWord n; // carries the number of intersections to the host
     std::mutex guard;
 };
 
@@ -951,8 +952,7 @@ static int isect_device(IsectDevice **out) {
         for (hipStream_t &a : s->aux) SPLATAD_CHECK_HIP(hipStreamCreateWithFlags(&a, hipStreamNonBlocking));
         SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->fork, hipEventDisableTiming));
         for (hipEvent_t &e : s->join) SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-        SPLATAD_CHECK_HIP(hipHostMalloc((void **)&s->n_host, 64, hipHostMallocDefault));
-        SPLATAD_CHECK_HIP(hipHostGetDevicePointer((void **)&s->n_device, s->n_host, 0));
+        if (int rc = host_word_create(&s->n)) return rc;
         table[dev] = s;
     }
     *out = table[dev];
@@ -1016,41 +1016,23 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
                     "isect: camera and tile ids need more than 32 bits");
     IsectWorkspace w;
     carve_isect(workspace, total, pl.segs, sort ? pl.cslots : 0, &w);
-    // the host waits for the count below, which a stream under graph capture would never deliver
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    SPLATAD_CHECK_HIP(hipStreamIsCapturing(stream, &capturing));
-    SPLATAD_REQUIRE(capturing == hipStreamCaptureStatusNone,
-                    "isect: the counting call returns a number to the host and cannot be captured in a graph");
+    if (int rc = host_word_refuse_capture(stream, "isect")) return rc;
     IsectDevice *dv = nullptr;
     if (int rc = isect_device(&dv)) return rc;
     std::lock_guard<std::mutex> lock(dv->guard);
-    volatile unsigned long long *slot = dv->n_host;
-    const unsigned long long pending = ~0ull;
-    *slot = pending;
+    *(volatile unsigned long long *)dv->n.host = kHostWordPending;
     hipLaunchKernelGGL(fill_zero_u64_kernel, dim3(1), dim3(2), 0, stream, w.n_isects);
     dim3 count_grid = grid_for(total);
     if (count_grid.x > 512) count_grid.x = 512;
     hipLaunchKernelGGL(isect_count_kernel<LIDAR>, count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
-                       total, means2d, radii, tiles_per_gauss, w.n_isects, dv->n_device);
+                       total, means2d, radii, tiles_per_gauss, w.n_isects, dv->n.device);
     SPLATAD_LAUNCH_CHECK();
     // work for the GPU while the host learns the count and sizes the lists
     if (sort)
         if (int rc = enqueue_coarse_count<LIDAR>(g, pl, w, total, N, camera_ids, means2d, radii, C, stream))
             return rc;
-    // wait for the counting kernel's word only, not for the work behind it; now and then ask
-    // the stream, so that a failed launch or a fault ends the wait with its error
-    unsigned long long n = pending;
-    for (uint32_t spin = 1; (n = *slot) == pending; ++spin) {
-        __builtin_ia32_pause();
-        if ((spin & 0xFFFFu) == 0) {
-            const hipError_t q = hipStreamQuery(stream);
-            if (q == hipErrorNotReady) { (void)hipGetLastError(); continue; }
-            SPLATAD_CHECK_HIP(q);
-            n = *slot; // the stream has drained: the word is there, or never will be
-            SPLATAD_REQUIRE(n != pending, "isect: the counting kernel left no result");
-            break;
-        }
-    }
+    unsigned long long n = 0;
+    if (int rc = host_word_wait(&dv->n, stream, "isect", &n)) return rc;
     SPLATAD_REQUIRE(n < (1ull << 31), "isect: %llu intersections exceed the int32 offset range", n);
     *n_isects_host = (int64_t)n;
     return 0;

@@ -10,6 +10,7 @@
 // (lidar) of the reference, except that rows of culled Gaussians are written as zeros
 // instead of being left uninitialised.
 #include "common.h"
+#include "host_word.h"
 #include "scan.h"
 
 #define RAD_TO_DEG 57.2957795131f
@@ -411,6 +412,26 @@ extern "C" int splatad_lidar_projection_fwd(uint32_t C, uint32_t N, const float 
     return 0;
 }
 
+// The pinned word through which the number of kept (camera, Gaussian) pairs reaches the host,
+// one per device, with the mutex that serialises its users.
+static int packed_host_word(HostWord **word, std::mutex **guard) {
+    static std::mutex table_guard;
+    static HostWord *table[64] = {};
+    static std::mutex guards[64];
+    int dev = 0;
+    SPLATAD_CHECK_HIP(hipGetDevice(&dev));
+    SPLATAD_REQUIRE(dev >= 0 && dev < 64, "packed projection: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(table_guard);
+    if (!table[dev]) {
+        HostWord *w = new HostWord();
+        if (int rc = host_word_create(w)) { delete w; return rc; }
+        table[dev] = w;
+    }
+    *word = table[dev];
+    *guard = &guards[dev];
+    return 0;
+}
+
 extern "C" size_t splatad_projection_packed_workspace_bytes(uint32_t C, uint32_t N) {
     const uint64_t T = (uint64_t)C * N;
     return 256 + splatad_align256(T * 8) * 3 + splatad_align256(T * 4) * 3 +
@@ -429,6 +450,12 @@ extern "C" int splatad_projection_packed_count(
     SPLATAD_REQUIRE(workspace != nullptr, "packed projection: workspace is null");
     const uint64_t T = (uint64_t)C * N;
     PackedWorkspace w = carve_packed(workspace, T);
+    if (int rc = host_word_refuse_capture((hipStream_t)stream, "packed projection")) return rc;
+    HostWord *pw = nullptr;
+    std::mutex *guard = nullptr;
+    if (int rc = packed_host_word(&pw, &guard)) return rc;
+    std::lock_guard<std::mutex> lock(*guard);
+    *(volatile unsigned long long *)pw->host = kHostWordPending;
     int rc = splatad_projection_fwd(C, N, means, covars, quats, scales, velocities, viewmats, Ks,
                                     W, H, lin_vel, ang_vel, rs_time, eps2d, near_plane, far_plane,
                                     radius_clip, w.radii, w.means2d, w.depths, w.conics,
@@ -437,9 +464,13 @@ extern "C" int splatad_projection_packed_count(
     rc = launch_exclusive_scan<int32_t>(w.radii, (int64_t)T, 2, 1, w.pos, w.total, w.block_sums,
                                         (hipStream_t)stream);
     if (rc) return rc;
-    SPLATAD_CHECK_HIP(hipMemcpyAsync(nnz_host, w.total, sizeof(int64_t), hipMemcpyDeviceToHost,
-                                     (hipStream_t)stream));
-    SPLATAD_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
+    hipLaunchKernelGGL(host_word_publish_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, w.total,
+                       pw->device);
+    SPLATAD_LAUNCH_CHECK();
+    unsigned long long nnz = 0;
+    rc = host_word_wait(pw, (hipStream_t)stream, "packed projection", &nnz);
+    if (rc) return rc;
+    *nnz_host = (int64_t)nnz;
     return 0;
 }
 

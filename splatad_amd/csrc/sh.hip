@@ -132,11 +132,20 @@ __device__ __forceinline__ bool sh_row(uint32_t e, const ShView &v, const float 
     const uint32_t g = v.gaussian_ids ? (uint32_t)v.gaussian_ids[e] : e % v.N;
     const uint32_t cam = v.camera_ids ? (uint32_t)v.camera_ids[e] : e / v.N;
     coeff_row = v.coeffs_per_sensor ? (v.camera_ids ? (size_t)cam * v.N + g : (size_t)e) : (size_t)g;
-    if (v.radii[(size_t)e * 2] <= 0) return false;
+    // the mean is requested together with the radius, not after the test on it
+    const int32_t radius = v.radii[(size_t)e * 2];
+    const float mx = v.means[(size_t)g * 3], my = v.means[(size_t)g * 3 + 1], mz = v.means[(size_t)g * 3 + 2];
     float px, py, pz;
     sensor_position(v.viewmats + (size_t)cam * 16, px, py, pz);
-    dx = v.means[(size_t)g * 3] - px; dy = v.means[(size_t)g * 3 + 1] - py; dz = v.means[(size_t)g * 3 + 2] - pz;
-    return true;
+    dx = mx - px; dy = my - py; dz = mz - pz;
+    return radius > 0;
+}
+
+// The coefficients of band L (bases L^2 .. (L+1)^2 - 1) of one row
+template <int L>
+__device__ __forceinline__ void sh_load_band(float *c, const float *__restrict__ cf) {
+#pragma unroll
+    for (int f = 3 * L * L; f < 3 * (L + 1) * (L + 1); ++f) c[f] = cf[f];
 }
 
 // Forward: every lane reads its own row; the rows are read completely, so the cache lines a
@@ -156,11 +165,17 @@ sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, ShView view, const float 
     if (sh_row<VIEW>(e, view, dirs, masks, dx, dy, dz, coeff_row)) {
         const float inorm = rsqrtf(dx * dx + dy * dy + dz * dz);
         const float *cf = coeffs + coeff_row * K * 3;
+        float c[75]; // the whole row is requested before the first use: one memory round trip
+        sh_load_band<0>(c, cf);
+        if (degree >= 1) sh_load_band<1>(c, cf); // uniform
+        if (degree >= 2) sh_load_band<2>(c, cf);
+        if (degree >= 3) sh_load_band<3>(c, cf);
+        if (degree >= 4) sh_load_band<4>(c, cf);
         sh_for_each_basis(degree, dx * inorm, dy * inorm, dz * inorm,
                           [&](int k, float v, float, float, float) {
-                              r += v * cf[k * 3];
-                              g += v * cf[k * 3 + 1];
-                              b += v * cf[k * 3 + 2];
+                              r += v * c[k * 3];
+                              g += v * c[k * 3 + 1];
+                              b += v * c[k * 3 + 2];
                           });
     }
     float *out = colors + (size_t)e * stride;
@@ -176,7 +191,10 @@ sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, ShView view, const float 
 
 // VIEW: v_colors are rows of `stride` floats, the gradients of the activated colours
 // `colors` (same layout), so a channel passes its gradient on only where it is positive.
-template <bool VIEW>
+// DIRS: the gradients of the directions are wanted too.  A compile-time switch, so that the
+// coefficient loads stand outside any branch and the compiler can issue a row's loads together
+// (behind a run-time test each basis function waited for its own three loads).
+template <bool VIEW, bool DIRS>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, ShView view, const float *__restrict__ dirs,
               const float *__restrict__ coeffs, const uint8_t *__restrict__ masks,
@@ -186,7 +204,6 @@ sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, ShView view, const float
     extern __shared__ float s_rows[];
     const uint32_t first = blockIdx.x * blockDim.x;
     const uint32_t here = min(blockDim.x, n - first);
-    const bool want_dirs = v_dirs != nullptr;
     const uint32_t e = first + threadIdx.x;
     // every lane writes its row of coefficient gradients to LDS, from where the workgroup
     // stores them coalesced; rows of masked directions are zeros (their gradients are zero)
@@ -199,24 +216,35 @@ sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, ShView view, const float
         const float inorm = active ? rsqrtf(dx * dx + dy * dy + dz * dz) : 0.f;
         const float x = dx * inorm, y = dy * inorm, z = active ? dz * inorm : 1.f;
         const float *vc = v_colors + (size_t)e * stride;
-        float vr = active ? vc[0] : 0.f, vg = active ? vc[1] : 0.f, vb = active ? vc[2] : 0.f;
+        float vr = vc[0], vg = vc[1], vb = vc[2]; // read whether active or not: no wait for the test
         if (VIEW) {
-            const float *c = colors + (size_t)e * stride;
-            vr = c[0] > 0.f ? vr : 0.f;
-            vg = c[1] > 0.f ? vg : 0.f;
-            vb = c[2] > 0.f ? vb : 0.f;
+            const float *col = colors + (size_t)e * stride;
+            vr = col[0] > 0.f ? vr : 0.f;
+            vg = col[1] > 0.f ? vg : 0.f;
+            vb = col[2] > 0.f ? vb : 0.f;
         }
+        if (!active) vr = vg = vb = 0.f;
         float gx = 0.f, gy = 0.f, gz = 0.f;
+        // the whole coefficient row is requested before the first use, one memory round trip
+        // instead of one per degree
+        float c[DIRS ? 75 : 1] = {};
+        if (DIRS && active) {
+            sh_load_band<0>(c, cf);
+            if (degree >= 1) sh_load_band<1>(c, cf); // uniform
+            if (degree >= 2) sh_load_band<2>(c, cf);
+            if (degree >= 3) sh_load_band<3>(c, cf);
+            if (degree >= 4) sh_load_band<4>(c, cf);
+        }
         sh_for_each_basis(degree, x, y, z, [&](int k, float v, float bx, float by, float bz) {
-            if (want_dirs) {
-                const float w = cf[k * 3] * vr + cf[k * 3 + 1] * vg + cf[k * 3 + 2] * vb;
+            if (DIRS) {
+                const float w = c[k * 3] * vr + c[k * 3 + 1] * vg + c[k * 3 + 2] * vb;
                 gx += w * bx; gy += w * by; gz += w * bz;
             }
             row[k * 3] = v * vr;
             row[k * 3 + 1] = v * vg;
             row[k * 3 + 2] = v * vb;
         });
-        if (want_dirs && (active || VIEW)) {
+        if (DIRS && (active || VIEW)) {
             // through the normalisation: (I - n n^T) g / |d|; zero for inactive rows
             const float dot = gx * x + gy * y + gz * z;
             v_dirs[(size_t)e * 3] = (gx - dot * x) * inorm;
@@ -271,10 +299,16 @@ static int sh_backward(uint32_t n, uint32_t K, uint32_t degree, const ShView &vi
                        hipStream_t stream) {
     const ShRows r = sh_rows(K, degree);
     size_t lds = 0;
-    if (int rc = sh_lds(sh_bwd_kernel<VIEW>, r, &lds)) return rc;
-    hipLaunchKernelGGL(sh_bwd_kernel<VIEW>, dim3((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS),
-                       dim3(SPLATAD_THREADS), lds, stream, n, r, degree, view, dirs, coeffs, masks,
-                       colors, stride, v_colors, v_coeffs, v_dirs);
+    const dim3 grid((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS);
+    if (v_dirs != nullptr) {
+        if (int rc = sh_lds(sh_bwd_kernel<VIEW, true>, r, &lds)) return rc;
+        hipLaunchKernelGGL((sh_bwd_kernel<VIEW, true>), grid, dim3(SPLATAD_THREADS), lds, stream, n, r,
+                           degree, view, dirs, coeffs, masks, colors, stride, v_colors, v_coeffs, v_dirs);
+    } else {
+        if (int rc = sh_lds(sh_bwd_kernel<VIEW, false>, r, &lds)) return rc;
+        hipLaunchKernelGGL((sh_bwd_kernel<VIEW, false>), grid, dim3(SPLATAD_THREADS), lds, stream, n, r,
+                           degree, view, dirs, coeffs, masks, colors, stride, v_colors, v_coeffs, v_dirs);
+    }
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }

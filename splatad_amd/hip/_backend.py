@@ -91,6 +91,17 @@ def _zeros_many(device, *shapes):
     return out
 
 
+def _gathered_outputs(device, means, covars, quats, scales, viewmats, velocities):
+    """Gradient outputs of a projection backward over unpacked input, by shape (None stays None):
+    the kernel stores every per-Gaussian row itself, only the pose gradient is accumulated and
+    has to start at zero."""
+    f = dict(dtype=torch.float32, device=device)
+    out = [None if sh is None else torch.empty(tuple(sh), **f) for sh in (means, covars, quats, scales)]
+    out.append(None if viewmats is None else torch.zeros(tuple(viewmats), **f))
+    out.append(None if velocities is None else torch.empty(tuple(velocities), **f))
+    return out
+
+
 def _zeros_like_many(*tensors):
     ref = next(t for t in tensors if t is not None)
     return _zeros_many(ref.device, *(None if t is None else t.shape for t in tensors))
@@ -248,11 +259,12 @@ class _Ops:
         nnz = camera_ids.shape[0] if packed else 0
         rows = nnz if (packed and sparse_grad) else N
         f = dict(dtype=torch.float32, device=dev)
-        v_means, v_covars, v_quats, v_scales, v_viewmats, v_velocities = _zeros_many(
-            dev, (rows, 3), (rows, 6) if covars is not None else None,
-            (rows, 4) if covars is None else None, (rows, 3) if covars is None else None,
-            viewmats.shape if viewmats_requires_grad else None,
-            velocities.shape if (velocities_requires_grad and velocities is not None) else None)
+        shapes = ((rows, 3), (rows, 6) if covars is not None else None,
+                  (rows, 4) if covars is None else None, (rows, 3) if covars is None else None,
+                  viewmats.shape if viewmats_requires_grad else None,
+                  velocities.shape if (velocities_requires_grad and velocities is not None) else None)
+        v_means, v_covars, v_quats, v_scales, v_viewmats, v_velocities = (
+            _zeros_many(dev, *shapes) if packed else _gathered_outputs(dev, *shapes))
         with torch.cuda.device(dev):
             _check(lib.splatad_projection_bwd(
                 _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
@@ -285,10 +297,11 @@ class _Ops:
         v_pix_vels = _in(v_pix_vels, "v_pix_vels")
         v_dc = _in(v_depth_compensations, "v_depth_compensations")
         N, C, dev = means.shape[0], viewmats.shape[0], means.device
-        v_means, v_covars, v_quats, v_scales, v_viewmats, v_velocities = _zeros_like_many(
-            means, covars, quats if covars is None else None, scales if covars is None else None,
-            viewmats if viewmats_requires_grad else None,
-            velocities if (velocities_requires_grad and velocities is not None) else None)
+        v_means, v_covars, v_quats, v_scales, v_viewmats, v_velocities = _gathered_outputs(
+            dev, *(None if t is None else t.shape for t in (
+                means, covars, quats if covars is None else None, scales if covars is None else None,
+                viewmats if viewmats_requires_grad else None,
+                velocities if (velocities_requires_grad and velocities is not None) else None)))
         with torch.cuda.device(dev):
             _check(lib.splatad_lidar_projection_bwd(
                 _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
