@@ -63,13 +63,12 @@ constexpr uint32_t kElevLds = 1025;
 
 // Tile rectangle of one projected Gaussian: x in [x0, x1), y in [y0, y1).  For lidars x
 // may be negative or exceed tile_w (wrapped at emission).
+// `radii` holds the two words of the Gaussian's radii: int32 for cameras, float for lidars.
 template <bool LIDAR>
-__device__ __forceinline__ bool tile_rect(const TileGrid &g, const float *__restrict__ means2d,
-                                          const void *__restrict__ radii_v, uint64_t idx,
-                                          int32_t &x0, int32_t &y0, int32_t &x1, int32_t &y1) {
-    const float2 mu = reinterpret_cast<const float2 *>(means2d)[idx];
+__device__ __forceinline__ bool tile_rect_of(const TileGrid &g, float2 mu, uint2 radii,
+                                             int32_t &x0, int32_t &y0, int32_t &x1, int32_t &y1) {
     if (!LIDAR) {
-        const int2 r = reinterpret_cast<const int2 *>(radii_v)[idx];
+        const int2 r = make_int2((int32_t)radii.x, (int32_t)radii.y);
         if (r.x <= 0) return false;
         const float ts = (float)g.tile_size;
         const float ex = (float)r.x / ts, ey = (float)r.y / ts;
@@ -79,7 +78,7 @@ __device__ __forceinline__ bool tile_rect(const TileGrid &g, const float *__rest
         x1 = (int32_t)min(f2u_sat(ceilf(tx + ex)), g.tile_w);
         y1 = (int32_t)min(f2u_sat(ceilf(ty + ey)), g.tile_h);
     } else {
-        const float2 r = reinterpret_cast<const float2 *>(radii_v)[idx];
+        const float2 r = make_float2(__uint_as_float(radii.x), __uint_as_float(radii.y));
         if (r.x <= 0.f) return false;
         const float elev_low = mu.y - r.y, elev_high = mu.y + r.y;
         const float azim = mu.x - g.min_azim;
@@ -109,6 +108,20 @@ __device__ __forceinline__ bool tile_rect(const TileGrid &g, const float *__rest
 }
 
 template <bool LIDAR>
+__device__ __forceinline__ bool tile_rect(const TileGrid &g, const float *__restrict__ means2d,
+                                          const void *__restrict__ radii_v, uint64_t idx,
+                                          int32_t &x0, int32_t &y0, int32_t &x1, int32_t &y1) {
+    return tile_rect_of<LIDAR>(g, reinterpret_cast<const float2 *>(means2d)[idx],
+                               reinterpret_cast<const uint2 *>(radii_v)[idx], x0, y0, x1, y1);
+}
+
+// Keeps the compiler from moving the loads of x and y down to their first use behind a
+// branch: both values have to be in registers here.  Emits no instruction.
+__device__ __forceinline__ void loaded_here(float2 &mu, uint2 &r) {
+    asm volatile("" : "+v"(mu.x), "+v"(mu.y), "+v"(r.x), "+v"(r.y));
+}
+
+template <bool LIDAR>
 __device__ __forceinline__ uint32_t tile_index(const TileGrid &g, int32_t y, int32_t x) {
     if (LIDAR) {
         // Mathematical modulo.  For x >= -tile_w this equals (x + tile_w) % tile_w of the
@@ -120,22 +133,46 @@ __device__ __forceinline__ uint32_t tile_index(const TileGrid &g, int32_t y, int
     return (uint32_t)y * g.tile_w + (uint32_t)x;
 }
 
-// Grid-stride: a few hundred workgroups, each ending in one atomic on the total (thousands
-// of atomics on one address would take longer than the rest of the kernel).
+// Grid-stride over the Gaussians.  `counters` (kCountWords words, zeroed) takes the partial
+// sums; the total goes to the host's pinned slot.
+constexpr uint32_t kCountGroups = 32;
+constexpr uint32_t kCountWords = 8 + 8 * kCountGroups;
 template <bool LIDAR>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d,
                    const void *__restrict__ radii, int32_t *__restrict__ tiles_per_gauss,
-                   unsigned long long *__restrict__ n_isects,
+                   unsigned long long *__restrict__ counters,
                    unsigned long long *__restrict__ n_isects_host) {
     SPLATAD_STAGE_ELEVATIONS(g)
     long long s = 0;
-    for (uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-         idx += (uint64_t)gridDim.x * blockDim.x) {
-        int32_t cnt = 0, x0, y0, x1, y1;
-        if (tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) cnt = (y1 - y0) * (x1 - x0);
-        tiles_per_gauss[idx] = cnt;
-        s += cnt;
+    // four Gaussians per lane and step, so that their loads are in flight together (the
+    // kernel is bound by memory latency otherwise)
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i0 = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i0 < total; i0 += 4 * stride) {
+        float2 mu[4];
+        uint2 rad[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint64_t idx = min(i0 + k * stride, total - 1); // in range; unused if clamped
+            mu[k] = reinterpret_cast<const float2 *>(means2d)[idx];
+            rad[k] = reinterpret_cast<const uint2 *>(radii)[idx];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) loaded_here(mu[k], rad[k]);
+        int32_t cnt[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            int32_t x0, y0, x1, y1;
+            cnt[k] = 0;
+            if (i0 + k * stride < total && tile_rect_of<LIDAR>(g, mu[k], rad[k], x0, y0, x1, y1))
+                cnt[k] = (y1 - y0) * (x1 - x0);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint64_t idx = i0 + k * stride;
+            if (idx < total) tiles_per_gauss[idx] = cnt[k];
+            s += cnt[k];
+        }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, SPLATAD_WAVE);
@@ -145,15 +182,28 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
     if (threadIdx.x == 0) {
         long long t = 0;
         for (int w = 0; w < SPLATAD_THREADS / SPLATAD_WAVE; ++w) t += wsum[w];
-        if (t != 0) atomicAdd(n_isects, (unsigned long long)t);
-        // The workgroup that finishes last hands the total to the host, which spins on the
-        // pinned slot: no copy command, no event and no system-scope fence (which would write
-        // back whatever other kernels have dirtied in L2) stand between this kernel and the
-        // host or the work enqueued behind it.  n_isects[1] counts the finished workgroups.
-        __threadfence();
-        if (atomicAdd(n_isects + 1, 1ull) == gridDim.x - 1)
-            __hip_atomic_store(n_isects_host, atomicAdd(n_isects, 0ull), __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_SYSTEM);
+        // A workgroup reports with one atomic that carries both its sum (low 48 bits) and a
+        // count of one (the bits above), so the workgroup that finds everybody else counted
+        // also holds the total and no fence has to order a sum before a counter (a device-scope
+        // release writes back the L2 cache of a multi-die GPU; one per workgroup was most of this
+        // kernel's time).  Atomics of different workgroups on one address are served one after
+        // the other, so the workgroups report in groups (a 64-byte line each, counters + 8 + 8
+        // group) and the last of a group reports the group's sum to the root, counters[0].
+        // The workgroup that finishes last of all hands the total to the host, which spins on
+        // the pinned slot: no copy command, no event and no system-scope fence stand between
+        // this kernel and the host or the work enqueued behind it.
+        const unsigned long long one = 1ull << 48, low = one - 1ull;
+        const uint32_t groups = min(gridDim.x, kCountGroups);
+        const uint32_t group = blockIdx.x % groups;
+        const uint32_t members = gridDim.x / groups + (group < gridDim.x % groups ? 1u : 0u);
+        const unsigned long long before = atomicAdd(counters + 8 + 8 * group, one | (unsigned long long)t);
+        if ((before >> 48) == members - 1) {
+            const unsigned long long group_sum = (before & low) + (unsigned long long)t;
+            const unsigned long long root = atomicAdd(counters, one | group_sum);
+            if ((root >> 48) == groups - 1)
+                __hip_atomic_store(n_isects_host, (root & low) + group_sum, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_SYSTEM);
+        }
     }
 }
 
@@ -209,6 +259,60 @@ __device__ __forceinline__ void for_each_tile_balanced(const LaneWork &mine, Emi
         for (int32_t t = 0; t < mine.cnt; ++t) emit(mine, mine.y0 + t / mine.w, mine.x0 + t % mine.w, t);
 }
 
+// What a lane reads for its work item, and the work item made from it.  Reading and making
+// are separate so that a loop can request the next round's inputs before it works on this
+// round's.
+struct WorkInputs {
+    float2 mu;
+    uint2 radii;
+    uint32_t cam, depth_bits;
+    int64_t cum;
+    uint64_t idx;
+    bool in_range;
+};
+
+__device__ __forceinline__ WorkInputs fetch_work(uint64_t idx, uint64_t total, uint32_t N,
+                                                 const int64_t *__restrict__ camera_ids,
+                                                 const float *__restrict__ means2d,
+                                                 const void *__restrict__ radii,
+                                                 const float *__restrict__ depths,
+                                                 const int64_t *__restrict__ cum_before) {
+    WorkInputs in;
+    in.idx = idx;
+    in.in_range = idx < total;
+    const uint64_t j = in.in_range ? idx : 0; // everything is read, whatever the radius says
+    in.mu = reinterpret_cast<const float2 *>(means2d)[j];
+    in.radii = reinterpret_cast<const uint2 *>(radii)[j];
+    in.cam = camera_of(j, N, camera_ids);
+    in.depth_bits = depths ? __float_as_uint(depths[j]) : 0u;
+    in.cum = cum_before ? cum_before[j] : 0;
+    return in;
+}
+
+template <bool LIDAR>
+__device__ __forceinline__ LaneWork make_work(const TileGrid &g, WorkInputs in) {
+    loaded_here(in.mu, in.radii);
+    LaneWork w;
+    w.x0 = w.y0 = w.cnt = 0;
+    w.w = 1;
+    w.base = 0;
+    w.idx = (uint32_t)in.idx;
+    w.depth_bits = 0;
+    w.cum = 0;
+    w.tx0 = w.ty0 = w.tx1 = w.ty1 = 0;
+    int32_t x0, y0, x1, y1;
+    if (in.in_range && tile_rect_of<LIDAR>(g, in.mu, in.radii, x0, y0, x1, y1)) {
+        w.tx0 = x0; w.ty0 = y0; w.tx1 = x1; w.ty1 = y1;
+        w.x0 = x0; w.y0 = y0;
+        w.w = max(x1 - x0, 1);
+        w.cnt = max(x1 - x0, 0) * max(y1 - y0, 0);
+        w.base = in.cam * g.tile_w * g.tile_h;
+        w.depth_bits = in.depth_bits;
+        w.cum = in.cum;
+    }
+    return w;
+}
+
 template <bool LIDAR>
 __device__ __forceinline__ LaneWork load_work(const TileGrid &g, uint64_t idx, uint64_t total,
                                               uint32_t N, const int64_t *__restrict__ camera_ids,
@@ -216,27 +320,7 @@ __device__ __forceinline__ LaneWork load_work(const TileGrid &g, uint64_t idx, u
                                               const void *__restrict__ radii,
                                               const float *__restrict__ depths,
                                               const int64_t *__restrict__ cum_before) {
-    LaneWork w;
-    w.x0 = w.y0 = w.cnt = 0;
-    w.w = 1;
-    w.base = 0;
-    w.idx = (uint32_t)idx;
-    w.depth_bits = 0;
-    w.cum = 0;
-    w.tx0 = w.ty0 = w.tx1 = w.ty1 = 0;
-    if (idx < total) {
-        int32_t x0, y0, x1, y1;
-        if (tile_rect<LIDAR>(g, means2d, radii, idx, x0, y0, x1, y1)) {
-            w.tx0 = x0; w.ty0 = y0; w.tx1 = x1; w.ty1 = y1;
-            w.x0 = x0; w.y0 = y0;
-            w.w = max(x1 - x0, 1);
-            w.cnt = max(x1 - x0, 0) * max(y1 - y0, 0);
-            w.base = camera_of(idx, N, camera_ids) * g.tile_w * g.tile_h;
-            if (depths) w.depth_bits = __float_as_uint(depths[idx]);
-            if (cum_before) w.cum = cum_before[idx];
-        }
-    }
-    return w;
+    return make_work<LIDAR>(g, fetch_work(idx, total, N, camera_ids, means2d, radii, depths, cum_before));
 }
 
 // Coarse blocks of (1 << bshift) x 4 tiles.  The width is 4 tiles for cameras; for lidars,
@@ -304,10 +388,14 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
     int32_t *row = table + (size_t)blockIdx.x * n_blocks + first;
     for (uint32_t b = threadIdx.x; b < count; b += blockDim.x) s_blocks[b] = FILL ? row[b] : 0;
     __syncthreads();
-    for (uint64_t base = (uint64_t)blockIdx.x * blockDim.x; base < total;
-         base += (uint64_t)gridDim.x * blockDim.x) { // uniform across the workgroup
-        LaneWork mine = load_work<LIDAR>(g, base + threadIdx.x, total, N, camera_ids, means2d,
-                                         radii, FILL ? depths : nullptr, nullptr);
+    const uint64_t round = (uint64_t)gridDim.x * blockDim.x;
+    WorkInputs ahead = fetch_work((uint64_t)blockIdx.x * blockDim.x + threadIdx.x, total, N, camera_ids,
+                                  means2d, radii, FILL ? depths : nullptr, nullptr);
+    for (uint64_t base = (uint64_t)blockIdx.x * blockDim.x; base < total; base += round) { // uniform
+        LaneWork mine = make_work<LIDAR>(g, ahead);
+        // the inputs of the next round are requested before this round's emission
+        ahead = fetch_work(base + round + threadIdx.x, total, N, camera_ids, means2d, radii,
+                           FILL ? depths : nullptr, nullptr);
         const uint32_t cam = mine.base / tiles_per_cam;
         if (cam < cam_lo || cam >= cam_hi) mine.cnt = 0;
         mine.base = (cam - cam_lo) * per_cam;
@@ -750,6 +838,73 @@ __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
     }
 }
 
+// The three upper classes in one launch, longest segments first.  Their workgroups need most
+// of a compute unit's LDS, so even a launch that finds its class empty waits for such a unit to
+// fall free once other sort kernels are running; one launch, enqueued before those, meets an
+// idle GPU and costs next to nothing when the scene has no long segments (the usual case for
+// cameras), while a lidar's long segments all start at once.
+constexpr uint32_t kSortBigThreads = 1024;
+constexpr uint32_t kSortBigInLds = 16384; // class 4 is staged in LDS
+
+__global__ void __launch_bounds__(kSortBigThreads)
+isect_big_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t tile_n_bits,
+                              int64_t n_isects, const uint32_t *__restrict__ seg_counts,
+                              const uint32_t *__restrict__ seg_lists,
+                              const int32_t *__restrict__ tile_starts,
+                              const uint64_t *__restrict__ pairs, int64_t *isect_ids,
+                              int32_t *__restrict__ flatten_ids) {
+    extern __shared__ uint64_t lds_staged[];
+    __shared__ uint32_t s_wave[2 * (1024 / SPLATAD_WAVE)];
+    __shared__ uint32_t s_big;
+    for (int cls = kSortClasses - 1; cls >= 4; --cls) { // uniform
+        const uint32_t count = seg_counts[cls];
+        const uint32_t *list = seg_lists + (size_t)cls * n_segments;
+        for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) { // uniform across the workgroup
+            if (cls == 4)
+                sort_segment<16, true>(list[k], n_segments, n_tiles, tile_n_bits, kSortBigInLds,
+                                       sort_bucket_capacity(kSortBigInLds), n_isects, tile_starts, pairs,
+                                       isect_ids, flatten_ids, lds_staged, s_wave, s_big);
+            else if (cls == 5)
+                sort_segment<32, false>(list[k], n_segments, n_tiles, tile_n_bits, kSortWindow,
+                                        sort_bucket_capacity(32768u), n_isects, tile_starts, pairs,
+                                        isect_ids, flatten_ids, lds_staged, s_wave, s_big);
+            else
+                sort_segment<0, false>(list[k], n_segments, n_tiles, tile_n_bits, kSortWindow,
+                                       sort_bucket_capacity(0x7FFFFFFFu), n_isects, tile_starts, pairs,
+                                       isect_ids, flatten_ids, lds_staged, s_wave, s_big);
+            __syncthreads(); // the next segment reuses the LDS
+        }
+    }
+}
+
+static size_t sort_lds_bytes(uint32_t lds_words, uint32_t max_n) {
+    return (size_t)lds_words * 8 + (kSortFineBins + 2 * (size_t)sort_bucket_capacity(max_n)) * 4;
+}
+
+static int launch_big_segment_sort(uint32_t workgroups, uint32_t segs, uint32_t n_tiles,
+                                   uint32_t tile_n_bits, int64_t n_isects, const uint32_t *seg_counts,
+                                   const uint32_t *seg_lists, const int32_t *tile_starts,
+                                   const uint64_t *pairs, int64_t *isect_ids, int32_t *flatten_ids,
+                                   hipStream_t stream) {
+    size_t lds_bytes = sort_lds_bytes(kSortBigInLds, kSortBigInLds);
+    if (sort_lds_bytes(kSortWindow, 0x7FFFFFFFu) > lds_bytes) lds_bytes = sort_lds_bytes(kSortWindow, 0x7FFFFFFFu);
+    {
+        static std::mutex guard;
+        static bool raised = false;
+        std::lock_guard<std::mutex> lock(guard);
+        if (!raised) {
+            SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)isect_big_segment_sort_kernel,
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL(isect_big_segment_sort_kernel, dim3(workgroups < segs ? workgroups : segs),
+                       dim3(kSortBigThreads), lds_bytes, stream, segs, n_tiles, tile_n_bits, n_isects,
+                       seg_counts, seg_lists, tile_starts, pairs, isect_ids, flatten_ids);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
+}
+
 template <int ER, bool IN_LDS>
 static int launch_segment_sort(int cls, uint32_t threads, uint32_t max_n, uint32_t workgroups,
                                uint32_t segs, uint32_t n_tiles, uint32_t tile_n_bits,
@@ -809,10 +964,9 @@ __global__ void fill_zero_i32_kernel(int32_t *p, int64_t n) {
     if (i < n) p[i] = 0;
 }
 
-__global__ void fill_zero_u64_kernel(unsigned long long *p) { p[threadIdx.x] = 0ull; }
 
 struct IsectWorkspace {
-    unsigned long long *n_isects; // [1]
+    unsigned long long *n_isects; // [kCountWords] counters of the counting kernel, total first
     int64_t *n_entries;           // [1] length of the coarse lists
     int64_t *scan_total;          // [1]
     int32_t *zeroed;              // tile_counts, tile_fill are contiguous, cleared together
@@ -890,7 +1044,7 @@ static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslo
     if (tslots > scan_n) scan_n = tslots;
     char *p = (char *)ws;
     IsectWorkspace w = {};
-    w.n_isects = (unsigned long long *)p;   p += 256;
+    w.n_isects = (unsigned long long *)p;   p += splatad_align256(kCountWords * 8);
     w.n_entries = (int64_t *)p;             p += 256;
     w.scan_total = (int64_t *)p;            p += 256;
     w.zeroed = (int32_t *)p;
@@ -959,9 +1113,9 @@ static int isect_device(IsectDevice **out) {
     return 0;
 }
 
-// First stages of the binning, which need no list memory: clear the tile counters, count the
-// coarse lists and scan the counts (the table is stored [workgroup][block] and scanned
-// block-major, which makes a block's list contiguous).
+// First stages of the binning, which need no list memory (the tile counters were cleared
+// together with the counting kernel's): count the coarse lists and scan the counts (the table is
+// stored [workgroup][block] and scanned block-major, which makes a block's list contiguous).
 template <bool LIDAR>
 static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const IsectWorkspace &w,
                                 uint64_t total, uint32_t N, const int64_t *camera_ids,
@@ -984,8 +1138,6 @@ static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const Is
             raised = true;
         }
     }
-    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(w.n_zeroed), dim3(SPLATAD_THREADS), 0, stream,
-                       w.zeroed, (int64_t)w.n_zeroed);
     for (uint32_t c0 = 0; c0 < C; c0 += pl.cams_per_launch) {
         const uint32_t c1 = C - c0 < pl.cams_per_launch ? C : c0 + pl.cams_per_launch;
         hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, false>), dim3(pl.coarse_wgs),
@@ -1021,9 +1173,14 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     if (int rc = isect_device(&dv)) return rc;
     std::lock_guard<std::mutex> lock(dv->guard);
     *(volatile unsigned long long *)dv->n.host = kHostWordPending;
-    hipLaunchKernelGGL(fill_zero_u64_kernel, dim3(1), dim3(2), 0, stream, w.n_isects);
+    // one fill clears the counters and, for the binning, everything up to the end of the tile
+    // counters (the two scan totals between them are written before they are read)
+    const uint64_t clear_words = sort ? (uint64_t)((char *)(w.zeroed + w.n_zeroed) - (char *)w.n_isects) / 4
+                                      : (uint64_t)kCountWords * 2;
+    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(clear_words), dim3(SPLATAD_THREADS), 0, stream,
+                       (int32_t *)w.n_isects, (int64_t)clear_words);
     dim3 count_grid = grid_for(total);
-    if (count_grid.x > 512) count_grid.x = 512;
+    if (count_grid.x > 1024) count_grid.x = 1024;
     hipLaunchKernelGGL(isect_count_kernel<LIDAR>, count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
                        total, means2d, radii, tiles_per_gauss, w.n_isects, dv->n.device);
     SPLATAD_LAUNCH_CHECK();
@@ -1104,11 +1261,12 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
                        w.tile_counts, (const int32_t *)w.tile_starts, w.tile_fill, w.pairs);
     SPLATAD_LAUNCH_CHECK();
-    // Size classes: one launch per class, so that the LDS per workgroup (and with it the number
-    // of resident workgroups) fits the segment length; the segments of a class come from a list
-    // made on the device.  The classes touch disjoint segments; they run on two helper streams
-    // beside the caller's, forked and joined with events, so that the few long workgroups of the
-    // upper classes overlap the many short ones of the lower classes.
+    // Size classes: a launch per class (one for the three upper classes), so that the LDS per
+    // workgroup (and with it the number of resident workgroups) fits the segment length; the
+    // segments of a class come from a list made on the device.  The classes touch disjoint
+    // segments; they run on two helper streams beside the caller's, forked and joined with
+    // events, so that the few long workgroups of the upper classes overlap the many short ones
+    // of the lower classes.
     const uint32_t nseg = (uint32_t)segs;
     hipLaunchKernelGGL(isect_classify_segments_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream,
                        nseg, n_isects, (const int32_t *)w.tile_starts, w.seg_counts, w.seg_lists,
@@ -1124,10 +1282,10 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                                               n_isects, w.seg_counts, w.seg_lists, w.tile_starts, \
                                               w.pairs, isect_ids, flatten_ids, on)) != 0)         \
         return rc;
-    // the longest workgroups first on every stream
-    SPLATAD_SORT_CLASS(5, 32, false, 1024, 32768u, 256u, ss->aux[0])
-    SPLATAD_SORT_CLASS(4, 16, true, 1024, 16384u, 256u, ss->aux[1])
-    SPLATAD_SORT_CLASS(6, 0, false, 1024, 0x7FFFFFFFu, 256u, stream)
+    // the upper classes go first, on the caller's stream, which does not wait for the fork
+    if ((rc = launch_big_segment_sort(256u, nseg, n_tiles, tile_n_bits, n_isects, w.seg_counts, w.seg_lists,
+                                      w.tile_starts, w.pairs, isect_ids, flatten_ids, stream)) != 0)
+        return rc;
     SPLATAD_SORT_CLASS(2, 8, true, 512, 4096u, 1024u, ss->aux[0])
     SPLATAD_SORT_CLASS(3, 8, true, 1024, 8192u, 512u, ss->aux[1])
     SPLATAD_SORT_CLASS(1, 8, true, 256, 2048u, 2048u, stream)

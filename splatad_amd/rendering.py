@@ -182,7 +182,7 @@ def rasterization(
         opacities = opacities[gaussian_ids]  # [nnz]
     else:
         radii, means2d, depths, conics, compensations, pix_vels = proj
-        opacities = opacities.repeat(C, 1)  # [C, N]
+        opacities = opacities.expand(C, -1)  # [C, N]; a view, copied by the first operator that needs it when C > 1
         camera_ids, gaussian_ids = None, None
     if compensations is not None:
         opacities = opacities * compensations
@@ -374,7 +374,7 @@ def lidar_rasterization(
     if packed:
         raise NotImplementedError("Packed mode is not supported for lidar_rasterization")
     radii, means2d, depths, conics, compensations, pix_vels, depth_compensations = proj
-    opacities = opacities.repeat(C, 1)  # [C, N]
+    opacities = opacities.expand(C, -1)  # [C, N], as above
     camera_ids, gaussian_ids = None, None
 
     if not use_depth_compensation:
