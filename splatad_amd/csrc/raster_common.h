@@ -12,6 +12,29 @@ constexpr float kLog2e = 1.44269504088896341f;
 constexpr float kLn2 = 0.693147180559945309f;
 constexpr float kLog2Of255 = 7.99435343685886f;
 
+// A pointer to kernel inputs that no kernel of the launch writes, in the constant address
+// space: loads through it at a wavefront-uniform address go through the scalar unit into
+// scalar registers (one request per wavefront, no vector registers, usable directly as an
+// operand of vector arithmetic).
+typedef const float __attribute__((address_space(4))) *uniform_f32_ptr;
+__device__ __forceinline__ uniform_f32_ptr uniform_input(const float *p) {
+    return (uniform_f32_ptr)(uintptr_t)p;
+}
+
+// v[0..N) = p[0..N) for a wavefront-uniform p, in scalar loads of four floats where N allows.
+template <int N>
+__device__ __forceinline__ void load_uniform_row(uniform_f32_ptr p, float (&v)[N]) {
+    typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
+    typedef const f4u __attribute__((address_space(4))) *uniform_f4_ptr;
+#pragma unroll
+    for (int j = 0; j + 4 <= N; j += 4) {
+        const f4u q = *(uniform_f4_ptr)(p + j);
+        v[j] = q.x; v[j + 1] = q.y; v[j + 2] = q.z; v[j + 3] = q.w;
+    }
+#pragma unroll
+    for (int j = N / 4 * 4; j < N; ++j) v[j] = p[j];
+}
+
 // Staged exponent of a Gaussian: alpha = exp2(L - (A dx^2 + B dx dy + C dy^2)), i.e.
 // A = a log2(e) / 2, B = b log2(e), C = c log2(e) / 2 for the conic (a, b, c) and
 // L = log2(opacity) (-inf for opacity <= 0, which can then never reach alpha >= 1/255).
@@ -37,18 +60,21 @@ __device__ __forceinline__ float angle_difference(float a, float b) {
 // p is convex for a positive definite conic, so off the centre its minimum over the box lies
 // on one of the four edges.  A margin covers the rounding of the test itself; Gaussians with
 // a degenerate conic are never rejected.  Returns false when no offset in the box can pass.
+// half_inv_free = 1 / (2 free_coef): the minimiser along the edge is -cross * fixed / (2 free_coef),
+// clamped to the edge; an error of a few ulp in it moves the minimum in second order only.
 __device__ __forceinline__ float edge_min(float fixed_coef, float free_coef, float cross,
-                                          float fixed, float lo, float hi) {
-    const float free_c = fminf(fmaxf(-cross * fixed / (2.f * free_coef), lo), hi);
-    return fixed_coef * fixed * fixed + free_coef * free_c * free_c + cross * fixed * free_c;
+                                          float half_inv_free, float fixed, float lo, float hi) {
+    const float free_c = fminf(fmaxf(-cross * fixed * half_inv_free, lo), hi);
+    return fixed_coef * fixed * fixed + free_c * (free_coef * free_c + cross * fixed);
 }
 
 __device__ __forceinline__ bool box_may_pass(const float4 e, float x0, float x1, float y0, float y1) {
     const float A = e.x, B = e.y, C = e.z;
     const bool definite = A > 0.f && C > 0.f && 4.f * A * C - B * B > 0.f;
     const bool centre_in = x0 <= 0.f && x1 >= 0.f && y0 <= 0.f && y1 >= 0.f;
-    const float q = fminf(fminf(edge_min(A, C, B, x0, y0, y1), edge_min(A, C, B, x1, y0, y1)),
-                          fminf(edge_min(C, A, B, y0, x0, x1), edge_min(C, A, B, y1, x0, x1)));
+    const float hA = 0.5f * __builtin_amdgcn_rcpf(A), hC = 0.5f * __builtin_amdgcn_rcpf(C);
+    const float q = fminf(fminf(edge_min(A, C, B, hC, x0, y0, y1), edge_min(A, C, B, hC, x1, y0, y1)),
+                          fminf(edge_min(C, A, B, hA, y0, x0, x1), edge_min(C, A, B, hA, y1, x0, x1)));
     const float limit = e.w + kLog2Of255;
     return !(definite && !centre_in && q > limit + 1e-3f * fabsf(limit) + 0.02f);
 }

@@ -41,13 +41,17 @@ struct BwdArgs {
     // arrays; unpack_gradients_kernel distributes them afterwards.
     float *packed;
     uint32_t packed_stride;
+    uint32_t batch; // Gaussians staged per batch, at most the workgroup size
 };
 
 // Geometry gradient slots per Gaussian in the LDS accumulator, after the CH colour slots;
 // the last three exist for lidars only.
 enum { G_CONIC = 0, G_XY = 3, G_ABS = 5, G_VEL = 7, G_OPAC = 9, G_VELZ = 10, G_DC = 11, G_COUNT = 13 };
 
-constexpr int pow2_at_least(int n) { return n <= 16 ? 16 : (n <= 32 ? 32 : 64); }
+// The per-Gaussian values are summed over the wavefront in one or two power-of-two groups (a
+// reduce-scatter of n values costs about 2 n operations): first(n) values, then second(n).
+constexpr int reduce_first(int n) { return n <= 24 ? 16 : (n <= 48 ? 32 : 64); }
+constexpr int reduce_second(int n) { return n <= 16 ? 0 : (n <= 24 ? 8 : (n <= 32 ? 0 : (n <= 48 ? 16 : 0))); }
 
 template <int CH, bool LIDAR>
 __global__ void __launch_bounds__(256)
@@ -62,11 +66,15 @@ rasterize_bwd_kernel(BwdArgs a) {
     constexpr int RECORD = LIDAR ? 3 : 2; // {x, y, vx, vy}, staged exponent, lidar extras
     constexpr int GEO = LIDAR ? G_COUNT : G_VELZ;
     constexpr int ACC = CH + GEO;
-    constexpr int NV = pow2_at_least(ACC);
+    constexpr int NA = reduce_first(ACC), NB = reduce_second(ACC), NV = NA + NB;
+    static_assert(ACC <= SPLATAD_WAVE, "the flush gives every accumulator slot a lane");
     float4 *s_rec = lds4;
-    float2 *s_aux = reinterpret_cast<float2 *>(lds4 + (size_t)RECORD * block_size); // {id, 1/opacity}
-    float *s_col = reinterpret_cast<float *>(s_aux + block_size);                   // [block_size][CH]
-    float *s_acc = s_col + (size_t)block_size * CH;                                 // [block_size][ACC]
+    // Gaussians per batch: the first `batch` lanes stage one each.  Fewer than the workgroup has
+    // lanes where the LDS of a full batch would leave a compute unit with a single workgroup.
+    const uint32_t batch = a.batch;
+    float2 *s_aux = reinterpret_cast<float2 *>(lds4 + (size_t)RECORD * batch); // {id, 1/opacity}
+    float *s_col = reinterpret_cast<float *>(s_aux + batch);                   // [batch][CH]
+    float *s_acc = s_col + (size_t)batch * CH;                                 // [batch][ACC]
 
     const uint32_t tiles_per_cam = a.grid_w * a.grid_h;
     const uint32_t cam = blockIdx.x / tiles_per_cam;
@@ -120,10 +128,14 @@ rasterize_bwd_kernel(BwdArgs a) {
     const float T_final = inside ? 1.0f - a.render_alphas[pix] : 1.0f;
     float T = T_final;
     const int32_t bin_final = inside ? a.last_ids[pix] : -1;
-    float buffer[CH], v_out[CH];
+    // The reference keeps, per channel, the colour accumulated behind the current Gaussian
+    // (`buffer`) and forms v_alpha = sum_k (c_k T - buffer_k / (1 - alpha)) v_out_k.  Only the
+    // product of the buffer with v_out is ever used, so one running number per lane replaces
+    // the CH buffers: with cv = sum_k c_k v_out_k, v_alpha = cv T - behind / (1 - alpha) and
+    // behind += cv alpha T.
+    float behind = 0.f, v_out[CH];
 #pragma unroll
     for (int k = 0; k < CH; ++k) {
-        buffer[k] = 0.f;
         v_out[k] = (inside && (uint32_t)k < a.n_ch) ? a.v_render_colors[pix * a.color_stride + a.ch_offset + k] : 0.f;
     }
     const float v_render_a = (inside && a.first_pass) ? a.v_render_alphas[pix] : 0.f;
@@ -138,7 +150,6 @@ rasterize_bwd_kernel(BwdArgs a) {
     const bool has_depth = LIDAR && a.depth_idx >= a.ch_offset && a.depth_idx < a.ch_offset + a.n_ch;
     const int depth_local = has_depth ? (int)(a.depth_idx - a.ch_offset) : -1;
     float v_out_depth = 0.f; // v_out of the depth channel, valid in the pass that owns it
-    float buffer_extra = 0.f; // depth-channel part of `buffer` coming from the extra terms
 #pragma unroll
     for (int k = 0; k < CH; ++k)
         if (k == depth_local) v_out_depth = v_out[k];
@@ -149,7 +160,7 @@ rasterize_bwd_kernel(BwdArgs a) {
     __syncthreads();
     const int32_t list_end = min(range_end, s_block_final + 1); // exclusive
     if (list_end <= range_start) return;
-    const uint32_t num_batches = (uint32_t)(list_end - range_start + block_size - 1) / block_size;
+    const uint32_t num_batches = (uint32_t)(list_end - range_start + batch - 1) / batch;
 
     // footprint of this wavefront over the lanes that consumed anything
     WaveCull cull;
@@ -157,31 +168,84 @@ rasterize_bwd_kernel(BwdArgs a) {
     if (LIDAR) pcull.init(inside && bin_final >= range_start, px, py, roll, true);
     else cull.init(px, py, roll, true);
 
-    for (uint32_t b = 0; b < num_batches; ++b) {
-        __syncthreads(); // previous batch fully flushed
-        const int32_t batch_end = list_end - 1 - (int32_t)(block_size * b);
-        const int32_t batch_size = min((int32_t)block_size, batch_end + 1 - range_start);
-        const int32_t idx = batch_end - (int32_t)tr;
-        if (idx >= range_start) {
-            const int32_t g = a.flatten_ids[idx];
-            const float2 xy = reinterpret_cast<const float2 *>(a.means2d)[g];
+    // What a lane reads for the Gaussian it stages.  Lidar launches keep the next batch's values
+    // in registers while the current batch is worked on (and the ids of the batch after that):
+    // their workgroups are few and long, one or two to a compute unit, so nothing else would
+    // hide the two dependent memory round trips of a batch.  The camera kernel has eight
+    // workgroups per compute unit for that and reads a batch when it needs it.
+    constexpr bool AHEAD = LIDAR;
+    struct Fetched {
+        float2 xy, dc;
+        float cn[3], v[3], opac, depth_col, col[CH];
+    };
+    auto id_of = [&](uint32_t b) -> int32_t { // Gaussian this lane stages in batch b, or -1
+        const int32_t idx = list_end - 1 - (int32_t)(batch * b) - (int32_t)tr;
+        return (b < num_batches && tr < batch && idx >= range_start) ? a.flatten_ids[idx] : -1;
+    };
+    auto fetch = [&](int32_t g) -> Fetched {
+        Fetched f = {};
+        if (g >= 0) {
+            f.xy = reinterpret_cast<const float2 *>(a.means2d)[g];
             const float *cn = a.conics + (size_t)g * 3;
-            const float opac = a.opacities[g];
+            f.cn[0] = cn[0]; f.cn[1] = cn[1]; f.cn[2] = cn[2];
+            f.opac = a.opacities[g];
             const float *crow = a.colors + (size_t)g * a.color_stride;
-            float4 *rec = s_rec + (size_t)RECORD * tr;
             if (LIDAR) {
                 const float *v = a.pix_vels + (size_t)g * 3;
-                const float2 dc = reinterpret_cast<const float2 *>(a.depth_comps)[g];
-                rec[0] = make_float4(angle_difference(xy.x, ref_x), angle_difference(xy.y, ref_y), v[0], v[1]);
-                rec[RECORD - 1] = make_float4(v[2], dc.x, dc.y, crow[a.depth_idx]);
+                f.v[0] = v[0]; f.v[1] = v[1]; f.v[2] = v[2];
+                f.dc = reinterpret_cast<const float2 *>(a.depth_comps)[g];
+                f.depth_col = crow[a.depth_idx];
             } else {
                 const float2 v = reinterpret_cast<const float2 *>(a.pix_vels)[g];
-                rec[0] = make_float4(xy.x, xy.y, v.x, v.y);
+                f.v[0] = v.x; f.v[1] = v.y;
             }
-            rec[1] = staged_exponent(cn[0], cn[1], cn[2], opac);
-            s_aux[tr] = make_float2(__int_as_float(g), opac > 0.f ? 1.0f / opac : 0.f); // finite
 #pragma unroll
-            for (int k = 0; k < CH; ++k) s_col[tr * CH + k] = (uint32_t)k < a.n_ch ? crow[a.ch_offset + k] : 0.f;
+            for (int k = 0; k < CH; ++k) f.col[k] = (uint32_t)k < a.n_ch ? crow[a.ch_offset + k] : 0.f;
+        }
+        return f;
+    };
+    // where slot `lane` of a Gaussian's accumulator goes: slot_base + id * slot_stride
+    float *slot_base = nullptr;
+    uint32_t slot_stride = 0;
+    if (lane < CH) {
+        if ((uint32_t)lane < a.n_ch) { slot_base = a.v_colors + a.ch_offset + lane; slot_stride = a.color_stride; }
+    } else if (lane < ACC) {
+        const int geo = lane - CH;
+        const uint32_t nv = LIDAR ? 3 : 2;
+        if (geo < G_XY) { slot_base = a.v_conics + geo; slot_stride = 3; }
+        else if (geo < G_ABS) { slot_base = a.v_means2d + (geo - G_XY); slot_stride = 2; }
+        else if (geo < G_VEL) { if (a.v_means2d_abs != nullptr) { slot_base = a.v_means2d_abs + (geo - G_ABS); slot_stride = 2; } }
+        else if (geo < G_OPAC) { slot_base = a.v_pix_vels + (geo - G_VEL); slot_stride = nv; }
+        else if (geo == G_OPAC) { slot_base = a.v_opacities; slot_stride = 1; }
+        else if (geo == G_VELZ) { slot_base = a.v_pix_vels + 2; slot_stride = 3; }
+        else { slot_base = a.v_depth_comps + (geo - G_DC); slot_stride = 2; }
+    }
+    int32_t g_now = id_of(0), g_ahead = AHEAD ? id_of(1) : -1;
+    Fetched now = {};
+    if (AHEAD) now = fetch(g_now);
+
+    for (uint32_t b = 0; b < num_batches; ++b) {
+        __syncthreads(); // previous batch fully flushed
+        const int32_t batch_end = list_end - 1 - (int32_t)(batch * b);
+        const int32_t batch_size = min((int32_t)batch, batch_end + 1 - range_start);
+        if (!AHEAD) { g_now = id_of(b); now = fetch(g_now); }
+        if (g_now >= 0) {
+            float4 *rec = s_rec + (size_t)RECORD * tr;
+            if (LIDAR) {
+                rec[0] = make_float4(angle_difference(now.xy.x, ref_x), angle_difference(now.xy.y, ref_y), now.v[0], now.v[1]);
+                rec[RECORD - 1] = make_float4(now.v[2], now.dc.x, now.dc.y, now.depth_col);
+            } else {
+                rec[0] = make_float4(now.xy.x, now.xy.y, now.v[0], now.v[1]);
+            }
+            rec[1] = staged_exponent(now.cn[0], now.cn[1], now.cn[2], now.opac);
+            s_aux[tr] = make_float2(__int_as_float(g_now), now.opac > 0.f ? 1.0f / now.opac : 0.f); // finite
+#pragma unroll
+            for (int k = 0; k < CH; ++k) s_col[tr * CH + k] = now.col[k];
+        }
+        if (AHEAD) { // requested now, needed after this batch has been worked on
+            g_now = g_ahead;
+            now = fetch(g_now);
+            g_ahead = id_of(b + 2);
         }
         for (uint32_t k = tr; k < (uint32_t)batch_size * ACC; k += block_size) s_acc[k] = 0.f;
         __syncthreads();
@@ -233,20 +297,21 @@ rasterize_bwd_kernel(BwdArgs a) {
                 float v[NV];
 #pragma unroll
                 for (int k = ACC; k < NV; ++k) v[k] = 0.f;
-                float v_alpha = 0.f;
+                float cv = 0.f;
 #pragma unroll
                 for (int k = 0; k < CH; ++k) {
                     v[k] = fac * v_out[k];
-                    v_alpha += (s_col[t * CH + k] * T - buffer[k] * ra) * v_out[k];
+                    cv += s_col[t * CH + k] * v_out[k];
                 }
                 float4 ext = make_float4(0.f, 0.f, 0.f, 0.f);
                 float extra = 0.f;
                 if constexpr (LIDAR) {
                     ext = rec[RECORD - 1];
                     extra = ext.y * dx + ext.z * dy + ext.x * roll;
-                    // depth channel = colour + extra: both enter c*T and the buffer
-                    v_alpha += (extra * T - buffer_extra * ra) * v_out_depth;
+                    cv += extra * v_out_depth; // depth channel = colour + extra
                 }
+                float v_alpha = cv * T - behind * ra;
+                behind += cv * fac;
                 v_alpha += T_final * ra * v_render_a;
                 v_alpha += -T_final * ra * bg_dot;
                 const float rop = s_aux[t].y;
@@ -269,10 +334,7 @@ rasterize_bwd_kernel(BwdArgs a) {
                 }
                 float g_ax = fabsf(g_x), g_ay = fabsf(g_y);
                 v[CH + G_OPAC] = au_g * rop * v_alpha;
-#pragma unroll
-                for (int k = 0; k < CH; ++k) buffer[k] += s_col[t * CH + k] * fac;
                 if constexpr (LIDAR) {
-                    buffer_extra += extra * fac;
                     if (a.compute_alpha_sum) { // uniform
                         const float au_s = (valid && ext.w < pz - a.threshold) ? au : 0.f;
                         const float v_sig2 = -v_asum * au_s;
@@ -292,10 +354,16 @@ rasterize_bwd_kernel(BwdArgs a) {
                 v[CH + G_VEL] = g_x * roll;
                 v[CH + G_VEL + 1] = g_y * roll;
                 // sum over the wavefront; the lane that ends up with slot s adds it in LDS
-                wave_reduce_scatter<NV>(v, lane);
-                const int slot = wave_reduce_slot<NV>(lane);
-                if (slot < ACC && (lane & (64 / NV - 1)) == 0 && v[0] != 0.f)
+                wave_reduce_scatter<NA>(*reinterpret_cast<float(*)[NA]>(&v[0]), lane);
+                const int slot = wave_reduce_slot<NA>(lane);
+                if (slot < ACC && (lane & (64 / NA - 1)) == 0 && v[0] != 0.f)
                     atomicAdd(s_acc + (size_t)t * ACC + slot, v[0]);
+                if constexpr (NB > 0) {
+                    wave_reduce_scatter<NB>(*reinterpret_cast<float(*)[NB]>(&v[NA]), lane);
+                    const int slot_b = NA + wave_reduce_slot<NB>(lane);
+                    if (slot_b < ACC && (lane & (64 / NB - 1)) == 0 && v[NA] != 0.f)
+                        atomicAdd(s_acc + (size_t)t * ACC + slot_b, v[NA]);
+                }
             }
         }
         __syncthreads();
@@ -312,37 +380,14 @@ rasterize_bwd_kernel(BwdArgs a) {
                 if (val != 0.f)
                     atomicAdd(a.packed + (size_t)__float_as_int(s_aux[t].x) * a.packed_stride + slot, val);
             }
-        } else if ((int32_t)tr < batch_size) { // lane tr owns Gaussian tr of the batch
-            const int32_t g = __float_as_int(s_aux[tr].x);
-            const float *acc = s_acc + (size_t)tr * ACC;
-            float *vc = a.v_colors + (size_t)g * a.color_stride + a.ch_offset;
-#pragma unroll
-            for (int k = 0; k < CH; ++k)
-                if ((uint32_t)k < a.n_ch && acc[k] != 0.f) atomicAdd(vc + k, acc[k]);
-            const float *geo = acc + CH;
-            if (geo[G_OPAC] != 0.f || geo[G_XY] != 0.f || geo[G_XY + 1] != 0.f || geo[G_CONIC] != 0.f ||
-                geo[G_CONIC + 1] != 0.f || geo[G_CONIC + 2] != 0.f || geo[G_ABS] != 0.f || geo[G_ABS + 1] != 0.f) {
-                atomicAdd(a.v_conics + (size_t)g * 3, geo[G_CONIC]);
-                atomicAdd(a.v_conics + (size_t)g * 3 + 1, geo[G_CONIC + 1]);
-                atomicAdd(a.v_conics + (size_t)g * 3 + 2, geo[G_CONIC + 2]);
-                atomicAdd(a.v_means2d + (size_t)g * 2, geo[G_XY]);
-                atomicAdd(a.v_means2d + (size_t)g * 2 + 1, geo[G_XY + 1]);
-                if (a.v_means2d_abs != nullptr) {
-                    atomicAdd(a.v_means2d_abs + (size_t)g * 2, geo[G_ABS]);
-                    atomicAdd(a.v_means2d_abs + (size_t)g * 2 + 1, geo[G_ABS + 1]);
-                }
-                const int nv = LIDAR ? 3 : 2;
-                atomicAdd(a.v_pix_vels + (size_t)g * nv, geo[G_VEL]);
-                atomicAdd(a.v_pix_vels + (size_t)g * nv + 1, geo[G_VEL + 1]);
-                atomicAdd(a.v_opacities + g, geo[G_OPAC]);
-            }
-            if constexpr (LIDAR) {
-                const float gz = acc[CH + G_VELZ], d0 = acc[CH + G_DC], d1 = acc[CH + G_DC + 1];
-                if (gz != 0.f || d0 != 0.f || d1 != 0.f) {
-                    atomicAdd(a.v_pix_vels + (size_t)g * 3 + 2, gz);
-                    atomicAdd(a.v_depth_comps + (size_t)g * 2, d0);
-                    atomicAdd(a.v_depth_comps + (size_t)g * 2 + 1, d1);
-                }
+        } else {
+            // lane = slot: a wavefront adds one Gaussian's values per instruction, so the channels
+            // of a Gaussian (neighbours in v_colors) and the members of each geometry gradient
+            // share memory requests
+            for (uint32_t t = tr / SPLATAD_WAVE; t < (uint32_t)batch_size; t += block_size / SPLATAD_WAVE) {
+                const float val = lane < ACC ? s_acc[t * ACC + lane] : 0.f;
+                if (slot_base != nullptr && val != 0.f)
+                    atomicAdd(slot_base + (size_t)__float_as_int(s_aux[t].x) * slot_stride, val);
             }
         }
     }
@@ -392,9 +437,13 @@ static inline int pick_width(uint32_t n) {
 }
 
 template <int CH, bool LIDAR>
-static int launch_bwd(const BwdArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
-    const size_t bs = (size_t)block.x * block.y;
-    const size_t lds = bs * ((LIDAR ? 48 : 32) + 8) + bs * 4 * CH + bs * 4 * (CH + (LIDAR ? G_COUNT : G_VELZ));
+static int launch_bwd(BwdArgs a, dim3 grid, dim3 block, hipStream_t stream) {
+    const size_t per_gaussian = ((LIDAR ? 48 : 32) + 8) + 4 * CH + 4 * (CH + (LIDAR ? G_COUNT : G_VELZ));
+    // batches of the whole workgroup, unless that leaves fewer than three workgroups to a
+    // compute unit (160 KB of LDS): then half, or a quarter
+    a.batch = block.x;
+    while (a.batch > 64 && a.batch * per_gaussian > 52 * 1024) a.batch /= 2;
+    const size_t lds = a.batch * per_gaussian;
     if (lds > 64 * 1024)
         SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_bwd_kernel<CH, LIDAR>,
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));

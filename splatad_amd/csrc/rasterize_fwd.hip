@@ -176,11 +176,15 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
     __shared__ uint32_t s_ref_thread;
     __shared__ float s_ref[2];
     const uint32_t block_size = blockDim.x * blockDim.y;
-    // per Gaussian: {u_az, u_el, v_az, v_el} (u relative to the tile's reference point),
-    // {A, B, C, L} as in the pixel kernel, {v_range, depth comp 0, depth comp 1, depth} and
-    // the CH colours padded to a multiple of four floats
-    constexpr int RECORD = 3 + (CH + 3) / 4; // float4 per Gaussian
+    // Staged per Gaussian: {u_az, u_el, v_az, v_el} (u relative to the tile's reference point),
+    // {A, B, C, L} as in the pixel kernel, and the Gaussian's id.  That is all the footprint test
+    // and the alpha need.  A lidar point is a sample, not an area: of the Gaussians in a tile's
+    // list only a few per cent reach alpha >= 1/255 at any of a wavefront's points, so the rest
+    // of a Gaussian (its CH features, the range velocity, the depth compensation) is read from
+    // global memory by the wavefronts that composite it, through wavefront-uniform loads.
+    constexpr int RECORD = 2; // float4 per Gaussian
     float4 *s_rec = lds4;
+    int32_t *s_gid = reinterpret_cast<int32_t *>(lds4 + (size_t)RECORD * blockDim.x * blockDim.y);
 
     const uint32_t tiles_per_cam = a.grid_w * a.grid_h;
     const uint32_t cam = blockIdx.x / tiles_per_cam;
@@ -232,27 +236,43 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
 #pragma unroll
     for (int k = 0; k < CH; ++k) out[k] = 0.f;
 
+    // A tile's list is long (thousands of Gaussians) and a compute unit holds few of these
+    // workgroups, so nothing but the workgroup itself can hide the two dependent memory round
+    // trips of a batch (id, then the Gaussian): the values of the next batch are requested
+    // before the current batch is worked on, the ids one batch earlier still.
+    struct Fetched { float2 xy; float vx, vy, cn[3], opac; };
+    auto id_of = [&](uint32_t b) -> int32_t { // Gaussian this lane stages in batch b, or -1
+        const uint32_t idx = (uint32_t)range_start + block_size * b + tr;
+        return (b < num_batches && idx < (uint32_t)range_end) ? a.flatten_ids[idx] : -1;
+    };
+    auto fetch = [&](int32_t g) -> Fetched {
+        Fetched f = {};
+        if (g >= 0) {
+            f.xy = reinterpret_cast<const float2 *>(a.means2d)[g];
+            const float *v = a.pix_vels + (size_t)g * 3;
+            f.vx = v[0]; f.vy = v[1];
+            const float *cn = a.conics + (size_t)g * 3;
+            f.cn[0] = cn[0]; f.cn[1] = cn[1]; f.cn[2] = cn[2];
+            f.opac = a.opacities[g];
+        }
+        return f;
+    };
+    int32_t g_now = id_of(0), g_ahead = id_of(1);
+    Fetched now = fetch(g_now);
+
     for (uint32_t b = 0; b < num_batches; ++b) {
         // also orders the previous batch's LDS reads before this batch's writes
         if (__syncthreads_count(!wave_lanes(alive_bits)) >= (int)block_size) break;
         const uint32_t batch_start = (uint32_t)range_start + block_size * b;
-        const uint32_t idx = batch_start + tr;
-        if (idx < (uint32_t)range_end) {
-            const int32_t g = a.flatten_ids[idx];
-            const float2 xy = reinterpret_cast<const float2 *>(a.means2d)[g];
-            const float *v = a.pix_vels + (size_t)g * 3;
-            const float2 dc = reinterpret_cast<const float2 *>(a.depth_comps)[g];
-            const float *cn = a.conics + (size_t)g * 3;
-            const float *crow = a.colors + (size_t)g * a.color_stride;
+        if (g_now >= 0) {
             float4 *rec = s_rec + RECORD * tr;
-            rec[0] = make_float4(angle_difference(xy.x, ref_x), angle_difference(xy.y, ref_y), v[0], v[1]);
-            rec[1] = staged_exponent(cn[0], cn[1], cn[2], a.opacities[g]);
-            rec[2] = make_float4(v[2], dc.x, dc.y, crow[a.depth_idx]);
-            const float *c = crow + a.ch_offset;
-#pragma unroll
-            for (int k = 0; k < CH; ++k)
-                reinterpret_cast<float *>(rec + 3)[k] = (uint32_t)k < a.n_ch ? c[k] : 0.f;
+            rec[0] = make_float4(angle_difference(now.xy.x, ref_x), angle_difference(now.xy.y, ref_y), now.vx, now.vy);
+            rec[1] = staged_exponent(now.cn[0], now.cn[1], now.cn[2], now.opac);
+            s_gid[tr] = g_now;
         }
+        g_now = g_ahead;
+        now = fetch(g_now);
+        g_ahead = id_of(b + 2);
         __syncthreads();
 
         const uint32_t batch_size = min(block_size, (uint32_t)range_end - batch_start);
@@ -287,9 +307,22 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
                 if (take_bits != 0) {
                     const bool take = wave_lanes(take_bits);
                     const float vis = take ? weight : 0.f;
+                    // the rest of the Gaussian, at addresses the whole wavefront shares
+                    const uint32_t g = (uint32_t)__builtin_amdgcn_readfirstlane(s_gid[t]);
+                    const uniform_f32_ptr crow = uniform_input(a.colors) + (size_t)g * a.color_stride;
+                    const uniform_f32_ptr dcp = uniform_input(a.depth_comps) + (size_t)g * 2;
+                    const float4 ext = make_float4(uniform_input(a.pix_vels)[(size_t)g * 3 + 2], dcp[0], dcp[1],
+                                                   crow[a.depth_idx]);
+                    float c[CH];
+                    if (a.n_ch == CH) { // uniform; the usual case
+                        load_uniform_row<CH>(crow + a.ch_offset, c);
+                    } else { // a pass narrower than the kernel: the spare accumulators are never stored
+                        const float *row = a.colors + (size_t)g * a.color_stride + a.ch_offset;
 #pragma unroll
-                    for (int k = 0; k < CH; ++k) out[k] += reinterpret_cast<const float *>(rec + 3)[k] * vis;
-                    const float4 ext = rec[2];
+                        for (int k = 0; k < CH; ++k) c[k] = row[min((uint32_t)k, a.n_ch - 1u)];
+                    }
+#pragma unroll
+                    for (int k = 0; k < CH; ++k) out[k] += c[k] * vis;
                     const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
                     depth_extra += extra * vis;
                     if (take && T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
@@ -346,7 +379,7 @@ static int launch_pixels(const PixelArgs &a, dim3 grid, dim3 block, hipStream_t 
 
 template <int CH>
 static int launch_points(const PointArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
-    const size_t lds = (size_t)block.x * block.y * 16 * (3 + (CH + 3) / 4);
+    const size_t lds = (size_t)block.x * block.y * (2 * 16 + 4); // two float4 and the id per Gaussian
     hipLaunchKernelGGL(rasterize_to_points_fwd_kernel<CH>, grid, block, lds, stream, a);
     SPLATAD_LAUNCH_CHECK();
     return 0;
