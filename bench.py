@@ -28,8 +28,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # 0.5 KiB per KiB, WRITE_SIZE 1.0).  Summaries: profiles/rasterize_kernels_counters_1M.txt.
 # They describe the 1M-Gaussian default only; other sizes report null.
 MEASURED_TRAFFIC_BYTES = {
-    "camera": int((12972.2 * 2.0 + 48600.0) * 1024),
-    "lidar": int((36864.9 * 2.0 + 40193.0) * 1024),
+    "camera": int((12972.0 * 2.0 + 48617.6) * 1024),
+    "lidar": int((27165.8 * 2.0 + 40098.4) * 1024),
 }
 
 
@@ -67,26 +67,15 @@ def time_kernel(fn, iters, warmup=2):
     return sum(s.elapsed_time(e) for s, e in zip(start, stop)) / iters
 
 
-def consumed_isects(last_ids, alphas, offsets, n_isects, tile_w, tile_h):
-    """Per-tile prefix of the sorted list that the tile's pixels/points really consume:
-    the whole list when some pixel never saturates, else up to the last contributing entry."""
+def staged_isects(tile_batches, offsets, n_isects, batch=256):
+    """List entries the compositing kernel staged: whole batches until every pixel / point of a
+    tile has saturated, as counted by the kernel itself, clipped to the tile's list."""
     import torch
 
-    C, H, W = last_ids.shape
-    gh, gw = offsets.shape[1:]
     flat_off = offsets.reshape(-1).long()
     ends = torch.cat([flat_off[1:], torch.tensor([n_isects], device=flat_off.device)])
-    Hp, Wp = gh * tile_h, gw * tile_w
-    li = torch.zeros((C, Hp, Wp), dtype=torch.long, device=last_ids.device)
-    li[:, :H, :W] = last_ids.long()
-    unsat = torch.zeros((C, Hp, Wp), dtype=torch.bool, device=last_ids.device)
-    unsat[:, :H, :W] = alphas.reshape(C, H, W) < 0.9998
-    li = li.reshape(C, gh, tile_h, gw, tile_w).permute(0, 1, 3, 2, 4).reshape(C * gh * gw, -1)
-    unsat = unsat.reshape(C, gh, tile_h, gw, tile_w).permute(0, 1, 3, 2, 4).reshape(C * gh * gw, -1)
     full = ends - flat_off
-    need = (li.max(dim=1).values + 1 - flat_off).clamp(min=0)
-    need = torch.where(unsat.any(dim=1), full, torch.minimum(need, full))
-    need = torch.where(full > 0, need, torch.zeros_like(need))
+    need = torch.minimum(tile_batches.reshape(-1).long() * batch, full)
     return int(need.sum().item()), int(full.sum().item())
 
 
@@ -129,9 +118,13 @@ def bench_camera(args):
                 s["rolling_shutter_time"], None, W, H, ts, meta["isect_offsets"], meta["flatten_ids"])
 
         k_ms = time_kernel(raster, iters=max(5, args.steps))
-        _, alphas, last_ids = raster()
         n_isects = int(meta["flatten_ids"].shape[0])
-        i_need, i_full = consumed_isects(last_ids, alphas, meta["isect_offsets"], n_isects, ts, ts)
+        batches = torch.zeros_like(meta["isect_offsets"])
+        _C.rasterize_to_pixels_fwd(
+            meta["means2d"], meta["conics"], cols, meta["opacities"], meta["pix_vels"],
+            s["rolling_shutter_time"], None, W, H, ts, meta["isect_offsets"], meta["flatten_ids"],
+            tile_batches=batches)
+        i_need, i_full = staged_isects(batches, meta["isect_offsets"], n_isects)
         D = cols.shape[-1]
         P, T = C * H * W, meta["isect_offsets"].numel()
         alg_bytes = i_need * (36 + 4 * D) + P * (4 * D + 8) + T * 4
@@ -197,12 +190,17 @@ def bench_lidar(args):
                 meta["isect_offsets"], meta["flatten_ids"], D - 1)
 
         k_ms = time_kernel(raster, iters=max(5, args.steps))
-        _, alphas, last_ids, _, _ = raster()
         n_isects = int(meta["flatten_ids"].shape[0])
-        i_need, _ = consumed_isects(last_ids, alphas, meta["isect_offsets"], n_isects,
-                                    s["tile_width"], s["tile_height"])
+        batches = torch.zeros_like(meta["isect_offsets"])
+        _C.rasterize_to_points_fwd(
+            meta["means2d"], meta["conics"], feats, meta["opacities"], meta["pix_vels"], proj[6],
+            None, s["raster_pts"], W, H, s["tile_width"], s["tile_height"], True, 0.2,
+            meta["isect_offsets"], meta["flatten_ids"], D - 1, tile_batches=batches)
+        i_need, _ = staged_isects(batches, meta["isect_offsets"], n_isects)
         P, T = C * H * W, meta["isect_offsets"].numel()
-        alg_bytes = i_need * (48 + 4 * D) + P * (4 * D + 32) + T * 4
+        # staged per list entry: id, mean, angular velocity, conic, opacity (40 bytes); the features
+        # of the Gaussians a wavefront composites are read on demand and not counted here
+        alg_bytes = i_need * 40 + P * (4 * D + 32) + T * 4
     return dict(sec=sec, sec_chunk32=sec_chunk32, points=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
                 n_isects=n_isects, i_need=i_need, channels=D)
 

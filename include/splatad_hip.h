@@ -246,7 +246,10 @@ int splatad_populate_image_from_points(uint32_t C, int64_t n_points, const float
 
 /* rasterize_to_pixels_fwd_tensor, rasterization.cu:1520-2018 (kernel
  * :1360-1518).  Any channel count >= 1 is accepted (wide inputs are rendered in
- * passes).  backgrounds may be NULL. */
+ * passes).  backgrounds may be NULL.  tile_batches may be NULL; otherwise it receives,
+ * per (camera, tile), the number of 256-entry batches of the tile's list that were staged
+ * before every pixel of the tile had saturated (a diagnostic: it tells how much of the
+ * sorted lists a frame really reads). */
 int splatad_rasterize_to_pixels_fwd(uint32_t C, int64_t n_isects, uint32_t channels,
                                     const float *means2d, const float *conics,
                                     const float *colors, const float *opacities,
@@ -256,7 +259,8 @@ int splatad_rasterize_to_pixels_fwd(uint32_t C, int64_t n_isects, uint32_t chann
                                     uint32_t tile_width, uint32_t tile_height,
                                     const int32_t *tile_offsets, const int32_t *flatten_ids,
                                     float *render_colors, float *render_alphas,
-                                    int32_t *last_ids, splatad_stream_t stream);
+                                    int32_t *last_ids, int32_t *tile_batches,
+                                    splatad_stream_t stream);
 
 /* rasterize_to_pixels_bwd_tensor, rasterization.cu:3091-3726 (kernel
  * :2833-3089).  Gradient outputs must be zero-filled; v_means2d_abs may be NULL.
@@ -287,7 +291,8 @@ int splatad_rasterize_to_pixels_bwd(uint32_t C, int64_t n_isects, uint32_t chann
 
 /* rasterize_to_points_fwd_tensor, rasterization.cu:2221-2831 (kernel
  * :2021-2219).  Outputs of inactive points (range <= 0) are zero.
- * alpha_sum_until_points may be NULL when compute_alpha_sum_until_points == 0. */
+ * alpha_sum_until_points may be NULL when compute_alpha_sum_until_points == 0.
+ * tile_batches: optional diagnostic as in splatad_rasterize_to_pixels_fwd. */
 int splatad_rasterize_to_points_fwd(uint32_t C, int64_t n_isects, uint32_t channels,
                                     const float *means2d, const float *conics,
                                     const float *colors, const float *opacities,
@@ -301,7 +306,7 @@ int splatad_rasterize_to_points_fwd(uint32_t C, int64_t n_isects, uint32_t chann
                                     uint32_t depth_channel_idx, float *render_colors,
                                     float *render_alphas, float *alpha_sum_until_points,
                                     int32_t *last_ids, float *median_depths,
-                                    splatad_stream_t stream);
+                                    int32_t *tile_batches, splatad_stream_t stream);
 
 /* rasterize_to_points_bwd_tensor, rasterization.cu:4056-4851 (kernel :3728-4054). */
 int splatad_rasterize_to_points_bwd(uint32_t C, int64_t n_isects, uint32_t channels,

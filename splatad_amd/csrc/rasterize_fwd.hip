@@ -32,6 +32,7 @@ struct PixelArgs {
     float *render_colors, *render_alphas;
     int32_t *last_ids;
     int write_aux; // first pass also writes alphas and last ids
+    int32_t *tile_batches; // optional diagnostic: batches each tile's workgroup went through
 };
 
 template <int CH>
@@ -80,9 +81,11 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
 #pragma unroll
     for (int k = 0; k < CH; ++k) out[k] = 0.f;
 
+    uint32_t batches_done = 0;
     for (uint32_t b = 0; b < num_batches; ++b) {
         // also orders the previous batch's LDS reads before this batch's writes
         if (__syncthreads_count(!wave_lanes(alive_bits)) >= (int)block_size) break;
+        batches_done = b + 1;
 
         const uint32_t batch_start = (uint32_t)range_start + block_size * b;
         const uint32_t idx = batch_start + tr;
@@ -138,6 +141,7 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
         }
     }
 
+    if (a.tile_batches != nullptr && a.write_aux && tr == 0) a.tile_batches[blockIdx.x] = (int32_t)batches_done;
     if (inside) {
         const size_t pix = ((size_t)cam * a.H + i) * a.W + j;
         float *dst = a.render_colors + pix * a.color_stride + a.ch_offset;
@@ -167,6 +171,7 @@ struct PointArgs {
     int32_t *last_ids;
     float *median_depths;
     int write_aux;
+    int32_t *tile_batches; // optional diagnostic, as in PixelArgs
 };
 
 template <int CH>
@@ -260,9 +265,11 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
     int32_t g_now = id_of(0), g_ahead = id_of(1);
     Fetched now = fetch(g_now);
 
+    uint32_t batches_done = 0;
     for (uint32_t b = 0; b < num_batches; ++b) {
         // also orders the previous batch's LDS reads before this batch's writes
         if (__syncthreads_count(!wave_lanes(alive_bits)) >= (int)block_size) break;
+        batches_done = b + 1;
         const uint32_t batch_start = (uint32_t)range_start + block_size * b;
         if (g_now >= 0) {
             float4 *rec = s_rec + RECORD * tr;
@@ -335,6 +342,7 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
         }
     }
 
+    if (a.tile_batches != nullptr && a.write_aux && tr == 0) a.tile_batches[blockIdx.x] = (int32_t)batches_done;
     if (in_image) {
         float *dst = a.render_colors + pix * a.color_stride + a.ch_offset;
         const float *bg = a.backgrounds ? a.backgrounds + (size_t)cam * a.color_stride + a.ch_offset : nullptr;
@@ -424,7 +432,8 @@ extern "C" int splatad_rasterize_to_pixels_fwd(
     const float *colors, const float *opacities, const float *pix_vels, const float *rs_time,
     const float *backgrounds, uint32_t W, uint32_t H, uint32_t tile_size, uint32_t tile_w,
     uint32_t tile_h, const int32_t *tile_offsets, const int32_t *flatten_ids,
-    float *render_colors, float *render_alphas, int32_t *last_ids, splatad_stream_t stream) {
+    float *render_colors, float *render_alphas, int32_t *last_ids, int32_t *tile_batches,
+    splatad_stream_t stream) {
     SPLATAD_REQUIRE(channels >= 1, "rasterize_to_pixels: zero channels");
     SPLATAD_REQUIRE(tile_size >= 1 && tile_size * tile_size <= 1024,
                     "rasterize_to_pixels: tile_size %u is outside 1..32", tile_size);
@@ -444,6 +453,7 @@ extern "C" int splatad_rasterize_to_pixels_fwd(
     a.W = W; a.H = H; a.tile_size = tile_size; a.tile_w = tile_w; a.tile_h = tile_h;
     a.tile_offsets = tile_offsets; a.flatten_ids = flatten_ids;
     a.render_colors = render_colors; a.render_alphas = render_alphas; a.last_ids = last_ids;
+    a.tile_batches = tile_batches;
     const dim3 grid(C * tile_w * tile_h), block(tile_size, tile_size);
     const uint32_t pass = channels <= (uint32_t)kMaxPass ? channels : 32u;
     for (uint32_t off = 0; off < channels; off += pass) {
@@ -463,7 +473,8 @@ extern "C" int splatad_rasterize_to_points_fwd(
     uint32_t tile_width, uint32_t tile_height, uint32_t grid_w, uint32_t grid_h,
     int compute_alpha_sum, float threshold, const int32_t *tile_offsets,
     const int32_t *flatten_ids, uint32_t depth_idx, float *render_colors, float *render_alphas,
-    float *alpha_sum, int32_t *last_ids, float *median_depths, splatad_stream_t stream) {
+    float *alpha_sum, int32_t *last_ids, float *median_depths, int32_t *tile_batches,
+    splatad_stream_t stream) {
     SPLATAD_REQUIRE(channels >= 1, "rasterize_to_points: zero channels");
     SPLATAD_REQUIRE(depth_idx < channels, "rasterize_to_points: depth channel %u of %u", depth_idx, channels);
     SPLATAD_REQUIRE(tile_width >= 1 && tile_height >= 1 && tile_width * tile_height <= 256,
@@ -487,7 +498,7 @@ extern "C" int splatad_rasterize_to_points_fwd(
     a.tile_offsets = tile_offsets; a.flatten_ids = flatten_ids; a.depth_idx = depth_idx;
     a.render_colors = render_colors; a.render_alphas = render_alphas;
     a.alpha_sum = compute_alpha_sum ? alpha_sum : nullptr;
-    a.last_ids = last_ids; a.median_depths = median_depths;
+    a.last_ids = last_ids; a.median_depths = median_depths; a.tile_batches = tile_batches;
     const dim3 grid(C * grid_w * grid_h), block(tile_width, tile_height);
     const uint32_t pass = channels <= (uint32_t)kMaxPass ? channels : 32u;
     for (uint32_t off = 0; off < channels; off += pass) {

@@ -694,7 +694,9 @@ class _Ops:
     # ------------------------------------------------------------------ rasterization
     def rasterize_to_pixels_fwd(self, means2d, conics, colors, opacities, pix_vels,
                                 rolling_shutter_time, backgrounds, image_width, image_height,
-                                tile_size, tile_offsets, flatten_ids):
+                                tile_size, tile_offsets, flatten_ids, tile_batches=None):
+        """tile_batches: optional int32 [C, tile_height, tile_width] tensor that receives the number
+        of list batches every tile went through (a diagnostic, not part of the reference's op)."""
         lib = load_library()
         means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
         colors = _in(colors, "colors"); opacities = _in(opacities, "opacities")
@@ -713,7 +715,8 @@ class _Ops:
                 _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics), _p(colors),
                 _p(opacities), _p(pix_vels), _p(rs), _p(backgrounds), _u32(image_width),
                 _u32(image_height), _u32(tile_size), _u32(tw), _u32(th), _p(tile_offsets),
-                _p(flatten_ids), _p(renders), _p(alphas), _p(last_ids), _stream(dev)))
+                _p(flatten_ids), _p(renders), _p(alphas), _p(last_ids),
+                _p(_in(tile_batches, "tile_batches", torch.int32)), _stream(dev)))
         return renders, alphas, last_ids
 
     def rasterize_to_pixels_bwd(self, means2d, conics, colors, opacities, pix_vels,
@@ -754,7 +757,7 @@ class _Ops:
                                 image_height, tile_width, tile_height,
                                 compute_alpha_sum_until_points,
                                 compute_alpha_sum_until_points_threshold, tile_offsets, flatten_ids,
-                                depth_channel_idx):
+                                depth_channel_idx, tile_batches=None):
         lib = load_library()
         means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
         colors = _in(colors, "colors"); opacities = _in(opacities, "opacities")
@@ -779,7 +782,7 @@ class _Ops:
                 _u32(gw), _u32(gh), _i32(bool(compute_alpha_sum_until_points)),
                 _f32(compute_alpha_sum_until_points_threshold), _p(tile_offsets), _p(flatten_ids),
                 _u32(depth_channel_idx), _p(renders), _p(alphas), _p(asum), _p(last_ids),
-                _p(medians), _stream(dev)))
+                _p(medians), _p(_in(tile_batches, "tile_batches", torch.int32)), _stream(dev)))
         return renders, alphas, last_ids, asum, medians
 
     def rasterize_to_points_bwd(self, means2d, conics, colors, opacities, pix_vels,
