@@ -43,6 +43,23 @@ __device__ __forceinline__ float4 staged_exponent(float a, float b, float c, flo
                        opacity > 0.f ? __log2f(opacity) : -INFINITY);
 }
 
+// The arithmetic behind the two discontinuous decisions of the compositing rule (alpha >=
+// 1/255, transmittance <= 1e-4), with every rounding spelled out.  All compositing kernels
+// (forward, backward, index lists, every channel width) go through these, so that they take
+// the same decisions for the same inputs; left to the compiler, the fusing of multiplies and
+// adds differs from one instantiation to the next and with it the last bit of alpha.
+__device__ __forceinline__ float gaussian_offset(float mean, float velocity, float roll, float at) {
+    return fmaf(roll, velocity, mean) - at;
+}
+__device__ __forceinline__ float gaussian_power(const float4 e, float dx, float dy) {
+    const float cross = fmaf(e.x, dx, e.y * dy);
+    const float along = dx * cross;
+    return fmaf(dy, e.z * dy, along);
+}
+__device__ __forceinline__ float transmittance_behind(float T, float alpha) {
+    return fmaf(-alpha, T, T); // T (1 - alpha)
+}
+
 // Difference of two angles in degrees folded into [-180, 180), as the reference's
 // fmodf(a - b + 180, 360) - 180 with negative results raised by 360
 // (gsplat/cuda/csrc/utils.cuh:552-555).  Without the detour through +180 / -180 the difference of two

@@ -269,13 +269,13 @@ rasterize_bwd_kernel(BwdArgs a) {
                 const float4 *rec = s_rec + (size_t)RECORD * t;
                 const float4 xyv = rec[0];
                 const float4 e = rec[1];
-                float dx = (xyv.x + roll * xyv.z) - px;
-                float dy = (xyv.y + roll * xyv.w) - py;
+                float dx = gaussian_offset(xyv.x, xyv.z, roll, px);
+                float dy = gaussian_offset(xyv.y, xyv.w, roll, py);
                 if (LIDAR && ((folded >> bit) & 1ull)) { // uniform, rare
-                    dx = angle_difference(xyv.x + roll * xyv.z, px);
-                    dy = angle_difference(xyv.y + roll * xyv.w, py);
+                    dx = angle_difference(fmaf(roll, xyv.z, xyv.x), px);
+                    dy = angle_difference(fmaf(roll, xyv.w, xyv.y), py);
                 }
-                const float power = dx * (e.x * dx + e.y * dy) + e.z * dy * dy;
+                const float power = gaussian_power(e, dx, dy);
                 const float au = __builtin_amdgcn_exp2f(e.w - power); // opacity * exp(-sigma)
                 const float alpha = fminf(0.999f, au);
                 // the lanes that took this Gaussian in the forward pass, by scalar logic on lane masks

@@ -116,12 +116,12 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
                 const float4 *rec = s_rec + RECORD * t;
                 const float4 xyv = rec[0];
                 const float4 con = rec[1];
-                const float dx = (xyv.x + roll * xyv.z) - px;
-                const float dy = (xyv.y + roll * xyv.w) - py;
-                const float power = dx * (con.x * dx + con.y * dy) + con.z * dy * dy;
+                const float dx = gaussian_offset(xyv.x, xyv.z, roll, px);
+                const float dy = gaussian_offset(xyv.y, xyv.w, roll, py);
+                const float power = gaussian_power(con, dx, dy);
                 const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
                 const float weight = alpha * T;
-                const float next_T = T - weight; // T (1 - alpha)
+                const float next_T = transmittance_behind(T, alpha);
                 // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
                 const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
                                             wave_ballot(!(alpha < 1.f / 255.f));
@@ -174,9 +174,23 @@ struct PointArgs {
     int32_t *tile_batches; // optional diagnostic, as in PixelArgs
 };
 
-template <int CH>
+// MATRIX (CH = 32 or 33, every channel in use, whole wavefronts): the first 32 channels are
+// accumulated by the matrix cores.  Compositing a Gaussian adds the outer product of 64 weights
+// (one per point) and its features to the wavefront's accumulators; two Gaussians at a time
+// that is C[64 x 32] += W[64 x 2] F[2 x 32], two v_mfma_f32_32x32x2_f32 (one per 32 points).
+// The weights of a pair are brought into the A layout (lanes 0-31: first Gaussian, lanes 32-63:
+// second; points 0-31 for the first instruction, 32-63 for the second) by one
+// v_permlane32_swap; the features are loaded in the B layout (lane = feature) with one
+// coalesced 128-byte load per Gaussian.  This takes 32 of the about 65 vector instructions of a
+// composited Gaussian off the vector ALUs, which bound this kernel.  The accumulators live in
+// the D layout (lane = feature, register = point) until the end, when every half wavefront
+// stores the 32 features of a point with one 128-byte store.
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+template <int CH, bool MATRIX>
 __global__ void __launch_bounds__(256)
 rasterize_to_points_fwd_kernel(PointArgs a) {
+    static_assert(!MATRIX || CH == 32 || CH == 33, "the matrix path accumulates 32 channels (+1)");
     extern __shared__ float4 lds4[];
     __shared__ uint32_t s_ref_thread;
     __shared__ float s_ref[2];
@@ -237,9 +251,19 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
 
     float T = 1.0f, asum = 0.f, median = 0.f, depth_extra = 0.f;
     uint32_t cur_idx = 0;
-    float out[CH];
+    constexpr int NOUT = MATRIX ? CH - 32 : CH; // channels accumulated by the vector ALUs
+    float out[NOUT > 0 ? NOUT : 1];
 #pragma unroll
-    for (int k = 0; k < CH; ++k) out[k] = 0.f;
+    for (int k = 0; k < NOUT; ++k) out[k] = 0.f;
+    floatx16 acc_lo = {0}, acc_hi = {0};     // points 0-31 and 32-63 of the wavefront, D layout
+    bool pair_open = false;                  // uniform: a Gaussian waits for its partner
+    float pair_weight = 0.f, pair_feature = 0.f;
+    auto add_pair = [&](float w0, float w1, float f0, float f1) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(w0), __float_as_uint(w1), false, false);
+        const float f = lane < 32 ? f0 : f1;
+        acc_lo = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(sw[0]), f, acc_lo, 0, 0, 0);
+        acc_hi = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(sw[1]), f, acc_hi, 0, 0, 0);
+    };
 
     // A tile's list is long (thousands of Gaussians) and a compute unit holds few of these
     // workgroups, so nothing but the workgroup itself can hide the two dependent memory round
@@ -295,16 +319,16 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
                 const float4 *rec = s_rec + RECORD * t;
                 const float4 uv = rec[0];
                 const float4 con = rec[1];
-                float dx = (uv.x + roll * uv.z) - rx;
-                float dy = (uv.y + roll * uv.w) - ry;
+                float dx = gaussian_offset(uv.x, uv.z, roll, rx);
+                float dy = gaussian_offset(uv.y, uv.w, roll, ry);
                 if ((folded >> bit) & 1ull) { // uniform, rare: half a turn away from the tile
-                    dx = angle_difference(uv.x + roll * uv.z, rx);
-                    dy = angle_difference(uv.y + roll * uv.w, ry);
+                    dx = angle_difference(fmaf(roll, uv.z, uv.x), rx);
+                    dy = angle_difference(fmaf(roll, uv.w, uv.y), ry);
                 }
-                const float power = dx * (con.x * dx + con.y * dy) + con.z * dy * dy;
+                const float power = gaussian_power(con, dx, dy);
                 const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
                 const float weight = alpha * T;
-                const float next_T = T - weight; // T (1 - alpha)
+                const float next_T = transmittance_behind(T, alpha);
                 // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
                 const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
                                             wave_ballot(!(alpha < 1.f / 255.f));
@@ -320,16 +344,24 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
                     const uniform_f32_ptr dcp = uniform_input(a.depth_comps) + (size_t)g * 2;
                     const float4 ext = make_float4(uniform_input(a.pix_vels)[(size_t)g * 3 + 2], dcp[0], dcp[1],
                                                    crow[a.depth_idx]);
-                    float c[CH];
-                    if (a.n_ch == CH) { // uniform; the usual case
-                        load_uniform_row<CH>(crow + a.ch_offset, c);
-                    } else { // a pass narrower than the kernel: the spare accumulators are never stored
-                        const float *row = a.colors + (size_t)g * a.color_stride + a.ch_offset;
+                    if constexpr (MATRIX) {
+                        const float feature = a.colors[(size_t)g * a.color_stride + a.ch_offset + (lane & 31u)];
+                        if constexpr (CH == 33) out[0] += crow[a.ch_offset + 32] * vis;
+                        if (pair_open) add_pair(pair_weight, vis, pair_feature, feature);
+                        else { pair_weight = vis; pair_feature = feature; }
+                        pair_open = !pair_open;
+                    } else {
+                        float c[CH];
+                        if (a.n_ch == CH) { // uniform; the usual case
+                            load_uniform_row<CH>(crow + a.ch_offset, c);
+                        } else { // a pass narrower than the kernel: the spare accumulators are never stored
+                            const float *row = a.colors + (size_t)g * a.color_stride + a.ch_offset;
 #pragma unroll
-                        for (int k = 0; k < CH; ++k) c[k] = row[min((uint32_t)k, a.n_ch - 1u)];
+                            for (int k = 0; k < CH; ++k) c[k] = row[min((uint32_t)k, a.n_ch - 1u)];
+                        }
+#pragma unroll
+                        for (int k = 0; k < CH; ++k) out[k] += c[k] * vis;
                     }
-#pragma unroll
-                    for (int k = 0; k < CH; ++k) out[k] += c[k] * vis;
                     const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
                     depth_extra += extra * vis;
                     if (take && T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
@@ -343,14 +375,43 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
     }
 
     if (a.tile_batches != nullptr && a.write_aux && tr == 0) a.tile_batches[blockIdx.x] = (int32_t)batches_done;
-    if (in_image) {
-        float *dst = a.render_colors + pix * a.color_stride + a.ch_offset;
-        const float *bg = a.backgrounds ? a.backgrounds + (size_t)cam * a.color_stride + a.ch_offset : nullptr;
+    if constexpr (MATRIX) {
+        if (pair_open) add_pair(pair_weight, 0.f, pair_feature, 0.f);
+        // what the D layout needs to know of a point: where it is stored, its transmittance
+        // (negative: nothing composited, store zero; NaN: outside the image, store nothing)
+        // and the depth term, through the LDS the batches no longer use
+        __syncthreads();
+        float4 *s_point = lds4;
+        s_point[tr] = make_float4(__uint_as_float((uint32_t)(pix & 0xFFFFFFFFu)), __uint_as_float((uint32_t)(pix >> 32)),
+                                  in_image ? (inside ? T : -1.f) : NAN, depth_extra);
+        __syncthreads();
+        const uint32_t n = lane & 31u, half = lane >> 5, wave_first = tr & ~(SPLATAD_WAVE - 1);
+        const float bg_n = a.backgrounds ? a.backgrounds[(size_t)cam * a.color_stride + a.ch_offset + n] : 0.f;
+        const bool depth_here = has_depth && n == a.depth_idx - a.ch_offset;
 #pragma unroll
-        for (int k = 0; k < CH; ++k) {
-            if ((uint32_t)k < a.n_ch) {
+        for (int m = 0; m < 2; ++m) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const uint32_t i = 8u * (j / 4) + 4u * half + (j % 4);
+                const float4 pt = s_point[wave_first + 32u * m + i];
+                if (pt.z == pt.z) { // inside the image
+                    const size_t at = ((size_t)__float_as_uint(pt.y) << 32) | __float_as_uint(pt.x);
+                    float v = m == 0 ? acc_lo[j] : acc_hi[j];
+                    if (depth_here) v += pt.w;
+                    v += pt.z * bg_n; // no background: bg_n = 0
+                    a.render_colors[at * a.color_stride + a.ch_offset + n] = pt.z >= 0.f ? v : 0.f;
+                }
+            }
+        }
+    }
+    if (in_image) {
+        float *dst = a.render_colors + pix * a.color_stride + a.ch_offset + (MATRIX ? 32 : 0);
+        const float *bg = a.backgrounds ? a.backgrounds + (size_t)cam * a.color_stride + a.ch_offset + (MATRIX ? 32 : 0) : nullptr;
+#pragma unroll
+        for (int k = 0; k < NOUT; ++k) {
+            if (MATRIX || (uint32_t)k < a.n_ch) {
                 float v = out[k];
-                if (has_depth && (uint32_t)k == a.depth_idx - a.ch_offset) v += depth_extra;
+                if (has_depth && (uint32_t)k + (MATRIX ? 32u : 0u) == a.depth_idx - a.ch_offset) v += depth_extra;
                 if (bg && inside) v += T * bg[k];
                 dst[k] = inside ? v : 0.f;
             }
@@ -388,7 +449,15 @@ static int launch_pixels(const PixelArgs &a, dim3 grid, dim3 block, hipStream_t 
 template <int CH>
 static int launch_points(const PointArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
     const size_t lds = (size_t)block.x * block.y * (2 * 16 + 4); // two float4 and the id per Gaussian
-    hipLaunchKernelGGL(rasterize_to_points_fwd_kernel<CH>, grid, block, lds, stream, a);
+    if constexpr (CH == 32 || CH == 33) {
+        // the matrix-core path: every channel of the kernel in use and whole wavefronts
+        if (a.n_ch == (uint32_t)CH && (block.x * block.y) % SPLATAD_WAVE == 0) {
+            hipLaunchKernelGGL((rasterize_to_points_fwd_kernel<CH, true>), grid, block, lds, stream, a);
+            SPLATAD_LAUNCH_CHECK();
+            return 0;
+        }
+    }
+    hipLaunchKernelGGL((rasterize_to_points_fwd_kernel<CH, false>), grid, block, lds, stream, a);
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }

@@ -149,15 +149,15 @@ rasterize_to_indices_kernel(IndexArgs a) {
                 todo &= todo - 1;
                 const float4 xyv = s_rec[2 * t];
                 const float4 con = s_rec[2 * t + 1];
-                float dx = (xyv.x + roll * xyv.z) - px;
-                float dy = (xyv.y + roll * xyv.w) - py;
+                float dx = gaussian_offset(xyv.x, xyv.z, roll, px);
+                float dy = gaussian_offset(xyv.y, xyv.w, roll, py);
                 if (LIDAR && ((folded >> bit) & 1ull)) { // uniform, rare: half a turn away
-                    dx = angle_difference(xyv.x + roll * xyv.z, px);
-                    dy = angle_difference(xyv.y + roll * xyv.w, py);
+                    dx = angle_difference(fmaf(roll, xyv.z, xyv.x), px);
+                    dy = angle_difference(fmaf(roll, xyv.w, xyv.y), py);
                 }
-                const float power = dx * (con.x * dx + con.y * dy) + con.z * dy * dy;
+                const float power = gaussian_power(con, dx, dy);
                 const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
-                const float next_T = T - alpha * T; // as in the compositing kernels
+                const float next_T = transmittance_behind(T, alpha); // as in the compositing kernels
                 const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
                                             wave_ballot(!(alpha < 1.f / 255.f));
                 const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);

@@ -347,8 +347,10 @@ def _lidar_scene(N, seed, H=16, W=256, tw=32, th=4, D=5, C=1):
     return d, proj
 
 
-@pytest.mark.parametrize("D,asum", [(5, True), (5, False), (33, True), (2, True), (40, True)])
-def test_rasterize_to_points(D, asum):
+@pytest.mark.parametrize("D,asum,with_bg", [(5, True, False), (5, False, False), (33, True, False),
+                                            (2, True, False), (40, True, False), (32, False, False),
+                                            (33, False, True), (32, True, True), (5, True, True)])
+def test_rasterize_to_points(D, asum, with_bg):
     from splatad_amd import isect_lidar_tiles, isect_offset_encode, rasterize_to_points
     H, W, tw, th = 16, 256, 32, 4
     d, proj = _lidar_scene(8000, 30 + D, H, W, tw, th, D)
@@ -358,12 +360,16 @@ def test_rasterize_to_points(D, asum):
     offs = isect_offset_encode(ids, 1, W // tw, H // th)
     feats = torch.cat([d["lidar_features"], depths[..., None]], -1)
     opac = d["opacities"][None].contiguous()
+    bg = None
+    if with_bg:
+        bg = torch.rand((1, D), device=DEV, generator=torch.Generator(device=DEV).manual_seed(D))
     rf, ra, rsum, med = rasterize_to_points(means2d, conics, feats, opac, pix_vels, dcomp,
-                                            d["raster_pts"], W, H, tw, th, offs, flat, asum, 0.3)
+                                            d["raster_pts"], W, H, tw, th, offs, flat, asum, 0.3,
+                                            backgrounds=bg)
     o = oracle.rasterize_to_points_fwd(
         to_np(means2d), to_np(conics), to_np(feats), to_np(opac), to_np(pix_vels), to_np(dcomp),
-        None, to_np(d["raster_pts"]), W, H, tw, th, asum, 0.3, to_np(offs), to_np(flat), D - 1,
-        precision="f64")
+        None if bg is None else to_np(bg), to_np(d["raster_pts"]), W, H, tw, th, asum, 0.3, to_np(offs),
+        to_np(flat), D - 1, precision="f64")
     assert_close(to_np(rf), o[0], atol=2e-4, rtol=1e-4, frac=RASTER_FRAC, name="features")
     assert_close(to_np(ra), o[1], atol=1e-4, frac=RASTER_FRAC, name="alphas")
     if asum:
