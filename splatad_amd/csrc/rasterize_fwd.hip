@@ -258,12 +258,26 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
     floatx16 acc_lo = {0}, acc_hi = {0};     // points 0-31 and 32-63 of the wavefront, D layout
     bool pair_open = false;                  // uniform: a Gaussian waits for its partner
     float pair_weight = 0.f, pair_feature = 0.f;
-    auto add_pair = [&](float w0, float w1, float f0, float f1) {
+    // w0, w1: the weights of two Gaussians (lane = point); p0, p1: their payload words, the
+    // features in lanes 0-31
+    auto add_pair = [&](float w0, float w1, float p0, float p1) {
         const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(w0), __float_as_uint(w1), false, false);
-        const float f = lane < 32 ? f0 : f1;
+        const auto sf = __builtin_amdgcn_permlane32_swap(__float_as_uint(p0), __float_as_uint(p1), false, false);
+        const float f = __uint_as_float(sf[0]); // lanes 0-31: features of the first, 32-63: of the second
         acc_lo = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(sw[0]), f, acc_lo, 0, 0, 0);
         acc_hi = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(sw[1]), f, acc_hi, 0, 0, 0);
     };
+
+    // MATRIX: one load per Gaussian brings everything compositing needs beyond the staged
+    // record, each lane its own word: lanes 0-31 the features of the matrix part (already in
+    // the B layout), lane 32 feature 32, lanes 33-36 the range velocity, the two depth
+    // compensations and the range.  payload_at + id * payload_step is lane's address.
+    const float *payload_at = a.colors + a.ch_offset + min(lane, 32u);
+    uint32_t payload_step = a.color_stride;
+    if (lane == 33) { payload_at = a.pix_vels + 2; payload_step = 3; }
+    if (lane == 34 || lane == 35) { payload_at = a.depth_comps + (lane - 34); payload_step = 2; }
+    if (lane >= 36) payload_at = a.colors + a.depth_idx;
+    if (!MATRIX || (CH == 32 && lane == 32)) payload_at = a.colors; // unused words: any valid address
 
     // A tile's list is long (thousands of Gaussians) and a compute unit holds few of these
     // workgroups, so nothing but the workgroup itself can hide the two dependent memory round
@@ -312,64 +326,138 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
             if (keep) keep = cull.may_touch(s_rec[RECORD * (base + lane)], s_rec[RECORD * (base + lane) + 1], unfolded_ok);
             uint64_t todo = wave_ballot(keep);
             const uint64_t folded = wave_ballot(keep && !unfolded_ok);
-            while (todo) {
-                const uint32_t bit = (uint32_t)__ffsll((unsigned long long)todo) - 1u;
-                const uint32_t t = base + bit;
-                todo &= todo - 1;
-                const float4 *rec = s_rec + RECORD * t;
-                const float4 uv = rec[0];
-                const float4 con = rec[1];
-                float dx = gaussian_offset(uv.x, uv.z, roll, rx);
-                float dy = gaussian_offset(uv.y, uv.w, roll, ry);
-                if ((folded >> bit) & 1ull) { // uniform, rare: half a turn away from the tile
-                    dx = angle_difference(fmaf(roll, uv.z, uv.x), rx);
-                    dy = angle_difference(fmaf(roll, uv.w, uv.y), ry);
-                }
-                const float power = gaussian_power(con, dx, dy);
-                const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
-                const float weight = alpha * T;
-                const float next_T = transmittance_behind(T, alpha);
-                // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
-                const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
-                                            wave_ballot(!(alpha < 1.f / 255.f));
-                const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
-                const uint64_t take_bits = valid_bits & ~stop_bits;
-                alive_bits &= ~stop_bits;
-                if (take_bits != 0) {
-                    const bool take = wave_lanes(take_bits);
-                    const float vis = take ? weight : 0.f;
-                    // the rest of the Gaussian, at addresses the whole wavefront shares
-                    const uint32_t g = (uint32_t)__builtin_amdgcn_readfirstlane(s_gid[t]);
-                    const uniform_f32_ptr crow = uniform_input(a.colors) + (size_t)g * a.color_stride;
-                    const uniform_f32_ptr dcp = uniform_input(a.depth_comps) + (size_t)g * 2;
-                    const float4 ext = make_float4(uniform_input(a.pix_vels)[(size_t)g * 3 + 2], dcp[0], dcp[1],
-                                                   crow[a.depth_idx]);
-                    if constexpr (MATRIX) {
-                        const float feature = a.colors[(size_t)g * a.color_stride + a.ch_offset + (lane & 31u)];
-                        if constexpr (CH == 33) out[0] += crow[a.ch_offset + 32] * vis;
-                        if (pair_open) add_pair(pair_weight, vis, pair_feature, feature);
-                        else { pair_weight = vis; pair_feature = feature; }
-                        pair_open = !pair_open;
-                    } else {
-                        float c[CH];
-                        if (a.n_ch == CH) { // uniform; the usual case
-                            load_uniform_row<CH>(crow + a.ch_offset, c);
-                        } else { // a pass narrower than the kernel: the spare accumulators are never stored
-                            const float *row = a.colors + (size_t)g * a.color_stride + a.ch_offset;
+            if constexpr (MATRIX) {
+                // The Gaussians that pass the footprint test are taken four at a time: list
+                // positions (scalar), ids from LDS, payloads from global memory and staged
+                // records from LDS are requested phase by phase for all four, so that the requests
+                // of a phase are in flight together; then the four are composited one after the
+                // other.  One at a time, a wavefront waits for a load from global memory per
+                // Gaussian, ten times longer than it works on it.  Slots beyond the last
+                // Gaussian repeat it.
+                constexpr int K = 4;
+                while (todo) {
+                    uint32_t ts[K];
+                    bool fold[K], have[K];
+                    uint32_t last_t = base, last_bit = 0;
 #pragma unroll
-                            for (int k = 0; k < CH; ++k) c[k] = row[min((uint32_t)k, a.n_ch - 1u)];
+                    for (int k = 0; k < K; ++k) {
+                        have[k] = todo != 0; // uniform
+                        if (have[k]) {
+                            last_bit = (uint32_t)__ffsll((unsigned long long)todo) - 1u;
+                            todo &= todo - 1;
+                            last_t = base + last_bit;
                         }
-#pragma unroll
-                        for (int k = 0; k < CH; ++k) out[k] += c[k] * vis;
+                        ts[k] = last_t;
+                        fold[k] = (folded >> last_bit) & 1ull;
                     }
-                    const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
-                    depth_extra += extra * vis;
-                    if (take && T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
-                    if (take && a.compute_alpha_sum && ext.w < pz - a.threshold) asum += alpha;
-                    cur_idx = take ? batch_start + t : cur_idx;
-                    T -= vis;
+                    int32_t ids[K];
+#pragma unroll
+                    for (int k = 0; k < K; ++k) ids[k] = s_gid[ts[k]];
+                    float pay[K];
+#pragma unroll
+                    for (int k = 0; k < K; ++k)
+                        pay[k] = payload_at[(size_t)(uint32_t)__builtin_amdgcn_readfirstlane(ids[k]) * payload_step];
+                    float4 uvs[K], cons[K];
+#pragma unroll
+                    for (int k = 0; k < K; ++k) {
+                        uvs[k] = s_rec[RECORD * ts[k]];
+                        cons[k] = s_rec[RECORD * ts[k] + 1];
+                    }
+#pragma unroll
+                    for (int k = 0; k < K; ++k) {
+                        if (!have[k] || alive_bits == 0) break; // uniform
+                        const float4 uv = uvs[k], con = cons[k];
+                        float dx = gaussian_offset(uv.x, uv.z, roll, rx);
+                        float dy = gaussian_offset(uv.y, uv.w, roll, ry);
+                        if (fold[k]) { // uniform, rare: half a turn away from the tile
+                            dx = angle_difference(fmaf(roll, uv.z, uv.x), rx);
+                            dy = angle_difference(fmaf(roll, uv.w, uv.y), ry);
+                        }
+                        const float power = gaussian_power(con, dx, dy);
+                        const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
+                        const float weight = alpha * T;
+                        const float next_T = transmittance_behind(T, alpha);
+                        const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
+                                                    wave_ballot(!(alpha < 1.f / 255.f));
+                        const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
+                        const uint64_t take_bits = valid_bits & ~stop_bits;
+                        alive_bits &= ~stop_bits;
+                        if (take_bits != 0) {
+                            const bool take = wave_lanes(take_bits);
+                            const float vis = take ? weight : 0.f;
+                            const int word = __float_as_int(pay[k]);
+                            const float4 ext = make_float4(__int_as_float(__builtin_amdgcn_readlane(word, 33)),
+                                                           __int_as_float(__builtin_amdgcn_readlane(word, 34)),
+                                                           __int_as_float(__builtin_amdgcn_readlane(word, 35)),
+                                                           __int_as_float(__builtin_amdgcn_readlane(word, 36)));
+                            if constexpr (CH == 33) out[0] += __int_as_float(__builtin_amdgcn_readlane(word, 32)) * vis;
+                            if (pair_open) add_pair(pair_weight, vis, pair_feature, pay[k]);
+                            else { pair_weight = vis; pair_feature = pay[k]; }
+                            pair_open = !pair_open;
+                            const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
+                            depth_extra += extra * vis;
+                            if (take && T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
+                            if (take && a.compute_alpha_sum && ext.w < pz - a.threshold) asum += alpha;
+                            cur_idx = take ? batch_start + ts[k] : cur_idx;
+                            T -= vis;
+                        }
+                    }
+                    if (alive_bits == 0) break;
                 }
-                if (alive_bits == 0) break;
+            } else {
+                while (todo) {
+                    const uint32_t bit = (uint32_t)__ffsll((unsigned long long)todo) - 1u;
+                    const uint32_t t = base + bit;
+                    todo &= todo - 1;
+                    const float4 *rec = s_rec + RECORD * t;
+                    const float4 uv = rec[0];
+                    const float4 con = rec[1];
+                    float dx = gaussian_offset(uv.x, uv.z, roll, rx);
+                    float dy = gaussian_offset(uv.y, uv.w, roll, ry);
+                    if ((folded >> bit) & 1ull) { // uniform, rare: half a turn away from the tile
+                        dx = angle_difference(fmaf(roll, uv.z, uv.x), rx);
+                        dy = angle_difference(fmaf(roll, uv.w, uv.y), ry);
+                    }
+                    const float power = gaussian_power(con, dx, dy);
+                    const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
+                    const float weight = alpha * T;
+                    const float next_T = transmittance_behind(T, alpha);
+                    // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
+                    const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
+                                                wave_ballot(!(alpha < 1.f / 255.f));
+                    const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
+                    const uint64_t take_bits = valid_bits & ~stop_bits;
+                    alive_bits &= ~stop_bits;
+                    if (take_bits != 0) {
+                        const bool take = wave_lanes(take_bits);
+                        const float vis = take ? weight : 0.f;
+                        // the rest of the Gaussian, at addresses the whole wavefront shares
+                        const uint32_t g = (uint32_t)__builtin_amdgcn_readfirstlane(s_gid[t]);
+                        const uniform_f32_ptr crow = uniform_input(a.colors) + (size_t)g * a.color_stride;
+                        const uniform_f32_ptr dcp = uniform_input(a.depth_comps) + (size_t)g * 2;
+                        const float4 ext = make_float4(uniform_input(a.pix_vels)[(size_t)g * 3 + 2], dcp[0], dcp[1],
+                                                       crow[a.depth_idx]);
+                        {
+                            float c[CH];
+                            if (a.n_ch == CH) { // uniform; the usual case
+                                load_uniform_row<CH>(crow + a.ch_offset, c);
+                            } else { // a pass narrower than the kernel: the spare accumulators are never stored
+                                const float *row = a.colors + (size_t)g * a.color_stride + a.ch_offset;
+#pragma unroll
+                                for (int k = 0; k < CH; ++k) c[k] = row[min((uint32_t)k, a.n_ch - 1u)];
+                            }
+#pragma unroll
+                            for (int k = 0; k < CH; ++k) out[k] += c[k] * vis;
+                        }
+                        const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
+                        depth_extra += extra * vis;
+                        if (take && T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
+                        if (take && a.compute_alpha_sum && ext.w < pz - a.threshold) asum += alpha;
+                        cur_idx = take ? batch_start + t : cur_idx;
+                        T -= vis;
+                    }
+                    if (alive_bits == 0) break;
+                }
             }
         }
     }
