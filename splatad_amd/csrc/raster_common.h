@@ -12,29 +12,6 @@ constexpr float kLog2e = 1.44269504088896341f;
 constexpr float kLn2 = 0.693147180559945309f;
 constexpr float kLog2Of255 = 7.99435343685886f;
 
-// A pointer to kernel inputs that no kernel of the launch writes, in the constant address
-// space: loads through it at a wavefront-uniform address go through the scalar unit into
-// scalar registers (one request per wavefront, no vector registers, usable directly as an
-// operand of vector arithmetic).
-typedef const float __attribute__((address_space(4))) *uniform_f32_ptr;
-__device__ __forceinline__ uniform_f32_ptr uniform_input(const float *p) {
-    return (uniform_f32_ptr)(uintptr_t)p;
-}
-
-// v[0..N) = p[0..N) for a wavefront-uniform p, in scalar loads of four floats where N allows.
-template <int N>
-__device__ __forceinline__ void load_uniform_row(uniform_f32_ptr p, float (&v)[N]) {
-    typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
-    typedef const f4u __attribute__((address_space(4))) *uniform_f4_ptr;
-#pragma unroll
-    for (int j = 0; j + 4 <= N; j += 4) {
-        const f4u q = *(uniform_f4_ptr)(p + j);
-        v[j] = q.x; v[j + 1] = q.y; v[j + 2] = q.z; v[j + 3] = q.w;
-    }
-#pragma unroll
-    for (int j = N / 4 * 4; j < N; ++j) v[j] = p[j];
-}
-
 // Staged exponent of a Gaussian: alpha = exp2(L - (A dx^2 + B dx dy + C dy^2)), i.e.
 // A = a log2(e) / 2, B = b log2(e), C = c log2(e) / 2 for the conic (a, b, c) and
 // L = log2(opacity) (-inf for opacity <= 0, which can then never reach alpha >= 1/255).

@@ -2,11 +2,14 @@
 //
 // One workgroup per (sensor, tile); one lane per pixel / point.  A tile's depth-sorted
 // Gaussian list is streamed through LDS in batches of one Gaussian per lane: the batch is
-// gathered once (coalesced over the id list, 16-byte records in LDS, colours included) and
-// then every lane walks the batch reading LDS at a wave-uniform address, which the LDS
-// serves as a broadcast without bank conflicts.  A 16x16 tile is four wavefronts of 16x4
-// pixels; a wavefront leaves the batch loop as soon as its 64 pixels are saturated and the
-// workgroup stops fetching batches once all of its pixels are.
+// gathered once (coalesced over the id list, 16-byte records in LDS; for cameras the colours
+// too, for lidars the many features only of the Gaussians a wavefront composites) and then
+// every wavefront tests 64 Gaussians at a time against its footprint and walks the survivors,
+// reading LDS at a wave-uniform address, which the LDS serves as a broadcast without bank
+// conflicts.  A 16x16 camera tile is four wavefronts of 8x8 pixels, a 64x4 lidar tile four
+// of 16x4 points; a wavefront leaves the batch loop as soon as its 64 pixels are saturated
+// and the workgroup stops fetching batches once all of its pixels are.  With 32 or 33
+// channels the lidar kernel accumulates 32 of them on the matrix cores.
 //
 // Compositing rules follow gsplat/cuda/csrc/rasterization.cu:1360-1518 (pixels) and
 // :2021-2219 (points) of the reference: alpha = min(0.999, o * exp(-sigma)); a Gaussian is
@@ -200,7 +203,7 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
     // and the alpha need.  A lidar point is a sample, not an area: of the Gaussians in a tile's
     // list only a few per cent reach alpha >= 1/255 at any of a wavefront's points, so the rest
     // of a Gaussian (its CH features, the range velocity, the depth compensation) is read from
-    // global memory by the wavefronts that composite it, through wavefront-uniform loads.
+    // global memory by the wavefronts that composite it, one word per lane.
     constexpr int RECORD = 2; // float4 per Gaussian
     float4 *s_rec = lds4;
     int32_t *s_gid = reinterpret_cast<int32_t *>(lds4 + (size_t)RECORD * blockDim.x * blockDim.y);
@@ -215,8 +218,10 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
     const uint32_t i = (tile_id / a.grid_w) * a.tile_height + ly;
     const uint32_t j = (tile_id % a.grid_w) * a.tile_width + lx;
 
-    const bool in_image = (i < a.H && j < a.W);
-    const size_t pix = ((size_t)cam * a.H + i) * a.W + j;
+    // the workgroup is padded to whole wavefronts (the payload words below need every lane of a
+    // wavefront to exist); lanes beyond the tile own no point
+    const bool in_image = (tr < a.tile_width * a.tile_height && i < a.H && j < a.W);
+    const size_t pix = in_image ? ((size_t)cam * a.H + i) * a.W + j : 0;
     float px = 0.f, py = 0.f, pz = 0.f, roll = 0.f;
     if (in_image) {
         const float4 p = reinterpret_cast<const float4 *>(a.raster_pts)[pix];
@@ -268,16 +273,16 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
         acc_hi = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(sw[1]), f, acc_hi, 0, 0, 0);
     };
 
-    // MATRIX: one load per Gaussian brings everything compositing needs beyond the staged
-    // record, each lane its own word: lanes 0-31 the features of the matrix part (already in
-    // the B layout), lane 32 feature 32, lanes 33-36 the range velocity, the two depth
-    // compensations and the range.  payload_at + id * payload_step is lane's address.
-    const float *payload_at = a.colors + a.ch_offset + min(lane, 32u);
+    // One load per Gaussian brings everything compositing needs beyond the staged record, each
+    // lane its own word: lanes 0-32 the features of this pass (for the matrix path lanes 0-31
+    // are the B layout), lanes 33-36 the range velocity, the two depth compensations and the
+    // range.  payload_at + id * payload_step is the lane's address; lanes without a word of
+    // their own repeat a neighbour's.
+    const float *payload_at = a.colors + a.ch_offset + min(lane, a.n_ch - 1u);
     uint32_t payload_step = a.color_stride;
     if (lane == 33) { payload_at = a.pix_vels + 2; payload_step = 3; }
     if (lane == 34 || lane == 35) { payload_at = a.depth_comps + (lane - 34); payload_step = 2; }
     if (lane >= 36) payload_at = a.colors + a.depth_idx;
-    if (!MATRIX || (CH == 32 && lane == 32)) payload_at = a.colors; // unused words: any valid address
 
     // A tile's list is long (thousands of Gaussians) and a compute unit holds few of these
     // workgroups, so nothing but the workgroup itself can hide the two dependent memory round
@@ -326,95 +331,49 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
             if (keep) keep = cull.may_touch(s_rec[RECORD * (base + lane)], s_rec[RECORD * (base + lane) + 1], unfolded_ok);
             uint64_t todo = wave_ballot(keep);
             const uint64_t folded = wave_ballot(keep && !unfolded_ok);
-            if constexpr (MATRIX) {
-                // The Gaussians that pass the footprint test are taken four at a time: list
-                // positions (scalar), ids from LDS, payloads from global memory and staged
-                // records from LDS are requested phase by phase for all four, so that the requests
-                // of a phase are in flight together; then the four are composited one after the
-                // other.  One at a time, a wavefront waits for a load from global memory per
-                // Gaussian, ten times longer than it works on it.  Slots beyond the last
-                // Gaussian repeat it.
-                constexpr int K = 4;
-                while (todo) {
-                    uint32_t ts[K];
-                    bool fold[K], have[K];
-                    uint32_t last_t = base, last_bit = 0;
+            // The Gaussians that pass the footprint test are taken four at a time: list
+            // positions (scalar), ids from LDS, payloads from global memory and staged
+            // records from LDS are requested phase by phase for all four, so that the requests
+            // of a phase are in flight together; then the four are composited one after the
+            // other.  One at a time, a wavefront waits for a load from global memory per
+            // Gaussian, ten times longer than it works on it.  Slots beyond the last
+            // Gaussian repeat it.
+            constexpr int K = 4;
+            while (todo) {
+                uint32_t ts[K];
+                bool fold[K], have[K];
+                uint32_t last_t = base, last_bit = 0;
 #pragma unroll
-                    for (int k = 0; k < K; ++k) {
-                        have[k] = todo != 0; // uniform
-                        if (have[k]) {
-                            last_bit = (uint32_t)__ffsll((unsigned long long)todo) - 1u;
-                            todo &= todo - 1;
-                            last_t = base + last_bit;
-                        }
-                        ts[k] = last_t;
-                        fold[k] = (folded >> last_bit) & 1ull;
+                for (int k = 0; k < K; ++k) {
+                    have[k] = todo != 0; // uniform
+                    if (have[k]) {
+                        last_bit = (uint32_t)__ffsll((unsigned long long)todo) - 1u;
+                        todo &= todo - 1;
+                        last_t = base + last_bit;
                     }
-                    int32_t ids[K];
-#pragma unroll
-                    for (int k = 0; k < K; ++k) ids[k] = s_gid[ts[k]];
-                    float pay[K];
-#pragma unroll
-                    for (int k = 0; k < K; ++k)
-                        pay[k] = payload_at[(size_t)(uint32_t)__builtin_amdgcn_readfirstlane(ids[k]) * payload_step];
-                    float4 uvs[K], cons[K];
-#pragma unroll
-                    for (int k = 0; k < K; ++k) {
-                        uvs[k] = s_rec[RECORD * ts[k]];
-                        cons[k] = s_rec[RECORD * ts[k] + 1];
-                    }
-#pragma unroll
-                    for (int k = 0; k < K; ++k) {
-                        if (!have[k] || alive_bits == 0) break; // uniform
-                        const float4 uv = uvs[k], con = cons[k];
-                        float dx = gaussian_offset(uv.x, uv.z, roll, rx);
-                        float dy = gaussian_offset(uv.y, uv.w, roll, ry);
-                        if (fold[k]) { // uniform, rare: half a turn away from the tile
-                            dx = angle_difference(fmaf(roll, uv.z, uv.x), rx);
-                            dy = angle_difference(fmaf(roll, uv.w, uv.y), ry);
-                        }
-                        const float power = gaussian_power(con, dx, dy);
-                        const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
-                        const float weight = alpha * T;
-                        const float next_T = transmittance_behind(T, alpha);
-                        const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
-                                                    wave_ballot(!(alpha < 1.f / 255.f));
-                        const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
-                        const uint64_t take_bits = valid_bits & ~stop_bits;
-                        alive_bits &= ~stop_bits;
-                        if (take_bits != 0) {
-                            const bool take = wave_lanes(take_bits);
-                            const float vis = take ? weight : 0.f;
-                            const int word = __float_as_int(pay[k]);
-                            const float4 ext = make_float4(__int_as_float(__builtin_amdgcn_readlane(word, 33)),
-                                                           __int_as_float(__builtin_amdgcn_readlane(word, 34)),
-                                                           __int_as_float(__builtin_amdgcn_readlane(word, 35)),
-                                                           __int_as_float(__builtin_amdgcn_readlane(word, 36)));
-                            if constexpr (CH == 33) out[0] += __int_as_float(__builtin_amdgcn_readlane(word, 32)) * vis;
-                            if (pair_open) add_pair(pair_weight, vis, pair_feature, pay[k]);
-                            else { pair_weight = vis; pair_feature = pay[k]; }
-                            pair_open = !pair_open;
-                            const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
-                            depth_extra += extra * vis;
-                            if (take && T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
-                            if (take && a.compute_alpha_sum && ext.w < pz - a.threshold) asum += alpha;
-                            cur_idx = take ? batch_start + ts[k] : cur_idx;
-                            T -= vis;
-                        }
-                    }
-                    if (alive_bits == 0) break;
+                    ts[k] = last_t;
+                    fold[k] = (folded >> last_bit) & 1ull;
                 }
-            } else {
-                while (todo) {
-                    const uint32_t bit = (uint32_t)__ffsll((unsigned long long)todo) - 1u;
-                    const uint32_t t = base + bit;
-                    todo &= todo - 1;
-                    const float4 *rec = s_rec + RECORD * t;
-                    const float4 uv = rec[0];
-                    const float4 con = rec[1];
+                int32_t ids[K];
+#pragma unroll
+                for (int k = 0; k < K; ++k) ids[k] = s_gid[ts[k]];
+                float pay[K];
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                    pay[k] = payload_at[(size_t)(uint32_t)__builtin_amdgcn_readfirstlane(ids[k]) * payload_step];
+                float4 uvs[K], cons[K];
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    uvs[k] = s_rec[RECORD * ts[k]];
+                    cons[k] = s_rec[RECORD * ts[k] + 1];
+                }
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    if (!have[k] || alive_bits == 0) break; // uniform
+                    const float4 uv = uvs[k], con = cons[k];
                     float dx = gaussian_offset(uv.x, uv.z, roll, rx);
                     float dy = gaussian_offset(uv.y, uv.w, roll, ry);
-                    if ((folded >> bit) & 1ull) { // uniform, rare: half a turn away from the tile
+                    if (fold[k]) { // uniform, rare: half a turn away from the tile
                         dx = angle_difference(fmaf(roll, uv.z, uv.x), rx);
                         dy = angle_difference(fmaf(roll, uv.w, uv.y), ry);
                     }
@@ -422,7 +381,6 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
                     const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
                     const float weight = alpha * T;
                     const float next_T = transmittance_behind(T, alpha);
-                    // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
                     const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
                                                 wave_ballot(!(alpha < 1.f / 255.f));
                     const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
@@ -431,33 +389,29 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
                     if (take_bits != 0) {
                         const bool take = wave_lanes(take_bits);
                         const float vis = take ? weight : 0.f;
-                        // the rest of the Gaussian, at addresses the whole wavefront shares
-                        const uint32_t g = (uint32_t)__builtin_amdgcn_readfirstlane(s_gid[t]);
-                        const uniform_f32_ptr crow = uniform_input(a.colors) + (size_t)g * a.color_stride;
-                        const uniform_f32_ptr dcp = uniform_input(a.depth_comps) + (size_t)g * 2;
-                        const float4 ext = make_float4(uniform_input(a.pix_vels)[(size_t)g * 3 + 2], dcp[0], dcp[1],
-                                                       crow[a.depth_idx]);
-                        {
-                            float c[CH];
-                            if (a.n_ch == CH) { // uniform; the usual case
-                                load_uniform_row<CH>(crow + a.ch_offset, c);
-                            } else { // a pass narrower than the kernel: the spare accumulators are never stored
-                                const float *row = a.colors + (size_t)g * a.color_stride + a.ch_offset;
+                        const int word = __float_as_int(pay[k]);
+                        const float4 ext = make_float4(__int_as_float(__builtin_amdgcn_readlane(word, 33)),
+                                                       __int_as_float(__builtin_amdgcn_readlane(word, 34)),
+                                                       __int_as_float(__builtin_amdgcn_readlane(word, 35)),
+                                                       __int_as_float(__builtin_amdgcn_readlane(word, 36)));
+                        if constexpr (MATRIX) {
+                            if constexpr (CH == 33) out[0] += __int_as_float(__builtin_amdgcn_readlane(word, 32)) * vis;
+                            if (pair_open) add_pair(pair_weight, vis, pair_feature, pay[k]);
+                            else { pair_weight = vis; pair_feature = pay[k]; }
+                            pair_open = !pair_open;
+                        } else { // accumulators beyond n_ch repeat the last channel and are never stored
 #pragma unroll
-                                for (int k = 0; k < CH; ++k) c[k] = row[min((uint32_t)k, a.n_ch - 1u)];
-                            }
-#pragma unroll
-                            for (int k = 0; k < CH; ++k) out[k] += c[k] * vis;
+                            for (int c = 0; c < CH; ++c) out[c] += __int_as_float(__builtin_amdgcn_readlane(word, c)) * vis;
                         }
                         const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
                         depth_extra += extra * vis;
                         if (take && T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
                         if (take && a.compute_alpha_sum && ext.w < pz - a.threshold) asum += alpha;
-                        cur_idx = take ? batch_start + t : cur_idx;
+                        cur_idx = take ? batch_start + ts[k] : cur_idx;
                         T -= vis;
                     }
-                    if (alive_bits == 0) break;
                 }
+                if (alive_bits == 0) break;
             }
         }
     }
@@ -538,8 +492,8 @@ template <int CH>
 static int launch_points(const PointArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
     const size_t lds = (size_t)block.x * block.y * (2 * 16 + 4); // two float4 and the id per Gaussian
     if constexpr (CH == 32 || CH == 33) {
-        // the matrix-core path: every channel of the kernel in use and whole wavefronts
-        if (a.n_ch == (uint32_t)CH && (block.x * block.y) % SPLATAD_WAVE == 0) {
+        // the matrix-core path: every channel of the kernel in use
+        if (a.n_ch == (uint32_t)CH) {
             hipLaunchKernelGGL((rasterize_to_points_fwd_kernel<CH, true>), grid, block, lds, stream, a);
             SPLATAD_LAUNCH_CHECK();
             return 0;
@@ -656,7 +610,7 @@ extern "C" int splatad_rasterize_to_points_fwd(
     a.render_colors = render_colors; a.render_alphas = render_alphas;
     a.alpha_sum = compute_alpha_sum ? alpha_sum : nullptr;
     a.last_ids = last_ids; a.median_depths = median_depths; a.tile_batches = tile_batches;
-    const dim3 grid(C * grid_w * grid_h), block(tile_width, tile_height);
+    const dim3 grid(C * grid_w * grid_h), block((tile_width * tile_height + SPLATAD_WAVE - 1) / SPLATAD_WAVE * SPLATAD_WAVE);
     const uint32_t pass = channels <= (uint32_t)kMaxPass ? channels : 32u;
     for (uint32_t off = 0; off < channels; off += pass) {
         a.ch_offset = off;

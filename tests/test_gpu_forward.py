@@ -347,12 +347,16 @@ def _lidar_scene(N, seed, H=16, W=256, tw=32, th=4, D=5, C=1):
     return d, proj
 
 
-@pytest.mark.parametrize("D,asum,with_bg", [(5, True, False), (5, False, False), (33, True, False),
-                                            (2, True, False), (40, True, False), (32, False, False),
-                                            (33, False, True), (32, True, True), (5, True, True)])
-def test_rasterize_to_points(D, asum, with_bg):
+@pytest.mark.parametrize("D,asum,with_bg,tile", [
+    (5, True, False, (32, 4)), (5, False, False, (32, 4)), (33, True, False, (32, 4)),
+    (2, True, False, (32, 4)), (40, True, False, (32, 4)), (32, False, False, (32, 4)),
+    (33, False, True, (32, 4)), (32, True, True, (32, 4)), (5, True, True, (32, 4)),
+    # tiles that do not fill a wavefront (the workgroup is padded) and one of four wavefronts
+    (5, True, False, (16, 2)), (33, True, True, (16, 1)), (3, False, False, (64, 4))])
+def test_rasterize_to_points(D, asum, with_bg, tile):
     from splatad_amd import isect_lidar_tiles, isect_offset_encode, rasterize_to_points
-    H, W, tw, th = 16, 256, 32, 4
+    H, W = 16, 256
+    tw, th = tile
     d, proj = _lidar_scene(8000, 30 + D, H, W, tw, th, D)
     radii, means2d, depths, conics, _, pix_vels, dcomp = proj
     res = d["azimuth_resolution"] * tw
