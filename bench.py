@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # They describe the 1M-Gaussian default only; other sizes report null.
 MEASURED_TRAFFIC_BYTES = {
     "camera": int((12972.0 * 2.0 + 48617.6) * 1024),
-    "lidar": int((27165.8 * 2.0 + 40098.4) * 1024),
+    "lidar": int((26334.2 * 2.0 + 40957.4) * 1024),
 }
 
 
@@ -365,7 +365,7 @@ def main():
             "workload": "128x2048 lidar sweep, %d Gaussians, 32 features + range, tile 64x4, "
                         "channel_chunk=33 (BASELINE configs[2])" % args.n,
             "n_isects": lid["n_isects"], "n_isects_consumed": lid["i_need"],
-            "roofline": {"kernel": "rasterize_to_points_fwd_kernel<%d>" % lid["channels"],
+            "roofline": {"kernel": "rasterize_to_points_fwd_kernel<%d, %s>" % (lid["channels"], "true" if lid["channels"] in (32, 33) else "false"),
                          "bound": "hbm", "achieved": l_ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": l_ach / HBM_PEAK_GBS,
                          "traffic": MEASURED_TRAFFIC_BYTES["lidar"] if args.n == 1_000_000 else None,
