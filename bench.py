@@ -207,7 +207,7 @@ def bench_lidar(args):
 
 def bench_backward(args):
     """Forward + backward (L1 losses on colour, depth and alpha against random targets, the
-    shape of BASELINE configs[4]) of the camera and the lidar call, ms per step."""
+    shape of a training step) of the camera and the lidar call, ms per step."""
     import torch
 
     from splatad_amd import lidar_rasterization, rasterization, workloads
@@ -311,7 +311,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build renders on one GPU; --gpus must be 1 "
-              "(sensors would shard across GPUs, see DESIGN.md)", file=sys.stderr)
+              "(with more GPUs each would render its own share of the sensors)", file=sys.stderr)
         sys.exit(2)
     import torch
 
