@@ -165,8 +165,11 @@ int splatad_view_colors_bwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint
  * and is shared by the two calls: with sort != 0, _count also enqueues the first
  * stages of the binning (they do not depend on n_isects) behind the counting
  * kernel, so that the GPU has work while the host sizes the outputs, and _fill
- * continues from what they left there.  Pass both calls the same sort flag, inputs
- * and stream, and leave the workspace untouched in between.  `lists` is
+ * continues from what they left there (_count reads depths for that: where a tile
+ * meets very many Gaussians the binning also cuts the depth axis into slabs, at
+ * quantiles of a sample of the depths; depths may be NULL when sort == 0).  Pass
+ * both calls the same sort flag, inputs and stream, and leave the workspace
+ * untouched in between.  `lists` is
  * splatad_isect_lists_bytes(total, n_isects) bytes of scratch for _fill alone.
  * _count waits for the counting kernel only (the kernel writes n_isects into a
  * pinned host slot, one per device, kept for the life of the process, and the
@@ -178,8 +181,8 @@ int splatad_view_colors_bwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint
 size_t splatad_isect_workspace_bytes(uint64_t total, uint32_t C, uint32_t n_tiles);
 size_t splatad_isect_lists_bytes(uint64_t total, int64_t n_isects);
 int splatad_isect_tiles_count(uint64_t total, uint32_t N, const int64_t *camera_ids,
-                              const float *means2d, const int32_t *radii, uint32_t C,
-                              uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
+                              const float *means2d, const int32_t *radii, const float *depths,
+                              uint32_t C, uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
                               int sort, int32_t *tiles_per_gauss, void *workspace,
                               int64_t *n_isects_host, splatad_stream_t stream);
 int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_ids,
@@ -190,8 +193,8 @@ int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_i
                              int64_t *isect_ids, int32_t *flatten_ids, int32_t *tile_offsets,
                              splatad_stream_t stream);
 int splatad_isect_lidar_tiles_count(uint64_t total, uint32_t N, const int64_t *camera_ids,
-                                    const float *means2d, const float *radii, uint32_t C,
-                                    const float *elev_boundaries, float tile_azim_resolution,
+                                    const float *means2d, const float *radii, const float *depths,
+                                    uint32_t C, const float *elev_boundaries, float tile_azim_resolution,
                                     float min_azim, uint32_t tile_width, uint32_t tile_height,
                                     int sort, int32_t *tiles_per_gauss, void *workspace,
                                     int64_t *n_isects_host, splatad_stream_t stream);
@@ -292,11 +295,23 @@ int splatad_rasterize_to_pixels_bwd(uint32_t C, int64_t n_isects, uint32_t chann
 /* rasterize_to_points_fwd_tensor, rasterization.cu:2221-2831 (kernel
  * :2021-2219).  Outputs of inactive points (range <= 0) are zero.
  * alpha_sum_until_points may be NULL when compute_alpha_sum_until_points == 0.
- * tile_batches: optional diagnostic as in splatad_rasterize_to_pixels_fwd. */
+ * tile_batches: optional diagnostic as in splatad_rasterize_to_pixels_fwd.
+ *
+ * range_channel (both directions; NULL for the reference's layout): the reference's
+ * callers concatenate the Gaussians' ranges behind their features first
+ * (gsplat/rendering.py:746 and :779, torch.cat of lidar_features and depths), a copy of the
+ * whole feature tensor per frame.  With range_channel given, `colors` keeps its
+ * channels - 1 feature values per Gaussian and the last channel (depth_channel_idx
+ * must be channels - 1, channels >= 2) is read from range_channel[total]; all
+ * [.., channels] image-side arrays are as before.  In the backward call v_colors
+ * then has channels - 1 values per Gaussian too and the last channel's gradient
+ * goes to v_range[total] (zero-filled like the others; NULL exactly when
+ * range_channel is). */
 int splatad_rasterize_to_points_fwd(uint32_t C, int64_t n_isects, uint32_t channels,
                                     const float *means2d, const float *conics,
-                                    const float *colors, const float *opacities,
-                                    const float *pix_vels, const float *depth_compensations,
+                                    const float *colors, const float *range_channel,
+                                    const float *opacities, const float *pix_vels,
+                                    const float *depth_compensations,
                                     const float *backgrounds, const float *raster_pts,
                                     uint32_t image_width, uint32_t image_height,
                                     uint32_t tile_width, uint32_t tile_height,
@@ -311,8 +326,9 @@ int splatad_rasterize_to_points_fwd(uint32_t C, int64_t n_isects, uint32_t chann
 /* rasterize_to_points_bwd_tensor, rasterization.cu:4056-4851 (kernel :3728-4054). */
 int splatad_rasterize_to_points_bwd(uint32_t C, int64_t n_isects, uint32_t channels,
                                     const float *means2d, const float *conics,
-                                    const float *colors, const float *opacities,
-                                    const float *pix_vels, const float *depth_compensations,
+                                    const float *colors, const float *range_channel,
+                                    const float *opacities, const float *pix_vels,
+                                    const float *depth_compensations,
                                     const float *backgrounds, const float *raster_pts,
                                     uint32_t image_width, uint32_t image_height,
                                     uint32_t tile_width, uint32_t tile_height,
@@ -324,7 +340,7 @@ int splatad_rasterize_to_points_bwd(uint32_t C, int64_t n_isects, uint32_t chann
                                     const float *v_render_alphas,
                                     const float *v_alpha_sum_until_points, float *v_means2d_abs,
                                     float *v_means2d, float *v_conics, float *v_colors,
-                                    float *v_opacities, float *v_pix_vels,
+                                    float *v_range, float *v_opacities, float *v_pix_vels,
                                     float *v_depth_compensations, uint64_t total, void *workspace,
                                     size_t workspace_bytes, splatad_stream_t stream);
 

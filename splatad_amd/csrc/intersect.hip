@@ -218,6 +218,7 @@ struct LaneWork {
     uint32_t base;          // camera * tiles per camera
     uint32_t idx;           // flatten id
     uint32_t depth_bits;
+    uint32_t slab;          // depth slab (binning with depth slabs only)
     int64_t cum;            // emission position of the first tile (unsorted output only)
     int32_t tx0, ty0, tx1, ty1; // tile rectangle, when x0.. describe coarse blocks instead
 };
@@ -231,6 +232,7 @@ __device__ __forceinline__ LaneWork broadcast_work(const LaneWork &w, int leader
     o.base = __shfl(w.base, leader, SPLATAD_WAVE);
     o.idx = __shfl(w.idx, leader, SPLATAD_WAVE);
     o.depth_bits = __shfl(w.depth_bits, leader, SPLATAD_WAVE);
+    o.slab = __shfl(w.slab, leader, SPLATAD_WAVE);
     o.cum = __shfl(w.cum, leader, SPLATAD_WAVE);
     o.tx0 = __shfl(w.tx0, leader, SPLATAD_WAVE);
     o.ty0 = __shfl(w.ty0, leader, SPLATAD_WAVE);
@@ -298,6 +300,7 @@ __device__ __forceinline__ LaneWork make_work(const TileGrid &g, WorkInputs in) 
     w.base = 0;
     w.idx = (uint32_t)in.idx;
     w.depth_bits = 0;
+    w.slab = 0;
     w.cum = 0;
     w.tx0 = w.ty0 = w.tx1 = w.ty1 = 0;
     int32_t x0, y0, x1, y1;
@@ -364,6 +367,32 @@ __device__ __forceinline__ uint32_t coarse_mask(const LaneWork &w, const CoarseG
     return m;
 }
 
+// Depth slabs.  Where a tile meets thousands of Gaussians (a lidar sweep's wide tiles), one
+// workgroup per tile segment sorts too few, too long segments to keep the GPU busy.  The
+// binning then cuts the depth axis into 1 << sshift slabs at bounds that are the same for all
+// tiles, and bins into (tile, slab) pairs: a tile's segment becomes consecutive sub-segments
+// in slab order, each sorted on its own, and since the slab is a non-decreasing function of
+// the depth bits the result is the same list.  The bounds are weighted quantiles of a sample
+// of the depths (weight = tiles met), so the sub-segments of an average tile are about equal;
+// any bounds whatsoever give the same output, balance is all they decide.
+constexpr uint32_t kSlabShiftMax = 4;
+constexpr uint32_t kSlabSamples = 512;
+
+// Slabs for `total` projected Gaussians on `segs` tiles, from the sizes alone.
+static uint32_t slab_shift_for(uint64_t total, uint64_t segs) {
+    const uint64_t per_tile = segs ? total / segs : 0;
+    uint32_t sshift = 0;
+    while (sshift < kSlabShiftMax && (128ull << sshift) <= per_tile) ++sshift;
+    return sshift;
+}
+
+// Number of bounds at or below the depth bits: non-decreasing in d whatever the bounds hold.
+__device__ __forceinline__ uint32_t slab_of(uint32_t d, const uint32_t *bounds, uint32_t n_bounds) {
+    uint32_t s = 0;
+    for (uint32_t k = 0; k < n_bounds; ++k) s += bounds[k] <= d ? 1u : 0u;
+    return s;
+}
+
 // Coarse binning without global atomics.  A fixed grid of workgroups strides over the
 // Gaussians; each keeps the counters of all coarse blocks in LDS.  COUNT pass: the
 // workgroup's counts go to its own row of a [workgroup][block] table.  The table is then
@@ -380,28 +409,35 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
                     const int64_t *__restrict__ camera_ids, const float *__restrict__ means2d,
                     const void *__restrict__ radii, const float *__restrict__ depths,
                     uint32_t cam_lo, uint32_t cam_hi, uint32_t n_blocks, int32_t *table,
-                    uint4 *__restrict__ entries) {
+                    uint4 *__restrict__ entries, uint32_t sshift,
+                    const uint32_t *__restrict__ slab_bounds) {
     extern __shared__ int32_t s_blocks[];
+    __shared__ uint32_t s_bounds[1u << kSlabShiftMax];
     SPLATAD_STAGE_ELEVATIONS(g)
-    const uint32_t per_cam = cg.cw * cg.ch, tiles_per_cam = g.tile_w * g.tile_h;
+    // blocks and block counters below are (coarse block, slab) pairs, the slab in the low bits
+    const uint32_t per_cam = (cg.cw * cg.ch) << sshift, tiles_per_cam = g.tile_w * g.tile_h;
     const uint32_t first = cam_lo * per_cam, count = (cam_hi - cam_lo) * per_cam;
+    const uint32_t n_bounds = (1u << sshift) - 1u;
     int32_t *row = table + (size_t)blockIdx.x * n_blocks + first;
     for (uint32_t b = threadIdx.x; b < count; b += blockDim.x) s_blocks[b] = FILL ? row[b] : 0;
+    if (threadIdx.x < n_bounds) s_bounds[threadIdx.x] = slab_bounds[threadIdx.x];
     __syncthreads();
+    const float *depths_needed = FILL || sshift ? depths : nullptr;
     const uint64_t round = (uint64_t)gridDim.x * blockDim.x;
     WorkInputs ahead = fetch_work((uint64_t)blockIdx.x * blockDim.x + threadIdx.x, total, N, camera_ids,
-                                  means2d, radii, FILL ? depths : nullptr, nullptr);
+                                  means2d, radii, depths_needed, nullptr);
     for (uint64_t base = (uint64_t)blockIdx.x * blockDim.x; base < total; base += round) { // uniform
         LaneWork mine = make_work<LIDAR>(g, ahead);
         // the inputs of the next round are requested before this round's emission
         ahead = fetch_work(base + round + threadIdx.x, total, N, camera_ids, means2d, radii,
-                           FILL ? depths : nullptr, nullptr);
+                           depths_needed, nullptr);
         const uint32_t cam = mine.base / tiles_per_cam;
         if (cam < cam_lo || cam >= cam_hi) mine.cnt = 0;
         mine.base = (cam - cam_lo) * per_cam;
+        mine.slab = slab_of(mine.depth_bits, s_bounds, n_bounds);
         to_coarse(mine, cg);
         for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t) {
-            const uint32_t local = w.base + coarse_index<LIDAR>(cg, y, x);
+            const uint32_t local = w.base + ((coarse_index<LIDAR>(cg, y, x) << sshift) | w.slab);
             const int32_t slot = atomicAdd(&s_blocks[local], 1);
             if (FILL) entries[slot] = make_uint4(w.idx, w.depth_bits, first + local, coarse_mask(w, cg, y, x));
         });
@@ -419,8 +455,8 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
 // FILL == true reserves the run in the tile's segment and writes the pairs.
 template <bool FILL>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
-isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t copies,
-                      uint32_t n_segments, const int64_t *__restrict__ n_entries_ptr,
+isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t sshift,
+                      uint32_t copies, uint32_t n_segments, const int64_t *__restrict__ n_entries_ptr,
                       const uint4 *__restrict__ entries, int32_t *__restrict__ tile_counts,
                       const int32_t *__restrict__ tile_starts, int32_t *__restrict__ tile_fill,
                       uint64_t *__restrict__ pairs) {
@@ -439,8 +475,10 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
         uint64_t todo = __ballot(has);
         while (todo) {
             const int leader = __ffsll((unsigned long long)todo) - 1;
-            const uint32_t block = (uint32_t)__shfl((int)rec.z, leader, SPLATAD_WAVE);
-            const bool in = has && rec.z == block;
+            // (coarse block, slab) of the leader; n_segments counts (tile, slab) pairs
+            const uint32_t block_slab = (uint32_t)__shfl((int)rec.z, leader, SPLATAD_WAVE);
+            const bool in = has && rec.z == block_slab;
+            const uint32_t block = block_slab >> sshift, slab = block_slab & ((1u << sshift) - 1u);
             todo &= ~__ballot(in);
             uint32_t my_cnt = 0;
             for (uint32_t t = 0; t < bits; ++t) {
@@ -453,7 +491,7 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
                 const uint32_t cam = block / per_cam, r = block % per_cam;
                 const uint32_t x = ((r % cg.cw) << cg.bshift) + (lane & ((1u << cg.bshift) - 1u));
                 const uint32_t y = ((r / cg.cw) << kCoarseRowShift) + (lane >> cg.bshift);
-                tile += (int64_t)cam * tile_w * tile_h + (int64_t)y * tile_w + x;
+                tile += (((int64_t)cam * tile_w * tile_h + (int64_t)y * tile_w + x) << sshift) | slab;
             }
             if (!FILL) {
                 if (my_cnt) atomicAdd(&tile_counts[tile], (int32_t)my_cnt);
@@ -571,6 +609,54 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t L, uint32_t ti
     return total;
 }
 
+// One workgroup, one sample per lane: kSlabSamples Gaussians at a fixed stride, ordered by
+// depth (every lane counts the smaller keys; all lanes read the same LDS words, which are
+// broadcasts).  A key is the depth bits with the sample's index in the low bits, which makes
+// the keys distinct at a depth resolution of 2^-14, plenty for a bound.  Bound k is the key at
+// which the running sum of the samples' tile counts passes k / n_slabs of the total.
+__global__ void __launch_bounds__(kSlabSamples)
+isect_slab_bounds_kernel(uint64_t total, const float *__restrict__ depths,
+                         const int32_t *__restrict__ tiles_per_gauss, uint32_t n_slabs,
+                         uint32_t *__restrict__ bounds) {
+    static_assert((kSlabSamples & (kSlabSamples - 1)) == 0 && kSlabSamples % 4 == 0, "power of two");
+    __shared__ __align__(16) uint32_t s_key[kSlabSamples];
+    __shared__ uint32_t s_sorted[kSlabSamples];
+    __shared__ uint32_t s_weight[kSlabSamples];
+    __shared__ uint32_t s_before[kSlabSamples];
+    __shared__ uint32_t s_wave[2 * (kSlabSamples / SPLATAD_WAVE)];
+    const uint32_t tid = threadIdx.x;
+    const uint64_t n = total < kSlabSamples ? total : kSlabSamples;
+    const uint64_t stride = n ? total / n : 1;
+    uint32_t key = ~(kSlabSamples - 1u) | tid, weight = 0; // no tiles: behind every depth
+    if (tid < n) {
+        const int32_t w = tiles_per_gauss[tid * stride];
+        if (w > 0) {
+            key = (__float_as_uint(depths[tid * stride]) & ~(kSlabSamples - 1u)) | tid;
+            weight = (uint32_t)min(w, 1 << 20); // capped: the sum stays below 2^32
+        }
+    }
+    s_key[tid] = key;
+    if (tid < n_slabs) bounds[tid] = 0xFFFFFFFFu;
+    __syncthreads();
+    uint32_t rank = 0;
+    for (uint32_t j = 0; j < kSlabSamples; j += 4) {
+        const uint4 q = *reinterpret_cast<const uint4 *>(&s_key[j]);
+        rank += (q.x < key ? 1u : 0u) + (q.y < key ? 1u : 0u) + (q.z < key ? 1u : 0u) + (q.w < key ? 1u : 0u);
+    }
+    s_sorted[rank] = key;
+    s_weight[rank] = weight;
+    __syncthreads();
+    const uint32_t sum = block_exclusive_scan(
+        kSlabSamples, tid, kSlabSamples, s_wave, [&](uint32_t i) { return s_weight[i]; },
+        [&](uint32_t i, uint32_t before, uint32_t) { s_before[i] = before; });
+    const uint32_t w = s_weight[tid], before = s_before[tid];
+    if (w == 0) return;
+    for (uint32_t k = 1; k < n_slabs; ++k) {
+        const uint32_t target = (uint32_t)((uint64_t)sum * k / n_slabs);
+        if (before < target && target <= before + w) bounds[k - 1] = s_sorted[tid];
+    }
+}
+
 // One workgroup per (camera, tile) segment: a bucket sort on the depth in three steps.
 //  1. The segment's range of depth bits (for positive floats a piecewise-linear logarithm
 //     of the depth) is cut into up to 512 equal fine bins and the entries are counted per
@@ -592,7 +678,7 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t L, uint32_t ti
 // Dynamic LDS: lds_words * 8 bytes of staging, the fine bins, 2 * bucket_cap counters.
 template <int ER, bool IN_LDS>
 __device__ __forceinline__ void sort_segment(uint32_t seg, uint32_t n_segments, uint32_t n_tiles,
-                                             uint32_t tile_n_bits, uint32_t lds_words,
+                                             uint32_t sshift, uint32_t tile_n_bits, uint32_t lds_words,
                                              uint32_t bucket_cap, int64_t n_isects,
                                              const int32_t *__restrict__ tile_starts,
                                              const uint64_t *__restrict__ pairs, int64_t *isect_ids,
@@ -611,7 +697,7 @@ __device__ __forceinline__ void sort_segment(uint32_t seg, uint32_t n_segments, 
     const uint32_t tid = threadIdx.x, nt = blockDim.x;
     const uint32_t lane = tid & (SPLATAD_WAVE - 1), wave = tid / SPLATAD_WAVE;
     const uint32_t n_waves = nt / SPLATAD_WAVE;
-    const uint64_t cam = seg / n_tiles, tile = seg % n_tiles;
+    const uint64_t cam = (seg >> sshift) / n_tiles, tile = (seg >> sshift) % n_tiles;
     const uint64_t key_hi = ((cam << tile_n_bits) | tile) << 32;
 
     constexpr int NR = ER > 0 ? ER : 1;
@@ -785,7 +871,7 @@ __constant__ const uint32_t kSortClassMin[kSortClasses + 1] = {0u,    512u,   20
 // beforehand).  The order inside a class is whatever the atomics give; every segment is sorted
 // on its own, so the result does not depend on it.
 __global__ void __launch_bounds__(SPLATAD_THREADS)
-isect_classify_segments_kernel(uint32_t n_segments, int64_t n_isects,
+isect_classify_segments_kernel(uint32_t n_segments, uint32_t sshift, int64_t n_isects,
                                const int32_t *__restrict__ tile_starts,
                                uint32_t *__restrict__ seg_counts, uint32_t *__restrict__ seg_lists,
                                int32_t *__restrict__ tile_offsets) {
@@ -796,7 +882,9 @@ isect_classify_segments_kernel(uint32_t n_segments, int64_t n_isects,
         const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
         n = (uint32_t)(stop - start);
         // a tile's offset is the start of its segment: the first row of the scanned table
-        if (tile_offsets != nullptr) tile_offsets[seg] = (int32_t)start;
+        // (with depth slabs: of its first slab's)
+        if (tile_offsets != nullptr && (seg & ((1u << sshift) - 1u)) == 0)
+            tile_offsets[seg >> sshift] = (int32_t)start;
     }
     int c = n == 0 ? -1 : 0;
     while (c >= 0 && c + 1 < kSortClasses && n > kSortClassMin[c + 1]) ++c;
@@ -818,7 +906,7 @@ isect_classify_segments_kernel(uint32_t n_segments, int64_t n_isects,
 // The workgroups of a launch share out the segments of one class; a launch has no more
 // workgroups than can be resident, so a class without segments costs next to nothing.
 template <int ER, bool IN_LDS>
-__global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
+__global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t sshift,
                                           uint32_t tile_n_bits, uint32_t lds_words,
                                           uint32_t bucket_cap, int64_t n_isects,
                                           const uint32_t *__restrict__ seg_count,
@@ -831,7 +919,7 @@ __global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles,
     __shared__ uint32_t s_big;
     const uint32_t count = *seg_count;
     for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) { // uniform across the workgroup
-        sort_segment<ER, IN_LDS>(seg_list[k], n_segments, n_tiles, tile_n_bits, lds_words, bucket_cap,
+        sort_segment<ER, IN_LDS>(seg_list[k], n_segments, n_tiles, sshift, tile_n_bits, lds_words, bucket_cap,
                                  n_isects, tile_starts, pairs, isect_ids, flatten_ids, lds_staged,
                                  s_wave, s_big);
         __syncthreads(); // the next segment reuses the LDS
@@ -847,8 +935,9 @@ constexpr uint32_t kSortBigThreads = 1024;
 constexpr uint32_t kSortBigInLds = 16384; // class 4 is staged in LDS
 
 __global__ void __launch_bounds__(kSortBigThreads)
-isect_big_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t tile_n_bits,
-                              int64_t n_isects, const uint32_t *__restrict__ seg_counts,
+isect_big_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t sshift,
+                              uint32_t tile_n_bits, int64_t n_isects,
+                              const uint32_t *__restrict__ seg_counts,
                               const uint32_t *__restrict__ seg_lists,
                               const int32_t *__restrict__ tile_starts,
                               const uint64_t *__restrict__ pairs, int64_t *isect_ids,
@@ -861,15 +950,15 @@ isect_big_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t ti
         const uint32_t *list = seg_lists + (size_t)cls * n_segments;
         for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) { // uniform across the workgroup
             if (cls == 4)
-                sort_segment<16, true>(list[k], n_segments, n_tiles, tile_n_bits, kSortBigInLds,
+                sort_segment<16, true>(list[k], n_segments, n_tiles, sshift, tile_n_bits, kSortBigInLds,
                                        sort_bucket_capacity(kSortBigInLds), n_isects, tile_starts, pairs,
                                        isect_ids, flatten_ids, lds_staged, s_wave, s_big);
             else if (cls == 5)
-                sort_segment<32, false>(list[k], n_segments, n_tiles, tile_n_bits, kSortWindow,
+                sort_segment<32, false>(list[k], n_segments, n_tiles, sshift, tile_n_bits, kSortWindow,
                                         sort_bucket_capacity(32768u), n_isects, tile_starts, pairs,
                                         isect_ids, flatten_ids, lds_staged, s_wave, s_big);
             else
-                sort_segment<0, false>(list[k], n_segments, n_tiles, tile_n_bits, kSortWindow,
+                sort_segment<0, false>(list[k], n_segments, n_tiles, sshift, tile_n_bits, kSortWindow,
                                        sort_bucket_capacity(0x7FFFFFFFu), n_isects, tile_starts, pairs,
                                        isect_ids, flatten_ids, lds_staged, s_wave, s_big);
             __syncthreads(); // the next segment reuses the LDS
@@ -882,7 +971,7 @@ static size_t sort_lds_bytes(uint32_t lds_words, uint32_t max_n) {
 }
 
 static int launch_big_segment_sort(uint32_t workgroups, uint32_t segs, uint32_t n_tiles,
-                                   uint32_t tile_n_bits, int64_t n_isects, const uint32_t *seg_counts,
+                                   uint32_t sshift, uint32_t tile_n_bits, int64_t n_isects, const uint32_t *seg_counts,
                                    const uint32_t *seg_lists, const int32_t *tile_starts,
                                    const uint64_t *pairs, int64_t *isect_ids, int32_t *flatten_ids,
                                    hipStream_t stream) {
@@ -899,7 +988,7 @@ static int launch_big_segment_sort(uint32_t workgroups, uint32_t segs, uint32_t 
         }
     }
     hipLaunchKernelGGL(isect_big_segment_sort_kernel, dim3(workgroups < segs ? workgroups : segs),
-                       dim3(kSortBigThreads), lds_bytes, stream, segs, n_tiles, tile_n_bits, n_isects,
+                       dim3(kSortBigThreads), lds_bytes, stream, segs, n_tiles, sshift, tile_n_bits, n_isects,
                        seg_counts, seg_lists, tile_starts, pairs, isect_ids, flatten_ids);
     SPLATAD_LAUNCH_CHECK();
     return 0;
@@ -907,7 +996,7 @@ static int launch_big_segment_sort(uint32_t workgroups, uint32_t segs, uint32_t 
 
 template <int ER, bool IN_LDS>
 static int launch_segment_sort(int cls, uint32_t threads, uint32_t max_n, uint32_t workgroups,
-                               uint32_t segs, uint32_t n_tiles, uint32_t tile_n_bits,
+                               uint32_t segs, uint32_t n_tiles, uint32_t sshift, uint32_t tile_n_bits,
                                int64_t n_isects, const uint32_t *seg_counts,
                                const uint32_t *seg_lists, const int32_t *tile_starts,
                                const uint64_t *pairs, int64_t *isect_ids, int32_t *flatten_ids,
@@ -927,7 +1016,7 @@ static int launch_segment_sort(int cls, uint32_t threads, uint32_t max_n, uint32
         }
     }
     hipLaunchKernelGGL((isect_segment_sort_kernel<ER, IN_LDS>), dim3(workgroups < segs ? workgroups : segs),
-                       dim3(threads), lds_bytes, stream, segs, n_tiles, tile_n_bits, lds_words,
+                       dim3(threads), lds_bytes, stream, segs, n_tiles, sshift, tile_n_bits, lds_words,
                        bucket_cap, n_isects, seg_counts + cls, seg_lists + (size_t)cls * segs,
                        tile_starts, pairs, isect_ids, flatten_ids);
     SPLATAD_LAUNCH_CHECK();
@@ -969,15 +1058,16 @@ struct IsectWorkspace {
     unsigned long long *n_isects; // [kCountWords] counters of the counting kernel, total first
     int64_t *n_entries;           // [1] length of the coarse lists
     int64_t *scan_total;          // [1]
+    uint32_t *slab_bounds;        // [1 << kSlabShiftMax] depth bits at which the slabs begin
     int32_t *zeroed;              // tile_counts, tile_fill are contiguous, cleared together
     uint64_t n_zeroed;
-    int32_t *tile_counts;         // [tile copies * C * n_tiles]
+    int32_t *tile_counts;         // [tile copies * segments], segments = C * n_tiles * slabs
     int32_t *tile_fill;           // same
     int32_t *coarse_counts;       // [coarse workgroups * C * blocks]
     int32_t *coarse_starts;       // same
-    int32_t *tile_starts;         // [tile copies * C * n_tiles]
+    int32_t *tile_starts;         // [tile copies * segments]
     uint32_t *seg_counts;         // [kSortClasses] segments per size class (in the cleared part)
-    uint32_t *seg_lists;          // [kSortClasses * C * n_tiles]
+    uint32_t *seg_lists;          // [kSortClasses * segments]
     int64_t *block_sums;          // scan scratch
     // the lists, whose size depends on the number of intersections
     int64_t *cum_before;          // [total] (sort == false)
@@ -1014,20 +1104,25 @@ static uint32_t coarse_workgroups(uint64_t total, uint64_t blocks) {
 }
 
 // Everything the two calls derive from the sizes alone, the same way in both.
+// With depth slabs (sshift > 0), segments are (tile, slab) pairs and blocks (coarse block,
+// slab) pairs.
 struct IsectPlan {
-    uint32_t n_tiles, tile_n_bits, per_cam, coarse_wgs, cams_per_launch;
+    uint32_t n_tiles, tile_n_bits, sshift, per_cam, coarse_wgs, cams_per_launch;
     uint64_t segs, blocks, cslots;
     CoarseGrid cg;
 };
 
 template <bool LIDAR>
-static IsectPlan isect_plan(const TileGrid &g, uint64_t total, uint32_t C) {
+static IsectPlan isect_plan(const TileGrid &g, uint64_t total, uint32_t C, int sort) {
     IsectPlan pl;
     pl.n_tiles = g.tile_w * g.tile_h;
     pl.tile_n_bits = splatad_bit_width(pl.n_tiles);
-    pl.segs = (uint64_t)C * pl.n_tiles;
     pl.cg = coarse_grid<LIDAR>(g);
-    pl.per_cam = pl.cg.cw * pl.cg.ch;
+    pl.sshift = sort ? slab_shift_for(total, (uint64_t)C * pl.n_tiles) : 0;
+    // one sensor's block counters have to fit the LDS of the coarse binning
+    while (pl.sshift > 0 && ((uint64_t)pl.cg.cw * pl.cg.ch << pl.sshift) > kCoarseLdsBlocks) --pl.sshift;
+    pl.segs = ((uint64_t)C * pl.n_tiles) << pl.sshift;
+    pl.per_cam = (pl.cg.cw * pl.cg.ch) << pl.sshift;
     pl.blocks = (uint64_t)C * pl.per_cam;
     pl.coarse_wgs = coarse_workgroups(total, pl.blocks);
     pl.cslots = pl.blocks * pl.coarse_wgs;
@@ -1047,6 +1142,7 @@ static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslo
     w.n_isects = (unsigned long long *)p;   p += splatad_align256(kCountWords * 8);
     w.n_entries = (int64_t *)p;             p += 256;
     w.scan_total = (int64_t *)p;            p += 256;
+    w.slab_bounds = (uint32_t *)p;          p += 256;
     w.zeroed = (int32_t *)p;
     w.tile_counts = (int32_t *)p;           p += splatad_align256(tslots * 4);
     w.tile_fill = (int32_t *)p;             p += splatad_align256(tslots * 4);
@@ -1075,6 +1171,7 @@ static size_t carve_lists(void *lists, uint64_t total, int64_t n_isects, IsectWo
 static size_t isect_ws_bytes(uint64_t total, uint64_t segs) {
     // there are at most as many coarse blocks as tiles, and coarse_workgroups() keeps the
     // table at 2^19 entries unless 64 rows exceed that
+    segs <<= slab_shift_for(total, segs); // the most slabs a plan for these sizes uses
     const uint64_t cslots_bound = segs * 64 > (1ull << 19) ? segs * 64 : (1ull << 19);
     return carve_isect(nullptr, total, segs, cslots_bound, nullptr);
 }
@@ -1119,8 +1216,8 @@ static int isect_device(IsectDevice **out) {
 template <bool LIDAR>
 static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const IsectWorkspace &w,
                                 uint64_t total, uint32_t N, const int64_t *camera_ids,
-                                const float *means2d, const void *radii, uint32_t C,
-                                hipStream_t stream) {
+                                const float *means2d, const void *radii, const float *depths,
+                                uint32_t C, hipStream_t stream) {
     SPLATAD_REQUIRE(pl.per_cam <= kCoarseLdsBlocks, "isect: %u x %u tiles per sensor exceed the "
                     "binning capacity", g.tile_w, g.tile_h);
     SPLATAD_REQUIRE(pl.blocks < (1ull << 31) && pl.cslots < (1ull << 31), "isect: tile grid too large");
@@ -1142,8 +1239,9 @@ static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const Is
         const uint32_t c1 = C - c0 < pl.cams_per_launch ? C : c0 + pl.cams_per_launch;
         hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, false>), dim3(pl.coarse_wgs),
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, pl.cg,
-                           total, N, camera_ids, means2d, radii, (const float *)nullptr, c0, c1,
-                           (uint32_t)pl.blocks, w.coarse_counts, (uint4 *)nullptr);
+                           total, N, camera_ids, means2d, radii, pl.sshift ? depths : nullptr, c0, c1,
+                           (uint32_t)pl.blocks, w.coarse_counts, (uint4 *)nullptr, pl.sshift,
+                           (const uint32_t *)w.slab_bounds);
     }
     SPLATAD_LAUNCH_CHECK();
     return launch_exclusive_scan<int32_t>(w.coarse_counts, (int64_t)pl.cslots,
@@ -1153,7 +1251,7 @@ static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const Is
 
 template <bool LIDAR>
 static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *camera_ids,
-                       const float *means2d, const void *radii, uint32_t C, int sort,
+                       const float *means2d, const void *radii, const float *depths, uint32_t C, int sort,
                        int32_t *tiles_per_gauss, void *workspace, int64_t *n_isects_host,
                        hipStream_t stream) {
     SPLATAD_REQUIRE(n_isects_host != nullptr, "isect: n_isects_host is null");
@@ -1162,7 +1260,8 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     SPLATAD_REQUIRE(total < (1ull << 31), "isect: number of projected Gaussians must be below 2^31");
     SPLATAD_REQUIRE(means2d && radii && tiles_per_gauss && workspace, "isect: null pointer argument");
     SPLATAD_REQUIRE(camera_ids != nullptr || N > 0, "isect: N is zero for unpacked input");
-    const IsectPlan pl = isect_plan<LIDAR>(g, total, C);
+    SPLATAD_REQUIRE(!sort || depths != nullptr, "isect: depths is null");
+    const IsectPlan pl = isect_plan<LIDAR>(g, total, C, sort);
     SPLATAD_REQUIRE(pl.n_tiles > 0 && C > 0, "isect: empty tile grid");
     SPLATAD_REQUIRE(pl.tile_n_bits + splatad_bit_width(C) <= 32,
                     "isect: camera and tile ids need more than 32 bits");
@@ -1185,9 +1284,16 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
                        total, means2d, radii, tiles_per_gauss, w.n_isects, dv->n.device);
     SPLATAD_LAUNCH_CHECK();
     // work for the GPU while the host learns the count and sizes the lists
-    if (sort)
-        if (int rc = enqueue_coarse_count<LIDAR>(g, pl, w, total, N, camera_ids, means2d, radii, C, stream))
+    if (sort) {
+        if (pl.sshift) {
+            hipLaunchKernelGGL(isect_slab_bounds_kernel, dim3(1), dim3(kSlabSamples), 0, stream, total,
+                               depths, (const int32_t *)tiles_per_gauss, 1u << pl.sshift, w.slab_bounds);
+            SPLATAD_LAUNCH_CHECK();
+        }
+        if (int rc = enqueue_coarse_count<LIDAR>(g, pl, w, total, N, camera_ids, means2d, radii, depths,
+                                                 C, stream))
             return rc;
+    }
     unsigned long long n = 0;
     if (int rc = host_word_wait(&dv->n, stream, "isect", &n)) return rc;
     SPLATAD_REQUIRE(n < (1ull << 31), "isect: %llu intersections exceed the int32 offset range", n);
@@ -1213,8 +1319,8 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     SPLATAD_REQUIRE(means2d && radii && depths && workspace && lists && isect_ids && flatten_ids,
                     "isect: null pointer argument");
     SPLATAD_REQUIRE(camera_ids != nullptr || N > 0, "isect: N is zero for unpacked input");
-    const IsectPlan pl = isect_plan<LIDAR>(g, total, C);
-    const uint32_t n_tiles = pl.n_tiles, tile_n_bits = pl.tile_n_bits;
+    const IsectPlan pl = isect_plan<LIDAR>(g, total, C, sort);
+    const uint32_t n_tiles = pl.n_tiles, tile_n_bits = pl.tile_n_bits, sshift = pl.sshift;
     const uint64_t segs = pl.segs;
     const CoarseGrid cg = pl.cg;
     IsectWorkspace w;
@@ -1238,7 +1344,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, true>), dim3(pl.coarse_wgs),
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, cg,
                            total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)pl.blocks,
-                           w.coarse_starts, w.entries);
+                           w.coarse_starts, w.entries, sshift, (const uint32_t *)w.slab_bounds);
     }
     SPLATAD_LAUNCH_CHECK();
     // tile segments: count, scan, fill.  The number of coarse entries stays on the device;
@@ -1247,7 +1353,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     uint64_t bin_wgs = ((uint64_t)n_isects + SPLATAD_THREADS - 1) / SPLATAD_THREADS;
     if (bin_wgs > 8192) bin_wgs = 8192;
     hipLaunchKernelGGL(isect_tile_bin_kernel<false>, dim3((uint32_t)bin_wgs),
-                       dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, tcopies,
+                       dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, sshift, tcopies,
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
                        w.tile_counts, (const int32_t *)nullptr, (int32_t *)nullptr,
                        (uint64_t *)nullptr);
@@ -1257,7 +1363,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                                         w.scan_total, w.block_sums, stream);
     if (rc) return rc;
     hipLaunchKernelGGL(isect_tile_bin_kernel<true>, dim3((uint32_t)bin_wgs),
-                       dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, tcopies,
+                       dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, sshift, tcopies,
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
                        w.tile_counts, (const int32_t *)w.tile_starts, w.tile_fill, w.pairs);
     SPLATAD_LAUNCH_CHECK();
@@ -1269,7 +1375,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     // of the lower classes.
     const uint32_t nseg = (uint32_t)segs;
     hipLaunchKernelGGL(isect_classify_segments_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream,
-                       nseg, n_isects, (const int32_t *)w.tile_starts, w.seg_counts, w.seg_lists,
+                       nseg, sshift, n_isects, (const int32_t *)w.tile_starts, w.seg_counts, w.seg_lists,
                        tile_offsets);
     SPLATAD_LAUNCH_CHECK();
     IsectDevice *ss = nullptr;
@@ -1278,12 +1384,12 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     SPLATAD_CHECK_HIP(hipEventRecord(ss->fork, stream));
     for (hipStream_t aux : ss->aux) SPLATAD_CHECK_HIP(hipStreamWaitEvent(aux, ss->fork, 0));
 #define SPLATAD_SORT_CLASS(cls, ER, IN_LDS, threads, hi, wgs, on)                                \
-    if ((rc = launch_segment_sort<ER, IN_LDS>(cls, threads, hi, wgs, nseg, n_tiles, tile_n_bits,  \
+    if ((rc = launch_segment_sort<ER, IN_LDS>(cls, threads, hi, wgs, nseg, n_tiles, sshift, tile_n_bits, \
                                               n_isects, w.seg_counts, w.seg_lists, w.tile_starts, \
                                               w.pairs, isect_ids, flatten_ids, on)) != 0)         \
         return rc;
     // the upper classes go first, on the caller's stream, which does not wait for the fork
-    if ((rc = launch_big_segment_sort(256u, nseg, n_tiles, tile_n_bits, n_isects, w.seg_counts, w.seg_lists,
+    if ((rc = launch_big_segment_sort(256u, nseg, n_tiles, sshift, tile_n_bits, n_isects, w.seg_counts, w.seg_lists,
                                       w.tile_starts, w.pairs, isect_ids, flatten_ids, stream)) != 0)
         return rc;
     SPLATAD_SORT_CLASS(2, 8, true, 512, 4096u, 1024u, ss->aux[0])
@@ -1310,14 +1416,15 @@ extern "C" size_t splatad_isect_lists_bytes(uint64_t total, int64_t n_isects) {
 }
 
 extern "C" int splatad_isect_tiles_count(uint64_t total, uint32_t N, const int64_t *camera_ids,
-                                         const float *means2d, const int32_t *radii, uint32_t C,
+                                         const float *means2d, const int32_t *radii,
+                                         const float *depths, uint32_t C,
                                          uint32_t tile_size, uint32_t tile_width,
                                          uint32_t tile_height, int sort, int32_t *tiles_per_gauss,
                                          void *workspace, int64_t *n_isects_host,
                                          splatad_stream_t stream) {
     SPLATAD_REQUIRE(tile_size > 0, "isect_tiles: tile_size is zero");
     TileGrid g{tile_size, tile_width, tile_height, 0.f, 0.f, nullptr};
-    return isect_count<false>(g, total, N, camera_ids, means2d, radii, C, sort, tiles_per_gauss,
+    return isect_count<false>(g, total, N, camera_ids, means2d, radii, depths, C, sort, tiles_per_gauss,
                               workspace, n_isects_host, (hipStream_t)stream);
 }
 
@@ -1338,7 +1445,7 @@ extern "C" int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_
 
 extern "C" int splatad_isect_lidar_tiles_count(uint64_t total, uint32_t N,
                                                const int64_t *camera_ids, const float *means2d,
-                                               const float *radii, uint32_t C,
+                                               const float *radii, const float *depths, uint32_t C,
                                                const float *elev_boundaries,
                                                float tile_azim_resolution, float min_azim,
                                                uint32_t tile_width, uint32_t tile_height, int sort,
@@ -1346,7 +1453,7 @@ extern "C" int splatad_isect_lidar_tiles_count(uint64_t total, uint32_t N,
                                                int64_t *n_isects_host, splatad_stream_t stream) {
     SPLATAD_REQUIRE(elev_boundaries != nullptr, "isect_lidar_tiles: elev_boundaries is null");
     TileGrid g{0u, tile_width, tile_height, tile_azim_resolution, min_azim, elev_boundaries};
-    return isect_count<true>(g, total, N, camera_ids, means2d, radii, C, sort, tiles_per_gauss,
+    return isect_count<true>(g, total, N, camera_ids, means2d, radii, depths, C, sort, tiles_per_gauss,
                              workspace, n_isects_host, (hipStream_t)stream);
 }
 

@@ -24,6 +24,12 @@ struct BwdArgs {
     uint32_t C;
     int64_t n_isects;
     uint32_t color_stride, ch_offset, n_ch;
+    // Lidar only: with range_channel given, `colors` and `v_colors` have rows of feat_stride =
+    // color_stride - 1 values and channel depth_idx (the last one) lives in range_channel /
+    // v_range, one value per Gaussian; otherwise feat_stride == color_stride.
+    uint32_t feat_stride;
+    const float *range_channel;
+    float *v_range;
     const float *means2d, *conics, *colors, *opacities, *pix_vels, *depth_comps, *rs_time,
         *backgrounds, *raster_pts;
     uint32_t W, H, tile_w_px, tile_h_px, grid_w, grid_h;
@@ -184,18 +190,24 @@ rasterize_bwd_kernel(BwdArgs a) {
             const float *cn = a.conics + (size_t)g * 3;
             f.cn[0] = cn[0]; f.cn[1] = cn[1]; f.cn[2] = cn[2];
             f.opac = a.opacities[g];
-            const float *crow = a.colors + (size_t)g * a.color_stride;
+            const float *crow = a.colors + (size_t)g * a.feat_stride;
+            const bool split = LIDAR && a.range_channel != nullptr;
             if (LIDAR) {
                 const float *v = a.pix_vels + (size_t)g * 3;
                 f.v[0] = v[0]; f.v[1] = v[1]; f.v[2] = v[2];
                 f.dc = reinterpret_cast<const float2 *>(a.depth_comps)[g];
-                f.depth_col = crow[a.depth_idx];
+                f.depth_col = split ? a.range_channel[g] : crow[a.depth_idx];
             } else {
                 const float2 v = reinterpret_cast<const float2 *>(a.pix_vels)[g];
                 f.v[0] = v.x; f.v[1] = v.y;
             }
 #pragma unroll
-            for (int k = 0; k < CH; ++k) f.col[k] = (uint32_t)k < a.n_ch ? crow[a.ch_offset + k] : 0.f;
+            for (int k = 0; k < CH; ++k) {
+                const uint32_t c = a.ch_offset + k;
+                float v = 0.f;
+                if ((uint32_t)k < a.n_ch) v = split && c == a.depth_idx ? f.depth_col : crow[min(c, a.feat_stride - 1u)];
+                f.col[k] = v;
+            }
         }
         return f;
     };
@@ -203,7 +215,11 @@ rasterize_bwd_kernel(BwdArgs a) {
     float *slot_base = nullptr;
     uint32_t slot_stride = 0;
     if (lane < CH) {
-        if ((uint32_t)lane < a.n_ch) { slot_base = a.v_colors + a.ch_offset + lane; slot_stride = a.color_stride; }
+        if ((uint32_t)lane < a.n_ch) {
+            const uint32_t c = a.ch_offset + lane;
+            if (LIDAR && a.v_range != nullptr && c == a.depth_idx) { slot_base = a.v_range; slot_stride = 1; }
+            else { slot_base = a.v_colors + c; slot_stride = a.feat_stride; }
+        }
     } else if (lane < ACC) {
         const int geo = lane - CH;
         const uint32_t nv = LIDAR ? 3 : 2;
@@ -396,7 +412,11 @@ unpack_gradients_kernel(uint64_t total, uint32_t stride, uint32_t width, BwdArgs
     const float val = a.packed[idx];
     if (val == 0.f) return;
     if (slot < width) {
-        if (slot < a.n_ch) a.v_colors[g * a.color_stride + a.ch_offset + slot] += val;
+        if (slot < a.n_ch) {
+            const uint32_t c = a.ch_offset + slot;
+            if (LIDAR && a.v_range != nullptr && c == a.depth_idx) a.v_range[g] += val;
+            else a.v_colors[g * a.feat_stride + c] += val;
+        }
         return;
     }
     const uint32_t geo = slot - width;
@@ -534,7 +554,7 @@ extern "C" int splatad_rasterize_to_pixels_bwd(
                         v_means2d && v_conics && v_colors && v_opacities && v_pix_vels,
                     "rasterize_to_pixels bwd: null pointer argument");
     BwdArgs a = {};
-    a.C = C; a.n_isects = n_isects; a.color_stride = channels;
+    a.C = C; a.n_isects = n_isects; a.color_stride = channels; a.feat_stride = channels;
     a.means2d = means2d; a.conics = conics; a.colors = colors; a.opacities = opacities;
     a.pix_vels = pix_vels; a.rs_time = rs_time; a.backgrounds = backgrounds;
     a.W = W; a.H = H; a.tile_w_px = tile_size; a.tile_h_px = tile_size; a.grid_w = tile_w; a.grid_h = tile_h;
@@ -550,17 +570,22 @@ extern "C" int splatad_rasterize_to_pixels_bwd(
 
 extern "C" int splatad_rasterize_to_points_bwd(
     uint32_t C, int64_t n_isects, uint32_t channels, const float *means2d, const float *conics,
-    const float *colors, const float *opacities, const float *pix_vels, const float *depth_comps,
-    const float *backgrounds, const float *raster_pts, uint32_t W, uint32_t H,
-    uint32_t tile_width, uint32_t tile_height, uint32_t grid_w, uint32_t grid_h,
+    const float *colors, const float *range_channel, const float *opacities, const float *pix_vels,
+    const float *depth_comps, const float *backgrounds, const float *raster_pts, uint32_t W,
+    uint32_t H, uint32_t tile_width, uint32_t tile_height, uint32_t grid_w, uint32_t grid_h,
     int compute_alpha_sum, float threshold, const int32_t *tile_offsets,
     const int32_t *flatten_ids, uint32_t depth_idx, const float *render_alphas,
     const int32_t *last_ids, const float *v_render_colors, const float *v_render_alphas,
     const float *v_alpha_sum, float *v_means2d_abs, float *v_means2d, float *v_conics,
-    float *v_colors, float *v_opacities, float *v_pix_vels, float *v_depth_comps, uint64_t total,
+    float *v_colors, float *v_range, float *v_opacities, float *v_pix_vels, float *v_depth_comps,
+    uint64_t total,
     void *workspace, size_t workspace_bytes, splatad_stream_t stream) {
     SPLATAD_REQUIRE(channels >= 1, "rasterize_to_points bwd: zero channels");
     SPLATAD_REQUIRE(depth_idx < channels, "rasterize_to_points bwd: depth channel %u of %u", depth_idx, channels);
+    SPLATAD_REQUIRE((range_channel == nullptr) == (v_range == nullptr),
+                    "rasterize_to_points bwd: range_channel and v_range go together");
+    SPLATAD_REQUIRE(range_channel == nullptr || (depth_idx + 1 == channels && channels >= 2),
+                    "rasterize_to_points bwd: a separate range channel must be the last of at least two");
     SPLATAD_REQUIRE(tile_width >= 1 && tile_height >= 1 && tile_width * tile_height <= 256,
                     "rasterize_to_points bwd: tile %ux%u exceeds 256 points", tile_width, tile_height);
     if (C == 0 || W == 0 || H == 0 || n_isects == 0) return 0;
@@ -574,6 +599,8 @@ extern "C" int splatad_rasterize_to_points_bwd(
                     "rasterize_to_points bwd: null pointer argument");
     BwdArgs a = {};
     a.C = C; a.n_isects = n_isects; a.color_stride = channels;
+    a.feat_stride = range_channel ? channels - 1 : channels;
+    a.range_channel = range_channel; a.v_range = v_range;
     a.means2d = means2d; a.conics = conics; a.colors = colors; a.opacities = opacities;
     a.pix_vels = pix_vels; a.depth_comps = depth_comps; a.backgrounds = backgrounds;
     a.raster_pts = raster_pts; a.W = W; a.H = H; a.tile_w_px = tile_width; a.tile_h_px = tile_height;

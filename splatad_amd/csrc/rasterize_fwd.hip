@@ -163,6 +163,11 @@ struct PointArgs {
     uint32_t C;
     int64_t n_isects;
     uint32_t color_stride, ch_offset, n_ch;
+    // With range_channel given, `colors` has rows of feat_stride = color_stride - 1 values and
+    // channel depth_idx (the last one) is range_channel[id]; otherwise feat_stride ==
+    // color_stride.
+    uint32_t feat_stride;
+    const float *range_channel;
     const float *means2d, *conics, *colors, *opacities, *pix_vels, *depth_comps, *backgrounds,
         *raster_pts;
     uint32_t W, H, tile_width, tile_height, grid_w, grid_h;
@@ -278,11 +283,12 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
     // are the B layout), lanes 33-36 the range velocity, the two depth compensations and the
     // range.  payload_at + id * payload_step is the lane's address; lanes without a word of
     // their own repeat a neighbour's.
-    const float *payload_at = a.colors + a.ch_offset + min(lane, a.n_ch - 1u);
-    uint32_t payload_step = a.color_stride;
+    const uint32_t payload_ch = lane >= 36 ? a.depth_idx : a.ch_offset + min(lane, a.n_ch - 1u);
+    const float *payload_at = a.colors + payload_ch;
+    uint32_t payload_step = a.feat_stride;
+    if (a.range_channel != nullptr && payload_ch == a.depth_idx) { payload_at = a.range_channel; payload_step = 1; }
     if (lane == 33) { payload_at = a.pix_vels + 2; payload_step = 3; }
     if (lane == 34 || lane == 35) { payload_at = a.depth_comps + (lane - 34); payload_step = 2; }
-    if (lane >= 36) payload_at = a.colors + a.depth_idx;
 
     // A tile's list is long (thousands of Gaussians) and a compute unit holds few of these
     // workgroups, so nothing but the workgroup itself can hide the two dependent memory round
@@ -579,15 +585,17 @@ extern "C" int splatad_rasterize_to_pixels_fwd(
 
 extern "C" int splatad_rasterize_to_points_fwd(
     uint32_t C, int64_t n_isects, uint32_t channels, const float *means2d, const float *conics,
-    const float *colors, const float *opacities, const float *pix_vels, const float *depth_comps,
-    const float *backgrounds, const float *raster_pts, uint32_t W, uint32_t H,
-    uint32_t tile_width, uint32_t tile_height, uint32_t grid_w, uint32_t grid_h,
+    const float *colors, const float *range_channel, const float *opacities, const float *pix_vels,
+    const float *depth_comps, const float *backgrounds, const float *raster_pts, uint32_t W,
+    uint32_t H, uint32_t tile_width, uint32_t tile_height, uint32_t grid_w, uint32_t grid_h,
     int compute_alpha_sum, float threshold, const int32_t *tile_offsets,
     const int32_t *flatten_ids, uint32_t depth_idx, float *render_colors, float *render_alphas,
     float *alpha_sum, int32_t *last_ids, float *median_depths, int32_t *tile_batches,
     splatad_stream_t stream) {
     SPLATAD_REQUIRE(channels >= 1, "rasterize_to_points: zero channels");
     SPLATAD_REQUIRE(depth_idx < channels, "rasterize_to_points: depth channel %u of %u", depth_idx, channels);
+    SPLATAD_REQUIRE(range_channel == nullptr || (depth_idx + 1 == channels && channels >= 2),
+                    "rasterize_to_points: a separate range channel must be the last of at least two");
     SPLATAD_REQUIRE(tile_width >= 1 && tile_height >= 1 && tile_width * tile_height <= 256,
                     "rasterize_to_points: tile %ux%u exceeds 256 points", tile_width, tile_height);
     if (C == 0 || W == 0 || H == 0) return 0;
@@ -601,6 +609,8 @@ extern "C" int splatad_rasterize_to_points_fwd(
                     "rasterize_to_points: null pointer argument");
     PointArgs a;
     a.C = C; a.n_isects = n_isects; a.color_stride = channels;
+    a.feat_stride = range_channel ? channels - 1 : channels;
+    a.range_channel = range_channel;
     a.means2d = means2d; a.conics = conics; a.colors = colors; a.opacities = opacities;
     a.pix_vels = pix_vels; a.depth_comps = depth_comps; a.backgrounds = backgrounds;
     a.raster_pts = raster_pts; a.W = W; a.H = H; a.tile_width = tile_width;

@@ -421,7 +421,7 @@ class _Ops:
             # ids so that isect_offset_encode() on the same, unmodified tensor is free
             offsets = (torch.empty((C, tile_h, tile_w), dtype=torch.int32, device=dev)
                        if sort else None)
-            head = (_u64(total), _u32(N), _p(camera_ids), _p(means2d), _p(radii))
+            head = (_u64(total), _u32(N), _p(camera_ids), _p(means2d), _p(radii), _p(depths))
             tail = (_u32(C), *grid_args, _u32(tile_w), _u32(tile_h), _i32(bool(sort)))
             n_host = _i64(0)
             _check(count(*head, *tail, _p(tiles_per_gauss), _p(ws), ctypes.byref(n_host),
@@ -431,7 +431,7 @@ class _Ops:
             flatten_ids = torch.empty((n_isects,), dtype=torch.int32, device=dev)
             if n_isects:
                 lists = _workspace(lib.splatad_isect_lists_bytes(_u64(total), _i64(n_isects)), dev)
-                _check(fill(*head, _p(depths), *tail, _i64(n_isects), _p(tiles_per_gauss), _p(ws),
+                _check(fill(*head, *tail, _i64(n_isects), _p(tiles_per_gauss), _p(ws),
                             _p(lists), _p(isect_ids), _p(flatten_ids), _p(offsets), _stream(dev)))
             else:
                 offsets = None
@@ -757,16 +757,19 @@ class _Ops:
                                 image_height, tile_width, tile_height,
                                 compute_alpha_sum_until_points,
                                 compute_alpha_sum_until_points_threshold, tile_offsets, flatten_ids,
-                                depth_channel_idx, tile_batches=None):
+                                depth_channel_idx, tile_batches=None, range_channel=None):
+        """With range_channel ([C, N] or [nnz]) the last channel is read from it and `colors`
+        holds the other channels only (depth_channel_idx counts it: colors.shape[-1])."""
         lib = load_library()
         means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
         colors = _in(colors, "colors"); opacities = _in(opacities, "opacities")
+        range_channel = _in(range_channel, "range_channel")
         pix_vels = _in(pix_vels, "pix_vels"); dc = _in(depth_compensations, "depth_compensations")
         backgrounds = _in(backgrounds, "backgrounds"); raster_pts = _in(raster_pts, "raster_pts")
         tile_offsets = _in(tile_offsets, "tile_offsets", torch.int32)
         flatten_ids = _in(flatten_ids, "flatten_ids", torch.int32)
         C, gh, gw = tile_offsets.shape
-        D, dev = colors.shape[-1], means2d.device
+        D, dev = colors.shape[-1] + (range_channel is not None), means2d.device
         f = dict(dtype=torch.float32, device=dev)
         renders = torch.empty((C, image_height, image_width, D), **f)
         alphas = torch.empty((C, image_height, image_width, 1), **f)
@@ -777,7 +780,8 @@ class _Ops:
         with torch.cuda.device(dev):
             _check(lib.splatad_rasterize_to_points_fwd(
                 _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics), _p(colors),
-                _p(opacities), _p(pix_vels), _p(dc), _p(backgrounds), _p(raster_pts),
+                _p(range_channel), _p(opacities), _p(pix_vels), _p(dc), _p(backgrounds),
+                _p(raster_pts),
                 _u32(image_width), _u32(image_height), _u32(tile_width), _u32(tile_height),
                 _u32(gw), _u32(gh), _i32(bool(compute_alpha_sum_until_points)),
                 _f32(compute_alpha_sum_until_points_threshold), _p(tile_offsets), _p(flatten_ids),
@@ -790,10 +794,13 @@ class _Ops:
                                 image_height, tile_width, tile_height, tile_offsets, flatten_ids,
                                 render_alphas, last_ids, v_render_colors, v_render_alphas,
                                 v_alpha_sum_until_points, absgrad, compute_alpha_sum_until_points,
-                                compute_alpha_sum_until_points_threshold, depth_channel_idx):
+                                compute_alpha_sum_until_points_threshold, depth_channel_idx,
+                                range_channel=None):
+        """With range_channel, an eighth result follows: its gradient."""
         lib = load_library()
         means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
         colors = _in(colors, "colors"); opacities = _in(opacities, "opacities")
+        range_channel = _in(range_channel, "range_channel")
         pix_vels = _in(pix_vels, "pix_vels"); dc = _in(depth_compensations, "depth_compensations")
         backgrounds = _in(backgrounds, "backgrounds"); raster_pts = _in(raster_pts, "raster_pts")
         tile_offsets = _in(tile_offsets, "tile_offsets", torch.int32)
@@ -804,25 +811,28 @@ class _Ops:
         v_render_alphas = _in(v_render_alphas, "v_render_alphas")
         v_asum = _in(v_alpha_sum_until_points, "v_alpha_sum_until_points")
         C, gh, gw = tile_offsets.shape
-        D, dev = colors.shape[-1], means2d.device
-        v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_dc, v_means2d_abs = _zeros_like_many(
-            means2d, conics, colors, opacities, pix_vels, dc, means2d if absgrad else None)
+        D, dev = colors.shape[-1] + (range_channel is not None), means2d.device
+        (v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_dc, v_means2d_abs,
+         v_range) = _zeros_like_many(means2d, conics, colors, opacities, pix_vels, dc,
+                                     means2d if absgrad else None, range_channel)
         if flatten_ids.shape[0]:
             total = means2d.numel() // 2
             with torch.cuda.device(dev):
                 ws = _bwd_workspace(lib, total, D, True, dev)
                 _check(lib.splatad_rasterize_to_points_bwd(
                     _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics),
-                    _p(colors), _p(opacities), _p(pix_vels), _p(dc), _p(backgrounds),
+                    _p(colors), _p(range_channel), _p(opacities), _p(pix_vels), _p(dc), _p(backgrounds),
                     _p(raster_pts), _u32(image_width), _u32(image_height), _u32(tile_width),
                     _u32(tile_height), _u32(gw), _u32(gh),
                     _i32(bool(compute_alpha_sum_until_points)),
                     _f32(compute_alpha_sum_until_points_threshold), _p(tile_offsets),
                     _p(flatten_ids), _u32(depth_channel_idx), _p(render_alphas), _p(last_ids),
                     _p(v_render_colors), _p(v_render_alphas), _p(v_asum), _p(v_means2d_abs),
-                    _p(v_means2d), _p(v_conics), _p(v_colors), _p(v_opacities), _p(v_pix_vels),
-                    _p(v_dc), _u64(total), _p(ws), ctypes.c_size_t(0 if ws is None else ws.numel()),
+                    _p(v_means2d), _p(v_conics), _p(v_colors), _p(v_range), _p(v_opacities),
+                    _p(v_pix_vels), _p(v_dc), _u64(total), _p(ws), ctypes.c_size_t(0 if ws is None else ws.numel()),
                     _stream(dev)))
+        if range_channel is not None:
+            return v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_dc, v_range
         return v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_dc
 
     # ------------------------------------------------------------------ index lists

@@ -414,10 +414,15 @@ def rasterize_to_points(
     backgrounds: Optional[Tensor] = None,  # [C, channels]
     packed: bool = False,
     absgrad: bool = False,
+    ranges: Optional[Tensor] = None,  # [C, N] or [nnz]
 ) -> Tuple[Tensor, Tensor, Optional[Tensor], Tensor]:
     """Alpha compositing onto a grid of lidar points given in spherical coordinates; the last
     feature channel is the Gaussian's range and receives the depth-compensation and range-rate
     terms.  Points with range <= 0 are skipped (zeros).
+
+    `ranges` (not in the reference) spares the caller the concatenation of features and
+    ranges: given it, `lidar_features` holds channels - 1 features per Gaussian and the range
+    channel is read from `ranges`; results and gradients are those of the concatenated call.
 
     Returns (render_features[C,H,W,channels], render_alphas[C,H,W,1],
     alpha_sum_until_points[C,H,W,1] | None, median_depths[C,H,W,1]).
@@ -431,6 +436,7 @@ def rasterize_to_points(
         assert opacities.shape == (nnz,), opacities.shape
         assert pix_vels.shape == (nnz, 3), pix_vels.shape
         assert depth_compensations.shape == (nnz, 2), depth_compensations.shape
+        assert ranges is None or ranges.shape == (nnz,), ranges.shape
     else:
         N = means2d.size(1)
         assert means2d.shape == (C, N, 2), means2d.shape
@@ -439,11 +445,14 @@ def rasterize_to_points(
         assert opacities.shape == (C, N), opacities.shape
         assert pix_vels.shape == (C, N, 3), pix_vels.shape
         assert depth_compensations.shape == (C, N, 2), depth_compensations.shape
+        assert ranges is None or ranges.shape == (C, N), ranges.shape
+    channels = lidar_features.shape[-1] + (ranges is not None)
     if backgrounds is not None:
-        assert backgrounds.shape == (C, lidar_features.shape[-1]), backgrounds.shape
+        assert backgrounds.shape == (C, channels), backgrounds.shape
         backgrounds = backgrounds.contiguous()
-    channels = lidar_features.shape[-1]
     depth_channel_idx = channels - 1
+    if ranges is not None and channels < 2:
+        raise ValueError("ranges needs at least one feature channel beside it")
     if channels > MAX_CHANNELS or channels == 0:
         raise ValueError(f"Unsupported number of lidar_features channels: {channels}")
     tile_grid_height, tile_grid_width = isect_offsets.shape[1:3]
@@ -457,6 +466,7 @@ def rasterize_to_points(
         backgrounds, raster_pts.contiguous(), image_width, image_height, tile_width, tile_height,
         isect_offsets.contiguous(), flatten_ids.contiguous(), compute_alpha_sum_until_points,
         compute_alpha_sum_until_points_threshold, absgrad, depth_channel_idx,
+        None if ranges is None else ranges.contiguous(),
     )
 
 
@@ -725,16 +735,17 @@ class _RasterizeToPoints(torch.autograd.Function):
     def forward(ctx, means2d, conics, colors, opacities, pix_vels, depth_compensations,
                 backgrounds, raster_pts, width, height, tile_width, tile_height, isect_offsets,
                 flatten_ids, compute_alpha_sum_until_points,
-                compute_alpha_sum_until_points_threshold, absgrad, depth_channel_idx):
+                compute_alpha_sum_until_points_threshold, absgrad, depth_channel_idx,
+                ranges=None):
         (render_colors, render_alphas, last_ids, alpha_sum_until_points,
          median_depths) = _make_lazy_hip_func("rasterize_to_points_fwd")(
             means2d, conics, colors, opacities, pix_vels, depth_compensations, backgrounds,
             raster_pts, width, height, tile_width, tile_height, compute_alpha_sum_until_points,
             compute_alpha_sum_until_points_threshold, isect_offsets, flatten_ids,
-            depth_channel_idx)
+            depth_channel_idx, range_channel=ranges)
         ctx.save_for_backward(means2d, conics, colors, opacities, pix_vels, depth_compensations,
                               backgrounds, raster_pts, isect_offsets, flatten_ids, render_alphas,
-                              last_ids)
+                              last_ids, ranges)
         ctx.geom = (width, height, tile_width, tile_height)
         ctx.absgrad = absgrad
         ctx.alpha_sum = (compute_alpha_sum_until_points, compute_alpha_sum_until_points_threshold)
@@ -748,25 +759,28 @@ class _RasterizeToPoints(torch.autograd.Function):
     @staticmethod
     def backward(ctx, v_render_colors, v_render_alphas, v_alpha_sum_until_points, v_median_depths):
         (means2d, conics, colors, opacities, pix_vels, depth_compensations, backgrounds,
-         raster_pts, isect_offsets, flatten_ids, render_alphas, last_ids) = ctx.saved_tensors
+         raster_pts, isect_offsets, flatten_ids, render_alphas, last_ids,
+         ranges) = ctx.saved_tensors
         compute_sum, threshold = ctx.alpha_sum
         if compute_sum and v_alpha_sum_until_points is not None:
             v_sum = v_alpha_sum_until_points.contiguous()
         else:
             v_sum = torch.zeros_like(v_render_alphas)
-        (v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities, v_pix_vels,
-         v_depth_compensations) = _make_lazy_hip_func("rasterize_to_points_bwd")(
+        grads = _make_lazy_hip_func("rasterize_to_points_bwd")(
             means2d, conics, colors, opacities, pix_vels, depth_compensations, backgrounds,
             raster_pts, *ctx.geom, isect_offsets, flatten_ids, render_alphas, last_ids,
             v_render_colors.contiguous(), v_render_alphas.contiguous(), v_sum, ctx.absgrad,
-            compute_sum, threshold, ctx.depth_channel_idx)
+            compute_sum, threshold, ctx.depth_channel_idx, range_channel=ranges)
+        (v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities, v_pix_vels,
+         v_depth_compensations) = grads[:7]
+        v_ranges = grads[7] if ranges is not None else None
         if ctx.absgrad:
             means2d.absgrad = v_means2d_abs
         v_backgrounds = None
         if ctx.needs_input_grad[6]:
             v_backgrounds = (v_render_colors * (1.0 - render_alphas).float()).sum(dim=(1, 2))
         return (v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_depth_compensations,
-                v_backgrounds) + (None,) * 11
+                v_backgrounds) + (None,) * 11 + (v_ranges,)
 
 
 # ---------------------------------------------------------------------------

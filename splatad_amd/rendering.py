@@ -385,16 +385,20 @@ def lidar_rasterization(
     n_elevation_tiles = math.ceil(n_elevation_channels / tile_height)
     tile_azimuth_resolution = azimuth_resolution * tile_width
     n_azimuth_tiles = math.ceil((max_azimuth - min_azimuth) / tile_azimuth_resolution)
-    # features to composite (the range is appended as last channel further down, on a helper
-    # stream beside the segment sort of the tile intersection).  Chunks carry channel_chunk-1 features plus the range; the
-    # chunk count is the reference's (rendering.py:735): features beyond
-    # n_chunks*(channel_chunk-1) are not rendered, e.g. D=63 with channel_chunk=32.
+    # Features to composite.  Chunks carry channel_chunk-1 features plus the range; the chunk
+    # count is the reference's (rendering.py:735): features beyond n_chunks*(channel_chunk-1)
+    # are not rendered, e.g. D=63 with channel_chunk=32.  The reference appends the range to
+    # every chunk (rendering.py:746, :779); here a single chunk hands the compositing kernels
+    # features and ranges as they are, and only the slices of a chunked call are copied
+    # together with the range, on a helper stream beside the segment sort.
     if (D + 1) > channel_chunk:
         n_chunks = (D + channel_chunk) // channel_chunk
         chunks = [lidar_features[..., i * (channel_chunk - 1) : (i + 1) * (channel_chunk - 1)]
                   for i in range(n_chunks)]
+    elif D == 0:
+        chunks = [lidar_features]  # the range alone: nothing to spare
     else:
-        chunks = [lidar_features]
+        chunks = None
     beside = _Beside(means.device)  # fork: features and ranges are enqueued
     tiles_per_gauss, isect_ids, flatten_ids = isect_lidar_tiles(
         means2d, radii, depths, elev_boundaries=tile_elevation_boundaries,
@@ -402,23 +406,27 @@ def lidar_rasterization(
         n_cameras=C, camera_ids=camera_ids, gaussian_ids=gaussian_ids,
     )
     isect_offsets = isect_offset_encode(isect_ids, C, n_azimuth_tiles, n_elevation_tiles)
-    chunks = [_AppendChannel.apply(beside, f, depths) for f in chunks]
-    beside.join(*chunks)
+    if chunks is not None:
+        chunks = [_AppendChannel.apply(beside, f, depths) for f in chunks]
+        beside.join(*chunks)
 
     image_width = raster_pts.shape[-2]
     image_height = raster_pts.shape[-3]
 
-    def composite(feats):
+    def composite(feats, ranges=None):
         return rasterize_to_points(
             means2d, conics, feats, opacities, pix_vels,
             depth_compensations, raster_pts, image_width, image_height, tile_width, tile_height,
             isect_offsets, flatten_ids,
             compute_alpha_sum_until_points=compute_alpha_sum_until_points,
             compute_alpha_sum_until_points_threshold=compute_alpha_sum_until_points_threshold,
-            packed=packed, absgrad=absgrad,
+            packed=packed, absgrad=absgrad, ranges=ranges,
         )
 
-    if len(chunks) > 1:
+    if chunks is None:
+        render_lidar_features, render_alphas, alpha_sum_until_points, median_depths = composite(
+            lidar_features, depths)
+    elif len(chunks) > 1:
         feats_out, alphas_out, sums_out, medians_out = [], [], [], []
         for i, chunk in enumerate(chunks):
             rf, ra, rs_, md = composite(chunk)

@@ -95,7 +95,10 @@ class OracleOps:
         return tuple(_t(o) for o in out)
 
     def rasterize_to_points_fwd(self, means2d, conics, colors, opacities, pix_vels, dcomp, backgrounds,
-                                raster_pts, W, H, tw, th, asum, thr, offsets, flatten_ids, depth_idx):
+                                raster_pts, W, H, tw, th, asum, thr, offsets, flatten_ids, depth_idx,
+                                range_channel=None):
+        if range_channel is not None:  # the oracle follows the reference: one concatenated tensor
+            colors = torch.cat([colors, range_channel[..., None]], dim=-1)
         out = oracle.rasterize_to_points_fwd(_n(means2d), _n(conics), _n(colors), _n(opacities),
                                              _n(pix_vels), _n(dcomp), _n(backgrounds), _n(raster_pts), W, H,
                                              tw, th, asum, thr, _n(offsets), _n(flatten_ids), depth_idx,

@@ -284,9 +284,23 @@ def test_rasterize_to_points_backward(D, asum):
         loss_r = loss_r + (o[2] * T64(ws)).sum()
     grads_g = torch.autograd.grad(loss_g, lg)
     grads_r = torch.autograd.grad(loss_r, lr)
-    for n, a, b in zip(("means2d", "conics", "features", "opacities", "pix_vels", "depth_compensations"),
-                       grads_g, grads_r):
+    names = ("means2d", "conics", "features", "opacities", "pix_vels", "depth_compensations")
+    for n, a, b in zip(names, grads_g, grads_r):
         assert_grad_close(to_np(a), b.numpy(), f"{n} D={D}")
+    # features and ranges handed over separately: the gradient of the last channel comes apart
+    ls = [to_dev(x).requires_grad_() for x in (means2d, conics, np.ascontiguousarray(feats[..., :-1]), opac,
+                                               pv, dc, depths)]
+    sf, sa, ssum, _ = rasterize_to_points(ls[0], ls[1], ls[2], ls[3], ls[4], ls[5], to_dev(rp), W, H, tw, th,
+                                          offs, flat, asum, 0.3, ranges=ls[6])
+    assert torch.equal(sf, rf) and torch.equal(sa, ra)
+    loss_s = (sf * to_dev(wc)).sum() + (sa * to_dev(wa)).sum()
+    if asum:
+        loss_s = loss_s + (ssum * to_dev(ws)).sum()
+    grads_s = torch.autograd.grad(loss_s, ls)
+    for n, a, b in zip(names, grads_s[:6], grads_r):
+        want = b.numpy()[..., :-1] if n == "features" else b.numpy()
+        assert_grad_close(to_np(a), want, f"split {n} D={D}")
+    assert_grad_close(to_np(grads_s[6]), grads_r[2].numpy()[..., -1], f"split ranges D={D}")
 
 
 @pytest.mark.parametrize("deg", [0, 1, 2, 3, 4])

@@ -384,6 +384,12 @@ def test_rasterize_to_points(D, asum, with_bg, tile):
     assert_close(to_np(med), o[4], atol=1e-3, rtol=1e-4, frac=0.999, name="median")
     assert float(ra.max()) > 0.5
     assert (to_np(rf)[0, 0, :7] == 0).all() and (to_np(ra)[0, 3, 5] == 0).all()
+    # features and ranges handed over separately: the same arithmetic on the same values
+    split = rasterize_to_points(means2d, conics, d["lidar_features"].contiguous(), opac, pix_vels, dcomp,
+                                d["raster_pts"], W, H, tw, th, offs, flat, asum, 0.3, backgrounds=bg,
+                                ranges=depths)
+    for got, want in zip(split, (rf, ra, rsum, med)):
+        assert (got is None and want is None) or torch.equal(got, want)
 
 
 @pytest.mark.parametrize("deg", [0, 1, 2, 3, 4])
