@@ -198,10 +198,13 @@ def test_isect_camera_sizes_and_packed(n, C, W, H, ts, rmax):
 
 
 @pytest.mark.parametrize("n,tie_frac", [(1500, 0.8), (6000, 0.0), (6000, 0.5), (12000, 0.3),
-                                        (20000, 0.1), (40000, 0.0), (40000, 0.4), (3000, 1.0)])
+                                        (20000, 0.1), (40000, 0.0), (40000, 0.4), (3000, 1.0),
+                                        (60000, 0.4), (100000, 0.5), (400, 0.2)])
 def test_isect_sort_long_segments_and_depth_ties(n, tie_frac):
-    # every Gaussian covers all four tiles, so each tile's segment has n entries: exercises
-    # every segment-length class of the sort and, with many equal depths, oversized buckets
+    # every Gaussian covers all four tiles, so each tile's segment has n entries.  From 512
+    # Gaussians on, the binning cuts the segments into depth slabs (up to 16), and equal depths
+    # share a slab: the sizes and tie fractions exercise every segment-length class of the sort
+    # (the longest through 24000 and 50000 equal depths) and, with them, oversized buckets
     from splatad_amd import isect_tiles
     rng = np.random.default_rng(n + int(10 * tie_frac))
     means2d = rng.uniform(10, 22, (1, n, 2)).astype(np.float32)
@@ -246,11 +249,12 @@ def test_isect_lidar_reference_recipe_and_wrap():
     assert not (isect_offset_encode(ids, C, n_az, 16) is offs)
 
 
-def test_isect_lidar_large_nonuniform():
+@pytest.mark.parametrize("N", [100000, 300000])  # without and with depth slabs (2 per tile)
+def test_isect_lidar_large_nonuniform(N):
     from splatad_amd import isect_lidar_tiles
     from splatad_amd import workloads
     rng = np.random.default_rng(5)
-    C, N = 2, 100000
+    C = 2
     elev = workloads.lidar_beam_elevations(128)
     eb = workloads.lidar_tile_elevation_boundaries(elev, 4).numpy()
     res, min_az = 360.0 / 2048 * 64, -180.0
