@@ -191,23 +191,34 @@ def rasterization(
     beside = _Beside(means.device)  # fork: everything the colours need is enqueued
     tile_width = math.ceil(width / float(tile_size))
     tile_height = math.ceil(height / float(tile_size))
+    fused_colors = sh_degree is not None and not viewmats.requires_grad
+    depth_appended = fused_colors and render_mode in ["RGB+D", "RGB+ED"]
+
+    def fused_view_colors():
+        # one kernel for directions, masks, SH, activation and the depth channel
+        return view_dependent_colors(sh_degree, means, viewmats, colors, radii,
+                                     depths if depth_appended else None, camera_ids,
+                                     gaussian_ids, launch_context=beside)
+
+    # The colours run on a helper stream beside the intersection.  Unpacked, they are enqueued
+    # behind it: the host is far ahead of the GPU, and the kernel then meets the segment sort,
+    # whose long workgroups leave most of the GPU idle (enqueued first, it would compete with
+    # the binning chain that everything else waits for).  Packed, the host has just waited for
+    # the projection's row count and will wait again in the intersection, the GPU idles in
+    # between, and a kernel enqueued after the intersection would find the sort over: there
+    # the colours go first.
+    if fused_colors and packed:
+        colors = fused_view_colors()
     tiles_per_gauss, isect_ids, flatten_ids = isect_tiles(
         means2d, radii, depths, tile_size, tile_width, tile_height, packed=packed, n_cameras=C,
         camera_ids=camera_ids, gaussian_ids=gaussian_ids,
     )
     isect_offsets = isect_offset_encode(isect_ids, C, tile_width, tile_height)
 
-    # 3. per-(camera, Gaussian) colours.  The intersection has just enqueued its segment sort,
-    # whose long workgroups leave most of the GPU idle: the colours are computed beside it, on
-    # a helper stream.
-    depth_appended = False
-    fused_colors = sh_degree is not None and not viewmats.requires_grad
+    # 3. per-(camera, Gaussian) colours
     if fused_colors:
-        # one kernel for directions, masks, SH, activation and the depth channel
-        depth_appended = render_mode in ["RGB+D", "RGB+ED"]
-        colors = view_dependent_colors(sh_degree, means, viewmats, colors, radii,
-                                       depths if depth_appended else None, camera_ids,
-                                       gaussian_ids, launch_context=beside)
+        if not packed:
+            colors = fused_view_colors()
         beside.join(colors)
     elif sh_degree is None:
         if packed:
