@@ -89,20 +89,6 @@ class _Beside:
                     t.record_stream(self.main)
 
 
-class _AppendChannel(torch.autograd.Function):
-    """torch.cat([features, extra[..., None]], -1) with the copy enqueued inside `beside`;
-    the autograd node, and with it the backward pass, stays on the caller's stream."""
-
-    @staticmethod
-    def forward(ctx, beside, features, extra):
-        with beside:
-            return torch.cat([features, extra[..., None]], dim=-1)
-
-    @staticmethod
-    def backward(ctx, v_out):
-        return None, v_out[..., :-1], v_out[..., -1]
-
-
 def rasterization(
     means: Tensor,  # [N, 3]
     quats: Tensor,  # [N, 4]
@@ -257,18 +243,10 @@ def rasterization(
             flatten_ids, rolling_shutter_time, backgrounds=bgs, packed=packed, absgrad=absgrad,
         )
 
-    if colors.shape[-1] > channel_chunk:
-        n_chunks = (colors.shape[-1] + channel_chunk - 1) // channel_chunk
-        chunks, chunk_alphas = [], []
-        for i in range(n_chunks):
-            sl = slice(i * channel_chunk, (i + 1) * channel_chunk)
-            rc, ra = composite(colors[..., sl], backgrounds[..., sl] if backgrounds is not None else None)
-            chunks.append(rc)
-            chunk_alphas.append(ra)
-        render_colors = torch.cat(chunks, dim=-1)
-        render_alphas = chunk_alphas[0]
-    else:
-        render_colors, render_alphas = composite(colors, backgrounds)
+    # The reference composites channel_chunk channels per call (rendering.py:362-391), copying
+    # a slice of the colours for each; the kernel here takes all channels in one call (in
+    # passes of 32 over the same lists), which renders the same images without the copies.
+    render_colors, render_alphas = composite(colors, backgrounds)
 
     if render_mode in ["ED", "RGB+ED"]:
         render_colors = torch.cat(
@@ -396,63 +374,40 @@ def lidar_rasterization(
     n_elevation_tiles = math.ceil(n_elevation_channels / tile_height)
     tile_azimuth_resolution = azimuth_resolution * tile_width
     n_azimuth_tiles = math.ceil((max_azimuth - min_azimuth) / tile_azimuth_resolution)
-    # Features to composite.  Chunks carry channel_chunk-1 features plus the range; the chunk
-    # count is the reference's (rendering.py:735): features beyond n_chunks*(channel_chunk-1)
-    # are not rendered, e.g. D=63 with channel_chunk=32.  The reference appends the range to
-    # every chunk (rendering.py:746, :779); here a single chunk hands the compositing kernels
-    # features and ranges as they are, and only the slices of a chunked call are copied
-    # together with the range, on a helper stream beside the segment sort.
-    if (D + 1) > channel_chunk:
-        n_chunks = (D + channel_chunk) // channel_chunk
-        chunks = [lidar_features[..., i * (channel_chunk - 1) : (i + 1) * (channel_chunk - 1)]
-                  for i in range(n_chunks)]
-    elif D == 0:
-        chunks = [lidar_features]  # the range alone: nothing to spare
-    else:
-        chunks = None
-    beside = _Beside(means.device)  # fork: features and ranges are enqueued
+    # Features to composite.  The reference composites chunks of channel_chunk-1 features plus
+    # the range, each a concatenated copy (rendering.py:733-771), because its kernels take 32
+    # channels at most; the kernels here take any number of channels in one call (in passes
+    # of 32 over the same lists) and read features and ranges where they are, so one call
+    # renders what the reference's loop renders: the features its chunks cover -- those beyond
+    # n_chunks*(channel_chunk-1) are not rendered, e.g. D=63 with channel_chunk=32 -- then the
+    # range, and one median column per chunk (the chunks' medians are equal: they depend on
+    # the opacities alone).
+    n_chunks = (D + channel_chunk) // channel_chunk if (D + 1) > channel_chunk else 1
+    n_feats = min(D, n_chunks * (channel_chunk - 1)) if n_chunks > 1 else D
     tiles_per_gauss, isect_ids, flatten_ids = isect_lidar_tiles(
         means2d, radii, depths, elev_boundaries=tile_elevation_boundaries,
         tile_azim_resolution=tile_azimuth_resolution, min_azim=min_azimuth, packed=packed,
         n_cameras=C, camera_ids=camera_ids, gaussian_ids=gaussian_ids,
     )
     isect_offsets = isect_offset_encode(isect_ids, C, n_azimuth_tiles, n_elevation_tiles)
-    if chunks is not None:
-        chunks = [_AppendChannel.apply(beside, f, depths) for f in chunks]
-        beside.join(*chunks)
 
     image_width = raster_pts.shape[-2]
     image_height = raster_pts.shape[-3]
-
-    def composite(feats, ranges=None):
-        return rasterize_to_points(
-            means2d, conics, feats, opacities, pix_vels,
-            depth_compensations, raster_pts, image_width, image_height, tile_width, tile_height,
-            isect_offsets, flatten_ids,
-            compute_alpha_sum_until_points=compute_alpha_sum_until_points,
-            compute_alpha_sum_until_points_threshold=compute_alpha_sum_until_points_threshold,
-            packed=packed, absgrad=absgrad, ranges=ranges,
-        )
-
-    if chunks is None:
-        render_lidar_features, render_alphas, alpha_sum_until_points, median_depths = composite(
-            lidar_features, depths)
-    elif len(chunks) > 1:
-        feats_out, alphas_out, sums_out, medians_out = [], [], [], []
-        for i, chunk in enumerate(chunks):
-            rf, ra, rs_, md = composite(chunk)
-            feats_out.append(rf if i == len(chunks) - 1 else rf[..., :-1])
-            alphas_out.append(ra)
-            sums_out.append(rs_)
-            medians_out.append(md)
-        render_lidar_features = torch.cat(feats_out, dim=-1)
-        median_depths = torch.cat(medians_out, dim=-1)
-        render_alphas = alphas_out[0]
-        alpha_sum_until_points = sums_out[0]
+    if n_feats > 0:
+        feats = lidar_features if n_feats == D else lidar_features[..., :n_feats]
+        ranges = depths
     else:
-        render_lidar_features, render_alphas, alpha_sum_until_points, median_depths = composite(
-            chunks[0]
-        )
+        feats, ranges = depths[..., None], None  # the range alone is a one-channel call
+    render_lidar_features, render_alphas, alpha_sum_until_points, median_depths = rasterize_to_points(
+        means2d, conics, feats, opacities, pix_vels,
+        depth_compensations, raster_pts, image_width, image_height, tile_width, tile_height,
+        isect_offsets, flatten_ids,
+        compute_alpha_sum_until_points=compute_alpha_sum_until_points,
+        compute_alpha_sum_until_points_threshold=compute_alpha_sum_until_points_threshold,
+        packed=packed, absgrad=absgrad, ranges=ranges,
+    )
+    if n_chunks > 1:
+        median_depths = median_depths.repeat(1, 1, 1, n_chunks)
 
     meta = {
         "camera_ids": camera_ids,
