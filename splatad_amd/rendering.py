@@ -165,13 +165,17 @@ def rasterization(
     )
     if packed:
         camera_ids, gaussian_ids, radii, means2d, depths, conics, compensations, pix_vels = proj
-        opacities = opacities[gaussian_ids]  # [nnz]
     else:
         radii, means2d, depths, conics, compensations, pix_vels = proj
-        opacities = opacities.expand(C, -1)  # [C, N]; a view, copied by the first operator that needs it when C > 1
         camera_ids, gaussian_ids = None, None
-    if compensations is not None:
-        opacities = opacities * compensations
+
+    def per_row_opacities():
+        # Compositing is the first to need these.  The packed gather is enqueued behind the
+        # intersection: ahead of it, it would only add host time between the two waits for
+        # counts, during which the GPU idles.
+        # [nnz], or [C, N]: a view, copied by the first operator that needs it when C > 1
+        o = opacities[gaussian_ids] if packed else opacities.expand(C, -1)
+        return o if compensations is None else o * compensations
 
     # 2. tile intersection, sort, offsets
     beside = _Beside(means.device)  # fork: everything the colours need is enqueued
@@ -200,6 +204,7 @@ def rasterization(
         camera_ids=camera_ids, gaussian_ids=gaussian_ids,
     )
     isect_offsets = isect_offset_encode(isect_ids, C, tile_width, tile_height)
+    opacities = per_row_opacities()
 
     # 3. per-(camera, Gaussian) colours
     if fused_colors:
