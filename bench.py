@@ -28,8 +28,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # 0.5 KiB per KiB, WRITE_SIZE 1.0).  Summaries: profiles/rasterize_kernels_counters_1M.txt.
 # They describe the 1M-Gaussian default only; other sizes report null.
 MEASURED_TRAFFIC_BYTES = {
-    "camera": int((12971.8 * 2.0 + 48617.7) * 1024),
-    "lidar": int((26328.2 * 2.0 + 40964.5) * 1024),
+    "camera": int((12972.4 * 2.0 + 48617.6) * 1024),
+    "lidar": int((26317.1 * 2.0 + 40989.5) * 1024),
 }
 
 
