@@ -109,6 +109,46 @@ def test_camera_render_modes_backgrounds_sh_and_determinism():
     assert sh.shape == (1, 20000, 3)
 
 
+@pytest.mark.parametrize("packed", [False, True])
+def test_surround_cameras_small_against_oracle(packed):
+    """Three yawed cameras over one set of Gaussians: every stage of the multi-camera call
+    against the oracle on the GPU's own inputs to that stage."""
+    C = 3
+    s = workloads.camera_driving(n=20000, width=320, height=180, n_cameras=C, with_velocities=True)
+    rc, ra, meta = _render(s, sh_degree=3, packed=packed, render_mode="RGB+D")
+    assert rc.shape == (C, 180, 320, 4)
+    m2, radii, depths = to_np(meta["means2d"]), to_np(meta["radii"]), to_np(meta["depths"])
+    cam_ids = to_np(meta["camera_ids"]) if packed else None
+    tw, th = meta["tile_width"], meta["tile_height"]
+    o_tpg, o_ids, o_flat = oracle.isect_tiles(m2, radii, depths, 16, tw, th, n_cameras=C, camera_ids=cam_ids)
+    np.testing.assert_array_equal(to_np(meta["tiles_per_gauss"]), o_tpg)
+    np.testing.assert_array_equal(to_np(meta["isect_ids"]), o_ids)
+    np.testing.assert_array_equal(to_np(meta["flatten_ids"]), o_flat)
+    np.testing.assert_array_equal(to_np(meta["isect_offsets"]), oracle.isect_offset_encode(o_ids, C, tw, th))
+    # colours: SH of the view directions, + 0.5, clamped, then the depth channel
+    cam2world = np.linalg.inv(s["viewmats"].numpy().astype(np.float64))
+    means = s["means"].numpy().astype(np.float64)
+    coeffs = s["colors"].numpy()
+    if packed:
+        gid = to_np(meta["gaussian_ids"])
+        dirs = means[gid] - cam2world[cam_ids, :3, 3]
+        sh = oracle.spherical_harmonics(3, dirs, coeffs[gid], None, "f64")
+    else:
+        dirs = means[None] - cam2world[:, None, :3, 3]
+        sh = oracle.spherical_harmonics(3, dirs, np.broadcast_to(coeffs[None], (C,) + coeffs.shape),
+                                        radii[..., 0] > 0, "f64")
+    cols = np.concatenate([np.maximum(sh + 0.5, 0.0), depths[..., None]], -1).astype(np.float32)
+    o_rc, o_ra, _ = oracle.rasterize_to_pixels_fwd(
+        m2, to_np(meta["conics"]), cols, to_np(meta["opacities"]), to_np(meta["pix_vels"]),
+        s["rolling_shutter_time"].numpy(), None, s["width"], s["height"], 16, to_np(meta["isect_offsets"]),
+        to_np(meta["flatten_ids"]), precision="f64")
+    # a float32 alpha or transmittance on the other side of a threshold than the float64
+    # oracle's moves a pixel: allowed on a sliver of them
+    assert_close(to_np(rc), o_rc, atol=1e-4, rtol=1e-4, frac=0.9999, name="render")
+    assert_close(to_np(ra), o_ra, atol=1e-4, frac=0.9999, name="alpha")
+    assert all(float(ra[c].max()) > 0.5 for c in range(C))  # every camera sees the scene
+
+
 def _lidar(n=20000, D=8, **kw):
     l = workloads.lidar_sweep(n=n, n_beams=32, n_azimuth=512, feature_dim=D, tile_width=64, tile_height=4,
                               with_velocities=True, **kw)
@@ -284,3 +324,44 @@ def test_full_size_lidar_sweep_properties():
     opaque = ra[..., 0] > 0.99
     rng_ch = rf[..., -1][opaque]
     assert float(rng_ch.min()) > 0.0 and float(rng_ch.max()) < 60.0
+    # the reference's chunk loop spelled out (rendering.py:733-771): concatenated chunks of 31
+    # features + range, the range kept from the last chunk only
+    from splatad_amd import fully_fused_lidar_projection, rasterize_to_points
+    dcomp = fully_fused_lidar_projection(  # the one projection output the meta does not carry
+        d["means"], None, d["quats"], d["scales"], d["velocities"], d["viewmats"], d["linear_velocity"],
+        d["angular_velocity"], d["rolling_shutter_time"], min_elevation=d["min_elevation"],
+        max_elevation=d["max_elevation"], min_azimuth=d["min_azimuth"], max_azimuth=d["max_azimuth"],
+        eps2d=d["eps2d"])[-1]
+    feats_out = []
+    for i in range(2):
+        chunk = torch.cat([d["lidar_features"][..., i * 31:(i + 1) * 31], meta["depths"][..., None]], -1)
+        out = rasterize_to_points(meta["means2d"], meta["conics"], chunk, meta["opacities"], meta["pix_vels"],
+                                  dcomp, d["raster_pts"], 2048, 128, d["tile_width"],
+                                  d["tile_height"], meta["isect_offsets"], meta["flatten_ids"], True, 0.3)
+        feats_out.append(out[0] if i == 1 else out[0][..., :-1])
+        torch.testing.assert_close(out[1], ra2, rtol=0, atol=1e-6)
+    torch.testing.assert_close(torch.cat(feats_out, -1), rf2, rtol=1e-5, atol=1e-4)
+
+
+def test_full_size_surround_rig_properties():
+    """2M Gaussians, six 1920x1080 cameras around the sensor in one call, and a lidar sweep
+    over the same number of Gaussians: each camera's image equals the image of a call with that
+    camera alone, and the lists keep their invariants with camera bits in the keys."""
+    C = 6
+    s = workloads.camera_driving(n=2_000_000, n_cameras=C)
+    d = workloads.to_device(s, DEV)
+    rc, ra, meta = _render(s, d, sh_degree=3, packed=False, render_mode="RGB+D")
+    assert rc.shape == (C, 1080, 1920, 4) and torch.isfinite(rc).all()
+    _check_isect_invariants(meta, C, meta["tile_width"] * meta["tile_height"])
+    for c in (0, 3, 5):
+        one = dict(d)
+        for k in ("viewmats", "Ks", "linear_velocity", "angular_velocity", "rolling_shutter_time"):
+            one[k] = d[k][c:c + 1].contiguous()
+        rc1, ra1, meta1 = _render(s, one, sh_degree=3, packed=False, render_mode="RGB+D")
+        assert torch.equal(rc1[0], rc[c]) and torch.equal(ra1[0], ra[c])
+        assert float(ra1.max()) > 0.5
+    del rc, ra, meta
+    l = workloads.lidar_sweep(n=2_000_000)
+    rf, la, asum, lmeta = _lidar_render(workloads.to_device(l, DEV), channel_chunk=33)
+    assert rf.shape == (1, 128, 2048, 33) and torch.isfinite(rf).all()
+    _check_isect_invariants(lmeta, 1, lmeta["tile_grid_width"] * lmeta["tile_grid_height"])
