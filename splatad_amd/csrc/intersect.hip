@@ -377,12 +377,18 @@ __device__ __forceinline__ uint32_t coarse_mask(const LaneWork &w, const CoarseG
 // any bounds whatsoever give the same output, balance is all they decide.
 constexpr uint32_t kSlabShiftMax = 4;
 constexpr uint32_t kSlabSamples = 512;
+// Slabs pay once a tile's segment outgrows the sort's short classes (beyond about 8000 entries,
+// i.e. several hundred Gaussians per tile); below that they only lengthen the binning.  Measured
+// on lidar sweeps of 0.25-4M Gaussians on 1024 tiles and camera frames of 1-4M on 8160 tiles:
+// no slabs win up to 490 Gaussians per tile, 4 win at 980, 8 at 1950, 8-16 at 3900.
+constexpr uint64_t kSlabMinPerTile = 704;
 
 // Slabs for `total` projected Gaussians on `segs` tiles, from the sizes alone.
 static uint32_t slab_shift_for(uint64_t total, uint64_t segs) {
     const uint64_t per_tile = segs ? total / segs : 0;
+    if (per_tile < kSlabMinPerTile) return 0;
     uint32_t sshift = 0;
-    while (sshift < kSlabShiftMax && (128ull << sshift) <= per_tile) ++sshift;
+    while (sshift < kSlabShiftMax && (256ull << sshift) <= per_tile) ++sshift;
     return sshift;
 }
 

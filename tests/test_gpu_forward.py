@@ -201,8 +201,8 @@ def test_isect_camera_sizes_and_packed(n, C, W, H, ts, rmax):
                                         (20000, 0.1), (40000, 0.0), (40000, 0.4), (3000, 1.0),
                                         (60000, 0.4), (100000, 0.5), (400, 0.2)])
 def test_isect_sort_long_segments_and_depth_ties(n, tie_frac):
-    # every Gaussian covers all four tiles, so each tile's segment has n entries.  From 512
-    # Gaussians on, the binning cuts the segments into depth slabs (up to 16), and equal depths
+    # every Gaussian covers all four tiles, so each tile's segment has n entries.  From 2816
+    # Gaussians on, the binning cuts the segments into depth slabs (4 to 16), and equal depths
     # share a slab: the sizes and tie fractions exercise every segment-length class of the sort
     # (the longest through 24000 and 50000 equal depths) and, with them, oversized buckets
     from splatad_amd import isect_tiles
@@ -249,7 +249,7 @@ def test_isect_lidar_reference_recipe_and_wrap():
     assert not (isect_offset_encode(ids, C, n_az, 16) is offs)
 
 
-@pytest.mark.parametrize("N", [100000, 300000])  # without and with depth slabs (2 per tile)
+@pytest.mark.parametrize("N", [100000, 750000])  # without and with depth slabs (4 per tile)
 def test_isect_lidar_large_nonuniform(N):
     from splatad_amd import isect_lidar_tiles
     from splatad_amd import workloads
