@@ -269,6 +269,45 @@ def test_isect_lidar_large_nonuniform(N):
     np.testing.assert_array_equal(to_np(flat), o[2])
 
 
+@pytest.mark.parametrize("case", range(10))
+def test_isect_random_grids_depth_distributions_and_slabs(case):
+    """Random small grids with 500-4000 Gaussians per tile (depth slabs on in most), one to three
+    sensors, and depth distributions that make slab bounds awkward: log-uniform over six decades,
+    70 % equal, two tight clusters, all equal."""
+    from splatad_amd import isect_lidar_tiles, isect_tiles
+    rng = np.random.default_rng(1000 + case)
+    lidar = case % 2 == 1
+    C = int(rng.integers(1, 4))
+    if lidar:
+        tw, th = int(rng.choice([4, 8, 16])), int(rng.integers(2, 6))
+        N = min(int(rng.integers(500, 4000)) * tw * th // C + 1, 80000)
+        eb = np.sort(rng.uniform(-30, 30, th + 1)).astype(np.float32)
+        means2d = np.stack([rng.uniform(-180, 180, (C, N)), rng.uniform(-35, 35, (C, N))], -1).astype(np.float32)
+        radii = rng.exponential(8.0, (C, N, 2)).astype(np.float32)
+    else:
+        tw, th = int(rng.integers(1, 6)), int(rng.integers(1, 5))
+        N = min(int(rng.integers(500, 4000)) * tw * th // C + 1, 60000)
+        means2d = np.stack([rng.uniform(-10, tw * 16 + 10, (C, N)),
+                            rng.uniform(-10, th * 16 + 10, (C, N))], -1).astype(np.float32)
+        radii = rng.integers(0, 40, (C, N, 2)).astype(np.int32)
+    radii[rng.random((C, N)) < 0.2] = 0
+    depths = [rng.uniform(0.5, 80, (C, N)),
+              np.exp(rng.uniform(-6, 8, (C, N))),
+              np.where(rng.random((C, N)) < 0.7, 3.25, rng.uniform(1, 100, (C, N))),
+              np.where(rng.random((C, N)) < 0.5, rng.normal(5, 0.01, (C, N)), rng.normal(50, 0.01, (C, N))).clip(0.1),
+              np.full((C, N), 7.0)][case // 2].astype(np.float32)
+    if lidar:
+        res = 360.0 / tw
+        got = isect_lidar_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), to_dev(eb), res, -180.0)
+        want = oracle.isect_lidar_tiles(means2d, radii, depths, eb, res, -180.0)
+    else:
+        got = isect_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), 16, tw, th)
+        want = oracle.isect_tiles(means2d, radii, depths, 16, tw, th)
+    assert want[1].shape[0] > 0
+    for g, w in zip(got, want):
+        np.testing.assert_array_equal(to_np(g), w)
+
+
 def _projected_scene(C, N, W, H, D, seed, rs=(0.02, 0.0)):
     from splatad_amd import fully_fused_projection
     rng, means, quats, scales, vel = _gaussians(N, seed, log_scale=-2.6)
