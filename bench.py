@@ -180,29 +180,38 @@ def bench_lidar(args):
             s["min_elevation"], s["max_elevation"], s["min_azimuth"], s["max_azimuth"],
             s["linear_velocity"], s["angular_velocity"], s["rolling_shutter_time"], s["eps2d"],
             s["near_plane"], s["far_plane"], 0.0, False)
-        feats = torch.cat([s["lidar_features"], meta["depths"][..., None]], -1).contiguous()
-        D = feats.shape[-1]
+        # the compositing kernel as lidar_rasterization() calls it: features and ranges apart
+        feats, ranges = s["lidar_features"], meta["depths"]
+        D = feats.shape[-1] + 1
 
-        def raster():
+        def raster(**kw):
             return _C.rasterize_to_points_fwd(
                 meta["means2d"], meta["conics"], feats, meta["opacities"], meta["pix_vels"], proj[6],
                 None, s["raster_pts"], W, H, s["tile_width"], s["tile_height"], True, 0.2,
-                meta["isect_offsets"], meta["flatten_ids"], D - 1)
+                meta["isect_offsets"], meta["flatten_ids"], D - 1, range_channel=ranges, **kw)
 
         k_ms = time_kernel(raster, iters=max(5, args.steps))
         n_isects = int(meta["flatten_ids"].shape[0])
         batches = torch.zeros_like(meta["isect_offsets"])
-        _C.rasterize_to_points_fwd(
-            meta["means2d"], meta["conics"], feats, meta["opacities"], meta["pix_vels"], proj[6],
-            None, s["raster_pts"], W, H, s["tile_width"], s["tile_height"], True, 0.2,
-            meta["isect_offsets"], meta["flatten_ids"], D - 1, tile_batches=batches)
+        raster(tile_batches=batches)
         i_need, _ = staged_isects(batches, meta["isect_offsets"], n_isects)
         P, T = C * H * W, meta["isect_offsets"].numel()
         # staged per list entry: id, mean, angular velocity, conic, opacity (40 bytes); the features
         # of the Gaussians a wavefront composites are read on demand and not counted here
         alg_bytes = i_need * 40 + P * (4 * D + 32) + T * 4
+        stages = {}
+        stages["projection_ms"] = time_kernel(lambda: _C.fully_fused_lidar_projection_fwd(
+            s["means"], None, s["quats"], s["scales"], s["velocities"], s["viewmats"],
+            s["min_elevation"], s["max_elevation"], s["min_azimuth"], s["max_azimuth"],
+            s["linear_velocity"], s["angular_velocity"], s["rolling_shutter_time"], s["eps2d"],
+            s["near_plane"], s["far_plane"], 0.0, False), 5)
+        stages["isect_sort_ms"] = time_kernel(lambda: _C.isect_lidar_tiles(
+            meta["means2d"], meta["radii"], meta["depths"], None, None, C,
+            s["tile_elevation_boundaries"], s["azimuth_resolution"] * s["tile_width"], s["min_azimuth"],
+            True, True), 5)
+        stages["rasterize_ms"] = k_ms
     return dict(sec=sec, sec_chunk32=sec_chunk32, points=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
-                n_isects=n_isects, i_need=i_need, channels=D)
+                n_isects=n_isects, i_need=i_need, channels=D, stages=stages)
 
 
 def bench_backward(args):
@@ -365,6 +374,7 @@ def main():
             "workload": "128x2048 lidar sweep, %d Gaussians, 32 features + range, tile 64x4, "
                         "channel_chunk=33 (BASELINE configs[2])" % args.n,
             "n_isects": lid["n_isects"], "n_isects_consumed": lid["i_need"],
+            "stage_ms": {k: round(v, 4) for k, v in lid["stages"].items()},
             "roofline": {"kernel": "rasterize_to_points_fwd_kernel<%d, %s>" % (lid["channels"], "true" if lid["channels"] in (32, 33) else "false"),
                          "bound": "hbm", "achieved": l_ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": l_ach / HBM_PEAK_GBS,
