@@ -187,11 +187,15 @@ def isect_tiles(means2d, radii, depths, tile_size, tile_width, tile_height, sort
 
 
 def isect_lidar_tiles(means2d, radii, depths, elev_boundaries, tile_azim_resolution, min_azim,
-                      sort=True, n_cameras=None, camera_ids=None):
-    """Restates ``isect_lidar_tiles`` (rasterization.cu:287-529)."""
+                      sort=True, n_cameras=None, camera_ids=None, n_tiles_azim=None):
+    """Restates ``isect_lidar_tiles`` (rasterization.cu:287-529).
+
+    ``n_tiles_azim`` defaults to the reference's full turn of tile columns; a caller of the
+    kernel-level interface may pass fewer (a sector)."""
     import math
-    # rasterization.cu:435-436: float32 division, ceil
-    n_tiles_azim = int(math.ceil(float(np.float32(360.0) / np.float32(tile_azim_resolution))))
+    if n_tiles_azim is None:
+        # rasterization.cu:435-436: float32 division, ceil
+        n_tiles_azim = int(math.ceil(float(np.float32(360.0) / np.float32(tile_azim_resolution))))
     n_tiles_elev = int(np.asarray(elev_boundaries).shape[0] - 1)
     return _isect(1, means2d, radii, depths, 0, n_tiles_azim, n_tiles_elev, elev_boundaries,
                   tile_azim_resolution, min_azim, sort, n_cameras, camera_ids)

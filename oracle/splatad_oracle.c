@@ -536,7 +536,14 @@ long oracle_isect_count(int lidar, long total, const float *means2d, const void 
                 int32_t rect[4];
                 lidar_tile_rect(means2d, r, idx, elev_boundaries, tile_azim_res, min_azim, tile_w,
                                 tile_h, rect);
-                cnt = (rect[3] - rect[1]) * (rect[2] - rect[0]);
+                /* An empty rectangle counts as zero tiles.  With tile columns that span
+                 * less than a full turn, a Gaussian that straddles min_azim gets
+                 * rect[2] < rect[0]; the reference's product goes negative there
+                 * (rasterization.cu:359-361), its cumulative sum and every list entry
+                 * behind that Gaussian are then corrupt.  The emission loop below emits
+                 * nothing for such a rectangle, so zero is the consistent count. */
+                int32_t h = rect[3] - rect[1], w = rect[2] - rect[0];
+                cnt = (h > 0 ? h : 0) * (w > 0 ? w : 0);
             }
         }
         tiles_per_gauss[idx] = cnt;
@@ -581,8 +588,10 @@ void oracle_isect_emit(int lidar, long total, long N, const int64_t *camera_ids,
             for (int32_t i = rect[1]; i < rect[3]; ++i)
                 for (int32_t j = rect[0]; j < rect[2]; ++j) {
                     /* mathematical modulo: identical to (j + n) % n of the reference
-                     * (rasterization.cu:384) for j >= -n; azimuth extents below -360
-                     * degrees (j < -n) would make that expression negative */
+                     * (rasterization.cu:384) for j >= -n.  The reference's sum is
+                     * unsigned, so for azimuth extents below -360 degrees (j < -n) it
+                     * wraps modulo 2^32 first: the same column as here when n is a power
+                     * of two, a column shifted by 2^32 mod n otherwise. */
                     int32_t wj = ((j % (int32_t)tile_w) + (int32_t)tile_w) % (int32_t)tile_w;
                     int64_t tile_id = (int64_t)i * tile_w + wj;
                     isect_ids[cur] = cid_enc | (tile_id << 32) | depth_enc;

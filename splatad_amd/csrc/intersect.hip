@@ -125,8 +125,10 @@ template <bool LIDAR>
 __device__ __forceinline__ uint32_t tile_index(const TileGrid &g, int32_t y, int32_t x) {
     if (LIDAR) {
         // Mathematical modulo.  For x >= -tile_w this equals (x + tile_w) % tile_w of the
-        // reference (rasterization.cu:384); an azimuth extent reaching below -360 degrees
-        // gives x < -tile_w, where that expression would go negative.
+        // reference (rasterization.cu:384).  That sum is unsigned there, so for x < -tile_w (an
+        // azimuth extent reaching below -360 degrees) it wraps modulo 2^32 first: the same
+        // column as here when tile_w is a power of two, a column shifted by 2^32 mod tile_w
+        // otherwise.
         const int32_t n = (int32_t)g.tile_w;
         x = ((x % n) + n) % n;
     }
@@ -164,8 +166,12 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
         for (int k = 0; k < 4; ++k) {
             int32_t x0, y0, x1, y1;
             cnt[k] = 0;
+            // An empty rectangle counts as zero tiles, as in make_work(): a lidar whose tile
+            // columns span less than a full turn gives x1 < x0 for a Gaussian that straddles
+            // min_azim (the reference's product goes negative there, rasterization.cu:359-361,
+            // and its lists are corrupt from that Gaussian on).
             if (i0 + k * stride < total && tile_rect_of<LIDAR>(g, mu[k], rad[k], x0, y0, x1, y1))
-                cnt[k] = (y1 - y0) * (x1 - x0);
+                cnt[k] = max(y1 - y0, 0) * max(x1 - x0, 0);
         }
 #pragma unroll
         for (int k = 0; k < 4; ++k) {

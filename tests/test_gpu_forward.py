@@ -249,6 +249,32 @@ def test_isect_lidar_reference_recipe_and_wrap():
     assert not (isect_offset_encode(ids, C, n_az, 16) is offs)
 
 
+def test_isect_lidar_sector_of_tile_columns():
+    """Tile columns that span 120 degrees only, reachable through the C entry points alone (the
+    operator always passes a full turn of columns): Gaussians that straddle min_azim count zero
+    tiles in the counting call and in the binning alike, so the lists have exactly n_isects
+    entries and equal the oracle's."""
+    from splatad_amd.hip import _backend
+    rng = np.random.default_rng(11)
+    C, N, n_az, res, min_az = 2, 40000, 16, 7.5, -60.0
+    eb = np.sort(rng.uniform(-20, 20, 9)).astype(np.float32)
+    means2d = np.stack([rng.uniform(-75, 75, (C, N)), rng.uniform(-25, 25, (C, N))], -1).astype(np.float32)
+    radii = rng.exponential(3.0, (C, N, 2)).astype(np.float32)
+    radii[rng.random((C, N)) < 0.2] = 0
+    depths = rng.uniform(0.5, 80, (C, N)).astype(np.float32)
+    straddle = (means2d[..., 0] - min_az - radii[..., 0] < 0) & (radii[..., 0] > 0)
+    assert straddle.sum() > 100
+    eb_dev = to_dev(eb)
+    for sort in (True, False):
+        got = _backend._C._isect(True, to_dev(means2d), to_dev(radii), to_dev(depths), None, None, C,
+                                 (_backend._p(eb_dev), _backend._f32(res), _backend._f32(min_az)),
+                                 n_az, 8, sort)
+        want = oracle.isect_lidar_tiles(means2d, radii, depths, eb, res, min_az, sort=sort, n_tiles_azim=n_az)
+        assert (want[0] >= 0).all() and (want[0][straddle] == 0).all() and want[1].shape[0] > 1000
+        for g, w in zip(got, want):
+            np.testing.assert_array_equal(to_np(g), w)
+
+
 @pytest.mark.parametrize("N", [100000, 750000])  # without and with depth slabs (4 per tile)
 def test_isect_lidar_large_nonuniform(N):
     from splatad_amd import isect_lidar_tiles

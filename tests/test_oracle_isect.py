@@ -222,3 +222,34 @@ def test_lidar_isect_extent_beyond_a_full_turn():
     # consecutive emissions walk the columns cyclically
     cols = tile[: tpg[0, 0] // 2] % 8
     assert ((np.diff(cols) % 8) == 1).all()
+
+
+def test_lidar_isect_sector_of_tile_columns():
+    # Tile columns that span 120 degrees only (the operator itself always uses a full turn,
+    # rasterization.cu:435-436; a sector can only come through the kernel-level interface).
+    # A Gaussian that straddles min_azim gets an empty column range and counts zero tiles
+    # (the reference's count goes negative there); everything else is the brute-force
+    # overlap, and the counts add up to the list length.
+    res, n_az, min_az = 7.5, 16, -60.0
+    eb = np.array([-20.0, -5.0, 0.0, 5.0, 20.0], np.float32)
+    means2d = np.array([[[-60.2, 1.0],      # straddles min_azim: nothing
+                         [-50.0, 1.0],      # inside, two columns
+                         [0.0, -7.0],       # inside, crosses an elevation boundary
+                         [59.0, 2.0],       # reaches the sector's upper edge
+                         [30.0, 30.0]]],    # above every boundary
+                       np.float32)
+    radii = np.array([[[1.0, 1.0], [4.0, 1.0], [1.0, 3.0], [2.0, 1.0], [1.0, 1.0]]], np.float32)
+    depths = np.array([[5.0, 4.0, 3.0, 2.0, 1.0]], np.float32)
+    tpg, ids, flat = oracle.isect_lidar_tiles(means2d, radii, depths, eb, res, min_az, sort=False,
+                                              n_tiles_azim=n_az)
+    assert (tpg >= 0).all() and tpg.sum() == ids.shape[0] == flat.shape[0]
+    assert tpg[0, 0] == 0 and tpg[0, 4] == 0
+    for g in (1, 2, 3):
+        a = means2d[0, g, 0] - min_az
+        lo, hi = a - radii[0, g, 0], a + radii[0, g, 0]
+        cols = list(range(int(math.floor(lo / res)), int(math.ceil(hi / res))))
+        elo, ehi = means2d[0, g, 1] - radii[0, g, 1], means2d[0, g, 1] + radii[0, g, 1]
+        rows = [e for e in range(4) if eb[e] < ehi and eb[e + 1] >= elo]
+        assert tpg[0, g] == len(rows) * len(cols), g
+        _, tile, _ = _decode(ids[flat == g], n_az * 4, 1)
+        assert sorted(tile.tolist()) == sorted(e * n_az + (k % n_az) for e in rows for k in cols)
