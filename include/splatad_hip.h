@@ -265,6 +265,22 @@ int splatad_rasterize_to_pixels_fwd(uint32_t C, int64_t n_isects, uint32_t chann
                                     int32_t *last_ids, int32_t *tile_batches,
                                     splatad_stream_t stream);
 
+/* Diagnostic without a counterpart in the reference: lane utilisation of the compositing loop
+ * of splatad_rasterize_to_pixels_fwd on the same inputs (nothing is rendered).  Adds to eight
+ * counters in stats (zero them first): [0] (wavefront, Gaussian) iterations of the inner loop,
+ * [1] lanes that composited their Gaussian, summed over the iterations, [2] lanes still alive,
+ * [3] iterations in which no lane composited, [4] list entries tested against a wavefront's
+ * footprint, [5] entries that passed the test, [6] wavefronts, [7] lanes with alpha >= 1/255. */
+int splatad_rasterize_to_pixels_lane_stats(uint32_t C, int64_t n_isects, const float *means2d,
+                                           const float *conics, const float *opacities,
+                                           const float *pix_vels,
+                                           const float *rolling_shutter_time,
+                                           uint32_t image_width, uint32_t image_height,
+                                           uint32_t tile_size, uint32_t tile_width,
+                                           uint32_t tile_height, const int32_t *tile_offsets,
+                                           const int32_t *flatten_ids, unsigned long long *stats,
+                                           splatad_stream_t stream);
+
 /* rasterize_to_pixels_bwd_tensor, rasterization.cu:3091-3726 (kernel
  * :2833-3089).  Gradient outputs must be zero-filled; v_means2d_abs may be NULL.
  *

@@ -288,6 +288,31 @@ def compute_relocation(opacities, scales, ratios, binoms):
 # ---------------------------------------------------------------------------
 # rasterization
 # ---------------------------------------------------------------------------
+class nudged_thresholds:
+    """Context manager: the fused compositing functions take their discontinuous decisions
+    at alpha_scale / 255, t_scale * 1e-4, median_scale * 0.5 and range - threshold +
+    asum_shift instead of the reference's values.  With it a parity test finds the pixels
+    whose value depends on a decision within a few rounding errors of its threshold."""
+
+    def __init__(self, precision="f64", alpha_scale=1.0, t_scale=1.0, median_scale=1.0,
+                 asum_shift=0.0):
+        self.precision = precision
+        self.args = (alpha_scale, t_scale, median_scale, asum_shift)
+
+    def _set(self, a, t, m, s):
+        fn = getattr(_lib(self.precision), f"oracle_{self.precision}_set_thresholds")
+        fn.restype = None
+        fn(ctypes.c_double(a), ctypes.c_double(t), ctypes.c_double(m), ctypes.c_double(s))
+
+    def __enter__(self):
+        self._set(*self.args)
+        return self
+
+    def __exit__(self, *exc):
+        self._set(1.0, 1.0, 1.0, 0.0)
+        return False
+
+
 def rasterize_to_pixels_fwd(means2d, conics, colors, opacities, pix_vels, rolling_shutter_time,
                             backgrounds, width, height, tile_size, isect_offsets, flatten_ids,
                             precision="f32"):

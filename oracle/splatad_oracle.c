@@ -761,6 +761,29 @@ void oracle_compute_relocation(long N, const float *opacities, const float *scal
 
 #endif /* !ORACLE_F64 */
 
+/* The discontinuous decisions of the compositing rule.  The values are the reference's
+ * (rasterization.cu:1476-1488, 2186-2197): a Gaussian is skipped below alpha = 1/255, a
+ * pixel stops when its transmittance would fall to 1e-4 or below, the median depth is
+ * taken where the transmittance crosses 0.5, alpha is summed while the Gaussian lies
+ * in front of range - threshold.  A float32 implementation whose alpha or transmittance
+ * differs from this file's in the last bits takes the other branch for inputs within
+ * rounding distance of a threshold.  Parity tests find exactly those pixels by rendering
+ * again with the thresholds moved by a few rounding errors (set_thresholds); with the
+ * defaults below the functions restate the reference. */
+static real g_alpha_min = RC(1) / RC(255);
+static real g_T_min = RC(1e-4);
+static real g_median_T = RC(0.5);
+static real g_asum_shift = RC(0);
+
+void NAME(set_thresholds)(double alpha_scale, double t_scale, double median_scale,
+                          double asum_shift) {
+    g_alpha_min = (real)(alpha_scale * (1.0 / 255.0));
+    if (alpha_scale == 1.0) g_alpha_min = RC(1) / RC(255);
+    g_T_min = t_scale == 1.0 ? RC(1e-4) : (real)(t_scale * 1e-4);
+    g_median_T = median_scale == 1.0 ? RC(0.5) : (real)(median_scale * 0.5);
+    g_asum_shift = (real)asum_shift;
+}
+
 /* ------------------------------------------------------------------ */
 /* R1: rasterize_to_pixels forward (rasterization.cu:1360-1518)          */
 /* One scalar loop per pixel over its tile's sorted list.                */
@@ -796,9 +819,9 @@ void NAME(rasterize_to_pixels_fwd)(int C, long n_isects, int D, const float *mea
             real ca = conics[g * 3], cb = conics[g * 3 + 1], cc = conics[g * 3 + 2];
             real sigma = RC(0.5) * (ca * dx * dx + cc * dy * dy) + cb * dx * dy;
             real alpha = R_FMIN(RC(0.999), RC(opacities[g]) * R_EXP(-sigma));
-            if (sigma < 0 || alpha < RC(1) / RC(255)) continue;
+            if (sigma < 0 || alpha < g_alpha_min) continue;
             real next_T = T * (RC(1) - alpha);
-            if (next_T <= RC(1e-4)) break; /* exclusive: :1485-1488 */
+            if (next_T <= g_T_min) break; /* exclusive: :1485-1488 */
             real vis = alpha * T;
             const float *c = colors + g * D;
             for (int k = 0; k < D; ++k) out[k] += RC(c[k]) * vis;
@@ -860,16 +883,16 @@ void NAME(rasterize_to_points_fwd)(int C, long n_isects, int D, const float *mea
             real ca = conics[g * 3], cb = conics[g * 3 + 1], cc = conics[g * 3 + 2];
             real sigma = RC(0.5) * (ca * dx * dx + cc * dy * dy) + cb * dx * dy;
             real alpha = R_FMIN(RC(0.999), RC(opacities[g]) * R_EXP(-sigma));
-            if (sigma < 0 || alpha < RC(1) / RC(255)) continue;
+            if (sigma < 0 || alpha < g_alpha_min) continue;
             real next_T = T * (RC(1) - alpha);
-            if (next_T <= RC(1e-4)) break;
+            if (next_T <= g_T_min) break;
             real vis = alpha * T;
             const float *c = colors + g * D;
             for (int k = 0; k < D; ++k) out[k] += RC(c[k]) * vis;
             real extra = RC(depth_comps[g * 2]) * dx + RC(depth_comps[g * 2 + 1]) * dy + vz * roll;
             out[depth_idx] += extra * vis; /* :2184-2185 */
-            if (T > RC(0.5) && next_T <= RC(0.5)) median_depths[pix] = RC(c[depth_idx]) + extra;
-            if (compute_alpha_sum && RC(c[depth_idx]) < pz - RC(alpha_sum_threshold)) asum += alpha;
+            if (T > g_median_T && next_T <= g_median_T) median_depths[pix] = RC(c[depth_idx]) + extra;
+            if (compute_alpha_sum && RC(c[depth_idx]) < pz - RC(alpha_sum_threshold) + g_asum_shift) asum += alpha;
             cur_idx = s;
             T = next_T;
         }

@@ -164,8 +164,9 @@ def _angle_difference(a, b):
 
 
 def rasterize_to_pixels(means2d, conics, colors, opacities, pix_vels, rs_time, backgrounds, width,
-                        height, tile_size, offsets, flatten_ids):
-    """Dense per-tile compositing; differentiable w.r.t. the float inputs.  [C,N,...] layout."""
+                        height, tile_size, offsets, flatten_ids, tiles=None):
+    """Dense per-tile compositing; differentiable w.r.t. the float inputs.  [C,N,...] layout.
+    With `tiles` (flat (camera, tile) indices) only those tiles are rendered, the rest stays 0."""
     C, th, tw = offsets.shape
     D = colors.shape[-1]
     n_isects = flatten_ids.shape[0]
@@ -181,7 +182,7 @@ def rasterize_to_pixels(means2d, conics, colors, opacities, pix_vels, rs_time, b
                 t = (c * th + ty) * tw + tx
                 i0, j0 = ty * tile_size, tx * tile_size
                 i1, j1 = min(i0 + tile_size, height), min(j0 + tile_size, width)
-                if i1 <= i0 or j1 <= j0:
+                if i1 <= i0 or j1 <= j0 or (tiles is not None and t not in tiles):
                     continue
                 ii, jj = torch.meshgrid(torch.arange(i0, i1), torch.arange(j0, j1), indexing="ij")
                 px = (jj.reshape(-1, 1) + 0.5).to(means2d.dtype)
@@ -209,8 +210,9 @@ def rasterize_to_pixels(means2d, conics, colors, opacities, pix_vels, rs_time, b
 
 def rasterize_to_points(means2d, conics, colors, opacities, pix_vels, depth_comps, backgrounds,
                         raster_pts, tile_width, tile_height, compute_alpha_sum, threshold, offsets,
-                        flatten_ids, depth_idx):
-    """Dense per-tile compositing onto lidar points. Returns (colors, alphas, alpha_sum, median)."""
+                        flatten_ids, depth_idx, tiles=None):
+    """Dense per-tile compositing onto lidar points. Returns (colors, alphas, alpha_sum, median).
+    With `tiles` (flat (sensor, tile) indices) only those tiles are rendered."""
     C, gh, gw = offsets.shape
     H, W = raster_pts.shape[1:3]
     D = colors.shape[-1]
@@ -230,7 +232,7 @@ def rasterize_to_points(means2d, conics, colors, opacities, pix_vels, depth_comp
                 t = (c * gh + ty) * gw + tx
                 i0, j0 = ty * tile_height, tx * tile_width
                 i1, j1 = min(i0 + tile_height, H), min(j0 + tile_width, W)
-                if i1 <= i0 or j1 <= j0:
+                if i1 <= i0 or j1 <= j0 or (tiles is not None and t not in tiles):
                     continue
                 P = raster_pts[c, i0:i1, j0:j1].reshape(-1, 4)
                 active = (P[:, 2] > 0).to(dt)

@@ -1193,13 +1193,11 @@ static inline dim3 grid_for(uint64_t n) {
 }
 
 // Per device, created at first use and kept for the life of the process: the helper streams
-// (default priority) and events of the segment sort, and the pinned host slot through which
-// the number of intersections reaches the host.  `guard` serialises the
-// enqueueing of sequences that share them.
+// (default priority) and events of the segment sort.  `guard` serialises the enqueueing of the
+// fork / join sequences that share them (enqueueing only: no call waits for the GPU under it).
 struct IsectDevice {
     hipStream_t aux[2];
     hipEvent_t fork, join[2];
-    HostWord n; // carries the number of intersections to the host
     std::mutex guard;
 };
 
@@ -1215,7 +1213,6 @@ static int isect_device(IsectDevice **out) {
         for (hipStream_t &a : s->aux) SPLATAD_CHECK_HIP(hipStreamCreateWithFlags(&a, hipStreamNonBlocking));
         SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->fork, hipEventDisableTiming));
         for (hipEvent_t &e : s->join) SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-        if (int rc = host_word_create(&s->n)) return rc;
         table[dev] = s;
     }
     *out = table[dev];
@@ -1280,10 +1277,9 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     IsectWorkspace w;
     carve_isect(workspace, total, pl.segs, sort ? pl.cslots : 0, &w);
     if (int rc = host_word_refuse_capture(stream, "isect")) return rc;
-    IsectDevice *dv = nullptr;
-    if (int rc = isect_device(&dv)) return rc;
-    std::lock_guard<std::mutex> lock(dv->guard);
-    *(volatile unsigned long long *)dv->n.host = kHostWordPending;
+    // the number of intersections reaches the host through a leased pinned word
+    HostWordLease lease(stream);
+    if (int rc = host_word_acquire(&lease.word)) return rc;
     // one fill clears the counters and, for the binning, everything up to the end of the tile
     // counters (the two scan totals between them are written before they are read)
     const uint64_t clear_words = sort ? (uint64_t)((char *)(w.zeroed + w.n_zeroed) - (char *)w.n_isects) / 4
@@ -1293,7 +1289,7 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     dim3 count_grid = grid_for(total);
     if (count_grid.x > 1024) count_grid.x = 1024;
     hipLaunchKernelGGL(isect_count_kernel<LIDAR>, count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
-                       total, means2d, radii, tiles_per_gauss, w.n_isects, dv->n.device);
+                       total, means2d, radii, tiles_per_gauss, w.n_isects, lease.word.device);
     SPLATAD_LAUNCH_CHECK();
     // work for the GPU while the host learns the count and sizes the lists
     if (sort) {
@@ -1307,7 +1303,7 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
             return rc;
     }
     unsigned long long n = 0;
-    if (int rc = host_word_wait(&dv->n, stream, "isect", &n)) return rc;
+    if (int rc = host_word_wait(&lease, "isect", &n)) return rc;
     SPLATAD_REQUIRE(n < (1ull << 31), "isect: %llu intersections exceed the int32 offset range", n);
     *n_isects_host = (int64_t)n;
     return 0;
@@ -1395,24 +1391,34 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     std::lock_guard<std::mutex> fork_lock(ss->guard);
     SPLATAD_CHECK_HIP(hipEventRecord(ss->fork, stream));
     for (hipStream_t aux : ss->aux) SPLATAD_CHECK_HIP(hipStreamWaitEvent(aux, ss->fork, 0));
+    // After the fork the helper streams are joined whatever happens: work already queued on
+    // them reads and writes the caller's buffers, so the caller's stream must not run past it.
+    auto enqueue_sorts = [&]() -> int {
+        int e;
 #define SPLATAD_SORT_CLASS(cls, ER, IN_LDS, threads, hi, wgs, on)                                \
-    if ((rc = launch_segment_sort<ER, IN_LDS>(cls, threads, hi, wgs, nseg, n_tiles, sshift, tile_n_bits, \
-                                              n_isects, w.seg_counts, w.seg_lists, w.tile_starts, \
-                                              w.pairs, isect_ids, flatten_ids, on)) != 0)         \
-        return rc;
-    // the upper classes go first, on the caller's stream, which does not wait for the fork
-    if ((rc = launch_big_segment_sort(256u, nseg, n_tiles, sshift, tile_n_bits, n_isects, w.seg_counts, w.seg_lists,
-                                      w.tile_starts, w.pairs, isect_ids, flatten_ids, stream)) != 0)
-        return rc;
-    SPLATAD_SORT_CLASS(2, 8, true, 512, 4096u, 1024u, ss->aux[0])
-    SPLATAD_SORT_CLASS(3, 8, true, 1024, 8192u, 512u, ss->aux[1])
-    SPLATAD_SORT_CLASS(1, 8, true, 256, 2048u, 2048u, stream)
-    SPLATAD_SORT_CLASS(0, 4, true, 128, 512u, 4096u, stream)
+        if ((e = launch_segment_sort<ER, IN_LDS>(cls, threads, hi, wgs, nseg, n_tiles, sshift, tile_n_bits, \
+                                                 n_isects, w.seg_counts, w.seg_lists, w.tile_starts, \
+                                                 w.pairs, isect_ids, flatten_ids, on)) != 0)      \
+            return e;
+        // the upper classes go first, on the caller's stream, which does not wait for the fork
+        if ((e = launch_big_segment_sort(256u, nseg, n_tiles, sshift, tile_n_bits, n_isects, w.seg_counts,
+                                         w.seg_lists, w.tile_starts, w.pairs, isect_ids, flatten_ids,
+                                         stream)) != 0)
+            return e;
+        SPLATAD_SORT_CLASS(2, 8, true, 512, 4096u, 1024u, ss->aux[0])
+        SPLATAD_SORT_CLASS(3, 8, true, 1024, 8192u, 512u, ss->aux[1])
+        SPLATAD_SORT_CLASS(1, 8, true, 256, 2048u, 2048u, stream)
+        SPLATAD_SORT_CLASS(0, 4, true, 128, 512u, 4096u, stream)
 #undef SPLATAD_SORT_CLASS
+        return 0;
+    };
+    rc = enqueue_sorts();
     for (int k = 0; k < 2; ++k) {
-        SPLATAD_CHECK_HIP(hipEventRecord(ss->join[k], ss->aux[k]));
-        SPLATAD_CHECK_HIP(hipStreamWaitEvent(stream, ss->join[k], 0));
+        const hipError_t r = hipEventRecord(ss->join[k], ss->aux[k]);
+        const hipError_t q = r == hipSuccess ? hipStreamWaitEvent(stream, ss->join[k], 0) : r;
+        if (q != hipSuccess && rc == 0) SPLATAD_CHECK_HIP(q);
     }
+    if (rc) return rc;
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }

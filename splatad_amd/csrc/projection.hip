@@ -412,26 +412,6 @@ extern "C" int splatad_lidar_projection_fwd(uint32_t C, uint32_t N, const float 
     return 0;
 }
 
-// The pinned word through which the number of kept (camera, Gaussian) pairs reaches the host,
-// one per device, with the mutex that serialises its users.
-static int packed_host_word(HostWord **word, std::mutex **guard) {
-    static std::mutex table_guard;
-    static HostWord *table[64] = {};
-    static std::mutex guards[64];
-    int dev = 0;
-    SPLATAD_CHECK_HIP(hipGetDevice(&dev));
-    SPLATAD_REQUIRE(dev >= 0 && dev < 64, "packed projection: device index %d out of range", dev);
-    std::lock_guard<std::mutex> lock(table_guard);
-    if (!table[dev]) {
-        HostWord *w = new HostWord();
-        if (int rc = host_word_create(w)) { delete w; return rc; }
-        table[dev] = w;
-    }
-    *word = table[dev];
-    *guard = &guards[dev];
-    return 0;
-}
-
 extern "C" size_t splatad_projection_packed_workspace_bytes(uint32_t C, uint32_t N) {
     const uint64_t T = (uint64_t)C * N;
     return 256 + splatad_align256(T * 8) * 3 + splatad_align256(T * 4) * 3 +
@@ -451,11 +431,9 @@ extern "C" int splatad_projection_packed_count(
     const uint64_t T = (uint64_t)C * N;
     PackedWorkspace w = carve_packed(workspace, T);
     if (int rc = host_word_refuse_capture((hipStream_t)stream, "packed projection")) return rc;
-    HostWord *pw = nullptr;
-    std::mutex *guard = nullptr;
-    if (int rc = packed_host_word(&pw, &guard)) return rc;
-    std::lock_guard<std::mutex> lock(*guard);
-    *(volatile unsigned long long *)pw->host = kHostWordPending;
+    // the number of kept (camera, Gaussian) pairs reaches the host through a leased pinned word
+    HostWordLease lease((hipStream_t)stream);
+    if (int rc = host_word_acquire(&lease.word)) return rc;
     int rc = splatad_projection_fwd(C, N, means, covars, quats, scales, velocities, viewmats, Ks,
                                     W, H, lin_vel, ang_vel, rs_time, eps2d, near_plane, far_plane,
                                     radius_clip, w.radii, w.means2d, w.depths, w.conics,
@@ -465,10 +443,10 @@ extern "C" int splatad_projection_packed_count(
                                         (hipStream_t)stream);
     if (rc) return rc;
     hipLaunchKernelGGL(host_word_publish_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, w.total,
-                       pw->device);
+                       lease.word.device);
     SPLATAD_LAUNCH_CHECK();
     unsigned long long nnz = 0;
-    rc = host_word_wait(pw, (hipStream_t)stream, "packed projection", &nnz);
+    rc = host_word_wait(&lease, "packed projection", &nnz);
     if (rc) return rc;
     *nnz_host = (int64_t)nnz;
     return 0;

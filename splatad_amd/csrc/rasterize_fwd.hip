@@ -36,9 +36,12 @@ struct PixelArgs {
     int32_t *last_ids;
     int write_aux; // first pass also writes alphas and last ids
     int32_t *tile_batches; // optional diagnostic: batches each tile's workgroup went through
+    unsigned long long *lane_stats; // STATS kernels only: kLaneStats counters, see the entry point
 };
 
-template <int CH>
+constexpr int kLaneStats = 8;
+
+template <int CH, bool STATS = false>
 __global__ void __launch_bounds__(1024)
 rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     extern __shared__ float4 lds4[];
@@ -85,6 +88,7 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     for (int k = 0; k < CH; ++k) out[k] = 0.f;
 
     uint32_t batches_done = 0;
+    uint32_t st_iter = 0, st_take = 0, st_alive = 0, st_idle = 0, st_tested = 0, st_kept = 0, st_valid = 0;
     for (uint32_t b = 0; b < num_batches; ++b) {
         // also orders the previous batch's LDS reads before this batch's writes
         if (__syncthreads_count(!wave_lanes(alive_bits)) >= (int)block_size) break;
@@ -113,6 +117,10 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
             bool keep = base + lane < batch_size;
             if (keep) keep = cull.may_touch(s_rec[RECORD * (base + lane)], s_rec[RECORD * (base + lane) + 1]);
             uint64_t todo = wave_ballot(keep);
+            if (STATS) {
+                st_tested += min(batch_size - base, (uint32_t)SPLATAD_WAVE);
+                st_kept += (uint32_t)__popcll(todo);
+            }
             while (todo) {
                 const uint32_t t = base + (uint32_t)__ffsll((unsigned long long)todo) - 1u;
                 todo &= todo - 1;
@@ -130,6 +138,13 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
                                             wave_ballot(!(alpha < 1.f / 255.f));
                 const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
                 const uint64_t take_bits = valid_bits & ~stop_bits;
+                if (STATS) {
+                    st_iter += 1;
+                    st_alive += (uint32_t)__popcll(alive_bits);
+                    st_valid += (uint32_t)__popcll(valid_bits);
+                    st_take += (uint32_t)__popcll(take_bits);
+                    st_idle += take_bits == 0 ? 1u : 0u;
+                }
                 alive_bits &= ~stop_bits;
                 const bool take = wave_lanes(take_bits);
                 const float vis = take ? weight : 0.f;
@@ -145,6 +160,13 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     }
 
     if (a.tile_batches != nullptr && a.write_aux && tr == 0) a.tile_batches[blockIdx.x] = (int32_t)batches_done;
+    if (STATS) {
+        if (lane == 0) {
+            const uint32_t v[kLaneStats] = {st_iter, st_take, st_alive, st_idle, st_tested, st_kept, 1u, st_valid};
+            for (int k = 0; k < kLaneStats; ++k) atomicAdd(a.lane_stats + k, (unsigned long long)v[k]);
+        }
+        return;
+    }
     if (inside) {
         const size_t pix = ((size_t)cam * a.H + i) * a.W + j;
         float *dst = a.render_colors + pix * a.color_stride + a.ch_offset;
@@ -571,6 +593,7 @@ extern "C" int splatad_rasterize_to_pixels_fwd(
     a.tile_offsets = tile_offsets; a.flatten_ids = flatten_ids;
     a.render_colors = render_colors; a.render_alphas = render_alphas; a.last_ids = last_ids;
     a.tile_batches = tile_batches;
+    a.lane_stats = nullptr;
     const dim3 grid(C * tile_w * tile_h), block(tile_size, tile_size);
     const uint32_t pass = channels <= (uint32_t)kMaxPass ? channels : 32u;
     for (uint32_t off = 0; off < channels; off += pass) {
@@ -580,6 +603,33 @@ extern "C" int splatad_rasterize_to_pixels_fwd(
         int rc = dispatch_pixels(pick_width(a.n_ch), a, grid, block, (hipStream_t)stream);
         if (rc) return rc;
     }
+    return 0;
+}
+
+extern "C" int splatad_rasterize_to_pixels_lane_stats(
+    uint32_t C, int64_t n_isects, const float *means2d, const float *conics, const float *opacities,
+    const float *pix_vels, const float *rs_time, uint32_t W, uint32_t H, uint32_t tile_size,
+    uint32_t tile_w, uint32_t tile_h, const int32_t *tile_offsets, const int32_t *flatten_ids,
+    unsigned long long *stats, splatad_stream_t stream) {
+    SPLATAD_REQUIRE(tile_size >= 1 && tile_size * tile_size <= 1024,
+                    "rasterize_to_pixels: tile_size %u is outside 1..32", tile_size);
+    if (C == 0 || W == 0 || H == 0 || n_isects == 0) return 0;
+    SPLATAD_REQUIRE((uint64_t)tile_w * tile_size >= W && (uint64_t)tile_h * tile_size >= H,
+                    "rasterize_to_pixels: tile grid does not cover the image");
+    SPLATAD_REQUIRE(n_isects > 0 && n_isects < (1ll << 31), "rasterize_to_pixels: bad n_isects");
+    SPLATAD_REQUIRE(rs_time && tile_offsets && means2d && conics && opacities && pix_vels && flatten_ids && stats,
+                    "rasterize_to_pixels: null pointer argument");
+    PixelArgs a = {};
+    a.C = C; a.n_isects = n_isects; a.color_stride = 0; a.ch_offset = 0; a.n_ch = 0;
+    a.means2d = means2d; a.conics = conics; a.opacities = opacities;
+    a.pix_vels = pix_vels; a.rs_time = rs_time;
+    a.W = W; a.H = H; a.tile_size = tile_size; a.tile_w = tile_w; a.tile_h = tile_h;
+    a.tile_offsets = tile_offsets; a.flatten_ids = flatten_ids;
+    a.lane_stats = stats;
+    const dim3 grid(C * tile_w * tile_h), block(tile_size, tile_size);
+    const size_t lds = (size_t)block.x * block.y * 16 * 3;
+    hipLaunchKernelGGL((rasterize_to_pixels_fwd_kernel<1, true>), grid, block, lds, (hipStream_t)stream, a);
+    SPLATAD_LAUNCH_CHECK();
     return 0;
 }
 

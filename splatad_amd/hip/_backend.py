@@ -719,6 +719,26 @@ class _Ops:
                 _p(_in(tile_batches, "tile_batches", torch.int32)), _stream(dev)))
         return renders, alphas, last_ids
 
+    def rasterize_to_pixels_lane_stats(self, means2d, conics, opacities, pix_vels, rolling_shutter_time,
+                                       image_width, image_height, tile_size, tile_offsets, flatten_ids):
+        """Diagnostic: the eight lane-utilisation counters of the camera compositing loop
+        (include/splatad_hip.h) as an int64 tensor."""
+        lib = load_library()
+        means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
+        opacities = _in(opacities, "opacities"); pix_vels = _in(pix_vels, "pix_vels")
+        rs = _in(rolling_shutter_time, "rolling_shutter_time")
+        tile_offsets = _in(tile_offsets, "tile_offsets", torch.int32)
+        flatten_ids = _in(flatten_ids, "flatten_ids", torch.int32)
+        C, th, tw = tile_offsets.shape
+        dev = means2d.device
+        stats = torch.zeros((8,), dtype=torch.int64, device=dev)
+        with torch.cuda.device(dev):
+            _check(lib.splatad_rasterize_to_pixels_lane_stats(
+                _u32(C), _i64(flatten_ids.shape[0]), _p(means2d), _p(conics), _p(opacities), _p(pix_vels),
+                _p(rs), _u32(image_width), _u32(image_height), _u32(tile_size), _u32(tw), _u32(th),
+                _p(tile_offsets), _p(flatten_ids), _p(stats), _stream(dev)))
+        return stats
+
     def rasterize_to_pixels_bwd(self, means2d, conics, colors, opacities, pix_vels,
                                 rolling_shutter_time, backgrounds, image_width, image_height,
                                 tile_size, tile_offsets, flatten_ids, render_alphas, last_ids,

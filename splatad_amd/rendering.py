@@ -5,6 +5,7 @@
 hand-written gfx950 kernel through the operators of `splatad_amd.hip._wrapper`.
 """
 import math
+import threading
 from typing import Dict, Optional, Tuple, Union
 
 import torch
@@ -41,7 +42,9 @@ def _sensor_motion(C, device, linear_velocity, angular_velocity, rolling_shutter
     return linear_velocity, angular_velocity, rolling_shutter_time
 
 
-_HELPER_STREAMS: Dict[int, "torch.cuda.Stream"] = {}
+# one helper stream per (device, host thread): calls from different threads do not wait for one
+# another's helper work
+_HELPER_STREAMS: Dict[Tuple[int, int], "torch.cuda.Stream"] = {}
 
 
 class _Beside:
@@ -62,10 +65,11 @@ class _Beside:
         self.main = self.side = self.fork = self._ctx = None
         if device.type == "cuda" and not torch.cuda.is_current_stream_capturing():
             idx = device.index if device.index is not None else torch.cuda.current_device()
-            if idx not in _HELPER_STREAMS:
-                _HELPER_STREAMS[idx] = torch.cuda.Stream(device=idx)
+            key = (idx, threading.get_ident())
+            if key not in _HELPER_STREAMS:
+                _HELPER_STREAMS[key] = torch.cuda.Stream(device=idx)
             self.main = torch.cuda.current_stream(idx)
-            self.side = _HELPER_STREAMS[idx]
+            self.side = _HELPER_STREAMS[key]
             self.fork = self.main.record_event()
 
     def __enter__(self):

@@ -17,7 +17,7 @@ import torch
 import oracle
 from tests.gpu_util import DEV, assert_close, to_dev, to_np
 from tests.test_gpu_backward import _raster_scene, assert_grad_close
-from tests.test_gpu_forward import RASTER_FRAC, _lidar_scene, _projected_scene
+from tests.test_gpu_forward import _lidar_scene, _projected_scene
 
 pytestmark = pytest.mark.gpu
 
@@ -154,8 +154,8 @@ def test_list_compositing_reproduces_fused_pixels_with_gradients(D, ts, per_iter
                                  rolling_shutter_time=rs, backgrounds=fused[5])
     l_rc, l_ra = _rasterize_to_pixels(lists[0], lists[1], lists[2], lists[3], lists[4], W, H, ts, offs, flat,
                                       rs, backgrounds=lists[5], batch_per_iter=per_iter)
-    assert_close(to_np(l_rc), to_np(rc), atol=1e-4, frac=RASTER_FRAC, name="colors")
-    assert_close(to_np(l_ra), to_np(ra), atol=1e-4, frac=RASTER_FRAC, name="alphas")
+    assert_close(to_np(l_rc), to_np(rc), atol=1e-4, name="colors")
+    assert_close(to_np(l_ra), to_np(ra), atol=1e-4, name="alphas")
     rng = np.random.default_rng(1)
     wc = to_dev(rng.normal(size=tuple(rc.shape)).astype(np.float32))
     wa = to_dev(rng.normal(size=tuple(ra.shape)).astype(np.float32))
@@ -183,14 +183,14 @@ def test_list_compositing_reproduces_fused_points_with_gradients(asum):
     lists = [t.detach().clone().requires_grad_() for t in base]
     rf, ra, rsum, _ = rasterize_to_points(*fused, d["raster_pts"], W, H, tw, th, offs, flat, asum, 0.3)
     l_rf, l_ra, l_sum = _rasterize_to_points(*lists, d["raster_pts"], W, H, tw, th, offs, flat, asum, 0.3)
-    assert_close(to_np(l_rf), to_np(rf), atol=2e-4, rtol=1e-4, frac=RASTER_FRAC, name="features")
-    assert_close(to_np(l_ra), to_np(ra), atol=1e-4, frac=RASTER_FRAC, name="alphas")
+    assert_close(to_np(l_rf), to_np(rf), atol=2e-4, rtol=1e-4, name="features")
+    assert_close(to_np(l_ra), to_np(ra), atol=1e-4, name="alphas")
     rng = np.random.default_rng(2)
     wf = to_dev(rng.normal(size=tuple(rf.shape)).astype(np.float32))
     wa = to_dev(rng.normal(size=tuple(ra.shape)).astype(np.float32))
     loss_f, loss_l = (rf * wf).sum() + (ra * wa).sum(), (l_rf * wf).sum() + (l_ra * wa).sum()
     if asum:
-        assert_close(to_np(l_sum), to_np(rsum), atol=1e-4, rtol=1e-4, frac=RASTER_FRAC, name="alpha_sum")
+        assert_close(to_np(l_sum), to_np(rsum), atol=1e-4, rtol=1e-4, name="alpha_sum")
         ws = to_dev(rng.normal(size=tuple(rsum.shape)).astype(np.float32))
         loss_f, loss_l = loss_f + (rsum * ws).sum(), loss_l + (l_sum * ws).sum()
     else:
