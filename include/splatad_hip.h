@@ -230,6 +230,27 @@ int splatad_map_points_to_lidar_tiles(uint64_t total, uint32_t N, const int64_t 
                                       int64_t *tile_ids, int32_t *flatten_ids,
                                       splatad_stream_t stream);
 
+/* splatad_map_points_to_lidar_tiles for callers that cannot allocate (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments without the workspace: the counter table of the sorted mode lives in
+ * a static device array of the library (about 2 MiB per GPU, held until the process ends), and
+ * the call allocates nothing, on the device or on the host.  Limits, beyond which it returns an
+ * error and launches nothing: total <= splatad_map_points_to_lidar_tiles_noalloc_max_points()
+ * (4 194 304 points) and C * n_tiles_azim * n_tiles_elev <=
+ * splatad_map_points_to_lidar_tiles_noalloc_max_tiles() (16 384).  Results are identical to
+ * splatad_map_points_to_lidar_tiles.  All calls on one GPU share that GPU's array: calls that
+ * overlap on one GPU (different streams, different threads) race; calls in stream order do not,
+ * and nothing has to be cleared between them. */
+uint64_t splatad_map_points_to_lidar_tiles_noalloc_max_points(void);
+uint32_t splatad_map_points_to_lidar_tiles_noalloc_max_tiles(void);
+int splatad_map_points_to_lidar_tiles_noalloc(uint64_t total, uint32_t N,
+                                              const int64_t *camera_ids, const float *points2d,
+                                              uint32_t C, const float *elev_boundaries,
+                                              float tile_azim_resolution, float min_azim,
+                                              uint32_t n_tiles_azim, uint32_t n_tiles_elev,
+                                              int sort, int64_t *tile_ids, int32_t *flatten_ids,
+                                              splatad_stream_t stream);
+
 /* points_mapping_offset_encode_tensor, rasterization.cu:576-594 (kernel :531-574). */
 int splatad_points_mapping_offset_encode(int64_t n_points, const int64_t *point_ids, uint32_t C,
                                          uint32_t n_tiles, int32_t *offsets,

@@ -202,32 +202,22 @@ extern "C" size_t splatad_map_points_to_lidar_tiles_workspace_bytes(uint64_t tot
     return carve_bin(nullptr, n_slots * bin_workgroups(total, n_slots), nullptr);
 }
 
-extern "C" int splatad_map_points_to_lidar_tiles(
-    uint64_t total, uint32_t N, const int64_t *camera_ids, const float *points2d, uint32_t C,
-    const float *elev_boundaries, float tile_azim_resolution, float min_azim,
-    uint32_t n_tiles_azim, uint32_t n_tiles_elev, int sort, void *workspace, int64_t *tile_ids,
-    int32_t *flatten_ids, splatad_stream_t stream_) {
-    hipStream_t stream = (hipStream_t)stream_;
-    if (total == 0) return 0;
-    SPLATAD_REQUIRE(total < (1ull << 31), "map_points_to_lidar_tiles: number of points must be below 2^31");
-    SPLATAD_REQUIRE(points2d && elev_boundaries && tile_ids && flatten_ids,
-                    "map_points_to_lidar_tiles: null pointer argument");
-    SPLATAD_REQUIRE(camera_ids != nullptr || N > 0, "map_points_to_lidar_tiles: N is zero for unpacked input");
-    SPLATAD_REQUIRE(C > 0 && n_tiles_azim > 0 && n_tiles_elev > 0, "map_points_to_lidar_tiles: empty tile grid");
-    PointGrid g{n_tiles_azim, n_tiles_elev, tile_azim_resolution, min_azim, elev_boundaries};
-    if (!sort) {
-        hipLaunchKernelGGL(points_keys_kernel, dim3((uint32_t)((total + SPLATAD_THREADS - 1) / SPLATAD_THREADS)),
-                           dim3(SPLATAD_THREADS), 0, stream, g, total, N, camera_ids, points2d,
-                           tile_ids, flatten_ids);
-        SPLATAD_LAUNCH_CHECK();
-        return 0;
-    }
-    SPLATAD_REQUIRE(workspace != nullptr, "map_points_to_lidar_tiles: workspace is null");
-    const uint64_t n_slots64 = (uint64_t)C * n_tiles_azim * n_tiles_elev;
+namespace {
+
+// The sorted binning behind both entry points.  `max_table` bounds the [workgroup][slot] counter
+// table (and with it the scratch the caller has to provide): fewer workgroups are used when
+// the plain choice would exceed it.
+static int map_points_sorted(const PointGrid &g, uint64_t total, uint32_t N, const int64_t *camera_ids,
+                             const float *points2d, uint32_t C, void *workspace, uint64_t max_table,
+                             int64_t *tile_ids, int32_t *flatten_ids, hipStream_t stream) {
+    const uint64_t n_slots64 = (uint64_t)C * g.n_tiles_azim * g.n_tiles_elev;
     SPLATAD_REQUIRE(n_slots64 <= kMaxSlots, "map_points_to_lidar_tiles: %llu (sensor, tile) pairs exceed "
                     "the binning capacity of %u", (unsigned long long)n_slots64, kMaxSlots);
     const uint32_t n_slots = (uint32_t)n_slots64;
-    const uint32_t wgs = bin_workgroups(total, n_slots);
+    uint32_t wgs = bin_workgroups(total, n_slots);
+    if ((uint64_t)wgs * n_slots > max_table) wgs = (uint32_t)(max_table / n_slots);
+    SPLATAD_REQUIRE(wgs >= 1, "map_points_to_lidar_tiles: %u (sensor, tile) pairs exceed the counter table "
+                    "of %llu entries", n_slots, (unsigned long long)max_table);
     const uint64_t span = ((total + wgs - 1) / wgs + SPLATAD_WAVE - 1) / SPLATAD_WAVE * SPLATAD_WAVE;
     BinWorkspace w;
     carve_bin(workspace, (uint64_t)n_slots * wgs, &w);
@@ -257,6 +247,110 @@ extern "C" int splatad_map_points_to_lidar_tiles(
                        span, N, camera_ids, points2d, n_slots, w.starts, tile_ids, flatten_ids);
     SPLATAD_LAUNCH_CHECK();
     return 0;
+}
+
+static int map_points_check(uint64_t total, uint32_t N, const int64_t *camera_ids, const float *points2d,
+                            uint32_t C, const float *elev_boundaries, uint32_t n_tiles_azim,
+                            uint32_t n_tiles_elev, const int64_t *tile_ids, const int32_t *flatten_ids) {
+    SPLATAD_REQUIRE(total < (1ull << 31), "map_points_to_lidar_tiles: number of points must be below 2^31");
+    SPLATAD_REQUIRE(points2d && elev_boundaries && tile_ids && flatten_ids,
+                    "map_points_to_lidar_tiles: null pointer argument");
+    SPLATAD_REQUIRE(camera_ids != nullptr || N > 0, "map_points_to_lidar_tiles: N is zero for unpacked input");
+    SPLATAD_REQUIRE(C > 0 && n_tiles_azim > 0 && n_tiles_elev > 0, "map_points_to_lidar_tiles: empty tile grid");
+    return 0;
+}
+
+static int map_points_unsorted(const PointGrid &g, uint64_t total, uint32_t N, const int64_t *camera_ids,
+                               const float *points2d, int64_t *tile_ids, int32_t *flatten_ids,
+                               hipStream_t stream) {
+    hipLaunchKernelGGL(points_keys_kernel, dim3((uint32_t)((total + SPLATAD_THREADS - 1) / SPLATAD_THREADS)),
+                       dim3(SPLATAD_THREADS), 0, stream, g, total, N, camera_ids, points2d, tile_ids,
+                       flatten_ids);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
+}
+
+// Scratch of the entry point that allocates nothing: a counter table of at most kStaticTable
+// entries, its scan, the scan's block sums and total, laid out by carve_bin().  Every GPU the
+// library runs on holds its own copy of this array from the moment the library is loaded until
+// the process ends (about 2 MiB).
+constexpr uint64_t kStaticTable = 1ull << 18;
+constexpr size_t kStaticScratchBytes =
+    256 + 2 * (size_t)kStaticTable * 4 + ((kStaticTable + SCAN_TILE - 1) / SCAN_TILE) * 8 + 256;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Address of the current device's copy of `scratch`, looked up once per device.  In host code
+// the array's name is only a handle for this lookup, never an address a kernel could use.
+static int static_scratch(void **out) {
+    static std::mutex guard;
+    static void *table[64] = {};
+    int dev = 0;
+    SPLATAD_CHECK_HIP(hipGetDevice(&dev));
+    SPLATAD_REQUIRE(dev >= 0 && dev < 64, "map_points_to_lidar_tiles: device index %d out of range", dev);
+    SPLATAD_REQUIRE(carve_bin(nullptr, kStaticTable, nullptr) <= kStaticScratchBytes,
+                    "map_points_to_lidar_tiles: the static scratch is smaller than its layout");
+    std::lock_guard<std::mutex> lock(guard);
+    if (table[dev] == nullptr) {
+        void *ptr = nullptr;
+        SPLATAD_CHECK_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+        SPLATAD_REQUIRE(ptr != nullptr, "map_points_to_lidar_tiles: the static scratch has no device address");
+        table[dev] = ptr;
+    }
+    *out = table[dev];
+    return 0;
+}
+
+} // namespace
+
+extern "C" int splatad_map_points_to_lidar_tiles(
+    uint64_t total, uint32_t N, const int64_t *camera_ids, const float *points2d, uint32_t C,
+    const float *elev_boundaries, float tile_azim_resolution, float min_azim,
+    uint32_t n_tiles_azim, uint32_t n_tiles_elev, int sort, void *workspace, int64_t *tile_ids,
+    int32_t *flatten_ids, splatad_stream_t stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (total == 0) return 0;
+    if (int rc = map_points_check(total, N, camera_ids, points2d, C, elev_boundaries, n_tiles_azim,
+                                  n_tiles_elev, tile_ids, flatten_ids))
+        return rc;
+    PointGrid g{n_tiles_azim, n_tiles_elev, tile_azim_resolution, min_azim, elev_boundaries};
+    if (!sort) return map_points_unsorted(g, total, N, camera_ids, points2d, tile_ids, flatten_ids, stream);
+    SPLATAD_REQUIRE(workspace != nullptr, "map_points_to_lidar_tiles: workspace is null");
+    return map_points_sorted(g, total, N, camera_ids, points2d, C, workspace, ~0ull, tile_ids, flatten_ids,
+                             stream);
+}
+
+extern "C" uint64_t splatad_map_points_to_lidar_tiles_noalloc_max_points(void) { return 1ull << 22; }
+extern "C" uint32_t splatad_map_points_to_lidar_tiles_noalloc_max_tiles(void) { return 16384u; }
+
+extern "C" int splatad_map_points_to_lidar_tiles_noalloc(
+    uint64_t total, uint32_t N, const int64_t *camera_ids, const float *points2d, uint32_t C,
+    const float *elev_boundaries, float tile_azim_resolution, float min_azim,
+    uint32_t n_tiles_azim, uint32_t n_tiles_elev, int sort, int64_t *tile_ids,
+    int32_t *flatten_ids, splatad_stream_t stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (total == 0) return 0;
+    if (int rc = map_points_check(total, N, camera_ids, points2d, C, elev_boundaries, n_tiles_azim,
+                                  n_tiles_elev, tile_ids, flatten_ids))
+        return rc;
+    SPLATAD_REQUIRE(total <= splatad_map_points_to_lidar_tiles_noalloc_max_points(),
+                    "map_points_to_lidar_tiles_noalloc: %llu points exceed the limit of %llu of the entry "
+                    "point that allocates nothing; use splatad_map_points_to_lidar_tiles with a workspace",
+                    (unsigned long long)total,
+                    (unsigned long long)splatad_map_points_to_lidar_tiles_noalloc_max_points());
+    const uint64_t n_slots = (uint64_t)C * n_tiles_azim * n_tiles_elev;
+    SPLATAD_REQUIRE(n_slots <= splatad_map_points_to_lidar_tiles_noalloc_max_tiles(),
+                    "map_points_to_lidar_tiles_noalloc: %llu (sensor, tile) pairs exceed the limit of %u of "
+                    "the entry point that allocates nothing; use splatad_map_points_to_lidar_tiles with a "
+                    "workspace", (unsigned long long)n_slots, splatad_map_points_to_lidar_tiles_noalloc_max_tiles());
+    PointGrid g{n_tiles_azim, n_tiles_elev, tile_azim_resolution, min_azim, elev_boundaries};
+    if (!sort) return map_points_unsorted(g, total, N, camera_ids, points2d, tile_ids, flatten_ids, stream);
+    void *ptr = nullptr;
+    if (int rc = static_scratch(&ptr)) return rc;
+    // Every word of the scratch that a kernel reads is written by an earlier kernel of the same
+    // call (the counting pass stores whole rows of the table, the scan its block sums, its
+    // output and its total), so nothing has to be cleared between calls.
+    return map_points_sorted(g, total, N, camera_ids, points2d, C, ptr, kStaticTable, tile_ids, flatten_ids,
+                             stream);
 }
 
 extern "C" int splatad_points_mapping_offset_encode(int64_t n_points, const int64_t *point_ids,
