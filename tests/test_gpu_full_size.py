@@ -254,7 +254,7 @@ def test_training_step_1m_lidar_backward_properties():
     ones = torch.zeros_like(rf)
     ones[..., :-1] = 1.0
     (v_feat,) = torch.autograd.grad((rf * ones).sum(), [p["lidar_features"]], retain_graph=True)
-    total_alpha = float(ra.double().sum())
+    total_alpha = float(ra.detach().double().sum())
     per_channel = v_feat.double().sum(dim=(0, 1))
     assert float((per_channel - total_alpha).abs().max()) <= 1e-4 * total_alpha
     # linear in the cotangent
