@@ -67,16 +67,10 @@ def time_kernel(fn, iters, warmup=2):
     return sum(s.elapsed_time(e) for s, e in zip(start, stop)) / iters
 
 
-def staged_isects(tile_batches, offsets, n_isects, batch=256):
+def staged_isects(tile_entries):
     """List entries the compositing kernel staged: whole batches until every pixel / point of a
-    tile has saturated, as counted by the kernel itself, clipped to the tile's list."""
-    import torch
-
-    flat_off = offsets.reshape(-1).long()
-    ends = torch.cat([flat_off[1:], torch.tensor([n_isects], device=flat_off.device)])
-    full = ends - flat_off
-    need = torch.minimum(tile_batches.reshape(-1).long() * batch, full)
-    return int(need.sum().item()), int(full.sum().item())
+    tile has saturated, clipped to the tile's list, as counted by the kernel itself."""
+    return int(tile_entries.sum().item())
 
 
 def bench_camera(args):
@@ -124,7 +118,7 @@ def bench_camera(args):
             meta["means2d"], meta["conics"], cols, meta["opacities"], meta["pix_vels"],
             s["rolling_shutter_time"], None, W, H, ts, meta["isect_offsets"], meta["flatten_ids"],
             tile_batches=batches)
-        i_need, i_full = staged_isects(batches, meta["isect_offsets"], n_isects)
+        i_need = staged_isects(batches)
         D = cols.shape[-1]
         P, T = C * H * W, meta["isect_offsets"].numel()
         alg_bytes = i_need * (36 + 4 * D) + P * (4 * D + 8) + T * 4
@@ -194,7 +188,7 @@ def bench_lidar(args):
         n_isects = int(meta["flatten_ids"].shape[0])
         batches = torch.zeros_like(meta["isect_offsets"])
         raster(tile_batches=batches)
-        i_need, _ = staged_isects(batches, meta["isect_offsets"], n_isects)
+        i_need = staged_isects(batches)
         P, T = C * H * W, meta["isect_offsets"].numel()
         # staged per list entry: id, mean, angular velocity, conic, opacity (40 bytes); the features
         # of the Gaussians a wavefront composites are read on demand and not counted here

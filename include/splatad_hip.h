@@ -271,9 +271,9 @@ int splatad_populate_image_from_points(uint32_t C, int64_t n_points, const float
 /* rasterize_to_pixels_fwd_tensor, rasterization.cu:1520-2018 (kernel
  * :1360-1518).  Any channel count >= 1 is accepted (wide inputs are rendered in
  * passes).  backgrounds may be NULL.  tile_batches may be NULL; otherwise it receives,
- * per (camera, tile), the number of 256-entry batches of the tile's list that were staged
- * before every pixel of the tile had saturated (a diagnostic: it tells how much of the
- * sorted lists a frame really reads). */
+ * per (camera, tile), the number of entries of the tile's list that were staged (whole
+ * batches, until every pixel of the tile had saturated, clipped to the list's length; a
+ * diagnostic: it tells how much of the sorted lists a frame really reads). */
 int splatad_rasterize_to_pixels_fwd(uint32_t C, int64_t n_isects, uint32_t channels,
                                     const float *means2d, const float *conics,
                                     const float *colors, const float *opacities,

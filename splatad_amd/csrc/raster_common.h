@@ -16,6 +16,7 @@ constexpr float kLog2Of255 = 7.99435343685886f;
 // A = a log2(e) / 2, B = b log2(e), C = c log2(e) / 2 for the conic (a, b, c) and
 // L = log2(opacity) (-inf for opacity <= 0, which can then never reach alpha >= 1/255).
 __device__ __forceinline__ float4 staged_exponent(float a, float b, float c, float opacity) {
+#pragma clang fp contract(off)
     return make_float4(0.5f * kLog2e * a, kLog2e * b, 0.5f * kLog2e * c,
                        opacity > 0.f ? __log2f(opacity) : -INFINITY);
 }
@@ -158,6 +159,129 @@ struct WavePointCull {
         unfolded_ok = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(y0), fabsf(y1))) < 179.f;
         if (!unfolded_ok || !enabled) return true;
         return box_may_pass(e, x0, x1, y0, y1);
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// The exponent of a camera pixel as a polynomial in tile-centred pixel coordinates.
+//
+// With the rolling-shutter factor linear in the pixel row, roll = roll_c + roll_s Y, the offset
+// of pixel (X, Y) (relative to the tile centre) from a Gaussian is dx = dx0 - X + sx Y, dy = dy0 +
+// sy Y, and log2(alpha) = L - (A dx^2 + B dx dy + C dy^2) is a quadratic polynomial in (X, Y)
+// whose six coefficients depend on the Gaussian and the tile only.  They are computed once per
+// (tile, Gaussian) when the Gaussian is staged; a pixel then needs five fused multiply-adds
+// with its own constants (X, Y, X^2, X Y, Y^2; exact in float32 for half-integers) instead of
+// the ten operations of the offset form, and every kernel that evaluates a pixel through
+// pixel_exponent() gets the same bits, whatever its lane layout.  Inside a 16 x 16 tile |X|, |Y|
+// <= 7.5, and the cancellation between the terms costs at most a few 1e-5 of absolute accuracy
+// in the exponent for the sharpest Gaussians the projection can produce (conic 1 / eps2d).
+struct TileFrame {
+    float cx, cy;         // tile centre in pixel coordinates
+    float roll_c, roll_s; // rolling-shutter factor at the centre row, and per row
+};
+
+__device__ __forceinline__ TileFrame tile_frame(uint32_t tile_x, uint32_t tile_y, uint32_t tile_size,
+                                                float rs_time, uint32_t H) {
+#pragma clang fp contract(off)
+    TileFrame f;
+    f.cx = (float)(tile_x * tile_size) + 0.5f * (float)tile_size;
+    f.cy = (float)(tile_y * tile_size) + 0.5f * (float)tile_size;
+    // rasterization.cu:1401: roll = rs_time * (row / (H - 1) - 0.5), row = pixel centre - 0.5
+    f.roll_s = rs_time / (float)(H - 1);
+    f.roll_c = rs_time * ((f.cy - 0.5f) / (float)(H - 1) - 0.5f);
+    return f;
+}
+
+// a = {c0, cX, cY, cXX}, b = {cXY, cYY, X*, Y* or L}: exponent(X, Y) = c0 + cX X + cY Y + cXX X^2
+// + cXY X Y + cYY Y^2.  For a positive definite conic with opacity <= 0.999 (alpha then never
+// reaches the 0.999 clamp and sigma is never negative) b.z, b.w hold the pixel offset (X*, Y*) at
+// which the exponent peaks, which the footprint test uses.  Otherwise b.z is NaN ("general": the
+// compositing loop applies the clamp and the sigma < 0 rule, the footprint test keeps the
+// Gaussian) and b.w holds L for an indefinite conic, +inf for a definite one (sigma < 0 <=>
+// exponent > L can then never hold).
+//
+// No implicit contraction in here: every kernel that stages a Gaussian has to arrive at the same
+// bits (they take the alpha >= 1/255 decisions from them), and left to itself the compiler fuses
+// multiplies and adds differently from one template instantiation to the next.
+__device__ __forceinline__ void pixel_polynomial(const TileFrame &f, float2 xy, float2 v, float ca,
+                                                 float cb, float cc, float opacity, float4 &a, float4 &b) {
+#pragma clang fp contract(off)
+    const float4 e = staged_exponent(ca, cb, cc, opacity);
+    const float A = e.x, B = e.y, C = e.z, L = e.w;
+    const float dx0 = fmaf(f.roll_c, v.x, xy.x - f.cx), dy0 = fmaf(f.roll_c, v.y, xy.y - f.cy);
+    const float sx = f.roll_s * v.x, sy = fmaf(f.roll_s, v.y, -1.f);
+    const float Adx = A * dx0, Cdy = C * dy0;
+    a.x = L - (dx0 * fmaf(B, dy0, Adx) + Cdy * dy0);
+    a.y = fmaf(2.f, Adx, B * dy0);
+    a.z = -(2.f * Adx * sx + B * fmaf(dx0, sy, sx * dy0) + 2.f * Cdy * sy);
+    a.w = -A;
+    b.x = fmaf(2.f * A, sx, B * sy);
+    b.y = -(sx * fmaf(A, sx, B * sy) + C * sy * sy);
+    const bool definite = A > 0.f && C > 0.f && 4.f * A * C - B * B > 0.f;
+    const bool plain = definite && opacity <= 0.999f && fabsf(sy) > 1e-3f && b.y < 0.f;
+    if (plain) {
+        const float ys = -dy0 * __builtin_amdgcn_rcpf(sy); // dy = 0
+        b.w = ys;
+        b.z = fmaf(sx, ys, dx0);                           // dx = 0
+    } else {
+        b.z = NAN;
+        b.w = definite ? INFINITY : L;
+    }
+}
+
+struct PixelConstants {
+    float X, Y, XX, XY, YY;
+    __device__ __forceinline__ void init(float px, float py, const TileFrame &f) {
+#pragma clang fp contract(off)
+        X = px - f.cx; Y = py - f.cy;
+        XX = X * X; XY = X * Y; YY = Y * Y;
+    }
+};
+
+__device__ __forceinline__ float pixel_exponent(const float4 a, float cXY, float cYY, const PixelConstants &p) {
+    return fmaf(cYY, p.YY, fmaf(cXY, p.XY, fmaf(a.w, p.XX, fmaf(a.z, p.Y, fmaf(a.y, p.X, a.x)))));
+}
+
+// Footprint of a wavefront of camera pixels in tile-centred coordinates, and the test whether
+// any pixel in it can reach alpha >= 1/255 for a staged polynomial: the exponent is concave for
+// a definite conic, so over a box that does not contain its peak it is largest on one of the
+// four edges, where it is a parabola.  A margin covers the rounding of the test itself.
+struct WaveBox {
+    bool enabled;
+    float x0, x1, y0, y1;
+
+    __device__ __forceinline__ void init(float x_lo, float x_hi, float y_lo, float y_hi, bool full_wavefront) {
+        enabled = full_wavefront;
+        if (enabled) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                x_lo = fminf(x_lo, __shfl_xor(x_lo, off, SPLATAD_WAVE));
+                x_hi = fmaxf(x_hi, __shfl_xor(x_hi, off, SPLATAD_WAVE));
+                y_lo = fminf(y_lo, __shfl_xor(y_lo, off, SPLATAD_WAVE));
+                y_hi = fmaxf(y_hi, __shfl_xor(y_hi, off, SPLATAD_WAVE));
+            }
+        }
+        x0 = x_lo; x1 = x_hi; y0 = y_lo; y1 = y_hi;
+    }
+
+    __device__ __forceinline__ float edge_x(const float4 a, float cXY, float cYY, float hYY, float xe) const {
+        const float a0 = fmaf(xe, fmaf(a.w, xe, a.y), a.x), a1 = fmaf(cXY, xe, a.z);
+        const float yc = __builtin_amdgcn_fmed3f(a1 * hYY, y0, y1);
+        return fmaf(yc, fmaf(cYY, yc, a1), a0);
+    }
+    __device__ __forceinline__ float edge_y(const float4 a, float cXY, float cYY, float hXX, float ye) const {
+        const float b0 = fmaf(ye, fmaf(cYY, ye, a.z), a.x), b1 = fmaf(cXY, ye, a.y);
+        const float xc = __builtin_amdgcn_fmed3f(b1 * hXX, x0, x1);
+        return fmaf(xc, fmaf(a.w, xc, b1), b0);
+    }
+
+    __device__ __forceinline__ bool may_touch(const float4 a, const float4 b) const {
+        if (!enabled || !(b.z == b.z)) return true;
+        if (b.z >= x0 && b.z <= x1 && b.w >= y0 && b.w <= y1) return true;
+        const float hYY = -0.5f * __builtin_amdgcn_rcpf(b.y), hXX = -0.5f * __builtin_amdgcn_rcpf(a.w);
+        const float m = fmaxf(fmaxf(edge_x(a, b.x, b.y, hYY, x0), edge_x(a, b.x, b.y, hYY, x1)),
+                              fmaxf(edge_y(a, b.x, b.y, hXX, y0), edge_y(a, b.x, b.y, hXX, y1)));
+        return !(m < -kLog2Of255 - 0.05f - 4e-6f * fabsf(a.x));
     }
 };
 

@@ -21,6 +21,8 @@
 // host-side padding (wide inputs in passes of up to 32 channels).
 #include "raster_common.h"
 
+#include <type_traits>
+
 namespace {
 
 struct PixelArgs {
@@ -35,148 +37,276 @@ struct PixelArgs {
     float *render_colors, *render_alphas;
     int32_t *last_ids;
     int write_aux; // first pass also writes alphas and last ids
-    int32_t *tile_batches; // optional diagnostic: batches each tile's workgroup went through
+    int32_t *tile_batches; // optional diagnostic: list entries each tile's workgroup staged
     unsigned long long *lane_stats; // STATS kernels only: kLaneStats counters, see the entry point
 };
 
 constexpr int kLaneStats = 8;
 
-template <int CH, bool STATS = false>
+// PPL pixels per lane.  With PPL == 2 (tiles whose side is a multiple of 8 and that make whole
+// wavefronts that way) a wavefront covers 8 columns x 16 rows, lane (lx, ly) the pixels (lx, ly)
+// and (lx, ly + 8): every staged value read from LDS and every scalar instruction of the loop
+// then serves two pixels.  A wavefront's LDS reads are broadcasts of 16 bytes to 64 lanes, which
+// the LDS delivers at 128 bytes per clock: with one pixel per lane the three reads of a
+// (wavefront, Gaussian) iteration keep the LDS of a compute unit as busy as the iteration's
+// vector instructions keep a SIMD, and four SIMDs share that LDS.
+//
+// Per batch of the tile's list the workgroup stages, for every Gaussian, the six coefficients
+// of its exponent polynomial (raster_common.h), what the footprint test needs and its colours.
+// Every wavefront then tests 64 staged Gaussians at a time against its footprint, copies the
+// survivors' records in list order into a private strip of LDS (its own writes and reads: no
+// barrier) and walks that strip: sequential addresses, no lane-mask bookkeeping per Gaussian.
+template <int CH, int PPL, bool STATS = false>
 __global__ void __launch_bounds__(1024)
 rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     extern __shared__ float4 lds4[];
-    const uint32_t block_size = blockDim.x * blockDim.y;
-    // per Gaussian: {x, y, vx, vy} and {A, B, C, L}, where sigma * log2(e) = A dx^2 + B dx dy +
-    // C dy^2 and L = log2(opacity), so that alpha = exp2(L - (A dx^2 + B dx dy + C dy^2))
-    // followed by the CH colours, padded to a multiple of four floats
-    constexpr int RECORD = 2 + (CH + 3) / 4; // float4 per Gaussian
+    const uint32_t block_size = blockDim.x;
+    const uint32_t batch = block_size; // list entries staged at a time, one per lane
+    constexpr bool COPY = CH <= 4;           // survivors carry their colours along
+    constexpr int RECORD = 2 + (CH + 3) / 4; // float4 per staged Gaussian
+    constexpr int LIST = COPY ? 3 : 2;       // float4 per survivor
     float4 *s_rec = lds4;
 
     const uint32_t tiles_per_cam = a.tile_w * a.tile_h;
     const uint32_t cam = blockIdx.x / tiles_per_cam;
     const uint32_t tile_id = blockIdx.x % tiles_per_cam;
     const uint32_t tile_y = tile_id / a.tile_w, tile_x = tile_id % a.tile_w;
-    const uint32_t tr = threadIdx.y * blockDim.x + threadIdx.x;
-    const uint32_t lane = tr & (SPLATAD_WAVE - 1);
-    uint32_t lx, ly;
-    pixel_of_lane(a.tile_size, tr, lx, ly);
-    const uint32_t i = tile_y * a.tile_size + ly;
-    const uint32_t j = tile_x * a.tile_size + lx;
+    const uint32_t tr = threadIdx.x;
+    const uint32_t lane = tr & (SPLATAD_WAVE - 1), wave = tr / SPLATAD_WAVE;
+    float4 *s_list = lds4 + (size_t)RECORD * batch + (size_t)wave * SPLATAD_WAVE * LIST;
 
-    const float px = (float)j + 0.5f, py = (float)i + 0.5f;
-    const float roll = a.rs_time[cam] * ((py - 0.5f) / (float)(a.H - 1) - 0.5f);
-    const bool inside = (i < a.H && j < a.W);
-    // lanes still compositing, as a lane mask: the decisions of the inner loop are taken with
-    // scalar logic on such masks
-    uint64_t alive_bits = wave_ballot(inside);
+    const TileFrame frame = tile_frame(tile_x, tile_y, a.tile_size, a.rs_time[cam], a.H);
+    uint32_t pi[PPL], pj;
+    if (PPL == 2) {
+        const uint32_t waves_per_row = a.tile_size / 8;
+        const uint32_t lx = (wave % waves_per_row) * 8 + (lane & 7);
+        const uint32_t ly = (wave / waves_per_row) * 16 + (lane >> 3);
+        pj = tile_x * a.tile_size + lx;
+#pragma unroll
+        for (int p = 0; p < PPL; ++p) pi[p] = tile_y * a.tile_size + ly + 8 * p;
+    } else {
+        uint32_t lx, ly;
+        pixel_of_lane(a.tile_size, tr, lx, ly);
+        pj = tile_x * a.tile_size + lx;
+        pi[0] = tile_y * a.tile_size + ly;
+    }
+    PixelConstants pc[PPL];
+    bool inside[PPL];
+    uint64_t alive_bits[PPL]; // lanes still compositing, as lane masks (scalar logic below)
+    float y_lo = 0.f, y_hi = 0.f;
+#pragma unroll
+    for (int p = 0; p < PPL; ++p) {
+        pc[p].init((float)pj + 0.5f, (float)pi[p] + 0.5f, frame);
+        inside[p] = pi[p] < a.H && pj < a.W;
+        alive_bits[p] = wave_ballot(inside[p]);
+        y_lo = p == 0 ? pc[p].Y : fminf(y_lo, pc[p].Y);
+        y_hi = p == 0 ? pc[p].Y : fmaxf(y_hi, pc[p].Y);
+    }
+    WaveBox box; // footprint of this wavefront (all 64 lanes exist in whole wavefronts)
+    box.init(pc[0].X, pc[0].X, y_lo, y_hi, block_size % SPLATAD_WAVE == 0);
 
     const int32_t *offs = a.tile_offsets + (size_t)cam * tiles_per_cam;
     const int32_t range_start = offs[tile_id];
     const int32_t range_end = (cam == a.C - 1 && tile_id == tiles_per_cam - 1)
                                   ? (int32_t)a.n_isects
                                   : offs[tile_id + 1];
-    const uint32_t num_batches = (uint32_t)(range_end - range_start + block_size - 1) / block_size;
+    const uint32_t num_batches = (uint32_t)(range_end - range_start + batch - 1) / batch;
 
-    // footprint of this wavefront (all 64 lanes exist when the workgroup is a multiple of 64)
-    WaveCull cull;
-    cull.init(px, py, roll, block_size % SPLATAD_WAVE == 0);
-
-    float T = 1.0f;
-    uint32_t cur_idx = 0;
-    float out[CH];
+    float T[PPL], out[PPL][CH];
+    uint32_t cur_idx[PPL];
 #pragma unroll
-    for (int k = 0; k < CH; ++k) out[k] = 0.f;
+    for (int p = 0; p < PPL; ++p) {
+        T[p] = 1.0f;
+        cur_idx[p] = 0;
+#pragma unroll
+        for (int k = 0; k < CH; ++k) out[p][k] = 0.f;
+    }
 
-    uint32_t batches_done = 0;
+    // One Gaussian of the survivor strip for all pixels of the lane.  GENERAL: some Gaussian of
+    // the strip needs the 0.999 clamp or the sigma < 0 rule (see pixel_polynomial).
     uint32_t st_iter = 0, st_take = 0, st_alive = 0, st_idle = 0, st_tested = 0, st_kept = 0, st_valid = 0;
+    struct Survivor { float4 pa, pb, col; };
+    // the three reads of a strip entry are requested together, ahead of their use
+    auto fetch = [&](uint32_t k) {
+        Survivor s;
+        s.pa = s_list[LIST * k];
+        s.pb = s_list[LIST * k + 1]; // {cXY, cYY, list position (bits), L or +inf}
+        s.col = COPY ? s_list[LIST * k + 2] : make_float4(0.f, 0.f, 0.f, 0.f);
+        return s;
+    };
+    auto composite = [&](Survivor &s, uint32_t batch_start, auto general) {
+        constexpr bool GENERAL = decltype(general)::value;
+        const float4 pa = s.pa, pb = s.pb;
+        const float *col;
+        if (COPY) {
+            // the colours are in registers before the lanes part ways (the compiler would
+            // otherwise read them behind each pixel's decision and wait for the LDS there)
+            asm volatile("" : "+v"(s.col.x), "+v"(s.col.y), "+v"(s.col.z), "+v"(s.col.w));
+            col = reinterpret_cast<const float *>(&s.col);
+        } else {
+            const uint32_t slot = __float_as_uint(pb.z) - batch_start;
+            col = reinterpret_cast<const float *>(s_rec + (size_t)RECORD * slot + 2);
+        }
+        uint64_t any_alive = 0, any_take = 0;
+#pragma unroll
+        for (int p = 0; p < PPL; ++p) {
+            const float e = pixel_exponent(pa, pb.x, pb.y, pc[p]);
+            float alpha = __builtin_amdgcn_exp2f(e);
+            if (GENERAL) alpha = fminf(0.999f, alpha);
+            const float next_T = transmittance_behind(T[p], alpha);
+            // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
+            uint64_t valid_bits = alive_bits[p] & wave_ballot(!(alpha < 1.f / 255.f));
+            if (GENERAL) valid_bits &= wave_ballot(!(e > pb.w));
+            const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
+            const uint64_t take_bits = valid_bits & ~stop_bits;
+            if (STATS) {
+                st_alive += (uint32_t)__popcll(alive_bits[p]);
+                st_valid += (uint32_t)__popcll(valid_bits);
+                st_take += (uint32_t)__popcll(take_bits);
+                any_take |= take_bits;
+            }
+            alive_bits[p] &= ~stop_bits;
+            any_alive |= alive_bits[p];
+            if (wave_lanes(take_bits)) {
+                const float weight = alpha * T[p];
+#pragma unroll
+                for (int c = 0; c < CH; ++c) out[p][c] = fmaf(col[c], weight, out[p][c]);
+                T[p] = next_T;
+                cur_idx[p] = __float_as_uint(pb.z);
+            }
+        }
+        if (STATS) { st_iter += 1; st_idle += any_take == 0 ? 1u : 0u; }
+        return any_alive;
+    };
+    // walks the n survivors of the strip, two per trip so that the second one's reads are in
+    // flight while the first is composited; returns the lanes still alive
+    auto walk = [&](uint32_t n, uint32_t batch_start, uint64_t any_alive, auto general) {
+        uint32_t k = 0;
+        for (; k + 1 < n; k += 2) {
+            Survivor s0 = fetch(k), s1 = fetch(k + 1);
+            any_alive = composite(s0, batch_start, general);
+            if (any_alive == 0) return any_alive;
+            any_alive = composite(s1, batch_start, general);
+            if (any_alive == 0) return any_alive;
+        }
+        if (k < n) {
+            Survivor s0 = fetch(k);
+            any_alive = composite(s0, batch_start, general);
+        }
+        return any_alive;
+    };
+
+    // Staging reads.  Every load is unconditional (entries beyond the list repeat its last one,
+    // channels beyond the pass its last one), so that all of them are in flight together: two
+    // dependent round trips to memory per batch (id, then the Gaussian), hidden by the other
+    // workgroups of the compute unit.  (Requesting the next batch before compositing the current
+    // one costs 15 registers, one resident wavefront per SIMD with them, and was slower.)
+    struct Staged { float2 xy, vel; float cn[3], opac, col[CH]; };
+    auto id_of = [&](uint32_t b) -> int32_t {
+        const uint32_t idx = min((uint32_t)range_start + batch * b + tr, (uint32_t)range_end - 1u);
+        return b < num_batches ? a.flatten_ids[idx] : 0;
+    };
+    auto gather = [&](int32_t g) {
+        Staged s;
+        s.xy = reinterpret_cast<const float2 *>(a.means2d)[g];
+        s.vel = reinterpret_cast<const float2 *>(a.pix_vels)[g];
+        const float *c3 = a.conics + (size_t)g * 3;
+        s.cn[0] = c3[0]; s.cn[1] = c3[1]; s.cn[2] = c3[2];
+        s.opac = a.opacities[g];
+        const float *c = a.colors + (size_t)g * a.color_stride + a.ch_offset;
+#pragma unroll
+        for (int k = 0; k < CH; ++k) s.col[k] = STATS ? 0.f : c[min((uint32_t)k, a.n_ch - 1u)]; // STATS: no colours
+        return s;
+    };
+    uint32_t batches_done = 0;
     for (uint32_t b = 0; b < num_batches; ++b) {
         // also orders the previous batch's LDS reads before this batch's writes
-        if (__syncthreads_count(!wave_lanes(alive_bits)) >= (int)block_size) break;
+        bool lane_alive = false;
+#pragma unroll
+        for (int p = 0; p < PPL; ++p) lane_alive = lane_alive || wave_lanes(alive_bits[p]);
+        if (__syncthreads_count(!lane_alive) >= (int)block_size) break;
         batches_done = b + 1;
 
-        const uint32_t batch_start = (uint32_t)range_start + block_size * b;
-        const uint32_t idx = batch_start + tr;
-        if (idx < (uint32_t)range_end) {
-            const int32_t g = a.flatten_ids[idx];
-            const float2 xy = reinterpret_cast<const float2 *>(a.means2d)[g];
-            const float2 v = reinterpret_cast<const float2 *>(a.pix_vels)[g];
-            const float *cn = a.conics + (size_t)g * 3;
-            s_rec[RECORD * tr] = make_float4(xy.x, xy.y, v.x, v.y);
-            s_rec[RECORD * tr + 1] = staged_exponent(cn[0], cn[1], cn[2], a.opacities[g]);
-            const float *c = a.colors + (size_t)g * a.color_stride + a.ch_offset;
+        const uint32_t batch_start = (uint32_t)range_start + batch * b;
+        {
+            const Staged staged = gather(id_of(b));
+            float4 pa, pb;
+            pixel_polynomial(frame, staged.xy, staged.vel, staged.cn[0], staged.cn[1], staged.cn[2], staged.opac,
+                             pa, pb);
+            s_rec[RECORD * tr] = pa;
+            s_rec[RECORD * tr + 1] = pb;
 #pragma unroll
             for (int k = 0; k < CH; ++k)
-                reinterpret_cast<float *>(s_rec + RECORD * tr + 2)[k] = (uint32_t)k < a.n_ch ? c[k] : 0.f;
+                reinterpret_cast<float *>(s_rec + RECORD * tr + 2)[k] = (uint32_t)k < a.n_ch ? staged.col[k] : 0.f;
         }
         __syncthreads();
 
-        const uint32_t batch_size = min(block_size, (uint32_t)range_end - batch_start);
-        for (uint32_t base = 0; base < batch_size && alive_bits != 0; base += SPLATAD_WAVE) {
-            // lanes test 64 Gaussians against the wavefront's footprint, then all lanes walk
-            // the survivors (a wave-uniform loop over the set bits)
-            bool keep = base + lane < batch_size;
-            if (keep) keep = cull.may_touch(s_rec[RECORD * (base + lane)], s_rec[RECORD * (base + lane) + 1]);
-            uint64_t todo = wave_ballot(keep);
+        const uint32_t batch_size = min(batch, (uint32_t)range_end - batch_start);
+        uint64_t any_alive = 0;
+#pragma unroll
+        for (int p = 0; p < PPL; ++p) any_alive |= alive_bits[p];
+        for (uint32_t base = 0; base < batch_size && any_alive != 0; base += SPLATAD_WAVE) {
+            // lanes test 64 Gaussians against the wavefront's footprint ...
+            const uint32_t slot = base + lane;
+            bool keep = slot < batch_size;
+            float4 pa = make_float4(0.f, 0.f, 0.f, 0.f), pb = pa;
+            if (keep) {
+                pa = s_rec[RECORD * slot];
+                pb = s_rec[RECORD * slot + 1];
+                keep = box.may_touch(pa, pb);
+            }
+            const uint64_t todo = wave_ballot(keep);
+            const uint32_t n = (uint32_t)__popcll(todo);
             if (STATS) {
                 st_tested += min(batch_size - base, (uint32_t)SPLATAD_WAVE);
-                st_kept += (uint32_t)__popcll(todo);
+                st_kept += n;
             }
-            while (todo) {
-                const uint32_t t = base + (uint32_t)__ffsll((unsigned long long)todo) - 1u;
-                todo &= todo - 1;
-                const float4 *rec = s_rec + RECORD * t;
-                const float4 xyv = rec[0];
-                const float4 con = rec[1];
-                const float dx = gaussian_offset(xyv.x, xyv.z, roll, px);
-                const float dy = gaussian_offset(xyv.y, xyv.w, roll, py);
-                const float power = gaussian_power(con, dx, dy);
-                const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
-                const float weight = alpha * T;
-                const float next_T = transmittance_behind(T, alpha);
-                // same decisions as: skip if sigma < 0 or alpha < 1/255; stop if next_T <= 1e-4
-                const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
-                                            wave_ballot(!(alpha < 1.f / 255.f));
-                const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
-                const uint64_t take_bits = valid_bits & ~stop_bits;
-                if (STATS) {
-                    st_iter += 1;
-                    st_alive += (uint32_t)__popcll(alive_bits);
-                    st_valid += (uint32_t)__popcll(valid_bits);
-                    st_take += (uint32_t)__popcll(take_bits);
-                    st_idle += take_bits == 0 ? 1u : 0u;
-                }
-                alive_bits &= ~stop_bits;
-                const bool take = wave_lanes(take_bits);
-                const float vis = take ? weight : 0.f;
-                if (CH > 8 ? take_bits != 0 : true) {
-#pragma unroll
-                    for (int k = 0; k < CH; ++k) out[k] += reinterpret_cast<const float *>(rec + 2)[k] * vis;
-                }
-                cur_idx = take ? batch_start + t : cur_idx;
-                T -= vis;
-                if (alive_bits == 0) break;
+            if (n == 0) continue; // uniform
+            const bool general = wave_ballot(keep && !(pb.z == pb.z)) != 0; // uniform
+            // ... and copy the survivors into the wavefront's strip, in list order
+            if (keep) {
+                const uint32_t pos = (uint32_t)__popcll(todo & ((1ull << lane) - 1ull));
+                s_list[LIST * pos] = pa;
+                // .w: what the sigma < 0 rule compares with in a strip that needs it (for a plain
+                // Gaussian pb.w is the peak's row, not a bound)
+                s_list[LIST * pos + 1] = make_float4(pb.x, pb.y, __uint_as_float(batch_start + slot),
+                                                     pb.z == pb.z ? INFINITY : pb.w);
+                if (COPY) s_list[LIST * pos + 2] = s_rec[RECORD * slot + 2];
             }
+            // the strip is written and read by this wavefront only, whose LDS accesses execute in
+            // order; the fence keeps the compiler from moving the reads above the writes
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (!general) any_alive = walk(n, batch_start, any_alive, std::false_type{});
+            else any_alive = walk(n, batch_start, any_alive, std::true_type{});
+            // the next round overwrites the strip: its reads above are done (same wavefront)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
     }
 
-    if (a.tile_batches != nullptr && a.write_aux && tr == 0) a.tile_batches[blockIdx.x] = (int32_t)batches_done;
+    if (a.tile_batches != nullptr && a.write_aux && tr == 0)
+        a.tile_batches[blockIdx.x] = (int32_t)min(batches_done * batch, (uint32_t)(range_end - range_start));
     if (STATS) {
         if (lane == 0) {
-            const uint32_t v[kLaneStats] = {st_iter, st_take, st_alive, st_idle, st_tested, st_kept, 1u, st_valid};
+            const uint32_t v[kLaneStats] = {st_iter, st_take, st_alive, st_idle, st_tested, st_kept, (uint32_t)PPL, st_valid};
             for (int k = 0; k < kLaneStats; ++k) atomicAdd(a.lane_stats + k, (unsigned long long)v[k]);
         }
         return;
     }
-    if (inside) {
-        const size_t pix = ((size_t)cam * a.H + i) * a.W + j;
+#pragma unroll
+    for (int p = 0; p < PPL; ++p) {
+        if (!inside[p]) continue;
+        const size_t pix = ((size_t)cam * a.H + pi[p]) * a.W + pj;
         float *dst = a.render_colors + pix * a.color_stride + a.ch_offset;
         const float *bg = a.backgrounds ? a.backgrounds + (size_t)cam * a.color_stride + a.ch_offset : nullptr;
 #pragma unroll
         for (int k = 0; k < CH; ++k)
-            if ((uint32_t)k < a.n_ch) dst[k] = bg ? out[k] + T * bg[k] : out[k];
+            if ((uint32_t)k < a.n_ch) dst[k] = bg ? out[p][k] + T[p] * bg[k] : out[p][k];
         if (a.write_aux) {
-            a.render_alphas[pix] = 1.0f - T;
-            a.last_ids[pix] = (int32_t)cur_idx;
+            a.render_alphas[pix] = 1.0f - T[p];
+            a.last_ids[pix] = (int32_t)cur_idx[p];
         }
     }
 }
@@ -444,7 +574,8 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
         }
     }
 
-    if (a.tile_batches != nullptr && a.write_aux && tr == 0) a.tile_batches[blockIdx.x] = (int32_t)batches_done;
+    if (a.tile_batches != nullptr && a.write_aux && tr == 0)
+        a.tile_batches[blockIdx.x] = (int32_t)min(batches_done * block_size, (uint32_t)(range_end - range_start));
     if constexpr (MATRIX) {
         if (pair_open) add_pair(pair_weight, 0.f, pair_feature, 0.f);
         // what the D layout needs to know of a point: where it is stored, its transmittance
@@ -505,15 +636,33 @@ static inline int pick_width(uint32_t n) {
     return -1;
 }
 
+// Two pixels per lane where the tile makes whole wavefronts of 8 x 16 pixels.
+static inline int pixels_per_lane(uint32_t tile_size) {
+    return tile_size % 8 == 0 && (tile_size * tile_size / 2) % SPLATAD_WAVE == 0 ? 2 : 1;
+}
+
 template <int CH>
-static int launch_pixels(const PixelArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
-    const size_t lds = (size_t)block.x * block.y * 16 * (2 + (CH + 3) / 4);
+static size_t pixel_lds_bytes(uint32_t threads) {
+    const size_t waves = (threads + SPLATAD_WAVE - 1) / SPLATAD_WAVE;
+    return 16 * ((size_t)threads * (2 + (CH + 3) / 4) + waves * SPLATAD_WAVE * (CH <= 4 ? 3 : 2));
+}
+
+template <int CH, int PPL, bool STATS>
+static int launch_pixels_as(const PixelArgs &a, dim3 grid, uint32_t threads, hipStream_t stream) {
+    const size_t lds = pixel_lds_bytes<CH>(threads);
     if (lds > 64 * 1024)
-        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_to_pixels_fwd_kernel<CH>,
+        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_to_pixels_fwd_kernel<CH, PPL, STATS>,
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(rasterize_to_pixels_fwd_kernel<CH>, grid, block, lds, stream, a);
+    hipLaunchKernelGGL((rasterize_to_pixels_fwd_kernel<CH, PPL, STATS>), grid, dim3(threads), lds, stream, a);
     SPLATAD_LAUNCH_CHECK();
     return 0;
+}
+
+template <int CH>
+static int launch_pixels(const PixelArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
+    const uint32_t pixels = block.x * block.y;
+    if (pixels_per_lane(a.tile_size) == 2) return launch_pixels_as<CH, 2, false>(a, grid, pixels / 2, stream);
+    return launch_pixels_as<CH, 1, false>(a, grid, pixels, stream);
 }
 
 template <int CH>
@@ -626,11 +775,10 @@ extern "C" int splatad_rasterize_to_pixels_lane_stats(
     a.W = W; a.H = H; a.tile_size = tile_size; a.tile_w = tile_w; a.tile_h = tile_h;
     a.tile_offsets = tile_offsets; a.flatten_ids = flatten_ids;
     a.lane_stats = stats;
-    const dim3 grid(C * tile_w * tile_h), block(tile_size, tile_size);
-    const size_t lds = (size_t)block.x * block.y * 16 * 3;
-    hipLaunchKernelGGL((rasterize_to_pixels_fwd_kernel<1, true>), grid, block, lds, (hipStream_t)stream, a);
-    SPLATAD_LAUNCH_CHECK();
-    return 0;
+    const dim3 grid(C * tile_w * tile_h);
+    const uint32_t pixels = tile_size * tile_size;
+    if (pixels_per_lane(tile_size) == 2) return launch_pixels_as<1, 2, true>(a, grid, pixels / 2, (hipStream_t)stream);
+    return launch_pixels_as<1, 1, true>(a, grid, pixels, (hipStream_t)stream);
 }
 
 extern "C" int splatad_rasterize_to_points_fwd(

@@ -696,7 +696,7 @@ class _Ops:
                                 rolling_shutter_time, backgrounds, image_width, image_height,
                                 tile_size, tile_offsets, flatten_ids, tile_batches=None):
         """tile_batches: optional int32 [C, tile_height, tile_width] tensor that receives the number
-        of list batches every tile went through (a diagnostic, not part of the reference's op)."""
+        of list entries every tile staged (a diagnostic, not part of the reference's op)."""
         lib = load_library()
         means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
         colors = _in(colors, "colors"); opacities = _in(opacities, "opacities")
