@@ -25,11 +25,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch of the two compositing kernels on the default workloads, from
 # `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this file (KiB per dispatch,
 # scaled by what the same counters read for a 1 GiB device-to-device copy: FETCH_SIZE reads
-# 0.5 KiB per KiB, WRITE_SIZE 1.0).  Summaries: profiles/rasterize_kernels_counters_1M.txt.
+# 0.5 KiB per KiB, WRITE_SIZE 1.0).  Summaries: profiles/kernels_counters_camera_1M_1080p_lidar_128x2048.txt.
 # They describe the 1M-Gaussian default only; other sizes report null.
 MEASURED_TRAFFIC_BYTES = {
-    "camera": int((12972.4 * 2.0 + 48617.6) * 1024),
-    "lidar": int((26317.1 * 2.0 + 40989.5) * 1024),
+    "camera": int((9527.2 * 2.0 + 48612.3) * 1024),
+    "lidar": int((26294.5 * 2.0 + 40927.0) * 1024),
 }
 
 
@@ -71,6 +71,20 @@ def staged_isects(tile_entries):
     """List entries the compositing kernel staged: whole batches until every pixel / point of a
     tile has saturated, clipped to the tile's list, as counted by the kernel itself."""
     return int(tile_entries.sum().item())
+
+
+def stage_rooflines(leg):
+    """Per stage of a forward call: event-timed duration of the stage's launches in isolation, the
+    bytes any implementation of the stage has to move, and what that makes of the HBM peak."""
+    out = {}
+    for k, ms in leg["stages"].items():
+        b = leg["stage_bytes"].get(k)
+        if b is None:
+            continue
+        gbs = b / (ms * 1e-3) / 1e9
+        out[k[:-3]] = {"ms": round(ms, 4), "algorithmic_bytes": int(b), "achieved_GBps": round(gbs, 1),
+                       "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+    return out
 
 
 def bench_camera(args):
@@ -132,15 +146,35 @@ def bench_camera(args):
         isect = lambda: _C.isect_tiles(meta["means2d"], meta["radii"], meta["depths"], None, None, C,
                                        ts, meta["tile_width"], meta["tile_height"], True, True)
         stages["isect_sort_ms"] = time_kernel(isect, 5)
+        # on a copy: the tensor returned by isect_tiles carries the table the binning made
+        ids_copy = meta["isect_ids"].clone()
         stages["offset_encode_ms"] = time_kernel(
-            lambda: _C.isect_offset_encode(meta["isect_ids"], C, meta["tile_width"], meta["tile_height"]), 5)
+            lambda: _C.isect_offset_encode(ids_copy, C, meta["tile_width"], meta["tile_height"]), 5)
         stages["view_colors_ms"] = time_kernel(
             lambda: _C.view_colors_fwd(3, s["means"], s["viewmats"], None, None, meta["radii"],
                                        s["colors"], meta["depths"]), 5)
         stages["rasterize_ms"] = k_ms
+        nnz = int((meta["radii"][..., 0] > 0).sum().item())
+        N, K = s["means"].shape[0], s["colors"].shape[-2]
+        stage_bytes = {
+            "projection_ms": N * 52 + C * N * 40,
+            # what any implementation has to move: read the projected (mean, radii, depth) rows, write
+            # a key and an id per intersection and the offsets
+            "isect_sort_ms": C * N * 20 + n_isects * 12 + T * 4,
+            "offset_encode_ms": n_isects * 8 + T * 4,
+            "view_colors_ms": nnz * (12 + 12 * K + 1 + 12),
+            "rasterize_ms": alg_bytes,
+        }
+        st = _C.rasterize_to_pixels_lane_stats(
+            meta["means2d"], meta["conics"], meta["opacities"], meta["pix_vels"], s["rolling_shutter_time"], W, H,
+            ts, meta["isect_offsets"], meta["flatten_ids"]).tolist()
+        lanes = dict(iterations=st[0], pixels_per_lane=st[6],
+                     compositing_lane_fraction=st[1] / max(1, st[0] * 64 * st[6]),
+                     footprint_test_pass_fraction=st[5] / max(1, st[4]),
+                     iterations_without_a_compositing_lane=st[3] / max(1, st[0]))
     return dict(sec=sec, sec_packed=sec_packed, pixels=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
-                n_isects=n_isects, i_need=i_need, nnz=int((meta["radii"][..., 0] > 0).sum().item()),
-                stages=stages, channels=D)
+                n_isects=n_isects, i_need=i_need, nnz=nnz, stages=stages, stage_bytes=stage_bytes,
+                channels=D, lanes=lanes)
 
 
 def bench_lidar(args):
@@ -204,8 +238,12 @@ def bench_lidar(args):
             s["tile_elevation_boundaries"], s["azimuth_resolution"] * s["tile_width"], s["min_azimuth"],
             True, True), 5)
         stages["rasterize_ms"] = k_ms
+        N = s["means"].shape[0]
+        stage_bytes = {"projection_ms": N * 52 + C * N * 52,
+                       "isect_sort_ms": C * N * 20 + n_isects * 12 + T * 4,
+                       "rasterize_ms": alg_bytes}
     return dict(sec=sec, sec_chunk32=sec_chunk32, points=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
-                n_isects=n_isects, i_need=i_need, channels=D, stages=stages)
+                n_isects=n_isects, i_need=i_need, channels=D, stages=stages, stage_bytes=stage_bytes)
 
 
 def bench_backward(args):
@@ -256,6 +294,53 @@ def bench_backward(args):
             t.grad = None
 
     out["lidar_fwd_bwd_ms"] = time_steps(lidar_step, max(3, args.steps // 2), 2) * 1e3
+
+    # the compositing backward in isolation: gradient of the compositing call alone with respect
+    # to its per-Gaussian inputs (kernels, clearing and unpacking of the gradient records), on
+    # the forward call's own lists
+    from splatad_amd.hip import _wrapper as ops
+
+    def leaves(*ts):
+        return [t.detach().clone().requires_grad_(True) for t in ts]
+
+    with torch.no_grad():
+        _, ra, _, meta = lidar_rasterization(
+            l["means"], l["quats"], l["scales"], l["opacities"], l["lidar_features"], l["velocities"],
+            l["viewmats"], l["raster_pts"], l["tile_elevation_boundaries"], l["linear_velocity"],
+            l["angular_velocity"], l["rolling_shutter_time"], min_azimuth=l["min_azimuth"],
+            max_azimuth=l["max_azimuth"], min_elevation=l["min_elevation"], max_elevation=l["max_elevation"],
+            n_elevation_channels=l["n_elevation_channels"], azimuth_resolution=l["azimuth_resolution"],
+            tile_width=l["tile_width"], tile_height=l["tile_height"], near_plane=l["near_plane"],
+            far_plane=l["far_plane"], eps2d=l["eps2d"], channel_chunk=33)
+        from splatad_amd.hip._backend import _C
+        dcomp = _C.fully_fused_lidar_projection_fwd(
+            l["means"], None, l["quats"], l["scales"], l["velocities"], l["viewmats"], l["min_elevation"],
+            l["max_elevation"], l["min_azimuth"], l["max_azimuth"], l["linear_velocity"], l["angular_velocity"],
+            l["rolling_shutter_time"], l["eps2d"], l["near_plane"], l["far_plane"], 0.0, False)[6]
+    H, W = ra.shape[1:3]
+    ins = leaves(meta["means2d"], meta["conics"], l["lidar_features"], meta["opacities"], meta["depths"])
+    rf, ra, asum, med = ops.rasterize_to_points(
+        ins[0], ins[1], ins[2], ins[3], meta["pix_vels"], dcomp, l["raster_pts"], W, H,
+        l["tile_width"], l["tile_height"], meta["isect_offsets"], meta["flatten_ids"], True, 0.2, ranges=ins[4])
+    loss = rf.abs().mean() + ra.mean()
+    out["lidar_rasterize_bwd_ms"] = time_kernel(lambda: torch.autograd.grad(loss, ins, retain_graph=True), 5)
+    del l, q, ins, rf, ra, asum, med, loss, meta
+
+    s = workloads.to_device(workloads.camera_driving(n=args.n), dev)
+    with torch.no_grad():
+        _, _, meta = rasterization(
+            s["means"], s["quats"], s["scales"], s["opacities"], s["colors"], s["velocities"], s["viewmats"],
+            s["Ks"], s["width"], s["height"], s["linear_velocity"], s["angular_velocity"],
+            s["rolling_shutter_time"], sh_degree=s["sh_degree"], packed=False, render_mode="RGB+D",
+            near_plane=s["near_plane"], far_plane=s["far_plane"], eps2d=s["eps2d"], tile_size=s["tile_size"])
+        cols = torch.rand((1, s["means"].shape[0], 4), device=dev)
+        target = torch.rand((1, s["height"], s["width"], 4), device=dev)
+    ins = leaves(meta["means2d"], meta["conics"], cols, meta["opacities"])
+    rc, ra = ops.rasterize_to_pixels(
+        ins[0], ins[1], ins[2], ins[3], meta["pix_vels"], s["width"], s["height"], s["tile_size"],
+        meta["isect_offsets"], meta["flatten_ids"], rolling_shutter_time=s["rolling_shutter_time"])
+    loss = (rc - target).abs().mean() + ra.mean()
+    out["camera_rasterize_bwd_ms"] = time_kernel(lambda: torch.autograd.grad(loss, ins, retain_graph=True), 5)
     return out
 
 
@@ -350,9 +435,11 @@ def main():
             "n_isects": cam["n_isects"], "n_isects_consumed": cam["i_need"],
             "visible_gaussians": cam["nnz"], "ms_per_step_packed": cam["sec_packed"] * 1e3,
             "stage_ms": {k: round(v, 4) for k, v in cam["stages"].items()},
+            "lane_utilisation": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in cam["lanes"].items()},
         },
+        "stages": stage_rooflines(cam),
         "roofline": {
-            "kernel": "rasterize_to_pixels_fwd_kernel<%d>" % cam["channels"],
+            "kernel": "rasterize_to_pixels_fwd_kernel<%d, 2, false>" % cam["channels"],
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": MEASURED_TRAFFIC_BYTES["camera"] if args.n == 1_000_000 else None,
@@ -369,6 +456,7 @@ def main():
                         "channel_chunk=33 (BASELINE configs[2])" % args.n,
             "n_isects": lid["n_isects"], "n_isects_consumed": lid["i_need"],
             "stage_ms": {k: round(v, 4) for k, v in lid["stages"].items()},
+            "stages": stage_rooflines(lid),
             "roofline": {"kernel": "rasterize_to_points_fwd_kernel<%d, %s>" % (lid["channels"], "true" if lid["channels"] in (32, 33) else "false"),
                          "bound": "hbm", "achieved": l_ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": l_ach / HBM_PEAK_GBS,
@@ -376,7 +464,7 @@ def main():
                          "algorithmic_bytes": lid["alg_bytes"], "kernel_ms": lid["kernel_ms"]},
         }
     if not args.no_bwd:
-        out["config"].update({k: round(v, 4) for k, v in bench_backward(args).items()})
+        out["backward"] = {k: round(v, 4) for k, v in bench_backward(args).items()}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_camera(args)
     print(json.dumps(out))

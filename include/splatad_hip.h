@@ -289,9 +289,11 @@ int splatad_rasterize_to_pixels_fwd(uint32_t C, int64_t n_isects, uint32_t chann
 /* Diagnostic without a counterpart in the reference: lane utilisation of the compositing loop
  * of splatad_rasterize_to_pixels_fwd on the same inputs (nothing is rendered).  Adds to eight
  * counters in stats (zero them first): [0] (wavefront, Gaussian) iterations of the inner loop,
- * [1] lanes that composited their Gaussian, summed over the iterations, [2] lanes still alive,
- * [3] iterations in which no lane composited, [4] list entries tested against a wavefront's
- * footprint, [5] entries that passed the test, [6] wavefronts, [7] lanes with alpha >= 1/255. */
+ * [1] pixels that composited their Gaussian, summed over the iterations, [2] pixels still
+ * alive, [3] iterations in which no pixel composited, [4] list entries tested against a
+ * wavefront's footprint, [5] entries that passed the test, [6] (stored, not added) pixels per
+ * lane of the kernel that ran, so that an iteration offers 64 * [6] pixels, [7] pixels with
+ * alpha >= 1/255. */
 int splatad_rasterize_to_pixels_lane_stats(uint32_t C, int64_t n_isects, const float *means2d,
                                            const float *conics, const float *opacities,
                                            const float *pix_vels,

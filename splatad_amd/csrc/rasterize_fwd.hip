@@ -290,8 +290,10 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
         a.tile_batches[blockIdx.x] = (int32_t)min(batches_done * batch, (uint32_t)(range_end - range_start));
     if (STATS) {
         if (lane == 0) {
-            const uint32_t v[kLaneStats] = {st_iter, st_take, st_alive, st_idle, st_tested, st_kept, (uint32_t)PPL, st_valid};
-            for (int k = 0; k < kLaneStats; ++k) atomicAdd(a.lane_stats + k, (unsigned long long)v[k]);
+            const uint32_t v[kLaneStats] = {st_iter, st_take, st_alive, st_idle, st_tested, st_kept, 0u, st_valid};
+            for (int k = 0; k < kLaneStats; ++k)
+                if (k != 6) atomicAdd(a.lane_stats + k, (unsigned long long)v[k]);
+            if (blockIdx.x == 0 && tr == 0) a.lane_stats[6] = (unsigned long long)PPL;
         }
         return;
     }
