@@ -873,6 +873,167 @@ __device__ __forceinline__ void sort_segment(uint32_t seg, uint32_t n_segments, 
     }
 }
 
+// The same sort for the short segments (n <= lds_words <= 8192, n <= ER * blockDim.x), shaped
+// for the latency of its LDS accesses, which bounds the generic version above:
+//  * an entry's bucket is computed once, kept in a register for the scatter, and written as
+//    16 bits beside the entry's staging position for the rank step;
+//  * the rank loop takes four staged entries per trip with no bounds test: what follows a
+//    bucket in the staging array belongs to later buckets, whose depth bits are strictly larger
+//    (the bucket is a non-decreasing function of the depth bits), and four words of all ones
+//    follow the segment's last entry, so an entry read beyond the bucket never counts;
+//  * without TIES the keys (depth bits, flatten id) of a segment are distinct and one 64-bit
+//    comparison decides; TIES (lidar: a rectangle wider than the grid lists a tile twice) orders
+//    equal keys by staging position.
+// Dynamic LDS: (lds_words + 4) * 8 bytes of staging, the fine bins, 2 * bucket_cap + 1
+// counters, lds_words * 2 bytes of bucket indices.
+__host__ __device__ inline size_t sort_small_lds_bytes(uint32_t lds_words, uint32_t bucket_cap) {
+    return ((size_t)lds_words + 4) * 8 + (kSortFineBins + 2 * (size_t)bucket_cap + 1) * 4 +
+           (((size_t)lds_words * 2 + 7) & ~(size_t)7);
+}
+
+template <int ER, bool TIES>
+__device__ __forceinline__ void sort_segment_small(uint32_t seg, uint32_t n_segments, uint32_t n_tiles,
+                                                   uint32_t sshift, uint32_t tile_n_bits, uint32_t lds_words,
+                                                   uint32_t bucket_cap, int64_t n_isects,
+                                                   const int32_t *__restrict__ tile_starts,
+                                                   const uint64_t *__restrict__ pairs,
+                                                   int64_t *__restrict__ isect_ids,
+                                                   int32_t *__restrict__ flatten_ids,
+                                                   uint64_t *lds_staged, uint32_t *s_wave, uint32_t &s_big) {
+    const int64_t start = tile_starts[seg];
+    const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
+    const uint32_t n = (uint32_t)(stop - start);
+    uint32_t *s_fine = reinterpret_cast<uint32_t *>(lds_staged + lds_words + 4);
+    uint32_t *s_first = s_fine + kSortFineBins;   // bucket_cap + 1 words: starts, then the end
+    uint32_t *s_cursor = s_first + bucket_cap + 1;
+    uint16_t *s_bucket = reinterpret_cast<uint16_t *>(s_cursor + bucket_cap);
+    const uint64_t *g = pairs + start;
+    int64_t *ids_out = isect_ids + start;
+    int32_t *flat_out = flatten_ids + start;
+    const uint32_t tid = threadIdx.x, nt = blockDim.x;
+    const uint32_t lane = tid & (SPLATAD_WAVE - 1), wave = tid / SPLATAD_WAVE;
+    const uint32_t n_waves = nt / SPLATAD_WAVE;
+    const uint64_t cam = (seg >> sshift) / n_tiles, tile = (seg >> sshift) % n_tiles;
+    const uint64_t key_hi = ((cam << tile_n_bits) | tile) << 32;
+
+    uint64_t held[ER];
+#pragma unroll
+    for (int k = 0; k < ER; ++k) {
+        const uint32_t i = tid + k * nt;
+        held[k] = i < n ? g[i] : ~0ull;
+    }
+    uint32_t lo = 0xFFFFFFFFu, hi = 0u;
+#pragma unroll
+    for (int k = 0; k < ER; ++k)
+        if (tid + k * nt < n) {
+            const uint32_t d = (uint32_t)(held[k] >> 32);
+            lo = min(lo, d);
+            hi = max(hi, d);
+        }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        lo = min(lo, (uint32_t)__shfl_xor((int)lo, off, SPLATAD_WAVE));
+        hi = max(hi, (uint32_t)__shfl_xor((int)hi, off, SPLATAD_WAVE));
+    }
+    if (lane == 0) { s_wave[2 * wave] = lo; s_wave[2 * wave + 1] = hi; }
+    if (tid == 0) s_big = 0;
+    if (tid < 4) lds_staged[n + tid] = ~0ull;
+    uint32_t n_fine = 1;
+    while (n_fine < kSortFineBins && n_fine * 16 < n) n_fine <<= 1;
+    for (uint32_t f = tid; f < n_fine; f += nt) s_fine[f] = 0;
+    __syncthreads();
+    for (uint32_t w = 0; w < n_waves; ++w) {
+        lo = min(lo, s_wave[2 * w]);
+        hi = max(hi, s_wave[2 * w + 1]);
+    }
+    const float scale = (float)n_fine / ((float)(hi - lo) + 1.f);
+    auto fine_pos = [&](uint64_t p, uint32_t &f) -> float {
+        const float x = (float)((uint32_t)(p >> 32) - lo) * scale;
+        f = min(n_fine - 1, (uint32_t)x);
+        return x;
+    };
+    __syncthreads(); // s_wave is reused by the scans
+
+#pragma unroll
+    for (int k = 0; k < ER; ++k)
+        if (tid + k * nt < n) {
+            uint32_t f;
+            fine_pos(held[k], f);
+            atomicAdd(&s_fine[f], 1u);
+        }
+    __syncthreads();
+
+    const uint32_t mean = kSortBucketMean;
+    const uint32_t nb = block_exclusive_scan(
+        n_fine, tid, nt, s_wave,
+        [&](uint32_t f) { return (s_fine[f] + mean - 1) / mean; },
+        [&](uint32_t f, uint32_t before, uint32_t v) { s_fine[f] = before | (v << 16); });
+    for (uint32_t b = tid; b < nb; b += nt) s_cursor[b] = 0;
+    __syncthreads();
+    uint32_t bucket[ER];
+#pragma unroll
+    for (int k = 0; k < ER; ++k) {
+        bucket[k] = 0;
+        if (tid + k * nt < n) {
+            uint32_t f;
+            const float x = fine_pos(held[k], f);
+            const uint32_t packed = s_fine[f];
+            const uint32_t c = packed >> 16;
+            bucket[k] = (packed & 0xFFFFu) + min(c - 1, (uint32_t)((x - (float)f) * (float)c));
+            atomicAdd(&s_cursor[bucket[k]], 1u);
+        }
+    }
+    __syncthreads();
+    block_exclusive_scan(
+        nb, tid, nt, s_wave, [&](uint32_t b) { return s_cursor[b]; },
+        [&](uint32_t b, uint32_t before, uint32_t v) {
+            s_cursor[b] = before;
+            s_first[b] = before;
+            if (v > kSortRankMax) s_big = 1;
+        });
+    if (tid == 0) s_first[nb] = n;
+#pragma unroll
+    for (int k = 0; k < ER; ++k)
+        if (tid + k * nt < n) {
+            const uint32_t at = atomicAdd(&s_cursor[bucket[k]], 1u);
+            lds_staged[at] = held[k];
+            s_bucket[at] = (uint16_t)bucket[k];
+        }
+    __syncthreads();
+
+    if (s_big) { // uniform: more than 1024 entries in a bucket, i.e. that many equal depths
+        for (uint32_t b = 0; b < nb; ++b) {
+            const uint32_t s0 = s_first[b], c = s_first[b + 1] - s0;
+            if (c > kSortRankMax) bitonic_sort_ascending(lds_staged + s0, c, tid, nt); // uniform
+        }
+    }
+
+    for (uint32_t i = tid; i < n; i += nt) {
+        const uint64_t p = lds_staged[i];
+        const uint32_t b = s_bucket[i];
+        const uint32_t s0 = s_first[b], s1 = s_first[b + 1];
+        uint32_t place = s0;
+        if (s1 - s0 > kSortRankMax) {
+            place = i; // ordered by the network above
+        } else {
+            for (uint32_t j = s0; j < s1; j += 4) {
+                const uint64_t q0 = lds_staged[j], q1 = lds_staged[j + 1];
+                const uint64_t q2 = lds_staged[j + 2], q3 = lds_staged[j + 3];
+                if (TIES) {
+                    place += (q0 < p || (q0 == p && j < i)) ? 1u : 0u;
+                    place += (q1 < p || (q1 == p && j + 1 < i)) ? 1u : 0u;
+                    place += (q2 < p || (q2 == p && j + 2 < i)) ? 1u : 0u;
+                    place += (q3 < p || (q3 == p && j + 3 < i)) ? 1u : 0u;
+                } else {
+                    place += (q0 < p ? 1u : 0u) + (q1 < p ? 1u : 0u) + (q2 < p ? 1u : 0u) + (q3 < p ? 1u : 0u);
+                }
+            }
+        }
+        ids_out[place] = (int64_t)(key_hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
+        flat_out[place] = (int32_t)(uint32_t)p;
+    }
+}
+
 // Size classes of the segment sort: class c holds the segments with kSortClassMin[c] < n <=
 // kSortClassMin[c + 1]; the host launches one kernel configuration per class.
 constexpr int kSortClasses = 7;
@@ -917,23 +1078,24 @@ isect_classify_segments_kernel(uint32_t n_segments, uint32_t sshift, int64_t n_i
 
 // The workgroups of a launch share out the segments of one class; a launch has no more
 // workgroups than can be resident, so a class without segments costs next to nothing.
-template <int ER, bool IN_LDS>
-__global__ void isect_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t sshift,
-                                          uint32_t tile_n_bits, uint32_t lds_words,
-                                          uint32_t bucket_cap, int64_t n_isects,
-                                          const uint32_t *__restrict__ seg_count,
-                                          const uint32_t *__restrict__ seg_list,
-                                          const int32_t *__restrict__ tile_starts,
-                                          const uint64_t *__restrict__ pairs, int64_t *isect_ids,
-                                          int32_t *__restrict__ flatten_ids) {
+template <int ER, bool TIES>
+__global__ void isect_small_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t sshift,
+                                                uint32_t tile_n_bits, uint32_t lds_words,
+                                                uint32_t bucket_cap, int64_t n_isects,
+                                                const uint32_t *__restrict__ seg_count,
+                                                const uint32_t *__restrict__ seg_list,
+                                                const int32_t *__restrict__ tile_starts,
+                                                const uint64_t *__restrict__ pairs,
+                                                int64_t *__restrict__ isect_ids,
+                                                int32_t *__restrict__ flatten_ids) {
     extern __shared__ uint64_t lds_staged[];
     __shared__ uint32_t s_wave[2 * (1024 / SPLATAD_WAVE)];
     __shared__ uint32_t s_big;
     const uint32_t count = *seg_count;
     for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) { // uniform across the workgroup
-        sort_segment<ER, IN_LDS>(seg_list[k], n_segments, n_tiles, sshift, tile_n_bits, lds_words, bucket_cap,
-                                 n_isects, tile_starts, pairs, isect_ids, flatten_ids, lds_staged,
-                                 s_wave, s_big);
+        sort_segment_small<ER, TIES>(seg_list[k], n_segments, n_tiles, sshift, tile_n_bits, lds_words,
+                                     bucket_cap, n_isects, tile_starts, pairs, isect_ids, flatten_ids,
+                                     lds_staged, s_wave, s_big);
         __syncthreads(); // the next segment reuses the LDS
     }
 }
@@ -1006,29 +1168,29 @@ static int launch_big_segment_sort(uint32_t workgroups, uint32_t segs, uint32_t 
     return 0;
 }
 
-template <int ER, bool IN_LDS>
-static int launch_segment_sort(int cls, uint32_t threads, uint32_t max_n, uint32_t workgroups,
-                               uint32_t segs, uint32_t n_tiles, uint32_t sshift, uint32_t tile_n_bits,
-                               int64_t n_isects, const uint32_t *seg_counts,
-                               const uint32_t *seg_lists, const int32_t *tile_starts,
-                               const uint64_t *pairs, int64_t *isect_ids, int32_t *flatten_ids,
-                               hipStream_t stream) {
-    const uint32_t lds_words = IN_LDS ? max_n : kSortWindow;
+template <int ER, bool TIES>
+static int launch_small_segment_sort(int cls, uint32_t threads, uint32_t max_n, uint32_t workgroups,
+                                     uint32_t segs, uint32_t n_tiles, uint32_t sshift, uint32_t tile_n_bits,
+                                     int64_t n_isects, const uint32_t *seg_counts,
+                                     const uint32_t *seg_lists, const int32_t *tile_starts,
+                                     const uint64_t *pairs, int64_t *isect_ids, int32_t *flatten_ids,
+                                     hipStream_t stream) {
+    SPLATAD_REQUIRE((uint64_t)ER * threads >= max_n && max_n <= 8192u, "segment sort: class %d does not fit", cls);
     const uint32_t bucket_cap = sort_bucket_capacity(max_n);
-    const size_t lds_bytes = (size_t)lds_words * 8 + (kSortFineBins + 2 * (size_t)bucket_cap) * 4;
+    const size_t lds_bytes = sort_small_lds_bytes(max_n, bucket_cap);
     {   // raise the kernel's dynamic LDS limit once per instantiation and size
         static std::mutex guard;
         static size_t allowed = 0;
         std::lock_guard<std::mutex> lock(guard);
         if (lds_bytes > allowed) {
             SPLATAD_CHECK_HIP(hipFuncSetAttribute(
-                (const void *)isect_segment_sort_kernel<ER, IN_LDS>,
+                (const void *)isect_small_segment_sort_kernel<ER, TIES>,
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
             allowed = lds_bytes;
         }
     }
-    hipLaunchKernelGGL((isect_segment_sort_kernel<ER, IN_LDS>), dim3(workgroups < segs ? workgroups : segs),
-                       dim3(threads), lds_bytes, stream, segs, n_tiles, sshift, tile_n_bits, lds_words,
+    hipLaunchKernelGGL((isect_small_segment_sort_kernel<ER, TIES>), dim3(workgroups < segs ? workgroups : segs),
+                       dim3(threads), lds_bytes, stream, segs, n_tiles, sshift, tile_n_bits, max_n,
                        bucket_cap, n_isects, seg_counts + cls, seg_lists + (size_t)cls * segs,
                        tile_starts, pairs, isect_ids, flatten_ids);
     SPLATAD_LAUNCH_CHECK();
@@ -1395,20 +1557,20 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     // them reads and writes the caller's buffers, so the caller's stream must not run past it.
     auto enqueue_sorts = [&]() -> int {
         int e;
-#define SPLATAD_SORT_CLASS(cls, ER, IN_LDS, threads, hi, wgs, on)                                \
-        if ((e = launch_segment_sort<ER, IN_LDS>(cls, threads, hi, wgs, nseg, n_tiles, sshift, tile_n_bits, \
-                                                 n_isects, w.seg_counts, w.seg_lists, w.tile_starts, \
-                                                 w.pairs, isect_ids, flatten_ids, on)) != 0)      \
+#define SPLATAD_SORT_CLASS(cls, ER, threads, hi, wgs, on)                                        \
+        if ((e = launch_small_segment_sort<ER, LIDAR>(cls, threads, hi, wgs, nseg, n_tiles, sshift, tile_n_bits, \
+                                                      n_isects, w.seg_counts, w.seg_lists, w.tile_starts, \
+                                                      w.pairs, isect_ids, flatten_ids, on)) != 0) \
             return e;
         // the upper classes go first, on the caller's stream, which does not wait for the fork
         if ((e = launch_big_segment_sort(256u, nseg, n_tiles, sshift, tile_n_bits, n_isects, w.seg_counts,
                                          w.seg_lists, w.tile_starts, w.pairs, isect_ids, flatten_ids,
                                          stream)) != 0)
             return e;
-        SPLATAD_SORT_CLASS(2, 8, true, 512, 4096u, 1024u, ss->aux[0])
-        SPLATAD_SORT_CLASS(3, 8, true, 1024, 8192u, 512u, ss->aux[1])
-        SPLATAD_SORT_CLASS(1, 8, true, 256, 2048u, 2048u, stream)
-        SPLATAD_SORT_CLASS(0, 4, true, 128, 512u, 4096u, stream)
+        SPLATAD_SORT_CLASS(2, 8, 512, 4096u, 1024u, ss->aux[0])
+        SPLATAD_SORT_CLASS(3, 8, 1024, 8192u, 512u, ss->aux[1])
+        SPLATAD_SORT_CLASS(1, 8, 256, 2048u, 2048u, stream)
+        SPLATAD_SORT_CLASS(0, 4, 128, 512u, 4096u, stream)
 #undef SPLATAD_SORT_CLASS
         return 0;
     };
