@@ -460,6 +460,47 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
     }
 }
 
+// Size classes of the segment sort: class c holds the segments with kSortClassMin[c] < n <=
+// kSortClassMin[c + 1]; the host launches one kernel configuration per class.
+constexpr int kSortClasses = 7;
+__constant__ const uint32_t kSortClassMin[kSortClasses + 1] = {0u,    512u,   2048u,  4096u,
+                                                               8192u, 16384u, 32768u, 0x7FFFFFFFu};
+
+// Enters segment `seg` (one per lane; lanes beyond n_segments idle) into the list of its size
+// class: seg_lists[c * n_segments + k], k < seg_counts[c] (zeroed beforehand).  The order inside
+// a class is whatever the atomics give; every segment is sorted on its own, so the result does
+// not depend on it.  Also writes the tile offsets: a tile's offset is the start of its segment
+// (with depth slabs: of its first slab's), the first row of the scanned table.
+__device__ __forceinline__ void classify_segment(uint32_t seg, uint32_t lane, uint32_t n_segments,
+                                                 uint32_t sshift, int64_t n_isects,
+                                                 const int32_t *__restrict__ tile_starts,
+                                                 uint32_t *__restrict__ seg_counts,
+                                                 uint32_t *__restrict__ seg_lists,
+                                                 int32_t *__restrict__ tile_offsets) {
+    uint32_t n = 0;
+    if (seg < n_segments) {
+        const int64_t start = tile_starts[seg];
+        const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
+        n = (uint32_t)(stop - start);
+        if (tile_offsets != nullptr && (seg & ((1u << sshift) - 1u)) == 0)
+            tile_offsets[seg >> sshift] = (int32_t)start;
+    }
+    int c = n == 0 ? -1 : 0;
+    while (c >= 0 && c + 1 < kSortClasses && n > kSortClassMin[c + 1]) ++c;
+    // one atomic per wavefront and class: thousands of segments share a class, and atomics on
+    // one address are served one after the other
+    for (int k = 0; k < kSortClasses; ++k) {
+        const uint64_t members = wave_ballot(c == k);
+        if (members == 0) continue; // uniform
+        const int leader = __ffsll((unsigned long long)members) - 1;
+        uint32_t base = 0;
+        if ((int)lane == leader) base = atomicAdd(&seg_counts[k], (uint32_t)__popcll(members));
+        base = (uint32_t)__shfl((int)base, leader, SPLATAD_WAVE);
+        if (c == k)
+            seg_lists[(size_t)k * n_segments + base + (uint32_t)__popcll(members & ((1ull << lane) - 1ull))] = seg;
+    }
+}
+
 // Tile binning.  A wavefront takes 64 consecutive coarse entries; those of one block (nearly
 // always all 64, the lists being contiguous) are handled together: for each tile of the
 // block a ballot over the mask bit gives the number of entries and every entry's rank, and
@@ -471,11 +512,19 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
                       uint32_t copies, uint32_t n_segments, const int64_t *__restrict__ n_entries_ptr,
                       const uint4 *__restrict__ entries, int32_t *__restrict__ tile_counts,
                       const int32_t *__restrict__ tile_starts, int32_t *__restrict__ tile_fill,
-                      uint64_t *__restrict__ pairs) {
+                      uint64_t *__restrict__ pairs, int64_t n_isects,
+                      uint32_t *__restrict__ seg_counts, uint32_t *__restrict__ seg_lists,
+                      int32_t *__restrict__ tile_offsets) {
     const int64_t n_entries = *n_entries_ptr;
     const uint32_t lane = threadIdx.x & (SPLATAD_WAVE - 1);
     const int64_t wave_id = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / SPLATAD_WAVE;
     const int64_t n_waves = (int64_t)gridDim.x * blockDim.x / SPLATAD_WAVE;
+    // the filling pass also lists the segments by size class for the sort that follows (the
+    // scanned starts are complete before this kernel begins): a lane per segment
+    if (FILL && seg_lists != nullptr)
+        for (int64_t s0 = wave_id * SPLATAD_WAVE; s0 < (int64_t)n_segments; s0 += n_waves * SPLATAD_WAVE)
+            classify_segment((uint32_t)s0 + lane, lane, n_segments, sshift, n_isects, tile_starts,
+                             seg_counts, seg_lists, tile_offsets);
     const uint32_t bits = 4u << cg.bshift, per_cam = cg.cw * cg.ch;
     const uint64_t below = (1ull << lane) - 1ull;
     // the tile counters are replicated like the coarse ones; both passes run on the same
@@ -1034,47 +1083,6 @@ __device__ __forceinline__ void sort_segment_small(uint32_t seg, uint32_t n_segm
     }
 }
 
-// Size classes of the segment sort: class c holds the segments with kSortClassMin[c] < n <=
-// kSortClassMin[c + 1]; the host launches one kernel configuration per class.
-constexpr int kSortClasses = 7;
-__constant__ const uint32_t kSortClassMin[kSortClasses + 1] = {0u,    512u,   2048u,  4096u,
-                                                               8192u, 16384u, 32768u, 0x7FFFFFFFu};
-
-// Lists the segments of every class: seg_lists[c * n_segments + k], k < seg_counts[c] (zeroed
-// beforehand).  The order inside a class is whatever the atomics give; every segment is sorted
-// on its own, so the result does not depend on it.
-__global__ void __launch_bounds__(SPLATAD_THREADS)
-isect_classify_segments_kernel(uint32_t n_segments, uint32_t sshift, int64_t n_isects,
-                               const int32_t *__restrict__ tile_starts,
-                               uint32_t *__restrict__ seg_counts, uint32_t *__restrict__ seg_lists,
-                               int32_t *__restrict__ tile_offsets) {
-    const uint32_t seg = blockIdx.x * blockDim.x + threadIdx.x;
-    uint32_t n = 0;
-    if (seg < n_segments) {
-        const int64_t start = tile_starts[seg];
-        const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
-        n = (uint32_t)(stop - start);
-        // a tile's offset is the start of its segment: the first row of the scanned table
-        // (with depth slabs: of its first slab's)
-        if (tile_offsets != nullptr && (seg & ((1u << sshift) - 1u)) == 0)
-            tile_offsets[seg >> sshift] = (int32_t)start;
-    }
-    int c = n == 0 ? -1 : 0;
-    while (c >= 0 && c + 1 < kSortClasses && n > kSortClassMin[c + 1]) ++c;
-    // one atomic per wavefront and class: thousands of segments share a class, and atomics on
-    // one address are served one after the other
-    const uint32_t lane = threadIdx.x & (SPLATAD_WAVE - 1);
-    for (int k = 0; k < kSortClasses; ++k) {
-        const uint64_t members = wave_ballot(c == k);
-        if (members == 0) continue; // uniform
-        const int leader = __ffsll((unsigned long long)members) - 1;
-        uint32_t base = 0;
-        if ((int)lane == leader) base = atomicAdd(&seg_counts[k], (uint32_t)__popcll(members));
-        base = (uint32_t)__shfl((int)base, leader, SPLATAD_WAVE);
-        if (c == k)
-            seg_lists[(size_t)k * n_segments + base + (uint32_t)__popcll(members & ((1ull << lane) - 1ull))] = seg;
-    }
-}
 
 // The workgroups of a launch share out the segments of one class; a launch has no more
 // workgroups than can be resident, so a class without segments costs next to nothing.
@@ -1526,7 +1534,8 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                        dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, sshift, tcopies,
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
                        w.tile_counts, (const int32_t *)nullptr, (int32_t *)nullptr,
-                       (uint64_t *)nullptr);
+                       (uint64_t *)nullptr, (int64_t)0, (uint32_t *)nullptr, (uint32_t *)nullptr,
+                       (int32_t *)nullptr);
     SPLATAD_LAUNCH_CHECK();
     rc = launch_exclusive_scan<int32_t>(w.tile_counts, (int64_t)(segs * tcopies),
                                         tcopies > 1 ? -(int)tcopies : 1, 0, w.tile_starts,
@@ -1535,7 +1544,8 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     hipLaunchKernelGGL(isect_tile_bin_kernel<true>, dim3((uint32_t)bin_wgs),
                        dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, sshift, tcopies,
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
-                       w.tile_counts, (const int32_t *)w.tile_starts, w.tile_fill, w.pairs);
+                       w.tile_counts, (const int32_t *)w.tile_starts, w.tile_fill, w.pairs, n_isects,
+                       w.seg_counts, w.seg_lists, tile_offsets);
     SPLATAD_LAUNCH_CHECK();
     // Size classes: a launch per class (one for the three upper classes), so that the LDS per
     // workgroup (and with it the number of resident workgroups) fits the segment length; the
@@ -1544,10 +1554,6 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     // events, so that the few long workgroups of the upper classes overlap the many short ones
     // of the lower classes.
     const uint32_t nseg = (uint32_t)segs;
-    hipLaunchKernelGGL(isect_classify_segments_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream,
-                       nseg, sshift, n_isects, (const int32_t *)w.tile_starts, w.seg_counts, w.seg_lists,
-                       tile_offsets);
-    SPLATAD_LAUNCH_CHECK();
     IsectDevice *ss = nullptr;
     if ((rc = isect_device(&ss)) != 0) return rc;
     std::lock_guard<std::mutex> fork_lock(ss->guard);

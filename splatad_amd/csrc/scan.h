@@ -24,11 +24,36 @@ __device__ __forceinline__ int64_t scan_phys(int64_t i, int64_t n, int stride) {
     return (i % rows) * cols + (i / rows);
 }
 
-// Value of logical element i of an int32 input, optionally reduced to a 0/1 flag (v > 0).
-__device__ __forceinline__ int32_t scan_load(const int32_t *in, int64_t i, int64_t n, int stride,
-                                             int as_flag) {
-    if (i >= n) return 0;
-    int32_t v = in[scan_phys(i, n, stride)];
+// Walks consecutive logical elements from i on: one division at the start (n < 2^32), an
+// addition per step.
+struct ScanCursor {
+    int64_t phys;
+    uint32_t row, rows, cols;
+    __device__ __forceinline__ ScanCursor(int64_t i, int64_t n, int stride) {
+        if (stride > 0) {
+            rows = 0; cols = (uint32_t)stride; row = 0;
+            phys = i * stride;
+        } else {
+            rows = (uint32_t)-stride;
+            cols = (uint32_t)n / rows;
+            const uint32_t col = (uint32_t)i / rows;
+            row = (uint32_t)i - col * rows;
+            phys = (int64_t)row * cols + col;
+        }
+    }
+    __device__ __forceinline__ void next() {
+        phys += cols; // the next row of the column, or the next element of a strided vector
+        if (rows != 0 && ++row == rows) {
+            row = 0;
+            phys -= (int64_t)rows * cols - 1; // top of the next column
+        }
+    }
+};
+
+// Value at a physical position, optionally reduced to a 0/1 flag (v > 0).
+__device__ __forceinline__ int32_t scan_load(const int32_t *in, const ScanCursor &c, bool valid, int as_flag) {
+    if (!valid) return 0;
+    const int32_t v = in[c.phys];
     return as_flag ? (v > 0 ? 1 : 0) : v;
 }
 
@@ -63,8 +88,12 @@ scan_block_totals_kernel(const int32_t *__restrict__ in, int64_t n, int stride, 
                          int64_t *__restrict__ block_sums) {
     const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
     int64_t s = 0;
+    ScanCursor c(base, n, stride);
 #pragma unroll
-    for (int k = 0; k < SCAN_ITEMS; ++k) s += scan_load(in, base + k, n, stride, as_flag);
+    for (int k = 0; k < SCAN_ITEMS; ++k) {
+        s += scan_load(in, c, base + k < n, as_flag);
+        c.next();
+    }
     int64_t tot;
     block_exclusive_scan(s, &tot);
     if (threadIdx.x == 0) block_sums[blockIdx.x] = tot;
@@ -105,18 +134,23 @@ scan_apply_kernel(const int32_t *__restrict__ in, int64_t n, int stride, int as_
     const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
     int32_t v[SCAN_ITEMS];
     int64_t s = 0;
+    ScanCursor c(base, n, stride);
 #pragma unroll
     for (int k = 0; k < SCAN_ITEMS; ++k) {
-        v[k] = scan_load(in, base + k, n, stride, as_flag);
+        v[k] = scan_load(in, c, base + k < n, as_flag);
         s += v[k];
+        c.next();
     }
     int64_t tot;
     int64_t run = block_exclusive_scan(s, &tot) + before;
     if (FOLD && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) *total = before + tot;
+    // the output is dense for a strided input and shares the layout of a transposed one
+    ScanCursor o(base, n, stride > 0 ? 1 : stride);
 #pragma unroll
     for (int k = 0; k < SCAN_ITEMS; ++k) {
-        if (base + k < n) out[stride > 0 ? base + k : scan_phys(base + k, n, stride)] = (OutT)run;
+        if (base + k < n) out[o.phys] = (OutT)run;
         run += v[k];
+        o.next();
     }
 }
 
@@ -134,6 +168,7 @@ template <typename OutT>
 static inline int launch_exclusive_scan(const int32_t *in, int64_t n, int stride, int as_flag,
                                         OutT *out, int64_t *total, int64_t *block_sums,
                                         hipStream_t stream) {
+    SPLATAD_REQUIRE(n >= 0 && n < ((int64_t)1 << 32), "scan: %lld elements exceed the 32-bit index range", (long long)n);
     int64_t n_blocks = (n + SCAN_TILE - 1) / SCAN_TILE;
     if (n_blocks > 0) {
         hipLaunchKernelGGL(scan_block_totals_kernel, dim3((uint32_t)n_blocks), dim3(SPLATAD_THREADS),
