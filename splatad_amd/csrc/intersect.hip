@@ -135,8 +135,10 @@ __device__ __forceinline__ uint32_t tile_index(const TileGrid &g, int32_t y, int
     return (uint32_t)y * g.tile_w + (uint32_t)x;
 }
 
-// Grid-stride over the Gaussians.  `counters` (kCountWords words, zeroed) takes the partial
-// sums; the total goes to the host's pinned slot.
+// Grid-stride over the Gaussians.  `counters` (kCountWords words, zero when the kernel starts
+// and zero again when it ends) takes the partial sums; the total goes to the host's pinned
+// slot.  On its way the kernel clears `clear_words` words from `clear` on: the counters of the
+// binning kernels behind it, which spares the launch of a clearing kernel.
 constexpr uint32_t kCountGroups = 32;
 constexpr uint32_t kCountWords = 8 + 8 * kCountGroups;
 template <bool LIDAR>
@@ -144,8 +146,12 @@ __global__ void __launch_bounds__(SPLATAD_THREADS)
 isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d,
                    const void *__restrict__ radii, int32_t *__restrict__ tiles_per_gauss,
                    unsigned long long *__restrict__ counters,
-                   unsigned long long *__restrict__ n_isects_host) {
+                   unsigned long long *__restrict__ n_isects_host, int32_t *__restrict__ clear,
+                   uint64_t clear_words) {
     SPLATAD_STAGE_ELEVATIONS(g)
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words;
+         i += (uint64_t)gridDim.x * blockDim.x)
+        clear[i] = 0;
     long long s = 0;
     // four Gaussians per lane and step, so that their loads are in flight together (the
     // kernel is bound by memory latency otherwise)
@@ -202,13 +208,19 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
         const uint32_t groups = min(gridDim.x, kCountGroups);
         const uint32_t group = blockIdx.x % groups;
         const uint32_t members = gridDim.x / groups + (group < gridDim.x % groups ? 1u : 0u);
-        const unsigned long long before = atomicAdd(counters + 8 + 8 * group, one | (unsigned long long)t);
+        // The counters are put back to zero on the way, each by the last workgroup that touches
+        // it, with an exchange whose result the next step needs: the exchange has been performed
+        // before the report that depends on it is issued, so by the time the host sees the total
+        // (and may start the next counting kernel on these counters, on any stream) they are zero.
+        unsigned long long *mine = counters + 8 + 8 * group;
+        const unsigned long long before = atomicAdd(mine, one | (unsigned long long)t);
         if ((before >> 48) == members - 1) {
-            const unsigned long long group_sum = (before & low) + (unsigned long long)t;
+            const unsigned long long group_sum = atomicExch(mine, 0ull) & low; // (before & low) + t
             const unsigned long long root = atomicAdd(counters, one | group_sum);
-            if ((root >> 48) == groups - 1)
-                __hip_atomic_store(n_isects_host, (root & low) + group_sum, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_SYSTEM);
+            if ((root >> 48) == groups - 1) {
+                const unsigned long long sum = atomicExch(counters, 0ull) & low; // (root & low) + group_sum
+                __hip_atomic_store(n_isects_host, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
         }
     }
 }
@@ -1235,9 +1247,7 @@ __global__ void fill_zero_i32_kernel(int32_t *p, int64_t n) {
     if (i < n) p[i] = 0;
 }
 
-
 struct IsectWorkspace {
-    unsigned long long *n_isects; // [kCountWords] counters of the counting kernel, total first
     int64_t *n_entries;           // [1] length of the coarse lists
     int64_t *scan_total;          // [1]
     uint32_t *slab_bounds;        // [1 << kSlabShiftMax] depth bits at which the slabs begin
@@ -1321,7 +1331,6 @@ static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslo
     if (tslots > scan_n) scan_n = tslots;
     char *p = (char *)ws;
     IsectWorkspace w = {};
-    w.n_isects = (unsigned long long *)p;   p += splatad_align256(kCountWords * 8);
     w.n_entries = (int64_t *)p;             p += 256;
     w.scan_total = (int64_t *)p;            p += 256;
     w.slab_bounds = (uint32_t *)p;          p += 256;
@@ -1428,6 +1437,31 @@ static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const Is
                                           w.coarse_starts, w.n_entries, w.block_sums, stream);
 }
 
+// The counting kernel's cross-workgroup counters: one set per leased host word (calls that
+// overlap hold different leases), in device memory of the library itself, zero when the library
+// is loaded and left at zero by every counting kernel that completes.
+static __device__ __align__(256) unsigned long long count_words[kHostWordSlots * kCountWords];
+
+// Address of the current device's copy of `count_words`, looked up once per device.  In host
+// code the array's name is only a handle for this lookup, never an address a kernel could use.
+static int count_words_of(int slot, unsigned long long **out) {
+    static std::mutex guard;
+    static unsigned long long *table[kHostWordDevices] = {};
+    int dev = 0;
+    SPLATAD_CHECK_HIP(hipGetDevice(&dev));
+    SPLATAD_REQUIRE(dev >= 0 && dev < kHostWordDevices, "isect: device index %d out of range", dev);
+    SPLATAD_REQUIRE(slot >= 0 && slot < kHostWordSlots, "isect: host word slot %d out of range", slot);
+    std::lock_guard<std::mutex> lock(guard);
+    if (table[dev] == nullptr) {
+        void *ptr = nullptr;
+        SPLATAD_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(count_words)));
+        SPLATAD_REQUIRE(ptr != nullptr, "isect: the counters have no device address");
+        table[dev] = (unsigned long long *)ptr;
+    }
+    *out = table[dev] + (size_t)slot * kCountWords;
+    return 0;
+}
+
 template <bool LIDAR>
 static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *camera_ids,
                        const float *means2d, const void *radii, const float *depths, uint32_t C, int sort,
@@ -1450,16 +1484,15 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     // the number of intersections reaches the host through a leased pinned word
     HostWordLease lease(stream);
     if (int rc = host_word_acquire(&lease.word)) return rc;
-    // one fill clears the counters and, for the binning, everything up to the end of the tile
-    // counters (the two scan totals between them are written before they are read)
-    const uint64_t clear_words = sort ? (uint64_t)((char *)(w.zeroed + w.n_zeroed) - (char *)w.n_isects) / 4
-                                      : (uint64_t)kCountWords * 2;
-    hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(clear_words), dim3(SPLATAD_THREADS), 0, stream,
-                       (int32_t *)w.n_isects, (int64_t)clear_words);
+    unsigned long long *counters = nullptr;
+    if (int rc = count_words_of(lease.word.slot, &counters)) return rc;
+    // the counting kernel clears the tile counters, the fill cursors and the class counters of
+    // the binning behind it
     dim3 count_grid = grid_for(total);
     if (count_grid.x > 1024) count_grid.x = 1024;
     hipLaunchKernelGGL(isect_count_kernel<LIDAR>, count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
-                       total, means2d, radii, tiles_per_gauss, w.n_isects, lease.word.device);
+                       total, means2d, radii, tiles_per_gauss, counters, lease.word.device,
+                       w.zeroed, sort ? w.n_zeroed : (uint64_t)0);
     SPLATAD_LAUNCH_CHECK();
     // work for the GPU while the host learns the count and sizes the lists
     if (sort) {
@@ -1575,7 +1608,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
             return e;
         SPLATAD_SORT_CLASS(2, 8, 512, 4096u, 1024u, ss->aux[0])
         SPLATAD_SORT_CLASS(3, 8, 1024, 8192u, 512u, ss->aux[1])
-        SPLATAD_SORT_CLASS(1, 8, 256, 2048u, 2048u, stream)
+        SPLATAD_SORT_CLASS(1, 8, 256, 2048u, 4096u, stream)
         SPLATAD_SORT_CLASS(0, 4, 128, 512u, 4096u, stream)
 #undef SPLATAD_SORT_CLASS
         return 0;
