@@ -106,7 +106,7 @@ def bench_camera(args):
 
     with torch.no_grad():
         sec = time_steps(run, args.steps, args.warmup)
-        sec_packed = time_steps(lambda: run(True), max(2, args.steps // 2), 1)
+        sec_packed = time_steps(lambda: run(True), args.steps, args.warmup)
         rc, ra, meta = run()
         C, H, W = 1, s["height"], s["width"]
         # dominant kernel, isolated

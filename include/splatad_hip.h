@@ -62,6 +62,35 @@ int splatad_projection_packed_count(uint32_t C, uint32_t N, const float *means,
                                     float near_plane, float far_plane, float radius_clip,
                                     int calc_compensations, void *workspace, int64_t *nnz_host,
                                     splatad_stream_t stream);
+/* The same counting call for a caller that goes on to intersect the packed rows with a
+ * camera tile grid (rendering.py:278-309 of the reference: projection, then isect_tiles with the
+ * same rows): it also counts the tiles the kept rows meet, rasterization.cu:44-62, and returns
+ * both numbers with its one wait, so that splatad_isect_tiles_prepare can replace
+ * splatad_isect_tiles_count and its wait. */
+int splatad_projection_packed_count_tiles(uint32_t C, uint32_t N, const float *means,
+                                          const float *covars, const float *quats, const float *scales,
+                                          const float *velocities, const float *viewmats,
+                                          const float *Ks, uint32_t image_width, uint32_t image_height,
+                                          const float *linear_velocity, const float *angular_velocity,
+                                          const float *rolling_shutter_time, float eps2d,
+                                          float near_plane, float far_plane, float radius_clip,
+                                          int calc_compensations, uint32_t tile_size,
+                                          uint32_t tile_width, uint32_t tile_height, void *workspace,
+                                          void *isect_workspace, int64_t *nnz_host,
+                                          int64_t *n_isects_host, splatad_stream_t stream);
+/* With isect_workspace (splatad_isect_workspace_bytes(C * N, C, tile_width * tile_height) bytes,
+ * may be NULL) the counting call above also enqueues, before it waits, the first stages of the
+ * tile intersection on the dense rows in its workspace, and this call completes it for the
+ * packed rows: the lists it writes are those of splatad_isect_tiles_count / _fill on the packed
+ * outputs of splatad_projection_packed_fill (tiles_per_gauss [nnz] included), without the wait.
+ * Both workspaces must be untouched since the counting call; `lists` is
+ * splatad_isect_lists_bytes(C * N, n_isects) bytes of scratch. */
+int splatad_isect_tiles_fill_packed(uint32_t C, uint32_t N, uint32_t tile_size, uint32_t tile_width,
+                                    uint32_t tile_height, int64_t n_isects,
+                                    const void *packed_workspace, void *isect_workspace, void *lists,
+                                    int32_t *tiles_per_gauss, int64_t *isect_ids,
+                                    int32_t *flatten_ids, int32_t *tile_offsets,
+                                    splatad_stream_t stream);
 int splatad_projection_packed_fill(uint32_t C, uint32_t N, int64_t nnz, const void *workspace,
                                    int32_t *indptr, int64_t *camera_ids, int64_t *gaussian_ids,
                                    int32_t *radii, float *means2d, float *depths, float *conics,
@@ -172,8 +201,8 @@ int splatad_view_colors_bwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint
  * untouched in between.  `lists` is
  * splatad_isect_lists_bytes(total, n_isects) bytes of scratch for _fill alone.
  * _count waits for the counting kernel only (the kernel writes n_isects into a
- * pinned host slot, one per device, kept for the life of the process, and the
- * host spins on it), not for the work enqueued behind it.
+ * pinned host word leased from a small per-device pool that is kept for the life of the
+ * process, and the host spins on it), not for the work enqueued behind it.
  *
  * tile_offsets may be NULL; with sort != 0 it receives the [C, tile_height,
  * tile_width] table that splatad_isect_offset_encode would derive from isect_ids
@@ -185,6 +214,25 @@ int splatad_isect_tiles_count(uint64_t total, uint32_t N, const int64_t *camera_
                               uint32_t C, uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
                               int sort, int32_t *tiles_per_gauss, void *workspace,
                               int64_t *n_isects_host, splatad_stream_t stream);
+/* splatad_isect_tiles_count for a caller that knows n_isects already (from
+ * splatad_projection_packed_count_tiles on the same rows and tile grid): enqueues the same work,
+ * returns no number and waits for nothing.  _fill follows with that n_isects, which must be
+ * the number _count would have returned. */
+int splatad_isect_tiles_prepare(uint64_t total, uint32_t N, const int64_t *camera_ids,
+                                const float *means2d, const int32_t *radii, const float *depths,
+                                uint32_t C, uint32_t tile_size, uint32_t tile_width,
+                                uint32_t tile_height, int sort, int32_t *tiles_per_gauss,
+                                void *workspace, splatad_stream_t stream);
+/* _fill for dense [C, N] rows that stand in for their packed rows: `remap` [C * N] holds each
+ * kept row's position among the kept rows (what flatten_ids must name); tiles_out, if not NULL,
+ * receives the kept rows' tile counts at those positions. */
+int splatad_isect_tiles_fill_remapped(uint64_t total, uint32_t N, const float *means2d,
+                                      const int32_t *radii, const float *depths, uint32_t C,
+                                      uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
+                                      int64_t n_isects, const int32_t *tiles_per_gauss,
+                                      const int32_t *remap, void *workspace, void *lists,
+                                      int32_t *tiles_out, int64_t *isect_ids, int32_t *flatten_ids,
+                                      int32_t *tile_offsets, splatad_stream_t stream);
 int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_ids,
                              const float *means2d, const int32_t *radii, const float *depths,
                              uint32_t C, uint32_t tile_size, uint32_t tile_width,

@@ -22,6 +22,7 @@
 #include "common.h"
 #include "host_word.h"
 #include "scan.h"
+#include "tile_rect.h"
 
 #include <mutex>
 
@@ -33,12 +34,6 @@ struct TileGrid {
     float azim_res, min_azim; // lidar only
     const float *elev_boundaries;
 };
-
-__device__ __forceinline__ uint32_t f2u_sat(float v) {
-    if (!(v > 0.0f)) return 0u;
-    if (v >= 4294967296.0f) return 0xFFFFFFFFu;
-    return (uint32_t)v;
-}
 
 // Number of leading boundaries below v (boundaries ascending).
 __device__ __forceinline__ int32_t elev_lower_bound(const float *b, int32_t count, float v) {
@@ -68,15 +63,8 @@ template <bool LIDAR>
 __device__ __forceinline__ bool tile_rect_of(const TileGrid &g, float2 mu, uint2 radii,
                                              int32_t &x0, int32_t &y0, int32_t &x1, int32_t &y1) {
     if (!LIDAR) {
-        const int2 r = make_int2((int32_t)radii.x, (int32_t)radii.y);
-        if (r.x <= 0) return false;
-        const float ts = (float)g.tile_size;
-        const float ex = (float)r.x / ts, ey = (float)r.y / ts;
-        const float tx = mu.x / ts, ty = mu.y / ts;
-        x0 = (int32_t)min(f2u_sat(floorf(tx - ex)), g.tile_w);
-        y0 = (int32_t)min(f2u_sat(floorf(ty - ey)), g.tile_h);
-        x1 = (int32_t)min(f2u_sat(ceilf(tx + ex)), g.tile_w);
-        y1 = (int32_t)min(f2u_sat(ceilf(ty + ey)), g.tile_h);
+        return splatad_camera_tile_rect(g.tile_size, g.tile_w, g.tile_h, mu,
+                                        make_int2((int32_t)radii.x, (int32_t)radii.y), x0, y0, x1, y1);
     } else {
         const float2 r = make_float2(__uint_as_float(radii.x), __uint_as_float(radii.y));
         if (r.x <= 0.f) return false;
@@ -191,7 +179,7 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
     __shared__ long long wsum[SPLATAD_THREADS / SPLATAD_WAVE];
     if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = s;
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (threadIdx.x == 0 && counters != nullptr) { // null: the caller knows the total already
         long long t = 0;
         for (int w = 0; w < SPLATAD_THREADS / SPLATAD_WAVE; ++w) t += wsum[w];
         // A workgroup reports with one atomic that carries both its sum (low 48 bits) and a
@@ -434,7 +422,8 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
                     const void *__restrict__ radii, const float *__restrict__ depths,
                     uint32_t cam_lo, uint32_t cam_hi, uint32_t n_blocks, int32_t *table,
                     uint4 *__restrict__ entries, uint32_t sshift,
-                    const uint32_t *__restrict__ slab_bounds) {
+                    const uint32_t *__restrict__ slab_bounds, const int32_t *__restrict__ remap,
+                    int32_t *__restrict__ tiles_out) {
     extern __shared__ int32_t s_blocks[];
     __shared__ uint32_t s_bounds[1u << kSlabShiftMax];
     SPLATAD_STAGE_ELEVATIONS(g)
@@ -451,12 +440,22 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
     WorkInputs ahead = fetch_work((uint64_t)blockIdx.x * blockDim.x + threadIdx.x, total, N, camera_ids,
                                   means2d, radii, depths_needed, nullptr);
     for (uint64_t base = (uint64_t)blockIdx.x * blockDim.x; base < total; base += round) { // uniform
+        const bool was_kept = ahead.in_range && (LIDAR ? __uint_as_float(ahead.radii.x) > 0.f
+                                                       : (int32_t)ahead.radii.x > 0);
         LaneWork mine = make_work<LIDAR>(g, ahead);
         // the inputs of the next round are requested before this round's emission
         ahead = fetch_work(base + round + threadIdx.x, total, N, camera_ids, means2d, radii,
                            depths_needed, nullptr);
         const uint32_t cam = mine.base / tiles_per_cam;
         if (cam < cam_lo || cam >= cam_hi) mine.cnt = 0;
+        // Rows of a dense [C, N] projection standing in for its packed rows: the entries carry
+        // the row's position among the kept rows (an increasing function of the dense index, so
+        // ties keep their order), and the kept rows' tile counts are gathered on the way.
+        if (FILL && remap != nullptr && was_kept) {
+            const uint32_t at = (uint32_t)remap[mine.idx];
+            if (tiles_out != nullptr && cam >= cam_lo && cam < cam_hi) tiles_out[at] = mine.cnt;
+            mine.idx = at;
+        }
         mine.base = (cam - cam_lo) * per_cam;
         mine.slab = slab_of(mine.depth_bits, s_bounds, n_bounds);
         to_coarse(mine, cg);
@@ -1429,7 +1428,7 @@ static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const Is
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, pl.cg,
                            total, N, camera_ids, means2d, radii, pl.sshift ? depths : nullptr, c0, c1,
                            (uint32_t)pl.blocks, w.coarse_counts, (uint4 *)nullptr, pl.sshift,
-                           (const uint32_t *)w.slab_bounds);
+                           (const uint32_t *)w.slab_bounds, (const int32_t *)nullptr, (int32_t *)nullptr);
     }
     SPLATAD_LAUNCH_CHECK();
     return launch_exclusive_scan<int32_t>(w.coarse_counts, (int64_t)pl.cslots,
@@ -1466,9 +1465,11 @@ template <bool LIDAR>
 static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *camera_ids,
                        const float *means2d, const void *radii, const float *depths, uint32_t C, int sort,
                        int32_t *tiles_per_gauss, void *workspace, int64_t *n_isects_host,
-                       hipStream_t stream) {
-    SPLATAD_REQUIRE(n_isects_host != nullptr, "isect: n_isects_host is null");
-    *n_isects_host = 0;
+                       hipStream_t stream, bool known = false) {
+    // known: the caller has the number of intersections from elsewhere (the packed projection
+    // counts them for its rows); everything is enqueued as usual, nothing is waited for
+    SPLATAD_REQUIRE(known || n_isects_host != nullptr, "isect: n_isects_host is null");
+    if (n_isects_host) *n_isects_host = 0;
     if (total == 0) return 0;
     SPLATAD_REQUIRE(total < (1ull << 31), "isect: number of projected Gaussians must be below 2^31");
     SPLATAD_REQUIRE(means2d && radii && tiles_per_gauss && workspace, "isect: null pointer argument");
@@ -1480,12 +1481,14 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
                     "isect: camera and tile ids need more than 32 bits");
     IsectWorkspace w;
     carve_isect(workspace, total, pl.segs, sort ? pl.cslots : 0, &w);
-    if (int rc = host_word_refuse_capture(stream, "isect")) return rc;
     // the number of intersections reaches the host through a leased pinned word
     HostWordLease lease(stream);
-    if (int rc = host_word_acquire(&lease.word)) return rc;
     unsigned long long *counters = nullptr;
-    if (int rc = count_words_of(lease.word.slot, &counters)) return rc;
+    if (!known) {
+        if (int rc = host_word_refuse_capture(stream, "isect")) return rc;
+        if (int rc = host_word_acquire(&lease.word)) return rc;
+        if (int rc = count_words_of(lease.word.slot, &counters)) return rc;
+    }
     // the counting kernel clears the tile counters, the fill cursors and the class counters of
     // the binning behind it
     dim3 count_grid = grid_for(total);
@@ -1505,6 +1508,7 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
                                                  C, stream))
             return rc;
     }
+    if (known) return 0;
     unsigned long long n = 0;
     if (int rc = host_word_wait(&lease, "isect", &n)) return rc;
     SPLATAD_REQUIRE(n < (1ull << 31), "isect: %llu intersections exceed the int32 offset range", n);
@@ -1517,7 +1521,10 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                       const float *means2d, const void *radii, const float *depths, uint32_t C,
                       int sort, int64_t n_isects, const int32_t *tiles_per_gauss,
                       void *workspace, void *lists, int64_t *isect_ids, int32_t *flatten_ids,
-                      int32_t *tile_offsets, hipStream_t stream) {
+                      int32_t *tile_offsets, hipStream_t stream, const int32_t *remap = nullptr,
+                      int32_t *tiles_out = nullptr) {
+    SPLATAD_REQUIRE(remap == nullptr || (sort && camera_ids == nullptr),
+                    "isect: remapped rows need sort != 0 and a dense [C, N] layout");
     if (total == 0 || n_isects == 0) {
         if (tile_offsets && sort && (uint64_t)C * g.tile_w * g.tile_h > 0) {
             const uint64_t tiles = (uint64_t)C * g.tile_w * g.tile_h;
@@ -1555,7 +1562,8 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, true>), dim3(pl.coarse_wgs),
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, cg,
                            total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)pl.blocks,
-                           w.coarse_starts, w.entries, sshift, (const uint32_t *)w.slab_bounds);
+                           w.coarse_starts, w.entries, sshift, (const uint32_t *)w.slab_bounds, remap,
+                           tiles_out);
     }
     SPLATAD_LAUNCH_CHECK();
     // tile segments: count, scan, fill.  The number of coarse entries stays on the device;
@@ -1647,6 +1655,18 @@ extern "C" int splatad_isect_tiles_count(uint64_t total, uint32_t N, const int64
                               workspace, n_isects_host, (hipStream_t)stream);
 }
 
+extern "C" int splatad_isect_tiles_prepare(uint64_t total, uint32_t N, const int64_t *camera_ids,
+                                           const float *means2d, const int32_t *radii,
+                                           const float *depths, uint32_t C, uint32_t tile_size,
+                                           uint32_t tile_width, uint32_t tile_height, int sort,
+                                           int32_t *tiles_per_gauss, void *workspace,
+                                           splatad_stream_t stream) {
+    SPLATAD_REQUIRE(tile_size > 0, "isect_tiles: tile_size is zero");
+    TileGrid g{tile_size, tile_width, tile_height, 0.f, 0.f, nullptr};
+    return isect_count<false>(g, total, N, camera_ids, means2d, radii, depths, C, sort, tiles_per_gauss,
+                              workspace, nullptr, (hipStream_t)stream, true);
+}
+
 extern "C" int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_ids,
                                         const float *means2d, const int32_t *radii,
                                         const float *depths, uint32_t C, uint32_t tile_size,
@@ -1660,6 +1680,22 @@ extern "C" int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_
     return isect_fill<false>(g, total, N, camera_ids, means2d, radii, depths, C, sort, n_isects,
                              tiles_per_gauss, workspace, lists, isect_ids, flatten_ids,
                              tile_offsets, (hipStream_t)stream);
+}
+
+extern "C" int splatad_isect_tiles_fill_remapped(uint64_t total, uint32_t N, const float *means2d,
+                                                 const int32_t *radii, const float *depths, uint32_t C,
+                                                 uint32_t tile_size, uint32_t tile_width,
+                                                 uint32_t tile_height, int64_t n_isects,
+                                                 const int32_t *tiles_per_gauss, const int32_t *remap,
+                                                 void *workspace, void *lists, int32_t *tiles_out,
+                                                 int64_t *isect_ids, int32_t *flatten_ids,
+                                                 int32_t *tile_offsets, splatad_stream_t stream) {
+    SPLATAD_REQUIRE(tile_size > 0, "isect_tiles: tile_size is zero");
+    SPLATAD_REQUIRE(remap != nullptr, "isect_tiles: remap is null");
+    TileGrid g{tile_size, tile_width, tile_height, 0.f, 0.f, nullptr};
+    return isect_fill<false>(g, total, N, nullptr, means2d, radii, depths, C, 1, n_isects, tiles_per_gauss,
+                             workspace, lists, isect_ids, flatten_ids, tile_offsets, (hipStream_t)stream,
+                             remap, tiles_out);
 }
 
 extern "C" int splatad_isect_lidar_tiles_count(uint64_t total, uint32_t N,

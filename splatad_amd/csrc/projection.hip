@@ -12,6 +12,7 @@
 #include "common.h"
 #include "host_word.h"
 #include "scan.h"
+#include "tile_rect.h"
 
 #define RAD_TO_DEG 57.2957795131f
 
@@ -301,6 +302,8 @@ struct PackedWorkspace {
     int32_t *pos;     // [T] exclusive prefix of the valid flags
     int64_t *total;   // [1]
     int64_t *block_sums;
+    int64_t *tile_sums; // [scan blocks] tiles met by the kept rows of a scan block (optional count)
+    int32_t *tiles;     // [T] tiles per dense row (intersection started by the counting call)
 };
 
 static PackedWorkspace carve_packed(void *ws, uint64_t T) {
@@ -314,8 +317,57 @@ static PackedWorkspace carve_packed(void *ws, uint64_t T) {
     w.comps = (float *)p;         p += splatad_align256(T * 4);
     w.pix_vels = (float *)p;      p += splatad_align256(T * 8);
     w.pos = (int32_t *)p;         p += splatad_align256(T * 4);
-    w.block_sums = (int64_t *)p;
+    w.block_sums = (int64_t *)p;  p += scan_workspace_bytes((int64_t)T);
+    w.tile_sums = (int64_t *)p;   p += scan_workspace_bytes((int64_t)T);
+    w.tiles = (int32_t *)p;
     return w;
+}
+
+// The per-block totals of the scan over the kept flags (radii.x > 0, SCAN_TILE rows per block,
+// as scan_block_totals_kernel makes them) and, on the same pass, the number of tiles the kept
+// rows of the block meet on the camera's tile grid.
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+packed_block_totals_kernel(uint64_t T, const int32_t *__restrict__ w_radii,
+                           const float *__restrict__ w_means2d, uint32_t tile_size, uint32_t tile_w,
+                           uint32_t tile_h, int64_t *__restrict__ block_sums,
+                           int64_t *__restrict__ tile_sums) {
+    const uint64_t base = (uint64_t)blockIdx.x * SCAN_TILE + (uint64_t)threadIdx.x * SCAN_ITEMS;
+    int64_t kept = 0, tiles = 0;
+#pragma unroll
+    for (int k = 0; k < SCAN_ITEMS; ++k) {
+        const uint64_t idx = base + k;
+        if (idx >= T) continue;
+        const int2 r = reinterpret_cast<const int2 *>(w_radii)[idx];
+        if (r.x <= 0) continue;
+        ++kept;
+        int32_t x0, y0, x1, y1;
+        splatad_camera_tile_rect(tile_size, tile_w, tile_h, reinterpret_cast<const float2 *>(w_means2d)[idx], r,
+                                 x0, y0, x1, y1);
+        tiles += (int64_t)max(y1 - y0, 0) * max(x1 - x0, 0);
+    }
+    int64_t kept_total, tiles_total;
+    block_exclusive_scan(kept, &kept_total);
+    block_exclusive_scan(tiles, &tiles_total);
+    if (threadIdx.x == 0) {
+        block_sums[blockIdx.x] = kept_total;
+        tile_sums[blockIdx.x] = tiles_total;
+    }
+}
+
+// One workgroup: publishes the number of kept rows (low 32 bits) and of their tile
+// intersections (high 32 bits, saturated at 2^31 - 1, which the caller refuses) in one word.
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+packed_publish_kernel(const int64_t *__restrict__ total, const int64_t *__restrict__ tile_sums,
+                      int64_t n_blocks, unsigned long long *__restrict__ word) {
+    int64_t part = 0;
+    for (int64_t b = threadIdx.x; b < n_blocks; b += SPLATAD_THREADS) part += tile_sums[b];
+    int64_t tiles;
+    block_exclusive_scan(part, &tiles);
+    if (threadIdx.x == 0) {
+        const unsigned long long hi = tiles > 0x7FFFFFFFll ? 0x7FFFFFFFull : (unsigned long long)tiles;
+        __hip_atomic_store(word, (hi << 32) | (unsigned long long)(uint32_t)*total, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_SYSTEM);
+    }
 }
 
 __global__ void __launch_bounds__(SPLATAD_THREADS)
@@ -415,7 +467,72 @@ extern "C" int splatad_lidar_projection_fwd(uint32_t C, uint32_t N, const float 
 extern "C" size_t splatad_projection_packed_workspace_bytes(uint32_t C, uint32_t N) {
     const uint64_t T = (uint64_t)C * N;
     return 256 + splatad_align256(T * 8) * 3 + splatad_align256(T * 4) * 3 +
-           splatad_align256(T * 12) + scan_workspace_bytes((int64_t)T);
+           splatad_align256(T * 12) + 2 * scan_workspace_bytes((int64_t)T) + splatad_align256(T * 4);
+}
+
+// tile_size == 0: only the kept rows are counted.
+static int packed_count(uint32_t C, uint32_t N, const float *means, const float *covars, const float *quats,
+                        const float *scales, const float *velocities, const float *viewmats, const float *Ks,
+                        uint32_t W, uint32_t H, const float *lin_vel, const float *ang_vel, const float *rs_time,
+                        float eps2d, float near_plane, float far_plane, float radius_clip, int calc_compensations,
+                        uint32_t tile_size, uint32_t tile_width, uint32_t tile_height, void *workspace,
+                        void *isect_workspace, int64_t *nnz_host, int64_t *n_isects_host,
+                        splatad_stream_t stream) {
+    SPLATAD_REQUIRE(nnz_host != nullptr, "packed projection: nnz_host is null");
+    *nnz_host = 0;
+    if (n_isects_host) *n_isects_host = 0;
+    if (C == 0 || N == 0) return 0;
+    SPLATAD_REQUIRE(workspace != nullptr, "packed projection: workspace is null");
+    const uint64_t T = (uint64_t)C * N;
+    PackedWorkspace w = carve_packed(workspace, T);
+    if (int rc = host_word_refuse_capture((hipStream_t)stream, "packed projection")) return rc;
+    // the counts reach the host through a leased pinned word
+    HostWordLease lease((hipStream_t)stream);
+    if (int rc = host_word_acquire(&lease.word)) return rc;
+    int rc = splatad_projection_fwd(C, N, means, covars, quats, scales, velocities, viewmats, Ks,
+                                    W, H, lin_vel, ang_vel, rs_time, eps2d, near_plane, far_plane,
+                                    radius_clip, w.radii, w.means2d, w.depths, w.conics,
+                                    calc_compensations ? w.comps : nullptr, w.pix_vels, stream);
+    if (rc) return rc;
+    if (tile_size == 0) {
+        rc = launch_exclusive_scan<int32_t>(w.radii, (int64_t)T, 2, 1, w.pos, w.total, w.block_sums,
+                                            (hipStream_t)stream);
+        if (rc) return rc;
+        hipLaunchKernelGGL(host_word_publish_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, w.total,
+                           lease.word.device);
+    } else {
+        const int64_t n_blocks = ((int64_t)T + SCAN_TILE - 1) / SCAN_TILE;
+        hipLaunchKernelGGL(packed_block_totals_kernel, dim3((uint32_t)n_blocks), dim3(SPLATAD_THREADS), 0,
+                           (hipStream_t)stream, T, (const int32_t *)w.radii, (const float *)w.means2d, tile_size,
+                           tile_width, tile_height, w.block_sums, w.tile_sums);
+        SPLATAD_LAUNCH_CHECK();
+        rc = launch_exclusive_scan_apply<int32_t>(w.radii, (int64_t)T, 2, 1, w.pos, w.total, w.block_sums,
+                                                  (hipStream_t)stream);
+        if (rc) return rc;
+        hipLaunchKernelGGL(packed_publish_kernel, dim3(1), dim3(SPLATAD_THREADS), 0, (hipStream_t)stream,
+                           (const int64_t *)w.total, (const int64_t *)w.tile_sums, n_blocks, lease.word.device);
+        SPLATAD_LAUNCH_CHECK();
+        // work for the GPU while the host learns the counts and sizes the outputs: the first
+        // stages of the tile intersection, on the dense rows (culled rows meet no tile)
+        if (isect_workspace != nullptr) {
+            rc = splatad_isect_tiles_prepare(T, N, nullptr, w.means2d, w.radii, w.depths, C, tile_size,
+                                             tile_width, tile_height, 1, w.tiles, isect_workspace, stream);
+            if (rc) return rc;
+        }
+    }
+    SPLATAD_LAUNCH_CHECK();
+    unsigned long long word = 0;
+    rc = host_word_wait(&lease, "packed projection", &word);
+    if (rc) return rc;
+    if (tile_size == 0) {
+        *nnz_host = (int64_t)word;
+    } else {
+        *nnz_host = (int64_t)(word & 0xFFFFFFFFull);
+        SPLATAD_REQUIRE((word >> 32) < 0x7FFFFFFFull,
+                        "packed projection: the kept rows meet 2^31 - 1 tiles or more, beyond the int32 offset range");
+        if (n_isects_host) *n_isects_host = (int64_t)(word >> 32);
+    }
+    return 0;
 }
 
 extern "C" int splatad_projection_packed_count(
@@ -424,32 +541,37 @@ extern "C" int splatad_projection_packed_count(
     uint32_t W, uint32_t H, const float *lin_vel, const float *ang_vel, const float *rs_time,
     float eps2d, float near_plane, float far_plane, float radius_clip, int calc_compensations,
     void *workspace, int64_t *nnz_host, splatad_stream_t stream) {
-    SPLATAD_REQUIRE(nnz_host != nullptr, "packed projection: nnz_host is null");
-    *nnz_host = 0;
-    if (C == 0 || N == 0) return 0;
-    SPLATAD_REQUIRE(workspace != nullptr, "packed projection: workspace is null");
+    return packed_count(C, N, means, covars, quats, scales, velocities, viewmats, Ks, W, H, lin_vel, ang_vel,
+                        rs_time, eps2d, near_plane, far_plane, radius_clip, calc_compensations, 0, 0, 0,
+                        workspace, nullptr, nnz_host, nullptr, stream);
+}
+
+extern "C" int splatad_projection_packed_count_tiles(
+    uint32_t C, uint32_t N, const float *means, const float *covars, const float *quats,
+    const float *scales, const float *velocities, const float *viewmats, const float *Ks,
+    uint32_t W, uint32_t H, const float *lin_vel, const float *ang_vel, const float *rs_time,
+    float eps2d, float near_plane, float far_plane, float radius_clip, int calc_compensations,
+    uint32_t tile_size, uint32_t tile_width, uint32_t tile_height, void *workspace, void *isect_workspace,
+    int64_t *nnz_host, int64_t *n_isects_host, splatad_stream_t stream) {
+    SPLATAD_REQUIRE(tile_size > 0 && n_isects_host != nullptr,
+                    "packed projection: tile_size is zero or n_isects_host is null");
+    return packed_count(C, N, means, covars, quats, scales, velocities, viewmats, Ks, W, H, lin_vel, ang_vel,
+                        rs_time, eps2d, near_plane, far_plane, radius_clip, calc_compensations, tile_size,
+                        tile_width, tile_height, workspace, isect_workspace, nnz_host, n_isects_host, stream);
+}
+
+extern "C" int splatad_isect_tiles_fill_packed(uint32_t C, uint32_t N, uint32_t tile_size, uint32_t tile_width,
+                                               uint32_t tile_height, int64_t n_isects,
+                                               const void *packed_workspace, void *isect_workspace,
+                                               void *lists, int32_t *tiles_per_gauss, int64_t *isect_ids,
+                                               int32_t *flatten_ids, int32_t *tile_offsets,
+                                               splatad_stream_t stream) {
+    SPLATAD_REQUIRE(packed_workspace && isect_workspace, "isect_tiles: null workspace");
     const uint64_t T = (uint64_t)C * N;
-    PackedWorkspace w = carve_packed(workspace, T);
-    if (int rc = host_word_refuse_capture((hipStream_t)stream, "packed projection")) return rc;
-    // the number of kept (camera, Gaussian) pairs reaches the host through a leased pinned word
-    HostWordLease lease((hipStream_t)stream);
-    if (int rc = host_word_acquire(&lease.word)) return rc;
-    int rc = splatad_projection_fwd(C, N, means, covars, quats, scales, velocities, viewmats, Ks,
-                                    W, H, lin_vel, ang_vel, rs_time, eps2d, near_plane, far_plane,
-                                    radius_clip, w.radii, w.means2d, w.depths, w.conics,
-                                    calc_compensations ? w.comps : nullptr, w.pix_vels, stream);
-    if (rc) return rc;
-    rc = launch_exclusive_scan<int32_t>(w.radii, (int64_t)T, 2, 1, w.pos, w.total, w.block_sums,
-                                        (hipStream_t)stream);
-    if (rc) return rc;
-    hipLaunchKernelGGL(host_word_publish_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, w.total,
-                       lease.word.device);
-    SPLATAD_LAUNCH_CHECK();
-    unsigned long long nnz = 0;
-    rc = host_word_wait(&lease, "packed projection", &nnz);
-    if (rc) return rc;
-    *nnz_host = (int64_t)nnz;
-    return 0;
+    PackedWorkspace w = carve_packed((void *)packed_workspace, T);
+    return splatad_isect_tiles_fill_remapped(T, N, w.means2d, w.radii, w.depths, C, tile_size, tile_width,
+                                             tile_height, n_isects, w.tiles, w.pos, isect_workspace, lists,
+                                             tiles_per_gauss, isect_ids, flatten_ids, tile_offsets, stream);
 }
 
 extern "C" int splatad_projection_packed_fill(uint32_t C, uint32_t N, int64_t nnz,

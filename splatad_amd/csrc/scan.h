@@ -164,17 +164,14 @@ static inline size_t scan_workspace_bytes(int64_t n) {
 // out[i] = sum_{j<i} f(in[phys(j)]); *total (device) = sum over all.  The output is dense for
 // stride > 0 and uses the input's transposed layout for stride < 0 (see scan_phys).
 // `block_sums` is scan_workspace_bytes(n) of scratch.  n == 0 only writes *total = 0.
+// Second half of a scan whose per-block totals (SCAN_TILE logical elements per block) are in
+// block_sums already: launch_exclusive_scan() below, or a caller that makes the totals with a
+// kernel of its own, which can gather something else on the same pass.
 template <typename OutT>
-static inline int launch_exclusive_scan(const int32_t *in, int64_t n, int stride, int as_flag,
-                                        OutT *out, int64_t *total, int64_t *block_sums,
-                                        hipStream_t stream) {
-    SPLATAD_REQUIRE(n >= 0 && n < ((int64_t)1 << 32), "scan: %lld elements exceed the 32-bit index range", (long long)n);
-    int64_t n_blocks = (n + SCAN_TILE - 1) / SCAN_TILE;
-    if (n_blocks > 0) {
-        hipLaunchKernelGGL(scan_block_totals_kernel, dim3((uint32_t)n_blocks), dim3(SPLATAD_THREADS),
-                           0, stream, in, n, stride, as_flag, block_sums);
-        SPLATAD_LAUNCH_CHECK();
-    }
+static inline int launch_exclusive_scan_apply(const int32_t *in, int64_t n, int stride, int as_flag,
+                                              OutT *out, int64_t *total, int64_t *block_sums,
+                                              hipStream_t stream) {
+    const int64_t n_blocks = (n + SCAN_TILE - 1) / SCAN_TILE;
     if (n_blocks > 0 && n_blocks <= kScanFoldBlocks && out != nullptr) {
         hipLaunchKernelGGL((scan_apply_kernel<OutT, true>), dim3((uint32_t)n_blocks),
                            dim3(SPLATAD_THREADS), 0, stream, in, n, stride, as_flag,
@@ -192,6 +189,20 @@ static inline int launch_exclusive_scan(const int32_t *in, int64_t n, int stride
         SPLATAD_LAUNCH_CHECK();
     }
     return 0;
+}
+
+template <typename OutT>
+static inline int launch_exclusive_scan(const int32_t *in, int64_t n, int stride, int as_flag,
+                                        OutT *out, int64_t *total, int64_t *block_sums,
+                                        hipStream_t stream) {
+    SPLATAD_REQUIRE(n >= 0 && n < ((int64_t)1 << 32), "scan: %lld elements exceed the 32-bit index range", (long long)n);
+    const int64_t n_blocks = (n + SCAN_TILE - 1) / SCAN_TILE;
+    if (n_blocks > 0) {
+        hipLaunchKernelGGL(scan_block_totals_kernel, dim3((uint32_t)n_blocks), dim3(SPLATAD_THREADS),
+                           0, stream, in, n, stride, as_flag, block_sums);
+        SPLATAD_LAUNCH_CHECK();
+    }
+    return launch_exclusive_scan_apply<OutT>(in, n, stride, as_flag, out, total, block_sums, stream);
 }
 
 } // namespace

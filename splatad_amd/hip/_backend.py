@@ -10,6 +10,7 @@ torch so that they live in torch's caching allocator, on torch's current stream.
 There is no CPU path: without the built library, or with non-GPU tensors, the ops raise.
 """
 import ctypes
+import weakref
 import math
 import os
 from typing import Optional
@@ -152,7 +153,11 @@ class _Ops:
     def fully_fused_projection_packed_fwd(self, means, covars, quats, scales, velocities, viewmats,
                                           Ks, image_width, image_height, linear_velocity,
                                           angular_velocity, rolling_shutter_time, eps2d, near_plane,
-                                          far_plane, radius_clip, calc_compensations):
+                                          far_plane, radius_clip, calc_compensations,
+                                          isect_grid=None):
+        """isect_grid = (tile_size, tile_width, tile_height): the counting call also counts the
+        tile intersections of the rows it keeps (no second wait for isect_tiles on them); the
+        number travels with the returned radii, see _isect()."""
         lib = load_library()
         means = _in(means, "means"); covars = _in(covars, "covars"); quats = _in(quats, "quats")
         scales = _in(scales, "scales"); velocities = _in(velocities, "velocities")
@@ -163,12 +168,23 @@ class _Ops:
         f = dict(dtype=torch.float32, device=dev)
         with torch.cuda.device(dev):
             ws = _workspace(lib.splatad_projection_packed_workspace_bytes(_u32(C), _u32(N)), dev)
-            nnz_host = _i64(0)
-            _check(lib.splatad_projection_packed_count(
-                _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
-                _p(viewmats), _p(Ks), _u32(image_width), _u32(image_height), _p(lv), _p(av), _p(rs),
-                _f32(eps2d), _f32(near_plane), _f32(far_plane), _f32(radius_clip),
-                _i32(bool(calc_compensations)), _p(ws), ctypes.byref(nnz_host), _stream(dev)))
+            nnz_host, n_isects_host = _i64(0), _i64(0)
+            head = (_u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
+                    _p(viewmats), _p(Ks), _u32(image_width), _u32(image_height), _p(lv), _p(av), _p(rs),
+                    _f32(eps2d), _f32(near_plane), _f32(far_plane), _f32(radius_clip),
+                    _i32(bool(calc_compensations)))
+            isect_ws = None
+            if isect_grid is None:
+                _check(lib.splatad_projection_packed_count(*head, _p(ws), ctypes.byref(nnz_host), _stream(dev)))
+            else:
+                # the counting call also starts the tile intersection, on the dense rows in its
+                # workspace, while the host waits for the counts; _isect() completes it
+                n_tiles = int(isect_grid[1]) * int(isect_grid[2])
+                assert n_tiles.bit_length() + int(C).bit_length() <= 32
+                isect_ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(C * N), _u32(C), _u32(n_tiles)), dev)
+                _check(lib.splatad_projection_packed_count_tiles(
+                    *head, *(_u32(v) for v in isect_grid), _p(ws), _p(isect_ws), ctypes.byref(nnz_host),
+                    ctypes.byref(n_isects_host), _stream(dev)))
             nnz = int(nnz_host.value)
             indptr = torch.empty((C + 1,), dtype=torch.int32, device=dev)
             camera_ids = torch.empty((nnz,), dtype=torch.int64, device=dev)
@@ -181,6 +197,11 @@ class _Ops:
                 _u32(C), _u32(N), _i64(nnz), _p(ws), _p(indptr), _p(camera_ids), _p(gaussian_ids),
                 _p(radii), _p(means2d), _p(depths), _p(conics), _p(comps), _p(pix_vels),
                 _stream(dev)))
+        if isect_grid is not None:
+            # valid for these very tensors as long as nobody writes to them
+            radii._splatad_isect_count = (tuple(int(v) for v in isect_grid), int(n_isects_host.value),
+                                          radii._version, weakref.ref(means2d), means2d._version,
+                                          weakref.ref(depths), depths._version, C, N, ws, isect_ws)
         return indptr, camera_ids, gaussian_ids, radii, means2d, depths, conics, comps, pix_vels
 
     def fully_fused_lidar_projection_fwd(self, means, covars, quats, scales, velocities, viewmats,
@@ -414,27 +435,48 @@ class _Ops:
         tiles_per_gauss = torch.empty(depths.shape, dtype=torch.int32, device=dev)
         count = lib.splatad_isect_lidar_tiles_count if lidar else lib.splatad_isect_tiles_count
         fill = lib.splatad_isect_lidar_tiles_fill if lidar else lib.splatad_isect_tiles_fill
+        # A packed projection that was told the tile grid has counted the intersections of these
+        # rows and started the binning on its dense copy of them (good for one call, and only for
+        # the very tensors it returned, unwritten since).
+        known = getattr(radii, "_splatad_isect_count", None) if packed and not lidar and sort else None
+        if known is not None:
+            del radii._splatad_isect_count  # the workspaces are freed with it
+            if not (known[0] == (int(grid_args[0].value), tile_w, tile_h) and known[2] == radii._version
+                    and known[3]() is means2d and known[4] == means2d._version
+                    and known[5]() is depths and known[6] == depths._version and known[7] == C):
+                known = None
         with torch.cuda.device(dev):
-            # one workspace for both calls: the counting call leaves the start of the binning in it
-            ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(total), _u32(C), _u32(n_tiles)), dev)
             # the binning knows every tile's first intersection: keep that table with the
             # ids so that isect_offset_encode() on the same, unmodified tensor is free
             offsets = (torch.empty((C, tile_h, tile_w), dtype=torch.int32, device=dev)
                        if sort else None)
-            head = (_u64(total), _u32(N), _p(camera_ids), _p(means2d), _p(radii), _p(depths))
-            tail = (_u32(C), *grid_args, _u32(tile_w), _u32(tile_h), _i32(bool(sort)))
-            n_host = _i64(0)
-            _check(count(*head, *tail, _p(tiles_per_gauss), _p(ws), ctypes.byref(n_host),
-                         _stream(dev)))
-            n_isects = int(n_host.value)
+            if known is not None:
+                n_isects, (kC, kN, packed_ws, ws) = known[1], known[7:11]  # no wait here
+            else:
+                # one workspace for both calls: the counting call leaves the start of the binning in it
+                ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(total), _u32(C), _u32(n_tiles)), dev)
+                head = (_u64(total), _u32(N), _p(camera_ids), _p(means2d), _p(radii), _p(depths))
+                tail = (_u32(C), *grid_args, _u32(tile_w), _u32(tile_h), _i32(bool(sort)))
+                n_host = _i64(0)
+                _check(count(*head, *tail, _p(tiles_per_gauss), _p(ws), ctypes.byref(n_host),
+                             _stream(dev)))
+                n_isects = int(n_host.value)
             isect_ids = torch.empty((n_isects,), dtype=torch.int64, device=dev)
             flatten_ids = torch.empty((n_isects,), dtype=torch.int32, device=dev)
-            if n_isects:
+            if n_isects and known is not None:
+                lists = _workspace(lib.splatad_isect_lists_bytes(_u64(kC * kN), _i64(n_isects)), dev)
+                _check(lib.splatad_isect_tiles_fill_packed(
+                    _u32(kC), _u32(kN), *grid_args, _u32(tile_w), _u32(tile_h), _i64(n_isects),
+                    _p(packed_ws), _p(ws), _p(lists), _p(tiles_per_gauss), _p(isect_ids),
+                    _p(flatten_ids), _p(offsets), _stream(dev)))
+            elif n_isects:
                 lists = _workspace(lib.splatad_isect_lists_bytes(_u64(total), _i64(n_isects)), dev)
                 _check(fill(*head, *tail, _i64(n_isects), _p(tiles_per_gauss), _p(ws),
                             _p(lists), _p(isect_ids), _p(flatten_ids), _p(offsets), _stream(dev)))
             else:
                 offsets = None
+                if known is not None:
+                    tiles_per_gauss.zero_()
             if offsets is not None:
                 isect_ids._splatad_tile_offsets = (offsets, isect_ids._version)
         return tiles_per_gauss, isect_ids, flatten_ids

@@ -132,9 +132,15 @@ def fully_fused_projection(
     packed: bool = False,
     sparse_grad: bool = False,
     calc_compensations: bool = False,
+    isect_grid: Optional[Tuple[int, int, int]] = None,
 ):
     """Projects Gaussians onto C pinhole image planes (EWA splatting) with rolling-shutter
     pixel velocities.
+
+    `isect_grid` = (tile_size, tile_width, tile_height) (not in the reference; packed only) says
+    that `isect_tiles` on that grid follows: the projection, which waits for its row count
+    anyway, then counts the tile intersections of the rows it keeps as well, and `isect_tiles`
+    on the returned (unmodified) `means2d` and `radii` starts without a wait of its own.
 
     Returns, unpacked: (radii int32[C,N,2], means2d[C,N,2], depths[C,N], conics[C,N,3],
     compensations[C,N] | None, pix_vels[C,N,2]); a zero radius marks a culled Gaussian.
@@ -157,7 +163,7 @@ def fully_fused_projection(
         far_plane, radius_clip,
     )
     if packed:
-        return _FullyFusedProjectionPacked.apply(*args, sparse_grad, calc_compensations)
+        return _FullyFusedProjectionPacked.apply(*args, sparse_grad, calc_compensations, isect_grid)
     return _FullyFusedProjection.apply(*args, calc_compensations)
 
 
@@ -649,12 +655,12 @@ class _FullyFusedProjectionPacked(torch.autograd.Function):
     @staticmethod
     def forward(ctx, means, covars, quats, scales, velocities, viewmats, Ks, width, height,
                 linear_velocity, angular_velocity, rolling_shutter_time, eps2d, near_plane,
-                far_plane, radius_clip, sparse_grad, calc_compensations):
+                far_plane, radius_clip, sparse_grad, calc_compensations, isect_grid=None):
         (indptr, camera_ids, gaussian_ids, radii, means2d, depths, conics, compensations,
          pix_vels) = _make_lazy_hip_func("fully_fused_projection_packed_fwd")(
             means, covars, quats, scales, velocities, viewmats, Ks, width, height,
             linear_velocity, angular_velocity, rolling_shutter_time, eps2d, near_plane, far_plane,
-            radius_clip, calc_compensations)
+            radius_clip, calc_compensations, isect_grid)
         if not calc_compensations:
             compensations = None
         ctx.save_for_backward(camera_ids, gaussian_ids, means, covars, quats, scales, velocities,
@@ -697,7 +703,7 @@ class _FullyFusedProjectionPacked(torch.autograd.Function):
                 v_scales = coo(v_scales, scales)
         grads = _gate((v_means, v_covars, v_quats, v_scales, v_velocities, v_viewmats),
                       ctx.needs_input_grad[:6])
-        return grads + (None,) * 12
+        return grads + (None,) * 13
 
 
 class _RasterizeToPixels(torch.autograd.Function):

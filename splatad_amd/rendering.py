@@ -160,12 +160,16 @@ def rasterization(
         ), colors.shape
         assert (sh_degree + 1) ** 2 <= colors.shape[-2], colors.shape
 
-    # 1. projection
+    # 1. projection (packed: it also counts the intersections with the tile grid of step 2,
+    # so that the host waits for the GPU once per call, not twice)
+    tile_width = math.ceil(width / float(tile_size))
+    tile_height = math.ceil(height / float(tile_size))
     proj = fully_fused_projection(
         means, None, quats, scales, velocities, viewmats, Ks, width, height, linear_velocity,
         angular_velocity, rolling_shutter_time, eps2d=eps2d, packed=packed, near_plane=near_plane,
         far_plane=far_plane, radius_clip=radius_clip, sparse_grad=sparse_grad,
         calc_compensations=(rasterize_mode == "antialiased"),
+        isect_grid=(tile_size, tile_width, tile_height) if packed else None,
     )
     if packed:
         camera_ids, gaussian_ids, radii, means2d, depths, conics, compensations, pix_vels = proj
@@ -174,17 +178,13 @@ def rasterization(
         camera_ids, gaussian_ids = None, None
 
     def per_row_opacities():
-        # Compositing is the first to need these.  The packed gather is enqueued behind the
-        # intersection: ahead of it, it would only add host time between the two waits for
-        # counts, during which the GPU idles.
-        # [nnz], or [C, N]: a view, copied by the first operator that needs it when C > 1
+        # Compositing is the first to need these: [nnz], or [C, N] (a view, copied by the first
+        # operator that needs it when C > 1).
         o = opacities[gaussian_ids] if packed else opacities.expand(C, -1)
         return o if compensations is None else o * compensations
 
     # 2. tile intersection, sort, offsets
     beside = _Beside(means.device)  # fork: everything the colours need is enqueued
-    tile_width = math.ceil(width / float(tile_size))
-    tile_height = math.ceil(height / float(tile_size))
     fused_colors = sh_degree is not None and not viewmats.requires_grad
     depth_appended = fused_colors and render_mode in ["RGB+D", "RGB+ED"]
 
@@ -194,26 +194,27 @@ def rasterization(
                                      depths if depth_appended else None, camera_ids,
                                      gaussian_ids, launch_context=beside)
 
-    # The colours run on a helper stream beside the intersection.  Unpacked, they are enqueued
-    # behind it: the host is far ahead of the GPU, and the kernel then meets the segment sort,
-    # whose long workgroups leave most of the GPU idle (enqueued first, it would compete with
-    # the binning chain that everything else waits for).  Packed, the host has just waited for
-    # the projection's row count and will wait again in the intersection, the GPU idles in
-    # between, and a kernel enqueued after the intersection would find the sort over: there
-    # the colours go first.
-    if fused_colors and packed:
-        colors = fused_view_colors()
+    # The colours run on a helper stream beside the intersection, enqueued behind it: the kernel
+    # then meets the segment sort, whose long workgroups leave part of the GPU idle (enqueued
+    # first, it would compete with the binning chain that everything else waits for, and its
+    # launch would stand between the host and the launches the GPU is waiting for).
     tiles_per_gauss, isect_ids, flatten_ids = isect_tiles(
         means2d, radii, depths, tile_size, tile_width, tile_height, packed=packed, n_cameras=C,
         camera_ids=camera_ids, gaussian_ids=gaussian_ids,
     )
     isect_offsets = isect_offset_encode(isect_ids, C, tile_width, tile_height)
-    opacities = per_row_opacities()
+    if packed:
+        # the gather (and the product with the compensations) goes beside the sort too:
+        # on the caller's stream it would stand alone between the sort and the compositing
+        with beside:
+            opacities = per_row_opacities()
+        beside.join(opacities)
+    else:
+        opacities = per_row_opacities()
 
     # 3. per-(camera, Gaussian) colours
     if fused_colors:
-        if not packed:
-            colors = fused_view_colors()
+        colors = fused_view_colors()
         beside.join(colors)
     elif sh_degree is None:
         if packed:

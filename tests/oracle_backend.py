@@ -31,7 +31,8 @@ class OracleOps:
         return tuple(_t(o) for o in out)
 
     def fully_fused_projection_packed_fwd(self, means, covars, quats, scales, velocities, viewmats, Ks,
-                                          W, H, lin, ang, rs, eps2d, near, far, radius_clip, calc_comp):
+                                          W, H, lin, ang, rs, eps2d, near, far, radius_clip, calc_comp,
+                                          isect_grid=None):
         radii, m2, d, con, comp, pv = self.fully_fused_projection_fwd(
             means, covars, quats, scales, velocities, viewmats, Ks, W, H, lin, ang, rs, eps2d, near, far,
             radius_clip, calc_comp)

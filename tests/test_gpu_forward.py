@@ -109,6 +109,62 @@ def test_projection_camera(use_covars, use_vel, comp):
             np.testing.assert_array_equal(to_np(a), to_np(b)[sel[:, 0], sel[:, 1]])
 
 
+@pytest.mark.parametrize("C,N,W,H,ts", [(3, 20000, 320, 240, 16), (1, 5000, 200, 120, 8), (2, 300, 64, 48, 16)])
+def test_packed_projection_counts_the_intersections_of_its_rows(C, N, W, H, ts):
+    """isect_grid: the packed projection returns rows that carry the number of their tile
+    intersections; isect_tiles on those tensors skips its own count and gives the same lists;
+    writing to the tensors, or another grid, makes it count again."""
+    from splatad_amd import fully_fused_projection, isect_tiles
+    rng, means, quats, scales, vel = _gaussians(N, 17)
+    viewmats, Ks = _cameras(rng, C, W, H)
+    lin = rng.normal(size=(C, 3)).astype(np.float32)
+    ang = (rng.normal(size=(C, 3)) * 0.3).astype(np.float32)
+    rs = np.linspace(0.0, 0.03, C).astype(np.float32)
+    t = [to_dev(a) if isinstance(a, np.ndarray) else a
+         for a in (means, None, quats, scales, vel, viewmats, Ks, W, H, lin, ang, rs)]
+    kw = dict(eps2d=0.3, near_plane=0.5, far_plane=4.5, radius_clip=0.0, packed=True)
+    tw, th = math.ceil(W / ts), math.ceil(H / ts)
+    plain = fully_fused_projection(*t, **kw)
+
+    def lists(rows, ts=ts, tw=tw, th=th):
+        cam, gid, radii, means2d, depths = rows[:5]
+        return isect_tiles(means2d, radii, depths, ts, tw, th, packed=True, n_cameras=C,
+                           camera_ids=cam, gaussian_ids=gid)
+
+    def oracle_lists(rows, ts=ts, tw=tw, th=th):
+        cam, gid, radii, means2d, depths = rows[:5]
+        return oracle.isect_tiles(to_np(means2d), to_np(radii), to_np(depths), ts, tw, th, n_cameras=C,
+                                  camera_ids=to_np(cam))
+
+    want = lists(plain)  # counts by itself
+    hinted = fully_fused_projection(*t, isect_grid=(ts, tw, th), **kw)
+    for a, b in zip(plain, hinted):
+        assert (a is None and b is None) or torch.equal(a, b)
+    grid, n_known = hinted[2]._splatad_isect_count[:2]
+    assert grid == (ts, tw, th)
+    assert int(want[0].sum().item()) == n_known == want[1].numel()
+    got = lists(hinted)  # completes what the projection started
+    assert not hasattr(hinted[2], "_splatad_isect_count")  # good for one call
+    for a, b in zip(want, got):
+        assert torch.equal(a, b)
+    for a, b in zip(got, oracle_lists(hinted)):
+        np.testing.assert_array_equal(to_np(a), b)
+    for a, b in zip(want, lists(hinted)):  # a second call counts by itself
+        assert torch.equal(a, b)
+    # another grid: the count does not apply
+    hinted = fully_fused_projection(*t, isect_grid=(ts, tw, th), **kw)
+    g2 = dict(ts=2 * ts, tw=math.ceil(W / (2 * ts)), th=math.ceil(H / (2 * ts)))
+    for a, b in zip(lists(hinted, **g2), oracle_lists(hinted, **g2)):
+        np.testing.assert_array_equal(to_np(a), b)
+    # rows written to after the projection: counted again
+    hinted = fully_fused_projection(*t, isect_grid=(ts, tw, th), **kw)
+    hinted[2][: hinted[2].shape[0] // 2] = 0
+    changed = lists(hinted)
+    assert changed[1].numel() < n_known
+    for a, b in zip(changed, oracle_lists(hinted)):
+        np.testing.assert_array_equal(to_np(a), b)
+
+
 @pytest.mark.parametrize("use_covars", [False, True])
 @pytest.mark.parametrize("use_vel", [False, True])
 def test_projection_lidar(use_covars, use_vel):
