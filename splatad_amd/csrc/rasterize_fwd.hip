@@ -349,8 +349,9 @@ struct PointArgs {
 // stores the 32 features of a point with one 128-byte store.
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// Four wavefronts per SIMD: the 1024 tiles of a 128 x 2048 sweep then run in one round.
 template <int CH, bool MATRIX>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4)))
 rasterize_to_points_fwd_kernel(PointArgs a) {
     static_assert(!MATRIX || CH == 32 || CH == 33, "the matrix path accumulates 32 channels (+1)");
     extern __shared__ float4 lds4[];
@@ -366,6 +367,9 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
     constexpr int RECORD = 2; // float4 per Gaussian
     float4 *s_rec = lds4;
     int32_t *s_gid = reinterpret_cast<int32_t *>(lds4 + (size_t)RECORD * blockDim.x * blockDim.y);
+    // per wavefront: {position in the batch, id} of the staged Gaussians that pass its footprint test
+    uint2 *s_surv = reinterpret_cast<uint2 *>(s_gid + block_size) +
+                    (size_t)((threadIdx.y * blockDim.x + threadIdx.x) / SPLATAD_WAVE) * block_size;
 
     const uint32_t tiles_per_cam = a.grid_w * a.grid_h;
     const uint32_t cam = blockIdx.x / tiles_per_cam;
@@ -486,92 +490,103 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
         __syncthreads();
 
         const uint32_t batch_size = min(block_size, (uint32_t)range_end - batch_start);
+        // The footprint test runs over the whole batch first, 64 staged Gaussians per round; a
+        // survivor's position in the batch and its id go to a list that belongs to the wavefront.
+        uint32_t n_surv = 0; // uniform
         for (uint32_t base = 0; base < batch_size && alive_bits != 0; base += SPLATAD_WAVE) {
             bool keep = base + lane < batch_size, unfolded_ok = true;
             if (keep) keep = cull.may_touch(s_rec[RECORD * (base + lane)], s_rec[RECORD * (base + lane) + 1], unfolded_ok);
-            uint64_t todo = wave_ballot(keep);
-            const uint64_t folded = wave_ballot(keep && !unfolded_ok);
-            // The Gaussians that pass the footprint test are taken four at a time: list
-            // positions (scalar), ids from LDS, payloads from global memory and staged
-            // records from LDS are requested phase by phase for all four, so that the requests
-            // of a phase are in flight together; then the four are composited one after the
-            // other.  One at a time, a wavefront waits for a load from global memory per
-            // Gaussian, ten times longer than it works on it.  Slots beyond the last
-            // Gaussian repeat it.
-            constexpr int K = 4;
-            while (todo) {
-                uint32_t ts[K];
-                bool fold[K], have[K];
-                uint32_t last_t = base, last_bit = 0;
+            const uint64_t kept = wave_ballot(keep);
+            if (keep)
+                s_surv[n_surv + (uint32_t)__popcll(kept & ((1ull << lane) - 1ull))] =
+                    make_uint2((base + lane) | (unfolded_ok ? 0u : 0x80000000u), (uint32_t)s_gid[base + lane]);
+            n_surv += (uint32_t)__popcll(kept);
+        }
+        // the list is written and read by the same wavefront, whose LDS operations complete in
+        // order; the fences keep the compiler from moving the reads above the writes
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // The survivors are composited four at a time.  What a Gaussian needs beyond its staged
+        // record comes from global memory, a wait ten times longer than the work on the
+        // Gaussian: a group's words are requested before the group ahead of it is composited
+        // (two groups in two sets of registers, taking turns), so that the wait overlaps that
+        // work.  Slots beyond the last survivor repeat it.
+        constexpr int K = 4;
+        struct Group {
+            uint32_t ts[K]; // position in the batch, bit 31: the offset needs folding (uniform)
+            float pay[K];
+        };
+        auto request = [&](Group &g, uint32_t first) {
 #pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    have[k] = todo != 0; // uniform
-                    if (have[k]) {
-                        last_bit = (uint32_t)__ffsll((unsigned long long)todo) - 1u;
-                        todo &= todo - 1;
-                        last_t = base + last_bit;
-                    }
-                    ts[k] = last_t;
-                    fold[k] = (folded >> last_bit) & 1ull;
+            for (int k = 0; k < K; ++k) {
+                const uint2 e = s_surv[min(first + (uint32_t)k, n_surv - 1u)];
+                g.ts[k] = (uint32_t)__builtin_amdgcn_readfirstlane((int)e.x);
+                g.pay[k] = payload_at[(size_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)e.y) * payload_step];
+            }
+        };
+        auto composite = [&](const Group &g, uint32_t count) {
+            float4 uvs[K], cons[K];
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                uvs[k] = s_rec[RECORD * (g.ts[k] & 0x7FFFFFFFu)];
+                cons[k] = s_rec[RECORD * (g.ts[k] & 0x7FFFFFFFu) + 1];
+            }
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                if ((uint32_t)k >= count || alive_bits == 0) break; // uniform
+                const float4 uv = uvs[k], con = cons[k];
+                float dx = gaussian_offset(uv.x, uv.z, roll, rx);
+                float dy = gaussian_offset(uv.y, uv.w, roll, ry);
+                if (g.ts[k] >> 31) { // uniform, rare: half a turn away from the tile
+                    dx = angle_difference(fmaf(roll, uv.z, uv.x), rx);
+                    dy = angle_difference(fmaf(roll, uv.w, uv.y), ry);
                 }
-                int32_t ids[K];
+                const float power = gaussian_power(con, dx, dy);
+                const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
+                const float weight = alpha * T;
+                const float next_T = transmittance_behind(T, alpha);
+                const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
+                                            wave_ballot(!(alpha < 1.f / 255.f));
+                const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
+                const uint64_t take_bits = valid_bits & ~stop_bits;
+                alive_bits &= ~stop_bits;
+                if (take_bits != 0) {
+                    const bool take = wave_lanes(take_bits);
+                    const float vis = take ? weight : 0.f;
+                    const int word = __float_as_int(g.pay[k]);
+                    const float4 ext = make_float4(__int_as_float(__builtin_amdgcn_readlane(word, 33)),
+                                                   __int_as_float(__builtin_amdgcn_readlane(word, 34)),
+                                                   __int_as_float(__builtin_amdgcn_readlane(word, 35)),
+                                                   __int_as_float(__builtin_amdgcn_readlane(word, 36)));
+                    if constexpr (MATRIX) {
+                        if constexpr (CH == 33) out[0] += __int_as_float(__builtin_amdgcn_readlane(word, 32)) * vis;
+                        if (pair_open) add_pair(pair_weight, vis, pair_feature, g.pay[k]);
+                        else { pair_weight = vis; pair_feature = g.pay[k]; }
+                        pair_open = !pair_open;
+                    } else { // accumulators beyond n_ch repeat the last channel and are never stored
 #pragma unroll
-                for (int k = 0; k < K; ++k) ids[k] = s_gid[ts[k]];
-                float pay[K];
-#pragma unroll
-                for (int k = 0; k < K; ++k)
-                    pay[k] = payload_at[(size_t)(uint32_t)__builtin_amdgcn_readfirstlane(ids[k]) * payload_step];
-                float4 uvs[K], cons[K];
-#pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    uvs[k] = s_rec[RECORD * ts[k]];
-                    cons[k] = s_rec[RECORD * ts[k] + 1];
-                }
-#pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    if (!have[k] || alive_bits == 0) break; // uniform
-                    const float4 uv = uvs[k], con = cons[k];
-                    float dx = gaussian_offset(uv.x, uv.z, roll, rx);
-                    float dy = gaussian_offset(uv.y, uv.w, roll, ry);
-                    if (fold[k]) { // uniform, rare: half a turn away from the tile
-                        dx = angle_difference(fmaf(roll, uv.z, uv.x), rx);
-                        dy = angle_difference(fmaf(roll, uv.w, uv.y), ry);
+                        for (int c = 0; c < CH; ++c) out[c] += __int_as_float(__builtin_amdgcn_readlane(word, c)) * vis;
                     }
-                    const float power = gaussian_power(con, dx, dy);
-                    const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
-                    const float weight = alpha * T;
-                    const float next_T = transmittance_behind(T, alpha);
-                    const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
-                                                wave_ballot(!(alpha < 1.f / 255.f));
-                    const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
-                    const uint64_t take_bits = valid_bits & ~stop_bits;
-                    alive_bits &= ~stop_bits;
-                    if (take_bits != 0) {
-                        const bool take = wave_lanes(take_bits);
-                        const float vis = take ? weight : 0.f;
-                        const int word = __float_as_int(pay[k]);
-                        const float4 ext = make_float4(__int_as_float(__builtin_amdgcn_readlane(word, 33)),
-                                                       __int_as_float(__builtin_amdgcn_readlane(word, 34)),
-                                                       __int_as_float(__builtin_amdgcn_readlane(word, 35)),
-                                                       __int_as_float(__builtin_amdgcn_readlane(word, 36)));
-                        if constexpr (MATRIX) {
-                            if constexpr (CH == 33) out[0] += __int_as_float(__builtin_amdgcn_readlane(word, 32)) * vis;
-                            if (pair_open) add_pair(pair_weight, vis, pair_feature, pay[k]);
-                            else { pair_weight = vis; pair_feature = pay[k]; }
-                            pair_open = !pair_open;
-                        } else { // accumulators beyond n_ch repeat the last channel and are never stored
-#pragma unroll
-                            for (int c = 0; c < CH; ++c) out[c] += __int_as_float(__builtin_amdgcn_readlane(word, c)) * vis;
-                        }
-                        const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
-                        depth_extra += extra * vis;
-                        if (take && T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
-                        if (take && a.compute_alpha_sum && ext.w < pz - a.threshold) asum += alpha;
-                        cur_idx = take ? batch_start + ts[k] : cur_idx;
-                        T -= vis;
-                    }
+                    const float extra = ext.y * dx + ext.z * dy + ext.x * roll;
+                    depth_extra += extra * vis;
+                    if (take && T > 0.5f && next_T <= 0.5f) median = ext.w + extra;
+                    if (take && a.compute_alpha_sum && ext.w < pz - a.threshold) asum += alpha;
+                    cur_idx = take ? batch_start + (g.ts[k] & 0x7FFFFFFFu) : cur_idx;
+                    T -= vis;
                 }
-                if (alive_bits == 0) break;
+            }
+        };
+        if (n_surv != 0) {
+            Group even, odd;
+            request(even, 0);
+            // (a request beyond the list repeats the last survivor: issued all the same, so that
+            // the number of loads in flight at every wait is known when the kernel is compiled)
+            for (uint32_t first = 0; first < n_surv && alive_bits != 0; first += 2 * K) { // uniform
+                request(odd, first + K);
+                composite(even, min((uint32_t)K, n_surv - first));
+                if (first + K >= n_surv || alive_bits == 0) break;
+                request(even, first + 2 * K);
+                composite(odd, min((uint32_t)K, n_surv - first - K));
             }
         }
     }
@@ -669,7 +684,9 @@ static int launch_pixels(const PixelArgs &a, dim3 grid, dim3 block, hipStream_t 
 
 template <int CH>
 static int launch_points(const PointArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
-    const size_t lds = (size_t)block.x * block.y * (2 * 16 + 4); // two float4 and the id per Gaussian
+    // two float4 and the id per staged Gaussian, and a survivor list of that length per wavefront
+    const size_t threads = (size_t)block.x * block.y;
+    const size_t lds = threads * (2 * 16 + 4) + (threads / SPLATAD_WAVE) * threads * 8;
     if constexpr (CH == 32 || CH == 33) {
         // the matrix-core path: every channel of the kernel in use
         if (a.n_ch == (uint32_t)CH) {
