@@ -69,7 +69,9 @@ rasterize_bwd_kernel(BwdArgs a) {
     // the workgroup is one-dimensional and padded to whole wavefronts: the wavefront
     // reductions below need all 64 lanes; lanes beyond the tile own no pixel
     const uint32_t block_size = blockDim.x;
-    constexpr int RECORD = LIDAR ? 3 : 2; // {x, y, vx, vy}, staged exponent, lidar extras
+    // {x, y, vx, vy}, staged exponent, then the lidar extras or, for cameras, the polynomial of
+    // the exponent as the forward kernel stages it (same functions, same bits)
+    constexpr int RECORD = LIDAR ? 3 : 4;
     constexpr int GEO = LIDAR ? G_COUNT : G_VELZ;
     constexpr int ACC = CH + GEO;
     constexpr int NA = reduce_first(ACC), NB = reduce_second(ACC), NV = NA + NB;
@@ -110,6 +112,16 @@ rasterize_bwd_kernel(BwdArgs a) {
     }
     const bool inside = in_image && pz > 0.f;
     const uint64_t inside_bits = wave_ballot(inside);
+    // Cameras: alpha comes from the forward kernel's polynomial in tile-centred pixel
+    // coordinates, evaluated by the same function on the same staged coefficients, so that this
+    // pass takes the forward pass's alpha >= 1/255 and sigma < 0 decisions bit for bit; the
+    // offsets to the Gaussian's centre are still needed, for the gradients.
+    TileFrame frame = {};
+    PixelConstants pc = {};
+    if (!LIDAR) {
+        frame = tile_frame(tile_id % a.grid_w, tile_id / a.grid_w, a.tile_w_px, a.rs_time[cam], a.H);
+        pc.init(px, py, frame);
+    }
 
     // lidar: angles relative to the tile's first valid point, as in the forward kernel
     float ref_x = 0.f, ref_y = 0.f;
@@ -245,6 +257,12 @@ rasterize_bwd_kernel(BwdArgs a) {
                 rec[RECORD - 1] = make_float4(now.v[2], now.dc.x, now.dc.y, now.depth_col);
             } else {
                 rec[0] = make_float4(now.xy.x, now.xy.y, now.v[0], now.v[1]);
+                float4 pa, pb;
+                pixel_polynomial(frame, now.xy, make_float2(now.v[0], now.v[1]), now.cn[0], now.cn[1], now.cn[2],
+                                 now.opac, pa, pb);
+                rec[2] = pa;
+                // {cXY, cYY, the exponent above which sigma < 0 (+inf where that cannot be), -}
+                rec[3] = make_float4(pb.x, pb.y, pb.z == pb.z ? INFINITY : pb.w, 0.f);
             }
             rec[1] = staged_exponent(now.cn[0], now.cn[1], now.cn[2], now.opac);
             s_aux[tr] = make_float2(__int_as_float(g_now), now.opac > 0.f ? 1.0f / now.opac : 0.f); // finite
@@ -279,12 +297,22 @@ rasterize_bwd_kernel(BwdArgs a) {
                     dx = angle_difference(fmaf(roll, xyv.z, xyv.x), px);
                     dy = angle_difference(fmaf(roll, xyv.w, xyv.y), py);
                 }
-                const float power = gaussian_power(e, dx, dy);
-                const float au = __builtin_amdgcn_exp2f(e.w - power); // opacity * exp(-sigma)
+                float au; // opacity * exp(-sigma)
+                bool sigma_ok;
+                if constexpr (LIDAR) {
+                    const float power = gaussian_power(e, dx, dy);
+                    au = __builtin_amdgcn_exp2f(e.w - power);
+                    sigma_ok = !(power < 0.f);
+                } else {
+                    const float4 pb = rec[3];
+                    const float ex = pixel_exponent(rec[2], pb.x, pb.y, pc);
+                    au = __builtin_amdgcn_exp2f(ex);
+                    sigma_ok = !(ex > pb.z);
+                }
                 const float alpha = fminf(0.999f, au);
                 // the lanes that took this Gaussian in the forward pass, by scalar logic on lane masks
                 const uint64_t valid_bits = inside_bits & wave_ballot(batch_end - t <= bin_final) &
-                                            wave_ballot(!(power < 0.f)) & wave_ballot(!(alpha < 1.f / 255.f));
+                                            wave_ballot(sigma_ok) & wave_ballot(!(alpha < 1.f / 255.f));
                 if (valid_bits == 0) continue;
                 const bool valid = wave_lanes(valid_bits);
 
@@ -446,7 +474,7 @@ static inline int pick_width(uint32_t n) {
 
 template <int CH, bool LIDAR>
 static int launch_bwd(BwdArgs a, dim3 grid, dim3 block, hipStream_t stream) {
-    const size_t per_gaussian = ((LIDAR ? 48 : 32) + 8) + 4 * CH + 4 * (CH + (LIDAR ? G_COUNT : G_VELZ));
+    const size_t per_gaussian = ((LIDAR ? 48 : 64) + 8) + 4 * CH + 4 * (CH + (LIDAR ? G_COUNT : G_VELZ));
     // Batches of the whole workgroup, unless that leaves fewer than four workgroups to a compute
     // unit (160 KB of LDS): a lidar sweep's 1024 tiles then run all at once instead of in two
     // rounds (with 33 channels: 104 Gaussians per batch, 0.39 ms instead of 0.51 ms with 128).

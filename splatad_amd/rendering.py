@@ -203,9 +203,10 @@ def rasterization(
         camera_ids=camera_ids, gaussian_ids=gaussian_ids,
     )
     isect_offsets = isect_offset_encode(isect_ids, C, tile_width, tile_height)
-    if packed:
-        # the gather (and the product with the compensations) goes beside the sort too:
-        # on the caller's stream it would stand alone between the sort and the compositing
+    if packed and not opacities.requires_grad:
+        # the gather (and the product with the compensations) goes beside the sort too: on the
+        # caller's stream it would stand alone between the sort and the compositing.  (Not for a
+        # leaf that takes a gradient: autograd would accumulate it on the helper stream.)
         with beside:
             opacities = per_row_opacities()
         beside.join(opacities)
