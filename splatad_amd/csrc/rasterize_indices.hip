@@ -101,11 +101,21 @@ rasterize_to_indices_kernel(IndexArgs a) {
         any_point ? (uint32_t)(list_end - list_start + block_size - 1) / block_size : 0u;
     const uint32_t batch_end = min(a.range_end, num_batches);
 
-    WaveCull cull;
+    // Cameras: the exponent is the polynomial in tile-centred pixel coordinates that the
+    // compositing kernels stage and evaluate (same functions, same bits, hence the same alpha >=
+    // 1/255 and sigma < 0 decisions); the footprint test works on the polynomial too.
+    WaveBox box;
     WavePointCull pcull;
+    TileFrame frame = {};
+    PixelConstants pc = {};
     const bool full = block_size % SPLATAD_WAVE == 0;
-    if (LIDAR) pcull.init(inside, px, py, roll, full);
-    else cull.init(px, py, roll, full);
+    if (LIDAR) {
+        pcull.init(inside, px, py, roll, full);
+    } else {
+        frame = tile_frame(tile_id % a.grid_w, tile_id / a.grid_w, a.tile_width, a.rs_time[cam], a.H);
+        pc.init(px, py, frame);
+        box.init(pc.X, pc.X, pc.Y, pc.Y, full);
+    }
 
     float T = inside ? a.transmittances[pix] : 0.f;
     int64_t *out_g = nullptr, *out_i = nullptr;
@@ -126,10 +136,15 @@ rasterize_to_indices_kernel(IndexArgs a) {
             const float2 xy = reinterpret_cast<const float2 *>(a.means2d)[g];
             const float *v = a.pix_vels + (size_t)g * (LIDAR ? 3 : 2);
             const float *cn = a.conics + (size_t)g * 3;
-            s_rec[2 * tr] = LIDAR ? make_float4(angle_difference(xy.x, ref_x),
-                                                angle_difference(xy.y, ref_y), v[0], v[1])
-                                  : make_float4(xy.x, xy.y, v[0], v[1]);
-            s_rec[2 * tr + 1] = staged_exponent(cn[0], cn[1], cn[2], a.opacities[g]);
+            if (LIDAR) {
+                s_rec[2 * tr] = make_float4(angle_difference(xy.x, ref_x), angle_difference(xy.y, ref_y), v[0], v[1]);
+                s_rec[2 * tr + 1] = staged_exponent(cn[0], cn[1], cn[2], a.opacities[g]);
+            } else {
+                float4 pa, pb;
+                pixel_polynomial(frame, xy, make_float2(v[0], v[1]), cn[0], cn[1], cn[2], a.opacities[g], pa, pb);
+                s_rec[2 * tr] = pa;
+                s_rec[2 * tr + 1] = pb;
+            }
             s_id[tr] = (int32_t)((uint32_t)g % a.N);
         }
         __syncthreads();
@@ -139,7 +154,7 @@ rasterize_to_indices_kernel(IndexArgs a) {
             bool keep = base + lane < batch_size, unfolded_ok = true;
             if (keep) {
                 const float4 r0 = s_rec[2 * (base + lane)], r1 = s_rec[2 * (base + lane) + 1];
-                keep = LIDAR ? pcull.may_touch(r0, r1, unfolded_ok) : cull.may_touch(r0, r1);
+                keep = LIDAR ? pcull.may_touch(r0, r1, unfolded_ok) : box.may_touch(r0, r1);
             }
             uint64_t todo = wave_ballot(keep);
             const uint64_t folded = LIDAR ? wave_ballot(keep && !unfolded_ok) : 0ull;
@@ -149,16 +164,25 @@ rasterize_to_indices_kernel(IndexArgs a) {
                 todo &= todo - 1;
                 const float4 xyv = s_rec[2 * t];
                 const float4 con = s_rec[2 * t + 1];
-                float dx = gaussian_offset(xyv.x, xyv.z, roll, px);
-                float dy = gaussian_offset(xyv.y, xyv.w, roll, py);
-                if (LIDAR && ((folded >> bit) & 1ull)) { // uniform, rare: half a turn away
-                    dx = angle_difference(fmaf(roll, xyv.z, xyv.x), px);
-                    dy = angle_difference(fmaf(roll, xyv.w, xyv.y), py);
+                float alpha;
+                bool sigma_ok;
+                if constexpr (LIDAR) {
+                    float dx = gaussian_offset(xyv.x, xyv.z, roll, px);
+                    float dy = gaussian_offset(xyv.y, xyv.w, roll, py);
+                    if ((folded >> bit) & 1ull) { // uniform, rare: half a turn away
+                        dx = angle_difference(fmaf(roll, xyv.z, xyv.x), px);
+                        dy = angle_difference(fmaf(roll, xyv.w, xyv.y), py);
+                    }
+                    const float power = gaussian_power(con, dx, dy);
+                    alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
+                    sigma_ok = !(power < 0.f);
+                } else { // xyv, con hold the polynomial {c0, cX, cY, cXX}, {cXY, cYY, X* or NaN, Y* or L}
+                    const float ex = pixel_exponent(xyv, con.x, con.y, pc);
+                    alpha = fminf(0.999f, __builtin_amdgcn_exp2f(ex));
+                    sigma_ok = !(ex > (con.z == con.z ? INFINITY : con.w));
                 }
-                const float power = gaussian_power(con, dx, dy);
-                const float alpha = fminf(0.999f, __builtin_amdgcn_exp2f(con.w - power));
                 const float next_T = transmittance_behind(T, alpha); // as in the compositing kernels
-                const uint64_t valid_bits = alive_bits & wave_ballot(!(power < 0.f)) &
+                const uint64_t valid_bits = alive_bits & wave_ballot(sigma_ok) &
                                             wave_ballot(!(alpha < 1.f / 255.f));
                 const uint64_t stop_bits = valid_bits & wave_ballot(next_T <= 1e-4f);
                 alive_bits &= ~stop_bits;
