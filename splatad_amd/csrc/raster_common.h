@@ -82,8 +82,14 @@ struct WaveCull {
     float roll_mid, roll_half;
 
     __device__ __forceinline__ void init(float px, float py, float roll, bool full_wavefront) {
+        init(px, py, py, roll, roll, full_wavefront);
+    }
+    // a lane with several pixels in one column: rows py_a .. py_b, factors roll_a .. roll_b
+    __device__ __forceinline__ void init(float px, float py_a, float py_b, float roll_a, float roll_b,
+                                         bool full_wavefront) {
         enabled = full_wavefront;
-        float x_lo = px, x_hi = px, y_lo = py, y_hi = py, r_lo = roll, r_hi = roll;
+        float x_lo = px, x_hi = px, y_lo = fminf(py_a, py_b), y_hi = fmaxf(py_a, py_b);
+        float r_lo = fminf(roll_a, roll_b), r_hi = fmaxf(roll_a, roll_b);
         if (enabled) {
 #pragma unroll
             for (int off = 32; off > 0; off >>= 1) {

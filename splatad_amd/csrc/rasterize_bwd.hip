@@ -59,9 +59,14 @@ enum { G_CONIC = 0, G_XY = 3, G_ABS = 5, G_VEL = 7, G_OPAC = 9, G_VELZ = 10, G_D
 constexpr int reduce_first(int n) { return n <= 24 ? 16 : (n <= 48 ? 32 : 64); }
 constexpr int reduce_second(int n) { return n <= 16 ? 0 : (n <= 24 ? 8 : (n <= 32 ? 0 : (n <= 48 ? 16 : 0))); }
 
-template <int CH, bool LIDAR>
+// PPL: pixels per lane.  Two for camera tiles that make whole wavefronts of 8 x 16 pixels (rows y
+// and y + 8 of a column, as in the forward kernel) and few channels: the wavefront reduction of
+// the per-Gaussian gradients, about 40 of the 110 vector instructions of a (wavefront, Gaussian)
+// step, is then paid once per 128 pixels, and a Gaussian is fetched from the LDS half as often.
+template <int CH, bool LIDAR, int PPL>
 __global__ void __launch_bounds__(256)
 rasterize_bwd_kernel(BwdArgs a) {
+    static_assert(PPL == 1 || (PPL == 2 && !LIDAR), "two pixels per lane are a camera layout");
     extern __shared__ float4 lds4[];
     __shared__ int32_t s_block_final;
     __shared__ uint32_t s_ref_thread;
@@ -90,37 +95,52 @@ rasterize_bwd_kernel(BwdArgs a) {
     const uint32_t tr = threadIdx.x;
     const int lane = tr & (SPLATAD_WAVE - 1);
     uint32_t lx, ly;
-    if (LIDAR) point_of_lane(a.tile_w_px, a.tile_h_px, tr, lx, ly);
-    else pixel_of_lane(a.tile_w_px, tr, lx, ly);
-    const uint32_t i = (tile_id / a.grid_w) * a.tile_h_px + ly;
-    const uint32_t j = (tile_id % a.grid_w) * a.tile_w_px + lx;
-
-    const bool in_image = (tr < a.tile_w_px * a.tile_h_px && i < a.H && j < a.W);
-    const size_t pix = in_image ? ((size_t)cam * a.H + i) * a.W + j : 0;
-    float px, py, pz = 1.f, roll;
     if (LIDAR) {
-        px = py = roll = 0.f;
-        pz = 0.f;
-        if (in_image) {
-            const float4 p = reinterpret_cast<const float4 *>(a.raster_pts)[pix];
-            px = p.x; py = p.y; pz = p.z; roll = p.w;
-        }
+        point_of_lane(a.tile_w_px, a.tile_h_px, tr, lx, ly);
+    } else if (PPL == 2) {
+        const uint32_t waves_per_row = a.tile_w_px / 8, wave = tr / SPLATAD_WAVE;
+        lx = (wave % waves_per_row) * 8 + ((uint32_t)lane & 7u);
+        ly = (wave / waves_per_row) * 16 + ((uint32_t)lane >> 3);
     } else {
-        px = (float)j + 0.5f;
-        py = (float)i + 0.5f;
-        roll = a.rs_time[cam] * ((py - 0.5f) / (float)(a.H - 1) - 0.5f);
+        pixel_of_lane(a.tile_w_px, tr, lx, ly);
     }
-    const bool inside = in_image && pz > 0.f;
-    const uint64_t inside_bits = wave_ballot(inside);
+    const uint32_t j = (tile_id % a.grid_w) * a.tile_w_px + lx;
+    // per pixel of the lane (index p below): row, position, rolling-shutter factor
+    uint32_t i[PPL];
+    bool in_image[PPL], inside[PPL];
+    size_t pix[PPL];
+    uint64_t inside_bits[PPL];
+    float px, py[PPL], pz = 1.f, roll[PPL];
+    px = (float)j + 0.5f;
+#pragma unroll
+    for (int p = 0; p < PPL; ++p) {
+        i[p] = (tile_id / a.grid_w) * a.tile_h_px + ly + 8u * p;
+        in_image[p] = (tr * PPL < a.tile_w_px * a.tile_h_px && i[p] < a.H && j < a.W);
+        pix[p] = in_image[p] ? ((size_t)cam * a.H + i[p]) * a.W + j : 0;
+        if (LIDAR) {
+            px = py[p] = roll[p] = 0.f;
+            pz = 0.f;
+            if (in_image[p]) {
+                const float4 pt = reinterpret_cast<const float4 *>(a.raster_pts)[pix[p]];
+                px = pt.x; py[p] = pt.y; pz = pt.z; roll[p] = pt.w;
+            }
+        } else {
+            py[p] = (float)i[p] + 0.5f;
+            roll[p] = a.rs_time[cam] * ((py[p] - 0.5f) / (float)(a.H - 1) - 0.5f);
+        }
+        inside[p] = in_image[p] && pz > 0.f;
+        inside_bits[p] = wave_ballot(inside[p]);
+    }
     // Cameras: alpha comes from the forward kernel's polynomial in tile-centred pixel
     // coordinates, evaluated by the same function on the same staged coefficients, so that this
     // pass takes the forward pass's alpha >= 1/255 and sigma < 0 decisions bit for bit; the
     // offsets to the Gaussian's centre are still needed, for the gradients.
     TileFrame frame = {};
-    PixelConstants pc = {};
+    PixelConstants pc[PPL] = {};
     if (!LIDAR) {
         frame = tile_frame(tile_id % a.grid_w, tile_id / a.grid_w, a.tile_w_px, a.rs_time[cam], a.H);
-        pc.init(px, py, frame);
+#pragma unroll
+        for (int p = 0; p < PPL; ++p) pc[p].init(px, py[p], frame);
     }
 
     // lidar: angles relative to the tile's first valid point, as in the forward kernel
@@ -128,13 +148,13 @@ rasterize_bwd_kernel(BwdArgs a) {
     if (tr == 0) { s_block_final = -1; s_ref_thread = 0xFFFFFFFFu; }
     __syncthreads();
     if (LIDAR) {
-        if (inside) atomicMin(&s_ref_thread, tr);
+        if (inside[0]) atomicMin(&s_ref_thread, tr);
         __syncthreads();
-        if (tr == s_ref_thread) { s_ref[0] = px; s_ref[1] = py; }
+        if (tr == s_ref_thread) { s_ref[0] = px; s_ref[1] = py[0]; }
         __syncthreads();
         if (s_ref_thread != 0xFFFFFFFFu) { ref_x = s_ref[0]; ref_y = s_ref[1]; }
         px = angle_difference(px, ref_x); // from here on px, py are relative
-        py = angle_difference(py, ref_y);
+        py[0] = angle_difference(py[0], ref_y);
     }
 
     const int32_t *offs = a.tile_offsets + (size_t)cam * tiles_per_cam;
@@ -143,37 +163,45 @@ rasterize_bwd_kernel(BwdArgs a) {
                                   ? (int32_t)a.n_isects
                                   : offs[tile_id + 1];
 
-    const float T_final = inside ? 1.0f - a.render_alphas[pix] : 1.0f;
-    float T = T_final;
-    const int32_t bin_final = inside ? a.last_ids[pix] : -1;
     // The reference keeps, per channel, the colour accumulated behind the current Gaussian
     // (`buffer`) and forms v_alpha = sum_k (c_k T - buffer_k / (1 - alpha)) v_out_k.  Only the
-    // product of the buffer with v_out is ever used, so one running number per lane replaces
+    // product of the buffer with v_out is ever used, so one running number per pixel replaces
     // the CH buffers: with cv = sum_k c_k v_out_k, v_alpha = cv T - behind / (1 - alpha) and
     // behind += cv alpha T.
-    float behind = 0.f, v_out[CH];
+    float T_final[PPL], T[PPL], behind[PPL], v_out[PPL][CH], v_render_a[PPL], bg_dot[PPL];
+    int32_t bin_final[PPL];
 #pragma unroll
-    for (int k = 0; k < CH; ++k) {
-        v_out[k] = (inside && (uint32_t)k < a.n_ch) ? a.v_render_colors[pix * a.color_stride + a.ch_offset + k] : 0.f;
-    }
-    const float v_render_a = (inside && a.first_pass) ? a.v_render_alphas[pix] : 0.f;
-    const float v_asum = (LIDAR && inside && a.first_pass && a.compute_alpha_sum && a.v_alpha_sum) ? a.v_alpha_sum[pix] : 0.f;
-    float bg_dot = 0.f; // sum_k background_k v_out_k
-    if (a.backgrounds != nullptr) {
-        const float *bg = a.backgrounds + (size_t)cam * a.color_stride + a.ch_offset;
+    for (int p = 0; p < PPL; ++p) {
+        T_final[p] = inside[p] ? 1.0f - a.render_alphas[pix[p]] : 1.0f;
+        T[p] = T_final[p];
+        bin_final[p] = inside[p] ? a.last_ids[pix[p]] : -1;
+        behind[p] = 0.f;
 #pragma unroll
         for (int k = 0; k < CH; ++k)
-            if ((uint32_t)k < a.n_ch) bg_dot += bg[k] * v_out[k];
+            v_out[p][k] = (inside[p] && (uint32_t)k < a.n_ch)
+                              ? a.v_render_colors[pix[p] * a.color_stride + a.ch_offset + k] : 0.f;
+        v_render_a[p] = (inside[p] && a.first_pass) ? a.v_render_alphas[pix[p]] : 0.f;
+        bg_dot[p] = 0.f; // sum_k background_k v_out_k
+        if (a.backgrounds != nullptr) {
+            const float *bg = a.backgrounds + (size_t)cam * a.color_stride + a.ch_offset;
+#pragma unroll
+            for (int k = 0; k < CH; ++k)
+                if ((uint32_t)k < a.n_ch) bg_dot[p] += bg[k] * v_out[p][k];
+        }
     }
+    const float v_asum = (LIDAR && inside[0] && a.first_pass && a.compute_alpha_sum && a.v_alpha_sum) ? a.v_alpha_sum[pix[0]] : 0.f;
     const bool has_depth = LIDAR && a.depth_idx >= a.ch_offset && a.depth_idx < a.ch_offset + a.n_ch;
     const int depth_local = has_depth ? (int)(a.depth_idx - a.ch_offset) : -1;
     float v_out_depth = 0.f; // v_out of the depth channel, valid in the pass that owns it
 #pragma unroll
     for (int k = 0; k < CH; ++k)
-        if (k == depth_local) v_out_depth = v_out[k];
+        if (k == depth_local) v_out_depth = v_out[0][k];
 
     // deepest entry any pixel of the tile consumed
-    const int32_t wave_final = wave_max_i32(bin_final);
+    int32_t lane_final = bin_final[0];
+#pragma unroll
+    for (int p = 1; p < PPL; ++p) lane_final = max(lane_final, bin_final[p]);
+    const int32_t wave_final = wave_max_i32(lane_final);
     if (lane == 0 && wave_final >= 0) atomicMax(&s_block_final, wave_final);
     __syncthreads();
     const int32_t list_end = min(range_end, s_block_final + 1); // exclusive
@@ -183,8 +211,8 @@ rasterize_bwd_kernel(BwdArgs a) {
     // footprint of this wavefront over the lanes that consumed anything
     WaveCull cull;
     WavePointCull pcull;
-    if (LIDAR) pcull.init(inside && bin_final >= range_start, px, py, roll, true);
-    else cull.init(px, py, roll, true);
+    if (LIDAR) pcull.init(inside[0] && bin_final[0] >= range_start, px, py[0], roll[0], true);
+    else cull.init(px, py[0], py[PPL - 1], roll[0], roll[PPL - 1], true);
 
     // what a lane reads for the Gaussian it stages
     struct Fetched {
@@ -291,100 +319,109 @@ rasterize_bwd_kernel(BwdArgs a) {
                 const float4 *rec = s_rec + (size_t)RECORD * t;
                 const float4 xyv = rec[0];
                 const float4 e = rec[1];
-                float dx = gaussian_offset(xyv.x, xyv.z, roll, px);
-                float dy = gaussian_offset(xyv.y, xyv.w, roll, py);
-                if (LIDAR && ((folded >> bit) & 1ull)) { // uniform, rare
-                    dx = angle_difference(fmaf(roll, xyv.z, xyv.x), px);
-                    dy = angle_difference(fmaf(roll, xyv.w, xyv.y), py);
+                // per pixel: offsets, alpha before the clamp, and the lanes that took this Gaussian
+                // in the forward pass (scalar logic on lane masks)
+                float dx[PPL], dy[PPL], au[PPL];
+                uint64_t valid_bits[PPL], any_valid = 0;
+#pragma unroll
+                for (int p = 0; p < PPL; ++p) {
+                    dx[p] = gaussian_offset(xyv.x, xyv.z, roll[p], px);
+                    dy[p] = gaussian_offset(xyv.y, xyv.w, roll[p], py[p]);
+                    if (LIDAR && ((folded >> bit) & 1ull)) { // uniform, rare
+                        dx[p] = angle_difference(fmaf(roll[p], xyv.z, xyv.x), px);
+                        dy[p] = angle_difference(fmaf(roll[p], xyv.w, xyv.y), py[p]);
+                    }
+                    bool sigma_ok;
+                    if constexpr (LIDAR) {
+                        const float power = gaussian_power(e, dx[p], dy[p]);
+                        au[p] = __builtin_amdgcn_exp2f(e.w - power); // opacity * exp(-sigma)
+                        sigma_ok = !(power < 0.f);
+                    } else {
+                        const float4 pb = rec[3];
+                        const float ex = pixel_exponent(rec[2], pb.x, pb.y, pc[p]);
+                        au[p] = __builtin_amdgcn_exp2f(ex);
+                        sigma_ok = !(ex > pb.z);
+                    }
+                    valid_bits[p] = inside_bits[p] & wave_ballot(batch_end - t <= bin_final[p]) &
+                                    wave_ballot(sigma_ok) & wave_ballot(!(fminf(0.999f, au[p]) < 1.f / 255.f));
+                    any_valid |= valid_bits[p];
                 }
-                float au; // opacity * exp(-sigma)
-                bool sigma_ok;
-                if constexpr (LIDAR) {
-                    const float power = gaussian_power(e, dx, dy);
-                    au = __builtin_amdgcn_exp2f(e.w - power);
-                    sigma_ok = !(power < 0.f);
-                } else {
-                    const float4 pb = rec[3];
-                    const float ex = pixel_exponent(rec[2], pb.x, pb.y, pc);
-                    au = __builtin_amdgcn_exp2f(ex);
-                    sigma_ok = !(ex > pb.z);
-                }
-                const float alpha = fminf(0.999f, au);
-                // the lanes that took this Gaussian in the forward pass, by scalar logic on lane masks
-                const uint64_t valid_bits = inside_bits & wave_ballot(batch_end - t <= bin_final) &
-                                            wave_ballot(sigma_ok) & wave_ballot(!(alpha < 1.f / 255.f));
-                if (valid_bits == 0) continue;
-                const bool valid = wave_lanes(valid_bits);
+                if (any_valid == 0) continue;
 
-                // Branch-free from here on: a lane that does not take this Gaussian runs the same
+                // Branch-free from here on: a pixel that does not take this Gaussian runs the same
                 // arithmetic with alpha = 0 and alpha-before-clamping = 0, which makes every
                 // gradient term an exact zero (all other factors are finite) and leaves its
-                // transmittance and colour buffer as they are.
-                const float alpha_s = valid ? alpha : 0.f;
-                const float ra = __builtin_amdgcn_rcpf(1.0f - alpha_s); // 1 ulp; exactly 1 for alpha = 0
-                T *= ra; // transmittance in front of this Gaussian
-                const float fac = alpha_s * T;
-                // a clamped alpha passes no gradient on to the exponent or the opacity
-                const float au_g = (valid && au <= 0.999f) ? au : 0.f;
+                // transmittance and colour buffer as they are.  The pixels of a lane add up in
+                // the lane before the wavefront reduction.
                 float v[NV];
 #pragma unroll
-                for (int k = ACC; k < NV; ++k) v[k] = 0.f;
-                float cv = 0.f;
-#pragma unroll
-                for (int k = 0; k < CH; ++k) {
-                    v[k] = fac * v_out[k];
-                    cv += s_col[t * CH + k] * v_out[k];
-                }
-                float4 ext = make_float4(0.f, 0.f, 0.f, 0.f);
-                float extra = 0.f;
-                if constexpr (LIDAR) {
-                    ext = rec[RECORD - 1];
-                    extra = ext.y * dx + ext.z * dy + ext.x * roll;
-                    cv += extra * v_out_depth; // depth channel = colour + extra
-                }
-                float v_alpha = cv * T - behind * ra;
-                behind += cv * fac;
-                v_alpha += T_final * ra * v_render_a;
-                v_alpha += -T_final * ra * bg_dot;
+                for (int k = 0; k < NV; ++k) v[k] = 0.f;
                 const float rop = s_aux[t].y;
-                // conic row products a dx + b dy and b dx + c dy from the staged form
-                const float row_x = kLn2 * (2.f * e.x * dx + e.y * dy);
-                const float row_y = kLn2 * (e.y * dx + 2.f * e.z * dy);
-                const float v_sigma = -au_g * v_alpha;
-                v[CH + G_CONIC] = 0.5f * v_sigma * dx * dx;
-                v[CH + G_CONIC + 1] = v_sigma * dx * dy;
-                v[CH + G_CONIC + 2] = 0.5f * v_sigma * dy * dy;
-                float g_x = v_sigma * row_x, g_y = v_sigma * row_y;
-                if constexpr (LIDAR) {
-                    // gradient of the depth channel value, under the same clamp rule
-                    const float g_depth = au_g != 0.f ? fac * v_out_depth : 0.f;
-                    v[CH + G_DC] = g_depth * dx;
-                    v[CH + G_DC + 1] = g_depth * dy;
-                    v[CH + G_VELZ] = g_depth * roll;
-                    g_x += g_depth * ext.y;
-                    g_y += g_depth * ext.z;
-                }
-                float g_ax = fabsf(g_x), g_ay = fabsf(g_y);
-                v[CH + G_OPAC] = au_g * rop * v_alpha;
-                if constexpr (LIDAR) {
-                    if (a.compute_alpha_sum) { // uniform
-                        const float au_s = (valid && ext.w < pz - a.threshold) ? au : 0.f;
-                        const float v_sig2 = -v_asum * au_s;
-                        const float ex = v_sig2 * row_x, ey = v_sig2 * row_y;
-                        g_x += ex; g_y += ey;
-                        g_ax += fabsf(ex); g_ay += fabsf(ey);
-                        v[CH + G_CONIC] += v_sig2 * 0.5f * dx * dx;
-                        v[CH + G_CONIC + 1] += v_sig2 * dx * dy;
-                        v[CH + G_CONIC + 2] += v_sig2 * 0.5f * dy * dy;
-                        v[CH + G_OPAC] += v_asum * au_s * rop;
+                float4 ext = make_float4(0.f, 0.f, 0.f, 0.f);
+                if constexpr (LIDAR) ext = rec[RECORD - 1];
+#pragma unroll
+                for (int p = 0; p < PPL; ++p) {
+                    const bool valid = wave_lanes(valid_bits[p]);
+                    const float alpha_s = valid ? fminf(0.999f, au[p]) : 0.f;
+                    const float ra = __builtin_amdgcn_rcpf(1.0f - alpha_s); // 1 ulp; exactly 1 for alpha = 0
+                    T[p] *= ra; // transmittance in front of this Gaussian
+                    const float fac = alpha_s * T[p];
+                    // a clamped alpha passes no gradient on to the exponent or the opacity
+                    const float au_g = (valid && au[p] <= 0.999f) ? au[p] : 0.f;
+                    float cv = 0.f;
+#pragma unroll
+                    for (int k = 0; k < CH; ++k) {
+                        v[k] += fac * v_out[p][k];
+                        cv += s_col[t * CH + k] * v_out[p][k];
                     }
+                    float extra = 0.f;
+                    if constexpr (LIDAR) {
+                        extra = ext.y * dx[p] + ext.z * dy[p] + ext.x * roll[p];
+                        cv += extra * v_out_depth; // depth channel = colour + extra
+                    }
+                    float v_alpha = cv * T[p] - behind[p] * ra;
+                    behind[p] += cv * fac;
+                    v_alpha += T_final[p] * ra * v_render_a[p];
+                    v_alpha += -T_final[p] * ra * bg_dot[p];
+                    // conic row products a dx + b dy and b dx + c dy from the staged form
+                    const float row_x = kLn2 * (2.f * e.x * dx[p] + e.y * dy[p]);
+                    const float row_y = kLn2 * (e.y * dx[p] + 2.f * e.z * dy[p]);
+                    const float v_sigma = -au_g * v_alpha;
+                    v[CH + G_CONIC] += 0.5f * v_sigma * dx[p] * dx[p];
+                    v[CH + G_CONIC + 1] += v_sigma * dx[p] * dy[p];
+                    v[CH + G_CONIC + 2] += 0.5f * v_sigma * dy[p] * dy[p];
+                    float g_x = v_sigma * row_x, g_y = v_sigma * row_y;
+                    if constexpr (LIDAR) {
+                        // gradient of the depth channel value, under the same clamp rule
+                        const float g_depth = au_g != 0.f ? fac * v_out_depth : 0.f;
+                        v[CH + G_DC] += g_depth * dx[p];
+                        v[CH + G_DC + 1] += g_depth * dy[p];
+                        v[CH + G_VELZ] += g_depth * roll[p];
+                        g_x += g_depth * ext.y;
+                        g_y += g_depth * ext.z;
+                    }
+                    float g_ax = fabsf(g_x), g_ay = fabsf(g_y);
+                    v[CH + G_OPAC] += au_g * rop * v_alpha;
+                    if constexpr (LIDAR) {
+                        if (a.compute_alpha_sum) { // uniform
+                            const float au_s = (valid && ext.w < pz - a.threshold) ? au[p] : 0.f;
+                            const float v_sig2 = -v_asum * au_s;
+                            const float ex = v_sig2 * row_x, ey = v_sig2 * row_y;
+                            g_x += ex; g_y += ey;
+                            g_ax += fabsf(ex); g_ay += fabsf(ey);
+                            v[CH + G_CONIC] += v_sig2 * 0.5f * dx[p] * dx[p];
+                            v[CH + G_CONIC + 1] += v_sig2 * dx[p] * dy[p];
+                            v[CH + G_CONIC + 2] += v_sig2 * 0.5f * dy[p] * dy[p];
+                            v[CH + G_OPAC] += v_asum * au_s * rop;
+                        }
+                    }
+                    v[CH + G_XY] += g_x;
+                    v[CH + G_XY + 1] += g_y;
+                    v[CH + G_ABS] += g_ax;
+                    v[CH + G_ABS + 1] += g_ay;
+                    v[CH + G_VEL] += g_x * roll[p];
+                    v[CH + G_VEL + 1] += g_y * roll[p];
                 }
-                v[CH + G_XY] = g_x;
-                v[CH + G_XY + 1] = g_y;
-                v[CH + G_ABS] = g_ax;
-                v[CH + G_ABS + 1] = g_ay;
-                v[CH + G_VEL] = g_x * roll;
-                v[CH + G_VEL + 1] = g_y * roll;
                 // sum over the wavefront; the lane that ends up with slot s adds it in LDS
                 wave_reduce_scatter<NA>(*reinterpret_cast<float(*)[NA]>(&v[0]), lane);
                 const int slot = wave_reduce_slot<NA>(lane);
@@ -472,8 +509,8 @@ static inline int pick_width(uint32_t n) {
     return -1;
 }
 
-template <int CH, bool LIDAR>
-static int launch_bwd(BwdArgs a, dim3 grid, dim3 block, hipStream_t stream) {
+template <int CH, bool LIDAR, int PPL>
+static int launch_bwd_as(BwdArgs a, dim3 grid, dim3 block, hipStream_t stream) {
     const size_t per_gaussian = ((LIDAR ? 48 : 64) + 8) + 4 * CH + 4 * (CH + (LIDAR ? G_COUNT : G_VELZ));
     // Batches of the whole workgroup, unless that leaves fewer than four workgroups to a compute
     // unit (160 KB of LDS): a lidar sweep's 1024 tiles then run all at once instead of in two
@@ -482,11 +519,22 @@ static int launch_bwd(BwdArgs a, dim3 grid, dim3 block, hipStream_t stream) {
     if (a.batch * per_gaussian > 40 * 1024) a.batch = (uint32_t)(40 * 1024 / per_gaussian) / 8 * 8;
     const size_t lds = a.batch * per_gaussian;
     if (lds > 64 * 1024)
-        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_bwd_kernel<CH, LIDAR>,
+        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_bwd_kernel<CH, LIDAR, PPL>,
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL((rasterize_bwd_kernel<CH, LIDAR>), grid, block, lds, stream, a);
+    hipLaunchKernelGGL((rasterize_bwd_kernel<CH, LIDAR, PPL>), grid, block, lds, stream, a);
     SPLATAD_LAUNCH_CHECK();
     return 0;
+}
+
+// Cameras with few channels and tiles of whole 8 x 16 wavefronts: two pixels per lane.
+template <int CH, bool LIDAR>
+static int launch_bwd(const BwdArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
+    if constexpr (!LIDAR && CH <= 5) {
+        const uint32_t pixels = a.tile_w_px * a.tile_h_px;
+        if (a.tile_w_px % 8 == 0 && (pixels / 2) % SPLATAD_WAVE == 0 && block.x == pixels)
+            return launch_bwd_as<CH, LIDAR, 2>(a, grid, dim3(pixels / 2), stream);
+    }
+    return launch_bwd_as<CH, LIDAR, 1>(a, grid, block, stream);
 }
 
 template <bool LIDAR>
