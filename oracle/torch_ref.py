@@ -164,9 +164,13 @@ def _angle_difference(a, b):
 
 
 def rasterize_to_pixels(means2d, conics, colors, opacities, pix_vels, rs_time, backgrounds, width,
-                        height, tile_size, offsets, flatten_ids, tiles=None):
+                        height, tile_size, offsets, flatten_ids, tiles=None, near=None):
     """Dense per-tile compositing; differentiable w.r.t. the float inputs.  [C,N,...] layout.
-    With `tiles` (flat (camera, tile) indices) only those tiles are rendered, the rest stays 0."""
+    With `tiles` (flat (camera, tile) indices) only those tiles are rendered, the rest stays 0.
+    With `near` (a dict with "margin"), near["rows"] becomes a bool [C * N]: the Gaussians whose
+    alpha lies within the relative margin of the 1/255 threshold at some pixel that is still
+    compositing when it reaches them -- the pairs a float32 evaluation may decide differently --
+    and the Gaussians composited at a pixel that has such a pair."""
     C, th, tw = offsets.shape
     D = colors.shape[-1]
     n_isects = flatten_ids.shape[0]
@@ -199,6 +203,19 @@ def rasterize_to_pixels(means2d, conics, colors, opacities, pix_vels, rs_time, b
                     alpha = torch.clamp(op[g][None] * torch.exp(-sigma), max=0.999)
                     w, T_final, _, _, _, _ = _composite(alpha, sigma)
                     pix = w @ col[g]
+                    if near is not None:
+                        with torch.no_grad():
+                            near.setdefault("rows", torch.zeros(m2.shape[0], dtype=torch.bool))
+                            raw = op[g][None] * torch.exp(-sigma)
+                            _, _, _, a_, _, T_incl = _composite(alpha, sigma)
+                            stop = (a_ > 0) & (T_incl <= 1e-4)
+                            before = torch.cumsum(stop.to(torch.int64), dim=1) - stop.to(torch.int64)
+                            close = ((raw * 255.0 - 1.0).abs() <= near["margin"]) & (before == 0)
+                            # such a pair, decided the other way, changes its pixel for every
+                            # Gaussian composited there: the transmittance of those behind it, the
+                            # colour accumulated behind those in front of it, by alpha ~ 0.4 %
+                            shared = close.any(1, keepdim=True) & (w > 0)
+                            near["rows"][g[(close | shared).any(0)]] = True
                 if backgrounds is not None:
                     pix = pix + T_final[:, None] * backgrounds[c][None]
                 rows.append((c, i0, i1, j0, j1, pix, T_final))

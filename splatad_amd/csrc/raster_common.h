@@ -176,7 +176,7 @@ struct WavePointCull {
 // sy Y, and log2(alpha) = L - (A dx^2 + B dx dy + C dy^2) is a quadratic polynomial in (X, Y)
 // whose six coefficients depend on the Gaussian and the tile only.  They are computed once per
 // (tile, Gaussian) when the Gaussian is staged; a pixel then needs five fused multiply-adds
-// with its own constants (X, Y, X^2, X Y, Y^2; exact in float32 for half-integers) instead of
+// with its own constants (X, Y, X^2, Y^2; exact in float32 for half-integers) instead of
 // the ten operations of the offset form, and every kernel that evaluates a pixel through
 // pixel_exponent() gets the same bits, whatever its lane layout.  Inside a 16 x 16 tile |X|, |Y|
 // <= 7.5, and the cancellation between the terms costs at most a few 1e-5 of absolute accuracy
@@ -236,16 +236,22 @@ __device__ __forceinline__ void pixel_polynomial(const TileFrame &f, float2 xy, 
 }
 
 struct PixelConstants {
-    float X, Y, XX, XY, YY;
+    float X, Y, XX, YY;
     __device__ __forceinline__ void init(float px, float py, const TileFrame &f) {
 #pragma clang fp contract(off)
         X = px - f.cx; Y = py - f.cy;
-        XX = X * X; XY = X * Y; YY = Y * Y;
+        XX = X * X; YY = Y * Y;
     }
 };
 
+// Evaluated as (c0 + cX X + cXX X^2) + (cY + cXY X) Y + cYY Y^2: the two brackets depend on the
+// pixel's column only, so a lane whose pixels share a column (rows y and y + 8 in the kernels with
+// two pixels per lane) computes them once, seven fused multiply-adds for two pixels instead of ten.
+// Every kernel evaluates in this order, one pixel per lane or two.
 __device__ __forceinline__ float pixel_exponent(const float4 a, float cXY, float cYY, const PixelConstants &p) {
-    return fmaf(cYY, p.YY, fmaf(cXY, p.XY, fmaf(a.w, p.XX, fmaf(a.z, p.Y, fmaf(a.y, p.X, a.x)))));
+    const float column = fmaf(a.w, p.XX, fmaf(a.y, p.X, a.x));
+    const float slope = fmaf(cXY, p.X, a.z);
+    return fmaf(cYY, p.YY, fmaf(slope, p.Y, column));
 }
 
 // Footprint of a wavefront of camera pixels in tile-centred coordinates, and the test whether
