@@ -73,6 +73,18 @@ def staged_isects(tile_entries):
     return int(tile_entries.sum().item())
 
 
+def cycle_spread(cycles):
+    """Spread of the per-tile run times of a compositing kernel (shader clock cycles of each
+    tile's workgroup): the kernel lasts as long as its slowest tiles."""
+    import torch
+
+    c = cycles.flatten().double()
+    c = c[c > 0]
+    q = torch.quantile(c, torch.tensor([0.5, 0.9, 0.99], dtype=torch.float64, device=c.device)).tolist()
+    return {"tiles": int(c.numel()), "mean": round(c.mean().item()), "p50": round(q[0]), "p90": round(q[1]),
+            "p99": round(q[2]), "max": round(c.max().item()), "max_over_mean": round((c.max() / c.mean()).item(), 3)}
+
+
 def stage_rooflines(leg):
     """Per stage of a forward call: event-timed duration of the stage's launches in isolation, the
     bytes any implementation of the stage has to move, and what that makes of the HBM peak."""
@@ -133,6 +145,12 @@ def bench_camera(args):
             s["rolling_shutter_time"], None, W, H, ts, meta["isect_offsets"], meta["flatten_ids"],
             tile_batches=batches)
         i_need = staged_isects(batches)
+        cycles = torch.zeros(meta["isect_offsets"].shape, dtype=torch.int64, device=dev)
+        _C.rasterize_to_pixels_fwd(
+            meta["means2d"], meta["conics"], cols, meta["opacities"], meta["pix_vels"],
+            s["rolling_shutter_time"], None, W, H, ts, meta["isect_offsets"], meta["flatten_ids"],
+            tile_cycles=cycles)
+        tile_cycles = cycle_spread(cycles)
         D = cols.shape[-1]
         P, T = C * H * W, meta["isect_offsets"].numel()
         alg_bytes = i_need * (36 + 4 * D) + P * (4 * D + 8) + T * 4
@@ -174,7 +192,7 @@ def bench_camera(args):
                      iterations_without_a_compositing_lane=st[3] / max(1, st[0]))
     return dict(sec=sec, sec_packed=sec_packed, pixels=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
                 n_isects=n_isects, i_need=i_need, nnz=nnz, stages=stages, stage_bytes=stage_bytes,
-                channels=D, lanes=lanes)
+                channels=D, lanes=lanes, tile_cycles=tile_cycles)
 
 
 def bench_lidar(args):
@@ -223,6 +241,9 @@ def bench_lidar(args):
         batches = torch.zeros_like(meta["isect_offsets"])
         raster(tile_batches=batches)
         i_need = staged_isects(batches)
+        cycles = torch.zeros(meta["isect_offsets"].shape, dtype=torch.int64, device=dev)
+        raster(tile_cycles=cycles)
+        tile_cycles = cycle_spread(cycles)
         P, T = C * H * W, meta["isect_offsets"].numel()
         # staged per list entry: id, mean, angular velocity, conic, opacity (40 bytes); the features
         # of the Gaussians a wavefront composites are read on demand and not counted here
@@ -243,7 +264,8 @@ def bench_lidar(args):
                        "isect_sort_ms": C * N * 20 + n_isects * 12 + T * 4,
                        "rasterize_ms": alg_bytes}
     return dict(sec=sec, sec_chunk32=sec_chunk32, points=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
-                n_isects=n_isects, i_need=i_need, channels=D, stages=stages, stage_bytes=stage_bytes)
+                n_isects=n_isects, i_need=i_need, channels=D, stages=stages, stage_bytes=stage_bytes,
+                tile_cycles=tile_cycles)
 
 
 def bench_backward(args):
@@ -436,6 +458,7 @@ def main():
             "visible_gaussians": cam["nnz"], "ms_per_step_packed": cam["sec_packed"] * 1e3,
             "stage_ms": {k: round(v, 4) for k, v in cam["stages"].items()},
             "lane_utilisation": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in cam["lanes"].items()},
+            "tile_cycles": cam["tile_cycles"],
         },
         "stages": stage_rooflines(cam),
         "roofline": {
@@ -457,6 +480,7 @@ def main():
             "n_isects": lid["n_isects"], "n_isects_consumed": lid["i_need"],
             "stage_ms": {k: round(v, 4) for k, v in lid["stages"].items()},
             "stages": stage_rooflines(lid),
+            "tile_cycles": lid["tile_cycles"],
             "roofline": {"kernel": "rasterize_to_points_fwd_kernel<%d, %s>" % (lid["channels"], "true" if lid["channels"] in (32, 33) else "false"),
                          "bound": "hbm", "achieved": l_ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": l_ach / HBM_PEAK_GBS,

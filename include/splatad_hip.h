@@ -321,7 +321,10 @@ int splatad_populate_image_from_points(uint32_t C, int64_t n_points, const float
  * passes).  backgrounds may be NULL.  tile_batches may be NULL; otherwise it receives,
  * per (camera, tile), the number of entries of the tile's list that were staged (whole
  * batches, until every pixel of the tile had saturated, clipped to the list's length; a
- * diagnostic: it tells how much of the sorted lists a frame really reads). */
+ * diagnostic: it tells how much of the sorted lists a frame really reads).  tile_cycles may be
+ * NULL; otherwise it receives, per (camera, tile), the shader clock cycles the tile's workgroup
+ * ran for (a diagnostic: the spread tells how far the slowest tiles set the kernel's duration;
+ * with channels in several passes, the last pass's). */
 int splatad_rasterize_to_pixels_fwd(uint32_t C, int64_t n_isects, uint32_t channels,
                                     const float *means2d, const float *conics,
                                     const float *colors, const float *opacities,
@@ -332,7 +335,7 @@ int splatad_rasterize_to_pixels_fwd(uint32_t C, int64_t n_isects, uint32_t chann
                                     const int32_t *tile_offsets, const int32_t *flatten_ids,
                                     float *render_colors, float *render_alphas,
                                     int32_t *last_ids, int32_t *tile_batches,
-                                    splatad_stream_t stream);
+                                    int64_t *tile_cycles, splatad_stream_t stream);
 
 /* Diagnostic without a counterpart in the reference: lane utilisation of the compositing loop
  * of splatad_rasterize_to_pixels_fwd on the same inputs (nothing is rendered).  Adds to eight
@@ -382,7 +385,7 @@ int splatad_rasterize_to_pixels_bwd(uint32_t C, int64_t n_isects, uint32_t chann
 /* rasterize_to_points_fwd_tensor, rasterization.cu:2221-2831 (kernel
  * :2021-2219).  Outputs of inactive points (range <= 0) are zero.
  * alpha_sum_until_points may be NULL when compute_alpha_sum_until_points == 0.
- * tile_batches: optional diagnostic as in splatad_rasterize_to_pixels_fwd.
+ * tile_batches, tile_cycles: optional diagnostics as in splatad_rasterize_to_pixels_fwd.
  *
  * range_channel (both directions; NULL for the reference's layout): the reference's
  * callers concatenate the Gaussians' ranges behind their features first
@@ -408,7 +411,8 @@ int splatad_rasterize_to_points_fwd(uint32_t C, int64_t n_isects, uint32_t chann
                                     uint32_t depth_channel_idx, float *render_colors,
                                     float *render_alphas, float *alpha_sum_until_points,
                                     int32_t *last_ids, float *median_depths,
-                                    int32_t *tile_batches, splatad_stream_t stream);
+                                    int32_t *tile_batches, int64_t *tile_cycles,
+                                    splatad_stream_t stream);
 
 /* rasterize_to_points_bwd_tensor, rasterization.cu:4056-4851 (kernel :3728-4054). */
 int splatad_rasterize_to_points_bwd(uint32_t C, int64_t n_isects, uint32_t channels,

@@ -38,6 +38,7 @@ struct PixelArgs {
     int32_t *last_ids;
     int write_aux; // first pass also writes alphas and last ids
     int32_t *tile_batches; // optional diagnostic: list entries each tile's workgroup staged
+    int64_t *tile_cycles;  // optional diagnostic: shader clock cycles each tile's workgroup ran for
     unsigned long long *lane_stats; // STATS kernels only: kLaneStats counters, see the entry point
 };
 
@@ -59,6 +60,7 @@ constexpr int kLaneStats = 8;
 template <int CH, int PPL, bool STATS = false>
 __global__ void __launch_bounds__(1024)
 rasterize_to_pixels_fwd_kernel(PixelArgs a) {
+    const long long t_begin = a.tile_cycles != nullptr ? clock64() : 0;
     extern __shared__ float4 lds4[];
     const uint32_t block_size = blockDim.x;
     const uint32_t batch = block_size; // list entries staged at a time, one per lane
@@ -288,6 +290,7 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
 
     if (a.tile_batches != nullptr && a.write_aux && tr == 0)
         a.tile_batches[blockIdx.x] = (int32_t)min(batches_done * batch, (uint32_t)(range_end - range_start));
+    if (a.tile_cycles != nullptr && a.write_aux && tr == 0) a.tile_cycles[blockIdx.x] = clock64() - t_begin;
     if (STATS) {
         if (lane == 0) {
             const uint32_t v[kLaneStats] = {st_iter, st_take, st_alive, st_idle, st_tested, st_kept, 0u, st_valid};
@@ -334,6 +337,7 @@ struct PointArgs {
     float *median_depths;
     int write_aux;
     int32_t *tile_batches; // optional diagnostic, as in PixelArgs
+    int64_t *tile_cycles;  // optional diagnostic, as in PixelArgs
 };
 
 // MATRIX (CH = 32 or 33, every channel in use, whole wavefronts): the first 32 channels are
@@ -353,6 +357,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 template <int CH, bool MATRIX>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4)))
 rasterize_to_points_fwd_kernel(PointArgs a) {
+    const long long t_begin = a.tile_cycles != nullptr ? clock64() : 0;
     static_assert(!MATRIX || CH == 32 || CH == 33, "the matrix path accumulates 32 channels (+1)");
     extern __shared__ float4 lds4[];
     __shared__ uint32_t s_ref_thread;
@@ -593,6 +598,7 @@ rasterize_to_points_fwd_kernel(PointArgs a) {
 
     if (a.tile_batches != nullptr && a.write_aux && tr == 0)
         a.tile_batches[blockIdx.x] = (int32_t)min(batches_done * block_size, (uint32_t)(range_end - range_start));
+    if (a.tile_cycles != nullptr && a.write_aux && tr == 0) a.tile_cycles[blockIdx.x] = clock64() - t_begin;
     if constexpr (MATRIX) {
         if (pair_open) add_pair(pair_weight, 0.f, pair_feature, 0.f);
         // what the D layout needs to know of a point: where it is stored, its transmittance
@@ -740,7 +746,7 @@ extern "C" int splatad_rasterize_to_pixels_fwd(
     const float *backgrounds, uint32_t W, uint32_t H, uint32_t tile_size, uint32_t tile_w,
     uint32_t tile_h, const int32_t *tile_offsets, const int32_t *flatten_ids,
     float *render_colors, float *render_alphas, int32_t *last_ids, int32_t *tile_batches,
-    splatad_stream_t stream) {
+    int64_t *tile_cycles, splatad_stream_t stream) {
     SPLATAD_REQUIRE(channels >= 1, "rasterize_to_pixels: zero channels");
     SPLATAD_REQUIRE(tile_size >= 1 && tile_size * tile_size <= 1024,
                     "rasterize_to_pixels: tile_size %u is outside 1..32", tile_size);
@@ -761,6 +767,7 @@ extern "C" int splatad_rasterize_to_pixels_fwd(
     a.tile_offsets = tile_offsets; a.flatten_ids = flatten_ids;
     a.render_colors = render_colors; a.render_alphas = render_alphas; a.last_ids = last_ids;
     a.tile_batches = tile_batches;
+    a.tile_cycles = tile_cycles;
     a.lane_stats = nullptr;
     const dim3 grid(C * tile_w * tile_h), block(tile_size, tile_size);
     const uint32_t pass = channels <= (uint32_t)kMaxPass ? channels : 32u;
@@ -808,7 +815,7 @@ extern "C" int splatad_rasterize_to_points_fwd(
     int compute_alpha_sum, float threshold, const int32_t *tile_offsets,
     const int32_t *flatten_ids, uint32_t depth_idx, float *render_colors, float *render_alphas,
     float *alpha_sum, int32_t *last_ids, float *median_depths, int32_t *tile_batches,
-    splatad_stream_t stream) {
+    int64_t *tile_cycles, splatad_stream_t stream) {
     SPLATAD_REQUIRE(channels >= 1, "rasterize_to_points: zero channels");
     SPLATAD_REQUIRE(depth_idx < channels, "rasterize_to_points: depth channel %u of %u", depth_idx, channels);
     SPLATAD_REQUIRE(range_channel == nullptr || (depth_idx + 1 == channels && channels >= 2),
@@ -837,6 +844,7 @@ extern "C" int splatad_rasterize_to_points_fwd(
     a.render_colors = render_colors; a.render_alphas = render_alphas;
     a.alpha_sum = compute_alpha_sum ? alpha_sum : nullptr;
     a.last_ids = last_ids; a.median_depths = median_depths; a.tile_batches = tile_batches;
+    a.tile_cycles = tile_cycles;
     const dim3 grid(C * grid_w * grid_h), block((tile_width * tile_height + SPLATAD_WAVE - 1) / SPLATAD_WAVE * SPLATAD_WAVE);
     const uint32_t pass = channels <= (uint32_t)kMaxPass ? channels : 32u;
     for (uint32_t off = 0; off < channels; off += pass) {

@@ -736,7 +736,7 @@ class _Ops:
     # ------------------------------------------------------------------ rasterization
     def rasterize_to_pixels_fwd(self, means2d, conics, colors, opacities, pix_vels,
                                 rolling_shutter_time, backgrounds, image_width, image_height,
-                                tile_size, tile_offsets, flatten_ids, tile_batches=None):
+                                tile_size, tile_offsets, flatten_ids, tile_batches=None, tile_cycles=None):
         """tile_batches: optional int32 [C, tile_height, tile_width] tensor that receives the number
         of list entries every tile staged (a diagnostic, not part of the reference's op)."""
         lib = load_library()
@@ -758,7 +758,8 @@ class _Ops:
                 _p(opacities), _p(pix_vels), _p(rs), _p(backgrounds), _u32(image_width),
                 _u32(image_height), _u32(tile_size), _u32(tw), _u32(th), _p(tile_offsets),
                 _p(flatten_ids), _p(renders), _p(alphas), _p(last_ids),
-                _p(_in(tile_batches, "tile_batches", torch.int32)), _stream(dev)))
+                _p(_in(tile_batches, "tile_batches", torch.int32)),
+                _p(_in(tile_cycles, "tile_cycles", torch.int64)), _stream(dev)))
         return renders, alphas, last_ids
 
     def rasterize_to_pixels_lane_stats(self, means2d, conics, opacities, pix_vels, rolling_shutter_time,
@@ -819,7 +820,7 @@ class _Ops:
                                 image_height, tile_width, tile_height,
                                 compute_alpha_sum_until_points,
                                 compute_alpha_sum_until_points_threshold, tile_offsets, flatten_ids,
-                                depth_channel_idx, tile_batches=None, range_channel=None):
+                                depth_channel_idx, tile_batches=None, range_channel=None, tile_cycles=None):
         """With range_channel ([C, N] or [nnz]) the last channel is read from it and `colors`
         holds the other channels only (depth_channel_idx counts it: colors.shape[-1])."""
         lib = load_library()
@@ -848,7 +849,8 @@ class _Ops:
                 _u32(gw), _u32(gh), _i32(bool(compute_alpha_sum_until_points)),
                 _f32(compute_alpha_sum_until_points_threshold), _p(tile_offsets), _p(flatten_ids),
                 _u32(depth_channel_idx), _p(renders), _p(alphas), _p(asum), _p(last_ids),
-                _p(medians), _p(_in(tile_batches, "tile_batches", torch.int32)), _stream(dev)))
+                _p(medians), _p(_in(tile_batches, "tile_batches", torch.int32)),
+                _p(_in(tile_cycles, "tile_cycles", torch.int64)), _stream(dev)))
         return renders, alphas, last_ids, asum, medians
 
     def rasterize_to_points_bwd(self, means2d, conics, colors, opacities, pix_vels,
