@@ -187,7 +187,8 @@ def _raster_scene(seed, C, N, W, H, D):
     return means2d, conics, colors, opac, depths, pix_vels, radii, bg
 
 
-@pytest.mark.parametrize("D,ts,N", [(3, 16, 600), (4, 16, 3000), (1, 8, 500), (33, 16, 500), (40, 16, 400), (5, 4, 300)])
+@pytest.mark.parametrize("D,ts,N", [(3, 16, 600), (4, 16, 3000), (1, 8, 500), (33, 16, 500), (40, 16, 400), (5, 4, 300),
+                                    (5, 16, 500), (1, 16, 400), (8, 16, 300)])
 def test_rasterize_to_pixels_backward(D, ts, N):
     from splatad_amd import isect_offset_encode, isect_tiles, rasterize_to_pixels
     C, W, H = 2, 72, 40
