@@ -491,8 +491,8 @@ __device__ __forceinline__ void classify_segment(uint32_t seg, uint32_t lane, ui
     uint32_t n = 0;
     if (seg < n_segments) {
         const int64_t start = tile_starts[seg];
-        const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
-        n = (uint32_t)(stop - start);
+        const int64_t stop = min(seg + 1 == n_segments ? n_isects : (int64_t)tile_starts[seg + 1], n_isects);
+        n = stop > start ? (uint32_t)(stop - start) : 0u;
         if (tile_offsets != nullptr && (seg & ((1u << sshift) - 1u)) == 0)
             tile_offsets[seg >> sshift] = (int32_t)start;
     }
@@ -575,7 +575,10 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
                     const bool hit = in && ((rec.w >> t) & 1u);
                     const uint64_t b = __ballot(hit);
                     const int32_t first = __shfl(dst, (int)t, SPLATAD_WAVE);
-                    if (hit) pairs[(int64_t)first + __popcll(b & below)] = pair;
+                    // (the bound holds whenever n_isects is the count of these very rows; it
+                    // keeps a caller's mismatch from writing outside the lists)
+                    const int64_t at = (int64_t)first + __popcll(b & below);
+                    if (hit && at < n_isects) pairs[at] = pair;
                 }
             }
         }
@@ -757,8 +760,8 @@ __device__ __forceinline__ void sort_segment(uint32_t seg, uint32_t n_segments, 
                                              int32_t *__restrict__ flatten_ids,
                                              uint64_t *lds_staged, uint32_t *s_wave, uint32_t &s_big) {
     const int64_t start = tile_starts[seg];
-    const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
-    const uint32_t n = (uint32_t)(stop - start);
+    const int64_t stop = min(seg + 1 == n_segments ? n_isects : (int64_t)tile_starts[seg + 1], n_isects);
+    const uint32_t n = stop > start ? (uint32_t)(stop - start) : 0u; // as classified
     uint32_t *s_fine = reinterpret_cast<uint32_t *>(lds_staged + lds_words);
     uint32_t *s_cursor = s_fine + kSortFineBins;
     uint32_t *s_first = s_cursor + bucket_cap;
@@ -961,8 +964,8 @@ __device__ __forceinline__ void sort_segment_small(uint32_t seg, uint32_t n_segm
                                                    int32_t *__restrict__ flatten_ids,
                                                    uint64_t *lds_staged, uint32_t *s_wave, uint32_t &s_big) {
     const int64_t start = tile_starts[seg];
-    const int64_t stop = seg + 1 == n_segments ? n_isects : tile_starts[seg + 1];
-    const uint32_t n = (uint32_t)(stop - start);
+    const int64_t stop = min(seg + 1 == n_segments ? n_isects : (int64_t)tile_starts[seg + 1], n_isects);
+    const uint32_t n = stop > start ? (uint32_t)(stop - start) : 0u; // as classified
     uint32_t *s_fine = reinterpret_cast<uint32_t *>(lds_staged + lds_words + 4);
     uint32_t *s_first = s_fine + kSortFineBins;   // bucket_cap + 1 words: starts, then the end
     uint32_t *s_cursor = s_first + bucket_cap + 1;
