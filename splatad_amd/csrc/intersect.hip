@@ -109,6 +109,14 @@ __device__ __forceinline__ void loaded_here(float2 &mu, uint2 &r) {
     asm volatile("" : "+v"(mu.x), "+v"(mu.y), "+v"(r.x), "+v"(r.y));
 }
 
+// Mathematical x mod n; columns within one turn of the grid (nearly all) need no division.
+__device__ __forceinline__ int32_t wrap_column(int32_t x, int32_t n) {
+    if (x >= 0 && x < n) return x;
+    if (x < 0 && x >= -n) return x + n;
+    if (x >= n && x < 2 * n) return x - n;
+    return ((x % n) + n) % n;
+}
+
 template <bool LIDAR>
 __device__ __forceinline__ uint32_t tile_index(const TileGrid &g, int32_t y, int32_t x) {
     if (LIDAR) {
@@ -117,8 +125,7 @@ __device__ __forceinline__ uint32_t tile_index(const TileGrid &g, int32_t y, int
         // azimuth extent reaching below -360 degrees) it wraps modulo 2^32 first: the same
         // column as here when tile_w is a power of two, a column shifted by 2^32 mod tile_w
         // otherwise.
-        const int32_t n = (int32_t)g.tile_w;
-        x = ((x % n) + n) % n;
+        x = wrap_column(x, (int32_t)g.tile_w);
     }
     return (uint32_t)y * g.tile_w + (uint32_t)x;
 }
@@ -215,7 +222,9 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
 
 __device__ __forceinline__ uint32_t camera_of(uint64_t idx, uint32_t N,
                                               const int64_t *__restrict__ camera_ids) {
-    return camera_ids ? (uint32_t)camera_ids[idx] : (uint32_t)(idx / N);
+    if (camera_ids) return (uint32_t)camera_ids[idx];
+    // idx < 2^31 (checked by the callers): a 32-bit division, and none at all for one sensor
+    return (uint32_t)idx < N ? 0u : (uint32_t)idx / N;
 }
 
 // Work item of one lane: the tile rectangle of its Gaussian plus what the emitters need.
@@ -261,10 +270,22 @@ __device__ __forceinline__ void for_each_tile_balanced(const LaneWork &mine, Emi
         const int leader = __ffsll((unsigned long long)big) - 1;
         big &= big - 1;
         const LaneWork w = broadcast_work(mine, leader);
-        for (int32_t t = lane; t < w.cnt; t += SPLATAD_WAVE) emit(w, w.y0 + t / w.w, w.x0 + t % w.w, t);
+        // t / w without an integer division: for t < 2^22, (t + 0.5) / w is never within
+        // 0.5 / w of an integer, far more than the rounding of the product
+        const float inv_w = 1.0f / (float)w.w;
+        for (int32_t t = lane; t < w.cnt; t += SPLATAD_WAVE) {
+            const int32_t row = w.cnt < (1 << 22) ? (int32_t)(((float)t + 0.5f) * inv_w) : t / w.w;
+            emit(w, w.y0 + row, w.x0 + (t - row * w.w), t);
+        }
     }
-    if (mine.cnt <= kCoopTiles)
-        for (int32_t t = 0; t < mine.cnt; ++t) emit(mine, mine.y0 + t / mine.w, mine.x0 + t % mine.w, t);
+    if (mine.cnt <= kCoopTiles) { // row by row, no division
+        int32_t x = mine.x0, y = mine.y0;
+        const int32_t x_end = mine.x0 + mine.w;
+        for (int32_t t = 0; t < mine.cnt; ++t) {
+            emit(mine, y, x, t);
+            if (++x == x_end) { x = mine.x0; ++y; }
+        }
+    }
 }
 
 // What a lane reads for its work item, and the work item made from it.  Reading and making
@@ -353,10 +374,7 @@ __device__ __forceinline__ void to_coarse(LaneWork &w, const CoarseGrid &cg) {
 
 template <bool LIDAR>
 __device__ __forceinline__ uint32_t coarse_index(const CoarseGrid &cg, int32_t cy, int32_t cx) {
-    if (LIDAR) {
-        const int32_t n = (int32_t)cg.cw;
-        cx = ((cx % n) + n) % n;
-    }
+    if (LIDAR) cx = wrap_column(cx, (int32_t)cg.cw);
     return (uint32_t)cy * cg.cw + (uint32_t)cx;
 }
 
