@@ -227,6 +227,14 @@ __device__ __forceinline__ uint32_t camera_of(uint64_t idx, uint32_t N,
     return (uint32_t)idx < N ? 0u : (uint32_t)idx / N;
 }
 
+// n / d for a divisor whose reciprocal (1.0f / (float)d, correctly rounded) is at hand: below
+// 2^20, (n + 0.5) / d stays at least 0.5 / d away from an integer, several times the rounding
+// error of the product, so truncation gives the quotient; above, the integer division.
+constexpr uint32_t kFloatDivLimit = 1u << 20;
+__device__ __forceinline__ uint32_t div_by(uint32_t n, uint32_t d, float inv_d) {
+    return n < kFloatDivLimit ? (uint32_t)(((float)n + 0.5f) * inv_d) : n / d;
+}
+
 // Work item of one lane: the tile rectangle of its Gaussian plus what the emitters need.
 struct LaneWork {
     int32_t x0, y0, w, cnt; // rectangle origin, width and number of tiles (0 = nothing)
@@ -270,11 +278,9 @@ __device__ __forceinline__ void for_each_tile_balanced(const LaneWork &mine, Emi
         const int leader = __ffsll((unsigned long long)big) - 1;
         big &= big - 1;
         const LaneWork w = broadcast_work(mine, leader);
-        // t / w without an integer division: for t < 2^22, (t + 0.5) / w is never within
-        // 0.5 / w of an integer, far more than the rounding of the product
         const float inv_w = 1.0f / (float)w.w;
         for (int32_t t = lane; t < w.cnt; t += SPLATAD_WAVE) {
-            const int32_t row = w.cnt < (1 << 22) ? (int32_t)(((float)t + 0.5f) * inv_w) : t / w.w;
+            const int32_t row = (int32_t)div_by((uint32_t)t, (uint32_t)w.w, inv_w);
             emit(w, w.y0 + row, w.x0 + (t - row * w.w), t);
         }
     }
@@ -343,16 +349,6 @@ __device__ __forceinline__ LaneWork make_work(const TileGrid &g, WorkInputs in) 
     return w;
 }
 
-template <bool LIDAR>
-__device__ __forceinline__ LaneWork load_work(const TileGrid &g, uint64_t idx, uint64_t total,
-                                              uint32_t N, const int64_t *__restrict__ camera_ids,
-                                              const float *__restrict__ means2d,
-                                              const void *__restrict__ radii,
-                                              const float *__restrict__ depths,
-                                              const int64_t *__restrict__ cum_before) {
-    return make_work<LIDAR>(g, fetch_work(idx, total, N, camera_ids, means2d, radii, depths, cum_before));
-}
-
 // Coarse blocks of (1 << bshift) x 4 tiles.  The width is 4 tiles for cameras; for lidars,
 // whose tile columns wrap around, it is the largest of 4, 2, 1 that divides the number of
 // columns, so that an unwrapped block column maps onto one wrapped block column.
@@ -385,10 +381,13 @@ __device__ __forceinline__ uint32_t coarse_mask(const LaneWork &w, const CoarseG
     const int32_t by = 1 << kCoarseRowShift;
     const int32_t xa = max(w.tx0 - cx * bx, 0), xb = min(w.tx1 - cx * bx, bx);
     const int32_t ya = max(w.ty0 - cy * by, 0), yb = min(w.ty1 - cy * by, by);
+    if (xb <= xa || yb <= ya) return 0u;
     const uint32_t row = ((1u << xb) - 1u) & ~((1u << xa) - 1u);
-    uint32_t m = 0;
-    for (int32_t ly = ya; ly < yb; ++ly) m |= row << (ly << cg.bshift);
-    return m;
+    // the row repeated in the block rows ya .. yb - 1: a product with one bit per block row
+    // (the rows do not overlap, so nothing carries)
+    const uint32_t every = cg.bshift == 2 ? 0x1111u : (cg.bshift == 1 ? 0x55u : 0xFu);
+    const uint32_t rows = every & ((1u << (yb << cg.bshift)) - 1u) & ~((1u << (ya << cg.bshift)) - 1u);
+    return __umul24(row, rows);
 }
 
 // Depth slabs.  Where a tile meets thousands of Gaussians (a lidar sweep's wide tiles), one
@@ -446,7 +445,7 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
     __shared__ uint32_t s_bounds[1u << kSlabShiftMax];
     SPLATAD_STAGE_ELEVATIONS(g)
     // blocks and block counters below are (coarse block, slab) pairs, the slab in the low bits
-    const uint32_t per_cam = (cg.cw * cg.ch) << sshift, tiles_per_cam = g.tile_w * g.tile_h;
+    const uint32_t per_cam = (cg.cw * cg.ch) << sshift;
     const uint32_t first = cam_lo * per_cam, count = (cam_hi - cam_lo) * per_cam;
     const uint32_t n_bounds = (1u << sshift) - 1u;
     int32_t *row = table + (size_t)blockIdx.x * n_blocks + first;
@@ -460,11 +459,11 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
     for (uint64_t base = (uint64_t)blockIdx.x * blockDim.x; base < total; base += round) { // uniform
         const bool was_kept = ahead.in_range && (LIDAR ? __uint_as_float(ahead.radii.x) > 0.f
                                                        : (int32_t)ahead.radii.x > 0);
+        const uint32_t cam = ahead.cam;
         LaneWork mine = make_work<LIDAR>(g, ahead);
         // the inputs of the next round are requested before this round's emission
         ahead = fetch_work(base + round + threadIdx.x, total, N, camera_ids, means2d, radii,
                            depths_needed, nullptr);
-        const uint32_t cam = mine.base / tiles_per_cam;
         if (cam < cam_lo || cam >= cam_hi) mine.cnt = 0;
         // Rows of a dense [C, N] projection standing in for its packed rows: the entries carry
         // the row's position among the kept rows (an increasing function of the dense index, so
@@ -535,7 +534,10 @@ __device__ __forceinline__ void classify_segment(uint32_t seg, uint32_t lane, ui
 // block a ballot over the mask bit gives the number of entries and every entry's rank, and
 // the lane that owns the tile issues the one atomic.  FILL == false adds to the tile counts,
 // FILL == true reserves the run in the tile's segment and writes the pairs.
-template <bool FILL>
+// BITS == 16: blocks of 4 x 4 tiles (every camera grid, lidar grids whose columns divide by 4),
+// the loops over the tiles unrolled with the ballots kept in scalar registers; BITS == 0: any
+// block width.
+template <bool FILL, int BITS>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t sshift,
                       uint32_t copies, uint32_t n_segments, const int64_t *__restrict__ n_entries_ptr,
@@ -555,6 +557,8 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
             classify_segment((uint32_t)s0 + lane, lane, n_segments, sshift, n_isects, tile_starts,
                              seg_counts, seg_lists, tile_offsets);
     const uint32_t bits = 4u << cg.bshift, per_cam = cg.cw * cg.ch;
+    const float inv_cw = 1.0f / (float)cg.cw;
+    const uint32_t cap = (uint32_t)n_isects; // below 2^31
     const uint64_t below = (1ull << lane) - 1ull;
     // the tile counters are replicated like the coarse ones; both passes run on the same
     // grid, so an entry meets the same copy in both
@@ -571,16 +575,28 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
             const uint32_t block = block_slab >> sshift, slab = block_slab & ((1u << sshift) - 1u);
             todo &= ~__ballot(in);
             uint32_t my_cnt = 0;
-            for (uint32_t t = 0; t < bits; ++t) {
-                const uint64_t b = __ballot(in && ((rec.w >> t) & 1u));
-                if (lane == t) my_cnt = (uint32_t)__popcll(b);
+            const uint32_t mask = in ? rec.w : 0u;
+            uint64_t hits[BITS > 0 ? BITS : 1];
+            if (BITS > 0) {
+#pragma unroll
+                for (int t = 0; t < BITS; ++t) {
+                    hits[t] = __ballot((mask >> t) & 1u);
+                    const uint32_t n_hits = (uint32_t)__popcll(hits[t]); // uniform
+                    asm("v_writelane_b32 %0, %1, %2" : "+v"(my_cnt) : "s"(n_hits), "n"(t));
+                }
+            } else {
+                for (uint32_t t = 0; t < bits; ++t) {
+                    const uint64_t b = __ballot((mask >> t) & 1u);
+                    if (lane == t) my_cnt = (uint32_t)__popcll(b);
+                }
             }
             // lane t < bits owns tile t of the block
             int64_t tile = copy_base;
             if (lane < bits) {
-                const uint32_t cam = block / per_cam, r = block % per_cam;
-                const uint32_t x = ((r % cg.cw) << cg.bshift) + (lane & ((1u << cg.bshift) - 1u));
-                const uint32_t y = ((r / cg.cw) << kCoarseRowShift) + (lane >> cg.bshift);
+                const uint32_t cam = block < per_cam ? 0u : block / per_cam, r = block - cam * per_cam;
+                const uint32_t by = div_by(r, cg.cw, inv_cw), bx = r - by * cg.cw;
+                const uint32_t x = (bx << cg.bshift) + (lane & ((1u << cg.bshift) - 1u));
+                const uint32_t y = (by << kCoarseRowShift) + (lane >> cg.bshift);
                 tile += (((int64_t)cam * tile_w * tile_h + (int64_t)y * tile_w + x) << sshift) | slab;
             }
             if (!FILL) {
@@ -589,14 +605,25 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
                 int32_t dst = 0;
                 if (my_cnt) dst = tile_starts[tile] + atomicAdd(&tile_fill[tile], (int32_t)my_cnt);
                 const uint64_t pair = ((uint64_t)rec.y << 32) | (uint64_t)rec.x;
-                for (uint32_t t = 0; t < bits; ++t) {
-                    const bool hit = in && ((rec.w >> t) & 1u);
-                    const uint64_t b = __ballot(hit);
-                    const int32_t first = __shfl(dst, (int)t, SPLATAD_WAVE);
-                    // (the bound holds whenever n_isects is the count of these very rows; it
-                    // keeps a caller's mismatch from writing outside the lists)
-                    const int64_t at = (int64_t)first + __popcll(b & below);
-                    if (hit && at < n_isects) pairs[at] = pair;
+                // (the bound `cap` holds whenever n_isects is the count of these very rows; it
+                // keeps a caller's mismatch from writing outside the lists)
+                if (BITS > 0) {
+#pragma unroll
+                    for (int t = 0; t < BITS; ++t) {
+                        if (hits[t] == 0) continue; // uniform
+                        const uint32_t first = (uint32_t)__builtin_amdgcn_readlane(dst, t);
+                        const uint32_t at = __builtin_amdgcn_mbcnt_hi(
+                            (uint32_t)(hits[t] >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)hits[t], first));
+                        if (((mask >> t) & 1u) && at < cap) pairs[at] = pair;
+                    }
+                } else {
+                    for (uint32_t t = 0; t < bits; ++t) {
+                        const bool hit = (mask >> t) & 1u;
+                        const uint64_t b = __ballot(hit);
+                        const int32_t first = __shfl(dst, (int)t, SPLATAD_WAVE);
+                        const uint32_t at = (uint32_t)first + (uint32_t)__popcll(b & below);
+                        if (hit && at < cap) pairs[at] = pair;
+                    }
                 }
             }
         }
@@ -613,10 +640,11 @@ isect_emit_kernel(TileGrid g, uint64_t total, uint32_t N, const int64_t *__restr
                   int32_t *__restrict__ flatten_ids) {
     SPLATAD_STAGE_ELEVATIONS(g)
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const LaneWork mine = load_work<LIDAR>(g, idx, total, N, camera_ids, means2d, radii, depths, cum_before);
-    const uint32_t tiles_per_cam = g.tile_w * g.tile_h;
+    const WorkInputs in = fetch_work(idx, total, N, camera_ids, means2d, radii, depths, cum_before);
+    LaneWork mine = make_work<LIDAR>(g, in);
+    mine.base = in.cam; // here the camera itself, not its first tile
     for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t t) {
-        const int64_t cid_enc = (int64_t)(w.base / tiles_per_cam) << (32 + tile_n_bits);
+        const int64_t cid_enc = (int64_t)w.base << (32 + tile_n_bits);
         const int64_t depth_enc = (int64_t)(int32_t)w.depth_bits;
         const int64_t tile_id = tile_index<LIDAR>(g, y, x);
         isect_ids[w.cum + t] = cid_enc | (tile_id << 32) | depth_enc;
@@ -1592,7 +1620,9 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     const uint32_t tcopies = isect_copies(segs);
     uint64_t bin_wgs = ((uint64_t)n_isects + SPLATAD_THREADS - 1) / SPLATAD_THREADS;
     if (bin_wgs > 8192) bin_wgs = 8192;
-    hipLaunchKernelGGL(isect_tile_bin_kernel<false>, dim3((uint32_t)bin_wgs),
+    const bool square = cg.bshift == 2; // 4 x 4 tiles per block: the unrolled kernels
+    hipLaunchKernelGGL((square ? isect_tile_bin_kernel<false, 16> : isect_tile_bin_kernel<false, 0>),
+                       dim3((uint32_t)bin_wgs),
                        dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, sshift, tcopies,
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
                        w.tile_counts, (const int32_t *)nullptr, (int32_t *)nullptr,
@@ -1603,7 +1633,8 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                                         tcopies > 1 ? -(int)tcopies : 1, 0, w.tile_starts,
                                         w.scan_total, w.block_sums, stream);
     if (rc) return rc;
-    hipLaunchKernelGGL(isect_tile_bin_kernel<true>, dim3((uint32_t)bin_wgs),
+    hipLaunchKernelGGL((square ? isect_tile_bin_kernel<true, 16> : isect_tile_bin_kernel<true, 0>),
+                       dim3((uint32_t)bin_wgs),
                        dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, sshift, tcopies,
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
                        w.tile_counts, (const int32_t *)w.tile_starts, w.tile_fill, w.pairs, n_isects,
