@@ -84,18 +84,28 @@ int splatad_projection_packed_count_tiles(uint32_t C, uint32_t N, const float *m
  * packed rows: the lists it writes are those of splatad_isect_tiles_count / _fill on the packed
  * outputs of splatad_projection_packed_fill (tiles_per_gauss [nnz] included), without the wait.
  * Both workspaces must be untouched since the counting call; `lists` is
- * splatad_isect_lists_bytes(C * N, n_isects) bytes of scratch. */
+ * splatad_isect_lists_bytes(C * N, n_isects) bytes of scratch.
+ * beside_stream (may be NULL): another stream of the caller's, which this call makes wait for
+ * the point where the binning is done and the segment sort starts; work the caller enqueues there
+ * afterwards (that needs the projection only: splatad_projection_packed_fill,
+ * splatad_view_colors_fwd_packed) runs beside the sort, whose long workgroups leave part of the
+ * GPU idle.  Nothing waits for that stream: the caller joins it.  (A cross-stream wait costs
+ * the host about 10 us on this runtime, four kernel launches; here it rides on the fork the
+ * sort makes anyway.) */
 int splatad_isect_tiles_fill_packed(uint32_t C, uint32_t N, uint32_t tile_size, uint32_t tile_width,
                                     uint32_t tile_height, int64_t n_isects,
                                     const void *packed_workspace, void *isect_workspace, void *lists,
                                     int32_t *tiles_per_gauss, int64_t *isect_ids,
                                     int32_t *flatten_ids, int32_t *tile_offsets,
-                                    splatad_stream_t stream);
+                                    splatad_stream_t beside_stream, splatad_stream_t stream);
+/* opacities [N] and row_opacities [nnz] (both or neither): the kept rows' opacity for the
+ * compositing, opacities[gaussian] times the row's compensation when compensations are
+ * computed (rendering.py:311-314 of the reference does this with a gather and a product). */
 int splatad_projection_packed_fill(uint32_t C, uint32_t N, int64_t nnz, const void *workspace,
                                    int32_t *indptr, int64_t *camera_ids, int64_t *gaussian_ids,
                                    int32_t *radii, float *means2d, float *depths, float *conics,
-                                   float *compensations, float *pix_vels,
-                                   splatad_stream_t stream);
+                                   float *compensations, float *pix_vels, const float *opacities,
+                                   float *row_opacities, splatad_stream_t stream);
 
 /* fully_fused_lidar_projection_fwd_tensor, projection.cu:2631-2714 (kernel :2268-2417). */
 int splatad_lidar_projection_fwd(uint32_t C, uint32_t N, const float *means, const float *covars,
@@ -172,6 +182,21 @@ int splatad_view_colors_fwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint
                             const int64_t *gaussian_ids, const int32_t *radii, const float *coeffs,
                             int coeffs_per_sensor, const float *depths, float *colors,
                             splatad_stream_t stream);
+/* _fwd over dense [C, N] rows that stand in for their packed rows: an active row e writes its
+ * colours to row remap[e] of `colors` (its position among the kept rows), inactive rows write
+ * nothing; depths, if given, is indexed by e as well.  Same values as _fwd on the packed rows
+ * (one dependent load less per row).  _packed takes the rows, positions and depths from the
+ * workspace of splatad_projection_packed_count[_tiles]: colors is [nnz, 3], or [nnz, 4]
+ * with_depth. */
+int splatad_view_colors_fwd_remapped(uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
+                                     const float *means, const float *viewmats, const int32_t *radii,
+                                     const int32_t *remap, const float *coeffs, int coeffs_per_sensor,
+                                     const float *depths, float *colors, splatad_stream_t stream);
+int splatad_view_colors_fwd_packed(uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
+                                   const float *means, const float *viewmats,
+                                   const void *packed_workspace, const float *coeffs,
+                                   int coeffs_per_sensor, int with_depth, float *colors,
+                                   splatad_stream_t stream);
 int splatad_view_colors_bwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
                             const float *means, const float *viewmats, const int64_t *camera_ids,
                             const int64_t *gaussian_ids, const int32_t *radii, const float *coeffs,
@@ -225,14 +250,16 @@ int splatad_isect_tiles_prepare(uint64_t total, uint32_t N, const int64_t *camer
                                 void *workspace, splatad_stream_t stream);
 /* _fill for dense [C, N] rows that stand in for their packed rows: `remap` [C * N] holds each
  * kept row's position among the kept rows (what flatten_ids must name); tiles_out, if not NULL,
- * receives the kept rows' tile counts at those positions. */
+ * receives the kept rows' tile counts at those positions.  beside_stream: see
+ * splatad_isect_tiles_fill_packed. */
 int splatad_isect_tiles_fill_remapped(uint64_t total, uint32_t N, const float *means2d,
                                       const int32_t *radii, const float *depths, uint32_t C,
                                       uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
                                       int64_t n_isects, const int32_t *tiles_per_gauss,
                                       const int32_t *remap, void *workspace, void *lists,
                                       int32_t *tiles_out, int64_t *isect_ids, int32_t *flatten_ids,
-                                      int32_t *tile_offsets, splatad_stream_t stream);
+                                      int32_t *tile_offsets, splatad_stream_t beside_stream,
+                                      splatad_stream_t stream);
 int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_ids,
                              const float *means2d, const int32_t *radii, const float *depths,
                              uint32_t C, uint32_t tile_size, uint32_t tile_width,

@@ -440,8 +440,13 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
                     uint32_t cam_lo, uint32_t cam_hi, uint32_t n_blocks, int32_t *table,
                     uint4 *__restrict__ entries, uint32_t sshift,
                     const uint32_t *__restrict__ slab_bounds, const int32_t *__restrict__ remap,
-                    int32_t *__restrict__ tiles_out) {
+                    int32_t *__restrict__ tiles_out, int32_t *__restrict__ clear, uint64_t clear_words) {
     extern __shared__ int32_t s_blocks[];
+    // (the counting pass can zero the counters of the later stages on the counting kernel's behalf)
+    if (!FILL)
+        for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words;
+             i += (uint64_t)gridDim.x * blockDim.x)
+            clear[i] = 0;
     __shared__ uint32_t s_bounds[1u << kSlabShiftMax];
     SPLATAD_STAGE_ELEVATIONS(g)
     // blocks and block counters below are (coarse block, slab) pairs, the slab in the low bits
@@ -1453,7 +1458,7 @@ template <bool LIDAR>
 static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const IsectWorkspace &w,
                                 uint64_t total, uint32_t N, const int64_t *camera_ids,
                                 const float *means2d, const void *radii, const float *depths,
-                                uint32_t C, hipStream_t stream) {
+                                uint32_t C, hipStream_t stream, bool clear) {
     SPLATAD_REQUIRE(pl.per_cam <= kCoarseLdsBlocks, "isect: %u x %u tiles per sensor exceed the "
                     "binning capacity", g.tile_w, g.tile_h);
     SPLATAD_REQUIRE(pl.blocks < (1ull << 31) && pl.cslots < (1ull << 31), "isect: tile grid too large");
@@ -1477,7 +1482,8 @@ static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const Is
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, pl.cg,
                            total, N, camera_ids, means2d, radii, pl.sshift ? depths : nullptr, c0, c1,
                            (uint32_t)pl.blocks, w.coarse_counts, (uint4 *)nullptr, pl.sshift,
-                           (const uint32_t *)w.slab_bounds, (const int32_t *)nullptr, (int32_t *)nullptr);
+                           (const uint32_t *)w.slab_bounds, (const int32_t *)nullptr, (int32_t *)nullptr,
+                           w.zeroed, clear && c0 == 0 ? w.n_zeroed : (uint64_t)0);
     }
     SPLATAD_LAUNCH_CHECK();
     return launch_exclusive_scan<int32_t>(w.coarse_counts, (int64_t)pl.cslots,
@@ -1540,12 +1546,17 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     }
     // the counting kernel clears the tile counters, the fill cursors and the class counters of
     // the binning behind it
-    dim3 count_grid = grid_for(total);
-    if (count_grid.x > 1024) count_grid.x = 1024;
-    hipLaunchKernelGGL(isect_count_kernel<LIDAR>, count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
-                       total, means2d, radii, tiles_per_gauss, counters, lease.word.device,
-                       w.zeroed, sort ? w.n_zeroed : (uint64_t)0);
-    SPLATAD_LAUNCH_CHECK();
+    // (a caller that knows the count and sorts without depth slabs needs nothing else of the
+    // counting kernel: the coarse counting pass then clears)
+    const bool skip_count = known && sort && pl.sshift == 0;
+    if (!skip_count) {
+        dim3 count_grid = grid_for(total);
+        if (count_grid.x > 1024) count_grid.x = 1024;
+        hipLaunchKernelGGL(isect_count_kernel<LIDAR>, count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
+                           total, means2d, radii, tiles_per_gauss, counters, lease.word.device,
+                           w.zeroed, sort ? w.n_zeroed : (uint64_t)0);
+        SPLATAD_LAUNCH_CHECK();
+    }
     // work for the GPU while the host learns the count and sizes the lists
     if (sort) {
         if (pl.sshift) {
@@ -1554,7 +1565,7 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
             SPLATAD_LAUNCH_CHECK();
         }
         if (int rc = enqueue_coarse_count<LIDAR>(g, pl, w, total, N, camera_ids, means2d, radii, depths,
-                                                 C, stream))
+                                                 C, stream, skip_count))
             return rc;
     }
     if (known) return 0;
@@ -1571,7 +1582,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                       int sort, int64_t n_isects, const int32_t *tiles_per_gauss,
                       void *workspace, void *lists, int64_t *isect_ids, int32_t *flatten_ids,
                       int32_t *tile_offsets, hipStream_t stream, const int32_t *remap = nullptr,
-                      int32_t *tiles_out = nullptr) {
+                      int32_t *tiles_out = nullptr, hipStream_t beside = nullptr) {
     SPLATAD_REQUIRE(remap == nullptr || (sort && camera_ids == nullptr),
                     "isect: remapped rows need sort != 0 and a dense [C, N] layout");
     if (total == 0 || n_isects == 0) {
@@ -1580,6 +1591,13 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
             hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(tiles), dim3(SPLATAD_THREADS), 0,
                                stream, tile_offsets, (int64_t)tiles);
             SPLATAD_LAUNCH_CHECK();
+        }
+        if (beside != nullptr && beside != stream) { // nothing to sort: ordered behind this point
+            IsectDevice *ss = nullptr;
+            if (int rc = isect_device(&ss)) return rc;
+            std::lock_guard<std::mutex> fork_lock(ss->guard);
+            SPLATAD_CHECK_HIP(hipEventRecord(ss->fork, stream));
+            SPLATAD_CHECK_HIP(hipStreamWaitEvent(beside, ss->fork, 0));
         }
         return 0;
     }
@@ -1612,7 +1630,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, cg,
                            total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)pl.blocks,
                            w.coarse_starts, w.entries, sshift, (const uint32_t *)w.slab_bounds, remap,
-                           tiles_out);
+                           tiles_out, (int32_t *)nullptr, (uint64_t)0);
     }
     SPLATAD_LAUNCH_CHECK();
     // tile segments: count, scan, fill.  The number of coarse entries stays on the device;
@@ -1652,6 +1670,8 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     std::lock_guard<std::mutex> fork_lock(ss->guard);
     SPLATAD_CHECK_HIP(hipEventRecord(ss->fork, stream));
     for (hipStream_t aux : ss->aux) SPLATAD_CHECK_HIP(hipStreamWaitEvent(aux, ss->fork, 0));
+    // a stream of the caller's for work of its own beside the sort: ordered behind the binning
+    if (beside != nullptr && beside != stream) SPLATAD_CHECK_HIP(hipStreamWaitEvent(beside, ss->fork, 0));
     // After the fork the helper streams are joined whatever happens: work already queued on
     // them reads and writes the caller's buffers, so the caller's stream must not run past it.
     auto enqueue_sorts = [&]() -> int {
@@ -1741,13 +1761,14 @@ extern "C" int splatad_isect_tiles_fill_remapped(uint64_t total, uint32_t N, con
                                                  const int32_t *tiles_per_gauss, const int32_t *remap,
                                                  void *workspace, void *lists, int32_t *tiles_out,
                                                  int64_t *isect_ids, int32_t *flatten_ids,
-                                                 int32_t *tile_offsets, splatad_stream_t stream) {
+                                                 int32_t *tile_offsets, splatad_stream_t beside_stream,
+                                                 splatad_stream_t stream) {
     SPLATAD_REQUIRE(tile_size > 0, "isect_tiles: tile_size is zero");
     SPLATAD_REQUIRE(remap != nullptr, "isect_tiles: remap is null");
     TileGrid g{tile_size, tile_width, tile_height, 0.f, 0.f, nullptr};
     return isect_fill<false>(g, total, N, nullptr, means2d, radii, depths, C, 1, n_isects, tiles_per_gauss,
                              workspace, lists, isect_ids, flatten_ids, tile_offsets, (hipStream_t)stream,
-                             remap, tiles_out);
+                             remap, tiles_out, (hipStream_t)beside_stream);
 }
 
 extern "C" int splatad_isect_lidar_tiles_count(uint64_t total, uint32_t N,

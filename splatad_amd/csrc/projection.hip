@@ -121,6 +121,10 @@ __device__ __forceinline__ void relative_velocity(const SensorPose &p, const flo
     }
 }
 
+// COUNT: every workgroup also writes how many of its rows are kept (radii.x > 0) and how many
+// tiles of the camera's grid those meet: the counts of the packed layout and of its tile
+// intersection, gathered while the rows are in registers.
+template <bool COUNT>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 projection_fwd_kernel(uint32_t C, uint32_t N, const float *__restrict__ means,
                       const float *__restrict__ covars, const float *__restrict__ quats,
@@ -131,10 +135,14 @@ projection_fwd_kernel(uint32_t C, uint32_t N, const float *__restrict__ means,
                       float eps2d, float near_plane, float far_plane, float radius_clip,
                       int32_t *__restrict__ radii, float *__restrict__ means2d,
                       float *__restrict__ depths, float *__restrict__ conics,
-                      float *__restrict__ compensations, float *__restrict__ pix_vels) {
+                      float *__restrict__ compensations, float *__restrict__ pix_vels,
+                      uint32_t tile_size, uint32_t tile_w, uint32_t tile_h,
+                      int64_t *__restrict__ kept_sums, int64_t *__restrict__ tile_sums) {
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (uint64_t)C * N) return;
-    const uint32_t cid = (uint32_t)(idx / N), gid = (uint32_t)(idx % N);
+    const bool live = idx < (uint64_t)C * N;
+    if (!COUNT && !live) return;
+    // (a lane beyond the last row works on row 0 and stores nothing: it is needed for the sums)
+    const uint32_t cid = live ? (uint32_t)(idx / N) : 0u, gid = live ? (uint32_t)(idx % N) : 0u;
 
     int2 o_radii = make_int2(0, 0);
     float2 o_mean = make_float2(0.f, 0.f), o_vel = make_float2(0.f, 0.f);
@@ -194,12 +202,38 @@ projection_fwd_kernel(uint32_t C, uint32_t N, const float *__restrict__ means,
             }
         }
     }
-    reinterpret_cast<int2 *>(radii)[idx] = o_radii;
-    reinterpret_cast<float2 *>(means2d)[idx] = o_mean;
-    depths[idx] = o_depth;
-    conics[idx * 3] = o_c0; conics[idx * 3 + 1] = o_c1; conics[idx * 3 + 2] = o_c2;
-    if (compensations != nullptr) compensations[idx] = o_comp;
-    reinterpret_cast<float2 *>(pix_vels)[idx] = o_vel;
+    if (live) {
+        reinterpret_cast<int2 *>(radii)[idx] = o_radii;
+        reinterpret_cast<float2 *>(means2d)[idx] = o_mean;
+        depths[idx] = o_depth;
+        conics[idx * 3] = o_c0; conics[idx * 3 + 1] = o_c1; conics[idx * 3 + 2] = o_c2;
+        if (compensations != nullptr) compensations[idx] = o_comp;
+        reinterpret_cast<float2 *>(pix_vels)[idx] = o_vel;
+    }
+    if (COUNT) {
+        __shared__ int64_t s_sums[2 * (SPLATAD_THREADS / SPLATAD_WAVE)];
+        int64_t kept = 0, tiles = 0;
+        if (live && o_radii.x > 0) {
+            int32_t x0, y0, x1, y1;
+            splatad_camera_tile_rect(tile_size, tile_w, tile_h, o_mean, o_radii, x0, y0, x1, y1);
+            kept = 1;
+            tiles = (int64_t)max(y1 - y0, 0) * max(x1 - x0, 0);
+        }
+#pragma unroll
+        for (int off = SPLATAD_WAVE / 2; off > 0; off >>= 1) {
+            kept += __shfl_xor(kept, off, SPLATAD_WAVE);
+            tiles += __shfl_xor(tiles, off, SPLATAD_WAVE);
+        }
+        const uint32_t wave = threadIdx.x / SPLATAD_WAVE;
+        if ((threadIdx.x & (SPLATAD_WAVE - 1)) == 0) { s_sums[2 * wave] = kept; s_sums[2 * wave + 1] = tiles; }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            kept = tiles = 0;
+            for (uint32_t w = 0; w < SPLATAD_THREADS / SPLATAD_WAVE; ++w) { kept += s_sums[2 * w]; tiles += s_sums[2 * w + 1]; }
+            kept_sums[blockIdx.x] = kept;
+            tile_sums[blockIdx.x] = tiles;
+        }
+    }
 }
 
 __global__ void __launch_bounds__(SPLATAD_THREADS)
@@ -302,7 +336,7 @@ struct PackedWorkspace {
     int32_t *pos;     // [T] exclusive prefix of the valid flags
     int64_t *total;   // [1]
     int64_t *block_sums;
-    int64_t *tile_sums; // [scan blocks] tiles met by the kept rows of a scan block (optional count)
+    int64_t *tile_sums; // tiles met by the kept rows of a scan block or projection workgroup (optional count)
     int32_t *tiles;     // [T] tiles per dense row (intersection started by the counting call)
 };
 
@@ -317,8 +351,9 @@ static PackedWorkspace carve_packed(void *ws, uint64_t T) {
     w.comps = (float *)p;         p += splatad_align256(T * 4);
     w.pix_vels = (float *)p;      p += splatad_align256(T * 8);
     w.pos = (int32_t *)p;         p += splatad_align256(T * 4);
-    w.block_sums = (int64_t *)p;  p += scan_workspace_bytes((int64_t)T);
-    w.tile_sums = (int64_t *)p;   p += scan_workspace_bytes((int64_t)T);
+    // (room for the counts of every projection workgroup, SCAN_ITEMS per scan block)
+    w.block_sums = (int64_t *)p;  p += SCAN_ITEMS * scan_workspace_bytes((int64_t)T);
+    w.tile_sums = (int64_t *)p;   p += SCAN_ITEMS * scan_workspace_bytes((int64_t)T);
     w.tiles = (int32_t *)p;
     return w;
 }
@@ -356,16 +391,23 @@ packed_block_totals_kernel(uint64_t T, const int32_t *__restrict__ w_radii,
 
 // One workgroup: publishes the number of kept rows (low 32 bits) and of their tile
 // intersections (high 32 bits, saturated at 2^31 - 1, which the caller refuses) in one word.
+// The kept rows are *total when that is given, the sum of kept_sums otherwise.
 __global__ void __launch_bounds__(SPLATAD_THREADS)
-packed_publish_kernel(const int64_t *__restrict__ total, const int64_t *__restrict__ tile_sums,
-                      int64_t n_blocks, unsigned long long *__restrict__ word) {
-    int64_t part = 0;
-    for (int64_t b = threadIdx.x; b < n_blocks; b += SPLATAD_THREADS) part += tile_sums[b];
-    int64_t tiles;
+packed_publish_kernel(const int64_t *__restrict__ total, const int64_t *__restrict__ kept_sums,
+                      const int64_t *__restrict__ tile_sums, int64_t n_blocks,
+                      unsigned long long *__restrict__ word) {
+    int64_t part = 0, part_kept = 0;
+    for (int64_t b = threadIdx.x; b < n_blocks; b += SPLATAD_THREADS) {
+        part += tile_sums[b];
+        if (total == nullptr) part_kept += kept_sums[b];
+    }
+    int64_t tiles, kept;
     block_exclusive_scan(part, &tiles);
+    block_exclusive_scan(part_kept, &kept);
     if (threadIdx.x == 0) {
+        if (total != nullptr) kept = *total;
         const unsigned long long hi = tiles > 0x7FFFFFFFll ? 0x7FFFFFFFull : (unsigned long long)tiles;
-        __hip_atomic_store(word, (hi << 32) | (unsigned long long)(uint32_t)*total, __ATOMIC_RELAXED,
+        __hip_atomic_store(word, (hi << 32) | (unsigned long long)(uint32_t)kept, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_SYSTEM);
     }
 }
@@ -379,7 +421,8 @@ packed_compact_kernel(uint32_t C, uint32_t N, int64_t nnz, const int32_t *__rest
                       int64_t *__restrict__ gaussian_ids, int32_t *__restrict__ radii,
                       float *__restrict__ means2d, float *__restrict__ depths,
                       float *__restrict__ conics, float *__restrict__ comps,
-                      float *__restrict__ pix_vels) {
+                      float *__restrict__ pix_vels, const float *__restrict__ opacities,
+                      float *__restrict__ row_opacities) {
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const uint64_t T = (uint64_t)C * N;
     if (idx >= T) return;
@@ -399,6 +442,9 @@ packed_compact_kernel(uint32_t C, uint32_t N, int64_t nnz, const int32_t *__rest
     conics[o * 3 + 2] = w_conics[idx * 3 + 2];
     if (comps != nullptr) comps[o] = w_comps[idx];
     reinterpret_cast<float2 *>(pix_vels)[o] = reinterpret_cast<const float2 *>(w_pix_vels)[idx];
+    // the opacity the compositing takes for the row: the Gaussian's, times the compensation
+    // when there is one (rendering.py:311-314 of the reference)
+    if (row_opacities != nullptr) row_opacities[o] = comps != nullptr ? opacities[gid] * w_comps[idx] : opacities[gid];
 }
 
 __global__ void fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {
@@ -407,6 +453,40 @@ __global__ void fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {
 }
 
 } // namespace
+
+// kept_sums / tile_sums (both or neither): per-workgroup counts for the packed layout, see
+// projection_fwd_kernel<true>.
+static int projection_fwd(uint32_t C, uint32_t N, const float *means,
+                                      const float *covars, const float *quats,
+                                      const float *scales, const float *velocities,
+                                      const float *viewmats, const float *Ks, uint32_t W,
+                                      uint32_t H, const float *lin_vel, const float *ang_vel,
+                                      const float *rs_time, float eps2d, float near_plane,
+                                      float far_plane, float radius_clip, int32_t *radii,
+                                      float *means2d, float *depths, float *conics,
+                                      float *compensations, float *pix_vels,
+                                      uint32_t tile_size, uint32_t tile_w, uint32_t tile_h,
+                                      int64_t *kept_sums, int64_t *tile_sums,
+                                      splatad_stream_t stream) {
+    SPLATAD_REQUIRE((covars != nullptr) != (quats != nullptr && scales != nullptr),
+                    "projection: pass either covars or (quats, scales)");
+    SPLATAD_REQUIRE((uint64_t)C * N < (1ull << 31), "projection: C*N must be below 2^31");
+    if (C == 0 || N == 0) return 0;
+    SPLATAD_REQUIRE(means && viewmats && Ks && lin_vel && ang_vel && rs_time && radii && means2d &&
+                        depths && conics && pix_vels,
+                    "projection: null pointer argument");
+    const uint64_t T = (uint64_t)C * N;
+    const bool count = kept_sums != nullptr;
+    SPLATAD_REQUIRE(!count || (tile_sums != nullptr && tile_size > 0), "projection: incomplete count arguments");
+    hipLaunchKernelGGL((count ? projection_fwd_kernel<true> : projection_fwd_kernel<false>),
+                       dim3((uint32_t)((T + SPLATAD_THREADS - 1) / SPLATAD_THREADS)),
+                       dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, C, N, means, covars, quats,
+                       scales, velocities, viewmats, Ks, W, H, lin_vel, ang_vel, rs_time, eps2d,
+                       near_plane, far_plane, radius_clip, radii, means2d, depths, conics,
+                       compensations, pix_vels, tile_size, tile_w, tile_h, kept_sums, tile_sums);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
+}
 
 extern "C" int splatad_projection_fwd(uint32_t C, uint32_t N, const float *means,
                                       const float *covars, const float *quats,
@@ -418,21 +498,9 @@ extern "C" int splatad_projection_fwd(uint32_t C, uint32_t N, const float *means
                                       float *means2d, float *depths, float *conics,
                                       float *compensations, float *pix_vels,
                                       splatad_stream_t stream) {
-    SPLATAD_REQUIRE((covars != nullptr) != (quats != nullptr && scales != nullptr),
-                    "projection: pass either covars or (quats, scales)");
-    SPLATAD_REQUIRE((uint64_t)C * N < (1ull << 31), "projection: C*N must be below 2^31");
-    if (C == 0 || N == 0) return 0;
-    SPLATAD_REQUIRE(means && viewmats && Ks && lin_vel && ang_vel && rs_time && radii && means2d &&
-                        depths && conics && pix_vels,
-                    "projection: null pointer argument");
-    const uint64_t T = (uint64_t)C * N;
-    hipLaunchKernelGGL(projection_fwd_kernel, dim3((uint32_t)((T + SPLATAD_THREADS - 1) / SPLATAD_THREADS)),
-                       dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, C, N, means, covars, quats,
-                       scales, velocities, viewmats, Ks, W, H, lin_vel, ang_vel, rs_time, eps2d,
-                       near_plane, far_plane, radius_clip, radii, means2d, depths, conics,
-                       compensations, pix_vels);
-    SPLATAD_LAUNCH_CHECK();
-    return 0;
+    return projection_fwd(C, N, means, covars, quats, scales, velocities, viewmats, Ks, W, H, lin_vel,
+                          ang_vel, rs_time, eps2d, near_plane, far_plane, radius_clip, radii, means2d,
+                          depths, conics, compensations, pix_vels, 0, 0, 0, nullptr, nullptr, stream);
 }
 
 extern "C" int splatad_lidar_projection_fwd(uint32_t C, uint32_t N, const float *means,
@@ -467,7 +535,7 @@ extern "C" int splatad_lidar_projection_fwd(uint32_t C, uint32_t N, const float 
 extern "C" size_t splatad_projection_packed_workspace_bytes(uint32_t C, uint32_t N) {
     const uint64_t T = (uint64_t)C * N;
     return 256 + splatad_align256(T * 8) * 3 + splatad_align256(T * 4) * 3 +
-           splatad_align256(T * 12) + 2 * scan_workspace_bytes((int64_t)T) + splatad_align256(T * 4);
+           splatad_align256(T * 12) + 2 * SCAN_ITEMS * scan_workspace_bytes((int64_t)T) + splatad_align256(T * 4);
 }
 
 // tile_size == 0: only the kept rows are counted.
@@ -489,19 +557,39 @@ static int packed_count(uint32_t C, uint32_t N, const float *means, const float 
     // the counts reach the host through a leased pinned word
     HostWordLease lease((hipStream_t)stream);
     if (int rc = host_word_acquire(&lease.word)) return rc;
-    int rc = splatad_projection_fwd(C, N, means, covars, quats, scales, velocities, viewmats, Ks,
-                                    W, H, lin_vel, ang_vel, rs_time, eps2d, near_plane, far_plane,
-                                    radius_clip, w.radii, w.means2d, w.depths, w.conics,
-                                    calc_compensations ? w.comps : nullptr, w.pix_vels, stream);
+    // Up to kScanFoldBlocks scan blocks the projection itself counts, per workgroup, the kept
+    // rows and their tiles: the host word is published right behind it, and the scan's second
+    // half adds up the workgroups' counts before its block (SCAN_ITEMS of them per scan block).
+    static_assert(SCAN_TILE == SCAN_ITEMS * SPLATAD_THREADS, "a scan block is SCAN_ITEMS projection workgroups");
+    const int64_t n_blocks = ((int64_t)T + SCAN_TILE - 1) / SCAN_TILE;
+    const int64_t n_groups = ((int64_t)T + SPLATAD_THREADS - 1) / SPLATAD_THREADS;
+    const bool fused = tile_size != 0 && n_blocks <= kScanFoldBlocks;
+    int rc = projection_fwd(C, N, means, covars, quats, scales, velocities, viewmats, Ks, W, H, lin_vel,
+                            ang_vel, rs_time, eps2d, near_plane, far_plane, radius_clip, w.radii, w.means2d,
+                            w.depths, w.conics, calc_compensations ? w.comps : nullptr, w.pix_vels,
+                            fused ? tile_size : 0, tile_width, tile_height, fused ? w.block_sums : nullptr,
+                            fused ? w.tile_sums : nullptr, stream);
     if (rc) return rc;
-    if (tile_size == 0) {
+    if (fused) {
+        hipLaunchKernelGGL(packed_publish_kernel, dim3(1), dim3(SPLATAD_THREADS), 0, (hipStream_t)stream,
+                           (const int64_t *)nullptr, (const int64_t *)w.block_sums, (const int64_t *)w.tile_sums,
+                           n_groups, lease.word.device);
+        SPLATAD_LAUNCH_CHECK();
+        rc = launch_exclusive_scan_apply<int32_t>(w.radii, (int64_t)T, 2, 1, w.pos, w.total, w.block_sums,
+                                                  (hipStream_t)stream, SCAN_ITEMS);
+        if (rc) return rc;
+        if (isect_workspace != nullptr) {
+            rc = splatad_isect_tiles_prepare(T, N, nullptr, w.means2d, w.radii, w.depths, C, tile_size,
+                                             tile_width, tile_height, 1, w.tiles, isect_workspace, stream);
+            if (rc) return rc;
+        }
+    } else if (tile_size == 0) {
         rc = launch_exclusive_scan<int32_t>(w.radii, (int64_t)T, 2, 1, w.pos, w.total, w.block_sums,
                                             (hipStream_t)stream);
         if (rc) return rc;
         hipLaunchKernelGGL(host_word_publish_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, w.total,
                            lease.word.device);
     } else {
-        const int64_t n_blocks = ((int64_t)T + SCAN_TILE - 1) / SCAN_TILE;
         hipLaunchKernelGGL(packed_block_totals_kernel, dim3((uint32_t)n_blocks), dim3(SPLATAD_THREADS), 0,
                            (hipStream_t)stream, T, (const int32_t *)w.radii, (const float *)w.means2d, tile_size,
                            tile_width, tile_height, w.block_sums, w.tile_sums);
@@ -510,7 +598,8 @@ static int packed_count(uint32_t C, uint32_t N, const float *means, const float 
                                                   (hipStream_t)stream);
         if (rc) return rc;
         hipLaunchKernelGGL(packed_publish_kernel, dim3(1), dim3(SPLATAD_THREADS), 0, (hipStream_t)stream,
-                           (const int64_t *)w.total, (const int64_t *)w.tile_sums, n_blocks, lease.word.device);
+                           (const int64_t *)w.total, (const int64_t *)nullptr, (const int64_t *)w.tile_sums,
+                           n_blocks, lease.word.device);
         SPLATAD_LAUNCH_CHECK();
         // work for the GPU while the host learns the counts and sizes the outputs: the first
         // stages of the tile intersection, on the dense rows (culled rows meet no tile)
@@ -565,13 +654,25 @@ extern "C" int splatad_isect_tiles_fill_packed(uint32_t C, uint32_t N, uint32_t 
                                                const void *packed_workspace, void *isect_workspace,
                                                void *lists, int32_t *tiles_per_gauss, int64_t *isect_ids,
                                                int32_t *flatten_ids, int32_t *tile_offsets,
-                                               splatad_stream_t stream) {
+                                               splatad_stream_t beside_stream, splatad_stream_t stream) {
     SPLATAD_REQUIRE(packed_workspace && isect_workspace, "isect_tiles: null workspace");
     const uint64_t T = (uint64_t)C * N;
     PackedWorkspace w = carve_packed((void *)packed_workspace, T);
     return splatad_isect_tiles_fill_remapped(T, N, w.means2d, w.radii, w.depths, C, tile_size, tile_width,
                                              tile_height, n_isects, w.tiles, w.pos, isect_workspace, lists,
-                                             tiles_per_gauss, isect_ids, flatten_ids, tile_offsets, stream);
+                                             tiles_per_gauss, isect_ids, flatten_ids, tile_offsets,
+                                             beside_stream, stream);
+}
+
+extern "C" int splatad_view_colors_fwd_packed(uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
+                                              const float *means, const float *viewmats,
+                                              const void *packed_workspace, const float *coeffs,
+                                              int coeffs_per_sensor, int with_depth, float *colors,
+                                              splatad_stream_t stream) {
+    SPLATAD_REQUIRE(packed_workspace != nullptr, "view colours: null workspace");
+    PackedWorkspace w = carve_packed((void *)packed_workspace, (uint64_t)C * N);
+    return splatad_view_colors_fwd_remapped(C, N, K, degree, means, viewmats, w.radii, w.pos, coeffs,
+                                            coeffs_per_sensor, with_depth ? w.depths : nullptr, colors, stream);
 }
 
 extern "C" int splatad_projection_packed_fill(uint32_t C, uint32_t N, int64_t nnz,
@@ -579,8 +680,11 @@ extern "C" int splatad_projection_packed_fill(uint32_t C, uint32_t N, int64_t nn
                                               int64_t *camera_ids, int64_t *gaussian_ids,
                                               int32_t *radii, float *means2d, float *depths,
                                               float *conics, float *compensations,
-                                              float *pix_vels, splatad_stream_t stream) {
+                                              float *pix_vels, const float *opacities,
+                                              float *row_opacities, splatad_stream_t stream) {
     SPLATAD_REQUIRE(indptr != nullptr, "packed projection: indptr is null");
+    SPLATAD_REQUIRE((opacities != nullptr) == (row_opacities != nullptr),
+                    "packed projection: opacities and row_opacities go together");
     const uint64_t T = (uint64_t)C * N;
     if (T == 0 || nnz == 0) {
         hipLaunchKernelGGL(fill_i32_kernel, dim3((C + 1 + 255) / 256), dim3(256), 0,
@@ -597,7 +701,7 @@ extern "C" int splatad_projection_packed_fill(uint32_t C, uint32_t N, int64_t nn
                        dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, C, N, nnz, w.radii,
                        w.means2d, w.depths, w.conics, w.comps, w.pix_vels, w.pos, indptr,
                        camera_ids, gaussian_ids, radii, means2d, depths, conics, compensations,
-                       pix_vels);
+                       pix_vels, opacities, row_opacities);
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }

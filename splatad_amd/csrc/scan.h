@@ -118,15 +118,18 @@ scan_block_sums_kernel(int64_t *__restrict__ block_sums, int64_t n_blocks,
 // FOLD: block_sums holds the blocks' totals, not yet scanned; every workgroup adds up the
 // totals before its own (a few hundred at most, see kScanFoldBlocks) and the last one writes
 // the grand total, which saves the launch of scan_block_sums_kernel.
+// fold_ratio > 1: block_sums holds that many finer totals per block (those of consecutive,
+// equally long parts of it).
 template <typename OutT, bool FOLD>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 scan_apply_kernel(const int32_t *__restrict__ in, int64_t n, int stride, int as_flag,
                   const int64_t *__restrict__ block_sums, OutT *__restrict__ out,
-                  int64_t *__restrict__ total) {
+                  int64_t *__restrict__ total, uint32_t fold_ratio) {
     int64_t before = 0;
     if (FOLD) {
         int64_t part = 0;
-        for (uint32_t j = threadIdx.x; j < blockIdx.x; j += SPLATAD_THREADS) part += block_sums[j];
+        const uint32_t parts_before = blockIdx.x * fold_ratio;
+        for (uint32_t j = threadIdx.x; j < parts_before; j += SPLATAD_THREADS) part += block_sums[j];
         block_exclusive_scan(part, &before);
     } else {
         before = block_sums[blockIdx.x];
@@ -170,22 +173,23 @@ static inline size_t scan_workspace_bytes(int64_t n) {
 template <typename OutT>
 static inline int launch_exclusive_scan_apply(const int32_t *in, int64_t n, int stride, int as_flag,
                                               OutT *out, int64_t *total, int64_t *block_sums,
-                                              hipStream_t stream) {
+                                              hipStream_t stream, uint32_t fold_ratio = 1) {
     const int64_t n_blocks = (n + SCAN_TILE - 1) / SCAN_TILE;
     if (n_blocks > 0 && n_blocks <= kScanFoldBlocks && out != nullptr) {
         hipLaunchKernelGGL((scan_apply_kernel<OutT, true>), dim3((uint32_t)n_blocks),
                            dim3(SPLATAD_THREADS), 0, stream, in, n, stride, as_flag,
-                           (const int64_t *)block_sums, out, total);
+                           (const int64_t *)block_sums, out, total, fold_ratio);
         SPLATAD_LAUNCH_CHECK();
         return 0;
     }
+    SPLATAD_REQUIRE(fold_ratio == 1, "scan: finer totals need the folding pass (%lld blocks)", (long long)n_blocks);
     hipLaunchKernelGGL(scan_block_sums_kernel, dim3(1), dim3(SPLATAD_THREADS), 0, stream,
                        block_sums, n_blocks, total);
     SPLATAD_LAUNCH_CHECK();
     if (n_blocks > 0 && out != nullptr) {
         hipLaunchKernelGGL((scan_apply_kernel<OutT, false>), dim3((uint32_t)n_blocks),
                            dim3(SPLATAD_THREADS), 0, stream, in, n, stride, as_flag,
-                           (const int64_t *)block_sums, out, total);
+                           (const int64_t *)block_sums, out, total, 1u);
         SPLATAD_LAUNCH_CHECK();
     }
     return 0;

@@ -156,13 +156,19 @@ template <bool VIEW>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, ShView view, const float *__restrict__ dirs,
               const float *__restrict__ coeffs, const uint8_t *__restrict__ masks,
-              const float *__restrict__ depths, uint32_t stride, float *__restrict__ colors) {
+              const float *__restrict__ depths, uint32_t stride, float *__restrict__ colors,
+              const int32_t *__restrict__ remap) {
     const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= n) return;
     float r = 0.f, g = 0.f, b = 0.f;
     float dx = 0.f, dy = 0.f, dz = 0.f;
     size_t coeff_row;
-    if (sh_row<VIEW>(e, view, dirs, masks, dx, dy, dz, coeff_row)) {
+    // remap: only the active rows have a place in the output, row e at remap[e]
+    uint32_t at = e;
+    if (VIEW && remap != nullptr) at = (uint32_t)remap[e];
+    const bool active = sh_row<VIEW>(e, view, dirs, masks, dx, dy, dz, coeff_row);
+    if (VIEW && remap != nullptr && !active) return;
+    if (active) {
         const float inorm = rsqrtf(dx * dx + dy * dy + dz * dz);
         const float *cf = coeffs + coeff_row * K * 3;
         float c[75]; // the whole row is requested before the first use: one memory round trip
@@ -178,7 +184,7 @@ sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, ShView view, const float 
                               b += v * c[k * 3 + 2];
                           });
     }
-    float *out = colors + (size_t)e * stride;
+    float *out = colors + (size_t)at * stride;
     if (VIEW) {
         out[0] = fmaxf(r + 0.5f, 0.f);
         out[1] = fmaxf(g + 0.5f, 0.f);
@@ -284,10 +290,10 @@ static int sh_check(uint32_t K, uint32_t degree) {
 template <bool VIEW>
 static int sh_forward(uint32_t n, uint32_t K, uint32_t degree, const ShView &view, const float *dirs,
                       const float *coeffs, const uint8_t *masks, const float *depths,
-                      uint32_t stride, float *colors, hipStream_t stream) {
+                      uint32_t stride, float *colors, hipStream_t stream, const int32_t *remap = nullptr) {
     hipLaunchKernelGGL(sh_fwd_kernel<VIEW>, dim3((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS),
                        dim3(SPLATAD_THREADS), 0, stream, n, K, degree, view, dirs, coeffs, masks,
-                       depths, stride, colors);
+                       depths, stride, colors, remap);
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }
@@ -362,6 +368,24 @@ extern "C" int splatad_view_colors_fwd(uint32_t n, uint32_t C, uint32_t N, uint3
     SPLATAD_REQUIRE(coeffs && colors, "view colours: null pointer argument");
     return sh_forward<true>(n, K, degree, view, nullptr, coeffs, nullptr, depths, depths ? 4u : 3u,
                             colors, (hipStream_t)stream);
+}
+
+extern "C" int splatad_view_colors_fwd_remapped(uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
+                                                const float *means, const float *viewmats,
+                                                const int32_t *radii, const int32_t *remap,
+                                                const float *coeffs, int coeffs_per_sensor,
+                                                const float *depths, float *colors,
+                                                splatad_stream_t stream) {
+    if (int rc = sh_check(K, degree)) return rc;
+    const uint64_t n = (uint64_t)C * N;
+    if (n == 0) return 0;
+    SPLATAD_REQUIRE(n < (1ull << 31), "view colours: C*N must be below 2^31");
+    ShView view;
+    if (int rc = sh_view_args((uint32_t)n, C, N, means, viewmats, nullptr, nullptr, radii, coeffs_per_sensor,
+                              &view)) return rc;
+    SPLATAD_REQUIRE(coeffs && colors && remap, "view colours: null pointer argument");
+    return sh_forward<true>((uint32_t)n, K, degree, view, nullptr, coeffs, nullptr, depths, depths ? 4u : 3u,
+                            colors, (hipStream_t)stream, remap);
 }
 
 extern "C" int splatad_view_colors_bwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K,

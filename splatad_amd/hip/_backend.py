@@ -72,7 +72,28 @@ def _p(t: Optional[Tensor]):
 
 
 def _stream(device):
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    """Handle of torch's current stream on the device (the raw query: the Stream object that
+    torch.cuda.current_stream() builds costs several microseconds per call)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(index))
+
+
+class _on:
+    """`with _on(device)`: torch.cuda.device(device), entered only when another device is current."""
+
+    def __init__(self, device):
+        self._ctx = None
+        if device.index is not None and device.index != torch.cuda.current_device():
+            self._ctx = torch.cuda.device(device)
+
+    def __enter__(self):
+        if self._ctx is not None:
+            self._ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self._ctx is not None:
+            return self._ctx.__exit__(*exc)
+        return False
 
 
 _u32, _i32, _i64, _u64, _f32 = ctypes.c_uint32, ctypes.c_int, ctypes.c_int64, ctypes.c_uint64, ctypes.c_float
@@ -142,7 +163,7 @@ class _Ops:
         means2d = torch.empty((C, N, 2), **f); depths = torch.empty((C, N), **f)
         conics = torch.empty((C, N, 3), **f); pix_vels = torch.empty((C, N, 2), **f)
         comps = torch.empty((C, N), **f) if calc_compensations else None
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_projection_fwd(
                 _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
                 _p(viewmats), _p(Ks), _u32(image_width), _u32(image_height), _p(lv), _p(av), _p(rs),
@@ -154,10 +175,21 @@ class _Ops:
                                           Ks, image_width, image_height, linear_velocity,
                                           angular_velocity, rolling_shutter_time, eps2d, near_plane,
                                           far_plane, radius_clip, calc_compensations,
-                                          isect_grid=None):
+                                          isect_grid=None, beside=None):
         """isect_grid = (tile_size, tile_width, tile_height): the counting call also counts the
-        tile intersections of the rows it keeps (no second wait for isect_tiles on them); the
-        number travels with the returned radii, see _isect()."""
+        tile intersections of the rows it keeps, and their lists are made here, ahead of the
+        packed outputs (the GPU is waiting for that work, not for the outputs); they travel with
+        the returned radii, see _isect().
+
+        beside: an object with `side` (a torch stream or None), `requests` and `results` (dicts).
+        With isect_grid and a side stream, the kernels that write the packed outputs go to that
+        stream, ordered behind the binning by the intersection call itself, and run beside the
+        segment sort; the caller joins the stream before anything reads the outputs on its own
+        stream (_isect() with the lists of these rows does not read them; without them it waits
+        for the stream left on the radii).  requests["colors"] = (degrees_to_use, coeffs,
+        with_depth) and requests["opacities"] = opacities [N] ask for what view_colors_fwd() and
+        the gather opacities[gaussian_ids] (* compensations) would give for the returned rows;
+        they are made on the same stream and left in results under the same keys."""
         lib = load_library()
         means = _in(means, "means"); covars = _in(covars, "covars"); quats = _in(quats, "quats")
         scales = _in(scales, "scales"); velocities = _in(velocities, "velocities")
@@ -166,26 +198,54 @@ class _Ops:
         rs = _in(rolling_shutter_time, "rolling_shutter_time")
         N, C, dev = means.shape[0], viewmats.shape[0], means.device
         f = dict(dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             ws = _workspace(lib.splatad_projection_packed_workspace_bytes(_u32(C), _u32(N)), dev)
             nnz_host, n_isects_host = _i64(0), _i64(0)
             head = (_u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
                     _p(viewmats), _p(Ks), _u32(image_width), _u32(image_height), _p(lv), _p(av), _p(rs),
                     _f32(eps2d), _f32(near_plane), _f32(far_plane), _f32(radius_clip),
                     _i32(bool(calc_compensations)))
-            isect_ws = None
+            main = _stream(dev)
             if isect_grid is None:
-                _check(lib.splatad_projection_packed_count(*head, _p(ws), ctypes.byref(nnz_host), _stream(dev)))
+                _check(lib.splatad_projection_packed_count(*head, _p(ws), ctypes.byref(nnz_host), main))
             else:
                 # the counting call also starts the tile intersection, on the dense rows in its
-                # workspace, while the host waits for the counts; _isect() completes it
+                # workspace, while the host waits for the counts
                 n_tiles = int(isect_grid[1]) * int(isect_grid[2])
                 assert n_tiles.bit_length() + int(C).bit_length() <= 32
                 isect_ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(C * N), _u32(C), _u32(n_tiles)), dev)
                 _check(lib.splatad_projection_packed_count_tiles(
                     *head, *(_u32(v) for v in isect_grid), _p(ws), _p(isect_ws), ctypes.byref(nnz_host),
-                    ctypes.byref(n_isects_host), _stream(dev)))
+                    ctypes.byref(n_isects_host), main))
             nnz = int(nnz_host.value)
+            isect_result = side = None
+            work = main  # the stream of the kernels that write the outputs
+            if isect_grid is not None:
+                # first what the GPU is waiting for: the rest of the tile intersection
+                side = getattr(beside, "side", None)
+                if side is not None:
+                    work = ctypes.c_void_p(side.cuda_stream)
+                n_isects = int(n_isects_host.value)
+                tile_w, tile_h = int(isect_grid[1]), int(isect_grid[2])
+                tiles_per_gauss = torch.empty((nnz,), dtype=torch.int32, device=dev)
+                isect_ids = torch.empty((n_isects,), dtype=torch.int64, device=dev)
+                flatten_ids = torch.empty((n_isects,), dtype=torch.int32, device=dev)
+                offsets = lists = None
+                if n_isects:
+                    offsets = torch.empty((C, tile_h, tile_w), dtype=torch.int32, device=dev)
+                    lists = _workspace(lib.splatad_isect_lists_bytes(_u64(C * N), _i64(n_isects)), dev)
+                else:
+                    tiles_per_gauss.zero_()
+                if n_isects or side is not None:  # (without lists the call only orders the side stream)
+                    _check(lib.splatad_isect_tiles_fill_packed(
+                        _u32(C), _u32(N), *(_u32(v) for v in isect_grid), _i64(n_isects), _p(ws),
+                        _p(isect_ws), _p(lists), _p(tiles_per_gauss), _p(isect_ids), _p(flatten_ids),
+                        _p(offsets), work if side is not None else None, main))
+                if offsets is not None:
+                    # isect_offset_encode() on the same, unmodified tensor is free
+                    isect_ids._splatad_tile_offsets = (offsets, isect_ids._version)
+                isect_result = (tiles_per_gauss, isect_ids, flatten_ids)
+            requests = getattr(beside, "requests", None) or {}
             indptr = torch.empty((C + 1,), dtype=torch.int32, device=dev)
             camera_ids = torch.empty((nnz,), dtype=torch.int64, device=dev)
             gaussian_ids = torch.empty((nnz,), dtype=torch.int64, device=dev)
@@ -193,15 +253,38 @@ class _Ops:
             means2d = torch.empty((nnz, 2), **f); depths = torch.empty((nnz,), **f)
             conics = torch.empty((nnz, 3), **f); pix_vels = torch.empty((nnz, 2), **f)
             comps = torch.empty((nnz,), **f) if calc_compensations else None
+            opacities = requests.get("opacities")
+            row_opacities = None
+            if opacities is not None:
+                opacities = _in(opacities, "opacities")
+                assert opacities.shape == (N,), opacities.shape
+                row_opacities = torch.empty((nnz,), **f)
             _check(lib.splatad_projection_packed_fill(
                 _u32(C), _u32(N), _i64(nnz), _p(ws), _p(indptr), _p(camera_ids), _p(gaussian_ids),
                 _p(radii), _p(means2d), _p(depths), _p(conics), _p(comps), _p(pix_vels),
-                _stream(dev)))
+                _p(opacities), _p(row_opacities), work))
+            results = {}
+            if row_opacities is not None:
+                results["opacities"] = row_opacities
+            if "colors" in requests:
+                degree, coeffs, with_depth = requests["colors"]
+                coeffs = _in(coeffs, "coeffs")
+                colors = torch.empty((nnz, 4 if with_depth else 3), **f)
+                if nnz:
+                    _check(lib.splatad_view_colors_fwd_packed(
+                        _u32(C), _u32(N), _u32(coeffs.shape[-2]), _u32(degree), _p(means), _p(viewmats),
+                        _p(ws), _p(coeffs), _i32(coeffs.dim() == 4), _i32(bool(with_depth)), _p(colors), work))
+                results["colors"] = colors
+            if beside is not None:
+                beside.results = results
+            if side is not None:
+                ws.record_stream(side)  # read there after the last use here
+                radii._splatad_fill_stream = side
         if isect_grid is not None:
             # valid for these very tensors as long as nobody writes to them
-            radii._splatad_isect_count = (tuple(int(v) for v in isect_grid), int(n_isects_host.value),
+            radii._splatad_isect_count = (tuple(int(v) for v in isect_grid), isect_result,
                                           radii._version, weakref.ref(means2d), means2d._version,
-                                          weakref.ref(depths), depths._version, C, N, ws, isect_ws)
+                                          weakref.ref(depths), depths._version, C)
         return indptr, camera_ids, gaussian_ids, radii, means2d, depths, conics, comps, pix_vels
 
     def fully_fused_lidar_projection_fwd(self, means, covars, quats, scales, velocities, viewmats,
@@ -222,7 +305,7 @@ class _Ops:
         conics = torch.empty((C, N, 3), **f); pix_vels = torch.empty((C, N, 3), **f)
         dcomps = torch.empty((C, N, 2), **f)
         comps = torch.empty((C, N), **f) if calc_compensations else None
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_lidar_projection_fwd(
                 _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
                 _p(viewmats), _f32(min_elevation), _f32(max_elevation), _f32(min_azimuth),
@@ -286,7 +369,7 @@ class _Ops:
                   velocities.shape if (velocities_requires_grad and velocities is not None) else None)
         v_means, v_covars, v_quats, v_scales, v_viewmats, v_velocities = (
             _zeros_many(dev, *shapes) if packed else _gathered_outputs(dev, *shapes))
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_projection_bwd(
                 _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
                 _p(viewmats), _p(Ks), _u32(image_width), _u32(image_height), _p(lv), _p(av), _p(rs),
@@ -323,7 +406,7 @@ class _Ops:
                 means, covars, quats if covars is None else None, scales if covars is None else None,
                 viewmats if viewmats_requires_grad else None,
                 velocities if (velocities_requires_grad and velocities is not None) else None)))
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_lidar_projection_bwd(
                 _u32(C), _u32(N), _p(means), _p(covars), _p(quats), _p(scales), _p(velocities),
                 _p(viewmats), _p(lv), _p(av), _p(rs), _f32(eps2d), _p(radii), _p(conics),
@@ -345,7 +428,7 @@ class _Ops:
             raise RuntimeError("dirs must have last dimension 3")
         K, n, dev = coeffs.shape[-2], dirs.numel() // 3, dirs.device
         colors = torch.empty_like(dirs)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_sh_fwd(_u32(n), _u32(K), _u32(degrees_to_use), _p(dirs), _p(coeffs),
                                       _p(masks), _p(colors), _stream(dev)))
         return colors
@@ -359,7 +442,7 @@ class _Ops:
         full = (degrees_to_use + 1) ** 2 == K
         v_coeffs = torch.empty_like(coeffs) if full else torch.zeros_like(coeffs)
         v_dirs = torch.zeros_like(dirs) if compute_v_dirs else None
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_sh_bwd(_u32(n), _u32(K), _u32(degrees_to_use), _p(dirs), _p(coeffs),
                                       _p(masks), _p(v_colors), _p(v_coeffs), _p(v_dirs),
                                       _stream(dev)))
@@ -380,7 +463,7 @@ class _Ops:
         lead = tuple(radii.shape[:-1])
         n = int(math.prod(lead))
         colors = torch.empty(lead + (4 if depths is not None else 3,), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_view_colors_fwd(
                 _u32(n), _u32(C), _u32(N), _u32(coeffs.shape[-2]), _u32(degrees_to_use), _p(means),
                 _p(viewmats), _p(camera_ids), _p(gaussian_ids), _p(radii), _p(coeffs),
@@ -404,7 +487,7 @@ class _Ops:
         full = (degrees_to_use + 1) ** 2 == K
         v_coeffs = (torch.empty if full else torch.zeros)(lead + (K, 3), **f)
         v_dirs = torch.empty(lead + (3,), **f) if compute_v_dirs else None
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_view_colors_bwd(
                 _u32(n), _u32(C), _u32(N), _u32(K), _u32(degrees_to_use), _p(means), _p(viewmats),
                 _p(camera_ids), _p(gaussian_ids), _p(radii), _p(coeffs), _i32(coeffs.dim() == 4),
@@ -415,6 +498,20 @@ class _Ops:
     # ------------------------------------------------------------------ intersection
     def _isect(self, lidar, means2d, radii, depths, camera_ids, gaussian_ids, C, grid_args,
                tile_w, tile_h, sort):
+        # A packed projection that was told the tile grid has made the lists of these rows from its
+        # dense copy of them (good for one call, and only for the very tensors it returned,
+        # unwritten since).
+        known = getattr(radii, "_splatad_isect_count", None) if not lidar and sort else None
+        if known is not None:
+            del radii._splatad_isect_count
+            if (known[0] == (int(grid_args[0].value), tile_w, tile_h) and known[2] == radii._version
+                    and known[3]() is means2d and known[4] == means2d._version
+                    and known[5]() is depths and known[6] == depths._version and known[7] == C):
+                return known[1]
+        filled = getattr(radii, "_splatad_fill_stream", None)
+        if filled is not None:
+            # rows of a packed projection whose outputs were written on another stream
+            torch.cuda.current_stream(radii.device).wait_stream(filled)
         lib = load_library()
         means2d = _in(means2d, "means2d"); depths = _in(depths, "depths")
         radii = _in(radii, "radii", torch.float32 if lidar else torch.int32)
@@ -435,48 +532,27 @@ class _Ops:
         tiles_per_gauss = torch.empty(depths.shape, dtype=torch.int32, device=dev)
         count = lib.splatad_isect_lidar_tiles_count if lidar else lib.splatad_isect_tiles_count
         fill = lib.splatad_isect_lidar_tiles_fill if lidar else lib.splatad_isect_tiles_fill
-        # A packed projection that was told the tile grid has counted the intersections of these
-        # rows and started the binning on its dense copy of them (good for one call, and only for
-        # the very tensors it returned, unwritten since).
-        known = getattr(radii, "_splatad_isect_count", None) if packed and not lidar and sort else None
-        if known is not None:
-            del radii._splatad_isect_count  # the workspaces are freed with it
-            if not (known[0] == (int(grid_args[0].value), tile_w, tile_h) and known[2] == radii._version
-                    and known[3]() is means2d and known[4] == means2d._version
-                    and known[5]() is depths and known[6] == depths._version and known[7] == C):
-                known = None
-        with torch.cuda.device(dev):
+        with _on(dev):
             # the binning knows every tile's first intersection: keep that table with the
             # ids so that isect_offset_encode() on the same, unmodified tensor is free
             offsets = (torch.empty((C, tile_h, tile_w), dtype=torch.int32, device=dev)
                        if sort else None)
-            if known is not None:
-                n_isects, (kC, kN, packed_ws, ws) = known[1], known[7:11]  # no wait here
-            else:
-                # one workspace for both calls: the counting call leaves the start of the binning in it
-                ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(total), _u32(C), _u32(n_tiles)), dev)
-                head = (_u64(total), _u32(N), _p(camera_ids), _p(means2d), _p(radii), _p(depths))
-                tail = (_u32(C), *grid_args, _u32(tile_w), _u32(tile_h), _i32(bool(sort)))
-                n_host = _i64(0)
-                _check(count(*head, *tail, _p(tiles_per_gauss), _p(ws), ctypes.byref(n_host),
-                             _stream(dev)))
-                n_isects = int(n_host.value)
+            # one workspace for both calls: the counting call leaves the start of the binning in it
+            ws = _workspace(lib.splatad_isect_workspace_bytes(_u64(total), _u32(C), _u32(n_tiles)), dev)
+            head = (_u64(total), _u32(N), _p(camera_ids), _p(means2d), _p(radii), _p(depths))
+            tail = (_u32(C), *grid_args, _u32(tile_w), _u32(tile_h), _i32(bool(sort)))
+            n_host = _i64(0)
+            _check(count(*head, *tail, _p(tiles_per_gauss), _p(ws), ctypes.byref(n_host),
+                         _stream(dev)))
+            n_isects = int(n_host.value)
             isect_ids = torch.empty((n_isects,), dtype=torch.int64, device=dev)
             flatten_ids = torch.empty((n_isects,), dtype=torch.int32, device=dev)
-            if n_isects and known is not None:
-                lists = _workspace(lib.splatad_isect_lists_bytes(_u64(kC * kN), _i64(n_isects)), dev)
-                _check(lib.splatad_isect_tiles_fill_packed(
-                    _u32(kC), _u32(kN), *grid_args, _u32(tile_w), _u32(tile_h), _i64(n_isects),
-                    _p(packed_ws), _p(ws), _p(lists), _p(tiles_per_gauss), _p(isect_ids),
-                    _p(flatten_ids), _p(offsets), _stream(dev)))
-            elif n_isects:
+            if n_isects:
                 lists = _workspace(lib.splatad_isect_lists_bytes(_u64(total), _i64(n_isects)), dev)
                 _check(fill(*head, *tail, _i64(n_isects), _p(tiles_per_gauss), _p(ws),
                             _p(lists), _p(isect_ids), _p(flatten_ids), _p(offsets), _stream(dev)))
             else:
                 offsets = None
-                if known is not None:
-                    tiles_per_gauss.zero_()
             if offsets is not None:
                 isect_ids._splatad_tile_offsets = (offsets, isect_ids._version)
         return tiles_per_gauss, isect_ids, flatten_ids
@@ -506,7 +582,7 @@ class _Ops:
         isect_ids = _in(isect_ids, "isect_ids", torch.int64)
         dev = isect_ids.device
         offsets = torch.empty((C, tile_height, tile_width), dtype=torch.int32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_isect_offset_encode(_i64(isect_ids.shape[0]), _p(isect_ids), _u32(C),
                                                    _u32(tile_width * tile_height), _p(offsets),
                                                    _stream(dev)))
@@ -534,7 +610,7 @@ class _Ops:
         tile_ids = torch.empty((total,), dtype=torch.int64, device=dev)
         flatten_ids = torch.empty((total,), dtype=torch.int32, device=dev)
         if total:
-            with torch.cuda.device(dev):
+            with _on(dev):
                 ws = _workspace(lib.splatad_map_points_to_lidar_tiles_workspace_bytes(
                     _u64(total), _u32(C), _u32(n_az * n_el)), dev) if sort else None
                 _check(lib.splatad_map_points_to_lidar_tiles(
@@ -548,7 +624,7 @@ class _Ops:
         point_ids = _in(point_ids, "point_ids", torch.int64)
         dev = point_ids.device
         offsets = torch.empty((C, tile_height, tile_width), dtype=torch.int32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_points_mapping_offset_encode(
                 _i64(point_ids.shape[0]), _p(point_ids), _u32(C), _u32(tile_width * tile_height),
                 _p(offsets), _stream(dev)))
@@ -565,7 +641,7 @@ class _Ops:
         dev = points.device
         C, gh, gw = tile_offsets.shape
         image = torch.empty((C, image_height, image_width, 5), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_populate_image_from_points(
                 _u32(C), _i64(flatten_ids.shape[0]), _p(points), _u32(image_width),
                 _u32(image_height), _u32(tile_width), _u32(tile_height), _u32(gw), _u32(gh),
@@ -580,7 +656,7 @@ class _Ops:
         shape = (N, 6) if triu else (N, 3, 3)
         covars = torch.empty(shape, dtype=torch.float32, device=dev) if compute_covar else None
         precis = torch.empty(shape, dtype=torch.float32, device=dev) if compute_preci else None
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_quat_scale_to_covar_preci_fwd(
                 _u32(N), _p(quats), _p(scales), _i32(bool(triu)), _p(covars), _p(precis), _stream(dev)))
         return covars, precis
@@ -591,7 +667,7 @@ class _Ops:
         v_covars = _in(v_covars, "v_covars"); v_precis = _in(v_precis, "v_precis")
         dev = quats.device
         v_quats = torch.empty_like(quats); v_scales = torch.empty_like(scales)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_quat_scale_to_covar_preci_bwd(
                 _u32(quats.shape[0]), _p(quats), _p(scales), _p(v_covars), _p(v_precis),
                 _i32(bool(triu)), _p(v_quats), _p(v_scales), _stream(dev)))
@@ -603,7 +679,7 @@ class _Ops:
         C, N, dev = viewmats.shape[0], means.shape[0], means.device
         means_c = torch.empty((C, N, 3), dtype=torch.float32, device=dev)
         covars_c = torch.empty((C, N, 3, 3), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_world_to_cam_fwd(_u32(C), _u32(N), _p(means), _p(covars), _p(viewmats),
                                                 _p(means_c), _p(covars_c), _stream(dev)))
         return means_c, covars_c
@@ -617,7 +693,7 @@ class _Ops:
         v_means = torch.zeros_like(means) if means_grad else None
         v_covars = torch.zeros_like(covars) if covars_grad else None
         v_viewmats = torch.zeros_like(viewmats) if viewmats_grad else None
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_world_to_cam_bwd(
                 _u32(C), _u32(N), _p(means), _p(covars), _p(viewmats), _p(v_means_c), _p(v_covars_c),
                 _p(v_means), _p(v_covars), _p(v_viewmats), _stream(dev)))
@@ -629,7 +705,7 @@ class _Ops:
         C, N, dev = means.shape[0], means.shape[1], means.device
         means2d = torch.empty((C, N, 2), dtype=torch.float32, device=dev)
         covars2d = torch.empty((C, N, 2, 2), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_persp_proj_fwd(_u32(C), _u32(N), _p(means), _p(covars), _p(Ks), _u32(width),
                                               _u32(height), _p(means2d), _p(covars2d), _stream(dev)))
         return means2d, covars2d
@@ -640,7 +716,7 @@ class _Ops:
         v_means2d = _in(v_means2d, "v_means2d"); v_covars2d = _in(v_covars2d, "v_covars2d")
         C, N, dev = means.shape[0], means.shape[1], means.device
         v_means = torch.empty_like(means); v_covars = torch.empty_like(covars)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_persp_proj_bwd(
                 _u32(C), _u32(N), _p(means), _p(covars), _p(Ks), _u32(width), _u32(height),
                 _p(v_means2d), _p(v_covars2d), _p(v_means), _p(v_covars), _stream(dev)))
@@ -652,7 +728,7 @@ class _Ops:
         velocities = _in(velocities, "velocities"); Ks = _in(Ks, "Ks")
         C, N, dev = p_view.shape[0], p_view.shape[1], p_view.device
         vel = torch.empty((C, N, 2), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_compute_pix_velocity_fwd(
                 _u32(C), _u32(N), _p(p_view), _p(lin_vel), _p(ang_vel), _p(velocities), _p(Ks),
                 _u32(width), _u32(height), _p(vel), _stream(dev)))
@@ -664,7 +740,7 @@ class _Ops:
         velocities = _in(velocities, "velocities"); Ks = _in(Ks, "Ks"); v_vel = _in(v_vel, "v_vel")
         C, N, dev = p_view.shape[0], p_view.shape[1], p_view.device
         v_p_view = torch.empty_like(p_view); v_velocities = torch.empty_like(velocities)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_compute_pix_velocity_bwd(
                 _u32(C), _u32(N), _p(p_view), _p(lin_vel), _p(ang_vel), _p(velocities), _p(Ks),
                 _u32(width), _u32(height), _p(v_vel), _p(v_p_view), _p(v_velocities), _stream(dev)))
@@ -677,7 +753,7 @@ class _Ops:
         means2d = torch.empty((C, N, 2), dtype=torch.float32, device=dev)
         covars2d = torch.empty((C, N, 2, 2), dtype=torch.float32, device=dev)
         depth_comps = torch.empty((C, N, 2), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_lidar_proj_fwd(_u32(C), _u32(N), _p(means), _p(covars), _f32(eps2d),
                                               _p(means2d), _p(covars2d), _p(depth_comps), _stream(dev)))
         return means2d, covars2d, depth_comps
@@ -689,7 +765,7 @@ class _Ops:
         v_dc = _in(v_depth_compensations, "v_depth_compensations")
         C, N, dev = means.shape[0], means.shape[1], means.device
         v_means = torch.empty_like(means); v_covars = torch.empty_like(covars)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_lidar_proj_bwd(
                 _u32(C), _u32(N), _p(means), _p(covars), _f32(eps2d), _p(v_means2d), _p(v_covars2d),
                 _p(v_dc), _p(v_means), _p(v_covars), _stream(dev)))
@@ -701,7 +777,7 @@ class _Ops:
         velocities = _in(velocities, "velocities")
         C, N, dev = p_view.shape[0], p_view.shape[1], p_view.device
         vel = torch.empty((C, N, 3), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_compute_lidar_velocity_fwd(
                 _u32(C), _u32(N), _p(p_view), _p(lin_vel), _p(ang_vel), _p(velocities), _p(vel),
                 _stream(dev)))
@@ -713,7 +789,7 @@ class _Ops:
         velocities = _in(velocities, "velocities"); v_vel = _in(v_vel, "v_vel")
         C, N, dev = p_view.shape[0], p_view.shape[1], p_view.device
         v_p_view = torch.empty_like(p_view); v_velocities = torch.empty_like(velocities)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_compute_lidar_velocity_bwd(
                 _u32(C), _u32(N), _p(p_view), _p(lin_vel), _p(ang_vel), _p(velocities), _p(v_vel),
                 _p(v_p_view), _p(v_velocities), _stream(dev)))
@@ -727,7 +803,7 @@ class _Ops:
         dev = opacities.device
         new_opacities = torch.empty_like(opacities)
         new_scales = torch.empty_like(scales)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_compute_relocation(
                 _u32(opacities.shape[0]), _p(opacities), _p(scales), _p(ratios), _p(binoms),
                 _i32(n_max), _p(new_opacities), _p(new_scales), _stream(dev)))
@@ -752,7 +828,7 @@ class _Ops:
         renders = torch.empty((C, image_height, image_width, D), **f)
         alphas = torch.empty((C, image_height, image_width, 1), **f)
         last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_rasterize_to_pixels_fwd(
                 _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics), _p(colors),
                 _p(opacities), _p(pix_vels), _p(rs), _p(backgrounds), _u32(image_width),
@@ -775,7 +851,7 @@ class _Ops:
         C, th, tw = tile_offsets.shape
         dev = means2d.device
         stats = torch.zeros((8,), dtype=torch.int64, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_rasterize_to_pixels_lane_stats(
                 _u32(C), _i64(flatten_ids.shape[0]), _p(means2d), _p(conics), _p(opacities), _p(pix_vels),
                 _p(rs), _u32(image_width), _u32(image_height), _u32(tile_size), _u32(tw), _u32(th),
@@ -803,7 +879,7 @@ class _Ops:
             means2d, conics, colors, opacities, pix_vels, means2d if absgrad else None)
         if flatten_ids.shape[0]:
             total = means2d.numel() // 2
-            with torch.cuda.device(dev):
+            with _on(dev):
                 ws = _bwd_workspace(lib, total, D, False, dev)
                 _check(lib.splatad_rasterize_to_pixels_bwd(
                     _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics),
@@ -840,7 +916,7 @@ class _Ops:
         asum = (torch.empty((C, image_height, image_width, 1), **f)
                 if compute_alpha_sum_until_points else None)
         last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
-        with torch.cuda.device(dev):
+        with _on(dev):
             _check(lib.splatad_rasterize_to_points_fwd(
                 _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics), _p(colors),
                 _p(range_channel), _p(opacities), _p(pix_vels), _p(dc), _p(backgrounds),
@@ -881,7 +957,7 @@ class _Ops:
                                      means2d if absgrad else None, range_channel)
         if flatten_ids.shape[0]:
             total = means2d.numel() // 2
-            with torch.cuda.device(dev):
+            with _on(dev):
                 ws = _bwd_workspace(lib, total, D, True, dev)
                 _check(lib.splatad_rasterize_to_points_bwd(
                     _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics),
@@ -927,7 +1003,7 @@ class _Ops:
                 _u32(N), _i64(n_isects), _p(transmittances), _p(means2d), _p(conics), _p(opacities),
                 _p(pix_vels), _p(sensor), _u32(image_width), _u32(image_height), *tiles,
                 _p(tile_offsets), _p(flatten_ids))
-        with torch.cuda.device(dev):
+        with _on(dev):
             nbytes = lib.splatad_rasterize_to_indices_workspace_bytes(
                 _u32(C), _u32(image_width), _u32(image_height))
             ws = _workspace(nbytes, dev)

@@ -29,6 +29,28 @@ def _make_lazy_hip_func(name: str) -> Callable:
     return call_hip
 
 
+class _NoGradContext:
+    """Takes the place of the autograd context when no gradient can be asked for."""
+
+    needs_input_grad = ()
+
+    def save_for_backward(self, *tensors):
+        pass
+
+    def mark_non_differentiable(self, *tensors):
+        pass
+
+
+def _apply(function, *args):
+    """`function.apply(*args)`, or just its forward when gradients are switched off or no
+    argument takes one (the bookkeeping of autograd costs as much host time as a kernel launch)."""
+    if torch.is_grad_enabled():
+        for a in args:
+            if isinstance(a, Tensor) and a.requires_grad:
+                return function.apply(*args)
+    return function.forward(_NoGradContext(), *args)
+
+
 def _c(t: Optional[Tensor]) -> Optional[Tensor]:
     return None if t is None else t.contiguous()
 
@@ -64,7 +86,7 @@ def spherical_harmonics(
     if masks is not None:
         assert masks.shape == dirs.shape[:-1], masks.shape
         masks = masks.contiguous()
-    return _SphericalHarmonics.apply(degrees_to_use, dirs.contiguous(), coeffs.contiguous(), masks)
+    return _apply(_SphericalHarmonics, degrees_to_use, dirs.contiguous(), coeffs.contiguous(), masks)
 
 
 def view_dependent_colors(
@@ -77,6 +99,7 @@ def view_dependent_colors(
     camera_ids: Optional[Tensor] = None,  # [nnz]
     gaussian_ids: Optional[Tensor] = None,  # [nnz]
     launch_context=None,
+    precomputed: Optional[Tensor] = None,
 ) -> Tensor:
     """Activated view-dependent colours of every (sensor, Gaussian) pair in one kernel:
     max(SH(mean - sensor position) + 1/2, 0) for pairs with a positive projected radius
@@ -87,7 +110,8 @@ def view_dependent_colors(
     `viewmats` are treated as constants (rows [A | t], last row (0, 0, 0, 1)).
     `launch_context`, if given, is a context manager entered around the forward kernel launch
     only (e.g. a helper stream); the autograd node, and with it the backward pass, stays on the
-    caller's stream.
+    caller's stream.  `precomputed`: the result of this very call, made elsewhere (by the packed
+    projection, see `fully_fused_projection`); it is taken instead of running the kernel.
 
     Returns [C, N, 3 or 4], or [nnz, 3 or 4] for packed input.
     """
@@ -107,9 +131,9 @@ def view_dependent_colors(
     if depths is not None:
         assert depths.shape == radii.shape[:-1], depths.shape
         depths = depths.contiguous()
-    return _ViewColors.apply(degrees_to_use, means.contiguous(), viewmats.contiguous(),
-                             coeffs.contiguous(), radii.contiguous(), depths, camera_ids, gaussian_ids,
-                             launch_context)
+    return _apply(_ViewColors, degrees_to_use, means.contiguous(), viewmats.contiguous(),
+                  coeffs.contiguous(), radii.contiguous(), depths, camera_ids, gaussian_ids,
+                  launch_context, precomputed)
 
 
 def fully_fused_projection(
@@ -133,6 +157,7 @@ def fully_fused_projection(
     sparse_grad: bool = False,
     calc_compensations: bool = False,
     isect_grid: Optional[Tuple[int, int, int]] = None,
+    beside=None,
 ):
     """Projects Gaussians onto C pinhole image planes (EWA splatting) with rolling-shutter
     pixel velocities.
@@ -141,6 +166,13 @@ def fully_fused_projection(
     that `isect_tiles` on that grid follows: the projection, which waits for its row count
     anyway, then counts the tile intersections of the rows it keeps as well, and `isect_tiles`
     on the returned (unmodified) `means2d` and `radii` starts without a wait of its own.
+    `beside` (packed with `isect_grid` only, not in the reference): an object with `side` (a
+    torch stream or None), `requests` and `results` (dicts).  The kernels that write the packed
+    outputs then run on that stream beside the sort of the tile intersection, and the caller
+    joins it before anything but `isect_tiles` reads the outputs.  requests["colors"] =
+    (degrees_to_use, coeffs, with_depth) and requests["opacities"] = opacities [N] ask for the
+    result of `view_dependent_colors` and of opacities[gaussian_ids] (* compensations) on the
+    returned rows; they are made on the same stream, without a gradient, and left in `results`.
 
     Returns, unpacked: (radii int32[C,N,2], means2d[C,N,2], depths[C,N], conics[C,N,3],
     compensations[C,N] | None, pix_vels[C,N,2]); a zero radius marks a culled Gaussian.
@@ -163,8 +195,9 @@ def fully_fused_projection(
         far_plane, radius_clip,
     )
     if packed:
-        return _FullyFusedProjectionPacked.apply(*args, sparse_grad, calc_compensations, isect_grid)
-    return _FullyFusedProjection.apply(*args, calc_compensations)
+        return _apply(_FullyFusedProjectionPacked, *args, sparse_grad, calc_compensations, isect_grid,
+                      beside)
+    return _apply(_FullyFusedProjection, *args, calc_compensations)
 
 
 def fully_fused_lidar_projection(
@@ -204,7 +237,7 @@ def fully_fused_lidar_projection(
         assert packed, "sparse_grad is only supported when packed is True"
     if packed:
         raise NotImplementedError("FullyFusedLidarProjectionPacked is not implemented yet")
-    return _FullyFusedLidarProjection.apply(
+    return _apply(_FullyFusedLidarProjection,
         means.contiguous(), _c(covars), _c(quats), _c(scales), _c(velocities),
         viewmats.contiguous(), min_elevation, max_elevation, min_azimuth, max_azimuth,
         linear_velocity.contiguous(), angular_velocity.contiguous(),
@@ -394,7 +427,7 @@ def rasterize_to_pixels(
     assert tile_height * tile_size >= image_height, f"Assert Failed: {tile_height} * {tile_size} >= {image_height}"
     assert tile_width * tile_size >= image_width, f"Assert Failed: {tile_width} * {tile_size} >= {image_width}"
 
-    return _RasterizeToPixels.apply(
+    return _apply(_RasterizeToPixels,
         means2d.contiguous(), conics.contiguous(), colors.contiguous(), opacities.contiguous(),
         pix_vels.contiguous(), rolling_shutter_time.contiguous(), backgrounds, image_width,
         image_height, tile_size, isect_offsets.contiguous(), flatten_ids.contiguous(), absgrad,
@@ -466,7 +499,7 @@ def rasterize_to_points(
     assert tile_grid_width * tile_width >= image_width, f"Assert Failed: {tile_grid_width} * {tile_width} >= {image_width}"
     assert raster_pts.shape == (C, image_height, image_width, 4), "raster_pts does not have the correct shape"
 
-    return _RasterizeToPoints.apply(
+    return _apply(_RasterizeToPoints,
         means2d.contiguous(), conics.contiguous(), lidar_features.contiguous(),
         opacities.contiguous(), pix_vels.contiguous(), depth_compensations.contiguous(),
         backgrounds, raster_pts.contiguous(), image_width, image_height, tile_width, tile_height,
@@ -655,12 +688,13 @@ class _FullyFusedProjectionPacked(torch.autograd.Function):
     @staticmethod
     def forward(ctx, means, covars, quats, scales, velocities, viewmats, Ks, width, height,
                 linear_velocity, angular_velocity, rolling_shutter_time, eps2d, near_plane,
-                far_plane, radius_clip, sparse_grad, calc_compensations, isect_grid=None):
+                far_plane, radius_clip, sparse_grad, calc_compensations, isect_grid=None,
+                beside=None):
         (indptr, camera_ids, gaussian_ids, radii, means2d, depths, conics, compensations,
          pix_vels) = _make_lazy_hip_func("fully_fused_projection_packed_fwd")(
             means, covars, quats, scales, velocities, viewmats, Ks, width, height,
             linear_velocity, angular_velocity, rolling_shutter_time, eps2d, near_plane, far_plane,
-            radius_clip, calc_compensations, isect_grid)
+            radius_clip, calc_compensations, isect_grid, beside)
         if not calc_compensations:
             compensations = None
         ctx.save_for_backward(camera_ids, gaussian_ids, means, covars, quats, scales, velocities,
@@ -703,7 +737,7 @@ class _FullyFusedProjectionPacked(torch.autograd.Function):
                 v_scales = coo(v_scales, scales)
         grads = _gate((v_means, v_covars, v_quats, v_scales, v_velocities, v_viewmats),
                       ctx.needs_input_grad[:6])
-        return grads + (None,) * 13
+        return grads + (None,) * 14
 
 
 class _RasterizeToPixels(torch.autograd.Function):
@@ -804,7 +838,7 @@ def quat_scale_to_covar_preci(
     for is None."""
     assert quats.dim() == 2 and quats.size(1) == 4, quats.size()
     assert scales.dim() == 2 and scales.size(1) == 3, scales.size()
-    covars, precis = _QuatScaleToCovarPreci.apply(
+    covars, precis = _apply(_QuatScaleToCovarPreci,
         quats.contiguous(), scales.contiguous(), compute_covar, compute_preci, triu)
     return covars if compute_covar else None, precis if compute_preci else None
 
@@ -816,7 +850,7 @@ def persp_proj(means: Tensor, covars: Tensor, Ks: Tensor, width: int, height: in
     assert means.shape == (C, N, 3), means.size()
     assert covars.shape == (C, N, 3, 3), covars.size()
     assert Ks.shape == (C, 3, 3), Ks.size()
-    return _PerspProj.apply(means.contiguous(), covars.contiguous(), Ks.contiguous(), width, height)
+    return _apply(_PerspProj, means.contiguous(), covars.contiguous(), Ks.contiguous(), width, height)
 
 
 def compute_pix_velocity(p_view: Tensor, lin_vel: Tensor, ang_vel: Tensor, velocities: Tensor,
@@ -829,7 +863,7 @@ def compute_pix_velocity(p_view: Tensor, lin_vel: Tensor, ang_vel: Tensor, veloc
     assert ang_vel.shape == (C, 3), ang_vel.size()
     assert velocities.shape == (C, N, 3), velocities.size()
     assert Ks.shape == (C, 3, 3), Ks.size()
-    return _ComputePixVelocity.apply(p_view.contiguous(), lin_vel.contiguous(), ang_vel.contiguous(),
+    return _apply(_ComputePixVelocity, p_view.contiguous(), lin_vel.contiguous(), ang_vel.contiguous(),
                                      velocities.contiguous(), Ks.contiguous(), width, height)
 
 
@@ -841,7 +875,7 @@ def world_to_cam(means: Tensor, covars: Tensor, viewmats: Tensor) -> Tuple[Tenso
     assert means.size() == (N, 3), means.size()
     assert covars.size() == (N, 3, 3), covars.size()
     assert viewmats.size() == (C, 4, 4), viewmats.size()
-    return _WorldToCam.apply(means.contiguous(), covars.contiguous(), viewmats.contiguous())
+    return _apply(_WorldToCam, means.contiguous(), covars.contiguous(), viewmats.contiguous())
 
 
 def lidar_proj(means: Tensor, covars: Tensor, eps2d: float) -> Tuple[Tensor, Tensor, Tensor]:
@@ -850,7 +884,7 @@ def lidar_proj(means: Tensor, covars: Tensor, eps2d: float) -> Tuple[Tensor, Ten
     C, N, _ = means.shape
     assert means.shape == (C, N, 3), means.size()
     assert covars.shape == (C, N, 3, 3), covars.size()
-    return _LidarProj.apply(means.contiguous(), covars.contiguous(), eps2d)
+    return _apply(_LidarProj, means.contiguous(), covars.contiguous(), eps2d)
 
 
 def compute_lidar_velocity(p_view: Tensor, lin_vel: Tensor, ang_vel: Tensor, velocities: Tensor) -> Tensor:
@@ -861,7 +895,7 @@ def compute_lidar_velocity(p_view: Tensor, lin_vel: Tensor, ang_vel: Tensor, vel
     assert lin_vel.shape == (C, 3), lin_vel.size()
     assert ang_vel.shape == (C, 3), ang_vel.size()
     assert velocities.shape == (C, N, 3), velocities.size()
-    return _ComputeLidarVelocity.apply(p_view.contiguous(), lin_vel.contiguous(), ang_vel.contiguous(),
+    return _apply(_ComputeLidarVelocity, p_view.contiguous(), lin_vel.contiguous(), ang_vel.contiguous(),
                                        velocities.contiguous())
 
 
@@ -971,10 +1005,14 @@ class _ComputeLidarVelocity(torch.autograd.Function):
 class _ViewColors(torch.autograd.Function):
     @staticmethod
     def forward(ctx, sh_degree, means, viewmats, coeffs, radii, depths, camera_ids, gaussian_ids,
-                launch_context):
-        with (launch_context if launch_context is not None else contextlib.nullcontext()):
-            colors = _make_lazy_hip_func("view_colors_fwd")(
-                sh_degree, means, viewmats, camera_ids, gaussian_ids, radii, coeffs, depths)
+                launch_context, precomputed=None):
+        if precomputed is not None:
+            assert precomputed.shape == radii.shape[:-1] + (4 if depths is not None else 3,), precomputed.shape
+            colors = precomputed
+        else:
+            with (launch_context if launch_context is not None else contextlib.nullcontext()):
+                colors = _make_lazy_hip_func("view_colors_fwd")(
+                    sh_degree, means, viewmats, camera_ids, gaussian_ids, radii, coeffs, depths)
         ctx.save_for_backward(means, viewmats, coeffs, radii, camera_ids, gaussian_ids, colors)
         ctx.sh_degree = sh_degree
         ctx.has_depths = depths is not None
@@ -1006,7 +1044,7 @@ class _ViewColors(torch.autograd.Function):
                     v_means = v_dirs[0] if v_dirs.shape[0] == 1 else v_dirs.sum(0)
         if ctx.has_depths and ctx.needs_input_grad[5]:
             v_depths = v_colors[..., 3]
-        return None, v_means, None, v_coeffs, None, v_depths, None, None, None
+        return None, v_means, None, v_coeffs, None, v_depths, None, None, None, None
 
 
 class _SphericalHarmonics(torch.autograd.Function):

@@ -62,7 +62,10 @@ class _Beside:
     """
 
     def __init__(self, device):
-        self.main = self.side = self.fork = self._ctx = None
+        self.main = self.side = self.fork = self._ctx = self._waited = None
+        # what the packed projection is asked to make on the helper stream, and what it made
+        self.requests: Dict[str, object] = {}
+        self.results: Dict[str, Tensor] = {}
         if device.type == "cuda" and not torch.cuda.is_current_stream_capturing():
             idx = device.index if device.index is not None else torch.cuda.current_device()
             key = (idx, threading.get_ident())
@@ -74,7 +77,9 @@ class _Beside:
 
     def __enter__(self):
         if self.side is not None:
-            self.side.wait_event(self.fork)
+            if self._waited is not self.fork:  # once per fork: the helper stream runs in order
+                self.side.wait_event(self.fork)
+                self._waited = self.fork
             self._ctx = torch.cuda.stream(self.side)
             self._ctx.__enter__()
         return self
@@ -84,6 +89,11 @@ class _Beside:
             self._ctx.__exit__(*exc)
             self._ctx = None
         return False
+
+    def refork(self):
+        """Moves the fork to what the caller's stream holds now."""
+        if self.side is not None:
+            self.fork = self.main.record_event()
 
     def join(self, *tensors):
         if self.side is not None:
@@ -164,12 +174,27 @@ def rasterization(
     # so that the host waits for the GPU once per call, not twice)
     tile_width = math.ceil(width / float(tile_size))
     tile_height = math.ceil(height / float(tile_size))
+    # (packed: the kernels that write the packed rows go to the helper stream, and with them
+    # what else only needs the projection, the colours of step 3 and the rows' opacities; the
+    # tile intersection works on the projection's dense rows and does not wait for any of it)
+    beside = _Beside(means.device)
+    fused_colors = sh_degree is not None and not viewmats.requires_grad
+    depth_appended = fused_colors and render_mode in ["RGB+D", "RGB+ED"]
+    if packed:
+        if fused_colors and colors.is_contiguous():
+            beside.requests["colors"] = (sh_degree, colors, depth_appended)
+        # the gather opacities[gaussian_ids] (* compensations), where no gradient passes through it
+        no_grad = not torch.is_grad_enabled() or not any(
+            t is not None and t.requires_grad for t in (means, quats, scales, opacities, velocities, viewmats))
+        if no_grad and opacities.is_contiguous() and opacities.dtype == torch.float32:
+            beside.requests["opacities"] = opacities
     proj = fully_fused_projection(
         means, None, quats, scales, velocities, viewmats, Ks, width, height, linear_velocity,
         angular_velocity, rolling_shutter_time, eps2d=eps2d, packed=packed, near_plane=near_plane,
         far_plane=far_plane, radius_clip=radius_clip, sparse_grad=sparse_grad,
         calc_compensations=(rasterize_mode == "antialiased"),
         isect_grid=(tile_size, tile_width, tile_height) if packed else None,
+        beside=beside if packed else None,
     )
     if packed:
         camera_ids, gaussian_ids, radii, means2d, depths, conics, compensations, pix_vels = proj
@@ -184,15 +209,15 @@ def rasterization(
         return o if compensations is None else o * compensations
 
     # 2. tile intersection, sort, offsets
-    beside = _Beside(means.device)  # fork: everything the colours need is enqueued
-    fused_colors = sh_degree is not None and not viewmats.requires_grad
-    depth_appended = fused_colors and render_mode in ["RGB+D", "RGB+ED"]
+    if not packed:
+        beside.refork()  # fork: everything the colours need is enqueued
 
     def fused_view_colors():
         # one kernel for directions, masks, SH, activation and the depth channel
         return view_dependent_colors(sh_degree, means, viewmats, colors, radii,
                                      depths if depth_appended else None, camera_ids,
-                                     gaussian_ids, launch_context=beside)
+                                     gaussian_ids, launch_context=beside,
+                                     precomputed=beside.results.get("colors"))
 
     # The colours run on a helper stream beside the intersection, enqueued behind it: the kernel
     # then meets the segment sort, whose long workgroups leave part of the GPU idle (enqueued
@@ -203,20 +228,30 @@ def rasterization(
         camera_ids=camera_ids, gaussian_ids=gaussian_ids,
     )
     isect_offsets = isect_offset_encode(isect_ids, C, tile_width, tile_height)
-    if packed and not opacities.requires_grad:
+    beside_opacities = packed and not opacities.requires_grad
+    if "opacities" in beside.results:
+        opacities = beside.results["opacities"]
+        if not fused_colors:
+            beside.join()
+    elif beside_opacities:
         # the gather (and the product with the compensations) goes beside the sort too: on the
         # caller's stream it would stand alone between the sort and the compositing.  (Not for a
         # leaf that takes a gradient: autograd would accumulate it on the helper stream.)
         with beside:
             opacities = per_row_opacities()
-        beside.join(opacities)
+        if not fused_colors:
+            beside.join(opacities)
     else:
+        if packed:
+            beside.join()  # the packed rows are written on the helper stream
         opacities = per_row_opacities()
 
     # 3. per-(camera, Gaussian) colours
     if fused_colors:
         colors = fused_view_colors()
-        beside.join(colors)
+        made_beside = "colors" not in beside.results  # (what the projection made was allocated here)
+        beside.join(colors if made_beside else None,
+                    opacities if beside_opacities and "opacities" not in beside.results else None)
     elif sh_degree is None:
         if packed:
             colors = colors[gaussian_ids] if colors.dim() == 2 else colors[camera_ids, gaussian_ids]

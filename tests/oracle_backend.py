@@ -32,7 +32,7 @@ class OracleOps:
 
     def fully_fused_projection_packed_fwd(self, means, covars, quats, scales, velocities, viewmats, Ks,
                                           W, H, lin, ang, rs, eps2d, near, far, radius_clip, calc_comp,
-                                          isect_grid=None):
+                                          isect_grid=None, beside=None):
         radii, m2, d, con, comp, pv = self.fully_fused_projection_fwd(
             means, covars, quats, scales, velocities, viewmats, Ks, W, H, lin, ang, rs, eps2d, near, far,
             radius_clip, calc_comp)

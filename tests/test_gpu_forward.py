@@ -111,9 +111,9 @@ def test_projection_camera(use_covars, use_vel, comp):
 
 @pytest.mark.parametrize("C,N,W,H,ts", [(3, 20000, 320, 240, 16), (1, 5000, 200, 120, 8), (2, 300, 64, 48, 16)])
 def test_packed_projection_counts_the_intersections_of_its_rows(C, N, W, H, ts):
-    """isect_grid: the packed projection returns rows that carry the number of their tile
-    intersections; isect_tiles on those tensors skips its own count and gives the same lists;
-    writing to the tensors, or another grid, makes it count again."""
+    """isect_grid: the packed projection returns rows that carry the lists of their tile
+    intersections; isect_tiles on those tensors hands them out without a count of its own and
+    they are the same lists; writing to the tensors, or another grid, makes it count again."""
     from splatad_amd import fully_fused_projection, isect_tiles
     rng, means, quats, scales, vel = _gaussians(N, 17)
     viewmats, Ks = _cameras(rng, C, W, H)
@@ -140,10 +140,10 @@ def test_packed_projection_counts_the_intersections_of_its_rows(C, N, W, H, ts):
     hinted = fully_fused_projection(*t, isect_grid=(ts, tw, th), **kw)
     for a, b in zip(plain, hinted):
         assert (a is None and b is None) or torch.equal(a, b)
-    grid, n_known = hinted[2]._splatad_isect_count[:2]
+    grid, made = hinted[2]._splatad_isect_count[:2]
     assert grid == (ts, tw, th)
-    assert int(want[0].sum().item()) == n_known == want[1].numel()
-    got = lists(hinted)  # completes what the projection started
+    assert int(want[0].sum().item()) == made[1].numel() == want[1].numel()
+    got = lists(hinted)  # what the projection made
     assert not hasattr(hinted[2], "_splatad_isect_count")  # good for one call
     for a, b in zip(want, got):
         assert torch.equal(a, b)
@@ -160,7 +160,7 @@ def test_packed_projection_counts_the_intersections_of_its_rows(C, N, W, H, ts):
     hinted = fully_fused_projection(*t, isect_grid=(ts, tw, th), **kw)
     hinted[2][: hinted[2].shape[0] // 2] = 0
     changed = lists(hinted)
-    assert changed[1].numel() < n_known
+    assert changed[1].numel() < want[1].numel()
     for a, b in zip(changed, oracle_lists(hinted)):
         np.testing.assert_array_equal(to_np(a), b)
 
