@@ -165,6 +165,57 @@ def test_packed_projection_counts_the_intersections_of_its_rows(C, N, W, H, ts):
         np.testing.assert_array_equal(to_np(a), b)
 
 
+@pytest.mark.parametrize("C,N,W,H,ts,comp,degree,per_sensor,with_depth",
+                         [(3, 20000, 320, 240, 16, False, 3, False, True),
+                          (2, 6000, 200, 120, 8, True, 2, True, False),
+                          (1, 400, 64, 48, 16, True, 0, False, True)])
+def test_packed_projection_makes_what_was_asked_for_beside_the_sort(C, N, W, H, ts, comp, degree, per_sensor,
+                                                                  with_depth):
+    """beside=: the packed rows, their opacities and their colours are written on the helper
+    stream; after the join they equal, bit for bit, the plain projection's rows, the gather
+    opacities[gaussian_ids] (* compensations) and view_dependent_colors on those rows."""
+    from splatad_amd import fully_fused_projection, isect_tiles
+    from splatad_amd.hip._wrapper import view_dependent_colors
+    from splatad_amd.rendering import _Beside
+    rng, means, quats, scales, vel = _gaussians(N, 23)
+    viewmats, Ks = _cameras(rng, C, W, H)
+    lin = rng.normal(size=(C, 3)).astype(np.float32)
+    ang = (rng.normal(size=(C, 3)) * 0.3).astype(np.float32)
+    rs = np.linspace(0.0, 0.03, C).astype(np.float32)
+    K = (degree + 1) ** 2 + 2
+    coeffs = to_dev(rng.normal(size=((C, N, K, 3) if per_sensor else (N, K, 3))).astype(np.float32) * 0.5)
+    opacities = to_dev(rng.uniform(0.05, 1.0, N).astype(np.float32))
+    t = [to_dev(a) if isinstance(a, np.ndarray) else a
+         for a in (means, None, quats, scales, vel, viewmats, Ks, W, H, lin, ang, rs)]
+    kw = dict(eps2d=0.3, near_plane=0.5, far_plane=4.5, radius_clip=0.0, packed=True, calc_compensations=comp)
+    tw, th = math.ceil(W / ts), math.ceil(H / ts)
+    plain = fully_fused_projection(*t, **kw)
+    cam, gid, radii, means2d, depths, conics, comps, pix_vels = plain
+    want_lists = isect_tiles(means2d, radii, depths, ts, tw, th, packed=True, n_cameras=C,
+                             camera_ids=cam, gaussian_ids=gid)
+    want_colors = view_dependent_colors(degree, t[0], t[5], coeffs, radii, depths if with_depth else None, cam, gid)
+    want_opacities = opacities[gid] * comps if comp else opacities[gid]
+    for _ in range(2):  # the second call meets the first one's memory on the helper stream
+        beside = _Beside(torch.device(DEV))
+        assert beside.side is not None
+        beside.requests["colors"] = (degree, coeffs, with_depth)
+        beside.requests["opacities"] = opacities
+        rows = fully_fused_projection(*t, isect_grid=(ts, tw, th), beside=beside, **kw)
+        lists = isect_tiles(rows[3], rows[2], rows[4], ts, tw, th, packed=True, n_cameras=C,
+                            camera_ids=rows[0], gaussian_ids=rows[1])
+        beside.join()
+        for a, b in zip(plain, rows):
+            assert (a is None and b is None) or torch.equal(a, b)
+        for a, b in zip(want_lists, lists):
+            assert torch.equal(a, b)
+        assert torch.equal(beside.results["colors"], want_colors)
+        assert torch.equal(beside.results["opacities"], want_opacities)
+        # view_dependent_colors takes what was made instead of running its kernel
+        taken = view_dependent_colors(degree, t[0], t[5], coeffs, rows[2], rows[4] if with_depth else None,
+                                      rows[0], rows[1], precomputed=beside.results["colors"])
+        assert taken is beside.results["colors"]
+
+
 @pytest.mark.parametrize("use_covars", [False, True])
 @pytest.mark.parametrize("use_vel", [False, True])
 def test_projection_lidar(use_covars, use_vel):
