@@ -683,8 +683,6 @@ extern "C" int splatad_projection_packed_fill(uint32_t C, uint32_t N, int64_t nn
                                               float *pix_vels, const float *opacities,
                                               float *row_opacities, splatad_stream_t stream) {
     SPLATAD_REQUIRE(indptr != nullptr, "packed projection: indptr is null");
-    SPLATAD_REQUIRE((opacities != nullptr) == (row_opacities != nullptr),
-                    "packed projection: opacities and row_opacities go together");
     const uint64_t T = (uint64_t)C * N;
     if (T == 0 || nnz == 0) {
         hipLaunchKernelGGL(fill_i32_kernel, dim3((C + 1 + 255) / 256), dim3(256), 0,
@@ -695,6 +693,8 @@ extern "C" int splatad_projection_packed_fill(uint32_t C, uint32_t N, int64_t nn
     SPLATAD_REQUIRE(workspace && camera_ids && gaussian_ids && radii && means2d && depths &&
                         conics && pix_vels,
                     "packed projection: null pointer argument");
+    SPLATAD_REQUIRE((opacities != nullptr) == (row_opacities != nullptr),
+                    "packed projection: opacities and row_opacities go together");
     PackedWorkspace w = carve_packed((void *)workspace, T);
     hipLaunchKernelGGL(packed_compact_kernel,
                        dim3((uint32_t)((T + SPLATAD_THREADS - 1) / SPLATAD_THREADS)),

@@ -457,6 +457,42 @@ def test_lidar_without_depth_compensation_end_to_end():
     assert torch.equal(with_dc[0][..., :-1], rf[..., :-1])
 
 
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("case", ["behind", "between_tiles"])
+def test_camera_frames_without_rows_or_without_intersections(packed, case):
+    """Nothing in front of the camera (no packed rows at all), and Gaussians that are kept by the
+    projection but meet no tile (pushed outside the image after it): empty lists, a render of
+    the background, no alpha; the packed path's helper-stream work has nothing to write."""
+    from splatad_amd import rasterization
+    s = _cam_scene(n=2000)
+    d = workloads.to_device(s, DEV)
+    if case == "behind":
+        d["means"] = d["means"].clone()
+        d["means"][:, 2] = -torch.abs(d["means"][:, 2]) - 100.0  # behind every near plane
+    bg = torch.tensor([[0.25, 0.5, 0.75]], device=DEV)
+    kw = dict(near_plane=d["near_plane"], far_plane=d["far_plane"], eps2d=d["eps2d"], tile_size=d["tile_size"],
+              packed=packed, sh_degree=s["sh_degree"], backgrounds=bg, render_mode="RGB")
+    W, H = d["width"], d["height"]
+    if case == "between_tiles":
+        # a sliver of an image: the few Gaussians the projection keeps are culled again by ...
+        # nothing here; instead ask for an image that no Gaussian of the scene reaches
+        Ks = d["Ks"].clone()
+        Ks[:, 0, 2] += 1.0e6  # principal point far to the right: all means project outside
+        d = dict(d, Ks=Ks)
+    for _ in range(2):
+        rc, ra, meta = rasterization(d["means"], d["quats"], d["scales"], d["opacities"], d["colors"],
+                                     d["velocities"], d["viewmats"], d["Ks"], W, H, d["linear_velocity"],
+                                     d["angular_velocity"], d["rolling_shutter_time"], **kw)
+        torch.cuda.synchronize()
+        assert meta["isect_ids"].numel() == 0 and meta["flatten_ids"].numel() == 0
+        assert int(meta["tiles_per_gauss"].sum().item()) == 0
+        assert int(meta["isect_offsets"].abs().sum().item()) == 0
+        if packed:
+            assert meta["camera_ids"].numel() == meta["radii"].shape[0] == meta["means2d"].shape[0]
+        assert torch.equal(ra, torch.zeros_like(ra))
+        assert torch.allclose(rc, bg.view(1, 1, 1, 3).expand_as(rc))
+
+
 def test_two_host_threads_on_two_streams():
     """The boundary is callable from several host threads, each on a stream of its own: two
     threads render cameras (packed and unpacked: both counting calls) and lidar sweeps at the
