@@ -422,12 +422,49 @@ __device__ __forceinline__ uint32_t slab_of(uint32_t d, const uint32_t *bounds, 
     return s;
 }
 
-// Coarse binning without global atomics.  A fixed grid of workgroups strides over the
-// Gaussians; each keeps the counters of all coarse blocks in LDS.  COUNT pass: the
-// workgroup's counts go to its own row of a [workgroup][block] table.  The table is then
-// scanned block-major, which gives every (block, workgroup) its own run in the block's
-// list.  FILL pass: the same workgroup meets the same Gaussians, starts its LDS cursors at
-// those runs and writes the entries {flatten id, depth bits, block, tile mask}.
+// Exclusive scan over L values held in LDS by a workgroup of nt threads (a multiple of 64):
+// thread t owns ceil(L / nt) consecutive values; load(i) gives value i, store(i, before, v)
+// receives the sum of the values before i.  Returns the total.  Ends with a barrier.
+template <typename Load, typename Store>
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t L, uint32_t tid, uint32_t nt,
+                                                         uint32_t *s_wave, Load &&load, Store &&store) {
+    const uint32_t lane = tid & (SPLATAD_WAVE - 1), wave = tid / SPLATAD_WAVE;
+    const uint32_t per = (L + nt - 1) / nt;
+    const uint32_t b0 = min(L, tid * per), b1 = min(L, b0 + per);
+    uint32_t sum = 0;
+    for (uint32_t b = b0; b < b1; ++b) sum += load(b);
+    uint32_t incl = sum;
+#pragma unroll
+    for (int off = 1; off < SPLATAD_WAVE; off <<= 1) {
+        const uint32_t o = (uint32_t)__shfl_up((int)incl, off, SPLATAD_WAVE);
+        if ((int)lane >= off) incl += o;
+    }
+    if (lane == SPLATAD_WAVE - 1) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - sum, total = 0;
+    for (uint32_t w = 0; w < nt / SPLATAD_WAVE; ++w) {
+        const uint32_t v = s_wave[w];
+        if (w < wave) run += v;
+        total += v;
+    }
+    for (uint32_t b = b0; b < b1; ++b) {
+        const uint32_t v = load(b);
+        store(b, run, v);
+        run += v;
+    }
+    __syncthreads();
+    return total;
+}
+
+// Coarse binning with one global atomic per (workgroup, block).  A fixed grid of workgroups
+// strides over the Gaussians; each keeps the counters of all coarse blocks in LDS.  COUNT pass:
+// at its end the workgroup adds its count of every block to the block's total (`totals`, zero
+// before the pass) and keeps what the addition returns, the start of its run inside the block's
+// list, in its own row of a [workgroup][block] table; the order of the runs inside a list is
+// whatever the atomics give, and no later stage depends on it.  FILL pass: the same workgroup
+// meets the same Gaussians; it scans the totals (a few hundred to a few thousand values, by
+// every workgroup for itself: no scan kernels between the passes), starts its LDS cursors at
+// block start + run start and writes the entries {flatten id, depth bits, block, tile mask}.
 // One launch covers the cameras [cam_lo, cam_hi) (as many as the LDS holds counters for).
 constexpr uint32_t kCoarseThreads = 1024;
 constexpr uint32_t kCoarseLdsBlocks = 36864; // counters per workgroup, 144 KB
@@ -440,21 +477,28 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
                     uint32_t cam_lo, uint32_t cam_hi, uint32_t n_blocks, int32_t *table,
                     uint4 *__restrict__ entries, uint32_t sshift,
                     const uint32_t *__restrict__ slab_bounds, const int32_t *__restrict__ remap,
-                    int32_t *__restrict__ tiles_out, int32_t *__restrict__ clear, uint64_t clear_words) {
+                    int32_t *__restrict__ tiles_out, int32_t *__restrict__ totals,
+                    int64_t *__restrict__ n_entries) {
     extern __shared__ int32_t s_blocks[];
-    // (the counting pass can zero the counters of the later stages on the counting kernel's behalf)
-    if (!FILL)
-        for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words;
-             i += (uint64_t)gridDim.x * blockDim.x)
-            clear[i] = 0;
     __shared__ uint32_t s_bounds[1u << kSlabShiftMax];
+    __shared__ uint32_t s_scan[kCoarseThreads / SPLATAD_WAVE];
     SPLATAD_STAGE_ELEVATIONS(g)
     // blocks and block counters below are (coarse block, slab) pairs, the slab in the low bits
     const uint32_t per_cam = (cg.cw * cg.ch) << sshift;
     const uint32_t first = cam_lo * per_cam, count = (cam_hi - cam_lo) * per_cam;
     const uint32_t n_bounds = (1u << sshift) - 1u;
     int32_t *row = table + (size_t)blockIdx.x * n_blocks + first;
-    for (uint32_t b = threadIdx.x; b < count; b += blockDim.x) s_blocks[b] = FILL ? row[b] : 0;
+    if (FILL) {
+        // cursor of block b: the blocks before it (of all launches) plus this workgroup's run start
+        const uint32_t all = block_exclusive_scan(
+            first + count, threadIdx.x, blockDim.x, s_scan, [&](uint32_t j) { return (uint32_t)totals[j]; },
+            [&](uint32_t j, uint32_t before, uint32_t) {
+                if (j >= first) s_blocks[j - first] = (int32_t)before + row[j - first];
+            });
+        if (blockIdx.x == 0 && threadIdx.x == 0 && first + count == n_blocks) *n_entries = (int64_t)all;
+    } else {
+        for (uint32_t b = threadIdx.x; b < count; b += blockDim.x) s_blocks[b] = 0;
+    }
     if (threadIdx.x < n_bounds) s_bounds[threadIdx.x] = slab_bounds[threadIdx.x];
     __syncthreads();
     const float *depths_needed = FILL || sshift ? depths : nullptr;
@@ -489,7 +533,10 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
     }
     if (!FILL) {
         __syncthreads();
-        for (uint32_t b = threadIdx.x; b < count; b += blockDim.x) row[b] = s_blocks[b];
+        for (uint32_t b = threadIdx.x; b < count; b += blockDim.x) {
+            const int32_t c = s_blocks[b];
+            row[b] = c ? atomicAdd(&totals[first + b], c) : 0;
+        }
     }
 }
 
@@ -699,40 +746,6 @@ constexpr uint32_t kSortWindow = 15360;     // LDS window (entries) when staging
 __host__ __device__ inline uint32_t sort_bucket_capacity(uint32_t max_n) {
     const uint32_t split = max_n / kSortBucketMean < kSortSplit ? max_n / kSortBucketMean : kSortSplit;
     return split + kSortFineBins + 1;
-}
-
-// Exclusive scan over L values held in LDS by a workgroup of nt threads (a multiple of 64):
-// thread t owns ceil(L / nt) consecutive values; load(i) gives value i, store(i, before, v)
-// receives the sum of the values before i.  Returns the total.  Ends with a barrier.
-template <typename Load, typename Store>
-__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t L, uint32_t tid, uint32_t nt,
-                                                         uint32_t *s_wave, Load &&load, Store &&store) {
-    const uint32_t lane = tid & (SPLATAD_WAVE - 1), wave = tid / SPLATAD_WAVE;
-    const uint32_t per = (L + nt - 1) / nt;
-    const uint32_t b0 = min(L, tid * per), b1 = min(L, b0 + per);
-    uint32_t sum = 0;
-    for (uint32_t b = b0; b < b1; ++b) sum += load(b);
-    uint32_t incl = sum;
-#pragma unroll
-    for (int off = 1; off < SPLATAD_WAVE; off <<= 1) {
-        const uint32_t o = (uint32_t)__shfl_up((int)incl, off, SPLATAD_WAVE);
-        if ((int)lane >= off) incl += o;
-    }
-    if (lane == SPLATAD_WAVE - 1) s_wave[wave] = incl;
-    __syncthreads();
-    uint32_t run = incl - sum, total = 0;
-    for (uint32_t w = 0; w < nt / SPLATAD_WAVE; ++w) {
-        const uint32_t v = s_wave[w];
-        if (w < wave) run += v;
-        total += v;
-    }
-    for (uint32_t b = b0; b < b1; ++b) {
-        const uint32_t v = load(b);
-        store(b, run, v);
-        run += v;
-    }
-    __syncthreads();
-    return total;
 }
 
 // One workgroup, one sample per lane: kSlabSamples Gaussians at a fixed stride, ordered by
@@ -1304,12 +1317,12 @@ struct IsectWorkspace {
     int64_t *n_entries;           // [1] length of the coarse lists
     int64_t *scan_total;          // [1]
     uint32_t *slab_bounds;        // [1 << kSlabShiftMax] depth bits at which the slabs begin
-    int32_t *zeroed;              // tile_counts, tile_fill are contiguous, cleared together
+    int32_t *zeroed;              // tile_counts, tile_fill, block_totals, seg_counts: contiguous, cleared together
     uint64_t n_zeroed;
     int32_t *tile_counts;         // [tile copies * segments], segments = C * n_tiles * slabs
     int32_t *tile_fill;           // same
-    int32_t *coarse_counts;       // [coarse workgroups * C * blocks]
-    int32_t *coarse_starts;       // same
+    int32_t *block_totals;        // [C * blocks] entries per coarse block (in the cleared part)
+    int32_t *coarse_counts;       // [coarse workgroups * C * blocks] run starts inside the blocks' lists
     int32_t *tile_starts;         // [tile copies * segments]
     uint32_t *seg_counts;         // [kSortClasses] segments per size class (in the cleared part)
     uint32_t *seg_lists;          // [kSortClasses * segments]
@@ -1380,8 +1393,7 @@ static IsectPlan isect_plan(const TileGrid &g, uint64_t total, uint32_t C, int s
 static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslots,
                           IsectWorkspace *out) {
     const uint64_t tslots = segs * isect_copies(segs);
-    uint64_t scan_n = total > cslots ? total : cslots;
-    if (tslots > scan_n) scan_n = tslots;
+    const uint64_t scan_n = total > tslots ? total : tslots;
     char *p = (char *)ws;
     IsectWorkspace w = {};
     w.n_entries = (int64_t *)p;             p += 256;
@@ -1390,10 +1402,10 @@ static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslo
     w.zeroed = (int32_t *)p;
     w.tile_counts = (int32_t *)p;           p += splatad_align256(tslots * 4);
     w.tile_fill = (int32_t *)p;             p += splatad_align256(tslots * 4);
+    w.block_totals = (int32_t *)p;          p += splatad_align256(segs * 4); // blocks <= segments
     w.seg_counts = (uint32_t *)p;           p += 256;
     w.n_zeroed = (uint64_t)(p - (char *)w.zeroed) / 4;
     w.coarse_counts = (int32_t *)p;         p += splatad_align256(cslots * 4);
-    w.coarse_starts = (int32_t *)p;         p += splatad_align256(cslots * 4);
     w.tile_starts = (int32_t *)p;           p += splatad_align256(tslots * 4);
     w.seg_lists = (uint32_t *)p;            p += splatad_align256(segs * kSortClasses * 4);
     w.block_sums = (int64_t *)p;            p += scan_workspace_bytes((int64_t)scan_n);
@@ -1451,14 +1463,13 @@ static int isect_device(IsectDevice **out) {
     return 0;
 }
 
-// First stages of the binning, which need no list memory (the tile counters were cleared
-// together with the counting kernel's): count the coarse lists and scan the counts (the table is
-// stored [workgroup][block] and scanned block-major, which makes a block's list contiguous).
+// First stage of the binning, which needs no list memory (the counters were cleared by the
+// kernel before it): count the coarse lists.
 template <bool LIDAR>
 static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const IsectWorkspace &w,
                                 uint64_t total, uint32_t N, const int64_t *camera_ids,
                                 const float *means2d, const void *radii, const float *depths,
-                                uint32_t C, hipStream_t stream, bool clear) {
+                                uint32_t C, hipStream_t stream) {
     SPLATAD_REQUIRE(pl.per_cam <= kCoarseLdsBlocks, "isect: %u x %u tiles per sensor exceed the "
                     "binning capacity", g.tile_w, g.tile_h);
     SPLATAD_REQUIRE(pl.blocks < (1ull << 31) && pl.cslots < (1ull << 31), "isect: tile grid too large");
@@ -1483,12 +1494,10 @@ static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const Is
                            total, N, camera_ids, means2d, radii, pl.sshift ? depths : nullptr, c0, c1,
                            (uint32_t)pl.blocks, w.coarse_counts, (uint4 *)nullptr, pl.sshift,
                            (const uint32_t *)w.slab_bounds, (const int32_t *)nullptr, (int32_t *)nullptr,
-                           w.zeroed, clear && c0 == 0 ? w.n_zeroed : (uint64_t)0);
+                           w.block_totals, (int64_t *)nullptr);
     }
     SPLATAD_LAUNCH_CHECK();
-    return launch_exclusive_scan<int32_t>(w.coarse_counts, (int64_t)pl.cslots,
-                                          pl.coarse_wgs > 1 ? -(int)pl.coarse_wgs : 1, 0,
-                                          w.coarse_starts, w.n_entries, w.block_sums, stream);
+    return 0;
 }
 
 // The counting kernel's cross-workgroup counters: one set per leased host word (calls that
@@ -1546,8 +1555,8 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     }
     // the counting kernel clears the tile counters, the fill cursors and the class counters of
     // the binning behind it
-    // (a caller that knows the count and sorts without depth slabs needs nothing else of the
-    // counting kernel: the coarse counting pass then clears)
+    // (a caller that knows the count and sorts without depth slabs needs nothing of the counting
+    // kernel but the cleared counters)
     const bool skip_count = known && sort && pl.sshift == 0;
     if (!skip_count) {
         dim3 count_grid = grid_for(total);
@@ -1555,6 +1564,10 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
         hipLaunchKernelGGL(isect_count_kernel<LIDAR>, count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
                            total, means2d, radii, tiles_per_gauss, counters, lease.word.device,
                            w.zeroed, sort ? w.n_zeroed : (uint64_t)0);
+        SPLATAD_LAUNCH_CHECK();
+    } else {
+        hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(w.n_zeroed), dim3(SPLATAD_THREADS), 0, stream,
+                           w.zeroed, (int64_t)w.n_zeroed);
         SPLATAD_LAUNCH_CHECK();
     }
     // work for the GPU while the host learns the count and sizes the lists
@@ -1565,7 +1578,7 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
             SPLATAD_LAUNCH_CHECK();
         }
         if (int rc = enqueue_coarse_count<LIDAR>(g, pl, w, total, N, camera_ids, means2d, radii, depths,
-                                                 C, stream, skip_count))
+                                                 C, stream))
             return rc;
     }
     if (known) return 0;
@@ -1623,14 +1636,14 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         SPLATAD_LAUNCH_CHECK();
         return 0;
     }
-    // the coarse lists were counted and scanned by the counting call; fill them
+    // the coarse lists were counted by the counting call; fill them
     for (uint32_t c0 = 0; c0 < C; c0 += pl.cams_per_launch) {
         const uint32_t c1 = C - c0 < pl.cams_per_launch ? C : c0 + pl.cams_per_launch;
         hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, true>), dim3(pl.coarse_wgs),
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, cg,
                            total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)pl.blocks,
-                           w.coarse_starts, w.entries, sshift, (const uint32_t *)w.slab_bounds, remap,
-                           tiles_out, (int32_t *)nullptr, (uint64_t)0);
+                           w.coarse_counts, w.entries, sshift, (const uint32_t *)w.slab_bounds, remap,
+                           tiles_out, w.block_totals, w.n_entries);
     }
     SPLATAD_LAUNCH_CHECK();
     // tile segments: count, scan, fill.  The number of coarse entries stays on the device;
