@@ -457,6 +457,48 @@ def test_lidar_without_depth_compensation_end_to_end():
     assert torch.equal(with_dc[0][..., :-1], rf[..., :-1])
 
 
+@pytest.mark.parametrize("opts", [
+    dict(sh_degree=3, render_mode="RGB"), dict(sh_degree=0, render_mode="RGB+ED"),
+    dict(sh_degree=None, render_mode="RGB+D"), dict(sh_degree=2, render_mode="D"),
+    dict(sh_degree=3, render_mode="RGB+D", rasterize_mode="antialiased", radius_clip=2.0),
+    dict(sh_degree=1, render_mode="ED", tile_size=8), dict(sh_degree=3, render_mode="RGB", per_sensor=True)])
+def test_surround_packed_equals_unpacked_for_every_option(opts):
+    """What the packed call makes beside the sort (rows, opacities, colours) feeds the same
+    compositing kernel as the unpacked call's tensors: the renders are equal bit for bit, with
+    gradients switched off and with them switched on (where the opacities come from a gather
+    that autograd sees)."""
+    from splatad_amd import rasterization
+    opts = dict(opts)
+    s = workloads.camera_driving(n=20000, width=320, height=180, n_cameras=3, with_velocities=True)
+    d = workloads.to_device(s, DEV)
+    C, N = d["viewmats"].shape[0], d["means"].shape[0]
+    colors = d["colors"]
+    if opts.get("sh_degree") is None:
+        colors = torch.rand((N, 3), device=DEV, generator=torch.Generator(device=DEV).manual_seed(5))
+    elif opts.pop("per_sensor", False):
+        colors = colors[None].expand(C, -1, -1, -1).contiguous() * torch.linspace(0.5, 1.5, C, device=DEV).view(C, 1, 1, 1)
+    opts.pop("per_sensor", None)
+    bg = torch.rand((C, 3 if "RGB" in opts["render_mode"] else 1), device=DEV,
+                    generator=torch.Generator(device=DEV).manual_seed(6))
+    if opts["render_mode"] in ("D", "ED"):
+        bg = None
+    kw = dict(near_plane=d["near_plane"], far_plane=d["far_plane"], eps2d=d["eps2d"],
+              tile_size=opts.pop("tile_size", d["tile_size"]), backgrounds=bg, **opts)
+    args = (d["means"], d["quats"], d["scales"], d["opacities"], colors, d["velocities"], d["viewmats"], d["Ks"],
+            d["width"], d["height"], d["linear_velocity"], d["angular_velocity"], d["rolling_shutter_time"])
+    with torch.no_grad():
+        dense = rasterization(*args, packed=False, **kw)
+        packed = rasterization(*args, packed=True, **kw)
+    assert torch.equal(dense[0], packed[0]) and torch.equal(dense[1], packed[1])
+    assert float(dense[1].max()) > 0.5  # something was rendered
+    sel = dense[2]["radii"][..., 0] > 0
+    assert torch.equal(dense[2]["opacities"].expand(C, N)[sel], packed[2]["opacities"])
+    # gradients on: the same images again
+    leaves = [t.clone().requires_grad_() for t in (d["means"], d["opacities"])]
+    packed_grad = rasterization(leaves[0], d["quats"], d["scales"], leaves[1], *args[4:], packed=True, **kw)
+    assert torch.equal(packed_grad[0].detach(), dense[0]) and torch.equal(packed_grad[1].detach(), dense[1])
+
+
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("case", ["behind", "between_tiles"])
 def test_camera_frames_without_rows_or_without_intersections(packed, case):
