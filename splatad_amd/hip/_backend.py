@@ -24,6 +24,9 @@ LIB_PATH = os.path.join(_PKG_DIR, "libsplatad_hip.so")
 _lib = None
 
 
+ABI_VERSION = 5  # splatad_abi_version() of the library these bindings were written for
+
+
 def load_library():
     """Returns the ctypes handle of libsplatad_hip.so; raises if it has not been built."""
     global _lib
@@ -36,6 +39,10 @@ def load_library():
         lib = ctypes.CDLL(LIB_PATH)
         lib.splatad_last_error.restype = ctypes.c_char_p
         lib.splatad_abi_version.restype = ctypes.c_int
+        if lib.splatad_abi_version() != ABI_VERSION:
+            raise RuntimeError(
+                f"{LIB_PATH} has ABI version {lib.splatad_abi_version()}, this package needs {ABI_VERSION}: "
+                "rebuild it with `python -m splatad_amd.build`")
         for name in ("splatad_projection_packed_workspace_bytes", "splatad_isect_workspace_bytes",
                      "splatad_isect_lists_bytes",
                      "splatad_map_points_to_lidar_tiles_workspace_bytes",
