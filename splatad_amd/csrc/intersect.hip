@@ -581,10 +581,11 @@ __device__ __forceinline__ void classify_segment(uint32_t seg, uint32_t lane, ui
     }
 }
 
-// Tile binning.  A wavefront takes 64 consecutive coarse entries; those of one block (nearly
-// always all 64, the lists being contiguous) are handled together: for each tile of the
-// block a ballot over the mask bit gives the number of entries and every entry's rank, and
-// the lane that owns the tile issues the one atomic.  FILL == false adds to the tile counts,
+// Tile binning.  A wavefront takes 64 consecutive coarse entries, a workgroup 256; those of one
+// block (nearly always all of them, the lists being contiguous) are handled together: for each
+// tile of the block a ballot over the mask bit gives the number of entries and every entry's
+// rank inside the wavefront, the wavefronts' counts are added up in LDS, and the lane that owns
+// the tile issues one atomic for the workgroup.  FILL == false adds to the tile counts,
 // FILL == true reserves the run in the tile's segment and writes the pairs.
 // BITS == 16: blocks of 4 x 4 tiles (every camera grid, lidar grids whose columns divide by 4),
 // the loops over the tiles unrolled with the ballots kept in scalar registers; BITS == 0: any
@@ -612,73 +613,143 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
     const float inv_cw = 1.0f / (float)cg.cw;
     const uint32_t cap = (uint32_t)n_isects; // below 2^31
     const uint64_t below = (1ull << lane) - 1ull;
+    constexpr uint32_t kWaves = SPLATAD_THREADS / SPLATAD_WAVE;
+    constexpr uint32_t kNone = 0xFFFFFFFFu, kMixed = 0xFFFFFFFEu; // no (block, slab) pair reaches 2^31
+    __shared__ uint32_t s_block[kWaves];   // the one block of a wavefront's entries, or kNone / kMixed
+    __shared__ uint32_t s_cnt[kWaves][16]; // entries per tile of that block, per wavefront
+    __shared__ int32_t s_base[16];         // where the workgroup's run starts in each tile's segment
+    const uint32_t wave = threadIdx.x / SPLATAD_WAVE;
     // the tile counters are replicated like the coarse ones; both passes run on the same
     // grid, so an entry meets the same copy in both
-    const int64_t copy_base = (int64_t)(wave_id & (copies - 1)) * n_segments;
-    for (int64_t e0 = wave_id * SPLATAD_WAVE; e0 < n_entries; e0 += n_waves * SPLATAD_WAVE) {
-        const bool has = e0 + lane < n_entries;
-        const uint4 rec = has ? entries[e0 + lane] : make_uint4(0, 0, 0xFFFFFFFFu, 0);
-        uint64_t todo = __ballot(has);
-        while (todo) {
-            const int leader = __ffsll((unsigned long long)todo) - 1;
-            // (coarse block, slab) of the leader; n_segments counts (tile, slab) pairs
-            const uint32_t block_slab = (uint32_t)__shfl((int)rec.z, leader, SPLATAD_WAVE);
-            const bool in = has && rec.z == block_slab;
-            const uint32_t block = block_slab >> sshift, slab = block_slab & ((1u << sshift) - 1u);
-            todo &= ~__ballot(in);
-            uint32_t my_cnt = 0;
-            const uint32_t mask = in ? rec.w : 0u;
-            uint64_t hits[BITS > 0 ? BITS : 1];
-            if (BITS > 0) {
+    const int64_t copy_base = (int64_t)(blockIdx.x & (copies - 1)) * n_segments;
+
+    // counts the entries of the group `in` per tile (lane t < bits gets tile t's) and keeps the ballots
+    uint64_t hits[BITS > 0 ? BITS : 1];
+    auto count_group = [&](uint32_t mask) -> uint32_t {
+        uint32_t my_cnt = 0;
+        if (BITS > 0) {
 #pragma unroll
-                for (int t = 0; t < BITS; ++t) {
-                    hits[t] = __ballot((mask >> t) & 1u);
-                    const uint32_t n_hits = (uint32_t)__popcll(hits[t]); // uniform
-                    asm("v_writelane_b32 %0, %1, %2" : "+v"(my_cnt) : "s"(n_hits), "n"(t));
-                }
-            } else {
-                for (uint32_t t = 0; t < bits; ++t) {
-                    const uint64_t b = __ballot((mask >> t) & 1u);
-                    if (lane == t) my_cnt = (uint32_t)__popcll(b);
-                }
+            for (int t = 0; t < BITS; ++t) {
+                hits[t] = __ballot((mask >> t) & 1u);
+                const uint32_t n_hits = (uint32_t)__popcll(hits[t]); // uniform
+                asm("v_writelane_b32 %0, %1, %2" : "+v"(my_cnt) : "s"(n_hits), "n"(t));
             }
-            // lane t < bits owns tile t of the block
-            int64_t tile = copy_base;
-            if (lane < bits) {
-                const uint32_t cam = block < per_cam ? 0u : block / per_cam, r = block - cam * per_cam;
-                const uint32_t by = div_by(r, cg.cw, inv_cw), bx = r - by * cg.cw;
-                const uint32_t x = (bx << cg.bshift) + (lane & ((1u << cg.bshift) - 1u));
-                const uint32_t y = (by << kCoarseRowShift) + (lane >> cg.bshift);
-                tile += (((int64_t)cam * tile_w * tile_h + (int64_t)y * tile_w + x) << sshift) | slab;
+        } else {
+            for (uint32_t t = 0; t < bits; ++t) {
+                const uint64_t b = __ballot((mask >> t) & 1u);
+                if (lane == t) my_cnt = (uint32_t)__popcll(b);
+            }
+        }
+        return my_cnt;
+    };
+    // counter of the tile that lane t < bits owns in the block
+    auto tile_of = [&](uint32_t block_slab) -> int64_t {
+        const uint32_t block = block_slab >> sshift, slab = block_slab & ((1u << sshift) - 1u);
+        int64_t tile = copy_base;
+        if (lane < bits) {
+            const uint32_t cam = block < per_cam ? 0u : block / per_cam, r = block - cam * per_cam;
+            const uint32_t by = div_by(r, cg.cw, inv_cw), bx = r - by * cg.cw;
+            const uint32_t x = (bx << cg.bshift) + (lane & ((1u << cg.bshift) - 1u));
+            const uint32_t y = (by << kCoarseRowShift) + (lane >> cg.bshift);
+            tile += (((int64_t)cam * tile_w * tile_h + (int64_t)y * tile_w + x) << sshift) | slab;
+        }
+        return tile;
+    };
+    // writes the group's pairs: tile t's run of this wavefront starts at dst of lane t
+    // (the bound `cap` holds whenever n_isects is the count of these very rows; it keeps a
+    // caller's mismatch from writing outside the lists)
+    auto write_group = [&](uint32_t mask, int32_t dst, uint64_t pair) {
+        if (BITS > 0) {
+#pragma unroll
+            for (int t = 0; t < BITS; ++t) {
+                if (hits[t] == 0) continue; // uniform
+                const uint32_t first = (uint32_t)__builtin_amdgcn_readlane(dst, t);
+                const uint32_t at = __builtin_amdgcn_mbcnt_hi(
+                    (uint32_t)(hits[t] >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)hits[t], first));
+                if (((mask >> t) & 1u) && at < cap) pairs[at] = pair;
+            }
+        } else {
+            for (uint32_t t = 0; t < bits; ++t) {
+                const bool hit = (mask >> t) & 1u;
+                const uint64_t b = __ballot(hit);
+                const int32_t first = __shfl(dst, (int)t, SPLATAD_WAVE);
+                const uint32_t at = (uint32_t)first + (uint32_t)__popcll(b & below);
+                if (hit && at < cap) pairs[at] = pair;
+            }
+        }
+    };
+
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t first_entry = (int64_t)blockIdx.x * blockDim.x; first_entry < n_entries;
+         first_entry += stride) { // uniform across the workgroup
+        const int64_t e0 = first_entry + (int64_t)wave * SPLATAD_WAVE;
+        const bool has = e0 + lane < n_entries;
+        const uint4 rec = has ? entries[e0 + lane] : make_uint4(0, 0, kNone, 0);
+        const uint64_t pair = ((uint64_t)rec.y << 32) | (uint64_t)rec.x;
+        const uint64_t have = __ballot(has);
+        // Nearly always the 256 entries of the workgroup belong to one block: then the four
+        // wavefronts add up their counts in LDS and one of them issues the atomics, a quarter of
+        // what the wavefronts would issue on their own (the kernel is bound by those atomics).
+        const uint32_t lead = (uint32_t)__builtin_amdgcn_readfirstlane((int)rec.z);
+        const bool one = __ballot(has && rec.z != lead) == 0;
+        if (lane == 0) s_block[wave] = have == 0 ? kNone : (one ? lead : kMixed);
+        __syncthreads();
+        uint32_t common = kNone;
+        bool together = true;
+#pragma unroll
+        for (uint32_t w = 0; w < kWaves; ++w) {
+            const uint32_t b = s_block[w];
+            if (b == kMixed) together = false;
+            else if (b != kNone) {
+                if (common == kNone) common = b;
+                else if (common != b) together = false;
+            }
+        }
+        if (together && common != kNone) { // uniform across the workgroup
+            const uint32_t mask = has ? rec.w : 0u;
+            const uint32_t my_cnt = count_group(mask);
+            if (lane < 16) s_cnt[wave][lane] = lane < bits ? my_cnt : 0u;
+            __syncthreads();
+            const int64_t tile = tile_of(common);
+            uint32_t before = 0, all = 0; // entries of the wavefronts before this one, and of all
+            if (lane < 16) {
+#pragma unroll
+                for (uint32_t w = 0; w < kWaves; ++w) {
+                    const uint32_t c = s_cnt[w][lane];
+                    if (w < wave) before += c;
+                    all += c;
+                }
             }
             if (!FILL) {
-                if (my_cnt) atomicAdd(&tile_counts[tile], (int32_t)my_cnt);
+                if (wave == 0 && all) atomicAdd(&tile_counts[tile], (int32_t)all);
             } else {
-                int32_t dst = 0;
-                if (my_cnt) dst = tile_starts[tile] + atomicAdd(&tile_fill[tile], (int32_t)my_cnt);
-                const uint64_t pair = ((uint64_t)rec.y << 32) | (uint64_t)rec.x;
-                // (the bound `cap` holds whenever n_isects is the count of these very rows; it
-                // keeps a caller's mismatch from writing outside the lists)
-                if (BITS > 0) {
-#pragma unroll
-                    for (int t = 0; t < BITS; ++t) {
-                        if (hits[t] == 0) continue; // uniform
-                        const uint32_t first = (uint32_t)__builtin_amdgcn_readlane(dst, t);
-                        const uint32_t at = __builtin_amdgcn_mbcnt_hi(
-                            (uint32_t)(hits[t] >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)hits[t], first));
-                        if (((mask >> t) & 1u) && at < cap) pairs[at] = pair;
-                    }
+                if (wave == 0 && lane < 16)
+                    s_base[lane] = all ? tile_starts[tile] + atomicAdd(&tile_fill[tile], (int32_t)all) : 0;
+                __syncthreads();
+                const int32_t dst = lane < 16 ? s_base[lane] + (int32_t)before : 0;
+                write_group(mask, dst, pair);
+            }
+        } else {
+            uint64_t todo = have;
+            while (todo) {
+                const int leader = __ffsll((unsigned long long)todo) - 1;
+                // (coarse block, slab) of the leader; n_segments counts (tile, slab) pairs
+                const uint32_t block_slab = (uint32_t)__shfl((int)rec.z, leader, SPLATAD_WAVE);
+                const bool in = has && rec.z == block_slab;
+                todo &= ~__ballot(in);
+                const uint32_t mask = in ? rec.w : 0u;
+                const uint32_t my_cnt = count_group(mask);
+                const int64_t tile = tile_of(block_slab);
+                if (!FILL) {
+                    if (my_cnt) atomicAdd(&tile_counts[tile], (int32_t)my_cnt);
                 } else {
-                    for (uint32_t t = 0; t < bits; ++t) {
-                        const bool hit = (mask >> t) & 1u;
-                        const uint64_t b = __ballot(hit);
-                        const int32_t first = __shfl(dst, (int)t, SPLATAD_WAVE);
-                        const uint32_t at = (uint32_t)first + (uint32_t)__popcll(b & below);
-                        if (hit && at < cap) pairs[at] = pair;
-                    }
+                    int32_t dst = 0;
+                    if (my_cnt) dst = tile_starts[tile] + atomicAdd(&tile_fill[tile], (int32_t)my_cnt);
+                    write_group(mask, dst, pair);
                 }
             }
         }
+        __syncthreads(); // the next round reuses the LDS
     }
 }
 
@@ -1342,11 +1413,13 @@ static CoarseGrid coarse_grid(const TileGrid &g) {
     return cg;
 }
 
-// Copies of a counter table: a power of two chosen so that the table has about half a
-// million entries, i.e. thousands of cache lines for the atomics to spread over.
+// Copies of a counter table: a power of two chosen so that the table has about a quarter of a
+// million entries, i.e. thousands of cache lines for the atomics to spread over (measured with
+// one atomic per tile and workgroup of the tile binning: half as many copies as before cost
+// nothing there and shorten the scan; a quarter starts to cost).
 static uint32_t isect_copies(uint64_t blocks) {
     uint32_t k = 1;
-    while (k < 256 && (uint64_t)(2 * k) * blocks <= (1ull << 19)) k *= 2;
+    while (k < 256 && (uint64_t)(2 * k) * blocks <= (1ull << 18)) k *= 2;
     return k;
 }
 
