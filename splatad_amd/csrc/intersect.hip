@@ -402,17 +402,22 @@ constexpr uint32_t kSlabShiftMax = 4;
 constexpr uint32_t kSlabSamples = 512;
 // Slabs pay once a tile's segment outgrows the sort's short classes (beyond about 8000 entries,
 // i.e. several hundred Gaussians per tile); below that they only lengthen the binning.  Measured
-// on lidar sweeps of 0.25-4M Gaussians on 1024 tiles and camera frames of 1-4M on 8160 tiles:
-// no slabs win up to 490 Gaussians per tile, 4 win at 980, 8 at 1950, 8-16 at 3900.
+// on lidar sweeps of 0.25-4M Gaussians on 1024 tiles (whole call in ms with 0 / 4 / 8 / 16 slabs:
+// 488 Gaussians per tile 0.255 / 0.267 / 0.266 / 0.281, 732: 0.320 / 0.296 / 0.297 / 0.311,
+// 977: 0.516 / 0.397 / 0.382 / 0.396, 1953: 0.582 / 0.445 / 0.428 / 0.448, 3906: 1.59 / 1.11 /
+// 0.96 / 0.90) and on camera frames: one camera with 1M Gaussians on 8160 tiles (123 per tile)
+// and a rig of six with 2M (245) are fastest without slabs, single frames with 2M and 4M
+// Gaussians would gain 7 % from 4 slabs, which the number of Gaussians per tile does not tell
+// from the rig.
 constexpr uint64_t kSlabMinPerTile = 704;
 
 // Slabs for `total` projected Gaussians on `segs` tiles, from the sizes alone.
 static uint32_t slab_shift_for(uint64_t total, uint64_t segs) {
     const uint64_t per_tile = segs ? total / segs : 0;
     if (per_tile < kSlabMinPerTile) return 0;
-    uint32_t sshift = 0;
-    while (sshift < kSlabShiftMax && (256ull << sshift) <= per_tile) ++sshift;
-    return sshift;
+    if (per_tile < 896) return 2;
+    if (per_tile < 2816) return 3;
+    return kSlabShiftMax;
 }
 
 // Number of bounds at or below the depth bits: non-decreasing in d whatever the bounds hold.
@@ -812,6 +817,9 @@ constexpr uint32_t kSortBucketMean = 8;     // aimed-at entries per bucket
 constexpr uint32_t kSortSplit = 4096;       // buckets at most, beyond the fine bins
 constexpr uint32_t kSortRankMax = 1024;     // largest bucket ordered by rank counting
 constexpr uint32_t kSortWindow = 15360;     // LDS window (entries) when staging is global
+constexpr uint32_t kSortDirectBins = 2048;  // short segments: bins of the direct path at most
+constexpr uint32_t kSortDirectMean = 2;     // entries per bin it aims at
+constexpr uint32_t kSortDirectMax = 64;     // fullest bin it accepts
 
 // Bucket counters a segment of up to max_n entries can need.
 __host__ __device__ inline uint32_t sort_bucket_capacity(uint32_t max_n) {
@@ -1071,8 +1079,15 @@ __device__ __forceinline__ void sort_segment(uint32_t seg, uint32_t n_segments, 
     }
 }
 
-// The same sort for the short segments (n <= lds_words <= 8192, n <= ER * blockDim.x), shaped
-// for the latency of its LDS accesses, which bounds the generic version above:
+// The sort for the short segments (n <= lds_words <= 8192, n <= ER * blockDim.x), shaped for the
+// latency of its LDS accesses, which bounds the generic version above.  Where the depths of a
+// segment are spread evenly enough, one histogram places the entries: bins that are linear in
+// the depth, four entries each on average, and the atomic that counts an entry into its bin
+// returns the entry's place inside the bin; after one scan of the bins every entry is written
+// to its staging position and ranked among the entries of its bin.  A segment with a bin of
+// more than kSortDirectMax entries (clustered depths, a range stretched by outliers), or with
+// depths that are not positive finite floats, takes the equalised buckets of the generic sort
+// instead (a second histogram, scan and scatter).  Both ways:
 //  * an entry's bucket is computed once, kept in a register for the scatter, and written as
 //    16 bits beside the entry's staging position for the rank step;
 //  * the rank loop takes four staged entries per trip with no bounds test: what follows a
@@ -1101,6 +1116,8 @@ __device__ __forceinline__ void sort_segment_small(uint32_t seg, uint32_t n_segm
     const int64_t start = tile_starts[seg];
     const int64_t stop = min(seg + 1 == n_segments ? n_isects : (int64_t)tile_starts[seg + 1], n_isects);
     const uint32_t n = stop > start ? (uint32_t)(stop - start) : 0u; // as classified
+    // (the direct path's bins and the end marker behind them take the words from s_fine on,
+    // across the bucket tables it does not use: see launch_small_segment_sort)
     uint32_t *s_fine = reinterpret_cast<uint32_t *>(lds_staged + lds_words + 4);
     uint32_t *s_first = s_fine + kSortFineBins;   // bucket_cap + 1 words: starts, then the end
     uint32_t *s_cursor = s_first + bucket_cap + 1;
@@ -1136,21 +1153,95 @@ __device__ __forceinline__ void sort_segment_small(uint32_t seg, uint32_t n_segm
     if (lane == 0) { s_wave[2 * wave] = lo; s_wave[2 * wave + 1] = hi; }
     if (tid == 0) s_big = 0;
     if (tid < 4) lds_staged[n + tid] = ~0ull;
-    uint32_t n_fine = 1;
-    while (n_fine < kSortFineBins && n_fine * 16 < n) n_fine <<= 1;
-    for (uint32_t f = tid; f < n_fine; f += nt) s_fine[f] = 0;
+    // Ranks the staged entries inside their buckets (first[b] .. first[b + 1]) and writes the lists.
+    auto rank_and_write = [&](const uint32_t *first) {
+        for (uint32_t i = tid; i < n; i += nt) {
+            const uint64_t p = lds_staged[i];
+            const uint32_t b = s_bucket[i];
+            const uint32_t s0 = first[b], s1 = first[b + 1];
+            uint32_t place = s0;
+            if (s1 - s0 > kSortRankMax) {
+                place = i; // ordered by the network
+            } else {
+                for (uint32_t j = s0; j < s1; j += 4) {
+                    const uint64_t q0 = lds_staged[j], q1 = lds_staged[j + 1];
+                    const uint64_t q2 = lds_staged[j + 2], q3 = lds_staged[j + 3];
+                    if (TIES) {
+                        place += (q0 < p || (q0 == p && j < i)) ? 1u : 0u;
+                        place += (q1 < p || (q1 == p && j + 1 < i)) ? 1u : 0u;
+                        place += (q2 < p || (q2 == p && j + 2 < i)) ? 1u : 0u;
+                        place += (q3 < p || (q3 == p && j + 3 < i)) ? 1u : 0u;
+                    } else {
+                        place += (q0 < p ? 1u : 0u) + (q1 < p ? 1u : 0u) + (q2 < p ? 1u : 0u) + (q3 < p ? 1u : 0u);
+                    }
+                }
+            }
+            ids_out[place] = (int64_t)(key_hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
+            flat_out[place] = (int32_t)(uint32_t)p;
+        }
+    };
+
+    // Direct path: bins of kSortDirectMean entries on average, linear in the depth; the atomic
+    // that counts an entry into its bin also tells the entry's place inside the bin, so one
+    // histogram and one scan place every entry.  Taken when no bin holds more than
+    // kSortDirectMax entries; segments whose depths cluster take the equalised buckets below.
+    uint32_t n_bins = 1;
+    while (n_bins < kSortDirectBins && n_bins * kSortDirectMean < n) n_bins <<= 1;
+    for (uint32_t f = tid; f < n_bins; f += nt) s_fine[f] = 0;
     __syncthreads();
     for (uint32_t w = 0; w < n_waves; ++w) {
         lo = min(lo, s_wave[2 * w]);
         hi = max(hi, s_wave[2 * w + 1]);
     }
+    __syncthreads(); // s_wave is reused by the scans
+    if (hi < 0x7F800000u) { // uniform; depths that are positive finite floats: bins linear in the depth
+        const float lo_depth = __uint_as_float(lo), range = __uint_as_float(hi) - lo_depth;
+        const float bin_scale = range > 0.f ? (float)n_bins / range : 0.f;
+        uint32_t where[ER]; // bin, and above it the place inside the bin
+#pragma unroll
+        for (int k = 0; k < ER; ++k) {
+            where[k] = 0;
+            if (tid + k * nt < n) {
+                const float x = (__uint_as_float((uint32_t)(held[k] >> 32)) - lo_depth) * bin_scale;
+                const uint32_t f = min(n_bins - 1, (uint32_t)x);
+                where[k] = f | (atomicAdd(&s_fine[f], 1u) << 16);
+            }
+        }
+        __syncthreads();
+        block_exclusive_scan(
+            n_bins, tid, nt, s_wave, [&](uint32_t f) { return s_fine[f]; },
+            [&](uint32_t f, uint32_t before, uint32_t v) {
+                s_fine[f] = before;
+                if (v > kSortDirectMax) s_big = 2;
+            });
+        if (s_big != 2) { // uniform
+            if (tid == 0) s_fine[n_bins] = n;
+#pragma unroll
+            for (int k = 0; k < ER; ++k)
+                if (tid + k * nt < n) {
+                    const uint32_t f = where[k] & 0xFFFFu;
+                    const uint32_t at = s_fine[f] + (where[k] >> 16);
+                    lds_staged[at] = held[k];
+                    s_bucket[at] = (uint16_t)f;
+                }
+            __syncthreads();
+            rank_and_write(s_fine);
+            return;
+        }
+        __syncthreads(); // every lane has read the flag
+        if (tid == 0) s_big = 0;
+    }
+
+    uint32_t n_fine = 1;
+    while (n_fine < kSortFineBins && n_fine * 16 < n) n_fine <<= 1;
+    for (uint32_t f = tid; f < n_fine; f += nt) s_fine[f] = 0;
     const float scale = (float)n_fine / ((float)(hi - lo) + 1.f);
     auto fine_pos = [&](uint64_t p, uint32_t &f) -> float {
         const float x = (float)((uint32_t)(p >> 32) - lo) * scale;
         f = min(n_fine - 1, (uint32_t)x);
         return x;
     };
-    __syncthreads(); // s_wave is reused by the scans
+    __syncthreads();
 
 #pragma unroll
     for (int k = 0; k < ER; ++k)
@@ -1205,31 +1296,7 @@ __device__ __forceinline__ void sort_segment_small(uint32_t seg, uint32_t n_segm
             if (c > kSortRankMax) bitonic_sort_ascending(lds_staged + s0, c, tid, nt); // uniform
         }
     }
-
-    for (uint32_t i = tid; i < n; i += nt) {
-        const uint64_t p = lds_staged[i];
-        const uint32_t b = s_bucket[i];
-        const uint32_t s0 = s_first[b], s1 = s_first[b + 1];
-        uint32_t place = s0;
-        if (s1 - s0 > kSortRankMax) {
-            place = i; // ordered by the network above
-        } else {
-            for (uint32_t j = s0; j < s1; j += 4) {
-                const uint64_t q0 = lds_staged[j], q1 = lds_staged[j + 1];
-                const uint64_t q2 = lds_staged[j + 2], q3 = lds_staged[j + 3];
-                if (TIES) {
-                    place += (q0 < p || (q0 == p && j < i)) ? 1u : 0u;
-                    place += (q1 < p || (q1 == p && j + 1 < i)) ? 1u : 0u;
-                    place += (q2 < p || (q2 == p && j + 2 < i)) ? 1u : 0u;
-                    place += (q3 < p || (q3 == p && j + 3 < i)) ? 1u : 0u;
-                } else {
-                    place += (q0 < p ? 1u : 0u) + (q1 < p ? 1u : 0u) + (q2 < p ? 1u : 0u) + (q3 < p ? 1u : 0u);
-                }
-            }
-        }
-        ids_out[place] = (int64_t)(key_hi | (uint64_t)(int64_t)(int32_t)(p >> 32));
-        flat_out[place] = (int32_t)(uint32_t)p;
-    }
+    rank_and_write(s_first);
 }
 
 
@@ -1332,8 +1399,14 @@ static int launch_small_segment_sort(int cls, uint32_t threads, uint32_t max_n, 
                                      const uint32_t *seg_lists, const int32_t *tile_starts,
                                      const uint64_t *pairs, int64_t *isect_ids, int32_t *flatten_ids,
                                      hipStream_t stream) {
-    SPLATAD_REQUIRE((uint64_t)ER * threads >= max_n && max_n <= 8192u, "segment sort: class %d does not fit", cls);
+    SPLATAD_REQUIRE((uint64_t)ER * threads >= max_n && max_n <= 8192u && (max_n & (max_n - 1)) == 0,
+                    "segment sort: class %d does not fit", cls);
     const uint32_t bucket_cap = sort_bucket_capacity(max_n);
+    {   // the bins of the direct path: a power of two, at most max_n / kSortDirectMean of them
+        const uint32_t bins = max_n / kSortDirectMean < kSortDirectBins ? max_n / kSortDirectMean : kSortDirectBins;
+        SPLATAD_REQUIRE(bins + 1 <= kSortFineBins + 2 * bucket_cap + 1 && bins <= 65536u,
+                        "segment sort: no room for the %u bins of class %d", bins, cls);
+    }
     const size_t lds_bytes = sort_small_lds_bytes(max_n, bucket_cap);
     {   // raise the kernel's dynamic LDS limit once per instantiation and size
         static std::mutex guard;

@@ -325,6 +325,31 @@ def test_isect_sort_long_segments_and_depth_ties(n, tie_frac):
     np.testing.assert_array_equal(to_np(flat), o_flat)
 
 
+@pytest.mark.parametrize("n,spread", [(300, "even"), (1800, "even"), (1800, "far"), (7000, "even"),
+                                      (1800, "infinite"), (5000, "infinite")])
+def test_isect_sort_of_short_segments_by_depth_spread(n, spread):
+    # The short-segment sort places entries by bins that are linear in the depth when no bin gets
+    # too full, and by equalised buckets otherwise: depths spread evenly over their range take
+    # the first way, a range stretched by a few far depths the second, and depths that are not
+    # finite floats (their bit patterns still order the keys, rasterization.cu:77-84) are
+    # never binned by value.
+    from splatad_amd import isect_tiles
+    rng = np.random.default_rng(n + len(spread))
+    means2d = rng.uniform(10, 22, (1, n, 2)).astype(np.float32)
+    radii = np.full((1, n, 2), 40, np.int32)
+    depths = rng.uniform(0.5, 90.0, (1, n)).astype(np.float32)
+    if spread == "far":
+        depths[0, : n // 100] = rng.uniform(1e6, 1e9, n // 100)
+    elif spread == "infinite":
+        depths[0, rng.random(n) < 0.05] = np.inf
+    tpg, ids, flat = isect_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), 16, 2, 2)
+    o_tpg, o_ids, o_flat = oracle.isect_tiles(means2d, radii, depths, 16, 2, 2)
+    assert o_ids.shape[0] == 4 * n
+    np.testing.assert_array_equal(to_np(tpg), o_tpg)
+    np.testing.assert_array_equal(to_np(ids), o_ids)
+    np.testing.assert_array_equal(to_np(flat), o_flat)
+
+
 def test_isect_lidar_reference_recipe_and_wrap():
     # input recipe of the reference's test_isect_lidar (tests/test_basic.py:733-751)
     from splatad_amd import isect_lidar_tiles, isect_offset_encode
