@@ -7,7 +7,8 @@ A step is one complete forward call of `rasterization()` (projection + SH + tile
 SH degree 3, rolling shutter, RGB+D.  All inputs are resident in HBM before the timed region.
 The same is done for `lidar_rasterization()` on the 128x2048 lidar sweep and reported in the
 "lidar" object of the same JSON line.  "roofline" describes the dominant kernel
-(rasterize_to_pixels forward), timed with events on the launch stream; "cpu_baseline" times the
+(rasterize_to_pixels forward, which in a forward-only call also evaluates the colours of the
+Gaussians it composites), timed with events on the launch stream; "cpu_baseline" times the
 CPU oracle (a C restatement of the reference's algorithm, OpenMP) on the host cores.
 """
 import argparse
@@ -137,7 +138,16 @@ def bench_camera(args):
                 meta["means2d"], meta["conics"], cols, meta["opacities"], meta["pix_vels"],
                 s["rolling_shutter_time"], None, W, H, ts, meta["isect_offsets"], meta["flatten_ids"])
 
-        k_ms = time_kernel(raster, iters=max(5, args.steps))
+        def raster_sh():
+            # what the step runs: the same kernel evaluating the colours of the entries it stages
+            return _C.rasterize_to_pixels_sh_fwd(
+                3, s["means"], s["viewmats"], s["colors"], None, meta["depths"], meta["means2d"],
+                meta["conics"], meta["opacities"], meta["pix_vels"], s["rolling_shutter_time"], None,
+                W, H, ts, meta["isect_offsets"], meta["flatten_ids"])
+
+        assert torch.equal(raster_sh()[0], raster()[0]) and torch.equal(raster_sh()[0], rc)
+        k_ms = time_kernel(raster_sh, iters=max(5, args.steps))
+        k_plain_ms = time_kernel(raster, iters=max(5, args.steps))
         n_isects = int(meta["flatten_ids"].shape[0])
         batches = torch.zeros_like(meta["isect_offsets"])
         _C.rasterize_to_pixels_fwd(
@@ -153,7 +163,17 @@ def bench_camera(args):
         tile_cycles = cycle_spread(cycles)
         D = cols.shape[-1]
         P, T = C * H * W, meta["isect_offsets"].numel()
-        alg_bytes = i_need * (36 + 4 * D) + P * (4 * D + 8) + T * 4
+        N, K = s["means"].shape[0], s["colors"].shape[-2]
+        # rows (camera, Gaussian) among the staged entries: each one's mean and coefficients
+        # have to be read at least once
+        first = meta["isect_offsets"].flatten().long()
+        marks = torch.zeros(n_isects + 1, dtype=torch.int32, device=dev)
+        marks.index_add_(0, first, torch.ones_like(first, dtype=torch.int32))
+        marks.index_add_(0, first + batches.flatten().long(), -torch.ones_like(first, dtype=torch.int32))
+        staged = torch.cumsum(marks[:-1], 0) > 0
+        rows_staged = int(torch.unique(meta["flatten_ids"][staged]).numel())
+        plain_bytes = i_need * (36 + 4 * D) + P * (4 * D + 8) + T * 4
+        alg_bytes = i_need * (36 + 4 * (D - 3)) + rows_staged * (12 + 12 * K) + P * (4 * D + 8) + T * 4
         # per-stage times of the same call
         stages = {}
         proj = lambda: _C.fully_fused_projection_fwd(
@@ -172,8 +192,8 @@ def bench_camera(args):
             lambda: _C.view_colors_fwd(3, s["means"], s["viewmats"], None, None, meta["radii"],
                                        s["colors"], meta["depths"]), 5)
         stages["rasterize_ms"] = k_ms
+        stages["rasterize_given_colors_ms"] = k_plain_ms
         nnz = int((meta["radii"][..., 0] > 0).sum().item())
-        N, K = s["means"].shape[0], s["colors"].shape[-2]
         stage_bytes = {
             "projection_ms": N * 52 + C * N * 40,
             # what any implementation has to move: read the projected (mean, radii, depth) rows, write
@@ -182,6 +202,7 @@ def bench_camera(args):
             "offset_encode_ms": n_isects * 8 + T * 4,
             "view_colors_ms": nnz * (12 + 12 * K + 1 + 12),
             "rasterize_ms": alg_bytes,
+            "rasterize_given_colors_ms": plain_bytes,
         }
         st = _C.rasterize_to_pixels_lane_stats(
             meta["means2d"], meta["conics"], meta["opacities"], meta["pix_vels"], s["rolling_shutter_time"], W, H,
@@ -191,7 +212,8 @@ def bench_camera(args):
                      footprint_test_pass_fraction=st[5] / max(1, st[4]),
                      iterations_without_a_compositing_lane=st[3] / max(1, st[0]))
     return dict(sec=sec, sec_packed=sec_packed, pixels=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
-                n_isects=n_isects, i_need=i_need, nnz=nnz, stages=stages, stage_bytes=stage_bytes,
+                n_isects=n_isects, i_need=i_need, rows_staged=rows_staged, nnz=nnz, stages=stages,
+                stage_bytes=stage_bytes,
                 channels=D, lanes=lanes, tile_cycles=tile_cycles)
 
 
@@ -468,11 +490,15 @@ def main():
         },
         "stages": stage_rooflines(cam),
         "roofline": {
-            "kernel": "rasterize_to_pixels_fwd_kernel<%d, 2, false>" % cam["channels"],
+            # the compositing kernel that evaluates the spherical-harmonic colours of the entries
+            # it stages: the entries' geometry and depth, the mean and coefficient row of every
+            # (camera, Gaussian) among them once, the image
+            "kernel": "rasterize_to_pixels_fwd_kernel<%d, 2, false, true>" % cam["channels"],
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": MEASURED_TRAFFIC_BYTES["camera"] if args.n == 1_000_000 else None,
             "algorithmic_bytes": cam["alg_bytes"], "kernel_ms": cam["kernel_ms"],
+            "rows_staged": cam["rows_staged"],
         },
     }
     if lid is not None:

@@ -364,6 +364,35 @@ int splatad_rasterize_to_pixels_fwd(uint32_t C, int64_t n_isects, uint32_t chann
                                     int32_t *last_ids, int32_t *tile_batches,
                                     int64_t *tile_cycles, splatad_stream_t stream);
 
+/* Steps 3 and 5 of rasterization() in one kernel (gsplat/rendering.py:325-347 and 362-391 of
+ * the reference: view directions, spherical harmonics, max(c + 1/2, 0), then
+ * rasterize_to_pixels): the compositing kernel evaluates the colour of every list entry it
+ * stages from `coeffs` ([N, K, 3], or [C, N, K, 3] with coeffs_per_sensor != 0), `means` [N, 3]
+ * and the sensor positions in `viewmats` [C, 4, 4], with the instructions of
+ * splatad_view_colors_fwd, so the images equal those of the two calls bit for bit.  It reads
+ * the coefficients of the entries that tiles reach before they saturate instead of those of
+ * every visible Gaussian, beside arithmetic that leaves the memory idle.  Rows (what
+ * flatten_ids index: means2d, conics, opacities, pix_vels, depths) are dense [C, N] with
+ * gaussian_ids == NULL, or packed [nnz] with gaussian_ids [nnz] naming each row's Gaussian (the
+ * camera of a row is that of the tile that lists it).  Renders 3 channels, or 4 with `depths`
+ * (not NULL) as the last one.  color_cache: 16 bytes per row, every float a NaN before the call
+ * (the workgroups that first stage a row leave its colour there for the tiles that list the
+ * Gaussian later, so a row is evaluated a few times at most however much of the lists is
+ * consumed); what it holds afterwards is of no use to the caller.  Forward only. */
+int splatad_rasterize_to_pixels_fwd_sh(uint32_t C, uint32_t N, int64_t n_isects, uint32_t K,
+                                       uint32_t degree, const float *means, const float *viewmats,
+                                       const float *coeffs, int coeffs_per_sensor,
+                                       const int64_t *gaussian_ids, const float *depths,
+                                       float *color_cache, const float *means2d,
+                                       const float *conics, const float *opacities,
+                                       const float *pix_vels, const float *rolling_shutter_time,
+                                       const float *backgrounds, uint32_t image_width,
+                                       uint32_t image_height, uint32_t tile_size,
+                                       uint32_t tile_width, uint32_t tile_height,
+                                       const int32_t *tile_offsets, const int32_t *flatten_ids,
+                                       float *render_colors, float *render_alphas,
+                                       int32_t *last_ids, splatad_stream_t stream);
+
 /* Diagnostic without a counterpart in the reference: lane utilisation of the compositing loop
  * of splatad_rasterize_to_pixels_fwd on the same inputs (nothing is rendered).  Adds to eight
  * counters in stats (zero them first): [0] (wavefront, Gaussian) iterations of the inner loop,

@@ -20,6 +20,7 @@
 // channel count, stride and offset at run time, so any channel count is rendered without
 // host-side padding (wide inputs in passes of up to 32 channels).
 #include "raster_common.h"
+#include "sh_eval.h"
 
 #include <type_traits>
 
@@ -40,6 +41,17 @@ struct PixelArgs {
     int32_t *tile_batches; // optional diagnostic: list entries each tile's workgroup staged
     int64_t *tile_cycles;  // optional diagnostic: shader clock cycles each tile's workgroup ran for
     unsigned long long *lane_stats; // STATS kernels only: kLaneStats counters, see the entry point
+    // SHC kernels: channels 0-2 are the view-dependent colours of the Gaussians, evaluated from
+    // their spherical-harmonic coefficients for the entries a tile stages (`colors` is unused);
+    // channel 3, if rendered, is sh_depths[id].  Dense rows [C, N]: id = camera * sh_N + Gaussian;
+    // packed rows: sh_gaussian_ids[id] (not null) is the Gaussian.
+    // sh_cache: a float4 per row, NaN before the launch; the first workgroups to stage a row
+    // leave its colour there for the later ones.
+    const float *sh_means, *sh_viewmats, *sh_coeffs, *sh_depths;
+    const int64_t *sh_gaussian_ids;
+    float *sh_cache;
+    uint32_t sh_N, sh_K, sh_degree;
+    int sh_per_sensor; // coefficient rows: 1 = one per (camera, Gaussian), 0 = one per Gaussian
 };
 
 constexpr int kLaneStats = 8;
@@ -57,7 +69,7 @@ constexpr int kLaneStats = 8;
 // Every wavefront then tests 64 staged Gaussians at a time against its footprint, copies the
 // survivors' records in list order into a private strip of LDS (its own writes and reads: no
 // barrier) and walks that strip: sequential addresses, no lane-mask bookkeeping per Gaussian.
-template <int CH, int PPL, bool STATS = false>
+template <int CH, int PPL, bool STATS = false, bool SHC = false>
 __global__ void __launch_bounds__(1024)
 rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     const long long t_begin = a.tile_cycles != nullptr ? clock64() : 0;
@@ -70,8 +82,9 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     float4 *s_rec = lds4;
 
     const uint32_t tiles_per_cam = a.tile_w * a.tile_h;
-    const uint32_t cam = blockIdx.x / tiles_per_cam;
-    const uint32_t tile_id = blockIdx.x % tiles_per_cam;
+    const uint32_t unit = blockIdx.x;
+    const uint32_t cam = unit / tiles_per_cam;
+    const uint32_t tile_id = unit % tiles_per_cam;
     const uint32_t tile_y = tile_id / a.tile_w, tile_x = tile_id % a.tile_w;
     const uint32_t tr = threadIdx.x;
     const uint32_t lane = tr & (SPLATAD_WAVE - 1), wave = tr / SPLATAD_WAVE;
@@ -204,6 +217,8 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     // workgroups of the compute unit.  (Requesting the next batch before compositing the current
     // one costs 15 registers, one resident wavefront per SIMD with them, and was slower.)
     struct Staged { float2 xy, vel; float cn[3], opac, col[CH]; };
+    float sensor_x = 0.f, sensor_y = 0.f, sensor_z = 0.f;
+    if (SHC) sensor_position(a.sh_viewmats + (size_t)cam * 16, sensor_x, sensor_y, sensor_z);
     auto id_of = [&](uint32_t b) -> int32_t {
         const uint32_t idx = min((uint32_t)range_start + batch * b + tr, (uint32_t)range_end - 1u);
         return b < num_batches ? a.flatten_ids[idx] : 0;
@@ -215,10 +230,52 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
         const float *c3 = a.conics + (size_t)g * 3;
         s.cn[0] = c3[0]; s.cn[1] = c3[1]; s.cn[2] = c3[2];
         s.opac = a.opacities[g];
+        if (SHC) return s; // the colours are staged by stage_sh_color
         const float *c = a.colors + (size_t)g * a.color_stride + a.ch_offset;
 #pragma unroll
         for (int k = 0; k < CH; ++k) s.col[k] = STATS ? 0.f : c[min((uint32_t)k, a.n_ch - 1u)]; // STATS: no colours
         return s;
+    };
+    // SHC: the colour of row g, what sh_fwd_kernel<true> writes for it, by the same instructions;
+    // staged before the rest of the Gaussian is requested, so that the coefficients of a band
+    // and the Gaussian's other values are not in registers at the same time.
+    // A row's colour is evaluated by the first workgroups that stage it and left in sh_cache for
+    // the others (a Gaussian is listed by every tile it touches).  Word-wise relaxed accesses
+    // with no wider scope than the workgroup, i.e. ordinary cached loads and stores: another
+    // workgroup sees each word either as the NaN the cache was filled with -- then it evaluates
+    // the colour itself, to the same value -- or as the colour; how soon it sees the colour is
+    // left to the caches (the dies' L2 caches do not see one another's lines before the kernel
+    // ends, so each die evaluates the rows its tiles stage).  Loads or stores of device scope,
+    // which would share the colours between the dies, go to memory every time and made the
+    // kernel three to four times slower.
+    auto stage_sh_color = [&](int32_t g) {
+        float *cached = a.sh_cache + (size_t)g * 4;
+        float cr = __hip_atomic_load(cached, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        float cg = __hip_atomic_load(cached + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        float cb = __hip_atomic_load(cached + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        const bool missing = !(cr == cr) || !(cg == cg) || !(cb == cb);
+        if (wave_ballot(missing) != 0) { // uniform
+            if (missing) {
+                const uint32_t gauss =
+                    a.sh_gaussian_ids ? (uint32_t)a.sh_gaussian_ids[g] : (uint32_t)g - cam * a.sh_N;
+                const float *m = a.sh_means + (size_t)gauss * 3;
+                const float dx = m[0] - sensor_x, dy = m[1] - sensor_y, dz = m[2] - sensor_z;
+                const size_t row = a.sh_per_sensor ? (size_t)cam * a.sh_N + gauss : (size_t)gauss;
+                float r = 0.f, gr = 0.f, bl = 0.f;
+                sh_color_by_band(a.sh_degree, a.sh_coeffs + row * a.sh_K * 3, dx, dy, dz, r, gr, bl);
+                cr = fmaxf(r + 0.5f, 0.f);
+                cg = fmaxf(gr + 0.5f, 0.f);
+                cb = fmaxf(bl + 0.5f, 0.f);
+                __hip_atomic_store(cached, cr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_store(cached + 1, cg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_store(cached + 2, cb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
+        float *col = reinterpret_cast<float *>(s_rec + RECORD * tr + 2);
+        col[0] = cr;
+        col[1 % CH] = cg;
+        col[2 % CH] = cb;
+        if (CH > 3) col[3 % CH] = a.sh_depths[g];
     };
     uint32_t batches_done = 0;
     for (uint32_t b = 0; b < num_batches; ++b) {
@@ -231,15 +288,19 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
 
         const uint32_t batch_start = (uint32_t)range_start + batch * b;
         {
-            const Staged staged = gather(id_of(b));
+            const int32_t g = id_of(b);
+            if (SHC) stage_sh_color(g);
+            const Staged staged = gather(g);
             float4 pa, pb;
             pixel_polynomial(frame, staged.xy, staged.vel, staged.cn[0], staged.cn[1], staged.cn[2], staged.opac,
                              pa, pb);
             s_rec[RECORD * tr] = pa;
             s_rec[RECORD * tr + 1] = pb;
+            if (!SHC) {
 #pragma unroll
-            for (int k = 0; k < CH; ++k)
-                reinterpret_cast<float *>(s_rec + RECORD * tr + 2)[k] = (uint32_t)k < a.n_ch ? staged.col[k] : 0.f;
+                for (int k = 0; k < CH; ++k)
+                    reinterpret_cast<float *>(s_rec + RECORD * tr + 2)[k] = (uint32_t)k < a.n_ch ? staged.col[k] : 0.f;
+            }
         }
         __syncthreads();
 
@@ -289,8 +350,8 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     }
 
     if (a.tile_batches != nullptr && a.write_aux && tr == 0)
-        a.tile_batches[blockIdx.x] = (int32_t)min(batches_done * batch, (uint32_t)(range_end - range_start));
-    if (a.tile_cycles != nullptr && a.write_aux && tr == 0) a.tile_cycles[blockIdx.x] = clock64() - t_begin;
+        a.tile_batches[unit] = (int32_t)min(batches_done * batch, (uint32_t)(range_end - range_start));
+    if (a.tile_cycles != nullptr && a.write_aux && tr == 0) a.tile_cycles[unit] = clock64() - t_begin;
     if (STATS) {
         if (lane == 0) {
             const uint32_t v[kLaneStats] = {st_iter, st_take, st_alive, st_idle, st_tested, st_kept, 0u, st_valid};
@@ -670,15 +731,23 @@ static size_t pixel_lds_bytes(uint32_t threads) {
     return 16 * ((size_t)threads * (2 + (CH + 3) / 4) + waves * SPLATAD_WAVE * (CH <= 4 ? 3 : 2));
 }
 
-template <int CH, int PPL, bool STATS>
+template <int CH, int PPL, bool STATS, bool SHC = false>
 static int launch_pixels_as(const PixelArgs &a, dim3 grid, uint32_t threads, hipStream_t stream) {
     const size_t lds = pixel_lds_bytes<CH>(threads);
     if (lds > 64 * 1024)
-        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_to_pixels_fwd_kernel<CH, PPL, STATS>,
+        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_to_pixels_fwd_kernel<CH, PPL, STATS, SHC>,
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL((rasterize_to_pixels_fwd_kernel<CH, PPL, STATS>), grid, dim3(threads), lds, stream, a);
+    hipLaunchKernelGGL((rasterize_to_pixels_fwd_kernel<CH, PPL, STATS, SHC>), grid, dim3(threads), lds, stream, a);
     SPLATAD_LAUNCH_CHECK();
     return 0;
+}
+
+// Colours from spherical harmonics: three or four channels in one pass.
+template <int CH>
+static int launch_pixels_sh(const PixelArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
+    const uint32_t pixels = block.x * block.y;
+    if (pixels_per_lane(a.tile_size) == 2) return launch_pixels_as<CH, 2, false, true>(a, grid, pixels / 2, stream);
+    return launch_pixels_as<CH, 1, false, true>(a, grid, pixels, stream);
 }
 
 template <int CH>
@@ -779,6 +848,46 @@ extern "C" int splatad_rasterize_to_pixels_fwd(
         if (rc) return rc;
     }
     return 0;
+}
+
+extern "C" int splatad_rasterize_to_pixels_fwd_sh(
+    uint32_t C, uint32_t N, int64_t n_isects, uint32_t K, uint32_t degree, const float *means,
+    const float *viewmats, const float *coeffs, int coeffs_per_sensor,
+    const int64_t *gaussian_ids, const float *depths, float *color_cache,
+    const float *means2d, const float *conics, const float *opacities, const float *pix_vels,
+    const float *rs_time, const float *backgrounds, uint32_t W, uint32_t H, uint32_t tile_size,
+    uint32_t tile_w, uint32_t tile_h, const int32_t *tile_offsets, const int32_t *flatten_ids,
+    float *render_colors, float *render_alphas, int32_t *last_ids, splatad_stream_t stream) {
+    SPLATAD_REQUIRE(degree <= 4 && K >= (degree + 1) * (degree + 1),
+                    "rasterize_to_pixels: %u coefficients do not hold degree %u", K, degree);
+    SPLATAD_REQUIRE(tile_size >= 1 && tile_size * tile_size <= 1024,
+                    "rasterize_to_pixels: tile_size %u is outside 1..32", tile_size);
+    if (C == 0 || W == 0 || H == 0) return 0;
+    SPLATAD_REQUIRE((uint64_t)tile_w * tile_size >= W && (uint64_t)tile_h * tile_size >= H,
+                    "rasterize_to_pixels: tile grid %ux%u of size %u does not cover %ux%u", tile_w,
+                    tile_h, tile_size, W, H);
+    SPLATAD_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31), "rasterize_to_pixels: bad n_isects");
+    SPLATAD_REQUIRE((uint64_t)C * N < (1ull << 31), "rasterize_to_pixels: %u x %u rows exceed the id range", C, N);
+    SPLATAD_REQUIRE(rs_time && viewmats && tile_offsets && render_colors && render_alphas && last_ids,
+                    "rasterize_to_pixels: null pointer argument");
+    SPLATAD_REQUIRE(n_isects == 0 || (means && coeffs && color_cache && means2d && conics && opacities &&
+                                      pix_vels && flatten_ids),
+                    "rasterize_to_pixels: null pointer argument");
+    PixelArgs a = {};
+    a.C = C; a.n_isects = n_isects;
+    a.color_stride = depths != nullptr ? 4u : 3u;
+    a.ch_offset = 0; a.n_ch = a.color_stride; a.write_aux = 1;
+    a.means2d = means2d; a.conics = conics; a.opacities = opacities;
+    a.pix_vels = pix_vels; a.rs_time = rs_time; a.backgrounds = backgrounds;
+    a.W = W; a.H = H; a.tile_size = tile_size; a.tile_w = tile_w; a.tile_h = tile_h;
+    a.tile_offsets = tile_offsets; a.flatten_ids = flatten_ids;
+    a.render_colors = render_colors; a.render_alphas = render_alphas; a.last_ids = last_ids;
+    a.sh_means = means; a.sh_viewmats = viewmats; a.sh_coeffs = coeffs; a.sh_depths = depths;
+    a.sh_gaussian_ids = gaussian_ids; a.sh_cache = color_cache;
+    a.sh_N = N; a.sh_K = K; a.sh_degree = degree; a.sh_per_sensor = coeffs_per_sensor;
+    const dim3 grid(C * tile_w * tile_h), block(tile_size, tile_size);
+    if (depths != nullptr) return launch_pixels_sh<4>(a, grid, block, (hipStream_t)stream);
+    return launch_pixels_sh<3>(a, grid, block, (hipStream_t)stream);
 }
 
 extern "C" int splatad_rasterize_to_pixels_lane_stats(

@@ -24,7 +24,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libsplatad_hip.so")
 _lib = None
 
 
-ABI_VERSION = 5  # splatad_abi_version() of the library these bindings were written for
+ABI_VERSION = 6  # splatad_abi_version() of the library these bindings were written for
 
 
 def load_library():
@@ -843,6 +843,45 @@ class _Ops:
                 _p(flatten_ids), _p(renders), _p(alphas), _p(last_ids),
                 _p(_in(tile_batches, "tile_batches", torch.int32)),
                 _p(_in(tile_cycles, "tile_cycles", torch.int64)), _stream(dev)))
+        return renders, alphas, last_ids
+
+    def rasterize_to_pixels_sh_fwd(self, sh_degree, means, viewmats, coeffs, gaussian_ids, depths,
+                                   means2d, conics, opacities, pix_vels, rolling_shutter_time,
+                                   backgrounds, image_width, image_height, tile_size, tile_offsets,
+                                   flatten_ids):
+        """rasterize_to_pixels_fwd for rows whose colours are the view-dependent colours of
+        `coeffs` ([N, K, 3] or [C, N, K, 3]): the kernel evaluates them for the entries it
+        stages.  Rows are dense [C, N], or packed [nnz] with gaussian_ids [nnz]; depths, if
+        given, is rendered as a fourth channel."""
+        lib = load_library()
+        means = _in(means, "means"); viewmats = _in(viewmats, "viewmats"); coeffs = _in(coeffs, "coeffs")
+        depths = _in(depths, "depths"); gaussian_ids = _in(gaussian_ids, "gaussian_ids", torch.int64)
+        means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
+        opacities = _in(opacities, "opacities")
+        pix_vels = _in(pix_vels, "pix_vels"); rs = _in(rolling_shutter_time, "rolling_shutter_time")
+        backgrounds = _in(backgrounds, "backgrounds")
+        tile_offsets = _in(tile_offsets, "tile_offsets", torch.int32)
+        flatten_ids = _in(flatten_ids, "flatten_ids", torch.int32)
+        C, th, tw = tile_offsets.shape
+        N, dev = means.shape[0], means2d.device
+        rows = (C, N) if gaussian_ids is None else tuple(gaussian_ids.shape)
+        assert means2d.shape == rows + (2,) and coeffs.shape[-1] == 3, (means2d.shape, coeffs.shape)
+        assert coeffs.shape[:-2] in ((N,), (C, N)), coeffs.shape
+        D = 3 if depths is None else 4
+        f = dict(dtype=torch.float32, device=dev)
+        renders = torch.empty((C, image_height, image_width, D), **f)
+        alphas = torch.empty((C, image_height, image_width, 1), **f)
+        last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
+        # colours of the rows that tiles stage, left by the first for the others; NaN = not yet
+        cache = torch.full(rows + (4,), float("nan"), **f)
+        with _on(dev):
+            _check(lib.splatad_rasterize_to_pixels_fwd_sh(
+                _u32(C), _u32(N), _i64(flatten_ids.shape[0]), _u32(coeffs.shape[-2]), _u32(sh_degree),
+                _p(means), _p(viewmats), _p(coeffs), _i32(coeffs.dim() == 4), _p(gaussian_ids),
+                _p(depths), _p(cache), _p(means2d),
+                _p(conics), _p(opacities), _p(pix_vels), _p(rs), _p(backgrounds), _u32(image_width),
+                _u32(image_height), _u32(tile_size), _u32(tw), _u32(th), _p(tile_offsets),
+                _p(flatten_ids), _p(renders), _p(alphas), _p(last_ids), _stream(dev)))
         return renders, alphas, last_ids
 
     def rasterize_to_pixels_lane_stats(self, means2d, conics, opacities, pix_vels, rolling_shutter_time,

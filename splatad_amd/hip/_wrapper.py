@@ -434,6 +434,67 @@ def rasterize_to_pixels(
     )
 
 
+def rasterize_to_pixels_with_sh(
+    sh_degree: int,
+    means: Tensor,  # [N, 3]
+    viewmats: Tensor,  # [C, 4, 4]
+    sh_coeffs: Tensor,  # [N, K, 3] or [C, N, K, 3]
+    depths: Optional[Tensor],  # [C, N] or [nnz]: rendered as a fourth channel
+    means2d: Tensor,  # [C, N, 2] or [nnz, 2]
+    conics: Tensor,  # [C, N, 3] or [nnz, 3]
+    opacities: Tensor,  # [C, N] or [nnz]
+    pix_vels: Tensor,  # [C, N, 2] or [nnz, 2]
+    image_width: int,
+    image_height: int,
+    tile_size: int,
+    isect_offsets: Tensor,  # [C, tile_height, tile_width]
+    flatten_ids: Tensor,  # [n_isects]
+    rolling_shutter_time: Optional[Tensor] = None,  # [C]
+    backgrounds: Optional[Tensor] = None,  # [C, 3 or 4]
+    gaussian_ids: Optional[Tensor] = None,  # [nnz]: the rows are packed
+) -> Tuple[Tensor, Tensor]:
+    """`view_dependent_colors` and `rasterize_to_pixels` in one kernel, forward only: the
+    compositing kernel evaluates the colour of the list entries it stages (the ones tiles reach
+    before they saturate) instead of reading colours made for every visible Gaussian
+    beforehand.  Same images, bit for bit, as the two operators one after the other.
+
+    Returns (render_colors[C,H,W,3 or 4], render_alphas[C,H,W,1]).
+    """
+    C = isect_offsets.size(0)
+    N = means.size(0)
+    rows = (C, N) if gaussian_ids is None else (gaussian_ids.size(0),)
+    assert gaussian_ids is None or gaussian_ids.dim() == 1, gaussian_ids.shape
+    assert means2d.shape == rows + (2,), means2d.shape
+    assert conics.shape == rows + (3,), conics.shape
+    assert opacities.shape == rows, opacities.shape
+    assert pix_vels.shape == rows + (2,), pix_vels.shape
+    assert viewmats.shape == (C, 4, 4), viewmats.shape
+    assert sh_coeffs.shape[-1] == 3 and sh_coeffs.shape[:-2] in ((N,), (C, N)), sh_coeffs.shape
+    assert (sh_degree + 1) ** 2 <= sh_coeffs.shape[-2], sh_coeffs.shape
+    assert depths is None or depths.shape == rows, depths.shape
+    channels = 3 if depths is None else 4
+    if rolling_shutter_time is not None:
+        assert rolling_shutter_time.shape == (C,), rolling_shutter_time.shape
+    else:
+        rolling_shutter_time = torch.zeros(C, device=means2d.device)
+    if backgrounds is not None:
+        assert backgrounds.shape == (C, channels), backgrounds.shape
+        backgrounds = backgrounds.contiguous()
+    tile_height, tile_width = isect_offsets.shape[1:3]
+    assert tile_height * tile_size >= image_height, f"Assert Failed: {tile_height} * {tile_size} >= {image_height}"
+    assert tile_width * tile_size >= image_width, f"Assert Failed: {tile_width} * {tile_size} >= {image_width}"
+    tensors = (means, viewmats, sh_coeffs, depths, means2d, conics, opacities, pix_vels, backgrounds)
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        raise ValueError("rasterize_to_pixels_with_sh is forward only: use view_dependent_colors "
+                         "and rasterize_to_pixels where a gradient is wanted")
+    render_colors, render_alphas, _ = _make_lazy_hip_func("rasterize_to_pixels_sh_fwd")(
+        sh_degree, means.contiguous(), viewmats.contiguous(), sh_coeffs.contiguous(), _c(gaussian_ids),
+        _c(depths), means2d.contiguous(), conics.contiguous(), opacities.contiguous(), pix_vels.contiguous(),
+        rolling_shutter_time.contiguous(), backgrounds, image_width, image_height, tile_size,
+        isect_offsets.contiguous(), flatten_ids.contiguous())
+    return render_colors, render_alphas
+
+
 def rasterize_to_points(
     means2d: Tensor,  # [C, N, 2] or [nnz, 2]
     conics: Tensor,  # [C, N, 3] or [nnz, 3]

@@ -19,6 +19,7 @@ from .hip._wrapper import (
     isect_offset_encode,
     isect_tiles,
     rasterize_to_pixels,
+    rasterize_to_pixels_with_sh,
     rasterize_to_points,
     spherical_harmonics,
     view_dependent_colors,
@@ -180,8 +181,17 @@ def rasterization(
     beside = _Beside(means.device)
     fused_colors = sh_degree is not None and not viewmats.requires_grad
     depth_appended = fused_colors and render_mode in ["RGB+D", "RGB+ED"]
+    # Colours from spherical harmonics and no gradient wanted: the compositing kernel evaluates
+    # the colours of the entries it stages itself (step 3 below falls away).
+    colors_while_compositing = (
+        fused_colors and means.is_cuda and render_mode in ["RGB", "RGB+D", "RGB+ED"]
+        and colors.dtype == torch.float32
+        and not (torch.is_grad_enabled() and any(
+            t is not None and t.requires_grad
+            for t in (means, quats, scales, opacities, colors, velocities, viewmats, backgrounds))))
+    colors_beside = fused_colors and not colors_while_compositing
     if packed:
-        if fused_colors and colors.is_contiguous():
+        if colors_beside and colors.is_contiguous():
             beside.requests["colors"] = (sh_degree, colors, depth_appended)
         # the gather opacities[gaussian_ids] (* compensations), where no gradient passes through it
         no_grad = not torch.is_grad_enabled() or not any(
@@ -209,7 +219,7 @@ def rasterization(
         return o if compensations is None else o * compensations
 
     # 2. tile intersection, sort, offsets
-    if not packed:
+    if not packed and not colors_while_compositing:
         beside.refork()  # fork: everything the colours need is enqueued
 
     def fused_view_colors():
@@ -231,7 +241,7 @@ def rasterization(
     beside_opacities = packed and not opacities.requires_grad
     if "opacities" in beside.results:
         opacities = beside.results["opacities"]
-        if not fused_colors:
+        if not colors_beside:
             beside.join()
     elif beside_opacities:
         # the gather (and the product with the compensations) goes beside the sort too: on the
@@ -239,7 +249,7 @@ def rasterization(
         # leaf that takes a gradient: autograd would accumulate it on the helper stream.)
         with beside:
             opacities = per_row_opacities()
-        if not fused_colors:
+        if not colors_beside:
             beside.join(opacities)
     else:
         if packed:
@@ -247,7 +257,9 @@ def rasterization(
         opacities = per_row_opacities()
 
     # 3. per-(camera, Gaussian) colours
-    if fused_colors:
+    if colors_while_compositing:
+        pass
+    elif fused_colors:
         colors = fused_view_colors()
         made_beside = "colors" not in beside.results  # (what the projection made was allocated here)
         beside.join(colors if made_beside else None,
@@ -272,7 +284,7 @@ def rasterization(
 
     # 4. channels to composite
     if render_mode in ["RGB+D", "RGB+ED"]:
-        if not depth_appended:
+        if not depth_appended and not colors_while_compositing:
             colors = torch.cat((colors, depths[..., None]), dim=-1)
         if backgrounds is not None:
             backgrounds = torch.cat(
@@ -292,7 +304,13 @@ def rasterization(
     # The reference composites channel_chunk channels per call (rendering.py:362-391), copying
     # a slice of the colours for each; the kernel here takes all channels in one call (in
     # passes of 32 over the same lists), which renders the same images without the copies.
-    render_colors, render_alphas = composite(colors, backgrounds)
+    if colors_while_compositing:
+        render_colors, render_alphas = rasterize_to_pixels_with_sh(
+            sh_degree, means, viewmats, colors, depths if depth_appended else None, means2d, conics,
+            opacities, pix_vels, width, height, tile_size, isect_offsets, flatten_ids,
+            rolling_shutter_time, backgrounds=backgrounds, gaussian_ids=gaussian_ids)
+    else:
+        render_colors, render_alphas = composite(colors, backgrounds)
 
     if render_mode in ["ED", "RGB+ED"]:
         render_colors = torch.cat(

@@ -1,0 +1,117 @@
+"""`rasterize_to_pixels_with_sh` -- the compositing kernel that evaluates the view-dependent
+colours of the entries it stages -- against the two operators it stands for,
+`view_dependent_colors` (gsplat/rendering.py:325-347 of the reference: directions, spherical
+harmonics, max(c + 1/2, 0)) followed by `rasterize_to_pixels` (rasterization.cu:1360-1518),
+which other tests compare with the oracle.  The bar is equality bit for bit: both paths run
+the same instructions on the same values.
+"""
+import math
+
+import pytest
+import torch
+
+from splatad_amd import workloads
+from tests.gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+
+
+def _projected(C, N, W, H, tile_size, packed, seed):
+    from splatad_amd import fully_fused_projection, isect_offset_encode, isect_tiles
+    s = workloads.camera_driving(n=N, seed=seed, width=W, height=H, n_cameras=C, with_velocities=True)
+    d = workloads.to_device(s, DEV)
+    proj = fully_fused_projection(d["means"], None, d["quats"], d["scales"], d["velocities"], d["viewmats"],
+                                  d["Ks"], W, H, d["linear_velocity"], d["angular_velocity"],
+                                  d["rolling_shutter_time"], eps2d=d["eps2d"], near_plane=d["near_plane"],
+                                  far_plane=d["far_plane"], packed=packed)
+    if packed:
+        camera_ids, gaussian_ids, radii, means2d, depths, conics, _, pix_vels = proj
+        opacities = d["opacities"][gaussian_ids]
+    else:
+        radii, means2d, depths, conics, _, pix_vels = proj
+        camera_ids = gaussian_ids = None
+        opacities = d["opacities"].expand(C, -1).contiguous()
+    tw, th = math.ceil(W / tile_size), math.ceil(H / tile_size)
+    _, isect_ids, flatten_ids = isect_tiles(means2d, radii, depths, tile_size, tw, th, packed=packed,
+                                            n_cameras=C, camera_ids=camera_ids, gaussian_ids=gaussian_ids)
+    offsets = isect_offset_encode(isect_ids, C, tw, th)
+    return d, dict(radii=radii, means2d=means2d, depths=depths, conics=conics, pix_vels=pix_vels,
+                   opacities=opacities, camera_ids=camera_ids, gaussian_ids=gaussian_ids,
+                   offsets=offsets, flatten_ids=flatten_ids)
+
+
+@pytest.mark.parametrize("C,degree,per_sensor,with_depth,tile_size,packed", [
+    (1, 3, False, True, 16, False),   # the driving camera's case: two pixels per lane, RGB+D
+    (1, 3, False, False, 16, False),
+    (3, 3, True, True, 16, False),    # coefficients of their own per camera
+    (2, 0, False, True, 16, False),
+    (2, 1, False, False, 16, True),
+    (2, 2, True, True, 16, True),
+    (2, 4, False, True, 16, True),    # 25 coefficients
+    (2, 4, True, False, 8, False),
+    (1, 3, False, True, 4, False),    # one pixel per lane
+    (2, 3, False, True, 8, True),
+])
+def test_colours_evaluated_while_compositing_equal_the_two_operators(C, degree, per_sensor, with_depth,
+                                                                      tile_size, packed):
+    from splatad_amd.hip._wrapper import (rasterize_to_pixels, rasterize_to_pixels_with_sh,
+                                          view_dependent_colors)
+    N, W, H = 6000, 200, 120
+    d, p = _projected(C, N, W, H, tile_size, packed, seed=20 + degree)
+    g = torch.Generator(device=DEV).manual_seed(3)
+    K = (degree + 1) ** 2 + (2 if degree == 2 else 0)  # more coefficients than the degree uses, once
+    coeffs = torch.randn(((C, N) if per_sensor else (N,)) + (K, 3), device=DEV, generator=g) * 0.4
+    bg = torch.rand((C, 4 if with_depth else 3), device=DEV, generator=g)
+    depths = p["depths"] if with_depth else None
+    with torch.no_grad():
+        colors = view_dependent_colors(degree, d["means"], d["viewmats"], coeffs, p["radii"], depths,
+                                       p["camera_ids"], p["gaussian_ids"])
+        want = rasterize_to_pixels(p["means2d"], p["conics"], colors, p["opacities"], p["pix_vels"], W, H,
+                                   tile_size, p["offsets"], p["flatten_ids"], d["rolling_shutter_time"],
+                                   backgrounds=bg, packed=packed)
+        got = rasterize_to_pixels_with_sh(degree, d["means"], d["viewmats"], coeffs, depths, p["means2d"],
+                                          p["conics"], p["opacities"], p["pix_vels"], W, H, tile_size,
+                                          p["offsets"], p["flatten_ids"], d["rolling_shutter_time"],
+                                          backgrounds=bg, gaussian_ids=p["gaussian_ids"])
+    assert got[0].shape == want[0].shape == (C, H, W, 4 if with_depth else 3)
+    assert float(want[1].max()) > 0.5 and float(want[1].min()) < 0.5  # rendered, and not everywhere
+    assert torch.equal(got[1], want[1])
+    assert torch.equal(got[0], want[0])
+
+
+def test_colours_while_compositing_is_forward_only_and_checks_its_rows():
+    from splatad_amd.hip._wrapper import rasterize_to_pixels_with_sh
+    d, p = _projected(1, 500, 64, 48, 16, False, seed=4)
+    coeffs = torch.zeros((500, 16, 3), device=DEV)
+    args = (3, d["means"], d["viewmats"], coeffs, None, p["means2d"], p["conics"], p["opacities"],
+            p["pix_vels"], 64, 48, 16, p["offsets"], p["flatten_ids"])
+    rc, ra = rasterize_to_pixels_with_sh(*args)
+    # zero coefficients: every colour is max(0 + 1/2, 0), so a pixel holds alpha / 2
+    torch.testing.assert_close(rc, (0.5 * ra).expand(-1, -1, -1, 3), atol=1e-6, rtol=1e-6)
+    with pytest.raises(ValueError, match="forward only"):
+        rasterize_to_pixels_with_sh(3, d["means"], d["viewmats"], coeffs.requires_grad_(), *args[4:])
+    with pytest.raises(AssertionError):  # degree 4 needs 25 coefficients
+        rasterize_to_pixels_with_sh(4, *args[1:])
+
+
+def test_rasterization_switches_to_the_colour_kernel_when_a_gradient_is_wanted():
+    """rasterization() evaluates the colours while compositing only when no input takes a
+    gradient; with one that does it runs the colour kernel and the differentiable operators,
+    and renders the same image."""
+    from splatad_amd import rasterization
+    s = workloads.camera_driving(n=8000, width=256, height=144, n_cameras=2)
+    d = workloads.to_device(s, DEV)
+    kw = dict(near_plane=d["near_plane"], far_plane=d["far_plane"], eps2d=d["eps2d"], tile_size=16,
+              sh_degree=3, render_mode="RGB+ED", backgrounds=torch.rand((2, 3), device=DEV))
+    rest = (d["velocities"], d["viewmats"], d["Ks"], d["width"], d["height"], d["linear_velocity"],
+            d["angular_velocity"], d["rolling_shutter_time"])
+    for packed in (False, True):
+        with torch.no_grad():
+            plain = rasterization(d["means"], d["quats"], d["scales"], d["opacities"], d["colors"], *rest,
+                                  packed=packed, **kw)
+        leaf = d["colors"].clone().requires_grad_()
+        grad = rasterization(d["means"], d["quats"], d["scales"], d["opacities"], leaf, *rest, packed=packed, **kw)
+        assert grad[0].requires_grad and not plain[0].requires_grad
+        assert torch.equal(grad[0].detach(), plain[0]) and torch.equal(grad[1].detach(), plain[1])
+        grad[0].sum().backward()
+        assert float(leaf.grad.abs().sum()) > 0
