@@ -68,6 +68,25 @@ def time_kernel(fn, iters, warmup=2):
     return sum(s.elapsed_time(e) for s, e in zip(start, stop)) / iters
 
 
+def time_kernel_on(make, fn, iters, warmup=2):
+    """As time_kernel, for fn(x) with x = make() made afresh, outside the timed interval, for
+    every call (a kernel that changes its input)."""
+    import torch
+
+    for _ in range(warmup):
+        fn(make())
+    xs = [make() for _ in range(iters)]
+    _sync()
+    start = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    stop = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    for i in range(iters):  # enqueued back to back, so that the GPU never waits for the host
+        start[i].record()
+        fn(xs[i])
+        stop[i].record()
+    _sync()
+    return sum(s.elapsed_time(e) for s, e in zip(start, stop)) / iters
+
+
 def staged_isects(tile_entries):
     """List entries the compositing kernel staged: whole batches until every pixel / point of a
     tile has saturated, clipped to the tile's list, as counted by the kernel itself."""
@@ -138,15 +157,25 @@ def bench_camera(args):
                 meta["means2d"], meta["conics"], cols, meta["opacities"], meta["pix_vels"],
                 s["rolling_shutter_time"], None, W, H, ts, meta["isect_offsets"], meta["flatten_ids"])
 
-        def raster_sh():
-            # what the step runs: the same kernel evaluating the colours of the entries it stages
+        # what the step runs: the same kernel evaluating the colours of the entries it stages,
+        # on a colour cache that two short launches prepare (left empty for this frame)
+        from splatad_amd.hip._wrapper import MIN_OPACITY_PER_TILE
+
+        def color_cache():
+            return _C.view_colors_cache(3, s["means"], s["viewmats"], None, None, meta["radii"], s["colors"],
+                                        meta["depths"], s["opacities"], ts, meta["tile_width"],
+                                        meta["tile_height"], MIN_OPACITY_PER_TILE)
+
+        def raster_sh(cache):
             return _C.rasterize_to_pixels_sh_fwd(
                 3, s["means"], s["viewmats"], s["colors"], None, meta["depths"], meta["means2d"],
                 meta["conics"], meta["opacities"], meta["pix_vels"], s["rolling_shutter_time"], None,
-                W, H, ts, meta["isect_offsets"], meta["flatten_ids"])
+                W, H, ts, meta["isect_offsets"], meta["flatten_ids"], cache=cache)
 
-        assert torch.equal(raster_sh()[0], raster()[0]) and torch.equal(raster_sh()[0], rc)
-        k_ms = time_kernel(raster_sh, iters=max(5, args.steps))
+        first = color_cache()
+        cache_left_empty = bool(torch.isnan(first).all().item())
+        assert torch.equal(raster_sh(first)[0], raster()[0]) and torch.equal(raster()[0], rc)
+        k_ms = time_kernel_on(color_cache, raster_sh, iters=max(5, args.steps))
         k_plain_ms = time_kernel(raster, iters=max(5, args.steps))
         n_isects = int(meta["flatten_ids"].shape[0])
         batches = torch.zeros_like(meta["isect_offsets"])
@@ -173,7 +202,9 @@ def bench_camera(args):
         staged = torch.cumsum(marks[:-1], 0) > 0
         rows_staged = int(torch.unique(meta["flatten_ids"][staged]).numel())
         plain_bytes = i_need * (36 + 4 * D) + P * (4 * D + 8) + T * 4
-        alg_bytes = i_need * (36 + 4 * (D - 3)) + rows_staged * (12 + 12 * K) + P * (4 * D + 8) + T * 4
+        # per staged entry its geometry and cache row, per staged row the evaluation (mean,
+        # coefficients, depth) and the cache row written back
+        alg_bytes = i_need * (36 + 16) + rows_staged * (12 + 12 * K + 4 + 16) + P * (4 * D + 8) + T * 4
         # per-stage times of the same call
         stages = {}
         proj = lambda: _C.fully_fused_projection_fwd(
@@ -191,6 +222,7 @@ def bench_camera(args):
         stages["view_colors_ms"] = time_kernel(
             lambda: _C.view_colors_fwd(3, s["means"], s["viewmats"], None, None, meta["radii"],
                                        s["colors"], meta["depths"]), 5)
+        stages["color_cache_ms"] = time_kernel(color_cache, 5)
         stages["rasterize_ms"] = k_ms
         stages["rasterize_given_colors_ms"] = k_plain_ms
         nnz = int((meta["radii"][..., 0] > 0).sum().item())
@@ -201,6 +233,7 @@ def bench_camera(args):
             "isect_sort_ms": C * N * 20 + n_isects * 12 + T * 4,
             "offset_encode_ms": n_isects * 8 + T * 4,
             "view_colors_ms": nnz * (12 + 12 * K + 1 + 12),
+            "color_cache_ms": C * N * (8 + 16) + N * 4,
             "rasterize_ms": alg_bytes,
             "rasterize_given_colors_ms": plain_bytes,
         }
@@ -212,7 +245,8 @@ def bench_camera(args):
                      footprint_test_pass_fraction=st[5] / max(1, st[4]),
                      iterations_without_a_compositing_lane=st[3] / max(1, st[0]))
     return dict(sec=sec, sec_packed=sec_packed, pixels=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
-                n_isects=n_isects, i_need=i_need, rows_staged=rows_staged, nnz=nnz, stages=stages,
+                n_isects=n_isects, i_need=i_need, rows_staged=rows_staged, cache_left_empty=cache_left_empty,
+                nnz=nnz, stages=stages,
                 stage_bytes=stage_bytes,
                 channels=D, lanes=lanes, tile_cycles=tile_cycles)
 
@@ -436,8 +470,8 @@ def cpu_baseline_camera(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--n", type=int, default=1_000_000, help="Gaussians (default: the benchmark's 1M)")
     ap.add_argument("--cpu-n", type=int, default=1_000_000, help="Gaussians of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -498,7 +532,7 @@ def main():
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": MEASURED_TRAFFIC_BYTES["camera"] if args.n == 1_000_000 else None,
             "algorithmic_bytes": cam["alg_bytes"], "kernel_ms": cam["kernel_ms"],
-            "rows_staged": cam["rows_staged"],
+            "rows_staged": cam["rows_staged"], "color_cache_left_empty": cam["cache_left_empty"],
         },
     }
     if lid is not None:

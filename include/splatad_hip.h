@@ -364,6 +364,24 @@ int splatad_rasterize_to_pixels_fwd(uint32_t C, int64_t n_isects, uint32_t chann
                                     int32_t *last_ids, int32_t *tile_batches,
                                     int64_t *tile_cycles, splatad_stream_t stream);
 
+/* Prepares the colour cache of splatad_rasterize_to_pixels_fwd_sh (no counterpart in the
+ * reference): `cache`, splatad_view_colors_cache_bytes(n) bytes, gets a NaN in every float of
+ * its n rows, and -- only where the lists will be consumed deeply -- the colours of all visible
+ * rows, as splatad_view_colors_fwd makes them, because then nearly every row is needed and a
+ * row per lane beforehand is cheaper than rows evaluated as the tiles reach them.  The test:
+ * sum over the visible rows of opacities[Gaussian] x tiles met (estimated from radii and
+ * tile_size), divided by the C x tile_width x tile_height tiles; below min_opacity_per_tile the
+ * colours are made here (0 = never, infinity = always), with the row's depth (depths may be
+ * NULL: zero) as fourth float, which the compositing kernel renders as its fourth channel.
+ * opacities is [N], one per Gaussian; the other arguments as for splatad_view_colors_fwd. */
+size_t splatad_view_colors_cache_bytes(uint64_t n_rows);
+int splatad_view_colors_cache(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
+                              const float *means, const float *viewmats, const int64_t *camera_ids,
+                              const int64_t *gaussian_ids, const int32_t *radii, const float *coeffs,
+                              int coeffs_per_sensor, const float *depths, const float *opacities,
+                              uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
+                              float min_opacity_per_tile, float *cache, splatad_stream_t stream);
+
 /* Steps 3 and 5 of rasterization() in one kernel (gsplat/rendering.py:325-347 and 362-391 of
  * the reference: view directions, spherical harmonics, max(c + 1/2, 0), then
  * rasterize_to_pixels): the compositing kernel evaluates the colour of every list entry it
@@ -375,10 +393,10 @@ int splatad_rasterize_to_pixels_fwd(uint32_t C, int64_t n_isects, uint32_t chann
  * flatten_ids index: means2d, conics, opacities, pix_vels, depths) are dense [C, N] with
  * gaussian_ids == NULL, or packed [nnz] with gaussian_ids [nnz] naming each row's Gaussian (the
  * camera of a row is that of the tile that lists it).  Renders 3 channels, or 4 with `depths`
- * (not NULL) as the last one.  color_cache: 16 bytes per row, every float a NaN before the call
- * (the workgroups that first stage a row leave its colour there for the tiles that list the
- * Gaussian later, so a row is evaluated a few times at most however much of the lists is
- * consumed); what it holds afterwards is of no use to the caller.  Forward only. */
+ * (not NULL) as the last one.  color_cache: 16 bytes per row, as splatad_view_colors_cache
+ * leaves them (every float a NaN, or the row's colour and depth; the workgroups that first
+ * stage a row without a colour leave it there for the tiles that list the Gaussian later); what
+ * it holds afterwards is of no use to the caller.  Forward only. */
 int splatad_rasterize_to_pixels_fwd_sh(uint32_t C, uint32_t N, int64_t n_isects, uint32_t K,
                                        uint32_t degree, const float *means, const float *viewmats,
                                        const float *coeffs, int coeffs_per_sensor,

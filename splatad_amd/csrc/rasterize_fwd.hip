@@ -236,24 +236,24 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
         for (int k = 0; k < CH; ++k) s.col[k] = STATS ? 0.f : c[min((uint32_t)k, a.n_ch - 1u)]; // STATS: no colours
         return s;
     };
-    // SHC: the colour of row g, what sh_fwd_kernel<true> writes for it, by the same instructions;
-    // staged before the rest of the Gaussian is requested, so that the coefficients of a band
-    // and the Gaussian's other values are not in registers at the same time.
+    // SHC: the colour of row g, what sh_fwd_kernel<true> writes for it, by the same instructions.
     // A row's colour is evaluated by the first workgroups that stage it and left in sh_cache for
-    // the others (a Gaussian is listed by every tile it touches).  Word-wise relaxed accesses
-    // with no wider scope than the workgroup, i.e. ordinary cached loads and stores: another
-    // workgroup sees each word either as the NaN the cache was filled with -- then it evaluates
-    // the colour itself, to the same value -- or as the colour; how soon it sees the colour is
-    // left to the caches (the dies' L2 caches do not see one another's lines before the kernel
-    // ends, so each die evaluates the rows its tiles stage).  Loads or stores of device scope,
-    // which would share the colours between the dies, go to memory every time and made the
-    // kernel three to four times slower.
-    auto stage_sh_color = [&](int32_t g) {
-        float *cached = a.sh_cache + (size_t)g * 4;
-        float cr = __hip_atomic_load(cached, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        float cg = __hip_atomic_load(cached + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        float cb = __hip_atomic_load(cached + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        const bool missing = !(cr == cr) || !(cg == cg) || !(cb == cb);
+    // the others (a Gaussian is listed by every tile it touches).  Ordinary cached loads and
+    // stores, on purpose without any ordering: a word of a row only ever changes from the NaN
+    // the cache was filled with to its colour, so another workgroup sees each word either as
+    // NaN -- then it evaluates the colour itself, to the same value -- or as the colour; how
+    // soon it sees the colour is left to the caches (the dies' L2 caches do not see one
+    // another's lines before the kernel ends, so each die evaluates the rows its tiles
+    // stage).  Atomic loads or stores of device scope, which would share the colours between
+    // the dies, go to memory every time and made the kernel three to four times slower.
+    struct Cached { float r, g, b, depth; };
+    auto cached_color = [&](int32_t g) { // requested together with the rest of the Gaussian
+        const float4 row = reinterpret_cast<const float4 *>(a.sh_cache)[g];
+        return Cached{row.x, row.y, row.z, row.w};
+    };
+    auto stage_sh_color = [&](int32_t g, const Cached &c) {
+        float cr = c.r, cg = c.g, cb = c.b, cd = c.depth; // the depth channel rides along
+        const bool missing = !(cr == cr) || !(cg == cg) || !(cb == cb) || (CH > 3 && !(cd == cd));
         if (wave_ballot(missing) != 0) { // uniform
             if (missing) {
                 const uint32_t gauss =
@@ -266,16 +266,15 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
                 cr = fmaxf(r + 0.5f, 0.f);
                 cg = fmaxf(gr + 0.5f, 0.f);
                 cb = fmaxf(bl + 0.5f, 0.f);
-                __hip_atomic_store(cached, cr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                __hip_atomic_store(cached + 1, cg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                __hip_atomic_store(cached + 2, cb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                cd = CH > 3 ? a.sh_depths[g] : 0.f;
+                reinterpret_cast<float4 *>(a.sh_cache)[g] = make_float4(cr, cg, cb, cd);
             }
         }
         float *col = reinterpret_cast<float *>(s_rec + RECORD * tr + 2);
         col[0] = cr;
         col[1 % CH] = cg;
         col[2 % CH] = cb;
-        if (CH > 3) col[3 % CH] = a.sh_depths[g];
+        if (CH > 3) col[3 % CH] = cd;
     };
     uint32_t batches_done = 0;
     for (uint32_t b = 0; b < num_batches; ++b) {
@@ -289,13 +288,17 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
         const uint32_t batch_start = (uint32_t)range_start + batch * b;
         {
             const int32_t g = id_of(b);
-            if (SHC) stage_sh_color(g);
+            Cached cached = {};
+            if (SHC) cached = cached_color(g);
             const Staged staged = gather(g);
             float4 pa, pb;
             pixel_polynomial(frame, staged.xy, staged.vel, staged.cn[0], staged.cn[1], staged.cn[2], staged.opac,
                              pa, pb);
             s_rec[RECORD * tr] = pa;
             s_rec[RECORD * tr + 1] = pb;
+            // (the colour last: where it has to be evaluated, nothing else of the Gaussian is in
+            // registers beside a band's coefficients)
+            if (SHC) stage_sh_color(g, cached);
             if (!SHC) {
 #pragma unroll
                 for (int k = 0; k < CH; ++k)

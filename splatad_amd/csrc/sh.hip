@@ -79,13 +79,11 @@ __device__ __forceinline__ bool sh_row(uint32_t e, const ShView &v, const float 
 // applies the colour activation of the pipeline, max(c + 1/2, 0) (gsplat/rendering.py:347),
 // and writes rows of `stride` floats, with the depth as fourth channel when given (:351).
 template <bool VIEW>
-__global__ void __launch_bounds__(SPLATAD_THREADS)
-sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, ShView view, const float *__restrict__ dirs,
-              const float *__restrict__ coeffs, const uint8_t *__restrict__ masks,
-              const float *__restrict__ depths, uint32_t stride, float *__restrict__ colors,
-              const int32_t *__restrict__ remap) {
-    const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n) return;
+__device__ __forceinline__ void sh_fwd_row(uint32_t e, uint32_t K, uint32_t degree, const ShView &view,
+                                           const float *__restrict__ dirs, const float *__restrict__ coeffs,
+                                           const uint8_t *__restrict__ masks, const float *__restrict__ depths,
+                                           uint32_t stride, float *__restrict__ colors,
+                                           const int32_t *__restrict__ remap) {
     float r = 0.f, g = 0.f, b = 0.f;
     float dx = 0.f, dy = 0.f, dz = 0.f;
     size_t coeff_row;
@@ -104,6 +102,75 @@ sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, ShView view, const float 
     } else {
         out[0] = r; out[1] = g; out[2] = b;
     }
+}
+
+template <bool VIEW>
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, ShView view, const float *__restrict__ dirs,
+              const float *__restrict__ coeffs, const uint8_t *__restrict__ masks,
+              const float *__restrict__ depths, uint32_t stride, float *__restrict__ colors,
+              const int32_t *__restrict__ remap) {
+    const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    sh_fwd_row<VIEW>(e, K, degree, view, dirs, coeffs, masks, depths, stride, colors, remap);
+}
+
+// The colour cache of the compositing kernel that evaluates colours itself
+// (rasterize_fwd.hip): a float4 per row, NaN = not evaluated yet.  Two launches prepare it.
+// The first fills it with NaN and adds up, per workgroup, opacity x tiles over the visible rows
+// (tiles estimated from the radii): divided by the number of tiles, the opacity a tile's list
+// carries.  Where that is large the tiles saturate on the first entries of their lists and the
+// compositing kernel evaluates those few rows itself; where it is small the lists are
+// consumed to their ends, every wavefront of the compositing kernel would meet a missing row
+// in every batch, and evaluating all visible rows beforehand, a row per lane, is cheaper: the
+// second launch does that unless the sum reaches `enough`.
+constexpr uint32_t kCachePartials = 1024; // workgroups of the first launch at most
+
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+sh_cache_clear_kernel(uint32_t n, ShView view, const float *__restrict__ opacities, float inv_tile,
+                      float tile_w, float tile_h, float4 *__restrict__ cache, float *__restrict__ partials) {
+    __shared__ float s_sum[SPLATAD_THREADS / SPLATAD_WAVE];
+    const float nan = __uint_as_float(0x7FC00000u);
+    float sum = 0.f;
+    for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
+        cache[e] = make_float4(nan, nan, nan, nan);
+        const int32_t rx = view.radii[(size_t)e * 2], ry = view.radii[(size_t)e * 2 + 1];
+        if (rx > 0 && ry > 0) {
+            const uint32_t g = view.gaussian_ids ? (uint32_t)view.gaussian_ids[e] : e % view.N;
+            sum += opacities[g] * fminf(2.f * (float)rx * inv_tile + 1.f, tile_w) *
+                   fminf(2.f * (float)ry * inv_tile + 1.f, tile_h);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, SPLATAD_WAVE);
+    if ((threadIdx.x & (SPLATAD_WAVE - 1)) == 0) s_sum[threadIdx.x / SPLATAD_WAVE] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float total = 0.f;
+        for (uint32_t w = 0; w < blockDim.x / SPLATAD_WAVE; ++w) total += s_sum[w];
+        partials[blockIdx.x] = total;
+    }
+}
+
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+sh_cache_fill_kernel(uint32_t n, uint32_t K, uint32_t degree, ShView view, const float *__restrict__ coeffs,
+                     const float *__restrict__ depths, float *__restrict__ cache,
+                     const float *__restrict__ partials, uint32_t n_partials, float enough) {
+    __shared__ float s_sum[SPLATAD_THREADS / SPLATAD_WAVE];
+    float sum = 0.f; // every workgroup adds up the same numbers in the same order
+    for (uint32_t k = threadIdx.x; k < n_partials; k += blockDim.x) sum += partials[k];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, SPLATAD_WAVE);
+    if ((threadIdx.x & (SPLATAD_WAVE - 1)) == 0) s_sum[threadIdx.x / SPLATAD_WAVE] = sum;
+    __syncthreads();
+    float total = 0.f;
+    for (uint32_t w = 0; w < blockDim.x / SPLATAD_WAVE; ++w) total += s_sum[w];
+    if (total >= enough) return; // uniform across the launch
+    const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    if (view.radii[(size_t)e * 2] <= 0) return; // rows no list names keep their NaN
+    sh_fwd_row<true>(e, K, degree, view, nullptr, coeffs, nullptr, depths, 4u, cache, nullptr);
+    if (depths == nullptr) cache[(size_t)e * 4 + 3] = 0.f;
 }
 
 // VIEW: v_colors are rows of `stride` floats, the gradients of the activated colours
@@ -279,6 +346,41 @@ extern "C" int splatad_view_colors_fwd(uint32_t n, uint32_t C, uint32_t N, uint3
     SPLATAD_REQUIRE(coeffs && colors, "view colours: null pointer argument");
     return sh_forward<true>(n, K, degree, view, nullptr, coeffs, nullptr, depths, depths ? 4u : 3u,
                             colors, (hipStream_t)stream);
+}
+
+extern "C" size_t splatad_view_colors_cache_bytes(uint64_t n_rows) {
+    return (size_t)n_rows * 16 + kCachePartials * sizeof(float);
+}
+
+extern "C" int splatad_view_colors_cache(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
+                                         const float *means, const float *viewmats,
+                                         const int64_t *camera_ids, const int64_t *gaussian_ids,
+                                         const int32_t *radii, const float *coeffs,
+                                         int coeffs_per_sensor, const float *depths,
+                                         const float *opacities,
+                                         uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
+                                         float min_opacity_per_tile, float *cache,
+                                         splatad_stream_t stream) {
+    if (int rc = sh_check(K, degree)) return rc;
+    if (n == 0) return 0;
+    ShView view;
+    if (int rc = sh_view_args(n, C, N, means, viewmats, camera_ids, gaussian_ids, radii,
+                              coeffs_per_sensor, &view)) return rc;
+    SPLATAD_REQUIRE(coeffs && opacities && cache, "view colours: null pointer argument");
+    SPLATAD_REQUIRE(tile_size > 0 && tile_width > 0 && tile_height > 0, "view colours: empty tile grid");
+    const float n_tiles = (float)C * (float)tile_width * (float)tile_height;
+    float *partials = cache + (size_t)n * 4;
+    uint32_t wgs = (n + SPLATAD_THREADS - 1) / SPLATAD_THREADS;
+    if (wgs > kCachePartials) wgs = kCachePartials;
+    hipLaunchKernelGGL(sh_cache_clear_kernel, dim3(wgs), dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, n,
+                       view, opacities, 1.f / (float)tile_size, (float)tile_width, (float)tile_height,
+                       reinterpret_cast<float4 *>(cache), partials);
+    SPLATAD_LAUNCH_CHECK();
+    hipLaunchKernelGGL(sh_cache_fill_kernel, dim3((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS),
+                       dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, n, K, degree, view, coeffs, depths, cache,
+                       (const float *)partials, wgs, min_opacity_per_tile * n_tiles);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
 }
 
 extern "C" int splatad_view_colors_fwd_remapped(uint32_t C, uint32_t N, uint32_t K, uint32_t degree,

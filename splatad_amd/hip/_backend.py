@@ -44,7 +44,7 @@ def load_library():
                 f"{LIB_PATH} has ABI version {lib.splatad_abi_version()}, this package needs {ABI_VERSION}: "
                 "rebuild it with `python -m splatad_amd.build`")
         for name in ("splatad_projection_packed_workspace_bytes", "splatad_isect_workspace_bytes",
-                     "splatad_isect_lists_bytes",
+                     "splatad_isect_lists_bytes", "splatad_view_colors_cache_bytes",
                      "splatad_map_points_to_lidar_tiles_workspace_bytes",
                      "splatad_rasterize_to_indices_workspace_bytes",
                      "splatad_rasterize_bwd_workspace_bytes"):
@@ -477,6 +477,32 @@ class _Ops:
                 _i32(coeffs.dim() == 4), _p(depths), _p(colors), _stream(dev)))
         return colors
 
+    def view_colors_cache(self, degrees_to_use, means, viewmats, camera_ids, gaussian_ids, radii, coeffs,
+                          depths, opacities, tile_size, tile_width, tile_height, min_opacity_per_tile):
+        """The colour cache that rasterize_to_pixels_sh_fwd takes ([rows, 4] floats, NaN = not
+        evaluated): all NaN where tiles will saturate early, the colours of the visible rows
+        where the estimate of the opacity per tile falls below min_opacity_per_tile."""
+        lib = load_library()
+        means = _in(means, "means"); viewmats = _in(viewmats, "viewmats")
+        camera_ids = _in(camera_ids, "camera_ids", torch.int64)
+        gaussian_ids = _in(gaussian_ids, "gaussian_ids", torch.int64)
+        radii = _in(radii, "radii", torch.int32); coeffs = _in(coeffs, "coeffs")
+        opacities = _in(opacities, "opacities"); depths = _in(depths, "depths")
+        C, N, dev = viewmats.shape[0], means.shape[0], means.device
+        assert opacities.shape == (N,), opacities.shape
+        assert depths is None or depths.shape == radii.shape[:-1], depths.shape
+        lead = tuple(radii.shape[:-1])
+        n = int(math.prod(lead))
+        words = lib.splatad_view_colors_cache_bytes(_u64(n)) // 4
+        buf = torch.empty((words,), dtype=torch.float32, device=dev)
+        with _on(dev):
+            _check(lib.splatad_view_colors_cache(
+                _u32(n), _u32(C), _u32(N), _u32(coeffs.shape[-2]), _u32(degrees_to_use), _p(means),
+                _p(viewmats), _p(camera_ids), _p(gaussian_ids), _p(radii), _p(coeffs),
+                _i32(coeffs.dim() == 4), _p(depths), _p(opacities), _u32(tile_size), _u32(tile_width),
+                _u32(tile_height), _f32(min_opacity_per_tile), _p(buf), _stream(dev)))
+        return buf[: n * 4].view(lead + (4,))
+
     def view_colors_bwd(self, degrees_to_use, means, viewmats, camera_ids, gaussian_ids, radii,
                         coeffs, colors, v_colors, compute_v_dirs):
         """Per-row gradients (v_coeffs [..., K, 3], v_dirs [..., 3] | None) of view_colors_fwd."""
@@ -848,7 +874,7 @@ class _Ops:
     def rasterize_to_pixels_sh_fwd(self, sh_degree, means, viewmats, coeffs, gaussian_ids, depths,
                                    means2d, conics, opacities, pix_vels, rolling_shutter_time,
                                    backgrounds, image_width, image_height, tile_size, tile_offsets,
-                                   flatten_ids):
+                                   flatten_ids, cache=None):
         """rasterize_to_pixels_fwd for rows whose colours are the view-dependent colours of
         `coeffs` ([N, K, 3] or [C, N, K, 3]): the kernel evaluates them for the entries it
         stages.  Rows are dense [C, N], or packed [nnz] with gaussian_ids [nnz]; depths, if
@@ -873,7 +899,10 @@ class _Ops:
         alphas = torch.empty((C, image_height, image_width, 1), **f)
         last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
         # colours of the rows that tiles stage, left by the first for the others; NaN = not yet
-        cache = torch.full(rows + (4,), float("nan"), **f)
+        if cache is None:
+            cache = torch.full(rows + (4,), float("nan"), **f)
+        cache = _in(cache, "cache")
+        assert cache.shape == rows + (4,), cache.shape
         with _on(dev):
             _check(lib.splatad_rasterize_to_pixels_fwd_sh(
                 _u32(C), _u32(N), _i64(flatten_ids.shape[0]), _u32(coeffs.shape[-2]), _u32(sh_degree),

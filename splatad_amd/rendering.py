@@ -22,6 +22,7 @@ from .hip._wrapper import (
     rasterize_to_pixels_with_sh,
     rasterize_to_points,
     spherical_harmonics,
+    view_dependent_color_cache,
     view_dependent_colors,
 )
 
@@ -185,13 +186,13 @@ def rasterization(
     # the colours of the entries it stages itself (step 3 below falls away).
     colors_while_compositing = (
         fused_colors and means.is_cuda and render_mode in ["RGB", "RGB+D", "RGB+ED"]
-        and colors.dtype == torch.float32
+        and colors.dtype == torch.float32 and opacities.dtype == torch.float32
         and not (torch.is_grad_enabled() and any(
             t is not None and t.requires_grad
             for t in (means, quats, scales, opacities, colors, velocities, viewmats, backgrounds))))
-    colors_beside = fused_colors and not colors_while_compositing
+    colors_beside = fused_colors and (packed or not colors_while_compositing)  # step 3 joins the helper stream
     if packed:
-        if colors_beside and colors.is_contiguous():
+        if fused_colors and not colors_while_compositing and colors.is_contiguous():
             beside.requests["colors"] = (sh_degree, colors, depth_appended)
         # the gather opacities[gaussian_ids] (* compensations), where no gradient passes through it
         no_grad = not torch.is_grad_enabled() or not any(
@@ -211,6 +212,8 @@ def rasterization(
     else:
         radii, means2d, depths, conics, compensations, pix_vels = proj
         camera_ids, gaussian_ids = None, None
+
+    opacities_per_gaussian = opacities
 
     def per_row_opacities():
         # Compositing is the first to need these: [nnz], or [C, N] (a view, copied by the first
@@ -257,8 +260,16 @@ def rasterization(
         opacities = per_row_opacities()
 
     # 3. per-(camera, Gaussian) colours
+    color_cache = None
     if colors_while_compositing:
-        pass
+        # the empty cache through which the tiles share the colours they evaluate, or, for a
+        # scene whose tiles will not saturate early, all colours after all (on the caller's
+        # stream: two short launches cost less there than a helper stream's fork and join)
+        if packed:
+            beside.join(opacities if beside_opacities and "opacities" not in beside.results else None)
+        color_cache = view_dependent_color_cache(
+            sh_degree, means, viewmats, colors, radii, depths if depth_appended else None,
+            opacities_per_gaussian, tile_size, tile_width, tile_height, camera_ids, gaussian_ids)
     elif fused_colors:
         colors = fused_view_colors()
         made_beside = "colors" not in beside.results  # (what the projection made was allocated here)
@@ -308,7 +319,8 @@ def rasterization(
         render_colors, render_alphas = rasterize_to_pixels_with_sh(
             sh_degree, means, viewmats, colors, depths if depth_appended else None, means2d, conics,
             opacities, pix_vels, width, height, tile_size, isect_offsets, flatten_ids,
-            rolling_shutter_time, backgrounds=backgrounds, gaussian_ids=gaussian_ids)
+            rolling_shutter_time, backgrounds=backgrounds, gaussian_ids=gaussian_ids,
+            color_cache=color_cache)
     else:
         render_colors, render_alphas = composite(colors, backgrounds)
 

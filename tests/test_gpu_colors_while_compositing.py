@@ -79,6 +79,56 @@ def test_colours_evaluated_while_compositing_equal_the_two_operators(C, degree, 
     assert torch.equal(got[0], want[0])
 
 
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("with_depth", [False, True])
+def test_colour_cache_empty_or_filled_by_the_opacity_a_tile_carries(packed, with_depth):
+    """view_dependent_color_cache leaves every row NaN where the visible Gaussians carry enough
+    opacity per tile for tiles to saturate early, and otherwise holds what view_dependent_colors
+    makes for the visible rows; compositing renders the same image from either."""
+    from splatad_amd.hip._wrapper import (MIN_OPACITY_PER_TILE, rasterize_to_pixels,
+                                          rasterize_to_pixels_with_sh, view_dependent_color_cache,
+                                          view_dependent_colors)
+    C, N, W, H, ts = 2, 6000, 200, 120, 16
+    d, p = _projected(C, N, W, H, ts, packed, seed=31)
+    tw, th = math.ceil(W / ts), math.ceil(H / ts)
+    coeffs = torch.randn((N, 16, 3), device=DEV, generator=torch.Generator(device=DEV).manual_seed(8)) * 0.4
+    depths = p["depths"] if with_depth else None
+    visible = p["radii"][..., 0] > 0
+    # the estimate the kernels make, restated: opacity x tiles met (from the radii, at most the grid)
+    gid = p["gaussian_ids"] if packed else torch.arange(N, device=DEV).expand(C, N)
+    r = p["radii"].float()
+    tiles = (2 * r[..., 0] / ts + 1).clamp(max=tw) * (2 * r[..., 1] / ts + 1).clamp(max=th)
+    estimate = float((d["opacities"][gid] * tiles)[visible & (p["radii"][..., 1] > 0)].sum()) / (C * tw * th)
+    assert 4 < estimate < 0.5 * MIN_OPACITY_PER_TILE  # a sparse little scene: the default fills
+    with torch.no_grad():
+        colors = view_dependent_colors(3, d["means"], d["viewmats"], coeffs, p["radii"], depths,
+                                       p["camera_ids"], p["gaussian_ids"])
+        want = rasterize_to_pixels(p["means2d"], p["conics"], colors, p["opacities"], p["pix_vels"], W, H,
+                                   ts, p["offsets"], p["flatten_ids"], d["rolling_shutter_time"], packed=packed)
+        for limit, filled in ((0.0, False), (0.5 * estimate, False), (2.0 * estimate, True),
+                              (float("inf"), True), (None, True)):
+            cache = view_dependent_color_cache(3, d["means"], d["viewmats"], coeffs, p["radii"], depths,
+                                               d["opacities"], ts, tw, th, p["camera_ids"], p["gaussian_ids"],
+                                               min_opacity_per_tile=limit)
+            assert cache.shape == tuple(visible.shape) + (4,)
+            if filled:
+                assert torch.equal(cache[visible][:, :3], colors[visible][:, :3])
+                assert torch.equal(cache[visible][:, 3],
+                                   depths[visible] if with_depth else torch.zeros_like(cache[visible][:, 3]))
+                assert bool(torch.isnan(cache[~visible]).all())
+            else:
+                assert bool(torch.isnan(cache).all())
+            got = rasterize_to_pixels_with_sh(3, d["means"], d["viewmats"], coeffs, depths, p["means2d"],
+                                              p["conics"], p["opacities"], p["pix_vels"], W, H, ts, p["offsets"],
+                                              p["flatten_ids"], d["rolling_shutter_time"],
+                                              gaussian_ids=p["gaussian_ids"], color_cache=cache)
+            assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+            if not filled:  # the rows that tiles staged now hold their colours, the others still NaN
+                held = ~torch.isnan(cache[..., 0])
+                assert bool(held.any()) and not bool(held[~visible].any())
+                assert torch.equal(cache[held][:, :3], colors[held][:, :3])
+
+
 def test_colours_while_compositing_is_forward_only_and_checks_its_rows():
     from splatad_amd.hip._wrapper import rasterize_to_pixels_with_sh
     d, p = _projected(1, 500, 64, 48, 16, False, seed=4)
