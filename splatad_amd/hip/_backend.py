@@ -193,7 +193,9 @@ class _Ops:
         stream, ordered behind the binning by the intersection call itself, and run beside the
         segment sort; the caller joins the stream before anything reads the outputs on its own
         stream (_isect() with the lists of these rows does not read them; without them it waits
-        for the stream left on the radii).  requests["colors"] = (degrees_to_use, coeffs,
+        for the stream left on the radii).  requests["color_cache"] = (degrees_to_use, coeffs,
+        with_depth, tile_size, tile_width, tile_height, min_opacity_per_tile) asks for what
+        view_colors_cache() makes of the packed rows; requests["colors"] = (degrees_to_use, coeffs,
         with_depth) and requests["opacities"] = opacities [N] ask for what view_colors_fwd() and
         the gather opacities[gaussian_ids] (* compensations) would give for the returned rows;
         they are made on the same stream and left in results under the same keys."""
@@ -282,6 +284,21 @@ class _Ops:
                         _u32(C), _u32(N), _u32(coeffs.shape[-2]), _u32(degree), _p(means), _p(viewmats),
                         _p(ws), _p(coeffs), _i32(coeffs.dim() == 4), _i32(bool(with_depth)), _p(colors), work))
                 results["colors"] = colors
+            if "color_cache" in requests:
+                # the colour cache of rasterize_to_pixels_sh_fwd for the packed rows, see
+                # view_colors_cache(); needs requests["opacities"]
+                degree, coeffs, with_depth, tile_size, tile_w, tile_h, limit = requests["color_cache"]
+                coeffs = _in(coeffs, "coeffs")
+                assert opacities is not None
+                words = lib.splatad_view_colors_cache_bytes(_u64(nnz)) // 4
+                buf = torch.empty((words,), **f)
+                if nnz:
+                    _check(lib.splatad_view_colors_cache(
+                        _u32(nnz), _u32(C), _u32(N), _u32(coeffs.shape[-2]), _u32(degree), _p(means),
+                        _p(viewmats), _p(camera_ids), _p(gaussian_ids), _p(radii), _p(coeffs),
+                        _i32(coeffs.dim() == 4), _p(depths if with_depth else None), _p(opacities),
+                        _u32(tile_size), _u32(tile_w), _u32(tile_h), _f32(limit), _p(buf), work))
+                results["color_cache"] = buf[: nnz * 4].view(nnz, 4)
             if beside is not None:
                 beside.results = results
             if side is not None:

@@ -13,6 +13,7 @@ from torch import Tensor
 from typing_extensions import Literal
 
 from .hip._wrapper import (
+    MIN_OPACITY_PER_TILE,
     fully_fused_lidar_projection,
     fully_fused_projection,
     isect_lidar_tiles,
@@ -199,6 +200,9 @@ def rasterization(
             t is not None and t.requires_grad for t in (means, quats, scales, opacities, velocities, viewmats))
         if no_grad and opacities.is_contiguous() and opacities.dtype == torch.float32:
             beside.requests["opacities"] = opacities
+            if colors_while_compositing and colors.is_contiguous():
+                beside.requests["color_cache"] = (sh_degree, colors, depth_appended, tile_size, tile_width,
+                                                  tile_height, MIN_OPACITY_PER_TILE)
     proj = fully_fused_projection(
         means, None, quats, scales, velocities, viewmats, Ks, width, height, linear_velocity,
         angular_velocity, rolling_shutter_time, eps2d=eps2d, packed=packed, near_plane=near_plane,
@@ -267,9 +271,11 @@ def rasterization(
         # stream: two short launches cost less there than a helper stream's fork and join)
         if packed:
             beside.join(opacities if beside_opacities and "opacities" not in beside.results else None)
-        color_cache = view_dependent_color_cache(
-            sh_degree, means, viewmats, colors, radii, depths if depth_appended else None,
-            opacities_per_gaussian, tile_size, tile_width, tile_height, camera_ids, gaussian_ids)
+        color_cache = beside.results.get("color_cache")  # made with the packed rows, beside the sort
+        if color_cache is None:
+            color_cache = view_dependent_color_cache(
+                sh_degree, means, viewmats, colors, radii, depths if depth_appended else None,
+                opacities_per_gaussian, tile_size, tile_width, tile_height, camera_ids, gaussian_ids)
     elif fused_colors:
         colors = fused_view_colors()
         made_beside = "colors" not in beside.results  # (what the projection made was allocated here)
