@@ -166,11 +166,11 @@ sh_cache_fill_kernel(uint32_t n, uint32_t K, uint32_t degree, ShView view, const
     float total = 0.f;
     for (uint32_t w = 0; w < blockDim.x / SPLATAD_WAVE; ++w) total += s_sum[w];
     if (total >= enough) return; // uniform across the launch
-    const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n) return;
-    if (view.radii[(size_t)e * 2] <= 0) return; // rows no list names keep their NaN
-    sh_fwd_row<true>(e, K, degree, view, nullptr, coeffs, nullptr, depths, 4u, cache, nullptr);
-    if (depths == nullptr) cache[(size_t)e * 4 + 3] = 0.f;
+    for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
+        if (view.radii[(size_t)e * 2] <= 0) continue; // rows no list names keep their NaN
+        sh_fwd_row<true>(e, K, degree, view, nullptr, coeffs, nullptr, depths, 4u, cache, nullptr);
+        if (depths == nullptr) cache[(size_t)e * 4 + 3] = 0.f;
+    }
 }
 
 // VIEW: v_colors are rows of `stride` floats, the gradients of the activated colours
@@ -376,7 +376,9 @@ extern "C" int splatad_view_colors_cache(uint32_t n, uint32_t C, uint32_t N, uin
                        view, opacities, 1.f / (float)tile_size, (float)tile_width, (float)tile_height,
                        reinterpret_cast<float4 *>(cache), partials);
     SPLATAD_LAUNCH_CHECK();
-    hipLaunchKernelGGL(sh_cache_fill_kernel, dim3((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS),
+    // (a launch that mostly finds nothing to do: no more workgroups than fill the GPU a few times)
+    const uint32_t rows_wgs = (n + SPLATAD_THREADS - 1) / SPLATAD_THREADS;
+    hipLaunchKernelGGL(sh_cache_fill_kernel, dim3(rows_wgs < 2048u ? rows_wgs : 2048u),
                        dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, n, K, degree, view, coeffs, depths, cache,
                        (const float *)partials, wgs, min_opacity_per_tile * n_tiles);
     SPLATAD_LAUNCH_CHECK();
