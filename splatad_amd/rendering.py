@@ -64,12 +64,14 @@ class _Beside:
     captured, the blocks simply run in place.
     """
 
-    def __init__(self, device):
+    def __init__(self, device, enabled=True):
+        # enabled=False: no helper stream; the blocks run in place, the requests to the packed
+        # projection are served on the caller's stream
         self.main = self.side = self.fork = self._ctx = self._waited = None
         # what the packed projection is asked to make on the helper stream, and what it made
         self.requests: Dict[str, object] = {}
         self.results: Dict[str, Tensor] = {}
-        if device.type == "cuda" and not torch.cuda.is_current_stream_capturing():
+        if enabled and device.type == "cuda" and not torch.cuda.is_current_stream_capturing():
             idx = device.index if device.index is not None else torch.cuda.current_device()
             key = (idx, threading.get_ident())
             if key not in _HELPER_STREAMS:
@@ -180,7 +182,6 @@ def rasterization(
     # (packed: the kernels that write the packed rows go to the helper stream, and with them
     # what else only needs the projection, the colours of step 3 and the rows' opacities; the
     # tile intersection works on the projection's dense rows and does not wait for any of it)
-    beside = _Beside(means.device)
     fused_colors = sh_degree is not None and not viewmats.requires_grad
     depth_appended = fused_colors and render_mode in ["RGB+D", "RGB+ED"]
     # Colours from spherical harmonics and no gradient wanted: the compositing kernel evaluates
@@ -192,6 +193,10 @@ def rasterization(
             t is not None and t.requires_grad
             for t in (means, quats, scales, opacities, colors, velocities, viewmats, backgrounds))))
     colors_beside = fused_colors and (packed or not colors_while_compositing)  # step 3 joins the helper stream
+    # (with the colours left to the compositing kernel nothing is worth a helper stream: a packed
+    # call's rows, opacities and colour cache, written on the caller's stream behind the sort, cost
+    # less than the fork, the join and a sort that shares the GPU)
+    beside = _Beside(means.device, enabled=not colors_while_compositing)
     if packed:
         if fused_colors and not colors_while_compositing and colors.is_contiguous():
             beside.requests["colors"] = (sh_degree, colors, depth_appended)
@@ -269,9 +274,7 @@ def rasterization(
         # the empty cache through which the tiles share the colours they evaluate, or, for a
         # scene whose tiles will not saturate early, all colours after all (on the caller's
         # stream: two short launches cost less there than a helper stream's fork and join)
-        if packed:
-            beside.join(opacities if beside_opacities and "opacities" not in beside.results else None)
-        color_cache = beside.results.get("color_cache")  # made with the packed rows, beside the sort
+        color_cache = beside.results.get("color_cache")  # what the packed projection made of its rows
         if color_cache is None:
             color_cache = view_dependent_color_cache(
                 sh_degree, means, viewmats, colors, radii, depths if depth_appended else None,
