@@ -423,28 +423,36 @@ packed_compact_kernel(uint32_t C, uint32_t N, int64_t nnz, const int32_t *__rest
                       float *__restrict__ conics, float *__restrict__ comps,
                       float *__restrict__ pix_vels, const float *__restrict__ opacities,
                       float *__restrict__ row_opacities) {
-    const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const uint64_t T = (uint64_t)C * N;
+    const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; // C * N < 2^31
+    const uint32_t T = C * N;
     if (idx >= T) return;
-    const uint32_t cid = (uint32_t)(idx / N), gid = (uint32_t)(idx % N);
+    const uint32_t cid = idx / N, gid = idx - cid * N;
+    // everything a kept row needs is requested before the test on the radius (culled rows of
+    // the workspace hold zeros): one memory round trip instead of two
     const int32_t o = pos[idx];
+    const int2 r = reinterpret_cast<const int2 *>(w_radii)[idx];
+    const float2 mean = reinterpret_cast<const float2 *>(w_means2d)[idx];
+    const float depth = w_depths[idx];
+    const float c0 = w_conics[(size_t)idx * 3], c1 = w_conics[(size_t)idx * 3 + 1], c2 = w_conics[(size_t)idx * 3 + 2];
+    const float2 vel = reinterpret_cast<const float2 *>(w_pix_vels)[idx];
+    const float comp = comps != nullptr ? w_comps[idx] : 1.f;
+    const float opacity = row_opacities != nullptr ? opacities[gid] : 0.f;
     if (gid == 0) indptr[cid] = o; // first element of each row holds the row start
     if (idx == T - 1) indptr[C] = (int32_t)nnz;
-    const int2 r = reinterpret_cast<const int2 *>(w_radii)[idx];
     if (r.x <= 0) return;
     camera_ids[o] = cid;
     gaussian_ids[o] = gid;
     reinterpret_cast<int2 *>(radii)[o] = r;
-    reinterpret_cast<float2 *>(means2d)[o] = reinterpret_cast<const float2 *>(w_means2d)[idx];
-    depths[o] = w_depths[idx];
-    conics[o * 3] = w_conics[idx * 3];
-    conics[o * 3 + 1] = w_conics[idx * 3 + 1];
-    conics[o * 3 + 2] = w_conics[idx * 3 + 2];
-    if (comps != nullptr) comps[o] = w_comps[idx];
-    reinterpret_cast<float2 *>(pix_vels)[o] = reinterpret_cast<const float2 *>(w_pix_vels)[idx];
+    reinterpret_cast<float2 *>(means2d)[o] = mean;
+    depths[o] = depth;
+    conics[(size_t)o * 3] = c0;
+    conics[(size_t)o * 3 + 1] = c1;
+    conics[(size_t)o * 3 + 2] = c2;
+    if (comps != nullptr) comps[o] = comp;
+    reinterpret_cast<float2 *>(pix_vels)[o] = vel;
     // the opacity the compositing takes for the row: the Gaussian's, times the compensation
     // when there is one (rendering.py:311-314 of the reference)
-    if (row_opacities != nullptr) row_opacities[o] = comps != nullptr ? opacities[gid] * w_comps[idx] : opacities[gid];
+    if (row_opacities != nullptr) row_opacities[o] = comps != nullptr ? opacity * comp : opacity;
 }
 
 __global__ void fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {

@@ -503,8 +503,10 @@ def rasterize_to_pixels_with_sh(
 
 # Opacity that a tile's list has to carry, by the estimate of view_dependent_color_cache, for the
 # colours to be left to the compositing kernel.  Measured on a 1080p frame of 1M Gaussians
-# whose opacities were scaled (estimate; colour kernel + compositing; colours while compositing):
-# 640: 0.156 / 0.135 ms; 128: 0.476 / 0.479 ms; 32: 1.150 / 1.551 ms.
+# whose opacities were scaled (estimate: colour kernel + compositing / compositing with the
+# colours left to it / with all colours put into the cache beforehand, in ms):
+# 1399: 0.159 / 0.139 / 0.178; 560: 0.284 / 0.274 / 0.294; 280: 0.445 / 0.456 / 0.453;
+# 140: 0.702 / 0.813 / 0.724; 70: 1.173 / 1.444 / 1.193.
 MIN_OPACITY_PER_TILE = 200.0
 
 
