@@ -551,6 +551,46 @@ constexpr int kSortClasses = 7;
 __constant__ const uint32_t kSortClassMin[kSortClasses + 1] = {0u,    512u,   2048u,  4096u,
                                                                8192u, 16384u, 32768u, 0x7FFFFFFFu};
 
+// A table scanned by scan_local_kernel holds prefixes inside scan blocks; what has to be added is
+// the sum of the blocks before an element's.  Every wavefront that needs it keeps those sums for
+// the (at most 128) blocks, two per lane.  before() is called by all lanes of the wavefront
+// together (it shuffles).
+struct ScanBlocks {
+    int32_t even, odd; // sums of the totals of the blocks before block 2 * lane and 2 * lane + 1
+    bool local;        // false: the table holds complete prefixes
+    bool summed;
+    // request() only issues the loads of the totals, so that a caller can issue other loads
+    // behind them before sum() waits for them.
+    __device__ __forceinline__ void request(const int64_t *__restrict__ totals, uint32_t n_blocks, uint32_t lane) {
+        local = totals != nullptr;
+        summed = !local;
+        even = odd = 0;
+        if (!local) return; // uniform
+        even = 2 * lane < n_blocks ? (int32_t)totals[2 * lane] : 0;
+        odd = 2 * lane + 1 < n_blocks ? (int32_t)totals[2 * lane + 1] : 0;
+    }
+    __device__ __forceinline__ void sum(uint32_t lane) {
+        if (summed) return; // uniform
+        summed = true;
+        const int32_t v0 = even, v1 = odd;
+        int32_t incl = v0 + v1;
+#pragma unroll
+        for (int off = 1; off < SPLATAD_WAVE; off <<= 1) {
+            const int32_t o = __shfl_up(incl, off, SPLATAD_WAVE);
+            if ((int)lane >= off) incl += o;
+        }
+        even = incl - v0 - v1;
+        odd = even + v0;
+    }
+    __device__ __forceinline__ int32_t before(uint32_t logical) const {
+        if (!local) return 0; // uniform
+        const uint32_t b = logical / SCAN_TILE;
+        const int32_t e = __shfl(even, (int)(b >> 1), SPLATAD_WAVE);
+        const int32_t o = __shfl(odd, (int)(b >> 1), SPLATAD_WAVE);
+        return (b & 1u) ? o : e;
+    }
+};
+
 // Enters segment `seg` (one per lane; lanes beyond n_segments idle) into the list of its size
 // class: seg_lists[c * n_segments + k], k < seg_counts[c] (zeroed beforehand).  The order inside
 // a class is whatever the atomics give; every segment is sorted on its own, so the result does
@@ -559,13 +599,20 @@ __constant__ const uint32_t kSortClassMin[kSortClasses + 1] = {0u,    512u,   20
 __device__ __forceinline__ void classify_segment(uint32_t seg, uint32_t lane, uint32_t n_segments,
                                                  uint32_t sshift, int64_t n_isects,
                                                  const int32_t *__restrict__ tile_starts,
+                                                 const ScanBlocks &scan, uint32_t copies,
+                                                 int32_t *__restrict__ seg_starts,
                                                  uint32_t *__restrict__ seg_counts,
                                                  uint32_t *__restrict__ seg_lists,
                                                  int32_t *__restrict__ tile_offsets) {
     uint32_t n = 0;
+    // the first copy of segment s is logical element s * copies of the scanned table
+    const int32_t before_here = scan.before(min(seg, n_segments - 1u) * copies);
+    const int32_t before_next = scan.before(min(seg + 1u, n_segments - 1u) * copies);
     if (seg < n_segments) {
-        const int64_t start = tile_starts[seg];
-        const int64_t stop = min(seg + 1 == n_segments ? n_isects : (int64_t)tile_starts[seg + 1], n_isects);
+        const int64_t start = (int64_t)tile_starts[seg] + before_here;
+        const int64_t stop = min(seg + 1 == n_segments ? n_isects : (int64_t)tile_starts[seg + 1] + before_next,
+                                 n_isects);
+        seg_starts[seg] = (int32_t)start; // what the sort kernels read
         n = stop > start ? (uint32_t)(stop - start) : 0u;
         if (tile_offsets != nullptr && (seg & ((1u << sshift) - 1u)) == 0)
             tile_offsets[seg >> sshift] = (int32_t)start;
@@ -603,17 +650,24 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
                       const int32_t *__restrict__ tile_starts, int32_t *__restrict__ tile_fill,
                       uint64_t *__restrict__ pairs, int64_t n_isects,
                       uint32_t *__restrict__ seg_counts, uint32_t *__restrict__ seg_lists,
-                      int32_t *__restrict__ tile_offsets) {
+                      int32_t *__restrict__ tile_offsets, const int64_t *__restrict__ scan_totals,
+                      uint32_t n_scan_blocks, int32_t *__restrict__ seg_starts) {
     const int64_t n_entries = *n_entries_ptr;
     const uint32_t lane = threadIdx.x & (SPLATAD_WAVE - 1);
     const int64_t wave_id = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / SPLATAD_WAVE;
     const int64_t n_waves = (int64_t)gridDim.x * blockDim.x / SPLATAD_WAVE;
+    // scan_totals: tile_starts holds prefixes inside scan blocks, and this kernel adds the
+    // blocks before (one scan launch instead of two)
+    ScanBlocks scan;
+    scan.request(FILL ? scan_totals : nullptr, n_scan_blocks, lane);
     // the filling pass also lists the segments by size class for the sort that follows (the
     // scanned starts are complete before this kernel begins): a lane per segment
     if (FILL && seg_lists != nullptr)
-        for (int64_t s0 = wave_id * SPLATAD_WAVE; s0 < (int64_t)n_segments; s0 += n_waves * SPLATAD_WAVE)
-            classify_segment((uint32_t)s0 + lane, lane, n_segments, sshift, n_isects, tile_starts,
-                             seg_counts, seg_lists, tile_offsets);
+        for (int64_t s0 = wave_id * SPLATAD_WAVE; s0 < (int64_t)n_segments; s0 += n_waves * SPLATAD_WAVE) {
+            scan.sum(lane);
+            classify_segment((uint32_t)s0 + lane, lane, n_segments, sshift, n_isects, tile_starts, scan,
+                             copies, seg_starts, seg_counts, seg_lists, tile_offsets);
+        }
     const uint32_t bits = 4u << cg.bshift, per_cam = cg.cw * cg.ch;
     const float inv_cw = 1.0f / (float)cg.cw;
     const uint32_t cap = (uint32_t)n_isects; // below 2^31
@@ -691,6 +745,7 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
         const bool has = e0 + lane < n_entries;
         const uint4 rec = has ? entries[e0 + lane] : make_uint4(0, 0, kNone, 0);
         const uint64_t pair = ((uint64_t)rec.y << 32) | (uint64_t)rec.x;
+        if (FILL) scan.sum(lane); // (the first round: behind the request for the entries)
         const uint64_t have = __ballot(has);
         // Nearly always the 256 entries of the workgroup belong to one block: then the four
         // wavefronts add up their counts in LDS and one of them issues the atomics, a quarter of
@@ -728,8 +783,11 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
             if (!FILL) {
                 if (wave == 0 && all) atomicAdd(&tile_counts[tile], (int32_t)all);
             } else {
+                // (tile - copy_base is the segment; its copy's logical element in the scanned table)
+                const int32_t blocks_before =
+                    scan.before((uint32_t)(tile - copy_base) * copies + (blockIdx.x & (copies - 1)));
                 if (wave == 0 && lane < 16)
-                    s_base[lane] = all ? tile_starts[tile] + atomicAdd(&tile_fill[tile], (int32_t)all) : 0;
+                    s_base[lane] = all ? tile_starts[tile] + blocks_before + atomicAdd(&tile_fill[tile], (int32_t)all) : 0;
                 __syncthreads();
                 const int32_t dst = lane < 16 ? s_base[lane] + (int32_t)before : 0;
                 write_group(mask, dst, pair);
@@ -749,7 +807,9 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
                     if (my_cnt) atomicAdd(&tile_counts[tile], (int32_t)my_cnt);
                 } else {
                     int32_t dst = 0;
-                    if (my_cnt) dst = tile_starts[tile] + atomicAdd(&tile_fill[tile], (int32_t)my_cnt);
+                    const int32_t blocks_before =
+                        scan.before((uint32_t)(tile - copy_base) * copies + (blockIdx.x & (copies - 1)));
+                    if (my_cnt) dst = tile_starts[tile] + blocks_before + atomicAdd(&tile_fill[tile], (int32_t)my_cnt);
                     write_group(mask, dst, pair);
                 }
             }
@@ -1468,6 +1528,7 @@ struct IsectWorkspace {
     int32_t *block_totals;        // [C * blocks] entries per coarse block (in the cleared part)
     int32_t *coarse_counts;       // [coarse workgroups * C * blocks] run starts inside the blocks' lists
     int32_t *tile_starts;         // [tile copies * segments]
+    int32_t *seg_starts;          // [segments] first entry of every segment, for the sort
     uint32_t *seg_counts;         // [kSortClasses] segments per size class (in the cleared part)
     uint32_t *seg_lists;          // [kSortClasses * segments]
     int64_t *block_sums;          // scan scratch
@@ -1554,6 +1615,7 @@ static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslo
     w.coarse_counts = (int32_t *)p;         p += splatad_align256(cslots * 4);
     w.tile_starts = (int32_t *)p;           p += splatad_align256(tslots * 4);
     w.seg_lists = (uint32_t *)p;            p += splatad_align256(segs * kSortClasses * 4);
+    w.seg_starts = (int32_t *)p;            p += splatad_align256(segs * 4);
     w.block_sums = (int64_t *)p;            p += scan_workspace_bytes((int64_t)scan_n);
     if (out) *out = w;
     return (size_t)(p - (char *)ws);
@@ -1804,18 +1866,29 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
                        w.tile_counts, (const int32_t *)nullptr, (int32_t *)nullptr,
                        (uint64_t *)nullptr, (int64_t)0, (uint32_t *)nullptr, (uint32_t *)nullptr,
-                       (int32_t *)nullptr);
+                       (int32_t *)nullptr, (const int64_t *)nullptr, 0u, (int32_t *)nullptr);
     SPLATAD_LAUNCH_CHECK();
-    rc = launch_exclusive_scan<int32_t>(w.tile_counts, (int64_t)(segs * tcopies),
-                                        tcopies > 1 ? -(int)tcopies : 1, 0, w.tile_starts,
-                                        w.scan_total, w.block_sums, stream);
+    // up to 128 scan blocks, i.e. any table of the size isect_copies() aims at: one scan launch,
+    // and the filling pass adds the blocks before an element itself
+    const int64_t scan_n = (int64_t)(segs * tcopies);
+    const int scan_stride = tcopies > 1 ? -(int)tcopies : 1;
+    uint32_t n_scan_blocks = 0;
+    const bool local_scan = scan_n <= kScanLocalBlocks * SCAN_TILE;
+    if (local_scan)
+        rc = launch_local_scan<int32_t>(w.tile_counts, scan_n, scan_stride, w.tile_starts, w.block_sums,
+                                        &n_scan_blocks, stream);
+    else
+        rc = launch_exclusive_scan<int32_t>(w.tile_counts, scan_n, scan_stride, 0, w.tile_starts,
+                                            w.scan_total, w.block_sums, stream);
     if (rc) return rc;
     hipLaunchKernelGGL((square ? isect_tile_bin_kernel<true, 16> : isect_tile_bin_kernel<true, 0>),
                        dim3((uint32_t)bin_wgs),
                        dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, sshift, tcopies,
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
                        w.tile_counts, (const int32_t *)w.tile_starts, w.tile_fill, w.pairs, n_isects,
-                       w.seg_counts, w.seg_lists, tile_offsets);
+                       w.seg_counts, w.seg_lists, tile_offsets,
+                       local_scan ? (const int64_t *)w.block_sums : (const int64_t *)nullptr, n_scan_blocks,
+                       w.seg_starts);
     SPLATAD_LAUNCH_CHECK();
     // Size classes: a launch per class (one for the three upper classes), so that the LDS per
     // workgroup (and with it the number of resident workgroups) fits the segment length; the
@@ -1837,12 +1910,12 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         int e;
 #define SPLATAD_SORT_CLASS(cls, ER, threads, hi, wgs, on)                                        \
         if ((e = launch_small_segment_sort<ER, LIDAR>(cls, threads, hi, wgs, nseg, n_tiles, sshift, tile_n_bits, \
-                                                      n_isects, w.seg_counts, w.seg_lists, w.tile_starts, \
+                                                      n_isects, w.seg_counts, w.seg_lists, w.seg_starts, \
                                                       w.pairs, isect_ids, flatten_ids, on)) != 0) \
             return e;
         // the upper classes go first, on the caller's stream, which does not wait for the fork
         if ((e = launch_big_segment_sort(256u, nseg, n_tiles, sshift, tile_n_bits, n_isects, w.seg_counts,
-                                         w.seg_lists, w.tile_starts, w.pairs, isect_ids, flatten_ids,
+                                         w.seg_lists, w.seg_starts, w.pairs, isect_ids, flatten_ids,
                                          stream)) != 0)
             return e;
         SPLATAD_SORT_CLASS(2, 8, 512, 4096u, 1024u, ss->aux[0])

@@ -159,6 +159,39 @@ scan_apply_kernel(const int32_t *__restrict__ in, int64_t n, int stride, int as_
 
 constexpr int64_t kScanFoldBlocks = 1024; // up to 2M elements: two launches instead of three
 
+// One launch for a consumer that finishes the scan itself: out holds every element's exclusive
+// prefix inside its block of SCAN_TILE logical elements, block_sums the blocks' totals; the
+// prefix of element i is out[phys(i)] + the sum of block_sums[0 .. i / SCAN_TILE).  For tables
+// of up to kScanLocalBlocks blocks, two per lane of a consumer's wavefront, which adds them up
+// with shuffles.
+constexpr int64_t kScanLocalBlocks = 2 * SPLATAD_WAVE;
+
+template <typename OutT>
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+scan_local_kernel(const int32_t *__restrict__ in, int64_t n, int stride, OutT *__restrict__ out,
+                  int64_t *__restrict__ block_sums) {
+    const int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+    int32_t v[SCAN_ITEMS];
+    int64_t s = 0;
+    ScanCursor c(base, n, stride);
+#pragma unroll
+    for (int k = 0; k < SCAN_ITEMS; ++k) {
+        v[k] = scan_load(in, c, base + k < n, 0);
+        s += v[k];
+        c.next();
+    }
+    int64_t tot;
+    int64_t run = block_exclusive_scan(s, &tot);
+    if (threadIdx.x == 0) block_sums[blockIdx.x] = tot;
+    ScanCursor o(base, n, stride > 0 ? 1 : stride);
+#pragma unroll
+    for (int k = 0; k < SCAN_ITEMS; ++k) {
+        if (base + k < n) out[o.phys] = (OutT)run;
+        run += v[k];
+        o.next();
+    }
+}
+
 static inline size_t scan_workspace_bytes(int64_t n) {
     int64_t n_blocks = (n + SCAN_TILE - 1) / SCAN_TILE;
     return splatad_align256((size_t)(n_blocks > 0 ? n_blocks : 1) * sizeof(int64_t));
@@ -192,6 +225,20 @@ static inline int launch_exclusive_scan_apply(const int32_t *in, int64_t n, int 
                            (const int64_t *)block_sums, out, total, 1u);
         SPLATAD_LAUNCH_CHECK();
     }
+    return 0;
+}
+
+// Returns the number of blocks through *n_blocks; the caller has checked n against
+// kScanLocalBlocks * SCAN_TILE.
+template <typename OutT>
+static inline int launch_local_scan(const int32_t *in, int64_t n, int stride, OutT *out,
+                                    int64_t *block_sums, uint32_t *n_blocks, hipStream_t stream) {
+    const int64_t blocks = (n + SCAN_TILE - 1) / SCAN_TILE;
+    SPLATAD_REQUIRE(n > 0 && blocks <= kScanLocalBlocks, "scan: %lld elements are too many for a local scan", (long long)n);
+    hipLaunchKernelGGL((scan_local_kernel<OutT>), dim3((uint32_t)blocks), dim3(SPLATAD_THREADS), 0, stream, in, n,
+                       stride, out, block_sums);
+    SPLATAD_LAUNCH_CHECK();
+    *n_blocks = (uint32_t)blocks;
     return 0;
 }
 
