@@ -179,9 +179,10 @@ def rasterization(
     # so that the host waits for the GPU once per call, not twice)
     tile_width = math.ceil(width / float(tile_size))
     tile_height = math.ceil(height / float(tile_size))
-    # (packed: the kernels that write the packed rows go to the helper stream, and with them
-    # what else only needs the projection, the colours of step 3 and the rows' opacities; the
-    # tile intersection works on the projection's dense rows and does not wait for any of it)
+    # (packed, in a call that wants gradients: the kernels that write the packed rows go to the
+    # helper stream, and with them what else only needs the projection, the colours of step 3 and
+    # the rows' opacities; the tile intersection works on the projection's dense rows and does
+    # not wait for any of it)
     fused_colors = sh_degree is not None and not viewmats.requires_grad
     depth_appended = fused_colors and render_mode in ["RGB+D", "RGB+ED"]
     # Colours from spherical harmonics and no gradient wanted: the compositing kernel evaluates
