@@ -176,7 +176,10 @@ int splatad_sh_bwd(uint32_t n, uint32_t K, uint32_t degree, const float *dirs,
  * (coeffs_per_sensor == 0) or [C, N, K, 3] (== 1).  colors has 3 channels, or 4 with depths.
  * _bwd takes the forward's colors (a channel passes its gradient only where it is positive)
  * and writes one row per e: v_coeffs [n, K, 3] (zero-filled by the caller) and, unless NULL,
- * v_dirs [n, 3]; the caller sums rows that share a Gaussian. */
+ * v_dirs [n, 3]; the caller sums rows that share a Gaussian.  With scatter_coeffs != 0 the
+ * kernel does that sum for the coefficients itself: v_coeffs then has the layout of coeffs
+ * ([N, K, 3] or [C, N, K, 3]), cleared by the caller, and every row's gradients are added, with
+ * atomics, at the coefficient row it read. */
 int splatad_view_colors_fwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
                             const float *means, const float *viewmats, const int64_t *camera_ids,
                             const int64_t *gaussian_ids, const int32_t *radii, const float *coeffs,
@@ -201,8 +204,8 @@ int splatad_view_colors_bwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint
                             const float *means, const float *viewmats, const int64_t *camera_ids,
                             const int64_t *gaussian_ids, const int32_t *radii, const float *coeffs,
                             int coeffs_per_sensor, uint32_t channels, const float *colors,
-                            const float *v_colors, float *v_coeffs, float *v_dirs,
-                            splatad_stream_t stream);
+                            const float *v_colors, int scatter_coeffs, float *v_coeffs,
+                            float *v_dirs, splatad_stream_t stream);
 
 /* ---- tile intersection, sort, offsets ----------------------------------- */
 

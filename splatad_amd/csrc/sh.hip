@@ -23,13 +23,13 @@ struct ShRows {
     uint32_t dq, dr; // blockDim.x / K3 and blockDim.x % K3
 };
 
-// f(lds_index, global_index) for every used float of the workgroup's `rows` rows
+// f(lds_index, global_index, row, column) for every used float of the workgroup's `rows` rows
 template <typename F>
 __device__ __forceinline__ void sh_for_each_float(const ShRows &r, uint32_t rows, F &&f) {
     uint32_t row = threadIdx.x / r.K3, col = threadIdx.x % r.K3;
     const uint32_t total = rows * r.K3;
     for (uint32_t e = threadIdx.x; e < total; e += blockDim.x) {
-        if (col < r.used) f(row * (r.used + 1) + col, e);
+        if (col < r.used) f(row * (r.used + 1) + col, e, row, col);
         row += r.dq;
         col += r.dr;
         if (col >= r.K3) { col -= r.K3; ++row; }
@@ -184,8 +184,11 @@ sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, ShView view, const float
               const float *__restrict__ coeffs, const uint8_t *__restrict__ masks,
               const float *__restrict__ colors, uint32_t stride,
               const float *__restrict__ v_colors, float *__restrict__ v_coeffs,
-              float *__restrict__ v_dirs) {
+              float *__restrict__ v_dirs, int scatter) {
     extern __shared__ float s_rows[];
+    // scatter: v_coeffs has the layout of coeffs, cleared by the caller, and every row's
+    // gradients are added at the coefficient row it read (packed rows: the Gaussian's)
+    uint32_t *s_dest = reinterpret_cast<uint32_t *>(s_rows + (size_t)blockDim.x * (rows.used + 1));
     const uint32_t first = blockIdx.x * blockDim.x;
     const uint32_t here = min(blockDim.x, n - first);
     const uint32_t e = first + threadIdx.x;
@@ -196,6 +199,7 @@ sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, ShView view, const float
         float dx = 0.f, dy = 0.f, dz = 0.f;
         size_t coeff_row;
         const bool active = sh_row<VIEW>(e, view, dirs, masks, dx, dy, dz, coeff_row);
+        if (scatter) s_dest[threadIdx.x] = (uint32_t)coeff_row;
         const float *cf = coeffs + coeff_row * rows.K3;
         const float inorm = active ? rsqrtf(dx * dx + dy * dy + dz * dz) : 0.f;
         const float x = dx * inorm, y = dy * inorm, z = active ? dz * inorm : 1.f;
@@ -237,8 +241,15 @@ sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, ShView view, const float
         }
     }
     __syncthreads();
+    if (scatter) { // uniform
+        sh_for_each_float(rows, here, [&](uint32_t l, uint32_t, uint32_t row_here, uint32_t col) {
+            const float v = s_rows[l];
+            if (v != 0.f) atomicAdd(v_coeffs + (size_t)s_dest[row_here] * rows.K3 + col, v);
+        });
+        return;
+    }
     float *gout = v_coeffs + (size_t)first * rows.K3;
-    sh_for_each_float(rows, here, [&](uint32_t l, uint32_t f) { gout[f] = s_rows[l]; });
+    sh_for_each_float(rows, here, [&](uint32_t l, uint32_t f, uint32_t, uint32_t) { gout[f] = s_rows[l]; });
 }
 
 static ShRows sh_rows(uint32_t K, uint32_t degree) {
@@ -252,7 +263,7 @@ static ShRows sh_rows(uint32_t K, uint32_t degree) {
 
 template <typename Kernel>
 static int sh_lds(Kernel kernel, const ShRows &r, size_t *bytes) {
-    *bytes = (size_t)SPLATAD_THREADS * (r.used + 1) * sizeof(float);
+    *bytes = (size_t)SPLATAD_THREADS * (r.used + 1) * sizeof(float) + SPLATAD_THREADS * sizeof(uint32_t);
     if (*bytes > 64 * 1024)
         SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)kernel,
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)*bytes));
@@ -280,18 +291,18 @@ template <bool VIEW>
 static int sh_backward(uint32_t n, uint32_t K, uint32_t degree, const ShView &view, const float *dirs,
                        const float *coeffs, const uint8_t *masks, const float *colors,
                        uint32_t stride, const float *v_colors, float *v_coeffs, float *v_dirs,
-                       hipStream_t stream) {
+                       hipStream_t stream, int scatter = 0) {
     const ShRows r = sh_rows(K, degree);
     size_t lds = 0;
     const dim3 grid((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS);
     if (v_dirs != nullptr) {
         if (int rc = sh_lds(sh_bwd_kernel<VIEW, true>, r, &lds)) return rc;
         hipLaunchKernelGGL((sh_bwd_kernel<VIEW, true>), grid, dim3(SPLATAD_THREADS), lds, stream, n, r,
-                           degree, view, dirs, coeffs, masks, colors, stride, v_colors, v_coeffs, v_dirs);
+                           degree, view, dirs, coeffs, masks, colors, stride, v_colors, v_coeffs, v_dirs, scatter);
     } else {
         if (int rc = sh_lds(sh_bwd_kernel<VIEW, false>, r, &lds)) return rc;
         hipLaunchKernelGGL((sh_bwd_kernel<VIEW, false>), grid, dim3(SPLATAD_THREADS), lds, stream, n, r,
-                           degree, view, dirs, coeffs, masks, colors, stride, v_colors, v_coeffs, v_dirs);
+                           degree, view, dirs, coeffs, masks, colors, stride, v_colors, v_coeffs, v_dirs, scatter);
     }
     SPLATAD_LAUNCH_CHECK();
     return 0;
@@ -408,8 +419,8 @@ extern "C" int splatad_view_colors_bwd(uint32_t n, uint32_t C, uint32_t N, uint3
                                        const int64_t *camera_ids, const int64_t *gaussian_ids,
                                        const int32_t *radii, const float *coeffs,
                                        int coeffs_per_sensor, uint32_t channels, const float *colors,
-                                       const float *v_colors, float *v_coeffs, float *v_dirs,
-                                       splatad_stream_t stream) {
+                                       const float *v_colors, int scatter_coeffs, float *v_coeffs,
+                                       float *v_dirs, splatad_stream_t stream) {
     if (int rc = sh_check(K, degree)) return rc;
     if (n == 0) return 0;
     ShView view;
@@ -418,5 +429,5 @@ extern "C" int splatad_view_colors_bwd(uint32_t n, uint32_t C, uint32_t N, uint3
     SPLATAD_REQUIRE(channels == 3 || channels == 4, "view colours: %u channels per row", channels);
     SPLATAD_REQUIRE(coeffs && colors && v_colors && v_coeffs, "view colours: null pointer argument");
     return sh_backward<true>(n, K, degree, view, nullptr, coeffs, nullptr, colors, channels, v_colors,
-                             v_coeffs, v_dirs, (hipStream_t)stream);
+                             v_coeffs, v_dirs, (hipStream_t)stream, scatter_coeffs);
 }

@@ -24,7 +24,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libsplatad_hip.so")
 _lib = None
 
 
-ABI_VERSION = 6  # splatad_abi_version() of the library these bindings were written for
+ABI_VERSION = 7  # splatad_abi_version() of the library these bindings were written for
 
 
 def load_library():
@@ -521,8 +521,9 @@ class _Ops:
         return buf[: n * 4].view(lead + (4,))
 
     def view_colors_bwd(self, degrees_to_use, means, viewmats, camera_ids, gaussian_ids, radii,
-                        coeffs, colors, v_colors, compute_v_dirs):
-        """Per-row gradients (v_coeffs [..., K, 3], v_dirs [..., 3] | None) of view_colors_fwd."""
+                        coeffs, colors, v_colors, compute_v_dirs, scatter_coeffs=False):
+        """Per-row gradients (v_coeffs [..., K, 3], v_dirs [..., 3] | None) of view_colors_fwd;
+        with scatter_coeffs, v_coeffs is summed over the rows of a Gaussian and shaped like coeffs."""
         lib = load_library()
         means = _in(means, "means"); viewmats = _in(viewmats, "viewmats")
         camera_ids = _in(camera_ids, "camera_ids", torch.int64)
@@ -535,14 +536,18 @@ class _Ops:
         f = dict(dtype=torch.float32, device=dev)
         # the kernel writes the floats of the bases in use; the others must read zero
         full = (degrees_to_use + 1) ** 2 == K
-        v_coeffs = (torch.empty if full else torch.zeros)(lead + (K, 3), **f)
+        if scatter_coeffs:
+            # gradients in the layout of coeffs: the kernel adds every row's at its Gaussian's
+            v_coeffs = torch.zeros_like(coeffs)
+        else:
+            v_coeffs = (torch.empty if full else torch.zeros)(lead + (K, 3), **f)
         v_dirs = torch.empty(lead + (3,), **f) if compute_v_dirs else None
         with _on(dev):
             _check(lib.splatad_view_colors_bwd(
                 _u32(n), _u32(C), _u32(N), _u32(K), _u32(degrees_to_use), _p(means), _p(viewmats),
                 _p(camera_ids), _p(gaussian_ids), _p(radii), _p(coeffs), _i32(coeffs.dim() == 4),
-                _u32(colors.shape[-1]), _p(colors), _p(v_colors), _p(v_coeffs), _p(v_dirs),
-                _stream(dev)))
+                _u32(colors.shape[-1]), _p(colors), _p(v_colors), _i32(bool(scatter_coeffs)), _p(v_coeffs),
+                _p(v_dirs), _stream(dev)))
         return v_coeffs, v_dirs
 
     # ------------------------------------------------------------------ intersection

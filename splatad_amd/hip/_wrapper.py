@@ -1128,13 +1128,18 @@ class _ViewColors(torch.autograd.Function):
         need_means, need_coeffs = ctx.needs_input_grad[1], ctx.needs_input_grad[3]
         v_means = v_coeffs = v_depths = None
         if need_means or need_coeffs:
+            # rows of one Gaussian seen by several sensors add up; for packed rows the kernel adds
+            # the coefficient gradients at their Gaussians itself (one pass over them instead of
+            # a [nnz, K, 3] tensor and an index_add_ over it)
+            packed = camera_ids is not None
+            scatter = packed and need_coeffs
             v_rows, v_dirs = _make_lazy_hip_func("view_colors_bwd")(
                 ctx.sh_degree, means, viewmats, camera_ids, gaussian_ids, radii, coeffs, colors,
-                v_colors.contiguous(), need_means)
-            # rows of one Gaussian seen by several sensors add up
-            packed = camera_ids is not None
+                v_colors.contiguous(), need_means, scatter)
             if need_coeffs:
-                if coeffs.dim() == 4:
+                if scatter:
+                    v_coeffs = v_rows
+                elif coeffs.dim() == 4:
                     v_coeffs = (torch.zeros_like(coeffs).index_put_((camera_ids, gaussian_ids), v_rows, accumulate=True)
                                 if packed else v_rows)
                 elif packed:
