@@ -45,6 +45,15 @@ def _sensor_motion(C, device, linear_velocity, angular_velocity, rolling_shutter
     return linear_velocity, angular_velocity, rolling_shutter_time
 
 
+# Whether rasterization() puts the work that only depends on the projection (colour kernel,
+# packed rows, their opacities) on a helper stream beside the tile intersection.  Off: measured
+# on the 1M-Gaussian 1080p frame, that work enqueued on the caller's stream behind the sort costs
+# the same or 6-9 us less in every mode but one (packed, colours from spherical harmonics and
+# gradients wanted: 0.468 against 0.462 ms) -- kernels that share the GPU share its wave slots
+# and memory system, and a fork and a join cost 20 us of their own -- and a call then uses one
+# stream only.
+HELPER_STREAM = False
+
 # one helper stream per (device, host thread): calls from different threads do not wait for one
 # another's helper work
 _HELPER_STREAMS: Dict[Tuple[int, int], "torch.cuda.Stream"] = {}
@@ -194,10 +203,7 @@ def rasterization(
             t is not None and t.requires_grad
             for t in (means, quats, scales, opacities, colors, velocities, viewmats, backgrounds))))
     colors_beside = fused_colors and (packed or not colors_while_compositing)  # step 3 joins the helper stream
-    # (with the colours left to the compositing kernel nothing is worth a helper stream: a packed
-    # call's rows, opacities and colour cache, written on the caller's stream behind the sort, cost
-    # less than the fork, the join and a sort that shares the GPU)
-    beside = _Beside(means.device, enabled=not colors_while_compositing)
+    beside = _Beside(means.device, enabled=HELPER_STREAM and not colors_while_compositing)
     if packed:
         if fused_colors and not colors_while_compositing and colors.is_contiguous():
             beside.requests["colors"] = (sh_degree, colors, depth_appended)

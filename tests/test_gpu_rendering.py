@@ -500,6 +500,32 @@ def test_surround_packed_equals_unpacked_for_every_option(opts):
 
 
 @pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("sh", [False, True])
+def test_helper_stream_switch_renders_the_same(packed, sh, monkeypatch):
+    """rendering.HELPER_STREAM (off by default) moves the colour kernel, the packed rows and their
+    opacities to a helper stream beside the tile intersection: same images and gradients."""
+    import splatad_amd.rendering as rendering
+    s = workloads.camera_driving(n=20000, width=320, height=180, n_cameras=2, sh_degree=3 if sh else None)
+    d = workloads.to_device(s, DEV)
+    kw = dict(near_plane=d["near_plane"], far_plane=d["far_plane"], eps2d=d["eps2d"], tile_size=16,
+              sh_degree=3 if sh else None, render_mode="RGB+D", packed=packed)
+    rest = (d["velocities"], d["viewmats"], d["Ks"], d["width"], d["height"], d["linear_velocity"],
+            d["angular_velocity"], d["rolling_shutter_time"])
+    out = {}
+    for helper in (False, True):
+        monkeypatch.setattr(rendering, "HELPER_STREAM", helper)
+        leaves = [d[k].clone().requires_grad_() for k in ("means", "opacities", "colors")]
+        rc, ra, _ = rendering.rasterization(leaves[0], d["quats"], d["scales"], leaves[1], leaves[2], *rest, **kw)
+        (rc.sum() + 2.0 * ra.sum()).backward()
+        torch.cuda.synchronize()
+        out[helper] = (rc.detach(), ra.detach(), [t.grad for t in leaves])
+    assert torch.equal(out[False][0], out[True][0]) and torch.equal(out[False][1], out[True][1])
+    # (the backward kernels add with float atomics, so two runs differ in the last bits anyway)
+    for a, b in zip(out[False][2], out[True][2]):
+        torch.testing.assert_close(a, b, rtol=1e-3, atol=1e-3 * float(a.abs().max()))
+
+
+@pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("case", ["behind", "between_tiles"])
 def test_camera_frames_without_rows_or_without_intersections(packed, case):
     """Nothing in front of the camera (no packed rows at all), and Gaussians that are kept by the
