@@ -399,7 +399,7 @@ __device__ __forceinline__ uint32_t coarse_mask(const LaneWork &w, const CoarseG
 // of the depths (weight = tiles met), so the sub-segments of an average tile are about equal;
 // any bounds whatsoever give the same output, balance is all they decide.
 constexpr uint32_t kSlabShiftMax = 4;
-constexpr uint32_t kSlabSamples = 512;
+constexpr uint32_t kSlabSamples = 256;
 // Slabs pay once a tile's segment outgrows the sort's short classes (beyond about 8000 entries,
 // i.e. several hundred Gaussians per tile); below that they only lengthen the binning.  Measured
 // on lidar sweeps of 0.25-4M Gaussians on 1024 tiles (whole call in ms with 0 / 4 / 8 / 16 slabs:
