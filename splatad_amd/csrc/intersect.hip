@@ -134,23 +134,122 @@ __device__ __forceinline__ uint32_t tile_index(const TileGrid &g, int32_t y, int
 // and zero again when it ends) takes the partial sums; the total goes to the host's pinned
 // slot.  On its way the kernel clears `clear_words` words from `clear` on: the counters of the
 // binning kernels behind it, which spares the launch of a clearing kernel.
+constexpr uint32_t kSlabSamples = 256;
+
+template <typename Load, typename Store>
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t L, uint32_t tid, uint32_t nt,
+                                                         uint32_t *s_wave, Load &&load, Store &&store) {
+    const uint32_t lane = tid & (SPLATAD_WAVE - 1), wave = tid / SPLATAD_WAVE;
+    const uint32_t per = (L + nt - 1) / nt;
+    const uint32_t b0 = min(L, tid * per), b1 = min(L, b0 + per);
+    uint32_t sum = 0;
+    for (uint32_t b = b0; b < b1; ++b) sum += load(b);
+    uint32_t incl = sum;
+#pragma unroll
+    for (int off = 1; off < SPLATAD_WAVE; off <<= 1) {
+        const uint32_t o = (uint32_t)__shfl_up((int)incl, off, SPLATAD_WAVE);
+        if ((int)lane >= off) incl += o;
+    }
+    if (lane == SPLATAD_WAVE - 1) s_wave[wave] = incl;
+    __syncthreads();
+    uint32_t run = incl - sum, total = 0;
+    for (uint32_t w = 0; w < nt / SPLATAD_WAVE; ++w) {
+        const uint32_t v = s_wave[w];
+        if (w < wave) run += v;
+        total += v;
+    }
+    for (uint32_t b = b0; b < b1; ++b) {
+        const uint32_t v = load(b);
+        store(b, run, v);
+        run += v;
+    }
+    __syncthreads();
+    return total;
+}
+
+// One workgroup, one sample per lane: kSlabSamples Gaussians at a fixed stride, ordered by
+// depth (every lane counts the smaller keys; all lanes read the same LDS words, which are
+// broadcasts).  A key is the depth bits with the sample's index in the low bits, which makes
+// the keys distinct at a depth resolution of 2^-14, plenty for a bound.  Bound k is the key at
+// which the running sum of the samples' tile counts passes k / n_slabs of the total.
+// weight_of(i): the tiles Gaussian i meets.  Run by one workgroup of the counting kernel, beside
+// the workgroups that count (as a launch of its own it stood in the chain of dependent kernels:
+// 6 us and a launch gap per lidar call).
+template <typename Weight>
+__device__ __forceinline__ void slab_bounds_workgroup(uint64_t total, const float *__restrict__ depths,
+                                                      Weight &&weight_of, uint32_t n_slabs,
+                                                      uint32_t *__restrict__ bounds) {
+    static_assert((kSlabSamples & (kSlabSamples - 1)) == 0 && kSlabSamples % 4 == 0, "power of two");
+    static_assert(kSlabSamples == SPLATAD_THREADS, "one sample per lane of a counting workgroup");
+    __shared__ __align__(16) uint32_t s_key[kSlabSamples];
+    __shared__ uint32_t s_sorted[kSlabSamples];
+    __shared__ uint32_t s_weight[kSlabSamples];
+    __shared__ uint32_t s_before[kSlabSamples];
+    __shared__ uint32_t s_wave[2 * (kSlabSamples / SPLATAD_WAVE)];
+    const uint32_t tid = threadIdx.x;
+    const uint64_t n = total < kSlabSamples ? total : kSlabSamples;
+    const uint64_t stride = n ? total / n : 1;
+    uint32_t key = ~(kSlabSamples - 1u) | tid, weight = 0; // no tiles: behind every depth
+    if (tid < n) {
+        const int32_t w = weight_of(tid * stride);
+        if (w > 0) {
+            key = (__float_as_uint(depths[tid * stride]) & ~(kSlabSamples - 1u)) | tid;
+            weight = (uint32_t)min(w, 1 << 20); // capped: the sum stays below 2^32
+        }
+    }
+    s_key[tid] = key;
+    if (tid < n_slabs) bounds[tid] = 0xFFFFFFFFu;
+    __syncthreads();
+    uint32_t rank = 0;
+    for (uint32_t j = 0; j < kSlabSamples; j += 4) {
+        const uint4 q = *reinterpret_cast<const uint4 *>(&s_key[j]);
+        rank += (q.x < key ? 1u : 0u) + (q.y < key ? 1u : 0u) + (q.z < key ? 1u : 0u) + (q.w < key ? 1u : 0u);
+    }
+    s_sorted[rank] = key;
+    s_weight[rank] = weight;
+    __syncthreads();
+    const uint32_t sum = block_exclusive_scan(
+        kSlabSamples, tid, kSlabSamples, s_wave, [&](uint32_t i) { return s_weight[i]; },
+        [&](uint32_t i, uint32_t before, uint32_t) { s_before[i] = before; });
+    const uint32_t w = s_weight[tid], before = s_before[tid];
+    if (w == 0) return;
+    for (uint32_t k = 1; k < n_slabs; ++k) {
+        const uint32_t target = (uint32_t)((uint64_t)sum * k / n_slabs);
+        if (before < target && target <= before + w) bounds[k - 1] = s_sorted[tid];
+    }
+}
+
 constexpr uint32_t kCountGroups = 32;
 constexpr uint32_t kCountWords = 8 + 8 * kCountGroups;
-template <bool LIDAR>
+template <bool LIDAR, bool SLABS>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d,
                    const void *__restrict__ radii, int32_t *__restrict__ tiles_per_gauss,
                    unsigned long long *__restrict__ counters,
                    unsigned long long *__restrict__ n_isects_host, int32_t *__restrict__ clear,
-                   uint64_t clear_words) {
+                   uint64_t clear_words, const float *__restrict__ depths, uint32_t n_slabs,
+                   uint32_t *__restrict__ slab_bounds) {
     SPLATAD_STAGE_ELEVATIONS(g)
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words;
          i += (uint64_t)gridDim.x * blockDim.x)
         clear[i] = 0;
+    // SLABS: the launch has one workgroup more than count, and that one finds the depth slabs'
+    // bounds meanwhile (it counts the tiles of its samples itself)
+    const uint32_t n_wgs = gridDim.x - (SLABS ? 1u : 0u);
+    if (SLABS && blockIdx.x == n_wgs) { // uniform across the workgroup
+        slab_bounds_workgroup(total, depths, [&](uint64_t i) -> int32_t {
+            float2 mu = reinterpret_cast<const float2 *>(means2d)[i];
+            uint2 rad = reinterpret_cast<const uint2 *>(radii)[i];
+            int32_t x0, y0, x1, y1;
+            if (!tile_rect_of<LIDAR>(g, mu, rad, x0, y0, x1, y1)) return 0;
+            return max(y1 - y0, 0) * max(x1 - x0, 0);
+        }, n_slabs, slab_bounds);
+        return;
+    }
     long long s = 0;
     // four Gaussians per lane and step, so that their loads are in flight together (the
     // kernel is bound by memory latency otherwise)
-    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    const uint64_t stride = (uint64_t)n_wgs * blockDim.x;
     for (uint64_t i0 = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i0 < total; i0 += 4 * stride) {
         float2 mu[4];
         uint2 rad[4];
@@ -200,9 +299,9 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
         // the pinned slot: no copy command, no event and no system-scope fence stand between
         // this kernel and the host or the work enqueued behind it.
         const unsigned long long one = 1ull << 48, low = one - 1ull;
-        const uint32_t groups = min(gridDim.x, kCountGroups);
+        const uint32_t groups = min(n_wgs, kCountGroups);
         const uint32_t group = blockIdx.x % groups;
-        const uint32_t members = gridDim.x / groups + (group < gridDim.x % groups ? 1u : 0u);
+        const uint32_t members = n_wgs / groups + (group < n_wgs % groups ? 1u : 0u);
         // The counters are put back to zero on the way, each by the last workgroup that touches
         // it, with an exchange whose result the next step needs: the exchange has been performed
         // before the report that depends on it is issued, so by the time the host sees the total
@@ -399,7 +498,6 @@ __device__ __forceinline__ uint32_t coarse_mask(const LaneWork &w, const CoarseG
 // of the depths (weight = tiles met), so the sub-segments of an average tile are about equal;
 // any bounds whatsoever give the same output, balance is all they decide.
 constexpr uint32_t kSlabShiftMax = 4;
-constexpr uint32_t kSlabSamples = 256;
 // Slabs pay once a tile's segment outgrows the sort's short classes (beyond about 8000 entries,
 // i.e. several hundred Gaussians per tile); below that they only lengthen the binning.  Measured
 // on lidar sweeps of 0.25-4M Gaussians on 1024 tiles (whole call in ms with 0 / 4 / 8 / 16 slabs:
@@ -430,37 +528,6 @@ __device__ __forceinline__ uint32_t slab_of(uint32_t d, const uint32_t *bounds, 
 // Exclusive scan over L values held in LDS by a workgroup of nt threads (a multiple of 64):
 // thread t owns ceil(L / nt) consecutive values; load(i) gives value i, store(i, before, v)
 // receives the sum of the values before i.  Returns the total.  Ends with a barrier.
-template <typename Load, typename Store>
-__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t L, uint32_t tid, uint32_t nt,
-                                                         uint32_t *s_wave, Load &&load, Store &&store) {
-    const uint32_t lane = tid & (SPLATAD_WAVE - 1), wave = tid / SPLATAD_WAVE;
-    const uint32_t per = (L + nt - 1) / nt;
-    const uint32_t b0 = min(L, tid * per), b1 = min(L, b0 + per);
-    uint32_t sum = 0;
-    for (uint32_t b = b0; b < b1; ++b) sum += load(b);
-    uint32_t incl = sum;
-#pragma unroll
-    for (int off = 1; off < SPLATAD_WAVE; off <<= 1) {
-        const uint32_t o = (uint32_t)__shfl_up((int)incl, off, SPLATAD_WAVE);
-        if ((int)lane >= off) incl += o;
-    }
-    if (lane == SPLATAD_WAVE - 1) s_wave[wave] = incl;
-    __syncthreads();
-    uint32_t run = incl - sum, total = 0;
-    for (uint32_t w = 0; w < nt / SPLATAD_WAVE; ++w) {
-        const uint32_t v = s_wave[w];
-        if (w < wave) run += v;
-        total += v;
-    }
-    for (uint32_t b = b0; b < b1; ++b) {
-        const uint32_t v = load(b);
-        store(b, run, v);
-        run += v;
-    }
-    __syncthreads();
-    return total;
-}
-
 // Coarse binning with one global atomic per (workgroup, block).  A fixed grid of workgroups
 // strides over the Gaussians; each keeps the counters of all coarse blocks in LDS.  COUNT pass:
 // at its end the workgroup adds its count of every block to the block's total (`totals`, zero
@@ -885,54 +952,6 @@ constexpr uint32_t kSortDirectMax = 64;     // fullest bin it accepts
 __host__ __device__ inline uint32_t sort_bucket_capacity(uint32_t max_n) {
     const uint32_t split = max_n / kSortBucketMean < kSortSplit ? max_n / kSortBucketMean : kSortSplit;
     return split + kSortFineBins + 1;
-}
-
-// One workgroup, one sample per lane: kSlabSamples Gaussians at a fixed stride, ordered by
-// depth (every lane counts the smaller keys; all lanes read the same LDS words, which are
-// broadcasts).  A key is the depth bits with the sample's index in the low bits, which makes
-// the keys distinct at a depth resolution of 2^-14, plenty for a bound.  Bound k is the key at
-// which the running sum of the samples' tile counts passes k / n_slabs of the total.
-__global__ void __launch_bounds__(kSlabSamples)
-isect_slab_bounds_kernel(uint64_t total, const float *__restrict__ depths,
-                         const int32_t *__restrict__ tiles_per_gauss, uint32_t n_slabs,
-                         uint32_t *__restrict__ bounds) {
-    static_assert((kSlabSamples & (kSlabSamples - 1)) == 0 && kSlabSamples % 4 == 0, "power of two");
-    __shared__ __align__(16) uint32_t s_key[kSlabSamples];
-    __shared__ uint32_t s_sorted[kSlabSamples];
-    __shared__ uint32_t s_weight[kSlabSamples];
-    __shared__ uint32_t s_before[kSlabSamples];
-    __shared__ uint32_t s_wave[2 * (kSlabSamples / SPLATAD_WAVE)];
-    const uint32_t tid = threadIdx.x;
-    const uint64_t n = total < kSlabSamples ? total : kSlabSamples;
-    const uint64_t stride = n ? total / n : 1;
-    uint32_t key = ~(kSlabSamples - 1u) | tid, weight = 0; // no tiles: behind every depth
-    if (tid < n) {
-        const int32_t w = tiles_per_gauss[tid * stride];
-        if (w > 0) {
-            key = (__float_as_uint(depths[tid * stride]) & ~(kSlabSamples - 1u)) | tid;
-            weight = (uint32_t)min(w, 1 << 20); // capped: the sum stays below 2^32
-        }
-    }
-    s_key[tid] = key;
-    if (tid < n_slabs) bounds[tid] = 0xFFFFFFFFu;
-    __syncthreads();
-    uint32_t rank = 0;
-    for (uint32_t j = 0; j < kSlabSamples; j += 4) {
-        const uint4 q = *reinterpret_cast<const uint4 *>(&s_key[j]);
-        rank += (q.x < key ? 1u : 0u) + (q.y < key ? 1u : 0u) + (q.z < key ? 1u : 0u) + (q.w < key ? 1u : 0u);
-    }
-    s_sorted[rank] = key;
-    s_weight[rank] = weight;
-    __syncthreads();
-    const uint32_t sum = block_exclusive_scan(
-        kSlabSamples, tid, kSlabSamples, s_wave, [&](uint32_t i) { return s_weight[i]; },
-        [&](uint32_t i, uint32_t before, uint32_t) { s_before[i] = before; });
-    const uint32_t w = s_weight[tid], before = s_before[tid];
-    if (w == 0) return;
-    for (uint32_t k = 1; k < n_slabs; ++k) {
-        const uint32_t target = (uint32_t)((uint64_t)sum * k / n_slabs);
-        if (before < target && target <= before + w) bounds[k - 1] = s_sorted[tid];
-    }
 }
 
 // One workgroup per (camera, tile) segment: a bucket sort on the depth in three steps.
@@ -1769,9 +1788,13 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     if (!skip_count) {
         dim3 count_grid = grid_for(total);
         if (count_grid.x > 1024) count_grid.x = 1024;
-        hipLaunchKernelGGL(isect_count_kernel<LIDAR>, count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
+        const bool slabs = sort && pl.sshift != 0; // one more workgroup finds the slabs' bounds
+        if (slabs) count_grid.x += 1;
+        hipLaunchKernelGGL((slabs ? isect_count_kernel<LIDAR, true> : isect_count_kernel<LIDAR, false>),
+                           count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
                            total, means2d, radii, tiles_per_gauss, counters, lease.word.device,
-                           w.zeroed, sort ? w.n_zeroed : (uint64_t)0);
+                           w.zeroed, sort ? w.n_zeroed : (uint64_t)0, depths, 1u << pl.sshift,
+                           slabs ? w.slab_bounds : (uint32_t *)nullptr);
         SPLATAD_LAUNCH_CHECK();
     } else {
         hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(w.n_zeroed), dim3(SPLATAD_THREADS), 0, stream,
@@ -1780,11 +1803,6 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     }
     // work for the GPU while the host learns the count and sizes the lists
     if (sort) {
-        if (pl.sshift) {
-            hipLaunchKernelGGL(isect_slab_bounds_kernel, dim3(1), dim3(kSlabSamples), 0, stream, total,
-                               depths, (const int32_t *)tiles_per_gauss, 1u << pl.sshift, w.slab_bounds);
-            SPLATAD_LAUNCH_CHECK();
-        }
         if (int rc = enqueue_coarse_count<LIDAR>(g, pl, w, total, N, camera_ids, means2d, radii, depths,
                                                  C, stream))
             return rc;
