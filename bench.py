@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # 0.5 KiB per KiB, WRITE_SIZE 1.0).  Summaries: profiles/kernels_counters_camera_1M_1080p_lidar_128x2048.txt.
 # They describe the 1M-Gaussian default only; other sizes report null.
 MEASURED_TRAFFIC_BYTES = {
-    "camera": int((14182.2 * 2.0 + 49098.5) * 1024),
-    "lidar": int((26517.9 * 2.0 + 42243.8) * 1024),
+    "camera": int((15075.7 * 2.0 + 53046.0) * 1024),
+    "lidar": int((26520.3 * 2.0 + 42266.5) * 1024),
 }
 
 
