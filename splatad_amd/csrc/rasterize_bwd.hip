@@ -515,8 +515,13 @@ static int launch_bwd_as(BwdArgs a, dim3 grid, dim3 block, hipStream_t stream) {
     // Batches of the whole workgroup, unless that leaves fewer than four workgroups to a compute
     // unit (160 KB of LDS): a lidar sweep's 1024 tiles then run all at once instead of in two
     // rounds (with 33 channels: 104 Gaussians per batch, 0.39 ms instead of 0.51 ms with 128).
+    // The two-pixel kernels' registers allow five wavefronts per SIMD, twenty per compute unit:
+    // their batches leave room for the workgroups that makes (ten of 128 lanes: 104 Gaussians per
+    // batch with four channels, 0.54 instead of 0.57 ms for the 1080p frame's backward pass).
     a.batch = block.x;
-    if (a.batch * per_gaussian > 40 * 1024) a.batch = (uint32_t)(40 * 1024 / per_gaussian) / 8 * 8;
+    const size_t wgs = PPL == 2 ? std::max<size_t>(4, 20 / ((block.x + SPLATAD_WAVE - 1) / SPLATAD_WAVE)) : 4;
+    const size_t room = 160 * 1024 / wgs - 1024; // LDS is granted in blocks, and 16 bytes are static
+    if (a.batch * per_gaussian > room) a.batch = (uint32_t)(room / per_gaussian) / 8 * 8;
     const size_t lds = a.batch * per_gaussian;
     if (lds > 64 * 1024)
         SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_bwd_kernel<CH, LIDAR, PPL>,
