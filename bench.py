@@ -23,15 +23,65 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# HBM bytes per launch of the two compositing kernels on the default workloads, from
-# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this file (KiB per dispatch,
-# scaled by what the same counters read for a 1 GiB device-to-device copy: FETCH_SIZE reads
-# 0.5 KiB per KiB, WRITE_SIZE 1.0).  Summaries: profiles/kernels_counters_camera_1M_1080p_lidar_128x2048.txt.
-# They describe the 1M-Gaussian default only; other sizes report null.
-MEASURED_TRAFFIC_BYTES = {
-    "camera": int((15075.7 * 2.0 + 53046.0) * 1024),
-    "lidar": int((26520.3 * 2.0 + 42266.5) * 1024),
-}
+VALU_CLOCK_HZ = 2.4e9  # MI355X peak engine clock, published
+N_SIMDS = 256 * 4      # 256 compute units, four SIMDs each; a wave64 vector instruction issues over 4 cycles
+# vector instructions a (pixel, composited Gaussian) pair costs the camera compositing kernel at
+# the least in its formulation (exact float32, no packed FP32): five multiply-adds of the exponent
+# polynomial, one v_exp_f32, the alpha test, the next transmittance and its test and update (4),
+# the weight and four channel multiply-adds (5) = 15
+MIN_VALU_PER_PIXEL_AND_GAUSSIAN = 15
+
+PROFILE = os.path.join(ROOT, "profiles", "kernels_counters_camera_1M_1080p_lidar_128x2048.txt")
+
+
+def profiled_counters():
+    """Per-kernel hardware counters of the default workloads, read from the committed rocprofv3
+    summary (its lines `@ kernel | FETCH_SIZE KiB | WRITE_SIZE KiB | SQ_INSTS_VALU`, averages per
+    dispatch, and `@ calibration | fetch factor | write factor` from a 1 GiB copy).  They describe
+    the 1M-Gaussian default only.  Returns {} when the summary is missing."""
+    out = {}
+    try:
+        with open(PROFILE) as f:
+            for line in f:
+                if not line.startswith("@ "):
+                    continue
+                parts = [x.strip() for x in line[2:].split("|")]
+                if parts[0] == "calibration":
+                    out["calibration"] = (float(parts[1]), float(parts[2]))
+                elif len(parts) == 4:
+                    out[parts[0]] = dict(fetch_kib=float(parts[1]), write_kib=float(parts[2]), insts_valu=float(parts[3]))
+    except OSError:
+        return {}
+    return out
+
+
+def hbm_traffic_bytes(counters, kernel):
+    """FETCH_SIZE and WRITE_SIZE of a kernel scaled by what the same counters read for a copy of
+    known size; None when the summary does not hold the kernel."""
+    if kernel not in counters or "calibration" not in counters:
+        return None
+    ff, wf = counters["calibration"]
+    c = counters[kernel]
+    return int((c["fetch_kib"] * ff + c["write_kib"] * wf) * 1024)
+
+
+def valu_roofline(counters, kernel, kernel_ms, pairs=None):
+    """The bound that holds the compositing kernels: vector instruction issue.  achieved = the
+    fraction of the GPU's issue cycles (four per wave64 instruction and SIMD) the kernel's
+    SQ_INSTS_VALU fill during its event-timed duration; floor_ms = the time the (pixel,
+    Gaussian) pairs that composite need at MIN_VALU_PER_PIXEL_AND_GAUSSIAN instructions each."""
+    if kernel not in counters:
+        return None
+    insts = counters[kernel]["insts_valu"]
+    busy_s = insts * 4.0 / (N_SIMDS * VALU_CLOCK_HZ)
+    out = {"kernel": kernel, "bound": "valu_issue", "achieved": busy_s / (kernel_ms * 1e-3), "peak": 1.0,
+           "unit": "fraction of vector issue cycles", "frac": busy_s / (kernel_ms * 1e-3),
+           "insts_valu_per_launch": insts, "issue_ms": busy_s * 1e3, "kernel_ms": kernel_ms}
+    if pairs is not None:
+        floor_s = pairs / 64.0 * MIN_VALU_PER_PIXEL_AND_GAUSSIAN * 4.0 / (N_SIMDS * VALU_CLOCK_HZ)
+        out.update(pixel_gaussian_pairs=int(pairs), min_insts_per_pair=MIN_VALU_PER_PIXEL_AND_GAUSSIAN,
+                   floor_ms=floor_s * 1e3, floor_over_kernel=floor_s / (kernel_ms * 1e-3))
+    return out
 
 
 def _sync():
@@ -422,6 +472,90 @@ def bench_backward(args):
     return out
 
 
+def bench_configs(args):
+    """Driver-timed legs for the benchmark's other forward configurations: configs[0] (10k
+    Gaussians, 320x240, RGB, packed and unpacked) and configs[3] (2M Gaussians around the sensor:
+    six 1920x1080 rolling-shutter cameras in one call, and the 128x2048 sweep), each with its
+    step time, its intersections and the event-timed stages of the call."""
+    import torch
+
+    from splatad_amd import lidar_rasterization, rasterization, workloads
+    from splatad_amd.hip._backend import _C
+
+    dev = torch.device("cuda:0")
+    out = {}
+    steps, warmup = max(5, args.steps // 2), max(2, args.warmup // 5)
+
+    def camera_leg(s, label, render_mode):
+        C = s["viewmats"].shape[0]
+
+        def run(packed=False):
+            return rasterization(
+                s["means"], s["quats"], s["scales"], s["opacities"], s["colors"], s["velocities"],
+                s["viewmats"], s["Ks"], s["width"], s["height"], s["linear_velocity"],
+                s["angular_velocity"], s["rolling_shutter_time"], sh_degree=s["sh_degree"],
+                packed=packed, render_mode=render_mode, near_plane=s["near_plane"],
+                far_plane=s["far_plane"], eps2d=s["eps2d"], tile_size=s["tile_size"])
+
+        sec = time_steps(run, steps, warmup)
+        sec_packed = time_steps(lambda: run(True), steps, warmup)
+        _, _, meta = run()
+        W, H, ts = s["width"], s["height"], s["tile_size"]
+        zeros = torch.zeros((C, 3), device=dev)  # a sensor at rest, as rasterization() passes it
+        lin = s["linear_velocity"] if s["linear_velocity"] is not None else zeros
+        ang = s["angular_velocity"] if s["angular_velocity"] is not None else zeros
+        rs = s["rolling_shutter_time"] if s["rolling_shutter_time"] is not None else zeros[:, 0].contiguous()
+        stages = {
+            "projection_ms": time_kernel(lambda: _C.fully_fused_projection_fwd(
+                s["means"], None, s["quats"], s["scales"], s["velocities"], s["viewmats"], s["Ks"], W, H,
+                lin, ang, rs, s["eps2d"], s["near_plane"], s["far_plane"], 0.0, False), 5),
+            "isect_sort_ms": time_kernel(lambda: _C.isect_tiles(
+                meta["means2d"], meta["radii"], meta["depths"], None, None, C, ts, meta["tile_width"],
+                meta["tile_height"], True, True), 5),
+        }
+        stages["rest_ms (colours + compositing + host gaps)"] = sec * 1e3 - sum(stages.values())
+        return {"workload": label, "ms": sec * 1e3, "ms_packed": sec_packed * 1e3,
+                "Mpix_per_s": C * W * H / sec / 1e6, "n_isects": int(meta["flatten_ids"].shape[0]),
+                "visible_rows": int((meta["radii"][..., 0] > 0).sum().item()),
+                "stage_ms": {k: round(v, 4) for k, v in stages.items()}}
+
+    with torch.no_grad():
+        s = workloads.to_device(workloads.camera_small(), dev)
+        out["config0"] = camera_leg(s, "10000 Gaussians, 320x240, RGB, no rolling shutter (BASELINE configs[0])", "RGB")
+        del s
+        s = workloads.to_device(workloads.camera_driving(n=2 * args.n, n_cameras=6), dev)
+        out["config3_cameras"] = camera_leg(
+            s, "%d Gaussians around the sensor, six 1920x1080 rolling-shutter cameras in one call, SH degree 3, "
+               "RGB+D (BASELINE configs[3])" % (2 * args.n), "RGB+D")
+        del s
+        torch.cuda.empty_cache()
+        l = workloads.to_device(workloads.lidar_sweep(n=2 * args.n), dev)
+
+        def lidar_run():
+            return lidar_rasterization(
+                l["means"], l["quats"], l["scales"], l["opacities"], l["lidar_features"],
+                l["velocities"], l["viewmats"], l["raster_pts"], l["tile_elevation_boundaries"],
+                l["linear_velocity"], l["angular_velocity"], l["rolling_shutter_time"],
+                min_azimuth=l["min_azimuth"], max_azimuth=l["max_azimuth"],
+                min_elevation=l["min_elevation"], max_elevation=l["max_elevation"],
+                n_elevation_channels=l["n_elevation_channels"],
+                azimuth_resolution=l["azimuth_resolution"], tile_width=l["tile_width"],
+                tile_height=l["tile_height"], near_plane=l["near_plane"], far_plane=l["far_plane"],
+                eps2d=l["eps2d"], channel_chunk=33)
+
+        sec = time_steps(lidar_run, steps, warmup)
+        rf, ra, _, meta = lidar_run()
+        stages = {"isect_sort_ms": time_kernel(lambda: _C.isect_lidar_tiles(
+            meta["means2d"], meta["radii"], meta["depths"], None, None, 1, l["tile_elevation_boundaries"],
+            l["azimuth_resolution"] * l["tile_width"], l["min_azimuth"], True, True), 5)}
+        out["config3_lidar"] = {
+            "workload": "%d Gaussians, 128x2048 sweep, 32 features + range (BASELINE configs[3])" % (2 * args.n),
+            "ms": sec * 1e3, "Mpts_per_s": ra.numel() / sec / 1e6, "n_isects": int(meta["flatten_ids"].shape[0]),
+            "stage_ms": {k: round(v, 4) for k, v in stages.items()}}
+        out["config3_frame_ms"] = out["config3_cameras"]["ms"] + out["config3_lidar"]["ms"]
+    return out
+
+
 def cpu_baseline_camera(args):
     """The CPU oracle on the same camera workload (same seed and distributions), OpenMP over
     all host cores given to the process; bounded by using fewer Gaussians when needed."""
@@ -477,6 +611,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-lidar", action="store_true")
     ap.add_argument("--no-bwd", action="store_true", help="skip the forward + backward timing")
+    ap.add_argument("--no-configs", action="store_true", help="skip the legs for configs[0] and configs[3]")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (known HBM traffic, used "
                          "to scale FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -500,6 +635,12 @@ def main():
     cam = bench_camera(args)
     lid = None if args.no_lidar else bench_lidar(args)
     achieved = cam["alg_bytes"] / (cam["kernel_ms"] * 1e-3) / 1e9
+    plain = cam["stage_bytes"]["rasterize_given_colors_ms"] / (cam["stages"]["rasterize_given_colors_ms"] * 1e-3) / 1e9
+    counters = profiled_counters() if args.n == 1_000_000 else {}
+    cam_kernel = "rasterize_to_pixels_fwd_kernel<%d, 2, false, true>" % cam["channels"]
+    cam_plain_kernel = "rasterize_to_pixels_fwd_kernel<%d, 2, false, false>" % cam["channels"]
+    lanes = cam["lanes"]
+    pairs = lanes["iterations"] * 64 * lanes["pixels_per_lane"] * lanes["compositing_lane_fraction"]
     out = {
         "metric": "camera Mpix/s (fwd)",
         "value": cam["pixels"] / cam["sec"] / 1e6,
@@ -526,17 +667,28 @@ def main():
         "roofline": {
             # the compositing kernel that evaluates the spherical-harmonic colours of the entries
             # it stages: the entries' geometry and depth, the mean and coefficient row of every
-            # (camera, Gaussian) among them once, the image
-            "kernel": "rasterize_to_pixels_fwd_kernel<%d, 2, false, true>" % cam["channels"],
+            # (camera, Gaussian) among them once, the image.  `frac` is this kernel against these
+            # bytes; `given_colors` is the same kernel handed the colours (as calls that want
+            # gradients run it) against the bytes of that formulation.
+            "kernel": cam_kernel,
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES["camera"] if args.n == 1_000_000 else None,
+            "traffic": hbm_traffic_bytes(counters, cam_kernel),
             "algorithmic_bytes": cam["alg_bytes"], "kernel_ms": cam["kernel_ms"],
             "rows_staged": cam["rows_staged"], "color_cache_left_empty": cam["cache_left_empty"],
+            "given_colors": {"kernel": cam_plain_kernel, "achieved": plain, "frac": plain / HBM_PEAK_GBS,
+                             "algorithmic_bytes": cam["stage_bytes"]["rasterize_given_colors_ms"],
+                             "kernel_ms": cam["stages"]["rasterize_given_colors_ms"],
+                             "traffic": hbm_traffic_bytes(counters, cam_plain_kernel)},
+            # what actually bounds the kernel: vector instruction issue
+            "valu_issue": valu_roofline(counters, cam_kernel, cam["kernel_ms"], pairs),
+            "valu_issue_given_colors": valu_roofline(counters, cam_plain_kernel,
+                                                     cam["stages"]["rasterize_given_colors_ms"], pairs),
         },
     }
     if lid is not None:
         l_ach = lid["alg_bytes"] / (lid["kernel_ms"] * 1e-3) / 1e9
+        lid_kernel = "rasterize_to_points_fwd_kernel<%d, %s>" % (lid["channels"], "true" if lid["channels"] in (32, 33) else "false")
         out["lidar"] = {
             "metric": "lidar Mpts/s (fwd)", "value": lid["points"] / lid["sec"] / 1e6,
             "unit": "Mpts/s", "ms_per_step": lid["sec"] * 1e3,
@@ -547,14 +699,26 @@ def main():
             "stage_ms": {k: round(v, 4) for k, v in lid["stages"].items()},
             "stages": stage_rooflines(lid),
             "tile_cycles": lid["tile_cycles"],
-            "roofline": {"kernel": "rasterize_to_points_fwd_kernel<%d, %s>" % (lid["channels"], "true" if lid["channels"] in (32, 33) else "false"),
+            "roofline": {"kernel": lid_kernel,
                          "bound": "hbm", "achieved": l_ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": l_ach / HBM_PEAK_GBS,
-                         "traffic": MEASURED_TRAFFIC_BYTES["lidar"] if args.n == 1_000_000 else None,
-                         "algorithmic_bytes": lid["alg_bytes"], "kernel_ms": lid["kernel_ms"]},
+                         "traffic": hbm_traffic_bytes(counters, lid_kernel),
+                         "algorithmic_bytes": lid["alg_bytes"], "kernel_ms": lid["kernel_ms"],
+                         # the kernel lasts as long as its slowest tile (all tiles resident at once):
+                         # vector issue fills less than half of it
+                         "valu_issue": valu_roofline(counters, lid_kernel, lid["kernel_ms"])},
         }
+    if not args.no_configs:
+        out["configs"] = bench_configs(args)
     if not args.no_bwd:
-        out["backward"] = {k: round(v, 4) for k, v in bench_backward(args).items()}
+        bwd = bench_backward(args)
+        out["backward"] = {k: round(v, 4) for k, v in bwd.items()}
+        for key, kernel in (("camera_rasterize_bwd_ms", "rasterize_bwd_kernel<4, false, 2>"),
+                            ("lidar_rasterize_bwd_ms", "rasterize_bwd_kernel<33, true, 1>")):
+            # (the timed interval also holds the clearing and unpacking launches around the kernel)
+            r = valu_roofline(counters, kernel, bwd[key])
+            if r is not None:
+                out["backward"][key.replace("_ms", "_valu_issue")] = r
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_camera(args)
     print(json.dumps(out))

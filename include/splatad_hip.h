@@ -318,7 +318,10 @@ int splatad_map_points_to_lidar_tiles(uint64_t total, uint32_t N, const int64_t 
  * splatad_map_points_to_lidar_tiles_noalloc_max_tiles() (16 384).  Results are identical to
  * splatad_map_points_to_lidar_tiles.  All calls on one GPU share that GPU's array: calls that
  * overlap on one GPU (different streams, different threads) race; calls in stream order do not,
- * and nothing has to be cleared between them. */
+ * and nothing has to be cleared between them.  The first sorted call on a device also does the
+ * library's one-time setup for that device (kernel attributes, the address of the static
+ * array): make one call outside any capture before capturing calls into a HIP graph; after
+ * that a call enqueues kernels only. */
 uint64_t splatad_map_points_to_lidar_tiles_noalloc_max_points(void);
 uint32_t splatad_map_points_to_lidar_tiles_noalloc_max_tiles(void);
 int splatad_map_points_to_lidar_tiles_noalloc(uint64_t total, uint32_t N,

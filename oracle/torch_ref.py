@@ -227,9 +227,13 @@ def rasterize_to_pixels(means2d, conics, colors, opacities, pix_vels, rs_time, b
 
 def rasterize_to_points(means2d, conics, colors, opacities, pix_vels, depth_comps, backgrounds,
                         raster_pts, tile_width, tile_height, compute_alpha_sum, threshold, offsets,
-                        flatten_ids, depth_idx, tiles=None):
+                        flatten_ids, depth_idx, tiles=None, near=None):
     """Dense per-tile compositing onto lidar points. Returns (colors, alphas, alpha_sum, median).
-    With `tiles` (flat (sensor, tile) indices) only those tiles are rendered."""
+    With `tiles` (flat (sensor, tile) indices) only those tiles are rendered.  With `near` (a dict
+    with "margin" and, for the alpha sum, "depth_margin" in metres), near["rows"] becomes a bool
+    [C * N] as in rasterize_to_pixels: the Gaussians with an alpha within the relative margin of
+    1/255 at a point still compositing, or a depth within depth_margin of the alpha sum's
+    range - threshold cut there, and the Gaussians composited at a point that has such a pair."""
     C, gh, gw = offsets.shape
     H, W = raster_pts.shape[1:3]
     D = colors.shape[-1]
@@ -273,6 +277,20 @@ def rasterize_to_points(means2d, conics, colors, opacities, pix_vels, depth_comp
                 al = (1.0 - T_final) * active
                 before = col[g, depth_idx][None] < (P[:, 2:3] - threshold)
                 s = (a_eff * used * before).sum(1) * active if compute_alpha_sum else torch.zeros_like(al)
+                if near is not None:
+                    with torch.no_grad():
+                        near.setdefault("rows", torch.zeros(m2.shape[0], dtype=torch.bool))
+                        raw = op[g][None] * torch.exp(-sigma)
+                        stop = (a_eff > 0) & (T_incl <= 1e-4)
+                        earlier = torch.cumsum(stop.to(torch.int64), dim=1) - stop.to(torch.int64)
+                        live = (earlier == 0) & (active[:, None] > 0)
+                        close = ((raw * 255.0 - 1.0).abs() <= near["margin"]) & live
+                        shared = close.any(1, keepdim=True) & (w > 0)
+                        hit = close | shared
+                        if compute_alpha_sum and near.get("depth_margin"):
+                            cut = (col[g, depth_idx][None] - (P[:, 2:3] - threshold)).abs() <= near["depth_margin"]
+                            hit = hit | (cut & used & live)
+                        near["rows"][g[hit.any(0)]] = True
                 cross = used & (T_excl > 0.5) & (T_incl <= 0.5)
                 m = ((col[g, depth_idx][None] + extra) * cross).sum(1) * active
                 pieces.append((c, i0, i1, j0, j1, pix, al, s, m))

@@ -222,18 +222,21 @@ static int map_points_sorted(const PointGrid &g, uint64_t total, uint32_t N, con
     BinWorkspace w;
     carve_bin(workspace, (uint64_t)n_slots * wgs, &w);
     const size_t lds = (size_t)n_slots * 4;
-    {
+    {   // once per device, at the first sorted call on it (which therefore cannot be a captured one)
         static std::mutex guard;
-        static bool raised = false;
+        static bool raised[64] = {};
+        int dev = 0;
+        SPLATAD_CHECK_HIP(hipGetDevice(&dev));
+        SPLATAD_REQUIRE(dev >= 0 && dev < 64, "map_points_to_lidar_tiles: device index %d out of range", dev);
         std::lock_guard<std::mutex> lock(guard);
-        if (!raised) {
+        if (!raised[dev]) {
             SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)points_bin_kernel<false>,
                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
                                                   (int)(kMaxSlots * 4)));
             SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)points_bin_kernel<true>,
                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
                                                   (int)(kMaxSlots * 4)));
-            raised = true;
+            raised[dev] = true;
         }
     }
     hipLaunchKernelGGL(points_bin_kernel<false>, dim3(wgs), dim3(SPLATAD_WAVE), lds, stream, g, total,

@@ -242,14 +242,19 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     };
     // SHC: the colour of row g, what sh_fwd_kernel<true> writes for it, by the same instructions.
     // A row's colour is evaluated by the first workgroups that stage it and left in sh_cache for
-    // the others (a Gaussian is listed by every tile it touches).  Ordinary cached loads and
-    // stores, on purpose without any ordering: a word of a row only ever changes from the NaN
-    // the cache was filled with to its colour, so another workgroup sees each word either as
-    // NaN -- then it evaluates the colour itself, to the same value -- or as the colour; how
-    // soon it sees the colour is left to the caches (the dies' L2 caches do not see one
-    // another's lines before the kernel ends, so each die evaluates the rows its tiles
-    // stage).  Atomic loads or stores of device scope, which would share the colours between
-    // the dies, go to memory every time and made the kernel three to four times slower.
+    // the others (a Gaussian is listed by every tile it touches), on purpose without any
+    // ordering: a word of a row only ever changes from the NaN the cache was filled with to its
+    // colour, so another workgroup sees each word either as NaN -- then it evaluates the colour
+    // itself, to the same value -- or as the colour; how soon it sees the colour is left to the
+    // caches (the dies' L2 caches do not see one another's lines before the kernel ends, so each
+    // die evaluates the rows its tiles stage).  A row is read once, by one aligned 16-byte load
+    // whose four words are pinned in registers before their first use (an empty asm statement
+    // takes and returns them, so the compiler can neither read the row a second time later nor
+    // assume anything about the values), and written by one aligned 16-byte store; the
+    // hardware moves a word whole, so a read sees each word before or after its one change.
+    // Measured alternatives: relaxed atomic accesses word by word (four requests per row
+    // instead of one) cost this kernel 8 %, volatile accesses and atomic accesses of device
+    // scope go to memory every time and made it three to four times slower.
     struct Cached { float r, g, b, depth; };
     auto cached_color = [&](int32_t g) { // requested together with the rest of the Gaussian
         const float4 row = reinterpret_cast<const float4 *>(a.sh_cache)[g];
@@ -257,6 +262,7 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
     };
     auto stage_sh_color = [&](int32_t g, const Cached &c) {
         float cr = c.r, cg = c.g, cb = c.b, cd = c.depth; // the depth channel rides along
+        asm volatile("" : "+v"(cr), "+v"(cg), "+v"(cb), "+v"(cd)); // the row as it was read, once (see above)
         const bool missing = !(cr == cr) || !(cg == cg) || !(cb == cb) || (CH > 3 && !(cd == cd));
         if (wave_ballot(missing) != 0) { // uniform
             if (missing) {

@@ -86,7 +86,7 @@ def render_variants(render, lidar=False):
     return outs
 
 
-def assert_matches_oracle_decisions(got, variants, tols, name="", max_attributed=1.5e-2, max_ambiguous=2):
+def assert_matches_oracle_decisions(got, variants, tols, name="", max_attributed=1.5e-2, max_ambiguous=None):
     """got: dict name -> array [..., ch]; variants: list of such dicts from render_variants();
     tols: dict name -> (atol, rtol).  Per output and pixel (all leading axes):
       * oracle value identical under every variant -> |got - nominal| <= atol + rtol |nominal|
@@ -95,10 +95,12 @@ def assert_matches_oracle_decisions(got, variants, tols, name="", max_attributed
         threshold) got must meet the tolerance against one of the variants; at most
         `max_ambiguous` pixels per output may match none (two near-threshold decisions in one
         pixel, moved in opposite directions), and those must lie within the variants' spread.
+        By default none (no test of this suite, up to the 1920x1080 frames, has needed one);
+        the number used is printed and returned.
     The near-threshold pixels may be at most `max_attributed` of all pixels (a plausibility
     bound: every saturating pixel ends on a transmittance decision, and a window of 6e-4 around
     1e-4 catches about half a per cent of them; measured 0.67 % on the 1920x1080 benchmark frame).
-    Returns {name: (attributed pixels, pixels that differ from the nominal render)}."""
+    Returns {name: (attributed pixels, pixels that differ from the nominal render, ambiguous pixels)}."""
     report = {}
     for key, (atol, rtol) in tols.items():
         g = np.asarray(got[key], np.float64)
@@ -123,13 +125,17 @@ def assert_matches_oracle_decisions(got, variants, tols, name="", max_attributed
         lo, hi = stack.min(0), stack.max(0)
         pad = atol + rtol * np.maximum(np.abs(lo), np.abs(hi)) + (hi - lo)
         inside = ((g >= lo - pad) & (g <= hi + pad)).all(-1)
-        assert int(ambiguous.sum()) <= max_ambiguous and inside[ambiguous].all(), (
-            f"{name} {key}: {int(ambiguous.sum())} near-threshold pixels match no decision variant")
         n_pix = max(attributed.size, 1)
+        allowed_ambiguous = 0 if max_ambiguous is None else max_ambiguous
+        assert int(ambiguous.sum()) <= allowed_ambiguous and inside[ambiguous].all(), (
+            f"{name} {key}: {int(ambiguous.sum())} near-threshold pixels match no decision variant "
+            f"(allowed {allowed_ambiguous})")
         # every point crosses T = 0.5 somewhere, in steps of ~alpha / 2: the median hinges on its
         # threshold five times as often as the other outputs on theirs
         allowed = max_attributed * (5 if key == "median" else 1)
         assert attributed.sum() <= max(allowed * n_pix, 3), (
             f"{name} {key}: {int(attributed.sum())}/{n_pix} pixels depend on a near-threshold decision")
-        report[key] = (int(attributed.sum()), int((~ok[0]).sum()))
+        report[key] = (int(attributed.sum()), int((~ok[0]).sum()), int(ambiguous.sum()))
+    print(f"{name}: per output (pixels on a near-threshold decision, pixels that differ from the nominal "
+          f"oracle render, pixels that match no variant): {report}")
     return report

@@ -20,17 +20,30 @@ pytestmark = pytest.mark.gpu
 T64 = lambda a: torch.from_numpy(np.ascontiguousarray(a)).double()
 
 
-def assert_grad_close(got, ref, name, rtol=1e-3, frac=0.995, loose=2e-2):
+def assert_grad_close(got, ref, name, rtol=1e-3, frac=0.995, loose=2e-2, near_rows=None, near_loose=5e-2):
+    """|got - ref| <= rtol (|ref| + rms) on at least `frac` of the entries and <= loose (|ref| + rms)
+    on every entry.  With `near_rows` (bool per leading row: the Gaussians for which the float64
+    comparator found an alpha >= 1/255 decision within rounding distance of its threshold, or
+    that share a pixel with such a pair) that bar holds for every other row without exception,
+    and the listed rows, whose gradient moves by the flipped pair's share, get `near_loose`."""
     got = np.asarray(got, np.float64)
     ref = np.asarray(ref, np.float64)
     assert got.shape == ref.shape, (name, got.shape, ref.shape)
     if ref.size == 0:
         return
     scale = math.sqrt(float((ref ** 2).mean())) + 1e-12
-    err = np.abs(got - ref)
-    tight = err <= rtol * (np.abs(ref) + scale)
-    ok = tight.mean()
-    worst = float((err / (np.abs(ref) + scale)).max())
+    rel = np.abs(got - ref) / (np.abs(ref) + scale)
+    if near_rows is not None:
+        near_rows = np.asarray(near_rows, bool).reshape(-1)
+        assert near_rows.shape[0] == got.shape[0], (name, near_rows.shape, got.shape)
+        if near_rows.any():
+            worst_near = float(rel[near_rows].max())
+            assert worst_near <= near_loose, f"{name}: worst rel {worst_near:.3e} on a row with a near-threshold pair"
+        rel = rel[~near_rows]
+        if rel.size == 0:
+            return
+    ok = (rel <= rtol).mean()
+    worst = float(rel.max())
     assert ok >= frac and worst <= loose, f"{name}: {ok:.4f} within {rtol}, worst rel {worst:.3e} (rms {scale:.3e})"
 
 

@@ -165,3 +165,33 @@ def test_rasterization_switches_to_the_colour_kernel_when_a_gradient_is_wanted()
         assert torch.equal(grad[0].detach(), plain[0]) and torch.equal(grad[1].detach(), plain[1])
         grad[0].sum().backward()
         assert float(leaf.grad.abs().sum()) > 0
+
+
+def test_colours_that_are_not_numbers_equal_the_two_operators():
+    """A colour cache row that is "not evaluated" is told by NaN; a row whose evaluated colour is
+    itself NaN (infinite or NaN coefficients, a NaN depth channel) therefore stays "not
+    evaluated" and every workgroup that stages it evaluates it again, to the same bits.  The
+    render has to equal the two operators' there too, NaN for NaN."""
+    from splatad_amd.hip._wrapper import (rasterize_to_pixels, rasterize_to_pixels_with_sh,
+                                          view_dependent_colors)
+    C, N, W, H, degree = 2, 6000, 200, 120, 3
+    d, p = _projected(C, N, W, H, 16, False, seed=31)
+    g = torch.Generator(device=DEV).manual_seed(5)
+    coeffs = torch.randn((N, 16, 3), device=DEV, generator=g) * 0.4
+    bad = torch.randperm(N, generator=torch.Generator().manual_seed(6))[:300].to(DEV)
+    coeffs[bad[:100], 0, 0] = float("nan")
+    coeffs[bad[100:200], 5, 1] = float("inf")
+    coeffs[bad[200:300], 9, 2] = -float("inf")
+    depths = p["depths"].clone()
+    depths[:, bad[250:]] = float("nan")
+    with torch.no_grad():
+        colors = view_dependent_colors(degree, d["means"], d["viewmats"], coeffs, p["radii"], depths)
+        want = rasterize_to_pixels(p["means2d"], p["conics"], colors, p["opacities"], p["pix_vels"], W, H, 16,
+                                   p["offsets"], p["flatten_ids"], d["rolling_shutter_time"])
+        got = rasterize_to_pixels_with_sh(degree, d["means"], d["viewmats"], coeffs, depths, p["means2d"],
+                                          p["conics"], p["opacities"], p["pix_vels"], W, H, 16, p["offsets"],
+                                          p["flatten_ids"], d["rolling_shutter_time"])
+    assert torch.isnan(want[0]).any() and not torch.isnan(want[0]).all()
+    assert torch.equal(torch.isnan(got[0]), torch.isnan(want[0]))
+    assert torch.equal(torch.nan_to_num(got[0], nan=-1.0), torch.nan_to_num(want[0], nan=-1.0))
+    assert torch.equal(got[1], want[1])

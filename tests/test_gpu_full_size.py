@@ -99,6 +99,11 @@ def test_surround_rig_2m_cameras_of_one_call_and_lidar_against_oracle():
     _lidar_stages_against_oracle(l, dl, lmeta, rf, la, asum, name="rig lidar 2M")
 
 
+def rows_of(flat, offs, ends, tiles):
+    """The Gaussians listed by the given tiles (sorted, unique)."""
+    return torch.unique(torch.cat([flat[int(offs.reshape(-1)[t]):int(ends[t])] for t in tiles])).cpu().long()
+
+
 def _directional_check(loss_of, x, grad, direction, h, name, rtol):
     """Central finite difference of a float64-accumulated loss along `direction` against the
     backward pass's gradient contracted with it."""
@@ -189,20 +194,27 @@ def test_training_step_1m_camera_backward_properties():
                                      rolling_shutter_time=d["rolling_shutter_time"])
     got = torch.autograd.grad((o_rc * v_c.to(DEV)).sum() + (o_ra * v_a.to(DEV)).sum(), leaves)
     rl = [T64(t).requires_grad_() for t in base]
+    near = {"margin": 1e-4}  # float32 alpha (a polynomial in tile coordinates) is good to a few 1e-5 relative
     r_rc, r_ra = torch_ref.rasterize_to_pixels(*rl, T64(d["rolling_shutter_time"]), None, 1920, 1080, 16,
-                                               offs.cpu(), flat.cpu(), tiles=set(pick))
+                                               offs.cpu(), flat.cpu(), tiles=set(pick), near=near)
+    near_rows = near["rows"][rows_of(flat, offs, ends, pick)].numpy()
     want = torch.autograd.grad((r_rc * v_c.double()).sum() + (r_ra * v_a.double()).sum(), rl)
-    rows = torch.unique(torch.cat([flat[int(offs.reshape(-1)[t]):int(ends[t])] for t in pick])).cpu().long()
+    rows = rows_of(flat, offs, ends, pick)
     assert rows.shape[0] > 5000
+    # the rows that may differ by a flipped pair's share are the comparator's own list, a
+    # plausibly short one (a window of 2e-4 around 1/255 and the Gaussians that share such pixels)
+    print(f"camera 1M, 40 tiles: {int(near_rows.sum())} of {rows.shape[0]} Gaussians have a near-threshold pair")
+    assert near_rows.sum() <= 3e-2 * rows.shape[0], int(near_rows.sum())
     for k, a, b in zip(("v_means2d", "v_conics", "v_colors", "v_opacities", "v_pix_vels"), got, want):
         a, b = a.detach().cpu().reshape(-1, *a.shape[2:]), b.reshape(-1, *b.shape[2:])
         untouched = torch.ones(a.shape[0], dtype=torch.bool)
         untouched[rows] = False
         assert float(a[untouched].abs().max()) == 0.0, k
-        # 1e-3 on 99.5 % of the entries, as in the operator tests; the float64 comparator takes
-        # its own alpha >= 1/255 decisions, and a Gaussian that it keeps in a pixel where float32
-        # drops it moves that Gaussian's entry by a few per cent (measured worst: 2.3e-2)
-        assert_grad_close(a[rows].numpy(), b[rows].numpy(), f"{k} (40 tiles of the 1M frame)", loose=5e-2)
+        # the operator tests' bar (1e-3 on 99.5 % of the entries, 2e-2 on all) for every row
+        # without a near-threshold pair; the float64 comparator takes its own alpha >= 1/255
+        # decisions, and a Gaussian that it keeps in a pixel where float32 drops it moves the
+        # rows it lists by a few per cent
+        assert_grad_close(a[rows].numpy(), b[rows].numpy(), f"{k} (40 tiles of the 1M frame)", near_rows=near_rows)
 
     # all-ones cotangent: the colour gradients of the compositing operator add up to sum(alpha)
     N = s["means"].shape[0]
@@ -308,12 +320,141 @@ def test_training_step_1m_lidar_backward_properties():
     got = torch.autograd.grad((o[0] * v_f.to(DEV)).sum() + (o[1] * v_a.to(DEV)).sum() + (o[2] * v_s.to(DEV)).sum(),
                               leaves)
     rl = [T64(t).requires_grad_() for t in base]
+    near = {"margin": 1e-4, "depth_margin": 1e-4}
     r = torch_ref.rasterize_to_points(*rl, None, T64(d["raster_pts"]), 64, 4, True, 0.2, offs.cpu(), flat.cpu(), 32,
-                                      tiles=set(pick))
+                                      tiles=set(pick), near=near)
     want = torch.autograd.grad((r[0] * v_f.double()).sum() + (r[1] * v_a.double()).sum()
                                + (r[2] * v_s.double()).sum(), rl)
-    rows = torch.unique(torch.cat([flat[int(offs.reshape(-1)[t]):int(ends[t])] for t in pick])).cpu().long()
+    rows = rows_of(flat, offs, ends, pick)
+    near_rows = near["rows"][rows].numpy()
+    print(f"lidar 1M, 12 tiles: {int(near_rows.sum())} of {rows.shape[0]} Gaussians have a near-threshold pair")
+    assert near_rows.sum() <= 3e-2 * rows.shape[0], int(near_rows.sum())
     names6 = ("v_means2d", "v_conics", "v_features", "v_opacities", "v_pix_vels", "v_depth_compensations")
     for k, a, b in zip(names6, got, want):
         a, b = a.detach().cpu().reshape(-1, *a.shape[2:]), b.reshape(-1, *b.shape[2:])
-        assert_grad_close(a[rows].numpy(), b[rows].numpy(), f"{k} (12 tiles of the 1M sweep)", loose=5e-2)
+        assert_grad_close(a[rows].numpy(), b[rows].numpy(), f"{k} (12 tiles of the 1M sweep)", near_rows=near_rows)
+
+
+def _subsample_reference(n_total, n_sample, seed, run_ref, leaves_full, chunk=100_000):
+    """Gradients of a float64 reference that is independent per Gaussian: per-Gaussian
+    gradients on a random subsample, and the gradient with respect to whatever is shared by all
+    Gaussians (the view matrices) summed over all of them, in chunks.
+    run_ref(idx) -> (loss, per_gaussian_leaves, shared_leaf) for the Gaussians `idx` (LongTensor)."""
+    pick = torch.randperm(n_total, generator=torch.Generator().manual_seed(seed))[:n_sample].sort().values
+    loss, per, shared = run_ref(pick)
+    per_grads = torch.autograd.grad(loss, per)
+    shared_sum = None
+    for c0 in range(0, n_total, chunk):
+        idx = torch.arange(c0, min(c0 + chunk, n_total))
+        loss, _, shared = run_ref(idx)
+        (g,) = torch.autograd.grad(loss, [shared])
+        shared_sum = g if shared_sum is None else shared_sum + g
+    return pick, per_grads, shared_sum
+
+
+def test_projection_and_sh_backward_1m_camera_against_float64():
+    """Backward of the camera projection and of the view-dependent colours at 1M Gaussians seen
+    by two 1920x1080 rolling-shutter cameras, per-Gaussian velocities included, against float64
+    autograd of the torch restatement: the gradients of an unpacked call are independent per
+    Gaussian, so they are compared on a random 20 000 of them, and the view-matrix gradient,
+    a sum over all Gaussians, on the float64 sum over all of them."""
+    from oracle import torch_ref
+    from splatad_amd import fully_fused_projection
+    from splatad_amd.hip._wrapper import view_dependent_colors
+    from tests.test_gpu_backward import assert_grad_close
+    s = workloads.camera_driving(n=1_000_000, n_cameras=2, with_velocities=True)
+    d = workloads.to_device(s, DEV)
+    N, C, W, H = s["means"].shape[0], 2, 1920, 1080
+    names = ("means", "quats", "scales", "velocities", "viewmats")
+    leaves = [d[k].clone().requires_grad_() for k in names]
+    out = fully_fused_projection(leaves[0], None, leaves[1], leaves[2], leaves[3], leaves[4], d["Ks"], W, H,
+                                 d["linear_velocity"], d["angular_velocity"], d["rolling_shutter_time"],
+                                 eps2d=d["eps2d"], calc_compensations=True)
+    radii, outs = out[0], out[1:]
+    valid = (radii[..., 0] > 0).cpu()
+    assert int(valid.sum()) > 500_000
+    gw = torch.Generator().manual_seed(21)
+    ws = [torch.randn(tuple(o.shape), generator=gw) for o in outs]
+    got = torch.autograd.grad(sum((o * w.to(DEV)).sum() for o, w in zip(outs, ws)), leaves)
+    T64 = lambda t: t.detach().cpu().double()
+    Ks, lin, ang, rs = T64(d["Ks"]), T64(d["linear_velocity"]), T64(d["angular_velocity"]), T64(d["rolling_shutter_time"])
+
+    def run_ref(idx):
+        per = [T64(d[k])[idx].requires_grad_() for k in names[:4]]
+        vm = T64(d["viewmats"]).requires_grad_()
+        ref = torch_ref.projection_fwd(per[0], None, per[1], per[2], per[3], vm, Ks, W, H, lin, ang, rs,
+                                       eps2d=s["eps2d"])
+        m = valid[:, idx]
+        loss = sum((r * w[:, idx].double() * (m if r.dim() == 2 else m[..., None])).sum() for r, w in zip(ref, ws))
+        return loss, per, vm
+
+    pick, per_grads, v_vm = _subsample_reference(N, 20_000, 22, run_ref, leaves)
+    assert int(valid[:, pick].sum()) > 10_000
+    for k, a, b in zip(names[:4], got[:4], per_grads):
+        assert_grad_close(a.cpu()[pick].numpy(), b.numpy(), f"projection {k} (20k of 1M, 2 cameras)")
+    assert_grad_close(got[4].cpu().numpy()[:, :3], v_vm.numpy()[:, :3], "projection viewmats (sum over 1M)")
+
+    # colours of degree 3 with the depth channel, the operator a training step runs
+    coeffs = d["colors"].clone().requires_grad_()
+    means = d["means"].clone().requires_grad_()
+    depths = outs[1].detach().clone().requires_grad_()
+    cols = view_dependent_colors(3, means, d["viewmats"], coeffs, radii, depths)
+    w_c = torch.randn(tuple(cols.shape), generator=gw)
+    got_c = torch.autograd.grad((cols * w_c.to(DEV)).sum(), [means, coeffs, depths])
+    c2w = torch.inverse(T64(d["viewmats"]))
+
+    def run_sh(idx):
+        m, cf = T64(d["means"])[idx].requires_grad_(), T64(d["colors"])[idx].requires_grad_()
+        dirs = m[None] - c2w[:, None, :3, 3]
+        rgb = torch.clamp_min(torch_ref.spherical_harmonics(3, dirs, cf[None].expand(C, -1, -1, -1)) + 0.5, 0.0)
+        return (rgb * w_c[:, idx, :3].double() * valid[:, idx, None]).sum(), [m, cf], None
+
+    pick = torch.randperm(N, generator=torch.Generator().manual_seed(23))[:20_000].sort().values
+    loss, per, _ = run_sh(pick)
+    want = torch.autograd.grad(loss, per)
+    assert_grad_close(got_c[0].cpu()[pick].numpy(), want[0].numpy(), "view colours: means (20k of 1M)")
+    assert_grad_close(got_c[1].cpu()[pick].numpy(), want[1].numpy(), "view colours: coefficients (20k of 1M)")
+    assert torch.equal(got_c[2].cpu(), w_c[..., 3].float())
+
+
+def test_projection_backward_1m_lidar_against_float64():
+    """Backward of the lidar projection at 1M Gaussians (per-Gaussian velocities included)
+    against float64 autograd of the torch restatement, as for the camera."""
+    from oracle import torch_ref
+    from splatad_amd import fully_fused_lidar_projection
+    from tests.test_gpu_backward import assert_grad_close
+    l = workloads.lidar_sweep(n=1_000_000, with_velocities=True)
+    d = workloads.to_device(l, DEV)
+    # a sensor pose that is not the identity, so that the view-matrix gradient has every entry
+    vm = torch.eye(4)
+    vm[:3, :3] = torch.tensor([[0.9950042, -0.0998334, 0.0], [0.0998334, 0.9950042, 0.0], [0.0, 0.0, 1.0]])
+    vm[:3, 3] = torch.tensor([0.5, -0.3, 0.2])
+    names = ("means", "quats", "scales", "velocities")
+    N = l["means"].shape[0]
+    leaves = [d[k].clone().requires_grad_() for k in names] + [vm[None].to(DEV).requires_grad_()]
+    out = fully_fused_lidar_projection(
+        leaves[0], None, leaves[1], leaves[2], leaves[3], leaves[4], d["linear_velocity"], d["angular_velocity"],
+        d["rolling_shutter_time"], min_elevation=l["min_elevation"], max_elevation=l["max_elevation"],
+        min_azimuth=l["min_azimuth"], max_azimuth=l["max_azimuth"], eps2d=l["eps2d"], calc_compensations=True)
+    radii, outs = out[0], out[1:]
+    valid = (radii[..., 0] > 0).cpu()
+    assert int(valid.sum()) > 300_000
+    gw = torch.Generator().manual_seed(31)
+    ws = [torch.randn(tuple(o.shape), generator=gw) for o in outs]
+    got = torch.autograd.grad(sum((o * w.to(DEV)).sum() for o, w in zip(outs, ws)), leaves)
+    T64 = lambda t: t.detach().cpu().double()
+    lin, ang, rs = T64(d["linear_velocity"]), T64(d["angular_velocity"]), T64(d["rolling_shutter_time"])
+
+    def run_ref(idx):
+        per = [T64(d[k])[idx].requires_grad_() for k in names]
+        v = vm[None].double().requires_grad_()
+        ref = torch_ref.lidar_projection_fwd(per[0], None, per[1], per[2], per[3], v, lin, ang, rs, eps2d=l["eps2d"])
+        m = valid[:, idx]
+        loss = sum((r * w[:, idx].double() * (m if r.dim() == 2 else m[..., None])).sum() for r, w in zip(ref, ws))
+        return loss, per, v
+
+    pick, per_grads, v_vm = _subsample_reference(N, 20_000, 32, run_ref, leaves)
+    assert int(valid[:, pick].sum()) > 5_000
+    for k, a, b in zip(names, got[:4], per_grads):
+        assert_grad_close(a.cpu()[pick].numpy(), b.numpy(), f"lidar projection {k} (20k of 1M)")
+    assert_grad_close(got[4].cpu().numpy()[:, :3], v_vm.numpy()[:, :3], "lidar projection viewmats (sum over 1M)")
