@@ -550,7 +550,7 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
                     uint4 *__restrict__ entries, uint32_t sshift,
                     const uint32_t *__restrict__ slab_bounds, const int32_t *__restrict__ remap,
                     int32_t *__restrict__ tiles_out, int32_t *__restrict__ totals,
-                    int64_t *__restrict__ n_entries) {
+                    int64_t *__restrict__ n_entries, uint32_t entries_cap) {
     extern __shared__ int32_t s_blocks[];
     __shared__ uint32_t s_bounds[1u << kSlabShiftMax];
     __shared__ uint32_t s_scan[kCoarseThreads / SPLATAD_WAVE];
@@ -567,7 +567,10 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
             [&](uint32_t j, uint32_t before, uint32_t) {
                 if (j >= first) s_blocks[j - first] = (int32_t)before + row[j - first];
             });
-        if (blockIdx.x == 0 && threadIdx.x == 0 && first + count == n_blocks) *n_entries = (int64_t)all;
+        // (entries_cap, the caller's number of intersections, bounds the list: it holds whenever the
+        // lists were sized for these very rows, and keeps a caller's mismatch inside the lists)
+        if (blockIdx.x == 0 && threadIdx.x == 0 && first + count == n_blocks)
+            *n_entries = (int64_t)min(all, entries_cap);
     } else {
         for (uint32_t b = threadIdx.x; b < count; b += blockDim.x) s_blocks[b] = 0;
     }
@@ -600,7 +603,8 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
         for_each_tile_balanced(mine, [&](const LaneWork &w, int32_t y, int32_t x, int32_t) {
             const uint32_t local = w.base + ((coarse_index<LIDAR>(cg, y, x) << sshift) | w.slab);
             const int32_t slot = atomicAdd(&s_blocks[local], 1);
-            if (FILL) entries[slot] = make_uint4(w.idx, w.depth_bits, first + local, coarse_mask(w, cg, y, x));
+            if (FILL && (uint32_t)slot < entries_cap)
+                entries[slot] = make_uint4(w.idx, w.depth_bits, first + local, coarse_mask(w, cg, y, x));
         });
     }
     if (!FILL) {
@@ -616,7 +620,7 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
 // kSortClassMin[c + 1]; the host launches one kernel configuration per class.
 constexpr int kSortClasses = 7;
 __constant__ const uint32_t kSortClassMin[kSortClasses + 1] = {0u,    512u,   2048u,  4096u,
-                                                               8192u, 16384u, 32768u, 0x7FFFFFFFu};
+                                                               8192u, 12288u, 32768u, 0x7FFFFFFFu};
 
 // A table scanned by scan_local_kernel holds prefixes inside scan blocks; what has to be added is
 // the sum of the blocks before an element's.  Every wavefront that needs it keeps those sums for
@@ -1158,7 +1162,7 @@ __device__ __forceinline__ void sort_segment(uint32_t seg, uint32_t n_segments, 
     }
 }
 
-// The sort for the short segments (n <= lds_words <= 8192, n <= ER * blockDim.x), shaped for the
+// The sort for the short segments (n <= lds_words <= 12288, n <= ER * blockDim.x), shaped for the
 // latency of its LDS accesses, which bounds the generic version above.  Where the depths of a
 // segment are spread evenly enough, one histogram places the entries: bins that are linear in
 // the depth, four entries each on average, and the atomic that counts an entry into its bin
@@ -1406,13 +1410,12 @@ isect_small_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t 
     }
 }
 
-// The three upper classes in one launch, longest segments first.  Their workgroups need most
-// of a compute unit's LDS, so even a launch that finds its class empty waits for such a unit to
+// The two upper classes (more than 12288 entries) in one launch, longest segments first.  Their
+// workgroups need most of a compute unit's LDS, so even a launch that finds its class empty waits for such a unit to
 // fall free once other sort kernels are running; one launch, enqueued before those, meets an
 // idle GPU and costs next to nothing when the scene has no long segments (the usual case for
 // cameras), while a lidar's long segments all start at once.
 constexpr uint32_t kSortBigThreads = 1024;
-constexpr uint32_t kSortBigInLds = 16384; // class 4 is staged in LDS
 
 __global__ void __launch_bounds__(kSortBigThreads)
 isect_big_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t sshift,
@@ -1425,15 +1428,11 @@ isect_big_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t ss
     extern __shared__ uint64_t lds_staged[];
     __shared__ uint32_t s_wave[2 * (1024 / SPLATAD_WAVE)];
     __shared__ uint32_t s_big;
-    for (int cls = kSortClasses - 1; cls >= 4; --cls) { // uniform
+    for (int cls = kSortClasses - 1; cls >= 5; --cls) { // uniform
         const uint32_t count = seg_counts[cls];
         const uint32_t *list = seg_lists + (size_t)cls * n_segments;
         for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) { // uniform across the workgroup
-            if (cls == 4)
-                sort_segment<16, true>(list[k], n_segments, n_tiles, sshift, tile_n_bits, kSortBigInLds,
-                                       sort_bucket_capacity(kSortBigInLds), n_isects, tile_starts, pairs,
-                                       isect_ids, flatten_ids, lds_staged, s_wave, s_big);
-            else if (cls == 5)
+            if (cls == 5)
                 sort_segment<32, false>(list[k], n_segments, n_tiles, sshift, tile_n_bits, kSortWindow,
                                         sort_bucket_capacity(32768u), n_isects, tile_starts, pairs,
                                         isect_ids, flatten_ids, lds_staged, s_wave, s_big);
@@ -1455,8 +1454,7 @@ static int launch_big_segment_sort(uint32_t workgroups, uint32_t segs, uint32_t 
                                    const uint32_t *seg_lists, const int32_t *tile_starts,
                                    const uint64_t *pairs, int64_t *isect_ids, int32_t *flatten_ids,
                                    hipStream_t stream) {
-    size_t lds_bytes = sort_lds_bytes(kSortBigInLds, kSortBigInLds);
-    if (sort_lds_bytes(kSortWindow, 0x7FFFFFFFu) > lds_bytes) lds_bytes = sort_lds_bytes(kSortWindow, 0x7FFFFFFFu);
+    const size_t lds_bytes = sort_lds_bytes(kSortWindow, 0x7FFFFFFFu);
     {
         static std::mutex guard;
         static bool raised = false;
@@ -1481,7 +1479,8 @@ static int launch_small_segment_sort(int cls, uint32_t threads, uint32_t max_n, 
                                      const uint32_t *seg_lists, const int32_t *tile_starts,
                                      const uint64_t *pairs, int64_t *isect_ids, int32_t *flatten_ids,
                                      hipStream_t stream) {
-    SPLATAD_REQUIRE((uint64_t)ER * threads >= max_n && max_n <= 8192u && (max_n & (max_n - 1)) == 0,
+    SPLATAD_REQUIRE((uint64_t)ER * threads >= max_n && max_n <= 12288u &&
+                        ((max_n & (max_n - 1)) == 0 || max_n % 4096u == 0),
                     "segment sort: class %d does not fit", cls);
     const uint32_t bucket_cap = sort_bucket_capacity(max_n);
     {   // the bins of the direct path: a power of two, at most max_n / kSortDirectMean of them
@@ -1724,7 +1723,7 @@ static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const Is
                            total, N, camera_ids, means2d, radii, pl.sshift ? depths : nullptr, c0, c1,
                            (uint32_t)pl.blocks, w.coarse_counts, (uint4 *)nullptr, pl.sshift,
                            (const uint32_t *)w.slab_bounds, (const int32_t *)nullptr, (int32_t *)nullptr,
-                           w.block_totals, (int64_t *)nullptr);
+                           w.block_totals, (int64_t *)nullptr, 0u);
     }
     SPLATAD_LAUNCH_CHECK();
     return 0;
@@ -1872,7 +1871,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, cg,
                            total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)pl.blocks,
                            w.coarse_counts, w.entries, sshift, (const uint32_t *)w.slab_bounds, remap,
-                           tiles_out, w.block_totals, w.n_entries);
+                           tiles_out, w.block_totals, w.n_entries, (uint32_t)n_isects);
     }
     SPLATAD_LAUNCH_CHECK();
     // tile segments: count, scan, fill.  The number of coarse entries stays on the device;
@@ -1911,7 +1910,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                        local_scan ? (const int64_t *)w.block_sums : (const int64_t *)nullptr, n_scan_blocks,
                        w.seg_starts);
     SPLATAD_LAUNCH_CHECK();
-    // Size classes: a launch per class (one for the three upper classes), so that the LDS per
+    // Size classes: a launch per class (one for the two upper classes), so that the LDS per
     // workgroup (and with it the number of resident workgroups) fits the segment length; the
     // segments of a class come from a list made on the device.  The classes touch disjoint
     // segments; they run on two helper streams beside the caller's, forked and joined with
@@ -1934,11 +1933,15 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                                                       n_isects, w.seg_counts, w.seg_lists, w.seg_starts, \
                                                       w.pairs, isect_ids, flatten_ids, on)) != 0) \
             return e;
-        // the upper classes go first, on the caller's stream, which does not wait for the fork
+        // the upper classes go first, on the caller's stream, which does not wait for the fork;
+        // then the segments of 8193 to 12288 entries (a driving frame's longest, a sixth of its
+        // entries), by the short-segment sort with twelve entries per lane: through the generic
+        // sort of the upper classes they took 30 us at the head of this stream
         if ((e = launch_big_segment_sort(256u, nseg, n_tiles, sshift, tile_n_bits, n_isects, w.seg_counts,
                                          w.seg_lists, w.seg_starts, w.pairs, isect_ids, flatten_ids,
                                          stream)) != 0)
             return e;
+        SPLATAD_SORT_CLASS(4, 12, 1024, 12288u, 256u, stream)
         SPLATAD_SORT_CLASS(2, 8, 512, 4096u, 1024u, ss->aux[0])
         SPLATAD_SORT_CLASS(3, 8, 1024, 8192u, 512u, ss->aux[1])
         SPLATAD_SORT_CLASS(1, 8, 256, 2048u, 4096u, stream)

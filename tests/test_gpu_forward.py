@@ -652,3 +652,50 @@ def test_isect_lidar_extent_beyond_a_full_turn():
     np.testing.assert_array_equal(to_np(tpg), o[0])
     np.testing.assert_array_equal(to_np(ids), o[1])
     np.testing.assert_array_equal(to_np(flat), o[2])
+
+
+def test_isect_fill_with_too_small_a_count_stays_inside_its_lists():
+    """The C ABI trusts the caller's n_isects for the size of `lists` and of the outputs.  A count
+    that is too small (a caller's mistake, or rows changed between the two calls) must not make
+    any stage write outside them: every buffer is followed by guard bytes, which have to survive."""
+    import ctypes
+    from splatad_amd.hip import _backend as b
+    lib = b.load_library()
+    rng = np.random.default_rng(77)
+    C, N, tile, tw, th = 1, 6000, 16, 20, 12
+    means2d = to_dev(np.stack([rng.uniform(0, tw * tile, (C, N)), rng.uniform(0, th * tile, (C, N))], -1).astype(np.float32))
+    radii = to_dev(rng.integers(1, 60, (C, N, 2)).astype(np.int32))
+    depths = to_dev(rng.uniform(0.1, 50.0, (C, N)).astype(np.float32))
+    total = C * N
+    tiles_per_gauss = torch.empty((C, N), dtype=torch.int32, device=DEV)
+    ws = b._workspace(lib.splatad_isect_workspace_bytes(b._u64(total), b._u32(C), b._u32(tw * th)), DEV)
+    head = (b._u64(total), b._u32(N), b._p(None), b._p(means2d), b._p(radii), b._p(depths))
+    tail = (b._u32(C), b._u32(tile), b._u32(tw), b._u32(th), b._i32(1))
+    n_host = b._i64(0)
+    b._check(lib.splatad_isect_tiles_count(*head, *tail, b._p(tiles_per_gauss), b._p(ws), ctypes.byref(n_host),
+                                           b._stream(DEV)))
+    n = int(n_host.value)
+    assert n > 100_000
+    small = n // 10
+    guard = 8 << 20  # more than every list of the true size takes
+    lists_bytes = lib.splatad_isect_lists_bytes(b._u64(total), b._i64(small))
+
+    def guarded(nbytes):
+        buf = torch.full((nbytes + guard,), 0xA5, dtype=torch.uint8, device=DEV)
+        return buf, buf[nbytes:]
+
+    lists, lists_guard = guarded(lists_bytes)
+    ids, ids_guard = guarded(small * 8)
+    flat, flat_guard = guarded(small * 4)
+    offsets = torch.empty((C, th, tw), dtype=torch.int32, device=DEV)
+    rc = lib.splatad_isect_tiles_fill(*head, *tail, b._i64(small), b._p(tiles_per_gauss), b._p(ws), b._p(lists),
+                                      b._p(ids), b._p(flat), b._p(offsets), b._stream(DEV))
+    torch.cuda.synchronize()
+    assert rc == 0, lib.splatad_last_error()
+    for name, g in (("lists", lists_guard), ("isect_ids", ids_guard), ("flatten_ids", flat_guard)):
+        assert bool((g == 0xA5).all()), f"{name}: written beyond the size the caller gave"
+    # and the library still gives the right lists for the right count afterwards
+    _, o_ids, o_flat = oracle.isect_tiles(to_np(means2d), to_np(radii), to_np(depths), tile, tw, th)
+    from splatad_amd.hip._backend import _C
+    _, g_ids, g_flat = _C.isect_tiles(means2d, radii, depths, None, None, C, tile, tw, th, True, True)
+    assert np.array_equal(to_np(g_ids), o_ids) and np.array_equal(to_np(g_flat), o_flat)
