@@ -151,10 +151,32 @@ def accumulate_lidar(
             accs.reshape(C, image_height, image_width, 1), alpha_sum)
 
 
-def _longest_list_batches(isect_offsets: Tensor, n_isects: int, block_size: int) -> int:
-    ends = torch.cat([isect_offsets.flatten()[1:], isect_offsets.new_tensor([n_isects])])
-    longest = int((ends - isect_offsets.flatten()).max().item()) if ends.numel() else 0
-    return (longest + block_size - 1) // block_size
+def _composite_in_windows(shape, channels, n_isects, isect_offsets, tile_points, batch_per_iter, device,
+                          list_window, composite_window, extra=False):
+    """Shared driver of the list-based rasterizers: the tiles' lists are walked in windows of
+    `batch_per_iter` batches of `tile_points` entries; `list_window(first, last, T)` emits the
+    (Gaussian, pixel, sensor) triples of a window for pixels that arrive with transmittance T,
+    `composite_window(triples)` composites them to (values, alphas[, extra]) as if the window
+    stood alone, and the driver scales each window by the transmittance in front of it.  The
+    optional third output (the lidar's alpha sum) is not scaled.  Returns (values [*shape,
+    channels], alphas [*shape, 1], extra | None)."""
+    values = torch.zeros((*shape, channels), device=device)
+    alphas = torch.zeros((*shape, 1), device=device)
+    extras = torch.zeros_like(alphas) if extra else None
+    starts = isect_offsets.flatten()
+    ends = torch.cat([starts[1:], starts.new_tensor([n_isects])])
+    longest = int((ends - starts).max().item()) if ends.numel() else 0
+    for first in range(0, -(-longest // tile_points), batch_per_iter):
+        in_front = 1.0 - alphas[..., 0]
+        triples = list_window(first, first + batch_per_iter, in_front)
+        if len(triples[0]) == 0:
+            break
+        out = composite_window(triples)
+        values = values + out[0] * in_front[..., None]
+        alphas = alphas + out[1] * in_front[..., None]
+        if extra:
+            extras = extras + out[2]
+    return values, alphas, extras
 
 
 def _rasterize_to_pixels(
@@ -178,23 +200,14 @@ def _rasterize_to_pixels(
     """
     from ._wrapper import rasterize_to_indices_in_range
 
-    C = means2d.shape[0]
-    dev = means2d.device
-    render_colors = torch.zeros((C, image_height, image_width, colors.shape[-1]), device=dev)
-    render_alphas = torch.zeros((C, image_height, image_width, 1), device=dev)
-    num_batches = _longest_list_batches(isect_offsets, len(flatten_ids), tile_size * tile_size)
-    for step in range(0, num_batches, batch_per_iter):
-        transmittances = 1.0 - render_alphas[..., 0]
-        gs_ids, pixel_ids, camera_ids = rasterize_to_indices_in_range(
-            step, step + batch_per_iter, transmittances, means2d, conics, opacities, pix_vels,
-            image_width, image_height, tile_size, isect_offsets, flatten_ids, rolling_shutter_time)
-        if len(gs_ids) == 0:
-            break
-        renders_step, accs_step = accumulate(
-            means2d, conics, opacities, colors, pix_vels, rolling_shutter_time, gs_ids, pixel_ids,
-            camera_ids, image_width, image_height)
-        render_colors = render_colors + renders_step * transmittances[..., None]
-        render_alphas = render_alphas + accs_step * transmittances[..., None]
+    render_colors, render_alphas, _ = _composite_in_windows(
+        (means2d.shape[0], image_height, image_width), colors.shape[-1], len(flatten_ids), isect_offsets,
+        tile_size * tile_size, batch_per_iter, means2d.device,
+        lambda first, last, T: rasterize_to_indices_in_range(
+            first, last, T, means2d, conics, opacities, pix_vels, image_width, image_height, tile_size,
+            isect_offsets, flatten_ids, rolling_shutter_time),
+        lambda ids: accumulate(means2d, conics, opacities, colors, pix_vels, rolling_shutter_time, *ids,
+                               image_width, image_height))
     if backgrounds is not None:
         render_colors = render_colors + backgrounds[:, None, None, :] * (1.0 - render_alphas)
     return render_colors, render_alphas
@@ -224,27 +237,14 @@ def _rasterize_to_points(
     """
     from ._wrapper import rasterize_to_indices_in_range_lidar
 
-    C = means2d.shape[0]
-    dev = means2d.device
-    render_features = torch.zeros((C, image_height, image_width, lidar_features.shape[-1]), device=dev)
-    render_alphas = torch.zeros((C, image_height, image_width, 1), device=dev)
-    alpha_sum = torch.zeros_like(render_alphas) if compute_alpha_sum_until_points else None
-    num_batches = _longest_list_batches(isect_offsets, len(flatten_ids), tile_width * tile_height)
-    for step in range(0, num_batches, batch_per_iter):
-        transmittances = 1.0 - render_alphas[..., 0]
-        gs_ids, pixel_ids, camera_ids = rasterize_to_indices_in_range_lidar(
-            step, step + batch_per_iter, transmittances, means2d, conics, opacities, pix_vels,
-            raster_pts, image_width, image_height, tile_width, tile_height, isect_offsets,
-            flatten_ids)
-        if len(gs_ids) == 0:
-            break
-        renders_step, accs_step, alpha_sum_step = accumulate_lidar(
-            means2d, conics, opacities, lidar_features, pix_vels, depth_compensations, raster_pts,
-            gs_ids, pixel_ids, camera_ids, image_width, image_height,
-            compute_alpha_sum_until_pts=compute_alpha_sum_until_points,
-            compute_alpha_sum_until_pts_threshold=compute_alpha_sum_until_points_threshold)
-        render_features = render_features + renders_step * transmittances[..., None]
-        render_alphas = render_alphas + accs_step * transmittances[..., None]
-        if compute_alpha_sum_until_points:
-            alpha_sum = alpha_sum + alpha_sum_step
-    return render_features, render_alphas, alpha_sum
+    return _composite_in_windows(
+        (means2d.shape[0], image_height, image_width), lidar_features.shape[-1], len(flatten_ids),
+        isect_offsets, tile_width * tile_height, batch_per_iter, means2d.device,
+        lambda first, last, T: rasterize_to_indices_in_range_lidar(
+            first, last, T, means2d, conics, opacities, pix_vels, raster_pts, image_width, image_height,
+            tile_width, tile_height, isect_offsets, flatten_ids),
+        lambda ids: accumulate_lidar(
+            means2d, conics, opacities, lidar_features, pix_vels, depth_compensations, raster_pts, *ids,
+            image_width, image_height, compute_alpha_sum_until_pts=compute_alpha_sum_until_points,
+            compute_alpha_sum_until_pts_threshold=compute_alpha_sum_until_points_threshold),
+        extra=compute_alpha_sum_until_points)

@@ -5,13 +5,13 @@
 hand-written gfx950 kernel through the operators of `splatad_amd.hip._wrapper`.
 """
 import math
-import threading
 from typing import Dict, Optional, Tuple, Union
 
 import torch
 from torch import Tensor
 from typing_extensions import Literal
 
+from ._helper_stream import HelperStream, InPlace
 from .hip._wrapper import (
     MIN_OPACITY_PER_TILE,
     fully_fused_lidar_projection,
@@ -54,67 +54,51 @@ def _sensor_motion(C, device, linear_velocity, angular_velocity, rolling_shutter
 # stream only.
 HELPER_STREAM = False
 
-# one helper stream per (device, host thread): calls from different threads do not wait for one
-# another's helper work
-_HELPER_STREAMS: Dict[Tuple[int, int], "torch.cuda.Stream"] = {}
 
+class _CameraPlan:
+    """What a `rasterization()` call does beyond the fixed stages, decided up front from its
+    arguments alone:
 
-class _Beside:
-    """Runs the work of `with` blocks on a helper stream, beside what the caller's stream does
-    between the creation of the object (the fork) and `join()`.
-
-    The tile intersection ends with a segment sort whose few long workgroups leave most of the
-    GPU idle; work that only depends on the projection -- the colours of the Gaussians -- is
-    enqueued on a helper stream (default priority) to run meanwhile.  Create the object when
-    the inputs of that work are enqueued on the caller's stream: the helper stream waits for
-    that point only, not for what the caller's stream is given afterwards.  `join()` makes the
-    caller's stream wait for the helper and tells the allocator that the tensors made there
-    are used on the caller's stream from now on.  On a CPU device, or while a graph is being
-    captured, the blocks simply run in place.
+    colors            who makes the per-row colours: "given" (post-activation features),
+                      "view_kernel" (one kernel: directions, SH, activation, depth channel),
+                      "while_compositing" (forward-only calls: the compositing kernel evaluates
+                      the colours of the entries it stages) or "sh_operators" (view matrices that
+                      take a gradient: directions and SH by differentiable operators);
+    depth_in_colors   the colour maker appends the depth channel itself;
+    requests          what a packed projection is asked to make of its rows besides the rows:
+                      their opacities, their colours, their colour cache;
+    helper_stream     whether that work runs on a helper stream beside the tile intersection.
     """
 
-    def __init__(self, device, enabled=True):
-        # enabled=False: no helper stream; the blocks run in place, the requests to the packed
-        # projection are served on the caller's stream
-        self.main = self.side = self.fork = self._ctx = self._waited = None
-        # what the packed projection is asked to make on the helper stream, and what it made
-        self.requests: Dict[str, object] = {}
-        self.results: Dict[str, Tensor] = {}
-        if enabled and device.type == "cuda" and not torch.cuda.is_current_stream_capturing():
-            idx = device.index if device.index is not None else torch.cuda.current_device()
-            key = (idx, threading.get_ident())
-            if key not in _HELPER_STREAMS:
-                _HELPER_STREAMS[key] = torch.cuda.Stream(device=idx)
-            self.main = torch.cuda.current_stream(idx)
-            self.side = _HELPER_STREAMS[key]
-            self.fork = self.main.record_event()
+    def __init__(self, packed, sh_degree, render_mode, tile, means, quats, scales, opacities, colors,
+                 velocities, viewmats, backgrounds):
+        def wanted(*tensors):  # does any of them take a gradient in this call?
+            return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
 
-    def __enter__(self):
-        if self.side is not None:
-            if self._waited is not self.fork:  # once per fork: the helper stream runs in order
-                self.side.wait_event(self.fork)
-                self._waited = self.fork
-            self._ctx = torch.cuda.stream(self.side)
-            self._ctx.__enter__()
-        return self
-
-    def __exit__(self, *exc):
-        if self._ctx is not None:
-            self._ctx.__exit__(*exc)
-            self._ctx = None
-        return False
-
-    def refork(self):
-        """Moves the fork to what the caller's stream holds now."""
-        if self.side is not None:
-            self.fork = self.main.record_event()
-
-    def join(self, *tensors):
-        if self.side is not None:
-            self.main.wait_stream(self.side)
-            for t in tensors:
-                if t is not None:
-                    t.record_stream(self.main)
+        with_depth = render_mode in ("RGB+D", "RGB+ED")
+        if sh_degree is None:
+            self.colors = "given"
+        elif viewmats.requires_grad:
+            self.colors = "sh_operators"
+        elif (means.is_cuda and render_mode in ("RGB", "RGB+D", "RGB+ED") and colors.dtype == torch.float32
+              and opacities.dtype == torch.float32
+              and not wanted(means, quats, scales, opacities, colors, velocities, viewmats, backgrounds)):
+            self.colors = "while_compositing"
+        else:
+            self.colors = "view_kernel"
+        self.depth_in_colors = with_depth and self.colors in ("view_kernel", "while_compositing")
+        self.helper_stream = HELPER_STREAM and self.colors != "while_compositing"
+        self.requests = {}
+        if packed:
+            if self.colors == "view_kernel" and colors.is_contiguous():
+                self.requests["colors"] = (sh_degree, colors, self.depth_in_colors)
+            # the gather opacities[gaussian_ids] (* compensations), where no gradient passes through it
+            if (not wanted(means, quats, scales, opacities, velocities, viewmats) and opacities.is_contiguous()
+                    and opacities.dtype == torch.float32):
+                self.requests["opacities"] = opacities
+                if self.colors == "while_compositing" and colors.is_contiguous():
+                    self.requests["color_cache"] = (sh_degree, colors, self.depth_in_colors, *tile,
+                                                    MIN_OPACITY_PER_TILE)
 
 
 def rasterization(
@@ -157,6 +141,12 @@ def rasterization(
     sqrt(det(Sigma) / det(Sigma + eps2d I)); `absgrad=True` leaves the accumulated absolute
     image-plane gradients in `meta["means2d"].absgrad` after backward.
 
+    Reproducibility: forward results are the same bits from run to run.  Gradients that add up
+    contributions of many pixels (those of the compositing stage) are summed with float atomics,
+    so they differ in the last bits between runs; with `packed=True` and more than one camera
+    this also holds for the sums over the cameras that see a Gaussian (opacities, colours or SH
+    coefficients, projection inputs), which the unpacked call adds in a fixed order.
+
     Returns (render_colors [C, H, W, X], render_alphas [C, H, W, 1], meta).
     """
     N = means.shape[0]
@@ -185,36 +175,13 @@ def rasterization(
         assert (sh_degree + 1) ** 2 <= colors.shape[-2], colors.shape
 
     # 1. projection (packed: it also counts the intersections with the tile grid of step 2,
-    # so that the host waits for the GPU once per call, not twice)
+    # so that the host waits for the GPU once per call, not twice, makes the lists of step 2
+    # on its dense rows, and is asked for what else only needs the projection: see the plan)
     tile_width = math.ceil(width / float(tile_size))
     tile_height = math.ceil(height / float(tile_size))
-    # (packed, in a call that wants gradients: the kernels that write the packed rows go to the
-    # helper stream, and with them what else only needs the projection, the colours of step 3 and
-    # the rows' opacities; the tile intersection works on the projection's dense rows and does
-    # not wait for any of it)
-    fused_colors = sh_degree is not None and not viewmats.requires_grad
-    depth_appended = fused_colors and render_mode in ["RGB+D", "RGB+ED"]
-    # Colours from spherical harmonics and no gradient wanted: the compositing kernel evaluates
-    # the colours of the entries it stages itself (step 3 below falls away).
-    colors_while_compositing = (
-        fused_colors and means.is_cuda and render_mode in ["RGB", "RGB+D", "RGB+ED"]
-        and colors.dtype == torch.float32 and opacities.dtype == torch.float32
-        and not (torch.is_grad_enabled() and any(
-            t is not None and t.requires_grad
-            for t in (means, quats, scales, opacities, colors, velocities, viewmats, backgrounds))))
-    colors_beside = fused_colors and (packed or not colors_while_compositing)  # step 3 joins the helper stream
-    beside = _Beside(means.device, enabled=HELPER_STREAM and not colors_while_compositing)
-    if packed:
-        if fused_colors and not colors_while_compositing and colors.is_contiguous():
-            beside.requests["colors"] = (sh_degree, colors, depth_appended)
-        # the gather opacities[gaussian_ids] (* compensations), where no gradient passes through it
-        no_grad = not torch.is_grad_enabled() or not any(
-            t is not None and t.requires_grad for t in (means, quats, scales, opacities, velocities, viewmats))
-        if no_grad and opacities.is_contiguous() and opacities.dtype == torch.float32:
-            beside.requests["opacities"] = opacities
-            if colors_while_compositing and colors.is_contiguous():
-                beside.requests["color_cache"] = (sh_degree, colors, depth_appended, tile_size, tile_width,
-                                                  tile_height, MIN_OPACITY_PER_TILE)
+    plan = _CameraPlan(packed, sh_degree, render_mode, (tile_size, tile_width, tile_height), means, quats,
+                       scales, opacities, colors, velocities, viewmats, backgrounds)
+    beside = HelperStream(means.device, plan.requests) if plan.helper_stream else InPlace(plan.requests)
     proj = fully_fused_projection(
         means, None, quats, scales, velocities, viewmats, Ks, width, height, linear_velocity,
         angular_velocity, rolling_shutter_time, eps2d=eps2d, packed=packed, near_plane=near_plane,
@@ -228,80 +195,61 @@ def rasterization(
     else:
         radii, means2d, depths, conics, compensations, pix_vels = proj
         camera_ids, gaussian_ids = None, None
+        beside.refork()  # everything the colours need is enqueued
 
-    opacities_per_gaussian = opacities
-
-    def per_row_opacities():
-        # Compositing is the first to need these: [nnz], or [C, N] (a view, copied by the first
-        # operator that needs it when C > 1).
-        # (index_select: its backward adds with atomics where that of opacities[gaussian_ids]
-        # sorts the indices first, 0.1 ms for a million rows; the sums can differ in the last
-        # bit from run to run where a Gaussian is seen by several cameras)
-        o = opacities.index_select(0, gaussian_ids) if packed else opacities.expand(C, -1)
-        return o if compensations is None else o * compensations
-
-    # 2. tile intersection, sort, offsets
-    if not packed and not colors_while_compositing:
-        beside.refork()  # fork: everything the colours need is enqueued
-
-    def fused_view_colors():
-        # one kernel for directions, masks, SH, activation and the depth channel
-        return view_dependent_colors(sh_degree, means, viewmats, colors, radii,
-                                     depths if depth_appended else None, camera_ids,
-                                     gaussian_ids, launch_context=beside,
-                                     precomputed=beside.results.get("colors"))
-
-    # The colours run on a helper stream beside the intersection, enqueued behind it: the kernel
-    # then meets the segment sort, whose long workgroups leave part of the GPU idle (enqueued
-    # first, it would compete with the binning chain that everything else waits for, and its
-    # launch would stand between the host and the launches the GPU is waiting for).
+    # 2. tile intersection, sort, offsets.  (Work beside it is enqueued behind it: the kernel then
+    # meets the segment sort; enqueued first, its launch would stand between the host and the
+    # launches the GPU is waiting for.)
     tiles_per_gauss, isect_ids, flatten_ids = isect_tiles(
         means2d, radii, depths, tile_size, tile_width, tile_height, packed=packed, n_cameras=C,
         camera_ids=camera_ids, gaussian_ids=gaussian_ids,
     )
     isect_offsets = isect_offset_encode(isect_ids, C, tile_width, tile_height)
-    beside_opacities = packed and not opacities.requires_grad
+
+    # per-row opacities: [nnz], or [C, N] (a view, copied by the first operator that needs it
+    # when C > 1).  (index_select: its backward adds with atomics where that of
+    # opacities[gaussian_ids] sorts the indices first, 0.1 ms for a million rows; the sums can
+    # differ in the last bit from run to run where a Gaussian is seen by several cameras.)
+    opacities_per_gaussian = opacities
+
+    def per_row_opacities():
+        o = opacities_per_gaussian.index_select(0, gaussian_ids) if packed else opacities_per_gaussian.expand(C, -1)
+        return o if compensations is None else o * compensations
+
     if "opacities" in beside.results:
         opacities = beside.results["opacities"]
-        if not colors_beside:
-            beside.join()
-    elif beside_opacities:
-        # the gather (and the product with the compensations) goes beside the sort too: on the
-        # caller's stream it would stand alone between the sort and the compositing.  (Not for a
-        # leaf that takes a gradient: autograd would accumulate it on the helper stream.)
-        with beside:
+    elif packed and not opacities.requires_grad:
+        with beside:  # (not for a leaf that takes a gradient: autograd would accumulate it there)
             opacities = per_row_opacities()
-        if not colors_beside:
-            beside.join(opacities)
     else:
         if packed:
-            beside.join()  # the packed rows are written on the helper stream
+            beside.join()  # the gather reads the packed rows' ids
         opacities = per_row_opacities()
 
     # 3. per-(camera, Gaussian) colours
     color_cache = None
-    if colors_while_compositing:
+    depths_for_colors = depths if plan.depth_in_colors else None
+    if plan.colors == "view_kernel":
+        colors = view_dependent_colors(sh_degree, means, viewmats, colors, radii, depths_for_colors, camera_ids,
+                                       gaussian_ids, launch_context=beside,
+                                       precomputed=beside.results.get("colors"))
+    beside.join(colors, opacities)  # from here on everything is on the caller's stream
+    if plan.colors == "while_compositing":
         # the empty cache through which the tiles share the colours they evaluate, or, for a
-        # scene whose tiles will not saturate early, all colours after all (on the caller's
-        # stream: two short launches cost less there than a helper stream's fork and join)
-        color_cache = beside.results.get("color_cache")  # what the packed projection made of its rows
+        # scene whose tiles will not saturate early, all colours after all: what the packed
+        # projection made of its rows, or two short launches here
+        color_cache = beside.results.get("color_cache")
         if color_cache is None:
             color_cache = view_dependent_color_cache(
-                sh_degree, means, viewmats, colors, radii, depths if depth_appended else None,
-                opacities_per_gaussian, tile_size, tile_width, tile_height, camera_ids, gaussian_ids)
-    elif fused_colors:
-        colors = fused_view_colors()
-        made_beside = "colors" not in beside.results  # (what the projection made was allocated here)
-        beside.join(colors if made_beside else None,
-                    opacities if beside_opacities and "opacities" not in beside.results else None)
-    elif sh_degree is None:
+                sh_degree, means, viewmats, colors, radii, depths_for_colors, opacities_per_gaussian,
+                tile_size, tile_width, tile_height, camera_ids, gaussian_ids)
+    elif plan.colors == "given":
         if packed:
             colors = colors.index_select(0, gaussian_ids) if colors.dim() == 2 else colors[camera_ids, gaussian_ids]
         elif colors.dim() == 2:
             colors = colors.expand(C, -1, -1)
-    else:
+    elif plan.colors == "sh_operators":
         camtoworlds = torch.inverse(viewmats)  # [C, 4, 4]
-        masks = radii[..., 0] > 0
         if packed:
             dirs = means[gaussian_ids, :] - camtoworlds[camera_ids, :3, 3]  # [nnz, 3]
             shs = (colors[gaussian_ids, :, :] if colors.dim() == 3
@@ -309,12 +257,12 @@ def rasterization(
         else:
             dirs = means[None, :, :] - camtoworlds[:, None, :3, 3]  # [C, N, 3]
             shs = colors.expand(C, -1, -1, -1) if colors.dim() == 3 else colors  # [C, N, K, 3]
-        colors = spherical_harmonics(sh_degree, dirs, shs, masks=masks)
+        colors = spherical_harmonics(sh_degree, dirs, shs, masks=radii[..., 0] > 0)
         colors = torch.clamp_min(colors + 0.5, 0.0)
 
     # 4. channels to composite
     if render_mode in ["RGB+D", "RGB+ED"]:
-        if not depth_appended and not colors_while_compositing:
+        if not plan.depth_in_colors:
             colors = torch.cat((colors, depths[..., None]), dim=-1)
         if backgrounds is not None:
             backgrounds = torch.cat(
@@ -334,9 +282,9 @@ def rasterization(
     # The reference composites channel_chunk channels per call (rendering.py:362-391), copying
     # a slice of the colours for each; the kernel here takes all channels in one call (in
     # passes of 32 over the same lists), which renders the same images without the copies.
-    if colors_while_compositing:
+    if plan.colors == "while_compositing":
         render_colors, render_alphas = rasterize_to_pixels_with_sh(
-            sh_degree, means, viewmats, colors, depths if depth_appended else None, means2d, conics,
+            sh_degree, means, viewmats, colors, depths_for_colors, means2d, conics,
             opacities, pix_vels, width, height, tile_size, isect_offsets, flatten_ids,
             rolling_shutter_time, backgrounds=backgrounds, gaussian_ids=gaussian_ids,
             color_cache=color_cache)

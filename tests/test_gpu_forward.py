@@ -176,7 +176,7 @@ def test_packed_projection_makes_what_was_asked_for_beside_the_sort(C, N, W, H, 
     opacities[gaussian_ids] (* compensations) and view_dependent_colors on those rows."""
     from splatad_amd import fully_fused_projection, isect_tiles
     from splatad_amd.hip._wrapper import view_dependent_colors
-    from splatad_amd.rendering import _Beside
+    from splatad_amd._helper_stream import HelperStream as _Beside
     rng, means, quats, scales, vel = _gaussians(N, 23)
     viewmats, Ks = _cameras(rng, C, W, H)
     lin = rng.normal(size=(C, 3)).astype(np.float32)
