@@ -220,7 +220,7 @@ def bench_camera(args):
             return _C.rasterize_to_pixels_sh_fwd(
                 3, s["means"], s["viewmats"], s["colors"], None, meta["depths"], meta["means2d"],
                 meta["conics"], meta["opacities"], meta["pix_vels"], s["rolling_shutter_time"], None,
-                W, H, ts, meta["isect_offsets"], meta["flatten_ids"], cache=cache)
+                W, H, ts, meta["isect_offsets"], meta["flatten_ids"], cache=cache, want_last_ids=False)
 
         first = color_cache()
         cache_left_empty = bool(torch.isnan(first).all().item())
@@ -637,8 +637,10 @@ def main():
     achieved = cam["alg_bytes"] / (cam["kernel_ms"] * 1e-3) / 1e9
     plain = cam["stage_bytes"]["rasterize_given_colors_ms"] / (cam["stages"]["rasterize_given_colors_ms"] * 1e-3) / 1e9
     counters = profiled_counters() if args.n == 1_000_000 else {}
-    cam_kernel = "rasterize_to_pixels_fwd_kernel<%d, 2, false, true>" % cam["channels"]
-    cam_plain_kernel = "rasterize_to_pixels_fwd_kernel<%d, 2, false, false>" % cam["channels"]
+    # (template arguments: channels, pixels per lane, diagnostic, colours evaluated in the kernel,
+    # last ids kept)
+    cam_kernel = "rasterize_to_pixels_fwd_kernel<%d, 2, false, true, false>" % cam["channels"]
+    cam_plain_kernel = "rasterize_to_pixels_fwd_kernel<%d, 2, false, false, true>" % cam["channels"]
     lanes = cam["lanes"]
     pairs = lanes["iterations"] * 64 * lanes["pixels_per_lane"] * lanes["compositing_lane_fraction"]
     out = {

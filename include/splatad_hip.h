@@ -402,7 +402,8 @@ int splatad_view_colors_cache(uint32_t n, uint32_t C, uint32_t N, uint32_t K, ui
  * (not NULL) as the last one.  color_cache: 16 bytes per row, as splatad_view_colors_cache
  * leaves them (every float a NaN, or the row's colour and depth; the workgroups that first
  * stage a row without a colour leave it there for the tiles that list the Gaussian later); what
- * it holds afterwards is of no use to the caller.  Forward only. */
+ * it holds afterwards is of no use to the caller.  Forward only; last_ids may be NULL (nobody
+ * will run a backward pass from this call), which spares the kernel their bookkeeping. */
 int splatad_rasterize_to_pixels_fwd_sh(uint32_t C, uint32_t N, int64_t n_isects, uint32_t K,
                                        uint32_t degree, const float *means, const float *viewmats,
                                        const float *coeffs, int coeffs_per_sensor,

@@ -50,9 +50,43 @@ struct BwdArgs {
     uint32_t batch; // Gaussians staged per batch, at most the workgroup size
 };
 
-// Geometry gradient slots per Gaussian in the LDS accumulator, after the CH colour slots;
-// the last three exist for lidars only.
-enum { G_CONIC = 0, G_XY = 3, G_ABS = 5, G_VEL = 7, G_OPAC = 9, G_VELZ = 10, G_DC = 11, G_COUNT = 13 };
+// Geometry slots per Gaussian in the LDS accumulator, after the CH colour slots; those from
+// G_VELZ on exist for lidars only.  While a batch is worked on the slots hold moments of the
+// pixels' gradients of the exponent, s = dL/dsigma per pixel, not yet the gradients themselves:
+// G_CONIC: sum s dx^2, s dx dy, s dy^2; G_XY: sum s dx, s dy; G_VEL: sum s dx roll, s dy roll;
+// G_OPAC: sum s; and for the lidar's depth term d = dL/d(depth value) per point, G_DC: sum d dx,
+// d dy; G_VELZ: sum d roll; G_D0: sum d.  Every geometry gradient is a combination of these
+// with coefficients that belong to the Gaussian, not the pixel (its conic, its opacity, its
+// depth compensation), so the pixels accumulate the moments -- a dozen multiply-adds instead of
+// the two conic rows and a product per gradient -- and the flush forms the gradients once per
+// (tile, Gaussian), see gradients_from_moments().  G_ABS (the absolute image-plane gradients, which
+// are sums of absolute values and do not factor) is accumulated as such, and only where wanted.
+enum { G_CONIC = 0, G_XY = 3, G_ABS = 5, G_VEL = 7, G_OPAC = 9, G_VELZ = 10, G_DC = 11, G_D0 = 13, G_COUNT = 14 };
+
+// Turns the moments `m` (the geometry slots of one Gaussian) into the gradients, in place, from
+// its staged exponent e = {A, B, C, L}, 1 / opacity and, for lidars, ext = {range velocity,
+// depth compensation x, y, depth}: with a = 2 ln2 A, b = ln2 B, c = 2 ln2 C the conic,
+//   v_conic = (m_xx / 2, m_xy, m_yy / 2),        v_mean = (a m_x + b m_y, b m_x + c m_y) [+ dc m_d0],
+//   v_vel   = the same of (m_xr, m_yr) [+ dc m_dr], v_opacity = -m_0 / opacity;
+// G_ABS, G_VELZ and G_DC are gradients as accumulated, G_D0 is none and is cleared.
+template <bool LIDAR>
+__device__ __forceinline__ void gradients_from_moments(float *m, float4 e, float rop, float4 ext) {
+    const float a = 2.f * kLn2 * e.x, b = kLn2 * e.y, c = 2.f * kLn2 * e.z;
+    const float mx = m[G_XY], my = m[G_XY + 1], mxr = m[G_VEL], myr = m[G_VEL + 1];
+    float gx = a * mx + b * my, gy = b * mx + c * my;
+    float vx = a * mxr + b * myr, vy = b * mxr + c * myr;
+    if constexpr (LIDAR) {
+        const float d0 = m[G_D0], dr = m[G_VELZ];
+        gx += ext.y * d0; gy += ext.z * d0;
+        vx += ext.y * dr; vy += ext.z * dr;
+        m[G_D0] = 0.f;
+    }
+    m[G_CONIC] *= 0.5f;
+    m[G_CONIC + 2] *= 0.5f;
+    m[G_XY] = gx; m[G_XY + 1] = gy;
+    m[G_VEL] = vx; m[G_VEL + 1] = vy;
+    m[G_OPAC] *= -rop;
+}
 
 // The per-Gaussian values are summed over the wavefront in one or two power-of-two groups (a
 // reduce-scatter of n values costs about 2 n operations): first(n) values, then second(n).
@@ -269,7 +303,7 @@ rasterize_bwd_kernel(BwdArgs a) {
         else if (geo < G_OPAC) { slot_base = a.v_pix_vels + (geo - G_VEL); slot_stride = nv; }
         else if (geo == G_OPAC) { slot_base = a.v_opacities; slot_stride = 1; }
         else if (geo == G_VELZ) { slot_base = a.v_pix_vels + 2; slot_stride = 3; }
-        else { slot_base = a.v_depth_comps + (geo - G_DC); slot_stride = 2; }
+        else if (geo < G_D0) { slot_base = a.v_depth_comps + (geo - G_DC); slot_stride = 2; }
     }
 
     for (uint32_t b = 0; b < num_batches; ++b) {
@@ -356,7 +390,6 @@ rasterize_bwd_kernel(BwdArgs a) {
                 float v[NV];
 #pragma unroll
                 for (int k = 0; k < NV; ++k) v[k] = 0.f;
-                const float rop = s_aux[t].y;
                 float4 ext = make_float4(0.f, 0.f, 0.f, 0.f);
                 if constexpr (LIDAR) ext = rec[RECORD - 1];
 #pragma unroll
@@ -383,44 +416,40 @@ rasterize_bwd_kernel(BwdArgs a) {
                     behind[p] += cv * fac;
                     v_alpha += T_final[p] * ra * v_render_a[p];
                     v_alpha += -T_final[p] * ra * bg_dot[p];
-                    // conic row products a dx + b dy and b dx + c dy from the staged form
-                    const float row_x = kLn2 * (2.f * e.x * dx[p] + e.y * dy[p]);
-                    const float row_y = kLn2 * (e.y * dx[p] + 2.f * e.z * dy[p]);
                     const float v_sigma = -au_g * v_alpha;
-                    v[CH + G_CONIC] += 0.5f * v_sigma * dx[p] * dx[p];
-                    v[CH + G_CONIC + 1] += v_sigma * dx[p] * dy[p];
-                    v[CH + G_CONIC + 2] += 0.5f * v_sigma * dy[p] * dy[p];
-                    float g_x = v_sigma * row_x, g_y = v_sigma * row_y;
+                    float s_all = v_sigma, v_sig2 = 0.f; // every term that multiplies the conic rows
+                    float g_depth = 0.f;
                     if constexpr (LIDAR) {
                         // gradient of the depth channel value, under the same clamp rule
-                        const float g_depth = au_g != 0.f ? fac * v_out_depth : 0.f;
+                        g_depth = au_g != 0.f ? fac * v_out_depth : 0.f;
                         v[CH + G_DC] += g_depth * dx[p];
                         v[CH + G_DC + 1] += g_depth * dy[p];
                         v[CH + G_VELZ] += g_depth * roll[p];
-                        g_x += g_depth * ext.y;
-                        g_y += g_depth * ext.z;
-                    }
-                    float g_ax = fabsf(g_x), g_ay = fabsf(g_y);
-                    v[CH + G_OPAC] += au_g * rop * v_alpha;
-                    if constexpr (LIDAR) {
+                        v[CH + G_D0] += g_depth;
                         if (a.compute_alpha_sum) { // uniform
                             const float au_s = (valid && ext.w < pz - a.threshold) ? au[p] : 0.f;
-                            const float v_sig2 = -v_asum * au_s;
-                            const float ex = v_sig2 * row_x, ey = v_sig2 * row_y;
-                            g_x += ex; g_y += ey;
-                            g_ax += fabsf(ex); g_ay += fabsf(ey);
-                            v[CH + G_CONIC] += v_sig2 * 0.5f * dx[p] * dx[p];
-                            v[CH + G_CONIC + 1] += v_sig2 * dx[p] * dy[p];
-                            v[CH + G_CONIC + 2] += v_sig2 * 0.5f * dy[p] * dy[p];
-                            v[CH + G_OPAC] += v_asum * au_s * rop;
+                            v_sig2 = -v_asum * au_s;
+                            s_all += v_sig2;
                         }
                     }
-                    v[CH + G_XY] += g_x;
-                    v[CH + G_XY + 1] += g_y;
-                    v[CH + G_ABS] += g_ax;
-                    v[CH + G_ABS + 1] += g_ay;
-                    v[CH + G_VEL] += g_x * roll[p];
-                    v[CH + G_VEL + 1] += g_y * roll[p];
+                    const float sx = s_all * dx[p], sy = s_all * dy[p];
+                    v[CH + G_CONIC] = fmaf(sx, dx[p], v[CH + G_CONIC]);
+                    v[CH + G_CONIC + 1] = fmaf(sx, dy[p], v[CH + G_CONIC + 1]);
+                    v[CH + G_CONIC + 2] = fmaf(sy, dy[p], v[CH + G_CONIC + 2]);
+                    v[CH + G_XY] += sx;
+                    v[CH + G_XY + 1] += sy;
+                    v[CH + G_VEL] = fmaf(sx, roll[p], v[CH + G_VEL]);
+                    v[CH + G_VEL + 1] = fmaf(sy, roll[p], v[CH + G_VEL + 1]);
+                    v[CH + G_OPAC] += s_all;
+                    if (a.v_means2d_abs != nullptr) { // uniform: sums of absolute values, pixel by pixel
+                        // conic row products a dx + b dy and b dx + c dy from the staged form
+                        const float row_x = kLn2 * (2.f * e.x * dx[p] + e.y * dy[p]);
+                        const float row_y = kLn2 * (e.y * dx[p] + 2.f * e.z * dy[p]);
+                        float g_x = v_sigma * row_x, g_y = v_sigma * row_y;
+                        if constexpr (LIDAR) { g_x += g_depth * ext.y; g_y += g_depth * ext.z; }
+                        v[CH + G_ABS] += fabsf(g_x) + fabsf(v_sig2 * row_x);
+                        v[CH + G_ABS + 1] += fabsf(g_y) + fabsf(v_sig2 * row_y);
+                    }
                 }
                 // sum over the wavefront; the lane that ends up with slot s adds it in LDS
                 wave_reduce_scatter<NA>(*reinterpret_cast<float(*)[NA]>(&v[0]), lane);
@@ -442,6 +471,14 @@ rasterize_bwd_kernel(BwdArgs a) {
         // packed layout the slots of one Gaussian are neighbours in memory and in the wavefront
         // (lane = (Gaussian, slot)), and a Gaussian costs one or two requests instead of one per
         // value.
+        // the geometry slots hold moments: the gradients are formed here, once per Gaussian of the
+        // batch (a lane per Gaussian, the same straight-line code for all)
+        for (uint32_t t = tr; t < (uint32_t)batch_size; t += block_size) {
+            const float4 *rec = s_rec + (size_t)RECORD * t;
+            gradients_from_moments<LIDAR>(s_acc + (size_t)t * ACC + CH, rec[1], s_aux[t].y,
+                                          LIDAR ? rec[RECORD - 1] : make_float4(0.f, 0.f, 0.f, 0.f));
+        }
+        __syncthreads();
         if (a.packed != nullptr) {
             for (uint32_t idx = tr; idx < (uint32_t)batch_size * ACC; idx += block_size) {
                 const uint32_t t = idx / ACC, slot = idx - t * ACC;
@@ -492,7 +529,7 @@ unpack_gradients_kernel(uint64_t total, uint32_t stride, uint32_t width, BwdArgs
     else if (geo < G_OPAC) a.v_pix_vels[g * nv + (geo - G_VEL)] += val;
     else if (geo == G_OPAC) a.v_opacities[g] += val;
     else if (geo == G_VELZ) a.v_pix_vels[g * 3 + 2] += val;
-    else a.v_depth_comps[g * 2 + (geo - G_DC)] += val;
+    else if (geo < G_D0) a.v_depth_comps[g * 2 + (geo - G_DC)] += val;
 }
 
 __global__ void __launch_bounds__(SPLATAD_THREADS) fill_zero_f32x4_kernel(float4 *p, uint64_t n4) {

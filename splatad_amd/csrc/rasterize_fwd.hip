@@ -69,7 +69,10 @@ constexpr int kLaneStats = 8;
 // Every wavefront then tests 64 staged Gaussians at a time against its footprint, copies the
 // survivors' records in list order into a private strip of LDS (its own writes and reads: no
 // barrier) and walks that strip: sequential addresses, no lane-mask bookkeeping per Gaussian.
-template <int CH, int PPL, bool STATS = false, bool SHC = false>
+// LAST: the index of the last entry a pixel composited is kept and written (what the backward
+// pass starts from); without it (last_ids null: calls that take no gradient) the loop is two
+// instructions per survivor shorter.
+template <int CH, int PPL, bool STATS = false, bool SHC = false, bool LAST = true>
 // (Two pixels per lane: at most 512 lanes per tile.  The narrow two-pixel kernels are held to the
 // 80 registers of six resident wavefronts per SIMD, which they exceeded by two: 0.116 -> 0.110 ms
 // for the 1080p frame.)
@@ -191,7 +194,7 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
 #pragma unroll
                 for (int c = 0; c < CH; ++c) out[p][c] = fmaf(col[c], weight, out[p][c]);
                 T[p] = next_T;
-                cur_idx[p] = __float_as_uint(pb.z);
+                if (LAST) cur_idx[p] = __float_as_uint(pb.z);
             }
         }
         if (STATS) { st_iter += 1; st_idle += any_take == 0 ? 1u : 0u; }
@@ -385,7 +388,7 @@ rasterize_to_pixels_fwd_kernel(PixelArgs a) {
             if ((uint32_t)k < a.n_ch) dst[k] = bg ? out[p][k] + T[p] * bg[k] : out[p][k];
         if (a.write_aux) {
             a.render_alphas[pix] = 1.0f - T[p];
-            a.last_ids[pix] = (int32_t)cur_idx[p];
+            if (LAST) a.last_ids[pix] = (int32_t)cur_idx[p];
         }
     }
 }
@@ -744,13 +747,13 @@ static size_t pixel_lds_bytes(uint32_t threads) {
     return 16 * ((size_t)threads * (2 + (CH + 3) / 4) + waves * SPLATAD_WAVE * (CH <= 4 ? 3 : 2));
 }
 
-template <int CH, int PPL, bool STATS, bool SHC = false>
+template <int CH, int PPL, bool STATS, bool SHC = false, bool LAST = true>
 static int launch_pixels_as(const PixelArgs &a, dim3 grid, uint32_t threads, hipStream_t stream) {
     const size_t lds = pixel_lds_bytes<CH>(threads);
     if (lds > 64 * 1024)
-        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_to_pixels_fwd_kernel<CH, PPL, STATS, SHC>,
+        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_to_pixels_fwd_kernel<CH, PPL, STATS, SHC, LAST>,
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL((rasterize_to_pixels_fwd_kernel<CH, PPL, STATS, SHC>), grid, dim3(threads), lds, stream, a);
+    hipLaunchKernelGGL((rasterize_to_pixels_fwd_kernel<CH, PPL, STATS, SHC, LAST>), grid, dim3(threads), lds, stream, a);
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }
@@ -759,8 +762,12 @@ static int launch_pixels_as(const PixelArgs &a, dim3 grid, uint32_t threads, hip
 template <int CH>
 static int launch_pixels_sh(const PixelArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
     const uint32_t pixels = block.x * block.y;
-    if (pixels_per_lane(a.tile_size) == 2) return launch_pixels_as<CH, 2, false, true>(a, grid, pixels / 2, stream);
-    return launch_pixels_as<CH, 1, false, true>(a, grid, pixels, stream);
+    const bool two = pixels_per_lane(a.tile_size) == 2;
+    if (a.last_ids == nullptr) // a call that takes no gradient wants no last ids
+        return two ? launch_pixels_as<CH, 2, false, true, false>(a, grid, pixels / 2, stream)
+                   : launch_pixels_as<CH, 1, false, true, false>(a, grid, pixels, stream);
+    return two ? launch_pixels_as<CH, 2, false, true>(a, grid, pixels / 2, stream)
+               : launch_pixels_as<CH, 1, false, true>(a, grid, pixels, stream);
 }
 
 template <int CH>
@@ -881,7 +888,7 @@ extern "C" int splatad_rasterize_to_pixels_fwd_sh(
                     tile_h, tile_size, W, H);
     SPLATAD_REQUIRE(n_isects >= 0 && n_isects < (1ll << 31), "rasterize_to_pixels: bad n_isects");
     SPLATAD_REQUIRE((uint64_t)C * N < (1ull << 31), "rasterize_to_pixels: %u x %u rows exceed the id range", C, N);
-    SPLATAD_REQUIRE(rs_time && viewmats && tile_offsets && render_colors && render_alphas && last_ids,
+    SPLATAD_REQUIRE(rs_time && viewmats && tile_offsets && render_colors && render_alphas,
                     "rasterize_to_pixels: null pointer argument");
     SPLATAD_REQUIRE(n_isects == 0 || (means && coeffs && color_cache && means2d && conics && opacities &&
                                       pix_vels && flatten_ids),

@@ -896,11 +896,12 @@ class _Ops:
     def rasterize_to_pixels_sh_fwd(self, sh_degree, means, viewmats, coeffs, gaussian_ids, depths,
                                    means2d, conics, opacities, pix_vels, rolling_shutter_time,
                                    backgrounds, image_width, image_height, tile_size, tile_offsets,
-                                   flatten_ids, cache=None):
+                                   flatten_ids, cache=None, want_last_ids=True):
         """rasterize_to_pixels_fwd for rows whose colours are the view-dependent colours of
         `coeffs` ([N, K, 3] or [C, N, K, 3]): the kernel evaluates them for the entries it
         stages.  Rows are dense [C, N], or packed [nnz] with gaussian_ids [nnz]; depths, if
-        given, is rendered as a fourth channel."""
+        given, is rendered as a fourth channel.  want_last_ids=False: the third result is None
+        and the kernel does not keep track of them."""
         lib = load_library()
         means = _in(means, "means"); viewmats = _in(viewmats, "viewmats"); coeffs = _in(coeffs, "coeffs")
         depths = _in(depths, "depths"); gaussian_ids = _in(gaussian_ids, "gaussian_ids", torch.int64)
@@ -919,7 +920,8 @@ class _Ops:
         f = dict(dtype=torch.float32, device=dev)
         renders = torch.empty((C, image_height, image_width, D), **f)
         alphas = torch.empty((C, image_height, image_width, 1), **f)
-        last_ids = torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
+        last_ids = (torch.empty((C, image_height, image_width), dtype=torch.int32, device=dev)
+                    if want_last_ids else None)
         # colours of the rows that tiles stage, left by the first for the others; NaN = not yet
         if cache is None:
             cache = torch.full(rows + (4,), float("nan"), **f)

@@ -497,7 +497,7 @@ def rasterize_to_pixels_with_sh(
         sh_degree, means.contiguous(), viewmats.contiguous(), sh_coeffs.contiguous(), _c(gaussian_ids),
         _c(depths), means2d.contiguous(), conics.contiguous(), opacities.contiguous(), pix_vels.contiguous(),
         rolling_shutter_time.contiguous(), backgrounds, image_width, image_height, tile_size,
-        isect_offsets.contiguous(), flatten_ids.contiguous(), cache=color_cache)
+        isect_offsets.contiguous(), flatten_ids.contiguous(), cache=color_cache, want_last_ids=False)
     return render_colors, render_alphas
 
 
