@@ -61,14 +61,19 @@ struct BwdArgs {
 // the two conic rows and a product per gradient -- and the flush forms the gradients once per
 // (tile, Gaussian), see gradients_from_moments().  G_ABS (the absolute image-plane gradients, which
 // are sums of absolute values and do not factor) is accumulated as such, and only where wanted.
-enum { G_CONIC = 0, G_XY = 3, G_ABS = 5, G_VEL = 7, G_OPAC = 9, G_VELZ = 10, G_DC = 11, G_D0 = 13, G_COUNT = 14 };
+// The two G_ABS slots come last (behind G_OPAC for cameras, behind G_D0 for lidars), so that a
+// kernel compiled without them sums two values less per Gaussian over the wavefront; records
+// and unpacking always have room for them.
+enum { G_CONIC = 0, G_XY = 3, G_VEL = 5, G_OPAC = 7, G_VELZ = 8, G_DC = 9, G_D0 = 11 };
+constexpr int geo_abs(bool lidar) { return lidar ? 12 : 8; }
+constexpr int geo_count(bool lidar, bool with_abs = true) { return geo_abs(lidar) + (with_abs ? 2 : 0); }
 
 // Turns the moments `m` (the geometry slots of one Gaussian) into the gradients, in place, from
 // its staged exponent e = {A, B, C, L}, 1 / opacity and, for lidars, ext = {range velocity,
 // depth compensation x, y, depth}: with a = 2 ln2 A, b = ln2 B, c = 2 ln2 C the conic,
 //   v_conic = (m_xx / 2, m_xy, m_yy / 2),        v_mean = (a m_x + b m_y, b m_x + c m_y) [+ dc m_d0],
 //   v_vel   = the same of (m_xr, m_yr) [+ dc m_dr], v_opacity = -m_0 / opacity;
-// G_ABS, G_VELZ and G_DC are gradients as accumulated, G_D0 is none and is cleared.
+// the absolute gradients, G_VELZ and G_DC are gradients as accumulated, G_D0 is none and is cleared.
 template <bool LIDAR>
 __device__ __forceinline__ void gradients_from_moments(float *m, float4 e, float rop, float4 ext) {
     const float a = 2.f * kLn2 * e.x, b = kLn2 * e.y, c = 2.f * kLn2 * e.z;
@@ -90,17 +95,21 @@ __device__ __forceinline__ void gradients_from_moments(float *m, float4 e, float
 
 // The per-Gaussian values are summed over the wavefront in one or two power-of-two groups (a
 // reduce-scatter of n values costs about 2 n operations): first(n) values, then second(n).
-constexpr int reduce_first(int n) { return n <= 24 ? 16 : (n <= 48 ? 32 : 64); }
-constexpr int reduce_second(int n) { return n <= 16 ? 0 : (n <= 24 ? 8 : (n <= 32 ? 0 : (n <= 48 ? 16 : 0))); }
+constexpr int reduce_first(int n) { return n <= 12 ? 8 : (n <= 24 ? 16 : (n <= 48 ? 32 : 64)); }
+constexpr int reduce_second(int n) {
+    return n <= 8 ? 0 : (n <= 12 ? 4 : (n <= 16 ? 0 : (n <= 24 ? 8 : (n <= 32 ? 0 : (n <= 48 ? 16 : 0)))));
+}
 
 // PPL: pixels per lane.  Two for camera tiles that make whole wavefronts of 8 x 16 pixels (rows y
 // and y + 8 of a column, as in the forward kernel) and few channels: the wavefront reduction of
 // the per-Gaussian gradients, about 40 of the 110 vector instructions of a (wavefront, Gaussian)
 // step, is then paid once per 128 pixels, and a Gaussian is fetched from the LDS half as often.
-template <int CH, bool LIDAR, int PPL>
+// ABS: the kernel also sums the absolute image-plane gradients (v_means2d_abs not null).
+template <int CH, bool LIDAR, int PPL, bool ABS = true>
 __global__ void __launch_bounds__(256)
 rasterize_bwd_kernel(BwdArgs a) {
     static_assert(PPL == 1 || (PPL == 2 && !LIDAR), "two pixels per lane are a camera layout");
+    constexpr int G_ABS = geo_abs(LIDAR);
     extern __shared__ float4 lds4[];
     __shared__ int32_t s_block_final;
     __shared__ uint32_t s_ref_thread;
@@ -111,7 +120,7 @@ rasterize_bwd_kernel(BwdArgs a) {
     // {x, y, vx, vy}, staged exponent, then the lidar extras or, for cameras, the polynomial of
     // the exponent as the forward kernel stages it (same functions, same bits)
     constexpr int RECORD = LIDAR ? 3 : 4;
-    constexpr int GEO = LIDAR ? G_COUNT : G_VELZ;
+    constexpr int GEO = geo_count(LIDAR, ABS);
     constexpr int ACC = CH + GEO;
     constexpr int NA = reduce_first(ACC), NB = reduce_second(ACC), NV = NA + NB;
     static_assert(ACC <= SPLATAD_WAVE, "the flush gives every accumulator slot a lane");
@@ -298,10 +307,10 @@ rasterize_bwd_kernel(BwdArgs a) {
         const int geo = lane - CH;
         const uint32_t nv = LIDAR ? 3 : 2;
         if (geo < G_XY) { slot_base = a.v_conics + geo; slot_stride = 3; }
-        else if (geo < G_ABS) { slot_base = a.v_means2d + (geo - G_XY); slot_stride = 2; }
-        else if (geo < G_VEL) { if (a.v_means2d_abs != nullptr) { slot_base = a.v_means2d_abs + (geo - G_ABS); slot_stride = 2; } }
+        else if (geo < G_VEL) { slot_base = a.v_means2d + (geo - G_XY); slot_stride = 2; }
         else if (geo < G_OPAC) { slot_base = a.v_pix_vels + (geo - G_VEL); slot_stride = nv; }
         else if (geo == G_OPAC) { slot_base = a.v_opacities; slot_stride = 1; }
+        else if (geo >= G_ABS) { if (a.v_means2d_abs != nullptr) { slot_base = a.v_means2d_abs + (geo - G_ABS); slot_stride = 2; } }
         else if (geo == G_VELZ) { slot_base = a.v_pix_vels + 2; slot_stride = 3; }
         else if (geo < G_D0) { slot_base = a.v_depth_comps + (geo - G_DC); slot_stride = 2; }
     }
@@ -441,7 +450,7 @@ rasterize_bwd_kernel(BwdArgs a) {
                     v[CH + G_VEL] = fmaf(sx, roll[p], v[CH + G_VEL]);
                     v[CH + G_VEL + 1] = fmaf(sy, roll[p], v[CH + G_VEL + 1]);
                     v[CH + G_OPAC] += s_all;
-                    if (a.v_means2d_abs != nullptr) { // uniform: sums of absolute values, pixel by pixel
+                    if (ABS && a.v_means2d_abs != nullptr) { // (uniform) sums of absolute values, pixel by pixel
                         // conic row products a dx + b dy and b dx + c dy from the staged form
                         const float row_x = kLn2 * (2.f * e.x * dx[p] + e.y * dy[p]);
                         const float row_y = kLn2 * (e.y * dx[p] + 2.f * e.z * dy[p]);
@@ -509,7 +518,7 @@ unpack_gradients_kernel(uint64_t total, uint32_t stride, uint32_t width, BwdArgs
     if (idx >= total * stride) return;
     const uint64_t g = idx / stride;
     const uint32_t slot = (uint32_t)(idx - g * stride);
-    constexpr uint32_t GEO = LIDAR ? G_COUNT : G_VELZ;
+    constexpr uint32_t GEO = geo_count(LIDAR), G_ABS = geo_abs(LIDAR);
     if (slot >= width + GEO) return;
     const float val = a.packed[idx];
     if (val == 0.f) return;
@@ -524,10 +533,10 @@ unpack_gradients_kernel(uint64_t total, uint32_t stride, uint32_t width, BwdArgs
     const uint32_t geo = slot - width;
     constexpr uint32_t nv = LIDAR ? 3 : 2;
     if (geo < G_XY) a.v_conics[g * 3 + geo] += val;
-    else if (geo < G_ABS) a.v_means2d[g * 2 + (geo - G_XY)] += val;
-    else if (geo < G_VEL) { if (a.v_means2d_abs != nullptr) a.v_means2d_abs[g * 2 + (geo - G_ABS)] += val; }
+    else if (geo < G_VEL) a.v_means2d[g * 2 + (geo - G_XY)] += val;
     else if (geo < G_OPAC) a.v_pix_vels[g * nv + (geo - G_VEL)] += val;
     else if (geo == G_OPAC) a.v_opacities[g] += val;
+    else if (geo >= G_ABS) { if (a.v_means2d_abs != nullptr) a.v_means2d_abs[g * 2 + (geo - G_ABS)] += val; }
     else if (geo == G_VELZ) a.v_pix_vels[g * 3 + 2] += val;
     else if (geo < G_D0) a.v_depth_comps[g * 2 + (geo - G_DC)] += val;
 }
@@ -546,9 +555,9 @@ static inline int pick_width(uint32_t n) {
     return -1;
 }
 
-template <int CH, bool LIDAR, int PPL>
+template <int CH, bool LIDAR, int PPL, bool ABS = true>
 static int launch_bwd_as(BwdArgs a, dim3 grid, dim3 block, hipStream_t stream) {
-    const size_t per_gaussian = ((LIDAR ? 48 : 64) + 8) + 4 * CH + 4 * (CH + (LIDAR ? G_COUNT : G_VELZ));
+    const size_t per_gaussian = ((LIDAR ? 48 : 64) + 8) + 4 * CH + 4 * (CH + geo_count(LIDAR, ABS));
     // Batches of the whole workgroup, unless that leaves fewer than four workgroups to a compute
     // unit (160 KB of LDS): a lidar sweep's 1024 tiles then run all at once instead of in two
     // rounds (with 33 channels: 104 Gaussians per batch, 0.39 ms instead of 0.51 ms with 128).
@@ -561,9 +570,9 @@ static int launch_bwd_as(BwdArgs a, dim3 grid, dim3 block, hipStream_t stream) {
     if (a.batch * per_gaussian > room) a.batch = (uint32_t)(room / per_gaussian) / 8 * 8;
     const size_t lds = a.batch * per_gaussian;
     if (lds > 64 * 1024)
-        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_bwd_kernel<CH, LIDAR, PPL>,
+        SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)rasterize_bwd_kernel<CH, LIDAR, PPL, ABS>,
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL((rasterize_bwd_kernel<CH, LIDAR, PPL>), grid, block, lds, stream, a);
+    hipLaunchKernelGGL((rasterize_bwd_kernel<CH, LIDAR, PPL, ABS>), grid, block, lds, stream, a);
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }
@@ -573,8 +582,11 @@ template <int CH, bool LIDAR>
 static int launch_bwd(const BwdArgs &a, dim3 grid, dim3 block, hipStream_t stream) {
     if constexpr (!LIDAR && CH <= 5) {
         const uint32_t pixels = a.tile_w_px * a.tile_h_px;
+        // (without the absolute gradients the two-pixel kernels sum 8 + 4 instead of 16 values per
+        // Gaussian over the wavefront)
         if (a.tile_w_px % 8 == 0 && (pixels / 2) % SPLATAD_WAVE == 0 && block.x == pixels)
-            return launch_bwd_as<CH, LIDAR, 2>(a, grid, dim3(pixels / 2), stream);
+            return a.v_means2d_abs != nullptr ? launch_bwd_as<CH, LIDAR, 2, true>(a, grid, dim3(pixels / 2), stream)
+                                              : launch_bwd_as<CH, LIDAR, 2, false>(a, grid, dim3(pixels / 2), stream);
     }
     return launch_bwd_as<CH, LIDAR, 1>(a, grid, block, stream);
 }
@@ -603,7 +615,7 @@ static int dispatch_bwd(int w, const BwdArgs &a, dim3 grid, dim3 block, hipStrea
 // slots, in whole 64-byte lines.
 static uint32_t packed_stride(uint32_t channels, bool lidar) {
     const uint32_t pass = channels <= (uint32_t)kMaxPass ? channels : 32u;
-    const uint32_t acc = (uint32_t)pick_width(pass) + (lidar ? G_COUNT : G_VELZ);
+    const uint32_t acc = (uint32_t)pick_width(pass) + (uint32_t)geo_count(lidar);
     return (acc + 15u) / 16u * 16u;
 }
 
