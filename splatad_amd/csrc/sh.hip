@@ -215,8 +215,11 @@ sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, ShView view, const float
         float gx = 0.f, gy = 0.f, gz = 0.f;
         // the whole coefficient row is requested before the first use, one memory round trip
         // instead of one per degree
+        // (only for rows that take a gradient: where few of the visible rows were composited
+        // -- a frame that saturates in its nearest Gaussians -- the coefficient rows are most
+        // of what this kernel would read)
         float c[DIRS ? 75 : 1] = {};
-        if (DIRS && active) {
+        if (DIRS && active && (vr != 0.f || vg != 0.f || vb != 0.f)) {
             sh_load_band<0>(c, cf);
             if (degree >= 1) sh_load_band<1>(c, cf); // uniform
             if (degree >= 2) sh_load_band<2>(c, cf);

@@ -453,11 +453,16 @@ def rasterize_to_pixels_with_sh(
     backgrounds: Optional[Tensor] = None,  # [C, 3 or 4]
     gaussian_ids: Optional[Tensor] = None,  # [nnz]: the rows are packed
     color_cache: Optional[Tensor] = None,  # [C, N, 4] or [nnz, 4], from view_dependent_color_cache
+    radii: Optional[Tensor] = None,  # [C, N, 2] or [nnz, 2]: needed where a gradient is wanted
+    camera_ids: Optional[Tensor] = None,  # [nnz], with gaussian_ids and radii
+    absgrad: bool = False,
 ) -> Tuple[Tensor, Tensor]:
-    """`view_dependent_colors` and `rasterize_to_pixels` in one kernel, forward only: the
-    compositing kernel evaluates the colour of the list entries it stages (the ones tiles reach
-    before they saturate) instead of reading colours made for every visible Gaussian
-    beforehand.  Same images, bit for bit, as the two operators one after the other.
+    """`view_dependent_colors` and `rasterize_to_pixels` in one kernel: the compositing kernel
+    evaluates the colour of the list entries it stages (the ones tiles reach before they
+    saturate) instead of reading colours made for every visible Gaussian beforehand.  Same
+    images, bit for bit, as the two operators one after the other.  Differentiable in what the
+    two operators are differentiable in (not the view matrices) when `radii` is given: the
+    backward pass takes the colours from what the forward pass left in the cache.
 
     color_cache: where the first tiles to stage a row leave its colour for the others; made by
     `view_dependent_color_cache`, which also decides whether to evaluate all rows beforehand
@@ -491,8 +496,19 @@ def rasterize_to_pixels_with_sh(
     assert tile_width * tile_size >= image_width, f"Assert Failed: {tile_width} * {tile_size} >= {image_width}"
     tensors = (means, viewmats, sh_coeffs, depths, means2d, conics, opacities, pix_vels, backgrounds)
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
-        raise ValueError("rasterize_to_pixels_with_sh is forward only: use view_dependent_colors "
-                         "and rasterize_to_pixels where a gradient is wanted")
+        if viewmats.requires_grad or radii is None:
+            raise ValueError("rasterize_to_pixels_with_sh: gradients need `radii` and view matrices "
+                             "that take none; use view_dependent_colors and rasterize_to_pixels otherwise")
+        assert radii.shape == rows + (2,), radii.shape
+        assert (camera_ids is None) == (gaussian_ids is None)
+        if color_cache is None:
+            color_cache = torch.full(rows + (4,), float("nan"), dtype=torch.float32, device=means2d.device)
+        return _RasterizeToPixelsWithSH.apply(
+            sh_degree, means.contiguous(), viewmats.contiguous(), sh_coeffs.contiguous(), _c(depths),
+            radii.contiguous(), _c(camera_ids), _c(gaussian_ids), means2d.contiguous(), conics.contiguous(),
+            opacities.contiguous(), pix_vels.contiguous(), rolling_shutter_time.contiguous(), backgrounds,
+            image_width, image_height, tile_size, isect_offsets.contiguous(), flatten_ids.contiguous(),
+            color_cache, absgrad)
     render_colors, render_alphas, _ = _make_lazy_hip_func("rasterize_to_pixels_sh_fwd")(
         sh_degree, means.contiguous(), viewmats.contiguous(), sh_coeffs.contiguous(), _c(gaussian_ids),
         _c(depths), means2d.contiguous(), conics.contiguous(), opacities.contiguous(), pix_vels.contiguous(),
@@ -1125,35 +1141,92 @@ class _ViewColors(torch.autograd.Function):
     @staticmethod
     def backward(ctx, v_colors):
         means, viewmats, coeffs, radii, camera_ids, gaussian_ids, colors = ctx.saved_tensors
-        need_means, need_coeffs = ctx.needs_input_grad[1], ctx.needs_input_grad[3]
-        v_means = v_coeffs = v_depths = None
-        if need_means or need_coeffs:
-            # rows of one Gaussian seen by several sensors add up; for packed rows the kernel adds
-            # the coefficient gradients at their Gaussians itself (one pass over them instead of
-            # a [nnz, K, 3] tensor and an index_add_ over it)
-            packed = camera_ids is not None
-            scatter = packed and need_coeffs
-            v_rows, v_dirs = _make_lazy_hip_func("view_colors_bwd")(
-                ctx.sh_degree, means, viewmats, camera_ids, gaussian_ids, radii, coeffs, colors,
-                v_colors.contiguous(), need_means, scatter)
-            if need_coeffs:
-                if scatter:
-                    v_coeffs = v_rows
-                elif coeffs.dim() == 4:
-                    v_coeffs = (torch.zeros_like(coeffs).index_put_((camera_ids, gaussian_ids), v_rows, accumulate=True)
-                                if packed else v_rows)
-                elif packed:
-                    v_coeffs = torch.zeros_like(coeffs).index_add_(0, gaussian_ids, v_rows)
-                else:
-                    v_coeffs = v_rows[0] if v_rows.shape[0] == 1 else v_rows.sum(0)
-            if need_means:
-                if packed:
-                    v_means = torch.zeros_like(means).index_add_(0, gaussian_ids, v_dirs)
-                else:
-                    v_means = v_dirs[0] if v_dirs.shape[0] == 1 else v_dirs.sum(0)
-        if ctx.has_depths and ctx.needs_input_grad[5]:
-            v_depths = v_colors[..., 3]
+        v_means, v_coeffs = _view_colors_backward(
+            ctx.sh_degree, means, viewmats, coeffs, radii, camera_ids, gaussian_ids, colors, v_colors,
+            ctx.needs_input_grad[1], ctx.needs_input_grad[3])
+        v_depths = v_colors[..., 3] if ctx.has_depths and ctx.needs_input_grad[5] else None
         return None, v_means, None, v_coeffs, None, v_depths, None, None, None, None
+
+
+def _view_colors_backward(sh_degree, means, viewmats, coeffs, radii, camera_ids, gaussian_ids, colors,
+                          v_colors, need_means, need_coeffs):
+    """Gradients of the view-dependent colours with respect to the means and the coefficients,
+    summed over the sensors that see a Gaussian; (None, None) where neither is wanted."""
+    v_means = v_coeffs = None
+    if need_means or need_coeffs:
+        # rows of one Gaussian seen by several sensors add up; for packed rows the kernel adds
+        # the coefficient gradients at their Gaussians itself (one pass over them instead of
+        # a [nnz, K, 3] tensor and an index_add_ over it)
+        packed = camera_ids is not None
+        scatter = packed and need_coeffs
+        v_rows, v_dirs = _make_lazy_hip_func("view_colors_bwd")(
+            sh_degree, means, viewmats, camera_ids, gaussian_ids, radii, coeffs, colors,
+            v_colors.contiguous(), need_means, scatter)
+        if need_coeffs:
+            if scatter:
+                v_coeffs = v_rows
+            elif coeffs.dim() == 4:
+                v_coeffs = (torch.zeros_like(coeffs).index_put_((camera_ids, gaussian_ids), v_rows, accumulate=True)
+                            if packed else v_rows)
+            elif packed:
+                v_coeffs = torch.zeros_like(coeffs).index_add_(0, gaussian_ids, v_rows)
+            else:
+                v_coeffs = v_rows[0] if v_rows.shape[0] == 1 else v_rows.sum(0)
+        if need_means:
+            if packed:
+                v_means = torch.zeros_like(means).index_add_(0, gaussian_ids, v_dirs)
+            else:
+                v_means = v_dirs[0] if v_dirs.shape[0] == 1 else v_dirs.sum(0)
+    return v_means, v_coeffs
+
+
+class _RasterizeToPixelsWithSH(torch.autograd.Function):
+    """rasterize_to_pixels_with_sh for calls that want gradients: the forward pass is the kernel
+    that evaluates the colours of the entries it stages; what it leaves in the colour cache --
+    the colour (and depth) of every row some tile staged -- is all the backward pass needs of the
+    colours, because a row that no tile staged was composited nowhere and takes no gradient."""
+
+    @staticmethod
+    def forward(ctx, sh_degree, means, viewmats, coeffs, depths, radii, camera_ids, gaussian_ids, means2d,
+                conics, opacities, pix_vels, rolling_shutter_time, backgrounds, width, height, tile_size,
+                isect_offsets, flatten_ids, color_cache, absgrad):
+        render_colors, render_alphas, last_ids = _make_lazy_hip_func("rasterize_to_pixels_sh_fwd")(
+            sh_degree, means, viewmats, coeffs, gaussian_ids, depths, means2d, conics, opacities, pix_vels,
+            rolling_shutter_time, backgrounds, width, height, tile_size, isect_offsets, flatten_ids,
+            cache=color_cache, want_last_ids=True)
+        ctx.save_for_backward(means, viewmats, coeffs, radii, camera_ids, gaussian_ids, means2d, conics,
+                              opacities, pix_vels, rolling_shutter_time, backgrounds, isect_offsets, flatten_ids,
+                              render_alphas, last_ids, color_cache)
+        ctx.sh_degree, ctx.has_depths = sh_degree, depths is not None
+        ctx.width, ctx.height, ctx.tile_size, ctx.absgrad = width, height, tile_size, absgrad
+        return render_colors, render_alphas.float()
+
+    @staticmethod
+    def backward(ctx, v_render_colors, v_render_alphas):
+        (means, viewmats, coeffs, radii, camera_ids, gaussian_ids, means2d, conics, opacities, pix_vels,
+         rolling_shutter_time, backgrounds, isect_offsets, flatten_ids, render_alphas, last_ids,
+         cache) = ctx.saved_tensors
+        # the rows' colours as the forward pass evaluated them; rows it never staged hold NaN,
+        # are read by no pixel that composited them, and count as zero
+        colors = torch.nan_to_num(cache, nan=0.0, posinf=float("inf"), neginf=-float("inf"))
+        if not ctx.has_depths:
+            colors = colors[..., :3].contiguous()
+        (v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities,
+         v_pix_vels) = _make_lazy_hip_func("rasterize_to_pixels_bwd")(
+            means2d, conics, colors, opacities, pix_vels, rolling_shutter_time, backgrounds,
+            ctx.width, ctx.height, ctx.tile_size, isect_offsets, flatten_ids, render_alphas,
+            last_ids, v_render_colors.contiguous(), v_render_alphas.contiguous(), ctx.absgrad)
+        if ctx.absgrad:
+            means2d.absgrad = v_means2d_abs
+        v_means, v_coeffs = _view_colors_backward(
+            ctx.sh_degree, means, viewmats, coeffs, radii, camera_ids, gaussian_ids, colors, v_colors,
+            ctx.needs_input_grad[1], ctx.needs_input_grad[3])
+        v_depths = v_colors[..., 3] if ctx.has_depths and ctx.needs_input_grad[4] else None
+        v_backgrounds = None
+        if ctx.needs_input_grad[13]:
+            v_backgrounds = (v_render_colors * (1.0 - render_alphas).float()).sum(dim=(1, 2))
+        return (None, v_means, None, v_coeffs, v_depths, None, None, None, v_means2d, v_conics, v_opacities,
+                v_pix_vels, None, v_backgrounds, None, None, None, None, None, None, None)
 
 
 class _SphericalHarmonics(torch.autograd.Function):

@@ -61,8 +61,9 @@ class _CameraPlan:
 
     colors            who makes the per-row colours: "given" (post-activation features),
                       "view_kernel" (one kernel: directions, SH, activation, depth channel),
-                      "while_compositing" (forward-only calls: the compositing kernel evaluates
-                      the colours of the entries it stages) or "sh_operators" (view matrices that
+                      "while_compositing" (the compositing kernel evaluates the colours of the
+                      entries it stages, and its backward pass takes them from what that left
+                      in the colour cache) or "sh_operators" (view matrices that
                       take a gradient: directions and SH by differentiable operators);
     depth_in_colors   the colour maker appends the depth channel itself;
     requests          what a packed projection is asked to make of its rows besides the rows:
@@ -81,8 +82,7 @@ class _CameraPlan:
         elif viewmats.requires_grad:
             self.colors = "sh_operators"
         elif (means.is_cuda and render_mode in ("RGB", "RGB+D", "RGB+ED") and colors.dtype == torch.float32
-              and opacities.dtype == torch.float32
-              and not wanted(means, quats, scales, opacities, colors, velocities, viewmats, backgrounds)):
+              and opacities.dtype == torch.float32):
             self.colors = "while_compositing"
         else:
             self.colors = "view_kernel"
@@ -287,7 +287,7 @@ def rasterization(
             sh_degree, means, viewmats, colors, depths_for_colors, means2d, conics,
             opacities, pix_vels, width, height, tile_size, isect_offsets, flatten_ids,
             rolling_shutter_time, backgrounds=backgrounds, gaussian_ids=gaussian_ids,
-            color_cache=color_cache)
+            color_cache=color_cache, radii=radii, camera_ids=camera_ids, absgrad=absgrad)
     else:
         render_colors, render_alphas = composite(colors, backgrounds)
 
