@@ -463,6 +463,27 @@ int splatad_rasterize_to_pixels_bwd(uint32_t C, int64_t n_isects, uint32_t chann
                                     uint64_t total, void *workspace, size_t workspace_bytes,
                                     splatad_stream_t stream);
 
+/* The backward pass of splatad_rasterize_to_pixels_fwd_sh (which has no counterpart in the
+ * reference): splatad_rasterize_to_pixels_bwd with `colors` = the colour cache that call left
+ * behind ([rows, 4], of which `channels` = 4 are composited; for 3 channels hand over a
+ * contiguous [rows, 3] copy).  Rows that no tile staged hold NaN there; no pixel composited
+ * them, their gradient is zero, and the kernel takes their colour as zero.  v_colors then goes
+ * to splatad_view_colors_bwd. */
+int splatad_rasterize_to_pixels_bwd_sh(uint32_t C, int64_t n_isects, uint32_t channels,
+                                    const float *means2d, const float *conics,
+                                    const float *colors, const float *opacities,
+                                    const float *pix_vels, const float *rolling_shutter_time,
+                                    const float *backgrounds, uint32_t image_width,
+                                    uint32_t image_height, uint32_t tile_size,
+                                    uint32_t tile_width, uint32_t tile_height,
+                                    const int32_t *tile_offsets, const int32_t *flatten_ids,
+                                    const float *render_alphas, const int32_t *last_ids,
+                                    const float *v_render_colors, const float *v_render_alphas,
+                                    float *v_means2d_abs, float *v_means2d, float *v_conics,
+                                    float *v_colors, float *v_opacities, float *v_pix_vels,
+                                    uint64_t total, void *workspace, size_t workspace_bytes,
+                                    splatad_stream_t stream);
+
 /* rasterize_to_points_fwd_tensor, rasterization.cu:2221-2831 (kernel
  * :2021-2219).  Outputs of inactive points (range <= 0) are zero.
  * alpha_sum_until_points may be NULL when compute_alpha_sum_until_points == 0.

@@ -48,6 +48,9 @@ struct BwdArgs {
     float *packed;
     uint32_t packed_stride;
     uint32_t batch; // Gaussians staged per batch, at most the workgroup size
+    // `colors` is the colour cache a forward pass that evaluated the colours itself left behind:
+    // rows no tile staged hold NaN; no pixel composited them, and they are taken as zero
+    int colors_from_cache;
 };
 
 // Geometry slots per Gaussian in the LDS accumulator, after the CH colour slots; those from
@@ -289,6 +292,7 @@ rasterize_bwd_kernel(BwdArgs a) {
                 const uint32_t c = a.ch_offset + k;
                 float v = 0.f;
                 if ((uint32_t)k < a.n_ch) v = split && c == a.depth_idx ? f.depth_col : crow[min(c, a.feat_stride - 1u)];
+                if (!LIDAR && a.colors_from_cache && !(v == v)) v = 0.f;
                 f.col[k] = v;
             }
         }
@@ -663,7 +667,7 @@ extern "C" size_t splatad_rasterize_bwd_workspace_bytes(uint64_t total, uint32_t
     return (size_t)(total * packed_stride(channels ? channels : 1, lidar != 0) * sizeof(float));
 }
 
-extern "C" int splatad_rasterize_to_pixels_bwd(
+static int pixels_bwd(int colors_from_cache,
     uint32_t C, int64_t n_isects, uint32_t channels, const float *means2d, const float *conics,
     const float *colors, const float *opacities, const float *pix_vels, const float *rs_time,
     const float *backgrounds, uint32_t W, uint32_t H, uint32_t tile_size, uint32_t tile_w,
@@ -684,6 +688,7 @@ extern "C" int splatad_rasterize_to_pixels_bwd(
                         v_means2d && v_conics && v_colors && v_opacities && v_pix_vels,
                     "rasterize_to_pixels bwd: null pointer argument");
     BwdArgs a = {};
+    a.colors_from_cache = colors_from_cache;
     a.C = C; a.n_isects = n_isects; a.color_stride = channels; a.feat_stride = channels;
     a.means2d = means2d; a.conics = conics; a.colors = colors; a.opacities = opacities;
     a.pix_vels = pix_vels; a.rs_time = rs_time; a.backgrounds = backgrounds;
@@ -696,6 +701,38 @@ extern "C" int splatad_rasterize_to_pixels_bwd(
     return run_passes<false>(a, channels, dim3(C * tile_w * tile_h),
                              dim3((tile_size * tile_size + 63) / 64 * 64), total, workspace,
                              workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int splatad_rasterize_to_pixels_bwd(
+    uint32_t C, int64_t n_isects, uint32_t channels, const float *means2d, const float *conics,
+    const float *colors, const float *opacities, const float *pix_vels, const float *rs_time,
+    const float *backgrounds, uint32_t W, uint32_t H, uint32_t tile_size, uint32_t tile_w,
+    uint32_t tile_h, const int32_t *tile_offsets, const int32_t *flatten_ids,
+    const float *render_alphas, const int32_t *last_ids, const float *v_render_colors,
+    const float *v_render_alphas, float *v_means2d_abs, float *v_means2d, float *v_conics,
+    float *v_colors, float *v_opacities, float *v_pix_vels, uint64_t total, void *workspace,
+    size_t workspace_bytes, splatad_stream_t stream) {
+    return pixels_bwd(0, C, n_isects, channels, means2d, conics, colors, opacities, pix_vels, rs_time,
+                      backgrounds, W, H, tile_size, tile_w, tile_h, tile_offsets, flatten_ids,
+                      render_alphas, last_ids, v_render_colors, v_render_alphas, v_means2d_abs, v_means2d,
+                      v_conics, v_colors, v_opacities, v_pix_vels, total, workspace, workspace_bytes,
+                      stream);
+}
+
+extern "C" int splatad_rasterize_to_pixels_bwd_sh(
+    uint32_t C, int64_t n_isects, uint32_t channels, const float *means2d, const float *conics,
+    const float *colors, const float *opacities, const float *pix_vels, const float *rs_time,
+    const float *backgrounds, uint32_t W, uint32_t H, uint32_t tile_size, uint32_t tile_w,
+    uint32_t tile_h, const int32_t *tile_offsets, const int32_t *flatten_ids,
+    const float *render_alphas, const int32_t *last_ids, const float *v_render_colors,
+    const float *v_render_alphas, float *v_means2d_abs, float *v_means2d, float *v_conics,
+    float *v_colors, float *v_opacities, float *v_pix_vels, uint64_t total, void *workspace,
+    size_t workspace_bytes, splatad_stream_t stream) {
+    return pixels_bwd(1, C, n_isects, channels, means2d, conics, colors, opacities, pix_vels, rs_time,
+                      backgrounds, W, H, tile_size, tile_w, tile_h, tile_offsets, flatten_ids,
+                      render_alphas, last_ids, v_render_colors, v_render_alphas, v_means2d_abs, v_means2d,
+                      v_conics, v_colors, v_opacities, v_pix_vels, total, workspace, workspace_bytes,
+                      stream);
 }
 
 extern "C" int splatad_rasterize_to_points_bwd(

@@ -960,7 +960,9 @@ class _Ops:
     def rasterize_to_pixels_bwd(self, means2d, conics, colors, opacities, pix_vels,
                                 rolling_shutter_time, backgrounds, image_width, image_height,
                                 tile_size, tile_offsets, flatten_ids, render_alphas, last_ids,
-                                v_render_colors, v_render_alphas, absgrad):
+                                v_render_colors, v_render_alphas, absgrad, colors_from_cache=False):
+        """colors_from_cache: `colors` is the colour cache rasterize_to_pixels_sh_fwd left behind
+        (NaN rows = never staged, taken as zero)."""
         lib = load_library()
         means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
         colors = _in(colors, "colors"); opacities = _in(opacities, "opacities")
@@ -980,7 +982,8 @@ class _Ops:
             total = means2d.numel() // 2
             with _on(dev):
                 ws = _bwd_workspace(lib, total, D, False, dev)
-                _check(lib.splatad_rasterize_to_pixels_bwd(
+                entry = lib.splatad_rasterize_to_pixels_bwd_sh if colors_from_cache else lib.splatad_rasterize_to_pixels_bwd
+                _check(entry(
                     _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics),
                     _p(colors), _p(opacities), _p(pix_vels), _p(rs), _p(backgrounds),
                     _u32(image_width), _u32(image_height), _u32(tile_size), _u32(tw), _u32(th),

@@ -1207,15 +1207,15 @@ class _RasterizeToPixelsWithSH(torch.autograd.Function):
          rolling_shutter_time, backgrounds, isect_offsets, flatten_ids, render_alphas, last_ids,
          cache) = ctx.saved_tensors
         # the rows' colours as the forward pass evaluated them; rows it never staged hold NaN,
-        # are read by no pixel that composited them, and count as zero
-        colors = torch.nan_to_num(cache, nan=0.0, posinf=float("inf"), neginf=-float("inf"))
-        if not ctx.has_depths:
-            colors = colors[..., :3].contiguous()
+        # are read by no pixel that composited them, and count as zero in both kernels below
+        # (the SH backward only asks whether a colour is positive)
+        colors = cache if ctx.has_depths else cache[..., :3].contiguous()
         (v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities,
          v_pix_vels) = _make_lazy_hip_func("rasterize_to_pixels_bwd")(
             means2d, conics, colors, opacities, pix_vels, rolling_shutter_time, backgrounds,
             ctx.width, ctx.height, ctx.tile_size, isect_offsets, flatten_ids, render_alphas,
-            last_ids, v_render_colors.contiguous(), v_render_alphas.contiguous(), ctx.absgrad)
+            last_ids, v_render_colors.contiguous(), v_render_alphas.contiguous(), ctx.absgrad,
+            colors_from_cache=True)
         if ctx.absgrad:
             means2d.absgrad = v_means2d_abs
         v_means, v_coeffs = _view_colors_backward(
