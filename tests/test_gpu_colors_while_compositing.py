@@ -129,7 +129,7 @@ def test_colour_cache_empty_or_filled_by_the_opacity_a_tile_carries(packed, with
                 assert torch.equal(cache[held][:, :3], colors[held][:, :3])
 
 
-def test_colours_while_compositing_is_forward_only_and_checks_its_rows():
+def test_colours_while_compositing_checks_its_rows_and_what_a_gradient_needs():
     from splatad_amd.hip._wrapper import rasterize_to_pixels_with_sh
     d, p = _projected(1, 500, 64, 48, 16, False, seed=4)
     coeffs = torch.zeros((500, 16, 3), device=DEV)
@@ -138,16 +138,77 @@ def test_colours_while_compositing_is_forward_only_and_checks_its_rows():
     rc, ra = rasterize_to_pixels_with_sh(*args)
     # zero coefficients: every colour is max(0 + 1/2, 0), so a pixel holds alpha / 2
     torch.testing.assert_close(rc, (0.5 * ra).expand(-1, -1, -1, 3), atol=1e-6, rtol=1e-6)
-    with pytest.raises(ValueError, match="forward only"):
-        rasterize_to_pixels_with_sh(3, d["means"], d["viewmats"], coeffs.requires_grad_(), *args[4:])
+    with pytest.raises(ValueError, match="gradients need `radii`"):
+        rasterize_to_pixels_with_sh(3, d["means"], d["viewmats"], coeffs.clone().requires_grad_(), *args[4:])
+    with pytest.raises(ValueError, match="view matrices"):
+        rasterize_to_pixels_with_sh(3, d["means"], d["viewmats"].clone().requires_grad_(), *args[3:],
+                                    radii=p["radii"])
     with pytest.raises(AssertionError):  # degree 4 needs 25 coefficients
         rasterize_to_pixels_with_sh(4, *args[1:])
 
 
-def test_rasterization_switches_to_the_colour_kernel_when_a_gradient_is_wanted():
-    """rasterization() evaluates the colours while compositing only when no input takes a
-    gradient; with one that does it runs the colour kernel and the differentiable operators,
-    and renders the same image."""
+@pytest.mark.parametrize("C,degree,with_depth,packed,absgrad", [
+    (1, 3, True, False, False),   # the driving camera's training step
+    (2, 3, False, False, True),
+    (2, 2, True, True, False),
+    (2, 1, True, True, True),
+])
+def test_gradients_through_colours_evaluated_while_compositing_equal_the_two_operators(C, degree, with_depth,
+                                                                                      packed, absgrad):
+    """The backward pass of `rasterize_to_pixels_with_sh` composites with the colours the forward
+    kernel left in its cache (rows no tile staged count as zero: no pixel's gradient reaches
+    them) and sends the colour gradients through the colour kernel's backward pass.  Every
+    gradient has to equal the one of `view_dependent_colors` + `rasterize_to_pixels`, which
+    other tests compare with the float64 oracle, up to the order of the float32 sums."""
+    from splatad_amd.hip._wrapper import (rasterize_to_pixels, rasterize_to_pixels_with_sh,
+                                          view_dependent_colors)
+    N, W, H, ts = 5000, 160, 96, 16
+    d, p = _projected(C, N, W, H, ts, packed, seed=40 + degree)
+    g = torch.Generator(device=DEV).manual_seed(5)
+    coeffs0 = torch.randn((N, (degree + 1) ** 2, 3), device=DEV, generator=g) * 0.4
+    bg0 = torch.rand((C, 4 if with_depth else 3), device=DEV, generator=g)
+    weights = torch.rand((C, H, W, 5 if with_depth else 4), device=DEV, generator=g)
+    names = ("means", "coeffs", "depths", "means2d", "conics", "opacities", "backgrounds")
+
+    def leaves():
+        out = dict(means=d["means"], coeffs=coeffs0, depths=p["depths"] if with_depth else None,
+                   means2d=p["means2d"], conics=p["conics"], opacities=p["opacities"], backgrounds=bg0)
+        return {k: (None if v is None else v.detach().clone().requires_grad_()) for k, v in out.items()}
+
+    def loss(render):
+        return (torch.cat(render, dim=-1) * weights).sum()
+
+    a = leaves()
+    if absgrad:
+        a["means2d"].absgrad = None
+    colors = view_dependent_colors(degree, a["means"], d["viewmats"], a["coeffs"], p["radii"], a["depths"],
+                                   p["camera_ids"], p["gaussian_ids"])
+    want = rasterize_to_pixels(a["means2d"], a["conics"], colors, a["opacities"], p["pix_vels"], W, H, ts,
+                               p["offsets"], p["flatten_ids"], d["rolling_shutter_time"],
+                               backgrounds=a["backgrounds"], packed=packed, absgrad=absgrad)
+    loss(want).backward()
+    b = leaves()
+    got = rasterize_to_pixels_with_sh(degree, b["means"], d["viewmats"], b["coeffs"], b["depths"], b["means2d"],
+                                      b["conics"], b["opacities"], p["pix_vels"], W, H, ts, p["offsets"],
+                                      p["flatten_ids"], d["rolling_shutter_time"], backgrounds=b["backgrounds"],
+                                      gaussian_ids=p["gaussian_ids"], radii=p["radii"],
+                                      camera_ids=p["camera_ids"], absgrad=absgrad)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    loss(got).backward()
+    for k in names:
+        if a[k] is None:
+            continue
+        assert b[k].grad is not None and float(a[k].grad.abs().max()) > 0, k
+        scale = float(a[k].grad.abs().max())
+        torch.testing.assert_close(b[k].grad, a[k].grad, atol=2e-5 * scale, rtol=1e-4, msg=lambda m, k=k: f"{k}: {m}")
+    if absgrad:
+        scale = float(a["means2d"].absgrad.abs().max())
+        torch.testing.assert_close(b["means2d"].absgrad, a["means2d"].absgrad, atol=2e-5 * scale, rtol=1e-4)
+
+
+def test_rasterization_renders_the_same_image_when_a_gradient_is_wanted():
+    """rasterization() renders the same image, bit for bit, whether or not an input takes a
+    gradient, and the gradient reaches the coefficients."""
     from splatad_amd import rasterization
     s = workloads.camera_driving(n=8000, width=256, height=144, n_cameras=2)
     d = workloads.to_device(s, DEV)
