@@ -134,7 +134,9 @@ __device__ __forceinline__ uint32_t tile_index(const TileGrid &g, int32_t y, int
 // and zero again when it ends) takes the partial sums; the total goes to the host's pinned
 // slot.  On its way the kernel clears `clear_words` words from `clear` on: the counters of the
 // binning kernels behind it, which spares the launch of a clearing kernel.
+constexpr uint32_t kSlabShiftMax = 4;
 constexpr uint32_t kSlabSamples = 256;
+constexpr uint32_t kSlabEstimates = 4; // independent sets of samples, a workgroup each
 
 template <typename Load, typename Store>
 __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t L, uint32_t tid, uint32_t nt,
@@ -167,6 +169,38 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t L, uint32_t ti
     return total;
 }
 
+// All comparators of this bitonic network point the same way (the first stage of every
+// merge is a "flip"), so a virtual +inf tail needs no storage: pairs whose upper index is
+// >= n are skipped.
+template <typename Ptr>
+__device__ __forceinline__ void bitonic_sort_ascending(Ptr a, uint32_t n, uint32_t tid,
+                                                       uint32_t nthreads) {
+    uint32_t m = 1;
+    while (m < n) m <<= 1;
+    for (uint32_t k = 2; k <= m; k <<= 1) {
+        for (uint32_t i = tid; i < m / 2; i += nthreads) {
+            const uint32_t lo = ((i / (k / 2)) * k) + (i % (k / 2));
+            const uint32_t hi = lo ^ (k - 1);
+            if (hi < n) {
+                const uint64_t x = a[lo], y = a[hi];
+                if (y < x) { a[lo] = y; a[hi] = x; }
+            }
+        }
+        __syncthreads();
+        for (uint32_t j = k / 4; j > 0; j >>= 1) {
+            for (uint32_t i = tid; i < m / 2; i += nthreads) {
+                const uint32_t lo = ((i / j) * (2 * j)) + (i % j);
+                const uint32_t hi = lo + j;
+                if (hi < n) {
+                    const uint64_t x = a[lo], y = a[hi];
+                    if (y < x) { a[lo] = y; a[hi] = x; }
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
 // One workgroup, one sample per lane: kSlabSamples Gaussians at a fixed stride, ordered by
 // depth (every lane counts the smaller keys; all lanes read the same LDS words, which are
 // broadcasts).  A key is the depth bits with the sample's index in the low bits, which makes
@@ -177,7 +211,7 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t L, uint32_t ti
 // 6 us and a launch gap per lidar call).
 template <typename Weight>
 __device__ __forceinline__ void slab_bounds_workgroup(uint64_t total, const float *__restrict__ depths,
-                                                      Weight &&weight_of, uint32_t n_slabs,
+                                                      Weight &&weight_of, uint32_t n_slabs, uint32_t estimate,
                                                       uint32_t *__restrict__ bounds) {
     static_assert((kSlabSamples & (kSlabSamples - 1)) == 0 && kSlabSamples % 4 == 0, "power of two");
     static_assert(kSlabSamples == SPLATAD_THREADS, "one sample per lane of a counting workgroup");
@@ -187,13 +221,16 @@ __device__ __forceinline__ void slab_bounds_workgroup(uint64_t total, const floa
     __shared__ uint32_t s_before[kSlabSamples];
     __shared__ uint32_t s_wave[2 * (kSlabSamples / SPLATAD_WAVE)];
     const uint32_t tid = threadIdx.x;
-    const uint64_t n = total < kSlabSamples ? total : kSlabSamples;
-    const uint64_t stride = n ? total / n : 1;
+    // (estimate e of kSlabEstimates takes every kSlabEstimates-th of the samples, from the e-th on)
+    const uint64_t n_all = total < kSlabSamples * kSlabEstimates ? total : kSlabSamples * kSlabEstimates;
+    const uint64_t stride = n_all ? total / n_all : 1;
+    const uint64_t at = ((uint64_t)tid * kSlabEstimates + estimate) * stride;
     uint32_t key = ~(kSlabSamples - 1u) | tid, weight = 0; // no tiles: behind every depth
-    if (tid < n) {
-        const int32_t w = weight_of(tid * stride);
+    bounds += (size_t)estimate << kSlabShiftMax;
+    if (at < total) {
+        const int32_t w = weight_of(at);
         if (w > 0) {
-            key = (__float_as_uint(depths[tid * stride]) & ~(kSlabSamples - 1u)) | tid;
+            key = (__float_as_uint(depths[at]) & ~(kSlabSamples - 1u)) | tid;
             weight = (uint32_t)min(w, 1 << 20); // capped: the sum stays below 2^32
         }
     }
@@ -228,22 +265,24 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
                    unsigned long long *__restrict__ counters,
                    unsigned long long *__restrict__ n_isects_host, int32_t *__restrict__ clear,
                    uint64_t clear_words, const float *__restrict__ depths, uint32_t n_slabs,
-                   uint32_t *__restrict__ slab_bounds) {
+                   uint32_t *__restrict__ slab_bounds, int unit_weights) {
     SPLATAD_STAGE_ELEVATIONS(g)
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words;
          i += (uint64_t)gridDim.x * blockDim.x)
         clear[i] = 0;
-    // SLABS: the launch has one workgroup more than count, and that one finds the depth slabs'
-    // bounds meanwhile (it counts the tiles of its samples itself)
-    const uint32_t n_wgs = gridDim.x - (SLABS ? 1u : 0u);
-    if (SLABS && blockIdx.x == n_wgs) { // uniform across the workgroup
+    // SLABS: the launch has kSlabEstimates workgroups more than count, and those find the depth
+    // slabs' bounds meanwhile, each from samples of its own (they count their samples' tiles
+    // themselves); the bounds used are the means of the estimates
+    const uint32_t n_wgs = gridDim.x - (SLABS ? kSlabEstimates : 0u);
+    if (SLABS && blockIdx.x >= n_wgs) { // uniform across the workgroup
         slab_bounds_workgroup(total, depths, [&](uint64_t i) -> int32_t {
             float2 mu = reinterpret_cast<const float2 *>(means2d)[i];
             uint2 rad = reinterpret_cast<const uint2 *>(radii)[i];
             int32_t x0, y0, x1, y1;
             if (!tile_rect_of<LIDAR>(g, mu, rad, x0, y0, x1, y1)) return 0;
-            return max(y1 - y0, 0) * max(x1 - x0, 0);
-        }, n_slabs, slab_bounds);
+            const int32_t tiles = max(y1 - y0, 0) * max(x1 - x0, 0);
+            return unit_weights ? min(tiles, 1) : tiles;
+        }, n_slabs, blockIdx.x - n_wgs, slab_bounds);
         return;
     }
     long long s = 0;
@@ -497,7 +536,6 @@ __device__ __forceinline__ uint32_t coarse_mask(const LaneWork &w, const CoarseG
 // the depth bits the result is the same list.  The bounds are weighted quantiles of a sample
 // of the depths (weight = tiles met), so the sub-segments of an average tile are about equal;
 // any bounds whatsoever give the same output, balance is all they decide.
-constexpr uint32_t kSlabShiftMax = 4;
 // Slabs pay once a tile's segment outgrows the sort's short classes (beyond about 8000 entries,
 // i.e. several hundred Gaussians per tile); below that they only lengthen the binning.  Measured
 // on lidar sweeps of 0.25-4M Gaussians on 1024 tiles (whole call in ms with 0 / 4 / 8 / 16 slabs:
@@ -516,6 +554,18 @@ static uint32_t slab_shift_for(uint64_t total, uint64_t segs) {
     if (per_tile < 896) return 2;
     if (per_tile < 2816) return 3;
     return kSlabShiftMax;
+}
+
+// Bound k from the kSlabEstimates estimates of it ([estimate][1 << kSlabShiftMax]): the mean of
+// those that found one (an estimate whose samples met no tile has none).
+__device__ __forceinline__ uint32_t slab_bound(const uint32_t *__restrict__ estimates, uint32_t k) {
+    uint64_t sum = 0;
+    uint32_t found = 0;
+    for (uint32_t e = 0; e < kSlabEstimates; ++e) {
+        const uint32_t b = estimates[(e << kSlabShiftMax) + k];
+        if (b != 0xFFFFFFFFu) { sum += b; ++found; }
+    }
+    return found ? (uint32_t)(sum / found) : 0xFFFFFFFFu;
 }
 
 // Number of bounds at or below the depth bits: non-decreasing in d whatever the bounds hold.
@@ -550,10 +600,12 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
                     uint4 *__restrict__ entries, uint32_t sshift,
                     const uint32_t *__restrict__ slab_bounds, const int32_t *__restrict__ remap,
                     int32_t *__restrict__ tiles_out, int32_t *__restrict__ totals,
-                    int64_t *__restrict__ n_entries, uint32_t entries_cap) {
+                    int64_t *__restrict__ n_entries, uint32_t entries_cap,
+                    uint32_t *__restrict__ list_starts, unsigned long long *__restrict__ longest_host) {
     extern __shared__ int32_t s_blocks[];
     __shared__ uint32_t s_bounds[1u << kSlabShiftMax];
     __shared__ uint32_t s_scan[kCoarseThreads / SPLATAD_WAVE];
+    __shared__ uint32_t s_longest;
     SPLATAD_STAGE_ELEVATIONS(g)
     // blocks and block counters below are (coarse block, slab) pairs, the slab in the low bits
     const uint32_t per_cam = (cg.cw * cg.ch) << sshift;
@@ -561,20 +613,60 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
     const uint32_t n_bounds = (1u << sshift) - 1u;
     int32_t *row = table + (size_t)blockIdx.x * n_blocks + first;
     if (FILL) {
-        // cursor of block b: the blocks before it (of all launches) plus this workgroup's run start
-        const uint32_t all = block_exclusive_scan(
-            first + count, threadIdx.x, blockDim.x, s_scan, [&](uint32_t j) { return (uint32_t)totals[j]; },
-            [&](uint32_t j, uint32_t before, uint32_t) {
-                if (j >= first) s_blocks[j - first] = (int32_t)before + row[j - first];
+        // Cursor of list j: the lists before it (of all launches) plus this workgroup's run start.
+        // The totals pass through LDS and the table rows are read lane by lane (a lane that walked
+        // its own consecutive lists in global memory waited for every load in turn: 25 us on a frame
+        // with 8160 lists).  list_starts: the first workgroup also leaves the lists' starts, and the
+        // end behind them, for the kernels that walk the lists; longest_host: and tells the host the
+        // longest list, a word in pinned memory like the number of intersections.
+        const bool tells = blockIdx.x == 0 && list_starts != nullptr;
+        uint32_t longest = 0, head = 0; // head: the entries of the launches before this one
+        if (threadIdx.x == 0) s_longest = 0;
+        for (uint32_t j = threadIdx.x; j < first; j += blockDim.x) {
+            const uint32_t v = (uint32_t)totals[j];
+            head += v;
+            longest = max(longest, v);
+        }
+        for (uint32_t j = threadIdx.x; j < count; j += blockDim.x) s_blocks[j] = totals[first + j];
+        if (first != 0) { // uniform
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) head += (uint32_t)__shfl_xor((int)head, off, SPLATAD_WAVE);
+            if ((threadIdx.x & (SPLATAD_WAVE - 1)) == 0) s_scan[threadIdx.x / SPLATAD_WAVE] = head;
+            __syncthreads();
+            head = 0;
+            for (uint32_t w = 0; w < blockDim.x / SPLATAD_WAVE; ++w) head += s_scan[w];
+        }
+        __syncthreads();
+        const uint32_t all = head + block_exclusive_scan(
+            count, threadIdx.x, blockDim.x, s_scan, [&](uint32_t j) { return (uint32_t)s_blocks[j]; },
+            [&](uint32_t j, uint32_t before, uint32_t v) {
+                s_blocks[j] = (int32_t)(head + before);
+                longest = max(longest, v);
             });
         // (entries_cap, the caller's number of intersections, bounds the list: it holds whenever the
         // lists were sized for these very rows, and keeps a caller's mismatch inside the lists)
-        if (blockIdx.x == 0 && threadIdx.x == 0 && first + count == n_blocks)
+        for (uint32_t j = threadIdx.x; j < count; j += blockDim.x) {
+            const int32_t start = s_blocks[j];
+            if (tells) list_starts[first + j] = min((uint32_t)start, entries_cap);
+            s_blocks[j] = start + row[j];
+        }
+        const bool last_launch = first + count == n_blocks;
+        if (blockIdx.x == 0 && threadIdx.x == 0 && last_launch) {
             *n_entries = (int64_t)min(all, entries_cap);
+            if (list_starts != nullptr) list_starts[n_blocks] = min(all, entries_cap);
+        }
+        if (blockIdx.x == 0 && last_launch && longest_host != nullptr) { // uniform
+            if (longest) atomicMax(&s_longest, longest);
+            __syncthreads();
+            // a list that would not fit the caller's memory counts as too long for everything
+            if (threadIdx.x == 0)
+                __hip_atomic_store(longest_host, (unsigned long long)(all > entries_cap ? 0xFFFFFFFFu : s_longest),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
     } else {
         for (uint32_t b = threadIdx.x; b < count; b += blockDim.x) s_blocks[b] = 0;
     }
-    if (threadIdx.x < n_bounds) s_bounds[threadIdx.x] = slab_bounds[threadIdx.x];
+    if (threadIdx.x < n_bounds) s_bounds[threadIdx.x] = slab_bound(slab_bounds, threadIdx.x);
     __syncthreads();
     const float *depths_needed = FILL || sshift ? depths : nullptr;
     const uint64_t round = (uint64_t)gridDim.x * blockDim.x;
@@ -609,9 +701,22 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
     }
     if (!FILL) {
         __syncthreads();
-        for (uint32_t b = threadIdx.x; b < count; b += blockDim.x) {
-            const int32_t c = s_blocks[b];
-            row[b] = c ? atomicAdd(&totals[first + b], c) : 0;
+        // (eight lists per lane and step, so that their atomics are in flight together)
+        for (uint32_t b0 = threadIdx.x; b0 < count; b0 += 8 * blockDim.x) {
+            int32_t c[8], start[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t b = b0 + k * blockDim.x;
+                c[k] = b < count ? s_blocks[b] : 0;
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                start[k] = c[k] ? atomicAdd(&totals[first + b0 + k * blockDim.x], c[k]) : 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t b = b0 + k * blockDim.x;
+                if (b < count) row[b] = start[k];
+            }
         }
     }
 }
@@ -722,7 +827,9 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
                       uint64_t *__restrict__ pairs, int64_t n_isects,
                       uint32_t *__restrict__ seg_counts, uint32_t *__restrict__ seg_lists,
                       int32_t *__restrict__ tile_offsets, const int64_t *__restrict__ scan_totals,
-                      uint32_t n_scan_blocks, int32_t *__restrict__ seg_starts) {
+                      uint32_t n_scan_blocks, int32_t *__restrict__ seg_starts, uint32_t kshift) {
+    // kshift: the coarse lists are cut into 1 << (sshift + kshift) depth slabs, the tile
+    // segments into 1 << sshift
     const int64_t n_entries = *n_entries_ptr;
     const uint32_t lane = threadIdx.x & (SPLATAD_WAVE - 1);
     const int64_t wave_id = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / SPLATAD_WAVE;
@@ -814,7 +921,8 @@ isect_tile_bin_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t 
          first_entry += stride) { // uniform across the workgroup
         const int64_t e0 = first_entry + (int64_t)wave * SPLATAD_WAVE;
         const bool has = e0 + lane < n_entries;
-        const uint4 rec = has ? entries[e0 + lane] : make_uint4(0, 0, kNone, 0);
+        uint4 rec = has ? entries[e0 + lane] : make_uint4(0, 0, kNone, 0);
+        if (has) rec.z >>= kshift; // (coarse block, slab of the tile segments)
         const uint64_t pair = ((uint64_t)rec.y << 32) | (uint64_t)rec.x;
         if (FILL) scan.sum(lane); // (the first round: behind the request for the entries)
         const uint64_t have = __ballot(has);
@@ -909,38 +1017,6 @@ isect_emit_kernel(TileGrid g, uint64_t total, uint32_t N, const int64_t *__restr
         isect_ids[w.cum + t] = cid_enc | (tile_id << 32) | depth_enc;
         flatten_ids[w.cum + t] = (int32_t)w.idx;
     });
-}
-
-// All comparators of this bitonic network point the same way (the first stage of every
-// merge is a "flip"), so a virtual +inf tail needs no storage: pairs whose upper index is
-// >= n are skipped.
-template <typename Ptr>
-__device__ __forceinline__ void bitonic_sort_ascending(Ptr a, uint32_t n, uint32_t tid,
-                                                       uint32_t nthreads) {
-    uint32_t m = 1;
-    while (m < n) m <<= 1;
-    for (uint32_t k = 2; k <= m; k <<= 1) {
-        for (uint32_t i = tid; i < m / 2; i += nthreads) {
-            const uint32_t lo = ((i / (k / 2)) * k) + (i % (k / 2));
-            const uint32_t hi = lo ^ (k - 1);
-            if (hi < n) {
-                const uint64_t x = a[lo], y = a[hi];
-                if (y < x) { a[lo] = y; a[hi] = x; }
-            }
-        }
-        __syncthreads();
-        for (uint32_t j = k / 4; j > 0; j >>= 1) {
-            for (uint32_t i = tid; i < m / 2; i += nthreads) {
-                const uint32_t lo = ((i / j) * (2 * j)) + (i % j);
-                const uint32_t hi = lo + j;
-                if (hi < n) {
-                    const uint64_t x = a[lo], y = a[hi];
-                    if (y < x) { a[lo] = y; a[hi] = x; }
-                }
-            }
-            __syncthreads();
-        }
-    }
 }
 
 constexpr uint32_t kSortFineBins = 512;     // first-level depth bins per segment
@@ -1410,6 +1486,526 @@ isect_small_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t 
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Cameras: the coarse lists are sorted, and the tile lists written in order.
+//
+// A Gaussian that covers many tiles is one entry of a coarse block's list and up to sixteen
+// intersections (6.3 on a 1080p driving frame).  Instead of expanding the coarse lists into
+// unordered tile segments and sorting every segment (each such Gaussian sorted sixteen times
+// over), a workgroup sorts a piece of a coarse list by (depth bits, flatten id) in LDS and then
+// walks the sorted piece once per tile of the block: the entries whose mask names the tile, in
+// their sorted order, are the piece's share of the tile's list.  Pieces are runs of consecutive
+// depth slabs of one block (the slab is a non-decreasing function of the depth bits, so the
+// pieces of a block follow each other in the tile lists as they do in depth); where a piece
+// lands in a tile's list follows from the tile's start (the scan of the per-tile counts) plus
+// the entries of the block's earlier slabs that name the tile, counted per list and tile
+// beforehand.  Coarse blocks differ wildly in length -- a block at the horizon of a driving
+// frame holds ten times the average -- which the depth slabs even out: their bounds are
+// quantiles of the visible Gaussians' depths.
+constexpr uint32_t kBlockSortCap = 10240;   // longest (block, slab) list the LDS sort takes
+constexpr uint32_t kBlockMergeCap = 4096;   // slabs of a block are sorted together up to this many entries,
+constexpr uint32_t kBlockPairsCap = 32768;  // and about this many intersections
+constexpr int kBlockClasses = 5;
+__constant__ const uint32_t kBlockClassMax[kBlockClasses] = {512u, 2048u, 4096u, 8192u, kBlockSortCap};
+
+// Dynamic LDS of the block sort: the staging array and its four end markers, the masks and
+// bucket numbers of the staged entries, the fine bins and two bucket tables.
+__host__ __device__ inline size_t block_sort_lds_bytes(uint32_t lds_words, uint32_t bucket_cap) {
+    return ((size_t)lds_words + 4) * 8 + (kSortFineBins + 2 * (size_t)bucket_cap + 1) * 4 +
+           2 * (((size_t)lds_words * 2 + 7) & ~(size_t)7);
+}
+
+// Counts, for every (block, slab) list, the entries that name each of the block's sixteen tiles:
+// counts[list * 16 + t], zero beforehand.  A wavefront takes 64 consecutive entries; those of
+// one list (nearly always all of them) are counted with a ballot per tile and added with one
+// atomic instruction of sixteen lanes.  The lists being short, no counter sees many atomics.
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+isect_list_count_kernel(const int64_t *__restrict__ n_entries_ptr, const uint4 *__restrict__ entries,
+                        int32_t *__restrict__ counts) {
+    const int64_t n_entries = *n_entries_ptr;
+    const uint32_t lane = threadIdx.x & (SPLATAD_WAVE - 1);
+    const int64_t wave_id = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / SPLATAD_WAVE;
+    const int64_t n_waves = (int64_t)gridDim.x * blockDim.x / SPLATAD_WAVE;
+    for (int64_t e0 = wave_id * SPLATAD_WAVE; e0 < n_entries; e0 += n_waves * SPLATAD_WAVE) { // uniform per wavefront
+        const bool has = e0 + lane < n_entries;
+        const uint4 rec = has ? entries[e0 + lane] : make_uint4(0u, 0u, 0xFFFFFFFFu, 0u);
+        uint64_t todo = __ballot(has);
+        while (todo) {
+            const int leader = __ffsll((unsigned long long)todo) - 1;
+            const uint32_t list = (uint32_t)__shfl((int)rec.z, leader, SPLATAD_WAVE);
+            const bool in = has && rec.z == list;
+            todo &= ~__ballot(in);
+            const uint32_t mask = in ? rec.w : 0u;
+            uint32_t cnt = 0;
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const uint32_t n_hits = (uint32_t)__popcll(__ballot((mask >> t) & 1u)); // uniform
+                asm("v_writelane_b32 %0, %1, %2" : "+v"(cnt) : "s"(n_hits), "n"(t));
+            }
+            if (lane < 16 && cnt) atomicAdd(&counts[(size_t)list * 16 + lane], (int32_t)cnt);
+        }
+    }
+}
+
+// A lane per tile: adds up the tile's counts over the slab lists of its block (the tile's number
+// of intersections, which the scan behind this kernel turns into the tile's start) and leaves in
+// their place the counts of the slabs before each (where a slab's entries start inside the
+// tile's list).
+__global__ void __launch_bounds__(SPLATAD_THREADS)
+isect_tile_totals_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t bsshift, uint32_t n_segments,
+                         int32_t *__restrict__ counts, int32_t *__restrict__ tile_counts) {
+    const uint32_t seg = blockIdx.x * blockDim.x + threadIdx.x;
+    if (seg >= n_segments) return;
+    const uint32_t n_tiles = tile_w * tile_h, cam = seg / n_tiles, r = seg - cam * n_tiles;
+    const uint32_t y = r / tile_w, x = r - y * tile_w;
+    const uint32_t block = cam * cg.cw * cg.ch + (y >> kCoarseRowShift) * cg.cw + (x >> 2);
+    const uint32_t t = ((y & 3u) << 2) | (x & 3u);
+    int32_t *mine = counts + ((size_t)block << bsshift) * 16 + t;
+    const uint32_t slabs = 1u << bsshift;
+    int32_t c[1u << kSlabShiftMax];
+#pragma unroll
+    for (uint32_t sl = 0; sl < (1u << kSlabShiftMax); ++sl) c[sl] = sl < slabs ? mine[(size_t)sl * 16] : 0;
+    int32_t run = 0;
+#pragma unroll
+    for (uint32_t sl = 0; sl < (1u << kSlabShiftMax); ++sl) {
+        if (sl < slabs) mine[(size_t)sl * 16] = run;
+        run += c[sl];
+    }
+    tile_counts[seg] = run;
+}
+
+// First workgroup: cuts every block's slab lists into pieces {first entry, entries, block, first
+// list}, a piece being as many consecutive slabs as stay within kBlockMergeCap entries (fewer
+// where the entries meet many tiles each, so that a piece writes about kBlockPairsCap
+// intersections at most; a single slab's list beyond that is a piece of its own), and lists the
+// pieces by size class: class c's are pieces[c * max_pieces ..] , class_count[c] of them.  The
+// other workgroups turn the scanned tile counts into the tiles' starts (seg_starts) and the
+// tile offsets.
+__global__ void __launch_bounds__(1024)
+isect_block_plan_kernel(uint32_t n_blocks, uint32_t bsshift, const int32_t *__restrict__ totals,
+                        const uint32_t *__restrict__ list_starts, const int32_t *__restrict__ tile_counts,
+                        CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t n_segments, uint32_t copies, const int32_t *__restrict__ tile_starts,
+                        const int64_t *__restrict__ scan_totals, uint32_t n_scan_blocks,
+                        int32_t *__restrict__ seg_starts, int32_t *__restrict__ tile_offsets,
+                        uint32_t *__restrict__ class_count, uint32_t max_pieces,
+                        uint4 *__restrict__ pieces) {
+    const uint32_t tid = threadIdx.x, nt = blockDim.x, lane = tid & (SPLATAD_WAVE - 1);
+    if (blockIdx.x != 0) { // uniform across the workgroup
+        ScanBlocks scan;
+        scan.request(scan_totals, n_scan_blocks, lane);
+        scan.sum(lane);
+        const uint32_t per_round = (gridDim.x - 1) * nt;
+        for (uint32_t s0 = (blockIdx.x - 1) * nt + (tid & ~(SPLATAD_WAVE - 1u)); s0 < n_segments; s0 += per_round) {
+            const uint32_t seg = s0 + lane;
+            // the first copy of segment s is logical element s * copies of the scanned table
+            const int32_t before = scan.before(min(seg, n_segments - 1u) * copies);
+            if (seg < n_segments) {
+                const int32_t start = tile_starts[seg] + before;
+                seg_starts[seg] = start;
+                if (tile_offsets != nullptr) tile_offsets[seg] = start;
+            }
+        }
+        return;
+    }
+    __shared__ uint32_t s_count[kBlockClasses];
+    if (tid < kBlockClasses) s_count[tid] = 0;
+    __syncthreads();
+    const uint32_t slabs = 1u << bsshift;
+    for (uint32_t b = tid; b < n_blocks; b += nt) {
+        const uint32_t list0 = b << bsshift;
+        // everything the block needs is requested before any of it is used
+        uint32_t v[1u << kSlabShiftMax];
+#pragma unroll
+        for (uint32_t sl = 0; sl < (1u << kSlabShiftMax); ++sl) v[sl] = sl < slabs ? (uint32_t)totals[list0 + sl] : 0u;
+        const uint32_t block_first = list_starts[list0];
+        // the block's intersections: its tiles' counts (copies == 1 here: one counter per tile)
+        uint32_t in_tiles[16];
+        {
+            const uint32_t per_cam = cg.cw * cg.ch, cam = b / per_cam, r = b - cam * per_cam;
+            const uint32_t by = r / cg.cw, bx = r - by * cg.cw;
+#pragma unroll
+            for (uint32_t t = 0; t < 16; ++t) {
+                const uint32_t x = (bx << 2) + (t & 3u), y = (by << kCoarseRowShift) + (t >> 2);
+                in_tiles[t] = x < tile_w && y < tile_h ? (uint32_t)tile_counts[cam * tile_w * tile_h + y * tile_w + x] : 0u;
+            }
+        }
+        uint64_t pairs = 0;
+#pragma unroll
+        for (uint32_t t = 0; t < 16; ++t) pairs += in_tiles[t];
+        uint32_t block_n = 0;
+#pragma unroll
+        for (uint32_t sl = 0; sl < (1u << kSlabShiftMax); ++sl) block_n += v[sl];
+        if (block_n == 0) continue;
+        uint32_t cap = kBlockMergeCap;
+        if (pairs * cap > (uint64_t)kBlockPairsCap * block_n)
+            cap = max(512u, (uint32_t)((uint64_t)kBlockPairsCap * block_n / pairs));
+        uint32_t piece_first = block_first, piece_n = 0, piece_list = list0;
+        auto emit = [&](uint32_t next_list) {
+            if (piece_n != 0) {
+                int c = 0;
+                while (c + 1 < kBlockClasses && piece_n > kBlockClassMax[c]) ++c;
+                const uint32_t k = atomicAdd(&s_count[c], 1u);
+                pieces[(size_t)c * max_pieces + k] = make_uint4(piece_first, piece_n, b, piece_list);
+                piece_first += piece_n;
+                piece_n = 0;
+            }
+            piece_list = next_list;
+        };
+#pragma unroll
+        for (uint32_t sl = 0; sl < (1u << kSlabShiftMax); ++sl) {
+            if (sl < slabs) {
+                if (piece_n != 0 && piece_n + v[sl] > cap) emit(list0 + sl);
+                if (piece_n == 0) piece_list = list0 + sl;
+                piece_n += v[sl];
+            }
+        }
+        emit(0u);
+    }
+    __syncthreads();
+    if (tid < kBlockClasses) class_count[tid] = s_count[tid];
+}
+
+// Sorts one piece (n <= ER * blockDim.x entries, n <= lds_words) in LDS -- sort_segment_small's
+// method, with the tile masks travelling beside the keys -- and writes its share of the lists
+// of the block's sixteen tiles.
+template <int ER>
+__device__ __forceinline__ void sort_expand_piece(uint4 piece, CoarseGrid cg, uint32_t tile_w, uint32_t tile_h,
+                                                  uint32_t n_tiles, uint32_t tile_n_bits, uint32_t lds_words,
+                                                  uint32_t bucket_cap, int64_t n_isects,
+                                                  const uint4 *__restrict__ entries,
+                                                  const int32_t *__restrict__ seg_starts,
+                                                  const int32_t *__restrict__ slabs_before,
+                                                  int64_t *__restrict__ isect_ids,
+                                                  int32_t *__restrict__ flatten_ids,
+                                                  uint64_t *lds_staged, uint32_t *s_wave, uint32_t &s_big,
+                                                  uint32_t (*s_cnt)[16]) {
+    const uint32_t n = piece.y;
+    uint32_t *s_fine = reinterpret_cast<uint32_t *>(lds_staged + lds_words + 4);
+    uint32_t *s_first = s_fine + kSortFineBins;   // bucket_cap + 1 words: starts, then the end
+    uint32_t *s_cursor = s_first + bucket_cap + 1;
+    uint16_t *s_bucket = reinterpret_cast<uint16_t *>(s_cursor + bucket_cap);
+    uint16_t *s_mask = s_bucket + ((lds_words + 3) & ~3u);
+    const uint4 *g = entries + piece.x;
+    const uint32_t tid = threadIdx.x, nt = blockDim.x;
+    const uint32_t lane = tid & (SPLATAD_WAVE - 1), wave = tid / SPLATAD_WAVE;
+    const uint32_t n_waves = nt / SPLATAD_WAVE;
+
+    uint64_t held[ER];
+    uint32_t held_mask[ER];
+#pragma unroll
+    for (int k = 0; k < ER; ++k) {
+        const uint32_t i = tid + k * nt;
+        const uint4 e = i < n ? g[i] : make_uint4(~0u, ~0u, 0u, 0u);
+        held[k] = ((uint64_t)e.y << 32) | (uint64_t)e.x;
+        held_mask[k] = e.w;
+    }
+    // lane t < 16: the entries of the block's earlier slabs that name tile t
+    const uint32_t pre = lane < 16 ? (uint32_t)slabs_before[(size_t)piece.w * 16 + lane] : 0u;
+    auto count16 = [&](uint32_t mask) -> uint32_t {
+        uint32_t cnt = 0;
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            const uint32_t n_hits = (uint32_t)__popcll(__ballot((mask >> t) & 1u)); // uniform
+            asm("v_writelane_b32 %0, %1, %2" : "+v"(cnt) : "s"(n_hits), "n"(t));
+        }
+        return cnt;
+    };
+    uint32_t lo = 0xFFFFFFFFu, hi = 0u, id_lo = 0xFFFFFFFFu, id_hi = 0u;
+#pragma unroll
+    for (int k = 0; k < ER; ++k)
+        if (tid + k * nt < n) {
+            const uint32_t d = (uint32_t)(held[k] >> 32), id = (uint32_t)held[k];
+            lo = min(lo, d);
+            hi = max(hi, d);
+            id_lo = min(id_lo, id);
+            id_hi = max(id_hi, id);
+        }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        lo = min(lo, (uint32_t)__shfl_xor((int)lo, off, SPLATAD_WAVE));
+        hi = max(hi, (uint32_t)__shfl_xor((int)hi, off, SPLATAD_WAVE));
+        id_lo = min(id_lo, (uint32_t)__shfl_xor((int)id_lo, off, SPLATAD_WAVE));
+        id_hi = max(id_hi, (uint32_t)__shfl_xor((int)id_hi, off, SPLATAD_WAVE));
+    }
+    if (lane == 0) {
+        s_wave[4 * wave] = lo; s_wave[4 * wave + 1] = hi;
+        s_wave[4 * wave + 2] = id_lo; s_wave[4 * wave + 3] = id_hi;
+    }
+    if (tid == 0) s_big = 0;
+    if (tid < 4) lds_staged[n + tid] = ~0ull;
+
+    // Places of the staged entries: an entry's bucket is first[b] .. first[b + 1], its place the
+    // bucket's start plus the bucket's smaller keys.  The keys (depth bits, flatten id) of a
+    // coarse list are distinct.  Kept in registers (with the mask above the place), for the
+    // staging array is where the sorted piece goes.
+    uint64_t placed[ER];
+    uint32_t place_mask[ER];
+    auto rank_all = [&](const uint32_t *first) {
+#pragma unroll
+        for (int k = 0; k < ER; ++k) {
+            const uint32_t i = tid + k * nt;
+            placed[k] = 0;
+            place_mask[k] = 0;
+            if (i < n) {
+                const uint64_t p = lds_staged[i];
+                const uint32_t b = s_bucket[i];
+                const uint32_t s0 = first[b], s1 = first[b + 1];
+                uint32_t place = s0;
+                for (uint32_t j = s0; j < s1; j += 4) {
+                    const uint64_t q0 = lds_staged[j], q1 = lds_staged[j + 1];
+                    const uint64_t q2 = lds_staged[j + 2], q3 = lds_staged[j + 3];
+                    place += (q0 < p ? 1u : 0u) + (q1 < p ? 1u : 0u) + (q2 < p ? 1u : 0u) + (q3 < p ? 1u : 0u);
+                }
+                placed[k] = p;
+                place_mask[k] = place | ((uint32_t)s_mask[i] << 16);
+            }
+        }
+    };
+
+    uint32_t n_bins = 1;
+    while (n_bins < kSortDirectBins && n_bins * kSortDirectMean < n) n_bins <<= 1;
+    for (uint32_t f = tid; f < n_bins; f += nt) s_fine[f] = 0;
+    __syncthreads();
+    for (uint32_t w = 0; w < n_waves; ++w) {
+        lo = min(lo, s_wave[4 * w]);
+        hi = max(hi, s_wave[4 * w + 1]);
+        id_lo = min(id_lo, s_wave[4 * w + 2]);
+        id_hi = max(id_hi, s_wave[4 * w + 3]);
+    }
+    __syncthreads(); // s_wave is reused by the scans
+    bool ranked = false;
+    if (hi < 0x7F800000u) { // uniform; depths that are positive finite floats
+        // Direct path, as in sort_segment_small: bins linear in the depth, and the atomic that
+        // counts an entry into its bin tells its place inside the bin.  A piece whose depths are
+        // all equal (a wall that faces the camera) is ordered by the flatten ids alone: bins
+        // linear in the id.
+        const bool by_id = hi == lo;
+        const float lo_depth = __uint_as_float(lo), range = __uint_as_float(hi) - lo_depth;
+        const float bin_scale = by_id ? (float)n_bins / ((float)(id_hi - id_lo) + 1.f)
+                                      : (float)n_bins / range;
+        uint32_t where[ER]; // bin, and above it the place inside the bin
+#pragma unroll
+        for (int k = 0; k < ER; ++k) {
+            where[k] = 0;
+            if (tid + k * nt < n) {
+                const float x = by_id ? (float)((uint32_t)held[k] - id_lo) * bin_scale
+                                      : (__uint_as_float((uint32_t)(held[k] >> 32)) - lo_depth) * bin_scale;
+                const uint32_t f = min(n_bins - 1, (uint32_t)x);
+                where[k] = f | (atomicAdd(&s_fine[f], 1u) << 16);
+            }
+        }
+        __syncthreads();
+        block_exclusive_scan(
+            n_bins, tid, nt, s_wave, [&](uint32_t f) { return s_fine[f]; },
+            [&](uint32_t f, uint32_t before, uint32_t v) {
+                s_fine[f] = before;
+                if (v > kSortDirectMax) s_big = 2;
+            });
+        if (s_big != 2) { // uniform
+            if (tid == 0) s_fine[n_bins] = n;
+#pragma unroll
+            for (int k = 0; k < ER; ++k)
+                if (tid + k * nt < n) {
+                    const uint32_t f = where[k] & 0xFFFFu;
+                    const uint32_t at = s_fine[f] + (where[k] >> 16);
+                    lds_staged[at] = held[k];
+                    s_bucket[at] = (uint16_t)f;
+                    s_mask[at] = (uint16_t)held_mask[k];
+                }
+            __syncthreads();
+            rank_all(s_fine);
+            ranked = true;
+        } else {
+            __syncthreads(); // every lane has read the flag
+            if (tid == 0) s_big = 0;
+        }
+    }
+    if (!ranked) { // uniform: buckets equalised over the depth bits, as in sort_segment_small
+        uint32_t n_fine = 1;
+        while (n_fine < kSortFineBins && n_fine * 16 < n) n_fine <<= 1;
+        for (uint32_t f = tid; f < n_fine; f += nt) s_fine[f] = 0;
+        const float scale = (float)n_fine / ((float)(hi - lo) + 1.f);
+        auto fine_pos = [&](uint64_t p, uint32_t &f) -> float {
+            const float x = (float)((uint32_t)(p >> 32) - lo) * scale;
+            f = min(n_fine - 1, (uint32_t)x);
+            return x;
+        };
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < ER; ++k)
+            if (tid + k * nt < n) {
+                uint32_t f;
+                fine_pos(held[k], f);
+                atomicAdd(&s_fine[f], 1u);
+            }
+        __syncthreads();
+        const uint32_t mean = kSortBucketMean;
+        const uint32_t nb = block_exclusive_scan(
+            n_fine, tid, nt, s_wave,
+            [&](uint32_t f) { return (s_fine[f] + mean - 1) / mean; },
+            [&](uint32_t f, uint32_t before, uint32_t v) { s_fine[f] = before | (v << 16); });
+        for (uint32_t b = tid; b < nb; b += nt) s_cursor[b] = 0;
+        __syncthreads();
+        uint32_t bucket[ER];
+#pragma unroll
+        for (int k = 0; k < ER; ++k) {
+            bucket[k] = 0;
+            if (tid + k * nt < n) {
+                uint32_t f;
+                const float x = fine_pos(held[k], f);
+                const uint32_t packed = s_fine[f];
+                const uint32_t c = packed >> 16;
+                bucket[k] = (packed & 0xFFFFu) + min(c - 1, (uint32_t)((x - (float)f) * (float)c));
+                atomicAdd(&s_cursor[bucket[k]], 1u);
+            }
+        }
+        __syncthreads();
+        block_exclusive_scan(
+            nb, tid, nt, s_wave, [&](uint32_t b) { return s_cursor[b]; },
+            [&](uint32_t b, uint32_t before, uint32_t) {
+                s_cursor[b] = before;
+                s_first[b] = before;
+            });
+        if (tid == 0) s_first[nb] = n;
+#pragma unroll
+        for (int k = 0; k < ER; ++k)
+            if (tid + k * nt < n) {
+                const uint32_t at = atomicAdd(&s_cursor[bucket[k]], 1u);
+                lds_staged[at] = held[k];
+                s_bucket[at] = (uint16_t)bucket[k];
+                s_mask[at] = (uint16_t)held_mask[k];
+            }
+        __syncthreads();
+        // (a bucket of many equal depths is ranked like any other: every entry counts the
+        // bucket's smaller keys)
+        rank_all(s_first);
+    }
+    __syncthreads(); // every place is known: the staging array takes the sorted piece
+#pragma unroll
+    for (int k = 0; k < ER; ++k)
+        if (tid + k * nt < n) {
+            const uint32_t place = place_mask[k] & 0xFFFFu;
+            lds_staged[place] = placed[k];
+            s_mask[place] = (uint16_t)(place_mask[k] >> 16);
+        }
+    __syncthreads();
+
+    // The sorted piece, tile by tile.  A wavefront takes consecutive chunks of 64 entries; it
+    // counts its chunks' entries per tile, learns from the other wavefronts' counts where its
+    // first chunk starts in every tile's list, and writes.
+    const uint32_t n_chunks = (n + SPLATAD_WAVE - 1) / SPLATAD_WAVE, per_wave = (n_chunks + n_waves - 1) / n_waves;
+    const uint32_t c0 = min(n_chunks, wave * per_wave), c1 = min(n_chunks, c0 + per_wave);
+    uint32_t mine = 0;
+    for (uint32_t c = c0; c < c1; ++c) { // uniform per wavefront
+        const uint32_t i = c * SPLATAD_WAVE + lane;
+        mine += count16(i < n ? (uint32_t)s_mask[i] : 0u);
+    }
+    if (lane < 16) s_cnt[wave][lane] = mine;
+    __syncthreads();
+    uint32_t base = 0, tile_key = 0;
+    if (lane < 16) {
+        const uint32_t per_cam = cg.cw * cg.ch;
+        const uint32_t cam = piece.z / per_cam, r = piece.z - cam * per_cam;
+        const uint32_t by = r / cg.cw, bx = r - by * cg.cw;
+        const uint32_t x = (bx << 2) + (lane & 3u), y = (by << kCoarseRowShift) + (lane >> 2);
+        if (x < tile_w && y < tile_h) { // (a tile beyond the grid's edge is in no mask)
+            const uint32_t tile = y * tile_w + x;
+            base = (uint32_t)seg_starts[cam * n_tiles + tile];
+            tile_key = (cam << tile_n_bits) | tile;
+        }
+        base += pre;
+        for (uint32_t w = 0; w < wave; ++w) base += s_cnt[w][lane];
+    }
+    // Where the wavefront's next entry of every tile goes, and the tiles' keys, are the same for all
+    // lanes: kept in scalar registers from here on.
+    uint32_t next_of[16], key_of[16];
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+        next_of[t] = (uint32_t)__builtin_amdgcn_readlane((int)base, t);
+        key_of[t] = (uint32_t)__builtin_amdgcn_readlane((int)tile_key, t);
+    }
+    const uint32_t cap = (uint32_t)n_isects; // below 2^31; keeps a caller's mismatch inside the lists
+    for (uint32_t c = c0; c < c1; ++c) { // uniform per wavefront
+        const uint32_t i = c * SPLATAD_WAVE + lane;
+        const uint64_t p = i < n ? lds_staged[i] : 0ull;
+        const uint32_t mask = i < n ? (uint32_t)s_mask[i] : 0u;
+        const uint32_t depth = (uint32_t)(p >> 32);
+        const uint32_t depth_sign = (uint32_t)((int32_t)depth >> 31);
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            const bool named = (mask >> t) & 1u;
+            const uint64_t hits = wave_ballot(named);
+            if (hits == 0) continue; // uniform
+            const uint32_t first = next_of[t];
+            next_of[t] = first + (uint32_t)__popcll(hits);
+            if (next_of[t] > cap) continue; // uniform: the caller's lists end before this run does
+            if (wave_lanes(hits)) { // (the lanes that name the tile, from the mask at hand)
+                const uint32_t at = __builtin_amdgcn_mbcnt_hi((uint32_t)(hits >> 32),
+                                                              __builtin_amdgcn_mbcnt_lo((uint32_t)hits, first));
+                // the key as the reference forms it: the depth bits sign-extended below the tile
+                isect_ids[at] = (int64_t)(((uint64_t)(key_of[t] | depth_sign) << 32) | (uint64_t)depth);
+                flatten_ids[at] = (int32_t)(uint32_t)p;
+            }
+        }
+    }
+}
+
+template <int ER>
+__global__ void isect_block_sort_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t n_tiles,
+                                        uint32_t tile_n_bits, uint32_t lds_words, uint32_t bucket_cap,
+                                        int64_t n_isects, const uint32_t *__restrict__ class_count,
+                                        const uint4 *__restrict__ pieces, const uint4 *__restrict__ entries,
+                                        const int32_t *__restrict__ seg_starts,
+                                        const int32_t *__restrict__ slabs_before,
+                                        int64_t *__restrict__ isect_ids, int32_t *__restrict__ flatten_ids) {
+    extern __shared__ uint64_t lds_staged[];
+    __shared__ uint32_t s_wave[4 * (1024 / SPLATAD_WAVE)];
+    __shared__ uint32_t s_big;
+    __shared__ uint32_t s_cnt[1024 / SPLATAD_WAVE][16];
+    const uint32_t count = *class_count;
+    for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) { // uniform across the workgroup
+        sort_expand_piece<ER>(pieces[k], cg, tile_w, tile_h, n_tiles, tile_n_bits, lds_words, bucket_cap, n_isects,
+                              entries, seg_starts, slabs_before, isect_ids, flatten_ids, lds_staged, s_wave,
+                              s_big, s_cnt);
+        __syncthreads(); // the next piece reuses the LDS
+    }
+}
+
+template <int ER>
+static int launch_block_sort(int cls, uint32_t threads, uint32_t max_n, uint32_t workgroups, uint32_t max_pieces,
+                             CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t n_tiles,
+                             uint32_t tile_n_bits, int64_t n_isects, const uint32_t *class_count,
+                             const uint4 *pieces, const uint4 *entries, const int32_t *seg_starts,
+                             const int32_t *slabs_before, int64_t *isect_ids, int32_t *flatten_ids,
+                             hipStream_t stream) {
+    SPLATAD_REQUIRE((uint64_t)ER * threads >= max_n && max_n <= kBlockSortCap && max_n % 512u == 0,
+                    "block sort: class %d does not fit", cls);
+    const uint32_t bucket_cap = sort_bucket_capacity(max_n);
+    {   // the bins of the direct path: a power of two, at most max_n / kSortDirectMean of them
+        uint32_t bins = 1;
+        while (bins < kSortDirectBins && bins * kSortDirectMean < max_n) bins <<= 1;
+        SPLATAD_REQUIRE(bins + 1 <= kSortFineBins + 2 * bucket_cap + 1 && bins <= 65536u,
+                        "block sort: no room for the %u bins of class %d", bins, cls);
+    }
+    const size_t lds_bytes = block_sort_lds_bytes(max_n, bucket_cap);
+    {   // raise the kernel's dynamic LDS limit once per instantiation and size
+        static std::mutex guard;
+        static size_t allowed = 0;
+        std::lock_guard<std::mutex> lock(guard);
+        if (lds_bytes > allowed) {
+            SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)isect_block_sort_kernel<ER>,
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+            allowed = lds_bytes;
+        }
+    }
+    hipLaunchKernelGGL((isect_block_sort_kernel<ER>), dim3(workgroups < max_pieces ? workgroups : max_pieces),
+                       dim3(threads), lds_bytes, stream, cg, tile_w, tile_h, n_tiles, tile_n_bits, max_n,
+                       bucket_cap, n_isects, class_count + cls, pieces + (size_t)cls * max_pieces, entries,
+                       seg_starts, slabs_before, isect_ids, flatten_ids);
+    SPLATAD_LAUNCH_CHECK();
+    return 0;
+}
+
 // The two upper classes (more than 12288 entries) in one launch, longest segments first.  Their
 // workgroups need most of a compute unit's LDS, so even a launch that finds its class empty waits for such a unit to
 // fall free once other sort kernels are running; one launch, enqueued before those, meets an
@@ -1552,6 +2148,10 @@ struct IsectWorkspace {
     int32_t *seg_starts;          // [segments] first entry of every segment, for the sort
     uint32_t *seg_counts;         // [kSortClasses] segments per size class (in the cleared part)
     uint32_t *seg_lists;          // [kSortClasses * segments]
+    int32_t *list_tile_counts;    // [lists * 16] entries per list and tile of the block (in the cleared part)
+    uint32_t *list_starts;        // [lists + 1] first entry of every (block, slab) list, and the end
+    uint32_t *piece_counts;       // [kBlockClasses] pieces per size class
+    uint4 *pieces;                // [kBlockClasses * lists] the pieces the block sort takes, by class
     int64_t *block_sums;          // scan scratch
     // the lists, whose size depends on the number of intersections
     int64_t *cum_before;          // [total] (sort == false)
@@ -1580,9 +2180,14 @@ static uint32_t isect_copies(uint64_t blocks) {
 
 // Workgroups of the coarse binning (= rows of its counter table): enough to fill the GPU,
 // fewer when many blocks would make the table long.
-static uint32_t coarse_workgroups(uint64_t total, uint64_t blocks) {
-    uint64_t wgs = (1ull << 19) / (blocks ? blocks : 1);
-    if (wgs > 512) wgs = 512;
+constexpr uint64_t kCoarseTable = 1ull << 19;          // entries of the [workgroup][block] table aimed at
+constexpr uint64_t kCoarseTableBlockSort = 1ull << 22; // with the block sort's depth slabs
+static uint32_t coarse_workgroups(uint64_t total, uint64_t blocks, uint64_t table) {
+    uint64_t wgs = table / (blocks ? blocks : 1);
+    // (with the block sort's lists a workgroup flushes thousands of counters with an atomic each:
+    // measured on a 1080p frame of 1M Gaussians, the intersection takes 0.228 / 0.219 / 0.240 ms
+    // with 512 / 256 / 128 workgroups)
+    if (wgs > (table == kCoarseTableBlockSort ? 256u : 512u)) wgs = table == kCoarseTableBlockSort ? 256 : 512;
     if (wgs < 64) wgs = 64;
     const uint64_t needed = (total + kCoarseThreads - 1) / kCoarseThreads;
     if (wgs > needed) wgs = needed ? needed : 1;
@@ -1594,9 +2199,23 @@ static uint32_t coarse_workgroups(uint64_t total, uint64_t blocks) {
 // slab) pairs.
 struct IsectPlan {
     uint32_t n_tiles, tile_n_bits, sshift, per_cam, coarse_wgs, cams_per_launch;
+    uint32_t bsshift;   // depth slabs of the coarse lists: sshift, or the block sort's own
+    bool block_sort;    // cameras: the coarse lists are sorted and the tile lists written in order
     uint64_t segs, blocks, cslots;
     CoarseGrid cg;
 };
+
+// Depth slabs of the coarse lists for the block sort: enough that a list holds about a hundred
+// Gaussians on average (the longest list of a driving frame, at its horizon, is some ten times
+// the average and has to fit the LDS sort: kBlockSortCap), but no more than lets the coarse
+// binning keep all sensors' counters in LDS at once, down to two slabs.
+static uint32_t block_slab_shift(uint64_t total, uint32_t C, uint64_t blocks_per_cam) {
+    const uint64_t per_block = total / ((uint64_t)C * blocks_per_cam);
+    uint32_t s = 0;
+    while (s < kSlabShiftMax && (per_block >> s) > 128) ++s;
+    while (s > 1 && (((uint64_t)C * blocks_per_cam) << s) > kCoarseLdsBlocks) --s;
+    return s;
+}
 
 template <bool LIDAR>
 static IsectPlan isect_plan(const TileGrid &g, uint64_t total, uint32_t C, int sort) {
@@ -1604,13 +2223,16 @@ static IsectPlan isect_plan(const TileGrid &g, uint64_t total, uint32_t C, int s
     pl.n_tiles = g.tile_w * g.tile_h;
     pl.tile_n_bits = splatad_bit_width(pl.n_tiles);
     pl.cg = coarse_grid<LIDAR>(g);
-    pl.sshift = sort ? slab_shift_for(total, (uint64_t)C * pl.n_tiles) : 0;
+    pl.block_sort = sort && !LIDAR;
+    pl.sshift = sort && !pl.block_sort ? slab_shift_for(total, (uint64_t)C * pl.n_tiles) : 0;
+    pl.bsshift = pl.block_sort ? block_slab_shift(total, C, (uint64_t)pl.cg.cw * pl.cg.ch) : pl.sshift;
     // one sensor's block counters have to fit the LDS of the coarse binning
-    while (pl.sshift > 0 && ((uint64_t)pl.cg.cw * pl.cg.ch << pl.sshift) > kCoarseLdsBlocks) --pl.sshift;
+    while (pl.bsshift > 0 && ((uint64_t)pl.cg.cw * pl.cg.ch << pl.bsshift) > kCoarseLdsBlocks) --pl.bsshift;
+    if (!pl.block_sort) pl.sshift = pl.bsshift;
     pl.segs = ((uint64_t)C * pl.n_tiles) << pl.sshift;
-    pl.per_cam = (pl.cg.cw * pl.cg.ch) << pl.sshift;
+    pl.per_cam = (pl.cg.cw * pl.cg.ch) << pl.bsshift;
     pl.blocks = (uint64_t)C * pl.per_cam;
-    pl.coarse_wgs = coarse_workgroups(total, pl.blocks);
+    pl.coarse_wgs = coarse_workgroups(total, pl.blocks, pl.block_sort ? kCoarseTableBlockSort : kCoarseTable);
     pl.cslots = pl.blocks * pl.coarse_wgs;
     pl.cams_per_launch = pl.per_cam ? kCoarseLdsBlocks / pl.per_cam : 0;
     return pl;
@@ -1618,8 +2240,9 @@ static IsectPlan isect_plan(const TileGrid &g, uint64_t total, uint32_t C, int s
 
 // Layout of the workspace from sizes only; cslots is the length of the coarse counter table,
 // or an upper bound of it when only the number of tiles is known (workspace sizing).
-static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslots,
-                          IsectWorkspace *out) {
+static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t lists, bool block_sort,
+                          uint64_t cslots, IsectWorkspace *out) {
+    const uint64_t block_sort_lists = block_sort ? lists : 0; // what only the block sort uses
     const uint64_t tslots = segs * isect_copies(segs);
     const uint64_t scan_n = total > tslots ? total : tslots;
     char *p = (char *)ws;
@@ -1630,13 +2253,17 @@ static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t cslo
     w.zeroed = (int32_t *)p;
     w.tile_counts = (int32_t *)p;           p += splatad_align256(tslots * 4);
     w.tile_fill = (int32_t *)p;             p += splatad_align256(tslots * 4);
-    w.block_totals = (int32_t *)p;          p += splatad_align256(segs * 4); // blocks <= segments
+    w.block_totals = (int32_t *)p;          p += splatad_align256(lists * 4);
+    w.list_tile_counts = (int32_t *)p;      p += splatad_align256(block_sort_lists * 64);
     w.seg_counts = (uint32_t *)p;           p += 256;
     w.n_zeroed = (uint64_t)(p - (char *)w.zeroed) / 4;
     w.coarse_counts = (int32_t *)p;         p += splatad_align256(cslots * 4);
     w.tile_starts = (int32_t *)p;           p += splatad_align256(tslots * 4);
     w.seg_lists = (uint32_t *)p;            p += splatad_align256(segs * kSortClasses * 4);
     w.seg_starts = (int32_t *)p;            p += splatad_align256(segs * 4);
+    w.list_starts = (uint32_t *)p;          p += splatad_align256((lists + 1) * 4);
+    w.piece_counts = (uint32_t *)p;         p += 256;
+    w.pieces = (uint4 *)p;                  p += splatad_align256(block_sort_lists * kBlockClasses * 16);
     w.block_sums = (int64_t *)p;            p += scan_workspace_bytes((int64_t)scan_n);
     if (out) *out = w;
     return (size_t)(p - (char *)ws);
@@ -1653,12 +2280,20 @@ static size_t carve_lists(void *lists, uint64_t total, int64_t n_isects, IsectWo
     return (size_t)(p - (char *)lists);
 }
 
-static size_t isect_ws_bytes(uint64_t total, uint64_t segs) {
-    // there are at most as many coarse blocks as tiles, and coarse_workgroups() keeps the
-    // table at 2^19 entries unless 64 rows exceed that
-    segs <<= slab_shift_for(total, segs); // the most slabs a plan for these sizes uses
-    const uint64_t cslots_bound = segs * 64 > (1ull << 19) ? segs * 64 : (1ull << 19);
-    return carve_isect(nullptr, total, segs, cslots_bound, nullptr);
+static size_t isect_ws_bytes(uint64_t total, uint32_t C, uint64_t n_tiles) {
+    uint64_t segs = (uint64_t)C * n_tiles;
+    // Bounds for both kinds of plan; coarse_workgroups() keeps the table at its aimed-at size
+    // unless 64 rows exceed that.
+    // The segment sort's plan: the most slabs a plan for these sizes uses, as many lists as segments
+    // at most.  The block sort's: tiles as segments, and a sensor's ceil(w / 4) * ceil(h / 4) blocks
+    // (at most a quarter of its w * h tiles, plus one) times 1 << kSlabShiftMax lists
+    const uint64_t slabbed = segs << slab_shift_for(total, segs);
+    const uint64_t lists = (uint64_t)C * (n_tiles / 4 + 1) << kSlabShiftMax;
+    const uint64_t a = carve_isect(nullptr, total, slabbed, slabbed, false,
+                                   slabbed * 64 > kCoarseTable ? slabbed * 64 : kCoarseTable, nullptr);
+    const uint64_t b = carve_isect(nullptr, total, segs, lists, true,
+                                   lists * 64 > kCoarseTableBlockSort ? lists * 64 : kCoarseTableBlockSort, nullptr);
+    return a > b ? a : b;
 }
 
 static inline dim3 grid_for(uint64_t n) {
@@ -1720,10 +2355,11 @@ static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const Is
         const uint32_t c1 = C - c0 < pl.cams_per_launch ? C : c0 + pl.cams_per_launch;
         hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, false>), dim3(pl.coarse_wgs),
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, pl.cg,
-                           total, N, camera_ids, means2d, radii, pl.sshift ? depths : nullptr, c0, c1,
-                           (uint32_t)pl.blocks, w.coarse_counts, (uint4 *)nullptr, pl.sshift,
+                           total, N, camera_ids, means2d, radii, pl.bsshift ? depths : nullptr, c0, c1,
+                           (uint32_t)pl.blocks, w.coarse_counts, (uint4 *)nullptr, pl.bsshift,
                            (const uint32_t *)w.slab_bounds, (const int32_t *)nullptr, (int32_t *)nullptr,
-                           w.block_totals, (int64_t *)nullptr, 0u);
+                           w.block_totals, (int64_t *)nullptr, 0u, (uint32_t *)nullptr,
+                           (unsigned long long *)nullptr);
     }
     SPLATAD_LAUNCH_CHECK();
     return 0;
@@ -1773,7 +2409,7 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     SPLATAD_REQUIRE(pl.tile_n_bits + splatad_bit_width(C) <= 32,
                     "isect: camera and tile ids need more than 32 bits");
     IsectWorkspace w;
-    carve_isect(workspace, total, pl.segs, sort ? pl.cslots : 0, &w);
+    carve_isect(workspace, total, pl.segs, pl.blocks, pl.block_sort, sort ? pl.cslots : 0, &w);
     // the number of intersections reaches the host through a leased pinned word
     HostWordLease lease(stream);
     unsigned long long *counters = nullptr;
@@ -1786,17 +2422,20 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     // the binning behind it
     // (a caller that knows the count and sorts without depth slabs needs nothing of the counting
     // kernel but the cleared counters)
-    const bool skip_count = known && sort && pl.sshift == 0;
+    const bool skip_count = known && sort && pl.bsshift == 0;
     if (!skip_count) {
         dim3 count_grid = grid_for(total);
         if (count_grid.x > 1024) count_grid.x = 1024;
-        const bool slabs = sort && pl.sshift != 0; // one more workgroup finds the slabs' bounds
-        if (slabs) count_grid.x += 1;
+        const bool slabs = sort && pl.bsshift != 0; // one more workgroup finds the slabs' bounds
+        if (slabs) count_grid.x += kSlabEstimates;
         hipLaunchKernelGGL((slabs ? isect_count_kernel<LIDAR, true> : isect_count_kernel<LIDAR, false>),
                            count_grid, dim3(SPLATAD_THREADS), 0, stream, g,
                            total, means2d, radii, tiles_per_gauss, counters, lease.word.device,
-                           w.zeroed, sort ? w.n_zeroed : (uint64_t)0, depths, 1u << pl.sshift,
-                           slabs ? w.slab_bounds : (uint32_t *)nullptr);
+                           w.zeroed, sort ? w.n_zeroed : (uint64_t)0, depths, 1u << pl.bsshift,
+                           slabs ? w.slab_bounds : (uint32_t *)nullptr,
+                           // the block sort's slabs even out the coarse lists, an entry per Gaussian
+                           // and block; the segment sort's the tile segments
+                           pl.block_sort ? 1 : 0);
         SPLATAD_LAUNCH_CHECK();
     } else {
         hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(w.n_zeroed), dim3(SPLATAD_THREADS), 0, stream,
@@ -1850,7 +2489,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     const uint64_t segs = pl.segs;
     const CoarseGrid cg = pl.cg;
     IsectWorkspace w;
-    carve_isect(workspace, total, segs, sort ? pl.cslots : 0, &w);
+    carve_isect(workspace, total, segs, pl.blocks, pl.block_sort, sort ? pl.cslots : 0, &w);
     carve_lists(lists, total, n_isects, &w);
     int rc;
     if (!sort) {
@@ -1864,29 +2503,49 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         SPLATAD_LAUNCH_CHECK();
         return 0;
     }
+    // The block sort takes coarse lists of up to kBlockSortCap entries.  Whether all lists are that
+    // short the host learns from the filling kernel, through a pinned word as it learnt the
+    // number of intersections (the wait below ends as soon as that kernel has begun: the GPU has
+    // the tile binning to do meanwhile); a scene with a longer list takes the segment sort.
+    HostWordLease longest(stream);
+    if (pl.block_sort) {
+        if ((rc = host_word_refuse_capture(stream, "isect")) != 0) return rc;
+        if ((rc = host_word_acquire(&longest.word)) != 0) return rc;
+    }
     // the coarse lists were counted by the counting call; fill them
     for (uint32_t c0 = 0; c0 < C; c0 += pl.cams_per_launch) {
         const uint32_t c1 = C - c0 < pl.cams_per_launch ? C : c0 + pl.cams_per_launch;
         hipLaunchKernelGGL((isect_coarse_kernel<LIDAR, true>), dim3(pl.coarse_wgs),
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, cg,
                            total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)pl.blocks,
-                           w.coarse_counts, w.entries, sshift, (const uint32_t *)w.slab_bounds, remap,
-                           tiles_out, w.block_totals, w.n_entries, (uint32_t)n_isects);
+                           w.coarse_counts, w.entries, pl.bsshift, (const uint32_t *)w.slab_bounds, remap,
+                           tiles_out, w.block_totals, w.n_entries, (uint32_t)n_isects,
+                           pl.block_sort ? w.list_starts : (uint32_t *)nullptr,
+                           pl.block_sort ? longest.word.device : (unsigned long long *)nullptr);
     }
     SPLATAD_LAUNCH_CHECK();
     // tile segments: count, scan, fill.  The number of coarse entries stays on the device;
     // the grid is sized for the bound n_isects and strides.
-    const uint32_t tcopies = isect_copies(segs);
+    const uint32_t tcopies = pl.block_sort ? 1u : isect_copies(segs);
     uint64_t bin_wgs = ((uint64_t)n_isects + SPLATAD_THREADS - 1) / SPLATAD_THREADS;
     if (bin_wgs > 8192) bin_wgs = 8192;
     const bool square = cg.bshift == 2; // 4 x 4 tiles per block: the unrolled kernels
+    if (pl.block_sort) {
+        // counts per list and tile, from which both the tiles' counts and the places of the
+        // lists inside the tiles' segments follow
+        hipLaunchKernelGGL(isect_list_count_kernel, dim3((uint32_t)bin_wgs), dim3(SPLATAD_THREADS), 0, stream,
+                           (const int64_t *)w.n_entries, (const uint4 *)w.entries, w.list_tile_counts);
+        hipLaunchKernelGGL(isect_tile_totals_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream, cg,
+                           g.tile_w, g.tile_h, pl.bsshift, (uint32_t)segs, w.list_tile_counts, w.tile_counts);
+    } else
     hipLaunchKernelGGL((square ? isect_tile_bin_kernel<false, 16> : isect_tile_bin_kernel<false, 0>),
                        dim3((uint32_t)bin_wgs),
                        dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, sshift, tcopies,
                        (uint32_t)segs, (const int64_t *)w.n_entries, (const uint4 *)w.entries,
                        w.tile_counts, (const int32_t *)nullptr, (int32_t *)nullptr,
                        (uint64_t *)nullptr, (int64_t)0, (uint32_t *)nullptr, (uint32_t *)nullptr,
-                       (int32_t *)nullptr, (const int64_t *)nullptr, 0u, (int32_t *)nullptr);
+                       (int32_t *)nullptr, (const int64_t *)nullptr, 0u, (int32_t *)nullptr,
+                       pl.bsshift - sshift);
     SPLATAD_LAUNCH_CHECK();
     // up to 128 scan blocks, i.e. any table of the size isect_copies() aims at: one scan launch,
     // and the filling pass adds the blocks before an element itself
@@ -1901,6 +2560,59 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         rc = launch_exclusive_scan<int32_t>(w.tile_counts, scan_n, scan_stride, 0, w.tile_starts,
                                             w.scan_total, w.block_sums, stream);
     if (rc) return rc;
+    IsectDevice *ss = nullptr;
+    if ((rc = isect_device(&ss)) != 0) return rc;
+    const uint32_t nseg = (uint32_t)segs;
+    bool short_lists = false;
+    if (pl.block_sort) {
+        unsigned long long longest_list = 0;
+        if ((rc = host_word_wait(&longest, "isect", &longest_list)) != 0) return rc;
+        short_lists = longest_list <= kBlockSortCap;
+    }
+    if (short_lists) {
+        // Pieces of the coarse lists by size class, and the tiles' starts; then a launch per
+        // class, the long pieces first, beside each other on the caller's stream and two helper
+        // streams like the classes of the segment sort below.
+        const uint32_t n_blocks = C * cg.cw * cg.ch;
+        uint32_t plan_wgs = 1 + (nseg + 1023) / 1024;
+        if (plan_wgs > 65) plan_wgs = 65;
+        hipLaunchKernelGGL(isect_block_plan_kernel, dim3(plan_wgs), dim3(1024), 0, stream, n_blocks, pl.bsshift,
+                           (const int32_t *)w.block_totals, (const uint32_t *)w.list_starts,
+                           (const int32_t *)w.tile_counts, cg, g.tile_w, g.tile_h, nseg, tcopies,
+                           (const int32_t *)w.tile_starts,
+                           local_scan ? (const int64_t *)w.block_sums : (const int64_t *)nullptr, n_scan_blocks,
+                           w.seg_starts, tile_offsets, w.piece_counts, (uint32_t)pl.blocks, w.pieces);
+        SPLATAD_LAUNCH_CHECK();
+        std::lock_guard<std::mutex> fork_lock(ss->guard);
+        SPLATAD_CHECK_HIP(hipEventRecord(ss->fork, stream));
+        for (hipStream_t aux : ss->aux) SPLATAD_CHECK_HIP(hipStreamWaitEvent(aux, ss->fork, 0));
+        if (beside != nullptr && beside != stream) SPLATAD_CHECK_HIP(hipStreamWaitEvent(beside, ss->fork, 0));
+        auto enqueue_block_sorts = [&]() -> int {
+            int e;
+#define SPLATAD_BLOCK_CLASS(cls, ER, threads, hi, wgs, on)                                                        \
+            if ((e = launch_block_sort<ER>(cls, threads, hi, wgs, (uint32_t)pl.blocks, cg, g.tile_w, g.tile_h,   \
+                                           n_tiles, tile_n_bits, n_isects, w.piece_counts, w.pieces, w.entries,  \
+                                           w.seg_starts, w.list_tile_counts, isect_ids, flatten_ids, on)) != 0)  \
+                return e;
+            SPLATAD_BLOCK_CLASS(4, 10, 1024, kBlockSortCap, 256u, stream)
+            SPLATAD_BLOCK_CLASS(3, 8, 1024, 8192u, 256u, stream)
+            SPLATAD_BLOCK_CLASS(2, 8, 512, 4096u, 512u, ss->aux[0])
+            SPLATAD_BLOCK_CLASS(1, 8, 256, 2048u, 1024u, ss->aux[1])
+            SPLATAD_BLOCK_CLASS(0, 4, 128, 512u, 2048u, ss->aux[1])
+#undef SPLATAD_BLOCK_CLASS
+            return 0;
+        };
+        rc = enqueue_block_sorts();
+        // (joined whatever happens: work already queued on the helper streams writes the caller's buffers)
+        for (int k = 0; k < 2; ++k) {
+            const hipError_t r = hipEventRecord(ss->join[k], ss->aux[k]);
+            const hipError_t q = r == hipSuccess ? hipStreamWaitEvent(stream, ss->join[k], 0) : r;
+            if (q != hipSuccess && rc == 0) SPLATAD_CHECK_HIP(q);
+        }
+        if (rc) return rc;
+        SPLATAD_LAUNCH_CHECK();
+        return 0;
+    }
     hipLaunchKernelGGL((square ? isect_tile_bin_kernel<true, 16> : isect_tile_bin_kernel<true, 0>),
                        dim3((uint32_t)bin_wgs),
                        dim3(SPLATAD_THREADS), 0, stream, cg, g.tile_w, g.tile_h, sshift, tcopies,
@@ -1908,7 +2620,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                        w.tile_counts, (const int32_t *)w.tile_starts, w.tile_fill, w.pairs, n_isects,
                        w.seg_counts, w.seg_lists, tile_offsets,
                        local_scan ? (const int64_t *)w.block_sums : (const int64_t *)nullptr, n_scan_blocks,
-                       w.seg_starts);
+                       w.seg_starts, pl.bsshift - sshift);
     SPLATAD_LAUNCH_CHECK();
     // Size classes: a launch per class (one for the two upper classes), so that the LDS per
     // workgroup (and with it the number of resident workgroups) fits the segment length; the
@@ -1916,9 +2628,6 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     // segments; they run on two helper streams beside the caller's, forked and joined with
     // events, so that the few long workgroups of the upper classes overlap the many short ones
     // of the lower classes.
-    const uint32_t nseg = (uint32_t)segs;
-    IsectDevice *ss = nullptr;
-    if ((rc = isect_device(&ss)) != 0) return rc;
     std::lock_guard<std::mutex> fork_lock(ss->guard);
     SPLATAD_CHECK_HIP(hipEventRecord(ss->fork, stream));
     for (hipStream_t aux : ss->aux) SPLATAD_CHECK_HIP(hipStreamWaitEvent(aux, ss->fork, 0));
@@ -1963,7 +2672,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
 } // namespace
 
 extern "C" size_t splatad_isect_workspace_bytes(uint64_t total, uint32_t C, uint32_t n_tiles) {
-    return isect_ws_bytes(total, (uint64_t)C * n_tiles);
+    return isect_ws_bytes(total, C, n_tiles);
 }
 
 extern "C" size_t splatad_isect_lists_bytes(uint64_t total, int64_t n_isects) {
