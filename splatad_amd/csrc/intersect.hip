@@ -265,7 +265,7 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
                    unsigned long long *__restrict__ counters,
                    unsigned long long *__restrict__ n_isects_host, int32_t *__restrict__ clear,
                    uint64_t clear_words, const float *__restrict__ depths, uint32_t n_slabs,
-                   uint32_t *__restrict__ slab_bounds, int unit_weights) {
+                   uint32_t *__restrict__ slab_bounds, int unit_weights, int count_rows) {
     SPLATAD_STAGE_ELEVATIONS(g)
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words;
          i += (uint64_t)gridDim.x * blockDim.x)
@@ -285,6 +285,7 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
         }, n_slabs, blockIdx.x - n_wgs, slab_bounds);
         return;
     }
+    if (!count_rows) return; // uniform: a caller that knows the count wants the clearing and the slabs only
     long long s = 0;
     // four Gaussians per lane and step, so that their loads are in flight together (the
     // kernel is bound by memory latency otherwise)
@@ -2304,8 +2305,8 @@ static inline dim3 grid_for(uint64_t n) {
 // (default priority) and events of the segment sort.  `guard` serialises the enqueueing of the
 // fork / join sequences that share them (enqueueing only: no call waits for the GPU under it).
 struct IsectDevice {
-    hipStream_t aux[2];
-    hipEvent_t fork, join[2];
+    hipStream_t aux[2], helper;
+    hipEvent_t fork, join[2], helper_fork, helper_done;
     std::mutex guard;
 };
 
@@ -2321,6 +2322,9 @@ static int isect_device(IsectDevice **out) {
         for (hipStream_t &a : s->aux) SPLATAD_CHECK_HIP(hipStreamCreateWithFlags(&a, hipStreamNonBlocking));
         SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->fork, hipEventDisableTiming));
         for (hipEvent_t &e : s->join) SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        SPLATAD_CHECK_HIP(hipStreamCreateWithFlags(&s->helper, hipStreamNonBlocking));
+        SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->helper_fork, hipEventDisableTiming));
+        SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->helper_done, hipEventDisableTiming));
         table[dev] = s;
     }
     *out = table[dev];
@@ -2401,7 +2405,10 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     if (n_isects_host) *n_isects_host = 0;
     if (total == 0) return 0;
     SPLATAD_REQUIRE(total < (1ull << 31), "isect: number of projected Gaussians must be below 2^31");
-    SPLATAD_REQUIRE(means2d && radii && tiles_per_gauss && workspace, "isect: null pointer argument");
+    // (tiles_per_gauss may be null for a caller that knows the count and wants sorted lists: the
+    // rows' counts are then not made)
+    SPLATAD_REQUIRE(means2d && radii && workspace && (tiles_per_gauss || (known && sort)),
+                    "isect: null pointer argument");
     SPLATAD_REQUIRE(camera_ids != nullptr || N > 0, "isect: N is zero for unpacked input");
     SPLATAD_REQUIRE(!sort || depths != nullptr, "isect: depths is null");
     const IsectPlan pl = isect_plan<LIDAR>(g, total, C, sort);
@@ -2426,6 +2433,9 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
     if (!skip_count) {
         dim3 count_grid = grid_for(total);
         if (count_grid.x > 1024) count_grid.x = 1024;
+        // (without the rows' counts the kernel only clears and finds the slabs' bounds)
+        const bool count_rows = tiles_per_gauss != nullptr;
+        if (!count_rows && count_grid.x > 256) count_grid.x = 256;
         const bool slabs = sort && pl.bsshift != 0; // one more workgroup finds the slabs' bounds
         if (slabs) count_grid.x += kSlabEstimates;
         hipLaunchKernelGGL((slabs ? isect_count_kernel<LIDAR, true> : isect_count_kernel<LIDAR, false>),
@@ -2435,7 +2445,7 @@ static int isect_count(TileGrid g, uint64_t total, uint32_t N, const int64_t *ca
                            slabs ? w.slab_bounds : (uint32_t *)nullptr,
                            // the block sort's slabs even out the coarse lists, an entry per Gaussian
                            // and block; the segment sort's the tile segments
-                           pl.block_sort ? 1 : 0);
+                           pl.block_sort ? 1 : 0, count_rows ? 1 : 0);
         SPLATAD_LAUNCH_CHECK();
     } else {
         hipLaunchKernelGGL(fill_zero_i32_kernel, grid_for(w.n_zeroed), dim3(SPLATAD_THREADS), 0, stream,
@@ -2765,6 +2775,26 @@ extern "C" int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N,
     return isect_fill<true>(g, total, N, camera_ids, means2d, radii, depths, C, sort, n_isects,
                             tiles_per_gauss, workspace, lists, isect_ids, flatten_ids, tile_offsets,
                             (hipStream_t)stream);
+}
+
+extern "C" int splatad_helper_stream_fork(splatad_stream_t stream, splatad_stream_t *helper) {
+    SPLATAD_REQUIRE(helper != nullptr, "helper stream: null pointer argument");
+    IsectDevice *ss = nullptr;
+    if (int rc = isect_device(&ss)) return rc;
+    std::lock_guard<std::mutex> lock(ss->guard);
+    SPLATAD_CHECK_HIP(hipEventRecord(ss->helper_fork, (hipStream_t)stream));
+    SPLATAD_CHECK_HIP(hipStreamWaitEvent(ss->helper, ss->helper_fork, 0));
+    *helper = (splatad_stream_t)ss->helper;
+    return 0;
+}
+
+extern "C" int splatad_helper_stream_join(splatad_stream_t stream) {
+    IsectDevice *ss = nullptr;
+    if (int rc = isect_device(&ss)) return rc;
+    std::lock_guard<std::mutex> lock(ss->guard);
+    SPLATAD_CHECK_HIP(hipEventRecord(ss->helper_done, ss->helper));
+    SPLATAD_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, ss->helper_done, 0));
+    return 0;
 }
 
 extern "C" int splatad_isect_offset_encode(int64_t n_isects, const int64_t *isect_ids, uint32_t C,
