@@ -2605,9 +2605,9 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                                            w.seg_starts, w.list_tile_counts, isect_ids, flatten_ids, on)) != 0)  \
                 return e;
             SPLATAD_BLOCK_CLASS(4, 10, 1024, kBlockSortCap, 256u, stream)
-            SPLATAD_BLOCK_CLASS(3, 8, 1024, 8192u, 256u, stream)
+            SPLATAD_BLOCK_CLASS(3, 8, 1024, 8192u, 256u, ss->aux[1])
             SPLATAD_BLOCK_CLASS(2, 8, 512, 4096u, 512u, ss->aux[0])
-            SPLATAD_BLOCK_CLASS(1, 8, 256, 2048u, 1024u, ss->aux[1])
+            SPLATAD_BLOCK_CLASS(1, 8, 256, 2048u, 1024u, stream)
             SPLATAD_BLOCK_CLASS(0, 4, 128, 512u, 2048u, ss->aux[1])
 #undef SPLATAD_BLOCK_CLASS
             return 0;
