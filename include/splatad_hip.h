@@ -287,17 +287,6 @@ int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N, const int64_t *ca
                                    int32_t *flatten_ids, int32_t *tile_offsets,
                                    splatad_stream_t stream);
 
-/* A stream of the library's (one per device, default priority, kept for the life of the
- * process) for work that only depends on what `stream` holds so far and may run beside what
- * `stream` is given next: _fork makes that stream wait for `stream`'s present end and returns
- * it; _join makes `stream` wait for everything enqueued on it since.  Every _fork is followed by
- * its _join before the buffers written in between are read on `stream` or released; calls that
- * overlap on one device share the stream and run on it one after the other.  rasterization()
- * uses it for the packed rows, which the tile intersection does not read.  No counterpart in
- * the reference. */
-int splatad_helper_stream_fork(splatad_stream_t stream, splatad_stream_t *helper);
-int splatad_helper_stream_join(splatad_stream_t stream);
-
 /* isect_offset_encode_tensor, rasterization.cu:264-285 (kernel :218-262). */
 int splatad_isect_offset_encode(int64_t n_isects, const int64_t *isect_ids, uint32_t C,
                                 uint32_t n_tiles, int32_t *offsets, splatad_stream_t stream);

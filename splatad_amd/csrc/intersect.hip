@@ -2305,8 +2305,8 @@ static inline dim3 grid_for(uint64_t n) {
 // (default priority) and events of the segment sort.  `guard` serialises the enqueueing of the
 // fork / join sequences that share them (enqueueing only: no call waits for the GPU under it).
 struct IsectDevice {
-    hipStream_t aux[2], helper;
-    hipEvent_t fork, join[2], helper_fork, helper_done;
+    hipStream_t aux[2];
+    hipEvent_t fork, join[2];
     std::mutex guard;
 };
 
@@ -2322,9 +2322,6 @@ static int isect_device(IsectDevice **out) {
         for (hipStream_t &a : s->aux) SPLATAD_CHECK_HIP(hipStreamCreateWithFlags(&a, hipStreamNonBlocking));
         SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->fork, hipEventDisableTiming));
         for (hipEvent_t &e : s->join) SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-        SPLATAD_CHECK_HIP(hipStreamCreateWithFlags(&s->helper, hipStreamNonBlocking));
-        SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->helper_fork, hipEventDisableTiming));
-        SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->helper_done, hipEventDisableTiming));
         table[dev] = s;
     }
     *out = table[dev];
@@ -2775,26 +2772,6 @@ extern "C" int splatad_isect_lidar_tiles_fill(uint64_t total, uint32_t N,
     return isect_fill<true>(g, total, N, camera_ids, means2d, radii, depths, C, sort, n_isects,
                             tiles_per_gauss, workspace, lists, isect_ids, flatten_ids, tile_offsets,
                             (hipStream_t)stream);
-}
-
-extern "C" int splatad_helper_stream_fork(splatad_stream_t stream, splatad_stream_t *helper) {
-    SPLATAD_REQUIRE(helper != nullptr, "helper stream: null pointer argument");
-    IsectDevice *ss = nullptr;
-    if (int rc = isect_device(&ss)) return rc;
-    std::lock_guard<std::mutex> lock(ss->guard);
-    SPLATAD_CHECK_HIP(hipEventRecord(ss->helper_fork, (hipStream_t)stream));
-    SPLATAD_CHECK_HIP(hipStreamWaitEvent(ss->helper, ss->helper_fork, 0));
-    *helper = (splatad_stream_t)ss->helper;
-    return 0;
-}
-
-extern "C" int splatad_helper_stream_join(splatad_stream_t stream) {
-    IsectDevice *ss = nullptr;
-    if (int rc = isect_device(&ss)) return rc;
-    std::lock_guard<std::mutex> lock(ss->guard);
-    SPLATAD_CHECK_HIP(hipEventRecord(ss->helper_done, ss->helper));
-    SPLATAD_CHECK_HIP(hipStreamWaitEvent((hipStream_t)stream, ss->helper_done, 0));
-    return 0;
 }
 
 extern "C" int splatad_isect_offset_encode(int64_t n_isects, const int64_t *isect_ids, uint32_t C,

@@ -14,8 +14,6 @@
 #include "scan.h"
 #include "tile_rect.h"
 
-#include <mutex>
-
 #define RAD_TO_DEG 57.2957795131f
 
 namespace {
@@ -542,44 +540,6 @@ extern "C" int splatad_lidar_projection_fwd(uint32_t C, uint32_t N, const float 
     return 0;
 }
 
-// Per device, created at first use and kept for the life of the process: a helper stream (default
-// priority) on which the scan over the kept flags runs beside the first stages of the tile
-// intersection, which do not read it, and the events that order it.  Whatever reads the rows'
-// positions afterwards waits for `scanned` first.
-struct PackedDevice {
-    hipStream_t aux;
-    hipEvent_t fork, scanned;
-    std::mutex guard; // enqueueing only: no call waits for the GPU under it
-};
-
-static int packed_device(PackedDevice **out) {
-    static std::mutex table_guard;
-    static PackedDevice *table[kHostWordDevices] = {};
-    int dev = 0;
-    SPLATAD_CHECK_HIP(hipGetDevice(&dev));
-    SPLATAD_REQUIRE(dev >= 0 && dev < kHostWordDevices, "packed projection: device index %d out of range", dev);
-    std::lock_guard<std::mutex> lock(table_guard);
-    if (!table[dev]) {
-        PackedDevice *s = new PackedDevice();
-        SPLATAD_CHECK_HIP(hipStreamCreateWithFlags(&s->aux, hipStreamNonBlocking));
-        SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->fork, hipEventDisableTiming));
-        SPLATAD_CHECK_HIP(hipEventCreateWithFlags(&s->scanned, hipEventDisableTiming));
-        table[dev] = s;
-    }
-    *out = table[dev];
-    return 0;
-}
-
-// Makes `stream` wait for the scan of the device's last counting call (nothing to wait for when
-// that scan ran on the caller's stream: the event is then older than the stream's own work).
-static int packed_wait_scanned(hipStream_t stream) {
-    PackedDevice *pd = nullptr;
-    if (int rc = packed_device(&pd)) return rc;
-    std::lock_guard<std::mutex> lock(pd->guard);
-    SPLATAD_CHECK_HIP(hipStreamWaitEvent(stream, pd->scanned, 0));
-    return 0;
-}
-
 extern "C" size_t splatad_projection_packed_workspace_bytes(uint32_t C, uint32_t N) {
     const uint64_t T = (uint64_t)C * N;
     return 256 + splatad_align256(T * 8) * 3 + splatad_align256(T * 4) * 3 +
@@ -623,28 +583,8 @@ static int packed_count(uint32_t C, uint32_t N, const float *means, const float 
                            (const int64_t *)nullptr, (const int64_t *)w.block_sums, (const int64_t *)w.tile_sums,
                            n_groups, lease.word.device);
         SPLATAD_LAUNCH_CHECK();
-        // the scan that gives every kept row its position, on the helper stream when the first
-        // stages of the tile intersection are there to run beside it (they read the dense rows)
-        hipStream_t scan_on = (hipStream_t)stream;
-        PackedDevice *pd = nullptr;
-        if (isect_workspace != nullptr) {
-            if ((rc = packed_device(&pd)) != 0) return rc;
-            pd->guard.lock();
-            const hipError_t r = hipEventRecord(pd->fork, (hipStream_t)stream);
-            const hipError_t q = r == hipSuccess ? hipStreamWaitEvent(pd->aux, pd->fork, 0) : r;
-            if (q != hipSuccess) {
-                pd->guard.unlock();
-                SPLATAD_CHECK_HIP(q);
-            }
-            scan_on = pd->aux;
-        }
         rc = launch_exclusive_scan_apply<int32_t>(w.radii, (int64_t)T, 2, 1, w.pos, w.total, w.block_sums,
-                                                  scan_on, SCAN_ITEMS);
-        if (pd != nullptr) {
-            const hipError_t r = hipEventRecord(pd->scanned, pd->aux);
-            pd->guard.unlock();
-            if (rc == 0) SPLATAD_CHECK_HIP(r);
-        }
+                                                  (hipStream_t)stream, SCAN_ITEMS);
         if (rc) return rc;
         if (isect_workspace != nullptr) {
             rc = splatad_isect_tiles_prepare(T, N, nullptr, w.means2d, w.radii, w.depths, C, tile_size,
@@ -726,7 +666,6 @@ extern "C" int splatad_isect_tiles_fill_packed(uint32_t C, uint32_t N, uint32_t 
     SPLATAD_REQUIRE(packed_workspace && isect_workspace, "isect_tiles: null workspace");
     const uint64_t T = (uint64_t)C * N;
     PackedWorkspace w = carve_packed((void *)packed_workspace, T);
-    if (int rc = packed_wait_scanned((hipStream_t)stream)) return rc; // the rows' positions
     return splatad_isect_tiles_fill_remapped(T, N, w.means2d, w.radii, w.depths, C, tile_size, tile_width,
                                              tile_height, n_isects, w.tiles, w.pos, isect_workspace, lists,
                                              tiles_per_gauss, isect_ids, flatten_ids, tile_offsets,
@@ -740,7 +679,6 @@ extern "C" int splatad_view_colors_fwd_packed(uint32_t C, uint32_t N, uint32_t K
                                               splatad_stream_t stream) {
     SPLATAD_REQUIRE(packed_workspace != nullptr, "view colours: null workspace");
     PackedWorkspace w = carve_packed((void *)packed_workspace, (uint64_t)C * N);
-    if (int rc = packed_wait_scanned((hipStream_t)stream)) return rc; // the rows' positions
     return splatad_view_colors_fwd_remapped(C, N, K, degree, means, viewmats, w.radii, w.pos, coeffs,
                                             coeffs_per_sensor, with_depth ? w.depths : nullptr, colors, stream);
 }
@@ -766,7 +704,6 @@ extern "C" int splatad_projection_packed_fill(uint32_t C, uint32_t N, int64_t nn
     SPLATAD_REQUIRE((opacities != nullptr) == (row_opacities != nullptr),
                     "packed projection: opacities and row_opacities go together");
     PackedWorkspace w = carve_packed((void *)workspace, T);
-    if (int rc = packed_wait_scanned((hipStream_t)stream)) return rc; // the rows' positions
     hipLaunchKernelGGL(packed_compact_kernel,
                        dim3((uint32_t)((T + SPLATAD_THREADS - 1) / SPLATAD_THREADS)),
                        dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, C, N, nnz, w.radii,

@@ -229,88 +229,76 @@ class _Ops:
             nnz = int(nnz_host.value)
             isect_result = side = None
             work = main  # the stream of the kernels that write the outputs
-            forked = False
             if isect_grid is not None:
                 # first what the GPU is waiting for: the rest of the tile intersection
                 side = getattr(beside, "side", None)
                 if side is not None:
                     work = ctypes.c_void_p(side.cuda_stream)
-                elif nnz and int(n_isects_host.value) and not torch.cuda.is_current_stream_capturing():
-                    # the packed outputs on the library's helper stream, beside the intersection,
-                    # which reads the dense rows of the workspace; joined below
-                    work = ctypes.c_void_p()
-                    _check(lib.splatad_helper_stream_fork(main, ctypes.byref(work)))
-                    forked = True
-            try:
-                if isect_grid is not None:
-                    n_isects = int(n_isects_host.value)
-                    tile_w, tile_h = int(isect_grid[1]), int(isect_grid[2])
-                    tiles_per_gauss = torch.empty((nnz,), dtype=torch.int32, device=dev)
-                    isect_ids = torch.empty((n_isects,), dtype=torch.int64, device=dev)
-                    flatten_ids = torch.empty((n_isects,), dtype=torch.int32, device=dev)
-                    offsets = lists = None
-                    if n_isects:
-                        offsets = torch.empty((C, tile_h, tile_w), dtype=torch.int32, device=dev)
-                        lists = _workspace(lib.splatad_isect_lists_bytes(_u64(C * N), _i64(n_isects)), dev)
-                    else:
-                        tiles_per_gauss.zero_()
-                    if n_isects or side is not None:  # (without lists the call only orders the side stream)
-                        _check(lib.splatad_isect_tiles_fill_packed(
-                            _u32(C), _u32(N), *(_u32(v) for v in isect_grid), _i64(n_isects), _p(ws),
-                            _p(isect_ws), _p(lists), _p(tiles_per_gauss), _p(isect_ids), _p(flatten_ids),
-                            _p(offsets), work if side is not None else None, main))
-                    if offsets is not None:
-                        # isect_offset_encode() on the same, unmodified tensor is free
-                        isect_ids._splatad_tile_offsets = (offsets, isect_ids._version)
-                    isect_result = (tiles_per_gauss, isect_ids, flatten_ids)
-                requests = getattr(beside, "requests", None) or {}
-                indptr = torch.empty((C + 1,), dtype=torch.int32, device=dev)
-                camera_ids = torch.empty((nnz,), dtype=torch.int64, device=dev)
-                gaussian_ids = torch.empty((nnz,), dtype=torch.int64, device=dev)
-                radii = torch.empty((nnz, 2), dtype=torch.int32, device=dev)
-                means2d = torch.empty((nnz, 2), **f); depths = torch.empty((nnz,), **f)
-                conics = torch.empty((nnz, 3), **f); pix_vels = torch.empty((nnz, 2), **f)
-                comps = torch.empty((nnz,), **f) if calc_compensations else None
-                opacities = requests.get("opacities")
-                row_opacities = None
-                if opacities is not None:
-                    opacities = _in(opacities, "opacities")
-                    assert opacities.shape == (N,), opacities.shape
-                    row_opacities = torch.empty((nnz,), **f)
-                _check(lib.splatad_projection_packed_fill(
-                    _u32(C), _u32(N), _i64(nnz), _p(ws), _p(indptr), _p(camera_ids), _p(gaussian_ids),
-                    _p(radii), _p(means2d), _p(depths), _p(conics), _p(comps), _p(pix_vels),
-                    _p(opacities), _p(row_opacities), work))
-                results = {}
-                if row_opacities is not None:
-                    results["opacities"] = row_opacities
-                if "colors" in requests:
-                    degree, coeffs, with_depth = requests["colors"]
-                    coeffs = _in(coeffs, "coeffs")
-                    colors = torch.empty((nnz, 4 if with_depth else 3), **f)
-                    if nnz:
-                        _check(lib.splatad_view_colors_fwd_packed(
-                            _u32(C), _u32(N), _u32(coeffs.shape[-2]), _u32(degree), _p(means), _p(viewmats),
-                            _p(ws), _p(coeffs), _i32(coeffs.dim() == 4), _i32(bool(with_depth)), _p(colors), work))
-                    results["colors"] = colors
-                if "color_cache" in requests:
-                    # the colour cache of rasterize_to_pixels_sh_fwd for the packed rows, see
-                    # view_colors_cache(); needs requests["opacities"]
-                    degree, coeffs, with_depth, tile_size, tile_w, tile_h, limit = requests["color_cache"]
-                    coeffs = _in(coeffs, "coeffs")
-                    assert opacities is not None
-                    words = lib.splatad_view_colors_cache_bytes(_u64(nnz)) // 4
-                    buf = torch.empty((words,), **f)
-                    if nnz:
-                        _check(lib.splatad_view_colors_cache(
-                            _u32(nnz), _u32(C), _u32(N), _u32(coeffs.shape[-2]), _u32(degree), _p(means),
-                            _p(viewmats), _p(camera_ids), _p(gaussian_ids), _p(radii), _p(coeffs),
-                            _i32(coeffs.dim() == 4), _p(depths if with_depth else None), _p(opacities),
-                            _u32(tile_size), _u32(tile_w), _u32(tile_h), _f32(limit), _p(buf), work))
-                    results["color_cache"] = buf[: nnz * 4].view(nnz, 4)
-            finally:
-                if forked:  # (also on an error: the helper stream reads this call's buffers)
-                    _check(lib.splatad_helper_stream_join(main))
+                n_isects = int(n_isects_host.value)
+                tile_w, tile_h = int(isect_grid[1]), int(isect_grid[2])
+                tiles_per_gauss = torch.empty((nnz,), dtype=torch.int32, device=dev)
+                isect_ids = torch.empty((n_isects,), dtype=torch.int64, device=dev)
+                flatten_ids = torch.empty((n_isects,), dtype=torch.int32, device=dev)
+                offsets = lists = None
+                if n_isects:
+                    offsets = torch.empty((C, tile_h, tile_w), dtype=torch.int32, device=dev)
+                    lists = _workspace(lib.splatad_isect_lists_bytes(_u64(C * N), _i64(n_isects)), dev)
+                else:
+                    tiles_per_gauss.zero_()
+                if n_isects or side is not None:  # (without lists the call only orders the side stream)
+                    _check(lib.splatad_isect_tiles_fill_packed(
+                        _u32(C), _u32(N), *(_u32(v) for v in isect_grid), _i64(n_isects), _p(ws),
+                        _p(isect_ws), _p(lists), _p(tiles_per_gauss), _p(isect_ids), _p(flatten_ids),
+                        _p(offsets), work if side is not None else None, main))
+                if offsets is not None:
+                    # isect_offset_encode() on the same, unmodified tensor is free
+                    isect_ids._splatad_tile_offsets = (offsets, isect_ids._version)
+                isect_result = (tiles_per_gauss, isect_ids, flatten_ids)
+            requests = getattr(beside, "requests", None) or {}
+            indptr = torch.empty((C + 1,), dtype=torch.int32, device=dev)
+            camera_ids = torch.empty((nnz,), dtype=torch.int64, device=dev)
+            gaussian_ids = torch.empty((nnz,), dtype=torch.int64, device=dev)
+            radii = torch.empty((nnz, 2), dtype=torch.int32, device=dev)
+            means2d = torch.empty((nnz, 2), **f); depths = torch.empty((nnz,), **f)
+            conics = torch.empty((nnz, 3), **f); pix_vels = torch.empty((nnz, 2), **f)
+            comps = torch.empty((nnz,), **f) if calc_compensations else None
+            opacities = requests.get("opacities")
+            row_opacities = None
+            if opacities is not None:
+                opacities = _in(opacities, "opacities")
+                assert opacities.shape == (N,), opacities.shape
+                row_opacities = torch.empty((nnz,), **f)
+            _check(lib.splatad_projection_packed_fill(
+                _u32(C), _u32(N), _i64(nnz), _p(ws), _p(indptr), _p(camera_ids), _p(gaussian_ids),
+                _p(radii), _p(means2d), _p(depths), _p(conics), _p(comps), _p(pix_vels),
+                _p(opacities), _p(row_opacities), work))
+            results = {}
+            if row_opacities is not None:
+                results["opacities"] = row_opacities
+            if "colors" in requests:
+                degree, coeffs, with_depth = requests["colors"]
+                coeffs = _in(coeffs, "coeffs")
+                colors = torch.empty((nnz, 4 if with_depth else 3), **f)
+                if nnz:
+                    _check(lib.splatad_view_colors_fwd_packed(
+                        _u32(C), _u32(N), _u32(coeffs.shape[-2]), _u32(degree), _p(means), _p(viewmats),
+                        _p(ws), _p(coeffs), _i32(coeffs.dim() == 4), _i32(bool(with_depth)), _p(colors), work))
+                results["colors"] = colors
+            if "color_cache" in requests:
+                # the colour cache of rasterize_to_pixels_sh_fwd for the packed rows, see
+                # view_colors_cache(); needs requests["opacities"]
+                degree, coeffs, with_depth, tile_size, tile_w, tile_h, limit = requests["color_cache"]
+                coeffs = _in(coeffs, "coeffs")
+                assert opacities is not None
+                words = lib.splatad_view_colors_cache_bytes(_u64(nnz)) // 4
+                buf = torch.empty((words,), **f)
+                if nnz:
+                    _check(lib.splatad_view_colors_cache(
+                        _u32(nnz), _u32(C), _u32(N), _u32(coeffs.shape[-2]), _u32(degree), _p(means),
+                        _p(viewmats), _p(camera_ids), _p(gaussian_ids), _p(radii), _p(coeffs),
+                        _i32(coeffs.dim() == 4), _p(depths if with_depth else None), _p(opacities),
+                        _u32(tile_size), _u32(tile_w), _u32(tile_h), _f32(limit), _p(buf), work))
+                results["color_cache"] = buf[: nnz * 4].view(nnz, 4)
             if beside is not None:
                 beside.results = results
             if side is not None:
