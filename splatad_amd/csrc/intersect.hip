@@ -1506,8 +1506,10 @@ isect_small_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t 
 constexpr uint32_t kBlockSortCap = 10240;   // longest (block, slab) list the LDS sort takes
 constexpr uint32_t kBlockMergeCap = 4096;   // slabs of a block are sorted together up to this many entries,
 constexpr uint32_t kBlockPairsCap = 32768;  // and about this many intersections
-constexpr int kBlockClasses = 5;
-__constant__ const uint32_t kBlockClassMax[kBlockClasses] = {512u, 2048u, 4096u, 8192u, kBlockSortCap};
+constexpr uint32_t kBlockLongMax = 8 * kBlockSortCap; // longest list the block sort takes at all (in parts)
+constexpr int kBlockClasses = 6;            // five by length, and the lists beyond kBlockSortCap
+constexpr int kBlockLongClass = 5;
+__constant__ const uint32_t kBlockClassMax[kBlockClasses] = {512u, 2048u, 4096u, 8192u, kBlockSortCap, 0xFFFFFFFFu};
 
 // Dynamic LDS of the block sort: the staging array and its four end markers, the masks and
 // bucket numbers of the staged entries, the fine bins and two bucket tables.
@@ -1679,8 +1681,13 @@ __device__ __forceinline__ void sort_expand_piece(uint4 piece, CoarseGrid cg, ui
                                                   int64_t *__restrict__ isect_ids,
                                                   int32_t *__restrict__ flatten_ids,
                                                   uint64_t *lds_staged, uint32_t *s_wave, uint32_t &s_big,
-                                                  uint32_t (*s_cnt)[16]) {
-    const uint32_t n = piece.y;
+                                                  uint32_t (*s_cnt)[16], bool gathered = false,
+                                                  uint32_t n_gathered = 0, uint32_t *carried = nullptr) {
+    // gathered: the piece is the first n_gathered entries of the staging array and their masks (a
+    // part of a long list, see sort_expand_long_list); *carried (lane t < 16) then holds the
+    // entries of the list's nearer parts and of the block's earlier slabs that name tile t, and
+    // takes this part's on top
+    const uint32_t n = gathered ? n_gathered : piece.y;
     uint32_t *s_fine = reinterpret_cast<uint32_t *>(lds_staged + lds_words + 4);
     uint32_t *s_first = s_fine + kSortFineBins;   // bucket_cap + 1 words: starts, then the end
     uint32_t *s_cursor = s_first + bucket_cap + 1;
@@ -1693,15 +1700,26 @@ __device__ __forceinline__ void sort_expand_piece(uint4 piece, CoarseGrid cg, ui
 
     uint64_t held[ER];
     uint32_t held_mask[ER];
+    uint32_t pre; // lane t < 16: the entries of the block's earlier slabs that name tile t
+    if (gathered) { // uniform
 #pragma unroll
-    for (int k = 0; k < ER; ++k) {
-        const uint32_t i = tid + k * nt;
-        const uint4 e = i < n ? g[i] : make_uint4(~0u, ~0u, 0u, 0u);
-        held[k] = ((uint64_t)e.y << 32) | (uint64_t)e.x;
-        held_mask[k] = e.w;
+        for (int k = 0; k < ER; ++k) {
+            const uint32_t i = tid + k * nt;
+            held[k] = i < n ? lds_staged[i] : ~0ull;
+            held_mask[k] = i < n ? (uint32_t)s_mask[i] : 0u;
+        }
+        pre = *carried;
+        __syncthreads(); // the staging array is free for the sort
+    } else {
+#pragma unroll
+        for (int k = 0; k < ER; ++k) {
+            const uint32_t i = tid + k * nt;
+            const uint4 e = i < n ? g[i] : make_uint4(~0u, ~0u, 0u, 0u);
+            held[k] = ((uint64_t)e.y << 32) | (uint64_t)e.x;
+            held_mask[k] = e.w;
+        }
+        pre = lane < 16 ? (uint32_t)slabs_before[(size_t)piece.w * 16 + lane] : 0u;
     }
-    // lane t < 16: the entries of the block's earlier slabs that name tile t
-    const uint32_t pre = lane < 16 ? (uint32_t)slabs_before[(size_t)piece.w * 16 + lane] : 0u;
     auto count16 = [&](uint32_t mask) -> uint32_t {
         uint32_t cnt = 0;
 #pragma unroll
@@ -1949,9 +1967,167 @@ __device__ __forceinline__ void sort_expand_piece(uint4 piece, CoarseGrid cg, ui
             }
         }
     }
+    if (gathered) { // uniform: what this part added to the tiles' lists
+        uint32_t total = pre;
+        if (lane < 16)
+            for (uint32_t w = 0; w < n_waves; ++w) total += s_cnt[w][lane];
+        *carried = total;
+    }
 }
 
+// A list too long for the LDS sort, by one workgroup, part by part in ascending key order.  The
+// key intervals still to do are kept on a small stack (nearest on top).  An interval of up to
+// lds_words entries is gathered from the list into the staging array (in any order), sorted and
+// written like any piece, and the tiles' cursors move on by what it wrote; a longer interval is
+// cut in two: a histogram of its keys (depth bits above flatten id, as one 64-bit number) over
+// kLongBins bins that are linear between its smallest and largest key, with every bin's
+// smallest and largest key beside the count, tells its nearest part and the rest.  The keys of
+// a coarse list are distinct, so an interval that still holds too much spans more keys than
+// bins, both halves of a cut are smaller than the interval, and the stack stays a few entries
+// deep (every level of cutting divides the span of the keys by kLongBins).
+constexpr uint32_t kLongBins = 2048;
+constexpr uint32_t kLongStack = 32;
+struct LongInterval { uint64_t lo, hi; uint32_t n, pad; };
+
 template <int ER>
+__device__ __forceinline__ void sort_expand_long_list(uint4 piece, CoarseGrid cg, uint32_t tile_w, uint32_t tile_h,
+                                                      uint32_t n_tiles, uint32_t tile_n_bits, uint32_t lds_words,
+                                                      uint32_t bucket_cap, int64_t n_isects,
+                                                      const uint4 *__restrict__ entries,
+                                                      const int32_t *__restrict__ seg_starts,
+                                                      const int32_t *__restrict__ slabs_before,
+                                                      int64_t *__restrict__ isect_ids,
+                                                      int32_t *__restrict__ flatten_ids, uint64_t *lds_staged,
+                                                      uint32_t *s_wave, uint32_t &s_big, uint32_t (*s_cnt)[16],
+                                                      LongInterval *s_stack, uint32_t &s_top, uint32_t &s_kept,
+                                                      unsigned long long *s_range) {
+    const uint32_t tid = threadIdx.x, nt = blockDim.x, lane = tid & (SPLATAD_WAVE - 1);
+    const uint4 *g = entries + piece.x;
+    const uint32_t n_all = piece.y;
+    uint16_t *s_mask;
+    {
+        uint32_t *s_fine = reinterpret_cast<uint32_t *>(lds_staged + lds_words + 4);
+        uint32_t *s_cursor = s_fine + kSortFineBins + bucket_cap + 1;
+        s_mask = reinterpret_cast<uint16_t *>(s_cursor + bucket_cap) + ((lds_words + 3) & ~3u);
+    }
+    // the histogram of an interval lies over the staging array, which is idle meanwhile
+    unsigned long long *h_lo = reinterpret_cast<unsigned long long *>(lds_staged);
+    unsigned long long *h_hi = h_lo + kLongBins;
+    uint32_t *h_n = reinterpret_cast<uint32_t *>(h_hi + kLongBins);
+    uint32_t *h_group = h_n + kLongBins; // a bin's sub-interval
+    // smallest and largest key of the list
+    {
+        unsigned long long lo = ~0ull, hi = 0ull;
+        for (uint32_t j = tid; j < n_all; j += nt) {
+            const uint4 e = g[j];
+            const unsigned long long key = ((unsigned long long)e.y << 32) | e.x;
+            lo = min(lo, key);
+            hi = max(hi, key);
+        }
+        if (tid == 0) { s_range[0] = ~0ull; s_range[1] = 0ull; }
+        __syncthreads();
+        if (lo <= hi) { atomicMin(&s_range[0], lo); atomicMax(&s_range[1], hi); }
+        __syncthreads();
+        if (tid == 0) {
+            s_stack[0].lo = s_range[0]; s_stack[0].hi = s_range[1]; s_stack[0].n = n_all;
+            s_top = 1;
+        }
+    }
+    uint32_t carried = lane < 16 ? (uint32_t)slabs_before[(size_t)piece.w * 16 + lane] : 0u;
+    for (;;) {
+        __syncthreads();
+        if (s_top == 0) break; // uniform
+        const LongInterval cur = s_stack[s_top - 1];
+        __syncthreads();
+        if (tid == 0) { s_top -= 1; s_kept = 0; }
+        if (cur.n <= lds_words) { // uniform: gather, sort, write
+            __syncthreads();
+            for (uint32_t j0 = (tid & ~(SPLATAD_WAVE - 1u)); j0 < n_all; j0 += 4 * nt) { // uniform per wavefront
+                uint4 e[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t j = j0 + u * nt + lane;
+                    e[u] = j < n_all ? g[j] : make_uint4(0u, 0u, 0u, 0u);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t j = j0 + u * nt + lane;
+                    const unsigned long long key = ((unsigned long long)e[u].y << 32) | e[u].x;
+                    const bool mine = j < n_all && key >= cur.lo && key <= cur.hi;
+                    const uint64_t keep = __ballot(mine);
+                    if (keep != 0) { // uniform
+                        uint32_t at = 0;
+                        const int leader = __ffsll((unsigned long long)keep) - 1;
+                        if ((int)lane == leader) at = atomicAdd(&s_kept, (uint32_t)__popcll(keep));
+                        at = (uint32_t)__shfl((int)at, leader, SPLATAD_WAVE) +
+                             (uint32_t)__popcll(keep & ((1ull << lane) - 1ull));
+                        if (mine && at < lds_words) { // (the interval's count says it fits)
+                            lds_staged[at] = key;
+                            s_mask[at] = (uint16_t)e[u].w;
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+            sort_expand_piece<ER>(piece, cg, tile_w, tile_h, n_tiles, tile_n_bits, lds_words, bucket_cap, n_isects,
+                                  entries, seg_starts, slabs_before, isect_ids, flatten_ids, lds_staged, s_wave,
+                                  s_big, s_cnt, true, min(s_kept, lds_words), &carried);
+            continue;
+        }
+        // cut the interval
+        for (uint32_t f = tid; f < kLongBins; f += nt) { h_lo[f] = ~0ull; h_hi[f] = 0ull; h_n[f] = 0; }
+        const float scale = (float)kLongBins / ((float)(cur.hi - cur.lo) + 1.f);
+        __syncthreads();
+        for (uint32_t j = tid; j < n_all; j += nt) {
+            const uint4 e = g[j];
+            const unsigned long long key = ((unsigned long long)e.y << 32) | e.x;
+            if (key < cur.lo || key > cur.hi) continue;
+            const uint32_t f = min(kLongBins - 1u, (uint32_t)((float)(key - cur.lo) * scale));
+            atomicAdd(&h_n[f], 1u);
+            atomicMin(&h_lo[f], key);
+            atomicMax(&h_hi[f], key);
+        }
+        __syncthreads();
+        // The nearest part: the leading bins that together fit the staging array, up to the first
+        // bin of more than half of it -- or that bin alone, if it comes first, to be cut again
+        // (its keys span less than this interval's: the smallest and the largest key of an
+        // interval lie in its first and last bin).  The part and, under it, the rest of the
+        // interval take the interval's place on the stack.
+        const uint32_t half = lds_words / 2;
+        if (tid == 0) { s_range[0] = ~0ull; s_range[1] = 0ull; s_kept = 0; s_big = kLongBins; }
+        block_exclusive_scan(
+            kLongBins, tid, nt, s_wave, [&](uint32_t f) { return h_n[f]; },
+            [&](uint32_t f, uint32_t before, uint32_t c) {
+                h_group[f] = before;
+                if (c > half) atomicMin(&s_big, f);
+            });
+        const uint32_t first_big = s_big;
+        __syncthreads();
+        for (uint32_t f = tid; f < kLongBins; f += nt) {
+            const uint32_t c = h_n[f];
+            if (c == 0) continue;
+            const bool leads = h_group[f] == 0; // the first bin that holds anything
+            const bool in_part = leads || (f < first_big && h_group[f] + c <= lds_words);
+            if (in_part) {
+                atomicAdd(&s_kept, c);
+                atomicMax(&s_range[1], h_hi[f]); // the part ends at its largest key
+            } else {
+                atomicMin(&s_range[0], h_lo[f]); // the rest begins at its smallest
+            }
+        }
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t top = s_top;
+            const uint32_t n_part = s_kept;
+            if (cur.n > n_part) { s_stack[top].lo = s_range[0]; s_stack[top].hi = cur.hi; s_stack[top].n = cur.n - n_part; ++top; }
+            s_stack[top].lo = cur.lo; s_stack[top].hi = s_range[1]; s_stack[top].n = n_part; ++top;
+            s_top = top;
+        }
+    }
+}
+
+// LONG: the launch takes the lists beyond the capacity of the LDS sort, part by part.
+template <int ER, bool LONG = false>
 __global__ void isect_block_sort_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t n_tiles,
                                         uint32_t tile_n_bits, uint32_t lds_words, uint32_t bucket_cap,
                                         int64_t n_isects, const uint32_t *__restrict__ class_count,
@@ -1964,6 +2140,18 @@ __global__ void isect_block_sort_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t
     __shared__ uint32_t s_big;
     __shared__ uint32_t s_cnt[1024 / SPLATAD_WAVE][16];
     const uint32_t count = *class_count;
+    if constexpr (LONG) {
+        __shared__ LongInterval s_stack[kLongStack];
+        __shared__ uint32_t s_top, s_kept;
+        __shared__ unsigned long long s_range[2];
+        for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) { // uniform across the workgroup
+            sort_expand_long_list<ER>(pieces[k], cg, tile_w, tile_h, n_tiles, tile_n_bits, lds_words, bucket_cap,
+                                      n_isects, entries, seg_starts, slabs_before, isect_ids, flatten_ids,
+                                      lds_staged, s_wave, s_big, s_cnt, s_stack, s_top, s_kept, s_range);
+            __syncthreads();
+        }
+        return;
+    }
     for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) { // uniform across the workgroup
         sort_expand_piece<ER>(pieces[k], cg, tile_w, tile_h, n_tiles, tile_n_bits, lds_words, bucket_cap, n_isects,
                               entries, seg_starts, slabs_before, isect_ids, flatten_ids, lds_staged, s_wave,
@@ -1972,7 +2160,7 @@ __global__ void isect_block_sort_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t
     }
 }
 
-template <int ER>
+template <int ER, bool LONG = false>
 static int launch_block_sort(int cls, uint32_t threads, uint32_t max_n, uint32_t workgroups, uint32_t max_pieces,
                              CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t n_tiles,
                              uint32_t tile_n_bits, int64_t n_isects, const uint32_t *class_count,
@@ -1994,12 +2182,12 @@ static int launch_block_sort(int cls, uint32_t threads, uint32_t max_n, uint32_t
         static size_t allowed = 0;
         std::lock_guard<std::mutex> lock(guard);
         if (lds_bytes > allowed) {
-            SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)isect_block_sort_kernel<ER>,
+            SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)isect_block_sort_kernel<ER, LONG>,
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
             allowed = lds_bytes;
         }
     }
-    hipLaunchKernelGGL((isect_block_sort_kernel<ER>), dim3(workgroups < max_pieces ? workgroups : max_pieces),
+    hipLaunchKernelGGL((isect_block_sort_kernel<ER, LONG>), dim3(workgroups < max_pieces ? workgroups : max_pieces),
                        dim3(threads), lds_bytes, stream, cg, tile_w, tile_h, n_tiles, tile_n_bits, max_n,
                        bucket_cap, n_isects, class_count + cls, pieces + (size_t)cls * max_pieces, entries,
                        seg_starts, slabs_before, isect_ids, flatten_ids);
@@ -2510,7 +2698,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         SPLATAD_LAUNCH_CHECK();
         return 0;
     }
-    // The block sort takes coarse lists of up to kBlockSortCap entries.  Whether all lists are that
+    // The block sort takes coarse lists of up to kBlockLongMax entries.  Whether all lists are that
     // short the host learns from the filling kernel, through a pinned word as it learnt the
     // number of intersections (the wait below ends as soon as that kernel has begun: the GPU has
     // the tile binning to do meanwhile); a scene with a longer list takes the segment sort.
@@ -2574,7 +2762,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     if (pl.block_sort) {
         unsigned long long longest_list = 0;
         if ((rc = host_word_wait(&longest, "isect", &longest_list)) != 0) return rc;
-        short_lists = longest_list <= kBlockSortCap;
+        short_lists = longest_list <= kBlockLongMax;
     }
     if (short_lists) {
         // Pieces of the coarse lists by size class, and the tiles' starts; then a launch per
@@ -2600,6 +2788,12 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
             if ((e = launch_block_sort<ER>(cls, threads, hi, wgs, (uint32_t)pl.blocks, cg, g.tile_w, g.tile_h,   \
                                            n_tiles, tile_n_bits, n_isects, w.piece_counts, w.pieces, w.entries,  \
                                            w.seg_starts, w.list_tile_counts, isect_ids, flatten_ids, on)) != 0)  \
+                return e;
+            // (the lists too long for one LDS sort first: a workgroup each, part by part)
+            if ((e = launch_block_sort<10, true>(kBlockLongClass, 1024, kBlockSortCap, 256u, (uint32_t)pl.blocks, cg,
+                                                 g.tile_w, g.tile_h, n_tiles, tile_n_bits, n_isects,
+                                                 w.piece_counts, w.pieces, w.entries, w.seg_starts,
+                                                 w.list_tile_counts, isect_ids, flatten_ids, stream)) != 0)
                 return e;
             SPLATAD_BLOCK_CLASS(4, 10, 1024, kBlockSortCap, 256u, stream)
             SPLATAD_BLOCK_CLASS(3, 8, 1024, 8192u, 256u, ss->aux[1])

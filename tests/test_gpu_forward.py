@@ -305,12 +305,14 @@ def test_isect_camera_sizes_and_packed(n, C, W, H, ts, rmax):
 
 @pytest.mark.parametrize("n,tie_frac", [(1500, 0.8), (6000, 0.0), (6000, 0.5), (12000, 0.3),
                                         (20000, 0.1), (40000, 0.0), (40000, 0.4), (3000, 1.0),
-                                        (60000, 0.4), (100000, 0.5), (400, 0.2)])
+                                        (60000, 0.4), (100000, 0.5), (400, 0.2), (300000, 0.0),
+                                        (100000, 0.9)])
 def test_isect_sort_long_segments_and_depth_ties(n, tie_frac):
-    # every Gaussian covers all four tiles, so each tile's segment has n entries.  From 2816
-    # Gaussians on, the binning cuts the segments into depth slabs (4 to 16), and equal depths
-    # share a slab: the sizes and tie fractions exercise every segment-length class of the sort
-    # (the longest through 24000 and 50000 equal depths) and, with them, oversized buckets
+    # every Gaussian covers all four tiles of the one coarse block.  The block's list is cut into
+    # up to 16 depth slabs, and equal depths share a slab: the sizes and tie fractions exercise
+    # every length class of the block sort, the lists it takes in parts (16000 to 50000 equal
+    # depths, ordered by id alone; 18750 distinct depths per slab) and, with 90000 equal depths,
+    # the list that is left to the per-tile segment sort with its own classes and oversized buckets
     from splatad_amd import isect_tiles
     rng = np.random.default_rng(n + int(10 * tie_frac))
     means2d = rng.uniform(10, 22, (1, n, 2)).astype(np.float32)
