@@ -134,7 +134,8 @@ __device__ __forceinline__ uint32_t tile_index(const TileGrid &g, int32_t y, int
 // and zero again when it ends) takes the partial sums; the total goes to the host's pinned
 // slot.  On its way the kernel clears `clear_words` words from `clear` on: the counters of the
 // binning kernels behind it, which spares the launch of a clearing kernel.
-constexpr uint32_t kSlabShiftMax = 4;
+constexpr uint32_t kSlabShiftMax = 6;          // 64 slabs at most (the block sort's lists)
+constexpr uint32_t kSegmentSlabShiftMax = 4;   // the segment sort cuts its tile segments into 16 at most
 constexpr uint32_t kSlabSamples = 256;
 constexpr uint32_t kSlabEstimates = 4; // independent sets of samples, a workgroup each
 
@@ -554,7 +555,7 @@ static uint32_t slab_shift_for(uint64_t total, uint64_t segs) {
     if (per_tile < kSlabMinPerTile) return 0;
     if (per_tile < 896) return 2;
     if (per_tile < 2816) return 3;
-    return kSlabShiftMax;
+    return kSegmentSlabShiftMax;
 }
 
 // Bound k from the kSlabEstimates estimates of it ([estimate][1 << kSlabShiftMax]): the mean of
@@ -2326,7 +2327,7 @@ __global__ void fill_zero_i32_kernel(int32_t *p, int64_t n) {
 struct IsectWorkspace {
     int64_t *n_entries;           // [1] length of the coarse lists
     int64_t *scan_total;          // [1]
-    uint32_t *slab_bounds;        // [1 << kSlabShiftMax] depth bits at which the slabs begin
+    uint32_t *slab_bounds;        // [kSlabEstimates][1 << kSlabShiftMax] depth bits at which the slabs begin
     int32_t *zeroed;              // tile_counts, tile_fill, block_totals, seg_counts: contiguous, cleared together
     uint64_t n_zeroed;
     int32_t *tile_counts;         // [tile copies * segments], segments = C * n_tiles * slabs
@@ -2396,8 +2397,11 @@ struct IsectPlan {
 
 // Depth slabs of the coarse lists for the block sort: enough that a list holds about a hundred
 // Gaussians on average (the longest list of a driving frame, at its horizon, is some ten times
-// the average and has to fit the LDS sort: kBlockSortCap), but no more than lets the coarse
-// binning keep all sensors' counters in LDS at once, down to two slabs.
+// the average and should fit the LDS sort, kBlockSortCap: a list taken in parts costs one
+// workgroup 100 us and more -- 1M Gaussians on a 1080p frame with 8 slabs instead of 16 take
+// 0.33 instead of 0.22 ms), but no more than lets the coarse binning keep all sensors' counters in
+// LDS at once, down to two slabs.  (Frames of 2M and 4M Gaussians take 32 and 64 slabs: 0.648
+// and 1.043 ms a frame against 0.671 and 1.052 with 16.)
 static uint32_t block_slab_shift(uint64_t total, uint32_t C, uint64_t blocks_per_cam) {
     const uint64_t per_block = total / ((uint64_t)C * blocks_per_cam);
     uint32_t s = 0;
@@ -2438,7 +2442,7 @@ static size_t carve_isect(void *ws, uint64_t total, uint64_t segs, uint64_t list
     IsectWorkspace w = {};
     w.n_entries = (int64_t *)p;             p += 256;
     w.scan_total = (int64_t *)p;            p += 256;
-    w.slab_bounds = (uint32_t *)p;          p += 256;
+    w.slab_bounds = (uint32_t *)p;          p += splatad_align256((kSlabEstimates << kSlabShiftMax) * 4);
     w.zeroed = (int32_t *)p;
     w.tile_counts = (int32_t *)p;           p += splatad_align256(tslots * 4);
     w.tile_fill = (int32_t *)p;             p += splatad_align256(tslots * 4);
