@@ -2371,12 +2371,14 @@ static uint32_t isect_copies(uint64_t blocks) {
 // Workgroups of the coarse binning (= rows of its counter table): enough to fill the GPU,
 // fewer when many blocks would make the table long.
 constexpr uint64_t kCoarseTable = 1ull << 19;          // entries of the [workgroup][block] table aimed at
-constexpr uint64_t kCoarseTableBlockSort = 1ull << 22; // with the block sort's depth slabs
+constexpr uint64_t kCoarseTableBlockSort = 1ull << 23; // with the block sort's depth slabs
 static uint32_t coarse_workgroups(uint64_t total, uint64_t blocks, uint64_t table) {
     uint64_t wgs = table / (blocks ? blocks : 1);
     // (with the block sort's lists a workgroup flushes thousands of counters with an atomic each:
     // measured on a 1080p frame of 1M Gaussians, the intersection takes 0.228 / 0.219 / 0.240 ms
-    // with 512 / 256 / 128 workgroups)
+    // with 512 / 256 / 128 workgroups; a workgroup per compute unit also where the lists are
+    // many -- six cameras' 24480 lists: 2.43 ms a frame with 171 workgroups, 2.25 with 256; a 4M
+    // frame's 32640 lists: 1.06 against 0.96 ms)
     if (wgs > (table == kCoarseTableBlockSort ? 256u : 512u)) wgs = table == kCoarseTableBlockSort ? 256 : 512;
     if (wgs < 64) wgs = 64;
     const uint64_t needed = (total + kCoarseThreads - 1) / kCoarseThreads;
