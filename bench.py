@@ -612,6 +612,9 @@ def main():
     ap.add_argument("--no-lidar", action="store_true")
     ap.add_argument("--no-bwd", action="store_true", help="skip the forward + backward timing")
     ap.add_argument("--no-configs", action="store_true", help="skip the legs for configs[0] and configs[3]")
+    ap.add_argument("--only-configs", action="store_true",
+                    help="run the legs for configs[0] and configs[3] alone and print their JSON object "
+                         "(what the kernel trace of the six-camera rig under profiles/ was made with)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (known HBM traffic, used "
                          "to scale FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -632,6 +635,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.only_configs:
+        print(json.dumps({"configs": bench_configs(args)}))
+        return
     cam = bench_camera(args)
     lid = None if args.no_lidar else bench_lidar(args)
     achieved = cam["alg_bytes"] / (cam["kernel_ms"] * 1e-3) / 1e9
@@ -715,8 +721,8 @@ def main():
     if not args.no_bwd:
         bwd = bench_backward(args)
         out["backward"] = {k: round(v, 4) for k, v in bwd.items()}
-        for key, kernel in (("camera_rasterize_bwd_ms", "rasterize_bwd_kernel<4, false, 2>"),
-                            ("lidar_rasterize_bwd_ms", "rasterize_bwd_kernel<33, true, 1>")):
+        for key, kernel in (("camera_rasterize_bwd_ms", "rasterize_bwd_kernel<4, false, 2, false>"),
+                            ("lidar_rasterize_bwd_ms", "rasterize_bwd_kernel<33, true, 1, true>")):
             # (the timed interval also holds the clearing and unpacking launches around the kernel)
             r = valu_roofline(counters, kernel, bwd[key])
             if r is not None:
