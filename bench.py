@@ -519,6 +519,18 @@ def bench_configs(args):
                 "visible_rows": int((meta["radii"][..., 0] > 0).sum().item()),
                 "stage_ms": {k: round(v, 4) for k, v in stages.items()}}
 
+    if args.only_configs == "rig":
+        with torch.no_grad():
+            s = workloads.to_device(workloads.camera_driving(n=2 * args.n, n_cameras=6), dev)
+            run = lambda: rasterization(
+                s["means"], s["quats"], s["scales"], s["opacities"], s["colors"], s["velocities"],
+                s["viewmats"], s["Ks"], s["width"], s["height"], s["linear_velocity"],
+                s["angular_velocity"], s["rolling_shutter_time"], sh_degree=s["sh_degree"],
+                packed=False, render_mode="RGB+D", near_plane=s["near_plane"],
+                far_plane=s["far_plane"], eps2d=s["eps2d"], tile_size=s["tile_size"])
+            sec = time_steps(run, steps, warmup)
+            return {"config3_cameras": {"ms": sec * 1e3, "steps": steps, "warmup": warmup,
+                                        "n_isects": int(run()[2]["flatten_ids"].shape[0])}}
     with torch.no_grad():
         s = workloads.to_device(workloads.camera_small(), dev)
         out["config0"] = camera_leg(s, "10000 Gaussians, 320x240, RGB, no rolling shutter (BASELINE configs[0])", "RGB")
@@ -612,9 +624,10 @@ def main():
     ap.add_argument("--no-lidar", action="store_true")
     ap.add_argument("--no-bwd", action="store_true", help="skip the forward + backward timing")
     ap.add_argument("--no-configs", action="store_true", help="skip the legs for configs[0] and configs[3]")
-    ap.add_argument("--only-configs", action="store_true",
-                    help="run the legs for configs[0] and configs[3] alone and print their JSON object "
-                         "(what the kernel trace of the six-camera rig under profiles/ was made with)")
+    ap.add_argument("--only-configs", nargs="?", const="all", default=None, choices=["all", "rig"],
+                    help="run the legs for configs[0] and configs[3] alone and print their JSON object; "
+                         "'rig' runs only the unpacked six-camera call of configs[3] (what the kernel "
+                         "trace of the rig under profiles/ was made with)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (known HBM traffic, used "
                          "to scale FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")

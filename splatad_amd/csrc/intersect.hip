@@ -12,6 +12,9 @@
 //      scan of the tile counts in between gives every tile's segment in the output;
 //   3. one workgroup per tile sorts its segment of (depth bits, flatten id) pairs in LDS and
 //      writes the final 64-bit keys and the ids.
+// Camera frames replace steps 2 and 3 by a sort of the coarse lists themselves (cut into depth
+// slabs), from which the tile lists are written in order ("Cameras: the coarse lists are
+// sorted" below); lidar sweeps, and frames with a coarse list too long for that, keep them.
 // A stable sort by (camera, tile, depth) with ties kept in emission order equals a sort
 // by (camera, tile, depth, flatten id), because the emission loop visits flatten ids in
 // ascending order; that is what makes the unordered binning legal.  Depths must have a
