@@ -469,7 +469,9 @@ int splatad_rasterize_to_pixels_bwd(uint32_t C, int64_t n_isects, uint32_t chann
  * behind ([rows, 4], of which `channels` = 4 are composited; for 3 channels hand over a
  * contiguous [rows, 3] copy).  Rows that no tile staged hold NaN there; no pixel composited
  * them, their gradient is zero, and the kernel takes their colour as zero.  v_colors then goes
- * to splatad_view_colors_bwd. */
+ * to splatad_view_colors_bwd.  v_depths (may be NULL; with channels = 4 only): [rows] floats,
+ * cleared by the caller, that receive the gradient of the fourth channel, the depth, instead
+ * of v_colors[.., 3] -- the contiguous array the projection's backward call takes. */
 int splatad_rasterize_to_pixels_bwd_sh(uint32_t C, int64_t n_isects, uint32_t channels,
                                     const float *means2d, const float *conics,
                                     const float *colors, const float *opacities,
@@ -481,9 +483,9 @@ int splatad_rasterize_to_pixels_bwd_sh(uint32_t C, int64_t n_isects, uint32_t ch
                                     const float *render_alphas, const int32_t *last_ids,
                                     const float *v_render_colors, const float *v_render_alphas,
                                     float *v_means2d_abs, float *v_means2d, float *v_conics,
-                                    float *v_colors, float *v_opacities, float *v_pix_vels,
-                                    uint64_t total, void *workspace, size_t workspace_bytes,
-                                    splatad_stream_t stream);
+                                    float *v_colors, float *v_depths, float *v_opacities,
+                                    float *v_pix_vels, uint64_t total, void *workspace,
+                                    size_t workspace_bytes, splatad_stream_t stream);
 
 /* rasterize_to_points_fwd_tensor, rasterization.cu:2221-2831 (kernel
  * :2021-2219).  Outputs of inactive points (range <= 0) are zero.

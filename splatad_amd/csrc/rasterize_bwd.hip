@@ -304,7 +304,7 @@ rasterize_bwd_kernel(BwdArgs a) {
     if (lane < CH) {
         if ((uint32_t)lane < a.n_ch) {
             const uint32_t c = a.ch_offset + lane;
-            if (LIDAR && a.v_range != nullptr && c == a.depth_idx) { slot_base = a.v_range; slot_stride = 1; }
+            if (a.v_range != nullptr && c == a.depth_idx) { slot_base = a.v_range; slot_stride = 1; }
             else { slot_base = a.v_colors + c; slot_stride = a.feat_stride; }
         }
     } else if (lane < ACC) {
@@ -529,7 +529,7 @@ unpack_gradients_kernel(uint64_t total, uint32_t stride, uint32_t width, BwdArgs
     if (slot < width) {
         if (slot < a.n_ch) {
             const uint32_t c = a.ch_offset + slot;
-            if (LIDAR && a.v_range != nullptr && c == a.depth_idx) a.v_range[g] += val;
+            if (a.v_range != nullptr && c == a.depth_idx) a.v_range[g] += val;
             else a.v_colors[g * a.feat_stride + c] += val;
         }
         return;
@@ -674,7 +674,7 @@ static int pixels_bwd(int colors_from_cache,
     uint32_t tile_h, const int32_t *tile_offsets, const int32_t *flatten_ids,
     const float *render_alphas, const int32_t *last_ids, const float *v_render_colors,
     const float *v_render_alphas, float *v_means2d_abs, float *v_means2d, float *v_conics,
-    float *v_colors, float *v_opacities, float *v_pix_vels, uint64_t total, void *workspace,
+    float *v_colors, float *v_depths, float *v_opacities, float *v_pix_vels, uint64_t total, void *workspace,
     size_t workspace_bytes, splatad_stream_t stream) {
     SPLATAD_REQUIRE(channels >= 1, "rasterize_to_pixels bwd: zero channels");
     SPLATAD_REQUIRE(tile_size >= 1 && tile_size * tile_size <= 256,
@@ -698,6 +698,8 @@ static int pixels_bwd(int colors_from_cache,
     a.v_render_colors = v_render_colors; a.v_render_alphas = v_render_alphas;
     a.v_means2d_abs = v_means2d_abs; a.v_means2d = v_means2d; a.v_conics = v_conics;
     a.v_colors = v_colors; a.v_opacities = v_opacities; a.v_pix_vels = v_pix_vels;
+    // the last channel's gradient in an array of its own (the depth channel of a colour cache row)
+    a.v_range = v_depths; a.depth_idx = channels - 1;
     return run_passes<false>(a, channels, dim3(C * tile_w * tile_h),
                              dim3((tile_size * tile_size + 63) / 64 * 64), total, workspace,
                              workspace_bytes, (hipStream_t)stream);
@@ -715,7 +717,7 @@ extern "C" int splatad_rasterize_to_pixels_bwd(
     return pixels_bwd(0, C, n_isects, channels, means2d, conics, colors, opacities, pix_vels, rs_time,
                       backgrounds, W, H, tile_size, tile_w, tile_h, tile_offsets, flatten_ids,
                       render_alphas, last_ids, v_render_colors, v_render_alphas, v_means2d_abs, v_means2d,
-                      v_conics, v_colors, v_opacities, v_pix_vels, total, workspace, workspace_bytes,
+                      v_conics, v_colors, nullptr, v_opacities, v_pix_vels, total, workspace, workspace_bytes,
                       stream);
 }
 
@@ -726,12 +728,14 @@ extern "C" int splatad_rasterize_to_pixels_bwd_sh(
     uint32_t tile_h, const int32_t *tile_offsets, const int32_t *flatten_ids,
     const float *render_alphas, const int32_t *last_ids, const float *v_render_colors,
     const float *v_render_alphas, float *v_means2d_abs, float *v_means2d, float *v_conics,
-    float *v_colors, float *v_opacities, float *v_pix_vels, uint64_t total, void *workspace,
+    float *v_colors, float *v_depths, float *v_opacities, float *v_pix_vels, uint64_t total, void *workspace,
     size_t workspace_bytes, splatad_stream_t stream) {
+    SPLATAD_REQUIRE(v_depths == nullptr || channels == 4,
+                    "rasterize_to_pixels bwd: v_depths goes with the four channels of a colour cache row");
     return pixels_bwd(1, C, n_isects, channels, means2d, conics, colors, opacities, pix_vels, rs_time,
                       backgrounds, W, H, tile_size, tile_w, tile_h, tile_offsets, flatten_ids,
                       render_alphas, last_ids, v_render_colors, v_render_alphas, v_means2d_abs, v_means2d,
-                      v_conics, v_colors, v_opacities, v_pix_vels, total, workspace, workspace_bytes,
+                      v_conics, v_colors, v_depths, v_opacities, v_pix_vels, total, workspace, workspace_bytes,
                       stream);
 }
 

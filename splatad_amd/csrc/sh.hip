@@ -195,16 +195,13 @@ sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, ShView view, const float
     // every lane writes its row of coefficient gradients to LDS, from where the workgroup
     // stores them coalesced; rows of masked directions are zeros (their gradients are zero)
     float *row = s_rows + (size_t)threadIdx.x * (rows.used + 1);
+    float dx = 0.f, dy = 0.f, dz = 0.f, vr = 0.f, vg = 0.f, vb = 0.f;
+    size_t coeff_row = 0;
+    bool active = false;
     if (e < n) {
-        float dx = 0.f, dy = 0.f, dz = 0.f;
-        size_t coeff_row;
-        const bool active = sh_row<VIEW>(e, view, dirs, masks, dx, dy, dz, coeff_row);
-        if (scatter) s_dest[threadIdx.x] = (uint32_t)coeff_row;
-        const float *cf = coeffs + coeff_row * rows.K3;
-        const float inorm = active ? rsqrtf(dx * dx + dy * dy + dz * dz) : 0.f;
-        const float x = dx * inorm, y = dy * inorm, z = active ? dz * inorm : 1.f;
+        active = sh_row<VIEW>(e, view, dirs, masks, dx, dy, dz, coeff_row);
         const float *vc = v_colors + (size_t)e * stride;
-        float vr = vc[0], vg = vc[1], vb = vc[2]; // read whether active or not: no wait for the test
+        vr = vc[0]; vg = vc[1]; vb = vc[2]; // read whether active or not: no wait for the test
         if (VIEW) {
             const float *col = colors + (size_t)e * stride;
             vr = col[0] > 0.f ? vr : 0.f;
@@ -212,6 +209,30 @@ sh_bwd_kernel(uint32_t n, ShRows rows, uint32_t degree, ShView view, const float
             vb = col[2] > 0.f ? vb : 0.f;
         }
         if (!active) vr = vg = vb = 0.f;
+    }
+    // A workgroup none of whose rows takes a gradient (rows that no pixel composited: most rows
+    // of a frame that saturates in its nearest Gaussians) only has zeros to write, and writes
+    // them without evaluating a basis or passing through LDS.
+    if (!__syncthreads_or(vr != 0.f || vg != 0.f || vb != 0.f)) {
+        if (DIRS && e < n && (active || VIEW))
+            v_dirs[(size_t)e * 3] = v_dirs[(size_t)e * 3 + 1] = v_dirs[(size_t)e * 3 + 2] = 0.f;
+        if (scatter) return; // nothing to add
+        float *gout = v_coeffs + (size_t)first * rows.K3;
+        const uint32_t total = here * rows.K3;
+        if (rows.used == rows.K3 && (reinterpret_cast<uintptr_t>(gout) & 15) == 0) {
+            float4 *g4 = reinterpret_cast<float4 *>(gout);
+            for (uint32_t i = threadIdx.x; i < total / 4; i += blockDim.x) g4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (uint32_t i = (total & ~3u) + threadIdx.x; i < total; i += blockDim.x) gout[i] = 0.f;
+        } else {
+            sh_for_each_float(rows, here, [&](uint32_t, uint32_t f, uint32_t, uint32_t) { gout[f] = 0.f; });
+        }
+        return;
+    }
+    if (e < n) {
+        if (scatter) s_dest[threadIdx.x] = (uint32_t)coeff_row;
+        const float *cf = coeffs + coeff_row * rows.K3;
+        const float inorm = active ? rsqrtf(dx * dx + dy * dy + dz * dz) : 0.f;
+        const float x = dx * inorm, y = dy * inorm, z = active ? dz * inorm : 1.f;
         float gx = 0.f, gy = 0.f, gz = 0.f;
         // the whole coefficient row is requested before the first use, one memory round trip
         // instead of one per degree

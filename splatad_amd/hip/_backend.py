@@ -24,7 +24,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libsplatad_hip.so")
 _lib = None
 
 
-ABI_VERSION = 7  # splatad_abi_version() of the library these bindings were written for
+ABI_VERSION = 8  # splatad_abi_version() of the library these bindings were written for
 
 
 def load_library():
@@ -962,7 +962,9 @@ class _Ops:
                                 tile_size, tile_offsets, flatten_ids, render_alphas, last_ids,
                                 v_render_colors, v_render_alphas, absgrad, colors_from_cache=False):
         """colors_from_cache: `colors` is the colour cache rasterize_to_pixels_sh_fwd left behind
-        (NaN rows = never staged, taken as zero)."""
+        (NaN rows = never staged, taken as zero); with its four channels the gradient of the
+        fourth, the depth, comes back as a seventh, contiguous tensor of one value per row (what
+        the projection's backward pass takes) and v_colors[..., 3] stays zero."""
         lib = load_library()
         means2d = _in(means2d, "means2d"); conics = _in(conics, "conics")
         colors = _in(colors, "colors"); opacities = _in(opacities, "opacities")
@@ -976,21 +978,28 @@ class _Ops:
         v_render_alphas = _in(v_render_alphas, "v_render_alphas")
         C, th, tw = tile_offsets.shape
         D, dev = colors.shape[-1], means2d.device
-        v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_means2d_abs = _zeros_like_many(
-            means2d, conics, colors, opacities, pix_vels, means2d if absgrad else None)
+        split_depth = colors_from_cache and D == 4
+        v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_means2d_abs, v_depths = _zeros_like_many(
+            means2d, conics, colors, opacities, pix_vels, means2d if absgrad else None,
+            opacities if split_depth else None)
         if flatten_ids.shape[0]:
             total = means2d.numel() // 2
             with _on(dev):
                 ws = _bwd_workspace(lib, total, D, False, dev)
-                entry = lib.splatad_rasterize_to_pixels_bwd_sh if colors_from_cache else lib.splatad_rasterize_to_pixels_bwd
-                _check(entry(
-                    _u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics),
-                    _p(colors), _p(opacities), _p(pix_vels), _p(rs), _p(backgrounds),
-                    _u32(image_width), _u32(image_height), _u32(tile_size), _u32(tw), _u32(th),
-                    _p(tile_offsets), _p(flatten_ids), _p(render_alphas), _p(last_ids),
-                    _p(v_render_colors), _p(v_render_alphas), _p(v_means2d_abs), _p(v_means2d),
-                    _p(v_conics), _p(v_colors), _p(v_opacities), _p(v_pix_vels), _u64(total), _p(ws),
-                    ctypes.c_size_t(0 if ws is None else ws.numel()), _stream(dev)))
+                head = (_u32(C), _i64(flatten_ids.shape[0]), _u32(D), _p(means2d), _p(conics),
+                        _p(colors), _p(opacities), _p(pix_vels), _p(rs), _p(backgrounds),
+                        _u32(image_width), _u32(image_height), _u32(tile_size), _u32(tw), _u32(th),
+                        _p(tile_offsets), _p(flatten_ids), _p(render_alphas), _p(last_ids),
+                        _p(v_render_colors), _p(v_render_alphas), _p(v_means2d_abs), _p(v_means2d),
+                        _p(v_conics), _p(v_colors))
+                tail = (_p(v_opacities), _p(v_pix_vels), _u64(total), _p(ws),
+                        ctypes.c_size_t(0 if ws is None else ws.numel()), _stream(dev))
+                if colors_from_cache:
+                    _check(lib.splatad_rasterize_to_pixels_bwd_sh(*head, _p(v_depths), *tail))
+                else:
+                    _check(lib.splatad_rasterize_to_pixels_bwd(*head, *tail))
+        if split_depth:
+            return v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities, v_pix_vels, v_depths
         return v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities, v_pix_vels
 
     def rasterize_to_points_fwd(self, means2d, conics, colors, opacities, pix_vels,

@@ -40,6 +40,9 @@ class _NoGradContext:
     def mark_non_differentiable(self, *tensors):
         pass
 
+    def set_materialize_grads(self, value):
+        pass
+
 
 def _apply(function, *args):
     """`function.apply(*args)`, or just its forward when gradients are switched off or no
@@ -728,6 +731,13 @@ def _gate(grads, needs):
     return tuple(g if n else None for g, n in zip(grads, needs))
 
 
+def _given(v: Optional[Tensor], like: Tensor, *last) -> Tensor:
+    """The incoming gradient, contiguous, or zeros of shape like.shape[:-1] + last where autograd
+    has none.  (The projections switch off autograd's own zero-filling of absent gradients: it
+    would also clear a tensor for the integer radii on every backward pass.)"""
+    return torch.zeros(like.shape[:-1] + last, dtype=torch.float32, device=like.device) if v is None else v.contiguous()
+
+
 class _FullyFusedProjection(torch.autograd.Function):
     @staticmethod
     def forward(ctx, means, covars, quats, scales, velocities, viewmats, Ks, width, height,
@@ -745,6 +755,7 @@ class _FullyFusedProjection(torch.autograd.Function):
                               conics, compensations)
         ctx.width, ctx.height, ctx.eps2d = width, height, eps2d
         ctx.mark_non_differentiable(radii)
+        ctx.set_materialize_grads(False)
         return radii, means2d, depths, conics, compensations, pix_vels
 
     @staticmethod
@@ -755,8 +766,8 @@ class _FullyFusedProjection(torch.autograd.Function):
         out = _make_lazy_hip_func("fully_fused_projection_bwd")(
             means, covars, quats, scales, velocities, viewmats, Ks, ctx.width, ctx.height,
             linear_velocity, angular_velocity, rolling_shutter_time, ctx.eps2d, radii, conics,
-            compensations, v_means2d.contiguous(), v_depths.contiguous(), v_conics.contiguous(),
-            _c(v_compensations), v_pix_vels.contiguous(), ctx.needs_input_grad[5], want_vel)
+            compensations, _given(v_means2d, conics, 2), _given(v_depths, conics), _given(v_conics, conics, 3),
+            _c(v_compensations), _given(v_pix_vels, conics, 2), ctx.needs_input_grad[5], want_vel)
         v_means, v_covars, v_quats, v_scales, v_viewmats = out[:5]
         v_velocities = out[5] if want_vel else None
         grads = _gate((v_means, v_covars, v_quats, v_scales, v_velocities, v_viewmats),
@@ -783,6 +794,7 @@ class _FullyFusedLidarProjection(torch.autograd.Function):
         ctx.bounds = (min_elevation, max_elevation, min_azimuth, max_azimuth)
         ctx.eps2d = eps2d
         ctx.mark_non_differentiable(radii)
+        ctx.set_materialize_grads(False)
         return radii, means2d, depths, conics, compensations, pix_vels, depth_compensations
 
     @staticmethod
@@ -794,8 +806,8 @@ class _FullyFusedLidarProjection(torch.autograd.Function):
         out = _make_lazy_hip_func("fully_fused_lidar_projection_bwd")(
             means, covars, quats, scales, velocities, viewmats, *ctx.bounds, linear_velocity,
             angular_velocity, rolling_shutter_time, ctx.eps2d, radii, conics, compensations,
-            v_means2d.contiguous(), v_depths.contiguous(), v_conics.contiguous(),
-            _c(v_compensations), v_pix_vels.contiguous(), v_depth_compensations.contiguous(),
+            _given(v_means2d, conics, 2), _given(v_depths, conics), _given(v_conics, conics, 3),
+            _c(v_compensations), _given(v_pix_vels, conics, 3), _given(v_depth_compensations, conics, 2),
             ctx.needs_input_grad[5], want_vel)
         v_means, v_covars, v_quats, v_scales, v_viewmats = out[:5]
         v_velocities = out[5] if want_vel else None
@@ -822,6 +834,7 @@ class _FullyFusedProjectionPacked(torch.autograd.Function):
                               rolling_shutter_time, conics, compensations, pix_vels)
         ctx.width, ctx.height, ctx.eps2d, ctx.sparse_grad = width, height, eps2d, sparse_grad
         ctx.mark_non_differentiable(camera_ids, gaussian_ids, radii)
+        ctx.set_materialize_grads(False)
         return camera_ids, gaussian_ids, radii, means2d, depths, conics, compensations, pix_vels
 
     @staticmethod
@@ -835,9 +848,9 @@ class _FullyFusedProjectionPacked(torch.autograd.Function):
         out = _make_lazy_hip_func("fully_fused_projection_packed_bwd")(
             means, covars, quats, scales, velocities, viewmats, Ks, ctx.width, ctx.height,
             linear_velocity, angular_velocity, rolling_shutter_time, ctx.eps2d, camera_ids,
-            gaussian_ids, conics, compensations, pix_vels, v_means2d.contiguous(),
-            v_depths.contiguous(), v_conics.contiguous(), _c(v_compensations),
-            v_pix_vels.contiguous(), ctx.needs_input_grad[5], sparse_grad, want_vel)
+            gaussian_ids, conics, compensations, pix_vels, _given(v_means2d, conics, 2),
+            _given(v_depths, conics), _given(v_conics, conics, 3), _c(v_compensations),
+            _given(v_pix_vels, conics, 2), ctx.needs_input_grad[5], sparse_grad, want_vel)
         v_means, v_covars, v_quats, v_scales, v_viewmats = out[:5]
         v_velocities = out[5] if want_vel else None
 
@@ -1210,8 +1223,10 @@ class _RasterizeToPixelsWithSH(torch.autograd.Function):
         # are read by no pixel that composited them, and count as zero in both kernels below
         # (the SH backward only asks whether a colour is positive)
         colors = cache if ctx.has_depths else cache[..., :3].contiguous()
-        (v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities,
-         v_pix_vels) = _make_lazy_hip_func("rasterize_to_pixels_bwd")(
+        # (with the depth channel: its gradient as a contiguous tensor of its own, which the
+        # projection's backward pass takes as it is)
+        (v_means2d_abs, v_means2d, v_conics, v_colors, v_opacities, v_pix_vels,
+         *v_depth_channel) = _make_lazy_hip_func("rasterize_to_pixels_bwd")(
             means2d, conics, colors, opacities, pix_vels, rolling_shutter_time, backgrounds,
             ctx.width, ctx.height, ctx.tile_size, isect_offsets, flatten_ids, render_alphas,
             last_ids, v_render_colors.contiguous(), v_render_alphas.contiguous(), ctx.absgrad,
@@ -1221,7 +1236,7 @@ class _RasterizeToPixelsWithSH(torch.autograd.Function):
         v_means, v_coeffs = _view_colors_backward(
             ctx.sh_degree, means, viewmats, coeffs, radii, camera_ids, gaussian_ids, colors, v_colors,
             ctx.needs_input_grad[1], ctx.needs_input_grad[3])
-        v_depths = v_colors[..., 3] if ctx.has_depths and ctx.needs_input_grad[4] else None
+        v_depths = v_depth_channel[0] if ctx.has_depths and ctx.needs_input_grad[4] else None
         v_backgrounds = None
         if ctx.needs_input_grad[13]:
             v_backgrounds = (v_render_colors * (1.0 - render_alphas).float()).sum(dim=(1, 2))

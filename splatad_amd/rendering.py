@@ -213,7 +213,9 @@ def rasterization(
     opacities_per_gaussian = opacities
 
     def per_row_opacities():
-        o = opacities_per_gaussian.index_select(0, gaussian_ids) if packed else opacities_per_gaussian.expand(C, -1)
+        # (one sensor: a view whose backward is a view; expand's is a sum, a kernel even over one row)
+        o = (opacities_per_gaussian.index_select(0, gaussian_ids) if packed
+             else opacities_per_gaussian[None] if C == 1 else opacities_per_gaussian.expand(C, -1))
         return o if compensations is None else o * compensations
 
     if "opacities" in beside.results:
