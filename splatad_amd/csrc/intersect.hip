@@ -1510,6 +1510,7 @@ isect_small_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t 
 constexpr uint32_t kBlockSortCap = 10240;   // longest (block, slab) list the LDS sort takes
 constexpr uint32_t kBlockMergeCap = 4096;   // slabs of a block are sorted together up to this many entries,
 constexpr uint32_t kBlockPairsCap = 32768;  // and about this many intersections
+static_assert(kBlockMergeCap <= 4096, "classes beyond 4096 entries hold single lists only: the host skips their launches by the longest list");
 constexpr uint32_t kBlockLongMax = 8 * kBlockSortCap; // longest list the block sort takes at all (in parts)
 constexpr int kBlockClasses = 6;            // five by length, and the lists beyond kBlockSortCap
 constexpr int kBlockLongClass = 5;
@@ -2768,8 +2769,8 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
     if ((rc = isect_device(&ss)) != 0) return rc;
     const uint32_t nseg = (uint32_t)segs;
     bool short_lists = false;
+    unsigned long long longest_list = 0;
     if (pl.block_sort) {
-        unsigned long long longest_list = 0;
         if ((rc = host_word_wait(&longest, "isect", &longest_list)) != 0) return rc;
         short_lists = longest_list <= kBlockLongMax;
     }
@@ -2799,13 +2800,16 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                                            w.seg_starts, w.list_tile_counts, isect_ids, flatten_ids, on)) != 0)  \
                 return e;
             // (the lists too long for one LDS sort first: a workgroup each, part by part)
-            if ((e = launch_block_sort<10, true>(kBlockLongClass, 1024, kBlockSortCap, 256u, (uint32_t)pl.blocks, cg,
+            // Pieces beyond kBlockMergeCap entries are single lists, so the longest list tells
+            // which of the upper classes are empty: their launches (5 us each on the way) are left out.
+            if (longest_list > kBlockSortCap &&
+                (e = launch_block_sort<10, true>(kBlockLongClass, 1024, kBlockSortCap, 256u, (uint32_t)pl.blocks, cg,
                                                  g.tile_w, g.tile_h, n_tiles, tile_n_bits, n_isects,
                                                  w.piece_counts, w.pieces, w.entries, w.seg_starts,
                                                  w.list_tile_counts, isect_ids, flatten_ids, stream)) != 0)
                 return e;
-            SPLATAD_BLOCK_CLASS(4, 10, 1024, kBlockSortCap, 256u, stream)
-            SPLATAD_BLOCK_CLASS(3, 8, 1024, 8192u, 256u, ss->aux[1])
+            if (longest_list > 8192u) SPLATAD_BLOCK_CLASS(4, 10, 1024, kBlockSortCap, 256u, stream)
+            if (longest_list > 4096u) SPLATAD_BLOCK_CLASS(3, 8, 1024, 8192u, 256u, ss->aux[1])
             SPLATAD_BLOCK_CLASS(2, 8, 512, 4096u, 512u, ss->aux[0])
             SPLATAD_BLOCK_CLASS(1, 8, 256, 2048u, 1024u, stream)
             SPLATAD_BLOCK_CLASS(0, 4, 128, 512u, 2048u, ss->aux[1])

@@ -102,3 +102,40 @@ def test_view_colors_packed(per_sensor):
     g_ref = torch.autograd.grad((ref * w).sum(), ref_leaves)
     for name, a, b in zip(("means", "coeffs", "depths"), g, g_ref):
         assert_grad_close(to_np(a), to_np(b), name)
+
+
+@pytest.mark.parametrize("C,degree,K,packed", [(1, 3, 16, False), (2, 2, 16, False), (2, 3, 16, True)])
+def test_view_colors_gradients_where_stretches_of_rows_take_none(C, degree, K, packed):
+    """Rows that no pixel composited have a zero colour gradient; a workgroup (256 rows) that
+    holds only such rows writes its zeros on a path of its own.  The cotangent here is zero on
+    stretches longer than a workgroup, beside stretches that are not; also with fewer bases in
+    use than the coefficient rows hold (degree 2 of 16)."""
+    from splatad_amd.hip._wrapper import view_dependent_colors
+    N = 3000
+    means, viewmats, coeffs, radii, depths = _scene(C, N, K, 71 + degree, False)
+    radii[...] = np.maximum(radii, 1)
+    vm = to_dev(viewmats)
+    if packed:
+        cam, gid = np.nonzero(radii[..., 0] > 0)
+        rd, dp = radii[cam, gid], depths[cam, gid]
+        ids = (to_dev(cam), to_dev(gid))
+    else:
+        rd, dp, ids = radii, depths, ()
+    rd_t = to_dev(rd)
+    leaves = [to_dev(a).requires_grad_() for a in (means, coeffs, dp)]
+    ref_leaves = [to_dev(a).requires_grad_() for a in (means, coeffs, dp)]
+    out = view_dependent_colors(degree, leaves[0], vm, leaves[1], rd_t, leaves[2], *ids)
+    ref = _chain(degree, ref_leaves[0], vm, ref_leaves[1], rd_t, ref_leaves[2], *ids)
+    w = np.random.default_rng(5).normal(size=tuple(out.shape)).astype(np.float32)
+    flat = w.reshape(-1, w.shape[-1])
+    flat[:700, :3] = 0
+    flat[1500:2300, :3] = 0
+    flat[2600:, :3] = 0  # the last, partial workgroup
+    w = to_dev(w)
+    g = torch.autograd.grad((out * w).sum(), leaves)
+    g_ref = torch.autograd.grad((ref * w).sum(), ref_leaves)
+    for name, a, b in zip(("means", "coeffs", "depths"), g, g_ref):
+        assert_grad_close(to_np(a), to_np(b), name)
+    if not packed and C == 1:  # rows without a gradient get exact zeros
+        assert (to_np(g[1])[:700] == 0).all() and (to_np(g[1])[1500:2300] == 0).all()
+        assert (to_np(g[0])[:700] == 0).all()
