@@ -1587,31 +1587,61 @@ isect_tile_totals_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32
 // where the entries meet many tiles each, so that a piece writes about kBlockPairsCap
 // intersections at most; a single slab's list beyond that is a piece of its own), and lists the
 // pieces by size class: class c's are pieces[c * max_pieces ..] , class_count[c] of them.  The
-// other workgroups turn the scanned tile counts into the tiles' starts (seg_starts) and the
-// tile offsets.
+// other workgroups scan the tile counts into the tiles' starts (seg_starts) and the tile
+// offsets: each takes a stretch of the tiles and adds up, for itself, the counts of all tiles
+// before it (a few thousand to some ten thousand words from L2: cheaper than a scan launch in
+// the chain of dependent kernels).
 __global__ void __launch_bounds__(1024)
 isect_block_plan_kernel(uint32_t n_blocks, uint32_t bsshift, const int32_t *__restrict__ totals,
                         const uint32_t *__restrict__ list_starts, const int32_t *__restrict__ tile_counts,
-                        CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t n_segments, uint32_t copies, const int32_t *__restrict__ tile_starts,
-                        const int64_t *__restrict__ scan_totals, uint32_t n_scan_blocks,
+                        CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t n_segments,
                         int32_t *__restrict__ seg_starts, int32_t *__restrict__ tile_offsets,
                         uint32_t *__restrict__ class_count, uint32_t max_pieces,
                         uint4 *__restrict__ pieces) {
     const uint32_t tid = threadIdx.x, nt = blockDim.x, lane = tid & (SPLATAD_WAVE - 1);
     if (blockIdx.x != 0) { // uniform across the workgroup
-        ScanBlocks scan;
-        scan.request(scan_totals, n_scan_blocks, lane);
-        scan.sum(lane);
-        const uint32_t per_round = (gridDim.x - 1) * nt;
-        for (uint32_t s0 = (blockIdx.x - 1) * nt + (tid & ~(SPLATAD_WAVE - 1u)); s0 < n_segments; s0 += per_round) {
-            const uint32_t seg = s0 + lane;
-            // the first copy of segment s is logical element s * copies of the scanned table
-            const int32_t before = scan.before(min(seg, n_segments - 1u) * copies);
-            if (seg < n_segments) {
-                const int32_t start = tile_starts[seg] + before;
+        __shared__ uint32_t s_wave[1024 / SPLATAD_WAVE];
+        const uint32_t workers = gridDim.x - 1, wave = tid / SPLATAD_WAVE, n_waves = nt / SPLATAD_WAVE;
+        const uint32_t per = ((n_segments + workers - 1) / workers + nt - 1) / nt * nt; // whole rounds of the workgroup
+        const uint32_t lo = min(n_segments, (blockIdx.x - 1) * per), hi = min(n_segments, lo + per);
+        if (lo >= hi) return;
+        // the counts before the stretch (lo is a multiple of the workgroup size: whole int4)
+        uint32_t sum = 0;
+        const int4 *counts4 = reinterpret_cast<const int4 *>(tile_counts);
+        for (uint32_t i = tid; i < lo / 4; i += nt) {
+            const int4 v = counts4[i];
+            sum += (uint32_t)(v.x + v.y + v.z + v.w);
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, SPLATAD_WAVE);
+        if (lane == 0) s_wave[wave] = sum;
+        __syncthreads();
+        uint32_t before = 0;
+        for (uint32_t k = 0; k < n_waves; ++k) before += s_wave[k];
+        for (uint32_t s0 = lo; s0 < hi; s0 += nt) { // uniform
+            const uint32_t seg = s0 + tid;
+            const uint32_t mine = seg < hi ? (uint32_t)tile_counts[seg] : 0u;
+            uint32_t incl = mine;
+#pragma unroll
+            for (int off = 1; off < SPLATAD_WAVE; off <<= 1) {
+                const uint32_t up = __shfl_up(incl, off, SPLATAD_WAVE);
+                if (lane >= (uint32_t)off) incl += up;
+            }
+            __syncthreads(); // the totals of the round before have been read
+            if (lane == SPLATAD_WAVE - 1) s_wave[wave] = incl;
+            __syncthreads();
+            uint32_t waves_before = 0, round = 0;
+            for (uint32_t k = 0; k < n_waves; ++k) {
+                const uint32_t v = s_wave[k];
+                if (k < wave) waves_before += v;
+                round += v;
+            }
+            if (seg < hi) {
+                const int32_t start = (int32_t)(before + waves_before + incl - mine);
                 seg_starts[seg] = start;
                 if (tile_offsets != nullptr) tile_offsets[seg] = start;
             }
+            before += round;
         }
         return;
     }
@@ -2752,19 +2782,6 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                        (int32_t *)nullptr, (const int64_t *)nullptr, 0u, (int32_t *)nullptr,
                        pl.bsshift - sshift);
     SPLATAD_LAUNCH_CHECK();
-    // up to 128 scan blocks, i.e. any table of the size isect_copies() aims at: one scan launch,
-    // and the filling pass adds the blocks before an element itself
-    const int64_t scan_n = (int64_t)(segs * tcopies);
-    const int scan_stride = tcopies > 1 ? -(int)tcopies : 1;
-    uint32_t n_scan_blocks = 0;
-    const bool local_scan = scan_n <= kScanLocalBlocks * SCAN_TILE;
-    if (local_scan)
-        rc = launch_local_scan<int32_t>(w.tile_counts, scan_n, scan_stride, w.tile_starts, w.block_sums,
-                                        &n_scan_blocks, stream);
-    else
-        rc = launch_exclusive_scan<int32_t>(w.tile_counts, scan_n, scan_stride, 0, w.tile_starts,
-                                            w.scan_total, w.block_sums, stream);
-    if (rc) return rc;
     IsectDevice *ss = nullptr;
     if ((rc = isect_device(&ss)) != 0) return rc;
     const uint32_t nseg = (uint32_t)segs;
@@ -2774,6 +2791,22 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         if ((rc = host_word_wait(&longest, "isect", &longest_list)) != 0) return rc;
         short_lists = longest_list <= kBlockLongMax;
     }
+    // up to 128 scan blocks, i.e. any table of the size isect_copies() aims at: one scan launch,
+    // and the filling pass adds the blocks before an element itself (the block sort's planning
+    // kernel scans its tile counts itself)
+    const int64_t scan_n = (int64_t)(segs * tcopies);
+    const int scan_stride = tcopies > 1 ? -(int)tcopies : 1;
+    uint32_t n_scan_blocks = 0;
+    const bool local_scan = scan_n <= kScanLocalBlocks * SCAN_TILE;
+    if (short_lists)
+        rc = 0;
+    else if (local_scan)
+        rc = launch_local_scan<int32_t>(w.tile_counts, scan_n, scan_stride, w.tile_starts, w.block_sums,
+                                        &n_scan_blocks, stream);
+    else
+        rc = launch_exclusive_scan<int32_t>(w.tile_counts, scan_n, scan_stride, 0, w.tile_starts,
+                                            w.scan_total, w.block_sums, stream);
+    if (rc) return rc;
     if (short_lists) {
         // Pieces of the coarse lists by size class, and the tiles' starts; then a launch per
         // class, the long pieces first, beside each other on the caller's stream and two helper
@@ -2783,9 +2816,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         if (plan_wgs > 65) plan_wgs = 65;
         hipLaunchKernelGGL(isect_block_plan_kernel, dim3(plan_wgs), dim3(1024), 0, stream, n_blocks, pl.bsshift,
                            (const int32_t *)w.block_totals, (const uint32_t *)w.list_starts,
-                           (const int32_t *)w.tile_counts, cg, g.tile_w, g.tile_h, nseg, tcopies,
-                           (const int32_t *)w.tile_starts,
-                           local_scan ? (const int64_t *)w.block_sums : (const int64_t *)nullptr, n_scan_blocks,
+                           (const int32_t *)w.tile_counts, cg, g.tile_w, g.tile_h, nseg,
                            w.seg_starts, tile_offsets, w.piece_counts, (uint32_t)pl.blocks, w.pieces);
         SPLATAD_LAUNCH_CHECK();
         std::lock_guard<std::mutex> fork_lock(ss->guard);
