@@ -408,7 +408,7 @@ def lidar_rasterization(
     if packed:
         raise NotImplementedError("Packed mode is not supported for lidar_rasterization")
     radii, means2d, depths, conics, compensations, pix_vels, depth_compensations = proj
-    opacities = opacities.expand(C, -1)  # [C, N], as above
+    opacities = opacities[None] if C == 1 else opacities.expand(C, -1)  # [C, N], as above
     camera_ids, gaussian_ids = None, None
 
     if not use_depth_compensation:
