@@ -1510,7 +1510,12 @@ isect_small_segment_sort_kernel(uint32_t n_segments, uint32_t n_tiles, uint32_t 
 constexpr uint32_t kBlockSortCap = 10240;   // longest (block, slab) list the LDS sort takes
 constexpr uint32_t kBlockMergeCap = 4096;   // slabs of a block are sorted together up to this many entries,
 constexpr uint32_t kBlockPairsCap = 32768;  // and about this many intersections
-static_assert(kBlockMergeCap <= 4096, "classes beyond 4096 entries hold single lists only: the host skips their launches by the longest list");
+// (a lidar's wide tiles: an entry names four tiles on average where a camera's names six, but its
+// lists come out evenly long, and pieces of 4096 entries all fall into one class whose single
+// launch then lasts 100 us: sweep intersection 0.254 ms with the camera's caps, 0.226 with these,
+// 0.238 with the per-tile segment sort)
+constexpr uint32_t kBlockMergeCapLidar = 2048, kBlockPairsCapLidar = 12288;
+static_assert(kBlockMergeCap <= 4096 && kBlockMergeCapLidar <= 4096, "classes beyond 4096 entries hold single lists only: the host skips their launches by the longest list");
 constexpr uint32_t kBlockLongMax = 8 * kBlockSortCap; // longest list the block sort takes at all (in parts)
 constexpr int kBlockClasses = 6;            // five by length, and the lists beyond kBlockSortCap
 constexpr int kBlockLongClass = 5;
@@ -1597,7 +1602,7 @@ isect_block_plan_kernel(uint32_t n_blocks, uint32_t bsshift, const int32_t *__re
                         CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t n_segments,
                         int32_t *__restrict__ seg_starts, int32_t *__restrict__ tile_offsets,
                         uint32_t *__restrict__ class_count, uint32_t max_pieces,
-                        uint4 *__restrict__ pieces) {
+                        uint4 *__restrict__ pieces, uint32_t merge_cap, uint32_t pairs_cap) {
     const uint32_t tid = threadIdx.x, nt = blockDim.x, lane = tid & (SPLATAD_WAVE - 1);
     if (blockIdx.x != 0) { // uniform across the workgroup
         __shared__ uint32_t s_wave[1024 / SPLATAD_WAVE];
@@ -1674,9 +1679,9 @@ isect_block_plan_kernel(uint32_t n_blocks, uint32_t bsshift, const int32_t *__re
 #pragma unroll
         for (uint32_t sl = 0; sl < (1u << kSlabShiftMax); ++sl) block_n += v[sl];
         if (block_n == 0) continue;
-        uint32_t cap = kBlockMergeCap;
-        if (pairs * cap > (uint64_t)kBlockPairsCap * block_n)
-            cap = max(512u, (uint32_t)((uint64_t)kBlockPairsCap * block_n / pairs));
+        uint32_t cap = merge_cap;
+        if (pairs * cap > (uint64_t)pairs_cap * block_n)
+            cap = max(512u, (uint32_t)((uint64_t)pairs_cap * block_n / pairs));
         uint32_t piece_first = block_first, piece_n = 0, piece_list = list0;
         auto emit = [&](uint32_t next_list) {
             if (piece_n != 0) {
@@ -1706,7 +1711,7 @@ isect_block_plan_kernel(uint32_t n_blocks, uint32_t bsshift, const int32_t *__re
 // Sorts one piece (n <= ER * blockDim.x entries, n <= lds_words) in LDS -- sort_segment_small's
 // method, with the tile masks travelling beside the keys -- and writes its share of the lists
 // of the block's sixteen tiles.
-template <int ER>
+template <int ER, bool TIES>
 __device__ __forceinline__ void sort_expand_piece(uint4 piece, CoarseGrid cg, uint32_t tile_w, uint32_t tile_h,
                                                   uint32_t n_tiles, uint32_t tile_n_bits, uint32_t lds_words,
                                                   uint32_t bucket_cap, int64_t n_isects,
@@ -1808,7 +1813,11 @@ __device__ __forceinline__ void sort_expand_piece(uint4 piece, CoarseGrid cg, ui
                 for (uint32_t j = s0; j < s1; j += 4) {
                     const uint64_t q0 = lds_staged[j], q1 = lds_staged[j + 1];
                     const uint64_t q2 = lds_staged[j + 2], q3 = lds_staged[j + 3];
-                    place += (q0 < p ? 1u : 0u) + (q1 < p ? 1u : 0u) + (q2 < p ? 1u : 0u) + (q3 < p ? 1u : 0u);
+                    if constexpr (TIES)
+                        place += (q0 < p || (q0 == p && j < i) ? 1u : 0u) + (q1 < p || (q1 == p && j + 1 < i) ? 1u : 0u) +
+                                 (q2 < p || (q2 == p && j + 2 < i) ? 1u : 0u) + (q3 < p || (q3 == p && j + 3 < i) ? 1u : 0u);
+                    else
+                        place += (q0 < p ? 1u : 0u) + (q1 < p ? 1u : 0u) + (q2 < p ? 1u : 0u) + (q3 < p ? 1u : 0u);
                 }
                 placed[k] = p;
                 place_mask[k] = place | ((uint32_t)s_mask[i] << 16);
@@ -2024,7 +2033,7 @@ constexpr uint32_t kLongBins = 2048;
 constexpr uint32_t kLongStack = 32;
 struct LongInterval { uint64_t lo, hi; uint32_t n, pad; };
 
-template <int ER>
+template <int ER, bool TIES>
 __device__ __forceinline__ void sort_expand_long_list(uint4 piece, CoarseGrid cg, uint32_t tile_w, uint32_t tile_h,
                                                       uint32_t n_tiles, uint32_t tile_n_bits, uint32_t lds_words,
                                                       uint32_t bucket_cap, int64_t n_isects,
@@ -2104,7 +2113,7 @@ __device__ __forceinline__ void sort_expand_long_list(uint4 piece, CoarseGrid cg
                 }
             }
             __syncthreads();
-            sort_expand_piece<ER>(piece, cg, tile_w, tile_h, n_tiles, tile_n_bits, lds_words, bucket_cap, n_isects,
+            sort_expand_piece<ER, TIES>(piece, cg, tile_w, tile_h, n_tiles, tile_n_bits, lds_words, bucket_cap, n_isects,
                                   entries, seg_starts, slabs_before, isect_ids, flatten_ids, lds_staged, s_wave,
                                   s_big, s_cnt, true, min(s_kept, lds_words), &carried);
             continue;
@@ -2162,7 +2171,7 @@ __device__ __forceinline__ void sort_expand_long_list(uint4 piece, CoarseGrid cg
 }
 
 // LONG: the launch takes the lists beyond the capacity of the LDS sort, part by part.
-template <int ER, bool LONG = false>
+template <int ER, bool TIES, bool LONG = false>
 __global__ void isect_block_sort_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t n_tiles,
                                         uint32_t tile_n_bits, uint32_t lds_words, uint32_t bucket_cap,
                                         int64_t n_isects, const uint32_t *__restrict__ class_count,
@@ -2180,7 +2189,7 @@ __global__ void isect_block_sort_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t
         __shared__ uint32_t s_top, s_kept;
         __shared__ unsigned long long s_range[2];
         for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) { // uniform across the workgroup
-            sort_expand_long_list<ER>(pieces[k], cg, tile_w, tile_h, n_tiles, tile_n_bits, lds_words, bucket_cap,
+            sort_expand_long_list<ER, TIES>(pieces[k], cg, tile_w, tile_h, n_tiles, tile_n_bits, lds_words, bucket_cap,
                                       n_isects, entries, seg_starts, slabs_before, isect_ids, flatten_ids,
                                       lds_staged, s_wave, s_big, s_cnt, s_stack, s_top, s_kept, s_range);
             __syncthreads();
@@ -2188,14 +2197,14 @@ __global__ void isect_block_sort_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t
         return;
     }
     for (uint32_t k = blockIdx.x; k < count; k += gridDim.x) { // uniform across the workgroup
-        sort_expand_piece<ER>(pieces[k], cg, tile_w, tile_h, n_tiles, tile_n_bits, lds_words, bucket_cap, n_isects,
+        sort_expand_piece<ER, TIES>(pieces[k], cg, tile_w, tile_h, n_tiles, tile_n_bits, lds_words, bucket_cap, n_isects,
                               entries, seg_starts, slabs_before, isect_ids, flatten_ids, lds_staged, s_wave,
                               s_big, s_cnt);
         __syncthreads(); // the next piece reuses the LDS
     }
 }
 
-template <int ER, bool LONG = false>
+template <int ER, bool TIES, bool LONG = false>
 static int launch_block_sort(int cls, uint32_t threads, uint32_t max_n, uint32_t workgroups, uint32_t max_pieces,
                              CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t n_tiles,
                              uint32_t tile_n_bits, int64_t n_isects, const uint32_t *class_count,
@@ -2217,12 +2226,12 @@ static int launch_block_sort(int cls, uint32_t threads, uint32_t max_n, uint32_t
         static size_t allowed = 0;
         std::lock_guard<std::mutex> lock(guard);
         if (lds_bytes > allowed) {
-            SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)isect_block_sort_kernel<ER, LONG>,
+            SPLATAD_CHECK_HIP(hipFuncSetAttribute((const void *)isect_block_sort_kernel<ER, TIES, LONG>,
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
             allowed = lds_bytes;
         }
     }
-    hipLaunchKernelGGL((isect_block_sort_kernel<ER, LONG>), dim3(workgroups < max_pieces ? workgroups : max_pieces),
+    hipLaunchKernelGGL((isect_block_sort_kernel<ER, TIES, LONG>), dim3(workgroups < max_pieces ? workgroups : max_pieces),
                        dim3(threads), lds_bytes, stream, cg, tile_w, tile_h, n_tiles, tile_n_bits, max_n,
                        bucket_cap, n_isects, class_count + cls, pieces + (size_t)cls * max_pieces, entries,
                        seg_starts, slabs_before, isect_ids, flatten_ids);
@@ -2452,7 +2461,7 @@ static IsectPlan isect_plan(const TileGrid &g, uint64_t total, uint32_t C, int s
     pl.n_tiles = g.tile_w * g.tile_h;
     pl.tile_n_bits = splatad_bit_width(pl.n_tiles);
     pl.cg = coarse_grid<LIDAR>(g);
-    pl.block_sort = sort && !LIDAR;
+    pl.block_sort = sort && (!LIDAR || pl.cg.bshift == 2);
     pl.sshift = sort && !pl.block_sort ? slab_shift_for(total, (uint64_t)C * pl.n_tiles) : 0;
     pl.bsshift = pl.block_sort ? block_slab_shift(total, C, (uint64_t)pl.cg.cw * pl.cg.ch) : pl.sshift;
     // one sensor's block counters have to fit the LDS of the coarse binning
@@ -2817,7 +2826,8 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         hipLaunchKernelGGL(isect_block_plan_kernel, dim3(plan_wgs), dim3(1024), 0, stream, n_blocks, pl.bsshift,
                            (const int32_t *)w.block_totals, (const uint32_t *)w.list_starts,
                            (const int32_t *)w.tile_counts, cg, g.tile_w, g.tile_h, nseg,
-                           w.seg_starts, tile_offsets, w.piece_counts, (uint32_t)pl.blocks, w.pieces);
+                           w.seg_starts, tile_offsets, w.piece_counts, (uint32_t)pl.blocks, w.pieces,
+                           LIDAR ? kBlockMergeCapLidar : kBlockMergeCap, LIDAR ? kBlockPairsCapLidar : kBlockPairsCap);
         SPLATAD_LAUNCH_CHECK();
         std::lock_guard<std::mutex> fork_lock(ss->guard);
         SPLATAD_CHECK_HIP(hipEventRecord(ss->fork, stream));
@@ -2826,7 +2836,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
         auto enqueue_block_sorts = [&]() -> int {
             int e;
 #define SPLATAD_BLOCK_CLASS(cls, ER, threads, hi, wgs, on)                                                        \
-            if ((e = launch_block_sort<ER>(cls, threads, hi, wgs, (uint32_t)pl.blocks, cg, g.tile_w, g.tile_h,   \
+            if ((e = launch_block_sort<ER, LIDAR>(cls, threads, hi, wgs, (uint32_t)pl.blocks, cg, g.tile_w, g.tile_h,   \
                                            n_tiles, tile_n_bits, n_isects, w.piece_counts, w.pieces, w.entries,  \
                                            w.seg_starts, w.list_tile_counts, isect_ids, flatten_ids, on)) != 0)  \
                 return e;
@@ -2834,7 +2844,7 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
             // Pieces beyond kBlockMergeCap entries are single lists, so the longest list tells
             // which of the upper classes are empty: their launches (5 us each on the way) are left out.
             if (longest_list > kBlockSortCap &&
-                (e = launch_block_sort<10, true>(kBlockLongClass, 1024, kBlockSortCap, 256u, (uint32_t)pl.blocks, cg,
+                (e = launch_block_sort<10, LIDAR, true>(kBlockLongClass, 1024, kBlockSortCap, 256u, (uint32_t)pl.blocks, cg,
                                                  g.tile_w, g.tile_h, n_tiles, tile_n_bits, n_isects,
                                                  w.piece_counts, w.pieces, w.entries, w.seg_starts,
                                                  w.list_tile_counts, isect_ids, flatten_ids, stream)) != 0)
