@@ -132,13 +132,30 @@ sh_cache_clear_kernel(uint32_t n, ShView view, const float *__restrict__ opaciti
     __shared__ float s_sum[SPLATAD_THREADS / SPLATAD_WAVE];
     const float nan = __uint_as_float(0x7FC00000u);
     float sum = 0.f;
-    for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
-        cache[e] = make_float4(nan, nan, nan, nan);
-        const int32_t rx = view.radii[(size_t)e * 2], ry = view.radii[(size_t)e * 2 + 1];
-        if (rx > 0 && ry > 0) {
-            const uint32_t g = view.gaussian_ids ? (uint32_t)view.gaussian_ids[e] : e % view.N;
-            sum += opacities[g] * fminf(2.f * (float)rx * inv_tile + 1.f, tile_w) *
-                   fminf(2.f * (float)ry * inv_tile + 1.f, tile_h);
+    // four rows per trip, their radii requested together: with many rows per lane (several
+    // sensors' worth) the loop is bound by the latency of its loads, not by the bytes
+    const uint32_t stride = gridDim.x * blockDim.x;
+    const int2 *radii2 = reinterpret_cast<const int2 *>(view.radii);
+    for (uint32_t e0 = blockIdx.x * blockDim.x + threadIdx.x; e0 < n; e0 += 4 * stride) {
+        int2 r[4];
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            const uint64_t e = (uint64_t)e0 + (uint64_t)k * stride;
+            r[k] = e < n ? radii2[e] : make_int2(0, 0);
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            const uint64_t e = (uint64_t)e0 + (uint64_t)k * stride;
+            if (e < n) cache[e] = make_float4(nan, nan, nan, nan);
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            const uint32_t e = e0 + k * stride; // (below n where the radii are positive)
+            if (r[k].x > 0 && r[k].y > 0) {
+                const uint32_t g = view.gaussian_ids ? (uint32_t)view.gaussian_ids[e] : e % view.N;
+                sum += opacities[g] * fminf(2.f * (float)r[k].x * inv_tile + 1.f, tile_w) *
+                       fminf(2.f * (float)r[k].y * inv_tile + 1.f, tile_h);
+            }
         }
     }
 #pragma unroll
