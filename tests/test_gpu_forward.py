@@ -327,6 +327,30 @@ def test_isect_sort_long_segments_and_depth_ties(n, tie_frac):
     np.testing.assert_array_equal(to_np(flat), o_flat)
 
 
+@pytest.mark.parametrize("n,tie_frac,turns", [(3000, 0.3, 1), (3000, 0.5, 2), (20000, 0.9, 1), (30000, 0.6, 2),
+                                              (120000, 0.9, 1)])
+def test_isect_lidar_long_lists_ties_and_rectangles_wider_than_the_grid(n, tie_frac, turns):
+    # a grid of 4 x 2 tiles (one coarse block) that every Gaussian covers; with turns == 2 the
+    # rectangles are wider than the full turn, so a tile is listed twice by the same Gaussian and
+    # the block's list holds equal keys.  Many equal depths put a slab's list beyond what one LDS
+    # sort takes (taken in parts) and, with 108000 of them, beyond what the block sort takes at
+    # all (the per-tile segment sort then).
+    from splatad_amd import isect_lidar_tiles
+    rng = np.random.default_rng(n + turns)
+    eb = np.array([-20.0, 0.0, 20.0], np.float32)
+    means2d = np.stack([rng.uniform(-180, 180, (1, n)), rng.uniform(-5, 5, (1, n))], -1).astype(np.float32)
+    radii = np.empty((1, n, 2), np.float32)
+    radii[..., 0] = 170.0 if turns == 1 else rng.uniform(185.0, 300.0, (1, n))
+    radii[..., 1] = 30.0
+    depths = np.exp(rng.uniform(-3, 5, (1, n))).astype(np.float32)
+    depths[0, rng.random(n) < tie_frac] = 3.25
+    got = isect_lidar_tiles(to_dev(means2d), to_dev(radii), to_dev(depths), to_dev(eb), 90.0, -180.0)
+    want = oracle.isect_lidar_tiles(means2d, radii, depths, eb, 90.0, -180.0)
+    assert want[1].shape[0] >= 6 * n
+    for g, w in zip(got, want):
+        np.testing.assert_array_equal(to_np(g), w)
+
+
 @pytest.mark.parametrize("n,spread", [(300, "even"), (1800, "even"), (1800, "far"), (7000, "even"),
                                       (1800, "infinite"), (5000, "infinite")])
 def test_isect_sort_of_short_segments_by_depth_spread(n, spread):
