@@ -254,8 +254,9 @@ __device__ __forceinline__ void slab_bounds_workgroup(uint64_t total, const floa
         [&](uint32_t i, uint32_t before, uint32_t) { s_before[i] = before; });
     const uint32_t w = s_weight[tid], before = s_before[tid];
     if (w == 0) return;
+    const uint32_t shift = 31u - (uint32_t)__clz((int)n_slabs); // the slabs are a power of two: no division per bound
     for (uint32_t k = 1; k < n_slabs; ++k) {
-        const uint32_t target = (uint32_t)((uint64_t)sum * k / n_slabs);
+        const uint32_t target = (uint32_t)(((uint64_t)sum * k) >> shift);
         if (before < target && target <= before + w) bounds[k - 1] = s_sorted[tid];
     }
 }
