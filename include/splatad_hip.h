@@ -91,13 +91,20 @@ int splatad_projection_packed_count_tiles(uint32_t C, uint32_t N, const float *m
  * splatad_view_colors_fwd_packed) runs beside the sort, whose long workgroups leave part of the
  * GPU idle.  Nothing waits for that stream: the caller joins it.  (A cross-stream wait costs
  * the host about 10 us on this runtime, four kernel launches; here it rides on the fork the
- * sort makes anyway.) */
+ * sort makes anyway.)
+ * beside_work (may be NULL): called once before this call returns, with beside_context and a
+ * stream on which the caller may enqueue such work from inside the callback; it runs beside the
+ * sort and has completed, as far as `stream` is concerned, when this call returns (the sort's own
+ * fork and join carry it: no further cross-stream wait).  When there is nothing to sort the
+ * stream handed over is `stream` itself.  A non-zero return value becomes this call's. */
+typedef int (*splatad_beside_fn)(void *context, splatad_stream_t stream);
 int splatad_isect_tiles_fill_packed(uint32_t C, uint32_t N, uint32_t tile_size, uint32_t tile_width,
                                     uint32_t tile_height, int64_t n_isects,
                                     const void *packed_workspace, void *isect_workspace, void *lists,
                                     int32_t *tiles_per_gauss, int64_t *isect_ids,
                                     int32_t *flatten_ids, int32_t *tile_offsets,
-                                    splatad_stream_t beside_stream, splatad_stream_t stream);
+                                    splatad_stream_t beside_stream, splatad_beside_fn beside_work,
+                                    void *beside_context, splatad_stream_t stream);
 /* opacities [N] and row_opacities [nnz] (both or neither): the kept rows' opacity for the
  * compositing, opacities[gaussian] times the row's compensation when compensations are
  * computed (rendering.py:311-314 of the reference does this with a gather and a product). */
@@ -254,7 +261,7 @@ int splatad_isect_tiles_prepare(uint64_t total, uint32_t N, const int64_t *camer
                                 void *workspace, splatad_stream_t stream);
 /* _fill for dense [C, N] rows that stand in for their packed rows: `remap` [C * N] holds each
  * kept row's position among the kept rows (what flatten_ids must name); tiles_out, if not NULL,
- * receives the kept rows' tile counts at those positions.  beside_stream: see
+ * receives the kept rows' tile counts at those positions.  beside_stream, beside_work: see
  * splatad_isect_tiles_fill_packed. */
 int splatad_isect_tiles_fill_remapped(uint64_t total, uint32_t N, const float *means2d,
                                       const int32_t *radii, const float *depths, uint32_t C,
@@ -263,6 +270,7 @@ int splatad_isect_tiles_fill_remapped(uint64_t total, uint32_t N, const float *m
                                       const int32_t *remap, void *workspace, void *lists,
                                       int32_t *tiles_out, int64_t *isect_ids, int32_t *flatten_ids,
                                       int32_t *tile_offsets, splatad_stream_t beside_stream,
+                                      splatad_beside_fn beside_work, void *beside_context,
                                       splatad_stream_t stream);
 int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_ids,
                              const float *means2d, const int32_t *radii, const float *depths,

@@ -662,14 +662,15 @@ extern "C" int splatad_isect_tiles_fill_packed(uint32_t C, uint32_t N, uint32_t 
                                                const void *packed_workspace, void *isect_workspace,
                                                void *lists, int32_t *tiles_per_gauss, int64_t *isect_ids,
                                                int32_t *flatten_ids, int32_t *tile_offsets,
-                                               splatad_stream_t beside_stream, splatad_stream_t stream) {
+                                               splatad_stream_t beside_stream, splatad_beside_fn beside_work,
+                                               void *beside_context, splatad_stream_t stream) {
     SPLATAD_REQUIRE(packed_workspace && isect_workspace, "isect_tiles: null workspace");
     const uint64_t T = (uint64_t)C * N;
     PackedWorkspace w = carve_packed((void *)packed_workspace, T);
     return splatad_isect_tiles_fill_remapped(T, N, w.means2d, w.radii, w.depths, C, tile_size, tile_width,
                                              tile_height, n_isects, w.tiles, w.pos, isect_workspace, lists,
                                              tiles_per_gauss, isect_ids, flatten_ids, tile_offsets,
-                                             beside_stream, stream);
+                                             beside_stream, beside_work, beside_context, stream);
 }
 
 extern "C" int splatad_view_colors_fwd_packed(uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
