@@ -193,15 +193,17 @@ int splatad_view_colors_fwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K, uint
                             int coeffs_per_sensor, const float *depths, float *colors,
                             splatad_stream_t stream);
 /* _fwd over dense [C, N] rows that stand in for their packed rows: an active row e writes its
- * colours to row remap[e] of `colors` (its position among the kept rows), inactive rows write
- * nothing; depths, if given, is indexed by e as well.  Same values as _fwd on the packed rows
+ * colours to row remap[e] (+ remap_offsets[e / 256] where remap_offsets is not NULL: positions
+ * kept as a place inside a group of 256 rows plus the group's place) of `colors` (its position
+ * among the kept rows), inactive rows write nothing; depths, if given, is indexed by e as well.  Same values as _fwd on the packed rows
  * (one dependent load less per row).  _packed takes the rows, positions and depths from the
  * workspace of splatad_projection_packed_count[_tiles]: colors is [nnz, 3], or [nnz, 4]
  * with_depth. */
 int splatad_view_colors_fwd_remapped(uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
                                      const float *means, const float *viewmats, const int32_t *radii,
-                                     const int32_t *remap, const float *coeffs, int coeffs_per_sensor,
-                                     const float *depths, float *colors, splatad_stream_t stream);
+                                     const int32_t *remap, const int32_t *remap_offsets,
+                                     const float *coeffs, int coeffs_per_sensor, const float *depths,
+                                     float *colors, splatad_stream_t stream);
 int splatad_view_colors_fwd_packed(uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
                                    const float *means, const float *viewmats,
                                    const void *packed_workspace, const float *coeffs,
@@ -261,14 +263,15 @@ int splatad_isect_tiles_prepare(uint64_t total, uint32_t N, const int64_t *camer
                                 void *workspace, splatad_stream_t stream);
 /* _fill for dense [C, N] rows that stand in for their packed rows: `remap` [C * N] holds each
  * kept row's position among the kept rows (what flatten_ids must name); tiles_out, if not NULL,
- * receives the kept rows' tile counts at those positions.  beside_stream, beside_work: see
- * splatad_isect_tiles_fill_packed. */
+ * receives the kept rows' tile counts at those positions.  remap_offsets (may be NULL): as for
+ * splatad_view_colors_fwd_remapped, row e's position is remap[e] + remap_offsets[e / 256].
+ * beside_stream, beside_work: see splatad_isect_tiles_fill_packed. */
 int splatad_isect_tiles_fill_remapped(uint64_t total, uint32_t N, const float *means2d,
                                       const int32_t *radii, const float *depths, uint32_t C,
                                       uint32_t tile_size, uint32_t tile_width, uint32_t tile_height,
                                       int64_t n_isects, const int32_t *tiles_per_gauss,
-                                      const int32_t *remap, void *workspace, void *lists,
-                                      int32_t *tiles_out, int64_t *isect_ids, int32_t *flatten_ids,
+                                      const int32_t *remap, const int32_t *remap_offsets,
+                                      void *workspace, void *lists, int32_t *tiles_out, int64_t *isect_ids, int32_t *flatten_ids,
                                       int32_t *tile_offsets, splatad_stream_t beside_stream,
                                       splatad_beside_fn beside_work, void *beside_context,
                                       splatad_stream_t stream);

@@ -605,6 +605,7 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
                     uint32_t cam_lo, uint32_t cam_hi, uint32_t n_blocks, int32_t *table,
                     uint4 *__restrict__ entries, uint32_t sshift,
                     const uint32_t *__restrict__ slab_bounds, const int32_t *__restrict__ remap,
+                    const int32_t *__restrict__ remap_offsets,
                     int32_t *__restrict__ tiles_out, int32_t *__restrict__ totals,
                     int64_t *__restrict__ n_entries, uint32_t entries_cap,
                     uint32_t *__restrict__ list_starts, unsigned long long *__restrict__ longest_host) {
@@ -691,7 +692,9 @@ isect_coarse_kernel(TileGrid g, CoarseGrid cg, uint64_t total, uint32_t N,
         // the row's position among the kept rows (an increasing function of the dense index, so
         // ties keep their order), and the kept rows' tile counts are gathered on the way.
         if (FILL && remap != nullptr && was_kept) {
-            const uint32_t at = (uint32_t)remap[mine.idx];
+            // (a row's place: remap, plus, where given, that of its group of SPLATAD_THREADS rows)
+            const uint32_t at = (uint32_t)(remap[mine.idx] +
+                                           (remap_offsets != nullptr ? remap_offsets[mine.idx / SPLATAD_THREADS] : 0));
             if (tiles_out != nullptr && cam >= cam_lo && cam < cam_hi) tiles_out[at] = mine.cnt;
             mine.idx = at;
         }
@@ -2596,8 +2599,8 @@ static int enqueue_coarse_count(const TileGrid &g, const IsectPlan &pl, const Is
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, pl.cg,
                            total, N, camera_ids, means2d, radii, pl.bsshift ? depths : nullptr, c0, c1,
                            (uint32_t)pl.blocks, w.coarse_counts, (uint4 *)nullptr, pl.bsshift,
-                           (const uint32_t *)w.slab_bounds, (const int32_t *)nullptr, (int32_t *)nullptr,
-                           w.block_totals, (int64_t *)nullptr, 0u, (uint32_t *)nullptr,
+                           (const uint32_t *)w.slab_bounds, (const int32_t *)nullptr, (const int32_t *)nullptr,
+                           (int32_t *)nullptr, w.block_totals, (int64_t *)nullptr, 0u, (uint32_t *)nullptr,
                            (unsigned long long *)nullptr);
     }
     SPLATAD_LAUNCH_CHECK();
@@ -2722,7 +2725,8 @@ static int isect_fill_with(TileGrid g, uint64_t total, uint32_t N, const int64_t
                       int sort, int64_t n_isects, const int32_t *tiles_per_gauss,
                       void *workspace, void *lists, int64_t *isect_ids, int32_t *flatten_ids,
                       int32_t *tile_offsets, hipStream_t stream, const int32_t *remap,
-                      int32_t *tiles_out, hipStream_t beside, BesideWork &beside_work);
+                      const int32_t *remap_offsets, int32_t *tiles_out, hipStream_t beside,
+                      BesideWork &beside_work);
 
 template <bool LIDAR>
 static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *camera_ids,
@@ -2731,13 +2735,14 @@ static int isect_fill(TileGrid g, uint64_t total, uint32_t N, const int64_t *cam
                       void *workspace, void *lists, int64_t *isect_ids, int32_t *flatten_ids,
                       int32_t *tile_offsets, hipStream_t stream, const int32_t *remap = nullptr,
                       int32_t *tiles_out = nullptr, hipStream_t beside = nullptr,
-                      splatad_beside_fn beside_fn = nullptr, void *beside_context = nullptr) {
+                      splatad_beside_fn beside_fn = nullptr, void *beside_context = nullptr,
+                      const int32_t *remap_offsets = nullptr) {
     BesideWork work;
     work.fn = beside_fn;
     work.context = beside_context;
     const int rc = isect_fill_with<LIDAR>(g, total, N, camera_ids, means2d, radii, depths, C, sort, n_isects,
                                           tiles_per_gauss, workspace, lists, isect_ids, flatten_ids, tile_offsets,
-                                          stream, remap, tiles_out, beside, work);
+                                          stream, remap, remap_offsets, tiles_out, beside, work);
     if (rc) return rc;
     return work.run(stream); // nothing was sorted on helper streams: on the call's own stream
 }
@@ -2748,7 +2753,8 @@ static int isect_fill_with(TileGrid g, uint64_t total, uint32_t N, const int64_t
                       int sort, int64_t n_isects, const int32_t *tiles_per_gauss,
                       void *workspace, void *lists, int64_t *isect_ids, int32_t *flatten_ids,
                       int32_t *tile_offsets, hipStream_t stream, const int32_t *remap,
-                      int32_t *tiles_out, hipStream_t beside, BesideWork &beside_work) {
+                      const int32_t *remap_offsets, int32_t *tiles_out, hipStream_t beside,
+                      BesideWork &beside_work) {
     SPLATAD_REQUIRE(remap == nullptr || (sort && camera_ids == nullptr),
                     "isect: remapped rows need sort != 0 and a dense [C, N] layout");
     if (total == 0 || n_isects == 0) {
@@ -2805,7 +2811,7 @@ static int isect_fill_with(TileGrid g, uint64_t total, uint32_t N, const int64_t
                            dim3(kCoarseThreads), (size_t)(c1 - c0) * pl.per_cam * 4, stream, g, cg,
                            total, N, camera_ids, means2d, radii, depths, c0, c1, (uint32_t)pl.blocks,
                            w.coarse_counts, w.entries, pl.bsshift, (const uint32_t *)w.slab_bounds, remap,
-                           tiles_out, w.block_totals, w.n_entries, (uint32_t)n_isects,
+                           remap_offsets, tiles_out, w.block_totals, w.n_entries, (uint32_t)n_isects,
                            pl.block_sort ? w.list_starts : (uint32_t *)nullptr,
                            pl.block_sort ? longest.word.device : (unsigned long long *)nullptr);
     }
@@ -3026,7 +3032,7 @@ extern "C" int splatad_isect_tiles_fill_remapped(uint64_t total, uint32_t N, con
                                                  uint32_t tile_size, uint32_t tile_width,
                                                  uint32_t tile_height, int64_t n_isects,
                                                  const int32_t *tiles_per_gauss, const int32_t *remap,
-                                                 void *workspace, void *lists, int32_t *tiles_out,
+                                                 const int32_t *remap_offsets, void *workspace, void *lists, int32_t *tiles_out,
                                                  int64_t *isect_ids, int32_t *flatten_ids,
                                                  int32_t *tile_offsets, splatad_stream_t beside_stream,
                                                  splatad_beside_fn beside_work, void *beside_context,
@@ -3036,7 +3042,8 @@ extern "C" int splatad_isect_tiles_fill_remapped(uint64_t total, uint32_t N, con
     TileGrid g{tile_size, tile_width, tile_height, 0.f, 0.f, nullptr};
     return isect_fill<false>(g, total, N, nullptr, means2d, radii, depths, C, 1, n_isects, tiles_per_gauss,
                              workspace, lists, isect_ids, flatten_ids, tile_offsets, (hipStream_t)stream,
-                             remap, tiles_out, (hipStream_t)beside_stream, beside_work, beside_context);
+                             remap, tiles_out, (hipStream_t)beside_stream, beside_work, beside_context,
+                             remap_offsets);
 }
 
 extern "C" int splatad_isect_lidar_tiles_count(uint64_t total, uint32_t N,

@@ -123,7 +123,9 @@ __device__ __forceinline__ void relative_velocity(const SensorPose &p, const flo
 
 // COUNT: every workgroup also writes how many of its rows are kept (radii.x > 0) and how many
 // tiles of the camera's grid those meet: the counts of the packed layout and of its tile
-// intersection, gathered while the rows are in registers.
+// intersection, gathered while the rows are in registers; and every row the number of kept
+// rows before it in its workgroup (kept_before), which with the exclusive prefix of the
+// workgroups' counts is the row's place among the kept rows: no scan pass over the rows.
 template <bool COUNT>
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 projection_fwd_kernel(uint32_t C, uint32_t N, const float *__restrict__ means,
@@ -137,7 +139,8 @@ projection_fwd_kernel(uint32_t C, uint32_t N, const float *__restrict__ means,
                       float *__restrict__ depths, float *__restrict__ conics,
                       float *__restrict__ compensations, float *__restrict__ pix_vels,
                       uint32_t tile_size, uint32_t tile_w, uint32_t tile_h,
-                      int64_t *__restrict__ kept_sums, int64_t *__restrict__ tile_sums) {
+                      int64_t *__restrict__ kept_sums, int64_t *__restrict__ tile_sums,
+                      int32_t *__restrict__ kept_before) {
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const bool live = idx < (uint64_t)C * N;
     if (!COUNT && !live) return;
@@ -213,12 +216,16 @@ projection_fwd_kernel(uint32_t C, uint32_t N, const float *__restrict__ means,
     if (COUNT) {
         __shared__ int64_t s_sums[2 * (SPLATAD_THREADS / SPLATAD_WAVE)];
         int64_t kept = 0, tiles = 0;
-        if (live && o_radii.x > 0) {
+        const bool keep = live && o_radii.x > 0;
+        if (keep) {
             int32_t x0, y0, x1, y1;
             splatad_camera_tile_rect(tile_size, tile_w, tile_h, o_mean, o_radii, x0, y0, x1, y1);
             kept = 1;
             tiles = (int64_t)max(y1 - y0, 0) * max(x1 - x0, 0);
         }
+        const uint64_t keepers = wave_ballot(keep);
+        const uint32_t before_in_wave =
+            __builtin_amdgcn_mbcnt_hi((uint32_t)(keepers >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)keepers, 0u));
 #pragma unroll
         for (int off = SPLATAD_WAVE / 2; off > 0; off >>= 1) {
             kept += __shfl_xor(kept, off, SPLATAD_WAVE);
@@ -227,6 +234,11 @@ projection_fwd_kernel(uint32_t C, uint32_t N, const float *__restrict__ means,
         const uint32_t wave = threadIdx.x / SPLATAD_WAVE;
         if ((threadIdx.x & (SPLATAD_WAVE - 1)) == 0) { s_sums[2 * wave] = kept; s_sums[2 * wave + 1] = tiles; }
         __syncthreads();
+        if (live) {
+            uint32_t before = before_in_wave;
+            for (uint32_t w = 0; w < wave; ++w) before += (uint32_t)s_sums[2 * w];
+            kept_before[idx] = (int32_t)before;
+        }
         if (threadIdx.x == 0) {
             kept = tiles = 0;
             for (uint32_t w = 0; w < SPLATAD_THREADS / SPLATAD_WAVE; ++w) { kept += s_sums[2 * w]; tiles += s_sums[2 * w + 1]; }
@@ -333,7 +345,8 @@ struct PackedWorkspace {
     float *conics;    // [T, 3]
     float *comps;     // [T]
     float *pix_vels;  // [T, 2]
-    int32_t *pos;     // [T] exclusive prefix of the valid flags
+    int32_t *pos;     // [T] kept rows before the row: in all, or in its projection workgroup, with
+    int32_t *offsets; // [T / SPLATAD_THREADS + 1] the kept rows before the workgroup (zeros in the first case)
     int64_t *total;   // [1]
     int64_t *block_sums;
     int64_t *tile_sums; // tiles met by the kept rows of a scan block or projection workgroup (optional count)
@@ -354,6 +367,7 @@ static PackedWorkspace carve_packed(void *ws, uint64_t T) {
     // (room for the counts of every projection workgroup, SCAN_ITEMS per scan block)
     w.block_sums = (int64_t *)p;  p += SCAN_ITEMS * scan_workspace_bytes((int64_t)T);
     w.tile_sums = (int64_t *)p;   p += SCAN_ITEMS * scan_workspace_bytes((int64_t)T);
+    w.offsets = (int32_t *)p;     p += splatad_align256((T / SPLATAD_THREADS + 1) * 4);
     w.tiles = (int32_t *)p;
     return w;
 }
@@ -392,18 +406,28 @@ packed_block_totals_kernel(uint64_t T, const int32_t *__restrict__ w_radii,
 // One workgroup: publishes the number of kept rows (low 32 bits) and of their tile
 // intersections (high 32 bits, saturated at 2^31 - 1, which the caller refuses) in one word.
 // The kept rows are *total when that is given, the sum of kept_sums otherwise.
+// offsets (with kept_sums): receives the exclusive prefix of kept_sums, the kept rows before
+// each workgroup of the projection.
 __global__ void __launch_bounds__(SPLATAD_THREADS)
 packed_publish_kernel(const int64_t *__restrict__ total, const int64_t *__restrict__ kept_sums,
                       const int64_t *__restrict__ tile_sums, int64_t n_blocks,
-                      unsigned long long *__restrict__ word) {
+                      unsigned long long *__restrict__ word, int32_t *__restrict__ offsets) {
+    // a lane takes a run of consecutive blocks, so that its prefix is that of its first block
+    const int64_t per = (n_blocks + SPLATAD_THREADS - 1) / SPLATAD_THREADS;
+    const int64_t b0 = min(n_blocks, (int64_t)threadIdx.x * per), b1 = min(n_blocks, b0 + per);
     int64_t part = 0, part_kept = 0;
-    for (int64_t b = threadIdx.x; b < n_blocks; b += SPLATAD_THREADS) {
+    for (int64_t b = b0; b < b1; ++b) {
         part += tile_sums[b];
         if (total == nullptr) part_kept += kept_sums[b];
     }
     int64_t tiles, kept;
     block_exclusive_scan(part, &tiles);
-    block_exclusive_scan(part_kept, &kept);
+    int64_t before = block_exclusive_scan(part_kept, &kept);
+    if (offsets != nullptr)
+        for (int64_t b = b0; b < b1; ++b) {
+            offsets[b] = (int32_t)before;
+            before += kept_sums[b];
+        }
     if (threadIdx.x == 0) {
         if (total != nullptr) kept = *total;
         const unsigned long long hi = tiles > 0x7FFFFFFFll ? 0x7FFFFFFFull : (unsigned long long)tiles;
@@ -417,7 +441,7 @@ packed_compact_kernel(uint32_t C, uint32_t N, int64_t nnz, const int32_t *__rest
                       const float *__restrict__ w_means2d, const float *__restrict__ w_depths,
                       const float *__restrict__ w_conics, const float *__restrict__ w_comps,
                       const float *__restrict__ w_pix_vels, const int32_t *__restrict__ pos,
-                      int32_t *__restrict__ indptr, int64_t *__restrict__ camera_ids,
+                      const int32_t *__restrict__ offsets, int32_t *__restrict__ indptr, int64_t *__restrict__ camera_ids,
                       int64_t *__restrict__ gaussian_ids, int32_t *__restrict__ radii,
                       float *__restrict__ means2d, float *__restrict__ depths,
                       float *__restrict__ conics, float *__restrict__ comps,
@@ -429,7 +453,7 @@ packed_compact_kernel(uint32_t C, uint32_t N, int64_t nnz, const int32_t *__rest
     const uint32_t cid = idx / N, gid = idx - cid * N;
     // everything a kept row needs is requested before the test on the radius (culled rows of
     // the workspace hold zeros): one memory round trip instead of two
-    const int32_t o = pos[idx];
+    const int32_t o = pos[idx] + offsets[idx / SPLATAD_THREADS];
     const int2 r = reinterpret_cast<const int2 *>(w_radii)[idx];
     const float2 mean = reinterpret_cast<const float2 *>(w_means2d)[idx];
     const float depth = w_depths[idx];
@@ -474,7 +498,7 @@ static int projection_fwd(uint32_t C, uint32_t N, const float *means,
                                       float *means2d, float *depths, float *conics,
                                       float *compensations, float *pix_vels,
                                       uint32_t tile_size, uint32_t tile_w, uint32_t tile_h,
-                                      int64_t *kept_sums, int64_t *tile_sums,
+                                      int64_t *kept_sums, int64_t *tile_sums, int32_t *kept_before,
                                       splatad_stream_t stream) {
     SPLATAD_REQUIRE((covars != nullptr) != (quats != nullptr && scales != nullptr),
                     "projection: pass either covars or (quats, scales)");
@@ -485,13 +509,14 @@ static int projection_fwd(uint32_t C, uint32_t N, const float *means,
                     "projection: null pointer argument");
     const uint64_t T = (uint64_t)C * N;
     const bool count = kept_sums != nullptr;
-    SPLATAD_REQUIRE(!count || (tile_sums != nullptr && tile_size > 0), "projection: incomplete count arguments");
+    SPLATAD_REQUIRE(!count || (tile_sums != nullptr && kept_before != nullptr && tile_size > 0),
+                    "projection: incomplete count arguments");
     hipLaunchKernelGGL((count ? projection_fwd_kernel<true> : projection_fwd_kernel<false>),
                        dim3((uint32_t)((T + SPLATAD_THREADS - 1) / SPLATAD_THREADS)),
                        dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, C, N, means, covars, quats,
                        scales, velocities, viewmats, Ks, W, H, lin_vel, ang_vel, rs_time, eps2d,
                        near_plane, far_plane, radius_clip, radii, means2d, depths, conics,
-                       compensations, pix_vels, tile_size, tile_w, tile_h, kept_sums, tile_sums);
+                       compensations, pix_vels, tile_size, tile_w, tile_h, kept_sums, tile_sums, kept_before);
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }
@@ -508,7 +533,7 @@ extern "C" int splatad_projection_fwd(uint32_t C, uint32_t N, const float *means
                                       splatad_stream_t stream) {
     return projection_fwd(C, N, means, covars, quats, scales, velocities, viewmats, Ks, W, H, lin_vel,
                           ang_vel, rs_time, eps2d, near_plane, far_plane, radius_clip, radii, means2d,
-                          depths, conics, compensations, pix_vels, 0, 0, 0, nullptr, nullptr, stream);
+                          depths, conics, compensations, pix_vels, 0, 0, 0, nullptr, nullptr, nullptr, stream);
 }
 
 extern "C" int splatad_lidar_projection_fwd(uint32_t C, uint32_t N, const float *means,
@@ -543,7 +568,8 @@ extern "C" int splatad_lidar_projection_fwd(uint32_t C, uint32_t N, const float 
 extern "C" size_t splatad_projection_packed_workspace_bytes(uint32_t C, uint32_t N) {
     const uint64_t T = (uint64_t)C * N;
     return 256 + splatad_align256(T * 8) * 3 + splatad_align256(T * 4) * 3 +
-           splatad_align256(T * 12) + 2 * SCAN_ITEMS * scan_workspace_bytes((int64_t)T) + splatad_align256(T * 4);
+           splatad_align256(T * 12) + 2 * SCAN_ITEMS * scan_workspace_bytes((int64_t)T) +
+           splatad_align256((T / SPLATAD_THREADS + 1) * 4) + splatad_align256(T * 4);
 }
 
 // tile_size == 0: only the kept rows are counted.
@@ -576,28 +602,31 @@ static int packed_count(uint32_t C, uint32_t N, const float *means, const float 
                             ang_vel, rs_time, eps2d, near_plane, far_plane, radius_clip, w.radii, w.means2d,
                             w.depths, w.conics, calc_compensations ? w.comps : nullptr, w.pix_vels,
                             fused ? tile_size : 0, tile_width, tile_height, fused ? w.block_sums : nullptr,
-                            fused ? w.tile_sums : nullptr, stream);
+                            fused ? w.tile_sums : nullptr, fused ? w.pos : nullptr, stream);
     if (rc) return rc;
     if (fused) {
         hipLaunchKernelGGL(packed_publish_kernel, dim3(1), dim3(SPLATAD_THREADS), 0, (hipStream_t)stream,
                            (const int64_t *)nullptr, (const int64_t *)w.block_sums, (const int64_t *)w.tile_sums,
-                           n_groups, lease.word.device);
+                           n_groups, lease.word.device, w.offsets);
         SPLATAD_LAUNCH_CHECK();
-        rc = launch_exclusive_scan_apply<int32_t>(w.radii, (int64_t)T, 2, 1, w.pos, w.total, w.block_sums,
-                                                  (hipStream_t)stream, SCAN_ITEMS);
-        if (rc) return rc;
+        // (no scan over the rows: the projection left every row's place inside its workgroup
+        // in w.pos, and the publishing kernel the workgroups' places in w.offsets)
         if (isect_workspace != nullptr) {
             rc = splatad_isect_tiles_prepare(T, N, nullptr, w.means2d, w.radii, w.depths, C, tile_size,
                                              tile_width, tile_height, 1, nullptr, isect_workspace, stream);
             if (rc) return rc;
         }
     } else if (tile_size == 0) {
+        hipLaunchKernelGGL(fill_i32_kernel, dim3((uint32_t)((n_groups + 1 + 255) / 256)), dim3(256), 0,
+                           (hipStream_t)stream, w.offsets, n_groups + 1, 0);
         rc = launch_exclusive_scan<int32_t>(w.radii, (int64_t)T, 2, 1, w.pos, w.total, w.block_sums,
                                             (hipStream_t)stream);
         if (rc) return rc;
         hipLaunchKernelGGL(host_word_publish_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, w.total,
                            lease.word.device);
     } else {
+        hipLaunchKernelGGL(fill_i32_kernel, dim3((uint32_t)((n_groups + 1 + 255) / 256)), dim3(256), 0,
+                           (hipStream_t)stream, w.offsets, n_groups + 1, 0);
         hipLaunchKernelGGL(packed_block_totals_kernel, dim3((uint32_t)n_blocks), dim3(SPLATAD_THREADS), 0,
                            (hipStream_t)stream, T, (const int32_t *)w.radii, (const float *)w.means2d, tile_size,
                            tile_width, tile_height, w.block_sums, w.tile_sums);
@@ -607,7 +636,7 @@ static int packed_count(uint32_t C, uint32_t N, const float *means, const float 
         if (rc) return rc;
         hipLaunchKernelGGL(packed_publish_kernel, dim3(1), dim3(SPLATAD_THREADS), 0, (hipStream_t)stream,
                            (const int64_t *)w.total, (const int64_t *)nullptr, (const int64_t *)w.tile_sums,
-                           n_blocks, lease.word.device);
+                           n_blocks, lease.word.device, (int32_t *)nullptr);
         SPLATAD_LAUNCH_CHECK();
         // work for the GPU while the host learns the counts and sizes the outputs: the first
         // stages of the tile intersection, on the dense rows (culled rows meet no tile)
@@ -668,7 +697,7 @@ extern "C" int splatad_isect_tiles_fill_packed(uint32_t C, uint32_t N, uint32_t 
     const uint64_t T = (uint64_t)C * N;
     PackedWorkspace w = carve_packed((void *)packed_workspace, T);
     return splatad_isect_tiles_fill_remapped(T, N, w.means2d, w.radii, w.depths, C, tile_size, tile_width,
-                                             tile_height, n_isects, w.tiles, w.pos, isect_workspace, lists,
+                                             tile_height, n_isects, w.tiles, w.pos, w.offsets, isect_workspace, lists,
                                              tiles_per_gauss, isect_ids, flatten_ids, tile_offsets,
                                              beside_stream, beside_work, beside_context, stream);
 }
@@ -680,7 +709,7 @@ extern "C" int splatad_view_colors_fwd_packed(uint32_t C, uint32_t N, uint32_t K
                                               splatad_stream_t stream) {
     SPLATAD_REQUIRE(packed_workspace != nullptr, "view colours: null workspace");
     PackedWorkspace w = carve_packed((void *)packed_workspace, (uint64_t)C * N);
-    return splatad_view_colors_fwd_remapped(C, N, K, degree, means, viewmats, w.radii, w.pos, coeffs,
+    return splatad_view_colors_fwd_remapped(C, N, K, degree, means, viewmats, w.radii, w.pos, w.offsets, coeffs,
                                             coeffs_per_sensor, with_depth ? w.depths : nullptr, colors, stream);
 }
 
@@ -708,7 +737,7 @@ extern "C" int splatad_projection_packed_fill(uint32_t C, uint32_t N, int64_t nn
     hipLaunchKernelGGL(packed_compact_kernel,
                        dim3((uint32_t)((T + SPLATAD_THREADS - 1) / SPLATAD_THREADS)),
                        dim3(SPLATAD_THREADS), 0, (hipStream_t)stream, C, N, nnz, w.radii,
-                       w.means2d, w.depths, w.conics, w.comps, w.pix_vels, w.pos, indptr,
+                       w.means2d, w.depths, w.conics, w.comps, w.pix_vels, w.pos, w.offsets, indptr,
                        camera_ids, gaussian_ids, radii, means2d, depths, conics, compensations,
                        pix_vels, opacities, row_opacities);
     SPLATAD_LAUNCH_CHECK();

@@ -83,13 +83,15 @@ __device__ __forceinline__ void sh_fwd_row(uint32_t e, uint32_t K, uint32_t degr
                                            const float *__restrict__ dirs, const float *__restrict__ coeffs,
                                            const uint8_t *__restrict__ masks, const float *__restrict__ depths,
                                            uint32_t stride, float *__restrict__ colors,
-                                           const int32_t *__restrict__ remap) {
+                                           const int32_t *__restrict__ remap,
+                                           const int32_t *__restrict__ remap_offsets = nullptr) {
     float r = 0.f, g = 0.f, b = 0.f;
     float dx = 0.f, dy = 0.f, dz = 0.f;
     size_t coeff_row;
     // remap: only the active rows have a place in the output, row e at remap[e]
     uint32_t at = e;
-    if (VIEW && remap != nullptr) at = (uint32_t)remap[e];
+    if (VIEW && remap != nullptr)
+        at = (uint32_t)(remap[e] + (remap_offsets != nullptr ? remap_offsets[e / SPLATAD_THREADS] : 0));
     const bool active = sh_row<VIEW>(e, view, dirs, masks, dx, dy, dz, coeff_row);
     if (VIEW && remap != nullptr && !active) return;
     if (active) sh_color(degree, coeffs + coeff_row * K * 3, dx, dy, dz, r, g, b);
@@ -109,10 +111,10 @@ __global__ void __launch_bounds__(SPLATAD_THREADS)
 sh_fwd_kernel(uint32_t n, uint32_t K, uint32_t degree, ShView view, const float *__restrict__ dirs,
               const float *__restrict__ coeffs, const uint8_t *__restrict__ masks,
               const float *__restrict__ depths, uint32_t stride, float *__restrict__ colors,
-              const int32_t *__restrict__ remap) {
+              const int32_t *__restrict__ remap, const int32_t *__restrict__ remap_offsets) {
     const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= n) return;
-    sh_fwd_row<VIEW>(e, K, degree, view, dirs, coeffs, masks, depths, stride, colors, remap);
+    sh_fwd_row<VIEW>(e, K, degree, view, dirs, coeffs, masks, depths, stride, colors, remap, remap_offsets);
 }
 
 // The colour cache of the compositing kernel that evaluates colours itself
@@ -320,10 +322,11 @@ static int sh_check(uint32_t K, uint32_t degree) {
 template <bool VIEW>
 static int sh_forward(uint32_t n, uint32_t K, uint32_t degree, const ShView &view, const float *dirs,
                       const float *coeffs, const uint8_t *masks, const float *depths,
-                      uint32_t stride, float *colors, hipStream_t stream, const int32_t *remap = nullptr) {
+                      uint32_t stride, float *colors, hipStream_t stream, const int32_t *remap = nullptr,
+                      const int32_t *remap_offsets = nullptr) {
     hipLaunchKernelGGL(sh_fwd_kernel<VIEW>, dim3((n + SPLATAD_THREADS - 1) / SPLATAD_THREADS),
                        dim3(SPLATAD_THREADS), 0, stream, n, K, degree, view, dirs, coeffs, masks,
-                       depths, stride, colors, remap);
+                       depths, stride, colors, remap, remap_offsets);
     SPLATAD_LAUNCH_CHECK();
     return 0;
 }
@@ -440,6 +443,7 @@ extern "C" int splatad_view_colors_cache(uint32_t n, uint32_t C, uint32_t N, uin
 extern "C" int splatad_view_colors_fwd_remapped(uint32_t C, uint32_t N, uint32_t K, uint32_t degree,
                                                 const float *means, const float *viewmats,
                                                 const int32_t *radii, const int32_t *remap,
+                                                const int32_t *remap_offsets,
                                                 const float *coeffs, int coeffs_per_sensor,
                                                 const float *depths, float *colors,
                                                 splatad_stream_t stream) {
@@ -452,7 +456,7 @@ extern "C" int splatad_view_colors_fwd_remapped(uint32_t C, uint32_t N, uint32_t
                               &view)) return rc;
     SPLATAD_REQUIRE(coeffs && colors && remap, "view colours: null pointer argument");
     return sh_forward<true>((uint32_t)n, K, degree, view, nullptr, coeffs, nullptr, depths, depths ? 4u : 3u,
-                            colors, (hipStream_t)stream, remap);
+                            colors, (hipStream_t)stream, remap, remap_offsets);
 }
 
 extern "C" int splatad_view_colors_bwd(uint32_t n, uint32_t C, uint32_t N, uint32_t K,

@@ -24,7 +24,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libsplatad_hip.so")
 _lib = None
 
 
-ABI_VERSION = 9  # splatad_abi_version() of the library these bindings were written for
+ABI_VERSION = 10  # splatad_abi_version() of the library these bindings were written for
 
 
 def load_library():
