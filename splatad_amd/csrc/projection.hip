@@ -372,37 +372,6 @@ static PackedWorkspace carve_packed(void *ws, uint64_t T) {
     return w;
 }
 
-// The per-block totals of the scan over the kept flags (radii.x > 0, SCAN_TILE rows per block,
-// as scan_block_totals_kernel makes them) and, on the same pass, the number of tiles the kept
-// rows of the block meet on the camera's tile grid.
-__global__ void __launch_bounds__(SPLATAD_THREADS)
-packed_block_totals_kernel(uint64_t T, const int32_t *__restrict__ w_radii,
-                           const float *__restrict__ w_means2d, uint32_t tile_size, uint32_t tile_w,
-                           uint32_t tile_h, int64_t *__restrict__ block_sums,
-                           int64_t *__restrict__ tile_sums) {
-    const uint64_t base = (uint64_t)blockIdx.x * SCAN_TILE + (uint64_t)threadIdx.x * SCAN_ITEMS;
-    int64_t kept = 0, tiles = 0;
-#pragma unroll
-    for (int k = 0; k < SCAN_ITEMS; ++k) {
-        const uint64_t idx = base + k;
-        if (idx >= T) continue;
-        const int2 r = reinterpret_cast<const int2 *>(w_radii)[idx];
-        if (r.x <= 0) continue;
-        ++kept;
-        int32_t x0, y0, x1, y1;
-        splatad_camera_tile_rect(tile_size, tile_w, tile_h, reinterpret_cast<const float2 *>(w_means2d)[idx], r,
-                                 x0, y0, x1, y1);
-        tiles += (int64_t)max(y1 - y0, 0) * max(x1 - x0, 0);
-    }
-    int64_t kept_total, tiles_total;
-    block_exclusive_scan(kept, &kept_total);
-    block_exclusive_scan(tiles, &tiles_total);
-    if (threadIdx.x == 0) {
-        block_sums[blockIdx.x] = kept_total;
-        tile_sums[blockIdx.x] = tiles_total;
-    }
-}
-
 // One workgroup: publishes the number of kept rows (low 32 bits) and of their tile
 // intersections (high 32 bits, saturated at 2^31 - 1, which the caller refuses) in one word.
 // The kept rows are *total when that is given, the sum of kept_sums otherwise.
@@ -591,13 +560,11 @@ static int packed_count(uint32_t C, uint32_t N, const float *means, const float 
     // the counts reach the host through a leased pinned word
     HostWordLease lease((hipStream_t)stream);
     if (int rc = host_word_acquire(&lease.word)) return rc;
-    // Up to kScanFoldBlocks scan blocks the projection itself counts, per workgroup, the kept
-    // rows and their tiles: the host word is published right behind it, and the scan's second
-    // half adds up the workgroups' counts before its block (SCAN_ITEMS of them per scan block).
-    static_assert(SCAN_TILE == SCAN_ITEMS * SPLATAD_THREADS, "a scan block is SCAN_ITEMS projection workgroups");
-    const int64_t n_blocks = ((int64_t)T + SCAN_TILE - 1) / SCAN_TILE;
+    // With a tile grid the projection itself counts, per workgroup, the kept rows and their
+    // tiles, and leaves every row's place among the kept rows of its workgroup: the host word is
+    // published right behind it by the kernel that also adds up the workgroups' places.
     const int64_t n_groups = ((int64_t)T + SPLATAD_THREADS - 1) / SPLATAD_THREADS;
-    const bool fused = tile_size != 0 && n_blocks <= kScanFoldBlocks;
+    const bool fused = tile_size != 0;
     int rc = projection_fwd(C, N, means, covars, quats, scales, velocities, viewmats, Ks, W, H, lin_vel,
                             ang_vel, rs_time, eps2d, near_plane, far_plane, radius_clip, w.radii, w.means2d,
                             w.depths, w.conics, calc_compensations ? w.comps : nullptr, w.pix_vels,
@@ -624,27 +591,6 @@ static int packed_count(uint32_t C, uint32_t N, const float *means, const float 
         if (rc) return rc;
         hipLaunchKernelGGL(host_word_publish_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, w.total,
                            lease.word.device);
-    } else {
-        hipLaunchKernelGGL(fill_i32_kernel, dim3((uint32_t)((n_groups + 1 + 255) / 256)), dim3(256), 0,
-                           (hipStream_t)stream, w.offsets, n_groups + 1, 0);
-        hipLaunchKernelGGL(packed_block_totals_kernel, dim3((uint32_t)n_blocks), dim3(SPLATAD_THREADS), 0,
-                           (hipStream_t)stream, T, (const int32_t *)w.radii, (const float *)w.means2d, tile_size,
-                           tile_width, tile_height, w.block_sums, w.tile_sums);
-        SPLATAD_LAUNCH_CHECK();
-        rc = launch_exclusive_scan_apply<int32_t>(w.radii, (int64_t)T, 2, 1, w.pos, w.total, w.block_sums,
-                                                  (hipStream_t)stream);
-        if (rc) return rc;
-        hipLaunchKernelGGL(packed_publish_kernel, dim3(1), dim3(SPLATAD_THREADS), 0, (hipStream_t)stream,
-                           (const int64_t *)w.total, (const int64_t *)nullptr, (const int64_t *)w.tile_sums,
-                           n_blocks, lease.word.device, (int32_t *)nullptr);
-        SPLATAD_LAUNCH_CHECK();
-        // work for the GPU while the host learns the counts and sizes the outputs: the first
-        // stages of the tile intersection, on the dense rows (culled rows meet no tile)
-        if (isect_workspace != nullptr) {
-            rc = splatad_isect_tiles_prepare(T, N, nullptr, w.means2d, w.radii, w.depths, C, tile_size,
-                                             tile_width, tile_height, 1, nullptr, isect_workspace, stream);
-            if (rc) return rc;
-        }
     }
     SPLATAD_LAUNCH_CHECK();
     unsigned long long word = 0;
