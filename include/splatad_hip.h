@@ -282,6 +282,20 @@ int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_t *camera_i
                              const int32_t *tiles_per_gauss, void *workspace, void *lists,
                              int64_t *isect_ids, int32_t *flatten_ids, int32_t *tile_offsets,
                              splatad_stream_t stream);
+/* splatad_isect_tiles_fill with work of the caller's beside the sort: beside_work (may be NULL)
+ * is called once before the call returns, with beside_context and a stream; what the callback
+ * enqueues there must need nothing that is enqueued on `stream` after this call began (the
+ * projection's outputs are fine: the colour cache of splatad_view_colors_cache, say), runs
+ * beside the sort, and has completed as far as `stream` is concerned when the call returns.  No
+ * counterpart in the reference; see splatad_isect_tiles_fill_packed for the mechanism. */
+int splatad_isect_tiles_fill_beside(uint64_t total, uint32_t N, const int64_t *camera_ids,
+                                    const float *means2d, const int32_t *radii, const float *depths,
+                                    uint32_t C, uint32_t tile_size, uint32_t tile_width,
+                                    uint32_t tile_height, int sort, int64_t n_isects,
+                                    const int32_t *tiles_per_gauss, void *workspace, void *lists,
+                                    int64_t *isect_ids, int32_t *flatten_ids, int32_t *tile_offsets,
+                                    splatad_beside_fn beside_work, void *beside_context,
+                                    splatad_stream_t stream);
 int splatad_isect_lidar_tiles_count(uint64_t total, uint32_t N, const int64_t *camera_ids,
                                     const float *means2d, const float *radii, const float *depths,
                                     uint32_t C, const float *elev_boundaries, float tile_azim_resolution,

@@ -15,4 +15,4 @@ void splatad_set_error(const char *fmt, ...) {
 
 extern "C" const char *splatad_last_error(void) { return g_last_error; }
 
-extern "C" int splatad_abi_version(void) { return 10; }
+extern "C" int splatad_abi_version(void) { return 11; }

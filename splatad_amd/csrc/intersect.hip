@@ -3020,11 +3020,26 @@ extern "C" int splatad_isect_tiles_fill(uint64_t total, uint32_t N, const int64_
                                         void *workspace, void *lists, int64_t *isect_ids,
                                         int32_t *flatten_ids, int32_t *tile_offsets,
                                         splatad_stream_t stream) {
+    return splatad_isect_tiles_fill_beside(total, N, camera_ids, means2d, radii, depths, C, tile_size, tile_width,
+                                           tile_height, sort, n_isects, tiles_per_gauss, workspace, lists,
+                                           isect_ids, flatten_ids, tile_offsets, nullptr, nullptr, stream);
+}
+
+extern "C" int splatad_isect_tiles_fill_beside(uint64_t total, uint32_t N, const int64_t *camera_ids,
+                                               const float *means2d, const int32_t *radii,
+                                               const float *depths, uint32_t C, uint32_t tile_size,
+                                               uint32_t tile_width, uint32_t tile_height, int sort,
+                                               int64_t n_isects, const int32_t *tiles_per_gauss,
+                                               void *workspace, void *lists, int64_t *isect_ids,
+                                               int32_t *flatten_ids, int32_t *tile_offsets,
+                                               splatad_beside_fn beside_work, void *beside_context,
+                                               splatad_stream_t stream) {
     SPLATAD_REQUIRE(tile_size > 0, "isect_tiles: tile_size is zero");
     TileGrid g{tile_size, tile_width, tile_height, 0.f, 0.f, nullptr};
     return isect_fill<false>(g, total, N, camera_ids, means2d, radii, depths, C, sort, n_isects,
                              tiles_per_gauss, workspace, lists, isect_ids, flatten_ids,
-                             tile_offsets, (hipStream_t)stream);
+                             tile_offsets, (hipStream_t)stream, nullptr, nullptr, nullptr, beside_work,
+                             beside_context);
 }
 
 extern "C" int splatad_isect_tiles_fill_remapped(uint64_t total, uint32_t N, const float *means2d,

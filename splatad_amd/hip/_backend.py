@@ -10,6 +10,7 @@ torch so that they live in torch's caching allocator, on torch's current stream.
 There is no CPU path: without the built library, or with non-GPU tensors, the ops raise.
 """
 import ctypes
+import threading
 import weakref
 import math
 import os
@@ -24,7 +25,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libsplatad_hip.so")
 _lib = None
 
 
-ABI_VERSION = 10  # splatad_abi_version() of the library these bindings were written for
+ABI_VERSION = 11  # splatad_abi_version() of the library these bindings were written for
 
 
 def load_library():
@@ -78,11 +79,35 @@ def _p(t: Optional[Tensor]):
     return ctypes.c_void_p(0 if t is None or t.numel() == 0 else t.data_ptr())
 
 
+_redirect = threading.local()  # .stream: where this thread's library calls go instead, see library_stream
+
+
 def _stream(device):
     """Handle of torch's current stream on the device (the raw query: the Stream object that
-    torch.cuda.current_stream() builds costs several microseconds per call)."""
+    torch.cuda.current_stream() builds costs several microseconds per call), or the stream that
+    library_stream() has put in its place."""
+    other = getattr(_redirect, "stream", None)
+    if other is not None:
+        return other
     index = device.index if device.index is not None else torch.cuda.current_device()
     return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(index))
+
+
+class library_stream:
+    """`with library_stream(handle)`: the calls this thread makes into the library enqueue on the
+    stream `handle` (a ctypes pointer) instead of torch's current one.  For the callbacks that an
+    intersection call runs beside its sort; torch's own kernels do not follow, so nothing inside
+    may launch one (allocations are fine)."""
+
+    def __init__(self, handle):
+        self.handle = handle
+
+    def __enter__(self):
+        self.before = getattr(_redirect, "stream", None)
+        _redirect.stream = self.handle
+
+    def __exit__(self, *exc):
+        _redirect.stream = self.before
 
 
 class _on:
@@ -587,7 +612,12 @@ class _Ops:
 
     # ------------------------------------------------------------------ intersection
     def _isect(self, lidar, means2d, radii, depths, camera_ids, gaussian_ids, C, grid_args,
-               tile_w, tile_h, sort):
+               tile_w, tile_h, sort, beside_work=None):
+        """beside_work: a callable without arguments, called once before this returns.  Where the
+        call sorts (cameras), it is called from inside the fill call with this thread's library
+        calls redirected to a helper stream of the sort (library_stream): what it enqueues runs
+        beside the sort and is joined with it.  It must launch no torch kernel and need nothing
+        but what was enqueued before this call."""
         # A packed projection that was told the tile grid has made the lists of these rows from its
         # dense copy of them (good for one call, and only for the very tensors it returned,
         # unwritten since).
@@ -597,6 +627,8 @@ class _Ops:
             if (known[0] == (int(grid_args[0].value), tile_w, tile_h) and known[2] == radii._version
                     and known[3]() is means2d and known[4] == means2d._version
                     and known[5]() is depths and known[6] == depths._version and known[7] == C):
+                if beside_work is not None:
+                    beside_work()
                 return known[1]
         filled = getattr(radii, "_splatad_fill_stream", None)
         if filled is not None:
@@ -639,18 +671,40 @@ class _Ops:
             flatten_ids = torch.empty((n_isects,), dtype=torch.int32, device=dev)
             if n_isects:
                 lists = _workspace(lib.splatad_isect_lists_bytes(_u64(total), _i64(n_isects)), dev)
-                _check(fill(*head, *tail, _i64(n_isects), _p(tiles_per_gauss), _p(ws),
-                            _p(lists), _p(isect_ids), _p(flatten_ids), _p(offsets), _stream(dev)))
+                if beside_work is not None and not lidar:
+                    caught = []
+
+                    def run_beside(_context, stream_handle):
+                        try:
+                            with library_stream(ctypes.c_void_p(stream_handle)):
+                                beside_work()
+                            return 0
+                        except BaseException as e:  # (an exception must not cross the C frames)
+                            caught.append(e)
+                            return 1
+
+                    rc = lib.splatad_isect_tiles_fill_beside(
+                        *head, *tail, _i64(n_isects), _p(tiles_per_gauss), _p(ws), _p(lists), _p(isect_ids),
+                        _p(flatten_ids), _p(offsets), _BESIDE_FN(run_beside), None, _stream(dev))
+                    beside_work = None
+                    if caught:
+                        raise caught[0]
+                    _check(rc)
+                else:
+                    _check(fill(*head, *tail, _i64(n_isects), _p(tiles_per_gauss), _p(ws),
+                                _p(lists), _p(isect_ids), _p(flatten_ids), _p(offsets), _stream(dev)))
             else:
                 offsets = None
+            if beside_work is not None:
+                beside_work()
             if offsets is not None:
                 isect_ids._splatad_tile_offsets = (offsets, isect_ids._version)
         return tiles_per_gauss, isect_ids, flatten_ids
 
     def isect_tiles(self, means2d, radii, depths, camera_ids, gaussian_ids, C, tile_size,
-                    tile_width, tile_height, sort, double_buffer):
+                    tile_width, tile_height, sort, double_buffer, beside_work=None):
         return self._isect(False, means2d, radii, depths, camera_ids, gaussian_ids, C,
-                           (_u32(tile_size),), tile_width, tile_height, sort)
+                           (_u32(tile_size),), tile_width, tile_height, sort, beside_work)
 
     def isect_lidar_tiles(self, means2d, radii, depths, camera_ids, gaussian_ids, C,
                           elev_boundaries, tile_azim_resolution, min_azim, sort, double_buffer):

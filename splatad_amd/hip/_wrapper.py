@@ -279,19 +279,27 @@ def isect_tiles(
     n_cameras: Optional[int] = None,
     camera_ids: Optional[Tensor] = None,
     gaussian_ids: Optional[Tensor] = None,
+    beside_work=None,
 ) -> Tuple[Tensor, Tensor, Tensor]:
     """Lists the image tiles every projected Gaussian touches.
 
     Returns (tiles_per_gauss int32[C,N] | [nnz], isect_ids int64[n_isects] with layout
     camera | tile | float bits of depth, flatten_ids int32[n_isects]); sorted by isect id
     (ties in emission order) when `sort`.
+
+    beside_work (not in the reference): a callable without arguments that is called once before
+    this returns, where possible from inside the call with the library's launches redirected to
+    a stream that runs beside the sort and is joined with it.  It may call operators of this
+    package that need only what was enqueued before this call, on contiguous tensors (no torch
+    kernel may be launched inside), e.g. `view_dependent_color_cache`.
     """
     C, camera_ids, gaussian_ids = _check_projected(
         means2d, radii, depths, packed, n_cameras, camera_ids, gaussian_ids
     )
+    more = {} if beside_work is None else {"beside_work": beside_work}
     return _make_lazy_hip_func("isect_tiles")(
         means2d.contiguous(), radii.contiguous(), depths.contiguous(), camera_ids, gaussian_ids,
-        C, tile_size, tile_width, tile_height, sort, True,
+        C, tile_size, tile_width, tile_height, sort, True, **more,
     )
 
 

@@ -199,11 +199,27 @@ def rasterization(
 
     # 2. tile intersection, sort, offsets.  (Work beside it is enqueued behind it: the kernel then
     # meets the segment sort; enqueued first, its launch would stand between the host and the
-    # launches the GPU is waiting for.)
+    # launches the GPU is waiting for.)  The colour cache of a call that evaluates its colours
+    # while compositing needs the projection only: its two short launches are made from inside
+    # the intersection call, on a stream that the sort forks and joins anyway (unpacked calls;
+    # a packed projection has made the cache of its rows the same way).
+    cache_beside_sort = None
+    if (plan.colors == "while_compositing" and not packed and "color_cache" not in beside.results
+            and all(t.is_contiguous() for t in (means, viewmats, colors, radii, depths, opacities))):
+        made = []
+        cache_depths = depths if plan.depth_in_colors else None
+
+        def cache_beside_sort():
+            made.append(view_dependent_color_cache(
+                sh_degree, means, viewmats, colors, radii, cache_depths, opacities, tile_size, tile_width,
+                tile_height, None, None))
+
     tiles_per_gauss, isect_ids, flatten_ids = isect_tiles(
         means2d, radii, depths, tile_size, tile_width, tile_height, packed=packed, n_cameras=C,
-        camera_ids=camera_ids, gaussian_ids=gaussian_ids,
+        camera_ids=camera_ids, gaussian_ids=gaussian_ids, beside_work=cache_beside_sort,
     )
+    if cache_beside_sort is not None:
+        beside.results["color_cache"] = made[0]
     isect_offsets = isect_offset_encode(isect_ids, C, tile_width, tile_height)
 
     # per-row opacities: [nnz], or [C, N] (a view, copied by the first operator that needs it

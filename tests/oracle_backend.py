@@ -74,7 +74,9 @@ class OracleOps:
         return _t(cols)
 
     def isect_tiles(self, means2d, radii, depths, camera_ids, gaussian_ids, C, tile_size, tw, th, sort,
-                    double_buffer):
+                    double_buffer, beside_work=None):
+        if beside_work is not None:
+            beside_work()
         out = oracle.isect_tiles(_n(means2d), _n(radii), _n(depths), tile_size, tw, th, sort, C,
                                  _n(camera_ids))
         return tuple(_t(o) for o in out)

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in include/splatad_hip.h but not exported"
     lib.splatad_abi_version.restype = ctypes.c_int
-    assert lib.splatad_abi_version() == 10
+    assert lib.splatad_abi_version() == 11
     lib.splatad_last_error.restype = ctypes.c_char_p
     assert isinstance(lib.splatad_last_error(), bytes)
     # size queries are pure host code
