@@ -256,3 +256,51 @@ def test_colours_that_are_not_numbers_equal_the_two_operators():
     assert torch.equal(torch.isnan(got[0]), torch.isnan(want[0]))
     assert torch.equal(torch.nan_to_num(got[0], nan=-1.0), torch.nan_to_num(want[0], nan=-1.0))
     assert torch.equal(got[1], want[1])
+
+
+def test_work_beside_the_sort_is_done_once_and_joined():
+    """isect_tiles(beside_work=...) calls the callable exactly once, from inside the fill call with
+    the library's launches on a stream of the sort's, and what it enqueued is complete for the
+    caller's stream when the call returns: the colour cache made there (with every row evaluated,
+    i.e. its filling kernel at work) equals the one made afterwards; the lists are the same; a
+    call that sorts nothing, a call without intersections and a failing callable behave."""
+    from splatad_amd import fully_fused_projection, isect_tiles
+    from splatad_amd.hip._wrapper import view_dependent_color_cache
+    C, N, W, H, ts = 2, 50000, 320, 192, 16
+    d = workloads.to_device(workloads.camera_driving(n=N, seed=3, width=W, height=H, n_cameras=C), DEV)
+    radii, means2d, depths, conics, _, pix_vels = fully_fused_projection(
+        d["means"], None, d["quats"], d["scales"], d["velocities"], d["viewmats"], d["Ks"], W, H,
+        d["linear_velocity"], d["angular_velocity"], d["rolling_shutter_time"], eps2d=d["eps2d"],
+        near_plane=d["near_plane"], far_plane=d["far_plane"], packed=False)
+    tw, th = math.ceil(W / ts), math.ceil(H / ts)
+    cache_args = (3, d["means"], d["viewmats"], d["colors"], radii, depths, d["opacities"], ts, tw, th, None, None)
+    made = []
+
+    def work():
+        # (a threshold that no scene reaches: the second launch evaluates every visible row)
+        made.append(view_dependent_color_cache(*cache_args, min_opacity_per_tile=1e30))
+
+    for sort in (True, False):
+        made.clear()
+        got = isect_tiles(means2d, radii, depths, ts, tw, th, sort=sort, beside_work=work)
+        want = isect_tiles(means2d, radii, depths, ts, tw, th, sort=sort)
+        assert len(made) == 1
+        for g, w in zip(got, want):
+            assert torch.equal(g, w)
+        direct = view_dependent_color_cache(*cache_args, min_opacity_per_tile=1e30)
+        visible = radii[..., 0] > 0
+        assert visible.any() and not torch.isnan(made[0][visible]).any()
+        assert torch.equal(made[0][visible], direct[visible]) and torch.isnan(made[0][~visible]).all()
+    # nothing to intersect: the work is still done, on the caller's stream
+    made.clear()
+    none = isect_tiles(means2d, torch.zeros_like(radii), depths, ts, tw, th, beside_work=work)
+    assert len(made) == 1 and none[1].numel() == 0
+
+    def failing():
+        raise ValueError("from the callable")
+
+    with pytest.raises(ValueError, match="from the callable"):
+        isect_tiles(means2d, radii, depths, ts, tw, th, beside_work=failing)
+    # and the library is in order afterwards
+    again = isect_tiles(means2d, radii, depths, ts, tw, th)
+    assert again[1].numel() == want[1].numel() > 0
