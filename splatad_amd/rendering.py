@@ -53,6 +53,8 @@ def _sensor_motion(C, device, linear_velocity, angular_velocity, rolling_shutter
 # and memory system, and a fork and a join cost 20 us of their own -- and a call then uses one
 # stream only.
 HELPER_STREAM = False
+# rows (sensors x Gaussians) up to which the colour cache is made beside the sort, see rasterization()
+CACHE_BESIDE_SORT_ROWS = 1_500_000
 
 
 class _CameraPlan:
@@ -202,9 +204,13 @@ def rasterization(
     # launches the GPU is waiting for.)  The colour cache of a call that evaluates its colours
     # while compositing needs the projection only: its two short launches are made from inside
     # the intersection call, on a stream that the sort forks and joins anyway (unpacked calls;
-    # a packed projection has made the cache of its rows the same way).
+    # a packed projection has made the cache of its rows the same way).  That stream has about
+    # 14 us to spare on a frame of a million rows, and clearing the cache takes 9 us per million
+    # rows: beyond a million and a half the launches stay behind the sort (measured: 1M rows
+    # 0.3675 -> 0.3585 ms beside the sort, 2M 0.639 -> 0.643, 4M 0.966 -> 0.996).
     cache_beside_sort = None
     if (plan.colors == "while_compositing" and not packed and "color_cache" not in beside.results
+            and C * N <= CACHE_BESIDE_SORT_ROWS
             and all(t.is_contiguous() for t in (means, viewmats, colors, radii, depths, opacities))):
         made = []
         cache_depths = depths if plan.depth_in_colors else None
