@@ -354,6 +354,9 @@ def bench_lidar(args):
         # staged per list entry: id, mean, angular velocity, conic, opacity (40 bytes); the features
         # of the Gaussians a wavefront composites are read on demand and not counted here
         alg_bytes = i_need * 40 + P * (4 * D + 32) + T * 4
+        # the figure with a staged entry's features counted too (4 * D bytes more per entry): what a
+        # kernel that stages whole Gaussians, as the reference's does, has to read
+        alg_bytes_features = i_need * (40 + 4 * D) + P * (4 * D + 32) + T * 4
         stages = {}
         stages["projection_ms"] = time_kernel(lambda: _C.fully_fused_lidar_projection_fwd(
             s["means"], None, s["quats"], s["scales"], s["velocities"], s["viewmats"],
@@ -371,7 +374,7 @@ def bench_lidar(args):
                        "rasterize_ms": alg_bytes}
     return dict(sec=sec, sec_chunk32=sec_chunk32, points=P, kernel_ms=k_ms, alg_bytes=alg_bytes,
                 n_isects=n_isects, i_need=i_need, channels=D, stages=stages, stage_bytes=stage_bytes,
-                tile_cycles=tile_cycles)
+                tile_cycles=tile_cycles, alg_bytes_features=alg_bytes_features)
 
 
 def bench_backward(args):
@@ -725,6 +728,9 @@ def main():
                          "frac": l_ach / HBM_PEAK_GBS,
                          "traffic": hbm_traffic_bytes(counters, lid_kernel),
                          "algorithmic_bytes": lid["alg_bytes"], "kernel_ms": lid["kernel_ms"],
+                         # (the kernel reads the features of the Gaussians it composites only, about
+                         # an eighth of those it stages: its traffic lies between the two figures)
+                         "algorithmic_bytes_with_staged_features": lid["alg_bytes_features"],
                          # the kernel lasts as long as its slowest tile (all tiles resident at once):
                          # vector issue fills less than half of it
                          "valu_issue": valu_roofline(counters, lid_kernel, lid["kernel_ms"])},
