@@ -1521,6 +1521,7 @@ constexpr uint32_t kBlockPairsCap = 32768;  // and about this many intersections
 constexpr uint32_t kBlockMergeCapLidar = 2048, kBlockPairsCapLidar = 12288;
 static_assert(kBlockMergeCap <= 4096 && kBlockMergeCapLidar <= 4096, "classes beyond 4096 entries hold single lists only: the host skips their launches by the longest list");
 constexpr uint32_t kBlockLongMax = 8 * kBlockSortCap; // longest list the block sort takes at all (in parts)
+constexpr int64_t kOneStreamIsects = 1 << 20;         // calls with fewer intersections sort on one stream
 constexpr int kBlockClasses = 6;            // five by length, and the lists beyond kBlockSortCap
 constexpr int kBlockLongClass = 5;
 __constant__ const uint32_t kBlockClassMax[kBlockClasses] = {512u, 2048u, 4096u, 8192u, kBlockSortCap, 0xFFFFFFFFu};
@@ -2877,16 +2878,27 @@ static int isect_fill_with(TileGrid g, uint64_t total, uint32_t N, const int64_t
                            w.seg_starts, tile_offsets, w.piece_counts, (uint32_t)pl.blocks, w.pieces,
                            LIDAR ? kBlockMergeCapLidar : kBlockMergeCap, LIDAR ? kBlockPairsCapLidar : kBlockPairsCap);
         SPLATAD_LAUNCH_CHECK();
-        std::lock_guard<std::mutex> fork_lock(ss->guard);
-        SPLATAD_CHECK_HIP(hipEventRecord(ss->fork, stream));
-        for (hipStream_t aux : ss->aux) SPLATAD_CHECK_HIP(hipStreamWaitEvent(aux, ss->fork, 0));
-        if (beside != nullptr && beside != stream) SPLATAD_CHECK_HIP(hipStreamWaitEvent(beside, ss->fork, 0));
+        // A small call (a few hundred thousand Gaussians at most) is bound by the host and by
+        // launch latencies, not by the GPU: its classes go one behind the other on the caller's
+        // stream, without the fork and the join of the helper streams (three event records and
+        // four cross-stream waits, 45 us of host time).
+        const bool one_stream = n_isects < kOneStreamIsects;
+        hipStream_t const aux0 = one_stream ? stream : ss->aux[0], aux1 = one_stream ? stream : ss->aux[1];
+        const bool orders_beside = beside != nullptr && beside != stream;
+        std::unique_lock<std::mutex> fork_lock(ss->guard, std::defer_lock);
+        if (!one_stream || orders_beside) {
+            fork_lock.lock();
+            SPLATAD_CHECK_HIP(hipEventRecord(ss->fork, stream));
+            if (!one_stream)
+                for (hipStream_t aux : ss->aux) SPLATAD_CHECK_HIP(hipStreamWaitEvent(aux, ss->fork, 0));
+            if (orders_beside) SPLATAD_CHECK_HIP(hipStreamWaitEvent(beside, ss->fork, 0));
+        }
         auto enqueue_block_sorts = [&]() -> int {
             int e;
             // (the caller's work first on the stream of the many mid-sized pieces: measured on a
             // packed frame, its compaction there costs the step 14 us less than behind the sort;
             // on the other helper stream 3 us less, on the caller's own 6 us more)
-            if ((e = beside_work.run(ss->aux[0])) != 0) return e;
+            if ((e = beside_work.run(aux0)) != 0) return e;
 #define SPLATAD_BLOCK_CLASS(cls, ER, threads, hi, wgs, on)                                                        \
             if ((e = launch_block_sort<ER, LIDAR>(cls, threads, hi, wgs, (uint32_t)pl.blocks, cg, g.tile_w, g.tile_h,   \
                                            n_tiles, tile_n_bits, n_isects, w.piece_counts, w.pieces, w.entries,  \
@@ -2902,16 +2914,16 @@ static int isect_fill_with(TileGrid g, uint64_t total, uint32_t N, const int64_t
                                                  w.list_tile_counts, isect_ids, flatten_ids, stream)) != 0)
                 return e;
             if (longest_list > 8192u) SPLATAD_BLOCK_CLASS(4, 10, 1024, kBlockSortCap, 256u, stream)
-            if (longest_list > 4096u) SPLATAD_BLOCK_CLASS(3, 8, 1024, 8192u, 256u, ss->aux[1])
-            SPLATAD_BLOCK_CLASS(2, 8, 512, 4096u, 512u, ss->aux[0])
+            if (longest_list > 4096u) SPLATAD_BLOCK_CLASS(3, 8, 1024, 8192u, 256u, aux1)
+            SPLATAD_BLOCK_CLASS(2, 8, 512, 4096u, 512u, aux0)
             SPLATAD_BLOCK_CLASS(1, 8, 256, 2048u, 1024u, stream)
-            SPLATAD_BLOCK_CLASS(0, 4, 128, 512u, 2048u, ss->aux[1])
+            SPLATAD_BLOCK_CLASS(0, 4, 128, 512u, 2048u, aux1)
 #undef SPLATAD_BLOCK_CLASS
             return 0;
         };
         rc = enqueue_block_sorts();
         // (joined whatever happens: work already queued on the helper streams writes the caller's buffers)
-        for (int k = 0; k < 2; ++k) {
+        for (int k = 0; k < (one_stream ? 0 : 2); ++k) {
             const hipError_t r = hipEventRecord(ss->join[k], ss->aux[k]);
             const hipError_t q = r == hipSuccess ? hipStreamWaitEvent(stream, ss->join[k], 0) : r;
             if (q != hipSuccess && rc == 0) SPLATAD_CHECK_HIP(q);
