@@ -1521,7 +1521,10 @@ constexpr uint32_t kBlockPairsCap = 32768;  // and about this many intersections
 constexpr uint32_t kBlockMergeCapLidar = 2048, kBlockPairsCapLidar = 12288;
 static_assert(kBlockMergeCap <= 4096 && kBlockMergeCapLidar <= 4096, "classes beyond 4096 entries hold single lists only: the host skips their launches by the longest list");
 constexpr uint32_t kBlockLongMax = 8 * kBlockSortCap; // longest list the block sort takes at all (in parts)
-constexpr int64_t kOneStreamIsects = 1 << 20;         // calls with fewer intersections sort on one stream
+// Calls with fewer intersections sort on one stream (measured: camera frames of 0.85 / 1.9 / 3.4 /
+// 8.3M intersections take 0.21 / 0.236 / 0.284 / 0.306 ms that way against 0.21 / 0.258 / 0.305 /
+// 0.31 with the helper streams, a sweep of 1.9M 0.265 against 0.31; the frame of 16.1M needs them)
+constexpr int64_t kOneStreamIsects = 1 << 23;
 constexpr int kBlockClasses = 6;            // five by length, and the lists beyond kBlockSortCap
 constexpr int kBlockLongClass = 5;
 __constant__ const uint32_t kBlockClassMax[kBlockClasses] = {512u, 2048u, 4096u, 8192u, kBlockSortCap, 0xFFFFFFFFu};
@@ -2878,7 +2881,7 @@ static int isect_fill_with(TileGrid g, uint64_t total, uint32_t N, const int64_t
                            w.seg_starts, tile_offsets, w.piece_counts, (uint32_t)pl.blocks, w.pieces,
                            LIDAR ? kBlockMergeCapLidar : kBlockMergeCap, LIDAR ? kBlockPairsCapLidar : kBlockPairsCap);
         SPLATAD_LAUNCH_CHECK();
-        // A small call (a few hundred thousand Gaussians at most) is bound by the host and by
+        // A small call (up to about half a million Gaussians) is bound by the host and by
         // launch latencies, not by the GPU: its classes go one behind the other on the caller's
         // stream, without the fork and the join of the helper streams (three event records and
         // four cross-stream waits, 45 us of host time).
