@@ -108,14 +108,15 @@ def time_kernel(fn, iters, warmup=2):
     for _ in range(warmup):
         fn()
     _sync()
-    start = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
-    stop = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    # one pair of events around all launches: a pair per launch adds the dispatch latency behind
+    # each start marker (4-5 us) to every kernel, which the kernel trace does not count
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
     for i in range(iters):
-        start[i].record()
         fn()
-        stop[i].record()
+    stop.record()
     _sync()
-    return sum(s.elapsed_time(e) for s, e in zip(start, stop)) / iters
+    return start.elapsed_time(stop) / iters
 
 
 def time_kernel_on(make, fn, iters, warmup=2):
@@ -127,14 +128,13 @@ def time_kernel_on(make, fn, iters, warmup=2):
         fn(make())
     xs = [make() for _ in range(iters)]
     _sync()
-    start = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
-    stop = [torch.cuda.Event(enable_timing=True) for _ in range(iters)]
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
     for i in range(iters):  # enqueued back to back, so that the GPU never waits for the host
-        start[i].record()
         fn(xs[i])
-        stop[i].record()
+    stop.record()
     _sync()
-    return sum(s.elapsed_time(e) for s, e in zip(start, stop)) / iters
+    return start.elapsed_time(stop) / iters
 
 
 def staged_isects(tile_entries):
