@@ -120,21 +120,24 @@ def time_kernel(fn, iters, warmup=2):
 
 
 def time_kernel_on(make, fn, iters, warmup=2):
-    """As time_kernel, for fn(x) with x = make() made afresh, outside the timed interval, for
-    every call (a kernel that changes its input)."""
+    """As time_kernel, for fn(x) with x = make() made afresh for every call (a kernel that changes
+    its input), right before the call as in a step, so that fn meets x as warm in the caches as a
+    step's kernel does: the time of make(); fn(x) less the time of make() alone."""
     import torch
 
-    for _ in range(warmup):
-        fn(make())
-    xs = [make() for _ in range(iters)]
-    _sync()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for i in range(iters):  # enqueued back to back, so that the GPU never waits for the host
-        fn(xs[i])
-    stop.record()
-    _sync()
-    return start.elapsed_time(stop) / iters
+    def timed(body):
+        for _ in range(warmup):
+            body()
+        _sync()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):  # enqueued back to back, so that the GPU never waits for the host
+            body()
+        stop.record()
+        _sync()
+        return start.elapsed_time(stop) / iters
+
+    return timed(lambda: fn(make())) - timed(make)
 
 
 def staged_isects(tile_entries):
