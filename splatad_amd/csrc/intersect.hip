@@ -277,9 +277,11 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
         clear[i] = 0;
     // SLABS: the launch has kSlabEstimates workgroups more than count, and those find the depth
     // slabs' bounds meanwhile, each from samples of its own (they count their samples' tiles
-    // themselves); the bounds used are the means of the estimates
+    // themselves); the bounds used are the means of the estimates.  They are the launch's first
+    // workgroups: theirs is the longest chain of dependent steps in the kernel, so they start first.
     const uint32_t n_wgs = gridDim.x - (SLABS ? kSlabEstimates : 0u);
-    if (SLABS && blockIdx.x >= n_wgs) { // uniform across the workgroup
+    const uint32_t slab_wgs = SLABS ? kSlabEstimates : 0u;
+    if (SLABS && blockIdx.x < slab_wgs) { // uniform across the workgroup
         slab_bounds_workgroup(total, depths, [&](uint64_t i) -> int32_t {
             float2 mu = reinterpret_cast<const float2 *>(means2d)[i];
             uint2 rad = reinterpret_cast<const uint2 *>(radii)[i];
@@ -287,7 +289,7 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
             if (!tile_rect_of<LIDAR>(g, mu, rad, x0, y0, x1, y1)) return 0;
             const int32_t tiles = max(y1 - y0, 0) * max(x1 - x0, 0);
             return unit_weights ? min(tiles, 1) : tiles;
-        }, n_slabs, blockIdx.x - n_wgs, slab_bounds);
+        }, n_slabs, blockIdx.x, slab_bounds);
         return;
     }
     if (!count_rows) return; // uniform: a caller that knows the count wants the clearing and the slabs only
@@ -295,7 +297,8 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
     // four Gaussians per lane and step, so that their loads are in flight together (the
     // kernel is bound by memory latency otherwise)
     const uint64_t stride = (uint64_t)n_wgs * blockDim.x;
-    for (uint64_t i0 = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i0 < total; i0 += 4 * stride) {
+    const uint32_t wg = blockIdx.x - slab_wgs;
+    for (uint64_t i0 = (uint64_t)wg * blockDim.x + threadIdx.x; i0 < total; i0 += 4 * stride) {
         float2 mu[4];
         uint2 rad[4];
 #pragma unroll
@@ -345,7 +348,7 @@ isect_count_kernel(TileGrid g, uint64_t total, const float *__restrict__ means2d
         // this kernel and the host or the work enqueued behind it.
         const unsigned long long one = 1ull << 48, low = one - 1ull;
         const uint32_t groups = min(n_wgs, kCountGroups);
-        const uint32_t group = blockIdx.x % groups;
+        const uint32_t group = wg % groups;
         const uint32_t members = n_wgs / groups + (group < n_wgs % groups ? 1u : 0u);
         // The counters are put back to zero on the way, each by the last workgroup that touches
         // it, with an exchange whose result the next step needs: the exchange has been performed
