@@ -1669,8 +1669,17 @@ isect_block_plan_kernel(uint32_t n_blocks, uint32_t bsshift, const int32_t *__re
         const uint32_t list0 = b << bsshift;
         // everything the block needs is requested before any of it is used
         uint32_t v[1u << kSlabShiftMax];
+        if (slabs >= 4) { // the block's totals are whole, aligned int4
+            const int4 *totals4 = reinterpret_cast<const int4 *>(totals + list0);
 #pragma unroll
-        for (uint32_t sl = 0; sl < (1u << kSlabShiftMax); ++sl) v[sl] = sl < slabs ? (uint32_t)totals[list0 + sl] : 0u;
+            for (uint32_t q = 0; q < (1u << kSlabShiftMax) / 4; ++q) {
+                const int4 t = 4 * q < slabs ? totals4[q] : make_int4(0, 0, 0, 0);
+                v[4 * q] = (uint32_t)t.x; v[4 * q + 1] = (uint32_t)t.y; v[4 * q + 2] = (uint32_t)t.z; v[4 * q + 3] = (uint32_t)t.w;
+            }
+        } else {
+#pragma unroll
+            for (uint32_t sl = 0; sl < (1u << kSlabShiftMax); ++sl) v[sl] = sl < slabs ? (uint32_t)totals[list0 + sl] : 0u;
+        }
         const uint32_t block_first = list_starts[list0];
         // the block's intersections: its tiles' counts (copies == 1 here: one counter per tile)
         uint32_t in_tiles[16];
