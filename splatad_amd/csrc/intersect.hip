@@ -1574,16 +1574,18 @@ isect_list_count_kernel(const int64_t *__restrict__ n_entries_ptr, const uint4 *
 // A lane per tile: adds up the tile's counts over the slab lists of its block (the tile's number
 // of intersections, which the scan behind this kernel turns into the tile's start) and leaves in
 // their place the counts of the slabs before each (where a slab's entries start inside the
-// tile's list).
+// tile's list).  Sixteen consecutive lanes take the sixteen tiles of one block, so that every
+// load and store of a wavefront is four whole 64-byte rows of the counter table.
 __global__ void __launch_bounds__(SPLATAD_THREADS)
-isect_tile_totals_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t bsshift, uint32_t n_segments,
+isect_tile_totals_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32_t bsshift, uint32_t n_blocks,
                          int32_t *__restrict__ counts, int32_t *__restrict__ tile_counts) {
-    const uint32_t seg = blockIdx.x * blockDim.x + threadIdx.x;
-    if (seg >= n_segments) return;
-    const uint32_t n_tiles = tile_w * tile_h, cam = seg / n_tiles, r = seg - cam * n_tiles;
-    const uint32_t y = r / tile_w, x = r - y * tile_w;
-    const uint32_t block = cam * cg.cw * cg.ch + (y >> kCoarseRowShift) * cg.cw + (x >> 2);
-    const uint32_t t = ((y & 3u) << 2) | (x & 3u);
+    const uint32_t id = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t block = id >> 4, t = id & 15u;
+    if (block >= n_blocks) return;
+    const uint32_t per_cam = cg.cw * cg.ch, cam = block / per_cam, r = block - cam * per_cam;
+    const uint32_t by = r / cg.cw, bx = r - by * cg.cw;
+    const uint32_t x = (bx << 2) + (t & 3u), y = (by << kCoarseRowShift) + (t >> 2);
+    if (x >= tile_w || y >= tile_h) return; // (a tile beyond the grid's edge: its counters stay zero)
     int32_t *mine = counts + ((size_t)block << bsshift) * 16 + t;
     const uint32_t slabs = 1u << bsshift;
     int32_t c[1u << kSlabShiftMax];
@@ -1595,7 +1597,7 @@ isect_tile_totals_kernel(CoarseGrid cg, uint32_t tile_w, uint32_t tile_h, uint32
         if (sl < slabs) mine[(size_t)sl * 16] = run;
         run += c[sl];
     }
-    tile_counts[seg] = run;
+    tile_counts[cam * tile_w * tile_h + y * tile_w + x] = run;
 }
 
 // First workgroup: cuts every block's slab lists into pieces {first entry, entries, block, first
@@ -2843,8 +2845,9 @@ static int isect_fill_with(TileGrid g, uint64_t total, uint32_t N, const int64_t
         // lists inside the tiles' segments follow
         hipLaunchKernelGGL(isect_list_count_kernel, dim3((uint32_t)bin_wgs), dim3(SPLATAD_THREADS), 0, stream,
                            (const int64_t *)w.n_entries, (const uint4 *)w.entries, w.list_tile_counts);
-        hipLaunchKernelGGL(isect_tile_totals_kernel, grid_for(segs), dim3(SPLATAD_THREADS), 0, stream, cg,
-                           g.tile_w, g.tile_h, pl.bsshift, (uint32_t)segs, w.list_tile_counts, w.tile_counts);
+        hipLaunchKernelGGL(isect_tile_totals_kernel, grid_for((uint64_t)C * cg.cw * cg.ch * 16), dim3(SPLATAD_THREADS), 0,
+                           stream, cg, g.tile_w, g.tile_h, pl.bsshift, C * cg.cw * cg.ch, w.list_tile_counts,
+                           w.tile_counts);
     } else
     hipLaunchKernelGGL((square ? isect_tile_bin_kernel<false, 16> : isect_tile_bin_kernel<false, 0>),
                        dim3((uint32_t)bin_wgs),
